@@ -1,0 +1,129 @@
+/*
+ * onenew_hip.h -- C ABI of the MI355X (gfx950) Conv / MatMul / Gemm backend.
+ *
+ * Two levels:
+ *
+ *  1. Plugin level (what the oneNew host binds).  Three shared objects, libConv_hip.so,
+ *     libMatMul_hip.so and libGemm_hip.so, each export `eval` with the signature of
+ *     onenew_abi.h; they forward to onhip_conv_eval / onhip_matmul_eval / onhip_gemm_eval below.
+ *     These replace device/x86/Conv/conv.c:13 `eval`, device/x86/MatMul/mat_mul.c:10 `eval`
+ *     and device/x86/Gemm/gemm.c:9 `eval` of the reference.
+ *
+ *  2. Kernel level: explicit shapes, device pointers and a HIP stream, no host<->device copies
+ *     and no synchronisation.  This is what benchmarks and parity tests time and check.
+ *
+ * Every function returns 0 on success and a negative code on failure; the text of the last
+ * failure on the calling thread is returned by onhip_last_error().  Nothing throws.
+ */
+#ifndef ONENEW_HIP_H
+#define ONENEW_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+#include "onenew_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ONHIP_OK 0
+#define ONHIP_ERR_ARG (-1)        /* shape / argument the path does not support */
+#define ONHIP_ERR_RUNTIME (-2)    /* a HIP call failed */
+#define ONHIP_ERR_WORKSPACE (-3)  /* caller workspace missing or too small */
+
+/* arithmetic of the multiply-accumulate; accumulation is always fp32 (int32 for W8A32) */
+enum {
+    ONHIP_COMPUTE_F32 = 0,   /* fp32 operands, fp32 MFMA */
+    ONHIP_COMPUTE_BF16 = 1,  /* operands rounded to bf16 (RNE) on the way into LDS */
+    ONHIP_COMPUTE_F16 = 2    /* operands rounded to fp16 (RNE) on the way into LDS */
+};
+
+/*
+ * Geometry and epilogue of one convolution.  Field meaning follows CONV_CONFIG_S and the
+ * OPERAND_S shapes the reference kernel reads (device/x86/Conv/conv.c:77-104,328-350):
+ * activations NCHW, weights [cout, cin/group, kh, kw], pads = top/left/bottom/right,
+ * dilation 1.  group == 1 is a dense convolution, any other value a depthwise convolution with
+ * cin == cout (conv.c:29,597-612).  n is the batch: the result equals n independent batch-1
+ * evaluations of the reference.
+ */
+typedef struct {
+    int32_t n, cin, h, w;
+    int32_t cout, kh, kw;
+    int32_t stride_h, stride_w;
+    int32_t pad_t, pad_l, pad_b, pad_r;
+    int32_t group;
+    int32_t has_bias;       /* 0: no bias and -- as in conv.c:18-27 -- no activation either */
+    int32_t act_type;       /* ACT_TYPE_E */
+    float clip_min, clip_max;
+    float leaky_relu_alpha;
+    float hard_sigmoid_alpha, hard_sigmoid_beta;
+    float input_scale;      /* W8A32 only: activation quantisation step */
+    int32_t compute;        /* ONHIP_COMPUTE_*; dense fp32-storage convolutions only */
+    int32_t out_s8;         /* W8A32 only: 1 = write int8 NCHW, re-quantised with output_scale */
+    float output_scale;
+} onhip_conv_desc_t;
+
+/*
+ * out[b] = A[b] (M x K, row-major) * B (K x N, row-major, shared when b_shared else per batch),
+ * optionally + bias[n] and then the table GELU of device/x86/Gelu/gelu.c:22-38.
+ * Plain MatMul (mat_mul.c:10-102) is bias == NULL, gelu_lut == NULL.
+ */
+typedef struct {
+    int32_t batch, m, k, n;
+    int32_t b_shared;
+    int32_t compute;        /* ONHIP_COMPUTE_* */
+} onhip_matmul_desc_t;
+
+/* ---- library -------------------------------------------------------------------------- */
+
+/* Selects the device, checks it is gfx950 and loads the kernels.  Idempotent. */
+int onhip_init(int device);
+/* Text of the last error on this thread ("" if none). */
+const char *onhip_last_error(void);
+/* Output height / width of a convolution (host/ops/conv.h:43-50). Returns 0 or ONHIP_ERR_ARG. */
+int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow);
+
+/* ---- kernel level: device pointers, asynchronous on `stream` (a hipStream_t, NULL = default) - */
+
+/* fp32 convolution + bias + activation.  Replaces conv.c eval_1x1j1 (:68), eval_mxn_img2col
+ * (:300), eval_mxn_img2col_no_bias (:417), eval_depthwise_conv_mxn_img2col (:527),
+ * eval_depthwise_conv_3x3_pad1 (:757) and do_act (:1216).  silu_lut (8192 floats) is required
+ * for act_type SILU only. */
+int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,
+                     const float *silu_lut, float *y, void *stream);
+
+/* Bytes of device scratch onhip_conv2d_w8a32 needs for `d` (the int8 copy of the activations). */
+size_t onhip_conv2d_w8a32_workspace(const onhip_conv_desc_t *d);
+
+/* W8A32 convolution: fp32 activations quantised with d->input_scale, int8 weights
+ * [cout, cin/group, kh, kw], int32 bias, int32 accumulation, fp32 de-quantisation with
+ * weight_aux[oc] / 127, activation.  Replaces conv.c eval_mxn_img2col_W8A32_with_input_scale
+ * (:901), ..._no_bias (:1061), eval_depthwise_conv_mxn_img2col_W8A32 (:617) and do_act.
+ * y is float* (d->out_s8 == 0) or int8_t* (d->out_s8 == 1).  acc32, when not NULL, receives
+ * the raw int32 accumulators (NCHW) for bit-exactness checks. */
+int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t *w8,
+                       const int32_t *bias32, const float *weight_aux, const float *silu_lut,
+                       void *y, int32_t *acc32, void *workspace, size_t workspace_bytes,
+                       void *stream);
+
+/* Batched MatMul with optional fused bias and table GELU.  Replaces mat_mul.c eval (:10) and,
+ * with bias/gelu_lut, the chain MatMul -> Add -> Gelu (device/x86/Gelu/gelu.c:9). */
+int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
+                 const float *gelu_lut, float *out, void *stream);
+
+/* out[m][n] = sum_k a[m][k] * w[n][k] + bias[n].  Replaces gemm.c eval (:9). */
+int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w,
+                   const float *bias, float *out, void *stream);
+
+/* ---- plugin level: the reference slot arrays; host or device pointers; synchronous --------- */
+
+int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* Drops the device copies of weights the plugin level keeps between calls. */
+int onhip_plugin_release(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ONENEW_HIP_H */

@@ -1,0 +1,250 @@
+"""Host side of the operator plugin boundary: the slot arrays the oneNew runtime hands to a
+plugin's ``eval`` and operator objects that fill them the way the reference host classes do.
+
+Mirrors, for the Conv / MatMul / Gemm path only:
+  host/op.h:35-39,109-185     params_vec / inputs_vec / outputs_vec, rt_prepare, forward
+  host/ops/conv.h:31-58,60-157,178-194   shape inference, slot filling, SiLU table
+  host/ops/mat_mul.h:32-57, host/ops/gemm.h:28-48    output shapes
+An operator object owns host buffers exactly like the reference (weights live for the lifetime of
+the object, activations are caller buffers) and calls whatever ``eval`` it is given: the HIP plugin
+of this package or any other shared object with the same symbol.
+"""
+import ctypes as C
+import numpy as np
+
+from . import abi
+from .abi import (BUFFER_INFO_S, OPERAND_S, CONV_CONFIG_S, GEMM_CONFIG_S, MATMUL_CONFIG_S, USEFUL_INFO_S,
+                  BUF_MAXNUM, ConvDesc)
+
+EVAL_T = C.CFUNCTYPE(C.c_int, C.POINTER(BUFFER_INFO_S), C.POINTER(BUFFER_INFO_S), C.POINTER(BUFFER_INFO_S))
+
+
+class Plugin:
+    """A shared object exporting ``eval`` (host/op.h:41-80 find_handle)."""
+
+    def __init__(self, path):
+        self.path = str(path)
+        self.lib = C.CDLL(self.path, mode=C.RTLD_LOCAL)
+        self.eval = self.lib.eval
+        self.eval.restype = C.c_int
+        self.eval.argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
+
+
+def aligned_empty(shape, dtype=np.float32, align=64, extra=16):
+    """host buffer aligned like the runtime's aligned_alloc(32, ...) (host/net.h:434-449), with a few
+    spare elements because the reference int8 quantiser reads past the end (conv.c:967-973)"""
+    dtype = np.dtype(dtype)
+    n = int(np.prod(shape))
+    raw = np.zeros((n + extra) * dtype.itemsize + align, dtype=np.uint8)
+    off = (-raw.ctypes.data) % align
+    return raw[off:off + n * dtype.itemsize].view(dtype).reshape(shape)
+
+
+def make_operand(shape, name=b"", fixed=False, dtype=abi.TYPE_FP32):
+    o = OPERAND_S()
+    o.operand_name = name
+    o.is_fixed_val = int(fixed)
+    o.dim_num_of_shapes = len(shape)
+    for i in range(abi.SHAPE_LEN):
+        o.shapes[i] = int(shape[i]) if i < len(shape) else 1
+    o.data_type = dtype
+    return o
+
+
+def make_useful_info(scratch_bytes=0):
+    """per-model tunables with the defaults onnx2one writes (tools/onnx2one/onnx2one.cpp:1332-1350);
+    returns (struct, scratch array or None)"""
+    u = USEFUL_INFO_S()
+    u.useful_info_magic_num = abi.USEFUL_INFO_MAGIC_NUM
+    bi = u.block_info
+    bi.x86_gemm_single_threads_tile_m, bi.x86_gemm_single_threads_tile_n, bi.x86_gemm_single_threads_tile_k = 32, 1024, 8
+    bi.x86_gemm_multi_threads_tile_m, bi.x86_gemm_multi_threads_tile_n, bi.x86_gemm_multi_threads_tile_k = 32, 1024, 8
+    bi.cuda_gemm_tile_m = bi.cuda_gemm_tile_n = bi.cuda_gemm_tile_k = 16
+    scratch = None
+    if scratch_bytes:
+        scratch = aligned_empty((scratch_bytes,), np.uint8, extra=0)
+        u.public_buf_info.public_buf_size = scratch_bytes
+        u.public_buf_info.public_buf_ptr = scratch.ctypes.data
+    return u, scratch
+
+
+def build_silu_lut():
+    """host/ops/conv.h:178-194, all-float: x = i/512 - 8, x / (1 + expf(-x)).  The table handed to a
+    plugin in production is built by the oneNew host with its libm; this numpy form is for callers
+    that have none.  Parity tests use the committed table in tests/golden."""
+    x = (np.arange(8192, dtype=np.float32) * np.float32(1.0 / 512) - np.float32(8.0)).astype(np.float32)
+    return (x / (np.float32(1.0) + np.exp(-x, dtype=np.float32))).astype(np.float32)
+
+
+class _Op:
+    def __init__(self, evalfn):
+        self.eval = evalfn
+        self.params_vec = (BUFFER_INFO_S * BUF_MAXNUM)()
+        self.inputs_vec = (BUFFER_INFO_S * BUF_MAXNUM)()
+        self.outputs_vec = (BUFFER_INFO_S * BUF_MAXNUM)()
+        self._keep = []
+
+    def _slot(self, vec, i, obj):
+        """obj: ctypes struct (address of), numpy array (data pointer) or int (raw address)"""
+        if isinstance(obj, np.ndarray):
+            addr = obj.ctypes.data
+        elif isinstance(obj, int):
+            addr = obj
+        else:
+            addr = C.addressof(obj)
+        self._keep.append(obj)
+        vec[i].addr = addr
+
+    def forward(self):
+        """host/op.h:171-185"""
+        return self.eval(self.params_vec, self.inputs_vec, self.outputs_vec)
+
+
+class Conv(_Op):
+    """host/ops/conv.h.  ``desc`` carries geometry and epilogue; weights are fp32 [cout, cin/g, kh, kw]
+    or, for the W8A32 form, int8 packed at the front of the fp32-sized buffer with an int32 bias
+    (tools/optimize/model_quant.hpp:14-25)."""
+
+    def __init__(self, evalfn, desc, weight, bias=None, weight_aux=None, silu_lut=None, scratch_bytes=0):
+        super().__init__(evalfn)
+        d = self.desc = ConvDesc.from_buffer_copy(desc)
+        cfg = self.conv_cfg = CONV_CONFIG_S()
+        cfg.op_base_cfg.op_type = b"Conv"
+        cfg.op_base_cfg.in_operand_num = 3 if d.has_bias else 2
+        cfg.op_base_cfg.out_operand_num = 1
+        cfg.has_bias = d.has_bias
+        cfg.dilations[0] = cfg.dilations[1] = 1
+        cfg.group = d.group
+        cfg.kernel_shape[0], cfg.kernel_shape[1] = d.kh, d.kw
+        cfg.pads[0], cfg.pads[1], cfg.pads[2], cfg.pads[3] = d.pad_t, d.pad_l, d.pad_b, d.pad_r
+        cfg.strides[0], cfg.strides[1] = d.stride_h, d.stride_w
+        cfg.act_type = d.act_type
+        cfg.clip_min, cfg.clip_max = d.clip_min, d.clip_max
+        cfg.leaky_relu_alpha = d.leaky_relu_alpha
+        cfg.hard_sigmoid_alpha, cfg.hard_sigmoid_beta = d.hard_sigmoid_alpha, d.hard_sigmoid_beta
+        self.int8 = weight_aux is not None
+        if self.int8:
+            cfg.ifmap_quant2 = abi.TYPE_INT8
+            cfg.input_scale = d.input_scale
+            aux = np.asarray(weight_aux, dtype=np.float32)
+            assert aux.shape == (d.cout,) and d.cout <= 4096
+            C.memmove(cfg.weight_aux, aux.ctypes.data, aux.nbytes)
+        kc = d.cin if d.group == 1 else 1
+        wshape = (d.cout, kc, d.kh, d.kw)
+        # weight / bias storage is always sized as fp32, as in std::vector<float> initial_datas
+        self.weight = aligned_empty(wshape, np.float32)
+        if self.int8:
+            w8 = np.ascontiguousarray(weight, dtype=np.int8).reshape(-1)
+            self.weight.reshape(-1).view(np.int8)[:w8.size] = w8
+        else:
+            self.weight[...] = np.asarray(weight, dtype=np.float32).reshape(wshape)
+        self.weight_operand = make_operand(wshape, b"weight", fixed=True)
+        self.useful, self._scratch = make_useful_info(scratch_bytes)
+        oh, ow = d.out_hw()
+        self.in_operand = make_operand((d.n, d.cin, d.h, d.w), b"in")
+        self.out_operand = make_operand((d.n, d.cout, oh, ow), b"out")
+        self._slot(self.params_vec, 0, cfg)
+        self._slot(self.params_vec, 1, self.in_operand)
+        self._slot(self.params_vec, 2, self.weight_operand)
+        self._slot(self.inputs_vec, 1, self.weight)
+        if d.has_bias:
+            self.bias = aligned_empty((d.cout,), np.float32)
+            if self.int8:
+                self.bias.view(np.int32)[...] = np.asarray(bias, dtype=np.int32)
+            else:
+                self.bias[...] = np.asarray(bias, dtype=np.float32)
+            self.bias_operand = make_operand((d.cout,), b"bias", fixed=True)
+            self._slot(self.params_vec, 3, self.bias_operand)
+            self._slot(self.inputs_vec, 2, self.bias)
+            self._slot(self.params_vec, 4, self.out_operand)
+        else:
+            self._slot(self.params_vec, 3, self.out_operand)
+        self._slot(self.params_vec, BUF_MAXNUM - 1, self.useful)
+        if d.act_type == abi.SILU:
+            self.lut = np.ascontiguousarray(silu_lut if silu_lut is not None else build_silu_lut(), dtype=np.float32)
+            self._slot(self.inputs_vec, BUF_MAXNUM - 1, self.lut)
+
+    def __call__(self, x, out=None):
+        d = self.desc
+        oh, ow = d.out_hw()
+        xin = x if isinstance(x, int) else np.ascontiguousarray(x, dtype=np.float32)
+        if out is None:
+            out = aligned_empty((d.n, d.cout, oh, ow), np.float32)
+        self._slot(self.inputs_vec, 0, xin)
+        self._slot(self.outputs_vec, 0, out)
+        rc = self.forward()
+        del self._keep[-2:]
+        if rc != 0:
+            raise RuntimeError(f"Conv eval returned {rc}")
+        return out
+
+
+class MatMul(_Op):
+    """host/ops/mat_mul.h: out = A[..., M, K] @ B, B either [K, N] shared or batched like A."""
+
+    def __init__(self, evalfn):
+        super().__init__(evalfn)
+        self.mat_mul_cfg = MATMUL_CONFIG_S()
+        self.mat_mul_cfg.op_base_cfg.op_type = b"MatMul"
+        self.mat_mul_cfg.op_base_cfg.in_operand_num = 2
+        self.mat_mul_cfg.op_base_cfg.out_operand_num = 1
+        self._slot(self.params_vec, 0, self.mat_mul_cfg)
+
+    def __call__(self, a, b, out=None):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        oshape = a.shape[:-1] + (b.shape[-1],)
+        if out is None:
+            out = aligned_empty(oshape, np.float32)
+        ops = [make_operand(a.shape, b"a"), make_operand(b.shape, b"b"), make_operand(oshape, b"out")]
+        for i, o in enumerate(ops):
+            self._slot(self.params_vec, 1 + i, o)
+        self._slot(self.inputs_vec, 0, a)
+        self._slot(self.inputs_vec, 1, b)
+        self._slot(self.outputs_vec, 0, out)
+        rc = self.forward()
+        del self._keep[-6:]
+        if rc != 0:
+            raise RuntimeError(f"MatMul eval returned {rc}")
+        return out
+
+
+class Gemm(_Op):
+    """host/ops/gemm.h: out[M, N] = A[M, K] @ W[N, K]^T + bias[N]; alpha, beta, transB ignored."""
+
+    def __init__(self, evalfn, weight, bias):
+        super().__init__(evalfn)
+        self.gemm_cfg = GEMM_CONFIG_S()
+        self.gemm_cfg.op_base_cfg.op_type = b"Gemm"
+        self.gemm_cfg.op_base_cfg.in_operand_num = 3
+        self.gemm_cfg.op_base_cfg.out_operand_num = 1
+        self.gemm_cfg.has_bias = 1
+        self.gemm_cfg.alpha = self.gemm_cfg.beta = 1.0
+        self.gemm_cfg.transB = 1
+        self.weight = aligned_empty(np.shape(weight), np.float32)
+        self.weight[...] = weight
+        self.bias = aligned_empty(np.shape(bias), np.float32)
+        self.bias[...] = bias
+        self.w_operand = make_operand(self.weight.shape, b"w", fixed=True)
+        self.b_operand = make_operand(self.bias.shape, b"bias", fixed=True)
+        self._slot(self.params_vec, 0, self.gemm_cfg)
+        self._slot(self.params_vec, 2, self.w_operand)
+        self._slot(self.params_vec, 3, self.b_operand)
+        self._slot(self.inputs_vec, 1, self.weight)
+        self._slot(self.inputs_vec, 2, self.bias)
+
+    def __call__(self, a, out=None):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        oshape = a.shape[:-1] + (self.bias.shape[0],)
+        if out is None:
+            out = aligned_empty(oshape, np.float32)
+        ain, aout = make_operand(a.shape, b"a"), make_operand(oshape, b"out")
+        self._slot(self.params_vec, 1, ain)
+        self._slot(self.params_vec, 4, aout)
+        self._slot(self.inputs_vec, 0, a)
+        self._slot(self.outputs_vec, 0, out)
+        rc = self.forward()
+        del self._keep[-4:]
+        if rc != 0:
+            raise RuntimeError(f"Gemm eval returned {rc}")
+        return out

@@ -1,0 +1,120 @@
+"""Layer-shape tables of the benchmark configurations (convolutions and matmuls at their real
+shapes).  ResNet-50 follows the torchvision v1.5 layout that the reference's recorded trace
+(tools/perf_profiling/timeline_info/resnet50.csv) confirms through its per-layer MFLOP counts."""
+from .abi import ConvDesc, MatmulDesc, NOT_ACT, RELU, CLIP, SILU
+
+
+def conv(name, cin, cout, k, s, p, hw, act=RELU, group=1, clip=(0.0, 6.0)):
+    d = ConvDesc(n=1, cin=cin, h=hw, w=hw, cout=cout, kh=k, kw=k, stride_h=s, stride_w=s,
+                 pad_t=p, pad_l=p, pad_b=p, pad_r=p, group=group, has_bias=1, act_type=act)
+    if act == CLIP:
+        d.clip_min, d.clip_max = clip
+    return name, d
+
+
+def resnet50(relu_everywhere=True):
+    """53 convolutions; 8174.3 MFLOP per image.  The real graph fuses ReLU into 33 of them (stem,
+    conv1, conv2); relu_everywhere=True applies it to all, as the benchmark configuration states."""
+    L = [conv("stem", 3, 64, 7, 2, 3, 224)]
+    lin = RELU if relu_everywhere else NOT_ACT
+    inplanes, hw = 64, 56
+    for li, (planes, blocks, stride) in enumerate([(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)], 1):
+        for b in range(blocks):
+            s = stride if b == 0 else 1
+            p = f"l{li}.{b}"
+            L.append(conv(p + ".conv1", inplanes, planes, 1, 1, 0, hw))
+            L.append(conv(p + ".conv2", planes, planes, 3, s, 1, hw))
+            if b == 0:
+                L.append(conv(p + ".down", inplanes, planes * 4, 1, s, 0, hw, act=lin))
+            hw //= s
+            L.append(conv(p + ".conv3", planes, planes * 4, 1, 1, 0, hw, act=lin))
+            inplanes = planes * 4
+    return L
+
+
+def mobilenet_v2():
+    """52 convolutions, 17 of them depthwise 3x3 pad 1; ReLU6 arrives as CLIP(0, 6)."""
+    L = [conv("stem", 3, 32, 3, 2, 1, 224, act=CLIP)]
+    cin, hw = 32, 112
+    cfg = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]
+    bi = 0
+    for t, c, n, s in cfg:
+        for i in range(n):
+            bi += 1
+            stride = s if i == 0 else 1
+            hidden = cin * t
+            if t != 1:
+                L.append(conv(f"b{bi}.expand", cin, hidden, 1, 1, 0, hw, act=CLIP))
+            L.append(conv(f"b{bi}.dw", hidden, hidden, 3, stride, 1, hw, act=CLIP, group=hidden))
+            hw //= stride
+            L.append(conv(f"b{bi}.project", hidden, c, 1, 1, 0, hw, act=NOT_ACT))
+            cin = c
+    L.append(conv("last", 320, 1280, 1, 1, 0, 7, act=CLIP))
+    return L
+
+
+def vit_tiny(batch=1):
+    """MatMuls of one ViT-Tiny/16 block at 197 tokens, dim 192, 3 heads x 64.
+    Returns (name, MatmulDesc, has_bias, gelu)."""
+    T, D, H = 197, 192, 3
+    return [
+        ("qkv", MatmulDesc(batch=batch, m=T, k=D, n=3 * D, b_shared=1), False, False),
+        ("scores", MatmulDesc(batch=batch * H, m=T, k=D // H, n=T, b_shared=0), False, False),
+        ("context", MatmulDesc(batch=batch * H, m=T, k=T, n=D // H, b_shared=0), False, False),
+        ("proj", MatmulDesc(batch=batch, m=T, k=D, n=D, b_shared=1), False, False),
+        ("fc1", MatmulDesc(batch=batch, m=T, k=D, n=4 * D, b_shared=1), True, True),
+        ("fc2", MatmulDesc(batch=batch, m=T, k=4 * D, n=D, b_shared=1), True, False),
+    ]
+
+
+def yolov8s():
+    """Convolutions of YOLOv8s at 640x640 (public ultralytics yolov8.yaml, scale s: widths
+    32/64/128/256/512, depth 1/2/2/1 bottlenecks).  SiLU everywhere except the final 1x1
+    predictors.  The reference ships no YOLO graph; this list restates the public definition."""
+    L = []
+
+    def cv(name, cin, cout, k, s, hw, act=SILU):
+        L.append(conv(name, cin, cout, k, s, k // 2, hw, act=act))
+
+    def c2f(name, cin, cout, n, hw):
+        c = cout // 2
+        cv(name + ".cv1", cin, cout, 1, 1, hw)
+        for i in range(n):
+            cv(f"{name}.m{i}.cv1", c, c, 3, 1, hw)
+            cv(f"{name}.m{i}.cv2", c, c, 3, 1, hw)
+        cv(name + ".cv2", (2 + n) * c, cout, 1, 1, hw)
+
+    cv("b0", 3, 32, 3, 2, 640)
+    cv("b1", 32, 64, 3, 2, 320)
+    c2f("b2", 64, 64, 1, 160)
+    cv("b3", 64, 128, 3, 2, 160)
+    c2f("b4", 128, 128, 2, 80)
+    cv("b5", 128, 256, 3, 2, 80)
+    c2f("b6", 256, 256, 2, 40)
+    cv("b7", 256, 512, 3, 2, 40)
+    c2f("b8", 512, 512, 1, 20)
+    cv("sppf.cv1", 512, 256, 1, 1, 20)
+    cv("sppf.cv2", 1024, 512, 1, 1, 20)
+    c2f("n12", 768, 256, 1, 40)
+    c2f("n15", 384, 128, 1, 80)
+    cv("n16", 128, 128, 3, 2, 80)
+    c2f("n18", 384, 256, 1, 40)
+    cv("n19", 256, 256, 3, 2, 40)
+    c2f("n21", 768, 512, 1, 20)
+    for c, hw in ((128, 80), (256, 40), (512, 20)):
+        cv(f"det{hw}.box0", c, 64, 3, 1, hw)
+        cv(f"det{hw}.box1", 64, 64, 3, 1, hw)
+        cv(f"det{hw}.box2", 64, 64, 1, 1, hw, act=NOT_ACT)
+        cv(f"det{hw}.cls0", c, 128, 3, 1, hw)
+        cv(f"det{hw}.cls1", 128, 128, 3, 1, hw)
+        cv(f"det{hw}.cls2", 128, 80, 1, 1, hw, act=NOT_ACT)
+    return L
+
+
+def with_batch(layers, n):
+    out = []
+    for name, d in layers:
+        e = ConvDesc.from_buffer_copy(d)
+        e.n = n
+        out.append((name, e))
+    return out

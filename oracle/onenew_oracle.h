@@ -1,0 +1,39 @@
+/*
+ * onenew_oracle.h -- CPU restatement of the oneNew x86 Conv / MatMul / Gemm arithmetic.
+ * TEST INFRASTRUCTURE ONLY: parity checker and timed CPU baseline, never part of the shipped
+ * library.  All pointers are host memory.  Functions return 0, -1 (bad argument), -2 (no memory).
+ */
+#ifndef ONENEW_ORACLE_H
+#define ONENEW_ORACLE_H
+
+#include <stdint.h>
+#include "../include/onenew_hip.h" /* onhip_conv_desc_t, ACT_TYPE_E values */
+
+#define ORACLE_LUT_LEN 8192
+
+void oracle_set_threads(int t);
+int oracle_get_threads(void);
+int oracle_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow);
+
+void oracle_build_silu_lut(float *lut);
+void oracle_build_gelu_lut(float *lut);
+void oracle_lut_act_f32(const float *x, const float *lut, float *y, int64_t count);
+
+int oracle_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,
+                      const float *silu_lut, float *y);
+
+void oracle_quantize_s8(const float *x, float scale, int8_t *q, int64_t count);
+void oracle_requantize_s8(const float *y, float output_scale, int8_t *q, int64_t count);
+int oracle_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, const int32_t *bias32,
+                        const float *weight_aux, const float *silu_lut, void *y, int32_t *acc32);
+void oracle_quant_weight_bias(const float *w, const float *bias, int cout, int per_channel, int8_t *w8,
+                              int32_t *bias32, float *weight_aux);
+
+int oracle_matmul_f32(int batch, int M, int K, int N, int b_shared, const float *A, const float *B, float *C);
+int oracle_gemm_f32(int M, int K, int N, const float *A, const float *W, const float *bias, float *C);
+int oracle_matmul_bias_gelu_f32(int batch, int M, int K, int N, int b_shared, const float *A, const float *B,
+                                const float *bias, const float *gelu_lut, float *C);
+void oracle_round_bf16(const float *x, float *y, int64_t count);
+void oracle_round_f16(const float *x, float *y, int64_t count);
+
+#endif

@@ -1,0 +1,80 @@
+"""Writes tests/golden/golden.npz and the two activation tables from the reference's own x86
+kernels, compiled in place by `make -C oracle ref` (outputs in oracle/_ref).  Runs only where the
+reference sources are mounted; the fixtures it writes are committed.
+
+    python tests/golden/make_golden.py
+
+For every case of tests/golden/cases.py the reference `eval` is called through the same slot
+arrays the oneNew host fills (onenew_amd.ops) and the output is summarised by cases.summarize."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, HERE)
+import cases  # noqa: E402
+from onenew_amd import abi, ops  # noqa: E402
+from oracle import oracle  # noqa: E402
+
+
+def main():
+    subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "ref"])
+    ref = os.path.join(ROOT, "oracle", "_ref")
+    subprocess.check_call([os.path.join(ref, "lutdump"), cases.SILU_LUT, cases.GELU_LUT])
+    silu, gelu = cases.silu_lut(), cases.gelu_lut()
+    conv = ops.Plugin(oracle.ref_path("Conv"))
+    matmul = ops.Plugin(oracle.ref_path("MatMul"))
+    gemm = ops.Plugin(oracle.ref_path("Gemm"))
+    gelu_so = ops.Plugin(os.path.join(ref, "libGelu_x86.so"))
+    out = {}
+
+    def put(name, tensor):
+        for k, v in cases.summarize(name, tensor).items():
+            out[f"{name}/{k}"] = v
+
+    for name, d in cases.conv_f32_cases().items():
+        x, w, b = cases.conv_inputs(name, d)
+        op = ops.Conv(conv.eval, d, w, b, silu_lut=silu, scratch_bytes=oracle.ref_scratch_bytes(d))
+        put(name, op(x))
+        print("conv f32", name, flush=True)
+    for name, d in cases.conv_w8a32_cases().items():
+        x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+        op = ops.Conv(conv.eval, d, w8, b32, weight_aux=aux, silu_lut=silu, scratch_bytes=oracle.ref_scratch_bytes(d))
+        xin = ops.aligned_empty(x.shape)
+        xin[...] = x
+        put(name, op(xin))
+        print("conv w8a32", name, flush=True)
+    for name, (ash, bsh) in cases.matmul_cases().items():
+        a, b = cases.matmul_inputs(name, ash, bsh)
+        aa, bb = ops.aligned_empty(a.shape), ops.aligned_empty(b.shape)
+        aa[...], bb[...] = a, b
+        put(name, ops.MatMul(matmul.eval)(aa, bb))
+        print("matmul", name, flush=True)
+    for name, (M, K, N) in cases.gemm_cases().items():
+        a, w, b = cases.gemm_inputs(name, M, K, N)
+        put(name, ops.Gemm(gemm.eval, w, b)(a))
+        print("gemm", name, flush=True)
+    # table GELU (device/x86/Gelu/gelu.c) on edge values
+    x = cases.gelu_input()
+    params = (abi.BUFFER_INFO_S * abi.BUF_MAXNUM)()
+    inputs = (abi.BUFFER_INFO_S * abi.BUF_MAXNUM)()
+    outputs = (abi.BUFFER_INFO_S * abi.BUF_MAXNUM)()
+    cfg = abi.MATMUL_CONFIG_S()          # GELU_CONFIG_S is a bare BASE_CONFIG_S as well
+    operand = ops.make_operand(x.shape)
+    y = np.empty_like(x)
+    import ctypes as C
+    params[0].addr, params[1].addr = C.addressof(cfg), C.addressof(operand)
+    inputs[0].addr, inputs[abi.BUF_MAXNUM - 1].addr = x.ctypes.data, gelu.ctypes.data
+    outputs[0].addr = y.ctypes.data
+    gelu_so.eval(params, inputs, outputs)
+    put("gelu_edges", y)
+    np.savez_compressed(cases.GOLDEN_NPZ, **out)
+    print("wrote", cases.GOLDEN_NPZ, os.path.getsize(cases.GOLDEN_NPZ), "bytes,", len(out), "arrays")
+
+
+if __name__ == "__main__":
+    main()

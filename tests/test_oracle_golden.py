@@ -1,0 +1,47 @@
+"""Pins the CPU oracle against outputs of the reference's own compiled x86 kernels
+(tests/golden/golden.npz, written by tests/golden/make_golden.py): bit-identical for every fp32 and
+W8A32 convolution path, MatMul, Gemm and the table activations."""
+import numpy as np
+import pytest
+
+import cases
+
+
+@pytest.mark.parametrize("name", list(cases.conv_f32_cases()))
+def test_conv_f32_bit_exact(name, golden, oracle):
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    y = oracle.conv2d_f32(d, x, w, b, cases.silu_lut())
+    cases.check_against(golden, name, y, exact=True)
+
+
+@pytest.mark.parametrize("name", list(cases.conv_w8a32_cases()))
+def test_conv_w8a32_bit_exact(name, golden, oracle):
+    d = cases.conv_w8a32_cases()[name]
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    y = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut())
+    cases.check_against(golden, name, y, exact=True)
+
+
+@pytest.mark.parametrize("name", list(cases.matmul_cases()))
+def test_matmul_bit_exact(name, golden, oracle):
+    a, b = cases.matmul_inputs(name, *cases.matmul_cases()[name])
+    cases.check_against(golden, name, oracle.matmul_f32(a, b), exact=True)
+
+
+@pytest.mark.parametrize("name", list(cases.gemm_cases()))
+def test_gemm_bit_exact(name, golden, oracle):
+    a, w, b = cases.gemm_inputs(name, *cases.gemm_cases()[name])
+    cases.check_against(golden, name, oracle.gemm_f32(a, w, b), exact=True)
+
+
+def test_gelu_table_apply(golden, oracle):
+    y = oracle.lut_act(cases.gelu_input(), cases.gelu_lut())
+    cases.check_against(golden, "gelu_edges", y, exact=True)
+
+
+def test_tables_regenerate(oracle):
+    """the table builders reproduce the tables dumped from the reference host classes"""
+    assert np.array_equal(oracle.silu_lut(), cases.silu_lut())
+    assert np.array_equal(oracle.gelu_lut(), cases.gelu_lut())
+    assert cases.silu_lut()[4608] == np.float32(0.731058598) and cases.gelu_lut()[4608] == np.float32(0.841347098)
