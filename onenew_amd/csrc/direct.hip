@@ -1,0 +1,222 @@
+// Bandwidth-bound kernels where MFMA does not pay: depthwise convolution (fp32 and W8A32), the
+// activation quantiser that stages NCHW fp32 as NHWC int8 for the int8 MFMA path, the int8 weight
+// re-layout, and the skinny Gemm  out = A * W^T + bias  with a wavefront-shuffle reduction.
+#include "onhip_internal.hpp"
+
+namespace onhip {
+
+// ---- depthwise convolution, fp32 -------------------------------------------------------------------
+// One thread per output element, lanes along ow (coalesced).  Taps are added in ascending (i, j)
+// order to a zero sum with separately rounded multiply and add, the bias last: the arithmetic of
+// device/x86/Conv/conv.c:597-612 and :853-894 exactly, so the result is bit-identical to it.
+__global__ __launch_bounds__(256) void depthwise_f32_kernel(onhip_conv_desc_t d, int OH, int OW, const float *x,
+                                                            const float *w, const float *bias, Epilogue ep, float *y,
+                                                            long long total) {
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int ow = (int) (idx % OW);
+    long long t = idx / OW;
+    const int oh = (int) (t % OH);
+    t /= OH;
+    const int c = (int) (t % d.cout);
+    const float *xc = x + t * (long long) d.h * d.w;  // t = img * C + c
+    const float *wc = w + (long long) c * d.kh * d.kw;
+    const int ih0 = oh * d.stride_h - d.pad_t, iw0 = ow * d.stride_w - d.pad_l;
+    float acc = 0.0f;
+    for (int i = 0; i < d.kh; ++i) {
+        const int ih = ih0 + i;
+        if ((unsigned) ih >= (unsigned) d.h) continue;
+        for (int j = 0; j < d.kw; ++j) {
+            const int iw = iw0 + j;
+            if ((unsigned) iw >= (unsigned) d.w) continue;
+            acc = __fadd_rn(acc, __fmul_rn(wc[i * d.kw + j], xc[(long long) ih * d.w + iw]));
+        }
+    }
+    acc = __fadd_rn(acc, bias[c]);
+    y[idx] = apply_act(acc, ep);
+}
+
+int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,
+                         const float *bias, const Epilogue &ep, float *y, hipStream_t stream) {
+    const long long total = (long long) d.n * d.cout * OH * OW;
+    const long long blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise: output too large");
+    hipLaunchKernelGGL(depthwise_f32_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, d, OH, OW, x, w, bias, ep,
+                       y, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+// activation quantiser of conv.c:961-973: t = x * (1/scale), clamp, roundf (ties away from zero)
+__device__ __forceinline__ int quant_s8(float x, float inv_scale) {
+    float t = __fmul_rn(x, inv_scale);
+    t = (t < -128.0f) ? -128.0f : (t > 127.0f) ? 127.0f : t;
+    return (int) roundf(t);
+}
+
+// ---- depthwise convolution, W8A32 (conv.c:617-755) -----------------------------------------------------
+__global__ __launch_bounds__(256) void depthwise_w8a32_kernel(onhip_conv_desc_t d, int OH, int OW, const float *x,
+                                                              const int8_t *w8, const int32_t *bias32,
+                                                              const float *weight_aux, Epilogue ep, void *y,
+                                                              int32_t *acc32, float inv_scale, float out_inv_scale,
+                                                              long long total) {
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int ow = (int) (idx % OW);
+    long long t = idx / OW;
+    const int oh = (int) (t % OH);
+    t /= OH;
+    const int c = (int) (t % d.cout);
+    const float *xc = x + t * (long long) d.h * d.w;
+    const int8_t *wc = w8 + (long long) c * d.kh * d.kw;
+    const int ih0 = oh * d.stride_h - d.pad_t, iw0 = ow * d.stride_w - d.pad_l;
+    int acc = 0;
+    for (int i = 0; i < d.kh; ++i) {
+        const int ih = ih0 + i;
+        if ((unsigned) ih >= (unsigned) d.h) continue;
+        for (int j = 0; j < d.kw; ++j) {
+            const int iw = iw0 + j;
+            if ((unsigned) iw >= (unsigned) d.w) continue;
+            acc += (int) wc[i * d.kw + j] * quant_s8(xc[(long long) ih * d.w + iw], inv_scale);
+        }
+    }
+    if (acc32) acc32[idx] = acc;
+    float f = __fadd_rn(__fmul_rn((float) acc, d.input_scale), (float) bias32[c]);
+    float v = apply_act(__fmul_rn(f, __fdiv_rn(weight_aux[c], 127.0f)), ep);
+    if (d.out_s8) {
+        float q = __fmul_rn(v, out_inv_scale);
+        q = (q < -128.0f) ? -128.0f : (q > 127.0f) ? 127.0f : q;
+        reinterpret_cast<int8_t *>(y)[idx] = (int8_t) roundf(q);
+    } else {
+        reinterpret_cast<float *>(y)[idx] = v;
+    }
+}
+
+int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const int8_t *w8,
+                           const int32_t *bias32, const float *weight_aux, const Epilogue &ep, void *y,
+                           int32_t *acc32, hipStream_t stream) {
+    const long long total = (long long) d.n * d.cout * OH * OW;
+    const long long blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise: output too large");
+    const float inv_scale = 1.0f / d.input_scale;
+    const float out_inv = d.out_s8 ? 1.0f / d.output_scale : 0.0f;
+    hipLaunchKernelGGL(depthwise_w8a32_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, d, OH, OW, x, w8, bias32,
+                       weight_aux, ep, y, acc32, inv_scale, out_inv, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+// ---- NCHW fp32 -> NHWC int8, channels zero-padded to cp (a multiple of 16) -----------------------------
+// One thread quantises 16 channels of one pixel: 16 loads that are each coalesced along the pixel
+// index, one 16-byte store.
+__global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float *x, int c, int hw, int cp, float inv_scale,
+                                                            int8_t *q, long long total) {
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;  // (img, cblock, pix), pix fastest
+    if (idx >= total) return;
+    const int cblocks = cp / 16;
+    const int pix = (int) (idx % hw);
+    const long long t = idx / hw;
+    const int cb = (int) (t % cblocks);
+    const long long img = t / cblocks;
+    const float *src = x + (img * c + (long long) cb * 16) * hw + pix;
+    unsigned out[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        unsigned word = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ch = cb * 16 + g * 4 + e;
+            const int v = ch < c ? quant_s8(src[(long long) (g * 4 + e) * hw], inv_scale) : 0;
+            word |= ((unsigned) v & 0xffu) << (8 * e);
+        }
+        out[g] = word;
+    }
+    *reinterpret_cast<uint4 *>(q + (img * hw + pix) * (long long) cp + cb * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
+                         hipStream_t stream) {
+    const long long total = (long long) n * (cp / 16) * h * w;
+    const long long blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "quantize: tensor too large");
+    hipLaunchKernelGGL(quantize_nhwc_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, x, c, h * w, cp, inv_scale,
+                       q, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+// ---- int8 weights [cout][cin][kh][kw] -> [cout][k_units * 16], k = (tap * cp + channel), zero padded ---
+__global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t *w8, int cin, int khkw, int cp, int row_bytes,
+                                                      int8_t *packed, long long total) {
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int kq = (int) (idx % row_bytes);
+    const long long oc = idx / row_bytes;
+    const int tap = kq / cp, ch = kq % cp;
+    int8_t v = 0;
+    if (tap < khkw && ch < cin) v = w8[(oc * cin + ch) * khkw + tap];
+    packed[idx] = v;
+}
+
+int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, int k_units, int8_t *packed,
+                   hipStream_t stream) {
+    const long long total = (long long) cout * k_units * 16;
+    const long long blocks = (total + 255) / 256;
+    hipLaunchKernelGGL(pack_w8_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, w8, cin, kh * kw, cp,
+                       k_units * 16, packed, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+// ---- skinny Gemm: out[m][n] = sum_k a[m][k] * w[n][k] + bias[n]  (device/x86/Gemm/gemm.c:9-79) ---------
+// One wavefront per output column n; lanes stride over k, eight rows of A at a time share each
+// weight load; butterfly reduction over the 64 lanes; the bias is added last.
+constexpr int GEMM_ROWS = 8;
+__global__ __launch_bounds__(256) void gemm_nt_kernel(int M, int K, int N, const float *a, const float *w,
+                                                      const float *bias, float *out, int vec) {
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const float *wr = w + (long long) n * K;
+    for (int m0 = 0; m0 < M; m0 += GEMM_ROWS) {
+        float acc[GEMM_ROWS];
+#pragma unroll
+        for (int r = 0; r < GEMM_ROWS; ++r) acc[r] = 0.0f;
+        if (vec) {
+            for (int k = lane * 4; k < K; k += 256) {
+                const float4 wv = *reinterpret_cast<const float4 *>(wr + k);
+#pragma unroll
+                for (int r = 0; r < GEMM_ROWS; ++r) {
+                    if (m0 + r < M) {
+                        const float4 av = *reinterpret_cast<const float4 *>(a + (long long) (m0 + r) * K + k);
+                        acc[r] = fmaf(av.x, wv.x, fmaf(av.y, wv.y, fmaf(av.z, wv.z, fmaf(av.w, wv.w, acc[r]))));
+                    }
+                }
+            }
+        } else {
+            for (int k = lane; k < K; k += 64) {
+                const float wv = wr[k];
+#pragma unroll
+                for (int r = 0; r < GEMM_ROWS; ++r)
+                    if (m0 + r < M) acc[r] = fmaf(a[(long long) (m0 + r) * K + k], wv, acc[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < GEMM_ROWS; ++r) {
+            float v = acc[r];
+#pragma unroll
+            for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s, 64);
+            if (lane == 0 && m0 + r < M) out[(long long) (m0 + r) * N + n] = __fadd_rn(v, bias[n]);
+        }
+    }
+}
+
+int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,
+                   hipStream_t stream) {
+    const int vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) % 16 == 0);
+    hipLaunchKernelGGL(gemm_nt_kernel, dim3((n + 3) / 4), dim3(256), 0, stream, m, k, n, a, w, bias, out, vec);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+}  // namespace onhip

@@ -1,0 +1,143 @@
+// Internal declarations shared by the gfx950 kernels and the C ABI layer.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/onenew_hip.h"
+
+namespace onhip {
+
+// ---- error plumbing ---------------------------------------------------------------------------
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+#define ONHIP_CHECK_HIP(expr)                                                                     \
+    do {                                                                                          \
+        hipError_t e_ = (expr);                                                                   \
+        if (e_ != hipSuccess)                                                                     \
+            return ::onhip::set_error(ONHIP_ERR_RUNTIME, "%s failed: %s (%s:%d)", #expr,          \
+                                      hipGetErrorString(e_), __FILE__, __LINE__);                 \
+    } while (0)
+
+// ---- epilogue description, common to every kernel ---------------------------------------------------
+struct Epilogue {
+    int act;                 // ACT_TYPE_E
+    float clip_min, clip_max;
+    float leaky_alpha;
+    float hs_alpha, hs_beta;
+    const float *lut;        // 8192-entry table for SILU (conv) / GELU (matmul), or nullptr
+};
+
+#define ONHIP_ACT_GELU_LUT 100  // internal: table GELU of device/x86/Gelu/gelu.c, matmul epilogue only
+
+// Activation with the rounding points of device/x86/Conv/conv.c:1216-1304 (no contraction).
+__device__ __forceinline__ float apply_act(float v, const Epilogue &e) {
+    switch (e.act) {
+        case RELU:
+            return v > 0.0f ? v : 0.0f;
+        case SILU:
+        case ONHIP_ACT_GELU_LUT: {
+            if (v < -8.0f) return 0.0f;
+            if (v >= 8.0f) return v;
+            int idx = (int) __fmul_rn(__fadd_rn(v, 8.0f), 512.0f);
+            // v just below 8 rounds v + 8 up to 16: the reference reads one past the table there
+            idx = idx > 8191 ? 8191 : idx;
+            return e.lut[idx];
+        }
+        case CLIP: {
+            float t = v > e.clip_min ? v : e.clip_min;
+            return t < e.clip_max ? t : e.clip_max;
+        }
+        case LEAKYRELU:
+            return v > 0.0f ? v : __fmul_rn(e.leaky_alpha, v);
+        case HARDSILU: {
+            float t = __fadd_rn(__fmul_rn(e.hs_alpha, v), e.hs_beta);
+            t = t > 0.0f ? t : 0.0f;
+            t = t < 1.0f ? t : 1.0f;
+            return __fmul_rn(v, t);
+        }
+        default:
+            return v;  // NOT_ACT and RELU6 (no branch in the reference)
+    }
+}
+
+// ---- implicit-GEMM kernel family (igemm.hip) ---------------------------------------------------------
+//
+// C[M, N] = A[M, K] * B[K, N] on MFMA 32x32 tiles.  A rows are K-contiguous (weights, or the left
+// MatMul operand).  B is produced on the fly by one of two loaders.
+
+enum { BL_GATHER = 0,  // element gather: NCHW activations (implicit im2col) or a row-major [K, N] matrix
+       BL_KVEC = 1 };  // 16-byte vectors along K: NHWC int8 activations, or an [N, K] matrix
+
+enum { OUT_CONV = 0,   // n = img * OHW + pix  ->  img * c_img_stride + m * c_stride_m + pix
+       OUT_PLAIN = 1 };// m * c_stride_m + n * c_stride_n
+
+enum { BIAS_NONE = 0, BIAS_M = 1, BIAS_N = 2 };
+
+struct IgemmParams {
+    int M, N, K;               // K counts real reduction elements (gather) or padded units*kpu (kvec)
+    int k_units;               // 16-byte units along K (multiple of 2 per MFMA step is NOT required)
+    int k_split_units;         // units handled by one blockIdx.y slice (split-K); == k_units if unsplit
+    // A
+    const void *A;
+    long long a_batch_stride;  // elements; 0 = shared
+    int lda;                   // elements between rows
+    int a_vec;                 // rows are 16-byte aligned and lda * elem is a multiple of 16
+    // B
+    const void *B;
+    long long b_batch_stride;  // elements
+    // gather geometry (BL_GATHER)
+    int H, W, OW, OHW, HW;
+    int kh, kw, khkw, sh, sw, pt, pl;
+    unsigned magic_khkw, magic_kw;
+    long long b_img_stride;    // Cin * H * W
+    // vector geometry (BL_KVEC)
+    int units_per_tap;         // units per filter tap (Cp / 16 for NHWC int8); k_units for a plain matrix
+    unsigned magic_upt;
+    int pix_stride;            // bytes between consecutive n ("pixels"): Cp, or ldb * elem
+    // C
+    void *C;
+    long long c_batch_stride, c_img_stride, c_stride_m, c_stride_n;
+    int out_mode;
+    // epilogue
+    const float *bias;
+    int bias_mode;
+    Epilogue ep;
+    // W8A32
+    float in_scale;            // activation scale s
+    const float *weight_aux;   // per output channel max|w|
+    const int32_t *bias32;
+    int32_t *acc_out;          // optional raw accumulators, same addressing as C
+    int out_s8;
+    float out_inv_scale;       // 1.0f / output_scale
+    // split-K workspace: partial sums [split][M][N] fp32 (nullptr when unsplit)
+    float *partial;
+};
+
+enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2, DT_I8 = 3 };
+
+struct IgemmLaunch {
+    int dtype;      // DT_*
+    int bl;         // BL_*
+    int bm, bn;     // tile
+    int batch;      // grid.z
+    int split;      // grid.y
+};
+
+int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
+// chooses a tile for the problem; fills cfg.bm / cfg.bn / cfg.split
+void igemm_pick_tile(IgemmLaunch &cfg, const IgemmParams &p);
+
+// ---- other kernels -------------------------------------------------------------------------------------
+int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,
+                         const float *bias, const Epilogue &ep, float *y, hipStream_t stream);
+int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const int8_t *w8,
+                           const int32_t *bias32, const float *weight_aux, const Epilogue &ep, void *y,
+                           int32_t *acc32, hipStream_t stream);
+int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
+                         hipStream_t stream);
+int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, int k_units, int8_t *packed,
+                   hipStream_t stream);
+int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,
+                   hipStream_t stream);
+
+}  // namespace onhip

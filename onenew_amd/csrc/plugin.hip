@@ -1,0 +1,341 @@
+// Plugin level of the C ABI: the three `eval` bodies the oneNew host binds.  They read the slot
+// arrays exactly like the reference kernels do (device/x86/Conv/conv.c:13-104, MatMul/mat_mul.c:10-33,
+// Gemm/gemm.c:9-33) and run the kernel-level entry points of api.hip.
+//
+// Residency.  The oneNew host hands out host pointers (weights in std::vector, activations from
+// aligned_alloc).  A slot whose address is device memory (hipMalloc / managed) is used in place;
+// a host address is staged: weights, bias and tables are uploaded once and cached by host address
+// and size (they live as long as the net, host/ops/conv.h:148-154), activations are copied in and
+// the result copied back on every call.  eval is synchronous: the output is complete on return,
+// like the reference's CUDA operators (device/cuda/MaxPool/maxpool.cu:76).
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <utility>
+
+#include "onhip_internal.hpp"
+
+namespace onhip {
+
+static std::mutex g_mu;
+static bool g_ready = false;
+
+struct DevBuf {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+// persistent staging buffers: [0] input, [1] second input, [2] output, [3] workspace
+static DevBuf g_stage[4];
+// uploaded constants keyed by (host address, bytes); the fingerprint of sampled content detects a
+// host buffer that was freed and reused for other data at the same address
+struct ConstEntry {
+    void *dev;
+    uint64_t fingerprint;
+};
+static std::map<std::pair<const void *, size_t>, ConstEntry> g_const;
+
+static uint64_t fingerprint(const void *host, size_t bytes) {
+    const unsigned char *b = static_cast<const unsigned char *>(host);
+    uint64_t h = 1469598103934665603ULL ^ bytes;
+    const size_t words = bytes / 8;
+    const size_t step = words > 4096 ? words / 4096 : 1;
+    for (size_t i = 0; i < words; i += step) {
+        uint64_t v;
+        memcpy(&v, b + i * 8, 8);
+        h = (h ^ v) * 1099511628211ULL;
+    }
+    for (size_t i = words * 8; i < bytes; ++i) h = (h ^ b[i]) * 1099511628211ULL;
+    if (words) {
+        uint64_t v;
+        memcpy(&v, b + (words - 1) * 8, 8);
+        h = (h ^ v) * 1099511628211ULL;
+    }
+    return h;
+}
+
+static int ensure_ready() {
+    if (g_ready) return ONHIP_OK;
+    int dev = 0;
+    ONHIP_CHECK_HIP(hipGetDevice(&dev));
+    int rc = onhip_init(dev);
+    if (rc) return rc;
+    g_ready = true;
+    return ONHIP_OK;
+}
+
+static bool is_device_ptr(const void *p) {
+    hipPointerAttribute_t attr;
+    hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void) hipGetLastError();  // plain host memory: clear the sticky error
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+static int stage_buf(int slot, size_t bytes, void **out) {
+    DevBuf &b = g_stage[slot];
+    if (bytes > b.bytes) {
+        if (b.ptr) ONHIP_CHECK_HIP(hipFree(b.ptr));
+        b.ptr = nullptr;
+        b.bytes = 0;
+        const size_t want = (bytes + (1u << 20) - 1) & ~((size_t) (1u << 20) - 1);
+        ONHIP_CHECK_HIP(hipMalloc(&b.ptr, want));
+        b.bytes = want;
+    }
+    *out = b.ptr;
+    return ONHIP_OK;
+}
+
+// device address of an input tensor: in place if already on the device, else staged copy
+static int input_on_device(int slot, const void *host, size_t bytes, const void **dev) {
+    if (is_device_ptr(host)) { *dev = host; return ONHIP_OK; }
+    void *d;
+    int rc = stage_buf(slot, bytes, &d);
+    if (rc) return rc;
+    ONHIP_CHECK_HIP(hipMemcpy(d, host, bytes, hipMemcpyHostToDevice));
+    *dev = d;
+    return ONHIP_OK;
+}
+
+// device address of a constant (weight, bias, table): uploaded once
+static int const_on_device(const void *host, size_t bytes, const void **dev) {
+    if (!host) { *dev = nullptr; return ONHIP_OK; }
+    if (is_device_ptr(host)) { *dev = host; return ONHIP_OK; }
+    auto key = std::make_pair(host, bytes);
+    const uint64_t fp = fingerprint(host, bytes);
+    auto it = g_const.find(key);
+    if (it != g_const.end()) {
+        if (it->second.fingerprint != fp) {
+            ONHIP_CHECK_HIP(hipMemcpy(it->second.dev, host, bytes, hipMemcpyHostToDevice));
+            it->second.fingerprint = fp;
+        }
+        *dev = it->second.dev;
+        return ONHIP_OK;
+    }
+    void *d = nullptr;
+    ONHIP_CHECK_HIP(hipMalloc(&d, bytes < 16 ? 16 : bytes));
+    ONHIP_CHECK_HIP(hipMemcpy(d, host, bytes, hipMemcpyHostToDevice));
+    g_const[key] = ConstEntry{d, fp};
+    *dev = d;
+    return ONHIP_OK;
+}
+
+static long long numel(const OPERAND_S *o) {
+    long long n = 1;
+    for (int i = 0; i < SHAPE_LEN; ++i) n *= o->shapes[i];  // unused dims hold 1 (common/utils_c.h:9-16)
+    return n;
+}
+
+static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const CONV_CONFIG_S *cfg = reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr);
+    const OPERAND_S *in_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *w_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
+    // params[3] is the bias descriptor, or the output when there is no bias (conv.c:434-436)
+    const OPERAND_S *out_t = reinterpret_cast<const OPERAND_S *>(params[cfg->has_bias ? 4 : 3].addr);
+    if (!cfg || !in_t || !w_t || !out_t) return set_error(ONHIP_ERR_ARG, "Conv eval: empty params slot");
+
+    onhip_conv_desc_t d;
+    memset(&d, 0, sizeof(d));
+    // the reference evaluates image 0 only (host/ops/conv.h:43); a batched output descriptor asks for more
+    d.n = out_t->shapes[0] < in_t->shapes[0] ? out_t->shapes[0] : in_t->shapes[0];
+    if (d.n < 1) d.n = 1;
+    d.cin = in_t->shapes[1]; d.h = in_t->shapes[2]; d.w = in_t->shapes[3];
+    d.cout = w_t->shapes[0]; d.kh = w_t->shapes[2]; d.kw = w_t->shapes[3];
+    d.stride_h = (int32_t) cfg->strides[0]; d.stride_w = (int32_t) cfg->strides[1];
+    d.pad_t = (int32_t) cfg->pads[0]; d.pad_l = (int32_t) cfg->pads[1];
+    d.pad_b = (int32_t) cfg->pads[2]; d.pad_r = (int32_t) cfg->pads[3];
+    // conv.c:18-29: without bias the dense path runs whatever the group says; with bias any group != 1
+    // (including a missing attribute, 0) is depthwise
+    d.group = !cfg->has_bias ? 1 : (cfg->group == 1 ? 1 : d.cin);
+    d.has_bias = cfg->has_bias ? 1 : 0;
+    d.act_type = cfg->act_type;
+    d.clip_min = cfg->clip_min; d.clip_max = cfg->clip_max;
+    d.leaky_relu_alpha = cfg->leaky_relu_alpha;
+    d.hard_sigmoid_alpha = cfg->hard_sigmoid_alpha; d.hard_sigmoid_beta = cfg->hard_sigmoid_beta;
+    d.input_scale = cfg->input_scale;
+    const bool int8 = cfg->ifmap_quant2 == TYPE_INT8;
+    if (d.group != 1 && d.cout != d.cin)
+        return set_error(ONHIP_ERR_ARG, "Conv eval: depthwise with cout %d != cin %d", d.cout, d.cin);
+
+    int32_t OH, OW;
+    int rc = onhip_conv_out_shape(&d, &OH, &OW);
+    if (rc) return rc;
+    if (out_t->shapes[1] != d.cout || out_t->shapes[2] != OH || out_t->shapes[3] != OW)
+        return set_error(ONHIP_ERR_ARG, "Conv eval: output descriptor %dx%dx%d does not match computed %dx%dx%d",
+                         out_t->shapes[1], out_t->shapes[2], out_t->shapes[3], d.cout, OH, OW);
+    const int kc = d.group == 1 ? d.cin : 1;
+    if (w_t->shapes[1] != kc)
+        return set_error(ONHIP_ERR_ARG, "Conv eval: weight has %d input channels, expected %d", w_t->shapes[1], kc);
+
+    const size_t in_bytes = (size_t) d.n * d.cin * d.h * d.w * 4;
+    const size_t out_bytes = (size_t) d.n * d.cout * OH * OW * 4;
+    const size_t w_elems = (size_t) d.cout * kc * d.kh * d.kw;
+    const void *x, *w, *b = nullptr, *lut = nullptr, *aux = nullptr;
+    rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
+    if (rc) return rc;
+    // int8 weights sit at the front of the fp32-sized buffer, the int32 bias in the fp32 bias buffer
+    rc = const_on_device(reinterpret_cast<const void *>(inputs[1].addr), int8 ? w_elems : w_elems * 4, &w);
+    if (rc) return rc;
+    if (d.has_bias) {
+        rc = const_on_device(reinterpret_cast<const void *>(inputs[2].addr), (size_t) d.cout * 4, &b);
+        if (rc) return rc;
+    }
+    if (d.has_bias && d.act_type == SILU) {
+        rc = const_on_device(reinterpret_cast<const void *>(inputs[BUF_MAXNUM - 1].addr), 8192 * 4, &lut);
+        if (rc) return rc;
+        if (!lut) return set_error(ONHIP_ERR_ARG, "Conv eval: SILU without a table in inputs[%d]", BUF_MAXNUM - 1);
+    }
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, out_bytes, &y);
+        if (rc) return rc;
+    }
+    if (int8) {
+        if (d.cout > 4096) return set_error(ONHIP_ERR_ARG, "Conv eval: weight_aux holds 4096 channels, cout is %d", d.cout);
+        rc = const_on_device(cfg->weight_aux, (size_t) d.cout * 4, &aux);
+        if (rc) return rc;
+        void *ws = nullptr;
+        const size_t ws_bytes = onhip_conv2d_w8a32_workspace(&d);
+        if (ws_bytes) {
+            rc = stage_buf(3, ws_bytes, &ws);
+            if (rc) return rc;
+        }
+        rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
+                                (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
+    } else {
+        rc = onhip_conv2d_f32(&d, (const float *) x, (const float *) w, (const float *) b, (const float *) lut,
+                              (float *) y, nullptr);
+    }
+    if (rc) return rc;
+    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, out_bytes, hipMemcpyDeviceToHost));
+    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    return ONHIP_OK;
+}
+
+static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *a_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *b_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
+    const OPERAND_S *o_t = reinterpret_cast<const OPERAND_S *>(params[3].addr);
+    if (!a_t || !b_t || !o_t) return set_error(ONHIP_ERR_ARG, "MatMul eval: empty params slot");
+    const int nd = a_t->dim_num_of_shapes;
+    if (nd < 2 || nd > SHAPE_LEN || o_t->dim_num_of_shapes < 1 || o_t->dim_num_of_shapes > SHAPE_LEN)
+        return set_error(ONHIP_ERR_ARG, "MatMul eval: rank %d", nd);
+    onhip_matmul_desc_t d;
+    memset(&d, 0, sizeof(d));
+    d.batch = 1;
+    for (int i = 0; i < nd - 2; ++i) d.batch *= a_t->shapes[i];  // mat_mul.c:24-27
+    d.m = a_t->shapes[nd - 2];
+    d.k = a_t->shapes[nd - 1];
+    d.n = o_t->shapes[o_t->dim_num_of_shapes - 1];
+    const long long b_elems = numel(b_t);
+    d.b_shared = b_elems == (long long) d.k * d.n;  // mat_mul.c:42-46
+    if (!d.b_shared && b_elems != (long long) d.batch * d.k * d.n)
+        return set_error(ONHIP_ERR_ARG, "MatMul eval: second operand has %lld elements, expected %lld or %lld", b_elems,
+                         (long long) d.k * d.n, (long long) d.batch * d.k * d.n);
+    const size_t a_bytes = (size_t) d.batch * d.m * d.k * 4, b_bytes = (size_t) b_elems * 4;
+    const size_t o_bytes = (size_t) d.batch * d.m * d.n * 4;
+    const void *a, *b;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), a_bytes, &a);
+    if (rc) return rc;
+    const void *b_host = reinterpret_cast<const void *>(inputs[1].addr);
+    // the second operand is a weight (fixed) or another activation
+    if (b_t->is_fixed_val) rc = const_on_device(b_host, b_bytes, &b);
+    else rc = input_on_device(1, b_host, b_bytes, &b);
+    if (rc) return rc;
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, o_bytes, &y);
+        if (rc) return rc;
+    }
+    rc = onhip_matmul(&d, (const float *) a, (const float *) b, nullptr, nullptr, (float *) y, nullptr);
+    if (rc) return rc;
+    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, o_bytes, hipMemcpyDeviceToHost));
+    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    return ONHIP_OK;
+}
+
+static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *a_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *o_t = reinterpret_cast<const OPERAND_S *>(params[4].addr);
+    if (!a_t || !o_t) return set_error(ONHIP_ERR_ARG, "Gemm eval: empty params slot");
+    const int nd = a_t->dim_num_of_shapes;
+    if (nd < 2 || nd > SHAPE_LEN || o_t->dim_num_of_shapes < 1 || o_t->dim_num_of_shapes > SHAPE_LEN)
+        return set_error(ONHIP_ERR_ARG, "Gemm eval: rank %d", nd);
+    // gemm.c:25-33: M and K from the last two dims of the input, N from the output; leading dims ignored
+    const int M = a_t->shapes[nd - 2], K = a_t->shapes[nd - 1], N = o_t->shapes[o_t->dim_num_of_shapes - 1];
+    if (M < 1 || K < 1 || N < 1) return set_error(ONHIP_ERR_ARG, "Gemm eval: bad shape %dx%dx%d", M, K, N);
+    const void *a, *w, *b;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), (size_t) M * K * 4, &a);
+    if (rc) return rc;
+    rc = const_on_device(reinterpret_cast<const void *>(inputs[1].addr), (size_t) N * K * 4, &w);
+    if (rc) return rc;
+    rc = const_on_device(reinterpret_cast<const void *>(inputs[2].addr), (size_t) N * 4, &b);
+    if (rc) return rc;
+    if (!b) return set_error(ONHIP_ERR_ARG, "Gemm eval: the reference Gemm always adds a bias; inputs[2] is empty");
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const size_t o_bytes = (size_t) M * N * 4;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, o_bytes, &y);
+        if (rc) return rc;
+    }
+    rc = onhip_gemm_f32(M, K, N, (const float *) a, (const float *) w, (const float *) b, (float *) y, nullptr);
+    if (rc) return rc;
+    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, o_bytes, hipMemcpyDeviceToHost));
+    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    return ONHIP_OK;
+}
+
+template <class F>
+static int guarded(const char *what, F f, BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    if (!params || !inputs || !outputs || !params[0].addr || !inputs[0].addr || !outputs[0].addr) {
+        int rc = set_error(ONHIP_ERR_ARG, "%s eval: null slot array or empty slot 0", what);
+        fprintf(stderr, "[onenew_hip] %s\n", onhip_last_error());
+        return rc;
+    }
+    std::lock_guard<std::mutex> lock(g_mu);
+    int rc = ensure_ready();
+    if (!rc) rc = f(params, inputs, outputs);
+    // the host ignores the return value (host/op.h:183): make failures visible
+    if (rc) fprintf(stderr, "[onenew_hip] %s eval failed (%d): %s\n", what, rc, onhip_last_error());
+    return rc;
+}
+
+}  // namespace onhip
+
+using namespace onhip;
+
+extern "C" {
+
+int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv", conv_eval_locked, params, inputs, outputs);
+}
+int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MatMul", matmul_eval_locked, params, inputs, outputs);
+}
+int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Gemm", gemm_eval_locked, params, inputs, outputs);
+}
+
+int onhip_plugin_release(void) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    ONHIP_CHECK_HIP(hipDeviceSynchronize());
+    for (auto &kv : g_const) (void) hipFree(kv.second.dev);
+    g_const.clear();
+    for (auto &b : g_stage) {
+        if (b.ptr) (void) hipFree(b.ptr);
+        b.ptr = nullptr;
+        b.bytes = 0;
+    }
+    return ONHIP_OK;
+}
+
+}  // extern "C"

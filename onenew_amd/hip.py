@@ -1,0 +1,136 @@
+"""Loader and thin Python front end of the gfx950 kernel library (include/onenew_hip.h).
+
+The shared objects are built in place by ``python -m onenew_amd.build``.  Nothing here falls back to
+another implementation: a missing library or a failing call raises.
+
+Tensor arguments are torch CUDA tensors (PyTorch is used for device memory and streams only) or
+raw integer device addresses; launches go to torch's current stream.
+"""
+import ctypes as C
+import os
+
+from . import abi
+from .abi import ConvDesc, MatmulDesc, BUFFER_INFO_S
+
+LIBDIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+_lib = None
+
+
+class OnhipError(RuntimeError):
+    pass
+
+
+def lib_path(name="libonenew_hip.so"):
+    return os.path.join(LIBDIR, name)
+
+
+def plugin_path(op):
+    """libConv_hip.so / libMatMul_hip.so / libGemm_hip.so"""
+    return os.path.join(LIBDIR, f"lib{op}_hip.so")
+
+
+EXPORTS = ["onhip_init", "onhip_last_error", "onhip_conv_out_shape", "onhip_conv2d_f32",
+           "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_matmul", "onhip_gemm_f32",
+           "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise OnhipError(f"{path} is missing: build it with `python -m onenew_amd.build`")
+    L = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    vp = C.c_void_p
+    L.onhip_init.argtypes = [C.c_int]
+    L.onhip_last_error.restype = C.c_char_p
+    L.onhip_conv_out_shape.argtypes = [C.POINTER(ConvDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    L.onhip_conv2d_f32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp]
+    L.onhip_conv2d_w8a32_workspace.argtypes = [C.POINTER(ConvDesc)]
+    L.onhip_conv2d_w8a32_workspace.restype = C.c_size_t
+    L.onhip_conv2d_w8a32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
+    L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
+    L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
+    for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval"):
+        getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
+    _lib = L
+    return L
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise OnhipError(f"{what} failed ({rc}): {load().onhip_last_error().decode()}")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    return t.data_ptr()
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def init(device=0):
+    _check(load().onhip_init(device), "onhip_init")
+
+
+def conv2d_f32(d, x, w, bias=None, silu_lut=None, out=None):
+    """fused Conv2d (+bias, +activation); returns the fp32 NCHW output tensor"""
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device=x.device)
+    _check(load().onhip_conv2d_f32(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(silu_lut), _ptr(out), _stream()),
+           "onhip_conv2d_f32")
+    return out
+
+
+def conv2d_w8a32_workspace(d):
+    return int(load().onhip_conv2d_w8a32_workspace(C.byref(d)))
+
+
+def conv2d_w8a32(d, x, w8, bias32, weight_aux, silu_lut=None, out=None, acc32=None, workspace=None):
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.int8 if d.out_s8 else torch.float32, device=x.device)
+    need = conv2d_w8a32_workspace(d)
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(load().onhip_conv2d_w8a32(C.byref(d), _ptr(x), _ptr(w8), _ptr(bias32), _ptr(weight_aux), _ptr(silu_lut),
+                                     _ptr(out), _ptr(acc32), _ptr(workspace), nbytes, _stream()),
+           "onhip_conv2d_w8a32")
+    return out
+
+
+def matmul(a, b, bias=None, gelu_lut=None, compute=abi.COMPUTE_F32, out=None):
+    """out = a @ b (b either [K, N] or batched like a), optional fused bias over N and table GELU"""
+    import torch
+    M, K = a.shape[-2], a.shape[-1]
+    N = b.shape[-1]
+    batch = 1
+    for s in a.shape[:-2]:
+        batch *= s
+    d = MatmulDesc(batch=batch, m=M, k=K, n=N, b_shared=int(b.numel() == K * N), compute=compute)
+    if out is None:
+        out = torch.empty(tuple(a.shape[:-1]) + (N,), dtype=torch.float32, device=a.device)
+    _check(load().onhip_matmul(C.byref(d), _ptr(a), _ptr(b), _ptr(bias), _ptr(gelu_lut), _ptr(out), _stream()),
+           "onhip_matmul")
+    return out
+
+
+def gemm_f32(a, w, bias, out=None):
+    import torch
+    M, K = a.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    _check(load().onhip_gemm_f32(M, K, N, _ptr(a), _ptr(w), _ptr(bias), _ptr(out), _stream()), "onhip_gemm_f32")
+    return out

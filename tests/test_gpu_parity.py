@@ -1,0 +1,315 @@
+"""GPU parity: the HIP kernels against the CPU oracle on the same seeded inputs and against the
+fixtures made from the reference's own compiled kernels.  Everything goes through the C ABI
+(kernel level via onenew_amd.hip, plugin level via `eval`).
+
+Bars: depthwise and W8A32 bit-exact (int32 accumulators included); fp32 MFMA paths
+max|a-b| / max|b| <= 1e-4 and |a-b| <= 1e-4 * |b| + 1e-5 element-wise; table activations are
+checked exactly on the kernel's own pre-activation; bf16 / fp16 modes within 1e-2 of the fp32
+reference."""
+import numpy as np
+import pytest
+
+import cases
+from onenew_amd import abi, hip, ops
+from onenew_amd.abi import ConvDesc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_dev():
+    import torch
+    assert torch.cuda.is_available(), "no GPU visible"
+    hip.init(0)
+    return torch
+
+
+def dev(torch, a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close_f32(got, ref, rel=1e-4, tag="", elementwise=True):
+    """max|a-b| / max|b| <= rel, and (fp32 paths) |a-b| <= rel*|b| + rel/10 for every element.  The
+    reduced-precision modes are judged on the normalised maximum only: with 8 mantissa bits the
+    rounding noise of a K-term sum exceeds any per-element bound near zero crossings."""
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    assert got.shape == ref.shape
+    scale = np.abs(ref).max() if ref.size else 0.0
+    diff = np.abs(got - ref)
+    assert diff.max() <= rel * max(scale, 1e-30), f"{tag}: max diff {diff.max():.3e} vs max|ref| {scale:.3e}"
+    if not elementwise:
+        return
+    bad = diff > rel * np.abs(ref) + rel * 0.1
+    assert not bad.any(), f"{tag}: {bad.sum()} elements outside |a-b| <= {rel}*|b| + {rel * 0.1}"
+
+
+def run_conv_f32(torch, name, d, compute=abi.COMPUTE_F32):
+    x, w, b = cases.conv_inputs(name, d)
+    dd = ConvDesc.from_buffer_copy(d)
+    dd.compute = compute
+    lut = dev(torch, cases.silu_lut())
+    y = hip.conv2d_f32(dd, dev(torch, x), dev(torch, w), dev(torch, b), lut)
+    torch.cuda.synchronize()
+    return x, w, b, y.cpu().numpy()
+
+
+@pytest.mark.parametrize("name", list(cases.conv_f32_cases()))
+def test_conv_f32(name, torch_dev, oracle, golden):
+    torch = torch_dev
+    d = cases.conv_f32_cases()[name]
+    print(f"case {name}", flush=True)
+    x, w, b, y = run_conv_f32(torch, name, d)
+    ref = oracle.conv2d_f32(d, x, w, b, cases.silu_lut())
+    if d.group != 1:
+        # depthwise: same operation order as the reference, bit-identical
+        assert np.array_equal(y, ref), f"{name}: {(y != ref).sum()} elements differ"
+        cases.check_against(golden, name, y, exact=True)
+        return
+    if d.has_bias and d.act_type == abi.SILU:
+        # table activation: compare the pre-activation, then the table applied to the kernel's own pre-activation
+        dn = ConvDesc.from_buffer_copy(d)
+        dn.act_type = abi.NOT_ACT
+        _, _, _, pre = run_conv_f32(torch, name, dn)
+        assert_close_f32(pre, oracle.conv2d_f32(dn, x, w, b), tag=name + " pre-activation")
+        assert np.array_equal(y, oracle.lut_act(pre, cases.silu_lut())), f"{name}: table lookup differs"
+        return
+    assert_close_f32(y, ref, tag=name)
+    scale = float(np.abs(ref).max())
+    cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * scale)
+
+
+@pytest.mark.parametrize("name", list(cases.conv_w8a32_cases()))
+def test_conv_w8a32_bit_exact(name, torch_dev, oracle, golden):
+    torch = torch_dev
+    d = cases.conv_w8a32_cases()[name]
+    print(f"case {name}", flush=True)
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    oh, ow = d.out_hw()
+    acc = torch.empty((d.n, d.cout, oh, ow), dtype=torch.int32, device="cuda")
+    y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux),
+                         dev(torch, cases.silu_lut()), acc32=acc)
+    torch.cuda.synchronize()
+    ref, ref_acc = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut(), want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), ref_acc), f"{name}: int32 accumulators differ"
+    y = y.cpu().numpy()
+    assert np.array_equal(y, ref), f"{name}: {(y != ref).sum()} de-quantised outputs differ"
+    cases.check_against(golden, name, y, exact=True)
+
+
+@pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_s2", "qdw3x3", "yolo_c2f_3x3_64_80"])
+def test_conv_w8a32_requant_s8(name, torch_dev, oracle):
+    """int8 output = the consumer's input quantisation of the fp32 result: exact, so <= 1 LSB"""
+    torch = torch_dev
+    d = ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()[name])
+    d.out_s8, d.output_scale = 1, 0.037
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()))
+    torch.cuda.synchronize()
+    ref = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut())
+    assert y.dtype == torch.int8 and np.array_equal(y.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("name,batch", [("c3x3_tiny_relu", 3), ("c1x1_unaligned_clip", 5), ("c7x7_s2_p3", 2),
+                                        ("dw3x3_s2_odd", 4), ("cfg1_64x56_3x3", 2), ("rn50_l4_3x3", 33)])
+def test_conv_f32_batched(name, batch, torch_dev, oracle):
+    """a batch is that many independent batch-1 evaluations of the reference"""
+    torch = torch_dev
+    d = ConvDesc.from_buffer_copy(cases.conv_f32_cases()[name])
+    d.n = batch
+    x, w, b, y = run_conv_f32(torch, name + "_batched", d)
+    ref = oracle.conv2d_f32(d, x, w, b, cases.silu_lut())
+    if d.group != 1:
+        assert np.array_equal(y, ref)
+    else:
+        assert_close_f32(y, ref, tag=name)
+
+
+def test_conv_w8a32_batched(torch_dev, oracle):
+    torch = torch_dev
+    d = ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()["q3x3_s2_odd"])
+    d.n = 5
+    x, w8, b32, aux = cases.conv_inputs("q_batched", d, quant=True)
+    y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut()))
+
+
+@pytest.mark.parametrize("compute,name", [(abi.COMPUTE_BF16, "cfg1_64x56_3x3"), (abi.COMPUTE_F16, "cfg1_64x56_3x3"),
+                                          (abi.COMPUTE_BF16, "c7x7_s2_p3"), (abi.COMPUTE_F16, "c1x1_unaligned_clip")])
+def test_conv_reduced_precision_modes(compute, name, torch_dev, oracle):
+    """bf16 / fp16 MFMA with fp32 accumulation: equals the reference arithmetic on operands rounded
+    to that type (tight), and stays within 1e-2 of the fp32 reference"""
+    torch = torch_dev
+    d = cases.conv_f32_cases()[name]
+    x, w, b, y = run_conv_f32(torch, name, d, compute=compute)
+    rnd = oracle.round_bf16 if compute == abi.COMPUTE_BF16 else oracle.round_f16
+    assert_close_f32(y, oracle.conv2d_f32(d, rnd(x), rnd(w), b, cases.silu_lut()), rel=1e-4, tag=name + " rounded operands")
+    assert_close_f32(y, oracle.conv2d_f32(d, x, w, b, cases.silu_lut()), rel=1e-2, tag=name + " vs fp32",
+                     elementwise=False)
+
+
+@pytest.mark.parametrize("name", list(cases.matmul_cases()))
+def test_matmul_f32(name, torch_dev, oracle, golden):
+    torch = torch_dev
+    a, b = cases.matmul_inputs(name, *cases.matmul_cases()[name])
+    y = hip.matmul(dev(torch, a), dev(torch, b))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+    ref = oracle.matmul_f32(a, b)
+    assert_close_f32(y, ref, tag=name)
+    cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(ref).max()))
+
+
+@pytest.mark.parametrize("compute", [abi.COMPUTE_F32, abi.COMPUTE_BF16, abi.COMPUTE_F16])
+@pytest.mark.parametrize("batch", [1, 4])
+def test_matmul_bias_gelu_fused(compute, batch, torch_dev, oracle):
+    """fused MatMul + bias + table GELU == the reference chain MatMul -> Add -> Gelu (ViT MLP fc1)"""
+    torch = torch_dev
+    a, w = cases.matmul_inputs("vit_fc1", (batch, 197, 192), (192, 768))
+    bias = cases.datagen.normal(cases.datagen.seed_for("vit_fc1", "bias"), (768,), 0.0, 0.02)
+    lut = cases.gelu_lut()
+    pre = hip.matmul(dev(torch, a), dev(torch, w), bias=dev(torch, bias), compute=compute)
+    y = hip.matmul(dev(torch, a), dev(torch, w), bias=dev(torch, bias), gelu_lut=dev(torch, lut), compute=compute)
+    torch.cuda.synchronize()
+    pre, y = pre.cpu().numpy(), y.cpu().numpy()
+    ref_pre = oracle.matmul_f32(a, w, bias=bias)
+    assert_close_f32(pre, ref_pre, rel=1e-4 if compute == abi.COMPUTE_F32 else 1e-2, tag="fc1 pre-activation",
+                     elementwise=compute == abi.COMPUTE_F32)
+    assert np.array_equal(y, oracle.lut_act(pre, lut)), "table GELU differs from the table applied to the kernel's sum"
+    if compute == abi.COMPUTE_F32:
+        # away from bin edges the fused result equals the reference chain
+        ref = oracle.matmul_f32(a, w, bias=bias, gelu=lut)
+        assert np.mean(y == ref) > 0.98 and np.abs(y - ref).max() < 5e-3
+
+
+@pytest.mark.parametrize("name", list(cases.gemm_cases()))
+def test_gemm_f32(name, torch_dev, oracle, golden):
+    torch = torch_dev
+    a, w, b = cases.gemm_inputs(name, *cases.gemm_cases()[name])
+    y = hip.gemm_f32(dev(torch, a), dev(torch, w), dev(torch, b))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+    ref = oracle.gemm_f32(a, w, b)
+    assert_close_f32(y, ref, tag=name)
+    cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(ref).max()))
+
+
+# ---- plugin level: host pointers through `eval`, as the oneNew runtime calls it -------------------------
+
+@pytest.mark.parametrize("name", ["c3x3_tiny_relu", "c1x1_unaligned_clip", "c3x3_silu", "c3x3_nobias", "dw3x3_s2_even",
+                                  "dw3x3_group0", "cfg1_64x56_3x3", "rn50_l4_1x1_2048_512"])
+def test_plugin_conv_eval_host_buffers(name, torch_dev, golden):
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    plug = ops.Plugin(hip.plugin_path("Conv"))
+    op = ops.Conv(plug.eval, d, w, b, silu_lut=cases.silu_lut())
+    y = op(x)
+    y2 = op(x)  # second call: cached weights
+    assert np.array_equal(y, y2)
+    exact = d.group != 1
+    # the SiLU case can flip a table bin on a last-bit difference of the sum
+    atol = 5e-3 if d.act_type == abi.SILU and d.has_bias else 1e-4 * float(np.abs(y).max())
+    cases.check_against(golden, name, y, exact=exact, rtol=1e-4, atol=atol)
+
+
+@pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_nobias", "qdw3x3_s2", "q3x3_bigacc", "yolo_sppf_1x1_1024"])
+def test_plugin_conv_eval_w8a32(name, torch_dev, golden):
+    d = cases.conv_w8a32_cases()[name]
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    plug = ops.Plugin(hip.plugin_path("Conv"))
+    op = ops.Conv(plug.eval, d, w8, b32, weight_aux=aux, silu_lut=cases.silu_lut())
+    cases.check_against(golden, name, op(x), exact=True)
+
+
+def test_plugin_matmul_and_gemm_eval(torch_dev, golden):
+    mm = ops.MatMul(ops.Plugin(hip.plugin_path("MatMul")).eval)
+    for name in ("mm_batched_shared", "mm_batched_b", "vit_scores", "mm_many_batches"):
+        a, b = cases.matmul_inputs(name, *cases.matmul_cases()[name])
+        y = mm(a, b)
+        cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(y).max()))
+    for name in ("gemm_n_tail", "rn50_fc"):
+        a, w, b = cases.gemm_inputs(name, *cases.gemm_cases()[name])
+        y = ops.Gemm(ops.Plugin(hip.plugin_path("Gemm")).eval, w, b)(a)
+        cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(y).max()))
+
+
+def test_plugin_conv_eval_device_buffers(torch_dev, golden):
+    """activation and output already in device memory: used in place, no staging"""
+    torch = torch_dev
+    name = "c3x3_s2_p1_even"
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    oh, ow = d.out_hw()
+    xd = dev(torch, x)
+    yd = torch.zeros((1, d.cout, oh, ow), dtype=torch.float32, device="cuda")
+    op = ops.Conv(ops.Plugin(hip.plugin_path("Conv")).eval, d, w, b)
+    op(xd.data_ptr(), out=yd.data_ptr())
+    y = yd.cpu().numpy()
+    cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(y).max()))
+
+
+def test_errors_are_reported_not_thrown(torch_dev):
+    d = cases.cd(4, 4, 3, 1, 1, 8)
+    d.stride_h = 0
+    import ctypes as C
+    L = hip.load()
+    rc = L.onhip_conv2d_f32(C.byref(d), 1, 1, 1, None, 1, None)
+    assert rc == -1 and b"bad geometry" in L.onhip_last_error()
+    q = cases.cd(4, 4, 3, 1, (1, 0, 1, 0), 8, input_scale=0.1)
+    rc = L.onhip_conv2d_w8a32(C.byref(q), 1, 1, 1, 1, None, 1, None, None, 0, None)
+    assert rc == -1 and b"uniform" in L.onhip_last_error()
+
+
+# ---- full-size properties ------------------------------------------------------------------------------
+
+def _sampled_conv_f64(d, x, w, b, idx):
+    """float64 cross-correlation at the sampled flat output indices (dense convolution, ReLU)"""
+    oh, ow = d.out_hw()
+    out = np.empty(len(idx))
+    xp = np.zeros((d.n, d.cin, d.h + d.pad_t + d.pad_b, d.w + d.pad_l + d.pad_r))
+    xp[:, :, d.pad_t:d.pad_t + d.h, d.pad_l:d.pad_l + d.w] = x
+    for t, f in enumerate(idx):
+        n, r = divmod(int(f), d.cout * oh * ow)
+        m, r = divmod(r, oh * ow)
+        i, j = divmod(r, ow)
+        patch = xp[n, :, i * d.stride_h:i * d.stride_h + d.kh, j * d.stride_w:j * d.stride_w + d.kw]
+        out[t] = max((patch * w[m].astype(np.float64)).sum() + float(b[m]), 0.0)
+    return out
+
+
+@pytest.mark.parametrize("layer", [0, 2, 13, 15, 26, 44, 49, 52])
+def test_resnet50_layers_batch32_sampled_f64(layer, torch_dev):
+    """ResNet-50 layers at their real shapes, batch 32: 1500 sampled outputs against float64"""
+    torch = torch_dev
+    from onenew_amd import stacks
+    name, d = stacks.with_batch(stacks.resnet50(), 32)[layer]
+    x, w, b = cases.conv_inputs("rn50b32_" + name, d)
+    y = hip.conv2d_f32(d, dev(torch, x), dev(torch, w), dev(torch, b))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy().reshape(-1)
+    idx = cases.datagen.integers(cases.datagen.seed_for(name, "probe"), (1500,), 0, y.size - 1)
+    ref = _sampled_conv_f64(d, x, w, b, idx)
+    assert np.abs(y[idx] - ref).max() <= 1e-4 * max(np.abs(ref).max(), 1e-6), name
+    # image 7 of the batch equals the batch-1 evaluation of image 7
+    d1 = ConvDesc.from_buffer_copy(d)
+    d1.n = 1
+    y1 = hip.conv2d_f32(d1, dev(torch, x[7:8]), dev(torch, w), dev(torch, b))
+    torch.cuda.synchronize()
+    per = y.size // 32
+    assert_close_f32(y[7 * per:8 * per], y1.cpu().numpy(), tag=name + " batch slice")
+
+
+def test_linearity_and_zero_input(torch_dev):
+    """conv(a*x) - bias == a * (conv(x) - bias) up to rounding; zero input gives act(bias)"""
+    torch = torch_dev
+    d = cases.cd(64, 128, 3, 1, 1, 28, act=abi.NOT_ACT, n=4)
+    x, w, b = cases.conv_inputs("lin", d)
+    xd, wd, bd = dev(torch, x), dev(torch, w), dev(torch, b)
+    y1 = hip.conv2d_f32(d, xd, wd, bd).cpu().numpy()
+    y2 = hip.conv2d_f32(d, xd * 2.0, wd, bd).cpu().numpy()
+    bb = b.reshape(1, -1, 1, 1)
+    assert_close_f32(y2 - bb, 2.0 * (y1 - bb), rel=1e-5, tag="linearity")
+    d.act_type = abi.RELU
+    y0 = hip.conv2d_f32(d, torch.zeros_like(xd), wd, bd).cpu().numpy()
+    assert np.array_equal(y0, np.broadcast_to(np.maximum(bb, 0), y0.shape))
