@@ -22,6 +22,7 @@ int set_error(int code, const char *fmt, ...) {
 }
 
 static unsigned magic_for(unsigned d) { return d <= 1 ? 0u : (unsigned) (0x100000000ULL / d) + 1u; }
+static unsigned pass_for(unsigned d) { return d <= 1 ? 0xFFFFFFFFu : 0u; }
 
 static Epilogue make_epilogue(const onhip_conv_desc_t &d, const float *lut) {
     Epilogue e;
@@ -175,14 +176,18 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
     p.k_units = (p.K + kpu - 1) / kpu;
     p.A = w;
     p.lda = p.K;
-    p.a_vec = (p.K % 4 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0);
     p.B = x;
     p.H = d->h; p.W = d->w; p.OW = OW; p.OHW = OH * OW; p.HW = d->h * d->w;
     p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
     p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
-    p.magic_khkw = magic_for(p.khkw);
-    p.magic_kw = magic_for(p.kw);
+    p.magic_khkw = magic_for(p.khkw); p.pass_khkw = pass_for(p.khkw);
+    p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
     p.b_img_stride = (long long) d->cin * d->h * d->w;
+    if (p.khkw == 1 && !d->pad_t && !d->pad_l && !d->pad_b && !d->pad_r) cfg.bl = BL_PLAIN;
+    p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * 4;
+    p.a_slice_bytes = (long long) p.M * p.K * 4;
+    p.b_slice_bytes = (long long) d->n * p.b_img_stride * 4 + 2 * p.b_shift_bytes;
+    p.c_slice_bytes = (long long) d->n * d->cout * OH * OW * 4;
     p.C = y;
     p.out_mode = OUT_CONV;
     p.c_img_stride = (long long) d->cout * OH * OW;
@@ -260,15 +265,18 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
     p.k_units = k_units;
     p.A = packed;
     p.lda = k_units * 16;
-    p.a_vec = 1;
     p.B = q;
     p.H = d->h; p.W = d->w; p.OW = OW; p.OHW = OH * OW; p.HW = d->h * d->w;
     p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
     p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
-    p.magic_kw = magic_for(p.kw);
+    p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
     p.units_per_tap = cp / 16;
-    p.magic_upt = magic_for(p.units_per_tap);
+    p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
     p.pix_stride = cp;
+    p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * cp;
+    p.a_slice_bytes = (long long) p.M * p.lda;
+    p.b_slice_bytes = (long long) d->n * d->h * d->w * cp + 2 * p.b_shift_bytes;
+    p.c_slice_bytes = (long long) d->n * d->cout * OH * OW * 4;
     p.C = y;
     p.out_mode = OUT_CONV;
     p.c_img_stride = (long long) d->cout * OH * OW;
@@ -300,7 +308,7 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     memset(&cfg, 0, sizeof(cfg));
     int rc = dtype_of_compute(d->compute, &cfg.dtype);
     if (rc) return rc;
-    cfg.bl = BL_GATHER;
+    cfg.bl = BL_PLAIN;
     cfg.batch = batch;
     IgemmParams p;
     memset(&p, 0, sizeof(p));
@@ -310,12 +318,14 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     p.A = a;
     p.lda = d->k;
     p.a_batch_stride = (long long) M * d->k;
-    p.a_vec = (d->k % 4 == 0) && (reinterpret_cast<uintptr_t>(a) % 16 == 0);
     p.B = b;
     p.b_batch_stride = (long long) d->k * d->n;
     // a row-major [K, N] matrix is the 1x1 "image" of N pixels and K channels
     p.H = 1; p.W = d->n; p.OW = d->n; p.OHW = d->n; p.HW = d->n;
     p.kh = p.kw = p.khkw = 1; p.sh = p.sw = 1;
+    p.a_slice_bytes = (long long) M * d->k * 4;
+    p.b_slice_bytes = (long long) d->k * d->n * 4;
+    p.c_slice_bytes = (long long) M * d->n * 4;
     p.C = out;
     p.out_mode = OUT_PLAIN;
     p.c_batch_stride = (long long) M * d->n;

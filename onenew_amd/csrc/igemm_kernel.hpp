@@ -1,0 +1,578 @@
+// Implicit-GEMM kernel family for gfx950 (MI355X): C[M, N] = A[M, K] * B[K, N] on 32x32 MFMA tiles
+// with the whole epilogue (bias, activation, W8A32 de-quantisation, re-quantisation) fused in
+// registers.
+//
+// Work decomposition
+//   * one workgroup = 256 threads = 4 wavefronts (64 lanes) computes a BM x BN tile of C; each
+//     wavefront owns a (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks held in accumulators;
+//   * K is walked in tiles of 4 "units"; a unit is 16 bytes of one A row / one B column along K
+//     (4 fp32, 8 bf16/fp16 or 16 int8 values), which is exactly what one lane feeds to the MFMA
+//     instructions v_mfma_f32_32x32x2_f32 (x4), v_mfma_f32_32x32x16_{bf16,f16},
+//     v_mfma_i32_32x32x32_i8;
+//   * LDS holds, double-buffered, A as [unit][row][16 B] and B as [unit][column][16 B]: a half
+//     wavefront reads 32 consecutive 16-byte slots (conflict-free ds_read_b128), lanes 0-31 take the
+//     even unit and lanes 32-63 the odd unit of an MFMA step;
+//   * global loads for tile t+1 are issued before the MFMAs of tile t and written to the other LDS
+//     buffer afterwards: one barrier per K tile.
+//
+// B never exists in memory.  BL_GATHER builds it element by element from NCHW activations
+// (implicit im2col) or from a row-major [K, N] matrix, with lanes running along N so every load
+// instruction is a coalesced run of pixels.  BL_KVEC reads 16-byte vectors along K from NHWC int8
+// activations (K ordered tap-major, channel-minor) or from an [N, K] matrix.
+//
+// Every global access is a raw buffer instruction: the per-lane byte offset (the pixel, fixed for
+// the whole K loop) goes in the vector offset, the wavefront-uniform part (channel, filter tap,
+// K tile) in the scalar offset, so a gathered element costs a handful of scalar operations and a
+// compare/select instead of 64-bit address arithmetic.  Padding, ragged tile edges and the K tail
+// are handled by pointing the vector offset outside the buffer, which makes the hardware return
+// zero: no branches, all loads of a tile in flight together.
+//
+// Replaces, for the dense cases: device/x86/Conv/conv.c im2col (:168,:260) + opt_gemm.h SGEMM (:17)
+// + bias sweep (:405) + do_act (:1216); the int32 GEMM and de-quantisation of conv.c:1024-1056;
+// device/x86/MatMul/mat_mul.c:10.
+#pragma once
+#include "onhip_internal.hpp"
+
+namespace onhip {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int UPT = 4;        // 16-byte units per K tile
+constexpr int THREADS = 256;
+constexpr unsigned OOB = 0x80000000u;       // vector offset outside every buffer: loads give 0, stores vanish
+constexpr unsigned RSRC_RANGE = 0x80000000u; // num_records of the data buffers (all offsets stay below 2 GiB)
+constexpr unsigned RSRC_FLAGS = 0x00020000u; // 32-bit data format, raw buffer
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) bytes, (int) RSRC_FLAGS);
+}
+__device__ __forceinline__ float buf_load_f32(rsrc_t r, unsigned voff, unsigned soff) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ uint4 buf_load_b128(rsrc_t r, unsigned voff, unsigned soff) {
+    u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+    return make_uint4(q.x, q.y, q.z, q.w);
+}
+
+template <int DT> struct Traits;
+template <> struct Traits<DT_F32> {
+    static constexpr int KPU = 4;
+    static constexpr int RAW = 4;          // fp32 values fetched per unit
+    typedef f32x16 acc_t;
+    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+    }
+};
+template <> struct Traits<DT_BF16> {
+    static constexpr int KPU = 8;
+    static constexpr int RAW = 8;
+    typedef f32x16 acc_t;
+    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                    0, 0, 0);
+    }
+};
+template <> struct Traits<DT_F16> {
+    static constexpr int KPU = 8;
+    static constexpr int RAW = 8;
+    typedef f32x16 acc_t;
+    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                   0, 0);
+    }
+};
+template <> struct Traits<DT_I8> {
+    static constexpr int KPU = 16;
+    static constexpr int RAW = 4;          // 4 dwords = 16 int8
+    typedef i32x16 acc_t;
+    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), c, 0, 0,
+                                                  0);
+    }
+};
+
+// what a thread keeps in flight for one unit between the global load and the LDS store
+template <int DT> struct RawUnit { float v[Traits<DT>::RAW]; };
+template <> struct RawUnit<DT_I8> { uint4 q; };
+
+template <int DT> __device__ __forceinline__ uint4 pack_unit(const RawUnit<DT> &r);
+template <> __device__ __forceinline__ uint4 pack_unit<DT_F32>(const RawUnit<DT_F32> &r) {
+    return make_uint4(__float_as_uint(r.v[0]), __float_as_uint(r.v[1]), __float_as_uint(r.v[2]),
+                      __float_as_uint(r.v[3]));
+}
+template <> __device__ __forceinline__ uint4 pack_unit<DT_BF16>(const RawUnit<DT_BF16> &r) {
+    uint4 o;
+    unsigned *w = reinterpret_cast<unsigned *>(&o);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bf16x2 t = {(__bf16) r.v[2 * i], (__bf16) r.v[2 * i + 1]};  // round to nearest even
+        w[i] = __builtin_bit_cast(unsigned, t);
+    }
+    return o;
+}
+template <> __device__ __forceinline__ uint4 pack_unit<DT_F16>(const RawUnit<DT_F16> &r) {
+    uint4 o;
+    unsigned *w = reinterpret_cast<unsigned *>(&o);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f16x2 t = {(_Float16) r.v[2 * i], (_Float16) r.v[2 * i + 1]};
+        w[i] = __builtin_bit_cast(unsigned, t);
+    }
+    return o;
+}
+template <> __device__ __forceinline__ uint4 pack_unit<DT_I8>(const RawUnit<DT_I8> &r) { return r.q; }
+
+// x / d for x * d < 2^32 with magic = floor(2^32 / d) + 1.  d == 1 is encoded as magic == 0 with
+// pass == ~0u (the quotient is x itself); otherwise pass == 0.  Branch-free on purpose: a scalar
+// branch between two loads would serialise them.
+__device__ __forceinline__ unsigned fast_div(unsigned x, unsigned magic, unsigned pass) {
+    return __umulhi(x, magic) + (x & pass);
+}
+
+// ---- A: one unit of one row ----------------------------------------------------------------------
+// voff: byte offset of (row, unit slot) fixed per thread, OOB for rows beyond M;
+// soff: byte offset of the K tile (uniform); k0: first reduction index of this unit; klim: end of K
+template <int DT>
+__device__ __forceinline__ void load_a_unit(RawUnit<DT> &r, rsrc_t ra, unsigned voff, unsigned soff, int k0, int klim) {
+    constexpr int KPU = Traits<DT>::KPU;
+    if constexpr (DT == DT_I8) {
+        r.q = buf_load_b128(ra, k0 < klim ? voff : OOB, soff);
+    } else {
+        // dwordx4 loads need dword alignment only.  A vector that straddles the end of a row brings
+        // in the head of the next row (the end of the buffer reads as zero, dwords are range-checked
+        // one by one); those lanes of K are cleared before they reach LDS (clear_a_tail).
+#pragma unroll
+        for (int q = 0; q < KPU / 4; ++q) {
+            const uint4 t = buf_load_b128(ra, (k0 + 4 * q < klim) ? voff + 16 * q : OOB, soff);
+            r.v[4 * q] = __uint_as_float(t.x); r.v[4 * q + 1] = __uint_as_float(t.y);
+            r.v[4 * q + 2] = __uint_as_float(t.z); r.v[4 * q + 3] = __uint_as_float(t.w);
+        }
+    }
+}
+
+// zero the elements of a unit whose reduction index is at or beyond klim (ragged end of K)
+template <int DT>
+__device__ __forceinline__ void clear_a_tail(RawUnit<DT> &r, int k0, int klim) {
+    if constexpr (DT != DT_I8) {
+#pragma unroll
+        for (int e = 0; e < Traits<DT>::KPU; ++e) r.v[e] = (k0 + e < klim) ? r.v[e] : 0.0f;
+    }
+}
+
+// ---- B: per-thread column state, fixed for the whole K loop -------------------------------------
+struct ColState {
+    unsigned pixoff;  // byte offset of the receptive field's origin in the (pad-shifted) buffer, OOB if n >= N
+    int ih0, iw0;     // top-left input coordinate of the receptive field
+};
+
+template <int BL>
+__device__ __forceinline__ ColState make_col(const IgemmParams &p, int n) {
+    ColState c;
+    const bool valid = n < p.N;
+    const int nn = valid ? n : 0;
+    const int img = nn / p.OHW;
+    const int pix = nn - img * p.OHW;
+    const int oh = pix / p.OW;
+    const int ow = pix - oh * p.OW;
+    c.ih0 = oh * p.sh - p.pt;
+    c.iw0 = ow * p.sw - p.pl;
+    unsigned off;
+    if constexpr (BL != BL_KVEC) off = (unsigned) (img * (int) p.b_img_stride + oh * p.sh * p.W + ow * p.sw) * 4u;
+    else off = (unsigned) ((img * p.H + oh * p.sh) * p.W + ow * p.sw) * (unsigned) p.pix_stride;
+    c.pixoff = valid ? off : OOB;
+    return c;
+}
+
+// u: unit index (wavefront-uniform); klim: end of the reduction range of this workgroup
+template <int DT, int BL>
+__device__ __forceinline__ void load_b_unit(RawUnit<DT> &r, const IgemmParams &p, rsrc_t rb, const ColState &c, int u,
+                                            int klim) {
+    constexpr int KPU = Traits<DT>::KPU;
+    if constexpr (BL == BL_PLAIN) {
+        static_assert(DT != DT_I8, "int8 activations are staged as NHWC vectors");
+        // 1x1 filter without padding (or a row-major [K, N] matrix): the pixel is always inside,
+        // only the channel moves, and it moves in the scalar offset
+#pragma unroll
+        for (int e = 0; e < KPU; ++e) {
+            const int k = u * KPU + e;
+            r.v[e] = buf_load_f32(rb, k < klim ? c.pixoff : OOB, (unsigned) k * (unsigned) p.HW * 4u);
+        }
+    } else if constexpr (BL == BL_GATHER) {
+        static_assert(DT != DT_I8, "int8 activations are staged as NHWC vectors");
+#pragma unroll
+        for (int e = 0; e < KPU; ++e) {
+            const unsigned k = (unsigned) (u * KPU + e);
+            const unsigned ch = fast_div(k, p.magic_khkw, p.pass_khkw);
+            const unsigned rem = k - ch * (unsigned) p.khkw;
+            const unsigned i = fast_div(rem, p.magic_kw, p.pass_kw);
+            const unsigned j = rem - i * (unsigned) p.kw;
+            const unsigned soff = (ch * (unsigned) p.HW + i * (unsigned) p.W + j) * 4u;
+            const bool ok = (int) k < klim && (unsigned) (c.ih0 + (int) i) < (unsigned) p.H &&
+                            (unsigned) (c.iw0 + (int) j) < (unsigned) p.W;
+            r.v[e] = buf_load_f32(rb, ok ? c.pixoff : OOB, soff);
+        }
+    } else {
+        // unit -> (tap, channel block); tap -> (i, j)
+        const unsigned tap = fast_div((unsigned) u, p.magic_upt, p.pass_upt);
+        const unsigned cb = (unsigned) u - tap * (unsigned) p.units_per_tap;
+        const unsigned i = fast_div(tap, p.magic_kw, p.pass_kw);
+        const unsigned j = tap - i * (unsigned) p.kw;
+        const unsigned soff = (i * (unsigned) p.W + j) * (unsigned) p.pix_stride + cb * 16u;
+        const bool ok = u * KPU < klim && (unsigned) (c.ih0 + (int) i) < (unsigned) p.H &&
+                        (unsigned) (c.iw0 + (int) j) < (unsigned) p.W;
+        const uint4 q = buf_load_b128(rb, ok ? c.pixoff : OOB, soff);
+        if constexpr (DT == DT_I8) {
+            r.q = q;
+        } else {
+            static_assert(DT == DT_F32 || DT == DT_I8, "vector B loader carries raw 16-byte units");
+            r.v[0] = __uint_as_float(q.x); r.v[1] = __uint_as_float(q.y);
+            r.v[2] = __uint_as_float(q.z); r.v[3] = __uint_as_float(q.w);
+        }
+    }
+}
+
+// ---- epilogue ----------------------------------------------------------------------------------------
+// byte offset of column n inside one batch slice of C (rows are added through the scalar offset)
+__device__ __forceinline__ unsigned out_col_offset(const IgemmParams &p, int n, int esz) {
+    if (p.out_mode == OUT_CONV) {
+        const int img = n / p.OHW;
+        const int pix = n - img * p.OHW;
+        return (unsigned) (img * (int) p.c_img_stride + pix) * (unsigned) esz;
+    }
+    return (unsigned) (n * (int) p.c_stride_n) * (unsigned) esz;
+}
+
+enum { EPI_NONE = 0, EPI_RELU = 1, EPI_CLIP = 2, EPI_GENERIC = 3 };
+
+template <int EPI>
+__device__ __forceinline__ float act_fast(float v, const Epilogue &e) {
+    if constexpr (EPI == EPI_NONE) return v;
+    else if constexpr (EPI == EPI_RELU) return v > 0.0f ? v : 0.0f;
+    else if constexpr (EPI == EPI_CLIP) {
+        const float t = v > e.clip_min ? v : e.clip_min;
+        return t < e.clip_max ? t : e.clip_max;
+    } else return apply_act(v, e);
+}
+
+// the consumer's activation quantiser (conv.c:961-973) applied to an fp32 result
+__device__ __forceinline__ int requant_s8(float y, float inv_scale) {
+    float t = __fmul_rn(y, inv_scale);
+    t = (t < -128.0f) ? -128.0f : (t > 127.0f) ? 127.0f : t;
+    return (int) roundf(t);
+}
+
+// Writes the accumulators of one wavefront.  Lane (li, lh) of a 32x32 block holds column li and rows
+// 8*(r/4) + 4*lh + (r%4): the column and the 4*lh part of the row go in the vector offset, the rest
+// of the row (uniform) in the scalar offset.
+template <int DT, int EPI, int TM, int TN, class ACC>
+__device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][TN], int batch, int m_wave, int n_wave,
+                                           int li, int lh) {
+    const int esz = (DT == DT_I8 && p.out_s8) ? 1 : 4;
+    const rsrc_t rc = make_rsrc(reinterpret_cast<const char *>(p.C) + (size_t) batch * p.c_batch_stride * esz,
+                                RSRC_RANGE);
+    const rsrc_t rbias = make_rsrc(p.bias, p.bias ? (unsigned) ((p.bias_mode == BIAS_N ? p.N : p.M) * 4) : 0u);
+    const rsrc_t raux = make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u);
+    const rsrc_t rb32 = make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u);
+    const rsrc_t racc = make_rsrc(p.acc_out ? p.acc_out + (size_t) batch * p.c_batch_stride : nullptr, RSRC_RANGE);
+    const bool m_edge = m_wave + TM * 32 > p.M;   // uniform: only the last row tile checks rows
+    const unsigned row_bytes = (unsigned) p.c_stride_m * (unsigned) esz;
+
+    unsigned col_voff[TN], col_voff4[TN];
+    float bias_n[TN];
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+        const int n = n_wave + b * 32 + li;
+        const bool ok = n < p.N;
+        const int nn = ok ? n : 0;
+        col_voff[b] = ok ? out_col_offset(p, nn, esz) + (unsigned) (4 * lh) * row_bytes : OOB;
+        col_voff4[b] = ok ? out_col_offset(p, nn, 4) + (unsigned) (4 * lh) * (unsigned) p.c_stride_m * 4u : OOB;
+        bias_n[b] = (p.bias_mode == BIAS_N) ? buf_load_f32(rbias, (unsigned) nn * 4u, 0) : 0.0f;
+    }
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);   // row of lanes with lh == 0
+            const int m = m_uni + 4 * lh;
+            const bool row_ok = !m_edge || m < p.M;
+            const unsigned soff = (unsigned) m_uni * row_bytes;
+            if constexpr (DT == DT_I8) {
+                // conv.c:1041-1056: acc * s, + bias, * (aux / 127): three separately rounded operations
+                const float coeff = __fdiv_rn(buf_load_f32(raux, (unsigned) m * 4u, 0), 127.0f);
+                const float fb = p.bias32 ? (float) (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, (unsigned) m * 4u, 0, 0) : 0.0f;
+#pragma unroll
+                for (int b = 0; b < TN; ++b) {
+                    const int av = acc[a][b][r];
+                    const unsigned voff = row_ok ? col_voff[b] : OOB;
+                    if (p.acc_out)
+                        __builtin_amdgcn_raw_buffer_store_b32((unsigned) av, racc, row_ok ? col_voff4[b] : OOB,
+                                                              (unsigned) m_uni * (unsigned) p.c_stride_m * 4u, 0);
+                    float f = __fmul_rn((float) av, p.in_scale);
+                    if (p.bias32) f = __fadd_rn(f, fb);
+                    const float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
+                    if (p.out_s8)
+                        __builtin_amdgcn_raw_buffer_store_b8((unsigned char) requant_s8(y, p.out_inv_scale), rc, voff, soff, 0);
+                    else
+                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), rc, voff, soff, 0);
+                }
+            } else {
+                const float bias_m = (p.bias_mode == BIAS_M) ? buf_load_f32(rbias, (unsigned) m * 4u, 0) : 0.0f;
+#pragma unroll
+                for (int b = 0; b < TN; ++b) {
+                    float v = acc[a][b][r];
+                    if (p.bias_mode == BIAS_M) v = __fadd_rn(v, bias_m);        // bias after the full sum
+                    else if (p.bias_mode == BIAS_N) v = __fadd_rn(v, bias_n[b]);
+                    v = act_fast<EPI>(v, p.ep);
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff[b] : OOB, soff, 0);
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ unsigned to_bits(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ unsigned to_bits(int v) { return (unsigned) v; }
+
+// split-K: raw partial sums [split][batch][M][N]; the finishing kernel applies the epilogue
+template <int TM, int TN, class ACC>
+__device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[TM][TN], int slice, int m_wave,
+                                              int n_wave, int li, int lh) {
+    const rsrc_t rp = make_rsrc(reinterpret_cast<const char *>(p.partial) + (size_t) slice * p.M * p.N * 4, RSRC_RANGE);
+    const bool m_edge = m_wave + TM * 32 > p.M;
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+        const int n = n_wave + b * 32 + li;
+        const unsigned cv = n < p.N ? (unsigned) (n + 4 * lh * p.N) * 4u : OOB;
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
+                const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
+                const auto val = acc[a][b][r];   // element copy first: bit-casting the vector element in place miscompiles
+                __builtin_amdgcn_raw_buffer_store_b32(to_bits(val), rp, row_ok ? cv : OOB,
+                                                      (unsigned) m_uni * (unsigned) p.N * 4u, 0);
+            }
+    }
+}
+
+// ---- the kernel --------------------------------------------------------------------------------
+template <int DT, int BL, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    static_assert(TM >= 1 && TN >= 1 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile / wave grid mismatch");
+    static_assert(THREADS % BN == 0 || BN % THREADS == 0, "B loader mapping");
+    constexpr int KPU = Traits<DT>::KPU;
+    constexpr int ESZ = DT == DT_I8 ? 1 : 4;   // bytes per stored operand element
+    constexpr int A_SLOTS = BM * UPT, B_SLOTS = BN * UPT;
+    constexpr int A_PER_T = (A_SLOTS + THREADS - 1) / THREADS;
+    constexpr int B_PER_T = B_SLOTS / THREADS;
+    static_assert(B_PER_T >= 1, "BN >= 64");
+    typedef typename Traits<DT>::acc_t acc_t;
+
+    __shared__ uint4 lds[2][A_SLOTS + B_SLOTS];
+
+    const int tid = threadIdx.x;
+    // the wavefront index is uniform; saying so keeps everything derived from it in scalar registers
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // XCD-aware tile order: consecutive workgroup ids go round-robin over the 8 XCDs (each with its
+    // own L2); give every XCD a contiguous run of tiles so neighbours in (m, n) share an L2.
+    const int tiles_m = (p.M + BM - 1) / BM;
+    int lid;
+    {
+        const int nb = gridDim.x, bid = blockIdx.x;
+        const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
+        lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+    }
+    const int tile_m = lid % tiles_m, tile_n = lid / tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int batch = blockIdx.z;
+    const int u_begin = blockIdx.y * p.k_split_units;
+    const int u_end = min(p.k_units, u_begin + p.k_split_units);
+    const int k_tiles = (u_end - u_begin + UPT - 1) / UPT;
+    const int klim = min(p.K, u_end * KPU);
+
+    // exact extent: the dwords of a row-end vector that fall past the matrix read as zero
+    const rsrc_t ra = make_rsrc(reinterpret_cast<const char *>(p.A) + (size_t) batch * p.a_batch_stride * ESZ,
+                                (unsigned) p.a_slice_bytes);
+    // the B buffer starts pad rows/columns before the tensor so that pixel offsets are never negative
+    const rsrc_t rb = make_rsrc(reinterpret_cast<const char *>(p.B) + (size_t) batch * p.b_batch_stride * ESZ -
+                                    (size_t) p.b_shift_bytes, RSRC_RANGE);
+
+    // per-thread A slots: (row, unit-in-tile) fixed for the whole K loop
+    unsigned a_voff[A_PER_T];
+    int a_unit[A_PER_T];
+#pragma unroll
+    for (int t = 0; t < A_PER_T; ++t) {
+        const int f = tid + t * THREADS;
+        const int ml = f / UPT, ua = f % UPT;
+        const bool ok = ((A_SLOTS % THREADS == 0) || f < A_SLOTS) && m0 + ml < p.M;
+        a_unit[t] = ua;
+        a_voff[t] = ok ? (unsigned) ((m0 + ml) * p.lda + ua * KPU) * (unsigned) ESZ : OOB;
+    }
+    // per-thread B column (same for all of its units)
+    const ColState col = make_col<BL>(p, n0 + (tid % BN));
+
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+
+    RawUnit<DT> qa[A_PER_T], qb[B_PER_T];
+
+    auto fetch = [&](int kt) {
+        const int ub = u_begin + kt * UPT;
+#pragma unroll
+        for (int t = 0; t < A_PER_T; ++t)
+            load_a_unit<DT>(qa[t], ra, a_voff[t], (unsigned) (ub * KPU * ESZ), (ub + a_unit[t]) * KPU, klim);
+#pragma unroll
+        for (int t = 0; t < B_PER_T; ++t) {
+            const int uu = __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN);
+            load_b_unit<DT, BL>(qb[t], p, rb, col, ub + uu, klim);
+        }
+    };
+    auto stage = [&](int buf, int kt) {
+        if ((u_begin + (kt + 1) * UPT) * KPU > klim) {   // uniform: only the tile holding the end of K
+#pragma unroll
+            for (int t = 0; t < A_PER_T; ++t) clear_a_tail<DT>(qa[t], (u_begin + kt * UPT + a_unit[t]) * KPU, klim);
+        }
+#pragma unroll
+        for (int t = 0; t < A_PER_T; ++t) {
+            const int f = tid + t * THREADS;
+            const int ml = f / UPT, ua = f % UPT;
+            if ((A_SLOTS % THREADS == 0) || f < A_SLOTS) lds[buf][ua * BM + ml] = pack_unit<DT>(qa[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < B_PER_T; ++t) {
+            const int f = tid + t * THREADS;
+            lds[buf][A_SLOTS + (f / BN) * BN + (f % BN)] = pack_unit<DT>(qb[t]);
+        }
+    };
+
+    if (k_tiles > 0) {
+        fetch(0);
+        stage(0, 0);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < k_tiles; ++kt) {
+        const int buf = kt & 1;
+        const bool more = kt + 1 < k_tiles;
+        if (more) fetch(kt + 1);
+        uint4 av[UPT / 2][TM], bv[UPT / 2][TN];
+#pragma unroll
+        for (int s = 0; s < UPT / 2; ++s) {
+#pragma unroll
+            for (int a = 0; a < TM; ++a) av[s][a] = lds[buf][(2 * s + lh) * BM + wm * (BM / WM) + a * 32 + li];
+#pragma unroll
+            for (int b = 0; b < TN; ++b) bv[s][b] = lds[buf][A_SLOTS + (2 * s + lh) * BN + wn * (BN / WN) + b * 32 + li];
+        }
+#pragma unroll
+        for (int s = 0; s < UPT / 2; ++s)
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b) Traits<DT>::mma(acc[a][b], av[s][a], bv[s][b]);
+        if (more) stage(buf ^ 1, kt + 1);
+        __syncthreads();
+    }
+
+    const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
+    if (p.partial) {
+        write_partial<TM, TN>(p, acc, blockIdx.y * gridDim.z + batch, m_wave, n_wave, li, lh);
+        return;
+    }
+    switch (p.ep.act) {
+        case NOT_ACT:
+        case RELU6: write_tile<DT, EPI_NONE, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case RELU: write_tile<DT, EPI_RELU, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case CLIP: write_tile<DT, EPI_CLIP, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        default: write_tile<DT, EPI_GENERIC, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+    }
+}
+
+// sums the split-K partials in slice order and applies the epilogue (one thread per output element)
+template <bool IS_INT>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p, int split, int batches) {
+    const long long total = (long long) batches * p.M * p.N;
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int n = (int) (idx % p.N);
+    const long long t = idx / p.N;
+    const int m = (int) (t % p.M);
+    const int batch = (int) (t / p.M);
+    const int esz = (IS_INT && p.out_s8) ? 1 : 4;
+    const size_t off4 = (size_t) batch * p.c_batch_stride + (size_t) m * p.c_stride_m + out_col_offset(p, n, 1);
+    char *cbase = reinterpret_cast<char *>(p.C);
+    if constexpr (IS_INT) {
+        int acc = 0;
+        for (int s = 0; s < split; ++s) acc += reinterpret_cast<const int *>(p.partial)[(size_t) s * total + idx];
+        if (p.acc_out) p.acc_out[off4] = acc;
+        float f = __fmul_rn((float) acc, p.in_scale);
+        if (p.bias32) f = __fadd_rn(f, (float) p.bias32[m]);
+        const float y = apply_act(__fmul_rn(f, __fdiv_rn(p.weight_aux[m], 127.0f)), p.ep);
+        if (p.out_s8) reinterpret_cast<int8_t *>(cbase)[off4] = (int8_t) requant_s8(y, p.out_inv_scale);
+        else reinterpret_cast<float *>(cbase)[off4] = y;
+        (void) esz;
+    } else {
+        float acc = 0.0f;
+        for (int s = 0; s < split; ++s) acc = __fadd_rn(acc, p.partial[(size_t) s * total + idx]);
+        if (p.bias_mode == BIAS_M) acc = __fadd_rn(acc, p.bias[m]);
+        else if (p.bias_mode == BIAS_N) acc = __fadd_rn(acc, p.bias[n]);
+        reinterpret_cast<float *>(cbase)[off4] = apply_act(acc, p.ep);
+    }
+}
+
+// ---- launch ------------------------------------------------------------------------------------------
+template <int DT, int BL, int BM, int BN, int WM, int WN>
+static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
+    const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    dim3 grid(tiles, cfg.split, cfg.batch);
+    hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN>), grid, dim3(THREADS), 0, stream, p);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    if (p.partial) {
+        const long long total = (long long) cfg.batch * p.M * p.N;
+        const int blocks = (int) ((total + 255) / 256);
+        if (DT == DT_I8)
+            hipLaunchKernelGGL((splitk_finish_kernel<true>), dim3(blocks), dim3(256), 0, stream, p, cfg.split, cfg.batch);
+        else
+            hipLaunchKernelGGL((splitk_finish_kernel<false>), dim3(blocks), dim3(256), 0, stream, p, cfg.split, cfg.batch);
+        ONHIP_CHECK_HIP(hipGetLastError());
+    }
+    return ONHIP_OK;
+}
+
+template <int DT, int BL>
+int launch_tile(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
+    const int key = cfg.bm * 1000 + cfg.bn;
+    switch (key) {
+        case 128128: return launch_one<DT, BL, 128, 128, 2, 2>(cfg, p, stream);
+        case 64128: return launch_one<DT, BL, 64, 128, 2, 2>(cfg, p, stream);
+        case 64064: return launch_one<DT, BL, 64, 64, 2, 2>(cfg, p, stream);
+        case 32128: return launch_one<DT, BL, 32, 128, 1, 4>(cfg, p, stream);
+        default: return set_error(ONHIP_ERR_ARG, "igemm: no kernel for tile %dx%d", cfg.bm, cfg.bn);
+    }
+}
+
+
+}  // namespace onhip

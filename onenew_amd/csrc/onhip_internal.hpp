@@ -65,8 +65,9 @@ __device__ __forceinline__ float apply_act(float v, const Epilogue &e) {
 // C[M, N] = A[M, K] * B[K, N] on MFMA 32x32 tiles.  A rows are K-contiguous (weights, or the left
 // MatMul operand).  B is produced on the fly by one of two loaders.
 
-enum { BL_GATHER = 0,  // element gather: NCHW activations (implicit im2col) or a row-major [K, N] matrix
-       BL_KVEC = 1 };  // 16-byte vectors along K: NHWC int8 activations, or an [N, K] matrix
+enum { BL_GATHER = 0,  // element gather from NCHW activations (implicit im2col), any filter / stride / padding
+       BL_KVEC = 1,    // 16-byte vectors along K from NHWC int8 activations
+       BL_PLAIN = 2 }; // 1x1 filter without padding, or a row-major [K, N] matrix: no tap arithmetic
 
 enum { OUT_CONV = 0,   // n = img * OHW + pix  ->  img * c_img_stride + m * c_stride_m + pix
        OUT_PLAIN = 1 };// m * c_stride_m + n * c_stride_n
@@ -81,18 +82,20 @@ struct IgemmParams {
     const void *A;
     long long a_batch_stride;  // elements; 0 = shared
     int lda;                   // elements between rows
-    int a_vec;                 // rows are 16-byte aligned and lda * elem is a multiple of 16
     // B
     const void *B;
     long long b_batch_stride;  // elements
     // gather geometry (BL_GATHER)
     int H, W, OW, OHW, HW;
     int kh, kw, khkw, sh, sw, pt, pl;
-    unsigned magic_khkw, magic_kw;
+    unsigned magic_khkw, magic_kw;   // multiply-high constants for / (kh*kw) and / kw
+    unsigned pass_khkw, pass_kw;     // ~0u when the divisor is 1 (quotient = dividend), else 0
     long long b_img_stride;    // Cin * H * W
+    long long b_shift_bytes;   // the B buffer descriptor starts this many bytes before the tensor (pad rows/cols)
+    long long a_slice_bytes, b_slice_bytes, c_slice_bytes;  // extent one batch slice can address (< 2 GiB)
     // vector geometry (BL_KVEC)
     int units_per_tap;         // units per filter tap (Cp / 16 for NHWC int8); k_units for a plain matrix
-    unsigned magic_upt;
+    unsigned magic_upt, pass_upt;
     int pix_stride;            // bytes between consecutive n ("pixels"): Cp, or ldb * elem
     // C
     void *C;
