@@ -123,6 +123,7 @@ def main():
     ap.add_argument("--workload", default="resnet50_b32")
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-tune", action="store_true", help="use the cost model instead of measured tile choice")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path runs on a single MI355X and nothing in this build "
@@ -132,6 +133,8 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
     hip.init(0)
+    # tile / split-K per layer shape is measured on first use (during the warm-up steps) and cached
+    hip.set_tuning(0 if args.no_tune else 1)
 
     desc, dtype, layer_descs = make_workload(args.workload)
     layers = [DeviceLayer(torch, n, d, args.workload) for n, d in layer_descs]

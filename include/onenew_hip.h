@@ -80,6 +80,12 @@ typedef struct {
 int onhip_init(int device);
 /* Text of the last error on this thread ("" if none). */
 const char *onhip_last_error(void);
+/* Tile / split-K selection.  mode 0: cost model only.  mode 1: the first call for each problem
+ * signature times the candidate launches on the caller's stream (it synchronises that stream once)
+ * and the winner is cached for the life of the process -- the counterpart of the reference's GEMM tile
+ * search (tools/optimize/auto_tuning.hpp:9-75).  Default: the ONHIP_TUNE environment variable, else 0.
+ * Returns the previous mode. */
+int onhip_set_tuning(int mode);
 /* Output height / width of a convolution (host/ops/conv.h:43-50). Returns 0 or ONHIP_ERR_ARG. */
 int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow);
 

@@ -5,7 +5,12 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <math.h>
+#include <stdlib.h>
+
+#include <map>
 #include <mutex>
+#include <vector>
 
 #include "onhip_internal.hpp"
 
@@ -86,29 +91,169 @@ static int get_scratch(size_t bytes, void **out) {
     return ONHIP_OK;
 }
 
-// Split K when the tile grid cannot occupy the chip: aim for about two workgroups per CU.
-static int plan_split(IgemmLaunch &cfg, IgemmParams &p) {
-    const long long tiles = (long long) ((p.M + cfg.bm - 1) / cfg.bm) * ((p.N + cfg.bn - 1) / cfg.bn) * cfg.batch;
-    cfg.split = 1;
+// ---- tile and split-K choice ----------------------------------------------------------------------
+//
+// A launch is described by (tile BM x BN, split): split > 1 cuts K into slices that write partial
+// sums to the scratch buffer and a finishing kernel adds them up.  The choice comes from a cost model
+// or, when tuning is on, from timing the candidates once per problem signature (the counterpart of
+// the reference's grid search over GEMM tiles, tools/optimize/auto_tuning.hpp:9-75).
+static const int kTiles[][2] = {{128, 128}, {64, 128}, {64, 64}, {32, 128}};
+static const int kNumTiles = 4;
+static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+static const int kNumSplits = 10;
+
+struct Choice { int bm, bn, split; };
+
+static std::mutex g_tune_mu;
+static int g_tune_mode = -1;   // -1: read ONHIP_TUNE on first use; 0 model only; 1 measure
+static std::map<std::vector<long long>, Choice> g_tuned;
+
+static int tune_mode() {
+    if (g_tune_mode < 0) {
+        const char *e = getenv("ONHIP_TUNE");
+        g_tune_mode = (e && atoi(e) > 0) ? 1 : 0;
+    }
+    return g_tune_mode;
+}
+
+static int mfma_k_per_unit(int dt) { return dt == DT_F32 ? 4 : dt == DT_I8 ? 16 : 8; }
+
+// cycles one CU needs for the MFMAs of one K tile of a BM x BN workgroup
+static double tile_mfma_cycles(int dt, int bm, int bn) {
+    const double flops = 2.0 * bm * bn * 4 * mfma_k_per_unit(dt);
+    const double per_clk = dt == DT_F32 ? 256.0 : dt == DT_I8 ? 8192.0 : 4096.0;
+    return flops / per_clk;
+}
+
+static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
+    cfg.bm = c.bm; cfg.bn = c.bn; cfg.split = 1;
     p.k_split_units = p.k_units;
     p.partial = nullptr;
-    const int k_tiles = (p.k_units + 3) / 4;
-    if (tiles >= 192 || k_tiles < 8) return ONHIP_OK;
-    int split = (int) ((512 + tiles - 1) / tiles);
-    if (split > k_tiles / 4) split = k_tiles / 4;
-    if (split > 32) split = 32;
-    if (split < 2) return ONHIP_OK;
-    const int tiles_per = (k_tiles + split - 1) / split;
-    split = (k_tiles + tiles_per - 1) / tiles_per;
-    void *buf = nullptr;
-    const size_t bytes = (size_t) split * cfg.batch * p.M * p.N * 4;
-    if (bytes > (512u << 20)) return ONHIP_OK;
-    int rc = get_scratch(bytes, &buf);
-    if (rc) return rc;
-    cfg.split = split;
-    p.k_split_units = tiles_per * 4;
-    p.partial = reinterpret_cast<float *>(buf);
+    if (c.split > 1) {
+        const int k_tiles = (p.k_units + 3) / 4;
+        const int tiles_per = (k_tiles + c.split - 1) / c.split;
+        const int split = (k_tiles + tiles_per - 1) / tiles_per;
+        if (split > 1) {
+            void *buf = nullptr;
+            const size_t bytes = (size_t) split * cfg.batch * p.M * p.N * 4;
+            int rc = get_scratch(bytes, &buf);
+            if (rc) return rc;
+            cfg.split = split;
+            p.k_split_units = tiles_per * 4;
+            p.partial = reinterpret_cast<float *>(buf);
+        }
+    }
     return ONHIP_OK;
+}
+
+static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
+    const int k_tiles = (p.k_units + 3) / 4;
+    if (c.split > 1 && (k_tiles < 2 * c.split)) return false;
+    if (c.split > 1 && (size_t) c.split * cfg.batch * p.M * p.N * 4 > ((size_t) 256 << 20)) return false;
+    return true;
+}
+
+// Cost model (cycles).  A CU works through its share of the workgroups; co-resident workgroups share
+// the MFMA pipes, so the MFMA time adds up while the per-workgroup fill/drain latency overlaps when
+// several are resident.  Split-K adds the partial-sum traffic and a second launch.
+static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
+    const long long tiles = (long long) ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * cfg.batch;
+    const int k_tiles = (p.k_units + 3) / 4;
+    const int per = (k_tiles + c.split - 1) / c.split;
+    const double wgs = (double) tiles * c.split;
+    const double per_cu = ceil(wgs / 256.0);
+    const int regs_occ = c.bm * c.bn >= 128 * 128 ? 3 : c.bm * c.bn >= 64 * 128 ? 4 : 6;
+    const double resident = per_cu < regs_occ ? per_cu : regs_occ;
+    const double overhead = cfg.bl == BL_GATHER ? 1.35 : 1.18;   // measured steady-state inefficiency
+    const double mfma = per * tile_mfma_cycles(cfg.dtype, c.bm, c.bn) * overhead;
+    const double fixed = 2600.0 + 12.0 * (c.bm * c.bn / 256);     // first loads in flight + epilogue stores
+    double cycles = per_cu * mfma + ceil(per_cu / resident) * fixed;
+    if (c.split > 1) cycles += 9000.0 + (double) (c.split + 1) * p.M * p.N * cfg.batch * 4.0 / 1500.0;
+    return cycles;
+}
+
+static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
+    Choice best = {64, 64, 1};
+    double best_cost = 1e300;
+    for (int t = 0; t < kNumTiles; ++t)
+        for (int s = 0; s < kNumSplits; ++s) {
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s]};
+            if (!candidate_ok(cfg, p, c)) continue;
+            const double cost = model_cost(cfg, p, c);
+            if (cost < best_cost) { best_cost = cost; best = c; }
+        }
+    return best;
+}
+
+static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st, hipEvent_t e0, hipEvent_t e1,
+                       float *best_ms) {
+    int rc = apply_choice(cfg, p, c);
+    if (rc) return rc;
+    rc = igemm_launch(cfg, p, st);   // warm-up
+    if (rc) return rc;
+    float best = 1e30f;
+    for (int rep = 0; rep < 2; ++rep) {
+        ONHIP_CHECK_HIP(hipEventRecord(e0, st));
+        for (int i = 0; i < 3; ++i) {
+            rc = igemm_launch(cfg, p, st);
+            if (rc) return rc;
+        }
+        ONHIP_CHECK_HIP(hipEventRecord(e1, st));
+        ONHIP_CHECK_HIP(hipEventSynchronize(e1));
+        float ms = 0.f;
+        ONHIP_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+        if (ms < best) best = ms;
+    }
+    *best_ms = best / 3.0f;
+    return ONHIP_OK;
+}
+
+// Chooses tile and split for the problem and makes p / cfg ready to launch.
+static int plan_launch(IgemmLaunch &cfg, IgemmParams &p, hipStream_t st) {
+    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT]
+        Choice c = {0, 0, 1};
+        if (sscanf(env, "%dx%dx%d", &c.bm, &c.bn, &c.split) >= 2) return apply_choice(cfg, p, c);
+    }
+    if (!tune_mode()) return apply_choice(cfg, p, model_choice(cfg, p));
+    std::vector<long long> key = {cfg.dtype, cfg.bl, cfg.batch, p.M, p.N, p.K, p.k_units, p.khkw, p.sh, p.sw,
+                                  p.H, p.W, p.out_mode, p.lda};
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mu);
+        auto it = g_tuned.find(key);
+        if (it != g_tuned.end()) return apply_choice(cfg, p, it->second);
+    }
+    // measure: the candidates the model ranks within 2.5x of its best, on the caller's stream
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone)
+        return apply_choice(cfg, p, model_choice(cfg, p));
+    const Choice guess = model_choice(cfg, p);
+    const double guess_cost = model_cost(cfg, p, guess);
+    hipEvent_t e0, e1;
+    ONHIP_CHECK_HIP(hipEventCreate(&e0));
+    ONHIP_CHECK_HIP(hipEventCreate(&e1));
+    Choice best = guess;
+    float best_ms = 1e30f;
+    int rc = ONHIP_OK;
+    for (int t = 0; t < kNumTiles && !rc; ++t)
+        for (int s = 0; s < kNumSplits && !rc; ++s) {
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s]};
+            if (!candidate_ok(cfg, p, c) || model_cost(cfg, p, c) > 2.5 * guess_cost) continue;
+            float ms = 0.f;
+            rc = time_choice(cfg, p, c, st, e0, e1, &ms);
+            if (!rc && ms < best_ms) { best_ms = ms; best = c; }
+        }
+    (void) hipEventDestroy(e0);
+    (void) hipEventDestroy(e1);
+    if (rc) return rc;
+    if (getenv("ONHIP_TUNE_VERBOSE"))
+        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d (%.4f ms; model said %dx%d split %d)\n",
+                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best_ms, guess.bm, guess.bn,
+                guess.split);
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mu);
+        g_tuned[key] = best;
+    }
+    return apply_choice(cfg, p, best);
 }
 
 static int dtype_of_compute(int compute, int *dt) {
@@ -138,6 +283,13 @@ int onhip_init(int device) {
         return set_error(ONHIP_ERR_RUNTIME, "device %d is %s; this library holds gfx950 code only", device,
                          prop.gcnArchName);
     return ONHIP_OK;
+}
+
+int onhip_set_tuning(int mode) {
+    std::lock_guard<std::mutex> lock(g_tune_mu);
+    const int prev = tune_mode();
+    g_tune_mode = mode > 0 ? 1 : 0;
+    return prev;
 }
 
 int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow) {
@@ -182,6 +334,7 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
     p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
     p.magic_khkw = magic_for(p.khkw); p.pass_khkw = pass_for(p.khkw);
     p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
+    p.use_tapmask = p.khkw <= 64;
     p.b_img_stride = (long long) d->cin * d->h * d->w;
     if (p.khkw == 1 && !d->pad_t && !d->pad_l && !d->pad_b && !d->pad_r) cfg.bl = BL_PLAIN;
     p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * 4;
@@ -195,8 +348,7 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
     p.bias = bias;
     p.bias_mode = d->has_bias ? BIAS_M : BIAS_NONE;
     p.ep = ep;
-    igemm_pick_tile(cfg, p);
-    rc = plan_split(cfg, p);
+    rc = plan_launch(cfg, p, st);
     if (rc) return rc;
     return igemm_launch(cfg, p, st);
 }
@@ -270,6 +422,7 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
     p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
     p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
     p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
+    p.use_tapmask = p.khkw <= 64;
     p.units_per_tap = cp / 16;
     p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
     p.pix_stride = cp;
@@ -288,8 +441,7 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
     p.acc_out = acc32;
     p.out_s8 = d->out_s8;
     p.out_inv_scale = d->out_s8 ? 1.0f / d->output_scale : 0.0f;
-    igemm_pick_tile(cfg, p);
-    rc = plan_split(cfg, p);
+    rc = plan_launch(cfg, p, st);
     if (rc) return rc;
     return igemm_launch(cfg, p, st);
 }
@@ -335,10 +487,10 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     p.bias_mode = bias ? BIAS_N : BIAS_NONE;
     p.ep.act = gelu_lut ? ONHIP_ACT_GELU_LUT : NOT_ACT;
     p.ep.lut = gelu_lut;
-    igemm_pick_tile(cfg, p);
-    rc = plan_split(cfg, p);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    rc = plan_launch(cfg, p, st);
     if (rc) return rc;
-    return igemm_launch(cfg, p, reinterpret_cast<hipStream_t>(stream));
+    return igemm_launch(cfg, p, st);
 }
 
 int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w, const float *bias, float *out,

@@ -1,5 +1,8 @@
 // Dispatch of the implicit-GEMM kernel family: picks the tile and the (element type, B loader)
 // variant; the kernels themselves are instantiated per element type in igemm_{f32,bf16,f16,i8}.hip.
+#include <stdio.h>
+#include <stdlib.h>
+
 #include "onhip_internal.hpp"
 
 namespace onhip {
@@ -24,24 +27,6 @@ int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t strea
         case DT_I8: return igemm_launch_i8(cfg, p, stream);
         default: return set_error(ONHIP_ERR_ARG, "igemm: unsupported element type %d", cfg.dtype);
     }
-}
-
-// Tile choice: largest tile whose padding waste is small and that still yields enough workgroups to
-// cover the 256 CUs a few times over.
-void igemm_pick_tile(IgemmLaunch &cfg, const IgemmParams &p) {
-    static const int cand[][2] = {{128, 128}, {64, 128}, {64, 64}, {32, 128}};
-    static const double weight[] = {1.0, 0.9, 0.75, 0.7};
-    double best = -1.0;
-    for (int i = 0; i < 4; ++i) {
-        const int bm = cand[i][0], bn = cand[i][1];
-        const long long tm = (p.M + bm - 1) / bm, tn = (p.N + bn - 1) / bn;
-        const double eff = ((double) p.M * p.N) / ((double) tm * bm * tn * bn);
-        const double wgs = (double) tm * tn * cfg.batch;
-        const double fill = wgs >= 512.0 ? 1.0 : (wgs / 512.0);
-        const double score = eff * weight[i] * (0.25 + 0.75 * fill);
-        if (score > best) { best = score; cfg.bm = bm; cfg.bn = bn; }
-    }
-    cfg.split = 1;
 }
 
 }  // namespace onhip

@@ -65,22 +65,24 @@ __device__ __forceinline__ uint4 buf_load_b128(rsrc_t r, unsigned voff, unsigned
 }
 
 template <int DT> struct Traits;
+// mma_part: one MFMA instruction of the PARTS that consume a pair of 16-byte units
 template <> struct Traits<DT_F32> {
     static constexpr int KPU = 4;
     static constexpr int RAW = 4;          // fp32 values fetched per unit
+    static constexpr int PARTS = 4;        // one v_mfma_f32_32x32x2_f32 per fp32 of the unit
     typedef f32x16 acc_t;
-    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
-        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+    static __device__ __forceinline__ void mma_part(acc_t &c, const uint4 &a, const uint4 &b, int part) {
+        const unsigned av = part == 0 ? a.x : part == 1 ? a.y : part == 2 ? a.z : a.w;
+        const unsigned bv = part == 0 ? b.x : part == 1 ? b.y : part == 2 ? b.z : b.w;
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(av), __uint_as_float(bv), c, 0, 0, 0);
     }
 };
 template <> struct Traits<DT_BF16> {
     static constexpr int KPU = 8;
     static constexpr int RAW = 8;
+    static constexpr int PARTS = 1;
     typedef f32x16 acc_t;
-    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+    static __device__ __forceinline__ void mma_part(acc_t &c, const uint4 &a, const uint4 &b, int) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
                                                     0, 0, 0);
     }
@@ -88,8 +90,9 @@ template <> struct Traits<DT_BF16> {
 template <> struct Traits<DT_F16> {
     static constexpr int KPU = 8;
     static constexpr int RAW = 8;
+    static constexpr int PARTS = 1;
     typedef f32x16 acc_t;
-    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+    static __device__ __forceinline__ void mma_part(acc_t &c, const uint4 &a, const uint4 &b, int) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
                                                    0, 0);
     }
@@ -97,8 +100,9 @@ template <> struct Traits<DT_F16> {
 template <> struct Traits<DT_I8> {
     static constexpr int KPU = 16;
     static constexpr int RAW = 4;          // 4 dwords = 16 int8
+    static constexpr int PARTS = 1;
     typedef i32x16 acc_t;
-    static __device__ __forceinline__ void mma(acc_t &c, const uint4 &a, const uint4 &b) {
+    static __device__ __forceinline__ void mma_part(acc_t &c, const uint4 &a, const uint4 &b, int) {
         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), c, 0, 0,
                                                   0);
     }
@@ -174,8 +178,9 @@ __device__ __forceinline__ void clear_a_tail(RawUnit<DT> &r, int k0, int klim) {
 
 // ---- B: per-thread column state, fixed for the whole K loop -------------------------------------
 struct ColState {
-    unsigned pixoff;  // byte offset of the receptive field's origin in the (pad-shifted) buffer, OOB if n >= N
-    int ih0, iw0;     // top-left input coordinate of the receptive field
+    unsigned pixoff;   // byte offset of the receptive field's origin in the (pad-shifted) buffer, OOB if n >= N
+    int ih0, iw0;      // top-left input coordinate of the receptive field
+    unsigned mask_lo, mask_hi;  // bit t set: filter tap t (t = i * kw + j, t < 64) falls inside the image
 };
 
 template <int BL>
@@ -193,54 +198,83 @@ __device__ __forceinline__ ColState make_col(const IgemmParams &p, int n) {
     if constexpr (BL != BL_KVEC) off = (unsigned) (img * (int) p.b_img_stride + oh * p.sh * p.W + ow * p.sw) * 4u;
     else off = (unsigned) ((img * p.H + oh * p.sh) * p.W + ow * p.sw) * (unsigned) p.pix_stride;
     c.pixoff = valid ? off : OOB;
+    c.mask_lo = c.mask_hi = 0;
+    if constexpr (BL != BL_PLAIN) {
+        if (p.use_tapmask) {
+            int i = 0, j = 0;
+            for (int t = 0; t < p.khkw; ++t) {
+                const bool ok = (unsigned) (c.ih0 + i) < (unsigned) p.H && (unsigned) (c.iw0 + j) < (unsigned) p.W;
+                if (ok) { if (t < 32) c.mask_lo |= 1u << t; else c.mask_hi |= 1u << (t - 32); }
+                if (++j == p.kw) { j = 0; ++i; }
+            }
+        }
+    }
     return c;
 }
 
-// u: unit index (wavefront-uniform); klim: end of the reduction range of this workgroup
+// Scalar description of one B load, computed a tile ahead in the shadow of the MFMAs: the
+// wavefront-uniform byte offset and the bit that selects the tap in the lane's validity mask
+// (0 when the reduction index is past the end of K).
+struct BPrep {
+    unsigned soff;
+    unsigned bit;
+    unsigned hi;   // the tap index is 32..63: test mask_hi
+};
+
+// item: (unit slot t, element e) for the element loaders, unit slot t for the vector loader
 template <int DT, int BL>
-__device__ __forceinline__ void load_b_unit(RawUnit<DT> &r, const IgemmParams &p, rsrc_t rb, const ColState &c, int u,
-                                            int klim) {
+__device__ __forceinline__ BPrep prep_b(const IgemmParams &p, int u, int e, int klim) {
     constexpr int KPU = Traits<DT>::KPU;
+    BPrep r;
     if constexpr (BL == BL_PLAIN) {
-        static_assert(DT != DT_I8, "int8 activations are staged as NHWC vectors");
-        // 1x1 filter without padding (or a row-major [K, N] matrix): the pixel is always inside,
-        // only the channel moves, and it moves in the scalar offset
-#pragma unroll
-        for (int e = 0; e < KPU; ++e) {
-            const int k = u * KPU + e;
-            r.v[e] = buf_load_f32(rb, k < klim ? c.pixoff : OOB, (unsigned) k * (unsigned) p.HW * 4u);
-        }
+        const int k = u * KPU + e;
+        r.soff = (unsigned) k * (unsigned) p.HW * 4u;
+        r.bit = k < klim ? 1u : 0u;
+        r.hi = 0;
     } else if constexpr (BL == BL_GATHER) {
-        static_assert(DT != DT_I8, "int8 activations are staged as NHWC vectors");
-#pragma unroll
-        for (int e = 0; e < KPU; ++e) {
-            const unsigned k = (unsigned) (u * KPU + e);
-            const unsigned ch = fast_div(k, p.magic_khkw, p.pass_khkw);
-            const unsigned rem = k - ch * (unsigned) p.khkw;
-            const unsigned i = fast_div(rem, p.magic_kw, p.pass_kw);
-            const unsigned j = rem - i * (unsigned) p.kw;
-            const unsigned soff = (ch * (unsigned) p.HW + i * (unsigned) p.W + j) * 4u;
-            const bool ok = (int) k < klim && (unsigned) (c.ih0 + (int) i) < (unsigned) p.H &&
-                            (unsigned) (c.iw0 + (int) j) < (unsigned) p.W;
-            r.v[e] = buf_load_f32(rb, ok ? c.pixoff : OOB, soff);
-        }
+        const unsigned k = (unsigned) (u * KPU + e);
+        const unsigned ch = fast_div(k, p.magic_khkw, p.pass_khkw);
+        const unsigned rem = k - ch * (unsigned) p.khkw;
+        const unsigned i = fast_div(rem, p.magic_kw, p.pass_kw);
+        const unsigned j = rem - i * (unsigned) p.kw;
+        r.soff = (ch * (unsigned) p.HW + i * (unsigned) p.W + j) * 4u;
+        r.bit = (int) k < klim ? (1u << (rem & 31u)) : 0u;
+        r.hi = rem >> 5;
     } else {
-        // unit -> (tap, channel block); tap -> (i, j)
         const unsigned tap = fast_div((unsigned) u, p.magic_upt, p.pass_upt);
         const unsigned cb = (unsigned) u - tap * (unsigned) p.units_per_tap;
         const unsigned i = fast_div(tap, p.magic_kw, p.pass_kw);
         const unsigned j = tap - i * (unsigned) p.kw;
-        const unsigned soff = (i * (unsigned) p.W + j) * (unsigned) p.pix_stride + cb * 16u;
-        const bool ok = u * KPU < klim && (unsigned) (c.ih0 + (int) i) < (unsigned) p.H &&
-                        (unsigned) (c.iw0 + (int) j) < (unsigned) p.W;
-        const uint4 q = buf_load_b128(rb, ok ? c.pixoff : OOB, soff);
-        if constexpr (DT == DT_I8) {
-            r.q = q;
-        } else {
-            static_assert(DT == DT_F32 || DT == DT_I8, "vector B loader carries raw 16-byte units");
-            r.v[0] = __uint_as_float(q.x); r.v[1] = __uint_as_float(q.y);
-            r.v[2] = __uint_as_float(q.z); r.v[3] = __uint_as_float(q.w);
+        r.soff = (i * (unsigned) p.W + j) * (unsigned) p.pix_stride + cb * 16u;
+        r.bit = u * KPU < klim ? (1u << (tap & 31u)) : 0u;
+        r.hi = tap >> 5;
+    }
+    return r;
+}
+
+// vector offset of a prepared B load for this lane: the pixel if the tap is inside, else OOB
+template <int BL>
+__device__ __forceinline__ unsigned b_voff(const IgemmParams &p, const ColState &c, const BPrep &q, int u_or_k) {
+    if constexpr (BL == BL_PLAIN) {
+        return q.bit ? c.pixoff : OOB;
+    } else {
+        if (p.use_tapmask) {
+            const unsigned word = q.hi ? c.mask_hi : c.mask_lo;
+            return (word & q.bit) ? c.pixoff : OOB;
         }
+        // more than 64 taps: validity by coordinates (slow path, large filters only)
+        unsigned tap;
+        if constexpr (BL == BL_GATHER) {
+            const unsigned k = (unsigned) u_or_k;
+            tap = k - fast_div(k, p.magic_khkw, p.pass_khkw) * (unsigned) p.khkw;
+        } else {
+            tap = fast_div((unsigned) u_or_k, p.magic_upt, p.pass_upt);
+        }
+        const unsigned i = fast_div(tap, p.magic_kw, p.pass_kw);
+        const unsigned j = tap - i * (unsigned) p.kw;
+        const bool ok = q.bit != 0 && (unsigned) (c.ih0 + (int) i) < (unsigned) p.H &&
+                        (unsigned) (c.iw0 + (int) j) < (unsigned) p.W;
+        return ok ? c.pixoff : OOB;
     }
 }
 
@@ -440,26 +474,51 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 
     RawUnit<DT> qa[A_PER_T], qb[B_PER_T];
 
-    auto fetch = [&](int kt) {
+    constexpr int PARTS = Traits<DT>::PARTS;
+    constexpr int BE = (BL == BL_KVEC) ? 1 : KPU;     // loads per B unit
+    constexpr int B_ITEMS = B_PER_T * BE;
+    constexpr int BLOCKS = (UPT / 2) * TM * TN;       // 32x32 blocks x unit pairs per K tile
+    constexpr int STEPS = BLOCKS * PARTS;             // MFMA instructions per K tile and wavefront
+    constexpr int HALF = STEPS / 2;
+    constexpr int READS = (UPT / 2) * (TM + TN);      // LDS operand reads per K tile and wavefront
+    struct Operands { uint4 a[UPT / 2][TM], b[UPT / 2][TN]; };
+
+    BPrep bp[B_ITEMS];                                // scalar descriptions of the next B loads
+
+    auto b_unit_of = [&](int t) { return __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN); };
+    auto prep_item = [&](int kt, int idx) {
+        const int t = idx / BE, e = idx % BE;
+        bp[idx] = prep_b<DT, BL>(p, u_begin + kt * UPT + b_unit_of(t), e, klim);
+    };
+    // issue every global load of K tile kt (B descriptions must have been prepared for kt)
+    auto issue = [&](int kt) {
         const int ub = u_begin + kt * UPT;
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t)
             load_a_unit<DT>(qa[t], ra, a_voff[t], (unsigned) (ub * KPU * ESZ), (ub + a_unit[t]) * KPU, klim);
 #pragma unroll
         for (int t = 0; t < B_PER_T; ++t) {
-            const int uu = __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN);
-            load_b_unit<DT, BL>(qb[t], p, rb, col, ub + uu, klim);
+            const int u = ub + b_unit_of(t);
+            if constexpr (BL == BL_KVEC) {
+                const uint4 q = buf_load_b128(rb, b_voff<BL>(p, col, bp[t], u), bp[t].soff);
+                if constexpr (DT == DT_I8) qb[t].q = q;
+                else {
+                    qb[t].v[0] = __uint_as_float(q.x); qb[t].v[1] = __uint_as_float(q.y);
+                    qb[t].v[2] = __uint_as_float(q.z); qb[t].v[3] = __uint_as_float(q.w);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < KPU; ++e)
+                    qb[t].v[e] = buf_load_f32(rb, b_voff<BL>(p, col, bp[t * KPU + e], u * KPU + e), bp[t * KPU + e].soff);
+            }
         }
     };
     auto stage = [&](int buf, int kt) {
-        if ((u_begin + (kt + 1) * UPT) * KPU > klim) {   // uniform: only the tile holding the end of K
-#pragma unroll
-            for (int t = 0; t < A_PER_T; ++t) clear_a_tail<DT>(qa[t], (u_begin + kt * UPT + a_unit[t]) * KPU, klim);
-        }
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t) {
             const int f = tid + t * THREADS;
             const int ml = f / UPT, ua = f % UPT;
+            clear_a_tail<DT>(qa[t], (u_begin + kt * UPT + a_unit[t]) * KPU, klim);
             if ((A_SLOTS % THREADS == 0) || f < A_SLOTS) lds[buf][ua * BM + ml] = pack_unit<DT>(qa[t]);
         }
 #pragma unroll
@@ -468,34 +527,64 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             lds[buf][A_SLOTS + (f / BN) * BN + (f % BN)] = pack_unit<DT>(qb[t]);
         }
     };
+    auto read_operand = [&](Operands &o, int buf, int idx) {   // idx-th of the READS LDS reads
+        const int s = idx / (TM + TN), t = idx % (TM + TN);
+        if (t < TM) o.a[s][t] = lds[buf][(2 * s + lh) * BM + wm * (BM / WM) + t * 32 + li];
+        else o.b[s][t - TM] = lds[buf][A_SLOTS + (2 * s + lh) * BN + wn * (BN / WN) + (t - TM) * 32 + li];
+    };
 
-    if (k_tiles > 0) {
-        fetch(0);
-        stage(0, 0);
-    }
+    // Pipeline.  While the MFMAs of K tile kt run (its operands are already in registers):
+    //   step 0            LDS store of tile kt+1 (loaded one tile ago), then all global loads of tile kt+2
+    //   steps 1..         scalar descriptions of the B loads of tile kt+3, spread over the MFMAs
+    //   after HALF steps  barrier
+    //   second half       LDS reads of tile kt+1 into the other operand set, spread over the MFMAs
+    // A wavefront therefore always has matrix work queued while it waits for LDS, the barrier or
+    // memory, and a global load has a whole tile of MFMAs to complete.  Past the last tile loads are
+    // fully masked (zero, no memory traffic), so the body has no branches.
+    Operands op0, op1;
+#pragma unroll
+    for (int i = 0; i < B_ITEMS; ++i) prep_item(0, i);
+    issue(0);
+    stage(0, 0);
+#pragma unroll
+    for (int i = 0; i < B_ITEMS; ++i) prep_item(1, i);
+    issue(1);
+#pragma unroll
+    for (int i = 0; i < B_ITEMS; ++i) prep_item(2, i);
     __syncthreads();
+#pragma unroll
+    for (int i = 0; i < READS; ++i) read_operand(op0, 0, i);
 
-    for (int kt = 0; kt < k_tiles; ++kt) {
-        const int buf = kt & 1;
-        const bool more = kt + 1 < k_tiles;
-        if (more) fetch(kt + 1);
-        uint4 av[UPT / 2][TM], bv[UPT / 2][TN];
+    auto body = [&](Operands &cur, Operands &nxt, int kt) {
+        const int nbuf = (kt + 1) & 1;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s = 0; s < UPT / 2; ++s) {
+        for (int st = 0; st < STEPS; ++st) {
+            const int blk = st / PARTS, part = st % PARTS;
+            const int s = blk / (TM * TN), a = (blk / TN) % TM, b = blk % TN;
+            Traits<DT>::mma_part(acc[a][b], cur.a[s][a], cur.b[s][b], part);
+            if (st == 0) {
+                stage(nbuf, kt + 1);
+                issue(kt + 2);
+            }
 #pragma unroll
-            for (int a = 0; a < TM; ++a) av[s][a] = lds[buf][(2 * s + lh) * BM + wm * (BM / WM) + a * 32 + li];
+            for (int i = 0; i < B_ITEMS; ++i)
+                if (STEPS > 1 ? (1 + (i * (STEPS - 1)) / B_ITEMS == st) : true) prep_item(kt + 3, i);
+            if (st >= HALF) {
 #pragma unroll
-            for (int b = 0; b < TN; ++b) bv[s][b] = lds[buf][A_SLOTS + (2 * s + lh) * BN + wn * (BN / WN) + b * 32 + li];
+                for (int i = 0; i < READS; ++i)
+                    if (HALF + (i * (STEPS - HALF)) / READS == st) read_operand(nxt, nbuf, i);
+            }
+            if (st == HALF - 1) __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int s = 0; s < UPT / 2; ++s)
-#pragma unroll
-            for (int a = 0; a < TM; ++a)
-#pragma unroll
-                for (int b = 0; b < TN; ++b) Traits<DT>::mma(acc[a][b], av[s][a], bv[s][b]);
-        if (more) stage(buf ^ 1, kt + 1);
-        __syncthreads();
+    };
+    int kt = 0;
+    for (; kt + 1 < k_tiles; kt += 2) {
+        body(op0, op1, kt);
+        body(op1, op0, kt + 1);
     }
+    if (kt < k_tiles) body(op0, op1, kt);
 
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
     if (p.partial) {

@@ -96,6 +96,7 @@ struct IgemmParams {
     // vector geometry (BL_KVEC)
     int units_per_tap;         // units per filter tap (Cp / 16 for NHWC int8); k_units for a plain matrix
     unsigned magic_upt, pass_upt;
+    int use_tapmask;           // kh*kw <= 64: per-lane tap validity is a 64-bit mask built once per tile
     int pix_stride;            // bytes between consecutive n ("pixels"): Cp, or ldb * elem
     // C
     void *C;
@@ -127,8 +128,6 @@ struct IgemmLaunch {
 };
 
 int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
-// chooses a tile for the problem; fills cfg.bm / cfg.bn / cfg.split
-void igemm_pick_tile(IgemmLaunch &cfg, const IgemmParams &p);
 
 // ---- other kernels -------------------------------------------------------------------------------------
 int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,

@@ -29,7 +29,7 @@ def plugin_path(op):
     return os.path.join(LIBDIR, f"lib{op}_hip.so")
 
 
-EXPORTS = ["onhip_init", "onhip_last_error", "onhip_conv_out_shape", "onhip_conv2d_f32",
+EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_matmul", "onhip_gemm_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
 
@@ -78,6 +78,11 @@ def _stream():
 
 def init(device=0):
     _check(load().onhip_init(device), "onhip_init")
+
+
+def set_tuning(mode):
+    """0: cost model; 1: time tile / split-K candidates on first use of each problem shape"""
+    return load().onhip_set_tuning(int(mode))
 
 
 def conv2d_f32(d, x, w, bias=None, silu_lut=None, out=None):
