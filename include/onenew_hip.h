@@ -98,6 +98,20 @@ int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow);
 int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,
                      const float *silu_lut, float *y, void *stream);
 
+/* Weights packed once at load time.  For dense convolutions other than unpadded 1x1 the kernel
+ * runs fastest on weights re-laid out tap-major, [cout][kh*kw][cin padded to the MFMA unit]: every
+ * group of input channels then shares one filter tap and the im2col arithmetic shrinks to one
+ * scalar description per group.  onhip_conv2d_packed_weight_bytes returns the size of that copy
+ * (0 when the convolution takes its weights as they are: 1x1 without padding, depthwise);
+ * onhip_conv2d_pack_weights writes it (device kernel on `stream`); onhip_conv2d_f32_packed is
+ * onhip_conv2d_f32 on such a copy.  Results of the two entry points agree to fp32 rounding (the
+ * summation order over K differs).  No counterpart in the reference, whose only weight
+ * re-layout is the offline int8 packing of tools/optimize/model_quant.hpp:14-25. */
+size_t onhip_conv2d_packed_weight_bytes(const onhip_conv_desc_t *d);
+int onhip_conv2d_pack_weights(const onhip_conv_desc_t *d, const float *w, float *packed, void *stream);
+int onhip_conv2d_f32_packed(const onhip_conv_desc_t *d, const float *x, const float *w_packed, const float *bias,
+                            const float *silu_lut, float *y, void *stream);
+
 /* Bytes of device scratch onhip_conv2d_w8a32 needs for `d` (the int8 copy of the activations). */
 size_t onhip_conv2d_w8a32_workspace(const onhip_conv_desc_t *d);
 

@@ -297,8 +297,33 @@ int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow) {
     return check_conv(d, oh, ow);
 }
 
-int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,
-                     const float *silu_lut, float *y, void *stream) {
+// channels per filter tap in the tap-major packed weight layout (padded to whole MFMA units)
+static int packed_cp(const onhip_conv_desc_t *d) {
+    const int kpu = d->compute == ONHIP_COMPUTE_F32 ? 4 : 8;
+    return (d->cin + kpu - 1) / kpu * kpu;
+}
+
+static bool wants_packed(const onhip_conv_desc_t *d) {
+    return d->group == 1 && !(d->kh == 1 && d->kw == 1 && !d->pad_t && !d->pad_l && !d->pad_b && !d->pad_r);
+}
+
+size_t onhip_conv2d_packed_weight_bytes(const onhip_conv_desc_t *d) {
+    if (!d || d->cin < 1 || d->cout < 1 || d->kh < 1 || d->kw < 1 || !wants_packed(d)) return 0;
+    return (size_t) d->cout * d->kh * d->kw * packed_cp(d) * sizeof(float);
+}
+
+int onhip_conv2d_pack_weights(const onhip_conv_desc_t *d, const float *w, float *packed, void *stream) {
+    int32_t OH, OW;
+    int rc = check_conv(d, &OH, &OW);
+    if (rc) return rc;
+    if (!w || !packed) return set_error(ONHIP_ERR_ARG, "conv pack: null pointer");
+    if (!wants_packed(d)) return set_error(ONHIP_ERR_ARG, "conv pack: this convolution takes its weights as they are");
+    return pack_wf32_launch(w, d->cout, d->cin, d->kh * d->kw, packed_cp(d), packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+// packed != 0: w holds the tap-major layout written by onhip_conv2d_pack_weights
+static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const float *w, int packed, const float *bias,
+                           const float *silu_lut, float *y, void *stream) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
@@ -306,6 +331,7 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
     if (d->has_bias && d->act_type == SILU && !silu_lut) return set_error(ONHIP_ERR_ARG, "conv: SILU needs the table");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const Epilogue ep = make_epilogue(*d, silu_lut);
+    if (packed && !wants_packed(d)) return set_error(ONHIP_ERR_ARG, "conv: this convolution has no packed weight form");
     if (d->group != 1) {
         if (d->compute != ONHIP_COMPUTE_F32)
             return set_error(ONHIP_ERR_ARG, "conv: depthwise runs in fp32 only");
@@ -315,31 +341,39 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
     memset(&cfg, 0, sizeof(cfg));
     rc = dtype_of_compute(d->compute, &cfg.dtype);
     if (rc) return rc;
-    cfg.bl = BL_GATHER;
     cfg.batch = 1;
     IgemmParams p;
     memset(&p, 0, sizeof(p));
+    const int kpu = kpu_of(cfg.dtype);
     p.M = d->cout;
     p.N = d->n * OH * OW;
-    p.K = d->cin * d->kh * d->kw;
-    if ((unsigned long long) p.K * (unsigned) (d->kh * d->kw) >= (1ULL << 32))
-        return set_error(ONHIP_ERR_ARG, "conv: reduction length %d too large", p.K);
-    const int kpu = kpu_of(cfg.dtype);
-    p.k_units = (p.K + kpu - 1) / kpu;
-    p.A = w;
-    p.lda = p.K;
-    p.B = x;
     p.H = d->h; p.W = d->w; p.OW = OW; p.OHW = OH * OW; p.HW = d->h * d->w;
     p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
     p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
     p.magic_khkw = magic_for(p.khkw); p.pass_khkw = pass_for(p.khkw);
     p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
     p.use_tapmask = p.khkw <= 64;
+    if (packed) {
+        // K = (tap, channel): every unit of KPU channels shares one filter tap
+        const int cp = packed_cp(d);
+        cfg.bl = BL_TAPC;
+        p.K = p.khkw * cp;
+        p.units_per_tap = cp / kpu;
+        p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
+    } else {
+        cfg.bl = wants_packed(d) ? BL_GATHER : BL_PLAIN;
+        p.K = d->cin * p.khkw;
+    }
+    if ((unsigned long long) p.K * (unsigned) p.khkw >= (1ULL << 32))
+        return set_error(ONHIP_ERR_ARG, "conv: reduction length %d too large", p.K);
+    p.k_units = (p.K + kpu - 1) / kpu;
+    p.A = w;
+    p.lda = p.K;
+    p.B = x;
     p.b_img_stride = (long long) d->cin * d->h * d->w;
-    if (p.khkw == 1 && !d->pad_t && !d->pad_l && !d->pad_b && !d->pad_r) cfg.bl = BL_PLAIN;
     p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * 4;
     p.a_slice_bytes = (long long) p.M * p.K * 4;
-    p.b_slice_bytes = (long long) d->n * p.b_img_stride * 4 + 2 * p.b_shift_bytes;
+    p.b_slice_bytes = (long long) d->n * p.b_img_stride * 4;
     p.c_slice_bytes = (long long) d->n * d->cout * OH * OW * 4;
     p.C = y;
     p.out_mode = OUT_CONV;
@@ -351,6 +385,16 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
     rc = plan_launch(cfg, p, st);
     if (rc) return rc;
     return igemm_launch(cfg, p, st);
+}
+
+int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,
+                     const float *silu_lut, float *y, void *stream) {
+    return conv2d_f32_impl(d, x, w, 0, bias, silu_lut, y, stream);
+}
+
+int onhip_conv2d_f32_packed(const onhip_conv_desc_t *d, const float *x, const float *w_packed, const float *bias,
+                            const float *silu_lut, float *y, void *stream) {
+    return conv2d_f32_impl(d, x, w_packed, 1, bias, silu_lut, y, stream);
 }
 
 static void w8a32_layout(const onhip_conv_desc_t *d, int *cp, int *k_units, size_t *packed_bytes, size_t *q_bytes) {
@@ -428,7 +472,7 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
     p.pix_stride = cp;
     p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * cp;
     p.a_slice_bytes = (long long) p.M * p.lda;
-    p.b_slice_bytes = (long long) d->n * d->h * d->w * cp + 2 * p.b_shift_bytes;
+    p.b_slice_bytes = (long long) d->n * d->h * d->w * cp;
     p.c_slice_bytes = (long long) d->n * d->cout * OH * OW * 4;
     p.C = y;
     p.out_mode = OUT_CONV;

@@ -145,6 +145,26 @@ int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, flo
     return ONHIP_OK;
 }
 
+// ---- fp32 weights [cout][cin][kh*kw] -> [cout][kh*kw][cp]: tap-major, channels zero-padded to cp -------
+__global__ __launch_bounds__(256) void pack_wf32_kernel(const float *w, int cin, int khkw, int cp, float *packed,
+                                                        long long total) {
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int c = (int) (idx % cp);
+    const long long t = idx / cp;
+    const int tap = (int) (t % khkw);
+    const long long oc = t / khkw;
+    packed[idx] = c < cin ? w[(oc * cin + c) * khkw + tap] : 0.0f;
+}
+
+int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream) {
+    const long long total = (long long) cout * khkw * cp;
+    const long long blocks = (total + 255) / 256;
+    hipLaunchKernelGGL(pack_wf32_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, w, cin, khkw, cp, packed, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
 // ---- int8 weights [cout][cin][kh][kw] -> [cout][k_units * 16], k = (tap * cp + channel), zero padded ---
 __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t *w8, int cin, int khkw, int cp, int row_bytes,
                                                       int8_t *packed, long long total) {

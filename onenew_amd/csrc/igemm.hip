@@ -18,7 +18,8 @@ int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t strea
     if (cfg.batch > 65535 || cfg.split > 65535) return set_error(ONHIP_ERR_ARG, "igemm: grid too large");
     if (cfg.split > 1 && !p.partial) return set_error(ONHIP_ERR_WORKSPACE, "igemm: split-K without workspace");
     // every byte offset a lane or a scalar register carries must stay below 2 GiB
-    if (p.a_slice_bytes >= (1LL << 31) || p.b_slice_bytes >= (1LL << 31) || p.c_slice_bytes >= (1LL << 31))
+    if (p.a_slice_bytes >= (1LL << 31) || p.b_slice_bytes + 2 * p.b_shift_bytes >= (1LL << 31) ||
+        p.c_slice_bytes >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "igemm: an operand slice of 2 GiB or more is not supported");
     switch (cfg.dtype) {
         case DT_F32: return igemm_launch_f32(cfg, p, stream);

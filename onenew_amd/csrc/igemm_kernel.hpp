@@ -241,11 +241,13 @@ __device__ __forceinline__ BPrep prep_b(const IgemmParams &p, int u, int e, int 
         r.bit = (int) k < klim ? (1u << (rem & 31u)) : 0u;
         r.hi = rem >> 5;
     } else {
+        // one description per unit: unit -> (tap, channel block), tap -> (i, j)
         const unsigned tap = fast_div((unsigned) u, p.magic_upt, p.pass_upt);
         const unsigned cb = (unsigned) u - tap * (unsigned) p.units_per_tap;
         const unsigned i = fast_div(tap, p.magic_kw, p.pass_kw);
         const unsigned j = tap - i * (unsigned) p.kw;
-        r.soff = (i * (unsigned) p.W + j) * (unsigned) p.pix_stride + cb * 16u;
+        if constexpr (BL == BL_TAPC) r.soff = (cb * (unsigned) KPU * (unsigned) p.HW + i * (unsigned) p.W + j) * 4u;
+        else r.soff = (i * (unsigned) p.W + j) * (unsigned) p.pix_stride + cb * 16u;
         r.bit = u * KPU < klim ? (1u << (tap & 31u)) : 0u;
         r.hi = tap >> 5;
     }
@@ -267,7 +269,7 @@ __device__ __forceinline__ unsigned b_voff(const IgemmParams &p, const ColState 
         if constexpr (BL == BL_GATHER) {
             const unsigned k = (unsigned) u_or_k;
             tap = k - fast_div(k, p.magic_khkw, p.pass_khkw) * (unsigned) p.khkw;
-        } else {
+        } else {   // unit index
             tap = fast_div((unsigned) u_or_k, p.magic_upt, p.pass_upt);
         }
         const unsigned i = fast_div(tap, p.magic_kw, p.pass_kw);
@@ -447,8 +449,9 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     const rsrc_t ra = make_rsrc(reinterpret_cast<const char *>(p.A) + (size_t) batch * p.a_batch_stride * ESZ,
                                 (unsigned) p.a_slice_bytes);
     // the B buffer starts pad rows/columns before the tensor so that pixel offsets are never negative
+    // and ends with the tensor: channel padding of the last image reads as zero
     const rsrc_t rb = make_rsrc(reinterpret_cast<const char *>(p.B) + (size_t) batch * p.b_batch_stride * ESZ -
-                                    (size_t) p.b_shift_bytes, RSRC_RANGE);
+                                    (size_t) p.b_shift_bytes, (unsigned) (p.b_slice_bytes + p.b_shift_bytes));
 
     // per-thread A slots: (row, unit-in-tile) fixed for the whole K loop
     unsigned a_voff[A_PER_T];
@@ -475,7 +478,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     RawUnit<DT> qa[A_PER_T], qb[B_PER_T];
 
     constexpr int PARTS = Traits<DT>::PARTS;
-    constexpr int BE = (BL == BL_KVEC) ? 1 : KPU;     // loads per B unit
+    constexpr int BE = (BL == BL_KVEC || BL == BL_TAPC) ? 1 : KPU;   // scalar descriptions per B unit
     constexpr int B_ITEMS = B_PER_T * BE;
     constexpr int BLOCKS = (UPT / 2) * TM * TN;       // 32x32 blocks x unit pairs per K tile
     constexpr int STEPS = BLOCKS * PARTS;             // MFMA instructions per K tile and wavefront
@@ -484,6 +487,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     struct Operands { uint4 a[UPT / 2][TM], b[UPT / 2][TN]; };
 
     BPrep bp[B_ITEMS];                                // scalar descriptions of the next B loads
+    const unsigned hw4 = (unsigned) p.HW * 4u;
 
     auto b_unit_of = [&](int t) { return __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN); };
     auto prep_item = [&](int kt, int idx) {
@@ -506,6 +510,11 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
                     qb[t].v[0] = __uint_as_float(q.x); qb[t].v[1] = __uint_as_float(q.y);
                     qb[t].v[2] = __uint_as_float(q.z); qb[t].v[3] = __uint_as_float(q.w);
                 }
+            } else if constexpr (BL == BL_TAPC) {
+                // the unit's KPU channels share the filter tap: one validity test, channel stride in the scalar offset
+                const unsigned voff = b_voff<BL>(p, col, bp[t], u);
+#pragma unroll
+                for (int e = 0; e < KPU; ++e) qb[t].v[e] = buf_load_f32(rb, voff, bp[t].soff + (unsigned) e * hw4);
             } else {
 #pragma unroll
                 for (int e = 0; e < KPU; ++e)

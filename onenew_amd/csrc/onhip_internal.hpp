@@ -67,7 +67,8 @@ __device__ __forceinline__ float apply_act(float v, const Epilogue &e) {
 
 enum { BL_GATHER = 0,  // element gather from NCHW activations (implicit im2col), any filter / stride / padding
        BL_KVEC = 1,    // 16-byte vectors along K from NHWC int8 activations
-       BL_PLAIN = 2 }; // 1x1 filter without padding, or a row-major [K, N] matrix: no tap arithmetic
+       BL_PLAIN = 2,   // 1x1 filter without padding, or a row-major [K, N] matrix: no tap arithmetic
+       BL_TAPC = 3 };  // NCHW activations against tap-major packed weights: K = (tap, channel), one tap per unit
 
 enum { OUT_CONV = 0,   // n = img * OHW + pix  ->  img * c_img_stride + m * c_stride_m + pix
        OUT_PLAIN = 1 };// m * c_stride_m + n * c_stride_n
@@ -137,6 +138,7 @@ int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const flo
                            int32_t *acc32, hipStream_t stream);
 int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
                          hipStream_t stream);
+int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
 int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, int k_units, int8_t *packed,
                    hipStream_t stream);
 int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,

@@ -30,6 +30,7 @@ def plugin_path(op):
 
 
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
+           "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_matmul", "onhip_gemm_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
 
@@ -47,6 +48,10 @@ def load():
     L.onhip_last_error.restype = C.c_char_p
     L.onhip_conv_out_shape.argtypes = [C.POINTER(ConvDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     L.onhip_conv2d_f32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp]
+    L.onhip_conv2d_packed_weight_bytes.argtypes = [C.POINTER(ConvDesc)]
+    L.onhip_conv2d_packed_weight_bytes.restype = C.c_size_t
+    L.onhip_conv2d_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    L.onhip_conv2d_f32_packed.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_conv2d_w8a32_workspace.argtypes = [C.POINTER(ConvDesc)]
     L.onhip_conv2d_w8a32_workspace.restype = C.c_size_t
     L.onhip_conv2d_w8a32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
@@ -85,15 +90,27 @@ def set_tuning(mode):
     return load().onhip_set_tuning(int(mode))
 
 
-def conv2d_f32(d, x, w, bias=None, silu_lut=None, out=None):
-    """fused Conv2d (+bias, +activation); returns the fp32 NCHW output tensor"""
+def conv2d_f32(d, x, w, bias=None, silu_lut=None, out=None, packed=False):
+    """fused Conv2d (+bias, +activation); returns the fp32 NCHW output tensor.  packed=True: `w` is
+    the result of pack_conv_weights"""
     import torch
     oh, ow = d.out_hw()
     if out is None:
         out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device=x.device)
-    _check(load().onhip_conv2d_f32(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(silu_lut), _ptr(out), _stream()),
-           "onhip_conv2d_f32")
+    fn = load().onhip_conv2d_f32_packed if packed else load().onhip_conv2d_f32
+    _check(fn(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(silu_lut), _ptr(out), _stream()), "onhip_conv2d_f32")
     return out
+
+
+def pack_conv_weights(d, w):
+    """tap-major copy of the weights for conv2d_f32(..., packed=True); None if the layer takes them as they are"""
+    import torch
+    nbytes = int(load().onhip_conv2d_packed_weight_bytes(C.byref(d)))
+    if nbytes == 0:
+        return None
+    packed = torch.empty(nbytes // 4, dtype=torch.float32, device=w.device)
+    _check(load().onhip_conv2d_pack_weights(C.byref(d), _ptr(w), _ptr(packed), _stream()), "onhip_conv2d_pack_weights")
+    return packed
 
 
 def conv2d_w8a32_workspace(d):

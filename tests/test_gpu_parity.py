@@ -79,6 +79,41 @@ def test_conv_f32(name, torch_dev, oracle, golden):
     cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * scale)
 
 
+PACKED_CASES = [n for n, d in cases.conv_f32_cases().items()
+                if d.group == 1 and not (d.kh == 1 and d.kw == 1 and d.pad_t == 0)]
+
+
+@pytest.mark.parametrize("name", PACKED_CASES)
+def test_conv_f32_packed_weights(name, torch_dev, oracle):
+    """tap-major packed weights: same convolution, the reduction merely runs in another order"""
+    torch = torch_dev
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    wd = dev(torch, w)
+    wp = hip.pack_conv_weights(d, wd)
+    assert wp is not None
+    dn = ConvDesc.from_buffer_copy(d)
+    if d.has_bias and d.act_type == abi.SILU:
+        dn.act_type = abi.NOT_ACT      # judged on the pre-activation; the table lookup is tested elsewhere
+    y = hip.conv2d_f32(dn, dev(torch, x), wp, dev(torch, b), None, packed=True)
+    torch.cuda.synchronize()
+    assert_close_f32(y.cpu().numpy(), oracle.conv2d_f32(dn, x, w, b), tag=name + " packed")
+
+
+@pytest.mark.parametrize("compute", [abi.COMPUTE_BF16, abi.COMPUTE_F16])
+def test_conv_packed_reduced_precision(compute, torch_dev, oracle):
+    torch = torch_dev
+    for name in ("cfg1_64x56_3x3", "c7x7_s2_p3"):
+        d = ConvDesc.from_buffer_copy(cases.conv_f32_cases()[name])
+        d.compute = compute
+        x, w, b = cases.conv_inputs(name, d)
+        wp = hip.pack_conv_weights(d, dev(torch, w))
+        y = hip.conv2d_f32(d, dev(torch, x), wp, dev(torch, b), None, packed=True)
+        torch.cuda.synchronize()
+        rnd = oracle.round_bf16 if compute == abi.COMPUTE_BF16 else oracle.round_f16
+        assert_close_f32(y.cpu().numpy(), oracle.conv2d_f32(d, rnd(x), rnd(w), b), rel=1e-4, tag=name + " packed")
+
+
 @pytest.mark.parametrize("name", list(cases.conv_w8a32_cases()))
 def test_conv_w8a32_bit_exact(name, torch_dev, oracle, golden):
     torch = torch_dev
@@ -285,7 +320,11 @@ def test_resnet50_layers_batch32_sampled_f64(layer, torch_dev):
     from onenew_amd import stacks
     name, d = stacks.with_batch(stacks.resnet50(), 32)[layer]
     x, w, b = cases.conv_inputs("rn50b32_" + name, d)
-    y = hip.conv2d_f32(d, dev(torch, x), dev(torch, w), dev(torch, b))
+    wp = hip.pack_conv_weights(d, dev(torch, w))
+    if wp is not None:
+        y = hip.conv2d_f32(d, dev(torch, x), wp, dev(torch, b), packed=True)
+    else:
+        y = hip.conv2d_f32(d, dev(torch, x), dev(torch, w), dev(torch, b))
     torch.cuda.synchronize()
     y = y.cpu().numpy().reshape(-1)
     idx = cases.datagen.integers(cases.datagen.seed_for(name, "probe"), (1500,), 0, y.size - 1)
