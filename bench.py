@@ -64,6 +64,16 @@ class DeviceLayer:
             hip.conv2d_f32(self.d, self.x, self.w, self.b, None, out=self.y)
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel from the committed counter summary
+    (profiles/<workload>_traffic.json: FETCH_SIZE / WRITE_SIZE scaled by the copy yardstick), else None"""
+    path = os.path.join(ROOT, "profiles", f"{workload}_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get("hbm_bytes_per_launch")
+
+
 def time_layers(torch, hip, layers, reps):
     """average launch duration of every layer, HIP events on the launch stream"""
     out = []
@@ -129,6 +139,7 @@ def main():
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-tune", action="store_true", help="use the cost model instead of measured tile choice")
+    ap.add_argument("--no-batch1", action="store_true", help="skip the extra batch-1 pass over the same stack")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path runs on a single MI355X and nothing in this build "
@@ -140,6 +151,17 @@ def main():
     hip.init(0)
     # tile / split-K per layer shape is measured on first use (during the warm-up steps) and cached
     hip.set_tuning(0 if args.no_tune else 1)
+
+    if args.workload == "copy":
+        # yardstick for the HBM traffic counters: a plain device copy of known size (1 GiB read + 1 GiB written)
+        src = torch.rand(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            hip.copy_f32(src, dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "copy", "bytes_read_per_launch": src.numel() * 4,
+                          "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
+        return
 
     desc, dtype, layer_descs = make_workload(args.workload)
     layers = [DeviceLayer(torch, n, d, args.workload) for n, d in layer_descs]
@@ -167,12 +189,12 @@ def main():
     achieved = dense_flops / (dense_ms * 1e-3) / 1e12
     roofline = {"kernel": "onhip::igemm_kernel (fp32 MFMA implicit GEMM)", "bound": "mfma",
                 "achieved": round(achieved, 3), "peak": PEAK[dtype], "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK[dtype], 4), "traffic": None,
+                "frac": round(achieved / PEAK[dtype], 4), "traffic": measured_traffic(args.workload),
                 "launches": len(dense), "avg_launch_ms": round(dense_ms / len(dense), 5),
                 "flops_per_launch": dense_flops / len(dense)}
 
     extra = {}
-    if args.workload.startswith("resnet50_b") and args.workload != "resnet50_b1":
+    if args.workload.startswith("resnet50_b") and args.workload != "resnet50_b1" and not args.no_batch1:
         # the same stack at batch 1 (the "conv stack ms" of the reference's recorded trace)
         _, _, l1 = make_workload("resnet50_b1")
         layers1 = [DeviceLayer(torch, n, d, "resnet50_b1") for n, d in l1]

@@ -135,6 +135,11 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
 int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w,
                    const float *bias, float *out, void *stream);
 
+/* Plain device-to-device copy of n floats (n % 4 == 0, 16-byte aligned).  A measuring aid with no
+ * counterpart in the reference: HBM traffic counters of the other kernels are scaled by what the
+ * same counters read for this copy of known size. */
+int onhip_copy_f32(const float *src, float *dst, long long n, void *stream);
+
 /* ---- plugin level: the reference slot arrays; host or device pointers; synchronous --------- */
 
 int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);

@@ -116,6 +116,43 @@ static int tune_mode() {
     return g_tune_mode;
 }
 
+// Optional persistence of measured choices: ONHIP_TUNE_CACHE names a text file, one line per problem
+// signature ("v0 v1 ... v13 : bm bn split"), read once and appended to after every measurement.
+static bool g_cache_loaded = false;
+static void load_tune_cache_locked() {
+    if (g_cache_loaded) return;
+    g_cache_loaded = true;
+    const char *path = getenv("ONHIP_TUNE_CACHE");
+    if (!path) return;
+    FILE *f = fopen(path, "r");
+    if (!f) return;
+    char line[512];
+    while (fgets(line, sizeof(line), f)) {
+        std::vector<long long> key;
+        char *s = line, *end = nullptr;
+        for (;;) {
+            while (*s == ' ') ++s;
+            if (*s == ':' || *s == 0 || *s == '\n') break;
+            const long long v = strtoll(s, &end, 10);
+            if (end == s) break;
+            key.push_back(v);
+            s = end;
+        }
+        Choice c;
+        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d", &c.bm, &c.bn, &c.split) == 3) g_tuned[key] = c;
+    }
+    fclose(f);
+}
+static void append_tune_cache_locked(const std::vector<long long> &key, const Choice &c) {
+    const char *path = getenv("ONHIP_TUNE_CACHE");
+    if (!path) return;
+    FILE *f = fopen(path, "a");
+    if (!f) return;
+    for (long long v : key) fprintf(f, "%lld ", v);
+    fprintf(f, ": %d %d %d\n", c.bm, c.bn, c.split);
+    fclose(f);
+}
+
 static int mfma_k_per_unit(int dt) { return dt == DT_F32 ? 4 : dt == DT_I8 ? 16 : 8; }
 
 // cycles one CU needs for the MFMAs of one K tile of a BM x BN workgroup
@@ -219,6 +256,7 @@ static int plan_launch(IgemmLaunch &cfg, IgemmParams &p, hipStream_t st) {
                                   p.H, p.W, p.out_mode, p.lda};
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
+        load_tune_cache_locked();
         auto it = g_tuned.find(key);
         if (it != g_tuned.end()) return apply_choice(cfg, p, it->second);
     }
@@ -252,6 +290,7 @@ static int plan_launch(IgemmLaunch &cfg, IgemmParams &p, hipStream_t st) {
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
         g_tuned[key] = best;
+        append_tune_cache_locked(key, best);
     }
     return apply_choice(cfg, p, best);
 }
@@ -535,6 +574,11 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     rc = plan_launch(cfg, p, st);
     if (rc) return rc;
     return igemm_launch(cfg, p, st);
+}
+
+int onhip_copy_f32(const float *src, float *dst, long long n, void *stream) {
+    if (!src || !dst || n < 0) return set_error(ONHIP_ERR_ARG, "copy: bad argument");
+    return copy_f32_launch(src, dst, n, reinterpret_cast<hipStream_t>(stream));
 }
 
 int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w, const float *bias, float *out,

@@ -240,3 +240,22 @@ int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const fl
 }
 
 }  // namespace onhip
+
+namespace onhip {
+
+// ---- plain device copy: the yardstick that HBM traffic counters are scaled by ------------------------
+__global__ __launch_bounds__(256) void copy_f32_kernel(const float4 *src, float4 *dst, long long n4) {
+    const long long stride = (long long) gridDim.x * blockDim.x;
+    for (long long i = (long long) blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
+}
+
+int copy_f32_launch(const float *src, float *dst, long long n, hipStream_t stream) {
+    if (n % 4 || (reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % 16)
+        return set_error(ONHIP_ERR_ARG, "copy: element count must be a multiple of 4 and pointers 16-byte aligned");
+    hipLaunchKernelGGL(copy_f32_kernel, dim3(256 * 8), dim3(256), 0, stream, reinterpret_cast<const float4 *>(src),
+                       reinterpret_cast<float4 *>(dst), n / 4);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+}  // namespace onhip

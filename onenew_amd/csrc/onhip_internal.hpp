@@ -143,5 +143,6 @@ int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, 
                    hipStream_t stream);
 int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,
                    hipStream_t stream);
+int copy_f32_launch(const float *src, float *dst, long long n, hipStream_t stream);
 
 }  // namespace onhip

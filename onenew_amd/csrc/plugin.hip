@@ -55,6 +55,39 @@ static uint64_t fingerprint(const void *host, size_t bytes) {
     return h;
 }
 
+// tap-major copies of k x k convolution weights, keyed by the device address of the original
+struct PackedEntry {
+    float *dev;
+    size_t bytes;
+};
+static std::map<const void *, PackedEntry> g_packed;
+
+static void drop_packed(const void *w_dev) {
+    auto it = g_packed.find(w_dev);
+    if (it == g_packed.end()) return;
+    (void) hipFree(it->second.dev);
+    g_packed.erase(it);
+}
+
+// *out = packed copy of the device weights w_dev for convolution d, or nullptr if d takes them as they are.
+// A weight that lives in device memory is packed when first seen; after changing it in place call
+// onhip_plugin_release().
+static int packed_weights(const onhip_conv_desc_t *d, const float *w_dev, const float **out) {
+    *out = nullptr;
+    const size_t bytes = onhip_conv2d_packed_weight_bytes(d);
+    if (!bytes) return ONHIP_OK;
+    auto it = g_packed.find(w_dev);
+    if (it != g_packed.end() && it->second.bytes == bytes) { *out = it->second.dev; return ONHIP_OK; }
+    drop_packed(w_dev);
+    float *p = nullptr;
+    ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&p), bytes));
+    int rc = onhip_conv2d_pack_weights(d, w_dev, p, nullptr);
+    if (rc) { (void) hipFree(p); return rc; }
+    g_packed[w_dev] = PackedEntry{p, bytes};
+    *out = p;
+    return ONHIP_OK;
+}
+
 static int ensure_ready() {
     if (g_ready) return ONHIP_OK;
     int dev = 0;
@@ -111,6 +144,7 @@ static int const_on_device(const void *host, size_t bytes, const void **dev) {
         if (it->second.fingerprint != fp) {
             ONHIP_CHECK_HIP(hipMemcpy(it->second.dev, host, bytes, hipMemcpyHostToDevice));
             it->second.fingerprint = fp;
+            drop_packed(it->second.dev);   // a packed copy of the old content is stale
         }
         *dev = it->second.dev;
         return ONHIP_OK;
@@ -208,8 +242,16 @@ static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
         rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
                                 (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
     } else {
-        rc = onhip_conv2d_f32(&d, (const float *) x, (const float *) w, (const float *) b, (const float *) lut,
-                              (float *) y, nullptr);
+        // k x k dense weights are re-laid out tap-major once, next to their device copy
+        const float *wp = nullptr;
+        rc = packed_weights(&d, (const float *) w, &wp);
+        if (rc) return rc;
+        if (wp)
+            rc = onhip_conv2d_f32_packed(&d, (const float *) x, wp, (const float *) b, (const float *) lut, (float *) y,
+                                         nullptr);
+        else
+            rc = onhip_conv2d_f32(&d, (const float *) x, (const float *) w, (const float *) b, (const float *) lut,
+                                  (float *) y, nullptr);
     }
     if (rc) return rc;
     if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, out_bytes, hipMemcpyDeviceToHost));
@@ -328,6 +370,8 @@ int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S 
 int onhip_plugin_release(void) {
     std::lock_guard<std::mutex> lock(g_mu);
     ONHIP_CHECK_HIP(hipDeviceSynchronize());
+    for (auto &kv : g_packed) (void) hipFree(kv.second.dev);
+    g_packed.clear();
     for (auto &kv : g_const) (void) hipFree(kv.second.dev);
     g_const.clear();
     for (auto &b : g_stage) {

@@ -31,7 +31,7 @@ def plugin_path(op):
 
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
-           "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_matmul", "onhip_gemm_f32",
+           "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
 
 
@@ -57,6 +57,7 @@ def load():
     L.onhip_conv2d_w8a32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
+    L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
     _lib = L
@@ -156,3 +157,9 @@ def gemm_f32(a, w, bias, out=None):
         out = torch.empty((M, N), dtype=torch.float32, device=a.device)
     _check(load().onhip_gemm_f32(M, K, N, _ptr(a), _ptr(w), _ptr(bias), _ptr(out), _stream()), "onhip_gemm_f32")
     return out
+
+
+def copy_f32(src, dst):
+    """plain device copy (the yardstick for HBM traffic counters)"""
+    _check(load().onhip_copy_f32(_ptr(src), _ptr(dst), src.numel(), _stream()), "onhip_copy_f32")
+    return dst
