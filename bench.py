@@ -3,12 +3,16 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
-A step is one pass over every layer of the workload: one launch per layer, inputs, weights and
-outputs resident in HBM, synthetic seeded data (x ~ U(-1,1), He-normal weights, bias N(0, 0.01)).
-Prints ONE JSON line: whole-stack throughput (`value`, TFLOP/s with 2 FLOP per multiply-accumulate,
-bias and activation not counted), the roofline position of the dominant kernel measured with HIP
-events on the launch stream, and the CPU baseline (the reference's own x86 kernels when their
-build is present, else the CPU restatement) timed on this machine's host cores.
+Workloads (BASELINE configurations): resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
+cfg1, mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
+the HBM traffic counters are scaled by).
+
+A step is one pass over every layer of the workload: one launch per layer, inputs, weights and outputs
+resident in HBM, synthetic seeded data.  Prints ONE JSON line: whole-stack throughput (`value`, TFLOP/s
+or TOP/s with 2 operations per multiply-accumulate; bias, activation and (de)quantisation not counted),
+the roofline position of the dominant kernel measured with HIP events on the launch stream, and the CPU
+baseline (the reference's own x86 kernels when their build is present, else the CPU restatement) timed on
+this machine's host cores.
 """
 import argparse
 import json
@@ -26,42 +30,159 @@ PEAK = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0, "i8": 5000.0}   # dense MFM
 HBM_PEAK_GBS = 8000.0
 
 
-def make_workload(name):
-    """-> (description, dtype, [(layer name, ConvDesc)])"""
-    from onenew_amd import stacks
-    if name.startswith("resnet50_b"):
-        n = int(name.split("_b")[1])
-        return f"ResNet-50 conv stack fp32, batch {n}, 224x224, 53 conv layers, fused ReLU", "f32", \
-            stacks.with_batch(stacks.resnet50(), n)
-    if name.startswith("mobilenetv2_b"):
-        n = int(name.split("_b")[1])
-        return f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers", "f32", \
-            stacks.with_batch(stacks.mobilenet_v2(), n)
-    if name == "cfg1":
+# ---- layers: device-resident operands + one launch -------------------------------------------------------
+
+class ConvF32Layer:
+    kind = "conv_f32"
+
+    def __init__(self, torch, hip, name, d, tag):
         import cases
-        return "Conv2d+ReLU fp32 64->64 56x56 3x3 s1 p1, batch 1", "f32", [("cfg1", cases.conv_f32_cases()["cfg1_64x56_3x3"])]
-    raise SystemExit(f"unknown workload {name}")
-
-
-class DeviceLayer:
-    """device-resident operands of one layer"""
-
-    def __init__(self, torch, name, d, seed_tag):
-        import cases
-        x, w, b = cases.conv_inputs(f"{seed_tag}/{name}", d)
+        x, w, b = cases.conv_inputs(f"{tag}/{name}", d)
         self.name, self.d = name, d
         self.x, self.w, self.b = (torch.from_numpy(t).cuda() for t in (x, w, b))
-        oh, ow = d.out_hw()
-        self.y = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device="cuda")
-        # weights are re-laid out once at load time (tap-major), as an inference runtime would
-        from onenew_amd import hip
+        self.y = torch.empty((d.n, d.cout) + d.out_hw(), dtype=torch.float32, device="cuda")
+        # k x k weights are re-laid out once at load time (tap-major), as an inference runtime would
         self.wp = hip.pack_conv_weights(d, self.w)
+        self.flops, self.bytes = d.flops(), d.algorithmic_bytes()
+        self.dense = d.group == 1
+        oh, ow = d.out_hw()
+        self.shape = f"M={d.cout} N={d.n * oh * ow} K={d.k_per_out()}"
 
     def launch(self, hip):
         if self.wp is not None:
             hip.conv2d_f32(self.d, self.x, self.wp, self.b, None, out=self.y, packed=True)
         else:
             hip.conv2d_f32(self.d, self.x, self.w, self.b, None, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        import cases
+        from onenew_amd import abi
+        d1 = abi.ConvDesc.from_buffer_copy(self.d)
+        d1.n = 1
+        x, w, b = cases.conv_inputs(f"{tag}/cpu/{self.name}", d1)
+        if oracle.have_ref():
+            op = ops.Conv(ops.Plugin(oracle.ref_path("Conv")).eval, d1, w, b, silu_lut=cases.silu_lut(),
+                          scratch_bytes=oracle.ref_scratch_bytes(d1))
+            xin = ops.aligned_empty(x.shape)
+            xin[...] = x
+            out = ops.aligned_empty((1, d1.cout) + d1.out_hw())
+            return d1.flops(), lambda: op(xin, out=out)
+        return d1.flops(), lambda: oracle.conv2d_f32(d1, x, w, b, cases.silu_lut())
+
+
+class ConvW8A32Layer:
+    kind = "conv_w8a32"
+
+    def __init__(self, torch, hip, name, d, tag):
+        import cases
+        x, w8, b32, aux = cases.conv_inputs(f"{tag}/{name}", d, quant=True)
+        self.name, self.d = name, d
+        self.x, self.w8, self.b32, self.aux = (torch.from_numpy(t).cuda() for t in (x, w8, b32, aux))
+        self.lut = torch.from_numpy(cases.silu_lut()).cuda()
+        self.y = torch.empty((d.n, d.cout) + d.out_hw(), dtype=torch.float32, device="cuda")
+        self.ws = torch.empty(max(16, hip.conv2d_w8a32_workspace(d)), dtype=torch.uint8, device="cuda")
+        self.flops, self.bytes = d.flops(), d.algorithmic_bytes(eb_x=4, eb_w=1, eb_y=4)
+        self.dense = d.group == 1
+        oh, ow = d.out_hw()
+        self.shape = f"M={d.cout} N={d.n * oh * ow} K={d.k_per_out()}"
+
+    def launch(self, hip):
+        hip.conv2d_w8a32(self.d, self.x, self.w8, self.b32, self.aux, self.lut, out=self.y, workspace=self.ws)
+
+    def cpu_runner(self, ops, oracle, tag):
+        import cases
+        from onenew_amd import abi
+        d1 = abi.ConvDesc.from_buffer_copy(self.d)
+        d1.n = 1
+        x, w8, b32, aux = cases.conv_inputs(f"{tag}/cpu/{self.name}", d1, quant=True)
+        if oracle.have_ref():
+            op = ops.Conv(ops.Plugin(oracle.ref_path("Conv")).eval, d1, w8, b32, weight_aux=aux, silu_lut=cases.silu_lut(),
+                          scratch_bytes=oracle.ref_scratch_bytes(d1))
+            xin = ops.aligned_empty(x.shape)
+            xin[...] = x
+            out = ops.aligned_empty((1, d1.cout) + d1.out_hw())
+            return d1.flops(), lambda: op(xin, out=out)
+        return d1.flops(), lambda: oracle.conv2d_w8a32(d1, x, w8, b32, aux, cases.silu_lut())
+
+
+class MatmulLayer:
+    kind = "matmul"
+
+    def __init__(self, torch, hip, name, md, has_bias, gelu, compute, tag):
+        import cases
+        from onenew_amd import datagen
+        self.name, self.md, self.compute = name, md, compute
+        ashape = (md.batch, md.m, md.k)
+        bshape = (md.k, md.n) if md.b_shared else (md.batch, md.k, md.n)
+        a = datagen.normal(datagen.seed_for(tag, name, "a"), ashape, 0.0, 1.0)
+        b = datagen.normal(datagen.seed_for(tag, name, "b"), bshape, 0.0, 0.02)
+        self.host = (a, b)
+        self.a, self.b = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+        self.bias = torch.from_numpy(datagen.normal(datagen.seed_for(tag, name, "bias"), (md.n,), 0.0, 0.02)).cuda() \
+            if has_bias else None
+        self.lut = torch.from_numpy(cases.gelu_lut()).cuda() if gelu else None
+        self.y = torch.empty((md.batch, md.m, md.n), dtype=torch.float32, device="cuda")
+        self.flops, self.bytes = md.flops(), md.algorithmic_bytes(bias=has_bias)
+        self.dense = True
+        self.shape = f"B={md.batch} M={md.m} N={md.n} K={md.k}"
+
+    def launch(self, hip):
+        hip.matmul(self.a, self.b, bias=self.bias, gelu_lut=self.lut, compute=self.compute, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        # reference semantics: MatMul (+ Add + Gelu as separate sweeps); one image's worth of the batch
+        md = self.md
+        per_image = md.batch if md.b_shared else md.batch      # the ViT batch is already folded into `batch`
+        a, b = self.host
+        flops = md.flops()
+        if oracle.have_ref():
+            mm = ops.MatMul(ops.Plugin(oracle.ref_path("MatMul")).eval)
+            aa, bb = ops.aligned_empty(a.shape), ops.aligned_empty(b.shape)
+            aa[...], bb[...] = a, b
+            out = ops.aligned_empty(a.shape[:-1] + (md.n,))
+            return flops, lambda: mm(aa, bb, out=out)
+        return flops, lambda: oracle.matmul_f32(a, b)
+
+
+def make_workload(torch, hip, name):
+    """-> (description, dtype, [layers])"""
+    from onenew_amd import abi, stacks, datagen
+    tag = name
+
+    def conv_stack(layers):
+        return [ConvF32Layer(torch, hip, n, d, tag) for n, d in layers]
+
+    if name.startswith("resnet50_b"):
+        n = int(name.split("_b")[1])
+        return (f"ResNet-50 conv stack fp32, batch {n}, 224x224, 53 conv layers, fused ReLU", "f32",
+                conv_stack(stacks.with_batch(stacks.resnet50(), n)))
+    if name.startswith("mobilenetv2_b"):
+        n = int(name.split("_b")[1])
+        return (f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers (17 depthwise), ReLU6 as CLIP", "f32",
+                conv_stack(stacks.with_batch(stacks.mobilenet_v2(), n)))
+    if name == "cfg1":
+        import cases
+        return ("Conv2d+ReLU fp32 64->64 56x56 3x3 s1 p1, batch 1", "f32",
+                conv_stack([("cfg1", cases.conv_f32_cases()["cfg1_64x56_3x3"])]))
+    if name.startswith("yolov8s_int8_b"):
+        n = int(name.split("_b")[1])
+        layers = []
+        for i, (lname, d) in enumerate(stacks.with_batch(stacks.yolov8s(), n)):
+            d.input_scale = float(datagen.uniform(datagen.seed_for(tag, i, "s_in"), (1,), 0.005, 0.05)[0])
+            layers.append(ConvW8A32Layer(torch, hip, lname, d, tag))
+        return (f"YOLOv8s conv stack W8A32 int8, batch {n}, 640x640, 63 conv layers, SiLU table, fp32 in/out", "i8", layers)
+    if name.startswith("vit_tiny_b"):
+        rest = name[len("vit_tiny_b"):]
+        compute, dtype = abi.COMPUTE_F32, "f32"
+        if rest.endswith("_bf16"):
+            compute, dtype, rest = abi.COMPUTE_BF16, "bf16", rest[:-5]
+        elif rest.endswith("_f16"):
+            compute, dtype, rest = abi.COMPUTE_F16, "f16", rest[:-4]
+        n = int(rest)
+        layers = [MatmulLayer(torch, hip, ln, md, hb, g, compute, tag) for ln, md, hb, g in stacks.vit_tiny(n)]
+        return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads; fc1 with fused bias + table GELU",
+                dtype, layers)
+    raise SystemExit(f"unknown workload {name}")
 
 
 def measured_traffic(workload):
@@ -90,30 +211,16 @@ def time_layers(torch, hip, layers, reps):
     return out
 
 
-def cpu_baseline(layer_descs, seed_tag, budget_s=20.0):
-    """the reference's x86 kernels (or the CPU restatement) on a bounded sample: batch-1 passes over the
-    same layer shapes, 8 threads as the reference builds by default"""
-    import cases
-    from onenew_amd import abi, ops
+def cpu_baseline(layers, tag, unit, budget_s=20.0):
+    """the reference's x86 kernels (or the CPU restatement) on a bounded sample: passes over the same layer
+    shapes at batch 1 (the reference evaluates one image per call), 8 threads as the reference builds"""
+    from onenew_amd import ops
     from oracle import oracle
     threads = 8
     os.environ.setdefault("OMP_NUM_THREADS", str(threads))
-    use_ref = oracle.have_ref()
     oracle.set_threads(threads)
-    runs = []
-    for name, d in layer_descs:
-        d1 = abi.ConvDesc.from_buffer_copy(d)
-        d1.n = 1
-        x, w, b = cases.conv_inputs(f"{seed_tag}/cpu/{name}", d1)
-        if use_ref:
-            op = ops.Conv(ops.Plugin(oracle.ref_path("Conv")).eval, d1, w, b, scratch_bytes=oracle.ref_scratch_bytes(d1))
-            xin = ops.aligned_empty(x.shape)
-            xin[...] = x
-            out = ops.aligned_empty((1, d1.cout) + d1.out_hw())
-            runs.append((d1, lambda op=op, xin=xin, out=out: op(xin, out=out)))
-        else:
-            runs.append((d1, lambda d1=d1, x=x, w=w, b=b: oracle.conv2d_f32(d1, x, w, b)))
-    flops = sum(d1.flops() for d1, _ in runs)
+    runs = [L.cpu_runner(ops, oracle, tag) for L in layers]
+    flops = sum(f for f, _ in runs)
     for _, f in runs:
         f()                      # warm-up pass
     times = []
@@ -124,9 +231,10 @@ def cpu_baseline(layer_descs, seed_tag, budget_s=20.0):
             f()
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
-    return {"value": round(flops / med / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
-            "kind": "reference" if use_ref else "port",
-            "sample": f"{len(times)} batch-1 passes over the {len(runs)} layer shapes, median; {med * 1e3:.1f} ms per pass",
+    return {"value": round(flops / med / 1e12, 5), "unit": unit, "cores": threads,
+            "kind": "reference" if oracle.have_ref() else "port",
+            "sample": f"{len(times)} passes over the {len(runs)} layer shapes, one image per call, median; "
+                      f"{med * 1e3:.1f} ms per pass",
             "ms_per_pass": round(med * 1e3, 2), "host_cpus": os.cpu_count()}
 
 
@@ -163,10 +271,10 @@ def main():
                           "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
         return
 
-    desc, dtype, layer_descs = make_workload(args.workload)
-    layers = [DeviceLayer(torch, n, d, args.workload) for n, d in layer_descs]
-    flops = sum(L.d.flops() for L in layers)
-    abytes = sum(L.d.algorithmic_bytes() for L in layers)
+    desc, dtype, layers = make_workload(torch, hip, args.workload)
+    unit = "TOP/s" if dtype == "i8" else "TFLOP/s"
+    flops = sum(L.flops for L in layers)
+    abytes = sum(L.bytes for L in layers)
 
     for _ in range(args.warmup):
         for L in layers:
@@ -180,48 +288,62 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
-    # roofline of the dominant kernel (the implicit-GEMM MFMA kernel runs every dense layer):
-    # algorithmic FLOPs of its launches / their average durations, from events on the launch stream
+    # Roofline of the dominant kernel.  Dense layers all run onhip::igemm_kernel (MFMA-bound); depthwise layers run
+    # onhip::depthwise_*_kernel (HBM-bound).  Whichever group takes more time is reported: algorithmic work of its
+    # launches / their average durations, from events on the launch stream.
     per_layer_ms = time_layers(torch, hip, layers, reps=max(10, args.steps))
-    dense = [(L, t) for L, t in zip(layers, per_layer_ms) if L.d.group == 1]
-    dense_flops = sum(L.d.flops() for L, _ in dense)
-    dense_ms = sum(t for _, t in dense)
-    achieved = dense_flops / (dense_ms * 1e-3) / 1e12
-    roofline = {"kernel": "onhip::igemm_kernel (fp32 MFMA implicit GEMM)", "bound": "mfma",
-                "achieved": round(achieved, 3), "peak": PEAK[dtype], "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK[dtype], 4), "traffic": measured_traffic(args.workload),
-                "launches": len(dense), "avg_launch_ms": round(dense_ms / len(dense), 5),
-                "flops_per_launch": dense_flops / len(dense)}
+    groups = {True: [], False: []}
+    for L, t in zip(layers, per_layer_ms):
+        groups[L.dense].append((L, t))
+    dom_dense = sum(t for _, t in groups[True]) >= sum(t for _, t in groups[False])
+    grp = groups[dom_dense]
+    g_ms = sum(t for _, t in grp)
+    if dom_dense:
+        achieved = sum(L.flops for L, _ in grp) / (g_ms * 1e-3) / 1e12
+        roofline = {"kernel": f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)", "bound": "mfma",
+                    "achieved": round(achieved, 3), "peak": PEAK[dtype], "unit": unit,
+                    "frac": round(achieved / PEAK[dtype], 4), "traffic": measured_traffic(args.workload),
+                    "launches": len(grp), "avg_launch_ms": round(g_ms / len(grp), 5),
+                    "work_per_launch": sum(L.flops for L, _ in grp) / len(grp)}
+    else:
+        achieved = sum(L.bytes for L, _ in grp) / (g_ms * 1e-3) / 1e9
+        roofline = {"kernel": "onhip::depthwise_f32_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    "traffic": measured_traffic(args.workload), "launches": len(grp),
+                    "avg_launch_ms": round(g_ms / len(grp), 5),
+                    "work_per_launch": sum(L.bytes for L, _ in grp) / len(grp)}
 
     extra = {}
     if args.workload.startswith("resnet50_b") and args.workload != "resnet50_b1" and not args.no_batch1:
         # the same stack at batch 1 (the "conv stack ms" of the reference's recorded trace)
-        _, _, l1 = make_workload("resnet50_b1")
-        layers1 = [DeviceLayer(torch, n, d, "resnet50_b1") for n, d in l1]
+        _, _, layers1 = make_workload(torch, hip, "resnet50_b1")
         ms1 = time_layers(torch, hip, layers1, reps=20)
         extra["resnet50_conv_stack_ms_batch1"] = round(sum(ms1), 4)
-    extra["conv_stack_ms_sum_of_layers"] = round(sum(per_layer_ms), 4)
+    extra["stack_ms_sum_of_layers"] = round(sum(per_layer_ms), 4)
     extra["algorithmic_GBps"] = round(abytes / (sum(per_layer_ms) * 1e-3) / 1e9, 1)
+    lowai = [(L, t) for L, t in zip(layers, per_layer_ms) if not L.dense]
+    if lowai:
+        extra["depthwise_GBps"] = round(sum(L.bytes for L, _ in lowai) / (sum(t for _, t in lowai) * 1e-3) / 1e9, 1)
+        extra["depthwise_ms"] = round(sum(t for _, t in lowai), 4)
 
     if args.layers:
-        print(f"{'layer':<18}{'M':>6}{'N':>9}{'K':>6}{'ms':>9}{'TFLOP/s':>9}{'%mfma':>7}{'GB/s':>8}", file=sys.stderr)
+        print(f"{'layer':<18}{'shape':<32}{'ms':>9}{unit:>9}{'%mfma':>7}{'GB/s':>8}{'%hbm':>6}", file=sys.stderr)
         for L, t in zip(layers, per_layer_ms):
-            d = L.d
-            oh, ow = d.out_hw()
-            tf = d.flops() / (t * 1e-3) / 1e12
-            print(f"{L.name:<18}{d.cout:>6}{d.n * oh * ow:>9}{d.k_per_out():>6}{t:>9.4f}{tf:>9.2f}"
-                  f"{100 * tf / PEAK[dtype]:>7.1f}{d.algorithmic_bytes() / (t * 1e-3) / 1e9:>8.0f}", file=sys.stderr)
+            tf = L.flops / (t * 1e-3) / 1e12
+            gb = L.bytes / (t * 1e-3) / 1e9
+            print(f"{L.name:<18}{L.shape:<32}{t:>9.4f}{tf:>9.2f}{100 * tf / PEAK[dtype]:>7.1f}{gb:>8.0f}"
+                  f"{100 * gb / HBM_PEAK_GBS:>6.1f}", file=sys.stderr)
 
-    cpu = None
-    if not args.no_cpu:
-        cpu = cpu_baseline(layer_descs, args.workload)
+    cpu = None if args.no_cpu else cpu_baseline(layers, args.workload, unit)
 
-    line = {"metric": "resnet50_conv_stack_fp32_tflops" if args.workload.startswith("resnet50") else
-            f"{args.workload}_tflops",
-            "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TFLOP/s", "n_gpus": 1,
+    metric = {"resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
+              "yolov8s": "yolov8s_conv_stack_w8a32_tops", "vit": f"vit_tiny_matmul_{dtype}_tflops",
+              "cfg1": "conv2d_relu_fp32_tflops"}
+    key = next(k for k in metric if args.workload.startswith(k))
+    line = {"metric": metric[key], "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": unit, "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-            "config": {"workload": desc, "layers": len(layers), "flops_per_step": flops,
+            "config": {"workload": desc, "layers": len(layers), "ops_per_step": flops,
                        "algorithmic_bytes_per_step": abytes},
             "roofline": roofline, "cpu_baseline": cpu}
     line.update(extra)

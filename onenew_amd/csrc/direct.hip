@@ -5,106 +5,6 @@
 
 namespace onhip {
 
-// ---- depthwise convolution, fp32 -------------------------------------------------------------------
-// One thread per output element, lanes along ow (coalesced).  Taps are added in ascending (i, j)
-// order to a zero sum with separately rounded multiply and add, the bias last: the arithmetic of
-// device/x86/Conv/conv.c:597-612 and :853-894 exactly, so the result is bit-identical to it.
-__global__ __launch_bounds__(256) void depthwise_f32_kernel(onhip_conv_desc_t d, int OH, int OW, const float *x,
-                                                            const float *w, const float *bias, Epilogue ep, float *y,
-                                                            long long total) {
-    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int ow = (int) (idx % OW);
-    long long t = idx / OW;
-    const int oh = (int) (t % OH);
-    t /= OH;
-    const int c = (int) (t % d.cout);
-    const float *xc = x + t * (long long) d.h * d.w;  // t = img * C + c
-    const float *wc = w + (long long) c * d.kh * d.kw;
-    const int ih0 = oh * d.stride_h - d.pad_t, iw0 = ow * d.stride_w - d.pad_l;
-    float acc = 0.0f;
-    for (int i = 0; i < d.kh; ++i) {
-        const int ih = ih0 + i;
-        if ((unsigned) ih >= (unsigned) d.h) continue;
-        for (int j = 0; j < d.kw; ++j) {
-            const int iw = iw0 + j;
-            if ((unsigned) iw >= (unsigned) d.w) continue;
-            acc = __fadd_rn(acc, __fmul_rn(wc[i * d.kw + j], xc[(long long) ih * d.w + iw]));
-        }
-    }
-    acc = __fadd_rn(acc, bias[c]);
-    y[idx] = apply_act(acc, ep);
-}
-
-int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,
-                         const float *bias, const Epilogue &ep, float *y, hipStream_t stream) {
-    const long long total = (long long) d.n * d.cout * OH * OW;
-    const long long blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise: output too large");
-    hipLaunchKernelGGL(depthwise_f32_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, d, OH, OW, x, w, bias, ep,
-                       y, total);
-    ONHIP_CHECK_HIP(hipGetLastError());
-    return ONHIP_OK;
-}
-
-// activation quantiser of conv.c:961-973: t = x * (1/scale), clamp, roundf (ties away from zero)
-__device__ __forceinline__ int quant_s8(float x, float inv_scale) {
-    float t = __fmul_rn(x, inv_scale);
-    t = (t < -128.0f) ? -128.0f : (t > 127.0f) ? 127.0f : t;
-    return (int) roundf(t);
-}
-
-// ---- depthwise convolution, W8A32 (conv.c:617-755) -----------------------------------------------------
-__global__ __launch_bounds__(256) void depthwise_w8a32_kernel(onhip_conv_desc_t d, int OH, int OW, const float *x,
-                                                              const int8_t *w8, const int32_t *bias32,
-                                                              const float *weight_aux, Epilogue ep, void *y,
-                                                              int32_t *acc32, float inv_scale, float out_inv_scale,
-                                                              long long total) {
-    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int ow = (int) (idx % OW);
-    long long t = idx / OW;
-    const int oh = (int) (t % OH);
-    t /= OH;
-    const int c = (int) (t % d.cout);
-    const float *xc = x + t * (long long) d.h * d.w;
-    const int8_t *wc = w8 + (long long) c * d.kh * d.kw;
-    const int ih0 = oh * d.stride_h - d.pad_t, iw0 = ow * d.stride_w - d.pad_l;
-    int acc = 0;
-    for (int i = 0; i < d.kh; ++i) {
-        const int ih = ih0 + i;
-        if ((unsigned) ih >= (unsigned) d.h) continue;
-        for (int j = 0; j < d.kw; ++j) {
-            const int iw = iw0 + j;
-            if ((unsigned) iw >= (unsigned) d.w) continue;
-            acc += (int) wc[i * d.kw + j] * quant_s8(xc[(long long) ih * d.w + iw], inv_scale);
-        }
-    }
-    if (acc32) acc32[idx] = acc;
-    float f = __fadd_rn(__fmul_rn((float) acc, d.input_scale), (float) bias32[c]);
-    float v = apply_act(__fmul_rn(f, __fdiv_rn(weight_aux[c], 127.0f)), ep);
-    if (d.out_s8) {
-        float q = __fmul_rn(v, out_inv_scale);
-        q = (q < -128.0f) ? -128.0f : (q > 127.0f) ? 127.0f : q;
-        reinterpret_cast<int8_t *>(y)[idx] = (int8_t) roundf(q);
-    } else {
-        reinterpret_cast<float *>(y)[idx] = v;
-    }
-}
-
-int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const int8_t *w8,
-                           const int32_t *bias32, const float *weight_aux, const Epilogue &ep, void *y,
-                           int32_t *acc32, hipStream_t stream) {
-    const long long total = (long long) d.n * d.cout * OH * OW;
-    const long long blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise: output too large");
-    const float inv_scale = 1.0f / d.input_scale;
-    const float out_inv = d.out_s8 ? 1.0f / d.output_scale : 0.0f;
-    hipLaunchKernelGGL(depthwise_w8a32_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, d, OH, OW, x, w8, bias32,
-                       weight_aux, ep, y, acc32, inv_scale, out_inv, total);
-    ONHIP_CHECK_HIP(hipGetLastError());
-    return ONHIP_OK;
-}
 
 // ---- NCHW fp32 -> NHWC int8, channels zero-padded to cp (a multiple of 16) -----------------------------
 // One thread quantises 16 channels of one pixel: 16 loads that are each coalesced along the pixel

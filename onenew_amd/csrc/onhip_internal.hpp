@@ -60,6 +60,13 @@ __device__ __forceinline__ float apply_act(float v, const Epilogue &e) {
     }
 }
 
+// activation quantiser of conv.c:961-973: t = x * (1/scale), clamp, roundf (ties away from zero)
+__device__ __forceinline__ int quant_s8(float x, float inv_scale) {
+    float t = __fmul_rn(x, inv_scale);
+    t = (t < -128.0f) ? -128.0f : (t > 127.0f) ? 127.0f : t;
+    return (int) roundf(t);
+}
+
 // ---- implicit-GEMM kernel family (igemm.hip) ---------------------------------------------------------
 //
 // C[M, N] = A[M, K] * B[K, N] on MFMA 32x32 tiles.  A rows are K-contiguous (weights, or the left
