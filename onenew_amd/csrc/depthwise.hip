@@ -17,6 +17,7 @@ namespace onhip {
 
 constexpr int DW_THREADS = 256;
 constexpr int DW_LDS_FLOATS = 8192;   // 32 KiB of LDS per workgroup: five workgroups per CU
+constexpr int DW_RT = 4;              // 3x3 specialisation: output rows per thread
 
 struct DwParams {
     int C, H, W, OH, OW, kh, kw, sh, sw, pt, pl;
@@ -24,14 +25,19 @@ struct DwParams {
     int planes_per_wg;   // >= 1 when whole planes fit in LDS, else 0
     int band_rows;       // output rows per workgroup when a plane is split into bands
     int bands;           // bands per plane (1 when planes_per_wg >= 1)
-    int strip_rows;      // 3x3 specialisation: output rows one thread walks down
+    int pitch;           // LDS row pitch: W plus the left and right padding columns the filter can touch
+    int flat_stage;      // small whole planes: stage by flat index
+    unsigned magic_hw, magic_w;   // floor(2^32 / d) + 1 for d = H*W and d = W (d >= 2)
     float in_scale, inv_in_scale, out_inv_scale;
     int out_s8;
 };
 
-// S3 > 0: 3x3 filter with stride S3, fully unrolled with a register window that slides down the
-// column (a new output row costs one new input row of three LDS reads for stride 1, two for stride 2).
-// S3 == 0: any filter, one output at a time.
+// The LDS tile holds, for each plane of the chunk, every input row and column the chunk's outputs
+// touch, padding included and zero-filled, so the compute phase reads it without predicates:
+// tile row = ih - (oh0 * sh - pt), tile column = iw + pl.
+//
+// S3 > 0: 3x3 filter with stride S3, fully unrolled: a thread computes DW_RT vertically adjacent
+// outputs from a (DW_RT - 1) * S3 + 3 by 3 register window.  S3 == 0: any filter, one output at a time.
 template <bool INT8, int S3>
 __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p, const float *__restrict__ x,
                                                                      const void *__restrict__ wv,
@@ -40,66 +46,82 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
                                                                      void *__restrict__ y, int32_t *__restrict__ acc32) {
     __shared__ float tile[DW_LDS_FLOATS];
     const int tid = threadIdx.x;
-    int plane0, nplanes, oh0, oh1, ih_lo, ih_hi;
+    int plane0, nplanes, oh0, oh1;
     if (p.planes_per_wg >= 1) {
         plane0 = blockIdx.x * p.planes_per_wg;
         nplanes = min(p.planes_per_wg, p.planes - plane0);
-        oh0 = 0; oh1 = p.OH; ih_lo = 0; ih_hi = p.H;
+        oh0 = 0; oh1 = p.OH;
     } else {
         plane0 = blockIdx.x / p.bands;
         nplanes = 1;
         const int band = blockIdx.x - plane0 * p.bands;
         oh0 = band * p.band_rows;
         oh1 = min(p.OH, oh0 + p.band_rows);
-        ih_lo = max(0, oh0 * p.sh - p.pt);
-        ih_hi = min(p.H, (oh1 - 1) * p.sh - p.pt + p.kh);
     }
-    const int rows = ih_hi - ih_lo;                 // input rows held per plane
-    const int plane_elems = rows * p.W;
-    // ---- stage the contiguous input chunk ---------------------------------------------------------
-    if (p.planes_per_wg >= 1) {
-        const long long start = (long long) plane0 * p.H * p.W;
-        const int total = nplanes * p.H * p.W;
-        const float *src = x + start;
-        if (((start | total) & 3) == 0) {
-            const float4 *s4 = reinterpret_cast<const float4 *>(src);
-            for (int i = tid; i < total / 4; i += DW_THREADS) {
-                float4 v = s4[i];
-                if (INT8) { v.x = (float) quant_s8(v.x, p.inv_in_scale); v.y = (float) quant_s8(v.y, p.inv_in_scale);
-                            v.z = (float) quant_s8(v.z, p.inv_in_scale); v.w = (float) quant_s8(v.w, p.inv_in_scale); }
-                reinterpret_cast<float4 *>(tile)[i] = v;
-            }
-        } else {
+    const int ih_first = oh0 * p.sh - p.pt;                      // input row of tile row 0 (may be negative)
+    const int trows = (oh1 - 1 - oh0) * p.sh + p.kh;             // tile rows per plane
+    const int pitch = p.pitch;
+    const int plane_cells = trows * pitch;
+    // ---- stage -----------------------------------------------------------------------------------------
+    // 1. clear the cells of the chunk (padding stays zero), 2. copy the rows that exist: a thread keeps its
+    // group of four columns and walks down the rows, 128-bit loads when rows are 16-byte aligned.
+    {
+        const int cells = nplanes * plane_cells;
+        float4 *t4 = reinterpret_cast<float4 *>(tile);
+        for (int i = tid; i < (cells + 3) / 4; i += DW_THREADS) t4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();
+        if (p.flat_stage) {
+            // small planes: the chunk is one contiguous run of nplanes * H * W inputs; walk it flat and scatter
+            // into the padded tile (flat index -> plane, row, column by multiply-high division)
+            const int hw = p.H * p.W;
+            const int total = nplanes * hw;
+            const float *src = x + (long long) plane0 * hw;
             for (int i = tid; i < total; i += DW_THREADS) {
+                const int pl = (int) __umulhi((unsigned) i, p.magic_hw);
+                const int rem = i - pl * hw;
+                const int r = (int) __umulhi((unsigned) rem, p.magic_w);
+                const int c = rem - r * p.W;
                 const float v = src[i];
-                tile[i] = INT8 ? (float) quant_s8(v, p.inv_in_scale) : v;
+                tile[pl * plane_cells + (r - ih_first) * pitch + c + p.pl] = INT8 ? (float) quant_s8(v, p.inv_in_scale) : v;
+            }
+            __syncthreads();
+        } else {
+        const int r_lo = max(0, -ih_first);                       // first tile row that exists in the image
+        const int r_hi = min(trows, p.H - ih_first);              // one past the last
+        const bool vec = (p.W & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+        const int groups = vec ? p.W / 4 : p.W;                   // column groups per row
+        const int gpp = groups < DW_THREADS ? groups : DW_THREADS;  // groups handled per pass
+        const int rows_per_pass = DW_THREADS / gpp;
+        const int ry = tid / gpp, gx = tid - ry * gpp;
+        if (ry < rows_per_pass) {
+            for (int pl = 0; pl < nplanes; ++pl) {
+                const float *src = x + ((long long) (plane0 + pl) * p.H + ih_first) * p.W;   // tile row 0 of this plane
+                float *dst = tile + pl * plane_cells + p.pl;
+                for (int g = gx; g < groups; g += gpp) {
+                    for (int tr = r_lo + ry; tr < r_hi; tr += rows_per_pass) {
+                        if (vec) {
+                            float4 v = *reinterpret_cast<const float4 *>(src + tr * p.W + 4 * g);
+                            if (INT8) { v.x = (float) quant_s8(v.x, p.inv_in_scale); v.y = (float) quant_s8(v.y, p.inv_in_scale);
+                                        v.z = (float) quant_s8(v.z, p.inv_in_scale); v.w = (float) quant_s8(v.w, p.inv_in_scale); }
+                            float *o = dst + tr * pitch + 4 * g;
+                            o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+                        } else {
+                            const float v = src[tr * p.W + g];
+                            dst[tr * pitch + g] = INT8 ? (float) quant_s8(v, p.inv_in_scale) : v;
+                        }
+                    }
+                }
             }
         }
-    } else {
-        const long long start = ((long long) plane0 * p.H + ih_lo) * p.W;
-        const float *src = x + start;
-        if (((start | plane_elems) & 3) == 0) {
-            const float4 *s4 = reinterpret_cast<const float4 *>(src);
-            for (int i = tid; i < plane_elems / 4; i += DW_THREADS) {
-                float4 v = s4[i];
-                if (INT8) { v.x = (float) quant_s8(v.x, p.inv_in_scale); v.y = (float) quant_s8(v.y, p.inv_in_scale);
-                            v.z = (float) quant_s8(v.z, p.inv_in_scale); v.w = (float) quant_s8(v.w, p.inv_in_scale); }
-                reinterpret_cast<float4 *>(tile)[i] = v;
-            }
-        } else {
-            for (int i = tid; i < plane_elems; i += DW_THREADS) {
-                const float v = src[i];
-                tile[i] = INT8 ? (float) quant_s8(v, p.inv_in_scale) : v;
-            }
+        __syncthreads();
         }
     }
-    __syncthreads();
     // ---- compute --------------------------------------------------------------------------------------
     const int out_rows = oh1 - oh0;
     const int khkw = p.kh * p.kw;
     if constexpr (S3 > 0) {
-        // a thread owns a strip: one output column, p.strip_rows consecutive output rows of one plane
-        const int nsr = (out_rows + p.strip_rows - 1) / p.strip_rows;
+        constexpr int WR = (DW_RT - 1) * S3 + 3;                  // window rows
+        const int nsr = (out_rows + DW_RT - 1) / DW_RT;
         const int strips_per_plane = nsr * p.OW;
         const int strips = nplanes * strips_per_plane;
         for (int sidx = tid; sidx < strips; sidx += DW_THREADS) {
@@ -109,7 +131,6 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
             const int ow = rem - sr * p.OW;
             const int plane = plane0 + pl;
             const int c = plane % p.C;
-            const float *tp = tile + pl * plane_elems;
             float wreg[9];
             float bias_f;
             if (INT8) {
@@ -124,33 +145,27 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
                 bias_f = reinterpret_cast<const float *>(bv)[c];
             }
             const float coeff = INT8 ? __fdiv_rn(weight_aux[c], 127.0f) : 0.0f;
-            const int iw0 = ow * p.sw - p.pl;
-            bool col_ok[3];
+            const int r0 = sr * DW_RT;                             // first output row of the strip, band-relative
+            const float *tp = tile + pl * plane_cells + ow * S3;
+            float win[WR][3];
 #pragma unroll
-            for (int j = 0; j < 3; ++j) col_ok[j] = (unsigned) (iw0 + j) < (unsigned) p.W;
-            // a tap outside the image multiplies a zero, as the reference's zero padding does
-            auto load_row = [&](int ih, float (&row)[3]) {
-                const bool rok = (unsigned) ih < (unsigned) p.H;
-                const int base = (ih - ih_lo) * p.W + iw0;
+            for (int r = 0; r < WR; ++r) {
+                // rows past the end of the band belong to outputs that are not stored: stay inside the tile
+                const int tr = min(r0 * S3 + r, trows - 1);
 #pragma unroll
-                for (int j = 0; j < 3; ++j) row[j] = (rok && col_ok[j]) ? tp[base + j] : 0.0f;
-            };
-            const int r_begin = oh0 + sr * p.strip_rows;
-            const int r_end = min(oh1, r_begin + p.strip_rows);
-            float win[3][3];
-            int ih = r_begin * S3 - p.pt;
-            load_row(ih, win[0]);
-            load_row(ih + 1, win[1]);
-            long long oidx = ((long long) plane * p.OH + r_begin) * p.OW + ow;
-            for (int oh = r_begin; oh < r_end; ++oh, oidx += p.OW) {
-                load_row(ih + 2, win[2]);
+                for (int j = 0; j < 3; ++j) win[r][j] = tp[tr * pitch + j];
+            }
+            long long oidx = ((long long) plane * p.OH + oh0 + r0) * p.OW + ow;
+#pragma unroll
+            for (int q = 0; q < DW_RT; ++q, oidx += p.OW) {
+                if (r0 + q >= out_rows) break;
                 float v;
                 if (INT8) {
                     int acc = 0;
 #pragma unroll
                     for (int i = 0; i < 3; ++i)
 #pragma unroll
-                        for (int j = 0; j < 3; ++j) acc += (int) wreg[i * 3 + j] * (int) win[i][j];
+                        for (int j = 0; j < 3; ++j) acc += (int) wreg[i * 3 + j] * (int) win[q * S3 + i][j];
                     if (acc32) acc32[oidx] = acc;
                     // conv.c:739 and :746-752: acc * s + bias32, then * (aux / 127): separately rounded
                     const float f = __fadd_rn(__fmul_rn((float) acc, p.in_scale), bias_f);
@@ -160,22 +175,11 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
 #pragma unroll
                     for (int i = 0; i < 3; ++i)
 #pragma unroll
-                        for (int j = 0; j < 3; ++j) acc = __fadd_rn(acc, __fmul_rn(wreg[i * 3 + j], win[i][j]));
+                        for (int j = 0; j < 3; ++j) acc = __fadd_rn(acc, __fmul_rn(wreg[i * 3 + j], win[q * S3 + i][j]));
                     v = apply_act(__fadd_rn(acc, bias_f), ep);
                 }
                 if (INT8 && p.out_s8) reinterpret_cast<int8_t *>(y)[oidx] = (int8_t) quant_s8(v, p.out_inv_scale);
                 else reinterpret_cast<float *>(y)[oidx] = v;
-                // slide the window down by the stride
-                if (S3 == 1) {
-#pragma unroll
-                    for (int j = 0; j < 3; ++j) { win[0][j] = win[1][j]; win[1][j] = win[2][j]; }
-                    ih += 1;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 3; ++j) win[0][j] = win[2][j];
-                    ih += 2;
-                    load_row(ih + 1, win[1]);
-                }
             }
         }
         return;
@@ -187,45 +191,28 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
         const int rem = o - pl * per_plane;
         const int r = rem / p.OW;
         const int ow = rem - r * p.OW;
-        const int oh = oh0 + r;
         const int plane = plane0 + pl;
         const int c = plane % p.C;
-        const float *tp = tile + pl * plane_elems;
-        const int ihb = oh * p.sh - p.pt, iwb = ow * p.sw - p.pl;
-        const long long oidx = ((long long) plane * p.OH + oh) * p.OW + ow;
+        const float *tp = tile + pl * plane_cells + (r * p.sh) * pitch + ow * p.sw;
+        const long long oidx = ((long long) plane * p.OH + oh0 + r) * p.OW + ow;
+        float v;
         if (INT8) {
             const int8_t *wc = reinterpret_cast<const int8_t *>(wv) + (long long) c * khkw;
             int acc = 0;
-            for (int i = 0; i < p.kh; ++i) {
-                const int ih = ihb + i;
-                if ((unsigned) ih >= (unsigned) p.H) continue;
-                for (int j = 0; j < p.kw; ++j) {
-                    const int iw = iwb + j;
-                    if ((unsigned) iw >= (unsigned) p.W) continue;
-                    acc += (int) wc[i * p.kw + j] * (int) tp[(ih - ih_lo) * p.W + iw];
-                }
-            }
+            for (int i = 0; i < p.kh; ++i)
+                for (int j = 0; j < p.kw; ++j) acc += (int) wc[i * p.kw + j] * (int) tp[i * pitch + j];
             if (acc32) acc32[oidx] = acc;
-            // conv.c:739 and :746-752: acc * s + bias32, then * (aux / 127): three separately rounded operations
-            float f = __fadd_rn(__fmul_rn((float) acc, p.in_scale), (float) reinterpret_cast<const int32_t *>(bv)[c]);
-            const float v = apply_act(__fmul_rn(f, __fdiv_rn(weight_aux[c], 127.0f)), ep);
-            if (p.out_s8) reinterpret_cast<int8_t *>(y)[oidx] = (int8_t) quant_s8(v, p.out_inv_scale);
-            else reinterpret_cast<float *>(y)[oidx] = v;
+            const float f = __fadd_rn(__fmul_rn((float) acc, p.in_scale), (float) reinterpret_cast<const int32_t *>(bv)[c]);
+            v = apply_act(__fmul_rn(f, __fdiv_rn(weight_aux[c], 127.0f)), ep);
         } else {
             const float *wc = reinterpret_cast<const float *>(wv) + (long long) c * khkw;
             float acc = 0.0f;
-            for (int i = 0; i < p.kh; ++i) {
-                const int ih = ihb + i;
-                if ((unsigned) ih >= (unsigned) p.H) continue;
-                for (int j = 0; j < p.kw; ++j) {
-                    const int iw = iwb + j;
-                    if ((unsigned) iw >= (unsigned) p.W) continue;
-                    acc = __fadd_rn(acc, __fmul_rn(wc[i * p.kw + j], tp[(ih - ih_lo) * p.W + iw]));
-                }
-            }
-            acc = __fadd_rn(acc, reinterpret_cast<const float *>(bv)[c]);
-            reinterpret_cast<float *>(y)[oidx] = apply_act(acc, ep);
+            for (int i = 0; i < p.kh; ++i)
+                for (int j = 0; j < p.kw; ++j) acc = __fadd_rn(acc, __fmul_rn(wc[i * p.kw + j], tp[i * pitch + j]));
+            v = apply_act(__fadd_rn(acc, reinterpret_cast<const float *>(bv)[c]), ep);
         }
+        if (INT8 && p.out_s8) reinterpret_cast<int8_t *>(y)[oidx] = (int8_t) quant_s8(v, p.out_inv_scale);
+        else reinterpret_cast<float *>(y)[oidx] = v;
     }
 }
 
@@ -239,33 +226,37 @@ static int dw_plan(const onhip_conv_desc_t &d, int OH, int OW, DwParams *p) {
     p->C = d.cout; p->H = d.h; p->W = d.w; p->OH = OH; p->OW = OW;
     p->kh = d.kh; p->kw = d.kw; p->sh = d.stride_h; p->sw = d.stride_w; p->pt = d.pad_t; p->pl = d.pad_l;
     p->planes = d.n * d.cout;
-    const int plane = d.h * d.w;
-    if (plane <= DW_LDS_FLOATS) {
-        // whole planes; keep at least a few hundred outputs per workgroup but leave enough workgroups for 256 CUs
-        int ppw = DW_LDS_FLOATS / plane;
+    // columns 0 .. (OW-1)*sw + kw - 1 of the padded row are read
+    p->pitch = (OW - 1) * d.stride_w + d.kw;
+    const int full_rows = (OH - 1) * d.stride_h + d.kh;
+    const int plane_cells = full_rows * p->pitch;
+    if (plane_cells <= DW_LDS_FLOATS) {
+        // whole planes: as many as fit, but leave enough workgroups to fill 256 CUs several times over
+        int ppw = DW_LDS_FLOATS / plane_cells;
         const int want_wgs = 256 * 8;
         const int cap = (p->planes + want_wgs - 1) / want_wgs;
         if (ppw > cap) ppw = cap < 1 ? 1 : cap;
-        while (ppw > 1 && ppw * OH * OW > 4096) --ppw;
         p->planes_per_wg = ppw;
         p->bands = 1;
         p->band_rows = OH;
-        // strips of rows per thread: long enough to amortise the set-up, short enough to keep 256 threads busy
-        int sr = (ppw * OH * OW) / (2 * DW_THREADS);
-        p->strip_rows = sr < 1 ? 1 : sr > 8 ? 8 : sr;
-        if (p->strip_rows > OH) p->strip_rows = OH;
+        // rows shorter than a wavefront: the row-walking copy would leave most lanes idle
+        p->flat_stage = d.w < 32 && d.w >= 2 && d.h * d.w >= 2 && (long long) ppw * d.h * d.w * d.h * d.w < (1LL << 32);
+        p->magic_hw = (unsigned) (0x100000000ULL / (unsigned) (d.h * d.w)) + 1u;
+        p->magic_w = (unsigned) (0x100000000ULL / (unsigned) d.w) + 1u;
         return (p->planes + ppw - 1) / ppw;
     }
-    // bands of output rows: (band_rows - 1) * sh + kh input rows must fit
-    int max_in_rows = DW_LDS_FLOATS / d.w;
-    int band = (max_in_rows - d.kh) / d.stride_h + 1;
-    if (band < 1) return -1;
+    // bands of output rows: (band_rows - 1) * sh + kh tile rows must fit
+    const int max_rows = DW_LDS_FLOATS / p->pitch;
+    int band = (max_rows - d.kh) / d.stride_h + 1;
+    if (max_rows < d.kh || band < 1) return -1;
     if (band > OH) band = OH;
+    // equal bands, a multiple of the per-thread strip where possible
+    const int nb = (OH + band - 1) / band;
+    band = (OH + nb - 1) / nb;
+    if (band % DW_RT && (band / DW_RT + 1) * DW_RT <= (max_rows - d.kh) / d.stride_h + 1) band = (band / DW_RT + 1) * DW_RT;
     p->planes_per_wg = 0;
     p->band_rows = band;
     p->bands = (OH + band - 1) / band;
-    int sr = (band * OW) / (2 * DW_THREADS);
-    p->strip_rows = sr < 1 ? 1 : sr > 8 ? 8 : sr;
     return p->planes * p->bands;
 }
 
