@@ -38,7 +38,7 @@ struct DwParams {
 //
 // S3 > 0: 3x3 filter with stride S3, fully unrolled: a thread computes DW_RT vertically adjacent
 // outputs from a (DW_RT - 1) * S3 + 3 by 3 register window.  S3 == 0: any filter, one output at a time.
-template <bool INT8, int S3>
+template <bool INT8, int S3, int EPI>
 __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p, const float *__restrict__ x,
                                                                      const void *__restrict__ wv,
                                                                      const void *__restrict__ bv,
@@ -155,10 +155,14 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
 #pragma unroll
                 for (int j = 0; j < 3; ++j) win[r][j] = tp[tr * pitch + j];
             }
-            long long oidx = ((long long) plane * p.OH + oh0 + r0) * p.OW + ow;
+            const long long obase = ((long long) plane * p.OH + oh0 + r0) * p.OW + ow;
+            float *yf = reinterpret_cast<float *>(y) + obase;
+            int8_t *y8 = reinterpret_cast<int8_t *>(y) + obase;
+            int32_t *ya = acc32 ? acc32 + obase : nullptr;
 #pragma unroll
-            for (int q = 0; q < DW_RT; ++q, oidx += p.OW) {
+            for (int q = 0; q < DW_RT; ++q) {
                 if (r0 + q >= out_rows) break;
+                const int oidx = q * p.OW;
                 float v;
                 if (INT8) {
                     int acc = 0;
@@ -166,20 +170,20 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
                     for (int i = 0; i < 3; ++i)
 #pragma unroll
                         for (int j = 0; j < 3; ++j) acc += (int) wreg[i * 3 + j] * (int) win[q * S3 + i][j];
-                    if (acc32) acc32[oidx] = acc;
+                    if (ya) ya[oidx] = acc;
                     // conv.c:739 and :746-752: acc * s + bias32, then * (aux / 127): separately rounded
                     const float f = __fadd_rn(__fmul_rn((float) acc, p.in_scale), bias_f);
-                    v = apply_act(__fmul_rn(f, coeff), ep);
+                    v = act_fast<EPI>(__fmul_rn(f, coeff), ep);
                 } else {
                     float acc = 0.0f;
 #pragma unroll
                     for (int i = 0; i < 3; ++i)
 #pragma unroll
                         for (int j = 0; j < 3; ++j) acc = __fadd_rn(acc, __fmul_rn(wreg[i * 3 + j], win[q * S3 + i][j]));
-                    v = apply_act(__fadd_rn(acc, bias_f), ep);
+                    v = act_fast<EPI>(__fadd_rn(acc, bias_f), ep);
                 }
-                if (INT8 && p.out_s8) reinterpret_cast<int8_t *>(y)[oidx] = (int8_t) quant_s8(v, p.out_inv_scale);
-                else reinterpret_cast<float *>(y)[oidx] = v;
+                if (INT8 && p.out_s8) y8[oidx] = (int8_t) quant_s8(v, p.out_inv_scale);
+                else yf[oidx] = v;
             }
         }
         return;
@@ -203,13 +207,13 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
                 for (int j = 0; j < p.kw; ++j) acc += (int) wc[i * p.kw + j] * (int) tp[i * pitch + j];
             if (acc32) acc32[oidx] = acc;
             const float f = __fadd_rn(__fmul_rn((float) acc, p.in_scale), (float) reinterpret_cast<const int32_t *>(bv)[c]);
-            v = apply_act(__fmul_rn(f, __fdiv_rn(weight_aux[c], 127.0f)), ep);
+            v = act_fast<EPI>(__fmul_rn(f, __fdiv_rn(weight_aux[c], 127.0f)), ep);
         } else {
             const float *wc = reinterpret_cast<const float *>(wv) + (long long) c * khkw;
             float acc = 0.0f;
             for (int i = 0; i < p.kh; ++i)
                 for (int j = 0; j < p.kw; ++j) acc = __fadd_rn(acc, __fmul_rn(wc[i * p.kw + j], tp[i * pitch + j]));
-            v = apply_act(__fadd_rn(acc, reinterpret_cast<const float *>(bv)[c]), ep);
+            v = act_fast<EPI>(__fadd_rn(acc, reinterpret_cast<const float *>(bv)[c]), ep);
         }
         if (INT8 && p.out_s8) reinterpret_cast<int8_t *>(y)[oidx] = (int8_t) quant_s8(v, p.out_inv_scale);
         else reinterpret_cast<float *>(y)[oidx] = v;
@@ -260,22 +264,28 @@ static int dw_plan(const onhip_conv_desc_t &d, int OH, int OW, DwParams *p) {
     return p->planes * p->bands;
 }
 
+template <bool INT8>
+static void dw_dispatch(int s3, int epi, unsigned wgs, hipStream_t stream, const DwParams &p, const float *x, const void *w,
+                        const void *b, const float *aux, const Epilogue &ep, void *y, int32_t *acc32) {
+#define ONHIP_DW_CASE(S, E)                                                                                             \
+    if (s3 == S && epi == E) {                                                                                          \
+        hipLaunchKernelGGL((depthwise_tiled_kernel<INT8, S, E>), dim3(wgs), dim3(DW_THREADS), 0, stream, p, x, w, b, aux, \
+                           ep, y, acc32);                                                                               \
+        return;                                                                                                         \
+    }
+#define ONHIP_DW_ROW(S) ONHIP_DW_CASE(S, EPI_NONE) ONHIP_DW_CASE(S, EPI_RELU) ONHIP_DW_CASE(S, EPI_CLIP) ONHIP_DW_CASE(S, EPI_GENERIC)
+    ONHIP_DW_ROW(0) ONHIP_DW_ROW(1) ONHIP_DW_ROW(2)
+#undef ONHIP_DW_ROW
+#undef ONHIP_DW_CASE
+}
+
 int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,
                          const float *bias, const Epilogue &ep, float *y, hipStream_t stream) {
     DwParams p;
     memset(&p, 0, sizeof(p));
     const long long wgs = dw_plan(d, OH, OW, &p);
     if (wgs < 1 || wgs > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise: image row of %d elements too wide", d.w);
-    const int s3 = dw_specialisation(d);
-    if (s3 == 1)
-        hipLaunchKernelGGL((depthwise_tiled_kernel<false, 1>), dim3((unsigned) wgs), dim3(DW_THREADS), 0, stream, p, x, w,
-                           bias, nullptr, ep, y, nullptr);
-    else if (s3 == 2)
-        hipLaunchKernelGGL((depthwise_tiled_kernel<false, 2>), dim3((unsigned) wgs), dim3(DW_THREADS), 0, stream, p, x, w,
-                           bias, nullptr, ep, y, nullptr);
-    else
-        hipLaunchKernelGGL((depthwise_tiled_kernel<false, 0>), dim3((unsigned) wgs), dim3(DW_THREADS), 0, stream, p, x, w,
-                           bias, nullptr, ep, y, nullptr);
+    dw_dispatch<false>(dw_specialisation(d), epi_of_act(ep.act), (unsigned) wgs, stream, p, x, w, bias, nullptr, ep, y, nullptr);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }
@@ -291,16 +301,8 @@ int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const flo
     p.inv_in_scale = 1.0f / d.input_scale;
     p.out_s8 = d.out_s8;
     p.out_inv_scale = d.out_s8 ? 1.0f / d.output_scale : 0.0f;
-    const int s3 = dw_specialisation(d);
-    if (s3 == 1)
-        hipLaunchKernelGGL((depthwise_tiled_kernel<true, 1>), dim3((unsigned) wgs), dim3(DW_THREADS), 0, stream, p, x, w8,
-                           bias32, weight_aux, ep, y, acc32);
-    else if (s3 == 2)
-        hipLaunchKernelGGL((depthwise_tiled_kernel<true, 2>), dim3((unsigned) wgs), dim3(DW_THREADS), 0, stream, p, x, w8,
-                           bias32, weight_aux, ep, y, acc32);
-    else
-        hipLaunchKernelGGL((depthwise_tiled_kernel<true, 0>), dim3((unsigned) wgs), dim3(DW_THREADS), 0, stream, p, x, w8,
-                           bias32, weight_aux, ep, y, acc32);
+    dw_dispatch<true>(dw_specialisation(d), epi_of_act(ep.act), (unsigned) wgs, stream, p, x, w8, bias32, weight_aux, ep, y,
+                      acc32);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }

@@ -291,18 +291,6 @@ __device__ __forceinline__ unsigned out_col_offset(const IgemmParams &p, int n, 
     return (unsigned) (n * (int) p.c_stride_n) * (unsigned) esz;
 }
 
-enum { EPI_NONE = 0, EPI_RELU = 1, EPI_CLIP = 2, EPI_GENERIC = 3 };
-
-template <int EPI>
-__device__ __forceinline__ float act_fast(float v, const Epilogue &e) {
-    if constexpr (EPI == EPI_NONE) return v;
-    else if constexpr (EPI == EPI_RELU) return v > 0.0f ? v : 0.0f;
-    else if constexpr (EPI == EPI_CLIP) {
-        const float t = v > e.clip_min ? v : e.clip_min;
-        return t < e.clip_max ? t : e.clip_max;
-    } else return apply_act(v, e);
-}
-
 // the consumer's activation quantiser (conv.c:961-973) applied to an fp32 result
 __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
     float t = __fmul_rn(y, inv_scale);

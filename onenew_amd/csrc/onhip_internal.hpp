@@ -60,6 +60,24 @@ __device__ __forceinline__ float apply_act(float v, const Epilogue &e) {
     }
 }
 
+// The activation kind as a template parameter, so the common ones cost one or two instructions and no
+// branch in an unrolled epilogue; EPI_GENERIC falls back to apply_act.
+enum { EPI_NONE = 0, EPI_RELU = 1, EPI_CLIP = 2, EPI_GENERIC = 3 };
+
+inline int epi_of_act(int act) {
+    return (act == NOT_ACT || act == RELU6) ? EPI_NONE : act == RELU ? EPI_RELU : act == CLIP ? EPI_CLIP : EPI_GENERIC;
+}
+
+template <int EPI>
+__device__ __forceinline__ float act_fast(float v, const Epilogue &e) {
+    if constexpr (EPI == EPI_NONE) return v;
+    else if constexpr (EPI == EPI_RELU) return v > 0.0f ? v : 0.0f;
+    else if constexpr (EPI == EPI_CLIP) {
+        const float t = v > e.clip_min ? v : e.clip_min;
+        return t < e.clip_max ? t : e.clip_max;
+    } else return apply_act(v, e);
+}
+
 // activation quantiser of conv.c:961-973: t = x * (1/scale), clamp, roundf (ties away from zero)
 __device__ __forceinline__ int quant_s8(float x, float inv_scale) {
     float t = __fmul_rn(x, inv_scale);
