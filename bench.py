@@ -185,14 +185,14 @@ def make_workload(torch, hip, name):
     raise SystemExit(f"unknown workload {name}")
 
 
-def measured_traffic(workload):
-    """HBM bytes per launch of the dominant kernel from the committed counter summary
+def measured_traffic(workload, group):
+    """HBM bytes per launch of a kernel group ("igemm" or "depthwise") from the committed counter summary
     (profiles/<workload>_traffic.json: FETCH_SIZE / WRITE_SIZE scaled by the copy yardstick), else None"""
     path = os.path.join(ROOT, "profiles", f"{workload}_traffic.json")
     if not os.path.exists(path):
         return None
     with open(path) as f:
-        return json.load(f).get("hbm_bytes_per_launch")
+        return json.load(f).get("groups", {}).get(group, {}).get("hbm_bytes_per_launch")
 
 
 def time_layers(torch, hip, layers, reps):
@@ -298,20 +298,20 @@ def main():
     dom_dense = sum(t for _, t in groups[True]) >= sum(t for _, t in groups[False])
     grp = groups[dom_dense]
     g_ms = sum(t for _, t in grp)
-    if dom_dense:
-        achieved = sum(L.flops for L, _ in grp) / (g_ms * 1e-3) / 1e12
-        roofline = {"kernel": f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)", "bound": "mfma",
-                    "achieved": round(achieved, 3), "peak": PEAK[dtype], "unit": unit,
-                    "frac": round(achieved / PEAK[dtype], 4), "traffic": measured_traffic(args.workload),
-                    "launches": len(grp), "avg_launch_ms": round(g_ms / len(grp), 5),
-                    "work_per_launch": sum(L.flops for L, _ in grp) / len(grp)}
+    g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
+    kernel = f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else "onhip::depthwise_tiled_kernel"
+    # the bound is the roof the group's arithmetic intensity puts it under
+    mfma_bound = dom_dense and g_flops / g_bytes >= PEAK[dtype] * 1e12 / (HBM_PEAK_GBS * 1e9)
+    if mfma_bound:
+        achieved, peak, r_unit, work = g_flops / (g_ms * 1e-3) / 1e12, PEAK[dtype], unit, g_flops
     else:
-        achieved = sum(L.bytes for L, _ in grp) / (g_ms * 1e-3) / 1e9
-        roofline = {"kernel": "onhip::depthwise_f32_kernel", "bound": "hbm", "achieved": round(achieved, 1),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                    "traffic": measured_traffic(args.workload), "launches": len(grp),
-                    "avg_launch_ms": round(g_ms / len(grp), 5),
-                    "work_per_launch": sum(L.bytes for L, _ in grp) / len(grp)}
+        achieved, peak, r_unit, work = g_bytes / (g_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", g_bytes
+    roofline = {"kernel": kernel, "bound": "mfma" if mfma_bound else "hbm", "achieved": round(achieved, 3),
+                "peak": peak, "unit": r_unit, "frac": round(achieved / peak, 4),
+                "traffic": measured_traffic(args.workload, "igemm" if dom_dense else "depthwise"),
+                "launches": len(grp), "avg_launch_ms": round(g_ms / len(grp), 5),
+                "work_per_launch": work / len(grp),
+                "arithmetic_intensity": round(g_flops / g_bytes, 2)}
 
     extra = {}
     if args.workload.startswith("resnet50_b") and args.workload != "resnet50_b1" and not args.no_batch1:
