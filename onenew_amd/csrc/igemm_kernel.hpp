@@ -32,6 +32,7 @@
 // device/x86/MatMul/mat_mul.c:10.
 #pragma once
 #include "onhip_internal.hpp"
+#include <type_traits>
 
 namespace onhip {
 
@@ -146,21 +147,27 @@ __device__ __forceinline__ unsigned fast_div(unsigned x, unsigned magic, unsigne
     return __umulhi(x, magic) + (x & pass);
 }
 
+// exact floor(x / d) for 0 <= x < 2^31 (see Div31)
+__device__ __forceinline__ unsigned div31(unsigned x, const Div31 &d) {
+    return (__umulhi(x, d.magic) >> d.shift) + (x & d.pass);
+}
+
 // ---- A: one unit of one row ----------------------------------------------------------------------
 // voff: byte offset of (row, unit slot) fixed per thread, OOB for rows beyond M;
 // soff: byte offset of the K tile (uniform); k0: first reduction index of this unit; klim: end of K
-template <int DT>
+// CHK == false: the tile is known to lie inside K, no per-unit test
+template <int DT, bool CHK>
 __device__ __forceinline__ void load_a_unit(RawUnit<DT> &r, rsrc_t ra, unsigned voff, unsigned soff, int k0, int klim) {
     constexpr int KPU = Traits<DT>::KPU;
     if constexpr (DT == DT_I8) {
-        r.q = buf_load_b128(ra, k0 < klim ? voff : OOB, soff);
+        r.q = buf_load_b128(ra, (!CHK || k0 < klim) ? voff : OOB, soff);
     } else {
         // dwordx4 loads need dword alignment only.  A vector that straddles the end of a row brings
         // in the head of the next row (the end of the buffer reads as zero, dwords are range-checked
         // one by one); those lanes of K are cleared before they reach LDS (clear_a_tail).
 #pragma unroll
         for (int q = 0; q < KPU / 4; ++q) {
-            const uint4 t = buf_load_b128(ra, (k0 + 4 * q < klim) ? voff + 16 * q : OOB, soff);
+            const uint4 t = buf_load_b128(ra, (!CHK || k0 + 4 * q < klim) ? voff + 16 * q : OOB, soff);
             r.v[4 * q] = __uint_as_float(t.x); r.v[4 * q + 1] = __uint_as_float(t.y);
             r.v[4 * q + 2] = __uint_as_float(t.z); r.v[4 * q + 3] = __uint_as_float(t.w);
         }
@@ -188,9 +195,9 @@ __device__ __forceinline__ ColState make_col(const IgemmParams &p, int n) {
     ColState c;
     const bool valid = n < p.N;
     const int nn = valid ? n : 0;
-    const int img = nn / p.OHW;
+    const int img = (int) div31((unsigned) nn, p.div_ohw);
     const int pix = nn - img * p.OHW;
-    const int oh = pix / p.OW;
+    const int oh = (int) div31((unsigned) pix, p.div_ow);
     const int ow = pix - oh * p.OW;
     c.ih0 = oh * p.sh - p.pt;
     c.iw0 = ow * p.sw - p.pl;
@@ -255,10 +262,10 @@ __device__ __forceinline__ BPrep prep_b(const IgemmParams &p, int u, int e, int 
 }
 
 // vector offset of a prepared B load for this lane: the pixel if the tap is inside, else OOB
-template <int BL>
+template <int BL, bool CHK = true>
 __device__ __forceinline__ unsigned b_voff(const IgemmParams &p, const ColState &c, const BPrep &q, int u_or_k) {
     if constexpr (BL == BL_PLAIN) {
-        return q.bit ? c.pixoff : OOB;
+        return (!CHK || q.bit) ? c.pixoff : OOB;
     } else {
         if (p.use_tapmask) {
             const unsigned word = q.hi ? c.mask_hi : c.mask_lo;
@@ -284,7 +291,7 @@ __device__ __forceinline__ unsigned b_voff(const IgemmParams &p, const ColState 
 // byte offset of column n inside one batch slice of C (rows are added through the scalar offset)
 __device__ __forceinline__ unsigned out_col_offset(const IgemmParams &p, int n, int esz) {
     if (p.out_mode == OUT_CONV) {
-        const int img = n / p.OHW;
+        const int img = (int) div31((unsigned) n, p.div_ohw);
         const int pix = n - img * p.OHW;
         return (unsigned) (img * (int) p.c_img_stride + pix) * (unsigned) esz;
     }
@@ -300,21 +307,23 @@ __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
 
 // Writes the accumulators of one wavefront.  Lane (li, lh) of a 32x32 block holds column li and rows
 // 8*(r/4) + 4*lh + (r%4): the column and the 4*lh part of the row go in the vector offset, the rest
-// of the row (uniform) in the scalar offset.
+// of the row (uniform) in the scalar offset.  Per-row operands (bias, weight_aux, int32 bias) are all
+// requested before the first one is used, through descriptors that are empty when the operand is
+// absent, so the epilogue has one memory round trip and no branches.
 template <int DT, int EPI, int TM, int TN, class ACC>
 __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][TN], int batch, int m_wave, int n_wave,
                                            int li, int lh) {
     const int esz = (DT == DT_I8 && p.out_s8) ? 1 : 4;
     const rsrc_t rc = make_rsrc(reinterpret_cast<const char *>(p.C) + (size_t) batch * p.c_batch_stride * esz,
                                 RSRC_RANGE);
-    const rsrc_t rbias = make_rsrc(p.bias, p.bias ? (unsigned) ((p.bias_mode == BIAS_N ? p.N : p.M) * 4) : 0u);
-    const rsrc_t raux = make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u);
-    const rsrc_t rb32 = make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u);
-    const rsrc_t racc = make_rsrc(p.acc_out ? p.acc_out + (size_t) batch * p.c_batch_stride : nullptr, RSRC_RANGE);
+    const bool bias_m_on = p.bias_mode == BIAS_M, bias_n_on = p.bias_mode == BIAS_N;
+    const rsrc_t rbias_m = make_rsrc(p.bias, bias_m_on ? (unsigned) (p.M * 4) : 0u);
+    const rsrc_t rbias_n = make_rsrc(p.bias, bias_n_on ? (unsigned) (p.N * 4) : 0u);
     const bool m_edge = m_wave + TM * 32 > p.M;   // uniform: only the last row tile checks rows
     const unsigned row_bytes = (unsigned) p.c_stride_m * (unsigned) esz;
+    const unsigned lh16 = (unsigned) lh * 16u;    // rows of the upper half wavefront are 4 further down
 
-    unsigned col_voff[TN], col_voff4[TN];
+    unsigned col_voff[TN];
     float bias_n[TN];
 #pragma unroll
     for (int b = 0; b < TN; ++b) {
@@ -322,48 +331,80 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
         const bool ok = n < p.N;
         const int nn = ok ? n : 0;
         col_voff[b] = ok ? out_col_offset(p, nn, esz) + (unsigned) (4 * lh) * row_bytes : OOB;
-        col_voff4[b] = ok ? out_col_offset(p, nn, 4) + (unsigned) (4 * lh) * (unsigned) p.c_stride_m * 4u : OOB;
-        bias_n[b] = (p.bias_mode == BIAS_N) ? buf_load_f32(rbias, (unsigned) nn * 4u, 0) : 0.0f;
+        bias_n[b] = buf_load_f32(rbias_n, (unsigned) nn * 4u, 0);
     }
+    if constexpr (DT == DT_I8) {
+        const rsrc_t raux = make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u);
+        const rsrc_t rb32 = make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u);
+        const rsrc_t racc = make_rsrc(p.acc_out ? p.acc_out + (size_t) batch * p.c_batch_stride : nullptr,
+                                      p.acc_out ? RSRC_RANGE : 0u);
+        const unsigned row_bytes4 = (unsigned) p.c_stride_m * 4u;
+        float aux[TM][16];
+        int b32[TM][16];
 #pragma unroll
-    for (int a = 0; a < TM; ++a) {
+        for (int a = 0; a < TM; ++a)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);   // row of lanes with lh == 0
-            const int m = m_uni + 4 * lh;
-            const bool row_ok = !m_edge || m < p.M;
-            const unsigned soff = (unsigned) m_uni * row_bytes;
-            if constexpr (DT == DT_I8) {
+            for (int r = 0; r < 16; ++r) {
+                const unsigned soff = (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u;
+                aux[a][r] = buf_load_f32(raux, lh16, soff);
+                b32[a][r] = (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
+            }
+        unsigned col_voff4[TN];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+            const int n = n_wave + b * 32 + li;
+            col_voff4[b] = n < p.N ? out_col_offset(p, n, 4) + (unsigned) (4 * lh) * row_bytes4 : OOB;
+        }
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
+                const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
                 // conv.c:1041-1056: acc * s, + bias, * (aux / 127): three separately rounded operations
-                const float coeff = __fdiv_rn(buf_load_f32(raux, (unsigned) m * 4u, 0), 127.0f);
-                const float fb = p.bias32 ? (float) (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, (unsigned) m * 4u, 0, 0) : 0.0f;
+                const float coeff = __fdiv_rn(aux[a][r], 127.0f);
+                const float fb = (float) b32[a][r];
 #pragma unroll
                 for (int b = 0; b < TN; ++b) {
                     const int av = acc[a][b][r];
-                    const unsigned voff = row_ok ? col_voff[b] : OOB;
-                    if (p.acc_out)
-                        __builtin_amdgcn_raw_buffer_store_b32((unsigned) av, racc, row_ok ? col_voff4[b] : OOB,
-                                                              (unsigned) m_uni * (unsigned) p.c_stride_m * 4u, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32((unsigned) av, racc, row_ok ? col_voff4[b] : OOB,
+                                                          (unsigned) m_uni * row_bytes4, 0);
                     float f = __fmul_rn((float) av, p.in_scale);
-                    if (p.bias32) f = __fadd_rn(f, fb);
+                    const float fbias = __fadd_rn(f, fb);
+                    f = p.bias32 ? fbias : f;
                     const float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
+                    const unsigned voff = row_ok ? col_voff[b] : OOB;
                     if (p.out_s8)
-                        __builtin_amdgcn_raw_buffer_store_b8((unsigned char) requant_s8(y, p.out_inv_scale), rc, voff, soff, 0);
+                        __builtin_amdgcn_raw_buffer_store_b8((unsigned char) requant_s8(y, p.out_inv_scale), rc, voff,
+                                                             (unsigned) m_uni * row_bytes, 0);
                     else
-                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), rc, voff, soff, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), rc, voff, (unsigned) m_uni * row_bytes, 0);
                 }
-            } else {
-                const float bias_m = (p.bias_mode == BIAS_M) ? buf_load_f32(rbias, (unsigned) m * 4u, 0) : 0.0f;
+            }
+    } else {
+        float bias_m[TM][16];
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                bias_m[a][r] = buf_load_f32(rbias_m, lh16, (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u);
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);   // row of lanes with lh == 0
+                const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
 #pragma unroll
                 for (int b = 0; b < TN; ++b) {
                     float v = acc[a][b][r];
-                    if (p.bias_mode == BIAS_M) v = __fadd_rn(v, bias_m);        // bias after the full sum
-                    else if (p.bias_mode == BIAS_N) v = __fadd_rn(v, bias_n[b]);
+                    // bias after the full sum; absent bias must not touch the value (the sign of a zero sum)
+                    const float vm = __fadd_rn(v, bias_m[a][r]), vn = __fadd_rn(v, bias_n[b]);
+                    v = bias_m_on ? vm : bias_n_on ? vn : v;
                     v = act_fast<EPI>(v, p.ep);
-                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff[b] : OOB, soff, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff[b] : OOB,
+                                                          (unsigned) m_uni * row_bytes, 0);
                 }
             }
-        }
     }
 }
 
@@ -425,7 +466,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
         lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
     }
-    const int tile_m = lid % tiles_m, tile_n = lid / tiles_m;
+    const int tile_n = (int) div31((unsigned) lid, p.div_tiles_m), tile_m = lid - tile_n * tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int batch = blockIdx.z;
     const int u_begin = blockIdx.y * p.k_split_units;
@@ -433,13 +474,17 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     const int k_tiles = (u_end - u_begin + UPT - 1) / UPT;
     const int klim = min(p.K, u_end * KPU);
 
+    // The last K tile of this slice is ragged when it is cut by the end of K or of the slice; only then do
+    // loads and LDS stores test reduction indices one by one (the CHK variants below).
+    const bool ragged = ((u_end - u_begin) % UPT) != 0 || klim < u_end * KPU;
+
     // exact extent: the dwords of a row-end vector that fall past the matrix read as zero
-    const rsrc_t ra = make_rsrc(reinterpret_cast<const char *>(p.A) + (size_t) batch * p.a_batch_stride * ESZ,
-                                (unsigned) p.a_slice_bytes);
+    const char *a_base = reinterpret_cast<const char *>(p.A) + (size_t) batch * p.a_batch_stride * ESZ;
     // the B buffer starts pad rows/columns before the tensor so that pixel offsets are never negative
     // and ends with the tensor: channel padding of the last image reads as zero
-    const rsrc_t rb = make_rsrc(reinterpret_cast<const char *>(p.B) + (size_t) batch * p.b_batch_stride * ESZ -
-                                    (size_t) p.b_shift_bytes, (unsigned) (p.b_slice_bytes + p.b_shift_bytes));
+    const char *b_base = reinterpret_cast<const char *>(p.B) + (size_t) batch * p.b_batch_stride * ESZ -
+                         (size_t) p.b_shift_bytes;
+    const unsigned a_bytes = (unsigned) p.a_slice_bytes, b_bytes = (unsigned) (p.b_slice_bytes + p.b_shift_bytes);
 
     // per-thread A slots: (row, unit-in-tile) fixed for the whole K loop
     unsigned a_voff[A_PER_T];
@@ -482,17 +527,23 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         const int t = idx / BE, e = idx % BE;
         bp[idx] = prep_b<DT, BL>(p, u_begin + kt * UPT + b_unit_of(t), e, klim);
     };
-    // issue every global load of K tile kt (B descriptions must have been prepared for kt)
-    auto issue = [&](int kt) {
+    // issue every global load of K tile kt (B descriptions must have been prepared for kt).  A tile past the
+    // end of the slice is switched off as a whole through empty buffer descriptors (a scalar select): its
+    // loads return zero without touching memory.  CHK adds the per-unit tests a ragged last tile needs.
+    auto issue = [&](int kt, auto chk) {
+        constexpr bool CHK = decltype(chk)::value;
         const int ub = u_begin + kt * UPT;
+        const bool live = kt < k_tiles;
+        const rsrc_t ra = make_rsrc(a_base, live ? a_bytes : 0u);
+        const rsrc_t rb = make_rsrc(b_base, live ? b_bytes : 0u);
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t)
-            load_a_unit<DT>(qa[t], ra, a_voff[t], (unsigned) (ub * KPU * ESZ), (ub + a_unit[t]) * KPU, klim);
+            load_a_unit<DT, CHK>(qa[t], ra, a_voff[t], (unsigned) (ub * KPU * ESZ), (ub + a_unit[t]) * KPU, klim);
 #pragma unroll
         for (int t = 0; t < B_PER_T; ++t) {
             const int u = ub + b_unit_of(t);
             if constexpr (BL == BL_KVEC) {
-                const uint4 q = buf_load_b128(rb, b_voff<BL>(p, col, bp[t], u), bp[t].soff);
+                const uint4 q = buf_load_b128(rb, b_voff<BL, CHK>(p, col, bp[t], u), bp[t].soff);
                 if constexpr (DT == DT_I8) qb[t].q = q;
                 else {
                     qb[t].v[0] = __uint_as_float(q.x); qb[t].v[1] = __uint_as_float(q.y);
@@ -500,22 +551,23 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
                 }
             } else if constexpr (BL == BL_TAPC) {
                 // the unit's KPU channels share the filter tap: one validity test, channel stride in the scalar offset
-                const unsigned voff = b_voff<BL>(p, col, bp[t], u);
+                const unsigned voff = b_voff<BL, CHK>(p, col, bp[t], u);
 #pragma unroll
                 for (int e = 0; e < KPU; ++e) qb[t].v[e] = buf_load_f32(rb, voff, bp[t].soff + (unsigned) e * hw4);
             } else {
 #pragma unroll
                 for (int e = 0; e < KPU; ++e)
-                    qb[t].v[e] = buf_load_f32(rb, b_voff<BL>(p, col, bp[t * KPU + e], u * KPU + e), bp[t * KPU + e].soff);
+                    qb[t].v[e] = buf_load_f32(rb, b_voff<BL, CHK>(p, col, bp[t * KPU + e], u * KPU + e), bp[t * KPU + e].soff);
             }
         }
     };
-    auto stage = [&](int buf, int kt) {
+    auto stage = [&](int buf, int kt, auto chk) {
+        constexpr bool CHK = decltype(chk)::value;
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t) {
             const int f = tid + t * THREADS;
             const int ml = f / UPT, ua = f % UPT;
-            clear_a_tail<DT>(qa[t], (u_begin + kt * UPT + a_unit[t]) * KPU, klim);
+            if constexpr (CHK) clear_a_tail<DT>(qa[t], (u_begin + kt * UPT + a_unit[t]) * KPU, klim);
             if ((A_SLOTS % THREADS == 0) || f < A_SLOTS) lds[buf][ua * BM + ml] = pack_unit<DT>(qa[t]);
         }
 #pragma unroll
@@ -539,20 +591,22 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     // memory, and a global load has a whole tile of MFMAs to complete.  Past the last tile loads are
     // fully masked (zero, no memory traffic), so the body has no branches.
     Operands op0, op1;
+    constexpr std::true_type CHECKED{};
+    constexpr std::false_type UNCHECKED{};
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(0, i);
-    issue(0);
-    stage(0, 0);
+    issue(0, CHECKED);
+    stage(0, 0, CHECKED);
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(1, i);
-    issue(1);
+    issue(1, CHECKED);
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(2, i);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < READS; ++i) read_operand(op0, 0, i);
 
-    auto body = [&](Operands &cur, Operands &nxt, int kt) {
+    auto body = [&](Operands &cur, Operands &nxt, int kt, auto chk) {
         const int nbuf = (kt + 1) & 1;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -561,8 +615,8 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             const int s = blk / (TM * TN), a = (blk / TN) % TM, b = blk % TN;
             Traits<DT>::mma_part(acc[a][b], cur.a[s][a], cur.b[s][b], part);
             if (st == 0) {
-                stage(nbuf, kt + 1);
-                issue(kt + 2);
+                stage(nbuf, kt + 1, chk);
+                issue(kt + 2, chk);
             }
 #pragma unroll
             for (int i = 0; i < B_ITEMS; ++i)
@@ -576,12 +630,20 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // Body kt stores tile kt+1 to LDS and loads tile kt+2; the ragged tile k_tiles-1 is therefore touched by
+    // bodies k_tiles-3 and k_tiles-2.  Everything before runs without per-element tests (an even count, so the
+    // two operand sets keep their roles).
+    const int n_plain = (ragged ? max(0, k_tiles - 3) : k_tiles) & ~1;
     int kt = 0;
-    for (; kt + 1 < k_tiles; kt += 2) {
-        body(op0, op1, kt);
-        body(op1, op0, kt + 1);
+    for (; kt < n_plain; kt += 2) {
+        body(op0, op1, kt, UNCHECKED);
+        body(op1, op0, kt + 1, UNCHECKED);
     }
-    if (kt < k_tiles) body(op0, op1, kt);
+    for (; kt + 1 < k_tiles; kt += 2) {
+        body(op0, op1, kt, CHECKED);
+        body(op1, op0, kt + 1, CHECKED);
+    }
+    if (kt < k_tiles) body(op0, op1, kt, CHECKED);
 
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
     if (p.partial) {
@@ -631,8 +693,13 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p,
 
 // ---- launch ------------------------------------------------------------------------------------------
 template <int DT, int BL, int BM, int BN, int WM, int WN>
-static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
-    const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream_t stream) {
+    IgemmParams p = p_in;
+    const int tiles_m = (p.M + BM - 1) / BM;
+    const int tiles = tiles_m * ((p.N + BN - 1) / BN);
+    p.div_ohw = make_div31((unsigned) (p.OHW > 0 ? p.OHW : 1));
+    p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
+    p.div_tiles_m = make_div31((unsigned) tiles_m);
     dim3 grid(tiles, cfg.split, cfg.batch);
     hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN>), grid, dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());

@@ -100,8 +100,24 @@ enum { OUT_CONV = 0,   // n = img * OHW + pix  ->  img * c_img_stride + m * c_st
 
 enum { BIAS_NONE = 0, BIAS_M = 1, BIAS_N = 2 };
 
+// floor(x / d) for 0 <= x < 2^31 as (mulhi(x, magic) >> shift) + (x & pass): with L = ceil(log2 d),
+// magic = floor(2^(31+L) / d) + 1 and shift = L - 1 the quotient is exact; d == 1 is magic 0, pass ~0.
+struct Div31 {
+    unsigned magic, shift, pass;
+};
+inline Div31 make_div31(unsigned d) {
+    Div31 r = {0u, 0u, 0xFFFFFFFFu};
+    if (d <= 1) return r;
+    unsigned L = 0;
+    while ((1ull << L) < d) ++L;
+    r.magic = (unsigned) ((1ull << (31 + L)) / d) + 1u;
+    r.shift = L - 1;
+    r.pass = 0;
+    return r;
+}
+
 struct IgemmParams {
-    int M, N, K;               // K counts real reduction elements (gather) or padded units*kpu (kvec)
+    int M, N, K;              // K counts real reduction elements (gather) or padded units*kpu (kvec)
     int k_units;               // 16-byte units along K (multiple of 2 per MFMA step is NOT required)
     int k_split_units;         // units handled by one blockIdx.y slice (split-K); == k_units if unsplit
     // A
@@ -141,6 +157,8 @@ struct IgemmParams {
     float out_inv_scale;       // 1.0f / output_scale
     // split-K workspace: partial sums [split][M][N] fp32 (nullptr when unsplit)
     float *partial;
+    // exact division of any x < 2^31 by OHW, OW and the number of row tiles (filled in by the launcher)
+    Div31 div_ohw, div_ow, div_tiles_m;
 };
 
 enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2, DT_I8 = 3 };
