@@ -160,6 +160,46 @@ def test_conv_f32_batched(name, batch, torch_dev, oracle):
         assert_close_f32(y, ref, tag=name)
 
 
+@pytest.mark.parametrize("tile", ["64x64x1", "64x64x3", "32x128x2", "64x128x5", "128x128x4", "128x128x1"])
+@pytest.mark.parametrize("kind", ["1x1_ragged_k", "3x3_packed"])
+def test_forced_tile_and_split_many_items(tile, kind, torch_dev, oracle, monkeypatch):
+    """every tile shape, with and without split-K, on problems with more work items than resident
+    workgroups (each workgroup walks through several tiles) and a K that ends inside a K tile;
+    run twice: the split-K arrival counters must be back at zero after a launch"""
+    torch = torch_dev
+    if kind == "1x1_ragged_k":
+        d = cases.cd(198, 96, 1, 1, 0, 48, n=24, act=abi.RELU)         # K = 198: ragged, odd
+    else:
+        d = cases.cd(24, 80, 3, 1, 1, 40, n=40, act=abi.CLIP, clip_min=-0.5, clip_max=0.7)
+    x, w, b = cases.conv_inputs("forced_" + kind, d)
+    ref = oracle.conv2d_f32(d, x, w, b, cases.silu_lut())
+    monkeypatch.setenv("ONHIP_TILE", tile)
+    xd, wd, bd = dev(torch, x), dev(torch, w), dev(torch, b)
+    wp = hip.pack_conv_weights(d, wd) if kind == "3x3_packed" else None
+    for rep in range(2):
+        if wp is not None:
+            y = hip.conv2d_f32(d, xd, wp, bd, packed=True)
+        else:
+            y = hip.conv2d_f32(d, xd, wd, bd)
+        torch.cuda.synchronize()
+        assert_close_f32(y.cpu().numpy(), ref, tag=f"{kind} {tile} run {rep}")
+
+
+@pytest.mark.parametrize("tile", ["64x64x4", "128x128x2", "32x128x1"])
+def test_forced_split_w8a32_bit_exact(tile, torch_dev, oracle, monkeypatch):
+    """integer partial sums add up exactly whatever the split"""
+    torch = torch_dev
+    d = ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()["q3x3_silu"])
+    d.n = 6
+    x, w8, b32, aux = cases.conv_inputs("q_forced_split", d, quant=True)
+    ref = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut())
+    monkeypatch.setenv("ONHIP_TILE", tile)
+    for rep in range(2):
+        y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()))
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy(), ref), f"{tile} run {rep}"
+
+
 def test_conv_w8a32_batched(torch_dev, oracle):
     torch = torch_dev
     d = ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()["q3x3_s2_odd"])
