@@ -659,32 +659,30 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     }
 }
 
-// sums the split-K partials in slice order and applies the epilogue (one thread per output element)
+// sums the split-K partials in slice order and applies the epilogue: one thread per output element; a
+// workgroup is 64 columns x 4 rows (one wavefront per row) and the grid (column blocks, row blocks, batch),
+// so no index has to be divided
 template <bool IS_INT>
 __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p, int split, int batches) {
-    const long long total = (long long) batches * p.M * p.N;
-    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int n = (int) (idx % p.N);
-    const long long t = idx / p.N;
-    const int m = (int) (t % p.M);
-    const int batch = (int) (t / p.M);
-    const int esz = (IS_INT && p.out_s8) ? 1 : 4;
+    const int n = blockIdx.x * 64 + threadIdx.x;
+    const int m = blockIdx.y * 4 + threadIdx.y, batch = blockIdx.z;
+    if (n >= p.N || m >= p.M) return;
+    const size_t slice = (size_t) batches * p.M * p.N;                    // elements per K slice
+    const size_t idx = ((size_t) batch * p.M + m) * p.N + n;
     const size_t off4 = (size_t) batch * p.c_batch_stride + (size_t) m * p.c_stride_m + out_col_offset(p, n, 1);
     char *cbase = reinterpret_cast<char *>(p.C);
     if constexpr (IS_INT) {
         int acc = 0;
-        for (int s = 0; s < split; ++s) acc += reinterpret_cast<const int *>(p.partial)[(size_t) s * total + idx];
+        for (int s = 0; s < split; ++s) acc += reinterpret_cast<const int *>(p.partial)[(size_t) s * slice + idx];
         if (p.acc_out) p.acc_out[off4] = acc;
         float f = __fmul_rn((float) acc, p.in_scale);
         if (p.bias32) f = __fadd_rn(f, (float) p.bias32[m]);
         const float y = apply_act(__fmul_rn(f, __fdiv_rn(p.weight_aux[m], 127.0f)), p.ep);
         if (p.out_s8) reinterpret_cast<int8_t *>(cbase)[off4] = (int8_t) requant_s8(y, p.out_inv_scale);
         else reinterpret_cast<float *>(cbase)[off4] = y;
-        (void) esz;
     } else {
         float acc = 0.0f;
-        for (int s = 0; s < split; ++s) acc = __fadd_rn(acc, p.partial[(size_t) s * total + idx]);
+        for (int s = 0; s < split; ++s) acc = __fadd_rn(acc, p.partial[(size_t) s * slice + idx]);
         if (p.bias_mode == BIAS_M) acc = __fadd_rn(acc, p.bias[m]);
         else if (p.bias_mode == BIAS_N) acc = __fadd_rn(acc, p.bias[n]);
         reinterpret_cast<float *>(cbase)[off4] = apply_act(acc, p.ep);
@@ -704,12 +702,13 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN>), grid, dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
     if (p.partial) {
-        const long long total = (long long) cfg.batch * p.M * p.N;
-        const int blocks = (int) ((total + 255) / 256);
+        if (p.M > 4 * 65535 || cfg.batch > 65535)
+            return set_error(ONHIP_ERR_ARG, "igemm: split-K with %d rows, %d batches", p.M, cfg.batch);
+        const dim3 fgrid((p.N + 63) / 64, (p.M + 3) / 4, cfg.batch);
         if (DT == DT_I8)
-            hipLaunchKernelGGL((splitk_finish_kernel<true>), dim3(blocks), dim3(256), 0, stream, p, cfg.split, cfg.batch);
+            hipLaunchKernelGGL((splitk_finish_kernel<true>), fgrid, dim3(64, 4), 0, stream, p, cfg.split, cfg.batch);
         else
-            hipLaunchKernelGGL((splitk_finish_kernel<false>), dim3(blocks), dim3(256), 0, stream, p, cfg.split, cfg.batch);
+            hipLaunchKernelGGL((splitk_finish_kernel<false>), fgrid, dim3(64, 4), 0, stream, p, cfg.split, cfg.batch);
         ONHIP_CHECK_HIP(hipGetLastError());
     }
     return ONHIP_OK;
