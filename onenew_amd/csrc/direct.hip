@@ -6,29 +6,30 @@
 namespace onhip {
 
 
-// ---- NCHW fp32 -> NHWC int8, channels zero-padded to cp (a multiple of 16) -----------------------------
-// One thread quantises 16 channels of one pixel: 16 loads that are each coalesced along the pixel
-// index, one 16-byte store.
+// ---- fp32 NCHW activations -> int8 NHWC with the channel count padded to cp (a multiple of 16) -------------
+// One thread quantises the 16 channels of one 16-byte block of one pixel (conv.c:961-973 per element).  A
+// wavefront covers CBW neighbouring channel blocks of 64 / CBW consecutive pixels, so its stores are runs of
+// CBW * 16 contiguous bytes per pixel (whole pixels when cp <= 64) and each of its 16 loads reads runs of
+// 64 / CBW consecutive pixels of a channel plane.  Grid: (pixel blocks, channel block groups, images).
+template <int CBW>
 __global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float *x, int c, int hw, int cp, float inv_scale,
-                                                            int8_t *q, long long total) {
-    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;  // (img, cblock, pix), pix fastest
-    if (idx >= total) return;
-    const int cblocks = cp / 16;
-    const int pix = (int) (idx % hw);
-    const long long t = idx / hw;
-    const int cb = (int) (t % cblocks);
-    const long long img = t / cblocks;
+                                                            int8_t *q) {
+    constexpr int PIXW = 64 / CBW;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pix = (blockIdx.x * 4 + wave) * PIXW + lane / CBW;
+    const int cb = blockIdx.y * CBW + lane % CBW;
+    if (pix >= hw || cb * 16 >= cp) return;
+    const long long img = blockIdx.z;
     const float *src = x + (img * c + (long long) cb * 16) * hw + pix;
+    float v[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = cb * 16 + e < c ? src[(long long) e * hw] : 0.0f;
     unsigned out[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         unsigned word = 0;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int ch = cb * 16 + g * 4 + e;
-            const int v = ch < c ? quant_s8(src[(long long) (g * 4 + e) * hw], inv_scale) : 0;
-            word |= ((unsigned) v & 0xffu) << (8 * e);
-        }
+        for (int e = 0; e < 4; ++e) word |= ((unsigned) quant_s8(v[g * 4 + e], inv_scale) & 0xffu) << (8 * e);
         out[g] = word;
     }
     *reinterpret_cast<uint4 *>(q + (img * hw + pix) * (long long) cp + cb * 16) = make_uint4(out[0], out[1], out[2], out[3]);
@@ -36,11 +37,13 @@ __global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float *x, int 
 
 int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
                          hipStream_t stream) {
-    const long long total = (long long) n * (cp / 16) * h * w;
-    const long long blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "quantize: tensor too large");
-    hipLaunchKernelGGL(quantize_nhwc_kernel, dim3((unsigned) blocks), dim3(256), 0, stream, x, c, h * w, cp, inv_scale,
-                       q, total);
+    const int hw = h * w, cblocks = cp / 16;
+    if (n > 65535) return set_error(ONHIP_ERR_ARG, "quantize: batch of %d", n);
+    const int cbw = cblocks >= 4 ? 4 : cblocks >= 2 ? 2 : 1;
+    const dim3 grid((hw + 4 * (64 / cbw) - 1) / (4 * (64 / cbw)), (cblocks + cbw - 1) / cbw, n);
+    if (cbw == 4) hipLaunchKernelGGL(quantize_nhwc_kernel<4>, grid, dim3(256), 0, stream, x, c, hw, cp, inv_scale, q);
+    else if (cbw == 2) hipLaunchKernelGGL(quantize_nhwc_kernel<2>, grid, dim3(256), 0, stream, x, c, hw, cp, inv_scale, q);
+    else hipLaunchKernelGGL(quantize_nhwc_kernel<1>, grid, dim3(256), 0, stream, x, c, hw, cp, inv_scale, q);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }

@@ -46,7 +46,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int UPT = 4;        // 16-byte units per K tile
 constexpr int THREADS = 256;
 constexpr unsigned OOB = 0x80000000u;       // vector offset outside every buffer: loads give 0, stores vanish
 constexpr unsigned RSRC_RANGE = 0x80000000u; // num_records of the data buffers (all offsets stay below 2 GiB)
@@ -443,13 +442,17 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     static_assert(THREADS % BN == 0 || BN % THREADS == 0, "B loader mapping");
     constexpr int KPU = Traits<DT>::KPU;
     constexpr int ESZ = DT == DT_I8 ? 1 : 4;   // bytes per stored operand element
+    constexpr int UPT = 4;                     // 16-byte units per K tile
     constexpr int A_SLOTS = BM * UPT, B_SLOTS = BN * UPT;
+    // A reaches LDS from threads that hold the UPT units of one row side by side: one spare slot per unit row
+    // puts those UPT stores in different banks
+    constexpr int A_LD = BM + 1, A_LDS = A_LD * UPT;
     constexpr int A_PER_T = (A_SLOTS + THREADS - 1) / THREADS;
     constexpr int B_PER_T = B_SLOTS / THREADS;
     static_assert(B_PER_T >= 1, "BN >= 64");
     typedef typename Traits<DT>::acc_t acc_t;
 
-    __shared__ uint4 lds[2][A_SLOTS + B_SLOTS];
+    __shared__ uint4 lds[2][A_LDS + B_SLOTS];
 
     const int tid = threadIdx.x;
     // the wavefront index is uniform; saying so keeps everything derived from it in scalar registers
@@ -568,18 +571,18 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             const int f = tid + t * THREADS;
             const int ml = f / UPT, ua = f % UPT;
             if constexpr (CHK) clear_a_tail<DT>(qa[t], (u_begin + kt * UPT + a_unit[t]) * KPU, klim);
-            if ((A_SLOTS % THREADS == 0) || f < A_SLOTS) lds[buf][ua * BM + ml] = pack_unit<DT>(qa[t]);
+            if ((A_SLOTS % THREADS == 0) || f < A_SLOTS) lds[buf][ua * A_LD + ml] = pack_unit<DT>(qa[t]);
         }
 #pragma unroll
         for (int t = 0; t < B_PER_T; ++t) {
             const int f = tid + t * THREADS;
-            lds[buf][A_SLOTS + (f / BN) * BN + (f % BN)] = pack_unit<DT>(qb[t]);
+            lds[buf][A_LDS + (f / BN) * BN + (f % BN)] = pack_unit<DT>(qb[t]);
         }
     };
     auto read_operand = [&](Operands &o, int buf, int idx) {   // idx-th of the READS LDS reads
         const int s = idx / (TM + TN), t = idx % (TM + TN);
-        if (t < TM) o.a[s][t] = lds[buf][(2 * s + lh) * BM + wm * (BM / WM) + t * 32 + li];
-        else o.b[s][t - TM] = lds[buf][A_SLOTS + (2 * s + lh) * BN + wn * (BN / WN) + (t - TM) * 32 + li];
+        if (t < TM) o.a[s][t] = lds[buf][(2 * s + lh) * A_LD + wm * (BM / WM) + t * 32 + li];
+        else o.b[s][t - TM] = lds[buf][A_LDS + (2 * s + lh) * BN + wn * (BN / WN) + (t - TM) * 32 + li];
     };
 
     // Pipeline.  While the MFMAs of K tile kt run (its operands are already in registers):

@@ -59,6 +59,7 @@ static uint64_t fingerprint(const void *host, size_t bytes) {
 struct PackedEntry {
     float *dev;
     size_t bytes;
+    bool int8;
 };
 static std::map<const void *, PackedEntry> g_packed;
 
@@ -72,18 +73,20 @@ static void drop_packed(const void *w_dev) {
 // *out = packed copy of the device weights w_dev for convolution d, or nullptr if d takes them as they are.
 // A weight that lives in device memory is packed when first seen; after changing it in place call
 // onhip_plugin_release().
-static int packed_weights(const onhip_conv_desc_t *d, const float *w_dev, const float **out) {
+static int packed_weights(const onhip_conv_desc_t *d, const float *w_dev, const float **out, bool int8 = false) {
     *out = nullptr;
-    const size_t bytes = onhip_conv2d_packed_weight_bytes(d);
+    const size_t bytes = int8 ? onhip_conv2d_w8a32_packed_weight_bytes(d) : onhip_conv2d_packed_weight_bytes(d);
     if (!bytes) return ONHIP_OK;
     auto it = g_packed.find(w_dev);
-    if (it != g_packed.end() && it->second.bytes == bytes) { *out = it->second.dev; return ONHIP_OK; }
+    if (it != g_packed.end() && it->second.bytes == bytes && it->second.int8 == int8) { *out = it->second.dev; return ONHIP_OK; }
     drop_packed(w_dev);
     float *p = nullptr;
     ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&p), bytes));
-    int rc = onhip_conv2d_pack_weights(d, w_dev, p, nullptr);
+    int rc = int8 ? onhip_conv2d_w8a32_pack_weights(d, reinterpret_cast<const int8_t *>(w_dev),
+                                                    reinterpret_cast<int8_t *>(p), nullptr)
+                  : onhip_conv2d_pack_weights(d, w_dev, p, nullptr);
     if (rc) { (void) hipFree(p); return rc; }
-    g_packed[w_dev] = PackedEntry{p, bytes};
+    g_packed[w_dev] = PackedEntry{p, bytes, int8};
     *out = p;
     return ONHIP_OK;
 }
@@ -239,8 +242,16 @@ static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
             rc = stage_buf(3, ws_bytes, &ws);
             if (rc) return rc;
         }
-        rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
-                                (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
+        // dense int8 weights are re-laid out for the kernel once, next to their device copy
+        const float *wp = nullptr;
+        rc = packed_weights(&d, (const float *) w, &wp, true);
+        if (rc) return rc;
+        if (wp)
+            rc = onhip_conv2d_w8a32_packed(&d, (const float *) x, (const int8_t *) wp, (const int32_t *) b,
+                                           (const float *) aux, (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
+        else
+            rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
+                                    (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
     } else {
         // k x k dense weights are re-laid out tap-major once, next to their device copy
         const float *wp = nullptr;

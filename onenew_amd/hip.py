@@ -31,7 +31,8 @@ def plugin_path(op):
 
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
-           "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
+           "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
+           "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
 
 
@@ -55,6 +56,10 @@ def load():
     L.onhip_conv2d_w8a32_workspace.argtypes = [C.POINTER(ConvDesc)]
     L.onhip_conv2d_w8a32_workspace.restype = C.c_size_t
     L.onhip_conv2d_w8a32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
+    L.onhip_conv2d_w8a32_packed_weight_bytes.argtypes = [C.POINTER(ConvDesc)]
+    L.onhip_conv2d_w8a32_packed_weight_bytes.restype = C.c_size_t
+    L.onhip_conv2d_w8a32_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    L.onhip_conv2d_w8a32_packed.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
     L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
@@ -118,7 +123,19 @@ def conv2d_w8a32_workspace(d):
     return int(load().onhip_conv2d_w8a32_workspace(C.byref(d)))
 
 
-def conv2d_w8a32(d, x, w8, bias32, weight_aux, silu_lut=None, out=None, acc32=None, workspace=None):
+def pack_conv_weights_w8(d, w8):
+    """the int8 weights in the kernel's layout (None for depthwise, which reads the reference layout)"""
+    import torch
+    nbytes = int(load().onhip_conv2d_w8a32_packed_weight_bytes(C.byref(d)))
+    if nbytes == 0:
+        return None
+    packed = torch.empty(nbytes, dtype=torch.int8, device=w8.device)
+    _check(load().onhip_conv2d_w8a32_pack_weights(C.byref(d), _ptr(w8), _ptr(packed), _stream()),
+           "onhip_conv2d_w8a32_pack_weights")
+    return packed
+
+
+def conv2d_w8a32(d, x, w8, bias32, weight_aux, silu_lut=None, out=None, acc32=None, workspace=None, packed=False):
     import torch
     oh, ow = d.out_hw()
     if out is None:
@@ -127,9 +144,10 @@ def conv2d_w8a32(d, x, w8, bias32, weight_aux, silu_lut=None, out=None, acc32=No
     if workspace is None and need:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    _check(load().onhip_conv2d_w8a32(C.byref(d), _ptr(x), _ptr(w8), _ptr(bias32), _ptr(weight_aux), _ptr(silu_lut),
-                                     _ptr(out), _ptr(acc32), _ptr(workspace), nbytes, _stream()),
-           "onhip_conv2d_w8a32")
+    fn = load().onhip_conv2d_w8a32_packed if packed else load().onhip_conv2d_w8a32
+    _check(fn(C.byref(d), _ptr(x), _ptr(w8), _ptr(bias32), _ptr(weight_aux), _ptr(silu_lut),
+              _ptr(out), _ptr(acc32), _ptr(workspace), nbytes, _stream()),
+           "onhip_conv2d_w8a32_packed" if packed else "onhip_conv2d_w8a32")
     return out
 
 

@@ -130,6 +130,14 @@ def test_conv_w8a32_bit_exact(name, torch_dev, oracle, golden):
     y = y.cpu().numpy()
     assert np.array_equal(y, ref), f"{name}: {(y != ref).sum()} de-quantised outputs differ"
     cases.check_against(golden, name, y, exact=True)
+    # the same through weights laid out once for the kernel
+    wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
+    assert (wp is None) == (d.group != 1)
+    if wp is not None:
+        y2 = hip.conv2d_w8a32(d, dev(torch, x), wp, dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()),
+                              packed=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(y2.cpu().numpy(), ref), f"{name}: packed weights give other results"
 
 
 @pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_s2", "qdw3x3", "yolo_c2f_3x3_64_80"])
