@@ -447,12 +447,17 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     // A reaches LDS from threads that hold the UPT units of one row side by side: one spare slot per unit row
     // puts those UPT stores in different banks
     constexpr int A_LD = BM + 1, A_LDS = A_LD * UPT;
+    // The vector loader (BL_KVEC) gives the UPT units of one column to neighbouring lanes as well: they are
+    // contiguous in memory (one 64-byte run per pixel instead of 64 scattered 16-byte pieces per load), and the
+    // filter tap of a unit becomes a per-lane quantity.
+    constexpr bool LANE_UNITS = BL == BL_KVEC;
+    constexpr int B_LD = LANE_UNITS ? BN + 1 : BN, B_LDS = B_LD * UPT;
     constexpr int A_PER_T = (A_SLOTS + THREADS - 1) / THREADS;
     constexpr int B_PER_T = B_SLOTS / THREADS;
     static_assert(B_PER_T >= 1, "BN >= 64");
     typedef typename Traits<DT>::acc_t acc_t;
 
-    __shared__ uint4 lds[2][A_LDS + B_SLOTS];
+    __shared__ uint4 lds[2][A_LDS + B_LDS];
 
     const int tid = threadIdx.x;
     // the wavefront index is uniform; saying so keeps everything derived from it in scalar registers
@@ -500,8 +505,13 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         a_unit[t] = ua;
         a_voff[t] = ok ? (unsigned) ((m0 + ml) * p.lda + ua * KPU) * (unsigned) ESZ : OOB;
     }
-    // per-thread B column (same for all of its units)
-    const ColState col = make_col<BL>(p, n0 + (tid % BN));
+    // per-thread B column(s): one for all of the thread's units, or (LANE_UNITS) one per slot
+    constexpr int NCOL = LANE_UNITS ? B_PER_T : 1;
+    ColState cols[NCOL];
+#pragma unroll
+    for (int t = 0; t < NCOL; ++t)
+        cols[t] = make_col<BL>(p, n0 + (LANE_UNITS ? (tid + t * THREADS) / UPT : tid % BN));
+    const ColState &col = cols[0];
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -514,15 +524,15 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     RawUnit<DT> qa[A_PER_T], qb[B_PER_T];
 
     constexpr int PARTS = Traits<DT>::PARTS;
-    constexpr int BE = (BL == BL_KVEC || BL == BL_TAPC) ? 1 : KPU;   // scalar descriptions per B unit
-    constexpr int B_ITEMS = B_PER_T * BE;
+    constexpr int BE = BL == BL_TAPC ? 1 : KPU;                      // scalar descriptions per B unit
+    constexpr int B_ITEMS = LANE_UNITS ? 0 : B_PER_T * BE;
     constexpr int BLOCKS = (UPT / 2) * TM * TN;       // 32x32 blocks x unit pairs per K tile
     constexpr int STEPS = BLOCKS * PARTS;             // MFMA instructions per K tile and wavefront
     constexpr int HALF = STEPS / 2;
     constexpr int READS = (UPT / 2) * (TM + TN);      // LDS operand reads per K tile and wavefront
     struct Operands { uint4 a[UPT / 2][TM], b[UPT / 2][TN]; };
 
-    BPrep bp[B_ITEMS];                                // scalar descriptions of the next B loads
+    BPrep bp[B_ITEMS > 0 ? B_ITEMS : 1];              // scalar descriptions of the next B loads
     const unsigned hw4 = (unsigned) p.HW * 4u;
 
     auto b_unit_of = [&](int t) { return __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN); };
@@ -542,25 +552,46 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t)
             load_a_unit<DT, CHK>(qa[t], ra, a_voff[t], (unsigned) (ub * KPU * ESZ), (ub + a_unit[t]) * KPU, klim);
+        if constexpr (LANE_UNITS) {
+            // this lane's unit: filter tap and channel block, then one 16-byte load per column
+            const unsigned u = (unsigned) ub + (unsigned) (tid % UPT);
+            const unsigned tap = fast_div(u, p.magic_upt, p.pass_upt);
+            const unsigned cb = u - tap * (unsigned) p.units_per_tap;
+            const unsigned ti = fast_div(tap, p.magic_kw, p.pass_kw);
+            const unsigned tj = tap - ti * (unsigned) p.kw;
+            const unsigned off = (ti * (unsigned) p.W + tj) * (unsigned) p.pix_stride + cb * 16u;
+            const bool k_ok = !CHK || (int) (u * KPU) < klim;
 #pragma unroll
-        for (int t = 0; t < B_PER_T; ++t) {
-            const int u = ub + b_unit_of(t);
-            if constexpr (BL == BL_KVEC) {
-                const uint4 q = buf_load_b128(rb, b_voff<BL, CHK>(p, col, bp[t], u), bp[t].soff);
+            for (int t = 0; t < B_PER_T; ++t) {
+                bool ok = k_ok;
+                if (p.use_tapmask) {
+                    const unsigned word = tap >= 32u ? cols[t].mask_hi : cols[t].mask_lo;
+                    ok = ok && ((word >> (tap & 31u)) & 1u);
+                } else {
+                    ok = ok && (unsigned) (cols[t].ih0 + (int) ti) < (unsigned) p.H &&
+                         (unsigned) (cols[t].iw0 + (int) tj) < (unsigned) p.W;
+                }
+                const uint4 q = buf_load_b128(rb, ok ? cols[t].pixoff + off : OOB, 0);
                 if constexpr (DT == DT_I8) qb[t].q = q;
                 else {
                     qb[t].v[0] = __uint_as_float(q.x); qb[t].v[1] = __uint_as_float(q.y);
                     qb[t].v[2] = __uint_as_float(q.z); qb[t].v[3] = __uint_as_float(q.w);
                 }
-            } else if constexpr (BL == BL_TAPC) {
-                // the unit's KPU channels share the filter tap: one validity test, channel stride in the scalar offset
-                const unsigned voff = b_voff<BL, CHK>(p, col, bp[t], u);
+            }
+        } else {
 #pragma unroll
-                for (int e = 0; e < KPU; ++e) qb[t].v[e] = buf_load_f32(rb, voff, bp[t].soff + (unsigned) e * hw4);
-            } else {
+            for (int t = 0; t < B_PER_T; ++t) {
+                const int u = ub + b_unit_of(t);
+                if constexpr (BL == BL_TAPC) {
+                    // the unit's KPU channels share the filter tap: one validity test, channel stride in the scalar offset
+                    const unsigned voff = b_voff<BL, CHK>(p, col, bp[t], u);
 #pragma unroll
-                for (int e = 0; e < KPU; ++e)
-                    qb[t].v[e] = buf_load_f32(rb, b_voff<BL, CHK>(p, col, bp[t * KPU + e], u * KPU + e), bp[t * KPU + e].soff);
+                    for (int e = 0; e < KPU; ++e) qb[t].v[e] = buf_load_f32(rb, voff, bp[t].soff + (unsigned) e * hw4);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < KPU; ++e)
+                        qb[t].v[e] = buf_load_f32(rb, b_voff<BL, CHK>(p, col, bp[t * KPU + e], u * KPU + e), bp[t * KPU + e].soff);
+                }
             }
         }
     };
@@ -576,13 +607,14 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 #pragma unroll
         for (int t = 0; t < B_PER_T; ++t) {
             const int f = tid + t * THREADS;
-            lds[buf][A_LDS + (f / BN) * BN + (f % BN)] = pack_unit<DT>(qb[t]);
+            if constexpr (LANE_UNITS) lds[buf][A_LDS + (f % UPT) * B_LD + (f / UPT)] = pack_unit<DT>(qb[t]);
+            else lds[buf][A_LDS + (f / BN) * B_LD + (f % BN)] = pack_unit<DT>(qb[t]);
         }
     };
     auto read_operand = [&](Operands &o, int buf, int idx) {   // idx-th of the READS LDS reads
         const int s = idx / (TM + TN), t = idx % (TM + TN);
         if (t < TM) o.a[s][t] = lds[buf][(2 * s + lh) * A_LD + wm * (BM / WM) + t * 32 + li];
-        else o.b[s][t - TM] = lds[buf][A_LDS + (2 * s + lh) * BN + wn * (BN / WN) + (t - TM) * 32 + li];
+        else o.b[s][t - TM] = lds[buf][A_LDS + (2 * s + lh) * B_LD + wn * (BN / WN) + (t - TM) * 32 + li];
     };
 
     // Pipeline.  While the MFMAs of K tile kt run (its operands are already in registers):
