@@ -149,6 +149,32 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
 int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w,
                    const float *bias, float *out, void *stream);
 
+/* ---- offline quantisation: what produces the operands of onhip_conv2d_w8a32 ------------------ */
+
+/* Per output channel: weight_aux = max|w|, w8 = (int8)(w * 127 / aux) (truncating),
+ * bias32 = (int32)(b * 127 / aux).  Replaces quant_weight_bias,
+ * tools/optimize/model_quant.hpp:6-29.  Host arrays (runs once per model); bias may be NULL. */
+int onhip_quant_weight_bias(const float *w, const float *bias, int32_t cout, int32_t per_channel,
+                            int8_t *w8, int32_t *bias32, float *weight_aux);
+
+/* Activation-scale calibration, the data passes of quant_kl / quant_mse / quant_percent
+ * (model_quant.hpp:197-435, :437-623, :83-185) over device-resident activations x:
+ *  - onhip_calib_abs_max: *max_abs (host, in/out) = max(*max_abs, max|x|)          (:287-296)
+ *  - onhip_calib_histogram: adds the 2048-bin histogram of |x| over [0, max_abs] (zeros skipped) to
+ *    hist (host, ONHIP_CALIB_BINS floats, counted like the reference's float counters) (:325-332)
+ *  - onhip_calib_threshold: the clipping threshold from such a histogram; elem_count is the
+ *    reference's "elements per image x images"                                   (:345-431, :585-618)
+ *  - onhip_calib_percentile: x holds `images` tensors of `elems` values; the 99.998 % magnitude (:99-183)
+ * The layer's input_scale is threshold / 127 (model_quant.hpp:668).  All four synchronise. */
+#define ONHIP_CALIB_BINS 2048
+#define ONHIP_CALIB_KL 0
+#define ONHIP_CALIB_MSE 1
+int onhip_calib_abs_max(const float *x, long long n, float *max_abs, void *stream);
+int onhip_calib_histogram(const float *x, long long n, float max_abs, float *hist, void *stream);
+int onhip_calib_threshold(int method, const float *hist, long long elem_count, float max_abs,
+                          float *threshold);
+int onhip_calib_percentile(const float *x, int images, int elems, float *threshold, void *stream);
+
 /* Plain device-to-device copy of n floats (n % 4 == 0, 16-byte aligned).  A measuring aid with no
  * counterpart in the reference: HBM traffic counters of the other kernels are scaled by what the
  * same counters read for this copy of known size. */

@@ -32,7 +32,9 @@ def plugin_path(op):
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
-           "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
+           "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quant_weight_bias",
+           "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
+           "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
 
 
@@ -60,6 +62,11 @@ def load():
     L.onhip_conv2d_w8a32_packed_weight_bytes.restype = C.c_size_t
     L.onhip_conv2d_w8a32_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
     L.onhip_conv2d_w8a32_packed.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
+    L.onhip_quant_weight_bias.argtypes = [vp, vp, C.c_int32, C.c_int32, vp, vp, vp]
+    L.onhip_calib_abs_max.argtypes = [vp, C.c_longlong, C.POINTER(C.c_float), vp]
+    L.onhip_calib_histogram.argtypes = [vp, C.c_longlong, C.c_float, vp, vp]
+    L.onhip_calib_threshold.argtypes = [C.c_int, vp, C.c_longlong, C.c_float, C.POINTER(C.c_float)]
+    L.onhip_calib_percentile.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
     L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
@@ -117,6 +124,56 @@ def pack_conv_weights(d, w):
     packed = torch.empty(nbytes // 4, dtype=torch.float32, device=w.device)
     _check(load().onhip_conv2d_pack_weights(C.byref(d), _ptr(w), _ptr(packed), _stream()), "onhip_conv2d_pack_weights")
     return packed
+
+
+CALIB_BINS, CALIB_KL, CALIB_MSE = 2048, 0, 1
+
+
+def quant_weight_bias(w, bias=None):
+    """host arrays: (w8, bias32, weight_aux) of model_quant.hpp:6-29"""
+    import numpy as np
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    cout = w.shape[0]
+    per = w.size // cout
+    w8 = np.empty(w.shape, np.int8)
+    aux = np.empty(cout, np.float32)
+    b32 = None
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
+        b32 = np.empty(cout, np.int32)
+    _check(load().onhip_quant_weight_bias(w.ctypes.data, bias.ctypes.data if bias is not None else None, cout, per,
+                                          w8.ctypes.data, b32.ctypes.data if b32 is not None else None,
+                                          aux.ctypes.data), "onhip_quant_weight_bias")
+    return w8, b32, aux
+
+
+def calib_abs_max(x, running=0.0):
+    m = C.c_float(running)
+    _check(load().onhip_calib_abs_max(_ptr(x), x.numel(), C.byref(m), _stream()), "onhip_calib_abs_max")
+    return m.value
+
+
+def calib_histogram(x, max_abs, hist=None):
+    """adds to (or creates) the host histogram of 2048 float counters"""
+    import numpy as np
+    if hist is None:
+        hist = np.zeros(CALIB_BINS, np.float32)
+    _check(load().onhip_calib_histogram(_ptr(x), x.numel(), max_abs, hist.ctypes.data, _stream()),
+           "onhip_calib_histogram")
+    return hist
+
+
+def calib_threshold(method, hist, elem_count, max_abs):
+    t = C.c_float(0.0)
+    _check(load().onhip_calib_threshold(method, hist.ctypes.data, elem_count, max_abs, C.byref(t)),
+           "onhip_calib_threshold")
+    return t.value
+
+
+def calib_percentile(x, images, elems):
+    t = C.c_float(0.0)
+    _check(load().onhip_calib_percentile(_ptr(x), images, elems, C.byref(t), _stream()), "onhip_calib_percentile")
+    return t.value
 
 
 def conv2d_w8a32_workspace(d):

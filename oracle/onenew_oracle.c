@@ -13,9 +13,15 @@
  * with their own flags the results are bit-identical for all fp32 and int8 paths whose output is
  * square (OH == OW); see the notes on im2col below.
  *
- * Every function of this file is pinned by tests/test_oracle_*.py: against the compiled
+ * The kernel functions of this file are pinned by tests/test_oracle_*.py: against the compiled
  * reference kernels (golden fixtures made by tests/golden/make_golden.py), against float64
  * brute force and against algebraic invariants.
+ *
+ * PARITY UNPINNED: oracle_quant_weight_bias and the oracle_calib_* functions restate
+ * tools/optimize/model_quant.hpp, which only builds together with the reference's host runtime,
+ * OpenCV and protobuf, and which leaves the overload of fabs / abs / log it calls on floats to the
+ * include order.  They are checked against closed forms and numpy (tests/test_oracle_math.py), not
+ * against reference output.
  */
 #include <immintrin.h>
 #include <math.h>
@@ -447,10 +453,140 @@ void oracle_quant_weight_bias(const float *w, const float *bias, int cout, int p
             mx = a > mx ? a : mx;
         }
         weight_aux[oc] = mx;
-        const float scale = 127.0f / mx;
-        for (int i = 0; i < per_channel; ++i) w8[(size_t) oc * per_channel + i] = (int8_t) (wc[i] * scale);
-        if (bias) bias32[oc] = (int32_t) (bias[oc] * scale);
+        /* "w * 127 / max": the product is rounded before the division (model_quant.hpp:22,25) */
+        for (int i = 0; i < per_channel; ++i) w8[(size_t) oc * per_channel + i] = (int8_t) ((wc[i] * 127.0f) / mx);
+        if (bias) bias32[oc] = (int32_t) ((bias[oc] * 127.0f) / mx);
     }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Activation-scale calibration (tools/optimize/model_quant.hpp:83-185 percentile, :197-435 KL,
+ * :437-623 MSE; input_scale = threshold / 127 at :668).  PARITY UNPINNED: the reference tool only
+ * builds with the whole host runtime and OpenCV, and it calls fabs / abs / log on floats without
+ * saying which overload it gets; float overloads (the evident intent) are used here.
+ * ------------------------------------------------------------------------------------------- */
+
+/* model_quant.hpp:287-292: running maximum of |x| over the calibration images */
+float oracle_calib_abs_max(const float *x, int64_t n, float running_max) {
+    float mx = running_max;
+    for (int64_t i = 0; i < n; ++i) {
+        const float a = fabsf(x[i]);
+        mx = mx > a ? mx : a;
+    }
+    return mx;
+}
+
+/* model_quant.hpp:325-332: 2048-bin histogram of |x| over [0, max], zeros skipped, counts kept as floats */
+void oracle_calib_histogram(const float *x, int64_t n, float max_abs, float *hist) {
+    for (int64_t i = 0; i < n; ++i) {
+        if (x[i] == 0.0f) continue;
+        int idx = (int) (fabsf(x[i]) * ORACLE_CALIB_BINS * 1.0f / max_abs);
+        idx = idx < ORACLE_CALIB_BINS - 1 ? idx : ORACLE_CALIB_BINS - 1;
+        hist[idx] += 1.0f;
+    }
+}
+
+/* model_quant.hpp:345-431: the clipping bin whose 128-level quantised distribution is closest (KL) to the
+ * clipped reference distribution; threshold = (best + 0.5) * max / 2048 */
+float oracle_calib_threshold_kl(const float *hist, int64_t elem_count, float max_abs) {
+    enum { TARGET = 128, MIN_BINS = 128 };
+    const float kl_eps = 1e-7f;
+    float best_kl = 32768.6f;
+    int best_bins = 0;
+    static float p[ORACLE_CALIB_BINS], accp[ORACLE_CALIB_BINS], q[TARGET], eq[ORACLE_CALIB_BINS];
+    for (int bins = MIN_BINS; bins < ORACLE_CALIB_BINS; ++bins) {
+        for (int i = 0; i < bins; ++i) p[i] = accp[i] = kl_eps + hist[i];
+        for (int i = bins; i < ORACLE_CALIB_BINS; ++i) accp[bins - 1] += hist[i];
+        for (int i = 0; i < bins; ++i) {
+            accp[i] = (float) (accp[i] / (double) elem_count);
+            p[i] = (float) (p[i] / (double) elem_count);
+        }
+        const float ratio = (float) bins * 1.0f / TARGET;
+        for (int i = 0; i < TARGET; ++i) {
+            const float st = i * ratio, ed = (i + 1) * ratio;
+            float v = 0.0f;
+            if (floorf(st) == floorf(ed)) {
+                v += (ed - st) * p[(int) floorf(st)];
+            } else {
+                v += (ceilf(st) - st) * p[(int) floorf(st)];
+                for (int j = (int) ceilf(st); j < (int) floorf(ed); ++j) v += p[j];
+                /* the reference reads p_histogram[floor(ed)], one past the end when ed == bins: that slot
+                 * is multiplied by ed - floor(ed) == 0 there, so it is skipped here */
+                if (ed - floorf(ed) != 0.0f) v += (ed - floorf(ed)) * p[(int) floorf(ed)];
+            }
+            q[i] = v / (ed - st);
+        }
+        for (int i = 0; i < bins; ++i) eq[i] = kl_eps;
+        for (int i = 0; i < TARGET; ++i) {
+            const float st = i * ratio, ed = (i + 1) * ratio;
+            if (floorf(st) == floorf(ed)) {
+                eq[(int) floorf(st)] += (ed - st) * q[i];
+            } else {
+                eq[(int) floorf(st)] += (ceilf(st) - st) * q[i];
+                for (int j = (int) ceilf(st); j < (int) floorf(ed); ++j) eq[j] += 1.0f * q[i];
+                const int tail = (int) floorf(ed) >= bins ? bins - 1 : (int) floorf(ed);
+                eq[tail] += (ed - floorf(ed)) / 1.0f * q[i];
+            }
+        }
+        float kl = 0.0f;
+        for (int i = 0; i < bins; ++i) kl += accp[i] * logf(accp[i] / eq[i]);
+        if (kl < best_kl) {
+            best_kl = kl;
+            best_bins = bins;
+        }
+    }
+    return (best_bins + 0.5f) * max_abs / ORACLE_CALIB_BINS;
+}
+
+/* model_quant.hpp:585-618: the clipping bin with the least squared error of a 128-level grid */
+float oracle_calib_threshold_mse(const float *hist, int64_t elem_count, float max_abs) {
+    enum { TARGET = 128, MIN_BINS = 128 };
+    int best_bins = 0;
+    float loss_min = 32768.0f;
+    const int32_t elem_size = (int32_t) elem_count;      /* the reference keeps the count in an int32 */
+    for (int bins = MIN_BINS; bins < ORACLE_CALIB_BINS; ++bins) {
+        float loss = 0.0f;
+        const float step = (float) bins / (TARGET - 1);
+        for (int idx = 0; idx < ORACLE_CALIB_BINS; ++idx) {
+            float iq = roundf(((float) idx + 0.5f) / step);
+            iq = iq > 127.0f ? 127.0f : iq;
+            iq *= step;
+            const float err = (float) ((float) idx + 0.5 - iq);      /* "+ 0.5" in double, stored to float */
+            loss += (hist[idx] * err * err) / elem_size;
+        }
+        if (loss < loss_min) {
+            loss_min = loss;
+            best_bins = bins;
+        }
+    }
+    return (best_bins + 0.5f) * max_abs / ORACLE_CALIB_BINS;
+}
+
+static int cmp_abs_desc(const void *a, const void *b) {
+    const float x = fabsf(*(const float *) a), y = fabsf(*(const float *) b);
+    return x > y ? -1 : x < y ? 1 : 0;
+}
+
+/* model_quant.hpp:99-183: every image keeps its (1 - 0.99998) * 10 * elems largest magnitudes; the threshold is
+ * the element of rank (1 - 0.99998) * images * elems among all kept ones.  x holds `images` tensors of `elems`
+ * values.  Returns the magnitude (the reference returns the signed element). */
+float oracle_calib_threshold_percent(const float *x, int images, int32_t elems) {
+    const float percent = 99.998 / 100;
+    const int32_t keep = (int32_t) (elems * (1 - percent) * 10);
+    const int32_t total = (int32_t) (images * elems * (1 - percent) * 10);
+    float *large = (float *) calloc(total > 0 ? total : 1, sizeof(float));
+    float *tmp = (float *) malloc((size_t) elems * sizeof(float));
+    for (int i = 0; i < images; ++i) {
+        memcpy(tmp, x + (size_t) i * elems, (size_t) elems * sizeof(float));
+        qsort(tmp, elems, sizeof(float), cmp_abs_desc);
+        if ((int64_t) i * keep + keep <= total) memcpy(large + (size_t) i * keep, tmp, (size_t) keep * sizeof(float));
+    }
+    qsort(large, total, sizeof(float), cmp_abs_desc);
+    const int32_t idx = (int32_t) ((1 - percent) * images * elems);
+    const float thr = (total > 0 && idx < total) ? fabsf(large[idx]) : 0.0f;
+    free(tmp);
+    free(large);
+    return thr;
 }
 
 /* ---------------------------------------------------------------------------------------------

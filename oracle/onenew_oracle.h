@@ -29,6 +29,13 @@ int oracle_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t
 void oracle_quant_weight_bias(const float *w, const float *bias, int cout, int per_channel, int8_t *w8,
                               int32_t *bias32, float *weight_aux);
 
+#define ORACLE_CALIB_BINS 2048
+float oracle_calib_abs_max(const float *x, int64_t n, float running_max);
+void oracle_calib_histogram(const float *x, int64_t n, float max_abs, float *hist);
+float oracle_calib_threshold_kl(const float *hist, int64_t elem_count, float max_abs);
+float oracle_calib_threshold_mse(const float *hist, int64_t elem_count, float max_abs);
+float oracle_calib_threshold_percent(const float *x, int images, int32_t elems);
+
 int oracle_matmul_f32(int batch, int M, int K, int N, int b_shared, const float *A, const float *B, float *C);
 int oracle_gemm_f32(int M, int K, int N, const float *A, const float *W, const float *bias, float *C);
 int oracle_matmul_bias_gelu_f32(int batch, int M, int K, int N, int b_shared, const float *A, const float *B,

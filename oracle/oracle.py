@@ -146,6 +146,35 @@ def quant_weight_bias(w, bias):
     return w8, b32, aux
 
 
+def calib_abs_max(x, running=0.0):
+    x = _f32(x)
+    fn = lib().oracle_calib_abs_max
+    fn.restype = C.c_float
+    return float(fn(_p(x, f32p), C.c_int64(x.size), C.c_float(running)))
+
+
+def calib_histogram(x, max_abs, hist=None):
+    x = _f32(x)
+    if hist is None:
+        hist = np.zeros(2048, np.float32)
+    lib().oracle_calib_histogram(_p(x, f32p), C.c_int64(x.size), C.c_float(max_abs), _p(hist, f32p))
+    return hist
+
+
+def calib_threshold(method, hist, elem_count, max_abs):
+    fn = lib().oracle_calib_threshold_kl if method == "kl" else lib().oracle_calib_threshold_mse
+    fn.restype = C.c_float
+    hist = _f32(hist)
+    return float(fn(_p(hist, f32p), C.c_int64(elem_count), C.c_float(max_abs)))
+
+
+def calib_percentile(x, images, elems):
+    x = _f32(x)
+    fn = lib().oracle_calib_threshold_percent
+    fn.restype = C.c_float
+    return float(fn(_p(x, f32p), int(images), C.c_int32(elems)))
+
+
 def round_bf16(x):
     x = _f32(x)
     y = np.empty_like(x)

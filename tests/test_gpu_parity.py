@@ -400,3 +400,41 @@ def test_linearity_and_zero_input(torch_dev):
     d.act_type = abi.RELU
     y0 = hip.conv2d_f32(d, torch.zeros_like(xd), wd, bd).cpu().numpy()
     assert np.array_equal(y0, np.broadcast_to(np.maximum(bb, 0), y0.shape))
+
+
+def _calib_tensor(seed, n):
+    x = cases.datagen.normal(seed, (n,), 1.0)
+    x[::997] *= 9.0
+    x[5::1231] = 0.0
+    return x.astype(np.float32)
+
+
+def test_calibration_passes_match_oracle(torch_dev, oracle):
+    """running max |x|, the 2048-bin histogram (two images accumulated) and the KL / MSE thresholds are the
+    oracle's, bit for bit; so is the weight / bias quantiser"""
+    torch = torch_dev
+    imgs = [_calib_tensor(cases.datagen.seed_for("calib_gpu", str(i)), 300000 + 1000 * i) for i in range(2)]
+    mx_ref, mx = 0.0, 0.0
+    for x in imgs:
+        mx_ref = oracle.calib_abs_max(x, mx_ref)
+        mx = hip.calib_abs_max(dev(torch, x), mx)
+    assert mx == mx_ref == max(float(np.abs(x).max()) for x in imgs)
+    h_ref, h = None, None
+    for x in imgs:
+        h_ref = oracle.calib_histogram(x, mx_ref, h_ref)
+        h = hip.calib_histogram(dev(torch, x), mx, h)
+    assert np.array_equal(h, h_ref)
+    count = sum(x.size for x in imgs)
+    for name, method in (("kl", hip.CALIB_KL), ("mse", hip.CALIB_MSE)):
+        assert hip.calib_threshold(method, h, count, mx) == oracle.calib_threshold(name, h_ref, count, mx_ref), name
+    w = cases.datagen.normal(21, (7, 5, 3, 3), 0.0, 0.1)
+    b = cases.datagen.normal(22, (7,), 0.0, 0.05)
+    got, ref = hip.quant_weight_bias(w, b), oracle.quant_weight_bias(w, b)
+    assert all(np.array_equal(g, r) for g, r in zip(got, ref))
+
+
+def test_calibration_percentile_matches_oracle(torch_dev, oracle):
+    torch = torch_dev
+    images, elems = 3, 400000
+    x = _calib_tensor(cases.datagen.seed_for("calib_gpu", "pct"), images * elems)
+    assert hip.calib_percentile(dev(torch, x), images, elems) == oracle.calib_percentile(x, images, elems)

@@ -138,9 +138,10 @@ def test_weight_quantiser_truncates_toward_zero(oracle):
     b = datagen.normal(12, (5,), 0.0, 0.05)
     w8, b32, aux = oracle.quant_weight_bias(w, b)
     assert np.array_equal(aux, np.abs(w).reshape(5, -1).max(axis=1))
-    scale = (np.float32(127.0) / aux).reshape(5, 1, 1, 1)
-    assert np.array_equal(w8, np.trunc(w * scale).astype(np.int8))
-    assert np.array_equal(b32, np.trunc(b * scale.reshape(5)).astype(np.int32))
+    # "w * 127 / max": the product is rounded to float before the division
+    a4 = aux.reshape(5, 1, 1, 1)
+    assert np.array_equal(w8, np.trunc((w * np.float32(127.0)) / a4).astype(np.int8))
+    assert np.array_equal(b32, np.trunc((b * np.float32(127.0)) / aux).astype(np.int32))
     assert np.abs(w8).max() == 127
     back = w8.astype(np.float32) * (aux / np.float32(127.0)).reshape(5, 1, 1, 1)
     assert np.all(np.abs(back) <= np.abs(w) + 1e-7) and np.abs(back - w).max() <= (aux / 127).max() + 1e-7
@@ -168,3 +169,74 @@ def test_bf16_f16_rounding_helpers(oracle):
     assert np.all((b.view(np.uint32) & 0xFFFF) == 0)
     h = oracle.round_f16(x)
     assert np.array_equal(h, x.astype(np.float16).astype(np.float32))
+
+
+def _calib_data(seed, n):
+    # a bell around zero with a few far outliers: the case clipping calibration exists for
+    x = datagen.normal(seed, (n,), 1.0)
+    x[::997] *= 9.0
+    x[5::1231] = 0.0
+    return x.astype(np.float32)
+
+
+def test_calibration_histogram_and_max(oracle):
+    """abs-max and the 2048-bin histogram against numpy; zeros are skipped, the top bin catches the maximum"""
+    x = _calib_data(datagen.seed_for("calib", "x"), 200000)
+    mx = oracle.calib_abs_max(x)
+    assert mx == np.abs(x).max()
+    assert oracle.calib_abs_max(x[:10], running=1e9) == np.float32(1e9)
+    h = oracle.calib_histogram(x, mx)
+    nz = np.abs(x[x != 0.0])
+    idx = np.minimum((nz * np.float32(2048) * np.float32(1.0) / np.float32(mx)).astype(np.int32), 2047)
+    assert np.array_equal(h, np.bincount(idx, minlength=2048).astype(np.float32))
+    assert h.sum() == nz.size and h[2047] >= 1
+    # a second call accumulates
+    h2 = oracle.calib_histogram(x, mx, hist=h.copy())
+    assert np.array_equal(h2, 2 * h)
+
+
+def test_calibration_thresholds_closed_cases(oracle):
+    """cases the definitions fix: (1) KL: a jagged distribution that lives in the first 128 bins is reproduced
+    exactly by 128 levels over 128 bins and blurred by every wider clipping range (neighbouring bins merge),
+    so the first candidate wins: threshold = 128.5 * max / 2048; (2) MSE: a single occupied
+    bin b has squared error (b + 0.5 - level)^2 minimised over the candidates - brute-forced in float64;
+    (3) thresholds scale linearly with max_abs; (4) outliers beyond the bulk are clipped: the KL threshold of a
+    bell with far outliers lies well below the maximum"""
+    h = np.zeros(2048, np.float32)
+    h[:128] = datagen.integers(datagen.seed_for("calib", "jagged"), (128,), 1, 2000).astype(np.float32)
+    t = oracle.calib_threshold("kl", h, int(h.sum()), 4.0)
+    assert t == np.float32((128 + 0.5) * 4.0 / 2048)
+    for b in (300, 1000, 2047):
+        h = np.zeros(2048, np.float32)
+        h[b] = 50.0
+        losses = []
+        for bins in range(128, 2048):
+            step = np.float32(bins) / np.float32(127)
+            level = min(np.floor((b + 0.5) / float(step) + 0.5), 127.0) * float(step)
+            losses.append((b + 0.5 - level) ** 2)
+        losses = np.array(losses)
+        t = oracle.calib_threshold("mse", h, 50, 2.0)
+        got_bins = round(t * 2048 / 2.0 - 0.5)
+        # float32 rounding of the step decides between candidates that both sit within 1e-3 bin^2 of zero error
+        assert losses[got_bins - 128] <= losses.min() + 1e-3, (b, got_bins, int(losses.argmin()) + 128)
+    x = _calib_data(datagen.seed_for("calib", "thr"), 400000)
+    mx = oracle.calib_abs_max(x)
+    h = oracle.calib_histogram(x, mx)
+    for method in ("kl", "mse"):
+        t1 = oracle.calib_threshold(method, h, x.size, mx)
+        t2 = oracle.calib_threshold(method, h, x.size, 2 * mx)
+        assert t2 == 2 * t1
+        assert 128.5 * mx / 2048 <= t1 <= mx
+    assert oracle.calib_threshold("kl", h, x.size, mx) < 0.8 * mx
+
+
+def test_calibration_percentile_rank(oracle):
+    """the 99.998 % rule against a numpy sort: rank (1-p)*images*elems among the kept largest magnitudes"""
+    images, elems = 3, 500000
+    x = _calib_data(datagen.seed_for("calib", "pct"), images * elems)
+    t = oracle.calib_percentile(x, images, elems)
+    p = np.float32(99.998 / 100)
+    keep = int(np.float32(elems) * (np.float32(1) - p) * 10)
+    kept = np.concatenate([np.sort(np.abs(x[i * elems:(i + 1) * elems]))[::-1][:keep] for i in range(images)])
+    rank = int((np.float32(1) - p) * images * elems)
+    assert t == np.sort(kept)[::-1][rank]
