@@ -217,7 +217,30 @@ def time_layers(torch, hip, layers, reps):
     return out
 
 
-def cpu_baseline(layers, tag, unit, budget_s=20.0):
+def plugin_eval_latency(hip):
+    """the drop-in boundary end to end: `eval` of libConv_hip.so on host buffers (BASELINE config 1), i.e. with the
+    activation copied in and the result copied out over PCIe on every call; never part of `value`"""
+    import cases
+    from onenew_amd import ops
+    d = cases.conv_f32_cases()["cfg1_64x56_3x3"]
+    x, w, b = cases.conv_inputs("bench/plugin_cfg1", d)
+    op = ops.Conv(ops.Plugin(hip.plugin_path("Conv")).eval, d, w, b, silu_lut=cases.silu_lut())
+    xin = ops.aligned_empty(x.shape)
+    xin[...] = x
+    out = ops.aligned_empty((1, d.cout) + d.out_hw())
+    for _ in range(5):
+        op(xin, out=out)
+    times = []
+    for _ in range(30):
+        t0 = time.perf_counter()
+        op(xin, out=out)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {"ms_per_call": round(med * 1e3, 4), "tflops": round(d.flops() / med / 1e12, 3),
+            "note": "host buffers in and out (PCIe-inclusive), synchronous, weights cached on the device"}
+
+
+def cpu_baseline(layers, tag, unit, budget_s=12.0):
     """the reference's x86 kernels (or the CPU restatement) on a bounded sample: passes over the same layer
     shapes at batch 1 (the reference evaluates one image per call), 8 threads as the reference builds"""
     from onenew_amd import ops
@@ -231,7 +254,8 @@ def cpu_baseline(layers, tag, unit, budget_s=20.0):
         f()                      # warm-up pass
     times = []
     t_start = time.perf_counter()
-    while len(times) < 10 and (time.perf_counter() - t_start < budget_s or len(times) < 2):
+    # about budget_s seconds of CPU work, at least 10 and at most 2000 passes
+    while len(times) < 2000 and (time.perf_counter() - t_start < budget_s or len(times) < 10):
         t0 = time.perf_counter()
         for _, f in runs:
             f()
@@ -325,6 +349,8 @@ def main():
         _, _, layers1 = make_workload(torch, hip, "resnet50_b1")
         ms1 = time_layers(torch, hip, layers1, reps=20)
         extra["resnet50_conv_stack_ms_batch1"] = round(sum(ms1), 4)
+    if args.workload.startswith("resnet50_b") or args.workload == "cfg1":
+        extra["plugin_eval_cfg1"] = plugin_eval_latency(hip)
     extra["stack_ms_sum_of_layers"] = round(sum(per_layer_ms), 4)
     extra["algorithmic_GBps"] = round(abytes / (sum(per_layer_ms) * 1e-3) / 1e9, 1)
     lowai = [(L, t) for L, t in zip(layers, per_layer_ms) if not L.dense]
