@@ -28,9 +28,15 @@ struct DwParams {
     int pitch;           // LDS row pitch: W plus the left and right padding columns the filter can touch
     int flat_stage;      // small whole planes: stage by flat index
     unsigned magic_hw, magic_w;   // floor(2^32 / d) + 1 for d = H*W and d = W (d >= 2)
+    Div31 div_ow, div_c;          // exact division by OW and by C
+    Div31 div_unit;               // whole-plane mode: by the work units (strips or outputs) of one plane
     float in_scale, inv_in_scale, out_inv_scale;
     int out_s8;
 };
+
+__device__ __forceinline__ int dw_div(int x, const Div31 &d) {
+    return (int) ((__umulhi((unsigned) x, d.magic) >> d.shift) + ((unsigned) x & d.pass));
+}
 
 // The LDS tile holds, for each plane of the chunk, every input row and column the chunk's outputs
 // touch, padding included and zero-filled, so the compute phase reads it without predicates:
@@ -125,12 +131,13 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
         const int strips_per_plane = nsr * p.OW;
         const int strips = nplanes * strips_per_plane;
         for (int sidx = tid; sidx < strips; sidx += DW_THREADS) {
-            const int pl = sidx / strips_per_plane;
+            // a band has one plane; whole planes have the host's divisor (no integer division in the loop)
+            const int pl = p.planes_per_wg >= 1 ? dw_div(sidx, p.div_unit) : 0;
             const int rem = sidx - pl * strips_per_plane;
-            const int sr = rem / p.OW;
+            const int sr = dw_div(rem, p.div_ow);
             const int ow = rem - sr * p.OW;
             const int plane = plane0 + pl;
-            const int c = plane % p.C;
+            const int c = plane - dw_div(plane, p.div_c) * p.C;
             float wreg[9];
             float bias_f;
             if (INT8) {
@@ -191,12 +198,12 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
     const int per_plane = out_rows * p.OW;
     const int total_out = nplanes * per_plane;
     for (int o = tid; o < total_out; o += DW_THREADS) {
-        const int pl = o / per_plane;
+        const int pl = p.planes_per_wg >= 1 ? dw_div(o, p.div_unit) : 0;
         const int rem = o - pl * per_plane;
-        const int r = rem / p.OW;
+        const int r = dw_div(rem, p.div_ow);
         const int ow = rem - r * p.OW;
         const int plane = plane0 + pl;
-        const int c = plane % p.C;
+        const int c = plane - dw_div(plane, p.div_c) * p.C;
         const float *tp = tile + pl * plane_cells + (r * p.sh) * pitch + ow * p.sw;
         const long long oidx = ((long long) plane * p.OH + oh0 + r) * p.OW + ow;
         float v;
@@ -226,8 +233,14 @@ static int dw_specialisation(const onhip_conv_desc_t &d) {
     return 0;
 }
 
+static int dw_specialisation(const onhip_conv_desc_t &d);
+
 static int dw_plan(const onhip_conv_desc_t &d, int OH, int OW, DwParams *p) {
     p->C = d.cout; p->H = d.h; p->W = d.w; p->OH = OH; p->OW = OW;
+    p->div_ow = make_div31((unsigned) OW);
+    p->div_c = make_div31((unsigned) d.cout);
+    // work units of one whole plane: strips of DW_RT rows in the 3x3 kernels, single outputs otherwise
+    p->div_unit = make_div31((unsigned) (dw_specialisation(d) ? ((OH + DW_RT - 1) / DW_RT) * OW : OH * OW));
     p->kh = d.kh; p->kw = d.kw; p->sh = d.stride_h; p->sw = d.stride_w; p->pt = d.pad_t; p->pl = d.pad_l;
     p->planes = d.n * d.cout;
     // columns 0 .. (OW-1)*sw + kw - 1 of the padded row are read
