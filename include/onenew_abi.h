@@ -8,7 +8,7 @@
  * The structs below are layout-identical (x86-64, LP64) to the ones the reference host fills
  * (reference: common/nn_common.h:20-26 constants, :28-62 USEFUL_INFO_S, :77-82 BUFFER_INFO_S,
  * :92-110 ELEM_TYPE_E, :129-138 ACT_TYPE_E, :146-155 OPERAND_S, :164-182 BASE_CONFIG_S,
- * :222-243 CONV_CONFIG_S, :312-320 GEMM_CONFIG_S, :366-369 MATMUL_CONFIG_S).  Only the types the
+ * :222-243 CONV_CONFIG_S, :312-320 GEMM_CONFIG_S, :366-369 MATMUL_CONFIG_S, :371-379 MAX_POOL_CONFIG_S).  Only the types the
  * Conv / MatMul / Gemm plugins read are declared.  The static assertions at the end pin every
  * size and offset a plugin depends on.
  */
@@ -157,6 +157,26 @@ typedef struct {
     BASE_CONFIG_S op_base_cfg;
 } MATMUL_CONFIG_S;
 
+/* common/nn_common.h:184-187, :327-330, :481-484: operators without parameters of their own */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+} ADD_CONFIG_S;
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+} GLOBAL_AVGPOOL_CONFIG_S;
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+} RELU_CONFIG_S;
+
+/* common/nn_common.h:371-379 */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    int64_t ceil_mode;          /* not read by the kernel */
+    int64_t kernel_shape[2];
+    int64_t pads[4];            /* the kernel pads all four sides by pads[0] */
+    int64_t strides[2];         /* [0] steps along w, [1] along h (maxpool.c:20-21,72) */
+} MAX_POOL_CONFIG_S;
+
 /* the one symbol a plugin exports */
 typedef int (*onenew_eval_fn)(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 
@@ -189,6 +209,12 @@ ONENEW_SA(offsetof(CONV_CONFIG_S, weight_aux) == 12988, "CONV.weight_aux");
 ONENEW_SA(sizeof(GEMM_CONFIG_S) == 12864, "GEMM_CONFIG_S");
 ONENEW_SA(offsetof(GEMM_CONFIG_S, transB) == 12856, "GEMM.transB");
 ONENEW_SA(sizeof(MATMUL_CONFIG_S) == 12840, "MATMUL_CONFIG_S");
+ONENEW_SA(sizeof(ADD_CONFIG_S) == 12840 && sizeof(RELU_CONFIG_S) == 12840 && sizeof(GLOBAL_AVGPOOL_CONFIG_S) == 12840,
+          "parameterless configs");
+ONENEW_SA(sizeof(MAX_POOL_CONFIG_S) == 12912, "MAX_POOL_CONFIG_S");
+ONENEW_SA(offsetof(MAX_POOL_CONFIG_S, kernel_shape) == 12848, "MAX_POOL.kernel_shape");
+ONENEW_SA(offsetof(MAX_POOL_CONFIG_S, pads) == 12864, "MAX_POOL.pads");
+ONENEW_SA(offsetof(MAX_POOL_CONFIG_S, strides) == 12896, "MAX_POOL.strides");
 ONENEW_SA(sizeof(USEFUL_INFO_S) == 96, "USEFUL_INFO_S");
 ONENEW_SA(offsetof(USEFUL_INFO_S, block_info) == 4, "USEFUL.block_info");
 ONENEW_SA(offsetof(USEFUL_INFO_S, public_buf_info) == 40, "USEFUL.public_buf_info");

@@ -149,6 +149,44 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
 int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w,
                    const float *bias, float *out, void *stream);
 
+/* ---- the operators around the convolutions of a residual network (device pointers) ------------ */
+
+/* Broadcasting add: out = large + small, out has the shape of `large`; `small` is aligned to the
+ * same rank (host pads its shape with leading 1s) and each of its extents is 1 or equal.  relu != 0
+ * applies max(x, 0) to the sum: the Add -> Relu pair that closes a residual block, in one pass.
+ * Replaces device/x86/Add/add.c eval (:18-80) and fun_0 / fun_1 / fun_2_dim3..6 (:87-365). */
+typedef struct {
+    int32_t ndim;            /* 1..6 */
+    int32_t large_shape[6];
+    int32_t small_shape[6];
+    int32_t relu;
+} onhip_add_desc_t;
+int onhip_add_f32(const onhip_add_desc_t *d, const float *large, const float *small, float *out,
+                  void *stream);
+
+/* y = relu(x) over n floats (16-byte aligned).  Replaces device/x86/Relu/relu.c eval (:8-55),
+ * including its two rules: the first n - n % 32 elements keep a NaN or a negative zero. */
+int onhip_relu_f32(const float *x, float *y, long long n, void *stream);
+
+/* Max pooling over NCHW planes, every side padded by `pad`; oh x ow is the extent of the output
+ * operand (at most the floor-mode shape onhip_maxpool_out_shape reports).  Replaces
+ * device/x86/MaxPool/maxpool.c eval (:7-92) with pad_maxpool.h; the running maximum starts at
+ * -3276800 as there. */
+typedef struct {
+    int32_t n, c, h, w;
+    int32_t kh, kw;
+    int32_t stride_w, stride_h;   /* strides[0] moves along w, strides[1] along h (maxpool.c:20-21,72) */
+    int32_t pad;
+} onhip_pool_desc_t;
+int onhip_maxpool_out_shape(const onhip_pool_desc_t *d, int32_t *oh, int32_t *ow);
+int onhip_maxpool_f32(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const float *x, float *y,
+                      void *stream);
+
+/* y[n][c] = (sum of the plane in memory order) * (1.0f / (h*w)).  Replaces
+ * device/x86/GlobalAveragePool/global_avgpool.c eval (:7-45). */
+int onhip_global_avgpool_f32(int32_t n, int32_t c, int32_t h, int32_t w, const float *x, float *y,
+                             void *stream);
+
 /* ---- offline quantisation: what produces the operands of onhip_conv2d_w8a32 ------------------ */
 
 /* Per output channel: weight_aux = max|w|, w8 = (int8)(w * 127 / aux) (truncating),
@@ -184,6 +222,11 @@ int onhip_copy_f32(const float *src, float *dst, long long n, void *stream);
 
 int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* Add (add.c:18), Relu (relu.c:8), MaxPool (maxpool.c:7), GlobalAveragePool (global_avgpool.c:7) */
+int onhip_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_maxpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_global_avgpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Drops the device copies of weights the plugin level keeps between calls. */
 int onhip_plugin_release(void);

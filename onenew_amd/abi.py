@@ -86,6 +86,32 @@ class MATMUL_CONFIG_S(C.Structure):
     _fields_ = [("op_base_cfg", BASE_CONFIG_S)]
 
 
+class PLAIN_CONFIG_S(C.Structure):
+    """ADD_CONFIG_S, RELU_CONFIG_S, GLOBAL_AVGPOOL_CONFIG_S: the base config and nothing else"""
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S)]
+
+
+class MAX_POOL_CONFIG_S(C.Structure):
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("ceil_mode", C.c_int64), ("kernel_shape", C.c_int64 * 2),
+                ("pads", C.c_int64 * 4), ("strides", C.c_int64 * 2)]
+
+
+class AddDesc(C.Structure):
+    """onhip_add_desc_t"""
+    _fields_ = [("ndim", C.c_int32), ("large_shape", C.c_int32 * 6), ("small_shape", C.c_int32 * 6),
+                ("relu", C.c_int32)]
+
+
+class PoolDesc(C.Structure):
+    """onhip_pool_desc_t"""
+    _fields_ = [("n", C.c_int32), ("c", C.c_int32), ("h", C.c_int32), ("w", C.c_int32), ("kh", C.c_int32),
+                ("kw", C.c_int32), ("stride_w", C.c_int32), ("stride_h", C.c_int32), ("pad", C.c_int32)]
+
+    def out_hw(self):
+        return ((self.h + 2 * self.pad - self.kh) // self.stride_h + 1,
+                (self.w + 2 * self.pad - self.kw) // self.stride_w + 1)
+
+
 class ConvDesc(C.Structure):
     """onhip_conv_desc_t"""
     _fields_ = [("n", C.c_int32), ("cin", C.c_int32), ("h", C.c_int32), ("w", C.c_int32),
@@ -144,6 +170,7 @@ def check_layout():
     assert CONV_CONFIG_S.weight_aux.offset == 12988
     assert C.sizeof(GEMM_CONFIG_S) == 12864 and GEMM_CONFIG_S.transB.offset == 12856
     assert C.sizeof(MATMUL_CONFIG_S) == 12840
+    assert C.sizeof(MAX_POOL_CONFIG_S) == 12912 and MAX_POOL_CONFIG_S.strides.offset == 12896
     assert C.sizeof(USEFUL_INFO_S) == 96 and USEFUL_INFO_S.public_buf_info.offset == 40
     assert C.sizeof(ConvDesc) == 25 * 4
     assert C.sizeof(MatmulDesc) == 24

@@ -1,0 +1,265 @@
+// The operators either side of the convolutions of a ResNet-style graph, so that a chain can stay in
+// HBM: broadcasting Add (optionally with the ReLU that follows a residual add fused in), ReLU, MaxPool
+// and GlobalAveragePool.  All four are bound by memory bandwidth; results are bit-identical to
+// device/x86/Add/add.c, Relu/relu.c, MaxPool/maxpool.c and GlobalAveragePool/global_avgpool.c.
+#include <string.h>
+
+#include "onhip_internal.hpp"
+
+namespace onhip {
+
+__device__ __forceinline__ unsigned ew_div(unsigned x, const Div31 &d) {
+    return (__umulhi(x, d.magic) >> d.shift) + (x & d.pass);
+}
+
+// ---- Add -------------------------------------------------------------------------------------------
+// out[i] = large[i] + small[j(i)] (add.c: the operand with fewer elements is broadcast onto the other).
+// MODE 0: same number of elements, 1: small is one value, 2: per-dimension broadcast (strides 0).
+struct AddParams {
+    long long n;              // output elements
+    int ndim;
+    Div31 div[6];             // by the extents of the large operand, innermost first
+    int extent[6];
+    int small_stride[6];      // innermost first; 0 where the small operand is broadcast
+    int relu;
+};
+
+template <int MODE>
+__global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__restrict__ large,
+                                                  const float *__restrict__ small, float *__restrict__ out) {
+    if constexpr (MODE == 0) {
+        // four elements per thread when everything is 16-byte aligned (checked by the launcher)
+        const long long i4 = (long long) blockIdx.x * 256 + threadIdx.x;
+        if (i4 * 4 + 3 < p.n) {
+            const float4 a = reinterpret_cast<const float4 *>(large)[i4], b = reinterpret_cast<const float4 *>(small)[i4];
+            // operand order of add.c:96: small + large
+            float4 r = make_float4(__fadd_rn(b.x, a.x), __fadd_rn(b.y, a.y), __fadd_rn(b.z, a.z), __fadd_rn(b.w, a.w));
+            if (p.relu) { r.x = r.x > 0 ? r.x : 0; r.y = r.y > 0 ? r.y : 0; r.z = r.z > 0 ? r.z : 0; r.w = r.w > 0 ? r.w : 0; }
+            reinterpret_cast<float4 *>(out)[i4] = r;
+        } else if (i4 * 4 < p.n) {
+            for (long long i = i4 * 4; i < p.n; ++i) {
+                const float r = __fadd_rn(small[i], large[i]);
+                out[i] = (p.relu && !(r > 0)) ? 0.0f : r;
+            }
+        }
+    } else {
+        const long long i = (long long) blockIdx.x * 256 + threadIdx.x;
+        if (i >= p.n) return;
+        long long j = 0;
+        if constexpr (MODE == 2) {
+            unsigned rest = (unsigned) i;
+#pragma unroll
+            for (int k = 0; k < 6; ++k) {
+                if (k < p.ndim) {
+                    const unsigned q = ew_div(rest, p.div[k]);
+                    j += (long long) (rest - q * (unsigned) p.extent[k]) * p.small_stride[k];
+                    rest = q;
+                }
+            }
+        }
+        const float r = __fadd_rn(large[i], small[j]);
+        out[i] = (p.relu && !(r > 0)) ? 0.0f : r;
+    }
+}
+
+// ---- ReLU ------------------------------------------------------------------------------------------
+// relu.c:27-52: the first n - n % 32 elements go through _mm256_max_ps(0, x), which is "0 > x ? 0 : x" (a NaN
+// or a negative zero comes back unchanged); the rest through "x > 0 ? x : 0".  Both rules are kept.
+__device__ __forceinline__ float relu_body(float v) { return 0.0f > v ? 0.0f : v; }
+__device__ __forceinline__ float relu_tail(float v) { return v > 0.0f ? v : 0.0f; }
+
+__global__ __launch_bounds__(256) void relu_kernel(const float *__restrict__ x, float *__restrict__ y, long long n,
+                                                   long long n_body) {
+    const long long i4 = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (i4 * 4 + 3 < n_body) {
+        float4 v = reinterpret_cast<const float4 *>(x)[i4];
+        v.x = relu_body(v.x); v.y = relu_body(v.y); v.z = relu_body(v.z); v.w = relu_body(v.w);
+        reinterpret_cast<float4 *>(y)[i4] = v;
+    } else if (i4 * 4 < n) {
+        for (long long i = i4 * 4; i < min(n, i4 * 4 + 4); ++i) y[i] = i < n_body ? relu_body(x[i]) : relu_tail(x[i]);
+    }
+}
+
+// ---- MaxPool -----------------------------------------------------------------------------------------
+// maxpool.c:62-86: the running maximum starts at -3276800 (smaller inputs are clamped to it) and the
+// padding value -32768000 never wins, so padded cells are simply skipped.  One thread per output, lanes
+// along ow.
+struct PoolParams {
+    int planes, H, W, OH, OW, kh, kw, sw, sh, pad;
+    Div31 div_ow, div_oh;
+};
+
+__global__ __launch_bounds__(256) void maxpool_kernel(PoolParams p, const float *__restrict__ x, float *__restrict__ y,
+                                                      long long total) {
+    const long long o = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (o >= total) return;
+    const unsigned t = ew_div((unsigned) o, p.div_ow);
+    const int ow = (int) ((unsigned) o - t * (unsigned) p.OW);
+    const unsigned plane = ew_div(t, p.div_oh);
+    const int oh = (int) (t - plane * (unsigned) p.OH);
+    const float *src = x + (long long) plane * p.H * p.W;
+    const int ih0 = oh * p.sh - p.pad, iw0 = ow * p.sw - p.pad;
+    float m = -3276800.0f;
+    for (int i = 0; i < p.kh; ++i) {
+        const int ih = ih0 + i;
+        if ((unsigned) ih >= (unsigned) p.H) continue;
+        for (int j = 0; j < p.kw; ++j) {
+            const int iw = iw0 + j;
+            if ((unsigned) iw >= (unsigned) p.W) continue;
+            const float v = src[ih * p.W + iw];
+            m = v > m ? v : m;
+        }
+    }
+    y[o] = m;
+}
+
+// ---- GlobalAveragePool -------------------------------------------------------------------------------
+// global_avgpool.c:27-42: the elements of a plane are added one after the other in memory order, then the
+// sum is multiplied by 1.0f / (H*W).  A workgroup copies a run of whole planes into LDS (coalesced), then
+// one thread per plane adds its elements in that same order.
+constexpr int GAP_LDS_FLOATS = 8192;
+
+__global__ __launch_bounds__(256) void gap_kernel(const float *__restrict__ x, float *__restrict__ y, int planes, int hw,
+                                                  int planes_per_wg, float coeff) {
+    __shared__ float tile[GAP_LDS_FLOATS];
+    const int plane0 = blockIdx.x * planes_per_wg;
+    const int np = min(planes_per_wg, planes - plane0);
+    if (planes_per_wg >= 1 && hw * planes_per_wg <= GAP_LDS_FLOATS) {
+        const float *src = x + (long long) plane0 * hw;
+        for (int i = threadIdx.x; i < np * hw; i += 256) tile[i] = src[i];
+        __syncthreads();
+        if ((int) threadIdx.x < np) {
+            float s = 0.0f;
+            const float *t = tile + threadIdx.x * hw;
+            for (int i = 0; i < hw; ++i) s = __fadd_rn(s, t[i]);
+            y[plane0 + threadIdx.x] = __fmul_rn(s, coeff);
+        }
+    } else {
+        // planes too large for LDS: one thread per plane straight from memory (rare: pooling large maps)
+        const int plane = blockIdx.x * 256 + threadIdx.x;
+        if (plane >= planes) return;
+        const float *t = x + (long long) plane * hw;
+        float s = 0.0f;
+        for (int i = 0; i < hw; ++i) s = __fadd_rn(s, t[i]);
+        y[plane] = __fmul_rn(s, coeff);
+    }
+}
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace onhip
+
+using namespace onhip;
+
+extern "C" {
+
+int onhip_add_f32(const onhip_add_desc_t *d, const float *large, const float *small, float *out, void *stream) {
+    if (!d || !large || !small || !out) return set_error(ONHIP_ERR_ARG, "add: null pointer");
+    if (d->ndim < 1 || d->ndim > 6) return set_error(ONHIP_ERR_ARG, "add: rank %d (1..6 supported)", d->ndim);
+    AddParams p;
+    memset(&p, 0, sizeof(p));
+    long long n = 1, ns = 1;
+    for (int i = 0; i < d->ndim; ++i) {
+        if (d->large_shape[i] < 1 || d->small_shape[i] < 1) return set_error(ONHIP_ERR_ARG, "add: empty dimension");
+        if (d->small_shape[i] != d->large_shape[i] && d->small_shape[i] != 1)
+            return set_error(ONHIP_ERR_ARG, "add: shapes do not broadcast (dim %d: %d onto %d)", i, d->small_shape[i],
+                             d->large_shape[i]);
+        n *= d->large_shape[i];
+        ns *= d->small_shape[i];
+    }
+    if (n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "add: tensors of 2^31 elements or more are not supported");
+    p.n = n;
+    p.ndim = d->ndim;
+    p.relu = d->relu ? 1 : 0;
+    int stride = 1;
+    for (int k = 0; k < d->ndim; ++k) {        // innermost first
+        const int dim = d->ndim - 1 - k;
+        p.extent[k] = d->large_shape[dim];
+        p.div[k] = make_div31((unsigned) d->large_shape[dim]);
+        p.small_stride[k] = d->small_shape[dim] == 1 ? 0 : stride;
+        stride *= d->small_shape[dim];
+    }
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (ns == n) {
+        if (aligned16(large) && aligned16(small) && aligned16(out)) {
+            hipLaunchKernelGGL(add_kernel<0>, dim3((unsigned) ((n / 4 + 1 + 255) / 256)), dim3(256), 0, st, p, large, small, out);
+        } else {
+            // unaligned operands: the broadcast kernel with unit strides is the same sum
+            hipLaunchKernelGGL(add_kernel<2>, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, st, p, large, small, out);
+        }
+    } else if (ns == 1) {
+        hipLaunchKernelGGL(add_kernel<1>, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, st, p, large, small, out);
+    } else {
+        hipLaunchKernelGGL(add_kernel<2>, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, st, p, large, small, out);
+    }
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_relu_f32(const float *x, float *y, long long n, void *stream) {
+    if (!x || !y || n < 1) return set_error(ONHIP_ERR_ARG, "relu: bad argument");
+    if (!aligned16(x) || !aligned16(y)) return set_error(ONHIP_ERR_ARG, "relu: tensors must be 16-byte aligned");
+    hipLaunchKernelGGL(relu_kernel, dim3((unsigned) ((n / 4 + 1 + 255) / 256)), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), x, y, n, n / 32 * 32);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_maxpool_out_shape(const onhip_pool_desc_t *d, int32_t *oh, int32_t *ow) {
+    if (!d || !oh || !ow) return set_error(ONHIP_ERR_ARG, "maxpool: null pointer");
+    if (d->n < 1 || d->c < 1 || d->h < 1 || d->w < 1 || d->kh < 1 || d->kw < 1 || d->stride_h < 1 || d->stride_w < 1 ||
+        d->pad < 0)
+        return set_error(ONHIP_ERR_ARG, "maxpool: bad shape");
+    if (d->h + 2 * d->pad < d->kh || d->w + 2 * d->pad < d->kw) return set_error(ONHIP_ERR_ARG, "maxpool: window larger than input");
+    *oh = (d->h + 2 * d->pad - d->kh) / d->stride_h + 1;   // host/ops/max_pool.h: floor mode
+    *ow = (d->w + 2 * d->pad - d->kw) / d->stride_w + 1;
+    return ONHIP_OK;
+}
+
+int onhip_maxpool_f32(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const float *x, float *y, void *stream) {
+    int32_t moh, mow;
+    int rc = onhip_maxpool_out_shape(d, &moh, &mow);
+    if (rc) return rc;
+    if (!x || !y) return set_error(ONHIP_ERR_ARG, "maxpool: null pointer");
+    // the output extent comes from the caller's operand descriptor, as in maxpool.c:35-38; every window must
+    // lie inside the padded input
+    if (oh < 1 || ow < 1 || oh > moh || ow > mow)
+        return set_error(ONHIP_ERR_ARG, "maxpool: output %dx%d does not fit (at most %dx%d)", oh, ow, moh, mow);
+    PoolParams p;
+    p.planes = d->n * d->c; p.H = d->h; p.W = d->w; p.OH = oh; p.OW = ow;
+    p.kh = d->kh; p.kw = d->kw; p.sw = d->stride_w; p.sh = d->stride_h; p.pad = d->pad;
+    p.div_ow = make_div31((unsigned) ow);
+    p.div_oh = make_div31((unsigned) oh);
+    const long long total = (long long) p.planes * oh * ow;
+    if (total >= (1LL << 31) || (long long) p.planes * d->h * d->w >= (1LL << 31))
+        return set_error(ONHIP_ERR_ARG, "maxpool: tensors of 2^31 elements or more are not supported");
+    hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), p, x, y, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_global_avgpool_f32(int32_t n, int32_t c, int32_t h, int32_t w, const float *x, float *y, void *stream) {
+    if (!x || !y || n < 1 || c < 1 || h < 1 || w < 1) return set_error(ONHIP_ERR_ARG, "global avgpool: bad argument");
+    const long long planes = (long long) n * c, hw = (long long) h * w;
+    if (planes * hw >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "global avgpool: tensor too large");
+    const float coeff = 1.0f / (h * w);
+    int ppw = (int) (GAP_LDS_FLOATS / hw);
+    if (ppw > 256) ppw = 256;
+    unsigned grid;
+    if (ppw >= 1) {
+        // keep at least a few workgroups per CU busy when there are few planes
+        const long long want = (planes + 1023) / 1024;
+        if (ppw > want) ppw = (int) (want < 1 ? 1 : want);
+        grid = (unsigned) ((planes + ppw - 1) / ppw);
+    } else {
+        ppw = 0;
+        grid = (unsigned) ((planes + 255) / 256);
+    }
+    hipLaunchKernelGGL(gap_kernel, dim3(grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x, y, (int) planes,
+                       (int) hw, ppw, coeff);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+}  // extern "C"

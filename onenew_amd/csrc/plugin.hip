@@ -347,6 +347,132 @@ static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
     return ONHIP_OK;
 }
 
+// ---- Add / Relu / MaxPool / GlobalAveragePool ----------------------------------------------------------
+// an output on the host is computed into a staging buffer and copied back; one on the device is written in place
+static int finish_output(void *host_out, void *y, size_t bytes, bool out_on_dev) {
+    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, bytes, hipMemcpyDeviceToHost));
+    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    return ONHIP_OK;
+}
+
+static int add_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *t0 = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *t1 = reinterpret_cast<const OPERAND_S *>(params[2].addr);
+    if (!t0 || !t1 || !inputs[1].addr) return set_error(ONHIP_ERR_ARG, "Add eval: empty slot");
+    // add.c:30-46: the operand with fewer elements is the one that is broadcast (the second one on a tie)
+    const long long n0 = numel(t0), n1 = numel(t1);
+    const bool small_is_0 = n0 < n1;
+    const OPERAND_S *lt = small_is_0 ? t1 : t0, *st = small_is_0 ? t0 : t1;
+    const void *lp = reinterpret_cast<const void *>(inputs[small_is_0 ? 1 : 0].addr);
+    const void *sp = reinterpret_cast<const void *>(inputs[small_is_0 ? 0 : 1].addr);
+    const long long nl = small_is_0 ? n1 : n0, ns = small_is_0 ? n0 : n1;
+    onhip_add_desc_t d;
+    memset(&d, 0, sizeof(d));
+    const int rank = lt->dim_num_of_shapes;
+    if (nl == ns || ns == 1) {
+        // add.c:48-53: shapes are not looked at
+        d.ndim = 1;
+        d.large_shape[0] = (int32_t) nl;
+        d.small_shape[0] = (int32_t) ns;
+        if (nl >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "Add eval: tensor too large");
+    } else {
+        if (rank < 3 || rank > 6) return set_error(ONHIP_ERR_ARG, "Add eval: broadcast over rank %d (3..6 as add.c:128-141)", rank);
+        const int srank = st->dim_num_of_shapes;
+        if (srank < 1 || srank > rank) return set_error(ONHIP_ERR_ARG, "Add eval: small operand of rank %d", srank);
+        d.ndim = rank;
+        for (int i = 0; i < rank; ++i) {
+            d.large_shape[i] = lt->shapes[i];
+            d.small_shape[i] = i < rank - srank ? 1 : st->shapes[i - (rank - srank)];   // add.c:56-70
+        }
+    }
+    const void *ld, *sd;
+    int rc = input_on_device(0, lp, (size_t) nl * 4, &ld);
+    if (rc) return rc;
+    rc = input_on_device(1, sp, (size_t) ns * 4, &sd);
+    if (rc) return rc;
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, (size_t) nl * 4, &y);
+        if (rc) return rc;
+    }
+    rc = onhip_add_f32(&d, (const float *) ld, (const float *) sd, (float *) y, nullptr);
+    if (rc) return rc;
+    return finish_output(host_out, y, (size_t) nl * 4, out_on_dev);
+}
+
+static int relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    if (!t) return set_error(ONHIP_ERR_ARG, "Relu eval: empty slot");
+    const long long n = numel(t);
+    if (n < 1 || n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "Relu eval: %lld elements", n);
+    const void *x;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), (size_t) n * 4, &x);
+    if (rc) return rc;
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, (size_t) n * 4, &y);
+        if (rc) return rc;
+    }
+    rc = onhip_relu_f32((const float *) x, (float *) y, n, nullptr);
+    if (rc) return rc;
+    return finish_output(host_out, y, (size_t) n * 4, out_on_dev);
+}
+
+static int maxpool_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const MAX_POOL_CONFIG_S *cfg = reinterpret_cast<const MAX_POOL_CONFIG_S *>(params[0].addr);
+    const OPERAND_S *it = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *ot = reinterpret_cast<const OPERAND_S *>(params[2].addr);
+    if (!it || !ot) return set_error(ONHIP_ERR_ARG, "MaxPool eval: empty slot");
+    onhip_pool_desc_t d;
+    // maxpool.c:67-69 loops over the output's batch and channels with the input's strides
+    d.n = ot->shapes[0]; d.c = ot->shapes[1]; d.h = it->shapes[2]; d.w = it->shapes[3];
+    if (d.n > it->shapes[0] || d.c != it->shapes[1])
+        return set_error(ONHIP_ERR_ARG, "MaxPool eval: output %dx%d planes against input %dx%d", d.n, d.c, it->shapes[0], it->shapes[1]);
+    d.kh = (int32_t) cfg->kernel_shape[0]; d.kw = (int32_t) cfg->kernel_shape[1];
+    d.stride_w = (int32_t) cfg->strides[0]; d.stride_h = (int32_t) cfg->strides[1];
+    d.pad = (int32_t) cfg->pads[0];
+    const int32_t oh = ot->shapes[2], ow = ot->shapes[3];
+    const size_t in_bytes = (size_t) d.n * d.c * d.h * d.w * 4, out_bytes = (size_t) d.n * d.c * oh * ow * 4;
+    const void *x;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
+    if (rc) return rc;
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, out_bytes, &y);
+        if (rc) return rc;
+    }
+    rc = onhip_maxpool_f32(&d, oh, ow, (const float *) x, (float *) y, nullptr);
+    if (rc) return rc;
+    return finish_output(host_out, y, out_bytes, out_on_dev);
+}
+
+static int gap_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *it = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    if (!it) return set_error(ONHIP_ERR_ARG, "GlobalAveragePool eval: empty slot");
+    const int n = it->shapes[0], c = it->shapes[1], h = it->shapes[2], w = it->shapes[3];
+    if (n < 1 || c < 1 || h < 1 || w < 1) return set_error(ONHIP_ERR_ARG, "GlobalAveragePool eval: bad shape");
+    const size_t in_bytes = (size_t) n * c * h * w * 4, out_bytes = (size_t) n * c * 4;
+    const void *x;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
+    if (rc) return rc;
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, out_bytes, &y);
+        if (rc) return rc;
+    }
+    rc = onhip_global_avgpool_f32(n, c, h, w, (const float *) x, (float *) y, nullptr);
+    if (rc) return rc;
+    return finish_output(host_out, y, out_bytes, out_on_dev);
+}
+
 template <class F>
 static int guarded(const char *what, F f, BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     if (!params || !inputs || !outputs || !params[0].addr || !inputs[0].addr || !outputs[0].addr) {
@@ -376,6 +502,22 @@ int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_
 }
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Gemm", gemm_eval_locked, params, inputs, outputs);
+}
+
+int onhip_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Add", add_eval_locked, params, inputs, outputs);
+}
+
+int onhip_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Relu", relu_eval_locked, params, inputs, outputs);
+}
+
+int onhip_maxpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MaxPool", maxpool_eval_locked, params, inputs, outputs);
+}
+
+int onhip_global_avgpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("GlobalAveragePool", gap_eval_locked, params, inputs, outputs);
 }
 
 int onhip_plugin_release(void) {

@@ -35,7 +35,9 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out
            "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quant_weight_bias",
            "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
-           "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_plugin_release"]
+           "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
+           "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
+           "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_plugin_release"]
 
 
 def load():
@@ -62,6 +64,10 @@ def load():
     L.onhip_conv2d_w8a32_packed_weight_bytes.restype = C.c_size_t
     L.onhip_conv2d_w8a32_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
     L.onhip_conv2d_w8a32_packed.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
+    L.onhip_add_f32.argtypes = [vp, vp, vp, vp, vp]
+    L.onhip_relu_f32.argtypes = [vp, vp, C.c_longlong, vp]
+    L.onhip_maxpool_f32.argtypes = [vp, C.c_int32, C.c_int32, vp, vp, vp]
+    L.onhip_global_avgpool_f32.argtypes = [C.c_int32] * 4 + [vp, vp, vp]
     L.onhip_quant_weight_bias.argtypes = [vp, vp, C.c_int32, C.c_int32, vp, vp, vp]
     L.onhip_calib_abs_max.argtypes = [vp, C.c_longlong, C.POINTER(C.c_float), vp]
     L.onhip_calib_histogram.argtypes = [vp, C.c_longlong, C.c_float, vp, vp]
@@ -124,6 +130,51 @@ def pack_conv_weights(d, w):
     packed = torch.empty(nbytes // 4, dtype=torch.float32, device=w.device)
     _check(load().onhip_conv2d_pack_weights(C.byref(d), _ptr(w), _ptr(packed), _stream()), "onhip_conv2d_pack_weights")
     return packed
+
+
+def add_f32(large, small, relu=False, out=None):
+    """out = large + small (small broadcast onto large, numpy rules), optionally followed by ReLU"""
+    import torch
+    from onenew_amd.abi import AddDesc
+    d = AddDesc()
+    ls, ss = list(large.shape), list(small.shape)
+    if large.numel() == small.numel() or small.numel() == 1:
+        ls, ss = [large.numel()], [small.numel()]
+    ss = [1] * (len(ls) - len(ss)) + ss
+    d.ndim, d.relu = len(ls), int(relu)
+    for i, (a, b) in enumerate(zip(ls, ss)):
+        d.large_shape[i], d.small_shape[i] = a, b
+    if out is None:
+        out = torch.empty_like(large)
+    _check(load().onhip_add_f32(C.byref(d), _ptr(large), _ptr(small), _ptr(out), _stream()), "onhip_add_f32")
+    return out
+
+
+def relu_f32(x, out=None):
+    import torch
+    if out is None:
+        out = torch.empty_like(x)
+    _check(load().onhip_relu_f32(_ptr(x), _ptr(out), x.numel(), _stream()), "onhip_relu_f32")
+    return out
+
+
+def maxpool_f32(d, x, out=None):
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        out = torch.empty((d.n, d.c, oh, ow), dtype=torch.float32, device=x.device)
+    _check(load().onhip_maxpool_f32(C.byref(d), out.shape[2], out.shape[3], _ptr(x), _ptr(out), _stream()),
+           "onhip_maxpool_f32")
+    return out
+
+
+def global_avgpool_f32(x, out=None):
+    import torch
+    n, c, h, w = x.shape
+    if out is None:
+        out = torch.empty((n, c, 1, 1), dtype=torch.float32, device=x.device)
+    _check(load().onhip_global_avgpool_f32(n, c, h, w, _ptr(x), _ptr(out), _stream()), "onhip_global_avgpool_f32")
+    return out
 
 
 CALIB_BINS, CALIB_KL, CALIB_MSE = 2048, 0, 1

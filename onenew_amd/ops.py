@@ -248,3 +248,99 @@ class Gemm(_Op):
         if rc != 0:
             raise RuntimeError(f"Gemm eval returned {rc}")
         return out
+
+
+class Add(_Op):
+    """host/ops/add.h: out = in0 + in1 with numpy broadcasting of the smaller operand (device/x86/Add/add.c)."""
+
+    def __init__(self, evalfn):
+        super().__init__(evalfn)
+        self.cfg = abi.PLAIN_CONFIG_S()
+        self.cfg.op_base_cfg.op_type = b"Add"
+        self.cfg.op_base_cfg.in_operand_num = 2
+        self.cfg.op_base_cfg.out_operand_num = 1
+        self._slot(self.params_vec, 0, self.cfg)
+
+    def __call__(self, a, b, out=None):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        oshape = a.shape if a.size >= b.size else b.shape
+        if out is None:
+            out = aligned_empty(oshape, np.float32)
+        descs = [make_operand(a.shape, b"a"), make_operand(b.shape, b"b"), make_operand(oshape, b"out")]
+        for i, o in enumerate(descs):
+            self._slot(self.params_vec, 1 + i, o)
+        self._slot(self.inputs_vec, 0, a)
+        self._slot(self.inputs_vec, 1, b)
+        self._slot(self.outputs_vec, 0, out)
+        rc = self.forward()
+        del self._keep[-6:]
+        if rc != 0:
+            raise RuntimeError(f"Add eval returned {rc}")
+        return out
+
+
+class _Unary(_Op):
+    op_type = b""
+
+    def __init__(self, evalfn, cfg=None):
+        super().__init__(evalfn)
+        self.cfg = cfg if cfg is not None else abi.PLAIN_CONFIG_S()
+        self.cfg.op_base_cfg.op_type = self.op_type
+        self.cfg.op_base_cfg.in_operand_num = 1
+        self.cfg.op_base_cfg.out_operand_num = 1
+        self._slot(self.params_vec, 0, self.cfg)
+
+    def out_shape(self, shape):
+        return shape
+
+    def __call__(self, x, out=None):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        oshape = self.out_shape(x.shape)
+        if out is None:
+            out = aligned_empty(oshape, np.float32)
+        descs = [make_operand(x.shape, b"in"), make_operand(oshape, b"out")]
+        self._slot(self.params_vec, 1, descs[0])
+        self._slot(self.params_vec, 2, descs[1])
+        self._slot(self.inputs_vec, 0, x)
+        self._slot(self.outputs_vec, 0, out)
+        rc = self.forward()
+        del self._keep[-4:]
+        if rc != 0:
+            raise RuntimeError(f"{self.op_type.decode()} eval returned {rc}")
+        return out
+
+
+class Relu(_Unary):
+    """host/ops/relu.h (device/x86/Relu/relu.c)"""
+    op_type = b"Relu"
+
+
+class GlobalAveragePool(_Unary):
+    """host/ops/global_avgpool.h (device/x86/GlobalAveragePool/global_avgpool.c)"""
+    op_type = b"GlobalAveragePool"
+
+    def out_shape(self, shape):
+        return (shape[0], shape[1], 1, 1)
+
+
+class MaxPool(_Unary):
+    """host/ops/max_pool.h (device/x86/MaxPool/maxpool.c): square padding pads[0], floor-mode output shape;
+    the kernel takes its scratch for the padded copy from USEFUL_INFO_S in params[11]."""
+    op_type = b"MaxPool"
+
+    def __init__(self, evalfn, kernel, stride, pad, scratch_bytes=0):
+        cfg = abi.MAX_POOL_CONFIG_S()
+        cfg.kernel_shape[0], cfg.kernel_shape[1] = kernel, kernel
+        cfg.strides[0], cfg.strides[1] = stride, stride
+        for i in range(4):
+            cfg.pads[i] = pad
+        super().__init__(evalfn, cfg)
+        self.kernel, self.stride, self.pad = kernel, stride, pad
+        self.useful, self._scratch = make_useful_info(scratch_bytes)
+        self._slot(self.params_vec, BUF_MAXNUM - 1, self.useful)
+
+    def out_shape(self, shape):
+        n, c, h, w = shape
+        return (n, c, (h + 2 * self.pad - self.kernel) // self.stride + 1,
+                (w + 2 * self.pad - self.kernel) // self.stride + 1)

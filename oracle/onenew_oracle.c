@@ -658,3 +658,75 @@ void oracle_round_f16(const float *x, float *y, int64_t count) {
     /* F16C conversion, round to nearest even */
     for (int64_t i = 0; i < count; ++i) y[i] = _cvtsh_ss(_cvtss_sh(x[i], _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC));
 }
+
+
+/* ---------------------------------------------------------------------------------------------
+ * The operators around the convolutions: Add, Relu, MaxPool, GlobalAveragePool
+ * ------------------------------------------------------------------------------------------- */
+
+/* device/x86/Add/add.c:18-80 and fun_0 / fun_1 / fun_2_dim3..6: out has the shape of the operand with
+ * more elements (`large`); `small` is aligned to the same rank and broadcast where its extent is 1 */
+int oracle_add_f32(int ndim, const int32_t *large_shape, const int32_t *small_shape, const float *large,
+                   const float *small, float *out) {
+    if (ndim < 1 || ndim > 6) return -1;
+    int64_t n = 1;
+    int32_t sstride[6], ext[6];
+    int64_t acc = 1;
+    for (int k = ndim - 1; k >= 0; --k) {
+        if (small_shape[k] != large_shape[k] && small_shape[k] != 1) return -1;
+        ext[k] = large_shape[k];
+        sstride[k] = small_shape[k] == 1 ? 0 : (int32_t) acc;      /* add.c:165-167: stride 0 on broadcast dims */
+        acc *= small_shape[k];
+        n *= large_shape[k];
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t rest = i, j = 0;
+        for (int k = ndim - 1; k >= 0; --k) {
+            j += (rest % ext[k]) * sstride[k];
+            rest /= ext[k];
+        }
+        out[i] = large[i] + small[j];
+    }
+    return 0;
+}
+
+/* device/x86/Relu/relu.c:21-52: 32 elements at a time through _mm256_max_ps(0, x) = (0 > x ? 0 : x), the
+ * remaining n % 32 through (x > 0 ? x : 0) */
+void oracle_relu_f32(const float *x, float *y, int64_t n) {
+    const int64_t body = n / 32 * 32;
+    for (int64_t i = 0; i < body; ++i) y[i] = 0.0f > x[i] ? 0.0f : x[i];
+    for (int64_t i = body; i < n; ++i) y[i] = x[i] > 0.0f ? x[i] : 0.0f;
+}
+
+/* device/x86/MaxPool/maxpool.c:40-88 with pad_maxpool.h: pad value -32768000, running maximum from -3276800;
+ * strides[0] steps along w and strides[1] along h */
+int oracle_maxpool_f32(int n, int c, int h, int w, int kh, int kw, int stride_w, int stride_h, int pad, int oh, int ow,
+                       const float *x, float *y) {
+    if ((oh - 1) * stride_h + kh > h + 2 * pad || (ow - 1) * stride_w + kw > w + 2 * pad) return -1;
+    const int ph = h + 2 * pad, pw = w + 2 * pad;
+    float *padded = (float *) malloc((size_t) ph * pw * sizeof(float));
+    for (int p = 0; p < n * c; ++p) {
+        for (int i = 0; i < ph * pw; ++i) padded[i] = -32768000.0f;
+        for (int i = 0; i < h; ++i) memcpy(padded + (size_t) (i + pad) * pw + pad, x + ((size_t) p * h + i) * w, (size_t) w * 4);
+        for (int i = 0; i < oh; ++i)
+            for (int j = 0; j < ow; ++j) {
+                const float *win = padded + (size_t) i * stride_h * pw + j * stride_w;
+                float m = -3276800.0f;
+                for (int a = 0; a < kh; ++a)
+                    for (int b = 0; b < kw; ++b) m = win[a * pw + b] > m ? win[a * pw + b] : m;
+                y[((size_t) p * oh + i) * ow + j] = m;
+            }
+    }
+    free(padded);
+    return 0;
+}
+
+/* device/x86/GlobalAveragePool/global_avgpool.c:27-42 */
+void oracle_global_avgpool_f32(int n, int c, int h, int w, const float *x, float *y) {
+    const float coeff = 1.0f / (h * w);
+    for (int p = 0; p < n * c; ++p) {
+        float psum = 0;
+        for (int i = 0; i < h * w; ++i) psum += x[(size_t) p * h * w + i];
+        y[p] = psum * coeff;
+    }
+}

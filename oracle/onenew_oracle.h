@@ -29,6 +29,13 @@ int oracle_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t
 void oracle_quant_weight_bias(const float *w, const float *bias, int cout, int per_channel, int8_t *w8,
                               int32_t *bias32, float *weight_aux);
 
+int oracle_add_f32(int ndim, const int32_t *large_shape, const int32_t *small_shape, const float *large,
+                   const float *small, float *out);
+void oracle_relu_f32(const float *x, float *y, int64_t n);
+int oracle_maxpool_f32(int n, int c, int h, int w, int kh, int kw, int stride_w, int stride_h, int pad, int oh, int ow,
+                       const float *x, float *y);
+void oracle_global_avgpool_f32(int n, int c, int h, int w, const float *x, float *y);
+
 #define ORACLE_CALIB_BINS 2048
 float oracle_calib_abs_max(const float *x, int64_t n, float running_max);
 void oracle_calib_histogram(const float *x, int64_t n, float max_abs, float *hist);

@@ -146,6 +146,46 @@ def quant_weight_bias(w, bias):
     return w8, b32, aux
 
 
+def add_f32(a, b):
+    """device/x86/Add semantics: the operand with fewer elements (the second on a tie) is broadcast"""
+    a, b = _f32(a), _f32(b)
+    large, small = (b, a) if a.size < b.size else (a, b)
+    ls, ss = list(large.shape), list(small.shape)
+    if large.size == small.size or small.size == 1:
+        ls, ss = [large.size], [small.size]
+    ss = [1] * (len(ls) - len(ss)) + ss
+    out = np.empty(large.shape, np.float32)
+    i32 = C.c_int32 * len(ls)
+    rc = lib().oracle_add_f32(len(ls), i32(*ls), i32(*ss), _p(large, f32p), _p(small, f32p), _p(out, f32p))
+    assert rc == 0, "shapes do not broadcast"
+    return out
+
+
+def relu_f32(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().oracle_relu_f32(_p(x, f32p), _p(y, f32p), C.c_int64(x.size))
+    return y
+
+
+def maxpool_f32(x, kernel, stride, pad):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    oh, ow = (h + 2 * pad - kernel) // stride + 1, (w + 2 * pad - kernel) // stride + 1
+    y = np.empty((n, c, oh, ow), np.float32)
+    rc = lib().oracle_maxpool_f32(n, c, h, w, kernel, kernel, stride, stride, pad, oh, ow, _p(x, f32p), _p(y, f32p))
+    assert rc == 0
+    return y
+
+
+def global_avgpool_f32(x):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    y = np.empty((n, c, 1, 1), np.float32)
+    lib().oracle_global_avgpool_f32(n, c, h, w, _p(x, f32p), _p(y, f32p))
+    return y
+
+
 def calib_abs_max(x, running=0.0):
     x = _f32(x)
     fn = lib().oracle_calib_abs_max

@@ -164,6 +164,68 @@ def gemm_inputs(name, M, K, N):
     return a, w, b
 
 
+def add_cases():
+    """name -> (shape of in0, shape of in1); the operand with fewer elements is broadcast"""
+    return {
+        "add_same": ((1, 64, 14, 14), (1, 64, 14, 14)),            # residual add
+        "add_same_unaligned": ((3, 5, 7), (3, 5, 7)),              # 105 elements: vector body + tail
+        "add_scalar": ((2, 9, 5), (1,)),
+        "add_scalar_first": ((1,), (4, 33)),
+        "add_bias_nchw": ((2, 16, 6, 6), (1, 16, 1, 1)),
+        "add_lower_rank": ((2, 7, 197, 24), (24,)),                # rank 1 onto rank 4 (ViT bias add)
+        "add_rank3_mid": ((5, 1, 12), (5, 9, 12)),                 # broadcast operand given first
+        "add_rank5": ((2, 3, 4, 5, 6), (1, 3, 1, 5, 1)),
+        "add_rank6": ((2, 2, 3, 2, 4, 5), (2, 1, 3, 1, 4, 1)),
+        "rn50_res_l1": ((1, 256, 56, 56), (1, 256, 56, 56)),
+    }
+
+
+def add_inputs(name, s0, s1):
+    return (datagen.normal(datagen.seed_for(name, "a"), s0, 0.0, 1.0),
+            datagen.normal(datagen.seed_for(name, "b"), s1, 0.0, 1.0))
+
+
+def relu_cases():
+    """name -> shape; sizes around the 32-element vector body of relu.c"""
+    return {"relu_31": (31,), "relu_32": (32,), "relu_100": (1, 4, 5, 5), "relu_rn50": (1, 256, 56, 56)}
+
+
+def relu_input(name, shape):
+    x = datagen.normal(datagen.seed_for(name, "x"), shape, 0.0, 1.0).reshape(-1)
+    # signed zeros and a NaN on both sides of the body / tail split: the two rules of relu.c differ there
+    for pos, v in ((0, -0.0), (1, np.nan), (x.size - 1, -0.0), (x.size - 2, np.nan), (x.size // 2, 0.0)):
+        if pos < x.size:
+            x[pos] = v
+    return x.reshape(shape).astype(np.float32)
+
+
+def maxpool_cases():
+    """name -> (input shape, kernel, stride, pad)"""
+    return {
+        "mp_rn50_stem": ((1, 64, 112, 112), 3, 2, 1),
+        "mp_2x2_s2": ((1, 5, 10, 12), 2, 2, 0),
+        "mp_3x3_s1_p1": ((1, 3, 9, 7), 3, 1, 1),
+        "mp_5x5_s1_p2_sppf": ((1, 8, 20, 20), 5, 1, 2),
+        "mp_odd_floor": ((1, 4, 11, 13), 3, 2, 0),
+        "mp_deep_negative": ((1, 2, 6, 6), 2, 2, 0),               # inputs below the -3276800 start value
+    }
+
+
+def maxpool_input(name, shape):
+    x = datagen.normal(datagen.seed_for(name, "x"), shape, 0.0, 1.0)
+    if name == "mp_deep_negative":
+        x = x * np.float32(1e6) - np.float32(4e6)
+    return x.astype(np.float32)
+
+
+def gap_cases():
+    return {"gap_rn50": (1, 2048, 7, 7), "gap_small": (1, 3, 2, 5), "gap_14": (1, 96, 14, 14), "gap_large_plane": (1, 2, 100, 100)}
+
+
+def gap_input(name, shape):
+    return datagen.normal(datagen.seed_for(name, "x"), shape, 0.5, 1.0)
+
+
 def gelu_input():
     """values across the table range, bin edges and both cut-offs"""
     x = datagen.uniform(datagen.seed_for("gelu", "x"), (5000,), -9.0, 9.0)

@@ -58,6 +58,28 @@ def main():
         a, w, b = cases.gemm_inputs(name, M, K, N)
         put(name, ops.Gemm(gemm.eval, w, b)(a))
         print("gemm", name, flush=True)
+    # the operators around the convolutions: Add, Relu, MaxPool, GlobalAveragePool
+    add = ops.Plugin(os.path.join(ref, "libAdd_x86.so"))
+    relu = ops.Plugin(os.path.join(ref, "libRelu_x86.so"))
+    maxpool = ops.Plugin(os.path.join(ref, "libMaxPool_x86.so"))
+    gap = ops.Plugin(os.path.join(ref, "libGlobalAveragePool_x86.so"))
+    for name, (s0, s1) in cases.add_cases().items():
+        a, b = cases.add_inputs(name, s0, s1)
+        put(name, ops.Add(add.eval)(a, b))
+        print("add", name, flush=True)
+    for name, shape in cases.relu_cases().items():
+        xin = ops.aligned_empty(shape)
+        xin[...] = cases.relu_input(name, shape)
+        put(name, ops.Relu(relu.eval)(xin))
+        print("relu", name, flush=True)
+    for name, (shape, k, st, pad) in cases.maxpool_cases().items():
+        x = cases.maxpool_input(name, shape)
+        scratch = 4 * x.size * 4 + (1 << 20)
+        put(name, ops.MaxPool(maxpool.eval, k, st, pad, scratch_bytes=scratch)(x))
+        print("maxpool", name, flush=True)
+    for name, shape in cases.gap_cases().items():
+        put(name, ops.GlobalAveragePool(gap.eval)(cases.gap_input(name, shape)))
+        print("gap", name, flush=True)
     # table GELU (device/x86/Gelu/gelu.c) on edge values
     x = cases.gelu_input()
     params = (abi.BUFFER_INFO_S * abi.BUF_MAXNUM)()

@@ -438,3 +438,71 @@ def test_calibration_percentile_matches_oracle(torch_dev, oracle):
     images, elems = 3, 400000
     x = _calib_tensor(cases.datagen.seed_for("calib_gpu", "pct"), images * elems)
     assert hip.calib_percentile(dev(torch, x), images, elems) == oracle.calib_percentile(x, images, elems)
+
+
+def _same_bits(a, b):
+    return np.array_equal(np.ascontiguousarray(a).reshape(-1).view(np.uint32),
+                          np.ascontiguousarray(b).reshape(-1).view(np.uint32))
+
+
+@pytest.mark.parametrize("name", list(cases.add_cases()))
+def test_add_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
+    """kernel level (incl. the fused ReLU) and the Add plugin on host buffers: bit-identical to the reference"""
+    torch = torch_dev
+    a, b = cases.add_inputs(name, *cases.add_cases()[name])
+    ref = oracle.add_f32(a, b)
+    large, small = (b, a) if a.size < b.size else (a, b)
+    y = hip.add_f32(dev(torch, large), dev(torch, small))
+    yr = hip.add_f32(dev(torch, large), dev(torch, small), relu=True)
+    torch.cuda.synchronize()
+    assert _same_bits(y.cpu().numpy(), ref)
+    assert _same_bits(yr.cpu().numpy(), np.where(ref > 0, ref, np.float32(0)))
+    cases.check_against(golden, name, y.cpu().numpy(), exact=True)
+    assert _same_bits(ops.Add(ops.Plugin(hip.plugin_path("Add")).eval)(a, b), ref)
+
+
+@pytest.mark.parametrize("name", list(cases.relu_cases()))
+def test_relu_matches_oracle_and_plugin(name, torch_dev, oracle):
+    torch = torch_dev
+    x = cases.relu_input(name, cases.relu_cases()[name])
+    ref = oracle.relu_f32(x)
+    y = hip.relu_f32(dev(torch, x))
+    torch.cuda.synchronize()
+    assert _same_bits(y.cpu().numpy(), ref)          # signed zeros and NaNs included
+    xin = ops.aligned_empty(x.shape)
+    xin[...] = x
+    assert _same_bits(ops.Relu(ops.Plugin(hip.plugin_path("Relu")).eval)(xin), ref)
+
+
+@pytest.mark.parametrize("name", list(cases.maxpool_cases()))
+def test_maxpool_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
+    torch = torch_dev
+    shape, k, st, pad = cases.maxpool_cases()[name]
+    x = cases.maxpool_input(name, shape)
+    ref = oracle.maxpool_f32(x, k, st, pad)
+    d = abi.PoolDesc(shape[0], shape[1], shape[2], shape[3], k, k, st, st, pad)
+    y = hip.maxpool_f32(d, dev(torch, x))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), ref)
+    cases.check_against(golden, name, y.cpu().numpy(), exact=True)
+    assert np.array_equal(ops.MaxPool(ops.Plugin(hip.plugin_path("MaxPool")).eval, k, st, pad)(x), ref)
+    # a batch is that many independent images
+    xb = np.concatenate([x, x[:, ::-1].copy()], axis=0)
+    db = abi.PoolDesc(2, shape[1], shape[2], shape[3], k, k, st, st, pad)
+    yb = hip.maxpool_f32(db, dev(torch, xb)).cpu().numpy()
+    assert np.array_equal(yb[0], ref[0]) and np.array_equal(yb[1], oracle.maxpool_f32(xb[1:2], k, st, pad)[0])
+
+
+@pytest.mark.parametrize("name", list(cases.gap_cases()))
+def test_global_avgpool_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
+    torch = torch_dev
+    x = cases.gap_input(name, cases.gap_cases()[name])
+    ref = oracle.global_avgpool_f32(x)
+    y = hip.global_avgpool_f32(dev(torch, x))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), ref)      # same summation order: bit-identical
+    cases.check_against(golden, name, y.cpu().numpy(), exact=True)
+    assert np.array_equal(ops.GlobalAveragePool(ops.Plugin(hip.plugin_path("GlobalAveragePool")).eval)(x), ref)
+    xb = np.concatenate([x] * 3, axis=0)
+    yb = hip.global_avgpool_f32(dev(torch, xb)).cpu().numpy()
+    assert np.array_equal(yb, np.concatenate([ref] * 3, axis=0))

@@ -45,3 +45,42 @@ def test_tables_regenerate(oracle):
     assert np.array_equal(oracle.silu_lut(), cases.silu_lut())
     assert np.array_equal(oracle.gelu_lut(), cases.gelu_lut())
     assert cases.silu_lut()[4608] == np.float32(0.731058598) and cases.gelu_lut()[4608] == np.float32(0.841347098)
+
+
+@pytest.mark.parametrize("name", list(cases.add_cases()))
+def test_add_bit_exact(name, golden, oracle):
+    a, b = cases.add_inputs(name, *cases.add_cases()[name])
+    y = oracle.add_f32(a, b)
+    cases.check_against(golden, name, y, exact=True)
+    if np.broadcast_shapes(a.shape, b.shape) == y.shape:
+        assert np.array_equal(y, a + b)            # numpy's broadcasting is the closed form
+
+
+@pytest.mark.parametrize("name", list(cases.relu_cases()))
+def test_relu_bit_exact(name, golden, oracle):
+    """bit patterns, so that the signed zeros and NaNs either side of the 32-element body count"""
+    x = cases.relu_input(name, cases.relu_cases()[name])
+    y = oracle.relu_f32(x)
+    key = f"{name}/full" if f"{name}/full" in golden else None
+    if key:
+        assert np.array_equal(golden[key].view(np.uint32), y.reshape(-1).view(np.uint32))
+    else:
+        idx = cases.sample_indices(name, y.size)
+        assert np.array_equal(golden[f"{name}/samples"].view(np.uint32), y.reshape(-1)[idx].view(np.uint32))
+
+
+@pytest.mark.parametrize("name", list(cases.maxpool_cases()))
+def test_maxpool_bit_exact(name, golden, oracle):
+    shape, k, st, pad = cases.maxpool_cases()[name]
+    y = oracle.maxpool_f32(cases.maxpool_input(name, shape), k, st, pad)
+    cases.check_against(golden, name, y, exact=True)
+    if name == "mp_deep_negative":
+        assert y.min() == np.float32(-3276800.0)   # the start value of the running maximum shows through
+
+
+@pytest.mark.parametrize("name", list(cases.gap_cases()))
+def test_global_avgpool_bit_exact(name, golden, oracle):
+    x = cases.gap_input(name, cases.gap_cases()[name])
+    y = oracle.global_avgpool_f32(x)
+    cases.check_against(golden, name, y, exact=True)
+    assert np.allclose(y.reshape(x.shape[:2]), x.astype(np.float64).mean(axis=(2, 3)), rtol=1e-5, atol=1e-6)
