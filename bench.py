@@ -111,6 +111,63 @@ class ConvW8A32Layer:
         return d1.flops(), lambda: oracle.conv2d_w8a32(d1, x, w8, b32, aux, cases.silu_lut())
 
 
+class GlueLayer:
+    """the memory-bound operators between the convolutions of ResNet-50: MaxPool after the stem, the residual
+    Add + ReLU of every block (one fused pass), GlobalAveragePool at the end"""
+    kind = "glue"
+    dense = False
+
+    def __init__(self, torch, hip, name, op, shape, tag):
+        from onenew_amd import abi, datagen
+        self.name, self.op = name, op
+        n, c, h, w = shape
+        rnd = lambda role: torch.from_numpy(datagen.normal(datagen.seed_for(f"{tag}/{name}", role), shape, 0.0, 1.0)).cuda()
+        self.x = rnd("x")
+        if op == "add_relu":
+            self.r = rnd("r")
+            self.y = torch.empty_like(self.x)
+            self.flops, self.bytes = 2 * self.x.numel(), 12 * self.x.numel()
+        elif op == "maxpool":
+            self.pd = abi.PoolDesc(n, c, h, w, 3, 3, 2, 2, 1)
+            oh, ow = self.pd.out_hw()
+            self.y = torch.empty((n, c, oh, ow), dtype=torch.float32, device="cuda")
+            self.flops, self.bytes = 9 * self.y.numel(), 4 * (self.x.numel() + self.y.numel())
+        else:
+            self.y = torch.empty((n, c, 1, 1), dtype=torch.float32, device="cuda")
+            self.flops, self.bytes = self.x.numel(), 4 * (self.x.numel() + self.y.numel())
+        self.shape = f"{op} {n}x{c}x{h}x{w}"
+
+    def launch(self, hip):
+        if self.op == "add_relu":
+            hip.add_f32(self.x, self.r, relu=True, out=self.y)
+        elif self.op == "maxpool":
+            hip.maxpool_f32(self.pd, self.x, out=self.y)
+        else:
+            hip.global_avgpool_f32(self.x, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        """the reference's own Add then Relu (two passes), MaxPool, GlobalAveragePool on one image"""
+        import os
+        x = self.x[:1].cpu().numpy()
+        ref = lambda op: ops.Plugin(os.path.join(os.path.dirname(oracle.ref_path("Conv")), f"lib{op}_x86.so")).eval
+        if self.op == "add_relu":
+            r = self.r[:1].cpu().numpy()
+            if oracle.have_ref():
+                add, relu = ops.Add(ref("Add")), ops.Relu(ref("Relu"))
+                buf = ops.aligned_empty(x.shape)
+                return self.flops // self.x.shape[0], lambda: relu(add(x, r, out=buf))
+            return self.flops // self.x.shape[0], lambda: oracle.relu_f32(oracle.add_f32(x, r))
+        if self.op == "maxpool":
+            if oracle.have_ref():
+                mp = ops.MaxPool(ref("MaxPool"), 3, 2, 1, scratch_bytes=8 * x.size + (1 << 20))
+                return self.flops // self.x.shape[0], lambda: mp(x)
+            return self.flops // self.x.shape[0], lambda: oracle.maxpool_f32(x, 3, 2, 1)
+        if oracle.have_ref():
+            gp = ops.GlobalAveragePool(ref("GlobalAveragePool"))
+            return self.flops // self.x.shape[0], lambda: gp(x)
+        return self.flops // self.x.shape[0], lambda: oracle.global_avgpool_f32(x)
+
+
 class MatmulLayer:
     kind = "matmul"
 
@@ -162,6 +219,15 @@ def make_workload(torch, hip, name):
         n = int(name.split("_b")[1])
         return (f"ResNet-50 conv stack fp32, batch {n}, 224x224, 53 conv layers, fused ReLU", "f32",
                 conv_stack(stacks.with_batch(stacks.resnet50(), n)))
+    if name.startswith("resnet50_glue_b"):
+        n = int(name.split("_b")[1])
+        spec = [("maxpool", "maxpool", (n, 64, 112, 112))]
+        for stage, (c, hw, blocks) in enumerate([(256, 56, 3), (512, 28, 4), (1024, 14, 6), (2048, 7, 3)], 1):
+            spec += [(f"l{stage}.{b}.add_relu", "add_relu", (n, c, hw, hw)) for b in range(blocks)]
+        spec.append(("avgpool", "gap", (n, 2048, 7, 7)))
+        return (f"ResNet-50 operators between the convolutions fp32, batch {n}: MaxPool 3x3 s2, 16 residual "
+                f"Add + ReLU (fused), GlobalAveragePool", "f32",
+                [GlueLayer(torch, hip, ln, op, shape, tag) for ln, op, shape in spec])
     if name.startswith("mobilenetv2_b"):
         n = int(name.split("_b")[1])
         return (f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers (17 depthwise), ReLU6 as CLIP", "f32",
@@ -329,7 +395,8 @@ def main():
     grp = groups[dom_dense]
     g_ms = sum(t for _, t in grp)
     g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
-    kernel = f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else "onhip::depthwise_tiled_kernel"
+    kernel = (f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
+              "onhip::add_kernel / maxpool_kernel / gap_kernel" if grp[0][0].kind == "glue" else "onhip::depthwise_tiled_kernel")
     # the bound is the roof the group's arithmetic intensity puts it under
     mfma_bound = dom_dense and g_flops / g_bytes >= PEAK[dtype] * 1e12 / (HBM_PEAK_GBS * 1e9)
     if mfma_bound:
@@ -338,7 +405,8 @@ def main():
         achieved, peak, r_unit, work = g_bytes / (g_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", g_bytes
     roofline = {"kernel": kernel, "bound": "mfma" if mfma_bound else "hbm", "achieved": round(achieved, 3),
                 "peak": peak, "unit": r_unit, "frac": round(achieved / peak, 4),
-                "traffic": measured_traffic(args.workload, "igemm" if dom_dense else "depthwise"),
+                "traffic": measured_traffic(args.workload, "igemm" if dom_dense else
+                                             "glue" if grp[0][0].kind == "glue" else "depthwise"),
                 "launches": len(grp), "avg_launch_ms": round(g_ms / len(grp), 5),
                 "work_per_launch": work / len(grp),
                 "arithmetic_intensity": round(g_flops / g_bytes, 2)}
@@ -368,7 +436,7 @@ def main():
 
     cpu = None if args.no_cpu else cpu_baseline(layers, args.workload, unit)
 
-    metric = {"resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
+    metric = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
               "yolov8s": "yolov8s_conv_stack_w8a32_tops", "vit": f"vit_tiny_matmul_{dtype}_tflops",
               "cfg1": "conv2d_relu_fp32_tflops"}
     key = next(k for k in metric if args.workload.startswith(k))
