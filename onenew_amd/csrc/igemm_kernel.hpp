@@ -16,9 +16,11 @@
 //     buffer afterwards: one barrier per K tile.
 //
 // B never exists in memory.  BL_GATHER builds it element by element from NCHW activations
-// (implicit im2col) or from a row-major [K, N] matrix, with lanes running along N so every load
-// instruction is a coalesced run of pixels.  BL_KVEC reads 16-byte vectors along K from NHWC int8
-// activations (K ordered tap-major, channel-minor) or from an [N, K] matrix.
+// (implicit im2col), BL_TAPC does the same against tap-major packed weights (one filter tap per
+// unit), BL_PLAIN reads a 1x1 convolution's input or a row-major [K, N] matrix; in all three lanes
+// run along N so every load instruction is a coalesced run of pixels.  BL_KVEC reads 16-byte
+// vectors along K from NHWC int8 activations (K ordered tap-major, channel-minor), the units of a
+// column on neighbouring lanes.
 //
 // Every global access is a raw buffer instruction: the per-lane byte offset (the pixel, fixed for
 // the whole K loop) goes in the vector offset, the wavefront-uniform part (channel, filter tap,
@@ -227,7 +229,7 @@ struct BPrep {
     unsigned hi;   // the tap index is 32..63: test mask_hi
 };
 
-// item: (unit slot t, element e) for the element loaders, unit slot t for the vector loader
+// item: (unit slot t, element e) for BL_PLAIN / BL_GATHER, unit slot t for BL_TAPC (BL_KVEC works per lane)
 template <int DT, int BL>
 __device__ __forceinline__ BPrep prep_b(const IgemmParams &p, int u, int e, int klim) {
     constexpr int KPU = Traits<DT>::KPU;
@@ -252,8 +254,7 @@ __device__ __forceinline__ BPrep prep_b(const IgemmParams &p, int u, int e, int 
         const unsigned cb = (unsigned) u - tap * (unsigned) p.units_per_tap;
         const unsigned i = fast_div(tap, p.magic_kw, p.pass_kw);
         const unsigned j = tap - i * (unsigned) p.kw;
-        if constexpr (BL == BL_TAPC) r.soff = (cb * (unsigned) KPU * (unsigned) p.HW + i * (unsigned) p.W + j) * 4u;
-        else r.soff = (i * (unsigned) p.W + j) * (unsigned) p.pix_stride + cb * 16u;
+        r.soff = (cb * (unsigned) KPU * (unsigned) p.HW + i * (unsigned) p.W + j) * 4u;
         r.bit = u * KPU < klim ? (1u << (tap & 31u)) : 0u;
         r.hi = tap >> 5;
     }
