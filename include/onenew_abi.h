@@ -177,6 +177,33 @@ typedef struct {
     int64_t strides[2];         /* [0] steps along w, [1] along h (maxpool.c:20-21,72) */
 } MAX_POOL_CONFIG_S;
 
+/* common/nn_common.h:322-325 */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+} GELU_CONFIG_S;
+
+/* common/nn_common.h:353-359 */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    int32_t axes[8];            /* axes[0] == 1 selects the strided form */
+    int32_t axes_num;
+    int32_t keepdims;
+} LAYERNORMALIZATION_CONFIG_S;
+
+/* common/nn_common.h:545-550 */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    int64_t dims;
+    int64_t axis;
+} SOFTMAX_CONFIG_S;
+
+/* common/nn_common.h:584-590 */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    int64_t perm[8];
+    int64_t perm_num;
+} TRANSPOSE_CONFIG_S;
+
 /* the one symbol a plugin exports */
 typedef int (*onenew_eval_fn)(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 
@@ -215,6 +242,10 @@ ONENEW_SA(sizeof(MAX_POOL_CONFIG_S) == 12912, "MAX_POOL_CONFIG_S");
 ONENEW_SA(offsetof(MAX_POOL_CONFIG_S, kernel_shape) == 12848, "MAX_POOL.kernel_shape");
 ONENEW_SA(offsetof(MAX_POOL_CONFIG_S, pads) == 12864, "MAX_POOL.pads");
 ONENEW_SA(offsetof(MAX_POOL_CONFIG_S, strides) == 12896, "MAX_POOL.strides");
+ONENEW_SA(sizeof(GELU_CONFIG_S) == 12840, "GELU_CONFIG_S");
+ONENEW_SA(sizeof(LAYERNORMALIZATION_CONFIG_S) == 12880 && offsetof(LAYERNORMALIZATION_CONFIG_S, axes) == 12840, "LAYERNORMALIZATION_CONFIG_S");
+ONENEW_SA(sizeof(SOFTMAX_CONFIG_S) == 12856 && offsetof(SOFTMAX_CONFIG_S, axis) == 12848, "SOFTMAX_CONFIG_S");
+ONENEW_SA(sizeof(TRANSPOSE_CONFIG_S) == 12912 && offsetof(TRANSPOSE_CONFIG_S, perm_num) == 12904, "TRANSPOSE_CONFIG_S");
 ONENEW_SA(sizeof(USEFUL_INFO_S) == 96, "USEFUL_INFO_S");
 ONENEW_SA(offsetof(USEFUL_INFO_S, block_info) == 4, "USEFUL.block_info");
 ONENEW_SA(offsetof(USEFUL_INFO_S, public_buf_info) == 40, "USEFUL.public_buf_info");

@@ -187,6 +187,33 @@ int onhip_maxpool_f32(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const 
 int onhip_global_avgpool_f32(int32_t n, int32_t c, int32_t h, int32_t w, const float *x, float *y,
                              void *stream);
 
+/* ---- the operators around the MatMuls of a transformer block (device pointers) ----------------- */
+
+/* y = table GELU of x: 0 below -8, x from 8 up, else gelu_lut[(int)((x + 8) * 512)] (8192 floats,
+ * host/ops/gelu.h:80-96).  Replaces device/x86/Gelu/gelu.c eval (:9-42). */
+int onhip_gelu_lut_f32(const float *x, const float *gelu_lut, float *y, long long n, void *stream);
+
+/* Layer normalisation of `rows` rows of `reduce` elements with per-element weight and bias, eps 1e-20.
+ * strided == 0: rows are contiguous (the last non-1 dimension is normalised,
+ * layer_normalization.c:62-97); strided != 0: element i of row r lies at i * rows + r (the "axes[0]
+ * == 1" form, :28-60).  Replaces device/x86/LayerNormalization/layer_normalization.c eval (:10-101). */
+int onhip_layernorm_f32(int32_t rows, int32_t reduce, int32_t strided, const float *x,
+                        const float *weight, const float *bias, float *y, void *stream);
+
+/* Softmax over `reduce` elements, `rows` times; strided as above (axis 1 of a batch-1 tensor).
+ * Replaces device/x86/Softmax/softmax.c eval_dim_last (:26-59) and eval_dim_1 (:62-118). */
+int onhip_softmax_f32(int32_t rows, int32_t reduce, int32_t strided, const float *x, float *y,
+                      void *stream);
+
+/* y = x with output dimension k taken from input dimension perm[k].  Replaces
+ * device/x86/Transpose/transpose.c eval_perm_num4 (:24-79) and eval_perm_num6 (:81-140). */
+typedef struct {
+    int32_t ndim;            /* 1..6 */
+    int32_t in_shape[6];
+    int32_t perm[6];
+} onhip_transpose_desc_t;
+int onhip_transpose_f32(const onhip_transpose_desc_t *d, const float *x, float *y, void *stream);
+
 /* ---- offline quantisation: what produces the operands of onhip_conv2d_w8a32 ------------------ */
 
 /* Per output channel: weight_aux = max|w|, w8 = (int8)(w * 127 / aux) (truncating),
@@ -227,6 +254,11 @@ int onhip_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *
 int onhip_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_maxpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_global_avgpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* Gelu (gelu.c:9), LayerNormalization (layer_normalization.c:10), Softmax (softmax.c:12), Transpose (transpose.c:13) */
+int onhip_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_layernorm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_softmax_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Drops the device copies of weights the plugin level keeps between calls. */
 int onhip_plugin_release(void);

@@ -96,6 +96,23 @@ class MAX_POOL_CONFIG_S(C.Structure):
                 ("pads", C.c_int64 * 4), ("strides", C.c_int64 * 2)]
 
 
+class LAYERNORMALIZATION_CONFIG_S(C.Structure):
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("axes", C.c_int32 * 8), ("axes_num", C.c_int32), ("keepdims", C.c_int32)]
+
+
+class SOFTMAX_CONFIG_S(C.Structure):
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("dims", C.c_int64), ("axis", C.c_int64)]
+
+
+class TRANSPOSE_CONFIG_S(C.Structure):
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("perm", C.c_int64 * 8), ("perm_num", C.c_int64)]
+
+
+class TransposeDesc(C.Structure):
+    """onhip_transpose_desc_t"""
+    _fields_ = [("ndim", C.c_int32), ("in_shape", C.c_int32 * 6), ("perm", C.c_int32 * 6)]
+
+
 class AddDesc(C.Structure):
     """onhip_add_desc_t"""
     _fields_ = [("ndim", C.c_int32), ("large_shape", C.c_int32 * 6), ("small_shape", C.c_int32 * 6),
@@ -171,6 +188,8 @@ def check_layout():
     assert C.sizeof(GEMM_CONFIG_S) == 12864 and GEMM_CONFIG_S.transB.offset == 12856
     assert C.sizeof(MATMUL_CONFIG_S) == 12840
     assert C.sizeof(MAX_POOL_CONFIG_S) == 12912 and MAX_POOL_CONFIG_S.strides.offset == 12896
+    assert C.sizeof(LAYERNORMALIZATION_CONFIG_S) == 12880 and C.sizeof(SOFTMAX_CONFIG_S) == 12856
+    assert C.sizeof(TRANSPOSE_CONFIG_S) == 12912 and TRANSPOSE_CONFIG_S.perm_num.offset == 12904
     assert C.sizeof(USEFUL_INFO_S) == 96 and USEFUL_INFO_S.public_buf_info.offset == 40
     assert C.sizeof(ConvDesc) == 25 * 4
     assert C.sizeof(MatmulDesc) == 24

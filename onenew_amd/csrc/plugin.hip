@@ -473,6 +473,126 @@ static int gap_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
     return finish_output(host_out, y, out_bytes, out_on_dev);
 }
 
+// ---- Gelu / LayerNormalization / Softmax / Transpose ------------------------------------------------------
+// shared shape of the unary operators: input 0 on the device, output staged or in place
+struct UnaryIo {
+    const void *x;
+    void *y, *host_out;
+    size_t out_bytes;
+    bool out_on_dev;
+};
+static int unary_io(BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, size_t in_bytes, size_t out_bytes, UnaryIo *io) {
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &io->x);
+    if (rc) return rc;
+    io->host_out = reinterpret_cast<void *>(outputs[0].addr);
+    io->y = io->host_out;
+    io->out_bytes = out_bytes;
+    io->out_on_dev = is_device_ptr(io->host_out);
+    if (!io->out_on_dev) rc = stage_buf(2, out_bytes, &io->y);
+    return rc;
+}
+
+static int gelu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    if (!t || !inputs[BUF_MAXNUM - 1].addr) return set_error(ONHIP_ERR_ARG, "Gelu eval: empty slot (the table is inputs[11])");
+    const long long n = numel(t);
+    if (n < 1 || n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "Gelu eval: %lld elements", n);
+    const void *lut;
+    int rc = const_on_device(reinterpret_cast<const void *>(inputs[BUF_MAXNUM - 1].addr), 8192 * 4, &lut);
+    if (rc) return rc;
+    UnaryIo io;
+    rc = unary_io(inputs, outputs, (size_t) n * 4, (size_t) n * 4, &io);
+    if (rc) return rc;
+    rc = onhip_gelu_lut_f32((const float *) io.x, (const float *) lut, (float *) io.y, n, nullptr);
+    if (rc) return rc;
+    return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
+}
+
+static int layernorm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const LAYERNORMALIZATION_CONFIG_S *cfg = reinterpret_cast<const LAYERNORMALIZATION_CONFIG_S *>(params[0].addr);
+    const OPERAND_S *t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    if (!t || !inputs[1].addr || !inputs[2].addr) return set_error(ONHIP_ERR_ARG, "LayerNormalization eval: empty slot");
+    const long long n = numel(t);
+    if (n < 1 || n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "LayerNormalization eval: %lld elements", n);
+    int reduce = 1, strided = 0;
+    if (cfg->axes[0] == 1) {
+        reduce = t->shapes[1];                         // layer_normalization.c:28-31
+        strided = 1;
+    } else {
+        for (int i = SHAPE_LEN - 1; i >= 0; --i)       // :63-68: the last dimension that is not 1
+            if (t->shapes[i] != 1) { reduce = t->shapes[i]; break; }
+    }
+    if (reduce < 1) return set_error(ONHIP_ERR_ARG, "LayerNormalization eval: bad shape");
+    const int rows = (int) (n / reduce);
+    const void *w, *b;
+    int rc = const_on_device(reinterpret_cast<const void *>(inputs[1].addr), (size_t) reduce * 4, &w);
+    if (rc) return rc;
+    rc = const_on_device(reinterpret_cast<const void *>(inputs[2].addr), (size_t) reduce * 4, &b);
+    if (rc) return rc;
+    UnaryIo io;
+    rc = unary_io(inputs, outputs, (size_t) n * 4, (size_t) n * 4, &io);
+    if (rc) return rc;
+    rc = onhip_layernorm_f32(rows, reduce, strided, (const float *) io.x, (const float *) w, (const float *) b, (float *) io.y,
+                             nullptr);
+    if (rc) return rc;
+    return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
+}
+
+static int softmax_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const SOFTMAX_CONFIG_S *cfg = reinterpret_cast<const SOFTMAX_CONFIG_S *>(params[0].addr);
+    const OPERAND_S *t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    if (!t) return set_error(ONHIP_ERR_ARG, "Softmax eval: empty slot");
+    const int nd = t->dim_num_of_shapes;
+    if (nd < 1 || nd > SHAPE_LEN) return set_error(ONHIP_ERR_ARG, "Softmax eval: rank %d", nd);
+    long long rows = 1;
+    int reduce, strided;
+    if (cfg->axis == -1 || cfg->axis == nd - 1) {      // softmax.c:18-19, :36-41
+        for (int i = 0; i < nd - 1; ++i) rows *= t->shapes[i];
+        reduce = t->shapes[nd - 1];
+        strided = 0;
+    } else if (cfg->axis == 1 && t->shapes[0] == 1) {  // :20-21, :72-77
+        for (int i = 2; i < nd; ++i) rows *= t->shapes[i];
+        reduce = t->shapes[1];
+        strided = 1;
+    } else {
+        return set_error(ONHIP_ERR_ARG, "Softmax eval: axis %lld of a rank-%d tensor is not supported (last axis, or axis 1 "
+                                        "of a batch-1 tensor, as the reference)", (long long) cfg->axis, nd);
+    }
+    if (rows < 1 || reduce < 1 || rows * reduce >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "Softmax eval: bad shape");
+    UnaryIo io;
+    int rc = unary_io(inputs, outputs, (size_t) rows * reduce * 4, (size_t) rows * reduce * 4, &io);
+    if (rc) return rc;
+    rc = onhip_softmax_f32((int) rows, reduce, strided, (const float *) io.x, (float *) io.y, nullptr);
+    if (rc) return rc;
+    return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
+}
+
+static int transpose_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const TRANSPOSE_CONFIG_S *cfg = reinterpret_cast<const TRANSPOSE_CONFIG_S *>(params[0].addr);
+    const OPERAND_S *t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    if (!t) return set_error(ONHIP_ERR_ARG, "Transpose eval: empty slot");
+    const int pn = (int) cfg->perm_num;
+    if (pn < 1 || pn > 6) return set_error(ONHIP_ERR_ARG, "Transpose eval: %d axes (up to 6 as transpose.c:18-24)", pn);
+    // transpose.c works on 4 (perm_num <= 4) or 6 dimensions; trailing dimensions keep their place
+    const int nd = pn <= 4 ? 4 : 6;
+    onhip_transpose_desc_t d;
+    memset(&d, 0, sizeof(d));
+    d.ndim = nd;
+    long long n = 1;
+    for (int i = 0; i < nd; ++i) {
+        d.in_shape[i] = t->shapes[i];
+        d.perm[i] = i < pn ? (int32_t) cfg->perm[i] : i;
+        n *= t->shapes[i];
+    }
+    if (n < 1 || n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "Transpose eval: %lld elements", n);
+    UnaryIo io;
+    int rc = unary_io(inputs, outputs, (size_t) n * 4, (size_t) n * 4, &io);
+    if (rc) return rc;
+    rc = onhip_transpose_f32(&d, (const float *) io.x, (float *) io.y, nullptr);
+    if (rc) return rc;
+    return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
+}
+
 template <class F>
 static int guarded(const char *what, F f, BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     if (!params || !inputs || !outputs || !params[0].addr || !inputs[0].addr || !outputs[0].addr) {
@@ -518,6 +638,22 @@ int onhip_maxpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO
 
 int onhip_global_avgpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("GlobalAveragePool", gap_eval_locked, params, inputs, outputs);
+}
+
+int onhip_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Gelu", gelu_eval_locked, params, inputs, outputs);
+}
+
+int onhip_layernorm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("LayerNormalization", layernorm_eval_locked, params, inputs, outputs);
+}
+
+int onhip_softmax_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Softmax", softmax_eval_locked, params, inputs, outputs);
+}
+
+int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Transpose", transpose_eval_locked, params, inputs, outputs);
 }
 
 int onhip_plugin_release(void) {

@@ -1,0 +1,265 @@
+// The operators either side of the MatMuls of a transformer block: table GELU, LayerNormalization,
+// Softmax and Transpose.  All are bound by memory bandwidth.  GELU, LayerNormalization and Transpose
+// reproduce device/x86/Gelu/gelu.c, LayerNormalization/layer_normalization.c and
+// Transpose/transpose.c bit for bit; Softmax (device/x86/Softmax/softmax.c) differs from the
+// reference by the last bits of expf and is held to the fp32 tolerance.
+#include <string.h>
+
+#include "onhip_internal.hpp"
+
+namespace onhip {
+
+__device__ __forceinline__ unsigned vg_div(unsigned x, const Div31 &d) {
+    return (__umulhi(x, d.magic) >> d.shift) + (x & d.pass);
+}
+
+// ---- table GELU (gelu.c:22-38) ------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gelu_lut_kernel(const float *__restrict__ x, const float *__restrict__ lut,
+                                                       float *__restrict__ y, long long n) {
+    const long long i = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    float r;
+    if (v < -8.0f) r = 0.0f;
+    else if (v >= 8.0f) r = v;
+    else {
+        int idx = (int) __fmul_rn(__fadd_rn(v, 8.0f), 512.0f);
+        idx = idx > 8191 ? 8191 : idx;     // v just below 8: v + 8 rounds to 16 and the reference reads one past the table
+        r = lut[idx];
+    }
+    y[i] = r;                              // a NaN fails both comparisons and indexes the table with (int) NaN
+}
+
+// ---- LayerNormalization ---------------------------------------------------------------------------------
+// layer_normalization.c:62-97: per row, psum and psum of squares added up element by element in float, then
+// mean = psum / n (as a product with 1/n), var = (1/n) * psq - mean * mean, + 1e-20 (a double constant),
+// 1 / sqrtf(var), and out = (x - mean) * inv_std * weight + bias with every operation rounded.
+__device__ __forceinline__ void ln_stats(float psum, float psq, float inv_n, float *mean, float *inv_std) {
+    const float m = __fmul_rn(psum, inv_n);
+    float var = __fsub_rn(__fmul_rn(inv_n, psq), __fmul_rn(m, m));
+    var = (float) ((double) var + 1e-20);
+    *mean = m;
+    // sqrtf, then 1 / std, each correctly rounded as on the CPU.  The single-precision square root of this
+    // toolchain is the bare v_sqrt_f32 (a last bit off on some inputs); the double-precision one rounded to float
+    // is exact (53 >= 2 * 24 + 2 bits).  The two steps are kept apart so that they cannot merge into v_rsq_f32.
+    float sd = (float) sqrt((double) var);
+    asm volatile("" : "+v"(sd));
+    *inv_std = __fdiv_rn(1.0f, sd);
+}
+
+constexpr int LN_LDS_FLOATS = 8192;
+
+// rows contiguous in memory: a workgroup stages `rpw` rows in LDS (pitch reduce + 1, so the threads that
+// each add up one row hit different banks), one thread per row does the sums in memory order, then all
+// threads normalise and store
+__global__ __launch_bounds__(256) void layernorm_rows_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                             const float *__restrict__ b, float *__restrict__ y, int rows,
+                                                             int reduce, int rpw, float inv_n) {
+    __shared__ float tile[LN_LDS_FLOATS];
+    __shared__ float s_mean[64], s_inv[64];
+    const int row0 = blockIdx.x * rpw;
+    const int nr = min(rpw, rows - row0);
+    const int pitch = reduce + 1;
+    const float *src = x + (long long) row0 * reduce;
+    const int total = nr * reduce;
+    for (int i = threadIdx.x; i < total; i += 256) {
+        const int r = i / reduce;
+        tile[r * pitch + (i - r * reduce)] = src[i];
+    }
+    __syncthreads();
+    if ((int) threadIdx.x < nr) {
+        const float *t = tile + threadIdx.x * pitch;
+        float psum = 0.0f, psq = 0.0f;
+        for (int i = 0; i < reduce; ++i) {
+            psum = __fadd_rn(psum, t[i]);
+            psq = __fadd_rn(psq, __fmul_rn(t[i], t[i]));
+        }
+        ln_stats(psum, psq, inv_n, &s_mean[threadIdx.x], &s_inv[threadIdx.x]);
+    }
+    __syncthreads();
+    float *dst = y + (long long) row0 * reduce;
+    for (int i = threadIdx.x; i < total; i += 256) {
+        const int r = i / reduce, e = i - r * reduce;
+        const float t = __fmul_rn(__fsub_rn(tile[r * pitch + e], s_mean[r]), s_inv[r]);
+        dst[i] = __fadd_rn(__fmul_rn(t, w[e]), b[e]);
+    }
+}
+
+// one thread per row straight from memory: rows too long for LDS (stride 1), or the "axis 1" form of
+// layer_normalization.c:28-60 where the elements of a row lie `stride` apart and neighbouring threads read
+// neighbouring addresses
+__global__ __launch_bounds__(256) void layernorm_thread_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                               const float *__restrict__ b, float *__restrict__ y,
+                                                               int rows, int reduce, long long row_step, long long stride,
+                                                               float inv_n) {
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    const float *src = x + r * row_step;
+    float *dst = y + r * row_step;
+    float psum = 0.0f, psq = 0.0f;
+    for (int i = 0; i < reduce; ++i) {
+        const float v = src[i * stride];
+        psum = __fadd_rn(psum, v);
+        psq = __fadd_rn(psq, __fmul_rn(v, v));
+    }
+    float mean, inv_std;
+    ln_stats(psum, psq, inv_n, &mean, &inv_std);
+    for (int i = 0; i < reduce; ++i) {
+        const float t = __fmul_rn(__fsub_rn(src[i * stride], mean), inv_std);
+        dst[i * stride] = __fadd_rn(__fmul_rn(t, w[i]), b[i]);
+    }
+}
+
+// ---- Softmax ----------------------------------------------------------------------------------------
+// softmax.c:40-58: max from -32768, exp(x - max), sum, times 1 / sum.  Last axis: one wavefront per row.
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float *__restrict__ x, float *__restrict__ y, int rows,
+                                                           int reduce) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    const float *src = x + (long long) row * reduce;
+    float *dst = y + (long long) row * reduce;
+    float m = -32768.0f;
+    for (int i = lane; i < reduce; i += 64) m = src[i] > m ? src[i] : m;
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const float o = __shfl_xor(m, s, 64);
+        m = o > m ? o : m;
+    }
+    float sum = 0.0f;
+    for (int i = lane; i < reduce; i += 64) {
+        const float e = expf(__fsub_rn(src[i], m));
+        dst[i] = e;
+        sum += e;
+    }
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) sum += __shfl_xor(sum, s, 64);
+    const float inv = __fdiv_rn(1.0f, sum);
+    for (int i = lane; i < reduce; i += 64) dst[i] = __fmul_rn(dst[i], inv);   // each lane re-reads its own stores
+}
+
+// axis 1 of a batch-1 tensor (softmax.c:85-117): element i of column c at i * cols + c; one thread per column
+__global__ __launch_bounds__(256) void softmax_cols_kernel(const float *__restrict__ x, float *__restrict__ y, int cols,
+                                                           int reduce) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    float m = -32768.0f;
+    for (int i = 0; i < reduce; ++i) {
+        const float v = x[(long long) i * cols + c];
+        m = v > m ? v : m;
+    }
+    float sum = 0.0f;
+    for (int i = 0; i < reduce; ++i) {
+        const float e = expf(__fsub_rn(x[(long long) i * cols + c], m));
+        y[(long long) i * cols + c] = e;
+        sum = __fadd_rn(sum, e);
+    }
+    const float inv = __fdiv_rn(1.0f, sum);
+    for (int i = 0; i < reduce; ++i) y[(long long) i * cols + c] = __fmul_rn(y[(long long) i * cols + c], inv);
+}
+
+// ---- Transpose ----------------------------------------------------------------------------------------
+// out[o0..o5] = in[...] with out dim k taken from in dim perm[k] (transpose.c:52-76, :118-137): one thread per
+// output element, the input offset is the dot product of the output coordinates with the permuted strides
+struct TransposeParams {
+    long long n;
+    int ndim;
+    Div31 div[6];          // by the output extents, innermost first
+    int extent[6];
+    int in_stride[6];      // input stride of the dimension each output dimension comes from, innermost first
+};
+
+__global__ __launch_bounds__(256) void transpose_kernel(TransposeParams p, const float *__restrict__ x, float *__restrict__ y) {
+    const long long o = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (o >= p.n) return;
+    unsigned rest = (unsigned) o;
+    long long src = 0;
+#pragma unroll
+    for (int k = 0; k < 6; ++k) {
+        if (k < p.ndim) {
+            const unsigned q = vg_div(rest, p.div[k]);
+            src += (long long) (rest - q * (unsigned) p.extent[k]) * p.in_stride[k];
+            rest = q;
+        }
+    }
+    y[o] = x[src];
+}
+
+}  // namespace onhip
+
+using namespace onhip;
+
+extern "C" {
+
+int onhip_gelu_lut_f32(const float *x, const float *gelu_lut, float *y, long long n, void *stream) {
+    if (!x || !gelu_lut || !y || n < 1) return set_error(ONHIP_ERR_ARG, "gelu: bad argument");
+    if ((n + 255) / 256 > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "gelu: tensor too large");
+    hipLaunchKernelGGL(gelu_lut_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       x, gelu_lut, y, n);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_layernorm_f32(int32_t rows, int32_t reduce, int32_t strided, const float *x, const float *weight,
+                        const float *bias, float *y, void *stream) {
+    if (!x || !weight || !bias || !y || rows < 1 || reduce < 1) return set_error(ONHIP_ERR_ARG, "layernorm: bad argument");
+    if ((long long) rows * reduce >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "layernorm: tensor too large");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const float inv_n = 1.0f / reduce;
+    if (strided) {
+        hipLaunchKernelGGL(layernorm_thread_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, x, weight, bias, y, rows,
+                           reduce, 1LL, (long long) rows, inv_n);
+    } else if (reduce + 1 <= LN_LDS_FLOATS / 4) {
+        int rpw = LN_LDS_FLOATS / (reduce + 1);
+        if (rpw > 64) rpw = 64;
+        hipLaunchKernelGGL(layernorm_rows_kernel, dim3((rows + rpw - 1) / rpw), dim3(256), 0, st, x, weight, bias, y, rows,
+                           reduce, rpw, inv_n);
+    } else {
+        hipLaunchKernelGGL(layernorm_thread_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, x, weight, bias, y, rows,
+                           reduce, (long long) reduce, 1LL, inv_n);
+    }
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_softmax_f32(int32_t rows, int32_t reduce, int32_t strided, const float *x, float *y, void *stream) {
+    if (!x || !y || rows < 1 || reduce < 1) return set_error(ONHIP_ERR_ARG, "softmax: bad argument");
+    if ((long long) rows * reduce >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "softmax: tensor too large");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (strided) hipLaunchKernelGGL(softmax_cols_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, x, y, rows, reduce);
+    else hipLaunchKernelGGL(softmax_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, st, x, y, rows, reduce);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_transpose_f32(const onhip_transpose_desc_t *d, const float *x, float *y, void *stream) {
+    if (!d || !x || !y) return set_error(ONHIP_ERR_ARG, "transpose: null pointer");
+    if (d->ndim < 1 || d->ndim > 6) return set_error(ONHIP_ERR_ARG, "transpose: rank %d (1..6 supported)", d->ndim);
+    int in_stride[6], seen = 0;
+    long long n = 1;
+    for (int i = d->ndim - 1; i >= 0; --i) {
+        if (d->in_shape[i] < 1) return set_error(ONHIP_ERR_ARG, "transpose: empty dimension");
+        in_stride[i] = (int) n;
+        n *= d->in_shape[i];
+        if (n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "transpose: tensor too large");
+    }
+    TransposeParams p;
+    memset(&p, 0, sizeof(p));
+    p.n = n;
+    p.ndim = d->ndim;
+    for (int k = 0; k < d->ndim; ++k) {        // innermost output dimension first
+        const int od = d->ndim - 1 - k;
+        const int id = d->perm[od];
+        if (id < 0 || id >= d->ndim || (seen & (1 << id))) return set_error(ONHIP_ERR_ARG, "transpose: perm is not a permutation");
+        seen |= 1 << id;
+        p.extent[k] = d->in_shape[id];
+        p.div[k] = make_div31((unsigned) d->in_shape[id]);
+        p.in_stride[k] = in_stride[id];
+    }
+    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       p, x, y);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+}  // extern "C"

@@ -36,8 +36,10 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out
            "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
+           "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
-           "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_plugin_release"]
+           "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_gelu_eval", "onhip_layernorm_eval",
+           "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_release"]
 
 
 def load():
@@ -68,6 +70,10 @@ def load():
     L.onhip_relu_f32.argtypes = [vp, vp, C.c_longlong, vp]
     L.onhip_maxpool_f32.argtypes = [vp, C.c_int32, C.c_int32, vp, vp, vp]
     L.onhip_global_avgpool_f32.argtypes = [C.c_int32] * 4 + [vp, vp, vp]
+    L.onhip_gelu_lut_f32.argtypes = [vp, vp, vp, C.c_longlong, vp]
+    L.onhip_layernorm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
+    L.onhip_softmax_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp]
+    L.onhip_transpose_f32.argtypes = [vp, vp, vp, vp]
     L.onhip_quant_weight_bias.argtypes = [vp, vp, C.c_int32, C.c_int32, vp, vp, vp]
     L.onhip_calib_abs_max.argtypes = [vp, C.c_longlong, C.POINTER(C.c_float), vp]
     L.onhip_calib_histogram.argtypes = [vp, C.c_longlong, C.c_float, vp, vp]
@@ -174,6 +180,49 @@ def global_avgpool_f32(x, out=None):
     if out is None:
         out = torch.empty((n, c, 1, 1), dtype=torch.float32, device=x.device)
     _check(load().onhip_global_avgpool_f32(n, c, h, w, _ptr(x), _ptr(out), _stream()), "onhip_global_avgpool_f32")
+    return out
+
+
+def gelu_lut_f32(x, lut, out=None):
+    import torch
+    if out is None:
+        out = torch.empty_like(x)
+    _check(load().onhip_gelu_lut_f32(_ptr(x), _ptr(lut), _ptr(out), x.numel(), _stream()), "onhip_gelu_lut_f32")
+    return out
+
+
+def layernorm_f32(x, weight, bias, axis1=False, out=None):
+    """normalises the last dimension of x, or (axis1) dimension 1 of a batch-1 tensor"""
+    import torch
+    reduce = x.shape[1] if axis1 else next((d for d in reversed(x.shape) if d != 1), 1)
+    rows = x.numel() // reduce
+    if out is None:
+        out = torch.empty_like(x)
+    _check(load().onhip_layernorm_f32(rows, reduce, int(axis1), _ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _stream()),
+           "onhip_layernorm_f32")
+    return out
+
+
+def softmax_f32(x, axis1=False, out=None):
+    import torch
+    reduce = x.shape[1] if axis1 else x.shape[-1]
+    rows = x.numel() // reduce
+    if out is None:
+        out = torch.empty_like(x)
+    _check(load().onhip_softmax_f32(rows, reduce, int(axis1), _ptr(x), _ptr(out), _stream()), "onhip_softmax_f32")
+    return out
+
+
+def transpose_f32(x, perm, out=None):
+    import torch
+    from onenew_amd.abi import TransposeDesc
+    d = TransposeDesc()
+    d.ndim = x.dim()
+    for i in range(x.dim()):
+        d.in_shape[i], d.perm[i] = x.shape[i], perm[i]
+    if out is None:
+        out = torch.empty([x.shape[p] for p in perm], dtype=torch.float32, device=x.device)
+    _check(load().onhip_transpose_f32(C.byref(d), _ptr(x), _ptr(out), _stream()), "onhip_transpose_f32")
     return out
 
 

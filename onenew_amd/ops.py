@@ -344,3 +344,55 @@ class MaxPool(_Unary):
         n, c, h, w = shape
         return (n, c, (h + 2 * self.pad - self.kernel) // self.stride + 1,
                 (w + 2 * self.pad - self.kernel) // self.stride + 1)
+
+
+class Gelu(_Unary):
+    """host/ops/gelu.h: table GELU, the 8192-entry table travels in inputs[11] (device/x86/Gelu/gelu.c)"""
+    op_type = b"Gelu"
+
+    def __init__(self, evalfn, gelu_lut):
+        super().__init__(evalfn)
+        self.lut = np.ascontiguousarray(gelu_lut, dtype=np.float32)
+        self._slot(self.inputs_vec, BUF_MAXNUM - 1, self.lut)
+
+
+class LayerNormalization(_Unary):
+    """host/ops/layer_normalization.h: weight in inputs[1], bias in inputs[2]; axes[0] == 1 normalises dimension 1
+    (device/x86/LayerNormalization/layer_normalization.c)"""
+    op_type = b"LayerNormalization"
+
+    def __init__(self, evalfn, weight, bias, axis=-1):
+        cfg = abi.LAYERNORMALIZATION_CONFIG_S()
+        cfg.axes[0] = axis
+        cfg.axes_num = 1
+        super().__init__(evalfn, cfg)
+        self.weight = np.ascontiguousarray(weight, dtype=np.float32)
+        self.bias = np.ascontiguousarray(bias, dtype=np.float32)
+        self._slot(self.inputs_vec, 1, self.weight)
+        self._slot(self.inputs_vec, 2, self.bias)
+
+
+class Softmax(_Unary):
+    """host/ops/softmax.h (device/x86/Softmax/softmax.c): the last axis, or axis 1 of a batch-1 tensor"""
+    op_type = b"Softmax"
+
+    def __init__(self, evalfn, axis=-1):
+        cfg = abi.SOFTMAX_CONFIG_S()
+        cfg.axis = axis
+        super().__init__(evalfn, cfg)
+
+
+class Transpose(_Unary):
+    """host/ops/transpose.h (device/x86/Transpose/transpose.c): out dim k = in dim perm[k]"""
+    op_type = b"Transpose"
+
+    def __init__(self, evalfn, perm):
+        cfg = abi.TRANSPOSE_CONFIG_S()
+        for i, p in enumerate(perm):
+            cfg.perm[i] = p
+        cfg.perm_num = len(perm)
+        super().__init__(evalfn, cfg)
+        self.perm = tuple(perm)
+
+    def out_shape(self, shape):
+        return tuple(shape[p] for p in self.perm)

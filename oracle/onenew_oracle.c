@@ -730,3 +730,76 @@ void oracle_global_avgpool_f32(int n, int c, int h, int w, const float *x, float
         y[p] = psum * coeff;
     }
 }
+
+
+/* ---------------------------------------------------------------------------------------------
+ * The operators around the MatMuls of a transformer block: LayerNormalization, Softmax, Transpose
+ * (table GELU is oracle_lut_act_f32)
+ * ------------------------------------------------------------------------------------------- */
+
+/* device/x86/LayerNormalization/layer_normalization.c:28-97.  strided == 0: rows contiguous; strided != 0:
+ * element i of row r at i * rows + r (the "axes[0] == 1" form).  EPSILON is the double 1e-20 (nn_common.h:19). */
+void oracle_layernorm_f32(int rows, int reduce, int strided, const float *x, const float *w, const float *b, float *y) {
+    const float inv_n = 1.0f / reduce;
+    const int64_t step = strided ? rows : 1;
+    for (int r = 0; r < rows; ++r) {
+        const float *src = x + (strided ? (int64_t) r : (int64_t) r * reduce);
+        float *dst = y + (strided ? (int64_t) r : (int64_t) r * reduce);
+        float psum = 0, psq = 0;
+        for (int i = 0; i < reduce; ++i) {
+            psum += src[i * step];
+            psq += src[i * step] * src[i * step];
+        }
+        const float mean = psum * inv_n;
+        float var = inv_n * psq - mean * mean;
+        var += 1e-20;
+        const float inv_std = 1.0f / sqrtf(var);
+        for (int i = 0; i < reduce; ++i) {
+            const float t = (src[i * step] - mean) * inv_std;
+            dst[i * step] = t * w[i] + b[i];
+        }
+    }
+}
+
+/* device/x86/Softmax/softmax.c:26-59 (last axis) and :62-118 (axis 1 of a batch-1 tensor, strided) */
+void oracle_softmax_f32(int rows, int reduce, int strided, const float *x, float *y) {
+    const int64_t step = strided ? rows : 1;
+    for (int r = 0; r < rows; ++r) {
+        const float *src = x + (strided ? (int64_t) r : (int64_t) r * reduce);
+        float *dst = y + (strided ? (int64_t) r : (int64_t) r * reduce);
+        float mx = -32768.0f;
+        for (int i = 0; i < reduce; ++i) mx = src[i * step] > mx ? src[i * step] : mx;
+        float total = 0;
+        for (int i = 0; i < reduce; ++i) {
+            dst[i * step] = expf(src[i * step] - mx);
+            total += dst[i * step];
+        }
+        const float inv = 1.0f / total;
+        for (int i = 0; i < reduce; ++i) dst[i * step] = dst[i * step] * inv;
+    }
+}
+
+/* device/x86/Transpose/transpose.c:24-140: output dimension k comes from input dimension perm[k] */
+int oracle_transpose_f32(int ndim, const int32_t *in_shape, const int32_t *perm, const float *x, float *y) {
+    if (ndim < 1 || ndim > 6) return -1;
+    int64_t in_stride[6], n = 1;
+    for (int i = ndim - 1; i >= 0; --i) {
+        in_stride[i] = n;
+        n *= in_shape[i];
+    }
+    int32_t out_shape[6];
+    int64_t cstride[6];
+    for (int k = 0; k < ndim; ++k) {
+        out_shape[k] = in_shape[perm[k]];
+        cstride[k] = in_stride[perm[k]];
+    }
+    for (int64_t o = 0; o < n; ++o) {
+        int64_t rest = o, src = 0;
+        for (int k = ndim - 1; k >= 0; --k) {
+            src += (rest % out_shape[k]) * cstride[k];
+            rest /= out_shape[k];
+        }
+        y[o] = x[src];
+    }
+    return 0;
+}

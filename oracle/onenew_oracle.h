@@ -36,6 +36,10 @@ int oracle_maxpool_f32(int n, int c, int h, int w, int kh, int kw, int stride_w,
                        const float *x, float *y);
 void oracle_global_avgpool_f32(int n, int c, int h, int w, const float *x, float *y);
 
+void oracle_layernorm_f32(int rows, int reduce, int strided, const float *x, const float *w, const float *b, float *y);
+void oracle_softmax_f32(int rows, int reduce, int strided, const float *x, float *y);
+int oracle_transpose_f32(int ndim, const int32_t *in_shape, const int32_t *perm, const float *x, float *y);
+
 #define ORACLE_CALIB_BINS 2048
 float oracle_calib_abs_max(const float *x, int64_t n, float running_max);
 void oracle_calib_histogram(const float *x, int64_t n, float max_abs, float *hist);

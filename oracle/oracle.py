@@ -186,6 +186,33 @@ def global_avgpool_f32(x):
     return y
 
 
+def layernorm_f32(x, weight, bias, axis1=False):
+    x, weight, bias = _f32(x), _f32(weight), _f32(bias)
+    # the reference normalises the last dimension that is not 1 (layer_normalization.c:63-68)
+    reduce = x.shape[1] if axis1 else next((d for d in reversed(x.shape) if d != 1), 1)
+    y = np.empty_like(x)
+    lib().oracle_layernorm_f32(x.size // reduce, reduce, int(axis1), _p(x, f32p), _p(weight, f32p), _p(bias, f32p),
+                               _p(y, f32p))
+    return y
+
+
+def softmax_f32(x, axis1=False):
+    x = _f32(x)
+    reduce = x.shape[1] if axis1 else x.shape[-1]
+    y = np.empty_like(x)
+    lib().oracle_softmax_f32(x.size // reduce, reduce, int(axis1), _p(x, f32p), _p(y, f32p))
+    return y
+
+
+def transpose_f32(x, perm):
+    x = _f32(x)
+    i32 = C.c_int32 * x.ndim
+    y = np.empty([x.shape[p] for p in perm], np.float32)
+    rc = lib().oracle_transpose_f32(x.ndim, i32(*x.shape), i32(*perm), _p(x, f32p), _p(y, f32p))
+    assert rc == 0
+    return y
+
+
 def calib_abs_max(x, running=0.0):
     x = _f32(x)
     fn = lib().oracle_calib_abs_max

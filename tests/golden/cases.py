@@ -226,6 +226,42 @@ def gap_input(name, shape):
     return datagen.normal(datagen.seed_for(name, "x"), shape, 0.5, 1.0)
 
 
+def layernorm_cases():
+    """name -> (shape, axis); axis -1 normalises the last non-1 dimension, axis 1 is the strided form"""
+    return {"ln_vit": ((1, 197, 192), -1), "ln_small": ((3, 5, 7), -1), "ln_trailing_ones": ((2, 6, 10, 1), -1),
+            "ln_axis1": ((1, 24, 6, 5), 1), "ln_long_row": ((2, 3000), -1)}
+
+
+def layernorm_inputs(name, shape, axis):
+    reduce = shape[1] if axis == 1 else [d for d in shape if d != 1][-1]
+    x = datagen.normal(datagen.seed_for(name, "x"), shape, 0.3, 1.5)
+    w = datagen.normal(datagen.seed_for(name, "w"), (reduce,), 1.0, 0.1)
+    b = datagen.normal(datagen.seed_for(name, "b"), (reduce,), 0.0, 0.1)
+    return x, w, b
+
+
+def softmax_cases():
+    """name -> (shape, axis)"""
+    return {"sm_vit_scores": ((3, 197, 197), -1), "sm_small": ((4, 9), -1), "sm_rank4": ((2, 3, 5, 33), 3),
+            "sm_axis1": ((1, 10, 7, 6), 1), "sm_wide": ((2, 1000), -1)}
+
+
+def softmax_input(name, shape):
+    return datagen.normal(datagen.seed_for(name, "x"), shape, 0.0, 3.0)
+
+
+def transpose_cases():
+    """name -> (shape, perm)"""
+    return {"tr_vit_heads": ((1, 197, 3, 64), (0, 2, 1, 3)), "tr_vit_kt": ((1, 3, 197, 64), (0, 1, 3, 2)),
+            "tr_nchw_nhwc": ((2, 5, 6, 7), (0, 2, 3, 1)), "tr_rank3": ((4, 6, 5), (2, 0, 1)),
+            "tr_rank2": ((9, 13), (1, 0)), "tr_rank6": ((2, 3, 2, 4, 3, 5), (0, 3, 1, 5, 2, 4)),
+            "tr_rank5": ((2, 3, 4, 5, 6), (4, 0, 2, 1, 3))}
+
+
+def transpose_input(name, shape):
+    return datagen.normal(datagen.seed_for(name, "x"), shape, 0.0, 1.0)
+
+
 def gelu_input():
     """values across the table range, bin edges and both cut-offs"""
     x = datagen.uniform(datagen.seed_for("gelu", "x"), (5000,), -9.0, 9.0)

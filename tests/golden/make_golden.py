@@ -80,6 +80,20 @@ def main():
     for name, shape in cases.gap_cases().items():
         put(name, ops.GlobalAveragePool(gap.eval)(cases.gap_input(name, shape)))
         print("gap", name, flush=True)
+    # the operators around the MatMuls: LayerNormalization, Softmax, Transpose
+    ln = ops.Plugin(os.path.join(ref, "libLayerNormalization_x86.so"))
+    sm = ops.Plugin(os.path.join(ref, "libSoftmax_x86.so"))
+    tr = ops.Plugin(os.path.join(ref, "libTranspose_x86.so"))
+    for name, (shape, axis) in cases.layernorm_cases().items():
+        x, w, b = cases.layernorm_inputs(name, shape, axis)
+        put(name, ops.LayerNormalization(ln.eval, w, b, axis)(x))
+        print("layernorm", name, flush=True)
+    for name, (shape, axis) in cases.softmax_cases().items():
+        put(name, ops.Softmax(sm.eval, axis)(cases.softmax_input(name, shape)))
+        print("softmax", name, flush=True)
+    for name, (shape, perm) in cases.transpose_cases().items():
+        put(name, ops.Transpose(tr.eval, perm)(cases.transpose_input(name, shape)))
+        print("transpose", name, flush=True)
     # table GELU (device/x86/Gelu/gelu.c) on edge values
     x = cases.gelu_input()
     params = (abi.BUFFER_INFO_S * abi.BUF_MAXNUM)()

@@ -506,3 +506,60 @@ def test_global_avgpool_matches_oracle_and_plugin(name, torch_dev, oracle, golde
     xb = np.concatenate([x] * 3, axis=0)
     yb = hip.global_avgpool_f32(dev(torch, xb)).cpu().numpy()
     assert np.array_equal(yb, np.concatenate([ref] * 3, axis=0))
+
+
+def test_gelu_table_matches_oracle_and_plugin(torch_dev, oracle, golden):
+    torch = torch_dev
+    x = cases.gelu_input()
+    lut = cases.gelu_lut()
+    ref = oracle.lut_act(x, lut)
+    y = hip.gelu_lut_f32(dev(torch, x), dev(torch, lut))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), ref)
+    cases.check_against(golden, "gelu_edges", y.cpu().numpy(), exact=True)
+    xin = ops.aligned_empty(x.shape)
+    xin[...] = x
+    assert np.array_equal(ops.Gelu(ops.Plugin(hip.plugin_path("Gelu")).eval, lut)(xin), ref)
+
+
+@pytest.mark.parametrize("name", list(cases.layernorm_cases()))
+def test_layernorm_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
+    """sums in memory order, every operation rounded as in the reference: bit-identical"""
+    torch = torch_dev
+    shape, axis = cases.layernorm_cases()[name]
+    x, w, b = cases.layernorm_inputs(name, shape, axis)
+    ref = oracle.layernorm_f32(x, w, b, axis1=(axis == 1))
+    y = hip.layernorm_f32(dev(torch, x), dev(torch, w), dev(torch, b), axis1=(axis == 1))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), ref), f"{name}: {(y.cpu().numpy() != ref).sum()} elements differ"
+    cases.check_against(golden, name, y.cpu().numpy(), exact=True)
+    plug = ops.LayerNormalization(ops.Plugin(hip.plugin_path("LayerNormalization")).eval, w, b, axis)
+    assert np.array_equal(plug(x), ref)
+
+
+@pytest.mark.parametrize("name", list(cases.softmax_cases()))
+def test_softmax_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
+    """expf on the GPU and in glibc agree to a few ulp: fp32 tolerance 1e-4 of the row maximum, rows sum to 1"""
+    torch = torch_dev
+    shape, axis = cases.softmax_cases()[name]
+    x = cases.softmax_input(name, shape)
+    ref = oracle.softmax_f32(x, axis1=(axis == 1))
+    y = hip.softmax_f32(dev(torch, x), axis1=(axis == 1)).cpu().numpy()
+    assert np.abs(y - ref).max() <= 1e-4 * ref.max() and np.allclose(y, ref, rtol=1e-4, atol=1e-9)
+    ax = 1 if axis == 1 else x.ndim - 1
+    assert np.allclose(y.sum(axis=ax), 1.0, atol=1e-5)
+    cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-9)
+    yp = ops.Softmax(ops.Plugin(hip.plugin_path("Softmax")).eval, axis)(x)
+    assert np.array_equal(yp, y)
+
+
+@pytest.mark.parametrize("name", list(cases.transpose_cases()))
+def test_transpose_matches_numpy_and_plugin(name, torch_dev):
+    torch = torch_dev
+    shape, perm = cases.transpose_cases()[name]
+    x = cases.transpose_input(name, shape)
+    y = hip.transpose_f32(dev(torch, x), perm)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), np.transpose(x, perm))
+    if len(shape) in (4, 6):
+        assert np.array_equal(ops.Transpose(ops.Plugin(hip.plugin_path("Transpose")).eval, perm)(x), np.transpose(x, perm))

@@ -84,3 +84,40 @@ def test_global_avgpool_bit_exact(name, golden, oracle):
     y = oracle.global_avgpool_f32(x)
     cases.check_against(golden, name, y, exact=True)
     assert np.allclose(y.reshape(x.shape[:2]), x.astype(np.float64).mean(axis=(2, 3)), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", list(cases.layernorm_cases()))
+def test_layernorm_bit_exact(name, golden, oracle):
+    shape, axis = cases.layernorm_cases()[name]
+    x, w, b = cases.layernorm_inputs(name, shape, axis)
+    y = oracle.layernorm_f32(x, w, b, axis1=(axis == 1))
+    cases.check_against(golden, name, y, exact=True)
+    # closed form in float64 (eps 1e-20 is invisible)
+    ax = 1 if axis == 1 else max(i for i, d in enumerate(shape) if d != 1)
+    x64 = x.astype(np.float64)
+    norm = (x64 - x64.mean(axis=ax, keepdims=True)) / np.sqrt(x64.var(axis=ax, keepdims=True))
+    bshape = [1] * x.ndim
+    bshape[ax] = -1
+    assert np.allclose(y, norm * w.reshape(bshape) + b.reshape(bshape), rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("name", list(cases.softmax_cases()))
+def test_softmax_bit_exact(name, golden, oracle):
+    """same libm as the reference build in this container, so the CPU restatement matches to the bit"""
+    shape, axis = cases.softmax_cases()[name]
+    x = cases.softmax_input(name, shape)
+    y = oracle.softmax_f32(x, axis1=(axis == 1))
+    cases.check_against(golden, name, y, exact=True)
+    ax = 1 if axis == 1 else x.ndim - 1
+    e = np.exp(x.astype(np.float64) - x.max(axis=ax, keepdims=True))
+    assert np.allclose(y, e / e.sum(axis=ax, keepdims=True), rtol=1e-5, atol=1e-8)
+
+
+@pytest.mark.parametrize("name", list(cases.transpose_cases()))
+def test_transpose_bit_exact(name, golden, oracle):
+    shape, perm = cases.transpose_cases()[name]
+    x = cases.transpose_input(name, shape)
+    y = oracle.transpose_f32(x, perm)
+    assert np.array_equal(y, np.transpose(x, perm))
+    if len(shape) in (4, 6) or len(perm) <= 4:
+        cases.check_against(golden, name, y, exact=True)
