@@ -168,6 +168,69 @@ class GlueLayer:
         return self.flops // self.x.shape[0], lambda: oracle.global_avgpool_f32(x)
 
 
+class VitGlueLayer:
+    """the memory-bound operators around the MatMuls of one ViT-Tiny block"""
+    kind = "glue"
+    dense = False
+
+    def __init__(self, torch, hip, name, op, shape, tag, perm=None):
+        import cases
+        from onenew_amd import datagen
+        self.name, self.op, self.perm = name, op, perm
+        rnd = lambda role, shp, sd=1.0: torch.from_numpy(datagen.normal(datagen.seed_for(f"{tag}/{name}", role), shp, 0.0, sd)).cuda()
+        self.x = rnd("x", shape)
+        self.y = torch.empty([shape[p] for p in perm] if perm else shape, dtype=torch.float32, device="cuda")
+        n = self.x.numel()
+        self.bytes, self.flops = 8 * n, n
+        if op == "layernorm":
+            self.w, self.b = rnd("w", (shape[-1],)), rnd("b", (shape[-1],))
+            self.flops = 8 * n
+        elif op == "bias_add":
+            self.b = rnd("b", (shape[-1],))
+        elif op == "residual_add":
+            self.r = rnd("r", shape)
+            self.bytes = 12 * n
+        elif op == "gelu":
+            self.lut = torch.from_numpy(cases.gelu_lut()).cuda()
+        elif op == "softmax":
+            self.flops = 4 * n
+        self.shape = f"{op} {'x'.join(map(str, shape))}"
+
+    def launch(self, hip):
+        if self.op == "layernorm":
+            hip.layernorm_f32(self.x, self.w, self.b, out=self.y)
+        elif self.op == "bias_add":
+            hip.add_f32(self.x, self.b, out=self.y)
+        elif self.op == "residual_add":
+            hip.add_f32(self.x, self.r, out=self.y)
+        elif self.op == "gelu":
+            hip.gelu_lut_f32(self.x, self.lut, out=self.y)
+        elif self.op == "softmax":
+            hip.softmax_f32(self.x, out=self.y)
+        else:
+            hip.transpose_f32(self.x, self.perm, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        import cases
+        x = self.x[:1].cpu().numpy()
+        fl = self.flops // self.x.shape[0]
+        if self.op == "layernorm":
+            w, b = self.w.cpu().numpy(), self.b.cpu().numpy()
+            return fl, lambda: oracle.layernorm_f32(x, w, b)
+        if self.op == "bias_add":
+            b = self.b.cpu().numpy()
+            return fl, lambda: oracle.add_f32(x, b)
+        if self.op == "residual_add":
+            r = self.r[:1].cpu().numpy()
+            return fl, lambda: oracle.add_f32(x, r)
+        if self.op == "gelu":
+            lut = cases.gelu_lut()
+            return fl, lambda: oracle.lut_act(x, lut)
+        if self.op == "softmax":
+            return fl, lambda: oracle.softmax_f32(x)
+        return fl, lambda: oracle.transpose_f32(x, self.perm)
+
+
 class MatmulLayer:
     kind = "matmul"
 
@@ -228,6 +291,19 @@ def make_workload(torch, hip, name):
         return (f"ResNet-50 operators between the convolutions fp32, batch {n}: MaxPool 3x3 s2, 16 residual "
                 f"Add + ReLU (fused), GlobalAveragePool", "f32",
                 [GlueLayer(torch, hip, ln, op, shape, tag) for ln, op, shape in spec])
+    if name.startswith("vit_tiny_glue_b"):
+        n = int(name.split("_b")[1])
+        t, c, h, hd = 197, 192, 3, 64
+        spec = [("ln1", "layernorm", (n, t, c), None), ("qkv.bias", "bias_add", (n, t, 3 * c), None),
+                ("q.heads", "transpose", (n, t, h, hd), (0, 2, 1, 3)), ("k.t", "transpose", (n, h, t, hd), (0, 1, 3, 2)),
+                ("softmax", "softmax", (n, h, t, t), None), ("ctx.merge", "transpose", (n, h, t, hd), (0, 2, 1, 3)),
+                ("proj.bias", "bias_add", (n, t, c), None), ("res1", "residual_add", (n, t, c), None),
+                ("ln2", "layernorm", (n, t, c), None), ("fc1.bias", "bias_add", (n, t, 4 * c), None),
+                ("gelu", "gelu", (n, t, 4 * c), None), ("fc2.bias", "bias_add", (n, t, c), None),
+                ("res2", "residual_add", (n, t, c), None)]
+        return (f"ViT-Tiny block, operators around the MatMuls fp32, batch {n}: LayerNorm x2, bias adds, head "
+                f"transposes, Softmax, table GELU, residual adds", "f32",
+                [VitGlueLayer(torch, hip, ln, op, shape, tag, perm) for ln, op, shape, perm in spec])
     if name.startswith("mobilenetv2_b"):
         n = int(name.split("_b")[1])
         return (f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers (17 depthwise), ReLU6 as CLIP", "f32",
@@ -396,7 +472,8 @@ def main():
     g_ms = sum(t for _, t in grp)
     g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
     kernel = (f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
-              "onhip::add_kernel / maxpool_kernel / gap_kernel" if grp[0][0].kind == "glue" else "onhip::depthwise_tiled_kernel")
+              "element-wise / pooling / normalisation kernels (elementwise.hip, vit_glue.hip)" if grp[0][0].kind == "glue"
+              else "onhip::depthwise_tiled_kernel")
     # the bound is the roof the group's arithmetic intensity puts it under
     mfma_bound = dom_dense and g_flops / g_bytes >= PEAK[dtype] * 1e12 / (HBM_PEAK_GBS * 1e9)
     if mfma_bound:
@@ -436,7 +513,7 @@ def main():
 
     cpu = None if args.no_cpu else cpu_baseline(layers, args.workload, unit)
 
-    metric = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
+    metric = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vit_tiny_glue_ops_fp32_tflops", "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
               "yolov8s": "yolov8s_conv_stack_w8a32_tops", "vit": f"vit_tiny_matmul_{dtype}_tflops",
               "cfg1": "conv2d_relu_fp32_tflops"}
     key = next(k for k in metric if args.workload.startswith(k))

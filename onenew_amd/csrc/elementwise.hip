@@ -14,7 +14,9 @@ __device__ __forceinline__ unsigned ew_div(unsigned x, const Div31 &d) {
 
 // ---- Add -------------------------------------------------------------------------------------------
 // out[i] = large[i] + small[j(i)] (add.c: the operand with fewer elements is broadcast onto the other).
-// MODE 0: same number of elements, 1: small is one value, 2: per-dimension broadcast (strides 0).
+// MODE 0: same number of elements, 1: small is one value, 2: per-dimension broadcast (strides 0),
+// 3: small covers the trailing dimensions of large (a bias vector): its index is i mod its size; both sizes are
+// multiples of 4 and everything is 16-byte aligned, four elements per thread.
 struct AddParams {
     long long n;              // output elements
     int ndim;
@@ -22,6 +24,8 @@ struct AddParams {
     int extent[6];
     int small_stride[6];      // innermost first; 0 where the small operand is broadcast
     int relu;
+    Div31 div_small;          // MODE 3: by the number of float4 groups of the small operand
+    int small4;
 };
 
 template <int MODE>
@@ -42,6 +46,15 @@ __global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__re
                 out[i] = (p.relu && !(r > 0)) ? 0.0f : r;
             }
         }
+    } else if constexpr (MODE == 3) {
+        const long long i4 = (long long) blockIdx.x * 256 + threadIdx.x;
+        if (i4 * 4 >= p.n) return;
+        const unsigned q = ew_div((unsigned) i4, p.div_small);
+        const unsigned j4 = (unsigned) i4 - q * (unsigned) p.small4;
+        const float4 a = reinterpret_cast<const float4 *>(large)[i4], b = reinterpret_cast<const float4 *>(small)[j4];
+        float4 r = make_float4(__fadd_rn(a.x, b.x), __fadd_rn(a.y, b.y), __fadd_rn(a.z, b.z), __fadd_rn(a.w, b.w));
+        if (p.relu) { r.x = r.x > 0 ? r.x : 0; r.y = r.y > 0 ? r.y : 0; r.z = r.z > 0 ? r.z : 0; r.w = r.w > 0 ? r.w : 0; }
+        reinterpret_cast<float4 *>(out)[i4] = r;
     } else {
         const long long i = (long long) blockIdx.x * 256 + threadIdx.x;
         if (i >= p.n) return;
@@ -180,6 +193,13 @@ int onhip_add_f32(const onhip_add_desc_t *d, const float *large, const float *sm
         stride *= d->small_shape[dim];
     }
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // a bias-like operand: leading extents 1, then exactly the trailing extents of the large operand
+    bool trailing = ns > 1 && ns < n;
+    {
+        int k = 0;
+        while (k < d->ndim && d->small_shape[k] == 1) ++k;
+        for (; k < d->ndim; ++k) trailing = trailing && d->small_shape[k] == d->large_shape[k];
+    }
     if (ns == n) {
         if (aligned16(large) && aligned16(small) && aligned16(out)) {
             hipLaunchKernelGGL(add_kernel<0>, dim3((unsigned) ((n / 4 + 1 + 255) / 256)), dim3(256), 0, st, p, large, small, out);
@@ -187,6 +207,10 @@ int onhip_add_f32(const onhip_add_desc_t *d, const float *large, const float *sm
             // unaligned operands: the broadcast kernel with unit strides is the same sum
             hipLaunchKernelGGL(add_kernel<2>, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, st, p, large, small, out);
         }
+    } else if (trailing && ns % 4 == 0 && n % 4 == 0 && aligned16(large) && aligned16(small) && aligned16(out)) {
+        p.small4 = (int) (ns / 4);
+        p.div_small = make_div31((unsigned) p.small4);
+        hipLaunchKernelGGL(add_kernel<3>, dim3((unsigned) ((n / 4 + 255) / 256)), dim3(256), 0, st, p, large, small, out);
     } else if (ns == 1) {
         hipLaunchKernelGGL(add_kernel<1>, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, st, p, large, small, out);
     } else {

@@ -14,20 +14,30 @@ __device__ __forceinline__ unsigned vg_div(unsigned x, const Div31 &d) {
 }
 
 // ---- table GELU (gelu.c:22-38) ------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_lut_one(float v, const float *__restrict__ lut) {
+    if (v < -8.0f) return 0.0f;
+    if (v >= 8.0f) return v;
+    int idx = (int) __fmul_rn(__fadd_rn(v, 8.0f), 512.0f);
+    idx = idx > 8191 ? 8191 : idx;         // v just below 8: v + 8 rounds to 16 and the reference reads one past the table
+    return lut[idx];                       // a NaN fails both comparisons and indexes the table with (int) NaN
+}
+
+// four elements per thread where the tensors allow 128-bit accesses (VEC), else one
+template <bool VEC>
 __global__ __launch_bounds__(256) void gelu_lut_kernel(const float *__restrict__ x, const float *__restrict__ lut,
                                                        float *__restrict__ y, long long n) {
     const long long i = (long long) blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    const float v = x[i];
-    float r;
-    if (v < -8.0f) r = 0.0f;
-    else if (v >= 8.0f) r = v;
-    else {
-        int idx = (int) __fmul_rn(__fadd_rn(v, 8.0f), 512.0f);
-        idx = idx > 8191 ? 8191 : idx;     // v just below 8: v + 8 rounds to 16 and the reference reads one past the table
-        r = lut[idx];
+    if constexpr (VEC) {
+        if (i * 4 + 3 < n) {
+            float4 v = reinterpret_cast<const float4 *>(x)[i];
+            v.x = gelu_lut_one(v.x, lut); v.y = gelu_lut_one(v.y, lut); v.z = gelu_lut_one(v.z, lut); v.w = gelu_lut_one(v.w, lut);
+            reinterpret_cast<float4 *>(y)[i] = v;
+        } else {
+            for (long long k = i * 4; k < n; ++k) y[k] = gelu_lut_one(x[k], lut);
+        }
+    } else {
+        if (i < n) y[i] = gelu_lut_one(x[i], lut);
     }
-    y[i] = r;                              // a NaN fails both comparisons and indexes the table with (int) NaN
 }
 
 // ---- LayerNormalization ---------------------------------------------------------------------------------
@@ -194,8 +204,11 @@ extern "C" {
 int onhip_gelu_lut_f32(const float *x, const float *gelu_lut, float *y, long long n, void *stream) {
     if (!x || !gelu_lut || !y || n < 1) return set_error(ONHIP_ERR_ARG, "gelu: bad argument");
     if ((n + 255) / 256 > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "gelu: tensor too large");
-    hipLaunchKernelGGL(gelu_lut_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                       x, gelu_lut, y, n);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0)
+        hipLaunchKernelGGL(gelu_lut_kernel<true>, dim3((unsigned) ((n / 4 + 1 + 255) / 256)), dim3(256), 0, st, x, gelu_lut, y, n);
+    else
+        hipLaunchKernelGGL(gelu_lut_kernel<false>, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, st, x, gelu_lut, y, n);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }
