@@ -111,6 +111,39 @@ class ConvW8A32Layer:
         return d1.flops(), lambda: oracle.conv2d_w8a32(d1, x, w8, b32, aux, cases.silu_lut())
 
 
+class ConvW8A8Layer(ConvW8A32Layer):
+    """the int8 chain form: int8 NHWC activations in and out, quantisation fused into the producer's epilogue"""
+    kind = "conv_w8a8"
+
+    def __init__(self, torch, hip, name, d, tag):
+        super().__init__(torch, hip, name, d, tag)
+        self.d.out_s8, self.d.output_scale = 1, 0.03
+        self.xq = hip.quantize_nhwc_s8(self.x, d.input_scale)
+        oh, ow = d.out_hw()
+        self.yq = torch.empty((d.n, oh, ow, (d.cout + 15) // 16 * 16), dtype=torch.int8, device="cuda")
+        self.bytes = d.algorithmic_bytes(eb_x=1, eb_w=1, eb_y=1)
+        del self.x, self.y
+
+    def launch(self, hip):
+        hip.conv2d_w8a8_nhwc(self.d, self.xq, self.wp, self.b32, self.aux, self.lut, out=self.yq)
+
+    def cpu_runner(self, ops, oracle, tag):
+        import cases
+        from onenew_amd import abi
+        d1 = abi.ConvDesc.from_buffer_copy(self.d)
+        d1.n, d1.out_s8 = 1, 0
+        x, w8, b32, aux = cases.conv_inputs(f"{tag}/cpu/{self.name}", d1, quant=True)
+        if oracle.have_ref():
+            # the reference has no int8-to-int8 form: its W8A32 convolution (fp32 in and out) is the baseline
+            op = ops.Conv(ops.Plugin(oracle.ref_path("Conv")).eval, d1, w8, b32, weight_aux=aux, silu_lut=cases.silu_lut(),
+                          scratch_bytes=oracle.ref_scratch_bytes(d1))
+            xin = ops.aligned_empty(x.shape)
+            xin[...] = x
+            out = ops.aligned_empty((1, d1.cout) + d1.out_hw())
+            return d1.flops(), lambda: op(xin, out=out)
+        return d1.flops(), lambda: oracle.conv2d_w8a32(d1, x, w8, b32, aux, cases.silu_lut())
+
+
 class GlueLayer:
     """the memory-bound operators between the convolutions of ResNet-50: MaxPool after the stem, the residual
     Add + ReLU of every block (one fused pass), GlobalAveragePool at the end"""
@@ -291,6 +324,14 @@ def make_workload(torch, hip, name):
         return (f"ResNet-50 operators between the convolutions fp32, batch {n}: MaxPool 3x3 s2, 16 residual "
                 f"Add + ReLU (fused), GlobalAveragePool", "f32",
                 [GlueLayer(torch, hip, ln, op, shape, tag) for ln, op, shape in spec])
+    if name.startswith("yolov8s_int8chain_b"):
+        n = int(name.split("_b")[1])
+        layers = []
+        for i, (ln, d) in enumerate(stacks.with_batch(stacks.yolov8s(), n)):
+            d.input_scale = float(datagen.uniform(datagen.seed_for(tag, i, "s_in"), (1,), 0.005, 0.05)[0])
+            layers.append(ConvW8A8Layer(torch, hip, ln, d, tag))
+        return (f"YOLOv8s conv stack int8 chain form (int8 NHWC activations in and out, int32 accumulate, SiLU table, "
+                f"requantise), batch {n}, 640x640, {len(layers)} conv layers", "i8", layers)
     if name.startswith("vit_tiny_glue_b"):
         n = int(name.split("_b")[1])
         t, c, h, hd = 197, 192, 3, 64
@@ -514,7 +555,7 @@ def main():
     cpu = None if args.no_cpu else cpu_baseline(layers, args.workload, unit)
 
     metric = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vit_tiny_glue_ops_fp32_tflops", "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
-              "yolov8s": "yolov8s_conv_stack_w8a32_tops", "vit": f"vit_tiny_matmul_{dtype}_tflops",
+              "yolov8s_int8chain": "yolov8s_conv_stack_w8a8_tops", "yolov8s": "yolov8s_conv_stack_w8a32_tops", "vit": f"vit_tiny_matmul_{dtype}_tflops",
               "cfg1": "conv2d_relu_fp32_tflops"}
     key = next(k for k in metric if args.workload.startswith(k))
     line = {"metric": metric[key], "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": unit, "n_gpus": 1,

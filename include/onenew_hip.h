@@ -140,6 +140,21 @@ int onhip_conv2d_w8a32_packed(const onhip_conv_desc_t *d, const float *x, const 
                               const float *silu_lut, void *y, int32_t *acc32, void *workspace,
                               size_t workspace_bytes, void *stream);
 
+/* The int8 chain form of the W8A32 convolution: activations stay int8 between layers.  Layout of
+ * both xq and yq: NHWC, channels padded with anything to a multiple of 16 ([n][h][w][cp], 16-byte
+ * aligned).  yq = quantise(y, d->output_scale) where y is exactly what onhip_conv2d_w8a32 computes
+ * from the activations de-quantised with d->input_scale — the quantiser every reference Conv applies
+ * to its input (conv.c:961-973), moved into the producer's epilogue, so a chain of these calls gives
+ * the consumer the same int8 values as a chain of reference convolutions.  No counterpart as a
+ * separate function in the reference.  Dense convolutions only; weights from
+ * onhip_conv2d_w8a32_pack_weights.  onhip_quantize_nhwc_s8 makes the first xq of a chain from
+ * NCHW fp32 (q 16-byte aligned, n*h*w*round_up(c,16) bytes). */
+int onhip_quantize_nhwc_s8(const float *x, int32_t n, int32_t c, int32_t h, int32_t w, float scale,
+                           int8_t *q, void *stream);
+int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const int8_t *w8_packed,
+                           const int32_t *bias32, const float *weight_aux, const float *silu_lut,
+                           int8_t *yq, void *stream);
+
 /* Batched MatMul with optional fused bias and table GELU.  Replaces mat_mul.c eval (:10) and,
  * with bias/gelu_lut, the chain MatMul -> Add -> Gelu (device/x86/Gelu/gelu.c:9). */
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

@@ -477,14 +477,18 @@ int onhip_conv2d_w8a32_pack_weights(const onhip_conv_desc_t *d, const int8_t *w8
 
 // packed != 0: w8 holds the layout written by onhip_conv2d_w8a32_pack_weights and the workspace only
 // takes the int8 copy of the activations
-static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, int packed_w,
+// xq != nullptr: the activations arrive already quantised (int8 NHWC, channels padded to 16) and x is not read;
+// nhwc_out != 0: the int8 result is written NHWC with its channels padded to 16, ready to be the next xq
+static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8, int packed_w,
                              const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y,
-                             int32_t *acc32, void *workspace, size_t workspace_bytes, void *stream) {
+                             int32_t *acc32, void *workspace, size_t workspace_bytes, int nhwc_out, void *stream) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
-    if (!x || !w8 || !y || !weight_aux || (d->has_bias && !bias32))
+    if ((!x && !xq) || !w8 || !y || !weight_aux || (d->has_bias && !bias32))
         return set_error(ONHIP_ERR_ARG, "conv w8a32: null tensor pointer");
+    if (nhwc_out && !d->out_s8) return set_error(ONHIP_ERR_ARG, "conv w8a8: the NHWC output form is int8 (out_s8 = 1)");
+    if ((xq || nhwc_out) && d->group != 1) return set_error(ONHIP_ERR_ARG, "conv w8a8: depthwise is not available in the NHWC int8 form");
     // the reference pads all four sides by pads[0] (conv.c:979-999) while shapes come from the four
     // pads: only uniform padding is self-consistent
     if (d->pad_t != d->pad_l || d->pad_t != d->pad_b || d->pad_t != d->pad_r)
@@ -503,11 +507,14 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     size_t packed_bytes, q_bytes;
     w8a32_layout(d, &cp, &k_units, &packed_bytes, &q_bytes);
     if (packed_w) packed_bytes = 0;
-    if (!workspace || workspace_bytes < packed_bytes + q_bytes)
+    if (xq) q_bytes = 0;
+    if (packed_bytes + q_bytes > 0 && (!workspace || workspace_bytes < packed_bytes + q_bytes))
         return set_error(ONHIP_ERR_WORKSPACE, "conv w8a32: workspace of %zu bytes needed, %zu given",
                          packed_bytes + q_bytes, workspace ? workspace_bytes : (size_t) 0);
-    if (reinterpret_cast<uintptr_t>(workspace) % 16)
+    if (packed_bytes + q_bytes > 0 && reinterpret_cast<uintptr_t>(workspace) % 16)
         return set_error(ONHIP_ERR_WORKSPACE, "conv w8a32: workspace must be 16-byte aligned");
+    if (xq && reinterpret_cast<uintptr_t>(xq) % 16)
+        return set_error(ONHIP_ERR_ARG, "conv w8a8: int8 activations must be 16-byte aligned");
     if ((long long) d->n * d->h * d->w * cp >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "conv w8a32: staged activations of 2 GiB or more are not supported");
     const int8_t *packed = w8;
@@ -520,8 +527,12 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     } else if (reinterpret_cast<uintptr_t>(w8) % 16) {
         return set_error(ONHIP_ERR_ARG, "conv w8a32: packed weights must be 16-byte aligned");
     }
-    rc = quantize_nhwc_launch(x, d->n, d->cin, d->h, d->w, cp, 1.0f / d->input_scale, q, st);
-    if (rc) return rc;
+    if (xq) {
+        q = const_cast<int8_t *>(xq);
+    } else {
+        rc = quantize_nhwc_launch(x, d->n, d->cin, d->h, d->w, cp, 1.0f / d->input_scale, q, st);
+        if (rc) return rc;
+    }
 
     IgemmLaunch cfg;
     memset(&cfg, 0, sizeof(cfg));
@@ -550,9 +561,16 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     p.b_slice_bytes = (long long) d->n * d->h * d->w * cp;
     p.c_slice_bytes = (long long) d->n * d->cout * OH * OW * 4;
     p.C = y;
-    p.out_mode = OUT_CONV;
-    p.c_img_stride = (long long) d->cout * OH * OW;
-    p.c_stride_m = (long long) OH * OW;
+    if (nhwc_out) {
+        // element (pixel n, channel m) at n * Cp_out + m
+        p.out_mode = OUT_PLAIN;
+        p.c_stride_m = 1;
+        p.c_stride_n = (d->cout + 15) / 16 * 16;
+    } else {
+        p.out_mode = OUT_CONV;
+        p.c_img_stride = (long long) d->cout * OH * OW;
+        p.c_stride_m = (long long) OH * OW;
+    }
     p.ep = ep;
     p.in_scale = d->input_scale;
     p.weight_aux = weight_aux;
@@ -568,14 +586,30 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
 int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, const int32_t *bias32,
                        const float *weight_aux, const float *silu_lut, void *y, int32_t *acc32, void *workspace,
                        size_t workspace_bytes, void *stream) {
-    return conv2d_w8a32_impl(d, x, w8, 0, bias32, weight_aux, silu_lut, y, acc32, workspace, workspace_bytes, stream);
+    return conv2d_w8a32_impl(d, x, nullptr, w8, 0, bias32, weight_aux, silu_lut, y, acc32, workspace, workspace_bytes, 0, stream);
 }
 
 int onhip_conv2d_w8a32_packed(const onhip_conv_desc_t *d, const float *x, const int8_t *w8_packed,
                               const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y,
                               int32_t *acc32, void *workspace, size_t workspace_bytes, void *stream) {
-    return conv2d_w8a32_impl(d, x, w8_packed, 1, bias32, weight_aux, silu_lut, y, acc32, workspace, workspace_bytes,
-                             stream);
+    return conv2d_w8a32_impl(d, x, nullptr, w8_packed, 1, bias32, weight_aux, silu_lut, y, acc32, workspace, workspace_bytes,
+                             0, stream);
+}
+
+int onhip_quantize_nhwc_s8(const float *x, int32_t n, int32_t c, int32_t h, int32_t w, float scale, int8_t *q, void *stream) {
+    if (!x || !q || n < 1 || c < 1 || h < 1 || w < 1 || !(scale > 0.0f)) return set_error(ONHIP_ERR_ARG, "quantize: bad argument");
+    const int cp = (c + 15) / 16 * 16;
+    if ((long long) n * h * w * cp >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "quantize: tensor too large");
+    if (reinterpret_cast<uintptr_t>(q) % 16) return set_error(ONHIP_ERR_ARG, "quantize: output must be 16-byte aligned");
+    return quantize_nhwc_launch(x, n, c, h, w, cp, 1.0f / scale, q, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const int8_t *w8_packed, const int32_t *bias32,
+                           const float *weight_aux, const float *silu_lut, int8_t *yq, void *stream) {
+    if (!d) return set_error(ONHIP_ERR_ARG, "conv w8a8: null descriptor");
+    onhip_conv_desc_t dd = *d;
+    dd.out_s8 = 1;
+    return conv2d_w8a32_impl(&dd, nullptr, xq, w8_packed, 1, bias32, weight_aux, silu_lut, yq, nullptr, nullptr, 0, 1, stream);
 }
 
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

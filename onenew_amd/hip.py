@@ -32,7 +32,8 @@ def plugin_path(op):
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
-           "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quant_weight_bias",
+           "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quantize_nhwc_s8",
+           "onhip_conv2d_w8a8_nhwc", "onhip_quant_weight_bias",
            "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
@@ -79,6 +80,8 @@ def load():
     L.onhip_calib_histogram.argtypes = [vp, C.c_longlong, C.c_float, vp, vp]
     L.onhip_calib_threshold.argtypes = [C.c_int, vp, C.c_longlong, C.c_float, C.POINTER(C.c_float)]
     L.onhip_calib_percentile.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), vp]
+    L.onhip_quantize_nhwc_s8.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float, vp, vp]
+    L.onhip_conv2d_w8a8_nhwc.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
     L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
@@ -290,6 +293,27 @@ def pack_conv_weights_w8(d, w8):
     _check(load().onhip_conv2d_w8a32_pack_weights(C.byref(d), _ptr(w8), _ptr(packed), _stream()),
            "onhip_conv2d_w8a32_pack_weights")
     return packed
+
+
+def quantize_nhwc_s8(x, scale, out=None):
+    """NCHW fp32 -> NHWC int8 with channels padded to 16: the input form of conv2d_w8a8_nhwc"""
+    import torch
+    n, c, h, w = x.shape
+    if out is None:
+        out = torch.empty((n, h, w, (c + 15) // 16 * 16), dtype=torch.int8, device=x.device)
+    _check(load().onhip_quantize_nhwc_s8(_ptr(x), n, c, h, w, scale, _ptr(out), _stream()), "onhip_quantize_nhwc_s8")
+    return out
+
+
+def conv2d_w8a8_nhwc(d, xq, w8_packed, bias32, weight_aux, silu_lut=None, out=None):
+    """int8 NHWC in, int8 NHWC out (d.input_scale, d.output_scale); out[..., :cout] holds the result"""
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        out = torch.empty((d.n, oh, ow, (d.cout + 15) // 16 * 16), dtype=torch.int8, device=xq.device)
+    _check(load().onhip_conv2d_w8a8_nhwc(C.byref(d), _ptr(xq), _ptr(w8_packed), _ptr(bias32), _ptr(weight_aux),
+                                         _ptr(silu_lut), _ptr(out), _stream()), "onhip_conv2d_w8a8_nhwc")
+    return out
 
 
 def conv2d_w8a32(d, x, w8, bias32, weight_aux, silu_lut=None, out=None, acc32=None, workspace=None, packed=False):

@@ -563,3 +563,23 @@ def test_transpose_matches_numpy_and_plugin(name, torch_dev):
     assert np.array_equal(y.cpu().numpy(), np.transpose(x, perm))
     if len(shape) in (4, 6):
         assert np.array_equal(ops.Transpose(ops.Plugin(hip.plugin_path("Transpose")).eval, perm)(x), np.transpose(x, perm))
+
+
+@pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_s2", "yolo_c2f_3x3_64_80", "yolo_sppf_1x1_1024", "q3x3_bigacc"])
+def test_conv_w8a8_nhwc_chain_form(name, torch_dev, oracle):
+    """int8 NHWC in / int8 NHWC out: the same int8 values as quantising the reference's fp32 result, and the
+    quantised input equals the reference's own input quantiser"""
+    torch = torch_dev
+    d = ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()[name])
+    d.n = 3
+    d.out_s8, d.output_scale = 1, 0.041
+    x, w8, b32, aux = cases.conv_inputs(name + "_chain", d, quant=True)
+    ref = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut())          # int8 NCHW
+    xq = hip.quantize_nhwc_s8(dev(torch, x), d.input_scale)
+    q_ref = oracle.quantize_s8(x, d.input_scale)                              # NCHW
+    assert np.array_equal(xq.cpu().numpy()[..., :d.cin], np.transpose(q_ref, (0, 2, 3, 1)))
+    assert not xq.cpu().numpy()[..., d.cin:].any()                            # channel padding is zero
+    wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
+    yq = hip.conv2d_w8a8_nhwc(d, xq, wp, dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()))
+    torch.cuda.synchronize()
+    assert np.array_equal(yq.cpu().numpy()[..., :d.cout], np.transpose(ref, (0, 2, 3, 1)))
