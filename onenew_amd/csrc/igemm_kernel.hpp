@@ -367,8 +367,9 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
 #pragma unroll
                 for (int b = 0; b < TN; ++b) {
                     const int av = acc[a][b][r];
-                    __builtin_amdgcn_raw_buffer_store_b32((unsigned) av, racc, row_ok ? col_voff4[b] : OOB,
-                                                          (unsigned) m_uni * row_bytes4, 0);
+                    if (p.acc_out)
+                        __builtin_amdgcn_raw_buffer_store_b32((unsigned) av, racc, row_ok ? col_voff4[b] : OOB,
+                                                              (unsigned) m_uni * row_bytes4, 0);
                     float f = __fmul_rn((float) av, p.in_scale);
                     const float fbias = __fadd_rn(f, fb);
                     f = p.bias32 ? fbias : f;
@@ -405,6 +406,66 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                                                           (unsigned) m_uni * row_bytes, 0);
                 }
             }
+    }
+}
+
+// int8 NHWC output (element (pixel n, channel m) at n * pitch + m, pitch a multiple of 16): the requantised
+// bytes of the workgroup's tile are transposed through LDS so that a thread stores 16 consecutive channels of
+// one pixel with a single 128-bit access instead of 16 single bytes to 16 different pixels.  A lane holds four
+// consecutive channels of a pixel (accumulator registers 4q .. 4q+3), which go to LDS as one dword.  Channels
+// between M and the pitch are written as zero.  stage: BN * (BM + 16) bytes of LDS nobody reads any more.
+template <int EPI, int BM, int BN, int TM, int TN, class ACC>
+__device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&acc)[TM][TN], unsigned char *stage, int m0,
+                                                   int n0, int m_wave, int n_wave, int li, int lh, int tid) {
+    constexpr int PITCH = BM + 16;
+    const rsrc_t raux = make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u);
+    const rsrc_t rb32 = make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u);
+    const unsigned lh16 = (unsigned) lh * 16u;
+    float aux[TM][16];
+    int b32[TM][16];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const unsigned soff = (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u;
+            aux[a][r] = buf_load_f32(raux, lh16, soff);
+            b32[a][r] = (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
+        }
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int ml = m_wave - m0 + a * 32 + 8 * q + 4 * lh;   // first of the lane's four channels, tile-local
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                unsigned packed = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int r = 4 * q + j;
+                    const float coeff = __fdiv_rn(aux[a][r], 127.0f);
+                    float f = __fmul_rn((float) acc[a][b][r], p.in_scale);
+                    const float fbias = __fadd_rn(f, (float) b32[a][r]);
+                    f = p.bias32 ? fbias : f;
+                    const float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
+                    const int v = (m0 + ml + j < p.M) ? requant_s8(y, p.out_inv_scale) : 0;
+                    packed |= ((unsigned) v & 0xffu) << (8 * j);
+                }
+                const int nl = n_wave - n0 + b * 32 + li;
+                *reinterpret_cast<unsigned *>(stage + nl * PITCH + ml) = packed;
+            }
+        }
+    __syncthreads();
+    constexpr int GROUPS = BM / 16;
+    const rsrc_t rc = make_rsrc(p.C, RSRC_RANGE);
+    const int pitch = (int) p.c_stride_n;
+#pragma unroll
+    for (int f0 = 0; f0 < BN * GROUPS; f0 += THREADS) {
+        const int f = f0 + tid;
+        const int nl = f / GROUPS, g = f % GROUPS;
+        const uint4 v = *reinterpret_cast<const uint4 *>(stage + nl * PITCH + g * 16);
+        const int n = n0 + nl, m = m0 + g * 16;
+        const bool ok = ((BN * GROUPS) % THREADS == 0 || f < BN * GROUPS) && n < p.N && m < pitch;
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{v.x, v.y, v.z, v.w}, rc, ok ? (unsigned) (n * pitch + m) : OOB, 0, 0);
     }
 }
 
@@ -686,11 +747,31 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         write_partial<TM, TN>(p, acc, blockIdx.y * gridDim.z + batch, m_wave, n_wave, li, lh);
         return;
     }
+    if constexpr (DT == DT_I8) {
+        // int8 NHWC output without the raw-accumulator copy: 128-bit stores through LDS (batch is 1 on this path)
+        if (p.out_s8 && p.out_mode == OUT_PLAIN && p.c_stride_m == 1 && !p.acc_out) {
+            static_assert(sizeof(lds) >= (size_t) BN * (BM + 16), "output staging fits the operand buffers");
+            unsigned char *stage = reinterpret_cast<unsigned char *>(&lds[0][0]);
+            __syncthreads();   // every wavefront is done with the operand buffers
+            switch (p.ep.act) {
+                case NOT_ACT:
+                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case SILU:
+                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+            }
+            return;
+        }
+    }
     switch (p.ep.act) {
         case NOT_ACT:
         case RELU6: write_tile<DT, EPI_NONE, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
         case RELU: write_tile<DT, EPI_RELU, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
         case CLIP: write_tile<DT, EPI_CLIP, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case SILU:
+        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
         default: write_tile<DT, EPI_GENERIC, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
     }
 }

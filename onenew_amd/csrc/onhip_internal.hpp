@@ -62,7 +62,7 @@ __device__ __forceinline__ float apply_act(float v, const Epilogue &e) {
 
 // The activation kind as a template parameter, so the common ones cost one or two instructions and no
 // branch in an unrolled epilogue; EPI_GENERIC falls back to apply_act.
-enum { EPI_NONE = 0, EPI_RELU = 1, EPI_CLIP = 2, EPI_GENERIC = 3 };
+enum { EPI_NONE = 0, EPI_RELU = 1, EPI_CLIP = 2, EPI_GENERIC = 3, EPI_LUT = 4 };
 
 inline int epi_of_act(int act) {
     return (act == NOT_ACT || act == RELU6) ? EPI_NONE : act == RELU ? EPI_RELU : act == CLIP ? EPI_CLIP : EPI_GENERIC;
@@ -75,6 +75,13 @@ __device__ __forceinline__ float act_fast(float v, const Epilogue &e) {
     else if constexpr (EPI == EPI_CLIP) {
         const float t = v > e.clip_min ? v : e.clip_min;
         return t < e.clip_max ? t : e.clip_max;
+    } else if constexpr (EPI == EPI_LUT) {
+        // the table activations of apply_act without branches: the load is unconditional (index clamped into
+        // the table) and the two outer ranges are selected afterwards
+        int idx = (int) __fmul_rn(__fadd_rn(v, 8.0f), 512.0f);
+        idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
+        const float l = e.lut[idx];
+        return v < -8.0f ? 0.0f : v >= 8.0f ? v : l;
     } else return apply_act(v, e);
 }
 
