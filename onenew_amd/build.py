@@ -16,7 +16,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 instructions are switched off for every device compile; floating-point contraction is
 # off because the epilogues and the depthwise kernels reproduce the reference's separately rounded
 # multiply and add (__fmul_rn / __fadd_rn are plain operators to this compiler, not barriers)
-HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-c++20-extensions",
              "-ffp-contract=off",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 KERNEL_SOURCES = ["depthwise.hip", "igemm_f32.hip", "igemm_bf16.hip", "igemm_f16.hip", "igemm_i8.hip", "igemm.hip", "direct.hip", "calib.hip", "elementwise.hip", "vit_glue.hip", "api.hip",

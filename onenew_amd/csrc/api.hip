@@ -555,6 +555,8 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     p.use_tapmask = p.khkw <= 64;
     p.units_per_tap = cp / 16;
     p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
+    // K tiles (4 units) inside one filter tap: the loader variant with scalar tap arithmetic
+    if (p.use_tapmask && p.units_per_tap % 4 == 0) cfg.bl = BL_KVEC_TAP;
     p.pix_stride = cp;
     p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * cp;
     p.a_slice_bytes = (long long) p.M * p.lda;

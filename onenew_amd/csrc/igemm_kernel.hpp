@@ -35,6 +35,7 @@
 #pragma once
 #include "onhip_internal.hpp"
 #include <type_traits>
+#include <utility>
 
 namespace onhip {
 
@@ -203,7 +204,7 @@ __device__ __forceinline__ ColState make_col(const IgemmParams &p, int n) {
     c.ih0 = oh * p.sh - p.pt;
     c.iw0 = ow * p.sw - p.pl;
     unsigned off;
-    if constexpr (BL != BL_KVEC) off = (unsigned) (img * (int) p.b_img_stride + oh * p.sh * p.W + ow * p.sw) * 4u;
+    if constexpr (BL != BL_KVEC && BL != BL_KVEC_TAP) off = (unsigned) (img * (int) p.b_img_stride + oh * p.sh * p.W + ow * p.sw) * 4u;
     else off = (unsigned) ((img * p.H + oh * p.sh) * p.W + ow * p.sw) * (unsigned) p.pix_stride;
     c.pixoff = valid ? off : OOB;
     c.mask_lo = c.mask_hi = 0;
@@ -496,7 +497,7 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
 }
 
 // ---- the kernel --------------------------------------------------------------------------------
-template <int DT, int BL, int BM, int BN, int WM, int WN>
+template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1>
 __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -512,7 +513,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     // The vector loader (BL_KVEC) gives the UPT units of one column to neighbouring lanes as well: they are
     // contiguous in memory (one 64-byte run per pixel instead of 64 scattered 16-byte pieces per load), and the
     // filter tap of a unit becomes a per-lane quantity.
-    constexpr bool LANE_UNITS = BL == BL_KVEC;
+    constexpr bool LANE_UNITS = BL == BL_KVEC || BL == BL_KVEC_TAP;
     constexpr int B_LD = LANE_UNITS ? BN + 1 : BN, B_LDS = B_LD * UPT;
     constexpr int A_PER_T = (A_SLOTS + THREADS - 1) / THREADS;
     constexpr int B_PER_T = B_SLOTS / THREADS;
@@ -574,6 +575,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     for (int t = 0; t < NCOL; ++t)
         cols[t] = make_col<BL>(p, n0 + (LANE_UNITS ? (tid + t * THREADS) / UPT : tid % BN));
     const ColState &col = cols[0];
+    const unsigned lane_unit_off = (unsigned) (tid % UPT) * 16u;
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -583,7 +585,10 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
 
-    RawUnit<DT> qa[A_PER_T], qb[B_PER_T];
+    // PF K tiles are in flight between global memory and LDS, each in a register set of its own (tile t in
+    // set t % PF).  One set covers one memory latency per K tile; short tiles (two int8 MFMAs per wavefront)
+    // need several.
+    RawUnit<DT> qa_[PF][A_PER_T], qb_[PF][B_PER_T];
 
     constexpr int PARTS = Traits<DT>::PARTS;
     constexpr int BE = BL == BL_TAPC ? 1 : KPU;                      // scalar descriptions per B unit
@@ -605,8 +610,10 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     // issue every global load of K tile kt (B descriptions must have been prepared for kt).  A tile past the
     // end of the slice is switched off as a whole through empty buffer descriptors (a scalar select): its
     // loads return zero without touching memory.  CHK adds the per-unit tests a ragged last tile needs.
-    auto issue = [&](int kt, auto chk) {
+    auto issue = [&](int kt, auto chk, auto slot) {
         constexpr bool CHK = decltype(chk)::value;
+        RawUnit<DT> (&qa)[A_PER_T] = qa_[decltype(slot)::value];
+        RawUnit<DT> (&qb)[B_PER_T] = qb_[decltype(slot)::value];
         const int ub = u_begin + kt * UPT;
         const bool live = kt < k_tiles;
         const rsrc_t ra = make_rsrc(a_base, live ? a_bytes : 0u);
@@ -614,7 +621,29 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t)
             load_a_unit<DT, CHK>(qa[t], ra, a_voff[t], (unsigned) (ub * KPU * ESZ), (ub + a_unit[t]) * KPU, klim);
-        if constexpr (LANE_UNITS) {
+        if constexpr (BL == BL_KVEC_TAP) {
+            // the UPT units of the tile share one filter tap: tap, offset and mask bit are scalar, a lane only
+            // adds its unit's 16 bytes (kept in lane_unit_off) and tests the tap in its column's mask
+            const unsigned tap = fast_div((unsigned) ub, p.magic_upt, p.pass_upt);
+            const unsigned cb0 = (unsigned) ub - tap * (unsigned) p.units_per_tap;
+            const unsigned ti = fast_div(tap, p.magic_kw, p.pass_kw);
+            const unsigned tj = tap - ti * (unsigned) p.kw;
+            const unsigned soff = (ti * (unsigned) p.W + tj) * (unsigned) p.pix_stride + cb0 * 16u;
+            const unsigned bit = 1u << (tap & 31u);
+            const bool hi = tap >= 32u;
+            const bool k_ok = !CHK || (int) (((unsigned) ub + (unsigned) (tid % UPT)) * KPU) < klim;
+#pragma unroll
+            for (int t = 0; t < B_PER_T; ++t) {
+                const unsigned word = hi ? cols[t].mask_hi : cols[t].mask_lo;
+                const bool ok = k_ok && (word & bit) != 0u;
+                const uint4 q = buf_load_b128(rb, ok ? cols[t].pixoff + lane_unit_off : OOB, soff);
+                if constexpr (DT == DT_I8) qb[t].q = q;
+                else {
+                    qb[t].v[0] = __uint_as_float(q.x); qb[t].v[1] = __uint_as_float(q.y);
+                    qb[t].v[2] = __uint_as_float(q.z); qb[t].v[3] = __uint_as_float(q.w);
+                }
+            }
+        } else if constexpr (BL == BL_KVEC) {
             // this lane's unit: filter tap and channel block, then one 16-byte load per column
             const unsigned u = (unsigned) ub + (unsigned) (tid % UPT);
             const unsigned tap = fast_div(u, p.magic_upt, p.pass_upt);
@@ -625,14 +654,12 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             const bool k_ok = !CHK || (int) (u * KPU) < klim;
 #pragma unroll
             for (int t = 0; t < B_PER_T; ++t) {
-                bool ok = k_ok;
-                if (p.use_tapmask) {
-                    const unsigned word = tap >= 32u ? cols[t].mask_hi : cols[t].mask_lo;
-                    ok = ok && ((word >> (tap & 31u)) & 1u);
-                } else {
-                    ok = ok && (unsigned) (cols[t].ih0 + (int) ti) < (unsigned) p.H &&
-                         (unsigned) (cols[t].iw0 + (int) tj) < (unsigned) p.W;
-                }
+                // both validity tests, then a select: no branch in the K loop
+                const unsigned word = tap >= 32u ? cols[t].mask_hi : cols[t].mask_lo;
+                const bool by_mask = ((word >> (tap & 31u)) & 1u) != 0u;
+                const bool by_coord = (unsigned) (cols[t].ih0 + (int) ti) < (unsigned) p.H &&
+                                      (unsigned) (cols[t].iw0 + (int) tj) < (unsigned) p.W;
+                const bool ok = k_ok & (p.use_tapmask ? by_mask : by_coord);
                 const uint4 q = buf_load_b128(rb, ok ? cols[t].pixoff + off : OOB, 0);
                 if constexpr (DT == DT_I8) qb[t].q = q;
                 else {
@@ -657,8 +684,10 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             }
         }
     };
-    auto stage = [&](int buf, int kt, auto chk) {
+    auto stage = [&](int buf, int kt, auto chk, auto slot) {
         constexpr bool CHK = decltype(chk)::value;
+        RawUnit<DT> (&qa)[A_PER_T] = qa_[decltype(slot)::value];
+        RawUnit<DT> (&qb)[B_PER_T] = qb_[decltype(slot)::value];
 #pragma unroll
         for (int t = 0; t < A_PER_T; ++t) {
             const int f = tid + t * THREADS;
@@ -680,30 +709,36 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     };
 
     // Pipeline.  While the MFMAs of K tile kt run (its operands are already in registers):
-    //   step 0            LDS store of tile kt+1 (loaded one tile ago), then all global loads of tile kt+2
-    //   steps 1..         scalar descriptions of the B loads of tile kt+3, spread over the MFMAs
+    //   step 0            LDS store of tile kt+1 (loaded PF tiles ago), then all global loads of tile kt+1+PF
+    //   steps 1..         scalar descriptions of the B loads of the tile after that, spread over the MFMAs
     //   after HALF steps  barrier
     //   second half       LDS reads of tile kt+1 into the other operand set, spread over the MFMAs
     // A wavefront therefore always has matrix work queued while it waits for LDS, the barrier or
-    // memory, and a global load has a whole tile of MFMAs to complete.  Past the last tile loads are
+    // memory, and a global load has PF tiles of MFMAs to complete.  Past the last tile loads are
     // fully masked (zero, no memory traffic), so the body has no branches.
     Operands op0, op1;
     constexpr std::true_type CHECKED{};
     constexpr std::false_type UNCHECKED{};
+    static_assert(PF == 1 || B_ITEMS == 0, "scalar B descriptions are prepared one tile ahead: PF == 1 only");
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(0, i);
-    issue(0, CHECKED);
-    stage(0, 0, CHECKED);
+    issue(0, CHECKED, std::integral_constant<int, 0>{});
+    stage(0, 0, CHECKED, std::integral_constant<int, 0>{});
+    // tiles 1 .. PF: tile t into set t % PF
+    [&]<int... T>(std::integer_sequence<int, T...>) __attribute__((always_inline)) {
+        ((void) ([&] {
 #pragma unroll
-    for (int i = 0; i < B_ITEMS; ++i) prep_item(1, i);
-    issue(1, CHECKED);
+            for (int i = 0; i < B_ITEMS; ++i) prep_item(T + 1, i);
+            issue(T + 1, CHECKED, std::integral_constant<int, (T + 1) % PF>{});
+        }()), ...);
+    }(std::make_integer_sequence<int, PF>{});
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(2, i);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < READS; ++i) read_operand(op0, 0, i);
 
-    auto body = [&](Operands &cur, Operands &nxt, int kt, auto chk) {
+    auto body = [&](Operands &cur, Operands &nxt, int kt, auto chk, auto slot) {
         const int nbuf = (kt + 1) & 1;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -712,8 +747,8 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             const int s = blk / (TM * TN), a = (blk / TN) % TM, b = blk % TN;
             Traits<DT>::mma_part(acc[a][b], cur.a[s][a], cur.b[s][b], part);
             if (st == 0) {
-                stage(nbuf, kt + 1, chk);
-                issue(kt + 2, chk);
+                stage(nbuf, kt + 1, chk, slot);
+                issue(kt + 1 + PF, chk, slot);
             }
 #pragma unroll
             for (int i = 0; i < B_ITEMS; ++i)
@@ -727,20 +762,24 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // Body kt stores tile kt+1 to LDS and loads tile kt+2; the ragged tile k_tiles-1 is therefore touched by
-    // bodies k_tiles-3 and k_tiles-2.  Everything before runs without per-element tests (an even count, so the
-    // two operand sets keep their roles).
-    const int n_plain = (ragged ? max(0, k_tiles - 3) : k_tiles) & ~1;
+    // Body kt stores tile kt+1 to LDS (register set (kt+1) % PF) and loads tile kt+1+PF into the same set; the
+    // ragged tile k_tiles-1 is therefore touched by bodies k_tiles-2-PF and k_tiles-2.  Everything before runs
+    // without per-element tests.  The loop is unrolled over U bodies so that operand sets and register sets are
+    // compile-time choices.
+    constexpr int U = (PF % 2 == 0) ? PF : 2 * PF;
+    auto group = [&](int kt0, auto chk, auto guarded) __attribute__((always_inline)) {
+        [&]<int... J>(std::integer_sequence<int, J...>) __attribute__((always_inline)) {
+            ((void) ([&] {
+                if (!decltype(guarded)::value || kt0 + J < k_tiles)
+                    body(J % 2 == 0 ? op0 : op1, J % 2 == 0 ? op1 : op0, kt0 + J, chk, std::integral_constant<int, (J + 1) % PF>{});
+            }()), ...);
+        }(std::make_integer_sequence<int, U>{});
+    };
+    const int n_plain = (ragged ? max(0, k_tiles - 2 - PF) : k_tiles) / U * U;
     int kt = 0;
-    for (; kt < n_plain; kt += 2) {
-        body(op0, op1, kt, UNCHECKED);
-        body(op1, op0, kt + 1, UNCHECKED);
-    }
-    for (; kt + 1 < k_tiles; kt += 2) {
-        body(op0, op1, kt, CHECKED);
-        body(op1, op0, kt + 1, CHECKED);
-    }
-    if (kt < k_tiles) body(op0, op1, kt, CHECKED);
+    for (; kt < n_plain; kt += U) group(kt, UNCHECKED, std::false_type{});
+    for (; kt + U <= k_tiles; kt += U) group(kt, CHECKED, std::false_type{});
+    if (kt < k_tiles) group(kt, CHECKED, std::true_type{});
 
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
     if (p.partial) {
@@ -807,7 +846,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p,
 }
 
 // ---- launch ------------------------------------------------------------------------------------------
-template <int DT, int BL, int BM, int BN, int WM, int WN>
+template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1>
 static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream_t stream) {
     IgemmParams p = p_in;
     const int tiles_m = (p.M + BM - 1) / BM;
@@ -816,7 +855,7 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
     p.div_tiles_m = make_div31((unsigned) tiles_m);
     dim3 grid(tiles, cfg.split, cfg.batch);
-    hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN>), grid, dim3(THREADS), 0, stream, p);
+    hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN, PF>), grid, dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
     if (p.partial) {
         if (p.M > 4 * 65535 || cfg.batch > 65535)
@@ -831,17 +870,16 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     return ONHIP_OK;
 }
 
-template <int DT, int BL>
+template <int DT, int BL, int PF = 1>
 int launch_tile(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
     const int key = cfg.bm * 1000 + cfg.bn;
     switch (key) {
-        case 128128: return launch_one<DT, BL, 128, 128, 2, 2>(cfg, p, stream);
-        case 64128: return launch_one<DT, BL, 64, 128, 2, 2>(cfg, p, stream);
-        case 64064: return launch_one<DT, BL, 64, 64, 2, 2>(cfg, p, stream);
-        case 32128: return launch_one<DT, BL, 32, 128, 1, 4>(cfg, p, stream);
+        case 128128: return launch_one<DT, BL, 128, 128, 2, 2, (PF > 2 ? 2 : PF)>(cfg, p, stream);
+        case 64128: return launch_one<DT, BL, 64, 128, 2, 2, PF>(cfg, p, stream);
+        case 64064: return launch_one<DT, BL, 64, 64, 2, 2, PF>(cfg, p, stream);
+        case 32128: return launch_one<DT, BL, 32, 128, 1, 4, PF>(cfg, p, stream);
         default: return set_error(ONHIP_ERR_ARG, "igemm: no kernel for tile %dx%d", cfg.bm, cfg.bn);
     }
 }
-
 
 }  // namespace onhip

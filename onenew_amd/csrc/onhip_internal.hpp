@@ -100,7 +100,9 @@ __device__ __forceinline__ int quant_s8(float x, float inv_scale) {
 enum { BL_GATHER = 0,  // element gather from NCHW activations (implicit im2col), any filter / stride / padding
        BL_KVEC = 1,    // 16-byte vectors along K from NHWC int8 activations
        BL_PLAIN = 2,   // 1x1 filter without padding, or a row-major [K, N] matrix: no tap arithmetic
-       BL_TAPC = 3 };  // NCHW activations against tap-major packed weights: K = (tap, channel), one tap per unit
+       BL_TAPC = 3,    // NCHW activations against tap-major packed weights: K = (tap, channel), one tap per unit
+       BL_KVEC_TAP = 4 };  // BL_KVEC whose K tiles never straddle a filter tap (units per tap a multiple of the
+                           // tile, at most 64 taps): tap arithmetic is scalar and the K loop has no branches
 
 enum { OUT_CONV = 0,   // n = img * OHW + pix  ->  img * c_img_stride + m * c_stride_m + pix
        OUT_PLAIN = 1 };// m * c_stride_m + n * c_stride_n

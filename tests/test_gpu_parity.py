@@ -565,12 +565,34 @@ def test_transpose_matches_numpy_and_plugin(name, torch_dev):
         assert np.array_equal(ops.Transpose(ops.Plugin(hip.plugin_path("Transpose")).eval, perm)(x), np.transpose(x, perm))
 
 
-@pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_s2", "yolo_c2f_3x3_64_80", "yolo_sppf_1x1_1024", "q3x3_bigacc"])
-def test_conv_w8a8_nhwc_chain_form(name, torch_dev, oracle):
+# chain-form shapes beyond the W8A32 case list: output channels that end inside a 16-channel group and inside a
+# row tile, channel counts whose K tiles do / do not straddle filter taps (64-channel multiples or not)
+CHAIN_EXTRA = {
+    "chain_128_80_3x3": cases.cd(128, 80, 3, 1, 1, 13, act=abi.SILU, input_scale=0.017),
+    "chain_48_24_3x3_s2": cases.cd(48, 24, 3, 2, 1, 17, act=abi.CLIP, clip_min=-0.5, clip_max=2.0, input_scale=0.02),
+    "chain_192_200_1x1": cases.cd(192, 200, 1, 1, 0, 9, act=abi.LEAKYRELU, leaky_relu_alpha=0.1, input_scale=0.012),
+    "chain_64_33_5x5": cases.cd(64, 33, 5, 1, 2, 11, act=abi.HARDSILU, hard_sigmoid_alpha=0.2, hard_sigmoid_beta=0.5, input_scale=0.015),
+}
+
+
+def _chain_desc(name):
+    if name in CHAIN_EXTRA:
+        return ConvDesc.from_buffer_copy(CHAIN_EXTRA[name])
+    return ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()[name])
+
+
+@pytest.mark.parametrize("tile", [None, "128x128", "64x128", "32x128", "64x64x2"])
+@pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_s2", "yolo_c2f_3x3_64_80", "yolo_sppf_1x1_1024", "q3x3_bigacc"]
+                         + list(CHAIN_EXTRA))
+def test_conv_w8a8_nhwc_chain_form(name, tile, torch_dev, oracle, monkeypatch):
     """int8 NHWC in / int8 NHWC out: the same int8 values as quantising the reference's fp32 result, and the
-    quantised input equals the reference's own input quantiser"""
+    quantised input equals the reference's own input quantiser; every tile shape and the split-K path"""
     torch = torch_dev
-    d = ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()[name])
+    if tile is not None and name in ("yolo_sppf_1x1_1024", "q3x3_silu", "q3x3_s2"):
+        pytest.skip("forced tiles run on the shapes with ragged rows and columns")
+    if tile:
+        monkeypatch.setenv("ONHIP_TILE", tile)
+    d = _chain_desc(name)
     d.n = 3
     d.out_s8, d.output_scale = 1, 0.041
     x, w8, b32, aux = cases.conv_inputs(name + "_chain", d, quant=True)
@@ -580,6 +602,11 @@ def test_conv_w8a8_nhwc_chain_form(name, torch_dev, oracle):
     assert np.array_equal(xq.cpu().numpy()[..., :d.cin], np.transpose(q_ref, (0, 2, 3, 1)))
     assert not xq.cpu().numpy()[..., d.cin:].any()                            # channel padding is zero
     wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
-    yq = hip.conv2d_w8a8_nhwc(d, xq, wp, dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()))
+    oh, ow = d.out_hw()
+    out = torch.full((d.n, oh, ow, (d.cout + 15) // 16 * 16), 77, dtype=torch.int8, device="cuda")
+    yq = hip.conv2d_w8a8_nhwc(d, xq, wp, dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()), out=out)
     torch.cuda.synchronize()
-    assert np.array_equal(yq.cpu().numpy()[..., :d.cout], np.transpose(ref, (0, 2, 3, 1)))
+    got = yq.cpu().numpy()
+    assert np.array_equal(got[..., :d.cout], np.transpose(ref, (0, 2, 3, 1)))
+    if tile is None or "x2" not in tile:
+        assert not got[..., d.cout:].any()                                    # unsplit launches zero the channel padding
