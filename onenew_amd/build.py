@@ -37,13 +37,35 @@ def _stale(target, sources):
     return any(os.path.getmtime(s) > t for s in sources)
 
 
+def _scratch_users(text):
+    """kernels that the compiler gave a stack frame (register arrays that fell out of registers): the resource
+    remarks come as a 'Function Name' line followed by that function's figures"""
+    bad, name = [], None
+    for line in text.splitlines():
+        if "remark:" not in line:
+            continue
+        body = line.split("remark:", 1)[1].strip()
+        if body.startswith("Function Name:"):
+            name = body.split(":", 1)[1].split("[")[0].strip()
+        elif body.startswith("ScratchSize [bytes/lane]:"):
+            if int(body.split(":", 1)[1].split("[")[0]) > 0 and name:
+                bad.append(name)
+    return bad
+
+
 def _run(cmd):
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l and "remark:" not in l)
     if res.returncode != 0:
         raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + out)
     if out.strip():
         print(out)
+    # the MFMA kernels keep tiles, operands and prefetched units in registers by construction: a kernel of those
+    # files that uses scratch memory has lost that (a lambda that was not inlined, an array indexed at run time)
+    if any(os.path.basename(a).startswith("igemm_") for a in cmd):
+        bad = _scratch_users(res.stdout)
+        if bad:
+            raise RuntimeError("kernels with a stack frame (scratch memory) in " + cmd[-3] + ":\n  " + "\n  ".join(bad))
 
 
 def build(force=False, verbose=True):
@@ -56,7 +78,7 @@ def build(force=False, verbose=True):
         o = os.path.join(OBJDIR, src + ".o")
         objs.append(o)
         if force or _stale(o, [s] + HEADERS):
-            jobs.append([HIPCC] + HIP_FLAGS + ["-c", s, "-o", o])
+            jobs.append([HIPCC] + HIP_FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", s, "-o", o])
     if verbose and jobs:
         print(f"[onenew_amd.build] compiling {len(jobs)} file(s) for gfx950", flush=True)
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:

@@ -602,15 +602,15 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     BPrep bp[B_ITEMS > 0 ? B_ITEMS : 1];              // scalar descriptions of the next B loads
     const unsigned hw4 = (unsigned) p.HW * 4u;
 
-    auto b_unit_of = [&](int t) { return __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN); };
-    auto prep_item = [&](int kt, int idx) {
+    auto b_unit_of = [&](int t) __attribute__((always_inline)) { return __builtin_amdgcn_readfirstlane((tid + t * THREADS) / BN); };
+    auto prep_item = [&](int kt, int idx) __attribute__((always_inline)) {
         const int t = idx / BE, e = idx % BE;
         bp[idx] = prep_b<DT, BL>(p, u_begin + kt * UPT + b_unit_of(t), e, klim);
     };
     // issue every global load of K tile kt (B descriptions must have been prepared for kt).  A tile past the
     // end of the slice is switched off as a whole through empty buffer descriptors (a scalar select): its
     // loads return zero without touching memory.  CHK adds the per-unit tests a ragged last tile needs.
-    auto issue = [&](int kt, auto chk, auto slot) {
+    auto issue = [&](int kt, auto chk, auto slot) __attribute__((always_inline)) {
         constexpr bool CHK = decltype(chk)::value;
         RawUnit<DT> (&qa)[A_PER_T] = qa_[decltype(slot)::value];
         RawUnit<DT> (&qb)[B_PER_T] = qb_[decltype(slot)::value];
@@ -684,7 +684,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             }
         }
     };
-    auto stage = [&](int buf, int kt, auto chk, auto slot) {
+    auto stage = [&](int buf, int kt, auto chk, auto slot) __attribute__((always_inline)) {
         constexpr bool CHK = decltype(chk)::value;
         RawUnit<DT> (&qa)[A_PER_T] = qa_[decltype(slot)::value];
         RawUnit<DT> (&qb)[B_PER_T] = qb_[decltype(slot)::value];
@@ -702,7 +702,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             else lds[buf][A_LDS + (f / BN) * B_LD + (f % BN)] = pack_unit<DT>(qb[t]);
         }
     };
-    auto read_operand = [&](Operands &o, int buf, int idx) {   // idx-th of the READS LDS reads
+    auto read_operand = [&](Operands &o, int buf, int idx) __attribute__((always_inline)) {   // idx-th of the READS LDS reads
         const int s = idx / (TM + TN), t = idx % (TM + TN);
         if (t < TM) o.a[s][t] = lds[buf][(2 * s + lh) * A_LD + wm * (BM / WM) + t * 32 + li];
         else o.b[s][t - TM] = lds[buf][A_LDS + (2 * s + lh) * B_LD + wn * (BN / WN) + (t - TM) * 32 + li];
@@ -726,7 +726,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     stage(0, 0, CHECKED, std::integral_constant<int, 0>{});
     // tiles 1 .. PF: tile t into set t % PF
     [&]<int... T>(std::integer_sequence<int, T...>) __attribute__((always_inline)) {
-        ((void) ([&] {
+        ((void) ([&]() __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < B_ITEMS; ++i) prep_item(T + 1, i);
             issue(T + 1, CHECKED, std::integral_constant<int, (T + 1) % PF>{});
@@ -738,7 +738,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 #pragma unroll
     for (int i = 0; i < READS; ++i) read_operand(op0, 0, i);
 
-    auto body = [&](Operands &cur, Operands &nxt, int kt, auto chk, auto slot) {
+    auto body = [&](Operands &cur, Operands &nxt, int kt, auto chk, auto slot) __attribute__((always_inline)) {
         const int nbuf = (kt + 1) & 1;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -769,7 +769,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     constexpr int U = (PF % 2 == 0) ? PF : 2 * PF;
     auto group = [&](int kt0, auto chk, auto guarded) __attribute__((always_inline)) {
         [&]<int... J>(std::integer_sequence<int, J...>) __attribute__((always_inline)) {
-            ((void) ([&] {
+            ((void) ([&]() __attribute__((always_inline)) {
                 if (!decltype(guarded)::value || kt0 + J < k_tiles)
                     body(J % 2 == 0 ? op0 : op1, J % 2 == 0 ? op1 : op0, kt0 + J, chk, std::integral_constant<int, (J + 1) % PF>{});
             }()), ...);
