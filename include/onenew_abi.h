@@ -204,6 +204,48 @@ typedef struct {
     int64_t perm_num;
 } TRANSPOSE_CONFIG_S;
 
+/* common/nn_common.h:296-300: Flatten keeps the data and only changes the shape (host/ops/flatten.h:29-62) */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    int64_t axis;
+} FLATTEN_CONFIG_S;
+
+/* common/nn_common.h:486-493: Reshape, likewise a view (host/ops/reshape.h:31-70) */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    int64_t allowzero;
+    int64_t dst_shape[8];
+    int64_t dst_shape_num;
+} RESHAPE_CONFIG_S;
+
+/* ---- the .one model file (tools/onnx2one/onnx2one.cpp:1294-1355, host/net.h:101-196) -------------------
+ * [ONE_MODEL_DESC_S][node configs][initialisers][io configs], every piece padded to 64 bytes:
+ *   node config   the op's *_CONFIG_S, BASE_CONFIG_S first (op_type selects the struct)
+ *   initialiser   OPERAND_S followed by the raw data (shape product * element size bytes)
+ *   io config     IO_CONFIG_S, op_type "io", op_name "input" or "output"
+ */
+#define ONE_MAGIC_NUM (0x6F6E65)
+
+/* common/nn_common.h:64-75 */
+typedef struct {
+    int32_t one_model_magic_num;
+    int32_t version;
+    int32_t node_cnt;
+    int32_t node_cfg_offset;
+    int32_t init_cnt;
+    int32_t init_info_offset;
+    int32_t io_cfg_cnt;
+    int32_t io_cfg_offset;
+    USEFUL_INFO_S useful_info;
+} ONE_MODEL_DESC_S;
+
+/* common/nn_common.h:157-162 */
+typedef struct {
+    char op_type[OP_TYPE_LEN];   /* "io" */
+    char op_name[OP_NAME_LEN];   /* "input" or "output" */
+    OPERAND_S operand;
+} IO_CONFIG_S;
+
 /* the one symbol a plugin exports */
 typedef int (*onenew_eval_fn)(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 
@@ -213,6 +255,11 @@ typedef int (*onenew_eval_fn)(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFF
 #define ONENEW_SA(c, m) _Static_assert(c, m)
 #endif
 ONENEW_SA(sizeof(BUFFER_INFO_S) == 16, "BUFFER_INFO_S");
+ONENEW_SA(sizeof(ONE_MODEL_DESC_S) == 32 + sizeof(USEFUL_INFO_S) && offsetof(ONE_MODEL_DESC_S, useful_info) == 32,
+          "ONE_MODEL_DESC_S");
+ONENEW_SA(sizeof(IO_CONFIG_S) == 512 + sizeof(OPERAND_S), "IO_CONFIG_S");
+ONENEW_SA(sizeof(FLATTEN_CONFIG_S) == sizeof(BASE_CONFIG_S) + 8, "FLATTEN_CONFIG_S");
+ONENEW_SA(sizeof(RESHAPE_CONFIG_S) == sizeof(BASE_CONFIG_S) + 80, "RESHAPE_CONFIG_S");
 ONENEW_SA(sizeof(OPERAND_S) == 312, "OPERAND_S");
 ONENEW_SA(offsetof(OPERAND_S, p_data) == 264, "OPERAND_S.p_data");
 ONENEW_SA(offsetof(OPERAND_S, dim_num_of_shapes) == 272, "OPERAND_S.dim_num_of_shapes");

@@ -275,6 +275,14 @@ int onhip_layernorm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_IN
 int onhip_softmax_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/*
+ * No counterpart in the reference, whose operators always finish before eval returns (device/cuda/MaxPool/
+ * maxpool.cu:76).  on != 0: an eval whose output is device memory returns as soon as its kernels are queued on
+ * the default stream; the caller orders its own reads after them (a blocking hipMemcpy, hipStreamSynchronize).
+ * Used by the device-resident runtime (onenew_rt.h) between the operators of one inference.  Outputs in host
+ * memory are still complete on return.
+ */
+int onhip_plugin_set_async(int on);
 /* Drops the device copies of weights the plugin level keeps between calls. */
 int onhip_plugin_release(void);
 

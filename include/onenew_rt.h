@@ -1,0 +1,82 @@
+/*
+ * onenew_rt.h -- device-resident execution of a .one model: the part of the oneNew host runtime that sits
+ * either side of the operator plugins, with every operand buffer and every initialiser in HBM.
+ *
+ * It restates the calling sequence of the reference host (host/net.h): load the file, build one operator
+ * object per node, order them, infer shapes, allocate one buffer per operand, fill the plugin slot arrays and
+ * call each plugin's `eval` in order.  What differs is where the bytes live: initialisers are uploaded once
+ * at load time, operand buffers are device memory, and between two operators nothing crosses PCIe.  Only the
+ * net's inputs are copied in and its outputs copied out.
+ *
+ * Operators: Conv, MatMul, Gemm, Add, Relu, MaxPool, GlobalAveragePool, Gelu, LayerNormalization, Softmax,
+ * Transpose through `lib<Op>_hip.so`; Flatten and Reshape as views (no buffer, no call: host/op.h:149-154).
+ * A model with any other node type is refused at load time.
+ *
+ * All functions return 0 on success or a negative ONRT_ERR_* code; onrt_last_error() describes the failure.
+ */
+#ifndef ONENEW_RT_H
+#define ONENEW_RT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ONRT_OK 0
+#define ONRT_ERR_ARG (-1)       /* null pointer, bad index, unknown operand name */
+#define ONRT_ERR_FORMAT (-2)    /* not a .one file, truncated file, node of an unsupported type */
+#define ONRT_ERR_PLUGIN (-3)    /* lib<Op>_hip.so not found, no `eval` in it, or eval returned non-zero */
+#define ONRT_ERR_RUNTIME (-4)   /* HIP call failed, out of memory */
+
+typedef struct onrt_net onrt_net_t;
+
+/* Message of the last failure on the calling thread. */
+const char *onrt_last_error(void);
+
+/*
+ * Loads a model and makes it ready to run: host/net.h:101-131 (load_one_model) or :133-136 (load_one_buf),
+ * :138-189 (instantiate_op), :191-221 (initialiser list), :378-389 (build_graph: order, operand list, shapes),
+ * :419-452 (new_output_buf) and :629-640 (prepare_for_op).  The buffer is copied; the caller may free it.
+ *
+ * op_lib_dir: where the operator plugins are looked up, in the order of host/op.h:41-80 with the HIP
+ * library in the place of the x86 one: <dir>/<Op>/lib<Op>_hip.so, then <dir>/lib<Op>_hip.so.  NULL means
+ * the environment variable ONENEW_OP_LIB_DIR, and without it the directory this library was loaded from.
+ */
+int onrt_net_load_file(const char *one_path, const char *op_lib_dir, onrt_net_t **net);
+int onrt_net_load_buf(const void *one_buf, size_t bytes, const char *op_lib_dir, onrt_net_t **net);
+
+/* Releases the device memory of the net and its operator objects (host/net.h:401-416). */
+void onrt_net_free(onrt_net_t *net);
+
+/* Counts of the io nodes named "input" / "output" (host/ops/io.h:56-70), in file order. */
+int onrt_net_io_count(const onrt_net_t *net, int32_t *n_inputs, int32_t *n_outputs);
+
+/* Name, rank and shape (SHAPE_LEN entries, unused ones 1) of input or output number idx. */
+int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, const char **name, int32_t *ndim,
+                     int32_t shape[8]);
+
+/* Operators in execution order (host/net.h:309-330): type and name of number idx, count through n_ops. */
+int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops);
+int onrt_net_op_info(const onrt_net_t *net, int32_t idx, const char **op_type, const char **op_name);
+
+/*
+ * Shape and device address of any operand by name, after shape inference: the counterpart of the per-layer
+ * dump mode (host/net.h:456-537), which reads operand_buf_map.  dev_ptr may be NULL.
+ */
+int onrt_net_operand(const onrt_net_t *net, const char *name, int32_t *ndim, int32_t shape[8], void **dev_ptr);
+
+/*
+ * One inference (extractor::impl, host/net.h:613-627).  inputs[i] / outputs[i] belong to input / output
+ * number i and hold fp32 elements of that operand's shape; each may be host or device memory.  Inputs are
+ * copied into the net's buffers, the operators run back to back on the device without a host wait in
+ * between, outputs are copied out and are complete on return.  An outputs[i] of NULL skips that copy
+ * (read the result in place through onrt_net_operand).
+ */
+int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ONENEW_RT_H */

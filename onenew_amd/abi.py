@@ -108,6 +108,29 @@ class TRANSPOSE_CONFIG_S(C.Structure):
     _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("perm", C.c_int64 * 8), ("perm_num", C.c_int64)]
 
 
+class FLATTEN_CONFIG_S(C.Structure):
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("axis", C.c_int64)]
+
+
+class RESHAPE_CONFIG_S(C.Structure):
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("allowzero", C.c_int64), ("dst_shape", C.c_int64 * 8),
+                ("dst_shape_num", C.c_int64)]
+
+
+ONE_MAGIC_NUM = 0x6F6E65
+
+
+class ONE_MODEL_DESC_S(C.Structure):
+    """header of a .one file (common/nn_common.h:64-75)"""
+    _fields_ = [("one_model_magic_num", C.c_int32), ("version", C.c_int32), ("node_cnt", C.c_int32),
+                ("node_cfg_offset", C.c_int32), ("init_cnt", C.c_int32), ("init_info_offset", C.c_int32),
+                ("io_cfg_cnt", C.c_int32), ("io_cfg_offset", C.c_int32), ("useful_info", USEFUL_INFO_S)]
+
+
+class IO_CONFIG_S(C.Structure):
+    _fields_ = [("op_type", C.c_char * NAME_LEN), ("op_name", C.c_char * NAME_LEN), ("operand", OPERAND_S)]
+
+
 class TransposeDesc(C.Structure):
     """onhip_transpose_desc_t"""
     _fields_ = [("ndim", C.c_int32), ("in_shape", C.c_int32 * 6), ("perm", C.c_int32 * 6)]
@@ -191,6 +214,8 @@ def check_layout():
     assert C.sizeof(LAYERNORMALIZATION_CONFIG_S) == 12880 and C.sizeof(SOFTMAX_CONFIG_S) == 12856
     assert C.sizeof(TRANSPOSE_CONFIG_S) == 12912 and TRANSPOSE_CONFIG_S.perm_num.offset == 12904
     assert C.sizeof(USEFUL_INFO_S) == 96 and USEFUL_INFO_S.public_buf_info.offset == 40
+    assert C.sizeof(ONE_MODEL_DESC_S) == 128 and C.sizeof(IO_CONFIG_S) == 824
+    assert C.sizeof(FLATTEN_CONFIG_S) == 12848 and C.sizeof(RESHAPE_CONFIG_S) == 12920
     assert C.sizeof(ConvDesc) == 25 * 4
     assert C.sizeof(MatmulDesc) == 24
 

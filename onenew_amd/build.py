@@ -1,5 +1,5 @@
 """Builds the gfx950 shared objects in place (onenew_amd/lib/): the kernel library
-libonenew_hip.so and the operator plugins lib{Conv,MatMul,Gemm,Add,Relu,MaxPool,GlobalAveragePool,Gelu,LayerNormalization,Softmax,Transpose}_hip.so.
+libonenew_hip.so, the model runtime libonenew_rt.so and the operator plugins lib{Conv,MatMul,Gemm,Add,Relu,MaxPool,GlobalAveragePool,Gelu,LayerNormalization,Softmax,Transpose}_hip.so.
 
     python -m onenew_amd.build [--force]
 """
@@ -92,6 +92,12 @@ def build(force=False, verbose=True):
         if force or _stale(so, [s, core] + HEADERS):
             _run(["g++", "-O2", "-fPIC", "-shared", "-fvisibility=hidden", s, "-o", so, "-L" + LIBDIR,
                   "-lonenew_hip", "-Wl,-rpath,$ORIGIN"])
+    # the device-resident model runtime: host code over the HIP runtime API, it reaches the kernels through the plugins
+    rt = os.path.join(LIBDIR, "libonenew_rt.so")
+    rt_src = os.path.join(CSRC, "runtime.cpp")
+    if force or _stale(rt, [rt_src, os.path.join(HERE, "..", "include", "onenew_rt.h")] + HEADERS):
+        _run(["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__",
+              "-I/opt/rocm/include", rt_src, "-o", rt, "-L/opt/rocm/lib", "-lamdhip64", "-ldl", "-Wl,-rpath,/opt/rocm/lib"])
     return LIBDIR
 
 

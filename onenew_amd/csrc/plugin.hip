@@ -21,6 +21,14 @@ namespace onhip {
 
 static std::mutex g_mu;
 static bool g_ready = false;
+// set by a caller that keeps consuming results on the device in stream order (onhip_plugin_set_async): an eval
+// whose output is device memory then returns without waiting for the kernels
+static bool g_async = false;
+
+static int wait_for_output() {
+    if (!g_async) ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    return ONHIP_OK;
+}
 
 struct DevBuf {
     void *ptr = nullptr;
@@ -266,7 +274,7 @@ static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
     }
     if (rc) return rc;
     if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, out_bytes, hipMemcpyDeviceToHost));
-    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    else return wait_for_output();
     return ONHIP_OK;
 }
 
@@ -310,7 +318,7 @@ static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFF
     rc = onhip_matmul(&d, (const float *) a, (const float *) b, nullptr, nullptr, (float *) y, nullptr);
     if (rc) return rc;
     if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, o_bytes, hipMemcpyDeviceToHost));
-    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    else return wait_for_output();
     return ONHIP_OK;
 }
 
@@ -343,7 +351,7 @@ static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
     rc = onhip_gemm_f32(M, K, N, (const float *) a, (const float *) w, (const float *) b, (float *) y, nullptr);
     if (rc) return rc;
     if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, o_bytes, hipMemcpyDeviceToHost));
-    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    else return wait_for_output();
     return ONHIP_OK;
 }
 
@@ -351,7 +359,7 @@ static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
 // an output on the host is computed into a staging buffer and copied back; one on the device is written in place
 static int finish_output(void *host_out, void *y, size_t bytes, bool out_on_dev) {
     if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, bytes, hipMemcpyDeviceToHost));
-    else ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    else return wait_for_output();
     return ONHIP_OK;
 }
 
@@ -654,6 +662,12 @@ int onhip_softmax_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO
 
 int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Transpose", transpose_eval_locked, params, inputs, outputs);
+}
+
+int onhip_plugin_set_async(int on) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_async = on != 0;
+    return ONHIP_OK;
 }
 
 int onhip_plugin_release(void) {

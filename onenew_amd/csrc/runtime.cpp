@@ -1,0 +1,634 @@
+// Device-resident execution of a .one model (include/onenew_rt.h): file reader, operator objects, execution
+// order, shape inference, buffers in HBM and the calls into the operator plugins.  Host code only; the
+// kernels live behind `eval` in lib<Op>_hip.so.
+//
+// Follows the reference host step by step (host/net.h, host/op.h, host/ops/*.h), with three deliberate
+// differences, all invisible to a batch-1 model the reference can run:
+//   * operand buffers and initialisers are device memory, carved out of two allocations made at load time
+//     (the reference makes one aligned_alloc per operand, host/net.h:434-449);
+//   * Conv and GlobalAveragePool keep the batch dimension of their input (the reference writes 1,
+//     host/ops/conv.h:43, host/ops/global_avgpool.h:33-36);
+//   * an initialiser goes to the slot with the index it has among the node's inputs (for every operator and
+//     operand order the reference host handles, this is the slot prepare_init_operand_data picks).
+#include <dlfcn.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <map>
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/onenew_abi.h"
+#include "../../include/onenew_rt.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define ONRT_HIP(expr)                                                                                     \
+    do {                                                                                                   \
+        hipError_t e_ = (expr);                                                                            \
+        if (e_ != hipSuccess) return fail(ONRT_ERR_RUNTIME, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+// common/utils_c.h:4-7
+inline size_t align64(size_t n) { return (n + 63) & ~(size_t) 63; }
+
+// bytes per element of the data types an initialiser may carry (ONNX numbering, common/nn_common.h:92-110)
+int elem_bytes(int32_t t) {
+    switch (t) {
+        case TYPE_FP32: case TYPE_INT32: return 4;
+        case TYPE_UINT8: case TYPE_INT8: return 1;
+        case TYPE_UINT16: case TYPE_INT16: case TYPE_FP16: case TYPE_BF16: return 2;
+        case TYPE_INT64: case TYPE_FP64: return 8;
+        default: return 0;
+    }
+}
+
+// common/utils_c.h:9-16: all SHAPE_LEN entries are multiplied, unused ones hold 1
+long long numel(const OPERAND_S &o) {
+    long long n = 1;
+    for (int i = 0; i < SHAPE_LEN; ++i) n *= o.shapes[i];
+    return n;
+}
+
+// the node types this runtime runs, with the size of their config struct (the reference keeps this table in
+// Manager::op_cfg_size_map, filled by OP_REGISTER_GLOBAL in each host/ops/*.h)
+struct OpKind {
+    const char *type;
+    size_t cfg_size;
+    bool view;   // no buffer of its own, no plugin call
+};
+const OpKind kOps[] = {
+    {"Conv", sizeof(CONV_CONFIG_S), false},
+    {"MatMul", sizeof(MATMUL_CONFIG_S), false},
+    {"Gemm", sizeof(GEMM_CONFIG_S), false},
+    {"Add", sizeof(ADD_CONFIG_S), false},
+    {"Relu", sizeof(RELU_CONFIG_S), false},
+    {"MaxPool", sizeof(MAX_POOL_CONFIG_S), false},
+    {"GlobalAveragePool", sizeof(GLOBAL_AVGPOOL_CONFIG_S), false},
+    {"Gelu", sizeof(GELU_CONFIG_S), false},
+    {"LayerNormalization", sizeof(LAYERNORMALIZATION_CONFIG_S), false},
+    {"Softmax", sizeof(SOFTMAX_CONFIG_S), false},
+    {"Transpose", sizeof(TRANSPOSE_CONFIG_S), false},
+    {"Flatten", sizeof(FLATTEN_CONFIG_S), true},
+    {"Reshape", sizeof(RESHAPE_CONFIG_S), true},
+};
+const OpKind *find_kind(const char *type) {
+    for (const OpKind &k : kOps)
+        if (!strcmp(k.type, type)) return &k;
+    return nullptr;
+}
+
+struct Tensor {
+    OPERAND_S desc;
+    void *dev = nullptr;
+    size_t bytes = 0;
+    bool is_init = false;
+    bool produced = false;   // an io input, an initialiser or the output of an operator already ordered
+};
+
+struct Node {
+    const OpKind *kind = nullptr;
+    std::vector<char> cfg;   // the node's config struct, as in the file
+    std::vector<std::string> in, out;
+    onenew_eval_fn eval = nullptr;
+    BUFFER_INFO_S params[BUF_MAXNUM], inputs[BUF_MAXNUM], outputs[BUF_MAXNUM];
+    const BASE_CONFIG_S *base() const { return reinterpret_cast<const BASE_CONFIG_S *>(cfg.data()); }
+};
+
+typedef int (*set_async_fn)(int);
+
+}  // namespace
+
+struct onrt_net {
+    std::vector<char> file;
+    std::vector<Node> nodes;
+    std::vector<int> order;
+    std::map<std::string, Tensor> tensors;   // operand_stu_map and operand_buf_map of the reference in one
+    std::vector<std::string> in_names, out_names;
+    USEFUL_INFO_S useful;
+    std::string lib_dir;
+    std::map<std::string, void *> handles;
+    std::vector<set_async_fn> async_switches;
+    void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
+    std::vector<float> silu_lut, gelu_lut;
+};
+
+namespace {
+
+const ONE_MODEL_DESC_S *header(const onrt_net &n) { return reinterpret_cast<const ONE_MODEL_DESC_S *>(n.file.data()); }
+
+// ---- reading the file (host/net.h:138-221) ------------------------------------------------------------
+int read_model(onrt_net &net) {
+    const size_t size = net.file.size();
+    if (size < sizeof(ONE_MODEL_DESC_S)) return fail(ONRT_ERR_FORMAT, "file of %zu bytes is shorter than the header", size);
+    const ONE_MODEL_DESC_S *h = header(net);
+    if (h->one_model_magic_num != ONE_MAGIC_NUM)
+        return fail(ONRT_ERR_FORMAT, "one_model_magic_num is 0x%x, a .one file starts with 0x%x", h->one_model_magic_num, ONE_MAGIC_NUM);
+    if (h->node_cnt < 0 || h->init_cnt < 0 || h->io_cfg_cnt < 0 || h->node_cfg_offset < 0 || h->init_info_offset < 0 ||
+        h->io_cfg_offset < 0)
+        return fail(ONRT_ERR_FORMAT, "negative count or offset in the header");
+    net.useful = h->useful_info;
+
+    // initialisers first: the operators look their inputs up among them
+    size_t off = (size_t) h->init_info_offset;
+    for (int i = 0; i < h->init_cnt; ++i) {
+        if (off + sizeof(OPERAND_S) > size) return fail(ONRT_ERR_FORMAT, "initialiser %d starts past the end of the file", i);
+        Tensor t;
+        memcpy(&t.desc, net.file.data() + off, sizeof(OPERAND_S));
+        t.desc.operand_name[OPERAND_NAME_LEN - 1] = 0;
+        const int eb = elem_bytes(t.desc.data_type);
+        const long long n = numel(t.desc);
+        if (!eb || n < 0 || n > (1LL << 40))
+            return fail(ONRT_ERR_FORMAT, "initialiser %s: data type %d / %lld elements", t.desc.operand_name, t.desc.data_type, n);
+        t.bytes = (size_t) n * eb;
+        if (off + sizeof(OPERAND_S) + t.bytes > size)
+            return fail(ONRT_ERR_FORMAT, "initialiser %s ends past the end of the file", t.desc.operand_name);
+        t.is_init = true;
+        t.produced = true;
+        t.desc.p_data = (int64_t) (off + sizeof(OPERAND_S));   // offset of the data in the file until uploaded
+        net.tensors[t.desc.operand_name] = t;
+        off += align64(sizeof(OPERAND_S) + t.bytes);
+    }
+
+    // io nodes (host/ops/io.h:56-70): "input" produces its operand, "output" names one to hand back
+    off = (size_t) h->io_cfg_offset;
+    for (int i = 0; i < h->io_cfg_cnt; ++i) {
+        if (off + sizeof(IO_CONFIG_S) > size) return fail(ONRT_ERR_FORMAT, "io config %d ends past the end of the file", i);
+        IO_CONFIG_S io;
+        memcpy(&io, net.file.data() + off, sizeof(io));
+        io.op_type[OP_TYPE_LEN - 1] = io.op_name[OP_NAME_LEN - 1] = io.operand.operand_name[OPERAND_NAME_LEN - 1] = 0;
+        if (strcmp(io.op_type, "io")) return fail(ONRT_ERR_FORMAT, "io config %d has op_type '%s'", i, io.op_type);
+        const std::string name(io.operand.operand_name);
+        if (!strcmp(io.op_name, "input")) {
+            if (io.operand.data_type != TYPE_FP32) return fail(ONRT_ERR_FORMAT, "input %s is not fp32", name.c_str());
+            Tensor t;
+            t.desc = io.operand;
+            t.produced = true;
+            net.tensors[name] = t;
+            net.in_names.push_back(name);
+        } else if (!strcmp(io.op_name, "output")) {
+            net.out_names.push_back(name);
+        } else {
+            return fail(ONRT_ERR_FORMAT, "io config %d is neither input nor output ('%s')", i, io.op_name);
+        }
+        off += align64(sizeof(IO_CONFIG_S));
+    }
+
+    // operator nodes
+    off = (size_t) h->node_cfg_offset;
+    for (int i = 0; i < h->node_cnt; ++i) {
+        if (off + sizeof(BASE_CONFIG_S) > size) return fail(ONRT_ERR_FORMAT, "node %d starts past the end of the file", i);
+        char type[OP_TYPE_LEN];
+        memcpy(type, net.file.data() + off, OP_TYPE_LEN);
+        type[OP_TYPE_LEN - 1] = 0;
+        const OpKind *kind = find_kind(type);
+        if (!kind) return fail(ONRT_ERR_FORMAT, "node %d: no HIP operator for type '%s'", i, type);
+        if (off + kind->cfg_size > size) return fail(ONRT_ERR_FORMAT, "node %d (%s) ends past the end of the file", i, type);
+        Node nd;
+        nd.kind = kind;
+        nd.cfg.assign(net.file.data() + off, net.file.data() + off + kind->cfg_size);
+        BASE_CONFIG_S *b = reinterpret_cast<BASE_CONFIG_S *>(nd.cfg.data());
+        b->op_name[OP_NAME_LEN - 1] = 0;
+        if (b->in_operand_num < 1 || b->in_operand_num > OPERAND_MAXNUM || b->out_operand_num < 1 || b->out_operand_num > OPERAND_MAXNUM)
+            return fail(ONRT_ERR_FORMAT, "node %s: %d inputs, %d outputs", b->op_name, b->in_operand_num, b->out_operand_num);
+        for (int k = 0; k < b->in_operand_num; ++k) {
+            b->in_operand_name[k][OPERAND_NAME_LEN - 1] = 0;
+            nd.in.push_back(b->in_operand_name[k]);
+        }
+        for (int k = 0; k < b->out_operand_num; ++k) {
+            b->out_operand_name[k][OPERAND_NAME_LEN - 1] = 0;
+            nd.out.push_back(b->out_operand_name[k]);
+        }
+        memset(nd.params, 0, sizeof(nd.params));
+        memset(nd.inputs, 0, sizeof(nd.inputs));
+        memset(nd.outputs, 0, sizeof(nd.outputs));
+        net.nodes.push_back(std::move(nd));
+        off += align64(kind->cfg_size);
+    }
+    return ONRT_OK;
+}
+
+// ---- execution order (host/net.h:274-330) -------------------------------------------------------------
+// A node is ready when every non-empty input is an initialiser, a net input or the output of a node already
+// placed; among ready nodes the first in file order goes next.
+int order_nodes(onrt_net &net) {
+    std::vector<bool> placed(net.nodes.size(), false);
+    for (size_t done = 0; done < net.nodes.size(); ++done) {
+        int pick = -1;
+        for (size_t i = 0; i < net.nodes.size() && pick < 0; ++i) {
+            if (placed[i]) continue;
+            bool ready = true;
+            for (const std::string &name : net.nodes[i].in) {
+                if (name.empty()) continue;
+                auto it = net.tensors.find(name);
+                if (it == net.tensors.end() || !it->second.produced) { ready = false; break; }
+            }
+            if (ready) pick = (int) i;
+        }
+        if (pick < 0) return fail(ONRT_ERR_FORMAT, "the graph has a cycle or an operand nobody produces (%zu of %zu nodes ordered)", done, net.nodes.size());
+        placed[pick] = true;
+        net.order.push_back(pick);
+        for (const std::string &name : net.nodes[pick].out) {
+            Tensor &t = net.tensors[name];
+            memset(&t.desc, 0, sizeof(t.desc));
+            snprintf(t.desc.operand_name, OPERAND_NAME_LEN, "%s", name.c_str());
+            t.desc.data_type = TYPE_FP32;
+            t.produced = true;
+        }
+    }
+    for (const std::string &name : net.out_names)
+        if (!net.tensors.count(name)) return fail(ONRT_ERR_FORMAT, "output %s is not produced by any node", name.c_str());
+    return ONRT_OK;
+}
+
+// ---- shape inference (shape_infer of each host/ops/*.h) -----------------------------------------------
+int infer_shapes(onrt_net &net) {
+    for (int idx : net.order) {
+        Node &nd = net.nodes[idx];
+        const char *type = nd.kind->type;
+        const Tensor &in0 = net.tensors[nd.in[0]];
+        const OPERAND_S &in = in0.desc;
+        OPERAND_S &out = net.tensors[nd.out[0]].desc;
+        auto init_at = [&](size_t k) -> const Tensor * {
+            if (k >= nd.in.size()) return nullptr;
+            auto it = net.tensors.find(nd.in[k]);
+            return it != net.tensors.end() && it->second.is_init ? &it->second : nullptr;
+        };
+        memcpy(out.shapes, in.shapes, sizeof(out.shapes));
+        out.dim_num_of_shapes = in.dim_num_of_shapes;
+        if (!strcmp(type, "Conv")) {   // host/ops/conv.h:31-58
+            const CONV_CONFIG_S *c = reinterpret_cast<const CONV_CONFIG_S *>(nd.cfg.data());
+            const Tensor *w = init_at(1);
+            if (!w) return fail(ONRT_ERR_FORMAT, "Conv %s: the weight is not an initialiser", nd.base()->op_name);
+            if (in.dim_num_of_shapes != 4) return fail(ONRT_ERR_FORMAT, "Conv %s: input of rank %d", nd.base()->op_name, in.dim_num_of_shapes);
+            if (c->has_bias && !init_at(2)) return fail(ONRT_ERR_FORMAT, "Conv %s: the bias is not an initialiser", nd.base()->op_name);
+            if (c->strides[0] < 1 || c->strides[1] < 1) return fail(ONRT_ERR_FORMAT, "Conv %s: stride below 1", nd.base()->op_name);
+            out.shapes[1] = w->desc.shapes[0];
+            out.shapes[2] = (int32_t) ((in.shapes[2] + c->pads[0] + c->pads[2] - c->kernel_shape[0]) / c->strides[0] + 1);
+            out.shapes[3] = (int32_t) ((in.shapes[3] + c->pads[1] + c->pads[3] - c->kernel_shape[1]) / c->strides[1] + 1);
+        } else if (!strcmp(type, "MaxPool")) {   // host/ops/maxpool.h:29-53
+            const MAX_POOL_CONFIG_S *c = reinterpret_cast<const MAX_POOL_CONFIG_S *>(nd.cfg.data());
+            if (c->strides[0] < 1 || c->strides[1] < 1) return fail(ONRT_ERR_FORMAT, "MaxPool %s: stride below 1", nd.base()->op_name);
+            out.shapes[2] = (int32_t) ((in.shapes[2] + c->pads[0] + c->pads[2] - c->kernel_shape[0]) / c->strides[0] + 1);
+            out.shapes[3] = (int32_t) ((in.shapes[3] + c->pads[1] + c->pads[3] - c->kernel_shape[1]) / c->strides[1] + 1);
+        } else if (!strcmp(type, "GlobalAveragePool")) {   // host/ops/global_avgpool.h:29-45
+            for (int i = 2; i < SHAPE_LEN; ++i) out.shapes[i] = 1;
+        } else if (!strcmp(type, "Gemm")) {   // host/ops/gemm.h:28-48: the last dimension becomes the bias length
+            const Tensor *b = init_at(2);
+            if (!init_at(1) || !b) return fail(ONRT_ERR_FORMAT, "Gemm %s: weight and bias must be initialisers", nd.base()->op_name);
+            out.shapes[out.dim_num_of_shapes - 1] = (int32_t) numel(b->desc);
+        } else if (!strcmp(type, "MatMul")) {   // host/ops/mat_mul.h:32-57
+            if (nd.in.size() < 2) return fail(ONRT_ERR_FORMAT, "MatMul %s: one input", nd.base()->op_name);
+            const OPERAND_S &b = net.tensors[nd.in[1]].desc;
+            out.shapes[out.dim_num_of_shapes - 1] = b.shapes[b.dim_num_of_shapes - 1];
+        } else if (!strcmp(type, "Add")) {   // host/ops/add.h:32-57
+            if (nd.in.size() < 2) return fail(ONRT_ERR_FORMAT, "Add %s: one input", nd.base()->op_name);
+            const Tensor &t1 = net.tensors[nd.in[1]];
+            if (in0.is_init) {
+                memcpy(out.shapes, t1.desc.shapes, sizeof(out.shapes));
+                out.dim_num_of_shapes = t1.desc.dim_num_of_shapes;
+            } else if (!t1.is_init && t1.desc.dim_num_of_shapes == in.dim_num_of_shapes) {
+                for (int i = 0; i < out.dim_num_of_shapes; ++i) out.shapes[i] = in.shapes[i] > t1.desc.shapes[i] ? in.shapes[i] : t1.desc.shapes[i];
+            }
+        } else if (!strcmp(type, "Transpose")) {   // host/ops/transpose.h:32-49
+            const TRANSPOSE_CONFIG_S *c = reinterpret_cast<const TRANSPOSE_CONFIG_S *>(nd.cfg.data());
+            if (c->perm_num < 0 || c->perm_num > SHAPE_LEN) return fail(ONRT_ERR_FORMAT, "Transpose %s: perm_num %lld", nd.base()->op_name, (long long) c->perm_num);
+            for (int i = 0; i < c->perm_num; ++i) {
+                if (c->perm[i] < 0 || c->perm[i] >= SHAPE_LEN) return fail(ONRT_ERR_FORMAT, "Transpose %s: perm[%d] = %lld", nd.base()->op_name, i, (long long) c->perm[i]);
+                out.shapes[i] = in.shapes[c->perm[i]];
+            }
+        } else if (!strcmp(type, "Flatten")) {   // host/ops/flatten.h:29-62
+            const FLATTEN_CONFIG_S *c = reinterpret_cast<const FLATTEN_CONFIG_S *>(nd.cfg.data());
+            if (c->axis < 0 || c->axis >= SHAPE_LEN) return fail(ONRT_ERR_FORMAT, "Flatten %s: axis %lld", nd.base()->op_name, (long long) c->axis);
+            out.not_need_buf = 1;
+            for (int i = 0; i < SHAPE_LEN; ++i) out.shapes[i] = 1;
+            for (int i = 0; i < c->axis; ++i) out.shapes[i] = in.shapes[i];
+            out.dim_num_of_shapes = (int32_t) c->axis + 1;
+            for (int i = (int) c->axis; i < SHAPE_LEN; ++i) out.shapes[c->axis] *= in.shapes[i];
+            if (in.dim_num_of_shapes == 3 && in.shapes[0] == 1 && c->axis == 2) {   // the reference's special case
+                out.shapes[0] = in.shapes[1];
+                out.shapes[1] = in.shapes[2];
+                out.shapes[2] = 1;
+                out.dim_num_of_shapes = 2;
+            }
+        } else if (!strcmp(type, "Reshape")) {   // host/ops/reshape.h:31-70
+            const RESHAPE_CONFIG_S *c = reinterpret_cast<const RESHAPE_CONFIG_S *>(nd.cfg.data());
+            if (c->dst_shape_num < 1 || c->dst_shape_num > SHAPE_LEN) return fail(ONRT_ERR_FORMAT, "Reshape %s: dst_shape_num %lld", nd.base()->op_name, (long long) c->dst_shape_num);
+            out.not_need_buf = 1;
+            const long long total = numel(in);
+            long long known = 1;
+            for (int i = 0; i < SHAPE_LEN; ++i) out.shapes[i] = 1;
+            for (int i = 0; i < c->dst_shape_num; ++i) {
+                out.shapes[i] = (int32_t) c->dst_shape[i];
+                if (c->dst_shape[i] != -1) known *= c->dst_shape[i];
+            }
+            for (int i = 0; i < c->dst_shape_num; ++i)
+                if (out.shapes[i] == -1) out.shapes[i] = known ? (int32_t) (total / known) : 0;
+            out.dim_num_of_shapes = (int32_t) c->dst_shape_num;
+            if (numel(out) != total) return fail(ONRT_ERR_FORMAT, "Reshape %s changes the element count (%lld to %lld)", nd.base()->op_name, total, numel(out));
+        }
+        // Relu, Gelu, LayerNormalization, Softmax: the input's shape
+        const long long n = numel(out);
+        if (n <= 0 || n >= (1LL << 31)) return fail(ONRT_ERR_FORMAT, "%s %s: output of %lld elements", type, nd.base()->op_name, n);
+    }
+    return ONRT_OK;
+}
+
+// ---- buffers (host/net.h:419-452) ---------------------------------------------------------------------
+int allocate(onrt_net &net) {
+    // initialisers: one allocation, uploaded once
+    size_t init_total = 0, act_total = 0;
+    for (auto &kv : net.tensors)
+        if (kv.second.is_init) init_total += (kv.second.bytes + 255) & ~(size_t) 255;
+    if (init_total) {
+        ONRT_HIP(hipMalloc(&net.init_arena, init_total));
+        size_t off = 0;
+        for (auto &kv : net.tensors) {
+            Tensor &t = kv.second;
+            if (!t.is_init) continue;
+            t.dev = static_cast<char *>(net.init_arena) + off;
+            if (t.bytes) ONRT_HIP(hipMemcpy(t.dev, net.file.data() + (size_t) t.desc.p_data, t.bytes, hipMemcpyHostToDevice));
+            t.desc.p_data = 0;
+            off += (t.bytes + 255) & ~(size_t) 255;
+        }
+    }
+    // operands: fp32 elements (elem_size * sizeof(float) in the reference), views excepted
+    for (auto &kv : net.tensors) {
+        Tensor &t = kv.second;
+        if (t.is_init || t.desc.not_need_buf) continue;
+        t.bytes = (size_t) numel(t.desc) * 4;
+        act_total += (t.bytes + 255) & ~(size_t) 255;
+    }
+    if (act_total) {
+        ONRT_HIP(hipMalloc(&net.act_arena, act_total));
+        size_t off = 0;
+        for (auto &kv : net.tensors) {
+            Tensor &t = kv.second;
+            if (t.is_init || t.desc.not_need_buf) continue;
+            t.dev = static_cast<char *>(net.act_arena) + off;
+            off += (t.bytes + 255) & ~(size_t) 255;
+        }
+    }
+    // a view shares the buffer of its input (host/op.h:149-154), in execution order so that chains resolve
+    for (int idx : net.order) {
+        const Node &nd = net.nodes[idx];
+        if (!nd.kind->view) continue;
+        const Tensor &src = net.tensors[nd.in[0]];
+        Tensor &dst = net.tensors[nd.out[0]];
+        dst.dev = src.dev;
+        dst.bytes = src.bytes;
+    }
+    return ONRT_OK;
+}
+
+// ---- activation tables (host/ops/conv.h:178-194, host/ops/gelu.h:80-96), built with the host's libm like
+// the reference host does, then kept on the device
+int build_tables(onrt_net &net) {
+    bool need_silu = false, need_gelu = false;
+    for (const Node &nd : net.nodes) {
+        if (!strcmp(nd.kind->type, "Conv") && reinterpret_cast<const CONV_CONFIG_S *>(nd.cfg.data())->act_type == SILU) need_silu = true;
+        if (!strcmp(nd.kind->type, "Gelu")) need_gelu = true;
+    }
+    if (!need_silu && !need_gelu) return ONRT_OK;
+    const float single_limit = 8.0f;
+    const float step = 1.0 / 512;
+    const int32_t lut_len = (int32_t) (2.0f * single_limit / step);
+    net.silu_lut.resize(lut_len);
+    net.gelu_lut.resize(lut_len);
+    const float inv_sqrt2 = 1.0f / 1.4142f;
+    for (int i = 0; i < lut_len; ++i) {
+        const float x = i * step - single_limit;
+        net.silu_lut[i] = x / (1 + expf(-x));
+        net.gelu_lut[i] = x * 0.5 * (1 + erf(x * inv_sqrt2));
+    }
+    ONRT_HIP(hipMalloc(&net.tables, 2 * (size_t) lut_len * 4));
+    ONRT_HIP(hipMemcpy(net.tables, net.silu_lut.data(), (size_t) lut_len * 4, hipMemcpyHostToDevice));
+    ONRT_HIP(hipMemcpy(static_cast<float *>(net.tables) + lut_len, net.gelu_lut.data(), (size_t) lut_len * 4, hipMemcpyHostToDevice));
+    return ONRT_OK;
+}
+
+// ---- plugins (host/op.h:41-80) ------------------------------------------------------------------------
+std::string own_directory() {
+    Dl_info info;
+    if (dladdr(reinterpret_cast<void *>(&own_directory), &info) && info.dli_fname) {
+        std::string p(info.dli_fname);
+        const size_t slash = p.rfind('/');
+        return slash == std::string::npos ? std::string(".") : p.substr(0, slash);
+    }
+    return ".";
+}
+
+int bind_plugins(onrt_net &net) {
+    for (Node &nd : net.nodes) {
+        if (nd.kind->view) continue;
+        const std::string type(nd.kind->type);
+        auto it = net.handles.find(type);
+        if (it == net.handles.end()) {
+            const std::string nested = net.lib_dir + "/" + type + "/lib" + type + "_hip.so";
+            const std::string flat = net.lib_dir + "/lib" + type + "_hip.so";
+            void *h = dlopen(nested.c_str(), RTLD_LAZY | RTLD_LOCAL);
+            if (!h) h = dlopen(flat.c_str(), RTLD_LAZY | RTLD_LOCAL);
+            if (!h) return fail(ONRT_ERR_PLUGIN, "the handle of %s op is not found: tried %s and %s (%s)", type.c_str(), nested.c_str(), flat.c_str(), dlerror());
+            it = net.handles.emplace(type, h).first;
+            // our plugins can leave a device-resident output to stream order instead of waiting for it
+            if (set_async_fn f = reinterpret_cast<set_async_fn>(dlsym(h, "onhip_plugin_set_async"))) net.async_switches.push_back(f);
+        }
+        nd.eval = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval"));
+        if (!nd.eval) return fail(ONRT_ERR_PLUGIN, "no eval in the %s plugin", type.c_str());
+    }
+    return ONRT_OK;
+}
+
+// ---- slot arrays (op::rt_prepare, host/op.h:109-168, and prepare_init_operand_data of each operator) ----
+int fill_slots(onrt_net &net) {
+    const size_t lut_len = net.silu_lut.size();
+    for (int idx : net.order) {
+        Node &nd = net.nodes[idx];
+        if (nd.kind->view) continue;
+        nd.params[0].addr = (int64_t) nd.cfg.data();
+        int act_slot = 0;   // activations are packed from slot 0 in input order (host/op.h:118-147) ...
+        for (size_t k = 0; k < nd.in.size(); ++k) {
+            if (nd.in[k].empty()) continue;
+            Tensor &t = net.tensors[nd.in[k]];
+            // ... and an initialiser sits at its own input index
+            const int slot = t.is_init ? (int) k : act_slot++;
+            if (1 + slot >= BUF_MAXNUM - 1) return fail(ONRT_ERR_FORMAT, "%s: too many inputs", nd.base()->op_name);
+            nd.params[1 + slot].addr = (int64_t) &t.desc;
+            nd.inputs[slot].addr = (int64_t) t.dev;
+        }
+        int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
+        for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
+            Tensor &t = net.tensors[nd.out[k]];
+            if (out_slot >= BUF_MAXNUM - 1) return fail(ONRT_ERR_FORMAT, "%s: too many operands", nd.base()->op_name);
+            nd.params[out_slot].addr = (int64_t) &t.desc;
+            nd.outputs[k].addr = (int64_t) t.dev;
+        }
+        // per-model tunables in the last params slot (host/ops/conv.h:66-69, host/ops/maxpool.h:57-62); the
+        // HIP operators bring their own workspace, so the shared scratch buffer stays unallocated
+        nd.params[BUF_MAXNUM - 1].addr = (int64_t) &net.useful;
+        if (!strcmp(nd.kind->type, "Conv") && reinterpret_cast<const CONV_CONFIG_S *>(nd.cfg.data())->act_type == SILU)
+            nd.inputs[BUF_MAXNUM - 1].addr = (int64_t) net.tables;
+        if (!strcmp(nd.kind->type, "Gelu")) nd.inputs[BUF_MAXNUM - 1].addr = (int64_t) (static_cast<float *>(net.tables) + lut_len);
+    }
+    return ONRT_OK;
+}
+
+int prepare(onrt_net &net, const char *op_lib_dir) {
+    if (op_lib_dir && *op_lib_dir) net.lib_dir = op_lib_dir;
+    else if (const char *env = getenv("ONENEW_OP_LIB_DIR")) net.lib_dir = env;
+    else net.lib_dir = own_directory();
+    int rc = read_model(net);
+    if (!rc) rc = order_nodes(net);
+    if (!rc) rc = infer_shapes(net);
+    if (!rc) rc = bind_plugins(net);
+    if (!rc) rc = allocate(net);
+    if (!rc) rc = build_tables(net);
+    if (!rc) rc = fill_slots(net);
+    net.useful.public_buf_info.public_buf_ptr = 0;
+    net.useful.public_buf_info.public_buf_size = 0;
+    return rc;
+}
+
+void set_async(onrt_net &net, int on) {
+    for (set_async_fn f : net.async_switches) f(on);
+}
+
+}  // namespace
+
+#define ONRT_API __attribute__((visibility("default")))
+
+extern "C" {
+
+ONRT_API const char *onrt_last_error(void) { return g_err; }
+
+ONRT_API int onrt_net_load_buf(const void *one_buf, size_t bytes, const char *op_lib_dir, onrt_net_t **out) {
+    if (!one_buf || !out) return fail(ONRT_ERR_ARG, "load: null argument");
+    *out = nullptr;
+    std::unique_ptr<onrt_net> net(new onrt_net);
+    net->file.assign(static_cast<const char *>(one_buf), static_cast<const char *>(one_buf) + bytes);
+    const int rc = prepare(*net, op_lib_dir);
+    if (rc) {
+        onrt_net_free(net.release());
+        return rc;
+    }
+    *out = net.release();
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_load_file(const char *one_path, const char *op_lib_dir, onrt_net_t **out) {
+    if (!one_path || !out) return fail(ONRT_ERR_ARG, "load: null argument");
+    FILE *f = fopen(one_path, "rb");
+    if (!f) return fail(ONRT_ERR_FORMAT, "can't open the one file %s", one_path);
+    std::vector<char> buf;
+    char chunk[1 << 16];
+    size_t got;
+    while ((got = fread(chunk, 1, sizeof(chunk), f)) > 0) buf.insert(buf.end(), chunk, chunk + got);
+    fclose(f);
+    return onrt_net_load_buf(buf.data(), buf.size(), op_lib_dir, out);
+}
+
+ONRT_API void onrt_net_free(onrt_net_t *net) {
+    if (!net) return;
+    (void) hipDeviceSynchronize();
+    if (net->init_arena) (void) hipFree(net->init_arena);
+    if (net->act_arena) (void) hipFree(net->act_arena);
+    if (net->tables) (void) hipFree(net->tables);
+    // plugin libraries stay loaded: they keep process-wide state (packed weights, staging buffers)
+    delete net;
+}
+
+ONRT_API int onrt_net_io_count(const onrt_net_t *net, int32_t *n_inputs, int32_t *n_outputs) {
+    if (!net) return fail(ONRT_ERR_ARG, "null net");
+    if (n_inputs) *n_inputs = (int32_t) net->in_names.size();
+    if (n_outputs) *n_outputs = (int32_t) net->out_names.size();
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, const char **name, int32_t *ndim, int32_t shape[8]) {
+    if (!net) return fail(ONRT_ERR_ARG, "null net");
+    const std::vector<std::string> &names = is_output ? net->out_names : net->in_names;
+    if (idx < 0 || idx >= (int32_t) names.size()) return fail(ONRT_ERR_ARG, "%s index %d of %zu", is_output ? "output" : "input", idx, names.size());
+    if (name) *name = names[idx].c_str();
+    return onrt_net_operand(net, names[idx].c_str(), ndim, shape, nullptr);
+}
+
+ONRT_API int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops) {
+    if (!net || !n_ops) return fail(ONRT_ERR_ARG, "null argument");
+    *n_ops = (int32_t) net->order.size();
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_op_info(const onrt_net_t *net, int32_t idx, const char **op_type, const char **op_name) {
+    if (!net) return fail(ONRT_ERR_ARG, "null net");
+    if (idx < 0 || idx >= (int32_t) net->order.size()) return fail(ONRT_ERR_ARG, "operator index %d of %zu", idx, net->order.size());
+    const Node &nd = net->nodes[net->order[idx]];
+    if (op_type) *op_type = nd.kind->type;
+    if (op_name) *op_name = nd.base()->op_name;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_operand(const onrt_net_t *net, const char *name, int32_t *ndim, int32_t shape[8], void **dev_ptr) {
+    if (!net || !name) return fail(ONRT_ERR_ARG, "null argument");
+    auto it = net->tensors.find(name);
+    if (it == net->tensors.end()) return fail(ONRT_ERR_ARG, "no operand named %s", name);
+    if (ndim) *ndim = it->second.desc.dim_num_of_shapes;
+    if (shape) memcpy(shape, it->second.desc.shapes, sizeof(int32_t) * SHAPE_LEN);
+    if (dev_ptr) *dev_ptr = it->second.dev;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs) {
+    if (!net || (!inputs && !net->in_names.empty()) || (!outputs && !net->out_names.empty())) return fail(ONRT_ERR_ARG, "run: null argument");
+    for (size_t i = 0; i < net->in_names.size(); ++i) {
+        if (!inputs[i]) return fail(ONRT_ERR_ARG, "run: input %zu is null", i);
+        const Tensor &t = net->tensors[net->in_names[i]];
+        if (inputs[i] != t.dev) ONRT_HIP(hipMemcpy(t.dev, inputs[i], t.bytes, hipMemcpyDefault));
+    }
+    set_async(*net, 1);
+    int rc = ONRT_OK;
+    for (int idx : net->order) {
+        Node &nd = net->nodes[idx];
+        if (nd.kind->view) continue;
+        const int r = nd.eval(nd.params, nd.inputs, nd.outputs);
+        if (r) {
+            rc = fail(ONRT_ERR_PLUGIN, "%s %s: eval returned %d", nd.kind->type, nd.base()->op_name, r);
+            break;
+        }
+    }
+    set_async(*net, 0);
+    if (rc) {
+        (void) hipDeviceSynchronize();
+        return rc;
+    }
+    bool copied = false;
+    for (size_t i = 0; i < net->out_names.size(); ++i) {
+        if (!outputs[i]) continue;
+        const Tensor &t = net->tensors[net->out_names[i]];
+        if (outputs[i] != t.dev) {
+            ONRT_HIP(hipMemcpy(outputs[i], t.dev, t.bytes, hipMemcpyDefault));
+            copied = true;
+        }
+    }
+    // a blocking copy has already waited for the operators; otherwise wait here: results are complete on return
+    if (!copied) ONRT_HIP(hipStreamSynchronize(nullptr));
+    return ONRT_OK;
+}
+
+}  // extern "C"

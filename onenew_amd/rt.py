@@ -1,0 +1,134 @@
+"""ctypes binding of the device-resident model runtime (include/onenew_rt.h, libonenew_rt.so)."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import hip
+
+EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
+           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run"]
+
+_lib = None
+
+
+class OnrtError(RuntimeError):
+    pass
+
+
+def lib_path():
+    return os.path.join(os.path.dirname(hip.lib_path()), "libonenew_rt.so")
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise OnrtError(f"{path} is missing: build it with `python -m onenew_amd.build`")
+    L = C.CDLL(path)
+    vp, i32p = C.c_void_p, C.POINTER(C.c_int32)
+    L.onrt_last_error.restype = C.c_char_p
+    L.onrt_net_load_file.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(vp)]
+    L.onrt_net_load_buf.argtypes = [C.c_char_p, C.c_size_t, C.c_char_p, C.POINTER(vp)]
+    L.onrt_net_free.argtypes = [vp]
+    L.onrt_net_free.restype = None
+    L.onrt_net_io_count.argtypes = [vp, i32p, i32p]
+    L.onrt_net_io_info.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(C.c_char_p), i32p, i32p]
+    L.onrt_net_op_count.argtypes = [vp, i32p]
+    L.onrt_net_op_info.argtypes = [vp, C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
+    L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
+    L.onrt_net_run.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
+    _lib = L
+    return L
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise OnrtError(f"{what} failed ({rc}): {load().onrt_last_error().decode(errors='replace')}")
+
+
+class Net:
+    """A loaded model.  ``model`` is a path or the bytes of a .one file; ``op_lib_dir`` defaults to the directory
+    of the built plugins."""
+
+    def __init__(self, model, op_lib_dir=None):
+        L = load()
+        self._h = C.c_void_p()
+        d = (op_lib_dir or os.path.dirname(lib_path())).encode()
+        if isinstance(model, (bytes, bytearray, memoryview)):
+            data = bytes(model)
+            _check(L.onrt_net_load_buf(data, len(data), d, C.byref(self._h)), "onrt_net_load_buf")
+        else:
+            _check(L.onrt_net_load_file(os.fspath(model).encode(), d, C.byref(self._h)), "onrt_net_load_file")
+        ni, no = C.c_int32(), C.c_int32()
+        _check(L.onrt_net_io_count(self._h, C.byref(ni), C.byref(no)), "onrt_net_io_count")
+        self.inputs = [self._io(0, i) for i in range(ni.value)]
+        self.outputs = [self._io(1, i) for i in range(no.value)]
+
+    def _io(self, is_output, idx):
+        name, nd, shape = C.c_char_p(), C.c_int32(), (C.c_int32 * 8)()
+        _check(load().onrt_net_io_info(self._h, is_output, idx, C.byref(name), C.byref(nd), shape), "onrt_net_io_info")
+        return name.value.decode(), tuple(shape[i] for i in range(nd.value))
+
+    def ops(self):
+        """(type, name) of every operator in execution order"""
+        L, n = load(), C.c_int32()
+        _check(L.onrt_net_op_count(self._h, C.byref(n)), "onrt_net_op_count")
+        out = []
+        for i in range(n.value):
+            t, nm = C.c_char_p(), C.c_char_p()
+            _check(L.onrt_net_op_info(self._h, i, C.byref(t), C.byref(nm)), "onrt_net_op_info")
+            out.append((t.value.decode(), nm.value.decode()))
+        return out
+
+    def operand(self, name):
+        """(shape, device address) of an operand"""
+        nd, shape, ptr = C.c_int32(), (C.c_int32 * 8)(), C.c_void_p()
+        _check(load().onrt_net_operand(self._h, name.encode(), C.byref(nd), shape, C.byref(ptr)), "onrt_net_operand")
+        return tuple(shape[i] for i in range(nd.value)), ptr.value
+
+    def fetch(self, name):
+        """host copy of an operand's current contents (fp32)"""
+        shape, ptr = self.operand(name)
+        n = int(np.prod(shape)) if shape else 1
+        out = np.empty(n, dtype=np.float32)
+        rt = C.CDLL("libamdhip64.so")
+        rt.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        rc = rt.hipMemcpy(out.ctypes.data, ptr, out.nbytes, 2)   # blocking device-to-host copy
+        if rc != 0:
+            raise OnrtError(f"hipMemcpy of operand {name} failed ({rc})")
+        return out.reshape(shape)
+
+    def run_raw(self, in_ptrs, out_ptrs):
+        """addresses (host or device) in input / output order; 0 / None among the outputs skips that copy"""
+        vp = C.c_void_p
+        ins = (vp * max(1, len(in_ptrs)))(*[vp(p) for p in in_ptrs])
+        outs = (vp * max(1, len(out_ptrs)))(*[vp(p or 0) for p in out_ptrs])
+        _check(load().onrt_net_run(self._h, ins, outs), "onrt_net_run")
+
+    def run(self, *arrays):
+        """numpy inputs in input order -> list of numpy outputs"""
+        if len(arrays) != len(self.inputs):
+            raise OnrtError(f"the net has {len(self.inputs)} inputs, {len(arrays)} given")
+        ins = []
+        for a, (name, shape) in zip(arrays, self.inputs):
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            if a.size != int(np.prod(shape)):
+                raise OnrtError(f"input {name} has shape {shape}, got {a.shape}")
+            ins.append(a)
+        outs = [np.empty(shape, dtype=np.float32) for _, shape in self.outputs]
+        self.run_raw([a.ctypes.data for a in ins], [o.ctypes.data for o in outs])
+        return outs
+
+    def close(self):
+        if self._h:
+            load().onrt_net_free(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,78 @@
+"""Small .one models for the runtime tests: every operator of the package, initialisers in each position the
+reference host handles, views, two inputs and two outputs.  Weights and inputs are seeded."""
+import numpy as np
+
+from onenew_amd import abi, onefile, datagen
+
+
+def _r(tag, shape, scale=1.0):
+    return (datagen.normal(datagen.seed_for("one_models", tag), shape, 0.0, 1.0) * np.float32(scale)).astype(np.float32)
+
+
+def resnet_block():
+    """conv+relu, conv, residual add, relu, maxpool, strided 1x1, global pool, flatten, gemm"""
+    m = onefile.OneModel()
+    m.input("x", (1, 16, 20, 20))
+    m.conv("c1", "x", _r("c1w", (16, 16, 3, 3), 0.08), _r("c1b", (16,), 0.1), "c1_out", pad=1, act=abi.RELU)
+    m.conv("c2", "c1_out", _r("c2w", (16, 16, 3, 3), 0.08), _r("c2b", (16,), 0.1), "c2_out", pad=1)
+    m.add("res", "c2_out", "x", "res_out")
+    m.relu("relu", "res_out", "relu_out")
+    m.maxpool("pool", "relu_out", "pool_out", 3, 2, 1)
+    m.conv("down", "pool_out", _r("dw", (40, 16, 1, 1), 0.2), None, "down_out", stride=2)
+    m.global_avgpool("gap", "down_out", "gap_out")
+    m.flatten("flat", "gap_out", "flat_out", axis=1)
+    m.gemm("fc", "flat_out", _r("fcw", (10, 40), 0.15), _r("fcb", (10,), 0.1), "logits")
+    m.output("logits", (1, 10))
+    return m.tobytes(), [_r("x", (1, 16, 20, 20))]
+
+
+def mobile_block():
+    """pointwise + CLIP, depthwise + CLIP, pointwise, SiLU conv: the fused activations and group != 1"""
+    m = onefile.OneModel()
+    m.input("x", (1, 8, 14, 14))
+    m.conv("expand", "x", _r("ew", (24, 8, 1, 1), 0.3), _r("eb", (24,), 0.1), "e", act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("dw", "e", _r("dww", (24, 1, 3, 3), 0.3), _r("dwb", (24,), 0.1), "d", stride=2, pad=1, group=24,
+           act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("project", "d", _r("pw", (12, 24, 1, 1), 0.2), _r("pb", (12,), 0.1), "p")
+    m.conv("silu", "p", _r("sw", (12, 12, 3, 3), 0.1), _r("sb", (12,), 0.1), "out", pad=1, act=abi.SILU)
+    m.output("out", (1, 12, 7, 7))
+    return m.tobytes(), [_r("xm", (1, 8, 14, 14))]
+
+
+def vit_block():
+    """layer norm, projection with a weight initialiser and a bias Add, table GELU, residual, then a token-mixing
+    pair of MatMuls over two activations with Transpose and Softmax, and a Reshape view"""
+    t, c = 17, 32
+    m = onefile.OneModel()
+    m.input("x", (1, t, c))
+    m.layernorm("ln1", "x", 1.0 + _r("g", (c,), 0.1), _r("b", (c,), 0.1), "ln1_out")
+    m.matmul("fc1", "ln1_out", _r("w1", (c, 64), 0.2), "fc1_out")
+    m.add("fc1_bias", "fc1_out", _r("b1", (64,), 0.1), "fc1_b")
+    m.gelu("gelu", "fc1_b", "gelu_out")
+    m.matmul("fc2", "gelu_out", _r("w2", (64, c), 0.2), "fc2_out")
+    m.add("fc2_bias", "fc2_out", _r("b2", (c,), 0.1), "fc2_b")
+    m.add("res", "fc2_b", "x", "h")
+    m.reshape("heads", "h", "h4", (1, 1, t, c))
+    m.transpose("kt", "h4", "h4_t", (0, 1, 3, 2))
+    m.matmul("scores", "h4", "h4_t", "scores_out")
+    m.softmax("attn", "scores_out", "attn_out")
+    m.matmul("ctx", "attn_out", "h4", "ctx_out")
+    m.output("ctx_out", (1, 1, t, c))
+    m.output("h", (1, t, c))
+    return m.tobytes(), [_r("xv", (1, t, c))]
+
+
+def two_inputs():
+    """two net inputs, an Add of them, a channel Softmax (axis 1) and an axis-1 layer norm"""
+    m = onefile.OneModel()
+    m.input("a", (1, 6, 5, 5))
+    m.input("b", (1, 6, 5, 5))
+    m.add("sum", "a", "b", "s")
+    m.softmax("sm", "s", "sm_out", axis=1)
+    m.output("sm_out", (1, 6, 5, 5))
+    m.relu("r", "s", "r_out")
+    m.output("r_out", (1, 6, 5, 5))
+    return m.tobytes(), [_r("a", (1, 6, 5, 5)), _r("b", (1, 6, 5, 5))]
+
+
+MODELS = {"resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
