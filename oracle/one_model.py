@@ -14,8 +14,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
-sys.path.insert(0, HERE)
-import oracle  # noqa: E402
+from oracle import oracle  # noqa: E402
 from onenew_amd import abi, onefile  # noqa: E402
 from onenew_amd.abi import ConvDesc  # noqa: E402
 

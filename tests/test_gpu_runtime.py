@@ -12,8 +12,8 @@ import numpy as np
 import pytest
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(os.path.dirname(HERE), "oracle"))
-import one_model  # noqa: E402
+sys.path.insert(0, os.path.dirname(HERE))
+from oracle import one_model  # noqa: E402
 import one_models  # noqa: E402
 from onenew_amd import hip, onefile, rt  # noqa: E402
 

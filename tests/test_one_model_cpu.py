@@ -11,8 +11,8 @@ import pytest
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-sys.path.insert(0, os.path.join(ROOT, "oracle"))
-import one_model  # noqa: E402
+sys.path.insert(0, ROOT)
+from oracle import one_model  # noqa: E402
 import one_models  # noqa: E402
 from onenew_amd import abi, onefile, rt  # noqa: E402
 
