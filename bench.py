@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
 Workloads (BASELINE configurations): resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
-cfg1, mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
+cfg1, resnet50_net_b{1,32} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
 the HBM traffic counters are scaled by).
 
 A step is one pass over every layer of the workload: one launch per layer, inputs, weights and outputs
@@ -451,6 +451,60 @@ def cpu_baseline(layers, tag, unit, budget_s=12.0):
             "ms_per_pass": round(med * 1e3, 2), "host_cpus": os.cpu_count()}
 
 
+def bench_net(torch, args):
+    """Whole ResNet-50 as a .one model through the device-resident runtime (libonenew_rt.so): every operator of the
+    graph (53 Conv, MaxPool, 16 Add, 16 Relu, GlobalAveragePool, Gemm) back to back on the device, input and
+    output in device memory.  A step is one inference of the batch."""
+    from onenew_amd import rt, stacks
+    n = int(args.workload.split("_b")[1])
+    data, in_shape, flops = stacks.resnet50_model(n)
+    net = rt.Net(data)
+    x = torch.randn(in_shape, dtype=torch.float32, device="cuda")
+    y = torch.empty((n, 1000), dtype=torch.float32, device="cuda")
+    ins, outs = [x.data_ptr()], [y.data_ptr()]
+    for _ in range(max(2, args.warmup)):     # the first inferences measure tile choices and pack the weights
+        net.run_raw(ins, outs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.run_raw(ins, outs)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    # device time of one inference: events around it on the default stream, where the plugins launch
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    dev_ms = []
+    for _ in range(max(5, args.steps)):
+        e0.record(torch.cuda.default_stream())
+        net.run_raw(ins, outs)
+        e1.record(torch.cuda.default_stream())
+        e1.synchronize()
+        dev_ms.append(e0.elapsed_time(e1))
+    dev = float(np.median(dev_ms))
+    ops = net.ops()
+    cpu = None
+    if not args.no_cpu:
+        from oracle import one_model
+        if one_model.have_ref_runner():
+            data1, shape1, flops1 = stacks.resnet50_model(1)
+            xin = np.random.default_rng(0).normal(size=shape1).astype(np.float32)
+            ms = one_model.time_reference(data1, [xin], repeats=40)
+            cpu = {"value": round(flops1 / (ms * 1e-3) / 1e12, 5), "unit": "TFLOP/s", "cores": 8, "kind": "reference",
+                   "sample": f"40 inferences of the same model at batch 1 through the reference's host operator classes "
+                             f"and x86 kernels, median {ms:.2f} ms", "ms_per_inference": round(ms, 3)}
+    line = {"metric": "resnet50_net_fp32_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"ResNet-50 .one model fp32, batch {n}, 224x224, {len(ops)} operators through the "
+                                   f"device-resident runtime, input and logits in HBM", "operators": len(ops),
+                       "ops_per_step": flops, "model_bytes": len(data)},
+            "roofline": {"kernel": "whole inference: every operator of the graph on the default stream", "bound": "mfma",
+                         "achieved": round(flops / (dev * 1e-3) / 1e12, 3), "peak": PEAK["f32"], "unit": "TFLOP/s",
+                         "frac": round(flops / (dev * 1e-3) / 1e12 / PEAK["f32"], 4), "traffic": None,
+                         "launches": len(ops), "device_ms_per_inference": round(dev, 4)},
+            "cpu_baseline": cpu, "images_per_s": round(n / (ms_per_step * 1e-3), 1)}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -483,6 +537,9 @@ def main():
         print(json.dumps({"workload": "copy", "bytes_read_per_launch": src.numel() * 4,
                           "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
         return
+
+    if args.workload.startswith("resnet50_net_b"):
+        return bench_net(torch, args)
 
     desc, dtype, layers = make_workload(torch, hip, args.workload)
     unit = "TOP/s" if dtype == "i8" else "TFLOP/s"

@@ -118,3 +118,51 @@ def with_batch(layers, n):
         e.n = n
         out.append((name, e))
     return out
+
+
+def resnet50_model(batch=1, classes=1000, tag="resnet50_model"):
+    """The whole ResNet-50 as a .one file, in the form the offline optimiser leaves it: batch norm folded into the
+    convolutions, ReLU fused into stem / conv1 / conv2 (33 of the 53), the residual Add and its ReLU as nodes of
+    their own, MaxPool 3x3 s2 after the stem, GlobalAveragePool, Flatten, Gemm.  Seeded He-scaled weights.
+    Returns (bytes, input shape, multiply-accumulates x 2 per inference)."""
+    import numpy as np
+    from . import datagen, onefile
+
+    def weights(name, shape, fan_in):
+        return datagen.normal(datagen.seed_for(tag, name), shape, 0.0, float(np.sqrt(2.0 / fan_in)))
+
+    m = onefile.OneModel()
+    flops = 0
+
+    def cv(name, x, cin, cout, k, s, p, hw, act, gain=1.0):
+        nonlocal flops
+        out_hw = (hw + 2 * p - k) // s + 1
+        flops += 2 * batch * cout * out_hw * out_hw * cin * k * k
+        w = weights(name + ".w", (cout, cin, k, k), cin * k * k) * gain   # the residual branch is damped: no batch norm here
+        b = datagen.normal(datagen.seed_for(tag, name + ".b"), (cout,), 0.0, 0.01)
+        return m.conv(name, x, w, b, name + "_out", stride=s, pad=p, act=act)
+
+    x = m.input("input", (batch, 3, 224, 224))
+    x = cv("stem", x, 3, 64, 7, 2, 3, 224, RELU)
+    x = m.maxpool("maxpool", x, "maxpool_out", 3, 2, 1)
+    inplanes, hw = 64, 56
+    for li, (planes, blocks, stride) in enumerate([(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)], 1):
+        for b in range(blocks):
+            s = stride if b == 0 else 1
+            p = f"l{li}.{b}"
+            y = cv(p + ".conv1", x, inplanes, planes, 1, 1, 0, hw, RELU)
+            y = cv(p + ".conv2", y, planes, planes, 3, s, 1, hw, RELU)
+            skip = cv(p + ".down", x, inplanes, planes * 4, 1, s, 0, hw, NOT_ACT) if b == 0 else x
+            hw //= s
+            y = cv(p + ".conv3", y, planes, planes * 4, 1, 1, 0, hw, NOT_ACT, gain=0.3)
+            y = m.add(p + ".add", y, skip, p + ".add_out")
+            x = m.relu(p + ".relu", y, p + ".relu_out")
+            inplanes = planes * 4
+    x = m.global_avgpool("avgpool", x, "avgpool_out")
+    x = m.flatten("flatten", x, "flatten_out", axis=1)
+    flops += 2 * batch * classes * inplanes
+    x = m.gemm("fc", x, weights("fc.w", (classes, inplanes), inplanes) * 0.5,
+               datagen.normal(datagen.seed_for(tag, "fc.b"), (classes,), 0.0, 0.01), "logits")
+    m.output("logits", (batch, classes))
+    return m.tobytes(), (batch, 3, 224, 224), flops
+

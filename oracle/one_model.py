@@ -92,6 +92,24 @@ def have_ref_runner():
     return os.path.exists(REF_RUNNER) and os.path.isdir(REF_OPS)
 
 
+def time_reference(one_bytes, inputs, repeats, threads=8):
+    """median milliseconds of one inference through the reference's operator classes and x86 kernels"""
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "m.one")
+        with open(path, "wb") as f:
+            f.write(one_bytes)
+        files = []
+        for i, a in enumerate(inputs):
+            files.append(os.path.join(tmp, f"in{i}.bin"))
+            np.ascontiguousarray(a, dtype=np.float32).tofile(files[-1])
+        env = dict(os.environ, ONENEW_REF_OP_DIR=REF_OPS, REF_REPEAT=str(repeats), OMP_NUM_THREADS=str(threads))
+        out = subprocess.run([REF_RUNNER, path, tmp] + files, check=True, env=env, capture_output=True, text=True).stdout
+        for line in out.splitlines():
+            if line.startswith("forward_ms"):
+                return float(line.split()[1])
+    raise RuntimeError("the reference runner printed no timing")
+
+
 def run_reference(one_bytes, inputs):
     """The same model through the reference's operator classes and x86 kernels (CPU).  Returns
     [(name, array)] for the outputs in io order."""

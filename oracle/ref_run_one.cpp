@@ -8,7 +8,8 @@
 //
 //   ref_run_one model.one out_dir input0.bin [input1.bin ...]     raw fp32 inputs in io order
 // writes out_dir/<n>.bin for output number n, and out_dir/shapes.txt with "<name> <ndim> <dims...>" per output;
-// REF_DUMP_ALL=1 also writes every operand as out_dir/op_<index>.bin with its name in shapes.txt.
+// REF_DUMP_ALL=1 also writes every operand as out_dir/op_<index>.bin with its name in shapes.txt;
+// REF_REPEAT=n times n further inferences and prints "forward_ms <median>".
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -16,6 +17,8 @@
 #include <vector>
 #include <set>
 #include <unordered_map>
+#include <algorithm>
+#include <omp.h>
 
 #include "io.h"
 #include "conv.h"
@@ -150,6 +153,17 @@ int main(int argc, char **argv) {
     }
     for (auto &o : order) o->rt_prepare(bufs, stu, init_list);
     for (auto &o : order) o->forward(bufs, stu, init_list);
+    // REF_REPEAT=n: n more inferences, the median time of one goes to stdout (the CPU baseline of the benchmark)
+    if (const char *rep = getenv("REF_REPEAT")) {
+        std::vector<double> ms;
+        for (int r = 0; r < atoi(rep); ++r) {
+            const double t0 = omp_get_wtime();
+            for (auto &o : order) o->forward(bufs, stu, init_list);
+            ms.push_back((omp_get_wtime() - t0) * 1e3);
+        }
+        std::sort(ms.begin(), ms.end());
+        if (!ms.empty()) printf("forward_ms %.4f\n", ms[ms.size() / 2]);
+    }
 
     const std::string dir(argv[2]);
     FILE *fs = fopen((dir + "/shapes.txt").c_str(), "w");
