@@ -8,6 +8,7 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <vector>
@@ -102,7 +103,9 @@ static const int kNumTiles = 4;
 static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
 static const int kNumSplits = 10;
 
-struct Choice { int bm, bn, split; };
+// tail > 1: the column blocks left over after whole rounds of 256 tiles run as a second launch, split `tail` ways
+// along K, next to the first one (launch_choice)
+struct Choice { int bm, bn, split, tail; };
 
 static std::mutex g_tune_mu;
 static int g_tune_mode = -1;   // -1: read ONHIP_TUNE on first use; 0 model only; 1 measure
@@ -138,8 +141,8 @@ static void load_tune_cache_locked() {
             key.push_back(v);
             s = end;
         }
-        Choice c;
-        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d", &c.bm, &c.bn, &c.split) == 3) g_tuned[key] = c;
+        Choice c = {0, 0, 1, 0};
+        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail) >= 3) g_tuned[key] = c;
     }
     fclose(f);
 }
@@ -149,7 +152,7 @@ static void append_tune_cache_locked(const std::vector<long long> &key, const Ch
     FILE *f = fopen(path, "a");
     if (!f) return;
     for (long long v : key) fprintf(f, "%lld ", v);
-    fprintf(f, ": %d %d %d\n", c.bm, c.bn, c.split);
+    fprintf(f, ": %d %d %d %d\n", c.bm, c.bn, c.split, c.tail);
     fclose(f);
 }
 
@@ -176,7 +179,7 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
         const int split = (k_tiles + tiles_per - 1) / tiles_per;
         if (split > 1) {
             void *buf = nullptr;
-            const size_t bytes = (size_t) split * cfg.batch * p.M * p.N * 4;
+            const size_t bytes = (size_t) split * cfg.batch * p.M * (p.N - p.n_begin) * 4;
             int rc = get_scratch(bytes, &buf);
             if (rc) return rc;
             cfg.split = split;
@@ -187,8 +190,32 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
     return ONHIP_OK;
 }
 
+// Tile quantisation.  All workgroups of these launches are resident at once, so the CUs that hold one workgroup more
+// than the others set the duration: 784 tiles on 256 CUs take as long as 1024.  When few tiles are left over after
+// whole rounds of 256, the launch is cut along N: the first dp_cols column blocks (a whole number of rounds) run as
+// they are, the rest runs as a second launch split along K so that it, too, puts about one small workgroup on every CU.
+// The two launches share the machine (caller's stream and a side stream of the library, joined by events).
+static bool tail_geometry(const IgemmLaunch &cfg, const IgemmParams &p, int bm, int bn, int *dp_cols, int *tail_tiles) {
+    if (cfg.batch != 1 || cfg.dtype == DT_I8 || p.n_begin != 0) return false;
+    const int tiles_m = (p.M + bm - 1) / bm, cols = (p.N + bn - 1) / bn;
+    const long long tiles = (long long) tiles_m * cols;
+    const int rounds = (int) (tiles / 256);
+    if (rounds < 1) return false;
+    const int dpc = rounds * 256 / tiles_m;
+    if (dpc < 1 || dpc >= cols) return false;
+    const int left = (cols - dpc) * tiles_m;
+    if (left > 128) return false;   // more than half a round left over: nothing to gain
+    *dp_cols = dpc;
+    *tail_tiles = left;
+    return true;
+}
+
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
+    if (c.tail > 1) {
+        int dpc, left;
+        return c.split == 1 && k_tiles >= 2 * c.tail && tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left);
+    }
     if (c.split > 1 && (k_tiles < 2 * c.split)) return false;
     if (c.split > 1 && (size_t) c.split * cfg.batch * p.M * p.N * 4 > ((size_t) 256 << 20)) return false;
     return true;
@@ -214,11 +241,11 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
 }
 
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
-    Choice best = {64, 64, 1};
+    Choice best = {64, 64, 1, 0};
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t)
         for (int s = 0; s < kNumSplits; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s]};
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0};
             if (!candidate_ok(cfg, p, c)) continue;
             const double cost = model_cost(cfg, p, c);
             if (cost < best_cost) { best_cost = cost; best = c; }
@@ -226,17 +253,77 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     return best;
 }
 
+// the side stream of the tail launches and a ring of event pairs to fork from and join the caller's stream
+static std::mutex g_side_mu;
+static hipStream_t g_side = nullptr;
+static const int kSideEvents = 32;
+static hipEvent_t g_fork[kSideEvents], g_join[kSideEvents];
+static int g_side_next = 0;
+static std::atomic<long long> g_tail_launches{0};
+
+static int side_stream(hipStream_t *side, hipEvent_t *fork, hipEvent_t *join) {
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    if (!g_side) {
+        hipStream_t s = nullptr;
+        ONHIP_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));   // default priority
+        for (int i = 0; i < kSideEvents; ++i) {
+            ONHIP_CHECK_HIP(hipEventCreateWithFlags(&g_fork[i], hipEventDisableTiming));
+            ONHIP_CHECK_HIP(hipEventCreateWithFlags(&g_join[i], hipEventDisableTiming));
+        }
+        g_side = s;
+    }
+    *side = g_side;
+    *fork = g_fork[g_side_next];
+    *join = g_join[g_side_next];
+    g_side_next = (g_side_next + 1) % kSideEvents;
+    return ONHIP_OK;
+}
+
+// Runs the problem the way the choice says.
+static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
+    int dpc = 0, left = 0;
+    if (c.tail <= 1 || !tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
+        const Choice plain = {c.bm, c.bn, c.split, 0};
+        int rc = apply_choice(cfg, p, plain);
+        return rc ? rc : igemm_launch(cfg, p, st);
+    }
+    // whole rounds: columns [0, dpc * bn), unsplit, on the caller's stream
+    IgemmLaunch cfg_dp = cfg, cfg_tail = cfg;
+    IgemmParams p_dp = p, p_tail = p;
+    p_dp.N = dpc * c.bn;
+    const Choice dp = {c.bm, c.bn, 1, 0}, tail = {c.bm, c.bn, c.tail, 0};
+    int rc = apply_choice(cfg_dp, p_dp, dp);
+    if (rc) return rc;
+    // the rest: columns [dpc * bn, N), split along K, on the side stream between a fork and a join
+    p_tail.n_begin = dpc * c.bn;
+    rc = apply_choice(cfg_tail, p_tail, tail);
+    if (rc) return rc;
+    hipStream_t side;
+    hipEvent_t fork, join;
+    rc = side_stream(&side, &fork, &join);
+    if (rc) return rc;
+    g_tail_launches.fetch_add(1, std::memory_order_relaxed);
+    ONHIP_CHECK_HIP(hipEventRecord(fork, st));
+    ONHIP_CHECK_HIP(hipStreamWaitEvent(side, fork, 0));
+    rc = igemm_launch(cfg_dp, p_dp, st);
+    if (!rc) rc = igemm_launch(cfg_tail, p_tail, side);
+    // join even after a failed launch, so the two streams never stay tied to a half-issued pair
+    hipError_t e1 = hipEventRecord(join, side);
+    hipError_t e2 = e1 == hipSuccess ? hipStreamWaitEvent(st, join, 0) : e1;
+    if (rc) return rc;
+    ONHIP_CHECK_HIP(e2);
+    return ONHIP_OK;
+}
+
 static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st, hipEvent_t e0, hipEvent_t e1,
                        float *best_ms) {
-    int rc = apply_choice(cfg, p, c);
-    if (rc) return rc;
-    rc = igemm_launch(cfg, p, st);   // warm-up
+    int rc = launch_choice(cfg, p, c, st);   // warm-up
     if (rc) return rc;
     float best = 1e30f;
     for (int rep = 0; rep < 2; ++rep) {
         ONHIP_CHECK_HIP(hipEventRecord(e0, st));
         for (int i = 0; i < 3; ++i) {
-            rc = igemm_launch(cfg, p, st);
+            rc = launch_choice(cfg, p, c, st);
             if (rc) return rc;
         }
         ONHIP_CHECK_HIP(hipEventRecord(e1, st));
@@ -249,25 +336,32 @@ static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStrea
     return ONHIP_OK;
 }
 
-// Chooses tile and split for the problem and makes p / cfg ready to launch.
-static int plan_launch(IgemmLaunch &cfg, IgemmParams &p, hipStream_t st) {
-    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT]
-        Choice c = {0, 0, 1};
-        if (sscanf(env, "%dx%dx%d", &c.bm, &c.bn, &c.split) >= 2) return apply_choice(cfg, p, c);
+// Chooses tile, split and tail handling for the problem and launches it.
+static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t st) {
+    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL]]
+        Choice c = {0, 0, 1, 0};
+        if (sscanf(env, "%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail) >= 2) {
+            if (c.tail > 1 && !candidate_ok(cfg, p, c)) c.tail = 0;   // no leftover to split on this shape
+            return launch_choice(cfg, p, c, st);
+        }
     }
-    if (!tune_mode()) return apply_choice(cfg, p, model_choice(cfg, p));
+    if (!tune_mode()) return launch_choice(cfg, p, model_choice(cfg, p), st);
     std::vector<long long> key = {cfg.dtype, cfg.bl, cfg.batch, p.M, p.N, p.K, p.k_units, p.khkw, p.sh, p.sw,
                                   p.H, p.W, p.out_mode, p.lda};
     {
-        std::lock_guard<std::mutex> lock(g_tune_mu);
+        std::unique_lock<std::mutex> lock(g_tune_mu);
         load_tune_cache_locked();
         auto it = g_tuned.find(key);
-        if (it != g_tuned.end()) return apply_choice(cfg, p, it->second);
+        if (it != g_tuned.end()) {
+            const Choice c = it->second;
+            lock.unlock();
+            return launch_choice(cfg, p, c, st);
+        }
     }
     // measure: the candidates the model ranks within 2.5x of its best, on the caller's stream
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone)
-        return apply_choice(cfg, p, model_choice(cfg, p));
+        return launch_choice(cfg, p, model_choice(cfg, p), st);
     const Choice guess = model_choice(cfg, p);
     const double guess_cost = model_cost(cfg, p, guess);
     hipEvent_t e0, e1;
@@ -276,27 +370,41 @@ static int plan_launch(IgemmLaunch &cfg, IgemmParams &p, hipStream_t st) {
     Choice best = guess;
     float best_ms = 1e30f;
     int rc = ONHIP_OK;
-    for (int t = 0; t < kNumTiles && !rc; ++t)
+    auto try_choice = [&](const Choice &c) {
+        float ms = 0.f;
+        rc = time_choice(cfg, p, c, st, e0, e1, &ms);
+        if (!rc && ms < best_ms) { best_ms = ms; best = c; }
+    };
+    for (int t = 0; t < kNumTiles && !rc; ++t) {
         for (int s = 0; s < kNumSplits && !rc; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s]};
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0};
             if (!candidate_ok(cfg, p, c) || model_cost(cfg, p, c) > 2.5 * guess_cost) continue;
-            float ms = 0.f;
-            rc = time_choice(cfg, p, c, st, e0, e1, &ms);
-            if (!rc && ms < best_ms) { best_ms = ms; best = c; }
+            try_choice(c);
         }
+        // the leftover column blocks as a K-split launch of about one workgroup per CU, and half as many
+        int dpc = 0, left = 0;
+        if (!rc && tail_geometry(cfg, p, kTiles[t][0], kTiles[t][1], &dpc, &left)) {
+            int want = 256 / left;
+            want = want > 16 ? 16 : want;
+            for (int ts = want; ts >= 2 && ts >= want / 2 && !rc; ts /= 2) {
+                const Choice c = {kTiles[t][0], kTiles[t][1], 1, ts};
+                if (candidate_ok(cfg, p, c) && model_cost(cfg, p, {c.bm, c.bn, 1, 0}) <= 2.5 * guess_cost) try_choice(c);
+            }
+        }
+    }
     (void) hipEventDestroy(e0);
     (void) hipEventDestroy(e1);
     if (rc) return rc;
     if (getenv("ONHIP_TUNE_VERBOSE"))
-        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d (%.4f ms; model said %dx%d split %d)\n",
-                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best_ms, guess.bm, guess.bn,
-                guess.split);
+        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d (%.4f ms; model said %dx%d split %d)\n",
+                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best_ms, guess.bm,
+                guess.bn, guess.split);
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
         g_tuned[key] = best;
         append_tune_cache_locked(key, best);
     }
-    return apply_choice(cfg, p, best);
+    return launch_choice(cfg, p, best, st);
 }
 
 static int dtype_of_compute(int compute, int *dt) {
@@ -334,6 +442,8 @@ int onhip_set_tuning(int mode) {
     g_tune_mode = mode > 0 ? 1 : 0;
     return prev;
 }
+
+long long onhip_split_tail_launches(void) { return g_tail_launches.load(std::memory_order_relaxed); }
 
 int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow) {
     if (!oh || !ow) return set_error(ONHIP_ERR_ARG, "conv: null output pointer");
@@ -425,9 +535,7 @@ static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const flo
     p.bias = bias;
     p.bias_mode = d->has_bias ? BIAS_M : BIAS_NONE;
     p.ep = ep;
-    rc = plan_launch(cfg, p, st);
-    if (rc) return rc;
-    return igemm_launch(cfg, p, st);
+    return plan_and_launch(cfg, p, st);
 }
 
 int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,
@@ -580,9 +688,7 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     p.acc_out = acc32;
     p.out_s8 = d->out_s8;
     p.out_inv_scale = d->out_s8 ? 1.0f / d->output_scale : 0.0f;
-    rc = plan_launch(cfg, p, st);
-    if (rc) return rc;
-    return igemm_launch(cfg, p, st);
+    return plan_and_launch(cfg, p, st);
 }
 
 int onhip_conv2d_w8a32(const onhip_conv_desc_t *d, const float *x, const int8_t *w8, const int32_t *bias32,
@@ -656,9 +762,7 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     p.ep.act = gelu_lut ? ONHIP_ACT_GELU_LUT : NOT_ACT;
     p.ep.lut = gelu_lut;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    rc = plan_launch(cfg, p, st);
-    if (rc) return rc;
-    return igemm_launch(cfg, p, st);
+    return plan_and_launch(cfg, p, st);
 }
 
 int onhip_copy_f32(const float *src, float *dst, long long n, void *stream) {

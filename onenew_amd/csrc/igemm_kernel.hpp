@@ -477,12 +477,13 @@ __device__ __forceinline__ unsigned to_bits(int v) { return (unsigned) v; }
 template <int TM, int TN, class ACC>
 __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[TM][TN], int slice, int m_wave,
                                               int n_wave, int li, int lh) {
-    const rsrc_t rp = make_rsrc(reinterpret_cast<const char *>(p.partial) + (size_t) slice * p.M * p.N * 4, RSRC_RANGE);
+    const int width = p.N - p.n_begin;   // partial sums cover the launch's own columns
+    const rsrc_t rp = make_rsrc(reinterpret_cast<const char *>(p.partial) + (size_t) slice * p.M * width * 4, RSRC_RANGE);
     const bool m_edge = m_wave + TM * 32 > p.M;
 #pragma unroll
     for (int b = 0; b < TN; ++b) {
         const int n = n_wave + b * 32 + li;
-        const unsigned cv = n < p.N ? (unsigned) (n + 4 * lh * p.N) * 4u : OOB;
+        const unsigned cv = n < p.N ? (unsigned) (n - p.n_begin + 4 * lh * width) * 4u : OOB;
 #pragma unroll
         for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -491,7 +492,7 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
                 const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
                 const auto val = acc[a][b][r];   // element copy first: bit-casting the vector element in place miscompiles
                 __builtin_amdgcn_raw_buffer_store_b32(to_bits(val), rp, row_ok ? cv : OOB,
-                                                      (unsigned) m_uni * (unsigned) p.N * 4u, 0);
+                                                      (unsigned) m_uni * (unsigned) width * 4u, 0);
             }
     }
 }
@@ -538,7 +539,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
     }
     const int tile_n = (int) div31((unsigned) lid, p.div_tiles_m), tile_m = lid - tile_n * tiles_m;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = p.n_begin + tile_n * BN;   // a launch may cover the columns [n_begin, N) only
     const int batch = blockIdx.z;
     const int u_begin = blockIdx.y * p.k_split_units;
     const int u_end = min(p.k_units, u_begin + p.k_split_units);
@@ -820,11 +821,12 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 // so no index has to be divided
 template <bool IS_INT>
 __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p, int split, int batches) {
-    const int n = blockIdx.x * 64 + threadIdx.x;
+    const int n = p.n_begin + blockIdx.x * 64 + threadIdx.x;
     const int m = blockIdx.y * 4 + threadIdx.y, batch = blockIdx.z;
     if (n >= p.N || m >= p.M) return;
-    const size_t slice = (size_t) batches * p.M * p.N;                    // elements per K slice
-    const size_t idx = ((size_t) batch * p.M + m) * p.N + n;
+    const int width = p.N - p.n_begin;
+    const size_t slice = (size_t) batches * p.M * width;                  // elements per K slice
+    const size_t idx = ((size_t) batch * p.M + m) * width + (n - p.n_begin);
     const size_t off4 = (size_t) batch * p.c_batch_stride + (size_t) m * p.c_stride_m + out_col_offset(p, n, 1);
     char *cbase = reinterpret_cast<char *>(p.C);
     if constexpr (IS_INT) {
@@ -850,7 +852,7 @@ template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1>
 static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream_t stream) {
     IgemmParams p = p_in;
     const int tiles_m = (p.M + BM - 1) / BM;
-    const int tiles = tiles_m * ((p.N + BN - 1) / BN);
+    const int tiles = tiles_m * ((p.N - p.n_begin + BN - 1) / BN);
     p.div_ohw = make_div31((unsigned) (p.OHW > 0 ? p.OHW : 1));
     p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
     p.div_tiles_m = make_div31((unsigned) tiles_m);
@@ -860,7 +862,7 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     if (p.partial) {
         if (p.M > 4 * 65535 || cfg.batch > 65535)
             return set_error(ONHIP_ERR_ARG, "igemm: split-K with %d rows, %d batches", p.M, cfg.batch);
-        const dim3 fgrid((p.N + 63) / 64, (p.M + 3) / 4, cfg.batch);
+        const dim3 fgrid((p.N - p.n_begin + 63) / 64, (p.M + 3) / 4, cfg.batch);
         if (DT == DT_I8)
             hipLaunchKernelGGL((splitk_finish_kernel<true>), fgrid, dim3(64, 4), 0, stream, p, cfg.split, cfg.batch);
         else

@@ -129,6 +129,7 @@ struct IgemmParams {
     int M, N, K;              // K counts real reduction elements (gather) or padded units*kpu (kvec)
     int k_units;               // 16-byte units along K (multiple of 2 per MFMA step is NOT required)
     int k_split_units;         // units handled by one blockIdx.y slice (split-K); == k_units if unsplit
+    int n_begin;               // first column of this launch (0 unless the columns are shared out between two launches)
     // A
     const void *A;
     long long a_batch_stride;  // elements; 0 = shared

@@ -29,7 +29,7 @@ def plugin_path(op):
     return os.path.join(LIBDIR, f"lib{op}_hip.so")
 
 
-EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_conv_out_shape", "onhip_conv2d_f32",
+EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
            "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quantize_nhwc_s8",
@@ -51,6 +51,7 @@ def load():
     if not os.path.exists(path):
         raise OnhipError(f"{path} is missing: build it with `python -m onenew_amd.build`")
     L = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    L.onhip_split_tail_launches.restype = C.c_longlong
     vp = C.c_void_p
     L.onhip_init.argtypes = [C.c_int]
     L.onhip_last_error.restype = C.c_char_p
@@ -362,3 +363,9 @@ def copy_f32(src, dst):
     """plain device copy (the yardstick for HBM traffic counters)"""
     _check(load().onhip_copy_f32(_ptr(src), _ptr(dst), src.numel(), _stream()), "onhip_copy_f32")
     return dst
+
+
+def split_tail_launches():
+    """launches so far whose leftover column blocks ran as a second, K-split launch"""
+    return int(load().onhip_split_tail_launches())
+

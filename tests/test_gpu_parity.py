@@ -193,6 +193,47 @@ def test_forced_tile_and_split_many_items(tile, kind, torch_dev, oracle, monkeyp
         assert_close_f32(y.cpu().numpy(), ref, tag=f"{kind} {tile} run {rep}")
 
 
+@pytest.mark.parametrize("tile,shape", [("64x64x1x8", (20, 30, 29)), ("64x64x1x16", (17, 32, 32)), ("64x128x1x4", (34, 32, 34)),
+                                        ("32x128x1x8", (33, 32, 33)), ("128x128x1x2", (80, 24, 36))])
+@pytest.mark.parametrize("kind", ["3x3_packed", "1x1", "matmul"])
+def test_leftover_tiles_as_a_split_launch(tile, shape, kind, torch_dev, oracle, monkeypatch):
+    """the launch cut along N: whole rounds of 256 tiles unsplit on the caller's stream, the leftover column blocks
+    split along K on the side stream, joined by events.  Shapes with more than 256 tiles, a ragged last column
+    block and (100 output channels) a ragged last row block; run three times, interleaved with an ordinary launch
+    on the same stream that reads the result"""
+    torch = torch_dev
+    n, h, w_ = shape
+    monkeypatch.setenv("ONHIP_TILE", tile)
+    if kind == "matmul":
+        rng = np.random.default_rng(7)
+        a = (rng.normal(size=(100, 528)) * 0.05).astype(np.float32)          # 100 rows, as many columns as the conv has pixels
+        b = rng.normal(size=(528, n * h * w_)).astype(np.float32)
+        ref = oracle.matmul_f32(a, b)
+        before = hip.split_tail_launches()
+        for rep in range(2):
+            y = hip.matmul(dev(torch, a), dev(torch, b))
+            torch.cuda.synchronize()
+            assert_close_f32(y.cpu().numpy(), ref, tag=f"matmul {tile} run {rep}")
+        assert hip.split_tail_launches() == before + 2
+        return
+    if kind == "3x3_packed":
+        d = cases.cd(64, 100, 3, 1, 1, h, w_, n=n, act=abi.RELU)              # K = 576: 36 K tiles, enough for 16 slices
+    else:
+        d = cases.cd(520, 100, 1, 1, 0, h, w_, n=n, act=abi.CLIP, clip_min=-0.4, clip_max=0.9)
+    x, w, b = cases.conv_inputs(f"tail_{kind}_{tile}", d)
+    ref = oracle.conv2d_f32(d, x, w, b, cases.silu_lut())
+    xd, wd, bd = dev(torch, x), dev(torch, w), dev(torch, b)
+    wp = hip.pack_conv_weights(d, wd) if kind == "3x3_packed" else None
+    before = hip.split_tail_launches()
+    for rep in range(3):
+        y = hip.conv2d_f32(d, xd, wp, bd, packed=True) if wp is not None else hip.conv2d_f32(d, xd, wd, bd)
+        doubled = hip.add_f32(y, y)                                            # stream-ordered consumer of the result
+        torch.cuda.synchronize()
+        assert_close_f32(y.cpu().numpy(), ref, tag=f"{kind} {tile} run {rep}")
+        assert np.array_equal(doubled.cpu().numpy(), 2 * y.cpu().numpy())
+    assert hip.split_tail_launches() == before + 3                             # the shape does have leftover tiles
+
+
 @pytest.mark.parametrize("tile", ["64x64x4", "128x128x2", "32x128x1"])
 def test_forced_split_w8a32_bit_exact(tile, torch_dev, oracle, monkeypatch):
     """integer partial sums add up exactly whatever the split"""
