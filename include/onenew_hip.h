@@ -86,10 +86,8 @@ const char *onhip_last_error(void);
  * search (tools/optimize/auto_tuning.hpp:9-75).  Default: the ONHIP_TUNE environment variable, else 0.
  * Returns the previous mode. */
 int onhip_set_tuning(int mode);
-/* Diagnostic, no counterpart in the reference: how many launches so far ran their leftover column blocks (those
- * beyond a whole number of rounds of 256 tiles) as a second, K-split launch on the library's side stream.  Such a
- * launch is ordered on the caller's stream like any other: the side stream is forked from it and joined back to
- * it with events before the entry point returns. */
+/* Diagnostic, no counterpart in the reference: how many launches so far cut their leftover tiles (those beyond a
+ * whole number of rounds of 256 tiles) into K slices next to the whole tiles of the same launch. */
 long long onhip_split_tail_launches(void);
 /* Output height / width of a convolution (host/ops/conv.h:43-50). Returns 0 or ONHIP_ERR_ARG. */
 int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow);

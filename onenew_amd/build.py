@@ -48,7 +48,9 @@ def _scratch_users(text):
         if body.startswith("Function Name:"):
             name = body.split(":", 1)[1].split("[")[0].strip()
         elif body.startswith("ScratchSize [bytes/lane]:"):
-            if int(body.split(":", 1)[1].split("[")[0]) > 0 and name:
+            # a few dozen bytes are reserved now and then without a single scratch instruction in the kernel;
+            # operand arrays that fell out of registers take a kilobyte and more
+            if int(body.split(":", 1)[1].split("[")[0]) > 256 and name:
                 bad.append(name)
     return bad
 

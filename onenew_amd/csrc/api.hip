@@ -103,8 +103,7 @@ static const int kNumTiles = 4;
 static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
 static const int kNumSplits = 10;
 
-// tail > 1: the column blocks left over after whole rounds of 256 tiles run as a second launch, split `tail` ways
-// along K, next to the first one (launch_choice)
+// tail > 1: the tiles left over after whole rounds of 256 are cut `tail` ways along K (launch_choice)
 struct Choice { int bm, bn, split, tail; };
 
 static std::mutex g_tune_mu;
@@ -179,7 +178,7 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
         const int split = (k_tiles + tiles_per - 1) / tiles_per;
         if (split > 1) {
             void *buf = nullptr;
-            const size_t bytes = (size_t) split * cfg.batch * p.M * (p.N - p.n_begin) * 4;
+            const size_t bytes = (size_t) split * cfg.batch * p.M * (p.N - p.part_begin) * 4;
             int rc = get_scratch(bytes, &buf);
             if (rc) return rc;
             cfg.split = split;
@@ -192,11 +191,12 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
 
 // Tile quantisation.  All workgroups of these launches are resident at once, so the CUs that hold one workgroup more
 // than the others set the duration: 784 tiles on 256 CUs take as long as 1024.  When few tiles are left over after
-// whole rounds of 256, the launch is cut along N: the first dp_cols column blocks (a whole number of rounds) run as
-// they are, the rest runs as a second launch split along K so that it, too, puts about one small workgroup on every CU.
-// The two launches share the machine (caller's stream and a side stream of the library, joined by events).
+// whole rounds of 256, the launch treats its tiles in two ways: the first dp_cols column blocks (a whole number of
+// rounds) are whole tiles, each of the remaining tiles is cut along K into slices so that the leftover, too, puts about
+// one small workgroup on every CU.  (Running the leftover as a second launch on another stream was tried first: the
+// cross-queue event waits cost more than the balance gained.)
 static bool tail_geometry(const IgemmLaunch &cfg, const IgemmParams &p, int bm, int bn, int *dp_cols, int *tail_tiles) {
-    if (cfg.batch != 1 || cfg.dtype == DT_I8 || p.n_begin != 0) return false;
+    if (cfg.batch != 1 || cfg.dtype == DT_I8) return false;
     const int tiles_m = (p.M + bm - 1) / bm, cols = (p.N + bn - 1) / bn;
     const long long tiles = (long long) tiles_m * cols;
     const int rounds = (int) (tiles / 256);
@@ -253,66 +253,31 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     return best;
 }
 
-// the side stream of the tail launches and a ring of event pairs to fork from and join the caller's stream
-static std::mutex g_side_mu;
-static hipStream_t g_side = nullptr;
-static const int kSideEvents = 32;
-static hipEvent_t g_fork[kSideEvents], g_join[kSideEvents];
-static int g_side_next = 0;
 static std::atomic<long long> g_tail_launches{0};
-
-static int side_stream(hipStream_t *side, hipEvent_t *fork, hipEvent_t *join) {
-    std::lock_guard<std::mutex> lock(g_side_mu);
-    if (!g_side) {
-        hipStream_t s = nullptr;
-        ONHIP_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));   // default priority
-        for (int i = 0; i < kSideEvents; ++i) {
-            ONHIP_CHECK_HIP(hipEventCreateWithFlags(&g_fork[i], hipEventDisableTiming));
-            ONHIP_CHECK_HIP(hipEventCreateWithFlags(&g_join[i], hipEventDisableTiming));
-        }
-        g_side = s;
-    }
-    *side = g_side;
-    *fork = g_fork[g_side_next];
-    *join = g_join[g_side_next];
-    g_side_next = (g_side_next + 1) % kSideEvents;
-    return ONHIP_OK;
-}
 
 // Runs the problem the way the choice says.
 static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
     int dpc = 0, left = 0;
+    p.part_begin = p.dp_tiles = p.tail_tiles = 0;
     if (c.tail <= 1 || !tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
         const Choice plain = {c.bm, c.bn, c.split, 0};
         int rc = apply_choice(cfg, p, plain);
         return rc ? rc : igemm_launch(cfg, p, st);
     }
-    // whole rounds: columns [0, dpc * bn), unsplit, on the caller's stream
-    IgemmLaunch cfg_dp = cfg, cfg_tail = cfg;
-    IgemmParams p_dp = p, p_tail = p;
-    p_dp.N = dpc * c.bn;
-    const Choice dp = {c.bm, c.bn, 1, 0}, tail = {c.bm, c.bn, c.tail, 0};
-    int rc = apply_choice(cfg_dp, p_dp, dp);
+    // one launch: dpc column blocks as whole tiles, the rest in c.tail K slices each; partial sums and the
+    // finishing pass cover the columns from dpc * bn on only
+    p.part_begin = dpc * c.bn;
+    const Choice tail = {c.bm, c.bn, c.tail, 0};
+    int rc = apply_choice(cfg, p, tail);
     if (rc) return rc;
-    // the rest: columns [dpc * bn, N), split along K, on the side stream between a fork and a join
-    p_tail.n_begin = dpc * c.bn;
-    rc = apply_choice(cfg_tail, p_tail, tail);
-    if (rc) return rc;
-    hipStream_t side;
-    hipEvent_t fork, join;
-    rc = side_stream(&side, &fork, &join);
-    if (rc) return rc;
+    if (cfg.split <= 1) {
+        p.part_begin = 0;
+        return igemm_launch(cfg, p, st);
+    }
+    p.dp_tiles = dpc * ((p.M + c.bm - 1) / c.bm);
+    p.tail_tiles = left;
     g_tail_launches.fetch_add(1, std::memory_order_relaxed);
-    ONHIP_CHECK_HIP(hipEventRecord(fork, st));
-    ONHIP_CHECK_HIP(hipStreamWaitEvent(side, fork, 0));
-    rc = igemm_launch(cfg_dp, p_dp, st);
-    if (!rc) rc = igemm_launch(cfg_tail, p_tail, side);
-    // join even after a failed launch, so the two streams never stay tied to a half-issued pair
-    hipError_t e1 = hipEventRecord(join, side);
-    hipError_t e2 = e1 == hipSuccess ? hipStreamWaitEvent(st, join, 0) : e1;
-    if (rc) return rc;
-    ONHIP_CHECK_HIP(e2);
-    return ONHIP_OK;
+    return igemm_launch(cfg, p, st);
 }
 
 static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st, hipEvent_t e0, hipEvent_t e1,

@@ -477,13 +477,13 @@ __device__ __forceinline__ unsigned to_bits(int v) { return (unsigned) v; }
 template <int TM, int TN, class ACC>
 __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[TM][TN], int slice, int m_wave,
                                               int n_wave, int li, int lh) {
-    const int width = p.N - p.n_begin;   // partial sums cover the launch's own columns
+    const int width = p.N - p.part_begin;   // partial sums cover the columns from part_begin on
     const rsrc_t rp = make_rsrc(reinterpret_cast<const char *>(p.partial) + (size_t) slice * p.M * width * 4, RSRC_RANGE);
     const bool m_edge = m_wave + TM * 32 > p.M;
 #pragma unroll
     for (int b = 0; b < TN; ++b) {
         const int n = n_wave + b * 32 + li;
-        const unsigned cv = n < p.N ? (unsigned) (n - p.n_begin + 4 * lh * width) * 4u : OOB;
+        const unsigned cv = n < p.N ? (unsigned) (n - p.part_begin + 4 * lh * width) * 4u : OOB;
 #pragma unroll
         for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -532,17 +532,29 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     // XCD-aware tile order: consecutive workgroup ids go round-robin over the 8 XCDs (each with its
     // own L2); give every XCD a contiguous run of tiles so neighbours in (m, n) share an L2.
     const int tiles_m = (p.M + BM - 1) / BM;
-    int lid;
+    // A launch with dp_tiles > 0 has two kinds of workgroups: the first dp_tiles take one whole tile each (all of K,
+    // result written directly), the others take one of `split` K slices of one of the tail_tiles tiles left over and
+    // write partial sums.  Slices of one tile are tail_tiles workgroup ids apart, so they land on different CUs.
+    int lid, slice = blockIdx.y;
+    bool whole_k = false;
     {
-        const int nb = gridDim.x, bid = blockIdx.x;
-        const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
-        lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+        const int bid = blockIdx.x;
+        if (p.dp_tiles > 0 && bid >= p.dp_tiles) {
+            const int r = bid - p.dp_tiles;
+            slice = r / p.tail_tiles;
+            lid = p.dp_tiles + (r - slice * p.tail_tiles);
+        } else {
+            const int nb = p.dp_tiles > 0 ? p.dp_tiles : (int) gridDim.x;
+            const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
+            lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+            whole_k = p.dp_tiles > 0;
+        }
     }
     const int tile_n = (int) div31((unsigned) lid, p.div_tiles_m), tile_m = lid - tile_n * tiles_m;
-    const int m0 = tile_m * BM, n0 = p.n_begin + tile_n * BN;   // a launch may cover the columns [n_begin, N) only
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int batch = blockIdx.z;
-    const int u_begin = blockIdx.y * p.k_split_units;
-    const int u_end = min(p.k_units, u_begin + p.k_split_units);
+    const int u_begin = whole_k ? 0 : slice * p.k_split_units;
+    const int u_end = whole_k ? p.k_units : min(p.k_units, u_begin + p.k_split_units);
     const int k_tiles = (u_end - u_begin + UPT - 1) / UPT;
     const int klim = min(p.K, u_end * KPU);
 
@@ -783,8 +795,8 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     if (kt < k_tiles) group(kt, CHECKED, std::true_type{});
 
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
-    if (p.partial) {
-        write_partial<TM, TN>(p, acc, blockIdx.y * gridDim.z + batch, m_wave, n_wave, li, lh);
+    if (p.partial && !whole_k) {
+        write_partial<TM, TN>(p, acc, slice * gridDim.z + batch, m_wave, n_wave, li, lh);
         return;
     }
     if constexpr (DT == DT_I8) {
@@ -821,12 +833,12 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 // so no index has to be divided
 template <bool IS_INT>
 __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p, int split, int batches) {
-    const int n = p.n_begin + blockIdx.x * 64 + threadIdx.x;
+    const int n = p.part_begin + blockIdx.x * 64 + threadIdx.x;
     const int m = blockIdx.y * 4 + threadIdx.y, batch = blockIdx.z;
     if (n >= p.N || m >= p.M) return;
-    const int width = p.N - p.n_begin;
+    const int width = p.N - p.part_begin;
     const size_t slice = (size_t) batches * p.M * width;                  // elements per K slice
-    const size_t idx = ((size_t) batch * p.M + m) * width + (n - p.n_begin);
+    const size_t idx = ((size_t) batch * p.M + m) * width + (n - p.part_begin);
     const size_t off4 = (size_t) batch * p.c_batch_stride + (size_t) m * p.c_stride_m + out_col_offset(p, n, 1);
     char *cbase = reinterpret_cast<char *>(p.C);
     if constexpr (IS_INT) {
@@ -852,17 +864,22 @@ template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1>
 static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream_t stream) {
     IgemmParams p = p_in;
     const int tiles_m = (p.M + BM - 1) / BM;
-    const int tiles = tiles_m * ((p.N - p.n_begin + BN - 1) / BN);
+    const int tiles = tiles_m * ((p.N + BN - 1) / BN);
     p.div_ohw = make_div31((unsigned) (p.OHW > 0 ? p.OHW : 1));
     p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
     p.div_tiles_m = make_div31((unsigned) tiles_m);
     dim3 grid(tiles, cfg.split, cfg.batch);
+    if (p.dp_tiles > 0) {   // whole tiles first, then the K slices of the leftover tiles (igemm_kernel)
+        if (cfg.batch != 1 || p.dp_tiles + p.tail_tiles != tiles || !p.partial || p.part_begin != p.dp_tiles / tiles_m * BN)
+            return set_error(ONHIP_ERR_ARG, "igemm: inconsistent leftover-tile launch");
+        grid = dim3(p.dp_tiles + p.tail_tiles * cfg.split, 1, 1);
+    }
     hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN, PF>), grid, dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
     if (p.partial) {
         if (p.M > 4 * 65535 || cfg.batch > 65535)
             return set_error(ONHIP_ERR_ARG, "igemm: split-K with %d rows, %d batches", p.M, cfg.batch);
-        const dim3 fgrid((p.N - p.n_begin + 63) / 64, (p.M + 3) / 4, cfg.batch);
+        const dim3 fgrid((p.N - p.part_begin + 63) / 64, (p.M + 3) / 4, cfg.batch);
         if (DT == DT_I8)
             hipLaunchKernelGGL((splitk_finish_kernel<true>), fgrid, dim3(64, 4), 0, stream, p, cfg.split, cfg.batch);
         else

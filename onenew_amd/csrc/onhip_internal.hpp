@@ -129,7 +129,9 @@ struct IgemmParams {
     int M, N, K;              // K counts real reduction elements (gather) or padded units*kpu (kvec)
     int k_units;               // 16-byte units along K (multiple of 2 per MFMA step is NOT required)
     int k_split_units;         // units handled by one blockIdx.y slice (split-K); == k_units if unsplit
-    int n_begin;               // first column of this launch (0 unless the columns are shared out between two launches)
+    int part_begin;            // first column the split-K partial sums cover (0 unless only leftover tiles are split)
+    int dp_tiles, tail_tiles;  // dp_tiles > 0: that many workgroups take whole tiles, the tail_tiles tiles after them are
+                               // cut into K slices (see igemm_kernel)
     // A
     const void *A;
     long long a_batch_stride;  // elements; 0 = shared
