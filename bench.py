@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
 Workloads (BASELINE configurations): resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
-cfg1, resnet50_net_b{1,32} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
+cfg1, resnet50_net_b{1,32} and mobilenetv2_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
 the HBM traffic counters are scaled by).
 
 A step is one pass over every layer of the workload: one launch per layer, inputs, weights and outputs
@@ -452,12 +452,15 @@ def cpu_baseline(layers, tag, unit, budget_s=12.0):
 
 
 def bench_net(torch, args):
-    """Whole ResNet-50 as a .one model through the device-resident runtime (libonenew_rt.so): every operator of the
-    graph (53 Conv, MaxPool, 16 Add, 16 Relu, GlobalAveragePool, Gemm) back to back on the device, input and
-    output in device memory.  A step is one inference of the batch."""
+    """A whole model (ResNet-50: 53 Conv, MaxPool, 16 Add, 16 Relu, GlobalAveragePool, Gemm; MobileNetV2: 52 Conv of
+    which 17 depthwise, 10 Add, GlobalAveragePool, Gemm) as a .one file through the device-resident runtime
+    (libonenew_rt.so): every operator back to back on the device, input and output in device memory.  A step is one
+    inference of the batch."""
     from onenew_amd import rt, stacks
     n = int(args.workload.split("_b")[1])
-    data, in_shape, flops = stacks.resnet50_model(n)
+    model = "ResNet-50" if args.workload.startswith("resnet50") else "MobileNetV2"
+    make = stacks.resnet50_model if model == "ResNet-50" else stacks.mobilenet_v2_model
+    data, in_shape, flops = make(n)
     net = rt.Net(data)
     x = torch.randn(in_shape, dtype=torch.float32, device="cuda")
     y = torch.empty((n, 1000), dtype=torch.float32, device="cuda")
@@ -485,16 +488,16 @@ def bench_net(torch, args):
     if not args.no_cpu:
         from oracle import one_model
         if one_model.have_ref_runner():
-            data1, shape1, flops1 = stacks.resnet50_model(1)
+            data1, shape1, flops1 = make(1)
             xin = np.random.default_rng(0).normal(size=shape1).astype(np.float32)
             ms = one_model.time_reference(data1, [xin], repeats=40)
             cpu = {"value": round(flops1 / (ms * 1e-3) / 1e12, 5), "unit": "TFLOP/s", "cores": 8, "kind": "reference",
                    "sample": f"40 inferences of the same model at batch 1 through the reference's host operator classes "
                              f"and x86 kernels, median {ms:.2f} ms", "ms_per_inference": round(ms, 3)}
-    line = {"metric": "resnet50_net_fp32_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
+    line = {"metric": f"{args.workload.split('_net_')[0]}_net_fp32_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": f"ResNet-50 .one model fp32, batch {n}, 224x224, {len(ops)} operators through the "
+            "config": {"workload": f"{model} .one model fp32, batch {n}, 224x224, {len(ops)} operators through the "
                                    f"device-resident runtime, input and logits in HBM", "operators": len(ops),
                        "ops_per_step": flops, "model_bytes": len(data)},
             "roofline": {"kernel": "whole inference: every operator of the graph on the default stream", "bound": "mfma",
@@ -538,7 +541,7 @@ def main():
                           "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
         return
 
-    if args.workload.startswith("resnet50_net_b"):
+    if args.workload.startswith("resnet50_net_b") or args.workload.startswith("mobilenetv2_net_b"):
         return bench_net(torch, args)
 
     desc, dtype, layers = make_workload(torch, hip, args.workload)

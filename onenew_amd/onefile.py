@@ -89,17 +89,31 @@ class OneModel:
         return outs[0]
 
     # ---- operators -------------------------------------------------------------------------------------
-    def conv(self, name, x, weight, bias, out, stride=1, pad=0, group=1, act=abi.NOT_ACT, clip=(0.0, 0.0)):
-        """weight [cout, cin/group, kh, kw] fp32 and bias [cout] (or None) become initialisers name.weight / name.bias"""
-        w = np.asarray(weight, dtype=np.float32)
-        ins = [x, self.init(name + ".weight", w)]
-        if bias is not None:
-            ins.append(self.init(name + ".bias", np.asarray(bias, dtype=np.float32)))
+    def conv(self, name, x, weight, bias, out, stride=1, pad=0, group=1, act=abi.NOT_ACT, clip=(0.0, 0.0), quant=None):
+        """weight [cout, cin/group, kh, kw] fp32 and bias [cout] (or None) become initialisers name.weight / name.bias.
+        quant=(weight_aux [cout], input_scale) marks the W8A32 form the offline quantiser writes
+        (tools/optimize/model_quant.hpp:14-25, :655-670): weight is then int8 and bias int32, both stored at the
+        front of initialisers that keep their fp32 size and type."""
         pads = (pad,) * 4 if isinstance(pad, int) else tuple(pad)
         strides = (stride, stride) if isinstance(stride, int) else tuple(stride)
-        return self.node("Conv", name, ins, [out], has_bias=int(bias is not None), dilations=(1, 1), group=group,
+        fields = {}
+        if quant is None:
+            w = np.asarray(weight, dtype=np.float32)
+            b = None if bias is None else np.asarray(bias, dtype=np.float32)
+        else:
+            aux, input_scale = quant
+            w8 = np.ascontiguousarray(weight, dtype=np.int8)
+            w = np.zeros(w8.shape, dtype=np.float32)
+            w.reshape(-1).view(np.int8)[:w8.size] = w8.reshape(-1)
+            b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32).view(np.float32)
+            fields = dict(ifmap_quant2=abi.TYPE_INT8, input_scale=float(input_scale),
+                          weight_aux=tuple(float(v) for v in np.asarray(aux, dtype=np.float32)))
+        ins = [x, self.init(name + ".weight", w)]
+        if b is not None:
+            ins.append(self.init(name + ".bias", b))
+        return self.node("Conv", name, ins, [out], has_bias=int(b is not None), dilations=(1, 1), group=group,
                          kernel_shape=w.shape[2:], pads=pads, strides=strides, act_type=act, clip_min=clip[0],
-                         clip_max=clip[1])
+                         clip_max=clip[1], **fields)
 
     def gemm(self, name, x, weight, bias, out):
         """out = x @ weight[N, K]^T + bias (device/x86/Gemm/gemm.c)"""

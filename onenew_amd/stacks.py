@@ -166,3 +166,50 @@ def resnet50_model(batch=1, classes=1000, tag="resnet50_model"):
     m.output("logits", (batch, classes))
     return m.tobytes(), (batch, 3, 224, 224), flops
 
+
+def mobilenet_v2_model(batch=1, classes=1000, tag="mobilenetv2_model"):
+    """The whole MobileNetV2 as a .one file in its optimised form: batch norm folded, ReLU6 fused as CLIP(0, 6) into
+    the stem, the expand and the depthwise convolutions, linear projections, residual Adds where stride is 1 and
+    the width does not change, the last 1x1 convolution, GlobalAveragePool, Flatten, Gemm.  Seeded weights.
+    Returns (bytes, input shape, multiply-accumulates x 2 per inference)."""
+    import numpy as np
+    from . import datagen, onefile
+
+    m = onefile.OneModel()
+    flops = 0
+
+    def cv(name, x, cin, cout, k, s, hw, act, group=1, gain=1.0):
+        nonlocal flops
+        p = k // 2
+        out_hw = (hw + 2 * p - k) // s + 1
+        kc = cin if group == 1 else 1
+        flops += 2 * batch * cout * out_hw * out_hw * kc * k * k
+        w = datagen.normal(datagen.seed_for(tag, name + ".w"), (cout, kc, k, k), 0.0, float(np.sqrt(2.0 / (kc * k * k)))) * gain
+        b = datagen.normal(datagen.seed_for(tag, name + ".b"), (cout,), 0.0, 0.01)
+        return m.conv(name, x, w, b, name + "_out", stride=s, pad=p, group=group, act=act, clip=(0.0, 6.0))
+
+    x = m.input("input", (batch, 3, 224, 224))
+    x = cv("stem", x, 3, 32, 3, 2, 224, CLIP)
+    cin, hw, bi = 32, 112, 0
+    for t, c, n, s in [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]:
+        for i in range(n):
+            bi += 1
+            stride = s if i == 0 else 1
+            hidden = cin * t
+            y = x
+            if t != 1:
+                y = cv(f"b{bi}.expand", y, cin, hidden, 1, 1, hw, CLIP)
+            y = cv(f"b{bi}.dw", y, hidden, hidden, 3, stride, hw, CLIP, group=hidden)
+            hw //= stride
+            y = cv(f"b{bi}.project", y, hidden, c, 1, 1, hw, NOT_ACT, gain=0.5)
+            x = m.add(f"b{bi}.add", y, x, f"b{bi}.add_out") if stride == 1 and cin == c else y
+            cin = c
+    x = cv("last", x, 320, 1280, 1, 1, hw, CLIP)
+    x = m.global_avgpool("avgpool", x, "avgpool_out")
+    x = m.flatten("flatten", x, "flatten_out", axis=1)
+    flops += 2 * batch * classes * 1280
+    x = m.gemm("fc", x, datagen.normal(datagen.seed_for(tag, "fc.w"), (classes, 1280), 0.0, 0.03),
+               datagen.normal(datagen.seed_for(tag, "fc.b"), (classes,), 0.0, 0.01), "logits")
+    m.output("logits", (batch, classes))
+    return m.tobytes(), (batch, 3, 224, 224), flops
+

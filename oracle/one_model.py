@@ -36,6 +36,13 @@ def _conv(cfg, x, w, bias):
                  clip_min=cfg.clip_min, clip_max=cfg.clip_max, leaky_relu_alpha=cfg.leaky_relu_alpha,
                  hard_sigmoid_alpha=cfg.hard_sigmoid_alpha, hard_sigmoid_beta=cfg.hard_sigmoid_beta)
     lut = oracle.silu_lut() if cfg.act_type == abi.SILU else None
+    if cfg.ifmap_quant2 == abi.TYPE_INT8:
+        # W8A32: int8 weights and int32 bias sit at the front of fp32-sized initialisers (conv.c:77-104)
+        d.input_scale = cfg.input_scale
+        w8 = np.ascontiguousarray(w).reshape(-1).view(np.int8)[:w.size].reshape(w.shape)
+        b32 = None if bias is None else np.ascontiguousarray(bias).view(np.int32)
+        aux = np.array([cfg.weight_aux[i] for i in range(d.cout)], dtype=np.float32)
+        return oracle.conv2d_w8a32(d, x, w8, b32, aux, lut)
     return oracle.conv2d_f32(d, x, w, bias, lut)
 
 

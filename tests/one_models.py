@@ -75,4 +75,27 @@ def two_inputs():
     return m.tobytes(), [_r("a", (1, 6, 5, 5)), _r("b", (1, 6, 5, 5))]
 
 
-MODELS = {"resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
+def quantised_block():
+    """W8A32 convolutions as the offline quantiser leaves them (int8 weights, int32 bias, per-channel weight_aux,
+    input_scale), dense with SiLU and RELU and one depthwise, between fp32 operators"""
+    from oracle import oracle
+    m = onefile.OneModel()
+    m.input("x", (1, 16, 18, 18))
+
+    def q(tag, shape, scale):
+        w = _r(tag + "w", shape, scale)
+        b = _r(tag + "b", (shape[0],), 0.2)
+        return oracle.quant_weight_bias(w, b)
+
+    w8, b32, aux = q("q1", (32, 16, 3, 3), 0.1)
+    m.conv("q1", "x", w8, b32, "q1_out", pad=1, act=abi.SILU, quant=(aux, 0.031))
+    w8, b32, aux = q("qd", (32, 1, 3, 3), 0.3)
+    m.conv("qd", "q1_out", w8, b32, "qd_out", stride=2, pad=1, group=32, act=abi.RELU, quant=(aux, 0.024))
+    w8, b32, aux = q("q2", (24, 32, 1, 1), 0.2)
+    m.conv("q2", "qd_out", w8, b32, "q2_out", act=abi.NOT_ACT, quant=(aux, 0.017))
+    m.relu("relu", "q2_out", "out")
+    m.output("out", (1, 24, 9, 9))
+    return m.tobytes(), [_r("xq", (1, 16, 18, 18))]
+
+
+MODELS = {"quantised_block": quantised_block, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}

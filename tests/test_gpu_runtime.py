@@ -45,6 +45,8 @@ def test_model_outputs_match_oracle(name, torch_dev):
     for (oname, _), got in zip(net.outputs, outs):
         assert got.shape == ref[oname].shape
         assert _close(got, ref[oname], 5e-4), oname                          # up to five MFMA operators deep, 1e-4 each
+        if name == "quantised_block":
+            assert np.array_equal(got, ref[oname])                           # integer accumulation: the chain is exact
     # every intermediate operand sits in device memory and holds what the oracle computed at that point
     for op_type, cfg in m["nodes"]:
         oname = cfg.op_base_cfg.out_operand_name[0].value.decode()
@@ -128,3 +130,24 @@ def test_plugin_lookup_prefers_the_per_operator_directory(torch_dev, tmp_path):
     a = np.linspace(-1, 1, 18, dtype=np.float32).reshape(1, 2, 3, 3)
     net = rt.Net(m.tobytes(), op_lib_dir=str(tmp_path))
     assert np.array_equal(net.run(a)[0], np.maximum(a + a, 0))
+
+
+@pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
+def test_whole_model_matches_the_reference_host_run(model, torch_dev):
+    """the full-size network at batch 1 (89 / 65 operators) through the runtime against the same file run by the
+    reference's host operator classes and x86 kernels on the CPU: logits within 1e-3 of their largest magnitude
+    (53 / 52 convolutions deep with fp32 sums in another order), same top-5 classes"""
+    from onenew_amd import stacks
+    if not one_model.have_ref_runner():
+        pytest.skip("oracle/_ref/ref_run_one is not built")
+    make = stacks.resnet50_model if model == "resnet50" else stacks.mobilenet_v2_model
+    data, shape, _ = make(1)
+    x = np.random.default_rng(3).normal(size=shape).astype(np.float32)
+    (_, ref), = one_model.run_reference(data, [x])
+    net = rt.Net(data)
+    (got,) = net.run(x)
+    assert got.shape == ref.shape == (1, 1000)
+    assert np.isfinite(got).all()
+    assert _close(got, ref, 1e-3)
+    assert set(np.argsort(got[0])[-5:]) == set(np.argsort(ref[0])[-5:])
+
