@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
-Workloads (BASELINE configurations): resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
+Workloads: resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
 cfg1, resnet50_net_b{1,32} and mobilenetv2_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
 the HBM traffic counters are scaled by).
 
@@ -401,7 +401,7 @@ def time_layers(torch, hip, layers, reps):
 
 
 def plugin_eval_latency(hip):
-    """the drop-in boundary end to end: `eval` of libConv_hip.so on host buffers (BASELINE config 1), i.e. with the
+    """the drop-in boundary end to end: `eval` of libConv_hip.so on host buffers (Conv2d+ReLU 64->64 56x56 3x3), i.e. with the
     activation copied in and the result copied out over PCIe on every call; never part of `value`"""
     import cases
     from onenew_amd import ops

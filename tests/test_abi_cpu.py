@@ -108,7 +108,7 @@ def test_layer_tables_match_published_counts():
     assert len(r) == 53
     # 8174.3 MFLOP per image: sum of the Conv rows of tools/perf_profiling/timeline_info/resnet50.csv
     assert abs(sum(d.flops() for _, d in r) / 1e6 - 8174.27) < 0.01
-    assert r[2][1].flops() == 231211008          # BASELINE configuration 1
+    assert r[2][1].flops() == 231211008          # Conv2d+ReLU 64->64 56x56 3x3, batch 1: 2 * 64 * 56 * 56 * 64 * 9
     m = stacks.mobilenet_v2()
     assert len(m) == 52 and sum(1 for _, d in m if d.group != 1) == 17
     assert len(stacks.yolov8s()) == 63
