@@ -104,7 +104,8 @@ static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
 static const int kNumSplits = 10;
 
 // tail > 1: the tiles left over after whole rounds of 256 are cut `tail` ways along K (launch_choice)
-struct Choice { int bm, bn, split, tail; };
+// rowb != 0: the kernel that feeds B from global memory straight into the MFMAs (igemm_rowb.hip), tile bm x bn
+struct Choice { int bm, bn, split, tail, rowb; };
 
 static std::mutex g_tune_mu;
 static int g_tune_mode = -1;   // -1: read ONHIP_TUNE on first use; 0 model only; 1 measure
@@ -140,8 +141,9 @@ static void load_tune_cache_locked() {
             key.push_back(v);
             s = end;
         }
-        Choice c = {0, 0, 1, 0};
-        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail) >= 3) g_tuned[key] = c;
+        Choice c = {0, 0, 1, 0, 0};
+        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb) >= 3)
+            g_tuned[key] = c;
     }
     fclose(f);
 }
@@ -151,7 +153,7 @@ static void append_tune_cache_locked(const std::vector<long long> &key, const Ch
     FILE *f = fopen(path, "a");
     if (!f) return;
     for (long long v : key) fprintf(f, "%lld ", v);
-    fprintf(f, ": %d %d %d %d\n", c.bm, c.bn, c.split, c.tail);
+    fprintf(f, ": %d %d %d %d %d\n", c.bm, c.bn, c.split, c.tail, c.rowb);
     fclose(f);
 }
 
@@ -212,6 +214,7 @@ static bool tail_geometry(const IgemmLaunch &cfg, const IgemmParams &p, int bm, 
 
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
+    if (c.rowb) return c.split == 1 && c.tail == 0 && rowb_f32_ok(cfg, p);
     if (c.tail > 1) {
         int dpc, left;
         return c.split == 1 && k_tiles >= 2 * c.tail && tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left);
@@ -241,11 +244,11 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
 }
 
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
-    Choice best = {64, 64, 1, 0};
+    Choice best = {64, 64, 1, 0, 0};
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t)
         for (int s = 0; s < kNumSplits; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0};
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0};
             if (!candidate_ok(cfg, p, c)) continue;
             const double cost = model_cost(cfg, p, c);
             if (cost < best_cost) { best_cost = cost; best = c; }
@@ -259,15 +262,21 @@ static std::atomic<long long> g_tail_launches{0};
 static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
     int dpc = 0, left = 0;
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
+    if (c.rowb) {
+        cfg.bm = c.bm; cfg.bn = c.bn; cfg.split = 1;
+        p.k_split_units = p.k_units;
+        p.partial = nullptr;
+        return rowb_f32_launch(cfg, p, st);
+    }
     if (c.tail <= 1 || !tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
-        const Choice plain = {c.bm, c.bn, c.split, 0};
+        const Choice plain = {c.bm, c.bn, c.split, 0, 0};
         int rc = apply_choice(cfg, p, plain);
         return rc ? rc : igemm_launch(cfg, p, st);
     }
     // one launch: dpc column blocks as whole tiles, the rest in c.tail K slices each; partial sums and the
     // finishing pass cover the columns from dpc * bn on only
     p.part_begin = dpc * c.bn;
-    const Choice tail = {c.bm, c.bn, c.tail, 0};
+    const Choice tail = {c.bm, c.bn, c.tail, 0, 0};
     int rc = apply_choice(cfg, p, tail);
     if (rc) return rc;
     if (cfg.split <= 1) {
@@ -303,9 +312,13 @@ static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStrea
 
 // Chooses tile, split and tail handling for the problem and launches it.
 static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t st) {
-    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL]]
-        Choice c = {0, 0, 1, 0};
-        if (sscanf(env, "%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail) >= 2) {
+    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB]]]
+        Choice c = {0, 0, 1, 0, 0};
+        if (sscanf(env, "%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb) >= 2) {
+            if (c.rowb && !candidate_ok(cfg, p, c)) {   // not a problem for that kernel: the tiled one, same tile if it has it
+                c.rowb = 0;
+                if (c.bn == 256) c.bn = 128;
+            }
             if (c.tail > 1 && !candidate_ok(cfg, p, c)) c.tail = 0;   // no leftover to split on this shape
             return launch_choice(cfg, p, c, st);
         }
@@ -342,7 +355,7 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     };
     for (int t = 0; t < kNumTiles && !rc; ++t) {
         for (int s = 0; s < kNumSplits && !rc; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0};
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0};
             if (!candidate_ok(cfg, p, c) || model_cost(cfg, p, c) > 2.5 * guess_cost) continue;
             try_choice(c);
         }
@@ -352,17 +365,23 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
             int want = 256 / left;
             want = want > 16 ? 16 : want;
             for (int ts = want; ts >= 2 && ts >= want / 2 && !rc; ts /= 2) {
-                const Choice c = {kTiles[t][0], kTiles[t][1], 1, ts};
-                if (candidate_ok(cfg, p, c) && model_cost(cfg, p, {c.bm, c.bn, 1, 0}) <= 2.5 * guess_cost) try_choice(c);
+                const Choice c = {kTiles[t][0], kTiles[t][1], 1, ts, 0};
+                if (candidate_ok(cfg, p, c) && model_cost(cfg, p, {c.bm, c.bn, 1, 0, 0}) <= 2.5 * guess_cost) try_choice(c);
             }
         }
+    }
+    // the kernel without LDS for B, where the problem allows it
+    static const int kRowbTiles[][2] = {{64, 128}, {128, 128}, {64, 256}};
+    for (int t = 0; t < 3 && !rc; ++t) {
+        const Choice c = {kRowbTiles[t][0], kRowbTiles[t][1], 1, 0, 1};
+        if (candidate_ok(cfg, p, c)) try_choice(c);
     }
     (void) hipEventDestroy(e0);
     (void) hipEventDestroy(e1);
     if (rc) return rc;
     if (getenv("ONHIP_TUNE_VERBOSE"))
-        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d (%.4f ms; model said %dx%d split %d)\n",
-                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best_ms, guess.bm,
+        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d rowb %d (%.4f ms; model said %dx%d split %d)\n",
+                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best.rowb, best_ms, guess.bm,
                 guess.bn, guess.split);
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);

@@ -184,6 +184,9 @@ struct IgemmLaunch {
 };
 
 int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
+// fp32 kernel for plain problems with B rows contiguous along N (igemm_rowb.hip): tiles 64x128, 128x128, 64x256
+bool rowb_f32_ok(const IgemmLaunch &cfg, const IgemmParams &p);
+int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
 
 // ---- other kernels -------------------------------------------------------------------------------------
 int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,

@@ -234,6 +234,53 @@ def test_leftover_tiles_as_a_split_launch(tile, shape, kind, torch_dev, oracle, 
     assert hip.split_tail_launches() == before + 3                             # the shape does have leftover tiles
 
 
+@pytest.mark.parametrize("tile", ["64x128x1x0x1", "128x128x1x0x1", "64x256x1x0x1"])
+@pytest.mark.parametrize("kind", ["conv_k200_m100", "conv_silu_k64", "conv_nobias", "matmul_batched_bias_gelu", "matmul_shared",
+                                  "not_applicable"])
+def test_kernel_with_b_straight_from_memory(tile, kind, torch_dev, oracle, monkeypatch):
+    """the fp32 kernel whose B operand never passes through LDS: 1x1 stride-1 convolutions and matrix products with K,
+    N and the pixels per image multiples of 4.  Ragged rows (100 channels), a last K tile of 8, column counts that end
+    inside a tile, several images, every epilogue; a problem it cannot take falls back to the tiled kernel."""
+    torch = torch_dev
+    monkeypatch.setenv("ONHIP_TILE", tile)
+    if kind.startswith("matmul"):
+        rng = np.random.default_rng(21)
+        if kind == "matmul_batched_bias_gelu":
+            a = (rng.normal(size=(3, 70, 136)) * 0.1).astype(np.float32)
+            b = rng.normal(size=(3, 136, 300)).astype(np.float32)
+            bias = rng.normal(size=(300,)).astype(np.float32)
+            lut = cases.gelu_lut()
+            ref = oracle.matmul_f32(a, b, bias, lut)
+            y = hip.matmul(dev(torch, a), dev(torch, b), bias=dev(torch, bias), gelu_lut=dev(torch, lut))
+        else:
+            a = (rng.normal(size=(2, 197, 192)) * 0.1).astype(np.float32)
+            b = rng.normal(size=(192, 576)).astype(np.float32)
+            ref = oracle.matmul_f32(a, b)
+            y = hip.matmul(dev(torch, a), dev(torch, b))
+        torch.cuda.synchronize()
+        if kind == "matmul_batched_bias_gelu":   # table activation: a step function of the sum (see the SILU case below)
+            err = np.abs(y.cpu().numpy() - ref)
+            assert err.max() <= 1.2 / 512 + 1e-4 * np.abs(ref).max() and np.mean(err > 1e-4 * np.abs(ref).max()) < 2e-3
+        else:
+            assert_close_f32(y.cpu().numpy(), ref, tag=f"{kind} {tile}")
+        return
+    d = {"conv_k200_m100": cases.cd(200, 100, 1, 1, 0, 20, 18, n=5, act=abi.RELU),
+         "conv_silu_k64": cases.cd(64, 256, 1, 1, 0, 28, 28, n=3, act=abi.SILU),
+         "conv_nobias": cases.cd(32, 48, 1, 1, 0, 12, 12, n=2, bias=0, act=abi.NOT_ACT),
+         "not_applicable": cases.cd(30, 40, 1, 1, 0, 7, 7, n=3, act=abi.RELU)}[kind]       # K = 30, 49 pixels per image
+    x, w, b = cases.conv_inputs(f"rowb_{kind}", d)
+    ref = oracle.conv2d_f32(d, x, w, b, cases.silu_lut())
+    y = hip.conv2d_f32(d, dev(torch, x), dev(torch, w), dev(torch, b), dev(torch, cases.silu_lut()))
+    torch.cuda.synchronize()
+    if d.act_type == abi.SILU:
+        # the table is a step function of the pre-activation: a last-bit difference in the sum may move an output to
+        # the neighbouring entry (slope below 1.1, step 1/512)
+        assert np.abs(y.cpu().numpy() - ref).max() <= 1.1 / 512 + 1e-4 * np.abs(ref).max()
+        assert np.mean(np.abs(y.cpu().numpy() - ref) > 1e-4 * np.abs(ref).max()) < 2e-3
+    else:
+        assert_close_f32(y.cpu().numpy(), ref, tag=f"{kind} {tile}")
+
+
 @pytest.mark.parametrize("tile", ["64x64x4", "128x128x2", "32x128x1"])
 def test_forced_split_w8a32_bit_exact(tile, torch_dev, oracle, monkeypatch):
     """integer partial sums add up exactly whatever the split"""
