@@ -214,7 +214,7 @@ static bool tail_geometry(const IgemmLaunch &cfg, const IgemmParams &p, int bm, 
 
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
-    if (c.rowb) return c.split == 1 && c.tail == 0 && rowb_f32_ok(cfg, p);
+    if (c.rowb && (c.split != 1 || !rowb_f32_ok(cfg, p))) return false;
     if (c.tail > 1) {
         int dpc, left;
         return c.split == 1 && k_tiles >= 2 * c.tail && tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left);
@@ -262,16 +262,11 @@ static std::atomic<long long> g_tail_launches{0};
 static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
     int dpc = 0, left = 0;
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
-    if (c.rowb) {
-        cfg.bm = c.bm; cfg.bn = c.bn; cfg.split = 1;
-        p.k_split_units = p.k_units;
-        p.partial = nullptr;
-        return rowb_f32_launch(cfg, p, st);
-    }
+    auto launch = [&]() { return c.rowb ? rowb_f32_launch(cfg, p, st) : igemm_launch(cfg, p, st); };
     if (c.tail <= 1 || !tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
-        const Choice plain = {c.bm, c.bn, c.split, 0, 0};
+        const Choice plain = {c.bm, c.bn, c.rowb ? 1 : c.split, 0, 0};
         int rc = apply_choice(cfg, p, plain);
-        return rc ? rc : igemm_launch(cfg, p, st);
+        return rc ? rc : launch();
     }
     // one launch: dpc column blocks as whole tiles, the rest in c.tail K slices each; partial sums and the
     // finishing pass cover the columns from dpc * bn on only
@@ -281,12 +276,12 @@ static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStr
     if (rc) return rc;
     if (cfg.split <= 1) {
         p.part_begin = 0;
-        return igemm_launch(cfg, p, st);
+        return launch();
     }
     p.dp_tiles = dpc * ((p.M + c.bm - 1) / c.bm);
     p.tail_tiles = left;
     g_tail_launches.fetch_add(1, std::memory_order_relaxed);
-    return igemm_launch(cfg, p, st);
+    return launch();
 }
 
 static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st, hipEvent_t e0, hipEvent_t e1,
@@ -374,7 +369,17 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     static const int kRowbTiles[][2] = {{64, 128}, {128, 128}, {64, 256}};
     for (int t = 0; t < 3 && !rc; ++t) {
         const Choice c = {kRowbTiles[t][0], kRowbTiles[t][1], 1, 0, 1};
-        if (candidate_ok(cfg, p, c)) try_choice(c);
+        if (!candidate_ok(cfg, p, c)) continue;
+        try_choice(c);
+        int dpc = 0, left = 0;
+        if (!rc && tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
+            int want = 256 / left;
+            want = want > 16 ? 16 : want;
+            for (int ts = want; ts >= 2 && ts >= want / 2 && !rc; ts /= 2) {
+                const Choice ct = {c.bm, c.bn, 1, ts, 1};
+                if (candidate_ok(cfg, p, ct)) try_choice(ct);
+            }
+        }
     }
     (void) hipEventDestroy(e0);
     (void) hipEventDestroy(e1);

@@ -12,7 +12,8 @@
 // instructions per MFMA.  The result of a lane is four neighbouring columns per row: 16-byte stores.
 //
 // Conditions (rowb_f32_ok): fp32, plain loader with unit strides, K, N and the pixels per image multiples of 4
-// (column quads never straddle an image or a row of B, A units are whole), unit column stride of C, no split-K.
+// (column quads never straddle an image or a row of B, A units are whole), unit column stride of C.  K is split only
+// for the tiles left over after whole rounds of 256 (dp_tiles / tail_tiles as in igemm_kernel).
 #include "igemm_kernel.hpp"
 
 namespace onhip {
@@ -53,6 +54,22 @@ __device__ __forceinline__ void rowb_store(const IgemmParams &p, f32x16 (&acc)[4
     }
 }
 
+// raw sums of one K slice: [slice][M][N - part_begin], four columns per store
+__device__ __forceinline__ void rowb_store_partial(const IgemmParams &p, f32x16 (&acc)[4], int slice, int m_wave, int n_quad, int lh) {
+    const int width = p.N - p.part_begin;
+    const rsrc_t rp = make_rsrc(reinterpret_cast<const char *>(p.partial) + (size_t) slice * p.M * width * 4, RSRC_RANGE);
+    const unsigned cv = n_quad < p.N ? (unsigned) (n_quad - p.part_begin + 4 * lh * width) * 4u : OOB;
+    const bool m_edge = m_wave + 32 > p.M;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m_uni = m_wave + 8 * (r / 4) + (r % 4);
+        const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
+        const float v0 = acc[0][r], v1 = acc[1][r], v2 = acc[2][r], v3 = acc[3][r];
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)},
+                                               rp, row_ok ? cv : OOB, (unsigned) m_uni * (unsigned) width * 4u, 0);
+    }
+}
+
 template <int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParams p) {
     constexpr int NT = 64 * WM * WN, BM = 32 * WM, BN = 128 * WN;
@@ -65,16 +82,29 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
     const int li = lane & 31, lh = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
     const int tiles_m = (p.M + BM - 1) / BM;
-    int lid;
-    {   // every XCD gets a contiguous run of tiles (its own L2)
-        const int nb = gridDim.x, bid = blockIdx.x;
-        const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
-        lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+    // workgroup -> (tile, K slice): whole tiles first, then the slices of the leftover tiles (see igemm_kernel)
+    int lid, slice = 0;
+    bool whole_k = true;
+    {
+        const int bid = blockIdx.x;
+        if (p.dp_tiles > 0 && bid >= p.dp_tiles) {
+            const int r = bid - p.dp_tiles;
+            slice = r / p.tail_tiles;
+            lid = p.dp_tiles + (r - slice * p.tail_tiles);
+            whole_k = false;
+        } else {   // every XCD gets a contiguous run of tiles (its own L2)
+            const int nb = p.dp_tiles > 0 ? p.dp_tiles : (int) gridDim.x;
+            const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
+            lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+        }
     }
     const int tile_n = (int) div31((unsigned) lid, p.div_tiles_m), tile_m = lid - tile_n * tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int batch = blockIdx.z;
-    const int k_tiles = (p.K + RB_KT - 1) / RB_KT;
+    // the slice's K tiles; a slice is a whole number of K tiles (4 units of 16 bytes each)
+    const int kt_begin = whole_k ? 0 : slice * p.k_split_units / 4;
+    const int k_end = whole_k ? p.K : min(p.K, (slice + 1) * p.k_split_units * 4);
+    const int k_tiles = (k_end + RB_KT - 1) / RB_KT - kt_begin;   // tiles of this workgroup, numbered from 0
 
     const char *a_base = reinterpret_cast<const char *>(p.A) + (size_t) batch * p.a_batch_stride * 4;
     const char *b_base = reinterpret_cast<const char *>(p.B) + (size_t) batch * p.b_batch_stride * 4;
@@ -113,9 +143,10 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
 
     auto issue_a = [&](int kt) __attribute__((always_inline)) {
         const rsrc_t ra = make_rsrc(a_base, kt < k_tiles ? a_bytes : 0u);
+        const int k0 = (kt_begin + kt) * RB_KT;
 #pragma unroll
-        for (int t = 0; t < A_PER_T; ++t)   // K is a multiple of 4: a unit lies inside K or outside it as a whole
-            qa[t] = buf_load_b128(ra, (kt * RB_KT + a_unit[t] * 4) < p.K ? a_voff[t] : OOB, (unsigned) (kt * RB_KT * 4));
+        for (int t = 0; t < A_PER_T; ++t)   // K and the slices are multiples of 4: a unit lies inside or outside as a whole
+            qa[t] = buf_load_b128(ra, (k0 + a_unit[t] * 4) < k_end ? a_voff[t] : OOB, (unsigned) (k0 * 4));
     };
     auto stage_a = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -124,13 +155,13 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
             if ((A_SLOTS % NT == 0) || f < A_SLOTS) lds[buf][(f % 4) * A_LD + f / 4] = qa[t];
         }
     };
-    // rows past K are read like any other (they hold finite tensor data or lie outside the buffer and read as
-    // zero); A is zero there.  A tile past the end is switched off as a whole.
+    // rows past the end of K or of the slice are read like any other (they hold finite tensor data or lie outside the
+    // buffer and read as zero); A is zero there.  A tile past the end is switched off as a whole.
     auto issue_b = [&](uint4 (&qb)[8], int kt, int slab) __attribute__((always_inline)) {
         const rsrc_t rb = make_rsrc(b_base, kt < k_tiles ? b_bytes : 0u);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
-            qb[slab * 4 + s] = buf_load_b128(rb, b_voff, (unsigned) (kt * RB_KT + slab * 8 + s) * row_bytes);
+            qb[slab * 4 + s] = buf_load_b128(rb, b_voff, (unsigned) ((kt_begin + kt) * RB_KT + slab * 8 + s) * row_bytes);
     };
     auto read_a = [&](uint4 (&oa)[2], int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -180,6 +211,10 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
     if (kt < k_tiles) body(qb0, oa0, oa1, kt);
 
     const int m_wave = m0 + wm * 32;
+    if (!whole_k) {
+        rowb_store_partial(p, acc, slice, m_wave, n_quad, lh);
+        return;
+    }
     switch (p.ep.act) {
         case NOT_ACT:
         case RELU6: rowb_store<EPI_NONE>(p, acc, batch, m_wave, n_quad, lh); break;
@@ -210,14 +245,26 @@ static int rowb_launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipS
     p.div_ohw = make_div31((unsigned) (p.OHW > 0 ? p.OHW : 1));
     p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
     p.div_tiles_m = make_div31((unsigned) tiles_m);
-    hipLaunchKernelGGL((rowb_f32_kernel<WM, WN>), dim3((unsigned) tiles, 1, cfg.batch), dim3(64 * WM * WN), 0, stream, p);
+    unsigned grid_x = (unsigned) tiles;
+    if (p.dp_tiles > 0) {   // whole tiles, then cfg.split K slices of each leftover tile
+        if (cfg.batch != 1 || p.dp_tiles + p.tail_tiles != tiles || !p.partial || cfg.split < 2 || (p.k_split_units % 4) ||
+            p.part_begin != p.dp_tiles / tiles_m * BN || p.M > 4 * 65535)
+            return set_error(ONHIP_ERR_ARG, "igemm: inconsistent leftover-tile launch");
+        grid_x = (unsigned) (p.dp_tiles + p.tail_tiles * cfg.split);
+    }
+    hipLaunchKernelGGL((rowb_f32_kernel<WM, WN>), dim3(grid_x, 1, cfg.batch), dim3(64 * WM * WN), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
+    if (p.dp_tiles > 0) {
+        const dim3 fgrid((p.N - p.part_begin + 63) / 64, (p.M + 3) / 4, 1);
+        hipLaunchKernelGGL((splitk_finish_kernel<false>), fgrid, dim3(64, 4), 0, stream, p, cfg.split, 1);
+        ONHIP_CHECK_HIP(hipGetLastError());
+    }
     return ONHIP_OK;
 }
 
 // cfg.bm x cfg.bn names the workgroup tile: 64x128 (2 wavefronts), 128x128 (4, stacked along M), 64x256 (2 x 2)
 int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
-    if (!rowb_f32_ok(cfg, p) || cfg.split != 1 || p.partial)
+    if (!rowb_f32_ok(cfg, p) || (p.dp_tiles > 0) != (cfg.split > 1) || (p.dp_tiles > 0) != (p.partial != nullptr))
         return set_error(ONHIP_ERR_ARG, "igemm: the row-B kernel does not take this problem");
     if (p.a_slice_bytes >= (1LL << 31) || p.b_slice_bytes >= (1LL << 31) || p.c_slice_bytes >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "igemm: an operand slice of 2 GiB or more is not supported");

@@ -194,7 +194,11 @@ def test_forced_tile_and_split_many_items(tile, kind, torch_dev, oracle, monkeyp
 
 
 @pytest.mark.parametrize("tile,shape", [("64x64x1x8", (20, 30, 29)), ("64x64x1x16", (17, 32, 32)), ("64x128x1x4", (34, 32, 34)),
-                                        ("32x128x1x8", (33, 32, 33)), ("128x128x1x2", (80, 24, 36))])
+                                        ("32x128x1x8", (33, 32, 33)), ("128x128x1x2", (80, 24, 36)),
+                                        # the same through the kernel that reads B straight from memory (1x1 and matmul;
+                                        # the 3x3 case falls back to the tiled kernel with the same split)
+                                        ("64x128x1x4x1", (34, 32, 34)), ("128x128x1x2x1", (80, 24, 36)),
+                                        ("64x256x1x4x1", (34, 32, 36))])
 @pytest.mark.parametrize("kind", ["3x3_packed", "1x1", "matmul"])
 def test_leftover_tiles_as_a_split_launch(tile, shape, kind, torch_dev, oracle, monkeypatch):
     """the launch cut along N: whole rounds of 256 tiles unsplit on the caller's stream, the leftover column blocks
