@@ -60,12 +60,19 @@ int elem_bytes(int32_t t) {
     }
 }
 
-// common/utils_c.h:9-16: all SHAPE_LEN entries are multiplied, unused ones hold 1
+// common/utils_c.h:9-16: all SHAPE_LEN entries are multiplied, unused ones hold 1.  -1 for a descriptor no tensor
+// can have (an entry below 1, or more than 2^40 elements), so that a damaged file is refused instead of followed.
 long long numel(const OPERAND_S &o) {
     long long n = 1;
-    for (int i = 0; i < SHAPE_LEN; ++i) n *= o.shapes[i];
+    for (int i = 0; i < SHAPE_LEN; ++i) {
+        if (o.shapes[i] < 1) return -1;
+        n *= o.shapes[i];
+        if (n > (1LL << 40)) return -1;
+    }
     return n;
 }
+
+bool sane_rank(const OPERAND_S &o) { return o.dim_num_of_shapes >= 1 && o.dim_num_of_shapes <= SHAPE_LEN; }
 
 // the node types this runtime runs, with the size of their config struct (the reference keeps this table in
 // Manager::op_cfg_size_map, filled by OP_REGISTER_GLOBAL in each host/ops/*.h)
@@ -155,8 +162,9 @@ int read_model(onrt_net &net) {
         t.desc.operand_name[OPERAND_NAME_LEN - 1] = 0;
         const int eb = elem_bytes(t.desc.data_type);
         const long long n = numel(t.desc);
-        if (!eb || n < 0 || n > (1LL << 40))
-            return fail(ONRT_ERR_FORMAT, "initialiser %s: data type %d / %lld elements", t.desc.operand_name, t.desc.data_type, n);
+        if (!eb || n < 0 || !sane_rank(t.desc))
+            return fail(ONRT_ERR_FORMAT, "initialiser %s: data type %d, rank %d, %lld elements", t.desc.operand_name, t.desc.data_type,
+                        t.desc.dim_num_of_shapes, n);
         t.bytes = (size_t) n * eb;
         if (off + sizeof(OPERAND_S) + t.bytes > size)
             return fail(ONRT_ERR_FORMAT, "initialiser %s ends past the end of the file", t.desc.operand_name);
@@ -178,6 +186,8 @@ int read_model(onrt_net &net) {
         const std::string name(io.operand.operand_name);
         if (!strcmp(io.op_name, "input")) {
             if (io.operand.data_type != TYPE_FP32) return fail(ONRT_ERR_FORMAT, "input %s is not fp32", name.c_str());
+            if (!sane_rank(io.operand) || numel(io.operand) < 1 || numel(io.operand) >= (1LL << 31))
+                return fail(ONRT_ERR_FORMAT, "input %s: rank %d, %lld elements", name.c_str(), io.operand.dim_num_of_shapes, numel(io.operand));
             Tensor t;
             t.desc = io.operand;
             t.produced = true;
@@ -336,6 +346,8 @@ int infer_shapes(onrt_net &net) {
             long long known = 1;
             for (int i = 0; i < SHAPE_LEN; ++i) out.shapes[i] = 1;
             for (int i = 0; i < c->dst_shape_num; ++i) {
+                if (c->dst_shape[i] != -1 && (c->dst_shape[i] < 1 || c->dst_shape[i] > total))
+                    return fail(ONRT_ERR_FORMAT, "Reshape %s: dimension %d is %lld", nd.base()->op_name, i, (long long) c->dst_shape[i]);
                 out.shapes[i] = (int32_t) c->dst_shape[i];
                 if (c->dst_shape[i] != -1) known *= c->dst_shape[i];
             }
@@ -346,7 +358,8 @@ int infer_shapes(onrt_net &net) {
         }
         // Relu, Gelu, LayerNormalization, Softmax: the input's shape
         const long long n = numel(out);
-        if (n <= 0 || n >= (1LL << 31)) return fail(ONRT_ERR_FORMAT, "%s %s: output of %lld elements", type, nd.base()->op_name, n);
+        if (n <= 0 || n >= (1LL << 31) || !sane_rank(out))
+            return fail(ONRT_ERR_FORMAT, "%s %s: output of rank %d, %lld elements", type, nd.base()->op_name, out.dim_num_of_shapes, n);
     }
     return ONRT_OK;
 }

@@ -109,3 +109,25 @@ def test_loader_reports_a_missing_plugin_directory():
     data, _ = one_models.two_inputs()
     rc, msg = _load_error(data)
     assert rc == -3 and "not found" in msg and "/nonexistent/Add/libAdd_hip.so" in msg
+
+
+def test_loader_rejects_damaged_descriptors():
+    """ranks and extents no tensor can have are refused before anything is indexed with them"""
+    import ctypes
+    data, _ = one_models.resnet_block()
+    m = onefile.parse(data)
+    io_off = m["header"].io_cfg_offset + 512                     # OPERAND_S of the first io config (the input)
+    for field, value, word in (("dim_num_of_shapes", 100, "rank"), ("dim_num_of_shapes", 0, "rank"), ("shapes", -3, "elements")):
+        bad = bytearray(data)
+        pos = io_off + getattr(abi.OPERAND_S, field).offset
+        bad[pos:pos + 4] = int(value & 0xffffffff).to_bytes(4, "little")
+        rc, msg = _load_error(bad)
+        assert rc == -2 and word in msg, (field, value, msg)
+    view = onefile.OneModel()
+    view.input("x", (1, 4, 3, 2))
+    view.reshape("r", "x", "y", (1, 0, 24))
+    view.relu("relu", "y", "z")
+    view.output("z", (1, 1, 24))
+    rc, msg = _load_error(view.tobytes())
+    assert rc == -2 and "Reshape" in msg
+
