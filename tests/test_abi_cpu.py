@@ -2,6 +2,7 @@
 import ctypes as C
 import os
 import re
+import sys
 
 import numpy as np
 
@@ -125,3 +126,13 @@ def test_datagen_is_deterministic_and_distributed():
     assert abs(z.mean()) < 0.02 and abs(z.std() - 2.0) < 0.02
     i = datagen.integers(9, (10000,), -127, 127)
     assert i.min() == -127 and i.max() == 127
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """the benchmark measures one GPU; asked for more it says so and exits before touching a device"""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0
+    assert "one GPU" in (res.stderr + res.stdout)
+
