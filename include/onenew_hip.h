@@ -115,6 +115,15 @@ int onhip_conv2d_pack_weights(const onhip_conv_desc_t *d, const float *w, float 
 int onhip_conv2d_f32_packed(const onhip_conv_desc_t *d, const float *x, const float *w_packed, const float *bias,
                             const float *silu_lut, float *y, void *stream);
 
+/* The convolution that ends a residual block with the operators after it folded into its store:
+ * y = conv(x) as onhip_conv2d_f32 (packed != 0: as onhip_conv2d_f32_packed), then y += addend (a tensor of
+ * y's shape, not y itself) as device/x86/Add/add.c:96, then, with relu_after != 0, relu as
+ * device/x86/Relu/relu.c:27-52 (both of its rules, by element index).  Bit-identical to the three operators
+ * run one after the other.  The reference fuses activations into Conv (tools/optimize/op_fusion.hpp:47-222)
+ * but not the Add; this is the same idea one operator further. */
+int onhip_conv2d_f32_add(const onhip_conv_desc_t *d, const float *x, const float *w, int32_t packed, const float *bias,
+                         const float *silu_lut, const float *addend, int32_t relu_after, float *y, void *stream);
+
 /* Bytes of device scratch onhip_conv2d_w8a32 needs for `d` (the int8 copy of the activations). */
 size_t onhip_conv2d_w8a32_workspace(const onhip_conv_desc_t *d);
 
@@ -266,6 +275,11 @@ int onhip_copy_f32(const float *src, float *dst, long long n, void *stream);
 /* ---- plugin level: the reference slot arrays; host or device pointers; synchronous --------- */
 
 int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* Conv with the Add (and Relu) that follow it in a residual block: slots as for Conv, inputs[3] = the other operand
+ * of the Add, outputs[0] = the block's result.  No counterpart in the reference; exported by libConv_hip.so as
+ * `eval_add` and `eval_add_relu` beside `eval`, for the device-resident runtime. */
+int onhip_conv_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Add (add.c:18), Relu (relu.c:8), MaxPool (maxpool.c:7), GlobalAveragePool (global_avgpool.c:7) */
 int onhip_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);

@@ -57,6 +57,18 @@ int onrt_net_io_count(const onrt_net_t *net, int32_t *n_inputs, int32_t *n_outpu
 int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, const char **name, int32_t *ndim,
                      int32_t shape[8]);
 
+/*
+ * Residual blocks.  Where a Conv's result is read only by an Add whose other operand has the same shape (and
+ * that sum perhaps only by a Relu), the loader folds the Add (and the Relu) into the convolution's store through
+ * the Conv plugin's `eval_add` / `eval_add_relu` entry points, when the plugin has them: one launch instead of
+ * three, and the tensors in between are never written.  The reference's offline optimiser folds the activation
+ * after a Conv the same way (tools/optimize/op_fusion.hpp:47-222).  Results are bit-identical to the separate
+ * operators.  The fused call runs at the Add's place in the order; the operands folded away stay in the operand
+ * table and read as the block's result.  Setting the environment variable ONENEW_RT_FUSE=0 before loading keeps
+ * every operator separate, for layer-by-layer comparison.  n_blocks: how many blocks were folded.
+ */
+int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks);
+
 /* Operators in execution order (host/net.h:309-330): type and name of number idx, count through n_ops. */
 int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops);
 int onrt_net_op_info(const onrt_net_t *net, int32_t idx, const char **op_type, const char **op_name);

@@ -320,7 +320,7 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     }
     if (!tune_mode()) return launch_choice(cfg, p, model_choice(cfg, p), st);
     std::vector<long long> key = {cfg.dtype, cfg.bl, cfg.batch, p.M, p.N, p.K, p.k_units, p.khkw, p.sh, p.sw,
-                                  p.H, p.W, p.out_mode, p.lda};
+                                  p.H, p.W, p.out_mode + (p.res ? 16 : 0), p.lda};   // a residual operand narrows the kernels
     {
         std::unique_lock<std::mutex> lock(g_tune_mu);
         load_tune_cache_locked();
@@ -464,12 +464,25 @@ int onhip_conv2d_pack_weights(const onhip_conv_desc_t *d, const float *w, float 
 }
 
 // packed != 0: w holds the tap-major layout written by onhip_conv2d_pack_weights
+// the Add (and Relu) of a residual block as separate passes over y, for the paths whose store cannot fold them in
+static int add_relu_in_place(const onhip_conv_desc_t *d, int OH, int OW, const float *addend, int relu, float *y, void *stream) {
+    onhip_add_desc_t ad;
+    memset(&ad, 0, sizeof(ad));
+    ad.ndim = 4;
+    const int32_t shape[4] = {d->n, d->cout, OH, OW};
+    for (int i = 0; i < 4; ++i) ad.large_shape[i] = ad.small_shape[i] = shape[i];
+    int rc = onhip_add_f32(&ad, y, addend, y, stream);
+    if (!rc && relu) rc = onhip_relu_f32(y, y, (long long) d->n * d->cout * OH * OW, stream);
+    return rc;
+}
+
 static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const float *w, int packed, const float *bias,
-                           const float *silu_lut, float *y, void *stream) {
+                           const float *silu_lut, float *y, void *stream, const float *addend = nullptr, int relu_after = 0) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
     if (!x || !w || !y || (d->has_bias && !bias)) return set_error(ONHIP_ERR_ARG, "conv: null tensor pointer");
+    if (addend == y) return set_error(ONHIP_ERR_ARG, "conv: the addend may not be the output buffer");
     if (d->has_bias && d->act_type == SILU && !silu_lut) return set_error(ONHIP_ERR_ARG, "conv: SILU needs the table");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const Epilogue ep = make_epilogue(*d, silu_lut);
@@ -477,7 +490,9 @@ static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const flo
     if (d->group != 1) {
         if (d->compute != ONHIP_COMPUTE_F32)
             return set_error(ONHIP_ERR_ARG, "conv: depthwise runs in fp32 only");
-        return depthwise_f32_launch(*d, OH, OW, x, w, bias, ep, y, st);
+        rc = depthwise_f32_launch(*d, OH, OW, x, w, bias, ep, y, st);
+        if (!rc && addend) rc = add_relu_in_place(d, OH, OW, addend, relu_after, y, stream);
+        return rc;
     }
     IgemmLaunch cfg;
     memset(&cfg, 0, sizeof(cfg));
@@ -524,7 +539,24 @@ static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const flo
     p.bias = bias;
     p.bias_mode = d->has_bias ? BIAS_M : BIAS_NONE;
     p.ep = ep;
+    if (addend && cfg.dtype != DT_F32) {   // reduced-precision operands: the two operators as passes over y
+        rc = plan_and_launch(cfg, p, st);
+        if (!rc) rc = add_relu_in_place(d, OH, OW, addend, relu_after, y, stream);
+        return rc;
+    }
+    if (addend) {
+        const long long n_out = (long long) d->n * d->cout * OH * OW;
+        p.res = addend;
+        p.res_relu = relu_after ? 1 : 0;
+        p.res_body = (unsigned) (n_out - n_out % 32);   // relu.c:27-52
+    }
     return plan_and_launch(cfg, p, st);
+}
+
+int onhip_conv2d_f32_add(const onhip_conv_desc_t *d, const float *x, const float *w, int32_t packed, const float *bias,
+                         const float *silu_lut, const float *addend, int32_t relu_after, float *y, void *stream) {
+    if (!addend) return set_error(ONHIP_ERR_ARG, "conv + add: null addend");
+    return conv2d_f32_impl(d, x, w, packed ? 1 : 0, bias, silu_lut, y, stream, addend, relu_after);
 }
 
 int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w, const float *bias,

@@ -76,10 +76,8 @@ __global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__re
 }
 
 // ---- ReLU ------------------------------------------------------------------------------------------
-// relu.c:27-52: the first n - n % 32 elements go through _mm256_max_ps(0, x), which is "0 > x ? 0 : x" (a NaN
-// or a negative zero comes back unchanged); the rest through "x > 0 ? x : 0".  Both rules are kept.
-__device__ __forceinline__ float relu_body(float v) { return 0.0f > v ? 0.0f : v; }
-__device__ __forceinline__ float relu_tail(float v) { return v > 0.0f ? v : 0.0f; }
+// relu.c:27-52: vector body and scalar tail differ on NaN and negative zero (relu_body / relu_tail); both rules
+// are kept.
 
 __global__ __launch_bounds__(256) void relu_kernel(const float *__restrict__ x, float *__restrict__ y, long long n,
                                                    long long n_body) {

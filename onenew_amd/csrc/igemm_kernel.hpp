@@ -311,7 +311,10 @@ __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
 // of the row (uniform) in the scalar offset.  Per-row operands (bias, weight_aux, int32 bias) are all
 // requested before the first one is used, through descriptors that are empty when the operand is
 // absent, so the epilogue has one memory round trip and no branches.
-template <int DT, int EPI, int TM, int TN, class ACC>
+// RES: the kernel variant for the last convolution of a residual block; the element of p.res at each output's place
+// is added after the activation (add_res).  All of a wavefront's addends are requested at once, ahead of the bias:
+// one memory round trip, paid for in registers, which is why the variant is a kernel of its own.
+template <int DT, int EPI, int TM, int TN, bool RES, class ACC>
 __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][TN], int batch, int m_wave, int n_wave,
                                            int li, int lh) {
     const int esz = (DT == DT_I8 && p.out_s8) ? 1 : 4;
@@ -384,6 +387,20 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                 }
             }
     } else {
+        float rv[RES ? TM : 1][RES ? 16 : 1][RES ? TN : 1];
+        if constexpr (RES) {
+            const rsrc_t rres = make_rsrc(reinterpret_cast<const char *>(p.res) + (size_t) batch * p.c_batch_stride * 4, RSRC_RANGE);
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
+                    const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+                        rv[a][r][b] = buf_load_f32(rres, row_ok ? col_voff[b] : OOB, (unsigned) m_uni * row_bytes);
+                }
+        }
         float bias_m[TM][16];
 #pragma unroll
         for (int a = 0; a < TM; ++a)
@@ -403,6 +420,8 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                     const float vm = __fadd_rn(v, bias_m[a][r]), vn = __fadd_rn(v, bias_n[b]);
                     v = bias_m_on ? vm : bias_n_on ? vn : v;
                     v = act_fast<EPI>(v, p.ep);
+                    if constexpr (RES)
+                        v = add_res(v, rv[a][r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
                     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff[b] : OOB,
                                                           (unsigned) m_uni * row_bytes, 0);
                 }
@@ -498,8 +517,9 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
 }
 
 // ---- the kernel --------------------------------------------------------------------------------
-template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1>
+template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1, bool RES = false>
 __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
+    static_assert(!RES || DT == DT_F32, "the residual store exists for fp32 operands");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     static_assert(TM >= 1 && TN >= 1 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile / wave grid mismatch");
@@ -819,12 +839,12 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     }
     switch (p.ep.act) {
         case NOT_ACT:
-        case RELU6: write_tile<DT, EPI_NONE, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
-        case RELU: write_tile<DT, EPI_RELU, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
-        case CLIP: write_tile<DT, EPI_CLIP, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case RELU6: write_tile<DT, EPI_NONE, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case RELU: write_tile<DT, EPI_RELU, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
         case SILU:
-        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
-        default: write_tile<DT, EPI_GENERIC, TM, TN>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        default: write_tile<DT, EPI_GENERIC, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
     }
 }
 
@@ -870,12 +890,14 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p,
         for (; s < split; ++s) acc = __fadd_rn(acc, part[(size_t) s * slice]);
         if (p.bias_mode == BIAS_M) acc = __fadd_rn(acc, p.bias[m]);
         else if (p.bias_mode == BIAS_N) acc = __fadd_rn(acc, p.bias[n]);
-        reinterpret_cast<float *>(cbase)[off4] = apply_act(acc, p.ep);
+        float y = apply_act(acc, p.ep);
+        if (p.res) y = add_res(y, p.res[off4], p.res_relu, (unsigned) off4, p.res_body);
+        reinterpret_cast<float *>(cbase)[off4] = y;
     }
 }
 
 // ---- launch ------------------------------------------------------------------------------------------
-template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1>
+template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1, bool RES = false>
 static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream_t stream) {
     IgemmParams p = p_in;
     const int tiles_m = (p.M + BM - 1) / BM;
@@ -889,7 +911,8 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
             return set_error(ONHIP_ERR_ARG, "igemm: inconsistent leftover-tile launch");
         grid = dim3(p.dp_tiles + p.tail_tiles * cfg.split, 1, 1);
     }
-    hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN, PF>), grid, dim3(THREADS), 0, stream, p);
+    if (RES != (p.res != nullptr)) return set_error(ONHIP_ERR_ARG, "igemm: residual operand and kernel variant do not match");
+    hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN, PF, RES>), grid, dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
     if (p.partial) {
         if (p.M > 4 * 65535 || cfg.batch > 65535)
@@ -904,14 +927,14 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     return ONHIP_OK;
 }
 
-template <int DT, int BL, int PF = 1>
+template <int DT, int BL, int PF = 1, bool RES = false>
 int launch_tile(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
     const int key = cfg.bm * 1000 + cfg.bn;
     switch (key) {
-        case 128128: return launch_one<DT, BL, 128, 128, 2, 2, (PF > 2 ? 2 : PF)>(cfg, p, stream);
-        case 64128: return launch_one<DT, BL, 64, 128, 2, 2, PF>(cfg, p, stream);
-        case 64064: return launch_one<DT, BL, 64, 64, 2, 2, PF>(cfg, p, stream);
-        case 32128: return launch_one<DT, BL, 32, 128, 1, 4, PF>(cfg, p, stream);
+        case 128128: return launch_one<DT, BL, 128, 128, 2, 2, (PF > 2 ? 2 : PF), RES>(cfg, p, stream);
+        case 64128: return launch_one<DT, BL, 64, 128, 2, 2, PF, RES>(cfg, p, stream);
+        case 64064: return launch_one<DT, BL, 64, 64, 2, 2, PF, RES>(cfg, p, stream);
+        case 32128: return launch_one<DT, BL, 32, 128, 1, 4, PF, RES>(cfg, p, stream);
         default: return set_error(ONHIP_ERR_ARG, "igemm: no kernel for tile %dx%d", cfg.bm, cfg.bn);
     }
 }

@@ -232,6 +232,7 @@ bool rowb_f32_ok(const IgemmLaunch &cfg, const IgemmParams &p) {
     if ((p.K % 4) || (p.N % 4) || (p.OHW % 4) || (p.HW % 4)) return false;
     if (p.out_mode == OUT_PLAIN && p.c_stride_n != 1) return false;
     if (p.lda % 4) return false;
+    if (p.res) return false;   // the store has no registers to spare for a residual operand: the tiled kernel takes those
     return true;
 }
 

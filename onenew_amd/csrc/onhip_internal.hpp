@@ -85,6 +85,17 @@ __device__ __forceinline__ float act_fast(float v, const Epilogue &e) {
     } else return apply_act(v, e);
 }
 
+// relu.c:27-52: the first n - n % 32 elements go through _mm256_max_ps(0, x), which is "0 > x ? 0 : x" (a NaN or a
+// negative zero comes back unchanged); the rest through "x > 0 ? x : 0"
+__device__ __forceinline__ float relu_body(float v) { return 0.0f > v ? 0.0f : v; }
+__device__ __forceinline__ float relu_tail(float v) { return v > 0.0f ? v : 0.0f; }
+// the Add and the Relu after a convolution, applied to one finished element at index `elem` of the output tensor
+__device__ __forceinline__ float add_res(float v, float r, int relu, unsigned elem, unsigned body) {
+    v = __fadd_rn(v, r);
+    const float vb = relu_body(v), vt = relu_tail(v);
+    return relu ? (elem < body ? vb : vt) : v;
+}
+
 // activation quantiser of conv.c:961-973: t = x * (1/scale), clamp, roundf (ties away from zero)
 __device__ __forceinline__ int quant_s8(float x, float inv_scale) {
     float t = __fmul_rn(x, inv_scale);
@@ -160,6 +171,12 @@ struct IgemmParams {
     const float *bias;
     int bias_mode;
     Epilogue ep;
+    // optional second pass of a residual block folded into the store (fp32 outputs): after the activation the
+    // element of `res` at the same place as in C is added (add.c), then, with res_relu, relu.c's rule is applied:
+    // the first res_body elements of the tensor go through its vector body, the rest through its scalar tail
+    const float *res;
+    int res_relu;
+    unsigned res_body;
     // W8A32
     float in_scale;            // activation scale s
     const float *weight_aux;   // per output channel max|w|

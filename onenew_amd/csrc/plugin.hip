@@ -174,7 +174,9 @@ static long long numel(const OPERAND_S *o) {
     return n;
 }
 
-static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+// fuse 0: the Conv of the reference.  1: inputs[3] holds a tensor of the output's shape that is added to the result
+// (the Add of a residual block); 2: and a Relu after that.
+static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, int fuse) {
     const CONV_CONFIG_S *cfg = reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr);
     const OPERAND_S *in_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
     const OPERAND_S *w_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
@@ -233,6 +235,12 @@ static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
         if (rc) return rc;
         if (!lut) return set_error(ONHIP_ERR_ARG, "Conv eval: SILU without a table in inputs[%d]", BUF_MAXNUM - 1);
     }
+    const void *addend = nullptr;
+    if (fuse) {
+        if (!inputs[3].addr) return set_error(ONHIP_ERR_ARG, "Conv eval: no addend in inputs[3]");
+        rc = input_on_device(1, reinterpret_cast<const void *>(inputs[3].addr), out_bytes, &addend);
+        if (rc) return rc;
+    }
     void *host_out = reinterpret_cast<void *>(outputs[0].addr);
     void *y = host_out;
     const bool out_on_dev = is_device_ptr(host_out);
@@ -260,6 +268,21 @@ static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
         else
             rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
                                     (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
+        if (!rc && fuse) {   // the int8 store does not fold the addend in: the two operators as passes over y
+            onhip_add_desc_t ad;
+            memset(&ad, 0, sizeof(ad));
+            ad.ndim = 4;
+            const int32_t shape[4] = {d.n, d.cout, OH, OW};
+            for (int i = 0; i < 4; ++i) ad.large_shape[i] = ad.small_shape[i] = shape[i];
+            rc = onhip_add_f32(&ad, (const float *) y, (const float *) addend, (float *) y, nullptr);
+            if (!rc && fuse == 2) rc = onhip_relu_f32((const float *) y, (float *) y, (long long) (out_bytes / 4), nullptr);
+        }
+    } else if (fuse) {
+        const float *wp = nullptr;
+        rc = packed_weights(&d, (const float *) w, &wp);
+        if (rc) return rc;
+        rc = onhip_conv2d_f32_add(&d, (const float *) x, wp ? wp : (const float *) w, wp ? 1 : 0, (const float *) b,
+                                  (const float *) lut, (const float *) addend, fuse == 2, (float *) y, nullptr);
     } else {
         // k x k dense weights are re-laid out tap-major once, next to their device copy
         const float *wp = nullptr;
@@ -276,6 +299,16 @@ static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
     if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, out_bytes, hipMemcpyDeviceToHost));
     else return wait_for_output();
     return ONHIP_OK;
+}
+
+static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return conv_eval_fused(params, inputs, outputs, 0);
+}
+static int conv_add_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return conv_eval_fused(params, inputs, outputs, 1);
+}
+static int conv_add_relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return conv_eval_fused(params, inputs, outputs, 2);
 }
 
 static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
@@ -625,6 +658,14 @@ extern "C" {
 int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Conv", conv_eval_locked, params, inputs, outputs);
 }
+int onhip_conv_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv + Add", conv_add_eval_locked, params, inputs, outputs);
+}
+
+int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv + Add + Relu", conv_add_relu_eval_locked, params, inputs, outputs);
+}
+
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MatMul", matmul_eval_locked, params, inputs, outputs);
 }

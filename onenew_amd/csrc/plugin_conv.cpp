@@ -6,3 +6,16 @@ extern "C" __attribute__((visibility("default"))) int eval(BUFFER_INFO_S *params
                                                            BUFFER_INFO_S *outputs) {
     return onhip_conv_eval(params, inputs, outputs);
 }
+
+// Not in the reference: the convolution that ends a residual block together with the Add (and the Relu) after it.
+// Slots as for `eval`, plus inputs[3] = the other operand of the Add (a tensor of the output's shape); outputs[0]
+// receives the block's result.  The device-resident runtime calls these when a model has that pattern.
+extern "C" __attribute__((visibility("default"))) int eval_add(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                               BUFFER_INFO_S *outputs) {
+    return onhip_conv_add_eval(params, inputs, outputs);
+}
+
+extern "C" __attribute__((visibility("default"))) int eval_add_relu(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                    BUFFER_INFO_S *outputs) {
+    return onhip_conv_add_relu_eval(params, inputs, outputs);
+}

@@ -17,6 +17,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <map>
 #include <memory>
 #include <set>
@@ -108,6 +109,7 @@ struct Tensor {
     size_t bytes = 0;
     bool is_init = false;
     bool produced = false;   // an io input, an initialiser or the output of an operator already ordered
+    std::string alias;       // an operand folded away with its producer reads as this one (fuse_residual_blocks)
 };
 
 struct Node {
@@ -115,6 +117,8 @@ struct Node {
     std::vector<char> cfg;   // the node's config struct, as in the file
     std::vector<std::string> in, out;
     onenew_eval_fn eval = nullptr;
+    int fuse = 0;            // Conv: 1 = the Add after it is folded in, 2 = and the Relu after that
+    std::string addend, fused_out;
     BUFFER_INFO_S params[BUF_MAXNUM], inputs[BUF_MAXNUM], outputs[BUF_MAXNUM];
     const BASE_CONFIG_S *base() const { return reinterpret_cast<const BASE_CONFIG_S *>(cfg.data()); }
 };
@@ -133,6 +137,8 @@ struct onrt_net {
     std::string lib_dir;
     std::map<std::string, void *> handles;
     std::vector<set_async_fn> async_switches;
+    onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
+    int fused_blocks = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -385,7 +391,7 @@ int allocate(onrt_net &net) {
     // operands: fp32 elements (elem_size * sizeof(float) in the reference), views excepted
     for (auto &kv : net.tensors) {
         Tensor &t = kv.second;
-        if (t.is_init || t.desc.not_need_buf) continue;
+        if (t.is_init || t.desc.not_need_buf || !t.alias.empty()) continue;
         t.bytes = (size_t) numel(t.desc) * 4;
         act_total += (t.bytes + 255) & ~(size_t) 255;
     }
@@ -394,10 +400,17 @@ int allocate(onrt_net &net) {
         size_t off = 0;
         for (auto &kv : net.tensors) {
             Tensor &t = kv.second;
-            if (t.is_init || t.desc.not_need_buf) continue;
+            if (t.is_init || t.desc.not_need_buf || !t.alias.empty()) continue;
             t.dev = static_cast<char *>(net.act_arena) + off;
             off += (t.bytes + 255) & ~(size_t) 255;
         }
+    }
+    for (auto &kv : net.tensors) {
+        Tensor &t = kv.second;
+        if (t.alias.empty()) continue;
+        const Tensor &target = net.tensors[t.alias];
+        t.dev = target.dev;
+        t.bytes = target.bytes;
     }
     // a view shares the buffer of its input (host/op.h:149-154), in execution order so that chains resolve
     for (int idx : net.order) {
@@ -465,7 +478,74 @@ int bind_plugins(onrt_net &net) {
         }
         nd.eval = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval"));
         if (!nd.eval) return fail(ONRT_ERR_PLUGIN, "no eval in the %s plugin", type.c_str());
+        if (type == "Conv") {
+            net.conv_add = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add"));
+            net.conv_add_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add_relu"));
+        }
     }
+    return ONRT_OK;
+}
+
+// ---- residual blocks ------------------------------------------------------------------------------------
+// Conv -> Add (-> Relu), where the convolution's result has no other reader and the other operand of the Add has the
+// same shape, becomes one call of the Conv plugin's `eval_add` / `eval_add_relu`: the sum is formed in the
+// convolution's store and the operands in between are never written.  The reference's optimiser does this for the
+// activation after a Conv (tools/optimize/op_fusion.hpp:47-222); here it goes one operator further, at load time.
+// The fused call takes the place of the Add in the order, where both of its inputs are complete.  The operands
+// folded away read as the block's result.  ONENEW_RT_FUSE=0 keeps every operator separate (layer-by-layer dumps).
+int fuse_residual_blocks(onrt_net &net) {
+    const char *env = getenv("ONENEW_RT_FUSE");
+    if ((env && !strcmp(env, "0")) || !net.conv_add) return ONRT_OK;
+    std::map<std::string, std::vector<int>> readers;
+    for (int idx : net.order)
+        for (const std::string &name : net.nodes[idx].in)
+            if (!name.empty()) readers[name].push_back(idx);
+    auto is_net_output = [&](const std::string &name) {
+        return std::find(net.out_names.begin(), net.out_names.end(), name) != net.out_names.end();
+    };
+    auto sole_reader = [&](const std::string &name, const char *type) -> int {
+        auto it = readers.find(name);
+        if (is_net_output(name) || it == readers.end() || it->second.size() != 1) return -1;
+        return strcmp(net.nodes[it->second[0]].kind->type, type) ? -1 : it->second[0];
+    };
+    std::map<int, int> runs_instead;   // Add node -> the Conv that takes its place
+    std::vector<bool> dropped(net.nodes.size(), false);
+    for (int idx : net.order) {
+        Node &conv = net.nodes[idx];
+        if (strcmp(conv.kind->type, "Conv") || conv.out.size() != 1 || conv.in.size() > 3) continue;
+        const std::string &mid = conv.out[0];
+        const int ai = sole_reader(mid, "Add");
+        if (ai < 0 || runs_instead.count(ai)) continue;
+        Node &add = net.nodes[ai];
+        if (add.in.size() != 2 || add.out.size() != 1 || add.in[0] == add.in[1]) continue;
+        const std::string &other = add.in[0] == mid ? add.in[1] : add.in[0];
+        const Tensor &ot = net.tensors[other], &mt = net.tensors[mid], &st = net.tensors[add.out[0]];
+        if (ot.is_init || !ot.alias.empty() || memcmp(ot.desc.shapes, mt.desc.shapes, sizeof(mt.desc.shapes)) ||
+            memcmp(st.desc.shapes, mt.desc.shapes, sizeof(mt.desc.shapes)))
+            continue;
+        conv.fuse = 1;
+        conv.addend = other;
+        conv.fused_out = add.out[0];
+        const int ri = net.conv_add_relu ? sole_reader(add.out[0], "Relu") : -1;
+        if (ri >= 0 && net.nodes[ri].in.size() == 1 && net.nodes[ri].out.size() == 1) {
+            conv.fuse = 2;
+            conv.fused_out = net.nodes[ri].out[0];
+            dropped[ri] = true;
+            net.tensors[add.out[0]].alias = conv.fused_out;
+        }
+        net.tensors[mid].alias = conv.fused_out;
+        conv.eval = conv.fuse == 2 ? net.conv_add_relu : net.conv_add;
+        dropped[idx] = true;
+        runs_instead[ai] = idx;
+        ++net.fused_blocks;
+    }
+    std::vector<int> order;
+    for (int idx : net.order) {
+        auto it = runs_instead.find(idx);
+        if (it != runs_instead.end()) order.push_back(it->second);
+        else if (!dropped[idx]) order.push_back(idx);
+    }
+    net.order.swap(order);
     return ONRT_OK;
 }
 
@@ -486,9 +566,10 @@ int fill_slots(onrt_net &net) {
             nd.params[1 + slot].addr = (int64_t) &t.desc;
             nd.inputs[slot].addr = (int64_t) t.dev;
         }
+        if (nd.fuse) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
-            Tensor &t = net.tensors[nd.out[k]];
+            Tensor &t = net.tensors[nd.fuse ? nd.fused_out : nd.out[k]];
             if (out_slot >= BUF_MAXNUM - 1) return fail(ONRT_ERR_FORMAT, "%s: too many operands", nd.base()->op_name);
             nd.params[out_slot].addr = (int64_t) &t.desc;
             nd.outputs[k].addr = (int64_t) t.dev;
@@ -511,6 +592,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
     if (!rc) rc = bind_plugins(net);
+    if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = allocate(net);
     if (!rc) rc = build_tables(net);
     if (!rc) rc = fill_slots(net);
@@ -585,6 +667,12 @@ ONRT_API int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t 
 ONRT_API int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops) {
     if (!net || !n_ops) return fail(ONRT_ERR_ARG, "null argument");
     *n_ops = (int32_t) net->order.size();
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks) {
+    if (!net || !n_blocks) return fail(ONRT_ERR_ARG, "null argument");
+    *n_blocks = (int32_t) net->fused_blocks;
     return ONRT_OK;
 }
 

@@ -28,6 +28,14 @@ class Plugin:
         self.eval = self.lib.eval
         self.eval.restype = C.c_int
         self.eval.argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
+        # entry points beside `eval` that the HIP Conv plugin has and the reference's plugins do not: the convolution
+        # with the Add (and Relu) of a residual block folded in, the other operand of the Add in inputs[3]
+        for extra in ("eval_add", "eval_add_relu"):
+            fn = getattr(self.lib, extra, None) if hasattr(self.lib, extra) else None
+            if fn is not None:
+                fn.restype = C.c_int
+                fn.argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
+            setattr(self, extra, fn)
 
 
 def aligned_empty(shape, dtype=np.float32, align=64, extra=16):
@@ -164,7 +172,8 @@ class Conv(_Op):
             self.lut = np.ascontiguousarray(silu_lut if silu_lut is not None else build_silu_lut(), dtype=np.float32)
             self._slot(self.inputs_vec, BUF_MAXNUM - 1, self.lut)
 
-    def __call__(self, x, out=None):
+    def __call__(self, x, out=None, addend=None):
+        """addend: the tensor of the output's shape that `eval_add` / `eval_add_relu` add to the result (inputs[3])"""
         d = self.desc
         oh, ow = d.out_hw()
         xin = x if isinstance(x, int) else np.ascontiguousarray(x, dtype=np.float32)
@@ -172,8 +181,13 @@ class Conv(_Op):
             out = aligned_empty((d.n, d.cout, oh, ow), np.float32)
         self._slot(self.inputs_vec, 0, xin)
         self._slot(self.outputs_vec, 0, out)
+        kept = 2
+        if addend is not None:
+            self._slot(self.inputs_vec, 3, addend if isinstance(addend, int) else np.ascontiguousarray(addend, dtype=np.float32))
+            kept = 3
         rc = self.forward()
-        del self._keep[-2:]
+        del self._keep[-kept:]
+        self.inputs_vec[3].addr = 0
         if rc != 0:
             raise RuntimeError(f"Conv eval returned {rc}")
         return out

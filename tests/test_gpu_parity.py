@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import cases
-from onenew_amd import abi, hip, ops
+from onenew_amd import abi, datagen, hip, ops
 from onenew_amd.abi import ConvDesc
 
 pytestmark = pytest.mark.gpu
@@ -368,6 +368,134 @@ def test_gemm_f32(name, torch_dev, oracle, golden):
     ref = oracle.gemm_f32(a, w, b)
     assert_close_f32(y, ref, tag=name)
     cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(ref).max()))
+
+
+# ---- the last convolution of a residual block with the Add and the Relu folded into its store ------------------
+
+def _residual_case(kind):
+    if kind == "1x1_resnet":          # a ResNet conv3: 1x1, no activation of its own
+        return cases.cd(64, 256, 1, 1, 0, 28, act=abi.NOT_ACT, n=2)
+    if kind == "1x1_ragged":          # 100 channels, 29x29: ragged tiles both ways, element count not a multiple of 32
+        return cases.cd(72, 100, 1, 1, 0, 29, act=abi.NOT_ACT, n=3)
+    if kind == "3x3_packed_relu":     # activation before the Add, then the block's Relu
+        return cases.cd(32, 48, 3, 1, 1, 19, 23, act=abi.RELU, n=2)
+    if kind == "3x3_s2_gather":       # weights as they are: the gathering loader
+        return cases.cd(24, 40, 3, 2, 1, 30, act=abi.CLIP, n=2, clip_min=-0.2, clip_max=0.5)
+    if kind == "mobilenet_project":   # MobileNetV2 project layer: few output channels, linear
+        return cases.cd(144, 24, 1, 1, 0, 56, act=abi.NOT_ACT, n=2)
+    if kind == "depthwise":           # no folded store on this path: the entry point runs the passes itself
+        return cases.cd(48, 48, 3, 1, 1, 20, act=abi.NOT_ACT, group=48, n=2)
+    if kind == "nobias":
+        return cases.cd(64, 64, 1, 1, 0, 16, act=abi.NOT_ACT, bias=0, n=1)
+    raise KeyError(kind)
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("tile", [None, "64x64x1", "64x64x3", "32x128x2", "128x128x1", "64x128x1x4", "64x128x1x0x1"])
+@pytest.mark.parametrize("kind", ["1x1_resnet", "1x1_ragged", "3x3_packed_relu", "3x3_s2_gather", "mobilenet_project",
+                                  "depthwise", "nobias"])
+def test_conv_with_add_and_relu_folded_in(kind, tile, relu, torch_dev, oracle, monkeypatch):
+    """onhip_conv2d_f32_add against the three operators run one after the other on the same launch configuration:
+    the same bits, whichever kernel stores the result (whole tiles, split K with its finishing pass, leftover tiles;
+    a forced row-B tile falls back to the tiled kernel).  The addend holds NaNs in the part of the tensor that
+    relu.c's vector body covers and in its scalar tail, where the two rules of that operator differ."""
+    torch = torch_dev
+    if tile is not None:
+        monkeypatch.setenv("ONHIP_TILE", tile)
+    d = _residual_case(kind)
+    if kind == "depthwise" and tile is not None:
+        pytest.skip("one kernel only")
+    x, w, b = cases.conv_inputs(f"res_{kind}", d)
+    oh, ow = d.out_hw()
+    r = datagen.uniform(datagen.seed_for(f"res_{kind}", "r"), (d.n, d.cout, oh, ow), -1.0, 1.0)
+    flat = r.reshape(-1)
+    flat[5] = np.nan
+    flat[-1] = np.nan                      # in the tail whenever the element count is not a multiple of 32
+    flat[7] = -0.0
+    xd, wd, rd = dev(torch, x), dev(torch, w), dev(torch, r)
+    bd = dev(torch, b) if b is not None else None
+    packed = kind.startswith("3x3_packed")
+    if packed:
+        wd = hip.pack_conv_weights(d, wd)
+    plain = hip.conv2d_f32(d, xd, wd, bd, packed=packed)
+    want = hip.add_f32(plain, rd)
+    if relu:
+        want = hip.relu_f32(want)
+    for rep in range(2):
+        got = hip.conv2d_f32_add(d, xd, wd, rd, bias=bd, relu=relu, packed=packed)
+        torch.cuda.synchronize()
+        assert _same_bits(got.cpu().numpy(), want.cpu().numpy()), f"{kind} tile {tile} relu {relu} run {rep}"
+    # and the sum is the sum: against the oracle's convolution, away from the planted NaNs
+    ref = oracle.conv2d_f32(d, x, w, b, cases.silu_lut()) + r
+    if relu:
+        ref = np.where(ref > 0, ref, 0).astype(np.float32)
+    ok = ~np.isnan(r)
+    assert_close_f32(np.where(ok, got.cpu().numpy(), 0), np.where(ok, ref, 0), tag=f"{kind} against the oracle")
+
+
+@pytest.mark.parametrize("relu", [False, True])
+def test_conv_with_add_folded_in_leftover_tiles(relu, torch_dev, monkeypatch):
+    """more tiles than one round of the chip: whole tiles store the sum themselves, the finishing pass of the split
+    leftover tiles adds it for its columns"""
+    torch = torch_dev
+    monkeypatch.setenv("ONHIP_TILE", "64x64x1x8")
+    d = cases.cd(520, 100, 1, 1, 0, 30, 29, n=20, act=abi.NOT_ACT)
+    x, w, b = cases.conv_inputs("res_tail", d)
+    r = datagen.uniform(datagen.seed_for("res_tail", "r"), (20, 100, 30, 29), -1.0, 1.0)
+    xd, wd, bd, rd = dev(torch, x), dev(torch, w), dev(torch, b), dev(torch, r)
+    before = hip.split_tail_launches()
+    want = hip.add_f32(hip.conv2d_f32(d, xd, wd, bd), rd)
+    if relu:
+        want = hip.relu_f32(want)
+    got = hip.conv2d_f32_add(d, xd, wd, rd, bias=bd, relu=relu)
+    torch.cuda.synchronize()
+    assert hip.split_tail_launches() == before + 2
+    assert _same_bits(got.cpu().numpy(), want.cpu().numpy())
+
+
+def test_conv_add_refuses_the_output_as_addend(torch_dev):
+    torch = torch_dev
+    d = _residual_case("nobias")
+    x, w, _ = cases.conv_inputs("res_alias", d)
+    y = torch.zeros((1, 64, 16, 16), dtype=torch.float32, device="cuda")
+    with pytest.raises(hip.OnhipError):
+        hip.conv2d_f32_add(d, dev(torch, x), dev(torch, w), y, out=y)
+
+
+@pytest.mark.parametrize("name", ["c3x3_tiny_relu", "c1x1_unaligned_clip", "dw3x3_s2_even", "rn50_l4_1x1_2048_512"])
+def test_plugin_conv_eval_add_host_buffers(name, torch_dev):
+    """libConv_hip.so's eval_add / eval_add_relu: slots as for eval plus the addend in inputs[3]; against eval
+    followed by the Add and Relu plugins"""
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    oh, ow = d.out_hw()
+    r = datagen.uniform(datagen.seed_for(name, "residual"), (d.n, d.cout, oh, ow), -1.0, 1.0)
+    plug = ops.Plugin(hip.plugin_path("Conv"))
+    assert plug.eval_add is not None and plug.eval_add_relu is not None
+    y = ops.Conv(plug.eval, d, w, b, silu_lut=cases.silu_lut())(x)
+    add = ops.Add(ops.Plugin(hip.plugin_path("Add")).eval)
+    relu = ops.Relu(ops.Plugin(hip.plugin_path("Relu")).eval)
+    summed = add(y, r)
+    got = ops.Conv(plug.eval_add, d, w, b, silu_lut=cases.silu_lut())(x, addend=r)
+    assert _same_bits(got, summed)
+    got = ops.Conv(plug.eval_add_relu, d, w, b, silu_lut=cases.silu_lut())(x, addend=r)
+    assert _same_bits(got, relu(summed))
+
+
+def test_plugin_conv_eval_add_w8a32(torch_dev):
+    """the int8 convolution has no folded store: the plugin runs the Add and the Relu as passes over its output"""
+    name = "q3x3_silu"
+    d = cases.conv_w8a32_cases()[name]
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    oh, ow = d.out_hw()
+    r = datagen.uniform(datagen.seed_for(name, "residual"), (d.n, d.cout, oh, ow), -1.0, 1.0)
+    plug = ops.Plugin(hip.plugin_path("Conv"))
+    y = ops.Conv(plug.eval, d, w8, b32, weight_aux=aux, silu_lut=cases.silu_lut())(x)
+    got = ops.Conv(plug.eval_add_relu, d, w8, b32, weight_aux=aux, silu_lut=cases.silu_lut())(x, addend=r)
+    want = y + r
+    want = np.concatenate([np.where(0.0 > want.reshape(-1)[:want.size // 32 * 32], 0.0, want.reshape(-1)[:want.size // 32 * 32]),
+                           np.where(want.reshape(-1)[want.size // 32 * 32:] > 0, want.reshape(-1)[want.size // 32 * 32:], 0.0)])
+    assert _same_bits(got, want.astype(np.float32).reshape(got.shape))
 
 
 # ---- plugin level: host pointers through `eval`, as the oneNew runtime calls it -------------------------

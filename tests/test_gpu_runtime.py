@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 from oracle import one_model  # noqa: E402
 import one_models  # noqa: E402
-from onenew_amd import hip, onefile, rt  # noqa: E402
+from onenew_amd import abi, hip, onefile, rt  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 
@@ -34,9 +34,11 @@ def _close(got, ref, rel):
 
 
 @pytest.mark.parametrize("name", list(one_models.MODELS))
-def test_model_outputs_match_oracle(name, torch_dev):
+def test_model_outputs_match_oracle(name, torch_dev, monkeypatch):
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")          # operator by operator, so that every operand can be compared
     data, ins = one_models.MODELS[name]()
     net = rt.Net(data)
+    assert net.fused_blocks() == 0
     m = onefile.parse(data)
     assert [n for n, _ in net.inputs] == [n for n, _ in m["inputs"]]
     assert net.outputs == [(n, tuple(s)) for n, s in m["outputs"]]          # inferred shapes equal the declared ones
@@ -130,6 +132,132 @@ def test_plugin_lookup_prefers_the_per_operator_directory(torch_dev, tmp_path):
     a = np.linspace(-1, 1, 18, dtype=np.float32).reshape(1, 2, 3, 3)
     net = rt.Net(m.tobytes(), op_lib_dir=str(tmp_path))
     assert np.array_equal(net.run(a)[0], np.maximum(a + a, 0))
+
+
+def _both_ways(data, ins, monkeypatch):
+    """outputs of the net loaded with residual blocks folded and with every operator separate"""
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    plain = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    fused = rt.Net(data)
+    return fused, plain, fused.run(*ins), plain.run(*ins)
+
+
+def test_residual_block_is_folded_into_the_convolution(torch_dev, monkeypatch):
+    """Conv -> Add -> Relu of the small ResNet block runs as one call of the Conv plugin: two operators fewer, the
+    operands in between share the block's buffer, and the net's output has the same bits as operator by operator"""
+    data, ins = one_models.resnet_block()
+    fused, plain, got, want = _both_ways(data, ins, monkeypatch)
+    assert plain.fused_blocks() == 0 and fused.fused_blocks() == 1
+    assert len(fused.ops()) == len(plain.ops()) - 2
+    assert [t for t, _ in fused.ops()].count("Add") == 0 and [t for t, _ in fused.ops()].count("Relu") == 0
+    assert np.array_equal(got[0], want[0])
+    assert fused.operand("c2_out")[1] == fused.operand("res_out")[1] == fused.operand("relu_out")[1]
+    assert np.array_equal(fused.fetch("relu_out"), plain.fetch("relu_out"))
+    (ref,) = one_model.run(data, ins)
+    assert _close(got[0], ref, 5e-4)
+    # a second run on another input: the folded call reads the addend afresh
+    x2 = (ins[0] * np.float32(0.5) - np.float32(0.1)).astype(np.float32)
+    assert np.array_equal(fused.run(x2)[0], plain.run(x2)[0])
+
+
+def _w(rng, *shape):
+    return (rng.normal(size=shape) * 0.2).astype(np.float32)
+
+
+def _residual_variants():
+    rng = np.random.default_rng(23)
+    out = {}
+
+    def base():
+        m = onefile.OneModel()
+        m.input("x", (2, 8, 12, 12))
+        return m
+
+    # the shortcut is itself a convolution that comes later in the file than the main branch (ResNet's first block of
+    # a stage): the folded call runs where the Add was, after both
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 8, 3, 3), _w(rng, 8), "main_out", pad=1)
+    m.conv("short", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "short_out")
+    m.add("sum", "main_out", "short_out", "s")
+    m.relu("relu", "s", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["shortcut_conv_later_in_the_file"] = (m.tobytes(), 1, 2)
+    # the Add without a Relu (MobileNetV2), addend first
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "main_out")
+    m.add("sum", "x", "main_out", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["add_only_addend_first"] = (m.tobytes(), 1, 1)
+    # the sum is read twice: the Add is folded, the Relu stays an operator
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 8, 3, 3), None, "main_out", pad=1, act=abi.RELU)
+    m.add("sum", "main_out", "x", "s")
+    m.relu("relu", "s", "r")
+    m.add("again", "s", "r", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["sum_read_twice"] = (m.tobytes(), 1, 1)
+    # depthwise convolution in front of the Add: the plugin runs the passes itself
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 1, 3, 3), _w(rng, 8), "main_out", pad=1, group=8)
+    m.add("sum", "main_out", "x", "s")
+    m.relu("relu", "s", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["depthwise_main_branch"] = (m.tobytes(), 1, 2)
+    # nothing to fold: the convolution's result is a net output / is read twice / the Add broadcasts a vector
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "main_out")
+    m.add("sum", "main_out", "x", "y")
+    m.output("y", (2, 8, 12, 12))
+    m.output("main_out", (2, 8, 12, 12))
+    out["conv_result_is_an_output"] = (m.tobytes(), 0, 0)
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "main_out")
+    m.add("sum", "main_out", "x", "s")
+    m.add("again", "s", "main_out", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["conv_result_read_twice"] = (m.tobytes(), 0, 0)
+    m = base()
+    m.conv("main", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "main_out")
+    m.add("sum", "main_out", _w(rng, 1, 8, 1, 1), "y")
+    m.output("y", (2, 8, 12, 12))
+    out["add_of_a_broadcast_initialiser"] = (m.tobytes(), 0, 0)
+    # two convolutions into one Add: one of them is folded, the other runs before it
+    m = base()
+    m.conv("a", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "a_out")
+    m.conv("b", "x", _w(rng, 8, 8, 3, 3), _w(rng, 8), "b_out", pad=1)
+    m.add("sum", "a_out", "b_out", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["two_convolutions_into_one_add"] = (m.tobytes(), 1, 1)
+    return out
+
+
+@pytest.mark.parametrize("name", list(_residual_variants()))
+def test_folding_rules(name, torch_dev, monkeypatch):
+    data, blocks, fewer_ops = _residual_variants()[name]
+    x = np.random.default_rng(29).normal(size=(2, 8, 12, 12)).astype(np.float32)
+    fused, plain, got, want = _both_ways(data, [x], monkeypatch)
+    assert fused.fused_blocks() == blocks
+    assert len(fused.ops()) == len(plain.ops()) - fewer_ops
+    for g, w_ in zip(got, want):
+        assert np.array_equal(g, w_)
+    ref = one_model.run(data, [x])
+    for g, r in zip(got, ref):
+        assert _close(g, r, 3e-4)
+
+
+@pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
+def test_whole_model_folds_every_residual_block(model, torch_dev, monkeypatch):
+    """16 bottleneck blocks of ResNet-50 (Add + Relu) and the 10 residual connections of MobileNetV2 (Add), batch 2:
+    the same logits, bit for bit, as operator by operator"""
+    from onenew_amd import stacks
+    make = stacks.resnet50_model if model == "resnet50" else stacks.mobilenet_v2_model
+    data, shape, _ = make(2)
+    x = np.random.default_rng(31).normal(size=shape).astype(np.float32)
+    fused, plain, got, want = _both_ways(data, [x], monkeypatch)
+    assert fused.fused_blocks() == (16 if model == "resnet50" else 10)
+    assert len(fused.ops()) == len(plain.ops()) - (32 if model == "resnet50" else 10)
+    assert np.array_equal(got[0], want[0])
 
 
 @pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
