@@ -300,6 +300,11 @@ int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S 
  * memory are still complete on return.
  */
 int onhip_plugin_set_async(int on);
+/* For a caller that hands `eval` weights in device memory and is about to free or overwrite them: drops the re-laid-out
+ * copies the plugin level made of weights whose address lies in [base, base + bytes), so that other data at the same
+ * address later is packed afresh.  The device-resident runtime calls it when a net is freed.  No counterpart in the
+ * reference (its weights live in host vectors for the life of the process). */
+int onhip_plugin_forget(const void *base, size_t bytes);
 /* Drops the device copies of weights the plugin level keeps between calls. */
 int onhip_plugin_release(void);
 

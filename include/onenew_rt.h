@@ -65,9 +65,13 @@ int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, cons
  * after a Conv the same way (tools/optimize/op_fusion.hpp:47-222).  Results are bit-identical to the separate
  * operators.  The fused call runs at the Add's place in the order; the operands folded away stay in the operand
  * table and read as the block's result.  Setting the environment variable ONENEW_RT_FUSE=0 before loading keeps
- * every operator separate, for layer-by-layer comparison.  n_blocks: how many blocks were folded.
+ * every operator separate, for layer-by-layer comparison.
+ *
+ * A Relu that alone reads the result of a Conv with a bias and no activation is folded first, the way that
+ * optimiser does it: the node goes and the Conv's act_type becomes RELU (a file that has been through the optimiser
+ * has none left).  n_blocks / n_relus (either may be NULL): how many residual blocks / Relu nodes were folded.
  */
-int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks);
+int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int32_t *n_relus);
 
 /* Operators in execution order (host/net.h:309-330): type and name of number idx, count through n_ops. */
 int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops);

@@ -711,6 +711,24 @@ int onhip_plugin_set_async(int on) {
     return ONHIP_OK;
 }
 
+int onhip_plugin_forget(const void *base, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    const char *lo = static_cast<const char *>(base), *hi = lo + bytes;
+    bool any = false;
+    for (auto it = g_packed.begin(); it != g_packed.end();) {
+        const char *k = static_cast<const char *>(it->first);
+        if (k >= lo && k < hi) {
+            if (!any) ONHIP_CHECK_HIP(hipDeviceSynchronize());   // a kernel may still be reading the copy
+            any = true;
+            (void) hipFree(it->second.dev);
+            it = g_packed.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    return ONHIP_OK;
+}
+
 int onhip_plugin_release(void) {
     std::lock_guard<std::mutex> lock(g_mu);
     ONHIP_CHECK_HIP(hipDeviceSynchronize());

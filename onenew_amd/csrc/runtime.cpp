@@ -124,6 +124,7 @@ struct Node {
 };
 
 typedef int (*set_async_fn)(int);
+typedef int (*forget_fn)(const void *, size_t);
 
 }  // namespace
 
@@ -137,8 +138,10 @@ struct onrt_net {
     std::string lib_dir;
     std::map<std::string, void *> handles;
     std::vector<set_async_fn> async_switches;
+    std::set<forget_fn> forgetters;   // plugins that keep re-laid-out copies of device-resident weights
+    size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    int fused_blocks = 0;
+    int fused_blocks = 0, folded_relus = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -378,6 +381,7 @@ int allocate(onrt_net &net) {
         if (kv.second.is_init) init_total += (kv.second.bytes + 255) & ~(size_t) 255;
     if (init_total) {
         ONRT_HIP(hipMalloc(&net.init_arena, init_total));
+        net.init_bytes = init_total;
         size_t off = 0;
         for (auto &kv : net.tensors) {
             Tensor &t = kv.second;
@@ -408,9 +412,10 @@ int allocate(onrt_net &net) {
     for (auto &kv : net.tensors) {
         Tensor &t = kv.second;
         if (t.alias.empty()) continue;
-        const Tensor &target = net.tensors[t.alias];
-        t.dev = target.dev;
-        t.bytes = target.bytes;
+        const Tensor *target = &net.tensors[t.alias];
+        while (!target->alias.empty()) target = &net.tensors[target->alias];   // a folded Relu inside a folded block
+        t.dev = target->dev;
+        t.bytes = target->bytes;
     }
     // a view shares the buffer of its input (host/op.h:149-154), in execution order so that chains resolve
     for (int idx : net.order) {
@@ -475,6 +480,7 @@ int bind_plugins(onrt_net &net) {
             it = net.handles.emplace(type, h).first;
             // our plugins can leave a device-resident output to stream order instead of waiting for it
             if (set_async_fn f = reinterpret_cast<set_async_fn>(dlsym(h, "onhip_plugin_set_async"))) net.async_switches.push_back(f);
+            if (forget_fn f = reinterpret_cast<forget_fn>(dlsym(h, "onhip_plugin_forget"))) net.forgetters.insert(f);
         }
         nd.eval = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval"));
         if (!nd.eval) return fail(ONRT_ERR_PLUGIN, "no eval in the %s plugin", type.c_str());
@@ -486,6 +492,58 @@ int bind_plugins(onrt_net &net) {
     return ONRT_OK;
 }
 
+// ---- Relu after Conv ------------------------------------------------------------------------------------
+// What the reference's offline optimiser does to Conv -> Relu (tools/optimize/op_fusion.hpp:47-222: the Relu node goes
+// and the Conv's act_type becomes RELU), done at load time for a file that has not been through it.  Only where the
+// reference's kernel would apply the activation: a convolution with a bias (conv.c:18-27 returns before do_act without
+// one) and no activation yet, whose result only the Relu reads.  As in the optimised file, the activation is then
+// do_act's "x > 0 ? x : 0" (a NaN becomes 0) instead of relu.c's vector rule.  ONENEW_RT_FUSE=0 leaves the file as it is.
+bool fusing_enabled() {
+    const char *env = getenv("ONENEW_RT_FUSE");
+    return !(env && !strcmp(env, "0"));
+}
+
+bool is_net_output(const onrt_net &net, const std::string &name) {
+    return std::find(net.out_names.begin(), net.out_names.end(), name) != net.out_names.end();
+}
+
+// index of the only node reading `name`, if it is of the given type and the operand is not a net output; else -1
+int sole_reader(const onrt_net &net, const std::string &name, const char *type) {
+    if (is_net_output(net, name)) return -1;
+    int found = -1;
+    for (int idx : net.order)
+        for (const std::string &in : net.nodes[idx].in)
+            if (in == name) {
+                if (found >= 0) return -1;   // a second reader, or the same node twice
+                found = idx;
+            }
+    if (found < 0 || strcmp(net.nodes[found].kind->type, type)) return -1;
+    return found;
+}
+
+int fold_relu_into_conv(onrt_net &net) {
+    if (!fusing_enabled()) return ONRT_OK;
+    std::vector<bool> dropped(net.nodes.size(), false);
+    for (int idx : net.order) {
+        Node &conv = net.nodes[idx];
+        if (strcmp(conv.kind->type, "Conv") || conv.out.size() != 1) continue;
+        CONV_CONFIG_S *cfg = reinterpret_cast<CONV_CONFIG_S *>(conv.cfg.data());
+        if (!cfg->has_bias || cfg->act_type != NOT_ACT) continue;
+        const int ri = sole_reader(net, conv.out[0], "Relu");
+        if (ri < 0 || net.nodes[ri].in.size() != 1 || net.nodes[ri].out.size() != 1) continue;
+        cfg->act_type = RELU;
+        conv.fused_out = net.nodes[ri].out[0];
+        net.tensors[conv.out[0]].alias = conv.fused_out;
+        dropped[ri] = true;
+        ++net.folded_relus;
+    }
+    std::vector<int> order;
+    for (int idx : net.order)
+        if (!dropped[idx]) order.push_back(idx);
+    net.order.swap(order);
+    return ONRT_OK;
+}
+
 // ---- residual blocks ------------------------------------------------------------------------------------
 // Conv -> Add (-> Relu), where the convolution's result has no other reader and the other operand of the Add has the
 // same shape, becomes one call of the Conv plugin's `eval_add` / `eval_add_relu`: the sum is formed in the
@@ -494,27 +552,14 @@ int bind_plugins(onrt_net &net) {
 // The fused call takes the place of the Add in the order, where both of its inputs are complete.  The operands
 // folded away read as the block's result.  ONENEW_RT_FUSE=0 keeps every operator separate (layer-by-layer dumps).
 int fuse_residual_blocks(onrt_net &net) {
-    const char *env = getenv("ONENEW_RT_FUSE");
-    if ((env && !strcmp(env, "0")) || !net.conv_add) return ONRT_OK;
-    std::map<std::string, std::vector<int>> readers;
-    for (int idx : net.order)
-        for (const std::string &name : net.nodes[idx].in)
-            if (!name.empty()) readers[name].push_back(idx);
-    auto is_net_output = [&](const std::string &name) {
-        return std::find(net.out_names.begin(), net.out_names.end(), name) != net.out_names.end();
-    };
-    auto sole_reader = [&](const std::string &name, const char *type) -> int {
-        auto it = readers.find(name);
-        if (is_net_output(name) || it == readers.end() || it->second.size() != 1) return -1;
-        return strcmp(net.nodes[it->second[0]].kind->type, type) ? -1 : it->second[0];
-    };
+    if (!fusing_enabled() || !net.conv_add) return ONRT_OK;
     std::map<int, int> runs_instead;   // Add node -> the Conv that takes its place
     std::vector<bool> dropped(net.nodes.size(), false);
     for (int idx : net.order) {
         Node &conv = net.nodes[idx];
         if (strcmp(conv.kind->type, "Conv") || conv.out.size() != 1 || conv.in.size() > 3) continue;
-        const std::string &mid = conv.out[0];
-        const int ai = sole_reader(mid, "Add");
+        const std::string mid = conv.fused_out.empty() ? conv.out[0] : conv.fused_out;   // after a folded Relu
+        const int ai = sole_reader(net, mid, "Add");
         if (ai < 0 || runs_instead.count(ai)) continue;
         Node &add = net.nodes[ai];
         if (add.in.size() != 2 || add.out.size() != 1 || add.in[0] == add.in[1]) continue;
@@ -526,13 +571,15 @@ int fuse_residual_blocks(onrt_net &net) {
         conv.fuse = 1;
         conv.addend = other;
         conv.fused_out = add.out[0];
-        const int ri = net.conv_add_relu ? sole_reader(add.out[0], "Relu") : -1;
+        const int ri = net.conv_add_relu ? sole_reader(net, add.out[0], "Relu") : -1;
         if (ri >= 0 && net.nodes[ri].in.size() == 1 && net.nodes[ri].out.size() == 1) {
             conv.fuse = 2;
             conv.fused_out = net.nodes[ri].out[0];
             dropped[ri] = true;
             net.tensors[add.out[0]].alias = conv.fused_out;
         }
+        // everything folded away on the way reads as the block's result
+        net.tensors[conv.out[0]].alias = conv.fused_out;
         net.tensors[mid].alias = conv.fused_out;
         conv.eval = conv.fuse == 2 ? net.conv_add_relu : net.conv_add;
         dropped[idx] = true;
@@ -569,7 +616,7 @@ int fill_slots(onrt_net &net) {
         if (nd.fuse) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
-            Tensor &t = net.tensors[nd.fuse ? nd.fused_out : nd.out[k]];
+            Tensor &t = net.tensors[nd.fused_out.empty() ? nd.out[k] : nd.fused_out];
             if (out_slot >= BUF_MAXNUM - 1) return fail(ONRT_ERR_FORMAT, "%s: too many operands", nd.base()->op_name);
             nd.params[out_slot].addr = (int64_t) &t.desc;
             nd.outputs[k].addr = (int64_t) t.dev;
@@ -592,6 +639,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
     if (!rc) rc = bind_plugins(net);
+    if (!rc) rc = fold_relu_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = allocate(net);
     if (!rc) rc = build_tables(net);
@@ -642,6 +690,9 @@ ONRT_API int onrt_net_load_file(const char *one_path, const char *op_lib_dir, on
 ONRT_API void onrt_net_free(onrt_net_t *net) {
     if (!net) return;
     (void) hipDeviceSynchronize();
+    // the plugins key their packed copies of the weights by device address: that address is about to be free for reuse
+    if (net->init_arena)
+        for (forget_fn f : net->forgetters) (void) f(net->init_arena, net->init_bytes);
     if (net->init_arena) (void) hipFree(net->init_arena);
     if (net->act_arena) (void) hipFree(net->act_arena);
     if (net->tables) (void) hipFree(net->tables);
@@ -670,9 +721,10 @@ ONRT_API int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops) {
     return ONRT_OK;
 }
 
-ONRT_API int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks) {
-    if (!net || !n_blocks) return fail(ONRT_ERR_ARG, "null argument");
-    *n_blocks = (int32_t) net->fused_blocks;
+ONRT_API int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int32_t *n_relus) {
+    if (!net) return fail(ONRT_ERR_ARG, "null argument");
+    if (n_blocks) *n_blocks = (int32_t) net->fused_blocks;
+    if (n_relus) *n_relus = (int32_t) net->folded_relus;
     return ONRT_OK;
 }
 

@@ -38,7 +38,7 @@ def load():
     L.onrt_net_io_info.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(C.c_char_p), i32p, i32p]
     L.onrt_net_op_count.argtypes = [vp, i32p]
     L.onrt_net_op_info.argtypes = [vp, C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
-    L.onrt_net_fused_count.argtypes = [vp, i32p]
+    L.onrt_net_fused_count.argtypes = [vp, i32p, i32p]
     L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
     L.onrt_net_run.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
     _lib = L
@@ -87,7 +87,13 @@ class Net:
     def fused_blocks(self):
         """number of Conv -> Add (-> Relu) groups the loader folded into one call"""
         n = C.c_int32()
-        _check(load().onrt_net_fused_count(self._h, C.byref(n)), "onrt_net_fused_count")
+        _check(load().onrt_net_fused_count(self._h, C.byref(n), None), "onrt_net_fused_count")
+        return n.value
+
+    def folded_relus(self):
+        """number of Relu nodes folded into the Conv in front of them (act_type RELU, as the offline optimiser does)"""
+        n = C.c_int32()
+        _check(load().onrt_net_fused_count(self._h, None, C.byref(n)), "onrt_net_fused_count")
         return n.value
 
     def operand(self, name):

@@ -100,6 +100,24 @@ def test_second_run_and_device_pointers(torch_dev):
     assert _close(net.fetch("logits"), ref2, 5e-4)
 
 
+def test_weights_of_a_freed_net_are_forgotten(torch_dev):
+    """nets of one shape with different weights, loaded and freed one after the other: the allocator hands the next
+    net the address the last one's weights had, and the Conv plugin must not run it on the packed copy it kept of
+    those"""
+    for seed in range(4):
+        rng = np.random.default_rng(100 + seed)
+        m = onefile.OneModel()
+        m.input("x", (1, 8, 10, 10))
+        m.conv("c", "x", (rng.normal(size=(8, 8, 3, 3)) * 0.2).astype(np.float32), rng.normal(size=8).astype(np.float32),
+               "y", pad=1)
+        m.output("y", (1, 8, 10, 10))
+        x = rng.normal(size=(1, 8, 10, 10)).astype(np.float32)
+        net = rt.Net(m.tobytes())
+        (y,) = net.run(x)
+        assert _close(y, one_model.run(m.tobytes(), [x])[0], 2e-4), seed
+        net.close()
+
+
 def test_batched_input_keeps_its_batch(torch_dev):
     """the reference host fixes Conv and GlobalAveragePool outputs to batch 1; this runtime carries the input's batch
     through (the plugins already take it from the operand descriptor), image by image equal to batch-1 runs"""
@@ -222,6 +240,27 @@ def _residual_variants():
     m.add("sum", "main_out", _w(rng, 1, 8, 1, 1), "y")
     m.output("y", (2, 8, 12, 12))
     out["add_of_a_broadcast_initialiser"] = (m.tobytes(), 0, 0)
+    # a Relu right after a convolution with a bias becomes the convolution's activation, as the offline optimiser
+    # does it; here in front of a residual Add, so the block folds on top of it: three operators fewer
+    m = base()
+    m.conv("pre", "x", _w(rng, 8, 8, 3, 3), _w(rng, 8), "pre_out", pad=1)
+    m.relu("pre_relu", "pre_out", "pre_act")
+    m.add("sum", "pre_act", "x", "s")
+    m.relu("relu", "s", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["relu_folded_then_block_folded"] = (m.tobytes(), 1, 3)
+    # the same Relu after a convolution without a bias stays: the reference's kernel returns before the activation
+    m = base()
+    m.conv("pre", "x", _w(rng, 8, 8, 3, 3), None, "pre_out", pad=1)
+    m.relu("pre_relu", "pre_out", "y")
+    m.output("y", (2, 8, 12, 12))
+    out["relu_after_a_convolution_without_bias"] = (m.tobytes(), 0, 0)
+    m = base()
+    m.conv("pre", "x", _w(rng, 8, 8, 3, 3), _w(rng, 8), "pre_out", pad=1)
+    m.relu("pre_relu", "pre_out", "mid")
+    m.conv("post", "mid", _w(rng, 8, 8, 1, 1), _w(rng, 8), "y", act=abi.RELU)
+    m.output("y", (2, 8, 12, 12))
+    out["relu_between_two_convolutions"] = (m.tobytes(), 0, 1)
     # two convolutions into one Add: one of them is folded, the other runs before it
     m = base()
     m.conv("a", "x", _w(rng, 8, 8, 1, 1), _w(rng, 8), "a_out")
@@ -239,11 +278,21 @@ def test_folding_rules(name, torch_dev, monkeypatch):
     fused, plain, got, want = _both_ways(data, [x], monkeypatch)
     assert fused.fused_blocks() == blocks
     assert len(fused.ops()) == len(plain.ops()) - fewer_ops
+    assert fused.folded_relus() == (1 if name in ("relu_folded_then_block_folded", "relu_between_two_convolutions") else 0)
     for g, w_ in zip(got, want):
         assert np.array_equal(g, w_)
     ref = one_model.run(data, [x])
     for g, r in zip(got, ref):
         assert _close(g, r, 3e-4)
+
+
+def test_relu_after_a_quantised_convolution_is_folded(torch_dev, monkeypatch):
+    """the W8A32 convolution takes the Relu as its activation too, and the integer chain stays exact"""
+    data, ins = one_models.quantised_block()
+    fused, plain, got, want = _both_ways(data, ins, monkeypatch)
+    assert fused.folded_relus() == 1 and len(fused.ops()) == len(plain.ops()) - 1
+    assert np.array_equal(got[0], want[0])
+    assert np.array_equal(got[0], one_model.run(data, ins)[0])
 
 
 @pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
