@@ -300,6 +300,10 @@ int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S 
  * memory are still complete on return.
  */
 int onhip_plugin_set_async(int on);
+/* The stream the evals queue their kernels on; NULL (the initial state) is the default stream.  No counterpart in the
+ * reference.  The device-resident runtime names its own stream for the length of a run so that the run can be
+ * recorded into a HIP graph.  Results into host buffers are still complete on return. */
+int onhip_plugin_set_stream(void *stream);
 /* For a caller that hands `eval` weights in device memory and is about to free or overwrite them: drops the re-laid-out
  * copies the plugin level made of weights whose address lies in [base, base + bytes), so that other data at the same
  * address later is packed afresh.  The device-resident runtime calls it when a net is freed.  No counterpart in the

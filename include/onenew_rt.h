@@ -73,6 +73,20 @@ int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, cons
  */
 int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int32_t *n_relus);
 
+/*
+ * One inference as a HIP graph, on request: with ONENEW_RT_GRAPH=1 in the environment at load time.  The operators
+ * of a net are the same launches with the same addresses on every run, so the second call of onrt_net_run records
+ * them (stream capture on a stream the net owns; the first call has packed the weights, sized the workspaces and
+ * chosen the tiles) and later calls replay the recording with one hipGraphLaunch.  The recorded kernels and their
+ * order are those of the plain run, so are the results.  It is not the default because onrt_net_run returns when
+ * the outputs are complete: launched one by one the first operator starts while the host is still queueing the
+ * rest, a replay starts nothing before the whole graph is submitted, and measured per-inference latency is higher
+ * with it (ResNet-50 batch 1: 0.64 against 0.56 ms).  It pays where the host thread is the bottleneck.  Needs
+ * plugins that export onhip_plugin_set_stream; when recording fails every run launches the operators one by one.
+ * n: replays so far.
+ */
+int onrt_net_graph_launches(const onrt_net_t *net, int64_t *n);
+
 /* Operators in execution order (host/net.h:309-330): type and name of number idx, count through n_ops. */
 int onrt_net_op_count(const onrt_net_t *net, int32_t *n_ops);
 int onrt_net_op_info(const onrt_net_t *net, int32_t idx, const char **op_type, const char **op_name);

@@ -24,9 +24,20 @@ static bool g_ready = false;
 // set by a caller that keeps consuming results on the device in stream order (onhip_plugin_set_async): an eval
 // whose output is device memory then returns without waiting for the kernels
 static bool g_async = false;
+// the stream every eval queues its kernels on: the default stream unless the caller named another
+// (onhip_plugin_set_stream)
+static hipStream_t g_stream = nullptr;
 
 static int wait_for_output() {
-    if (!g_async) ONHIP_CHECK_HIP(hipStreamSynchronize(nullptr));
+    if (!g_async) ONHIP_CHECK_HIP(hipStreamSynchronize(g_stream));
+    return ONHIP_OK;
+}
+
+// result back into a host buffer: the blocking copy orders itself after the default stream and after streams created
+// without hipStreamNonBlocking; a named stream of the other kind is waited for first
+static int copy_out(void *host_out, const void *y, size_t bytes) {
+    if (g_stream) ONHIP_CHECK_HIP(hipStreamSynchronize(g_stream));
+    ONHIP_CHECK_HIP(hipMemcpy(host_out, y, bytes, hipMemcpyDeviceToHost));
     return ONHIP_OK;
 }
 
@@ -91,8 +102,8 @@ static int packed_weights(const onhip_conv_desc_t *d, const float *w_dev, const 
     float *p = nullptr;
     ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&p), bytes));
     int rc = int8 ? onhip_conv2d_w8a32_pack_weights(d, reinterpret_cast<const int8_t *>(w_dev),
-                                                    reinterpret_cast<int8_t *>(p), nullptr)
-                  : onhip_conv2d_pack_weights(d, w_dev, p, nullptr);
+                                                    reinterpret_cast<int8_t *>(p), g_stream)
+                  : onhip_conv2d_pack_weights(d, w_dev, p, g_stream);
     if (rc) { (void) hipFree(p); return rc; }
     g_packed[w_dev] = PackedEntry{p, bytes, int8};
     *out = p;
@@ -264,25 +275,25 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         if (rc) return rc;
         if (wp)
             rc = onhip_conv2d_w8a32_packed(&d, (const float *) x, (const int8_t *) wp, (const int32_t *) b,
-                                           (const float *) aux, (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
+                                           (const float *) aux, (const float *) lut, y, nullptr, ws, ws_bytes, g_stream);
         else
             rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
-                                    (const float *) lut, y, nullptr, ws, ws_bytes, nullptr);
+                                    (const float *) lut, y, nullptr, ws, ws_bytes, g_stream);
         if (!rc && fuse) {   // the int8 store does not fold the addend in: the two operators as passes over y
             onhip_add_desc_t ad;
             memset(&ad, 0, sizeof(ad));
             ad.ndim = 4;
             const int32_t shape[4] = {d.n, d.cout, OH, OW};
             for (int i = 0; i < 4; ++i) ad.large_shape[i] = ad.small_shape[i] = shape[i];
-            rc = onhip_add_f32(&ad, (const float *) y, (const float *) addend, (float *) y, nullptr);
-            if (!rc && fuse == 2) rc = onhip_relu_f32((const float *) y, (float *) y, (long long) (out_bytes / 4), nullptr);
+            rc = onhip_add_f32(&ad, (const float *) y, (const float *) addend, (float *) y, g_stream);
+            if (!rc && fuse == 2) rc = onhip_relu_f32((const float *) y, (float *) y, (long long) (out_bytes / 4), g_stream);
         }
     } else if (fuse) {
         const float *wp = nullptr;
         rc = packed_weights(&d, (const float *) w, &wp);
         if (rc) return rc;
         rc = onhip_conv2d_f32_add(&d, (const float *) x, wp ? wp : (const float *) w, wp ? 1 : 0, (const float *) b,
-                                  (const float *) lut, (const float *) addend, fuse == 2, (float *) y, nullptr);
+                                  (const float *) lut, (const float *) addend, fuse == 2, (float *) y, g_stream);
     } else {
         // k x k dense weights are re-laid out tap-major once, next to their device copy
         const float *wp = nullptr;
@@ -290,13 +301,13 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         if (rc) return rc;
         if (wp)
             rc = onhip_conv2d_f32_packed(&d, (const float *) x, wp, (const float *) b, (const float *) lut, (float *) y,
-                                         nullptr);
+                                         g_stream);
         else
             rc = onhip_conv2d_f32(&d, (const float *) x, (const float *) w, (const float *) b, (const float *) lut,
-                                  (float *) y, nullptr);
+                                  (float *) y, g_stream);
     }
     if (rc) return rc;
-    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, out_bytes, hipMemcpyDeviceToHost));
+    if (!out_on_dev) return copy_out(host_out, y, out_bytes);
     else return wait_for_output();
     return ONHIP_OK;
 }
@@ -348,9 +359,9 @@ static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFF
         rc = stage_buf(2, o_bytes, &y);
         if (rc) return rc;
     }
-    rc = onhip_matmul(&d, (const float *) a, (const float *) b, nullptr, nullptr, (float *) y, nullptr);
+    rc = onhip_matmul(&d, (const float *) a, (const float *) b, nullptr, nullptr, (float *) y, g_stream);
     if (rc) return rc;
-    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, o_bytes, hipMemcpyDeviceToHost));
+    if (!out_on_dev) return copy_out(host_out, y, o_bytes);
     else return wait_for_output();
     return ONHIP_OK;
 }
@@ -381,9 +392,9 @@ static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
         rc = stage_buf(2, o_bytes, &y);
         if (rc) return rc;
     }
-    rc = onhip_gemm_f32(M, K, N, (const float *) a, (const float *) w, (const float *) b, (float *) y, nullptr);
+    rc = onhip_gemm_f32(M, K, N, (const float *) a, (const float *) w, (const float *) b, (float *) y, g_stream);
     if (rc) return rc;
-    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, o_bytes, hipMemcpyDeviceToHost));
+    if (!out_on_dev) return copy_out(host_out, y, o_bytes);
     else return wait_for_output();
     return ONHIP_OK;
 }
@@ -391,7 +402,7 @@ static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
 // ---- Add / Relu / MaxPool / GlobalAveragePool ----------------------------------------------------------
 // an output on the host is computed into a staging buffer and copied back; one on the device is written in place
 static int finish_output(void *host_out, void *y, size_t bytes, bool out_on_dev) {
-    if (!out_on_dev) ONHIP_CHECK_HIP(hipMemcpy(host_out, y, bytes, hipMemcpyDeviceToHost));
+    if (!out_on_dev) return copy_out(host_out, y, bytes);
     else return wait_for_output();
     return ONHIP_OK;
 }
@@ -438,7 +449,7 @@ static int add_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         rc = stage_buf(2, (size_t) nl * 4, &y);
         if (rc) return rc;
     }
-    rc = onhip_add_f32(&d, (const float *) ld, (const float *) sd, (float *) y, nullptr);
+    rc = onhip_add_f32(&d, (const float *) ld, (const float *) sd, (float *) y, g_stream);
     if (rc) return rc;
     return finish_output(host_out, y, (size_t) nl * 4, out_on_dev);
 }
@@ -458,7 +469,7 @@ static int relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
         rc = stage_buf(2, (size_t) n * 4, &y);
         if (rc) return rc;
     }
-    rc = onhip_relu_f32((const float *) x, (float *) y, n, nullptr);
+    rc = onhip_relu_f32((const float *) x, (float *) y, n, g_stream);
     if (rc) return rc;
     return finish_output(host_out, y, (size_t) n * 4, out_on_dev);
 }
@@ -488,7 +499,7 @@ static int maxpool_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUF
         rc = stage_buf(2, out_bytes, &y);
         if (rc) return rc;
     }
-    rc = onhip_maxpool_f32(&d, oh, ow, (const float *) x, (float *) y, nullptr);
+    rc = onhip_maxpool_f32(&d, oh, ow, (const float *) x, (float *) y, g_stream);
     if (rc) return rc;
     return finish_output(host_out, y, out_bytes, out_on_dev);
 }
@@ -509,7 +520,7 @@ static int gap_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         rc = stage_buf(2, out_bytes, &y);
         if (rc) return rc;
     }
-    rc = onhip_global_avgpool_f32(n, c, h, w, (const float *) x, (float *) y, nullptr);
+    rc = onhip_global_avgpool_f32(n, c, h, w, (const float *) x, (float *) y, g_stream);
     if (rc) return rc;
     return finish_output(host_out, y, out_bytes, out_on_dev);
 }
@@ -544,7 +555,7 @@ static int gelu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
     UnaryIo io;
     rc = unary_io(inputs, outputs, (size_t) n * 4, (size_t) n * 4, &io);
     if (rc) return rc;
-    rc = onhip_gelu_lut_f32((const float *) io.x, (const float *) lut, (float *) io.y, n, nullptr);
+    rc = onhip_gelu_lut_f32((const float *) io.x, (const float *) lut, (float *) io.y, n, g_stream);
     if (rc) return rc;
     return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
 }
@@ -574,7 +585,7 @@ static int layernorm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, B
     rc = unary_io(inputs, outputs, (size_t) n * 4, (size_t) n * 4, &io);
     if (rc) return rc;
     rc = onhip_layernorm_f32(rows, reduce, strided, (const float *) io.x, (const float *) w, (const float *) b, (float *) io.y,
-                             nullptr);
+                             g_stream);
     if (rc) return rc;
     return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
 }
@@ -603,7 +614,7 @@ static int softmax_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUF
     UnaryIo io;
     int rc = unary_io(inputs, outputs, (size_t) rows * reduce * 4, (size_t) rows * reduce * 4, &io);
     if (rc) return rc;
-    rc = onhip_softmax_f32((int) rows, reduce, strided, (const float *) io.x, (float *) io.y, nullptr);
+    rc = onhip_softmax_f32((int) rows, reduce, strided, (const float *) io.x, (float *) io.y, g_stream);
     if (rc) return rc;
     return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
 }
@@ -629,7 +640,7 @@ static int transpose_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, B
     UnaryIo io;
     int rc = unary_io(inputs, outputs, (size_t) n * 4, (size_t) n * 4, &io);
     if (rc) return rc;
-    rc = onhip_transpose_f32(&d, (const float *) io.x, (float *) io.y, nullptr);
+    rc = onhip_transpose_f32(&d, (const float *) io.x, (float *) io.y, g_stream);
     if (rc) return rc;
     return finish_output(io.host_out, io.y, io.out_bytes, io.out_on_dev);
 }
@@ -708,6 +719,12 @@ int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_IN
 int onhip_plugin_set_async(int on) {
     std::lock_guard<std::mutex> lock(g_mu);
     g_async = on != 0;
+    return ONHIP_OK;
+}
+
+int onhip_plugin_set_stream(void *stream) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_stream = reinterpret_cast<hipStream_t>(stream);
     return ONHIP_OK;
 }
 

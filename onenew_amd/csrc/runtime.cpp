@@ -125,6 +125,7 @@ struct Node {
 
 typedef int (*set_async_fn)(int);
 typedef int (*forget_fn)(const void *, size_t);
+typedef int (*set_stream_fn)(void *);
 
 }  // namespace
 
@@ -139,6 +140,16 @@ struct onrt_net {
     std::map<std::string, void *> handles;
     std::vector<set_async_fn> async_switches;
     std::set<forget_fn> forgetters;   // plugins that keep re-laid-out copies of device-resident weights
+    std::set<set_stream_fn> stream_setters;
+    size_t plugin_libs = 0;           // libraries bound; a graph needs every one of them to follow set_stream
+    // one inference as a HIP graph: recorded on the net's own stream during the second run (the first one packs
+    // weights, sizes workspaces and measures tile choices, none of which can be recorded), replayed from then on
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    bool graph_wanted = false, graph_failed = false;   // asked for with ONENEW_RT_GRAPH=1
+    bool graph_refused = false;
+    long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
     int fused_blocks = 0, folded_relus = 0;
@@ -481,6 +492,9 @@ int bind_plugins(onrt_net &net) {
             // our plugins can leave a device-resident output to stream order instead of waiting for it
             if (set_async_fn f = reinterpret_cast<set_async_fn>(dlsym(h, "onhip_plugin_set_async"))) net.async_switches.push_back(f);
             if (forget_fn f = reinterpret_cast<forget_fn>(dlsym(h, "onhip_plugin_forget"))) net.forgetters.insert(f);
+            ++net.plugin_libs;
+            if (set_stream_fn f = reinterpret_cast<set_stream_fn>(dlsym(h, "onhip_plugin_set_stream"))) net.stream_setters.insert(f);
+            else net.graph_refused = true;   // a plugin that launches where it likes cannot be recorded
         }
         nd.eval = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval"));
         if (!nd.eval) return fail(ONRT_ERR_PLUGIN, "no eval in the %s plugin", type.c_str());
@@ -646,11 +660,58 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = fill_slots(net);
     net.useful.public_buf_info.public_buf_ptr = 0;
     net.useful.public_buf_info.public_buf_size = 0;
+    if (const char *env = getenv("ONENEW_RT_GRAPH")) net.graph_wanted = !strcmp(env, "1");
+    if (net.stream_setters.empty() || net.graph_refused) net.graph_wanted = false;
+    // a stream of the blocking kind: the synchronous copies either side of a run order themselves against it
+    if (!rc && net.graph_wanted) ONRT_HIP(hipStreamCreate(&net.stream));
     return rc;
 }
 
 void set_async(onrt_net &net, int on) {
     for (set_async_fn f : net.async_switches) f(on);
+}
+
+void set_stream(onrt_net &net, hipStream_t s) {
+    for (set_stream_fn f : net.stream_setters) f(s);
+}
+
+// every operator once, in order, on whatever stream the plugins currently launch on
+int run_operators(onrt_net &net) {
+    for (int idx : net.order) {
+        Node &nd = net.nodes[idx];
+        if (nd.kind->view) continue;
+        const int r = nd.eval(nd.params, nd.inputs, nd.outputs);
+        if (r) return fail(ONRT_ERR_PLUGIN, "%s %s: eval returned %d", nd.kind->type, nd.base()->op_name, r);
+    }
+    return ONRT_OK;
+}
+
+// Records one inference into net.graph_exec.  Relaxed capture mode: the plugins look pointers up
+// (hipPointerGetAttributes) while they queue their kernels.  Any failure leaves the net on plain launches for good.
+int record_graph(onrt_net &net) {
+    if (hipStreamBeginCapture(net.stream, hipStreamCaptureModeRelaxed) != hipSuccess) {
+        (void) hipGetLastError();
+        net.graph_failed = true;
+        return ONRT_OK;
+    }
+    const int rc = run_operators(net);
+    hipGraph_t g = nullptr;
+    const hipError_t e = hipStreamEndCapture(net.stream, &g);
+    if (rc || e != hipSuccess || !g) {
+        (void) hipGetLastError();
+        if (g) (void) hipGraphDestroy(g);
+        net.graph_failed = true;
+        return rc;
+    }
+    if (hipGraphInstantiate(&net.graph_exec, g, nullptr, nullptr, 0) != hipSuccess) {
+        (void) hipGetLastError();
+        (void) hipGraphDestroy(g);
+        net.graph_exec = nullptr;
+        net.graph_failed = true;
+        return ONRT_OK;
+    }
+    net.graph = g;
+    return ONRT_OK;
 }
 
 }  // namespace
@@ -690,6 +751,9 @@ ONRT_API int onrt_net_load_file(const char *one_path, const char *op_lib_dir, on
 ONRT_API void onrt_net_free(onrt_net_t *net) {
     if (!net) return;
     (void) hipDeviceSynchronize();
+    if (net->graph_exec) (void) hipGraphExecDestroy(net->graph_exec);
+    if (net->graph) (void) hipGraphDestroy(net->graph);
+    if (net->stream) (void) hipStreamDestroy(net->stream);
     // the plugins key their packed copies of the weights by device address: that address is about to be free for reuse
     if (net->init_arena)
         for (forget_fn f : net->forgetters) (void) f(net->init_arena, net->init_bytes);
@@ -728,6 +792,12 @@ ONRT_API int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int3
     return ONRT_OK;
 }
 
+ONRT_API int onrt_net_graph_launches(const onrt_net_t *net, int64_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "null argument");
+    *n = net->graph_launches;
+    return ONRT_OK;
+}
+
 ONRT_API int onrt_net_op_info(const onrt_net_t *net, int32_t idx, const char **op_type, const char **op_name) {
     if (!net) return fail(ONRT_ERR_ARG, "null net");
     if (idx < 0 || idx >= (int32_t) net->order.size()) return fail(ONRT_ERR_ARG, "operator index %d of %zu", idx, net->order.size());
@@ -755,21 +825,25 @@ ONRT_API int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *cons
         if (inputs[i] != t.dev) ONRT_HIP(hipMemcpy(t.dev, inputs[i], t.bytes, hipMemcpyDefault));
     }
     set_async(*net, 1);
+    set_stream(*net, net->stream);
     int rc = ONRT_OK;
-    for (int idx : net->order) {
-        Node &nd = net->nodes[idx];
-        if (nd.kind->view) continue;
-        const int r = nd.eval(nd.params, nd.inputs, nd.outputs);
-        if (r) {
-            rc = fail(ONRT_ERR_PLUGIN, "%s %s: eval returned %d", nd.kind->type, nd.base()->op_name, r);
-            break;
+    if (net->stream && !net->graph_exec && !net->graph_failed && net->runs >= 1) rc = record_graph(*net);
+    if (!rc) {
+        if (net->graph_exec) {
+            if (hipGraphLaunch(net->graph_exec, net->stream) != hipSuccess) rc = fail(ONRT_ERR_RUNTIME, "hipGraphLaunch failed");
+            else ++net->graph_launches;
+        } else {
+            rc = run_operators(*net);
         }
     }
+    set_stream(*net, nullptr);
     set_async(*net, 0);
+    ++net->runs;
     if (rc) {
         (void) hipDeviceSynchronize();
         return rc;
     }
+    if (net->stream) ONRT_HIP(hipStreamSynchronize(net->stream));
     bool copied = false;
     for (size_t i = 0; i < net->out_names.size(); ++i) {
         if (!outputs[i]) continue;

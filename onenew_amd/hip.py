@@ -41,7 +41,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
            "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_gelu_eval", "onhip_layernorm_eval",
-           "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_set_async", "onhip_plugin_forget", "onhip_plugin_release"]
+           "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_set_async", "onhip_plugin_set_stream", "onhip_plugin_forget", "onhip_plugin_release"]
 
 
 def load():

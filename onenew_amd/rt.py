@@ -7,7 +7,7 @@ import numpy as np
 from . import hip
 
 EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
-           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count"]
+           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches"]
 
 _lib = None
 
@@ -38,6 +38,7 @@ def load():
     L.onrt_net_io_info.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(C.c_char_p), i32p, i32p]
     L.onrt_net_op_count.argtypes = [vp, i32p]
     L.onrt_net_op_info.argtypes = [vp, C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
+    L.onrt_net_graph_launches.argtypes = [vp, C.POINTER(C.c_int64)]
     L.onrt_net_fused_count.argtypes = [vp, i32p, i32p]
     L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
     L.onrt_net_run.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
@@ -88,6 +89,12 @@ class Net:
         """number of Conv -> Add (-> Relu) groups the loader folded into one call"""
         n = C.c_int32()
         _check(load().onrt_net_fused_count(self._h, C.byref(n), None), "onrt_net_fused_count")
+        return n.value
+
+    def graph_launches(self):
+        """runs so far that replayed the recorded HIP graph of the net"""
+        n = C.c_int64()
+        _check(load().onrt_net_graph_launches(self._h, C.byref(n)), "onrt_net_graph_launches")
         return n.value
 
     def folded_relus(self):

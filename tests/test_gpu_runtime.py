@@ -179,6 +179,35 @@ def test_residual_block_is_folded_into_the_convolution(torch_dev, monkeypatch):
     assert np.array_equal(fused.run(x2)[0], plain.run(x2)[0])
 
 
+@pytest.mark.parametrize("name", list(one_models.MODELS) + ["resnet50", "mobilenetv2"])
+def test_graph_replay_matches_plain_launches(name, torch_dev, monkeypatch):
+    """loaded with ONENEW_RT_GRAPH=1 a net replays a recorded HIP graph of its operators from its second run on: five runs on changing inputs, with
+    unrelated eager work and a device-wide wait between them, each against a net of the same file that launches its
+    operators one by one -- the same bits every time"""
+    torch = torch_dev
+    if name in one_models.MODELS:
+        data, ins = one_models.MODELS[name]()
+    else:
+        from onenew_amd import stacks
+        data, shape, _ = (stacks.resnet50_model if name == "resnet50" else stacks.mobilenet_v2_model)(1)
+        ins = [np.random.default_rng(41).normal(size=shape).astype(np.float32)]
+    plain = rt.Net(data)
+    monkeypatch.setenv("ONENEW_RT_GRAPH", "1")
+    graphed = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_GRAPH")
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for rep in range(5):
+        cur = [(a * np.float32(1.0 - 0.3 * rep) + np.float32(0.05 * rep)).astype(np.float32) for a in ins]
+        got = graphed.run(*cur)
+        scratch.add_(1.0)                       # the program's own work on another stream between the replays
+        torch.cuda.synchronize()
+        want = plain.run(*cur)
+        for g, w_ in zip(got, want):
+            assert np.array_equal(g, w_), (name, rep)
+    assert graphed.graph_launches() == 4 and plain.graph_launches() == 0
+    assert float(scratch[0]) == 5.0
+
+
 def _w(rng, *shape):
     return (rng.normal(size=shape) * 0.2).astype(np.float32)
 
