@@ -124,6 +124,39 @@ __global__ __launch_bounds__(256) void maxpool_kernel(PoolParams p, const float 
     y[o] = m;
 }
 
+// The pooling of a ResNet stem, 3x3 stride 2 padding 1 on rows of a multiple of four floats: a thread produces two
+// neighbouring outputs from one 16-byte load and one single float per input row (columns 4p-1 .. 4p+3 cover both
+// windows), instead of nine single loads per output.  The maximum does not depend on the order of its operands, and a
+// NaN never wins in either kernel, so the results are those of maxpool_kernel bit for bit.
+__global__ __launch_bounds__(256) void maxpool_3x3s2_kernel(PoolParams p, const float *__restrict__ x, float *__restrict__ y,
+                                                            long long pairs, Div31 div_owp) {
+    const long long o = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (o >= pairs) return;
+    const unsigned t = ew_div((unsigned) o, div_owp);
+    const int owp = (int) ((unsigned) o - t * (unsigned) (p.OW / 2));
+    const unsigned plane = ew_div(t, p.div_oh);
+    const int oh = (int) (t - plane * (unsigned) p.OH);
+    const float *src = x + (long long) plane * p.H * p.W + 4 * owp;
+    float m0 = -3276800.0f, m1 = -3276800.0f;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const int ih = 2 * oh - 1 + i;
+        if ((unsigned) ih >= (unsigned) p.H) continue;
+        const float *row = src + (long long) ih * p.W;
+        const float4 v = *reinterpret_cast<const float4 *>(row);
+        if (owp > 0) {
+            const float l = row[-1];
+            m0 = l > m0 ? l : m0;
+        }
+        m0 = v.x > m0 ? v.x : m0;
+        m0 = v.y > m0 ? v.y : m0;
+        m1 = v.y > m1 ? v.y : m1;
+        m1 = v.z > m1 ? v.z : m1;
+        m1 = v.w > m1 ? v.w : m1;
+    }
+    *reinterpret_cast<float2 *>(y + ((long long) plane * p.OH + oh) * p.OW + 2 * owp) = make_float2(m0, m1);
+}
+
 // ---- GlobalAveragePool -------------------------------------------------------------------------------
 // global_avgpool.c:27-42: the elements of a plane are added one after the other in memory order, then the
 // sum is multiplied by 1.0f / (H*W).  A workgroup copies a run of whole planes into LDS (coalesced), then
@@ -255,8 +288,15 @@ int onhip_maxpool_f32(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const 
     const long long total = (long long) p.planes * oh * ow;
     if (total >= (1LL << 31) || (long long) p.planes * d->h * d->w >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "maxpool: tensors of 2^31 elements or more are not supported");
-    hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0,
-                       reinterpret_cast<hipStream_t>(stream), p, x, y, total);
+    if (d->kh == 3 && d->kw == 3 && d->stride_h == 2 && d->stride_w == 2 && d->pad == 1 && d->w % 4 == 0 && ow == d->w / 2 &&
+        aligned16(x) && (reinterpret_cast<uintptr_t>(y) & 7) == 0) {
+        const long long pairs = total / 2;   // ow is even here
+        hipLaunchKernelGGL(maxpool_3x3s2_kernel, dim3((unsigned) ((pairs + 255) / 256)), dim3(256), 0,
+                           reinterpret_cast<hipStream_t>(stream), p, x, y, pairs, make_div31((unsigned) (ow / 2)));
+    } else {
+        hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0,
+                           reinterpret_cast<hipStream_t>(stream), p, x, y, total);
+    }
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }

@@ -713,6 +713,23 @@ def test_maxpool_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
     assert np.array_equal(yb[0], ref[0]) and np.array_equal(yb[1], oracle.maxpool_f32(xb[1:2], k, st, pad)[0])
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 9, 8), (1, 5, 16, 4), (3, 2, 7, 20), (1, 1, 2, 12), (2, 4, 10, 10)])
+def test_maxpool_3x3_stride2_two_outputs_per_thread(shape, torch_dev, oracle):
+    """the stem pooling (3x3, stride 2, padding 1) on rows of a multiple of four floats runs a kernel of its own:
+    odd and even heights, a single column pair, inputs below the reference's start value, NaNs (which never win),
+    and a width that is not a multiple of four (the general kernel) -- all equal to the oracle bit for bit"""
+    torch = torch_dev
+    rng = np.random.default_rng(sum(shape))
+    x = rng.normal(size=shape).astype(np.float32)
+    x[0, 0, 0, :] = -5e6                                   # below -3276800: the start value wins
+    x[-1, -1, -1, 1::3] = np.nan
+    ref = oracle.maxpool_f32(x, 3, 2, 1)
+    d = abi.PoolDesc(shape[0], shape[1], shape[2], shape[3], 3, 3, 2, 2, 1)
+    y = hip.maxpool_f32(d, dev(torch, x))
+    torch.cuda.synchronize()
+    assert _same_bits(y.cpu().numpy(), ref)
+
+
 @pytest.mark.parametrize("name", list(cases.gap_cases()))
 def test_global_avgpool_matches_oracle_and_plugin(name, torch_dev, oracle, golden):
     torch = torch_dev
