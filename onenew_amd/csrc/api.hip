@@ -795,6 +795,17 @@ int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float 
                    void *stream) {
     if (m < 1 || k < 1 || n < 1) return set_error(ONHIP_ERR_ARG, "gemm: bad shape %dx%dx%d", m, k, n);
     if (!a || !w || !bias || !out) return set_error(ONHIP_ERR_ARG, "gemm: null tensor pointer");
+    // Up to eight rows of A the skinny kernel reads the weights once and is bound by that read.  More rows are a
+    // matrix product worth the MFMA kernel: A [m, k] is m images of k channels and one pixel, W [n, k] the weights
+    // of a 1x1 convolution, out [m, n] its NCHW result (measured at k = 2048, n = 1000: 13 us from 16 to 64 rows,
+    // against 21 to 78 us).
+    if (m > 8) {
+        onhip_conv_desc_t d;
+        memset(&d, 0, sizeof(d));
+        d.n = m; d.cin = k; d.h = d.w = 1; d.cout = n; d.kh = d.kw = 1; d.stride_h = d.stride_w = 1;
+        d.group = 1; d.has_bias = 1; d.act_type = NOT_ACT; d.compute = ONHIP_COMPUTE_F32;
+        return conv2d_f32_impl(&d, a, w, 0, bias, nullptr, out, stream);
+    }
     return gemm_nt_launch(m, k, n, a, w, bias, out, reinterpret_cast<hipStream_t>(stream));
 }
 

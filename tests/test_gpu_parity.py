@@ -370,6 +370,17 @@ def test_gemm_f32(name, torch_dev, oracle, golden):
     cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(ref).max()))
 
 
+@pytest.mark.parametrize("shape", [(9, 2048, 1000), (32, 2048, 1000), (33, 1283, 37), (200, 64, 5), (8, 300, 70)])
+def test_gemm_many_rows_runs_as_a_matrix_product(shape, torch_dev, oracle):
+    """more than eight rows of A go through the MFMA kernel (the rows as one-pixel images of a 1x1 convolution), eight
+    and fewer through the skinny kernel; odd K, N below a tile, ragged M"""
+    torch = torch_dev
+    a, w, b = cases.gemm_inputs(f"gemm_rows_{shape}", *shape)
+    y = hip.gemm_f32(dev(torch, a), dev(torch, w), dev(torch, b))
+    torch.cuda.synchronize()
+    assert_close_f32(y.cpu().numpy(), oracle.gemm_f32(a, w, b), tag=str(shape))
+
+
 # ---- the last convolution of a residual block with the Add and the Relu folded into its store ------------------
 
 def _residual_case(kind):
