@@ -312,7 +312,8 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
         if (sscanf(env, "%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb) >= 2) {
             if (c.rowb && !candidate_ok(cfg, p, c)) {   // not a problem for that kernel: the tiled one, same tile if it has it
                 c.rowb = 0;
-                if (c.bn == 256) c.bn = 128;
+                if (c.bn > 128) c.bn = 128;
+                if (c.bm == 96) c.bm = 64;
             }
             if (c.tail > 1 && !candidate_ok(cfg, p, c)) c.tail = 0;   // no leftover to split on this shape
             return launch_choice(cfg, p, c, st);
@@ -366,8 +367,10 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
         }
     }
     // the kernel without LDS for B, where the problem allows it
-    static const int kRowbTiles[][2] = {{64, 128}, {128, 128}, {64, 256}};
-    for (int t = 0; t < 3 && !rc; ++t) {
+    static const int kRowbTiles[][2] = {{64, 128}, {128, 128}, {64, 256}, {96, 128}, {32, 256}, {32, 512}};
+    for (int t = 0; t < 6 && !rc; ++t) {
+        if (kRowbTiles[t][0] == 32 && p.M > 32) continue;   // one row tile of up to 32 output channels
+        if (kRowbTiles[t][0] == 96 && p.M % 96 > 0 && p.M % 96 <= 64) continue;   // a last row tile that a 64-row tile covers as well
         const Choice c = {kRowbTiles[t][0], kRowbTiles[t][1], 1, 0, 1};
         if (!candidate_ok(cfg, p, c)) continue;
         try_choice(c);

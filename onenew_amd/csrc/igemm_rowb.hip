@@ -263,7 +263,8 @@ static int rowb_launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipS
     return ONHIP_OK;
 }
 
-// cfg.bm x cfg.bn names the workgroup tile: 64x128 (2 wavefronts), 128x128 (4, stacked along M), 64x256 (2 x 2)
+// cfg.bm x cfg.bn names the workgroup tile: 64x128 (2 wavefronts), 128x128 (4, stacked along M), 64x256 (2 x 2),
+// 96x128 (3 stacked), 32x256 and 32x512 (2 and 4 side by side)
 int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
     if (!rowb_f32_ok(cfg, p) || (p.dp_tiles > 0) != (cfg.split > 1) || (p.dp_tiles > 0) != (p.partial != nullptr))
         return set_error(ONHIP_ERR_ARG, "igemm: the row-B kernel does not take this problem");
@@ -273,6 +274,9 @@ int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t st
         case 64128: return rowb_launch_one<2, 1>(cfg, p, stream);
         case 128128: return rowb_launch_one<4, 1>(cfg, p, stream);
         case 64256: return rowb_launch_one<2, 2>(cfg, p, stream);
+        case 96128: return rowb_launch_one<3, 1>(cfg, p, stream);   // six-fold channel expansions are multiples of 96
+        case 32256: return rowb_launch_one<1, 2>(cfg, p, stream);   // few output channels (projection layers)
+        case 32512: return rowb_launch_one<1, 4>(cfg, p, stream);
         default: return set_error(ONHIP_ERR_ARG, "igemm: no row-B kernel for tile %dx%d", cfg.bm, cfg.bn);
     }
 }

@@ -198,7 +198,8 @@ def test_forced_tile_and_split_many_items(tile, kind, torch_dev, oracle, monkeyp
                                         # the same through the kernel that reads B straight from memory (1x1 and matmul;
                                         # the 3x3 case falls back to the tiled kernel with the same split)
                                         ("64x128x1x4x1", (34, 32, 34)), ("128x128x1x2x1", (80, 24, 36)),
-                                        ("64x256x1x4x1", (34, 32, 36))])
+                                        ("64x256x1x4x1", (34, 32, 36)), ("96x128x1x4x1", (34, 32, 34)),
+                                        ("32x512x1x8x1", (34, 32, 32))])
 @pytest.mark.parametrize("kind", ["3x3_packed", "1x1", "matmul"])
 def test_leftover_tiles_as_a_split_launch(tile, shape, kind, torch_dev, oracle, monkeypatch):
     """the launch cut along N: whole rounds of 256 tiles unsplit on the caller's stream, the leftover column blocks
@@ -238,7 +239,7 @@ def test_leftover_tiles_as_a_split_launch(tile, shape, kind, torch_dev, oracle, 
     assert hip.split_tail_launches() == before + 3                             # the shape does have leftover tiles
 
 
-@pytest.mark.parametrize("tile", ["64x128x1x0x1", "128x128x1x0x1", "64x256x1x0x1"])
+@pytest.mark.parametrize("tile", ["64x128x1x0x1", "128x128x1x0x1", "64x256x1x0x1", "96x128x1x0x1", "32x256x1x0x1", "32x512x1x0x1"])
 @pytest.mark.parametrize("kind", ["conv_k200_m100", "conv_silu_k64", "conv_nobias", "matmul_batched_bias_gelu", "matmul_shared",
                                   "not_applicable"])
 def test_kernel_with_b_straight_from_memory(tile, kind, torch_dev, oracle, monkeypatch):
