@@ -16,7 +16,7 @@
 namespace onhip {
 
 constexpr int DW_THREADS = 256;
-constexpr int DW_LDS_FLOATS = 8192;   // 32 KiB of LDS per workgroup: five workgroups per CU
+constexpr int DW_LDS_FLOATS = 8192;   // at most 32 KiB of LDS per workgroup (five per CU); the launch asks for what the chunk needs
 constexpr int DW_RT = 4;              // 3x3 specialisation: output rows per thread
 
 struct DwParams {
@@ -27,6 +27,7 @@ struct DwParams {
     int bands;           // bands per plane (1 when planes_per_wg >= 1)
     int pitch;           // LDS row pitch: W plus the left and right padding columns the filter can touch
     int flat_stage;      // small whole planes: stage by flat index
+    int lds_floats;      // LDS cells of one workgroup's chunk (a multiple of 4)
     unsigned magic_hw, magic_w;   // floor(2^32 / d) + 1 for d = H*W and d = W (d >= 2)
     Div31 div_ow, div_c;          // exact division by OW and by C
     Div31 div_unit;               // whole-plane mode: by the work units (strips or outputs) of one plane
@@ -50,7 +51,9 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
                                                                      const void *__restrict__ bv,
                                                                      const float *__restrict__ weight_aux, Epilogue ep,
                                                                      void *__restrict__ y, int32_t *__restrict__ acc32) {
-    __shared__ float tile[DW_LDS_FLOATS];
+    // sized by the launch to the chunk (at most DW_LDS_FLOATS): a small chunk leaves LDS for more resident workgroups,
+    // which is what hides the stage -> compute dependency of each one
+    extern __shared__ __align__(16) float tile[];
     const int tid = threadIdx.x;
     int plane0, nplanes, oh0, oh1;
     if (p.planes_per_wg >= 1) {
@@ -260,6 +263,7 @@ static int dw_plan(const onhip_conv_desc_t &d, int OH, int OW, DwParams *p) {
         p->flat_stage = d.w < 32 && d.w >= 2 && d.h * d.w >= 2 && (long long) ppw * d.h * d.w * d.h * d.w < (1LL << 32);
         p->magic_hw = (unsigned) (0x100000000ULL / (unsigned) (d.h * d.w)) + 1u;
         p->magic_w = (unsigned) (0x100000000ULL / (unsigned) d.w) + 1u;
+        p->lds_floats = (ppw * plane_cells + 3) / 4 * 4;
         return (p->planes + ppw - 1) / ppw;
     }
     // bands of output rows: (band_rows - 1) * sh + kh tile rows must fit
@@ -274,6 +278,7 @@ static int dw_plan(const onhip_conv_desc_t &d, int OH, int OW, DwParams *p) {
     p->planes_per_wg = 0;
     p->band_rows = band;
     p->bands = (OH + band - 1) / band;
+    p->lds_floats = (((band - 1) * d.stride_h + d.kh) * p->pitch + 3) / 4 * 4;
     return p->planes * p->bands;
 }
 
@@ -282,7 +287,7 @@ static void dw_dispatch(int s3, int epi, unsigned wgs, hipStream_t stream, const
                         const void *b, const float *aux, const Epilogue &ep, void *y, int32_t *acc32) {
 #define ONHIP_DW_CASE(S, E)                                                                                             \
     if (s3 == S && epi == E) {                                                                                          \
-        hipLaunchKernelGGL((depthwise_tiled_kernel<INT8, S, E>), dim3(wgs), dim3(DW_THREADS), 0, stream, p, x, w, b, aux, \
+        hipLaunchKernelGGL((depthwise_tiled_kernel<INT8, S, E>), dim3(wgs), dim3(DW_THREADS), (size_t) p.lds_floats * 4, stream, p, x, w, b, aux, \
                            ep, y, acc32);                                                                               \
         return;                                                                                                         \
     }
