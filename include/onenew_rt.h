@@ -47,6 +47,15 @@ const char *onrt_last_error(void);
 int onrt_net_load_file(const char *one_path, const char *op_lib_dir, onrt_net_t **net);
 int onrt_net_load_buf(const void *one_buf, size_t bytes, const char *op_lib_dir, onrt_net_t **net);
 
+/*
+ * The host-side half of loading, without plugins, device or memory: reads the file, orders the nodes, infers the
+ * shapes and folds what the loader folds when the Conv plugin of this package is bound.  The result answers
+ * onrt_net_io_count / _io_info / _op_count / _op_info / _operand (addresses NULL) / _fused_count and is released
+ * with onrt_net_free; onrt_net_run refuses it.  For tools that want to know what a model will run as, and for
+ * checking a file on a machine without a GPU.
+ */
+int onrt_net_plan_buf(const void *one_buf, size_t bytes, onrt_net_t **net);
+
 /* Releases the device memory of the net and its operator objects (host/net.h:401-416). */
 void onrt_net_free(onrt_net_t *net);
 

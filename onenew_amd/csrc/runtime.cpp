@@ -149,6 +149,7 @@ struct onrt_net {
     hipGraphExec_t graph_exec = nullptr;
     bool graph_wanted = false, graph_failed = false;   // asked for with ONENEW_RT_GRAPH=1
     bool graph_refused = false;
+    bool plan_only = false;           // onrt_net_plan_buf: no plugins, no device memory
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
@@ -667,6 +668,20 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     return rc;
 }
 
+int plan_stub_eval(BUFFER_INFO_S *, BUFFER_INFO_S *, BUFFER_INFO_S *) { return ONRT_ERR_ARG; }
+
+// the host-side part of prepare: what would run, in which order, on which shapes
+int plan(onrt_net &net) {
+    net.plan_only = true;
+    int rc = read_model(net);
+    if (!rc) rc = order_nodes(net);
+    if (!rc) rc = infer_shapes(net);
+    net.conv_add = net.conv_add_relu = plan_stub_eval;   // as with the Conv plugin of this package
+    if (!rc) rc = fold_relu_into_conv(net);
+    if (!rc) rc = fuse_residual_blocks(net);
+    return rc;
+}
+
 void set_async(onrt_net &net, int on) {
     for (set_async_fn f : net.async_switches) f(on);
 }
@@ -736,6 +751,17 @@ ONRT_API int onrt_net_load_buf(const void *one_buf, size_t bytes, const char *op
     return ONRT_OK;
 }
 
+ONRT_API int onrt_net_plan_buf(const void *one_buf, size_t bytes, onrt_net_t **out) {
+    if (!one_buf || !out) return fail(ONRT_ERR_ARG, "plan: null argument");
+    *out = nullptr;
+    std::unique_ptr<onrt_net> net(new onrt_net);
+    net->file.assign(static_cast<const char *>(one_buf), static_cast<const char *>(one_buf) + bytes);
+    const int rc = plan(*net);
+    if (rc) return rc;
+    *out = net.release();
+    return ONRT_OK;
+}
+
 ONRT_API int onrt_net_load_file(const char *one_path, const char *op_lib_dir, onrt_net_t **out) {
     if (!one_path || !out) return fail(ONRT_ERR_ARG, "load: null argument");
     FILE *f = fopen(one_path, "rb");
@@ -750,6 +776,10 @@ ONRT_API int onrt_net_load_file(const char *one_path, const char *op_lib_dir, on
 
 ONRT_API void onrt_net_free(onrt_net_t *net) {
     if (!net) return;
+    if (net->plan_only) {
+        delete net;
+        return;
+    }
     (void) hipDeviceSynchronize();
     if (net->graph_exec) (void) hipGraphExecDestroy(net->graph_exec);
     if (net->graph) (void) hipGraphDestroy(net->graph);
@@ -819,6 +849,7 @@ ONRT_API int onrt_net_operand(const onrt_net_t *net, const char *name, int32_t *
 
 ONRT_API int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs) {
     if (!net || (!inputs && !net->in_names.empty()) || (!outputs && !net->out_names.empty())) return fail(ONRT_ERR_ARG, "run: null argument");
+    if (net->plan_only) return fail(ONRT_ERR_ARG, "run: this net is a plan (onrt_net_plan_buf): load it to run it");
     for (size_t i = 0; i < net->in_names.size(); ++i) {
         if (!inputs[i]) return fail(ONRT_ERR_ARG, "run: input %zu is null", i);
         const Tensor &t = net->tensors[net->in_names[i]];

@@ -7,7 +7,7 @@ import numpy as np
 from . import hip
 
 EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
-           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches"]
+           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf"]
 
 _lib = None
 
@@ -38,6 +38,7 @@ def load():
     L.onrt_net_io_info.argtypes = [vp, C.c_int32, C.c_int32, C.POINTER(C.c_char_p), i32p, i32p]
     L.onrt_net_op_count.argtypes = [vp, i32p]
     L.onrt_net_op_info.argtypes = [vp, C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
+    L.onrt_net_plan_buf.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(vp)]
     L.onrt_net_graph_launches.argtypes = [vp, C.POINTER(C.c_int64)]
     L.onrt_net_fused_count.argtypes = [vp, i32p, i32p]
     L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
@@ -55,11 +56,15 @@ class Net:
     """A loaded model.  ``model`` is a path or the bytes of a .one file; ``op_lib_dir`` defaults to the directory
     of the built plugins."""
 
-    def __init__(self, model, op_lib_dir=None):
+    def __init__(self, model, op_lib_dir=None, plan_only=False):
+        """plan_only: the host-side half only (order, shapes, folding) -- needs no GPU, cannot run"""
         L = load()
         self._h = C.c_void_p()
         d = (op_lib_dir or os.path.dirname(lib_path())).encode()
-        if isinstance(model, (bytes, bytearray, memoryview)):
+        if plan_only:
+            data = bytes(model) if isinstance(model, (bytes, bytearray, memoryview)) else open(os.fspath(model), "rb").read()
+            _check(L.onrt_net_plan_buf(data, len(data), C.byref(self._h)), "onrt_net_plan_buf")
+        elif isinstance(model, (bytes, bytearray, memoryview)):
             data = bytes(model)
             _check(L.onrt_net_load_buf(data, len(data), d, C.byref(self._h)), "onrt_net_load_buf")
         else:

@@ -131,3 +131,79 @@ def test_loader_rejects_damaged_descriptors():
     rc, msg = _load_error(view.tobytes())
     assert rc == -2 and "Reshape" in msg
 
+
+
+# ---- the host-side half of the runtime (order, shape inference, folding) on the CPU -----------------------------
+
+@pytest.mark.parametrize("name", list(one_models.MODELS))
+def test_plan_infers_the_shapes_the_oracle_computes(name, monkeypatch):
+    """onrt_net_plan_buf needs no GPU: with folding off every operand of every test model gets the shape the oracle's
+    execution of the file produces, in an order in which every input is ready"""
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    data, ins = one_models.MODELS[name]()
+    net = rt.Net(data, plan_only=True)
+    m = onefile.parse(data)
+    ref = one_model.run(data, ins, keep_all=True)
+    assert net.outputs == [(n, tuple(s)) for n, s in m["outputs"]]
+    assert sorted(t for t, _ in net.ops()) == sorted(t for t, _ in m["nodes"])
+    produced = {n for n, _ in m["inputs"]}
+    by_name = {cfg.op_base_cfg.op_name.decode(): cfg for _, cfg in m["nodes"]}
+    for _, op_name in net.ops():
+        cfg = by_name[op_name].op_base_cfg
+        for k in range(cfg.in_operand_num):
+            iname = cfg.in_operand_name[k].value.decode()
+            assert iname in produced or iname not in ref or iname.startswith(op_name + "."), (op_name, iname)
+        oname = cfg.out_operand_name[0].value.decode()
+        produced.add(oname)
+        shape, ptr = net.operand(oname)
+        assert ptr is None and tuple(shape) == tuple(ref[oname].shape), oname
+    with pytest.raises(rt.OnrtError, match="plan"):
+        net.run(*ins)
+    net.close()
+
+
+def test_plan_folds_residual_blocks_and_relus():
+    from onenew_amd import stacks
+    data, _ = one_models.resnet_block()
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 1 and net.folded_relus() == 0
+    types = [t for t, _ in net.ops()]
+    assert "Add" not in types and types.count("Relu") == 0 and len(types) == len(onefile.parse(data)["nodes"]) - 2
+    data, _ = one_models.quantised_block()
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 0 and net.folded_relus() == 1
+    # the full-size models: 16 bottleneck blocks, 10 inverted-residual connections
+    data, shape, _ = stacks.resnet50_model(2)
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 16 and len(net.ops()) == 89 - 32
+    assert net.inputs[0][1] == tuple(shape) and net.outputs[0][1] == (2, 1000)
+    data, shape, _ = stacks.mobilenet_v2_model(3)
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 10 and len(net.ops()) == 65 - 10
+    assert net.outputs[0][1] == (3, 1000)
+
+
+def test_plan_keeps_what_must_not_be_folded(monkeypatch):
+    """a convolution whose result is a net output, or has two readers, or meets a broadcast Add, stays as it is; with
+    ONENEW_RT_FUSE=0 so does everything"""
+    rng = np.random.default_rng(1)
+    w = lambda *s: (rng.normal(size=s) * 0.2).astype(np.float32)   # noqa: E731
+    m = onefile.OneModel()
+    m.input("x", (1, 4, 6, 6))
+    m.conv("a", "x", w(4, 4, 1, 1), w(4), "a_out")
+    m.add("s1", "a_out", "x", "y1")                    # a_out is also an output
+    m.conv("b", "x", w(4, 4, 1, 1), w(4), "b_out")
+    m.add("s2", "b_out", w(1, 4, 1, 1), "y2")          # broadcast of a per-channel initialiser
+    m.conv("c", "x", w(4, 4, 1, 1), w(4), "c_out")
+    m.add("s3", "c_out", "x", "t3")
+    m.add("s4", "t3", "c_out", "y3")                   # c_out read twice
+    m.conv("d", "x", w(4, 4, 1, 1), None, "d_out")
+    m.relu("r", "d_out", "y4")                         # no bias: the reference kernel skips the activation
+    for n in ("a_out", "y1", "y2", "y3", "y4"):
+        m.output(n, (1, 4, 6, 6))
+    net = rt.Net(m.tobytes(), plan_only=True)
+    assert net.fused_blocks() == 0 and net.folded_relus() == 0 and len(net.ops()) == 9
+    data, _ = one_models.resnet_block()
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 0 and len(net.ops()) == len(onefile.parse(data)["nodes"])
