@@ -302,6 +302,8 @@ int infer_shapes(onrt_net &net) {
             auto it = net.tensors.find(nd.in[k]);
             return it != net.tensors.end() && it->second.is_init ? &it->second : nullptr;
         };
+        if (nd.in[0].empty() || !sane_rank(in))
+            return fail(ONRT_ERR_FORMAT, "%s %s: first input of rank %d", type, nd.base()->op_name, in.dim_num_of_shapes);
         memcpy(out.shapes, in.shapes, sizeof(out.shapes));
         out.dim_num_of_shapes = in.dim_num_of_shapes;
         if (!strcmp(type, "Conv")) {   // host/ops/conv.h:31-58
@@ -328,6 +330,8 @@ int infer_shapes(onrt_net &net) {
         } else if (!strcmp(type, "MatMul")) {   // host/ops/mat_mul.h:32-57
             if (nd.in.size() < 2) return fail(ONRT_ERR_FORMAT, "MatMul %s: one input", nd.base()->op_name);
             const OPERAND_S &b = net.tensors[nd.in[1]].desc;
+            if (nd.in[1].empty() || !sane_rank(b))
+                return fail(ONRT_ERR_FORMAT, "MatMul %s: second input of rank %d", nd.base()->op_name, b.dim_num_of_shapes);
             out.shapes[out.dim_num_of_shapes - 1] = b.shapes[b.dim_num_of_shapes - 1];
         } else if (!strcmp(type, "Add")) {   // host/ops/add.h:32-57
             if (nd.in.size() < 2) return fail(ONRT_ERR_FORMAT, "Add %s: one input", nd.base()->op_name);

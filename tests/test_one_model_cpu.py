@@ -207,3 +207,22 @@ def test_plan_keeps_what_must_not_be_folded(monkeypatch):
     monkeypatch.setenv("ONENEW_RT_FUSE", "0")
     net = rt.Net(data, plan_only=True)
     assert net.fused_blocks() == 0 and len(net.ops()) == len(onefile.parse(data)["nodes"])
+
+
+def test_plan_refuses_a_node_whose_first_input_is_unnamed():
+    """found by fuzzing the plan under the host sanitizers: an empty first input name made a rank-0 operand whose last
+    dimension Gemm and MatMul then indexed"""
+    data, _ = one_models.resnet_block()
+    m = onefile.parse(data)
+    off = m["header"].node_cfg_offset
+    for op_type, cfg in m["nodes"]:
+        if op_type == "Gemm":
+            name_off = off + abi.BASE_CONFIG_S.in_operand_name.offset
+            bad = bytearray(data)
+            bad[name_off:name_off + 8] = b"\0" * 8
+            h = C.c_void_p()
+            rc = rt.load().onrt_net_plan_buf(bytes(bad), len(bad), C.byref(h))
+            assert rc == -2 and not h.value and "first input" in rt.load().onrt_last_error().decode()
+            return
+        off += onefile.align64(C.sizeof(cfg))
+    raise AssertionError("the test model has no Gemm")
