@@ -752,7 +752,6 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     Operands op0, op1;
     constexpr std::true_type CHECKED{};
     constexpr std::false_type UNCHECKED{};
-    static_assert(PF == 1 || B_ITEMS == 0, "scalar B descriptions are prepared one tile ahead: PF == 1 only");
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(0, i);
     issue(0, CHECKED, std::integral_constant<int, 0>{});
@@ -766,7 +765,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         }()), ...);
     }(std::make_integer_sequence<int, PF>{});
 #pragma unroll
-    for (int i = 0; i < B_ITEMS; ++i) prep_item(2, i);
+    for (int i = 0; i < B_ITEMS; ++i) prep_item(PF + 1, i);   // for the first load of the loop: tile 1 + PF
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < READS; ++i) read_operand(op0, 0, i);
@@ -785,7 +784,7 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             }
 #pragma unroll
             for (int i = 0; i < B_ITEMS; ++i)
-                if (STEPS > 1 ? (1 + (i * (STEPS - 1)) / B_ITEMS == st) : true) prep_item(kt + 3, i);
+                if (STEPS > 1 ? (1 + (i * (STEPS - 1)) / B_ITEMS == st) : true) prep_item(kt + 2 + PF, i);   // one body ahead of its issue
             if (st >= HALF) {
 #pragma unroll
                 for (int i = 0; i < READS; ++i)
