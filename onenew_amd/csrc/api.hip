@@ -32,6 +32,7 @@ static unsigned pass_for(unsigned d) { return d <= 1 ? 0xFFFFFFFFu : 0u; }
 
 static Epilogue make_epilogue(const onhip_conv_desc_t &d, const float *lut) {
     Epilogue e;
+    e.qlut = nullptr;
     // conv.c:18-27: a convolution without bias returns before the activation
     e.act = d.has_bias ? d.act_type : NOT_ACT;
     e.clip_min = d.clip_min;
@@ -609,6 +610,34 @@ int onhip_conv2d_w8a32_pack_weights(const onhip_conv_desc_t *d, const int8_t *w8
 
 // packed != 0: w8 holds the layout written by onhip_conv2d_w8a32_pack_weights and the workspace only
 // takes the int8 copy of the activations
+// Tables that have been through an output quantiser, by (table address, 1 / output scale): built on first use on the
+// caller's stream and kept for the life of the process.  The activation tables are constants of the model runtime
+// (host/ops/conv.h:178-194 builds one per process); a caller that rewrites one in place gets the old bytes.
+static std::mutex g_qlut_mu;
+static std::map<std::pair<const float *, uint32_t>, signed char *> g_qlut;
+
+static int quantised_table(const float *lut, float out_inv_scale, hipStream_t st, const signed char **out) {
+    uint32_t bits;
+    memcpy(&bits, &out_inv_scale, 4);
+    std::lock_guard<std::mutex> lock(g_qlut_mu);
+    auto key = std::make_pair(lut, bits);
+    auto it = g_qlut.find(key);
+    if (it == g_qlut.end()) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            *out = nullptr;   // no allocation while a graph is being recorded: the float table serves
+            return ONHIP_OK;
+        }
+        signed char *q = nullptr;
+        ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&q), 8192));
+        int rc = build_qlut_launch(lut, out_inv_scale, q, st);
+        if (rc) { (void) hipFree(q); return rc; }
+        it = g_qlut.emplace(key, q).first;
+    }
+    *out = it->second;
+    return ONHIP_OK;
+}
+
 // xq != nullptr: the activations arrive already quantised (int8 NHWC, channels padded to 16) and x is not read;
 // nhwc_out != 0: the int8 result is written NHWC with its channels padded to 16, ready to be the next xq
 static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8, int packed_w,
@@ -712,6 +741,10 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     p.acc_out = acc32;
     p.out_s8 = d->out_s8;
     p.out_inv_scale = d->out_s8 ? 1.0f / d->output_scale : 0.0f;
+    if (nhwc_out && ep.act == SILU && ep.lut && !acc32) {   // the staged int8 store: gather quantised table entries
+        rc = quantised_table(ep.lut, p.out_inv_scale, st, &p.ep.qlut);
+        if (rc) return rc;
+    }
     return plan_and_launch(cfg, p, st);
 }
 

@@ -91,6 +91,21 @@ int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, 
     return ONHIP_OK;
 }
 
+// ---- the activation table through the output quantiser --------------------------------------------------
+// qlut[i] = quantiser(lut[i]): what the int8 store of a table activation would compute per element, once per table
+// entry.  requant_s8(0) is 0, so the table's "below -8" rule needs no entry of its own.
+__global__ __launch_bounds__(256) void build_qlut_kernel(const float *__restrict__ lut, float out_inv_scale,
+                                                         signed char *__restrict__ qlut) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < 8192) qlut[i] = (signed char) quant_s8(lut[i], out_inv_scale);
+}
+
+int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream) {
+    hipLaunchKernelGGL(build_qlut_kernel, dim3(32), dim3(256), 0, stream, lut, out_inv_scale, qlut);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
 // ---- skinny Gemm: out[m][n] = sum_k a[m][k] * w[n][k] + bias[n]  (device/x86/Gemm/gemm.c:9-79) ---------
 // One wavefront per output column n; lanes stride over k, eight rows of A at a time share each
 // weight load; butterfly reduction over the 64 lanes; the bias is added last.

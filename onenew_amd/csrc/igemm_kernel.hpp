@@ -466,8 +466,18 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
                     float f = __fmul_rn((float) acc[a][b][r], p.in_scale);
                     const float fbias = __fadd_rn(f, (float) b32[a][r]);
                     f = p.bias32 ? fbias : f;
-                    const float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
-                    const int v = (m0 + ml + j < p.M) ? requant_s8(y, p.out_inv_scale) : 0;
+                    const float x = __fmul_rn(f, coeff);
+                    int q8;
+                    if (EPI == EPI_LUT && p.ep.qlut) {   // uniform: the table entry arrives quantised (act_fast<EPI_LUT>'s rules)
+                        int idx = (int) __fmul_rn(__fadd_rn(x, 8.0f), 512.0f);
+                        idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
+                        const int l = p.ep.qlut[idx];
+                        const int hi = requant_s8(x, p.out_inv_scale);
+                        q8 = x < -8.0f ? 0 : x >= 8.0f ? hi : l;
+                    } else {
+                        q8 = requant_s8(act_fast<EPI>(x, p.ep), p.out_inv_scale);
+                    }
+                    const int v = (m0 + ml + j < p.M) ? q8 : 0;
                     packed |= ((unsigned) v & 0xffu) << (8 * j);
                 }
                 const int nl = n_wave - n0 + b * 32 + li;

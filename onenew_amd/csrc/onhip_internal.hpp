@@ -25,6 +25,9 @@ struct Epilogue {
     float leaky_alpha;
     float hs_alpha, hs_beta;
     const float *lut;        // 8192-entry table for SILU (conv) / GELU (matmul), or nullptr
+    // int8 outputs only: the same table already passed through the output quantiser (one byte per entry), so that the
+    // store gathers a byte from 8 KiB instead of a float from 32 KiB and quantises it; nullptr = use `lut`
+    const signed char *qlut;
 };
 
 #define ONHIP_ACT_GELU_LUT 100  // internal: table GELU of device/x86/Gelu/gelu.c, matmul epilogue only
@@ -214,6 +217,7 @@ int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const flo
 int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
                          hipStream_t stream);
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
+int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
 int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, int k_units, int8_t *packed,
                    hipStream_t stream);
 int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,
