@@ -434,7 +434,7 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
 // one pixel with a single 128-bit access instead of 16 single bytes to 16 different pixels.  A lane holds four
 // consecutive channels of a pixel (accumulator registers 4q .. 4q+3), which go to LDS as one dword.  Channels
 // between M and the pitch are written as zero.  stage: BN * (BM + 16) bytes of LDS nobody reads any more.
-template <int EPI, int BM, int BN, int TM, int TN, class ACC>
+template <int EPI, int BM, int BN, int TM, int TN, bool QLUT_IN_LDS, class ACC>
 __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&acc)[TM][TN], unsigned char *stage, int m0,
                                                    int n0, int m_wave, int n_wave, int li, int lh, int tid) {
     constexpr int PITCH = BM + 16;
@@ -451,6 +451,16 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
             aux[a][r] = buf_load_f32(raux, lh16, soff);
             b32[a][r] = (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
         }
+    // the quantised activation table (8 KiB) next to the staging area: byte gathers from LDS instead of memory
+    const signed char *qtab = p.ep.qlut;
+    if (EPI == EPI_LUT && p.ep.qlut && QLUT_IN_LDS) {
+        unsigned char *ql = stage + BN * PITCH;
+        const uint4 *src = reinterpret_cast<const uint4 *>(p.ep.qlut);
+#pragma unroll
+        for (int i = 0; i < 8192 / 16 / THREADS; ++i) reinterpret_cast<uint4 *>(ql)[tid + i * THREADS] = src[tid + i * THREADS];
+        __syncthreads();
+        qtab = reinterpret_cast<const signed char *>(ql);
+    }
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -471,7 +481,7 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
                     if (EPI == EPI_LUT && p.ep.qlut) {   // uniform: the table entry arrives quantised (act_fast<EPI_LUT>'s rules)
                         int idx = (int) __fmul_rn(__fadd_rn(x, 8.0f), 512.0f);
                         idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
-                        const int l = p.ep.qlut[idx];
+                        const int l = qtab[idx];
                         const int hi = requant_s8(x, p.out_inv_scale);
                         q8 = x < -8.0f ? 0 : x >= 8.0f ? hi : l;
                     } else {
@@ -832,16 +842,17 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
         // int8 NHWC output without the raw-accumulator copy: 128-bit stores through LDS (batch is 1 on this path)
         if (p.out_s8 && p.out_mode == OUT_PLAIN && p.c_stride_m == 1 && !p.acc_out) {
             static_assert(sizeof(lds) >= (size_t) BN * (BM + 16), "output staging fits the operand buffers");
+            constexpr bool QL = sizeof(lds) >= (size_t) BN * (BM + 16) + 8192;   // room for the quantised activation table
             unsigned char *stage = reinterpret_cast<unsigned char *>(&lds[0][0]);
             __syncthreads();   // every wavefront is done with the operand buffers
             switch (p.ep.act) {
                 case NOT_ACT:
-                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
-                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
-                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
                 case SILU:
-                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
-                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
             }
             return;
         }
