@@ -101,8 +101,8 @@ static int get_scratch(size_t bytes, void **out) {
 // the reference's grid search over GEMM tiles, tools/optimize/auto_tuning.hpp:9-75).
 static const int kTiles[][2] = {{128, 128}, {64, 128}, {64, 64}, {32, 128}};
 static const int kNumTiles = 4;
-static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
-static const int kNumSplits = 10;
+static const int kSplits[] = {1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 24, 32};
+static const int kNumSplits = 13;
 
 // tail > 1: the tiles left over after whole rounds of 256 are cut `tail` ways along K (launch_choice)
 // rowb != 0: the kernel that feeds B from global memory straight into the MFMAs (igemm_rowb.hip), tile bm x bn
