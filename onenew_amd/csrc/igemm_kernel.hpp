@@ -902,12 +902,37 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const IgemmParams p,
         const float *part = p.partial + idx;
         float acc = 0.0f;
         int s = 0;
-        for (; s + 4 <= split; s += 4) {   // loads four at a time, added in slice order as before
+        // the loads of up to sixteen slices are in flight together (a small problem is one memory round trip, not one
+        // per group of four); the sums are added one after the other in slice order whatever the grouping
+        for (; s + 16 <= split; s += 16) {
+            float a[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) a[i] = part[(size_t) (s + i) * slice];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc = __fadd_rn(acc, a[i]);
+        }
+        if (s + 8 <= split) {
+            float a[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[i] = part[(size_t) (s + i) * slice];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc = __fadd_rn(acc, a[i]);
+            s += 8;
+        }
+        if (s + 4 <= split) {
             const float a0 = part[(size_t) s * slice], a1 = part[(size_t) (s + 1) * slice];
             const float a2 = part[(size_t) (s + 2) * slice], a3 = part[(size_t) (s + 3) * slice];
             acc = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(acc, a0), a1), a2), a3);
+            s += 4;
         }
-        for (; s < split; ++s) acc = __fadd_rn(acc, part[(size_t) s * slice]);
+        if (s < split) {   // up to three left: requested together as well
+            const float a0 = part[(size_t) s * slice];
+            const float a1 = s + 1 < split ? part[(size_t) (s + 1) * slice] : 0.0f;
+            const float a2 = s + 2 < split ? part[(size_t) (s + 2) * slice] : 0.0f;
+            acc = __fadd_rn(acc, a0);
+            if (s + 1 < split) acc = __fadd_rn(acc, a1);
+            if (s + 2 < split) acc = __fadd_rn(acc, a2);
+        }
         if (p.bias_mode == BIAS_M) acc = __fadd_rn(acc, p.bias[m]);
         else if (p.bias_mode == BIAS_N) acc = __fadd_rn(acc, p.bias[n]);
         float y = apply_act(acc, p.ep);
