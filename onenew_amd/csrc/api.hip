@@ -835,7 +835,8 @@ int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float 
     // matrix product worth the MFMA kernel: A [m, k] is m images of k channels and one pixel, W [n, k] the weights
     // of a 1x1 convolution, out [m, n] its NCHW result (measured at k = 2048, n = 1000: 13 us from 16 to 64 rows,
     // against 21 to 78 us).
-    if (m > 8) {
+    const long long lim = 1LL << 29;   // elements: the MFMA kernel addresses an operand with 32-bit byte offsets
+    if (m > 8 && (long long) m * k < lim && (long long) m * n < lim && (long long) n * k < lim) {
         onhip_conv_desc_t d;
         memset(&d, 0, sizeof(d));
         d.n = m; d.cin = k; d.h = d.w = 1; d.cout = n; d.kh = d.kw = 1; d.stride_h = d.stride_w = 1;
