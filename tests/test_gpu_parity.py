@@ -79,6 +79,79 @@ def test_conv_f32(name, torch_dev, oracle, golden):
     cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * scale)
 
 
+def _random_conv(rng, quant):
+    """a convolution the path accepts, drawn at random: filter 1..5 (rectangular now and then), stride 1..3, padding up
+    to the filter's reach, odd channel counts and image sides, batch 1..3, dense or depthwise, any activation"""
+    kh = int(rng.choice([1, 1, 3, 3, 3, 5, 2]))
+    kw = kh if rng.random() < 0.8 else int(rng.choice([1, 3]))
+    s = int(rng.choice([1, 1, 2, 3]))
+    pad = int(rng.integers(0, max(kh, kw) // 2 + 1))
+    depthwise = rng.random() < 0.25
+    cin = int(rng.integers(1, 70))
+    cout = cin if depthwise else int(rng.integers(1, 140))
+    h = int(rng.integers(max(kh, 1), 40))
+    w = int(rng.integers(max(kw, 1), 40))
+    acts = [abi.NOT_ACT, abi.RELU, abi.CLIP, abi.SILU, abi.LEAKYRELU, abi.HARDSILU]
+    act = int(rng.choice(acts))
+    bias = 1 if (depthwise or rng.random() < 0.8) else 0
+    kw_args = dict(clip_min=-0.3, clip_max=0.6, leaky_relu_alpha=0.1, hard_sigmoid_alpha=1.0 / 6, hard_sigmoid_beta=0.5)
+    if quant:
+        pad = min(pad, kh // 2)
+        kw_args["input_scale"] = float(rng.uniform(0.005, 0.05))
+    return cases.cd(cin, cout, (kh, kw), s, pad, h, w, act=act, group=cin if depthwise else 1, bias=bias,
+                    n=int(rng.integers(1, 4)), **kw_args)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_conv_f32_random_shapes(seed, torch_dev, oracle):
+    """forty seeded random convolutions through the measured tile choice and through the cost model's"""
+    torch = torch_dev
+    rng = np.random.default_rng(1000 + seed)
+    d = _random_conv(rng, quant=False)
+    name = f"random_f32_{seed}"
+    x, w, b = cases.conv_inputs(name, d)
+    lut = cases.silu_lut()
+    xd, wd, ld = dev(torch, x), dev(torch, w), dev(torch, lut)
+    bd = dev(torch, b) if b is not None else None
+    table = bool(d.has_bias) and d.act_type == abi.SILU
+    dn = ConvDesc.from_buffer_copy(d)
+    if table:
+        dn.act_type = abi.NOT_ACT                          # judged on the pre-activation: the table is a step function
+    ref = oracle.conv2d_f32(dn, x, w, b, lut)
+    for tune in (0, 1):
+        hip.set_tuning(tune)
+        try:
+            y = hip.conv2d_f32(dn, xd, wd, bd, ld).cpu().numpy()
+            yt = hip.conv2d_f32(d, xd, wd, bd, ld).cpu().numpy() if table else None
+        finally:
+            hip.set_tuning(0)
+        if d.group != 1:
+            assert np.array_equal(y, ref), f"{name}: depthwise differs from the reference's order of operations"
+        else:
+            assert_close_f32(y, ref, tag=f"{name} tuning {tune}", elementwise=False)
+        if table:
+            assert np.array_equal(yt, oracle.lut_act(y, lut)), f"{name}: table lookup differs"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_conv_w8a32_random_shapes_bit_exact(seed, torch_dev, oracle):
+    torch = torch_dev
+    rng = np.random.default_rng(2000 + seed)
+    d = _random_conv(rng, quant=True)
+    if not d.has_bias:
+        d.act_type = abi.NOT_ACT
+    name = f"random_q_{seed}"
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    oh, ow = d.out_hw()
+    acc = torch.empty((d.n, d.cout, oh, ow), dtype=torch.int32, device="cuda")
+    y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32) if b32 is not None else None, dev(torch, aux),
+                         dev(torch, cases.silu_lut()), acc32=acc)
+    torch.cuda.synchronize()
+    ref, ref_acc = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut(), want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), ref_acc), f"{name}: int32 accumulators differ"
+    assert np.array_equal(y.cpu().numpy(), ref), f"{name}: de-quantised outputs differ"
+
+
 PACKED_CASES = [n for n, d in cases.conv_f32_cases().items()
                 if d.group == 1 and not (d.kh == 1 and d.kw == 1 and d.pad_t == 0)]
 
