@@ -25,7 +25,8 @@ struct DwParams {
     int planes_per_wg;   // >= 1 when whole planes fit in LDS, else 0
     int band_rows;       // output rows per workgroup when a plane is split into bands
     int bands;           // bands per plane (1 when planes_per_wg >= 1)
-    int pitch;           // LDS row pitch: W plus the left and right padding columns the filter can touch
+    int pitch;           // LDS row pitch: the padded columns the windows reach, and at least left padding + W
+    int tile_rows;       // whole planes: tile rows per plane (the rows the windows reach, at least top padding + H)
     int flat_stage;      // small whole planes: stage by flat index
     int lds_floats;      // LDS cells of one workgroup's chunk (a multiple of 4)
     unsigned magic_hw, magic_w;   // floor(2^32 / d) + 1 for d = H*W and d = W (d >= 2)
@@ -68,7 +69,9 @@ __global__ __launch_bounds__(DW_THREADS) void depthwise_tiled_kernel(DwParams p,
         oh1 = min(p.OH, oh0 + p.band_rows);
     }
     const int ih_first = oh0 * p.sh - p.pt;                      // input row of tile row 0 (may be negative)
-    const int trows = (oh1 - 1 - oh0) * p.sh + p.kh;             // tile rows per plane
+    // tile rows per plane: what the band's windows reach, or (whole planes) at least every row of the image, so that
+    // the flat copy below has a cell for each input even where a stride above 1 leaves the last rows unread
+    const int trows = p.planes_per_wg >= 1 ? p.tile_rows : (oh1 - 1 - oh0) * p.sh + p.kh;
     const int pitch = p.pitch;
     const int plane_cells = trows * pitch;
     // ---- stage -----------------------------------------------------------------------------------------
@@ -246,9 +249,13 @@ static int dw_plan(const onhip_conv_desc_t &d, int OH, int OW, DwParams *p) {
     p->div_unit = make_div31((unsigned) (dw_specialisation(d) ? ((OH + DW_RT - 1) / DW_RT) * OW : OH * OW));
     p->kh = d.kh; p->kw = d.kw; p->sh = d.stride_h; p->sw = d.stride_w; p->pt = d.pad_t; p->pl = d.pad_l;
     p->planes = d.n * d.cout;
-    // columns 0 .. (OW-1)*sw + kw - 1 of the padded row are read
-    p->pitch = (OW - 1) * d.stride_w + d.kw;
-    const int full_rows = (OH - 1) * d.stride_h + d.kh;
+    // columns 0 .. (OW-1)*sw + kw - 1 of the padded row are read; the copy into the tile writes every column of the
+    // image, so the pitch also covers those a stride above 1 leaves unread at the right edge (same for the rows of a
+    // whole plane)
+    const int reach_w = (OW - 1) * d.stride_w + d.kw, reach_h = (OH - 1) * d.stride_h + d.kh;
+    p->pitch = reach_w > d.w + d.pad_l ? reach_w : d.w + d.pad_l;
+    const int full_rows = reach_h > d.h + d.pad_t ? reach_h : d.h + d.pad_t;
+    p->tile_rows = full_rows;
     const int plane_cells = full_rows * p->pitch;
     if (plane_cells <= DW_LDS_FLOATS) {
         // whole planes: as many as fit, but leave enough workgroups to fill 256 CUs several times over

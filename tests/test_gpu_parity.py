@@ -152,6 +152,29 @@ def test_conv_w8a32_random_shapes_bit_exact(seed, torch_dev, oracle):
     assert np.array_equal(y.cpu().numpy(), ref), f"{name}: de-quantised outputs differ"
 
 
+@pytest.mark.parametrize("shape", [(58, 13, 32, 3, 3, 0), (39, 33, 11, 3, 3, 0), (4, 22, 36, 1, 3, 0), (31, 39, 20, 3, 2, 0),
+                                   (64, 29, 23, 5, 3, 1), (30, 14, 12, 3, 3, 1), (7, 16, 32, 5, 2, 0), (9, 61, 100, 3, 3, 1)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_depthwise_stride_leaves_rows_and_columns_unread(shape, quant, torch_dev, oracle):
+    """a stride above 1 whose last window ends before the image does (found by the random sweep: the copy of the image
+    into the LDS tile had no cells for those rows and columns and wrote over its neighbours); small planes staged flat
+    and a plane wide enough for the row-walking copy, fp32 and W8A32, bit for bit"""
+    torch = torch_dev
+    c, h, w, k, s, pad = shape
+    d = cases.cd(c, c, k, s, pad, h, w, act=abi.RELU, group=c, n=2, input_scale=0.02)
+    name = f"dw_unread_{shape}_{quant}"
+    if quant:
+        x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+        y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, cases.silu_lut()))
+        ref = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut())
+    else:
+        x, wt, b = cases.conv_inputs(name, d)
+        y = hip.conv2d_f32(d, dev(torch, x), dev(torch, wt), dev(torch, b))
+        ref = oracle.conv2d_f32(d, x, wt, b, cases.silu_lut())
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), ref)
+
+
 PACKED_CASES = [n for n, d in cases.conv_f32_cases().items()
                 if d.group == 1 and not (d.kh == 1 and d.kw == 1 and d.pad_t == 0)]
 
