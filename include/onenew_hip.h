@@ -119,7 +119,9 @@ int onhip_conv2d_f32_packed(const onhip_conv_desc_t *d, const float *x, const fl
  * y = conv(x) as onhip_conv2d_f32 (packed != 0: as onhip_conv2d_f32_packed), then y += addend (a tensor of
  * y's shape, not y itself) as device/x86/Add/add.c:96, then, with relu_after != 0, relu as
  * device/x86/Relu/relu.c:27-52 (both of its rules, by element index).  Bit-identical to the three operators
- * run one after the other.  The reference fuses activations into Conv (tools/optimize/op_fusion.hpp:47-222)
+ * run one after the other when the convolution runs the same tile and split in both (always so with the cost model's
+ * choice; with measured choices, onhip_set_tuning(1), the two may be measured differently and then differ in the
+ * rounding of the sums, within the fp32 tolerance).  The reference fuses activations into Conv (tools/optimize/op_fusion.hpp:47-222)
  * but not the Add; this is the same idea one operator further. */
 int onhip_conv2d_f32_add(const onhip_conv_desc_t *d, const float *x, const float *w, int32_t packed, const float *bias,
                          const float *silu_lut, const float *addend, int32_t relu_after, float *y, void *stream);

@@ -72,7 +72,8 @@ int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, cons
  * the Conv plugin's `eval_add` / `eval_add_relu` entry points, when the plugin has them: one launch instead of
  * three, and the tensors in between are never written.  The reference's offline optimiser folds the activation
  * after a Conv the same way (tools/optimize/op_fusion.hpp:47-222).  Results are bit-identical to the separate
- * operators.  The fused call runs at the Add's place in the order; the operands folded away stay in the operand
+ * operators as long as the convolution runs the same tile and split either way (the cost model's choice always does;
+ * measured choices may differ between the two forms, and the sums then differ in their rounding).  The fused call runs at the Add's place in the order; the operands folded away stay in the operand
  * table and read as the block's result.  Setting the environment variable ONENEW_RT_FUSE=0 before loading keeps
  * every operator separate, for layer-by-layer comparison.
  *
