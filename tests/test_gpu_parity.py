@@ -152,6 +152,51 @@ def test_conv_w8a32_random_shapes_bit_exact(seed, torch_dev, oracle):
     assert np.array_equal(y.cpu().numpy(), ref), f"{name}: de-quantised outputs differ"
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_conv_w8a8_chain_random_shapes(seed, torch_dev, oracle):
+    """the int8 NHWC chain form on seeded random dense convolutions: the reference's int8 values exactly"""
+    torch = torch_dev
+    rng = np.random.default_rng(9000 + seed)
+    d = _random_conv(rng, quant=True)
+    if d.group != 1:
+        d.group, d.cout = 1, int(rng.integers(1, 100))
+    if not d.has_bias:
+        d.act_type = abi.NOT_ACT
+    d.out_s8, d.output_scale = 1, float(rng.uniform(0.01, 0.08))
+    x, w8, b32, aux = cases.conv_inputs(f"random_chain_{seed}", d, quant=True)
+    ref = oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut())
+    xq = hip.quantize_nhwc_s8(dev(torch, x), d.input_scale)
+    wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
+    oh, ow = d.out_hw()
+    out = torch.full((d.n, oh, ow, (d.cout + 15) // 16 * 16), 77, dtype=torch.int8, device="cuda")
+    yq = hip.conv2d_w8a8_nhwc(d, xq, wp, dev(torch, b32) if b32 is not None else None, dev(torch, aux),
+                              dev(torch, cases.silu_lut()), out=out)
+    torch.cuda.synchronize()
+    assert np.array_equal(yq.cpu().numpy()[..., :d.cout], np.transpose(ref, (0, 2, 3, 1)))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_conv_add_random_shapes(seed, torch_dev):
+    """the folded residual store on seeded random convolutions (cost model's tile choice, the same for both forms):
+    the bits of conv, Add and Relu run one after the other"""
+    torch = torch_dev
+    rng = np.random.default_rng(5000 + seed)
+    d = _random_conv(rng, quant=False)
+    x, w, b = cases.conv_inputs(f"random_res_{seed}", d)
+    oh, ow = d.out_hw()
+    r = rng.normal(size=(d.n, d.cout, oh, ow)).astype(np.float32)
+    lut = dev(torch, cases.silu_lut())
+    xd, wd, rd = dev(torch, x), dev(torch, w), dev(torch, r)
+    bd = dev(torch, b) if b is not None else None
+    for relu in (False, True):
+        want = hip.add_f32(hip.conv2d_f32(d, xd, wd, bd, lut), rd)
+        if relu:
+            want = hip.relu_f32(want)
+        got = hip.conv2d_f32_add(d, xd, wd, rd, bias=bd, silu_lut=lut, relu=relu)
+        torch.cuda.synchronize()
+        assert _same_bits(got.cpu().numpy(), want.cpu().numpy()), (seed, relu)
+
+
 @pytest.mark.parametrize("shape", [(58, 13, 32, 3, 3, 0), (39, 33, 11, 3, 3, 0), (4, 22, 36, 1, 3, 0), (31, 39, 20, 3, 2, 0),
                                    (64, 29, 23, 5, 3, 1), (30, 14, 12, 3, 3, 1), (7, 16, 32, 5, 2, 0), (9, 61, 100, 3, 3, 1)])
 @pytest.mark.parametrize("quant", [False, True])
