@@ -690,6 +690,31 @@ def test_plugin_matmul_and_gemm_eval(torch_dev, golden):
         cases.check_against(golden, name, y, exact=False, rtol=1e-4, atol=1e-4 * float(np.abs(y).max()))
 
 
+def test_plugin_evals_on_a_named_stream(torch_dev):
+    """onhip_plugin_set_stream: the evals queue their kernels on a caller's stream (here one created non-blocking, which
+    a blocking copy does not wait for by itself) and results in host buffers are still complete on return"""
+    import ctypes as C
+    torch = torch_dev
+    name = "c3x3_tiny_relu"
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    plug = ops.Plugin(hip.plugin_path("Conv"))
+    op = ops.Conv(plug.eval, d, w, b)
+    want = op(x).copy()
+    lib = hip.load()
+    lib.onhip_plugin_set_stream.argtypes = [C.c_void_p]
+    s = torch.cuda.Stream()
+    assert lib.onhip_plugin_set_stream(C.c_void_p(s.cuda_stream)) == 0
+    try:
+        for _ in range(3):
+            assert np.array_equal(op(x), want)
+        relu = ops.Relu(ops.Plugin(hip.plugin_path("Relu")).eval)
+        assert np.array_equal(relu(x), np.maximum(x, 0))
+    finally:
+        assert lib.onhip_plugin_set_stream(None) == 0
+    assert np.array_equal(op(x), want)
+
+
 def test_plugin_conv_eval_device_buffers(torch_dev, golden):
     """activation and output already in device memory: used in place, no staging"""
     torch = torch_dev
