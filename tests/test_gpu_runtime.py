@@ -324,6 +324,74 @@ def test_relu_after_a_quantised_convolution_is_folded(torch_dev, monkeypatch):
     assert np.array_equal(got[0], one_model.run(data, ins)[0])
 
 
+def _random_residual_graph(seed):
+    """convolutions (dense and depthwise, 1x1 and 3x3, with and without bias and activation), Relu and Add nodes over
+    tensors of one shape, wired at random: residual adds in either operand order, results read twice, results that are
+    net outputs, chains of folded blocks"""
+    rng = np.random.default_rng(13000 + seed)
+    C, H, W, N = int(rng.choice([4, 8, 12])), int(rng.integers(5, 14)), int(rng.integers(5, 14)), int(rng.integers(1, 3))
+    m = onefile.OneModel()
+    m.input("x", (N, C, H, W))
+    tensors, outs, nid = ["x"], [], 0
+
+    def w(*shape):
+        return (rng.normal(size=shape) * 0.2).astype(np.float32)
+
+    for _ in range(int(rng.integers(2, 7))):
+        kind = rng.random()
+        src = tensors[int(rng.integers(len(tensors)))] if rng.random() < 0.3 else tensors[-1]
+        nid += 1
+        if kind < 0.55:
+            k = int(rng.choice([1, 3]))
+            bias = w(C) if rng.random() < 0.8 else None
+            act = int(rng.choice([abi.NOT_ACT, abi.NOT_ACT, abi.RELU, abi.CLIP]))
+            group = C if (rng.random() < 0.2 and bias is not None) else 1
+            m.conv(f"c{nid}", src, w(C, 1 if group != 1 else C, k, k), bias, f"t{nid}", pad=k // 2, act=act,
+                   clip=(-0.5, 0.8), group=group)
+            cur = f"t{nid}"
+            if rng.random() < 0.3:
+                m.relu(f"r{nid}", cur, f"t{nid}r")
+                cur = f"t{nid}r"
+            if rng.random() < 0.6:
+                other = tensors[int(rng.integers(len(tensors)))]
+                if rng.random() < 0.5:
+                    m.add(f"a{nid}", cur, other, f"t{nid}a")
+                else:
+                    m.add(f"a{nid}", other, cur, f"t{nid}a")
+                if rng.random() < 0.2:
+                    outs.append(cur)
+                cur = f"t{nid}a"
+                if rng.random() < 0.6:
+                    m.relu(f"ar{nid}", cur, f"t{nid}ar")
+                    cur = f"t{nid}ar"
+            tensors.append(cur)
+        elif kind < 0.75:
+            m.add(f"a{nid}", src, tensors[int(rng.integers(len(tensors)))], f"t{nid}")
+            tensors.append(f"t{nid}")
+        else:
+            m.relu(f"r{nid}", src, f"t{nid}")
+            tensors.append(f"t{nid}")
+    outs.append(tensors[-1])
+    if rng.random() < 0.3 and len(tensors) > 2:
+        outs.append(tensors[int(rng.integers(1, len(tensors)))])
+    outs = list(dict.fromkeys(o for o in outs if o != "x"))
+    for o in outs:
+        m.output(o, (N, C, H, W))
+    return (m.tobytes() if outs else None), rng.normal(size=(N, C, H, W)).astype(np.float32)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_residual_graphs_fold_without_changing_a_bit(seed, torch_dev, monkeypatch):
+    data, x = _random_residual_graph(seed)
+    if data is None:
+        pytest.skip("the draw has no output")
+    fused, plain, got, want = _both_ways(data, [x], monkeypatch)
+    ref = one_model.run(data, [x])
+    for g, w_, r in zip(got, want, ref):
+        assert np.array_equal(g, w_)
+        assert _close(w_, r, 5e-4)
+
+
 @pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
 def test_whole_model_folds_every_residual_block(model, torch_dev, monkeypatch):
     """16 bottleneck blocks of ResNet-50 (Add + Relu) and the 10 residual connections of MobileNetV2 (Add), batch 2:

@@ -226,3 +226,20 @@ def test_plan_refuses_a_node_whose_first_input_is_unnamed():
             return
         off += onefile.align64(C.sizeof(cfg))
     raise AssertionError("the test model has no Gemm")
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_plan_of_random_residual_graphs(seed):
+    """the folding passes on the random graphs of the GPU suite, without a GPU: the plan loads, keeps every output, and
+    never runs more operators than the file has"""
+    sys.path.insert(0, HERE)
+    from test_gpu_runtime import _random_residual_graph
+    data, _ = _random_residual_graph(seed)
+    if data is None:
+        pytest.skip("the draw has no output")
+    m = onefile.parse(data)
+    net = rt.Net(data, plan_only=True)
+    assert net.outputs == [(n, tuple(s)) for n, s in m["outputs"]]
+    folded = len(m["nodes"]) - len(net.ops())
+    assert 0 <= folded <= 2 * net.fused_blocks() + net.folded_relus()
+    assert folded >= net.fused_blocks() + net.folded_relus()
