@@ -93,6 +93,24 @@ static int get_scratch(size_t bytes, void **out) {
     return ONHIP_OK;
 }
 
+// Workspace of the split-K reduction that runs inside the launch: partial sums and one arrival counter per tile in
+// uncached device memory, so that what one XCD wrote is what another reads without flushing anybody's L2.  Allocated
+// once at first use and kept for the life of the process.
+static void *g_uc = nullptr;
+static int *g_arrive = nullptr;
+static const size_t kUcBytes = (size_t) 256 << 20;
+static int get_uc(void **buf, int **arrive) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_uc) {
+        ONHIP_CHECK_HIP(hipExtMallocWithFlags(&g_uc, kUcBytes, hipDeviceMallocUncached));
+        ONHIP_CHECK_HIP(hipExtMallocWithFlags(reinterpret_cast<void **>(&g_arrive), 4 << 20, hipDeviceMallocUncached));
+        ONHIP_CHECK_HIP(hipMemset(g_arrive, 0, 4 << 20));
+        ONHIP_CHECK_HIP(hipDeviceSynchronize());
+    }
+    *buf = g_uc; *arrive = g_arrive;
+    return ONHIP_OK;
+}
+
 // ---- tile and split-K choice ----------------------------------------------------------------------
 //
 // A launch is described by (tile BM x BN, split): split > 1 cuts K into slices that write partial
@@ -106,7 +124,9 @@ static const int kNumSplits = 13;
 
 // tail > 1: the tiles left over after whole rounds of 256 are cut `tail` ways along K (launch_choice)
 // rowb != 0: the kernel that feeds B from global memory straight into the MFMAs (igemm_rowb.hip), tile bm x bn
-struct Choice { int bm, bn, split, tail, rowb; };
+// fin != 0 (with split > 1 or tail > 1): the slices of a tile are added up by the last of them to arrive, inside the
+// launch, instead of by a finishing launch (igemm_kernel, `arrive`)
+struct Choice { int bm, bn, split, tail, rowb, fin; };
 
 static std::mutex g_tune_mu;
 static int g_tune_mode = -1;   // -1: read ONHIP_TUNE on first use; 0 model only; 1 measure
@@ -142,8 +162,8 @@ static void load_tune_cache_locked() {
             key.push_back(v);
             s = end;
         }
-        Choice c = {0, 0, 1, 0, 0};
-        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb) >= 3)
+        Choice c = {0, 0, 1, 0, 0, 0};
+        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 3)
             g_tuned[key] = c;
     }
     fclose(f);
@@ -154,7 +174,7 @@ static void append_tune_cache_locked(const std::vector<long long> &key, const Ch
     FILE *f = fopen(path, "a");
     if (!f) return;
     for (long long v : key) fprintf(f, "%lld ", v);
-    fprintf(f, ": %d %d %d %d %d\n", c.bm, c.bn, c.split, c.tail, c.rowb);
+    fprintf(f, ": %d %d %d %d %d %d\n", c.bm, c.bn, c.split, c.tail, c.rowb, c.fin);
     fclose(f);
 }
 
@@ -187,6 +207,15 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
             cfg.split = split;
             p.k_split_units = tiles_per * upt;
             p.partial = reinterpret_cast<float *>(buf);
+            p.arrive = nullptr;
+            if (c.fin && cfg.dtype != DT_I8 && bytes <= kUcBytes) {
+                void *uc; int *arr;
+                rc = get_uc(&uc, &arr);
+                if (rc) return rc;
+                p.partial = reinterpret_cast<float *>(uc);
+                p.arrive = arr;
+                p.n_slices = split;
+            }
         }
     }
     return ONHIP_OK;
@@ -216,6 +245,12 @@ static bool tail_geometry(const IgemmLaunch &cfg, const IgemmParams &p, int bm, 
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
     if (c.rowb && (c.split != 1 || !rowb_f32_ok(cfg, p))) return false;
+    if (c.fin) {
+        static const bool off = getenv("ONHIP_NO_FIN") != nullptr;   // tuning hook: finishing launches only
+        if (off) return false;
+        const long long tiles = (long long) ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * cfg.batch;
+        if (cfg.dtype == DT_I8 || c.rowb || (c.split <= 1 && c.tail <= 1) || tiles > (1 << 20)) return false;
+    }
     if (c.tail > 1) {
         int dpc, left;
         return c.split == 1 && k_tiles >= 2 * c.tail && tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left);
@@ -245,11 +280,11 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
 }
 
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
-    Choice best = {64, 64, 1, 0, 0};
+    Choice best = {64, 64, 1, 0, 0, 0};
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t)
         for (int s = 0; s < kNumSplits; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0};
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0, 0};
             if (!candidate_ok(cfg, p, c)) continue;
             const double cost = model_cost(cfg, p, c);
             if (cost < best_cost) { best_cost = cost; best = c; }
@@ -265,14 +300,14 @@ static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStr
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
     auto launch = [&]() { return c.rowb ? rowb_f32_launch(cfg, p, st) : igemm_launch(cfg, p, st); };
     if (c.tail <= 1 || !tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
-        const Choice plain = {c.bm, c.bn, c.rowb ? 1 : c.split, 0, 0};
+        const Choice plain = {c.bm, c.bn, c.rowb ? 1 : c.split, 0, 0, c.rowb ? 0 : c.fin};
         int rc = apply_choice(cfg, p, plain);
         return rc ? rc : launch();
     }
     // one launch: dpc column blocks as whole tiles, the rest in c.tail K slices each; partial sums and the
     // finishing pass cover the columns from dpc * bn on only
     p.part_begin = dpc * c.bn;
-    const Choice tail = {c.bm, c.bn, c.tail, 0, 0};
+    const Choice tail = {c.bm, c.bn, c.tail, 0, 0, c.rowb ? 0 : c.fin};
     int rc = apply_choice(cfg, p, tail);
     if (rc) return rc;
     if (cfg.split <= 1) {
@@ -308,9 +343,10 @@ static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStrea
 
 // Chooses tile, split and tail handling for the problem and launches it.
 static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t st) {
-    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB]]]
-        Choice c = {0, 0, 1, 0, 0};
-        if (sscanf(env, "%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb) >= 2) {
+    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB[xFIN]]]]
+        Choice c = {0, 0, 1, 0, 0, 0};
+        if (sscanf(env, "%dx%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 2) {
+            if (c.fin && !candidate_ok(cfg, p, c)) c.fin = 0;
             if (c.rowb && !candidate_ok(cfg, p, c)) {   // not a problem for that kernel: the tiled one, same tile if it has it
                 c.rowb = 0;
                 if (c.bn > 128) c.bn = 128;
@@ -352,9 +388,11 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     };
     for (int t = 0; t < kNumTiles && !rc; ++t) {
         for (int s = 0; s < kNumSplits && !rc; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0};
+            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0, 0};
             if (!candidate_ok(cfg, p, c) || model_cost(cfg, p, c) > 2.5 * guess_cost) continue;
             try_choice(c);
+            const Choice cf = {c.bm, c.bn, c.split, 0, 0, 1};   // the same with the reduction inside the launch
+            if (!rc && candidate_ok(cfg, p, cf)) try_choice(cf);
         }
         // the leftover column blocks as a K-split launch of about one workgroup per CU, and half as many
         int dpc = 0, left = 0;
@@ -362,8 +400,12 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
             int want = 256 / left;
             want = want > 16 ? 16 : want;
             for (int ts = want; ts >= 2 && ts >= want / 2 && !rc; ts /= 2) {
-                const Choice c = {kTiles[t][0], kTiles[t][1], 1, ts, 0};
-                if (candidate_ok(cfg, p, c) && model_cost(cfg, p, {c.bm, c.bn, 1, 0, 0}) <= 2.5 * guess_cost) try_choice(c);
+                const Choice c = {kTiles[t][0], kTiles[t][1], 1, ts, 0, 0};
+                if (candidate_ok(cfg, p, c) && model_cost(cfg, p, {c.bm, c.bn, 1, 0, 0, 0}) <= 2.5 * guess_cost) {
+                    try_choice(c);
+                    const Choice cf = {c.bm, c.bn, 1, ts, 0, 1};
+                    if (!rc && candidate_ok(cfg, p, cf)) try_choice(cf);
+                }
             }
         }
     }
@@ -372,7 +414,7 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     for (int t = 0; t < 6 && !rc; ++t) {
         if (kRowbTiles[t][0] == 32 && p.M > 32) continue;   // one row tile of up to 32 output channels
         if (kRowbTiles[t][0] == 96 && p.M % 96 > 0 && p.M % 96 <= 64) continue;   // a last row tile that a 64-row tile covers as well
-        const Choice c = {kRowbTiles[t][0], kRowbTiles[t][1], 1, 0, 1};
+        const Choice c = {kRowbTiles[t][0], kRowbTiles[t][1], 1, 0, 1, 0};
         if (!candidate_ok(cfg, p, c)) continue;
         try_choice(c);
         int dpc = 0, left = 0;
@@ -380,7 +422,7 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
             int want = 256 / left;
             want = want > 16 ? 16 : want;
             for (int ts = want; ts >= 2 && ts >= want / 2 && !rc; ts /= 2) {
-                const Choice ct = {c.bm, c.bn, 1, ts, 1};
+                const Choice ct = {c.bm, c.bn, 1, ts, 1, 0};
                 if (candidate_ok(cfg, p, ct)) try_choice(ct);
             }
         }
@@ -389,8 +431,8 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     (void) hipEventDestroy(e1);
     if (rc) return rc;
     if (getenv("ONHIP_TUNE_VERBOSE"))
-        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d rowb %d (%.4f ms; model said %dx%d split %d)\n",
-                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best.rowb, best_ms, guess.bm,
+        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d rowb %d fin %d (%.4f ms; model said %dx%d split %d)\n",
+                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best.rowb, best.fin, best_ms, guess.bm,
                 guess.bn, guess.split);
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);

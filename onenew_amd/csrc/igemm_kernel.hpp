@@ -836,7 +836,61 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
     if (p.partial && !whole_k) {
         write_partial<TM, TN>(p, acc, slice * gridDim.z + batch, m_wave, n_wave, li, lh);
-        return;
+        if (DT == DT_I8 || !p.arrive) return;   // a finishing launch adds the slices up
+        // The reduction inside the launch.  Partial sums and counters live in uncached memory: once this workgroup's
+        // stores are acknowledged it counts itself in, and the last of a tile's slices to arrive adds all of them up
+        // in slice order (the order of the finishing kernel: the same bits) and goes on to the epilogue as if it had
+        // computed the whole tile.  Nobody waits for anybody, so the launch cannot hang; the counter is back at zero
+        // for the next launch.
+        __shared__ int s_last;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            int *ctr = p.arrive + lid + batch * (int) gridDim.x;
+            const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = old == p.n_slices - 1;
+            if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = last;
+        }
+        __syncthreads();
+        if (!s_last) return;
+        if constexpr (DT != DT_I8) {
+            const int width = p.N - p.part_begin;
+            const bool m_edge = m_wave + TM * 32 > p.M;
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+            for (int s = 0; s < p.n_slices; ++s) {
+                const rsrc_t rp = make_rsrc(reinterpret_cast<const char *>(p.partial) +
+                                            (size_t) (s * gridDim.z + batch) * p.M * width * 4, RSRC_RANGE);
+                // half a 32x32 block at a time: eight loads in flight, not sixteen per block of the tile, which would
+                // cost the kernels registers and with them occupancy
+#pragma unroll
+                for (int a = 0; a < TM; ++a)
+#pragma unroll
+                    for (int b = 0; b < TN; ++b) {
+                        const int n = n_wave + b * 32 + li;
+                        const unsigned cv = n < p.N ? (unsigned) (n - p.part_begin + 4 * lh * width) * 4u : OOB;
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            float v[8];
+#pragma unroll
+                            for (int q = 0; q < 8; ++q) {
+                                const int r = 8 * h + q;
+                                const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
+                                const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
+                                v[q] = buf_load_f32(rp, row_ok ? cv : OOB, (unsigned) m_uni * (unsigned) width * 4u);
+                            }
+#pragma unroll
+                            for (int q = 0; q < 8; ++q) acc[a][b][8 * h + q] = __fadd_rn(acc[a][b][8 * h + q], v[q]);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+            }
+        }
     }
     if constexpr (DT == DT_I8) {
         // int8 NHWC output without the raw-accumulator copy: 128-bit stores through LDS (batch is 1 on this path)
@@ -959,7 +1013,7 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     if (RES != (p.res != nullptr)) return set_error(ONHIP_ERR_ARG, "igemm: residual operand and kernel variant do not match");
     hipLaunchKernelGGL((igemm_kernel<DT, BL, BM, BN, WM, WN, PF, RES>), grid, dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
-    if (p.partial) {
+    if (p.partial && !p.arrive) {
         if (p.M > 4 * 65535 || cfg.batch > 65535)
             return set_error(ONHIP_ERR_ARG, "igemm: split-K with %d rows, %d batches", p.M, cfg.batch);
         const dim3 fgrid((p.N - p.part_begin + 63) / 64, (p.M + 3) / 4, cfg.batch);

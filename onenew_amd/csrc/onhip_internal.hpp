@@ -189,6 +189,10 @@ struct IgemmParams {
     float out_inv_scale;       // 1.0f / output_scale
     // split-K workspace: partial sums [split][M][N] fp32 (nullptr when unsplit)
     float *partial;
+    // reduction inside the launch by the last slice of a tile to arrive: one counter per tile (uncached memory, like
+    // `partial` then) and the number of slices; nullptr = a finishing launch adds the slices up
+    int *arrive;
+    int n_slices;
     // exact division of any x < 2^31 by OHW, OW and the number of row tiles (filled in by the launcher)
     Div31 div_ohw, div_ow, div_tiles_m;
 };

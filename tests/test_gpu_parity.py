@@ -309,7 +309,9 @@ def test_conv_f32_batched(name, batch, torch_dev, oracle):
         assert_close_f32(y, ref, tag=name)
 
 
-@pytest.mark.parametrize("tile", ["64x64x1", "64x64x3", "32x128x2", "64x128x5", "128x128x4", "128x128x1"])
+@pytest.mark.parametrize("tile", ["64x64x1", "64x64x3", "32x128x2", "64x128x5", "128x128x4", "128x128x1",
+                                  # the same splits with the slices added up inside the launch by the last to arrive
+                                  "64x64x3x0x0x1", "32x128x2x0x0x1", "64x128x5x0x0x1", "128x128x4x0x0x1"])
 @pytest.mark.parametrize("kind", ["1x1_ragged_k", "3x3_packed"])
 def test_forced_tile_and_split_many_items(tile, kind, torch_dev, oracle, monkeypatch):
     """every tile shape, with and without split-K, on problems with more work items than resident
@@ -334,13 +336,40 @@ def test_forced_tile_and_split_many_items(tile, kind, torch_dev, oracle, monkeyp
         assert_close_f32(y.cpu().numpy(), ref, tag=f"{kind} {tile} run {rep}")
 
 
+@pytest.mark.parametrize("tile", ["64x64x4x0x0x1", "64x128x3x0x0x1", "64x64x16x0x0x1"])
+def test_split_k_added_up_inside_the_launch_is_the_finishing_pass_bit_for_bit(tile, torch_dev, monkeypatch):
+    """the last slice of a tile to arrive adds the partial sums up in slice order, as the finishing kernel does: the same
+    bits as that kernel on the same split, two hundred launches in a row (whichever slice arrives last), with a launch
+    of another shape in between so that the counters and the workspace are reused"""
+    torch = torch_dev
+    d = cases.cd(200, 100, 3, 1, 1, 14, 15, n=6, act=abi.RELU)           # K = 1800: 113 K tiles, ragged rows and columns
+    x, w, b = cases.conv_inputs("inlaunch_" + tile, d)
+    xd, wd, bd = dev(torch, x), dev(torch, w), dev(torch, b)
+    wp = hip.pack_conv_weights(d, wd)
+    d2 = cases.cd(64, 40, 1, 1, 0, 9, n=2, act=abi.NOT_ACT)
+    x2, w2, b2 = cases.conv_inputs("inlaunch_other", d2)
+    x2d, w2d, b2d = dev(torch, x2), dev(torch, w2), dev(torch, b2)
+    monkeypatch.setenv("ONHIP_TILE", tile.rsplit("x", 3)[0])               # the same tile and split, finishing launch
+    want = hip.conv2d_f32(d, xd, wp, bd, packed=True).cpu().numpy()
+    want2 = hip.conv2d_f32(d2, x2d, w2d, b2d).cpu().numpy()
+    monkeypatch.setenv("ONHIP_TILE", tile)
+    for rep in range(200):
+        y = hip.conv2d_f32(d, xd, wp, bd, packed=True)
+        if rep % 10 == 0:
+            y2 = hip.conv2d_f32(d2, x2d, w2d, b2d)
+            assert _same_bits(y2.cpu().numpy(), want2), rep
+        assert _same_bits(y.cpu().numpy(), want), rep
+
+
 @pytest.mark.parametrize("tile,shape", [("64x64x1x8", (20, 30, 29)), ("64x64x1x16", (17, 32, 32)), ("64x128x1x4", (34, 32, 34)),
                                         ("32x128x1x8", (33, 32, 33)), ("128x128x1x2", (80, 24, 36)),
                                         # the same through the kernel that reads B straight from memory (1x1 and matmul;
                                         # the 3x3 case falls back to the tiled kernel with the same split)
                                         ("64x128x1x4x1", (34, 32, 34)), ("128x128x1x2x1", (80, 24, 36)),
                                         ("64x256x1x4x1", (34, 32, 36)), ("96x128x1x4x1", (34, 32, 34)),
-                                        ("32x512x1x8x1", (34, 32, 32))])
+                                        ("32x512x1x8x1", (34, 32, 32)),
+                                        # leftover tiles whose slices are added up inside the launch
+                                        ("64x64x1x8x0x1", (20, 30, 29)), ("64x128x1x4x0x1", (34, 32, 34))])
 @pytest.mark.parametrize("kind", ["3x3_packed", "1x1", "matmul"])
 def test_leftover_tiles_as_a_split_launch(tile, shape, kind, torch_dev, oracle, monkeypatch):
     """the launch cut along N: whole rounds of 256 tiles unsplit on the caller's stream, the leftover column blocks
@@ -544,7 +573,8 @@ def _residual_case(kind):
 
 
 @pytest.mark.parametrize("relu", [False, True])
-@pytest.mark.parametrize("tile", [None, "64x64x1", "64x64x3", "32x128x2", "128x128x1", "64x128x1x4", "64x128x1x0x1"])
+@pytest.mark.parametrize("tile", [None, "64x64x1", "64x64x3", "32x128x2", "128x128x1", "64x128x1x4", "64x128x1x0x1",
+                                  "64x64x3x0x0x1", "128x128x2x0x0x1"])
 @pytest.mark.parametrize("kind", ["1x1_resnet", "1x1_ragged", "3x3_packed_relu", "3x3_s2_gather", "mobilenet_project",
                                   "depthwise", "nobias"])
 def test_conv_with_add_and_relu_folded_in(kind, tile, relu, torch_dev, oracle, monkeypatch):
