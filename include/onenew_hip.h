@@ -14,6 +14,11 @@
  *
  * Every function returns 0 on success and a negative code on failure; the text of the last
  * failure on the calling thread is returned by onhip_last_error().  Nothing throws.
+ *
+ * Like the reference's kernels, which share one scratch buffer (host/net.h:419-429), the convolution and matrix
+ * entry points share per-process device workspaces (split-K partial sums, arrival counters, the plugin level's staging
+ * buffers): launches that may overlap on the device, i.e. on different streams without an ordering between them,
+ * race.  One stream at a time, as the single-threaded reference host calls its operators, is the contract.
  */
 #ifndef ONENEW_HIP_H
 #define ONENEW_HIP_H
