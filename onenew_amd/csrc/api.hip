@@ -101,11 +101,13 @@ static int *g_arrive = nullptr;
 static const size_t kUcBytes = (size_t) 256 << 20;
 static int get_uc(void **buf, int **arrive) {
     std::lock_guard<std::mutex> lock(g_scratch_mu);
-    if (!g_uc) {
-        ONHIP_CHECK_HIP(hipExtMallocWithFlags(&g_uc, kUcBytes, hipDeviceMallocUncached));
-        ONHIP_CHECK_HIP(hipExtMallocWithFlags(reinterpret_cast<void **>(&g_arrive), 4 << 20, hipDeviceMallocUncached));
-        ONHIP_CHECK_HIP(hipMemset(g_arrive, 0, 4 << 20));
+    if (!g_uc || !g_arrive) {   // both or neither: a call that fails half-way leaves what it got for the next one
+        if (!g_uc) ONHIP_CHECK_HIP(hipExtMallocWithFlags(&g_uc, kUcBytes, hipDeviceMallocUncached));
+        void *ctr = nullptr;
+        ONHIP_CHECK_HIP(hipExtMallocWithFlags(&ctr, 4 << 20, hipDeviceMallocUncached));
+        ONHIP_CHECK_HIP(hipMemset(ctr, 0, 4 << 20));
         ONHIP_CHECK_HIP(hipDeviceSynchronize());
+        g_arrive = static_cast<int *>(ctr);
     }
     *buf = g_uc; *arrive = g_arrive;
     return ONHIP_OK;
