@@ -311,9 +311,9 @@ int onhip_plugin_set_async(int on);
  * reference.  The device-resident runtime names its own stream for the length of a run so that the run can be
  * recorded into a HIP graph.  Results into host buffers are still complete on return. */
 int onhip_plugin_set_stream(void *stream);
-/* For a caller that hands `eval` weights in device memory and is about to free or overwrite them: drops the re-laid-out
- * copies the plugin level made of weights whose address lies in [base, base + bytes), so that other data at the same
- * address later is packed afresh.  The device-resident runtime calls it when a net is freed.  No counterpart in the
+/* For a caller that hands `eval` weights or activation tables in device memory and is about to free or overwrite them:
+ * drops the re-laid-out copies the library made of weights (and the quantised copies of tables) whose address lies in
+ * [base, base + bytes), so that other data at the same address later is packed afresh.  The device-resident runtime calls it when a net is freed.  No counterpart in the
  * reference (its weights live in host vectors for the life of the process). */
 int onhip_plugin_forget(const void *base, size_t bytes);
 /* Drops the device copies of weights the plugin level keeps between calls. */

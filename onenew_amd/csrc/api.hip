@@ -682,6 +682,28 @@ static int quantised_table(const float *lut, float out_inv_scale, hipStream_t st
     return ONHIP_OK;
 }
 
+// Drops the quantised copies of tables whose address lies in [base, base + bytes): that memory is about to be freed or
+// rewritten, and another table at the same address must be quantised afresh.
+extern "C++" {
+int onhip::forget_quantised_tables(const void *base, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_qlut_mu);
+    const char *lo = static_cast<const char *>(base), *hi = lo + bytes;
+    bool any = false;
+    for (auto it = g_qlut.begin(); it != g_qlut.end();) {
+        const char *k = reinterpret_cast<const char *>(it->first.first);
+        if (k >= lo && k < hi) {
+            if (!any) ONHIP_CHECK_HIP(hipDeviceSynchronize());   // a kernel may still be reading the copy
+            any = true;
+            (void) hipFree(it->second);
+            it = g_qlut.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    return ONHIP_OK;
+}
+}   // extern "C++"
+
 // xq != nullptr: the activations arrive already quantised (int8 NHWC, channels padded to 16) and x is not read;
 // nhwc_out != 0: the int8 result is written NHWC with its channels padded to 16, ready to be the next xq
 static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8, int packed_w,

@@ -222,6 +222,7 @@ int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, flo
                          hipStream_t stream);
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
 int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
+int forget_quantised_tables(const void *base, size_t bytes);   // api.hip: the cache of tables behind an output quantiser
 int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, int k_units, int8_t *packed,
                    hipStream_t stream);
 int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,

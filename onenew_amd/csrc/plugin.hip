@@ -743,7 +743,7 @@ int onhip_plugin_forget(const void *base, size_t bytes) {
             ++it;
         }
     }
-    return ONHIP_OK;
+    return forget_quantised_tables(base, bytes);
 }
 
 int onhip_plugin_release(void) {

@@ -791,6 +791,8 @@ ONRT_API void onrt_net_free(onrt_net_t *net) {
     // the plugins key their packed copies of the weights by device address: that address is about to be free for reuse
     if (net->init_arena)
         for (forget_fn f : net->forgetters) (void) f(net->init_arena, net->init_bytes);
+    if (net->tables)   // and the quantised copies of the activation tables by theirs
+        for (forget_fn f : net->forgetters) (void) f(net->tables, 2 * net->silu_lut.size() * sizeof(float));
     if (net->init_arena) (void) hipFree(net->init_arena);
     if (net->act_arena) (void) hipFree(net->act_arena);
     if (net->tables) (void) hipFree(net->tables);

@@ -88,10 +88,17 @@ def load():
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
     L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
+    L.onhip_plugin_forget.argtypes = [vp, C.c_size_t]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
     _lib = L
     return L
+
+
+def forget(t):
+    """tell the library that the device tensor t (weights or an activation table it may hold copies of) is about to be
+    freed or rewritten"""
+    _check(load().onhip_plugin_forget(_ptr(t), t.numel() * t.element_size()), "onhip_plugin_forget")
 
 
 def _check(rc, what):

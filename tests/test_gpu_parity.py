@@ -1026,6 +1026,30 @@ def _chain_desc(name):
     return ConvDesc.from_buffer_copy(cases.conv_w8a32_cases()[name])
 
 
+def test_quantised_copy_of_a_table_is_dropped_with_the_table(torch_dev, oracle):
+    """the chain form keeps a quantised copy of the activation table by the table's address; once the caller says
+    that address is being rewritten, the next call quantises what is there now"""
+    torch = torch_dev
+    d = _chain_desc("q3x3_silu")
+    d.n = 2
+    d.out_s8, d.output_scale = 1, 0.041
+    x, w8, b32, aux = cases.conv_inputs("q3x3_silu_table", d, quant=True)
+    xq = hip.quantize_nhwc_s8(dev(torch, x), d.input_scale)
+    wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
+    lut = dev(torch, cases.silu_lut())
+    other = -cases.silu_lut()
+    args = (d, xq, wp, dev(torch, b32), dev(torch, aux), lut)
+    got = hip.conv2d_w8a8_nhwc(*args).cpu().numpy()
+    assert np.array_equal(got[..., :d.cout], np.transpose(oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut()), (0, 2, 3, 1)))
+    hip.forget(lut)
+    lut.copy_(dev(torch, other))
+    got = hip.conv2d_w8a8_nhwc(*args).cpu().numpy()
+    want = np.transpose(oracle.conv2d_w8a32(d, x, w8, b32, aux, other), (0, 2, 3, 1))
+    assert np.array_equal(got[..., :d.cout], want)
+    assert not np.array_equal(got[..., :d.cout], np.transpose(oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut()), (0, 2, 3, 1)))
+    hip.forget(lut)
+
+
 @pytest.mark.parametrize("tile", [None, "128x128", "64x128", "32x128", "64x64x2"])
 @pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_s2", "yolo_c2f_3x3_64_80", "yolo_sppf_1x1_1024", "q3x3_bigacc"]
                          + list(CHAIN_EXTRA))
