@@ -165,7 +165,8 @@ static void load_tune_cache_locked() {
             s = end;
         }
         Choice c = {0, 0, 1, 0, 0, 0};
-        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 3)
+        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 3 &&
+            c.bm > 0 && c.bn > 0 && c.split >= 1 && c.split <= 64 && c.tail >= 0 && c.tail <= 64)
             g_tuned[key] = c;
     }
     fclose(f);
@@ -367,8 +368,11 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
         auto it = g_tuned.find(key);
         if (it != g_tuned.end()) {
             const Choice c = it->second;
-            lock.unlock();
-            return launch_choice(cfg, p, c, st);
+            if (candidate_ok(cfg, p, c)) {
+                lock.unlock();
+                return launch_choice(cfg, p, c, st);
+            }
+            g_tuned.erase(it);   // a line of the cache file that this build would not have written: measure again
         }
     }
     // measure: the candidates the model ranks within 2.5x of its best, on the caller's stream

@@ -1079,3 +1079,44 @@ def test_conv_w8a8_nhwc_chain_form(name, tile, torch_dev, oracle, monkeypatch):
     assert np.array_equal(got[..., :d.cout], np.transpose(ref, (0, 2, 3, 1)))
     if tile is None or "x2" not in tile:
         assert not got[..., d.cout:].any()                                    # unsplit launches zero the channel padding
+
+
+_TUNE_CHILD = r"""
+import sys, numpy as np, torch
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests/golden")
+import cases
+from onenew_amd import abi, hip
+hip.init(0)
+d = cases.cd(96, 80, 3, 1, 1, 20, n=4, act=abi.NOT_ACT)
+x, w, b = cases.conv_inputs("tune_cache_file", d)
+y = hip.conv2d_f32(d, torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()).cpu()
+ref = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(b).double(), padding=1)
+print("ERR", float((y.double() - ref).abs().max() / ref.abs().max()))
+"""
+
+
+@pytest.mark.gpu
+def test_tune_cache_file_is_validated_and_rewritten(tmp_path):
+    """measured choices persist in the file ONHIP_TUNE_CACHE names; lines that are not choices of this build (garbage,
+    or a choice the problem does not admit) are passed over and the problem is measured again"""
+    import os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cache = tmp_path / "tune.txt"
+    env = dict(os.environ, ONHIP_TUNE="1", ONHIP_TUNE_CACHE=str(cache))
+    env.pop("ONHIP_TILE", None)
+
+    def run():
+        out = subprocess.run([sys.executable, "-c", _TUNE_CHILD, root], env=env, capture_output=True, text=True, timeout=100)
+        assert out.returncode == 0, out.stderr[-2000:]
+        err = [float(l.split()[1]) for l in out.stdout.splitlines() if l.startswith("ERR")]
+        assert err and err[0] <= 1e-4
+        return [l for l in cache.read_text().splitlines() if l.strip()]
+
+    lines = run()                                   # measured and written
+    assert len(lines) == 1 and ":" in lines[0]
+    assert run() == lines                           # read back: nothing measured, nothing appended
+    key = lines[0].split(":")[0]
+    cache.write_text("not a line of this file\n" + key + ": 64 64 0 0 0 0\n" + key + ": 64 64 1 0 0 1\n")
+    after = run()       # split 0 is no choice; in-launch reduction without slices is none either: measured again
+    assert len(after) == 4 and after[3].startswith(key + ":")
+    assert run() == after                           # the last line for a problem is the one that counts
