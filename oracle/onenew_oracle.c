@@ -17,11 +17,14 @@
  * reference kernels (golden fixtures made by tests/golden/make_golden.py), against float64
  * brute force and against algebraic invariants.
  *
- * PARITY UNPINNED: oracle_quant_weight_bias and the oracle_calib_* functions restate
- * tools/optimize/model_quant.hpp, which only builds together with the reference's host runtime,
- * OpenCV and protobuf, and which leaves the overload of fabs / abs / log it calls on floats to the
- * include order.  They are checked against closed forms and numpy (tests/test_oracle_math.py), not
- * against reference output.
+ * oracle_quant_weight_bias and the oracle_calib_* functions restate tools/optimize/model_quant.hpp,
+ * which only builds together with the reference's host runtime, OpenCV and protobuf: there is no
+ * reference output for them.  They are pinned by what the mathematics fixes instead
+ * (tests/test_oracle_math.py): the quantiser by its closed form (product rounded before the division,
+ * truncation), the histogram by numpy's bincount, the percentile by a sort, the KL and MSE searches
+ * by float64 brute force of their definitions at every candidate range.  What stays open is the
+ * overload of fabs / abs / log the reference gets for floats (left to its include order); the
+ * float overloads are used here.
  */
 #include <immintrin.h>
 #include <math.h>
@@ -461,9 +464,13 @@ void oracle_quant_weight_bias(const float *w, const float *bias, int cout, int p
 
 /* ---------------------------------------------------------------------------------------------
  * Activation-scale calibration (tools/optimize/model_quant.hpp:83-185 percentile, :197-435 KL,
- * :437-623 MSE; input_scale = threshold / 127 at :668).  PARITY UNPINNED: the reference tool only
- * builds with the whole host runtime and OpenCV, and it calls fabs / abs / log on floats without
- * saying which overload it gets; float overloads (the evident intent) are used here.
+ * :437-623 MSE; input_scale = threshold / 127 at :668).  The reference tool only builds with the whole
+ * host runtime and OpenCV, so no reference output exists for these; it calls fabs / abs / log on floats
+ * without saying which overload it gets, float overloads (the evident intent) are used here.  What pins
+ * them instead (tests/test_oracle_math.py): the histogram against numpy's bincount, the percentile against
+ * a sort, and the value of the KL and the MSE search at every one of the 1920 candidate ranges against the
+ * float64 definition (interval-overlap matrix / nearest-level brute force) on histograms whose winner is
+ * inside the range, off the multiples of 128 and has mass beyond it.
  * ------------------------------------------------------------------------------------------- */
 
 /* model_quant.hpp:287-292: running maximum of |x| over the calibration images */
@@ -486,13 +493,13 @@ void oracle_calib_histogram(const float *x, int64_t n, float max_abs, float *his
     }
 }
 
-/* model_quant.hpp:345-431: the clipping bin whose 128-level quantised distribution is closest (KL) to the
- * clipped reference distribution; threshold = (best + 0.5) * max / 2048 */
-float oracle_calib_threshold_kl(const float *hist, int64_t elem_count, float max_abs) {
+/* model_quant.hpp:345-431, one value per candidate clipping range (128 ... 2047 bins): the KL divergence between
+ * the clipped reference distribution (mass beyond the range folded into its last bin, :356-358) and the same range
+ * seen through 128 levels (fractional bin edges, :376-392, spread back over the bins, :398-415).  kl has
+ * ORACLE_CALIB_BINS - 128 entries. */
+void oracle_calib_kl_curve(const float *hist, int64_t elem_count, float *kl_out) {
     enum { TARGET = 128, MIN_BINS = 128 };
     const float kl_eps = 1e-7f;
-    float best_kl = 32768.6f;
-    int best_bins = 0;
     static float p[ORACLE_CALIB_BINS], accp[ORACLE_CALIB_BINS], q[TARGET], eq[ORACLE_CALIB_BINS];
     for (int bins = MIN_BINS; bins < ORACLE_CALIB_BINS; ++bins) {
         for (int i = 0; i < bins; ++i) p[i] = accp[i] = kl_eps + hist[i];
@@ -530,19 +537,29 @@ float oracle_calib_threshold_kl(const float *hist, int64_t elem_count, float max
         }
         float kl = 0.0f;
         for (int i = 0; i < bins; ++i) kl += accp[i] * logf(accp[i] / eq[i]);
-        if (kl < best_kl) {
-            best_kl = kl;
+        kl_out[bins - MIN_BINS] = kl;
+    }
+}
+
+/* model_quant.hpp:420-431: the first candidate with the least divergence (below the starting value 32768.6);
+ * threshold = (best + 0.5) * max / 2048 */
+float oracle_calib_threshold_kl(const float *hist, int64_t elem_count, float max_abs) {
+    static float kl[ORACLE_CALIB_BINS];
+    oracle_calib_kl_curve(hist, elem_count, kl);
+    float best_kl = 32768.6f;
+    int best_bins = 0;
+    for (int bins = 128; bins < ORACLE_CALIB_BINS; ++bins)
+        if (kl[bins - 128] < best_kl) {
+            best_kl = kl[bins - 128];
             best_bins = bins;
         }
-    }
     return (best_bins + 0.5f) * max_abs / ORACLE_CALIB_BINS;
 }
 
-/* model_quant.hpp:585-618: the clipping bin with the least squared error of a 128-level grid */
-float oracle_calib_threshold_mse(const float *hist, int64_t elem_count, float max_abs) {
+/* model_quant.hpp:585-610, one value per candidate clipping range: the mean squared distance (in bins) of every
+ * bin centre from its level on a 128-level grid over the range, values beyond it clipped to the top level */
+void oracle_calib_mse_curve(const float *hist, int64_t elem_count, float *loss_out) {
     enum { TARGET = 128, MIN_BINS = 128 };
-    int best_bins = 0;
-    float loss_min = 32768.0f;
     const int32_t elem_size = (int32_t) elem_count;      /* the reference keeps the count in an int32 */
     for (int bins = MIN_BINS; bins < ORACLE_CALIB_BINS; ++bins) {
         float loss = 0.0f;
@@ -554,11 +571,21 @@ float oracle_calib_threshold_mse(const float *hist, int64_t elem_count, float ma
             const float err = (float) ((float) idx + 0.5 - iq);      /* "+ 0.5" in double, stored to float */
             loss += (hist[idx] * err * err) / elem_size;
         }
-        if (loss < loss_min) {
-            loss_min = loss;
+        loss_out[bins - MIN_BINS] = loss;
+    }
+}
+
+/* model_quant.hpp:611-618: the first candidate with the least loss (below the starting value 32768) */
+float oracle_calib_threshold_mse(const float *hist, int64_t elem_count, float max_abs) {
+    static float loss[ORACLE_CALIB_BINS];
+    oracle_calib_mse_curve(hist, elem_count, loss);
+    int best_bins = 0;
+    float loss_min = 32768.0f;
+    for (int bins = 128; bins < ORACLE_CALIB_BINS; ++bins)
+        if (loss[bins - 128] < loss_min) {
+            loss_min = loss[bins - 128];
             best_bins = bins;
         }
-    }
     return (best_bins + 0.5f) * max_abs / ORACLE_CALIB_BINS;
 }
 

@@ -43,6 +43,8 @@ int oracle_transpose_f32(int ndim, const int32_t *in_shape, const int32_t *perm,
 #define ORACLE_CALIB_BINS 2048
 float oracle_calib_abs_max(const float *x, int64_t n, float running_max);
 void oracle_calib_histogram(const float *x, int64_t n, float max_abs, float *hist);
+void oracle_calib_kl_curve(const float *hist, int64_t elem_count, float *kl_out);
+void oracle_calib_mse_curve(const float *hist, int64_t elem_count, float *loss_out);
 float oracle_calib_threshold_kl(const float *hist, int64_t elem_count, float max_abs);
 float oracle_calib_threshold_mse(const float *hist, int64_t elem_count, float max_abs);
 float oracle_calib_threshold_percent(const float *x, int images, int32_t elems);

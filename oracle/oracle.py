@@ -235,6 +235,16 @@ def calib_threshold(method, hist, elem_count, max_abs):
     return float(fn(_p(hist, f32p), C.c_int64(elem_count), C.c_float(max_abs)))
 
 
+def calib_curve(method, hist, elem_count):
+    """the search's value for every candidate clipping range (128 ... 2047 bins)"""
+    fn = lib().oracle_calib_kl_curve if method == "kl" else lib().oracle_calib_mse_curve
+    fn.restype = None
+    hist = _f32(hist)
+    out = np.empty(2048 - 128, np.float32)
+    fn(_p(hist, f32p), C.c_int64(elem_count), _p(out, f32p))
+    return out
+
+
 def calib_percentile(x, images, elems):
     x = _f32(x)
     fn = lib().oracle_calib_threshold_percent

@@ -230,6 +230,114 @@ def test_calibration_thresholds_closed_cases(oracle):
     assert oracle.calib_threshold("kl", h, x.size, mx) < 0.8 * mx
 
 
+def _tailed_histogram(tag, n, tail_frac, tail_scale):
+    """2048-bin histogram of a half-normal bulk with an exponential tail from 4 sigma outwards: the bulk fills a few
+    hundred bins, the tail reaches the last one, so every candidate range leaves mass beyond itself"""
+    x = np.abs(datagen.normal(datagen.seed_for("calib", tag, "bulk"), (n,), 0.0, 1.0).astype(np.float64))
+    k = int(n * tail_frac)
+    x[:k] = 4.0 - tail_scale * np.log(datagen.unit(datagen.seed_for("calib", tag, "tail"), k))
+    idx = np.minimum((x * 2048 / x.max()).astype(np.int64), 2047)
+    return np.bincount(idx, minlength=2048).astype(np.float32)
+
+
+def _overlap(bins, shift_last=False):
+    """W[i, j] = length of [i r, (i + 1) r) inside bin [j, j + 1), r = bins / 128: the 128 levels as intervals"""
+    r = bins / 128.0
+    i = np.arange(128)[:, None]
+    j = np.arange(bins)[None, :]
+    w = np.clip(np.minimum((i + 1) * r, j + 1.0) - np.maximum(i * r, j * 1.0), 0.0, None)
+    if shift_last:          # the mistake of giving a level's last, fractional piece to the bin before it
+        e = np.floor((np.arange(128) + 1) * r).astype(int)
+        for lvl in range(127):
+            if 0 < e[lvl] < bins and w[lvl, e[lvl]] > 0:
+                w[lvl, e[lvl] - 1] += w[lvl, e[lvl]]
+                w[lvl, e[lvl]] = 0.0
+    return w
+
+
+def _kl_curve_f64(h, n, fold=True, shift_last=False, eps=1e-7):
+    """the entropy calibration as its definition reads, in float64, for every clipping range: P = the range's bins
+    with everything beyond folded into the last one; Q = the same bins (not folded) averaged over 128 equal
+    intervals and spread back over the bins by interval overlap; KL(P || Q)"""
+    h = h.astype(np.float64)
+    out = np.empty(2048 - 128)
+    for bins in range(128, 2048):
+        p = (eps + h[:bins]) / n
+        P = p.copy()
+        if fold:
+            P[bins - 1] += h[bins:].sum() / n
+        w = _overlap(bins, shift_last)
+        q = (w @ p) / (bins / 128.0)
+        Q = eps + w.T @ q
+        out[bins - 128] = (P * np.log(P / Q)).sum()
+    return out
+
+
+def _mse_curve_f64(h, n, levels=128):
+    """squared distance of every bin centre to the nearest of `levels` equidistant levels from 0 to the clipping
+    point (centres beyond it are nearest to the top level), weighted by the histogram; float64"""
+    h = h.astype(np.float64)
+    c = np.arange(2048) + 0.5
+    out = np.empty(2048 - 128)
+    for bins in range(128, 2048):
+        grid = np.arange(levels) * (bins / (levels - 1.0))
+        d = np.abs(c[:, None] - grid[None, :]).min(axis=1)
+        out[bins - 128] = (h * d * d).sum() / n
+    return out
+
+
+# histograms on which the winner of the float64 search stands clear of its runner-up by more than ten times the
+# float32 rounding noise of the search under test
+_TAILED = [("t1", 0.002, 3.0), ("t2", 0.0005, 6.0), ("t6", 0.02, 1.0), ("t4", 0.0001, 10.0)]
+_TAILED_MSE = [("t1", 0.002, 3.0), ("t2", 0.0005, 6.0), ("t3", 0.01, 1.5), ("t7", 0.001, 4.0)]
+
+
+@pytest.mark.parametrize("tag,frac,scale", _TAILED)
+def test_kl_search_matches_float64_definition(oracle, tag, frac, scale):
+    """the KL value of every one of the 1920 candidates against the float64 definition written with an
+    interval-overlap matrix; the winner lies inside the range, is not a multiple of 128 (fractional level edges
+    decide) and has mass beyond it (the fold into the last bin decides).  Two plausible mistakes - leaving the
+    mass beyond the range out of P, giving a level's fractional last piece to the neighbouring bin - are shown to
+    move the curve by orders of magnitude more than the tolerance, and the first also moves the winner."""
+    h = _tailed_histogram(tag, 300000, frac, scale)
+    n = int(h.sum())
+    got = oracle.calib_curve("kl", h, n).astype(np.float64)
+    want = _kl_curve_f64(h, n)
+    tol = 2e-6 + 2e-5 * np.abs(want)
+    assert np.all(np.abs(got - want) <= tol), float(np.abs(got - want).max())
+    best = int(want.argmin()) + 128
+    srt = np.sort(want)
+    assert srt[1] - srt[0] > 10 * np.abs(got - want).max()          # the winner is decided beyond float32 noise
+    assert int(got.argmin()) + 128 == best
+    assert 128 < best < 2047 and best % 128 != 0 and h[best:].sum() > 0
+    t = oracle.calib_threshold("kl", h, n, 6.5)
+    assert t == np.float32(np.float32(best + 0.5) * np.float32(6.5) / np.float32(2048))
+    nofold = _kl_curve_f64(h, n, fold=False)
+    assert np.abs(nofold - want).max() > 1e3 * tol.max() and int(nofold.argmin()) + 128 != best
+    shifted = _kl_curve_f64(h, n, shift_last=True)
+    assert np.abs(shifted - want).max() > 1e2 * tol.max()
+
+
+@pytest.mark.parametrize("tag,frac,scale", _TAILED_MSE)
+def test_mse_search_matches_float64_definition(oracle, tag, frac, scale):
+    """the loss of every candidate against nearest-level quantisation brute-forced in float64 over a histogram with
+    hundreds of occupied bins; same winner, decided beyond float32 noise.  A 128-interval grid (step = range / 128
+    instead of range / 127) is shown to fail the same comparison."""
+    h = _tailed_histogram(tag, 300000, frac, scale)
+    n = int(h.sum())
+    got = oracle.calib_curve("mse", h, n).astype(np.float64)
+    want = _mse_curve_f64(h, n)
+    assert np.all(np.abs(got - want) <= 2e-5 * want), float((np.abs(got - want) / want).max())
+    best = int(want.argmin()) + 128
+    srt = np.sort(want)
+    assert (srt[1] - srt[0]) / srt[0] > 10 * (np.abs(got - want) / want).max()
+    assert int(got.argmin()) + 128 == best and 128 < best < 2047
+    t = oracle.calib_threshold("mse", h, n, 3.25)
+    assert t == np.float32(np.float32(best + 0.5) * np.float32(3.25) / np.float32(2048))
+    wrong = _mse_curve_f64(h, n, levels=129)
+    assert (np.abs(wrong - want) / want).max() > 1e-2
+
+
 def test_calibration_percentile_rank(oracle):
     """the 99.998 % rule against a numpy sort: rank (1-p)*images*elems among the kept largest magnitudes"""
     images, elems = 3, 500000
