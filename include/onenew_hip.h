@@ -120,6 +120,18 @@ int onhip_conv2d_pack_weights(const onhip_conv_desc_t *d, const float *w, float 
 int onhip_conv2d_f32_packed(const onhip_conv_desc_t *d, const float *x, const float *w_packed, const float *bias,
                             const float *silu_lut, float *y, void *stream);
 
+/* onhip_conv2d_f32 (packed == 0) or onhip_conv2d_f32_packed (packed != 0) for callers that cannot allocate device
+ * memory: code under HIP graph capture, serving loops, harnesses that forbid it.  No counterpart in the reference.
+ * It calls no allocating routine: the partial sums of a split-K launch go to a 32 MiB array built into the library's
+ * code object (one copy per GPU, held until the process ends), tile and split come from the cost model only, and the
+ * slices are added up by a finishing launch.  A problem whose chosen split needs more than 32 MiB of partial sums
+ * (split x output bytes) is refused with ONHIP_ERR_WORKSPACE.  The array keeps the last call's contents; every
+ * element read is written first by the same call, so nothing needs clearing.  All calls on one GPU share the array:
+ * calls that may overlap there (different streams without an ordering between them) race.  Same results as the entry
+ * point it mirrors when that one runs the cost model's choice (tuning off). */
+int onhip_conv2d_f32_noalloc(const onhip_conv_desc_t *d, const float *x, const float *w, int32_t packed, const float *bias,
+                             const float *silu_lut, float *y, void *stream);
+
 /* The convolution that ends a residual block with the operators after it folded into its store:
  * y = conv(x) as onhip_conv2d_f32 (packed != 0: as onhip_conv2d_f32_packed), then y += addend (a tensor of
  * y's shape, not y itself) as device/x86/Add/add.c:96, then, with relu_after != 0, relu as

@@ -76,7 +76,40 @@ static std::mutex g_scratch_mu;
 static void *g_scratch = nullptr;
 static size_t g_scratch_bytes = 0;
 
+// ---- the entry point that allocates nothing ------------------------------------------------------
+// Its split-K partial sums go to a device array that is part of the code object: every GPU the library runs on holds
+// its own copy for the life of the process.  The name `scratch` is a host-side handle, not a device address: host code
+// asks the runtime for the array's address once per device and passes that on.
+static const size_t kNoAllocScratchBytes = (size_t) 32 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+static const int kMaxDevices = 64;
+static void *g_noalloc_ptr[kMaxDevices];      // address of `scratch` on each device, once looked up there
+static thread_local void *tl_noalloc = nullptr;   // non-null while this thread runs the entry point: get_scratch hands it out
+
+// address of this device's copy of `scratch`; looked up with that device current, no allocation involved
+static int noalloc_scratch(void **out) {
+    int dev = -1;
+    ONHIP_CHECK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return set_error(ONHIP_ERR_RUNTIME, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_noalloc_ptr[dev]) {
+        void *ptr = nullptr;
+        ONHIP_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return set_error(ONHIP_ERR_RUNTIME, "no device address for the built-in scratch array");
+        g_noalloc_ptr[dev] = ptr;
+    }
+    *out = g_noalloc_ptr[dev];
+    return ONHIP_OK;
+}
+
 static int get_scratch(size_t bytes, void **out) {
+    if (tl_noalloc) {
+        if (bytes > kNoAllocScratchBytes)
+            return set_error(ONHIP_ERR_WORKSPACE, "conv (no allocation): the split-K partial sums of this problem take %zu bytes, "
+                             "the built-in scratch holds %zu; use onhip_conv2d_f32", bytes, kNoAllocScratchBytes);
+        *out = tl_noalloc;
+        return ONHIP_OK;
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     if (bytes > g_scratch_bytes) {
         if (g_scratch) {
@@ -346,6 +379,9 @@ static int time_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStrea
 
 // Chooses tile, split and tail handling for the problem and launches it.
 static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t st) {
+    // the entry point that allocates nothing: the cost model's choice (never the in-launch reduction, whose uncached
+    // workspace is allocated on first use; no measuring, which creates events and may grow buffers)
+    if (tl_noalloc) return launch_choice(cfg, p, model_choice(cfg, p), st);
     if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB[xFIN]]]]
         Choice c = {0, 0, 1, 0, 0, 0};
         if (sscanf(env, "%dx%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 2) {
@@ -474,7 +510,8 @@ int onhip_init(int device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(ONHIP_ERR_RUNTIME, "device %d is %s; this library holds gfx950 code only", device,
                          prop.gcnArchName);
-    return ONHIP_OK;
+    void *ptr = nullptr;
+    return noalloc_scratch(&ptr);   // this device's address of the built-in scratch array, for onhip_conv2d_f32_noalloc
 }
 
 int onhip_set_tuning(int mode) {
@@ -619,6 +656,17 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
 int onhip_conv2d_f32_packed(const onhip_conv_desc_t *d, const float *x, const float *w_packed, const float *bias,
                             const float *silu_lut, float *y, void *stream) {
     return conv2d_f32_impl(d, x, w_packed, 1, bias, silu_lut, y, stream);
+}
+
+int onhip_conv2d_f32_noalloc(const onhip_conv_desc_t *d, const float *x, const float *w, int32_t packed, const float *bias,
+                             const float *silu_lut, float *y, void *stream) {
+    void *ptr = nullptr;
+    int rc = noalloc_scratch(&ptr);   // a lookup on the first call on a device (onhip_init has done it already), no allocation
+    if (rc) return rc;
+    tl_noalloc = ptr;
+    rc = conv2d_f32_impl(d, x, w, packed ? 1 : 0, bias, silu_lut, y, stream);
+    tl_noalloc = nullptr;
+    return rc;
 }
 
 static void w8a32_layout(const onhip_conv_desc_t *d, int *cp, int *k_units, size_t *packed_bytes, size_t *q_bytes) {

@@ -31,7 +31,7 @@ def plugin_path(op):
 
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
-           "onhip_conv2d_f32_add", "onhip_conv_add_eval", "onhip_conv_add_relu_eval",
+           "onhip_conv2d_f32_add", "onhip_conv2d_f32_noalloc", "onhip_conv_add_eval", "onhip_conv_add_relu_eval",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
            "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quantize_nhwc_s8",
            "onhip_conv2d_w8a8_nhwc", "onhip_quant_weight_bias",
@@ -63,6 +63,7 @@ def load():
     L.onhip_conv2d_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
     L.onhip_conv2d_f32_packed.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_conv2d_f32_add.argtypes = [C.POINTER(ConvDesc), vp, vp, C.c_int32, vp, vp, vp, C.c_int32, vp, vp]
+    L.onhip_conv2d_f32_noalloc.argtypes = [C.POINTER(ConvDesc), vp, vp, C.c_int32, vp, vp, vp, vp]
     L.onhip_conv2d_w8a32_workspace.argtypes = [C.POINTER(ConvDesc)]
     L.onhip_conv2d_w8a32_workspace.restype = C.c_size_t
     L.onhip_conv2d_w8a32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t, vp]
@@ -137,6 +138,14 @@ def conv2d_f32(d, x, w, bias=None, silu_lut=None, out=None, packed=False):
         out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device=x.device)
     fn = load().onhip_conv2d_f32_packed if packed else load().onhip_conv2d_f32
     _check(fn(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(silu_lut), _ptr(out), _stream()), "onhip_conv2d_f32")
+    return out
+
+
+def conv2d_f32_noalloc(d, x, w, out, bias=None, silu_lut=None, packed=False):
+    """conv2d_f32 through the entry point that allocates nothing: the caller brings the output tensor, split-K partial
+    sums go to the array built into the library"""
+    _check(load().onhip_conv2d_f32_noalloc(C.byref(d), _ptr(x), _ptr(w), int(bool(packed)), _ptr(bias), _ptr(silu_lut),
+                                           _ptr(out), _stream()), "onhip_conv2d_f32_noalloc")
     return out
 
 
