@@ -1,0 +1,254 @@
+"""The benchmark configurations at their stated sizes, every layer: ResNet-50 batch 32 (53 convolutions), MobileNetV2
+batch 64 (52, of which 17 depthwise), the ViT-Tiny MatMuls at B = 64 in fp32 and bf16, YOLOv8s int8 batch 16 (63
+convolutions, fp32-in/out W8A32 form and int8 NHWC chain form).  What the benchmark times is what is checked here.
+
+Tensors of this size are drawn on the device (seeded) and only what the check needs comes back to the host: for a
+dense convolution the input patches of a few thousand sampled outputs, which are then evaluated on the CPU - float64
+cross-correlation for fp32 (bar 1e-4 of the largest sampled value), the exact integer closed form of
+device/x86/Conv/conv.c:961-973,1024-1056 for int8 (int64 sum, then the three separately rounded fp32 operations,
+the table and the re-quantisation through the oracle's own functions; bar: equality).  Depthwise layers are compared
+bit for bit with the oracle on whole images of the batch; the MatMuls with the oracle on the whole product."""
+import numpy as np
+import pytest
+
+import cases
+from onenew_amd import abi, datagen, hip, stacks
+from onenew_amd.abi import ConvDesc
+
+pytestmark = pytest.mark.gpu
+
+SAMPLES = 2000
+
+
+@pytest.fixture(scope="module")
+def torch_dev():
+    import torch
+    assert torch.cuda.is_available(), "no GPU visible"
+    hip.init(0)
+    return torch
+
+
+def _seed(*parts):
+    return datagen.seed_for("fullsize", *parts) & 0x7FFFFFFFFFFF
+
+
+def _device_uniform(torch, seed, shape, lo=-1.0, hi=1.0):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    return torch.rand(shape, generator=g, device="cuda", dtype=torch.float32) * (hi - lo) + lo
+
+
+def _sample_index(seed, d, count=SAMPLES):
+    """sampled outputs as (image, channel, row, column) index arrays; corners and edges of the first and last image and
+    channel are always among them (padding, the last tile's ragged rows and columns)"""
+    oh, ow = d.out_hw()
+    total = d.n * d.cout * oh * ow
+    flat = datagen.integers(seed, (min(count, total),), 0, total - 1)
+    fixed = [((n * d.cout + m) * oh + i) * ow + j for n in (0, d.n - 1) for m in (0, d.cout - 1)
+             for i in (0, oh - 1) for j in (0, ow - 1)]
+    flat = np.unique(np.concatenate([flat, np.array(fixed, np.int64)]))
+    n, r = np.divmod(flat, d.cout * oh * ow)
+    m, r = np.divmod(r, oh * ow)
+    i, j = np.divmod(r, ow)
+    return flat, n, m, i, j
+
+
+def _patches(torch, x, d, n, i, j):
+    """input patches [S, cin, kh, kw] of the sampled outputs, zero where the window hangs over the padding; pure data
+    movement on the device, returned as a host array"""
+    dv = x.device
+    n_t = torch.from_numpy(n).to(dv)
+    ih = torch.from_numpy(i * d.stride_h - d.pad_t).to(dv)[:, None] + torch.arange(d.kh, device=dv)[None, :]
+    iw = torch.from_numpy(j * d.stride_w - d.pad_l).to(dv)[:, None] + torch.arange(d.kw, device=dv)[None, :]
+    ok = ((ih >= 0) & (ih < d.h))[:, :, None] & ((iw >= 0) & (iw < d.w))[:, None, :]           # [S, kh, kw]
+    ihc, iwc = ih.clamp(0, d.h - 1), iw.clamp(0, d.w - 1)
+    c = torch.arange(d.cin, device=dv)
+    p = x[n_t[:, None, None, None], c[None, :, None, None], ihc[:, None, :, None], iwc[:, None, None, :]]
+    p = p * ok[:, None, :, :].to(p.dtype)
+    return p.cpu().numpy()
+
+
+def _act_f64(d, v):
+    if not d.has_bias or d.act_type == abi.NOT_ACT:
+        return v
+    if d.act_type == abi.RELU:
+        return np.maximum(v, 0.0)
+    if d.act_type == abi.CLIP:
+        return np.minimum(np.maximum(v, d.clip_min), d.clip_max)
+    raise AssertionError("activation not used by these stacks")
+
+
+def _check_dense_f32(torch, tag, name, d, w_std=None):
+    x = _device_uniform(torch, _seed(tag, name, "x"), (d.n, d.cin, d.h, d.w))
+    fan_in = d.cin * d.kh * d.kw
+    w = datagen.normal(_seed(tag, name, "w"), (d.cout, d.cin, d.kh, d.kw), 0.0, w_std or float(np.sqrt(2.0 / fan_in)))
+    b = datagen.normal(_seed(tag, name, "b"), (d.cout,), 0.0, 0.01)
+    wd, bd = torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()
+    wp = hip.pack_conv_weights(d, wd)
+    y = hip.conv2d_f32(d, x, wp if wp is not None else wd, bd, packed=wp is not None)
+    torch.cuda.synchronize()
+    flat, n, m, i, j = _sample_index(_seed(tag, name, "probe"), d)
+    got = y.reshape(-1)[torch.from_numpy(flat).cuda()].cpu().numpy().astype(np.float64)
+    p = _patches(torch, x, d, n, i, j).astype(np.float64)
+    ref = _act_f64(d, np.einsum("sckl,sckl->s", p, w[m].astype(np.float64)) + b[m].astype(np.float64))
+    scale = max(float(np.abs(ref).max()), 1e-6)
+    assert np.abs(got - ref).max() <= 1e-4 * scale, f"{name}: {np.abs(got - ref).max():.3e} against {scale:.3e}"
+    assert np.all(np.abs(got - ref) <= 1e-4 * np.abs(ref) + 1e-5), name
+    assert bool(torch.isfinite(y).all())
+
+
+def _check_depthwise_f32(torch, oracle, tag, name, d):
+    x = _device_uniform(torch, _seed(tag, name, "x"), (d.n, d.cin, d.h, d.w))
+    w = datagen.normal(_seed(tag, name, "w"), (d.cout, 1, d.kh, d.kw), 0.0, 0.05)
+    b = datagen.normal(_seed(tag, name, "b"), (d.cout,), 0.0, 0.01)
+    y = hip.conv2d_f32(d, x, torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda())
+    torch.cuda.synchronize()
+    d1 = ConvDesc.from_buffer_copy(d)
+    d1.n = 1
+    pick = sorted({0, d.n - 1, int(datagen.integers(_seed(tag, name, "img"), (1,), 0, d.n - 1)[0])})
+    for img in pick:
+        ref = oracle.conv2d_f32(d1, x[img:img + 1].cpu().numpy(), w, b)
+        assert np.array_equal(y[img:img + 1].cpu().numpy(), ref), f"{name}: image {img} differs from the oracle"
+    # the images the oracle did not see: each is a function of its own input alone, so a copy of image `a` put
+    # in place of image `c` must reproduce image a's result there
+    a, c = pick[0], (pick[0] + 1) % d.n
+    x2 = x.clone()
+    x2[c] = x[a]
+    y2 = hip.conv2d_f32(d, x2, torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(y2[c], y[a])
+    keep = [k for k in range(d.n) if k != c]
+    assert torch.equal(y2[keep], y[keep])
+
+
+RESNET = stacks.with_batch(stacks.resnet50(), 32)
+MOBILENET = stacks.with_batch(stacks.mobilenet_v2(), 64)
+YOLO = stacks.with_batch(stacks.yolov8s(), 16)
+
+
+@pytest.mark.parametrize("layer", range(len(RESNET)), ids=[n for n, _ in RESNET])
+def test_resnet50_batch32_every_layer(layer, torch_dev):
+    name, d = RESNET[layer]
+    print(f"resnet50 b32 {name}", flush=True)
+    _check_dense_f32(torch_dev, "rn50b32", name, d)
+
+
+@pytest.mark.parametrize("layer", range(len(MOBILENET)), ids=[n for n, _ in MOBILENET])
+def test_mobilenetv2_batch64_every_layer(layer, torch_dev, oracle):
+    name, d = MOBILENET[layer]
+    print(f"mobilenetv2 b64 {name}", flush=True)
+    if d.group != 1:
+        _check_depthwise_f32(torch_dev, oracle, "mbv2b64", name, d)
+    else:
+        _check_dense_f32(torch_dev, "mbv2b64", name, d, w_std=0.05)
+
+
+# ---- ViT-Tiny MatMuls at B = 64 -------------------------------------------------------------------------------
+
+VIT = stacks.vit_tiny(64)
+
+
+@pytest.mark.parametrize("compute", [abi.COMPUTE_F32, abi.COMPUTE_BF16, abi.COMPUTE_F16], ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("layer", range(len(VIT)), ids=[v[0] for v in VIT])
+def test_vit_tiny_batch64_every_matmul(layer, compute, torch_dev, oracle):
+    torch = torch_dev
+    name, md, has_bias, gelu = VIT[layer]
+    print(f"vit b64 {name} compute {compute}", flush=True)
+    ashape = (md.batch, md.m, md.k)
+    bshape = (md.k, md.n) if md.b_shared else (md.batch, md.k, md.n)
+    a = datagen.normal(_seed("vit", name, "a"), ashape, 0.0, 1.0)
+    b = datagen.normal(_seed("vit", name, "b"), bshape, 0.0, 0.02)
+    bias = datagen.normal(_seed("vit", name, "bias"), (md.n,), 0.0, 0.02) if has_bias else None
+    lut = cases.gelu_lut() if gelu else None
+    cu = lambda t: None if t is None else torch.from_numpy(t).cuda()
+    y = hip.matmul(cu(a), cu(b), bias=cu(bias), compute=compute)          # pre-activation
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+
+    def full(aa, bb):
+        r = oracle.matmul_f32(aa, bb)
+        return r + bias if has_bias else r
+
+    ref32 = full(a, b)
+    scale = float(np.abs(ref32).max())
+    if compute == abi.COMPUTE_F32:
+        assert np.abs(y - ref32).max() <= 1e-4 * scale, name
+        assert np.all(np.abs(y - ref32) <= 1e-4 * np.abs(ref32) + 1e-5), name
+    else:
+        rnd = oracle.round_bf16 if compute == abi.COMPUTE_BF16 else oracle.round_f16
+        ref16 = full(rnd(a), rnd(b))                 # operands rounded to the 16-bit type, fp32 accumulation
+        assert np.abs(y - ref16).max() <= 1e-4 * scale, name
+        assert np.abs(y - ref32).max() <= 1e-2 * scale, name
+    if gelu:
+        # the fused table activation, judged exactly on the kernel's own pre-activation
+        yg = hip.matmul(cu(a), cu(b), bias=cu(bias), gelu_lut=cu(lut), compute=compute)
+        torch.cuda.synchronize()
+        assert np.array_equal(yg.cpu().numpy(), oracle.lut_act(y, lut)), name
+
+
+# ---- YOLOv8s int8, batch 16 ---------------------------------------------------------------------------------------
+
+def _yolo_operands(torch, i, name, d):
+    d = ConvDesc.from_buffer_copy(d)
+    d.input_scale = float(datagen.uniform(_seed("yolo", i, "s_in"), (1,), 0.005, 0.05)[0])
+    # activations as the configuration draws them: U(-1, 1), scaled so that a few per cent clip at +-127 steps
+    x = _device_uniform(torch, _seed("yolo", name, "x"), (d.n, d.cin, d.h, d.w)) * float(d.input_scale * 140.0)
+    w8 = datagen.integers(_seed("yolo", name, "w"), (d.cout, d.cin, d.kh, d.kw), -127, 127).astype(np.int8)
+    b32 = datagen.integers(_seed("yolo", name, "b"), (d.cout,), -100, 100).astype(np.int32)
+    s_w = float(datagen.uniform(_seed("yolo", name, "aux"), (1,), 0.005, 0.05)[0])
+    aux = np.full((d.cout,), np.float32(127.0) * np.float32(s_w), np.float32)      # per-tensor weight scale
+    return d, x, w8, b32, aux
+
+
+def _int8_closed_form(oracle, d, patches, w8, b32, aux, m, lut):
+    """conv.c:961-973 (quantise), :1024-1039 (int32 sum), :1041-1056 (three rounded fp32 operations), do_act"""
+    q = oracle.quantize_s8(patches, d.input_scale).astype(np.int64)
+    acc = np.einsum("sckl,sckl->s", q, w8[m].astype(np.int64))
+    assert np.abs(acc).max() < 2 ** 31
+    f = acc.astype(np.int32).astype(np.float32)
+    f = f * np.float32(d.input_scale)
+    f = f + b32[m].astype(np.float32)
+    y = f * (aux[m] * np.float32(1.0) / np.float32(127.0))
+    if d.act_type == abi.SILU:
+        y = oracle.lut_act(y, lut)
+    return acc.astype(np.int32), y.astype(np.float32)
+
+
+@pytest.mark.parametrize("layer", range(len(YOLO)), ids=[n for n, _ in YOLO])
+def test_yolov8s_int8_batch16_every_layer(layer, torch_dev, oracle):
+    torch = torch_dev
+    name, d0 = YOLO[layer]
+    print(f"yolov8s b16 {name}", flush=True)
+    d, x, w8, b32, aux = _yolo_operands(torch, layer, name, d0)
+    lut = cases.silu_lut()
+    cu = lambda t: torch.from_numpy(t).cuda()
+    w8d, b32d, auxd, lutd = cu(w8), cu(b32), cu(aux), cu(lut)
+    oh, ow = d.out_hw()
+    flat, n, m, i, j = _sample_index(_seed("yolo", name, "probe"), d)
+    flat_t = torch.from_numpy(flat).cuda()
+    acc_ref, y_ref = _int8_closed_form(oracle, d, _patches(torch, x, d, n, i, j), w8, b32, aux, m, lut)
+
+    # the reference's form: fp32 NCHW in and out, int32 accumulators on request
+    wp = hip.pack_conv_weights_w8(d, w8d)
+    acc = torch.empty((d.n, d.cout, oh, ow), dtype=torch.int32, device="cuda")
+    y = hip.conv2d_w8a32(d, x, wp, b32d, auxd, lutd, acc32=acc, packed=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.reshape(-1)[flat_t].cpu().numpy(), acc_ref), f"{name}: int32 accumulators differ"
+    assert np.array_equal(y.reshape(-1)[flat_t].cpu().numpy(), y_ref), f"{name}: de-quantised outputs differ"
+    y_full = y
+    del acc
+
+    # the chain form: int8 NHWC in, int8 NHWC out; equals the consumer's own quantisation of the fp32 result
+    dq = ConvDesc.from_buffer_copy(d)
+    dq.out_s8, dq.output_scale = 1, 0.03
+    xq = hip.quantize_nhwc_s8(x, d.input_scale)
+    cpo = (d.cout + 15) // 16 * 16
+    out = torch.full((d.n, oh, ow, cpo), 77, dtype=torch.int8, device="cuda")
+    hip.conv2d_w8a8_nhwc(dq, xq, wp, b32d, auxd, lutd, out=out)
+    torch.cuda.synchronize()
+    q_ref = oracle.quantize_s8(y_ref, dq.output_scale)
+    nhwc = ((n * oh + i) * ow + j) * cpo + m
+    assert np.array_equal(out.reshape(-1)[torch.from_numpy(nhwc).cuda()].cpu().numpy(), q_ref), f"{name}: chain form differs"
+    # and, over the whole tensor, the chain form is the quantisation of the fp32 form's result (same accumulators)
+    want = hip.quantize_nhwc_s8(y_full, dq.output_scale)
+    assert torch.equal(out[..., :d.cout], want[..., :d.cout]), f"{name}: chain form is not the quantised fp32 form everywhere"
