@@ -408,20 +408,19 @@ def test_whole_model_folds_every_residual_block(model, torch_dev, monkeypatch):
 
 @pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
 def test_whole_model_matches_the_reference_host_run(model, torch_dev):
-    """the full-size network at batch 1 (89 / 65 operators) through the runtime against the same file run by the
-    reference's host operator classes and x86 kernels on the CPU: logits within 1e-3 of their largest magnitude
-    (53 / 52 convolutions deep with fp32 sums in another order), same top-5 classes"""
-    from onenew_amd import stacks
-    if not one_model.have_ref_runner():
-        pytest.skip("oracle/_ref/ref_run_one is not built")
-    make = stacks.resnet50_model if model == "resnet50" else stacks.mobilenet_v2_model
-    data, shape, _ = make(1)
-    x = np.random.default_rng(3).normal(size=shape).astype(np.float32)
-    (_, ref), = one_model.run_reference(data, [x])
+    """the full-size network at batch 1 (89 / 65 operators) through the runtime against the logits the reference's
+    host operator classes and x86 kernels gave for the same file and input (tests/golden/model_logits.npz, written by
+    tests/golden/make_model_logits.py): within 1e-3 of their largest magnitude (53 / 52 convolutions deep with fp32
+    sums in another order), same top-5 classes"""
+    import hashlib
+    import make_model_logits
+    data, x = make_model_logits.model_and_input(model)
+    fix = np.load(make_model_logits.OUT)
+    assert hashlib.sha256(data).digest() == fix[model + "_sha256"].tobytes(), "the model file changed: regenerate the fixture"
+    ref = fix[model + "_logits"]
     net = rt.Net(data)
     (got,) = net.run(x)
     assert got.shape == ref.shape == (1, 1000)
     assert np.isfinite(got).all()
     assert _close(got, ref, 1e-3)
     assert set(np.argsort(got[0])[-5:]) == set(np.argsort(ref[0])[-5:])
-

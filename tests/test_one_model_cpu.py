@@ -243,3 +243,16 @@ def test_plan_of_random_residual_graphs(seed):
     folded = len(m["nodes"]) - len(net.ops())
     assert 0 <= folded <= 2 * net.fused_blocks() + net.folded_relus()
     assert folded >= net.fused_blocks() + net.folded_relus()
+
+
+@pytest.mark.parametrize("model", ["resnet50", "mobilenetv2"])
+def test_full_size_model_oracle_reproduces_the_reference_logits(model):
+    """the CPU restatement of the runtime on the full-size model files against the logits the reference's host classes
+    gave for them (tests/golden/model_logits.npz): the same convolution arithmetic, so the same bits"""
+    import hashlib
+    import make_model_logits
+    data, x = make_model_logits.model_and_input(model)
+    fix = np.load(make_model_logits.OUT)
+    assert hashlib.sha256(data).digest() == fix[model + "_sha256"].tobytes(), "the model file changed: regenerate the fixture"
+    (got,) = one_model.run(data, [x])
+    assert np.array_equal(got, fix[model + "_logits"])
