@@ -32,14 +32,25 @@ HBM_PEAK_GBS = 8000.0
 
 # ---- layers: device-resident operands + one launch -------------------------------------------------------
 
+def device_uniform(torch, seed, shape, lo=-1.0, hi=1.0):
+    """activations U(lo, hi) drawn on the device from a seeded generator (the large tensors of batch 16 to 64 take
+    longer to draw on the host than the whole measurement)"""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed & 0x7FFFFFFFFFFF)
+    return torch.rand(shape, generator=g, device="cuda", dtype=torch.float32) * (hi - lo) + lo
+
+
 class ConvF32Layer:
     kind = "conv_f32"
 
     def __init__(self, torch, hip, name, d, tag):
-        import cases
-        x, w, b = cases.conv_inputs(f"{tag}/{name}", d)
+        from onenew_amd import datagen
+        kc = d.cin if d.group == 1 else 1
+        w = datagen.normal(datagen.seed_for(f"{tag}/{name}", "w"), (d.cout, kc, d.kh, d.kw), 0.0, float(np.sqrt(2.0 / (kc * d.kh * d.kw))))
+        b = datagen.normal(datagen.seed_for(f"{tag}/{name}", "b"), (d.cout,), 0.0, 0.01)
         self.name, self.d = name, d
-        self.x, self.w, self.b = (torch.from_numpy(t).cuda() for t in (x, w, b))
+        self.x = device_uniform(torch, datagen.seed_for(f"{tag}/{name}", "x"), (d.n, d.cin, d.h, d.w))
+        self.w, self.b = torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()
         self.y = torch.empty((d.n, d.cout) + d.out_hw(), dtype=torch.float32, device="cuda")
         # k x k weights are re-laid out once at load time (tap-major), as an inference runtime would
         self.wp = hip.pack_conv_weights(d, self.w)
@@ -75,9 +86,13 @@ class ConvW8A32Layer:
 
     def __init__(self, torch, hip, name, d, tag):
         import cases
-        x, w8, b32, aux = cases.conv_inputs(f"{tag}/{name}", d, quant=True)
+        from onenew_amd import datagen
+        d1 = type(d).from_buffer_copy(d)
+        d1.n, d1.h, d1.w = 1, d.kh, d.kw          # the weight-side operands of the case, without its activations
+        _, w8, b32, aux = cases.conv_inputs(f"{tag}/{name}", d1, quant=True)
         self.name, self.d = name, d
-        self.x, self.w8, self.b32, self.aux = (torch.from_numpy(t).cuda() for t in (x, w8, b32, aux))
+        self.x = device_uniform(torch, datagen.seed_for(f"{tag}/{name}", "x"), (d.n, d.cin, d.h, d.w))
+        self.w8, self.b32, self.aux = (torch.from_numpy(t).cuda() for t in (w8, b32, aux))
         self.lut = torch.from_numpy(cases.silu_lut()).cuda()
         self.y = torch.empty((d.n, d.cout) + d.out_hw(), dtype=torch.float32, device="cuda")
         self.ws = torch.empty(max(16, hip.conv2d_w8a32_workspace(d)), dtype=torch.uint8, device="cuda")
@@ -508,6 +523,99 @@ def bench_net(torch, args):
     print(json.dumps(line))
 
 
+METRIC = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vit_tiny_glue_ops_fp32_tflops",
+          "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
+          "yolov8s_int8chain": "yolov8s_conv_stack_w8a8_tops", "yolov8s": "yolov8s_conv_stack_w8a32_tops",
+          "vit": "vit_tiny_matmul_{dtype}_tflops", "cfg1": "conv2d_relu_fp32_tflops"}
+
+# the other configurations of the benchmark, timed after the headline one in a default run
+OTHER_CONFIGS = ["cfg1", "resnet50_b1", "mobilenetv2_b64", "mobilenetv2_b1", "vit_tiny_b64", "vit_tiny_b64_bf16", "vit_tiny_b1",
+                 "yolov8s_int8_b16", "yolov8s_int8chain_b16", "yolov8s_int8chain_b1"]
+
+
+def run_workload(torch, hip, name, steps, warmup, layers_table=False):
+    """times one workload: `warmup` untimed passes (tile choices are measured there when tuning is on), `steps` timed
+    passes between two device synchronisations, then every layer on its own with HIP events on the launch stream"""
+    desc, dtype, layers = make_workload(torch, hip, name)
+    unit = "TOP/s" if dtype == "i8" else "TFLOP/s"
+    flops = sum(L.flops for L in layers)
+    abytes = sum(L.bytes for L in layers)
+
+    for _ in range(warmup):
+        for L in layers:
+            L.launch(hip)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for L in layers:
+            L.launch(hip)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+
+    # Roofline of the dominant kernel.  Dense layers all run onhip::igemm_kernel (MFMA-bound); depthwise layers run
+    # onhip::depthwise_*_kernel (HBM-bound).  Whichever group takes more time is reported: algorithmic work of its
+    # launches / their average durations, from events on the launch stream.
+    per_layer_ms = time_layers(torch, hip, layers, reps=max(10, steps))
+    groups = {True: [], False: []}
+    for L, t in zip(layers, per_layer_ms):
+        groups[L.dense].append((L, t))
+    dom_dense = sum(t for _, t in groups[True]) >= sum(t for _, t in groups[False])
+    grp = groups[dom_dense]
+    g_ms = sum(t for _, t in grp)
+    g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
+    kernel = (f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
+              "element-wise / pooling / normalisation kernels (elementwise.hip, vit_glue.hip)" if grp[0][0].kind == "glue"
+              else "onhip::depthwise_tiled_kernel")
+    # the bound is the roof the group's arithmetic intensity puts it under
+    mfma_bound = dom_dense and g_flops / g_bytes >= PEAK[dtype] * 1e12 / (HBM_PEAK_GBS * 1e9)
+    if mfma_bound:
+        achieved, peak, r_unit, work = g_flops / (g_ms * 1e-3) / 1e12, PEAK[dtype], unit, g_flops
+        step_frac = flops / (ms_per_step * 1e-3) / 1e12 / peak
+    else:
+        achieved, peak, r_unit, work = g_bytes / (g_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", g_bytes
+        step_frac = abytes / (ms_per_step * 1e-3) / 1e9 / peak
+    group = "igemm" if dom_dense else "glue" if grp[0][0].kind == "glue" else "depthwise"
+    traffic = measured_traffic(name, group)
+    roofline = {"kernel": kernel, "bound": "mfma" if mfma_bound else "hbm", "achieved": round(achieved, 3),
+                "peak": peak, "unit": r_unit, "frac": round(achieved / peak, 4),
+                "traffic": traffic,
+                "traffic_source": None if traffic is None else
+                f"profiles/{name}_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload, summarised by "
+                f"onenew_amd/profile_summary.py; a committed figure, not measured in this run)",
+                "launches": len(grp), "avg_launch_ms": round(g_ms / len(grp), 5),
+                "work_per_launch": work / len(grp),
+                "arithmetic_intensity": round(g_flops / g_bytes, 2),
+                # the same fraction from the wall time of the timed passes (layers back to back, cold caches between them)
+                "frac_whole_step": round(step_frac, 4)}
+    res = {"name": name, "desc": desc, "dtype": dtype, "unit": unit, "flops": flops, "abytes": abytes,
+           "ms_per_step": ms_per_step, "per_layer_ms": per_layer_ms, "roofline": roofline, "layers": layers,
+           "value": flops / (ms_per_step * 1e-3) / 1e12}
+    if layers_table:
+        print(f"{'layer':<18}{'shape':<32}{'ms':>9}{unit:>9}{'%mfma':>7}{'GB/s':>8}{'%hbm':>6}", file=sys.stderr)
+        for L, t in zip(layers, per_layer_ms):
+            tf = L.flops / (t * 1e-3) / 1e12
+            gb = L.bytes / (t * 1e-3) / 1e9
+            print(f"{L.name:<18}{L.shape:<32}{t:>9.4f}{tf:>9.2f}{100 * tf / PEAK[dtype]:>7.1f}{gb:>8.0f}"
+                  f"{100 * gb / HBM_PEAK_GBS:>6.1f}", file=sys.stderr)
+    return res
+
+
+def config_summary(res):
+    """the short form of a workload's result for the `configs` array of the headline line"""
+    rf = res["roofline"]
+    per = res["per_layer_ms"]
+    out = {"workload": res["name"], "what": res["desc"], "dtype": res["dtype"], "value": round(res["value"], 3), "unit": res["unit"],
+           "ms_per_step": round(res["ms_per_step"], 4), "ms_sum_of_layers": round(sum(per), 4), "layers": len(per),
+           "roofline": {k: rf[k] for k in ("bound", "achieved", "peak", "unit", "frac", "frac_whole_step", "avg_launch_ms", "launches")},
+           "algorithmic_GBps": round(res["abytes"] / (res["ms_per_step"] * 1e-3) / 1e9, 1),
+           "hbm_frac_whole_step": round(res["abytes"] / (res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    lowai = [(L, t) for L, t in zip(res["layers"], per) if not L.dense]
+    if lowai:
+        out["depthwise_GBps"] = round(sum(L.bytes for L, _ in lowai) / (sum(t for _, t in lowai) * 1e-3) / 1e9, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -518,6 +626,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-tune", action="store_true", help="use the cost model instead of measured tile choice")
     ap.add_argument("--no-batch1", action="store_true", help="skip the extra batch-1 pass over the same stack")
+    ap.add_argument("--only", action="store_true", help="time the named workload only, not the other configurations after it")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path runs on a single MI355X and nothing in this build "
@@ -544,87 +653,68 @@ def main():
     if args.workload.startswith("resnet50_net_b") or args.workload.startswith("mobilenetv2_net_b"):
         return bench_net(torch, args)
 
-    desc, dtype, layers = make_workload(torch, hip, args.workload)
-    unit = "TOP/s" if dtype == "i8" else "TFLOP/s"
-    flops = sum(L.flops for L in layers)
-    abytes = sum(L.bytes for L in layers)
+    res = run_workload(torch, hip, args.workload, args.steps, args.warmup, layers_table=args.layers)
+    layers, per_layer_ms, dtype, unit = res["layers"], res["per_layer_ms"], res["dtype"], res["unit"]
 
-    for _ in range(args.warmup):
-        for L in layers:
-            L.launch(hip)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        for L in layers:
-            L.launch(hip)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-
-    # Roofline of the dominant kernel.  Dense layers all run onhip::igemm_kernel (MFMA-bound); depthwise layers run
-    # onhip::depthwise_*_kernel (HBM-bound).  Whichever group takes more time is reported: algorithmic work of its
-    # launches / their average durations, from events on the launch stream.
-    per_layer_ms = time_layers(torch, hip, layers, reps=max(10, args.steps))
-    groups = {True: [], False: []}
-    for L, t in zip(layers, per_layer_ms):
-        groups[L.dense].append((L, t))
-    dom_dense = sum(t for _, t in groups[True]) >= sum(t for _, t in groups[False])
-    grp = groups[dom_dense]
-    g_ms = sum(t for _, t in grp)
-    g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
-    kernel = (f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
-              "element-wise / pooling / normalisation kernels (elementwise.hip, vit_glue.hip)" if grp[0][0].kind == "glue"
-              else "onhip::depthwise_tiled_kernel")
-    # the bound is the roof the group's arithmetic intensity puts it under
-    mfma_bound = dom_dense and g_flops / g_bytes >= PEAK[dtype] * 1e12 / (HBM_PEAK_GBS * 1e9)
-    if mfma_bound:
-        achieved, peak, r_unit, work = g_flops / (g_ms * 1e-3) / 1e12, PEAK[dtype], unit, g_flops
-    else:
-        achieved, peak, r_unit, work = g_bytes / (g_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", g_bytes
-    roofline = {"kernel": kernel, "bound": "mfma" if mfma_bound else "hbm", "achieved": round(achieved, 3),
-                "peak": peak, "unit": r_unit, "frac": round(achieved / peak, 4),
-                "traffic": measured_traffic(args.workload, "igemm" if dom_dense else
-                                             "glue" if grp[0][0].kind == "glue" else "depthwise"),
-                "launches": len(grp), "avg_launch_ms": round(g_ms / len(grp), 5),
-                "work_per_launch": work / len(grp),
-                "arithmetic_intensity": round(g_flops / g_bytes, 2)}
-
-    extra = {}
+    extra = {"tuning": "cost model only" if args.no_tune else
+             "tile and split-K measured once per layer shape during the warm-up passes (onhip_set_tuning(1)); the library's "
+             "default is the cost model"}
+    if not args.no_tune and args.workload == "resnet50_b32" and not args.only:
+        # the same stack with the choices a host gets by default: the cost model, nothing measured
+        hip.set_tuning(0)
+        for _ in range(2):
+            for L in layers:
+                L.launch(hip)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            for L in layers:
+                L.launch(hip)
+        torch.cuda.synchronize()
+        ms_model = (time.perf_counter() - t0) * 1e3 / args.steps
+        hip.set_tuning(1)
+        extra["cost_model_choices"] = {"ms_per_step": round(ms_model, 4), "value": round(res["flops"] / (ms_model * 1e-3) / 1e12, 3)}
     if args.workload.startswith("resnet50_b") and args.workload != "resnet50_b1" and not args.no_batch1:
         # the same stack at batch 1 (the "conv stack ms" of the reference's recorded trace)
         _, _, layers1 = make_workload(torch, hip, "resnet50_b1")
         ms1 = time_layers(torch, hip, layers1, reps=20)
         extra["resnet50_conv_stack_ms_batch1"] = round(sum(ms1), 4)
+        del layers1
     if args.workload.startswith("resnet50_b") or args.workload == "cfg1":
         extra["plugin_eval_cfg1"] = plugin_eval_latency(hip)
     extra["stack_ms_sum_of_layers"] = round(sum(per_layer_ms), 4)
-    extra["algorithmic_GBps"] = round(abytes / (sum(per_layer_ms) * 1e-3) / 1e9, 1)
+    extra["algorithmic_GBps"] = round(res["abytes"] / (sum(per_layer_ms) * 1e-3) / 1e9, 1)
     lowai = [(L, t) for L, t in zip(layers, per_layer_ms) if not L.dense]
     if lowai:
         extra["depthwise_GBps"] = round(sum(L.bytes for L, _ in lowai) / (sum(t for _, t in lowai) * 1e-3) / 1e9, 1)
         extra["depthwise_ms"] = round(sum(t for _, t in lowai), 4)
 
-    if args.layers:
-        print(f"{'layer':<18}{'shape':<32}{'ms':>9}{unit:>9}{'%mfma':>7}{'GB/s':>8}{'%hbm':>6}", file=sys.stderr)
-        for L, t in zip(layers, per_layer_ms):
-            tf = L.flops / (t * 1e-3) / 1e12
-            gb = L.bytes / (t * 1e-3) / 1e9
-            print(f"{L.name:<18}{L.shape:<32}{t:>9.4f}{tf:>9.2f}{100 * tf / PEAK[dtype]:>7.1f}{gb:>8.0f}"
-                  f"{100 * gb / HBM_PEAK_GBS:>6.1f}", file=sys.stderr)
-
     cpu = None if args.no_cpu else cpu_baseline(layers, args.workload, unit)
 
-    metric = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vit_tiny_glue_ops_fp32_tflops", "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
-              "yolov8s_int8chain": "yolov8s_conv_stack_w8a8_tops", "yolov8s": "yolov8s_conv_stack_w8a32_tops", "vit": f"vit_tiny_matmul_{dtype}_tflops",
-              "cfg1": "conv2d_relu_fp32_tflops"}
-    key = next(k for k in metric if args.workload.startswith(k))
-    line = {"metric": metric[key], "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": unit, "n_gpus": 1,
-            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+    key = next(k for k in METRIC if args.workload.startswith(k))
+    line = {"metric": METRIC[key].format(dtype=dtype), "value": round(res["value"], 3), "unit": unit, "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-            "config": {"workload": desc, "layers": len(layers), "ops_per_step": flops,
-                       "algorithmic_bytes_per_step": abytes},
-            "roofline": roofline, "cpu_baseline": cpu}
+            "config": {"workload": res["desc"], "layers": len(layers), "ops_per_step": res["flops"],
+                       "algorithmic_bytes_per_step": res["abytes"]},
+            "roofline": res["roofline"], "cpu_baseline": cpu}
     line.update(extra)
+
+    if args.workload == "resnet50_b32" and not args.only:
+        # every other configuration of the benchmark, each timed the same way (fewer passes), as extra keys
+        del layers, res, lowai
+        configs = []
+        for name in OTHER_CONFIGS:
+            torch.cuda.empty_cache()
+            t0 = time.perf_counter()
+            r = run_workload(torch, hip, name, steps=10, warmup=3)
+            c = config_summary(r)
+            c["bench_seconds"] = round(time.perf_counter() - t0, 1)
+            configs.append(c)
+            print(f"[bench] {name}: {c['value']} {c['unit']}, {c['ms_per_step']} ms per step, roofline {c['roofline']['bound']} "
+                  f"{c['roofline']['frac']}", file=sys.stderr, flush=True)
+            del r
+        line["configs"] = configs
     print(json.dumps(line))
 
 
