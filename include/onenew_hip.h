@@ -94,6 +94,10 @@ int onhip_set_tuning(int mode);
 /* Diagnostic, no counterpart in the reference: how many launches so far cut their leftover tiles (those beyond a
  * whole number of rounds of 256 tiles) into K slices next to the whole tiles of the same launch. */
 long long onhip_split_tail_launches(void);
+/* Diagnostic, no counterpart in the reference: size in bytes of the library's split-K scratch block (0 before the first
+ * split launch).  The block grows by allocating a larger one; an outgrown block is kept until the process ends, because
+ * a HIP graph recorded by the caller may hold its address. */
+long long onhip_scratch_bytes(void);
 /* Output height / width of a convolution (host/ops/conv.h:43-50). Returns 0 or ONHIP_ERR_ARG. */
 int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow);
 

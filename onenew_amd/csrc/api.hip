@@ -75,6 +75,7 @@ static int check_conv(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow) {
 static std::mutex g_scratch_mu;
 static void *g_scratch = nullptr;
 static size_t g_scratch_bytes = 0;
+static long long g_scratch_generation = 0;   // how many blocks have been allocated so far
 
 // ---- the entry point that allocates nothing ------------------------------------------------------
 // Its split-K partial sums go to a device array that is part of the code object: every GPU the library runs on holds
@@ -112,15 +113,17 @@ static int get_scratch(size_t bytes, void **out) {
     }
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     if (bytes > g_scratch_bytes) {
-        if (g_scratch) {
-            ONHIP_CHECK_HIP(hipDeviceSynchronize());
-            ONHIP_CHECK_HIP(hipFree(g_scratch));
-            g_scratch = nullptr;
-            g_scratch_bytes = 0;
-        }
-        const size_t want = bytes < (64u << 20) ? (64u << 20) : bytes;
-        ONHIP_CHECK_HIP(hipMalloc(&g_scratch, want));
+        // A HIP graph recorded by a caller holds the current block's address in its kernel arguments, and its replays
+        // keep writing and reading partial sums there: a block that is outgrown is kept until the process ends (the
+        // replays then have it to themselves), never freed.  Sizes at least double, so all retired blocks together are
+        // smaller than the live one.
+        size_t want = bytes < (64u << 20) ? (64u << 20) : bytes;
+        if (want < 2 * g_scratch_bytes) want = 2 * g_scratch_bytes;
+        void *fresh = nullptr;
+        ONHIP_CHECK_HIP(hipMalloc(&fresh, want));
+        g_scratch = fresh;
         g_scratch_bytes = want;
+        ++g_scratch_generation;
     }
     *out = g_scratch;
     return ONHIP_OK;
@@ -132,8 +135,15 @@ static int get_scratch(size_t bytes, void **out) {
 static void *g_uc = nullptr;
 static int *g_arrive = nullptr;
 static const size_t kUcBytes = (size_t) 256 << 20;
+static bool g_arrive_dirty = false;   // a launch that counts arrivals failed: the counters may not be back at zero
 static int get_uc(void **buf, int **arrive) {
     std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_arrive && g_arrive_dirty) {
+        ONHIP_CHECK_HIP(hipDeviceSynchronize());
+        ONHIP_CHECK_HIP(hipMemset(g_arrive, 0, 4 << 20));
+        ONHIP_CHECK_HIP(hipDeviceSynchronize());
+        g_arrive_dirty = false;
+    }
     if (!g_uc || !g_arrive) {   // both or neither: a call that fails half-way leaves what it got for the next one
         if (!g_uc) ONHIP_CHECK_HIP(hipExtMallocWithFlags(&g_uc, kUcBytes, hipDeviceMallocUncached));
         void *ctr = nullptr;
@@ -236,21 +246,23 @@ static int apply_choice(IgemmLaunch &cfg, IgemmParams &p, const Choice &c) {
         const int tiles_per = (k_tiles + c.split - 1) / c.split;
         const int split = (k_tiles + tiles_per - 1) / tiles_per;
         if (split > 1) {
-            void *buf = nullptr;
             const size_t bytes = (size_t) split * cfg.batch * p.M * (p.N - p.part_begin) * 4;
-            int rc = get_scratch(bytes, &buf);
-            if (rc) return rc;
+            int rc;
             cfg.split = split;
             p.k_split_units = tiles_per * upt;
-            p.partial = reinterpret_cast<float *>(buf);
             p.arrive = nullptr;
-            if (c.fin && cfg.dtype != DT_I8 && bytes <= kUcBytes) {
+            if (c.fin && cfg.dtype != DT_I8 && bytes <= kUcBytes && !tl_noalloc) {
                 void *uc; int *arr;
                 rc = get_uc(&uc, &arr);
                 if (rc) return rc;
                 p.partial = reinterpret_cast<float *>(uc);
                 p.arrive = arr;
                 p.n_slices = split;
+            } else {
+                void *buf = nullptr;
+                rc = get_scratch(bytes, &buf);
+                if (rc) return rc;
+                p.partial = reinterpret_cast<float *>(buf);
             }
         }
     }
@@ -278,7 +290,20 @@ static bool tail_geometry(const IgemmLaunch &cfg, const IgemmParams &p, int bm, 
     return true;
 }
 
+static const int kRowbTiles[][2] = {{64, 128}, {128, 128}, {64, 256}, {96, 128}, {32, 256}, {32, 512}};
+static const int kNumRowbTiles = 6;
+
+// (bm, bn) is a tile this build has a kernel for
+static bool tile_exists(const Choice &c) {
+    const int (*list)[2] = c.rowb ? kRowbTiles : kTiles;
+    const int n = c.rowb ? kNumRowbTiles : kNumTiles;
+    for (int t = 0; t < n; ++t)
+        if (list[t][0] == c.bm && list[t][1] == c.bn) return true;
+    return false;
+}
+
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
+    if (!tile_exists(c)) return false;   // e.g. a line of the cache file written by another build or by hand
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
     if (c.rowb && (c.split != 1 || !rowb_f32_ok(cfg, p))) return false;
     if (c.fin) {
@@ -334,7 +359,14 @@ static std::atomic<long long> g_tail_launches{0};
 static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
     int dpc = 0, left = 0;
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
-    auto launch = [&]() { return c.rowb ? rowb_f32_launch(cfg, p, st) : igemm_launch(cfg, p, st); };
+    auto launch = [&]() {
+        const int rc = c.rowb ? rowb_f32_launch(cfg, p, st) : igemm_launch(cfg, p, st);
+        if (rc && p.arrive) {   // whatever part of the launch ran may have left arrival counters above zero
+            std::lock_guard<std::mutex> lock(g_scratch_mu);
+            g_arrive_dirty = true;
+        }
+        return rc;
+    };
     if (c.tail <= 1 || !tail_geometry(cfg, p, c.bm, c.bn, &dpc, &left)) {
         const Choice plain = {c.bm, c.bn, c.rowb ? 1 : c.split, 0, 0, c.rowb ? 0 : c.fin};
         int rc = apply_choice(cfg, p, plain);
@@ -452,8 +484,7 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
         }
     }
     // the kernel without LDS for B, where the problem allows it
-    static const int kRowbTiles[][2] = {{64, 128}, {128, 128}, {64, 256}, {96, 128}, {32, 256}, {32, 512}};
-    for (int t = 0; t < 6 && !rc; ++t) {
+    for (int t = 0; t < kNumRowbTiles && !rc; ++t) {
         if (kRowbTiles[t][0] == 32 && p.M > 32) continue;   // one row tile of up to 32 output channels
         if (kRowbTiles[t][0] == 96 && p.M % 96 > 0 && p.M % 96 <= 64) continue;   // a last row tile that a 64-row tile covers as well
         const Choice c = {kRowbTiles[t][0], kRowbTiles[t][1], 1, 0, 1, 0};
@@ -519,6 +550,11 @@ int onhip_set_tuning(int mode) {
     const int prev = tune_mode();
     g_tune_mode = mode > 0 ? 1 : 0;
     return prev;
+}
+
+long long onhip_scratch_bytes(void) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    return (long long) g_scratch_bytes;
 }
 
 long long onhip_split_tail_launches(void) { return g_tail_launches.load(std::memory_order_relaxed); }

@@ -512,8 +512,14 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
 __device__ __forceinline__ unsigned to_bits(float v) { return __float_as_uint(v); }
 __device__ __forceinline__ unsigned to_bits(int v) { return (unsigned) v; }
 
-// split-K: raw partial sums [split][batch][M][N]; the finishing kernel applies the epilogue
-template <int TM, int TN, class ACC>
+// cache policy bits of the raw-buffer instructions on gfx950: sc0 (bit 0) and sc1 (bit 4) together give an access system
+// scope: a store is written through to memory before it is acknowledged, a load does not hit a line that another XCD's
+// store has made stale.  The in-launch split-K reduction puts them on the partial sums it publishes and reads back.
+constexpr int AUX_SYSTEM_SCOPE = 0x11;
+
+// split-K: raw partial sums [split][batch][M][N]; the finishing kernel applies the epilogue.  PUBLISH: the sums are read
+// back by another workgroup of the same launch (system-scope stores); otherwise by the finishing launch.
+template <int TM, int TN, bool PUBLISH, class ACC>
 __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[TM][TN], int slice, int m_wave,
                                               int n_wave, int li, int lh) {
     const int width = p.N - p.part_begin;   // partial sums cover the columns from part_begin on
@@ -531,7 +537,7 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
                 const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
                 const auto val = acc[a][b][r];   // element copy first: bit-casting the vector element in place miscompiles
                 __builtin_amdgcn_raw_buffer_store_b32(to_bits(val), rp, row_ok ? cv : OOB,
-                                                      (unsigned) m_uni * (unsigned) width * 4u, 0);
+                                                      (unsigned) m_uni * (unsigned) width * 4u, PUBLISH ? AUX_SYSTEM_SCOPE : 0);
             }
     }
 }
@@ -835,13 +841,17 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
 
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
     if (p.partial && !whole_k) {
-        write_partial<TM, TN>(p, acc, slice * gridDim.z + batch, m_wave, n_wave, li, lh);
-        if (DT == DT_I8 || !p.arrive) return;   // a finishing launch adds the slices up
-        // The reduction inside the launch.  Partial sums and counters live in uncached memory: once this workgroup's
-        // stores are acknowledged it counts itself in, and the last of a tile's slices to arrive adds all of them up
-        // in slice order (the order of the finishing kernel: the same bits) and goes on to the epilogue as if it had
-        // computed the whole tile.  Nobody waits for anybody, so the launch cannot hang; the counter is back at zero
-        // for the next launch.
+        if (DT == DT_I8 || !p.arrive) {   // a finishing launch adds the slices up
+            write_partial<TM, TN, false>(p, acc, slice * gridDim.z + batch, m_wave, n_wave, li, lh);
+            return;
+        }
+        write_partial<TM, TN, true>(p, acc, slice * gridDim.z + batch, m_wave, n_wave, li, lh);
+        // The reduction inside the launch.  Partial sums and counters live in uncached memory and are stored and
+        // loaded with system scope (AUX_SYSTEM_SCOPE): once this workgroup's stores are acknowledged (written
+        // through, vmcnt(0)) it counts itself in with a device-scope atomic, and the last of a tile's slices to arrive
+        // adds all of them up in slice order (the order of the finishing kernel: the same bits) with loads that
+        // bypass the caches, and goes on to the epilogue as if it had computed the whole tile.  Nobody waits for
+        // anybody, so the launch cannot hang; the counter is back at zero for the next launch.
         __shared__ int s_last;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -882,7 +892,8 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
                                 const int r = 8 * h + q;
                                 const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
                                 const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
-                                v[q] = buf_load_f32(rp, row_ok ? cv : OOB, (unsigned) m_uni * (unsigned) width * 4u);
+                                v[q] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(
+                                    rp, row_ok ? cv : OOB, (unsigned) m_uni * (unsigned) width * 4u, AUX_SYSTEM_SCOPE));
                             }
 #pragma unroll
                             for (int q = 0; q < 8; ++q) acc[a][b][8 * h + q] = __fadd_rn(acc[a][b][8 * h + q], v[q]);

@@ -133,10 +133,17 @@ static bool is_device_ptr(const void *p) {
 static int stage_buf(int slot, size_t bytes, void **out) {
     DevBuf &b = g_stage[slot];
     if (bytes > b.bytes) {
-        if (b.ptr) ONHIP_CHECK_HIP(hipFree(b.ptr));
+        size_t want = (bytes + (1u << 20) - 1) & ~((size_t) (1u << 20) - 1);
+        if (slot == 3) {
+            // the workspace is a kernel argument of launches a caller may have recorded into a HIP graph (the int8 copy
+            // of a W8A32 convolution's activations): an outgrown block stays allocated for those replays, sizes at least
+            // double so the retired blocks together stay below the live one
+            if (want < 2 * b.bytes) want = 2 * b.bytes;
+        } else if (b.ptr) {
+            ONHIP_CHECK_HIP(hipFree(b.ptr));   // host staging: only synchronous copies of this library touch it
+        }
         b.ptr = nullptr;
         b.bytes = 0;
-        const size_t want = (bytes + (1u << 20) - 1) & ~((size_t) (1u << 20) - 1);
         ONHIP_CHECK_HIP(hipMalloc(&b.ptr, want));
         b.bytes = want;
     }

@@ -208,6 +208,53 @@ def test_graph_replay_matches_plain_launches(name, torch_dev, monkeypatch):
     assert float(scratch[0]) == 5.0
 
 
+def test_recorded_graph_survives_growth_of_the_shared_workspaces(torch_dev, monkeypatch):
+    """net A (a split-K convolution and a W8A32 convolution) records its graph; then a net with larger operands makes
+    the library's split-K scratch and the plugin's int8 workspace grow; replays of A afterwards still equal plain
+    launches bit for bit, because the blocks its recording points at are retired, not freed"""
+    from oracle import oracle as orc
+    torch = torch_dev
+    rng = np.random.default_rng(77)
+
+    def model(n, c, hw, q_hw):
+        m = onefile.OneModel()
+        m.input("x", (n, c, hw, hw))
+        m.conv("c1", "x", _w(rng, c, c, 3, 3) * 0.2, _w(rng, c), "c1_out", pad=1, act=abi.RELU)
+        w8, b32, aux = orc.quant_weight_bias(_w(rng, 32, c, 3, 3), _w(rng, 32))
+        m.conv("q1", "c1_out", w8, b32, "out", pad=1, act=abi.RELU, quant=(aux, 0.05))
+        m.output("out", (n, 32, hw, hw))
+        return m.tobytes(), rng.normal(size=(n, c, hw, hw)).astype(np.float32)
+
+    data_a, xa = model(1, 256, 14, 14)          # 256 -> 256 3x3 on 14 x 14: sixteen tiles, the cost model splits K
+    plain = rt.Net(data_a)
+    monkeypatch.setenv("ONENEW_RT_GRAPH", "1")
+    graphed = rt.Net(data_a)
+    monkeypatch.delenv("ONENEW_RT_GRAPH")
+    for rep in range(2):                        # the second run records
+        got = graphed.run(xa * np.float32(1.0 + rep))
+    before = hip.load().onhip_scratch_bytes()
+    assert before > 0, "net A did not use the split-K scratch"
+    # a larger net, every convolution forced to eight K slices: 8 x n x 64 x 56 x 56 x 4 B of partial sums, with the batch
+    # n chosen so that they exceed the block the process has so far (other tests may have grown it already)
+    n_b = before // (8 * 64 * 56 * 56 * 4) + 2
+    data_b, xb = model(int(n_b), 64, 56, 56)
+    monkeypatch.setenv("ONHIP_TILE", "64x64x8")
+    big = rt.Net(data_b)
+    big.run(xb)
+    monkeypatch.delenv("ONHIP_TILE")
+    torch.cuda.synchronize()
+    assert hip.load().onhip_scratch_bytes() > before, "the scratch did not grow: the test does not test what it says"
+    filler = torch.full((64 << 20,), 3.0, device="cuda")      # whatever the allocator hands out next
+    for rep in range(3):
+        cur = (xa * np.float32(0.5 + rep)).astype(np.float32)
+        got = graphed.run(cur)
+        filler.mul_(1.0)
+        torch.cuda.synchronize()
+        want = plain.run(cur)
+        assert np.array_equal(got[0], want[0]), rep
+    assert graphed.graph_launches() >= 3
+
+
 def _w(rng, *shape):
     return (rng.normal(size=shape) * 0.2).astype(np.float32)
 
