@@ -94,6 +94,15 @@ int onhip_set_tuning(int mode);
 /* Diagnostic, no counterpart in the reference: how many launches so far cut their leftover tiles (those beyond a
  * whole number of rounds of 256 tiles) into K slices next to the whole tiles of the same launch. */
 long long onhip_split_tail_launches(void);
+/* The model-wide GEMM tile of a .one file: BLOCK_INFO_S.cuda_gemm_tile_{m,n} (common/nn_common.h:28-39), which the
+ * reference's tuner fills for its x86 kernels (tools/optimize/auto_tuning.hpp:9-75) and its converter defaults to
+ * 16 x 16 (tools/onnx2one/onnx2one.cpp:1346-1349).  onhip_set_tile_hint(bm, bn) makes the cost model of the calling
+ * thread choose among the K splits of that workgroup tile only, when bm x bn is a tile this library has kernels for
+ * (returns 1); any other pair, 16 x 16 included, clears the hint (returns 0).  Measured choices (onhip_set_tuning(1))
+ * and ONHIP_TILE take precedence.  The Conv plugin sets it around each call from params[11] (USEFUL_INFO_S).
+ * onhip_tile_candidate(idx, ...) lists the tiles (ONHIP_ERR_ARG past the last one). */
+int onhip_set_tile_hint(int32_t bm, int32_t bn);
+int onhip_tile_candidate(int32_t idx, int32_t *bm, int32_t *bn);
 /* Diagnostic, no counterpart in the reference: size in bytes of the library's split-K scratch block (0 before the first
  * split launch).  The block grows by allocating a larger one; an outgrown block is kept until the process ends, because
  * a HIP graph recorded by the caller may hold its address. */

@@ -116,6 +116,24 @@ int onrt_net_operand(const onrt_net_t *net, const char *name, int32_t *ndim, int
  */
 int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs);
 
+/*
+ * The model-wide GEMM tile: BLOCK_INFO_S.cuda_gemm_tile_{m,n,k} in the file header (common/nn_common.h:28-39;
+ * the converter writes 16 / 16 / 16, tools/onnx2one/onnx2one.cpp:1346-1349), which every Conv call finds in its last
+ * params slot (host/ops/conv.h:65-68).  The reference's tuner searches the tiles of its x86 GEMM on one 1024-cubed
+ * product and writes them to the header (tools/optimize/auto_tuning.hpp:9-75); this one measures the loaded model
+ * itself: onrt_net_tune_tiles runs the net with every workgroup tile the Conv plugin's library has kernels for, and
+ * with none (each layer's tile from the cost model), `reps` timed inferences each on whatever the input buffers hold,
+ * keeps the fastest (a candidate must win by 2 %, as auto_tuning.hpp:41) and leaves it set on the net; best_ms /
+ * default_ms (may be NULL) are the fastest inference with it and with the converter's default.  tiles[2] is the depth
+ * of a K tile in fp32 values (16), informational.  onrt_one_set_tiles writes a triple into the header of a file
+ * image, so that every later load (onrt_net_load_*) starts from it; onrt_net_get_tiles / _set_tiles read and replace
+ * the triple of a loaded net or a plan (a recorded graph is dropped and recorded again).
+ */
+int onrt_net_tune_tiles(onrt_net_t *net, int32_t reps, int32_t tiles[3], float *best_ms, float *default_ms);
+int onrt_net_get_tiles(const onrt_net_t *net, int32_t tiles[3]);
+int onrt_net_set_tiles(onrt_net_t *net, const int32_t tiles[3]);
+int onrt_one_set_tiles(void *one_buf, size_t bytes, const int32_t tiles[3]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -340,16 +340,25 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
     return cycles;
 }
 
+// A tile the caller asks for (onhip_set_tile_hint): the model-wide GEMM tile a .one file carries in
+// BLOCK_INFO_S.cuda_gemm_tile_{m,n} (common/nn_common.h:28-39).  While it is set on a thread, the cost model chooses
+// among the splits of that tile only; measured choices (tuning mode 1) and ONHIP_TILE take precedence.
+static thread_local int tl_hint_bm = 0, tl_hint_bn = 0;
+
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     Choice best = {64, 64, 1, 0, 0, 0};
-    double best_cost = 1e300;
-    for (int t = 0; t < kNumTiles; ++t)
-        for (int s = 0; s < kNumSplits; ++s) {
-            const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0, 0};
-            if (!candidate_ok(cfg, p, c)) continue;
-            const double cost = model_cost(cfg, p, c);
-            if (cost < best_cost) { best_cost = cost; best = c; }
-        }
+    for (int pass = tl_hint_bm ? 0 : 1; pass < 2; ++pass) {   // pass 0: the hinted tile; pass 1: every tile
+        double best_cost = 1e300;
+        for (int t = 0; t < kNumTiles; ++t)
+            for (int s = 0; s < kNumSplits; ++s) {
+                const Choice c = {kTiles[t][0], kTiles[t][1], kSplits[s], 0, 0, 0};
+                if (pass == 0 && (c.bm != tl_hint_bm || c.bn != tl_hint_bn)) continue;
+                if (!candidate_ok(cfg, p, c)) continue;
+                const double cost = model_cost(cfg, p, c);
+                if (cost < best_cost) { best_cost = cost; best = c; }
+            }
+        if (best_cost < 1e300) break;
+    }
     return best;
 }
 
@@ -550,6 +559,22 @@ int onhip_set_tuning(int mode) {
     const int prev = tune_mode();
     g_tune_mode = mode > 0 ? 1 : 0;
     return prev;
+}
+
+int onhip_set_tile_hint(int32_t bm, int32_t bn) {
+    const Choice c = {bm, bn, 1, 0, 0, 0};
+    if (bm > 0 && bn > 0 && tile_exists(c)) {
+        tl_hint_bm = bm; tl_hint_bn = bn;
+        return 1;
+    }
+    tl_hint_bm = tl_hint_bn = 0;
+    return 0;
+}
+
+int onhip_tile_candidate(int32_t idx, int32_t *bm, int32_t *bn) {
+    if (idx < 0 || idx >= kNumTiles || !bm || !bn) return set_error(ONHIP_ERR_ARG, "tile candidate: index %d of %d", idx, kNumTiles);
+    *bm = kTiles[idx][0]; *bn = kTiles[idx][1];
+    return ONHIP_OK;
 }
 
 long long onhip_scratch_bytes(void) {

@@ -266,6 +266,12 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         rc = stage_buf(2, out_bytes, &y);
         if (rc) return rc;
     }
+    // the model-wide GEMM tile the file carries (host/ops/conv.h:65-68 puts USEFUL_INFO_S in the last params slot): a
+    // tile this library has kernels for narrows the cost model's choice, anything else (the converter's 16 x 16) does not
+    struct HintScope {
+        HintScope(const USEFUL_INFO_S *u) { if (u) onhip_set_tile_hint(u->block_info.cuda_gemm_tile_m, u->block_info.cuda_gemm_tile_n); }
+        ~HintScope() { onhip_set_tile_hint(0, 0); }
+    } hint(reinterpret_cast<const USEFUL_INFO_S *>(params[BUF_MAXNUM - 1].addr));
     if (int8) {
         if (d.cout > 4096) return set_error(ONHIP_ERR_ARG, "Conv eval: weight_aux holds 4096 channels, cout is %d", d.cout);
         rc = const_on_device(cfg->weight_aux, (size_t) d.cout * 4, &aux);

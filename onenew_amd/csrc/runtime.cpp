@@ -22,6 +22,7 @@
 #include <memory>
 #include <set>
 #include <string>
+#include <array>
 #include <vector>
 
 #include <hip/hip_runtime_api.h>
@@ -851,6 +852,107 @@ ONRT_API int onrt_net_operand(const onrt_net_t *net, const char *name, int32_t *
     if (shape) memcpy(shape, it->second.desc.shapes, sizeof(int32_t) * SHAPE_LEN);
     if (dev_ptr) *dev_ptr = it->second.dev;
     return ONRT_OK;
+}
+
+// ---- the model-wide GEMM tile (tools/optimize/auto_tuning.hpp:9-75 is the reference's search for its x86 kernels) ----
+
+// drops a recorded graph: its launches were chosen under another tile
+static void forget_graph(onrt_net &net) {
+    if (net.graph_exec) (void) hipGraphExecDestroy(net.graph_exec);
+    if (net.graph) (void) hipGraphDestroy(net.graph);
+    net.graph_exec = nullptr;
+    net.graph = nullptr;
+    net.graph_launches = 0;
+    net.runs = 0;
+}
+
+ONRT_API int onrt_net_get_tiles(const onrt_net_t *net, int32_t tiles[3]) {
+    if (!net || !tiles) return fail(ONRT_ERR_ARG, "tiles: null argument");
+    const BLOCK_INFO_S &b = net->useful.block_info;
+    tiles[0] = b.cuda_gemm_tile_m; tiles[1] = b.cuda_gemm_tile_n; tiles[2] = b.cuda_gemm_tile_k;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_set_tiles(onrt_net_t *net, const int32_t tiles[3]) {
+    if (!net || !tiles) return fail(ONRT_ERR_ARG, "tiles: null argument");
+    BLOCK_INFO_S &b = net->useful.block_info;   // the struct every Conv call finds in its last params slot
+    b.cuda_gemm_tile_m = tiles[0]; b.cuda_gemm_tile_n = tiles[1]; b.cuda_gemm_tile_k = tiles[2];
+    if (!net->plan_only) {
+        (void) hipDeviceSynchronize();
+        forget_graph(*net);
+    }
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_one_set_tiles(void *one_buf, size_t bytes, const int32_t tiles[3]) {
+    if (!one_buf || !tiles) return fail(ONRT_ERR_ARG, "tiles: null argument");
+    if (bytes < sizeof(ONE_MODEL_DESC_S)) return fail(ONRT_ERR_FORMAT, "the buffer is shorter than a .one header");
+    ONE_MODEL_DESC_S *h = static_cast<ONE_MODEL_DESC_S *>(one_buf);
+    if (h->one_model_magic_num != ONE_MAGIC_NUM)
+        return fail(ONRT_ERR_FORMAT, "one_model_magic_num is 0x%x, a .one file starts with 0x%x", h->one_model_magic_num, ONE_MAGIC_NUM);
+    BLOCK_INFO_S &b = h->useful_info.block_info;
+    b.cuda_gemm_tile_m = tiles[0]; b.cuda_gemm_tile_n = tiles[1]; b.cuda_gemm_tile_k = tiles[2];
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_tune_tiles(onrt_net_t *net, int32_t reps, int32_t tiles[3], float *best_ms, float *default_ms) {
+    if (!net || !tiles) return fail(ONRT_ERR_ARG, "tune: null argument");
+    if (net->plan_only) return fail(ONRT_ERR_ARG, "tune: this net is a plan (onrt_net_plan_buf): load it to tune it");
+    if (reps < 1) reps = 5;
+    // the candidates come from the Conv plugin's library when it lists them (onhip_tile_candidate), in the process
+    // already; a library without the list has nothing to choose from
+    typedef int (*cand_fn)(int32_t, int32_t *, int32_t *);
+    cand_fn cand = nullptr;
+    auto conv = net->handles.find("Conv");   // a handle's lookup covers the libraries it depends on
+    if (conv != net->handles.end()) cand = reinterpret_cast<cand_fn>(dlsym(conv->second, "onhip_tile_candidate"));
+    std::vector<std::array<int32_t, 3>> options;
+    options.push_back({16, 16, 16});   // the converter's default: no tile this library has, every layer by the cost model
+    for (int32_t i = 0; cand; ++i) {
+        int32_t bm = 0, bn = 0;
+        if (cand(i, &bm, &bn) != 0) break;
+        options.push_back({bm, bn, 16});   // a K tile is four 16-byte units: 16 fp32 values
+    }
+    std::vector<const void *> ins;
+    for (const std::string &name : net->in_names) ins.push_back(net->tensors[name].dev);   // whatever the buffers hold
+    std::vector<void *> outs(net->out_names.size(), nullptr);
+    hipEvent_t e0, e1;
+    ONRT_HIP(hipEventCreate(&e0));
+    ONRT_HIP(hipEventCreate(&e1));
+    const bool graph_wanted = net->graph_wanted;
+    net->graph_wanted = false;
+    hipStream_t keep = net->stream;
+    net->stream = nullptr;            // plain launches on the default stream while measuring
+    int rc = ONRT_OK;
+    float best = 1e30f, deflt = 0.f;
+    std::array<int32_t, 3> best_opt = options[0];
+    for (const auto &o : options) {
+        rc = onrt_net_set_tiles(net, o.data());
+        for (int i = 0; i < 2 && !rc; ++i) rc = onrt_net_run(net, ins.data(), outs.data());   // packs weights, warms caches
+        float fastest = 1e30f;
+        for (int i = 0; i < reps && !rc; ++i) {
+            if (hipEventRecord(e0, nullptr) != hipSuccess) { rc = fail(ONRT_ERR_RUNTIME, "hipEventRecord failed"); break; }
+            rc = onrt_net_run(net, ins.data(), outs.data());
+            if (rc) break;
+            float ms = 0.f;
+            if (hipEventRecord(e1, nullptr) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+                hipEventElapsedTime(&ms, e0, e1) != hipSuccess) { rc = fail(ONRT_ERR_RUNTIME, "event timing failed"); break; }
+            fastest = ms < fastest ? ms : fastest;
+        }
+        if (rc) break;
+        if (&o == &options[0]) deflt = fastest;
+        // like the reference's search (auto_tuning.hpp:41), a candidate has to win by 2 % to replace the one before it
+        if (fastest < 0.98f * best) { best = fastest; best_opt = o; }
+    }
+    (void) hipEventDestroy(e0);
+    (void) hipEventDestroy(e1);
+    net->stream = keep;
+    net->graph_wanted = graph_wanted;
+    if (rc) return rc;
+    rc = onrt_net_set_tiles(net, best_opt.data());
+    for (int k = 0; k < 3; ++k) tiles[k] = best_opt[k];
+    if (best_ms) *best_ms = best;
+    if (default_ms) *default_ms = deflt;
+    return rc;
 }
 
 ONRT_API int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs) {

@@ -7,7 +7,8 @@ import numpy as np
 from . import hip
 
 EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
-           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf"]
+           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf",
+           "onrt_net_tune_tiles", "onrt_net_get_tiles", "onrt_net_set_tiles", "onrt_one_set_tiles"]
 
 _lib = None
 
@@ -43,6 +44,10 @@ def load():
     L.onrt_net_fused_count.argtypes = [vp, i32p, i32p]
     L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
     L.onrt_net_run.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
+    L.onrt_net_tune_tiles.argtypes = [vp, C.c_int32, i32p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    L.onrt_net_get_tiles.argtypes = [vp, i32p]
+    L.onrt_net_set_tiles.argtypes = [vp, i32p]
+    L.onrt_one_set_tiles.argtypes = [C.c_char_p, C.c_size_t, i32p]
     _lib = L
     return L
 
@@ -50,6 +55,14 @@ def load():
 def _check(rc, what):
     if rc != 0:
         raise OnrtError(f"{what} failed ({rc}): {load().onrt_last_error().decode(errors='replace')}")
+
+
+def with_tiles(one_bytes, tiles):
+    """a copy of a .one file image with BLOCK_INFO_S.cuda_gemm_tile_{m,n,k} of its header set to `tiles`"""
+    buf = C.create_string_buffer(bytes(one_bytes), len(one_bytes))
+    t = (C.c_int32 * 3)(*tiles)
+    _check(load().onrt_one_set_tiles(buf, len(one_bytes), t), "onrt_one_set_tiles")
+    return buf.raw
 
 
 class Net:
@@ -107,6 +120,24 @@ class Net:
         n = C.c_int32()
         _check(load().onrt_net_fused_count(self._h, None, C.byref(n)), "onrt_net_fused_count")
         return n.value
+
+    def tiles(self):
+        """the model-wide GEMM tile (m, n, k) the net runs with: BLOCK_INFO_S.cuda_gemm_tile_* of its file, or what
+        tune_tiles / set_tiles left"""
+        t = (C.c_int32 * 3)()
+        _check(load().onrt_net_get_tiles(self._h, t), "onrt_net_get_tiles")
+        return tuple(t)
+
+    def set_tiles(self, tiles):
+        t = (C.c_int32 * 3)(*tiles)
+        _check(load().onrt_net_set_tiles(self._h, t), "onrt_net_set_tiles")
+
+    def tune_tiles(self, reps=5):
+        """measures the net with every workgroup tile of the Conv plugin's library and with none; leaves the fastest
+        set and returns (tiles, ms with it, ms with the converter's default)"""
+        t, best, deflt = (C.c_int32 * 3)(), C.c_float(), C.c_float()
+        _check(load().onrt_net_tune_tiles(self._h, reps, t, C.byref(best), C.byref(deflt)), "onrt_net_tune_tiles")
+        return tuple(t), best.value, deflt.value
 
     def operand(self, name):
         """(shape, device address) of an operand"""

@@ -5,6 +5,7 @@ the reference's host classes and x86 kernels in tests/test_one_model_cpu.py).
 Tolerances: a chain that contains Conv / MatMul / Gemm accumulates in a different order than the CPU, fp32
 relative 1e-4 of the output's largest magnitude per operator it passes through (stated per test); chains of the
 exact operators (Add, Relu, MaxPool, Transpose, views) are bit-exact."""
+import ctypes as C
 import os
 import sys
 
@@ -471,3 +472,43 @@ def test_whole_model_matches_the_reference_host_run(model, torch_dev):
     assert np.isfinite(got).all()
     assert _close(got, ref, 1e-3)
     assert set(np.argsort(got[0])[-5:]) == set(np.argsort(ref[0])[-5:])
+
+
+def test_tile_tuner_writes_the_header_and_the_runtime_reads_it_back(torch_dev):
+    """onrt_net_tune_tiles measures the loaded model under every workgroup tile of the library and leaves the fastest
+    set; written into the file header (BLOCK_INFO_S.cuda_gemm_tile_*) it is what the next load runs with; whatever the
+    tile, the results stay those of the oracle"""
+    from onenew_amd import stacks
+    data, ins = one_models.resnet_block()
+    ref = one_model.run(data, ins)
+    net = rt.Net(data)
+    assert net.tiles() == (16, 16, 16)
+    tiles, best_ms, default_ms = net.tune_tiles(reps=3)
+    cands = [(16, 16, 16)]
+    i, bm, bn = 0, C.c_int32(), C.c_int32()
+    while hip.load().onhip_tile_candidate(i, C.byref(bm), C.byref(bn)) == 0:
+        cands.append((bm.value, bn.value, 16))
+        i += 1
+    assert len(cands) >= 4 and tiles in cands and net.tiles() == tiles
+    assert 0 < best_ms <= default_ms
+    for g, r in zip(net.run(*ins), ref):
+        assert _close(g, r, 5e-4)
+    # every tile, forced through the header of the file: same results within the fp32 bar, and the tile is really used
+    # (a 3x3 convolution on 20 x 20 pixels and 16 channels under 128 x 128 and 32 x 128 tiles sums in another order)
+    outs = {}
+    for t in cands[1:]:
+        n2 = rt.Net(rt.with_tiles(data, t))
+        assert n2.tiles() == t
+        outs[t] = n2.run(*ins)
+        for g, r in zip(outs[t], ref):
+            assert _close(g, r, 5e-4), t
+    # the full-size model: the tuner's choice is at least as fast as the default and keeps the logits
+    data, shape, _ = stacks.resnet50_model(1)
+    x = np.random.default_rng(5).normal(size=shape).astype(np.float32)
+    net = rt.Net(data)
+    (before,) = net.run(x)
+    tiles, best_ms, default_ms = net.tune_tiles(reps=3)
+    print("ResNet-50 batch 1: tile", tiles, "best", best_ms, "ms, default", default_ms, "ms", flush=True)
+    (after,) = net.run(x)
+    assert best_ms <= default_ms and _close(after, before, 1e-3)
+    assert set(np.argsort(after[0])[-5:]) == set(np.argsort(before[0])[-5:])

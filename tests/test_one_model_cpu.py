@@ -256,3 +256,25 @@ def test_full_size_model_oracle_reproduces_the_reference_logits(model):
     assert hashlib.sha256(data).digest() == fix[model + "_sha256"].tobytes(), "the model file changed: regenerate the fixture"
     (got,) = one_model.run(data, [x])
     assert np.array_equal(got, fix[model + "_logits"])
+
+
+def test_header_tiles_are_written_and_read_back():
+    """BLOCK_INFO_S.cuda_gemm_tile_{m,n,k} of the file header (common/nn_common.h:28-39): the writer's default is the
+    converter's 16 / 16 / 16, onrt_one_set_tiles changes those three fields and nothing else, a plan reads them back"""
+    data, _ = one_models.resnet_block()
+    assert rt.Net(data, plan_only=True).tiles() == (16, 16, 16)
+    tuned = rt.with_tiles(data, (64, 128, 16))
+    assert len(tuned) == len(data)
+    h0, h1 = abi.ONE_MODEL_DESC_S.from_buffer_copy(data), abi.ONE_MODEL_DESC_S.from_buffer_copy(tuned)
+    b = h1.useful_info.block_info
+    assert (b.cuda_gemm_tile_m, b.cuda_gemm_tile_n, b.cuda_gemm_tile_k) == (64, 128, 16)
+    assert (b.x86_gemm_multi_threads_tile_m, b.x86_gemm_multi_threads_tile_n, b.x86_gemm_multi_threads_tile_k) == (32, 1024, 8)
+    off = abi.ONE_MODEL_DESC_S.useful_info.offset + abi.USEFUL_INFO_S.block_info.offset + 6 * 4
+    assert tuned[:off] == data[:off] and tuned[off + 12:] == data[off + 12:]
+    assert h0.node_cnt == h1.node_cnt
+    plan = rt.Net(tuned, plan_only=True)
+    assert plan.tiles() == (64, 128, 16)
+    plan.set_tiles((128, 128, 16))
+    assert plan.tiles() == (128, 128, 16)
+    with pytest.raises(rt.OnrtError):
+        rt.with_tiles(b"\0" * 4096, (64, 64, 16))
