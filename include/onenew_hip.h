@@ -289,15 +289,20 @@ int onhip_quant_weight_bias(const float *w, const float *bias, int32_t cout, int
  *  - onhip_calib_threshold: the clipping threshold from such a histogram; elem_count is the
  *    reference's "elements per image x images"                                   (:345-431, :585-618)
  *  - onhip_calib_percentile: x holds `images` tensors of `elems` values; the 99.998 % magnitude (:99-183)
- * The layer's input_scale is threshold / 127 (model_quant.hpp:668).  All four synchronise. */
+ * The layer's input_scale is threshold / 127 (model_quant.hpp:668).  All four synchronise.  The three passes over
+ * device data allocate nothing: they work in `workspace`, device memory of at least onhip_calib_workspace_bytes(images)
+ * bytes (images = 1 for abs_max and histogram), 8-byte aligned, which the caller may reuse from call to call. */
 #define ONHIP_CALIB_BINS 2048
 #define ONHIP_CALIB_KL 0
 #define ONHIP_CALIB_MSE 1
-int onhip_calib_abs_max(const float *x, long long n, float *max_abs, void *stream);
-int onhip_calib_histogram(const float *x, long long n, float max_abs, float *hist, void *stream);
+size_t onhip_calib_workspace_bytes(int images);
+int onhip_calib_abs_max(const float *x, long long n, float *max_abs, void *workspace, size_t workspace_bytes, void *stream);
+int onhip_calib_histogram(const float *x, long long n, float max_abs, float *hist, void *workspace, size_t workspace_bytes,
+                          void *stream);
 int onhip_calib_threshold(int method, const float *hist, long long elem_count, float max_abs,
                           float *threshold);
-int onhip_calib_percentile(const float *x, int images, int elems, float *threshold, void *stream);
+int onhip_calib_percentile(const float *x, int images, int elems, float *threshold, void *workspace, size_t workspace_bytes,
+                           void *stream);
 
 /* Plain device-to-device copy of n floats (n % 4 == 0, 16-byte aligned).  A measuring aid with no
  * counterpart in the reference: HBM traffic counters of the other kernels are scaled by what the

@@ -1,15 +1,15 @@
 // Offline quantisation support: what turns an fp32 model into the operands the W8A32 kernels take.
 //   * per-output-channel weight / bias quantiser (tools/optimize/model_quant.hpp:6-29), host arrays;
 //   * activation-scale calibration (model_quant.hpp:83-185 percentile, :197-435 KL, :437-623 MSE): the
-//     passes over the activations (running max |x|, 2048-bin histogram, largest magnitudes) run on the GPU
-//     over device-resident tensors, the search over 1920 candidate clipping bins runs on the host.
+//     passes over the activations (running max |x|, 2048-bin histogram, digit histograms of a radix selection)
+//     run on the GPU over device-resident tensors in a workspace the caller brings (nothing is allocated here),
+//     the search over 1920 candidate clipping bins and the walk over the digit histograms run on the host.
 // input_scale = threshold / 127 (model_quant.hpp:668).
-#include <hipcub/hipcub.hpp>
-
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "onhip_internal.hpp"
@@ -53,9 +53,33 @@ __global__ __launch_bounds__(256) void abs_histogram_kernel(const float *x, long
         if (local[i]) atomicAdd(&hist[i], (unsigned long long) local[i]);
 }
 
-__global__ __launch_bounds__(256) void abs_bits_kernel(const float *x, long long n, unsigned *keys) {
+// ---- radix selection on the bit patterns of |x| (which order like the values) -----------------------------------
+// One pass: the 256-bin histogram of the digit at `shift` over the keys of image blockIdx.y whose digits above it equal
+// prefix[image] (union == 0) or the single prefix[0] (union != 0: one histogram for all images, and a key takes part
+// only if it lies above its image's threshold thr[image]; images with skip[image] != 0 take no part).
+__global__ __launch_bounds__(256) void select_hist_kernel(const float *x, int elems, int shift, unsigned mask,
+                                                          const unsigned *prefix, const unsigned *thr, const unsigned *skip,
+                                                          int united, unsigned long long *hist) {
+    __shared__ unsigned local[256];
+    local[threadIdx.x] = 0;
+    __syncthreads();
+    const int img = blockIdx.y;
+    if (!united || !skip[img]) {
+        const unsigned want = prefix[united ? 0 : img];
+        const unsigned floor_key = united ? thr[img] : 0u;
+        const float *xi = x + (size_t) img * elems;
+        for (int i = blockIdx.x * 256 + threadIdx.x; i < elems; i += gridDim.x * 256) {
+            const unsigned key = __float_as_uint(xi[i]) & 0x7fffffffu;
+            if ((key & mask) == want && (!united || key > floor_key)) atomicAdd(&local[(key >> shift) & 255u], 1u);
+        }
+    }
+    __syncthreads();
+    if (local[threadIdx.x]) atomicAdd(&hist[(size_t) (united ? 0 : img) * 256 + threadIdx.x], (unsigned long long) local[threadIdx.x]);
+}
+
+__global__ __launch_bounds__(256) void fill_u64_kernel(unsigned long long *p, long long n) {
     const long long i = (long long) blockIdx.x * 256 + threadIdx.x;
-    if (i < n) keys[i] = __float_as_uint(x[i]) & 0x7fffffffu;
+    if (i < n) p[i] = 0;
 }
 
 static int grid_for(long long n) {
@@ -69,11 +93,28 @@ using namespace onhip;
 
 extern "C" {
 
-int onhip_calib_abs_max(const float *x, long long n, float *max_abs, void *stream) {
+size_t onhip_calib_workspace_bytes(int images) {
+    if (images < 1) images = 1;
+    // the 2048-bin histogram; or per image a 256-bin digit histogram, its prefix, its threshold and its skip flag
+    const size_t hist = ONHIP_CALIB_BINS * sizeof(unsigned long long);
+    const size_t sel = (size_t) images * (256 * sizeof(unsigned long long) + 3 * sizeof(unsigned));
+    return ((hist > sel ? hist : sel) + 255) / 256 * 256;
+}
+
+static int check_workspace(const char *what, void *workspace, size_t bytes, size_t need) {
+    if (!workspace || bytes < need)
+        return set_error(ONHIP_ERR_WORKSPACE, "%s: workspace of %zu bytes needed (onhip_calib_workspace_bytes), %zu given", what, need,
+                         workspace ? bytes : (size_t) 0);
+    if (reinterpret_cast<uintptr_t>(workspace) % 8) return set_error(ONHIP_ERR_WORKSPACE, "%s: workspace must be 8-byte aligned", what);
+    return ONHIP_OK;
+}
+
+int onhip_calib_abs_max(const float *x, long long n, float *max_abs, void *workspace, size_t workspace_bytes, void *stream) {
     if (!x || !max_abs || n < 1) return set_error(ONHIP_ERR_ARG, "calib abs max: bad argument");
+    int rc = check_workspace("calib abs max", workspace, workspace_bytes, sizeof(unsigned));
+    if (rc) return rc;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    unsigned *bits = nullptr;
-    ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&bits), sizeof(unsigned)));
+    unsigned *bits = static_cast<unsigned *>(workspace);
     unsigned start;
     const float cur = *max_abs > 0.0f ? *max_abs : 0.0f;
     memcpy(&start, &cur, sizeof(start));
@@ -85,27 +126,28 @@ int onhip_calib_abs_max(const float *x, long long n, float *max_abs, void *strea
     unsigned result = start;
     if (e == hipSuccess) e = hipMemcpyAsync(&result, bits, sizeof(result), hipMemcpyDeviceToHost, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void) hipFree(bits);
     if (e != hipSuccess) return set_error(ONHIP_ERR_RUNTIME, "calib abs max: %s", hipGetErrorString(e));
     memcpy(max_abs, &result, sizeof(result));
     return ONHIP_OK;
 }
 
-int onhip_calib_histogram(const float *x, long long n, float max_abs, float *hist, void *stream) {
+int onhip_calib_histogram(const float *x, long long n, float max_abs, float *hist, void *workspace, size_t workspace_bytes,
+                          void *stream) {
     if (!x || !hist || n < 1 || !(max_abs > 0.0f)) return set_error(ONHIP_ERR_ARG, "calib histogram: bad argument");
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    unsigned long long *dev = nullptr;
     const size_t bytes = ONHIP_CALIB_BINS * sizeof(unsigned long long);
-    ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&dev), bytes));
+    int rc = check_workspace("calib histogram", workspace, workspace_bytes, bytes);
+    if (rc) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    unsigned long long *dev = static_cast<unsigned long long *>(workspace);
     std::vector<unsigned long long> counts(ONHIP_CALIB_BINS, 0);
-    hipError_t e = hipMemcpyAsync(dev, counts.data(), bytes, hipMemcpyHostToDevice, st);
+    hipLaunchKernelGGL(fill_u64_kernel, dim3(ONHIP_CALIB_BINS / 256), dim3(256), 0, st, dev, (long long) ONHIP_CALIB_BINS);
+    hipError_t e = hipGetLastError();
     if (e == hipSuccess) {
         hipLaunchKernelGGL(abs_histogram_kernel, dim3(grid_for(n)), dim3(256), 0, st, x, n, max_abs, dev);
         e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipMemcpyAsync(counts.data(), dev, bytes, hipMemcpyDeviceToHost, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void) hipFree(dev);
     if (e != hipSuccess) return set_error(ONHIP_ERR_RUNTIME, "calib histogram: %s", hipGetErrorString(e));
     // the reference keeps float counters and adds 1.0f per element: past 2^24 a float counter stops growing
     for (int i = 0; i < ONHIP_CALIB_BINS; ++i) {
@@ -203,9 +245,13 @@ int onhip_calib_threshold(int method, const float *hist, long long elem_count, f
 }
 
 // Percentile (model_quant.hpp:99-183): per image the (1 - 0.99998) * 10 * elems largest magnitudes are kept; the
-// threshold is the magnitude of rank (1 - 0.99998) * images * elems among all kept ones.  Magnitudes are sorted
-// as integers (the bit pattern of |x| orders like the value) with a device radix sort.
-int onhip_calib_percentile(const float *x, int images, int elems, float *threshold, void *stream) {
+// threshold is the magnitude of rank (1 - 0.99998) * images * elems among all kept ones.  Nothing is sorted: a radix
+// selection, most significant byte first, finds per image the smallest kept magnitude T_i and how many copies of it are
+// kept, and then the wanted rank among everything kept (the keys above their image's T_i, counted on the device, plus
+// the kept copies of each T_i and the zeros the reference's list starts from, added on the host).  Eight passes over
+// the data, each a 256-bin histogram per image in the caller's workspace.
+int onhip_calib_percentile(const float *x, int images, int elems, float *threshold, void *workspace, size_t workspace_bytes,
+                           void *stream) {
     if (!x || !threshold || images < 1 || elems < 1) return set_error(ONHIP_ERR_ARG, "calib percentile: bad argument");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const float percent = 99.998 / 100;
@@ -214,35 +260,74 @@ int onhip_calib_percentile(const float *x, int images, int elems, float *thresho
     const int rank = (int) ((1 - percent) * images * elems);
     *threshold = 0.0f;
     if (total < 1 || rank >= total || keep < 1) return ONHIP_OK;
-    unsigned *keys = nullptr, *sorted = nullptr, *large = nullptr, *large_sorted = nullptr;
-    void *tmp = nullptr;
-    size_t tmp_bytes = 0, tmp2 = 0;
-    hipError_t e = hipcub::DeviceRadixSort::SortKeysDescending(nullptr, tmp_bytes, keys, sorted, elems, 0, 32, st);
-    if (e == hipSuccess) e = hipcub::DeviceRadixSort::SortKeysDescending(nullptr, tmp2, large, large_sorted, total, 0, 32, st);
-    if (tmp2 > tmp_bytes) tmp_bytes = tmp2;
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&keys), (size_t) elems * 4);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&sorted), (size_t) elems * 4);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&large), (size_t) total * 4);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&large_sorted), (size_t) total * 4);
-    if (e == hipSuccess) e = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 16);
-    if (e == hipSuccess) e = hipMemsetAsync(large, 0, (size_t) total * 4, st);
-    for (int i = 0; i < images && e == hipSuccess; ++i) {
-        hipLaunchKernelGGL(abs_bits_kernel, dim3((elems + 255) / 256), dim3(256), 0, st, x + (size_t) i * elems,
-                           (long long) elems, keys);
-        e = hipGetLastError();
-        size_t tb = tmp_bytes;
-        if (e == hipSuccess) e = hipcub::DeviceRadixSort::SortKeysDescending(tmp, tb, keys, sorted, elems, 0, 32, st);
-        if (e == hipSuccess && (long long) i * keep + keep <= total)
-            e = hipMemcpyAsync(large + (size_t) i * keep, sorted, (size_t) keep * 4, hipMemcpyDeviceToDevice, st);
+    int rc = check_workspace("calib percentile", workspace, workspace_bytes, onhip_calib_workspace_bytes(images));
+    if (rc) return rc;
+    unsigned long long *hist = static_cast<unsigned long long *>(workspace);
+    unsigned *d_prefix = reinterpret_cast<unsigned *>(hist + (size_t) images * 256);
+    unsigned *d_thr = d_prefix + images, *d_skip = d_thr + images;
+    std::vector<unsigned long long> h((size_t) images * 256);
+    std::vector<unsigned> prefix(images, 0), skip(images, 0);
+    std::vector<long long> left(images, keep - 1);   // how many larger keys of the current prefix group still precede the wanted one
+    const int blocks = elems / 2048 + 1 > 1024 ? 1024 : elems / 2048 + 1;
+    auto pass = [&](int shift, unsigned mask, int united) -> int {
+        const long long bins = (long long) (united ? 1 : images) * 256;
+        hipLaunchKernelGGL(fill_u64_kernel, dim3((unsigned) ((bins + 255) / 256)), dim3(256), 0, st, hist, bins);
+        ONHIP_CHECK_HIP(hipGetLastError());
+        ONHIP_CHECK_HIP(hipMemcpyAsync(d_prefix, prefix.data(), (size_t) images * 4, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(select_hist_kernel, dim3(blocks, images), dim3(256), 0, st, x, elems, shift, mask, d_prefix, d_thr, d_skip,
+                           united, hist);
+        ONHIP_CHECK_HIP(hipGetLastError());
+        ONHIP_CHECK_HIP(hipMemcpyAsync(h.data(), hist, (size_t) bins * 8, hipMemcpyDeviceToHost, st));
+        ONHIP_CHECK_HIP(hipStreamSynchronize(st));
+        return ONHIP_OK;
+    };
+    // per image: the keep-th largest key
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        const unsigned mask = shift == 24 ? 0u : 0xffffffffu << (shift + 8);
+        rc = pass(shift, mask, 0);
+        if (rc) return rc;
+        for (int i = 0; i < images; ++i) {
+            long long before = 0;
+            int b = 255;
+            for (; b > 0; --b) {
+                const long long c = (long long) h[(size_t) i * 256 + b];
+                if (before + c > left[i]) break;
+                before += c;
+            }
+            left[i] -= before;
+            prefix[i] |= (unsigned) b << shift;
+        }
     }
-    size_t tb = tmp_bytes;
-    if (e == hipSuccess) e = hipcub::DeviceRadixSort::SortKeysDescending(tmp, tb, large, large_sorted, total, 0, 32, st);
-    unsigned bits = 0;
-    if (e == hipSuccess) e = hipMemcpyAsync(&bits, large_sorted + rank, 4, hipMemcpyDeviceToHost, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void) hipFree(keys); (void) hipFree(sorted); (void) hipFree(large); (void) hipFree(large_sorted); (void) hipFree(tmp);
-    if (e != hipSuccess) return set_error(ONHIP_ERR_RUNTIME, "calib percentile: %s", hipGetErrorString(e));
-    memcpy(threshold, &bits, 4);
+    // image i keeps every key above T_i = prefix[i] and left[i] + 1 copies of T_i; an image whose slice would run past the
+    // list is not copied (model_quant.hpp:150-160 as restated by the oracle) and the list's untouched tail stays zero
+    std::vector<unsigned> thr = prefix;
+    long long zeros = total;
+    for (int i = 0; i < images; ++i) {
+        skip[i] = ((long long) i * keep + keep <= total) ? 0u : 1u;
+        if (!skip[i]) zeros -= keep;
+    }
+    ONHIP_CHECK_HIP(hipMemcpyAsync(d_thr, thr.data(), (size_t) images * 4, hipMemcpyHostToDevice, st));
+    ONHIP_CHECK_HIP(hipMemcpyAsync(d_skip, skip.data(), (size_t) images * 4, hipMemcpyHostToDevice, st));
+    std::fill(prefix.begin(), prefix.end(), 0u);
+    long long want = rank;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        const unsigned mask = shift == 24 ? 0u : 0xffffffffu << (shift + 8);
+        rc = pass(shift, mask, 1);
+        if (rc) return rc;
+        for (int i = 0; i < images; ++i)
+            if (!skip[i] && (thr[i] & mask) == prefix[0]) h[(thr[i] >> shift) & 255u] += (unsigned long long) (left[i] + 1);
+        if (prefix[0] == 0u) h[0] += (unsigned long long) zeros;
+        long long before = 0;
+        int b = 255;
+        for (; b > 0; --b) {
+            const long long c = (long long) h[b];
+            if (before + c > want) break;
+            before += c;
+        }
+        want -= before;
+        prefix[0] |= (unsigned) b << shift;
+    }
+    memcpy(threshold, &prefix[0], 4);
     return ONHIP_OK;
 }
 

@@ -35,7 +35,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
            "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quantize_nhwc_s8",
            "onhip_conv2d_w8a8_nhwc", "onhip_quant_weight_bias",
-           "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
+           "onhip_calib_workspace_bytes", "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
@@ -81,10 +81,12 @@ def load():
     L.onhip_softmax_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp]
     L.onhip_transpose_f32.argtypes = [vp, vp, vp, vp]
     L.onhip_quant_weight_bias.argtypes = [vp, vp, C.c_int32, C.c_int32, vp, vp, vp]
-    L.onhip_calib_abs_max.argtypes = [vp, C.c_longlong, C.POINTER(C.c_float), vp]
-    L.onhip_calib_histogram.argtypes = [vp, C.c_longlong, C.c_float, vp, vp]
+    L.onhip_calib_workspace_bytes.argtypes = [C.c_int]
+    L.onhip_calib_workspace_bytes.restype = C.c_size_t
+    L.onhip_calib_abs_max.argtypes = [vp, C.c_longlong, C.POINTER(C.c_float), vp, C.c_size_t, vp]
+    L.onhip_calib_histogram.argtypes = [vp, C.c_longlong, C.c_float, vp, vp, C.c_size_t, vp]
     L.onhip_calib_threshold.argtypes = [C.c_int, vp, C.c_longlong, C.c_float, C.POINTER(C.c_float)]
-    L.onhip_calib_percentile.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), vp]
+    L.onhip_calib_percentile.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), vp, C.c_size_t, vp]
     L.onhip_quantize_nhwc_s8.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float, vp, vp]
     L.onhip_conv2d_w8a8_nhwc.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
@@ -282,9 +284,25 @@ def quant_weight_bias(w, bias=None):
     return w8, b32, aux
 
 
+_calib_ws = None
+
+
+def calib_workspace(images=1):
+    """device workspace of the calibration passes: allocated by the caller (here: once per process, grown on demand)"""
+    import torch
+    global _calib_ws
+    L = load()
+    need = int(L.onhip_calib_workspace_bytes(int(images)))
+    if _calib_ws is None or _calib_ws.numel() < need:
+        _calib_ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    return _calib_ws
+
+
 def calib_abs_max(x, running=0.0):
     m = C.c_float(running)
-    _check(load().onhip_calib_abs_max(_ptr(x), x.numel(), C.byref(m), _stream()), "onhip_calib_abs_max")
+    ws = calib_workspace()
+    _check(load().onhip_calib_abs_max(_ptr(x), x.numel(), C.byref(m), _ptr(ws), ws.numel(), _stream()),
+           "onhip_calib_abs_max")
     return m.value
 
 
@@ -293,8 +311,9 @@ def calib_histogram(x, max_abs, hist=None):
     import numpy as np
     if hist is None:
         hist = np.zeros(CALIB_BINS, np.float32)
-    _check(load().onhip_calib_histogram(_ptr(x), x.numel(), max_abs, hist.ctypes.data, _stream()),
-           "onhip_calib_histogram")
+    ws = calib_workspace()
+    _check(load().onhip_calib_histogram(_ptr(x), x.numel(), max_abs, hist.ctypes.data, _ptr(ws),
+                                        C.c_size_t(ws.numel()), _stream()), "onhip_calib_histogram")
     return hist
 
 
@@ -307,7 +326,9 @@ def calib_threshold(method, hist, elem_count, max_abs):
 
 def calib_percentile(x, images, elems):
     t = C.c_float(0.0)
-    _check(load().onhip_calib_percentile(_ptr(x), images, elems, C.byref(t), _stream()), "onhip_calib_percentile")
+    ws = calib_workspace(images)
+    _check(load().onhip_calib_percentile(_ptr(x), int(images), int(elems), C.byref(t), _ptr(ws), ws.numel(), _stream()),
+           "onhip_calib_percentile")
     return t.value
 
 

@@ -861,11 +861,31 @@ def test_calibration_passes_match_oracle(torch_dev, oracle):
     assert all(np.array_equal(g, r) for g, r in zip(got, ref))
 
 
-def test_calibration_percentile_matches_oracle(torch_dev, oracle):
+@pytest.mark.parametrize("images,elems,step", [(3, 400000, 0.0), (1, 100000, 0.0), (5, 70001, 0.0), (7, 50000, 0.125),
+                                               (4, 250000, 0.5), (2, 1000000, 0.03125), (16, 50001, 0.25)])
+def test_calibration_percentile_matches_oracle(images, elems, step, torch_dev, oracle):
+    """the radix selection against the oracle's sort, also on data with many equal magnitudes (values rounded to a
+    step, so the kept set of an image ends inside a run of ties) and with zeros"""
     torch = torch_dev
-    images, elems = 3, 400000
-    x = _calib_tensor(cases.datagen.seed_for("calib_gpu", "pct"), images * elems)
+    x = _calib_tensor(cases.datagen.seed_for("calib_gpu", "pct", images, elems), images * elems)
+    if step:
+        x = (np.round(x / np.float32(step)) * np.float32(step)).astype(np.float32)
     assert hip.calib_percentile(dev(torch, x), images, elems) == oracle.calib_percentile(x, images, elems)
+
+
+def test_calibration_passes_refuse_a_missing_workspace(torch_dev):
+    import ctypes as C
+    torch = torch_dev
+    x = torch.ones(1000, device="cuda")
+    m, t = C.c_float(0.0), C.c_float(0.0)
+    L = hip.load()
+    assert L.onhip_calib_abs_max(x.data_ptr(), 1000, C.byref(m), None, 0, None) == -3
+    hist = np.zeros(2048, np.float32)
+    assert L.onhip_calib_histogram(x.data_ptr(), 1000, 1.0, hist.ctypes.data, None, 0, None) == -3
+    small = torch.empty(64, dtype=torch.uint8, device="cuda")
+    big = torch.ones(4 * 300000, device="cuda")
+    assert L.onhip_calib_percentile(big.data_ptr(), 4, 300000, C.byref(t), small.data_ptr(), 64, None) == -3
+    assert b"onhip_calib_workspace_bytes" in L.onhip_last_error()
 
 
 def _same_bits(a, b):
