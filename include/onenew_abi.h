@@ -168,6 +168,33 @@ typedef struct {
     BASE_CONFIG_S op_base_cfg;
 } RELU_CONFIG_S;
 
+/* The activation nodes the offline optimiser folds into the Conv in front of them (tools/optimize/op_fusion.hpp:75-192):
+ * common/nn_common.h:208-213 (Clip), :340-351 (HardSigmoid, LeakyRelu), :381-384 (Mul), :524-527 (Sigmoid). */
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    float min;
+    float max;
+} CLIP_CONFIG_S;
+
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    float alpha;
+    float beta;
+} HARD_SIGMOID_CONFIG_S;
+
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+    float alpha;
+} LEAKYRELU_CONFIG_S;
+
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+} MUL_CONFIG_S;
+
+typedef struct {
+    BASE_CONFIG_S op_base_cfg;
+} SIGMOID_CONFIG_S;
+
 /* common/nn_common.h:371-379 */
 typedef struct {
     BASE_CONFIG_S op_base_cfg;
@@ -294,6 +321,10 @@ ONENEW_SA(sizeof(LAYERNORMALIZATION_CONFIG_S) == 12880 && offsetof(LAYERNORMALIZ
 ONENEW_SA(sizeof(SOFTMAX_CONFIG_S) == 12856 && offsetof(SOFTMAX_CONFIG_S, axis) == 12848, "SOFTMAX_CONFIG_S");
 ONENEW_SA(sizeof(TRANSPOSE_CONFIG_S) == 12912 && offsetof(TRANSPOSE_CONFIG_S, perm_num) == 12904, "TRANSPOSE_CONFIG_S");
 ONENEW_SA(sizeof(USEFUL_INFO_S) == 96, "USEFUL_INFO_S");
+ONENEW_SA(sizeof(CLIP_CONFIG_S) == 12848 && offsetof(CLIP_CONFIG_S, min) == sizeof(BASE_CONFIG_S), "CLIP_CONFIG_S");
+ONENEW_SA(sizeof(HARD_SIGMOID_CONFIG_S) == 12848 && offsetof(HARD_SIGMOID_CONFIG_S, alpha) == sizeof(BASE_CONFIG_S), "HARD_SIGMOID_CONFIG_S");
+ONENEW_SA(sizeof(LEAKYRELU_CONFIG_S) == 12848 && offsetof(LEAKYRELU_CONFIG_S, alpha) == 12840, "LEAKYRELU_CONFIG_S");
+ONENEW_SA(sizeof(MUL_CONFIG_S) == sizeof(BASE_CONFIG_S) && sizeof(SIGMOID_CONFIG_S) == sizeof(BASE_CONFIG_S), "MUL / SIGMOID CONFIG");
 ONENEW_SA(offsetof(USEFUL_INFO_S, block_info) == 4, "USEFUL.block_info");
 ONENEW_SA(offsetof(USEFUL_INFO_S, public_buf_info) == 40, "USEFUL.public_buf_info");
 ONENEW_SA(offsetof(USEFUL_INFO_S, kv_cache_info) == 56, "USEFUL.kv_cache_info");

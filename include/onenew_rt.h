@@ -9,7 +9,8 @@
  * net's inputs are copied in and its outputs copied out.
  *
  * Operators: Conv, MatMul, Gemm, Add, Relu, MaxPool, GlobalAveragePool, Gelu, LayerNormalization, Softmax,
- * Transpose through `lib<Op>_hip.so`; Flatten and Reshape as views (no buffer, no call: host/op.h:149-154).
+ * Transpose through `lib<Op>_hip.so`; Flatten and Reshape as views (no buffer, no call: host/op.h:149-154); Clip,
+ * LeakyRelu, Sigmoid x Mul and HardSigmoid x Mul only as the activation of the Conv in front of them.
  * A model with any other node type is refused at load time.
  *
  * All functions return 0 on success or a negative ONRT_ERR_* code; onrt_last_error() describes the failure.
@@ -82,6 +83,17 @@ int onrt_net_io_info(const onrt_net_t *net, int32_t is_output, int32_t idx, cons
  * has none left).  n_blocks / n_relus (either may be NULL): how many residual blocks / Relu nodes were folded.
  */
 int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int32_t *n_relus);
+
+/*
+ * The other activations the offline optimiser folds into a Conv are folded the same way at load time: Conv -> Clip
+ * (act_type CLIP with the node's min / max, tools/optimize/op_fusion.hpp:75-103), Conv -> LeakyRelu (:105-132), Conv ->
+ * Sigmoid and Mul of the two (SILU, evaluated through the 8192-entry table like any fused SiLU, :134-160), Conv ->
+ * HardSigmoid and Mul (HARDSILU with the node's alpha / beta, :162-192); patterns as in :485-539, for a Conv with a bias
+ * and no activation yet.  This runtime has no operators of these five types: they are folded whatever ONENEW_RT_FUSE
+ * says, and a model in which one of them does not follow such a Conv is refused at load time.  n: how many Conv nodes
+ * took an activation this way.
+ */
+int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n);
 
 /*
  * One inference as a HIP graph, on request: with ONENEW_RT_GRAPH=1 in the environment at load time.  The operators

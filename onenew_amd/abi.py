@@ -91,6 +91,21 @@ class PLAIN_CONFIG_S(C.Structure):
     _fields_ = [("op_base_cfg", BASE_CONFIG_S)]
 
 
+class CLIP_CONFIG_S(C.Structure):
+    """common/nn_common.h:208-213"""
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("min", C.c_float), ("max", C.c_float)]
+
+
+class HARD_SIGMOID_CONFIG_S(C.Structure):
+    """common/nn_common.h:340-345"""
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("alpha", C.c_float), ("beta", C.c_float)]
+
+
+class LEAKYRELU_CONFIG_S(C.Structure):
+    """common/nn_common.h:347-351"""
+    _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("alpha", C.c_float)]
+
+
 class MAX_POOL_CONFIG_S(C.Structure):
     _fields_ = [("op_base_cfg", BASE_CONFIG_S), ("ceil_mode", C.c_int64), ("kernel_shape", C.c_int64 * 2),
                 ("pads", C.c_int64 * 4), ("strides", C.c_int64 * 2)]

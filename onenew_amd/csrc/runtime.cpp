@@ -82,6 +82,7 @@ struct OpKind {
     const char *type;
     size_t cfg_size;
     bool view;   // no buffer of its own, no plugin call
+    bool fold_only = false;   // runs only as part of the Conv in front of it (fold_activations_into_conv), no plugin of its own
 };
 const OpKind kOps[] = {
     {"Conv", sizeof(CONV_CONFIG_S), false},
@@ -97,6 +98,12 @@ const OpKind kOps[] = {
     {"Transpose", sizeof(TRANSPOSE_CONFIG_S), false},
     {"Flatten", sizeof(FLATTEN_CONFIG_S), true},
     {"Reshape", sizeof(RESHAPE_CONFIG_S), true},
+    // what the offline optimiser folds into a Conv (tools/optimize/op_fusion.hpp:75-192), for files that have not been through it
+    {"Clip", sizeof(CLIP_CONFIG_S), false, true},
+    {"LeakyRelu", sizeof(LEAKYRELU_CONFIG_S), false, true},
+    {"Sigmoid", sizeof(SIGMOID_CONFIG_S), false, true},
+    {"HardSigmoid", sizeof(HARD_SIGMOID_CONFIG_S), false, true},
+    {"Mul", sizeof(MUL_CONFIG_S), false, true},
 };
 const OpKind *find_kind(const char *type) {
     for (const OpKind &k : kOps)
@@ -154,7 +161,7 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    int fused_blocks = 0, folded_relus = 0;
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -485,7 +492,7 @@ std::string own_directory() {
 
 int bind_plugins(onrt_net &net) {
     for (Node &nd : net.nodes) {
-        if (nd.kind->view) continue;
+        if (nd.kind->view || nd.kind->fold_only) continue;
         const std::string type(nd.kind->type);
         auto it = net.handles.find(type);
         if (it == net.handles.end()) {
@@ -541,25 +548,93 @@ int sole_reader(const onrt_net &net, const std::string &name, const char *type) 
     return found;
 }
 
-int fold_relu_into_conv(onrt_net &net) {
-    if (!fusing_enabled()) return ONRT_OK;
+// every node that reads `name`, in execution order
+std::vector<int> readers_of(const onrt_net &net, const std::string &name) {
+    std::vector<int> out;
+    for (int idx : net.order)
+        for (const std::string &in : net.nodes[idx].in)
+            if (in == name) out.push_back(idx);
+    return out;
+}
+
+// The activation after a Conv becomes the Conv's act_type, as the offline optimiser does it (tools/optimize/
+// op_fusion.hpp: Relu :47-73, Clip :75-103, LeakyRelu :105-132, Sigmoid x Mul = SiLU :134-160, HardSigmoid x Mul
+// :162-192; sub-graph patterns :485-539), so a file that has not been through the optimiser runs like one that has.
+// Only for a Conv with a bias and no activation yet: a Conv without bias returns before the activation in the
+// reference's kernel (device/x86/Conv/conv.c:18-27).  The Relu fold obeys ONENEW_RT_FUSE (this package has a Relu
+// operator to run instead); the other node types exist here only folded, so they are folded whatever the switch
+// says, and one that no Conv takes is refused.
+int fold_activations_into_conv(onrt_net &net) {
     std::vector<bool> dropped(net.nodes.size(), false);
+    auto unary = [&](int ni) { return net.nodes[ni].in.size() == 1 && net.nodes[ni].out.size() == 1; };
     for (int idx : net.order) {
         Node &conv = net.nodes[idx];
         if (strcmp(conv.kind->type, "Conv") || conv.out.size() != 1) continue;
         CONV_CONFIG_S *cfg = reinterpret_cast<CONV_CONFIG_S *>(conv.cfg.data());
         if (!cfg->has_bias || cfg->act_type != NOT_ACT) continue;
-        const int ri = sole_reader(net, conv.out[0], "Relu");
-        if (ri < 0 || net.nodes[ri].in.size() != 1 || net.nodes[ri].out.size() != 1) continue;
-        cfg->act_type = RELU;
-        conv.fused_out = net.nodes[ri].out[0];
-        net.tensors[conv.out[0]].alias = conv.fused_out;
-        dropped[ri] = true;
-        ++net.folded_relus;
+        const std::string &mid = conv.out[0];
+        if (is_net_output(net, mid)) continue;
+        const std::vector<int> rd = readers_of(net, mid);
+        std::string result;
+        if (rd.size() == 1 && unary(rd[0])) {
+            Node &act = net.nodes[rd[0]];
+            const char *t = act.kind->type;
+            if (!strcmp(t, "Relu")) {
+                if (!fusing_enabled()) continue;
+                cfg->act_type = RELU;
+                ++net.folded_relus;
+            } else if (!strcmp(t, "Clip")) {
+                const CLIP_CONFIG_S *c = reinterpret_cast<const CLIP_CONFIG_S *>(act.cfg.data());
+                cfg->act_type = CLIP;
+                cfg->clip_min = c->min;
+                cfg->clip_max = c->max;
+                ++net.folded_acts;
+            } else if (!strcmp(t, "LeakyRelu")) {
+                cfg->act_type = LEAKYRELU;
+                cfg->leaky_relu_alpha = reinterpret_cast<const LEAKYRELU_CONFIG_S *>(act.cfg.data())->alpha;
+                ++net.folded_acts;
+            } else {
+                continue;
+            }
+            result = act.out[0];
+            dropped[rd[0]] = true;
+        } else if (rd.size() == 2 && rd[0] != rd[1]) {
+            // x -> gate(x), then x * gate(x): the gate reads the convolution alone, the Mul reads the convolution and the gate
+            int gi = rd[0], mi = rd[1];
+            if (!strcmp(net.nodes[gi].kind->type, "Mul")) std::swap(gi, mi);
+            Node &gate = net.nodes[gi], &mul = net.nodes[mi];
+            const bool sig = !strcmp(gate.kind->type, "Sigmoid"), hard = !strcmp(gate.kind->type, "HardSigmoid");
+            if ((!sig && !hard) || strcmp(mul.kind->type, "Mul") || !unary(gi) || mul.in.size() != 2 || mul.out.size() != 1) continue;
+            const std::string &g = gate.out[0];
+            if (!((mul.in[0] == mid && mul.in[1] == g) || (mul.in[1] == mid && mul.in[0] == g))) continue;
+            if (is_net_output(net, g) || readers_of(net, g).size() != 1) continue;
+            if (sig) {
+                cfg->act_type = SILU;
+            } else {
+                const HARD_SIGMOID_CONFIG_S *c = reinterpret_cast<const HARD_SIGMOID_CONFIG_S *>(gate.cfg.data());
+                cfg->act_type = HARDSILU;
+                cfg->hard_sigmoid_alpha = c->alpha;
+                cfg->hard_sigmoid_beta = c->beta;
+            }
+            ++net.folded_acts;
+            result = mul.out[0];
+            net.tensors[g].alias = result;
+            dropped[gi] = dropped[mi] = true;
+        } else {
+            continue;
+        }
+        conv.fused_out = result;
+        net.tensors[mid].alias = result;
     }
     std::vector<int> order;
-    for (int idx : net.order)
-        if (!dropped[idx]) order.push_back(idx);
+    for (int idx : net.order) {
+        if (dropped[idx]) continue;
+        const Node &nd = net.nodes[idx];
+        if (nd.kind->fold_only)
+            return fail(ONRT_ERR_FORMAT, "%s %s does not follow a Conv (with bias, without activation) it can be folded into, and this "
+                        "runtime has no %s operator of its own", nd.kind->type, nd.base()->op_name, nd.kind->type);
+        order.push_back(idx);
+    }
     net.order.swap(order);
     return ONRT_OK;
 }
@@ -659,7 +734,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
     if (!rc) rc = bind_plugins(net);
-    if (!rc) rc = fold_relu_into_conv(net);
+    if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = allocate(net);
     if (!rc) rc = build_tables(net);
@@ -682,7 +757,7 @@ int plan(onrt_net &net) {
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
     net.conv_add = net.conv_add_relu = plan_stub_eval;   // as with the Conv plugin of this package
-    if (!rc) rc = fold_relu_into_conv(net);
+    if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     return rc;
 }
@@ -864,6 +939,12 @@ static void forget_graph(onrt_net &net) {
     net.graph = nullptr;
     net.graph_launches = 0;
     net.runs = 0;
+}
+
+ONRT_API int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "folded activations: null argument");
+    *n = (int32_t) net->folded_acts;
+    return ONRT_OK;
 }
 
 ONRT_API int onrt_net_get_tiles(const onrt_net_t *net, int32_t tiles[3]) {

@@ -23,6 +23,9 @@ CFG_TYPES = {
     "MaxPool": abi.MAX_POOL_CONFIG_S, "LayerNormalization": abi.LAYERNORMALIZATION_CONFIG_S,
     "Softmax": abi.SOFTMAX_CONFIG_S, "Transpose": abi.TRANSPOSE_CONFIG_S, "Flatten": abi.FLATTEN_CONFIG_S,
     "Reshape": abi.RESHAPE_CONFIG_S,
+    # activation nodes of a file that has not been through the offline optimiser (tools/optimize/op_fusion.hpp:75-192)
+    "Clip": abi.CLIP_CONFIG_S, "LeakyRelu": abi.LEAKYRELU_CONFIG_S, "HardSigmoid": abi.HARD_SIGMOID_CONFIG_S,
+    "Sigmoid": abi.PLAIN_CONFIG_S, "Mul": abi.PLAIN_CONFIG_S,
 }
 # ONNX element type numbers (common/nn_common.h:92-110)
 DTYPES = {abi.TYPE_FP32: np.float32, abi.TYPE_INT8: np.int8, abi.TYPE_INT32: np.int32, 7: np.int64}
@@ -89,7 +92,8 @@ class OneModel:
         return outs[0]
 
     # ---- operators -------------------------------------------------------------------------------------
-    def conv(self, name, x, weight, bias, out, stride=1, pad=0, group=1, act=abi.NOT_ACT, clip=(0.0, 0.0), quant=None):
+    def conv(self, name, x, weight, bias, out, stride=1, pad=0, group=1, act=abi.NOT_ACT, clip=(0.0, 0.0), quant=None, leaky=0.0,
+             hard=(0.0, 0.0)):
         """weight [cout, cin/group, kh, kw] fp32 and bias [cout] (or None) become initialisers name.weight / name.bias.
         quant=(weight_aux [cout], input_scale) marks the W8A32 form the offline quantiser writes
         (tools/optimize/model_quant.hpp:14-25, :655-670): weight is then int8 and bias int32, both stored at the
@@ -113,7 +117,7 @@ class OneModel:
             ins.append(self.init(name + ".bias", b))
         return self.node("Conv", name, ins, [out], has_bias=int(b is not None), dilations=(1, 1), group=group,
                          kernel_shape=w.shape[2:], pads=pads, strides=strides, act_type=act, clip_min=clip[0],
-                         clip_max=clip[1], **fields)
+                         clip_max=clip[1], leaky_relu_alpha=leaky, hard_sigmoid_alpha=hard[0], hard_sigmoid_beta=hard[1], **fields)
 
     def gemm(self, name, x, weight, bias, out):
         """out = x @ weight[N, K]^T + bias (device/x86/Gemm/gemm.c)"""
@@ -135,6 +139,21 @@ class OneModel:
 
     def relu(self, name, x, out):
         return self.node("Relu", name, [x], [out])
+
+    def clip(self, name, x, out, lo, hi):
+        return self.node("Clip", name, [x], [out], min=lo, max=hi)
+
+    def leaky_relu(self, name, x, out, alpha):
+        return self.node("LeakyRelu", name, [x], [out], alpha=alpha)
+
+    def sigmoid(self, name, x, out):
+        return self.node("Sigmoid", name, [x], [out])
+
+    def hard_sigmoid(self, name, x, out, alpha, beta):
+        return self.node("HardSigmoid", name, [x], [out], alpha=alpha, beta=beta)
+
+    def mul(self, name, a, b, out):
+        return self.node("Mul", name, [a, b], [out])
 
     def gelu(self, name, x, out):
         return self.node("Gelu", name, [x], [out])

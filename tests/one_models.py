@@ -99,3 +99,37 @@ def quantised_block():
 
 
 MODELS = {"quantised_block": quantised_block, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
+
+
+def unfused_activations(optimised=False):
+    """A file as the converter leaves it, before tools/optimize: every activation a node of its own after its Conv
+    (Clip, LeakyRelu, Sigmoid and Mul, HardSigmoid and Mul, Relu).  optimised=True: the same model as the optimiser
+    writes it, the activations in the convolutions' act_type (tools/optimize/op_fusion.hpp:47-192)."""
+    m = onefile.OneModel()
+    m.input("x", (2, 8, 12, 12))
+
+    def cv(name, x, cin, cout, k, act, out, **kw):
+        w, b = _r(name + "w", (cout, cin, k, k), 0.25), _r(name + "b", (cout,), 0.2)
+        if optimised:
+            return m.conv(name, x, w, b, out, pad=k // 2, act=act, **kw)
+        return m.conv(name, x, w, b, name + "_raw", pad=k // 2)
+
+    cv("c1", "x", 8, 16, 3, abi.CLIP, "a1", clip=(0.0, 6.0))
+    if not optimised:
+        m.clip("clip", "c1_raw", "a1", 0.0, 6.0)
+    cv("c2", "a1", 16, 16, 1, abi.LEAKYRELU, "a2", leaky=0.1)
+    if not optimised:
+        m.leaky_relu("leaky", "c2_raw", "a2", 0.1)
+    cv("c3", "a2", 16, 16, 3, abi.SILU, "a3")
+    if not optimised:
+        m.sigmoid("sig", "c3_raw", "c3_gate")
+        m.mul("silu_mul", "c3_raw", "c3_gate", "a3")
+    cv("c4", "a3", 16, 12, 3, abi.HARDSILU, "a4", hard=(0.2, 0.5))
+    if not optimised:
+        m.hard_sigmoid("hsig", "c4_raw", "c4_gate", 0.2, 0.5)
+        m.mul("hsilu_mul", "c4_gate", "c4_raw", "a4")          # operands the other way round
+    cv("c5", "a4", 12, 12, 1, abi.RELU, "out")
+    if not optimised:
+        m.relu("relu", "c5_raw", "out")
+    m.output("out", (2, 12, 12, 12))
+    return m.tobytes(), [_r("xu", (2, 8, 12, 12))]

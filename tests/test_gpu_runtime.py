@@ -512,3 +512,23 @@ def test_tile_tuner_writes_the_header_and_the_runtime_reads_it_back(torch_dev):
     (after,) = net.run(x)
     assert best_ms <= default_ms and _close(after, before, 1e-3)
     assert set(np.argsort(after[0])[-5:]) == set(np.argsort(before[0])[-5:])
+
+
+def test_unoptimised_file_runs_like_the_optimised_one(torch_dev, monkeypatch):
+    """a file with Clip / LeakyRelu / Sigmoid x Mul / HardSigmoid x Mul / Relu nodes after its convolutions, loaded as
+    it is: the same bits as the file the offline optimiser would have made of it, which in turn matches the oracle;
+    also with ONENEW_RT_FUSE=0, which cannot leave these nodes unfolded"""
+    raw, ins = one_models.unfused_activations()
+    opt, _ = one_models.unfused_activations(optimised=True)
+    want = rt.Net(opt).run(*ins)
+    ref = one_model.run(opt, ins)
+    assert _close(want[0], ref[0], 5e-4)
+    net = rt.Net(raw)
+    assert net.folded_activations() == 4 and [t for t, _ in net.ops()] == ["Conv"] * 5
+    got = net.run(*ins)
+    assert np.array_equal(got[0], want[0])
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    unfused = rt.Net(raw)                       # the Relu stays a node of its own here, the other four are folded
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    assert unfused.folded_activations() == 4 and [t for t, _ in unfused.ops()] == ["Conv"] * 5 + ["Relu"]
+    assert np.array_equal(unfused.run(*ins)[0], want[0])

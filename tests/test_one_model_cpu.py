@@ -278,3 +278,54 @@ def test_header_tiles_are_written_and_read_back():
     assert plan.tiles() == (128, 128, 16)
     with pytest.raises(rt.OnrtError):
         rt.with_tiles(b"\0" * 4096, (64, 64, 16))
+
+
+def test_plan_folds_the_optimisers_activation_patterns():
+    """Conv -> Clip / LeakyRelu / Sigmoid x Mul / HardSigmoid x Mul / Relu of a file that has not been through the
+    offline optimiser: the plan runs five Conv calls and nothing else, exactly as for the optimised file, with the
+    activation parameters in the convolutions' configuration (tools/optimize/op_fusion.hpp:47-192)"""
+    raw, _ = one_models.unfused_activations()
+    opt, _ = one_models.unfused_activations(optimised=True)
+    p_raw, p_opt = rt.Net(raw, plan_only=True), rt.Net(opt, plan_only=True)
+    assert [t for t, _ in p_raw.ops()] == ["Conv"] * 5 == [t for t, _ in p_opt.ops()]
+    assert p_raw.folded_activations() == 4 and p_raw.folded_relus() == 1
+    assert p_opt.folded_activations() == 0 and p_opt.folded_relus() == 0
+    # the folded-away operands read as the activation's result
+    for name in ("c1_raw", "c3_raw", "c3_gate", "c4_gate"):
+        assert p_raw.operand(name)[0] == p_raw.operand({"c1_raw": "a1", "c3_raw": "a3", "c3_gate": "a3", "c4_gate": "a4"}[name])[0]
+    assert p_raw.operand("out")[0] == (2, 12, 12, 12)
+
+
+def test_plan_refuses_an_activation_node_no_conv_takes():
+    """a Clip after a MaxPool, a Sigmoid whose Mul partner is missing, a Clip after a Conv without bias: refused"""
+    def base():
+        m = onefile.OneModel()
+        m.input("x", (1, 4, 8, 8))
+        return m
+    w, b = np.ones((4, 4, 1, 1), np.float32), np.zeros(4, np.float32)
+    m = base()
+    m.maxpool("pool", "x", "p", 3, 1, 1)
+    m.clip("clip", "p", "out", 0.0, 6.0)
+    m.output("out", (1, 4, 8, 8))
+    with pytest.raises(rt.OnrtError, match="Clip"):
+        rt.Net(m.tobytes(), plan_only=True)
+    m = base()
+    m.conv("c", "x", w, b, "c_out")
+    m.sigmoid("sig", "c_out", "out")
+    m.output("out", (1, 4, 8, 8))
+    with pytest.raises(rt.OnrtError, match="Sigmoid"):
+        rt.Net(m.tobytes(), plan_only=True)
+    m = base()
+    m.conv("c", "x", w, None, "c_out")
+    m.clip("clip", "c_out", "out", 0.0, 6.0)
+    m.output("out", (1, 4, 8, 8))
+    with pytest.raises(rt.OnrtError, match="Clip"):
+        rt.Net(m.tobytes(), plan_only=True)
+    # the convolution's own result is also read elsewhere: the Clip cannot be folded
+    m = base()
+    m.conv("c", "x", w, b, "c_out")
+    m.clip("clip", "c_out", "y", 0.0, 6.0)
+    m.add("sum", "y", "c_out", "out")
+    m.output("out", (1, 4, 8, 8))
+    with pytest.raises(rt.OnrtError, match="Clip"):
+        rt.Net(m.tobytes(), plan_only=True)
