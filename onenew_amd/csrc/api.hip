@@ -171,7 +171,8 @@ static const int kNumSplits = 13;
 // rowb != 0: the kernel that feeds B from global memory straight into the MFMAs (igemm_rowb.hip), tile bm x bn
 // fin != 0 (with split > 1 or tail > 1): the slices of a tile are added up by the last of them to arrive, inside the
 // launch, instead of by a finishing launch (igemm_kernel, `arrive`)
-struct Choice { int bm, bn, split, tail, rowb, fin; };
+// dma != 0: the int8 kernel that loads its operand tiles straight into LDS (igemm_dma.hip), tile bm x bn, never split
+struct Choice { int bm, bn, split, tail, rowb, fin, dma; };
 
 static std::mutex g_tune_mu;
 static int g_tune_mode = -1;   // -1: read ONHIP_TUNE on first use; 0 model only; 1 measure
@@ -207,8 +208,8 @@ static void load_tune_cache_locked() {
             key.push_back(v);
             s = end;
         }
-        Choice c = {0, 0, 1, 0, 0, 0};
-        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 3 &&
+        Choice c = {0, 0, 1, 0, 0, 0, 0};
+        if (*s == ':' && key.size() == 14 && sscanf(s + 1, "%d %d %d %d %d %d %d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin, &c.dma) >= 3 &&
             c.bm > 0 && c.bn > 0 && c.split >= 1 && c.split <= 64 && c.tail >= 0 && c.tail <= 64)
             g_tuned[key] = c;
     }
@@ -220,7 +221,7 @@ static void append_tune_cache_locked(const std::vector<long long> &key, const Ch
     FILE *f = fopen(path, "a");
     if (!f) return;
     for (long long v : key) fprintf(f, "%lld ", v);
-    fprintf(f, ": %d %d %d %d %d %d\n", c.bm, c.bn, c.split, c.tail, c.rowb, c.fin);
+    fprintf(f, ": %d %d %d %d %d %d %d\n", c.bm, c.bn, c.split, c.tail, c.rowb, c.fin, c.dma);
     fclose(f);
 }
 
@@ -295,6 +296,7 @@ static const int kNumRowbTiles = 6;
 
 // (bm, bn) is a tile this build has a kernel for
 static bool tile_exists(const Choice &c) {
+    if (c.dma) return dma_i8_tile_ok(c.bm, c.bn);
     const int (*list)[2] = c.rowb ? kRowbTiles : kTiles;
     const int n = c.rowb ? kNumRowbTiles : kNumTiles;
     for (int t = 0; t < n; ++t)
@@ -305,6 +307,10 @@ static bool tile_exists(const Choice &c) {
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
     if (!tile_exists(c)) return false;   // e.g. a line of the cache file written by another build or by hand
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
+    if (c.dma) {
+        static const bool off = getenv("ONHIP_NO_DMA") != nullptr;   // tuning hook: the register-staged kernel only
+        return !off && c.split == 1 && c.tail <= 1 && !c.rowb && !c.fin && dma_i8_ok(cfg, p);
+    }
     if (c.rowb && (c.split != 1 || !rowb_f32_ok(cfg, p))) return false;
     if (c.fin) {
         static const bool off = getenv("ONHIP_NO_FIN") != nullptr;   // tuning hook: finishing launches only
@@ -345,8 +351,29 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
 // among the splits of that tile only; measured choices (tuning mode 1) and ONHIP_TILE take precedence.
 static thread_local int tl_hint_bm = 0, tl_hint_bn = 0;
 
+// The direct-to-LDS int8 kernel where the problem allows it (measured on YOLOv8s layer shapes: about twice as fast as the
+// register-staged kernel wherever it has work for most of the CUs): the largest tile that still gives every CU a
+// workgroup and then some.  Problems with so few tiles that only a split along K reaches all CUs stay with the
+// register-staged kernel, which has one.
+static bool dma_model_choice(const IgemmLaunch &cfg, const IgemmParams &p, Choice *out) {
+    static const int order[4][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
+    for (int t = 0; t < 4; ++t) {
+        const Choice c = {order[t][0], order[t][1], 1, 0, 0, 0, 1};
+        if (!candidate_ok(cfg, p, c)) return false;
+        if (c.bm == 128 && p.M <= 64) continue;
+        const long long tiles = (long long) ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
+        if (tiles >= 320 || t == 3) {
+            if (tiles < 96 && p.k_units >= 128) return false;
+            *out = c;
+            return true;
+        }
+    }
+    return false;
+}
+
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     Choice best = {64, 64, 1, 0, 0, 0};
+    if (cfg.dtype == DT_I8 && !tl_hint_bm && dma_model_choice(cfg, p, &best)) return best;
     for (int pass = tl_hint_bm ? 0 : 1; pass < 2; ++pass) {   // pass 0: the hinted tile; pass 1: every tile
         double best_cost = 1e300;
         for (int t = 0; t < kNumTiles; ++t)
@@ -363,11 +390,20 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
 }
 
 static std::atomic<long long> g_tail_launches{0};
+static std::atomic<long long> g_dma_launches{0};
 
 // Runs the problem the way the choice says.
 static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
     int dpc = 0, left = 0;
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
+    if (c.dma) {
+        cfg.bm = c.bm; cfg.bn = c.bn; cfg.split = 1;
+        p.k_split_units = p.k_units;
+        p.partial = nullptr;
+        p.arrive = nullptr;
+        g_dma_launches.fetch_add(1, std::memory_order_relaxed);
+        return dma_i8_launch(cfg, p, st);
+    }
     auto launch = [&]() {
         const int rc = c.rowb ? rowb_f32_launch(cfg, p, st) : igemm_launch(cfg, p, st);
         if (rc && p.arrive) {   // whatever part of the launch ran may have left arrival counters above zero
@@ -423,9 +459,13 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     // the entry point that allocates nothing: the cost model's choice (never the in-launch reduction, whose uncached
     // workspace is allocated on first use; no measuring, which creates events and may grow buffers)
     if (tl_noalloc) return launch_choice(cfg, p, model_choice(cfg, p), st);
-    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB[xFIN]]]]
-        Choice c = {0, 0, 1, 0, 0, 0};
-        if (sscanf(env, "%dx%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin) >= 2) {
+    if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB[xFIN[xDMA]]]]]
+        Choice c = {0, 0, 1, 0, 0, 0, 0};
+        if (sscanf(env, "%dx%dx%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin, &c.dma) >= 2) {
+            if (c.dma && !candidate_ok(cfg, p, c)) {   // not a problem (or a tile) for that kernel: the register-staged one
+                c.dma = 0;
+                if (c.bm == 128 && c.bn == 64) c.bm = 64;
+            }
             if (c.fin && !candidate_ok(cfg, p, c)) c.fin = 0;
             if (c.rowb && !candidate_ok(cfg, p, c)) {   // not a problem for that kernel: the tiled one, same tile if it has it
                 c.rowb = 0;
@@ -509,13 +549,19 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
             }
         }
     }
+    // the int8 kernel that loads its tiles straight into LDS
+    static const int kDmaTiles[][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
+    for (int t = 0; t < 4 && !rc; ++t) {
+        const Choice c = {kDmaTiles[t][0], kDmaTiles[t][1], 1, 0, 0, 0, 1};
+        if (candidate_ok(cfg, p, c)) try_choice(c);
+    }
     (void) hipEventDestroy(e0);
     (void) hipEventDestroy(e1);
     if (rc) return rc;
     if (getenv("ONHIP_TUNE_VERBOSE"))
-        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d rowb %d fin %d (%.4f ms; model said %dx%d split %d)\n",
-                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best.rowb, best.fin, best_ms, guess.bm,
-                guess.bn, guess.split);
+        fprintf(stderr, "[onenew_hip] tuned dt=%d bl=%d M=%d N=%d K=%d batch=%d -> %dx%d split %d tail %d rowb %d fin %d dma %d (%.4f ms; model said %dx%d split %d dma %d)\n",
+                cfg.dtype, cfg.bl, p.M, p.N, p.K, cfg.batch, best.bm, best.bn, best.split, best.tail, best.rowb, best.fin, best.dma, best_ms, guess.bm,
+                guess.bn, guess.split, guess.dma);
     {
         std::lock_guard<std::mutex> lock(g_tune_mu);
         g_tuned[key] = best;
@@ -581,6 +627,8 @@ long long onhip_scratch_bytes(void) {
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     return (long long) g_scratch_bytes;
 }
+
+long long onhip_direct_lds_launches(void) { return g_dma_launches.load(std::memory_order_relaxed); }
 
 long long onhip_split_tail_launches(void) { return g_tail_launches.load(std::memory_order_relaxed); }
 

@@ -303,7 +303,7 @@ __device__ __forceinline__ unsigned out_col_offset(const IgemmParams &p, int n, 
 __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
     float t = __fmul_rn(y, inv_scale);
     t = (t < -128.0f) ? -128.0f : (t > 127.0f) ? 127.0f : t;
-    return (int) roundf(t);
+    return round_half_away_small(t);
 }
 
 // Writes the accumulators of one wavefront.  Lane (li, lh) of a 32x32 block holds column li and rows
@@ -434,60 +434,120 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
 // one pixel with a single 128-bit access instead of 16 single bytes to 16 different pixels.  A lane holds four
 // consecutive channels of a pixel (accumulator registers 4q .. 4q+3), which go to LDS as one dword.  Channels
 // between M and the pitch are written as zero.  stage: BN * (BM + 16) bytes of LDS nobody reads any more.
+// rows: when not null, LDS holding the tile's per-row constants, BM de-quantisation factors weight_aux / 127 followed by
+// the BM int32 biases as floats (rows m0 .. m0 + BM - 1), which the caller computed once per row; otherwise every lane
+// fetches and divides for its own 16 x TM rows.
 template <int EPI, int BM, int BN, int TM, int TN, bool QLUT_IN_LDS, class ACC>
 __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&acc)[TM][TN], unsigned char *stage, int m0,
-                                                   int n0, int m_wave, int n_wave, int li, int lh, int tid) {
+                                                   int n0, int m_wave, int n_wave, int li, int lh, int tid,
+                                                   const float *rows = nullptr) {
     constexpr int PITCH = BM + 16;
-    const rsrc_t raux = make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u);
-    const rsrc_t rb32 = make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u);
     const unsigned lh16 = (unsigned) lh * 16u;
-    float aux[TM][16];
-    int b32[TM][16];
+    float aux[TM][16];      // the factor weight_aux / 127 of each of the lane's rows
+    float fb32[TM][16];     // and the row's int32 bias as a float
+    if (rows) {
+        // a lane's rows come in runs of four (8 (r / 4) + 4 lh + r % 4): one 16-byte read per run and constant
 #pragma unroll
-    for (int a = 0; a < TM; ++a)
+        for (int a = 0; a < TM; ++a)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const unsigned soff = (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u;
-            aux[a][r] = buf_load_f32(raux, lh16, soff);
-            b32[a][r] = (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
-        }
-    // the quantised activation table (8 KiB) next to the staging area: byte gathers from LDS instead of memory
+            for (int q = 0; q < 4; ++q) {
+                const int ml = m_wave - m0 + a * 32 + 8 * q + 4 * lh;
+                const float4 c = *reinterpret_cast<const float4 *>(rows + ml);
+                const float4 f = *reinterpret_cast<const float4 *>(rows + BM + ml);
+                aux[a][4 * q] = c.x; aux[a][4 * q + 1] = c.y; aux[a][4 * q + 2] = c.z; aux[a][4 * q + 3] = c.w;
+                fb32[a][4 * q] = f.x; fb32[a][4 * q + 1] = f.y; fb32[a][4 * q + 2] = f.z; fb32[a][4 * q + 3] = f.w;
+            }
+    } else {
+        const rsrc_t raux = make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u);
+        const rsrc_t rb32 = make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u);
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const unsigned soff = (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u;
+                aux[a][r] = buf_load_f32(raux, lh16, soff);
+                fb32[a][r] = (float) (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
+            }
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) aux[a][r] = __fdiv_rn(aux[a][r], 127.0f);
+    }
+    // the quantised activation table (8 KiB) next to the staging area: byte gathers from LDS instead of memory, through
+    // a pointer the compiler knows to be LDS (a pointer that may be either makes every gather a flat access)
+    typedef const __attribute__((address_space(3))) signed char *lds_s8_t;
     const signed char *qtab = p.ep.qlut;
+    lds_s8_t qtab_lds = nullptr;
     if (EPI == EPI_LUT && p.ep.qlut && QLUT_IN_LDS) {
         unsigned char *ql = stage + BN * PITCH;
         const uint4 *src = reinterpret_cast<const uint4 *>(p.ep.qlut);
 #pragma unroll
         for (int i = 0; i < 8192 / 16 / THREADS; ++i) reinterpret_cast<uint4 *>(ql)[tid + i * THREADS] = src[tid + i * THREADS];
         __syncthreads();
-        qtab = reinterpret_cast<const signed char *>(ql);
+        qtab_lds = (lds_s8_t) ql;
     }
+    const bool has_bias = p.bias32 != nullptr;
+    const bool table = EPI == EPI_LUT && p.ep.qlut != nullptr;   // uniform: the table entries arrive quantised
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int ml = m_wave - m0 + a * 32 + 8 * q + 4 * lh;   // first of the lane's four channels, tile-local
+            // the lane's 4 x TN values of this row group in three sweeps (arithmetic, table reads, selection), so that
+            // the table reads of a group are all in flight together instead of each being waited for on its own
+            float x[TN][4];
+            int q8[TN][4];
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int r = 4 * q + j;
+                    float f = __fmul_rn((float) acc[a][b][r], p.in_scale);
+                    const float fbias = __fadd_rn(f, fb32[a][r]);
+                    f = has_bias ? fbias : f;
+                    x[b][j] = __fmul_rn(f, aux[a][r]);
+                }
+            if (table) {   // act_fast<EPI_LUT>'s rules with the table behind the output quantiser
+                int l[TN][4];
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        int idx = (int) __fmul_rn(__fadd_rn(x[b][j], 8.0f), 512.0f);
+                        idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
+                        if constexpr (QLUT_IN_LDS) l[b][j] = qtab_lds[idx];
+                        else l[b][j] = qtab[idx];
+                    }
+                bool beyond = false;
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        q8[b][j] = x[b][j] < -8.0f ? 0 : l[b][j];
+                        beyond |= x[b][j] >= 8.0f;
+                    }
+                // beyond the table the activation is the identity: rare enough that a wavefront usually skips this whole
+                if (__builtin_amdgcn_ballot_w64(beyond) != 0ull) {
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int hi = requant_s8(x[b][j], p.out_inv_scale);
+                            q8[b][j] = x[b][j] >= 8.0f ? hi : q8[b][j];
+                        }
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) q8[b][j] = requant_s8(act_fast<EPI>(x[b][j], p.ep), p.out_inv_scale);
+            }
 #pragma unroll
             for (int b = 0; b < TN; ++b) {
                 unsigned packed = 0;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int r = 4 * q + j;
-                    const float coeff = __fdiv_rn(aux[a][r], 127.0f);
-                    float f = __fmul_rn((float) acc[a][b][r], p.in_scale);
-                    const float fbias = __fadd_rn(f, (float) b32[a][r]);
-                    f = p.bias32 ? fbias : f;
-                    const float x = __fmul_rn(f, coeff);
-                    int q8;
-                    if (EPI == EPI_LUT && p.ep.qlut) {   // uniform: the table entry arrives quantised (act_fast<EPI_LUT>'s rules)
-                        int idx = (int) __fmul_rn(__fadd_rn(x, 8.0f), 512.0f);
-                        idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
-                        const int l = qtab[idx];
-                        const int hi = requant_s8(x, p.out_inv_scale);
-                        q8 = x < -8.0f ? 0 : x >= 8.0f ? hi : l;
-                    } else {
-                        q8 = requant_s8(act_fast<EPI>(x, p.ep), p.out_inv_scale);
-                    }
-                    const int v = (m0 + ml + j < p.M) ? q8 : 0;
+                    const int v = (m0 + ml + j < p.M) ? q8[b][j] : 0;
                     packed |= ((unsigned) v & 0xffu) << (8 * j);
                 }
                 const int nl = n_wave - n0 + b * 32 + li;

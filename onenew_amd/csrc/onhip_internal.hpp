@@ -99,11 +99,20 @@ __device__ __forceinline__ float add_res(float v, float r, int relu, unsigned el
     return relu ? (elem < body ? vb : vt) : v;
 }
 
+// (int) roundf(t), ties away from zero, for |t| <= 128.5 in three instructions: adding the largest float below one half
+// with t's sign and truncating gives the same integer for every such float (checked exhaustively on the CPU, all
+// 2.2e9 of them: a tie k + 0.5 lands within a quarter ulp below k + 1 and rounds up to it, nothing else crosses an
+// integer); roundf itself is a dozen instructions
+__device__ __forceinline__ int round_half_away_small(float t) {
+    const float half = __uint_as_float((__float_as_uint(t) & 0x80000000u) | 0x3effffffu);
+    return (int) __fadd_rn(t, half);
+}
+
 // activation quantiser of conv.c:961-973: t = x * (1/scale), clamp, roundf (ties away from zero)
 __device__ __forceinline__ int quant_s8(float x, float inv_scale) {
     float t = __fmul_rn(x, inv_scale);
     t = (t < -128.0f) ? -128.0f : (t > 127.0f) ? 127.0f : t;
-    return (int) roundf(t);
+    return round_half_away_small(t);
 }
 
 // ---- implicit-GEMM kernel family (igemm.hip) ---------------------------------------------------------
@@ -211,6 +220,11 @@ int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t strea
 // fp32 kernel for plain problems with B rows contiguous along N (igemm_rowb.hip): tiles 64x128, 128x128, 64x256
 bool rowb_f32_ok(const IgemmLaunch &cfg, const IgemmParams &p);
 int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
+// int8 kernel with operand tiles loaded from global memory straight into LDS (igemm_dma.hip): NHWC int8 activations whose
+// padded channel count is a multiple of 64, tiles 128x128, 128x64, 64x128, 64x64, no split-K
+bool dma_i8_ok(const IgemmLaunch &cfg, const IgemmParams &p);
+bool dma_i8_tile_ok(int bm, int bn);
+int dma_i8_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
 
 // ---- other kernels -------------------------------------------------------------------------------------
 int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,

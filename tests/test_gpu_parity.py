@@ -1101,6 +1101,45 @@ def test_conv_w8a8_nhwc_chain_form(name, tile, torch_dev, oracle, monkeypatch):
         assert not got[..., d.cout:].any()                                    # unsplit launches zero the channel padding
 
 
+@pytest.mark.parametrize("tile", ["128x128", "128x64", "64x128", "64x64"])
+@pytest.mark.parametrize("shape", [(2, 64, 19, 72, 3, 1, 1), (1, 128, 23, 200, 3, 2, 1), (3, 192, 9, 130, 1, 1, 0), (2, 128, 12, 64, 5, 1, 2),
+                                   (1, 256, 7, 33, 3, 1, 1), (2, 64, 16, 128, 1, 2, 0)])
+@pytest.mark.parametrize("act", [abi.SILU, abi.RELU, abi.NOT_ACT])
+def test_conv_int8_direct_to_lds_kernel_every_tile(tile, shape, act, torch_dev, oracle, monkeypatch):
+    """the int8 kernel that loads its tiles from global memory straight into LDS, every tile it has, on shapes with ragged
+    rows and columns, strides, padding, 64- and 128-byte stages (channels a multiple of 64 / of 128), one and many taps,
+    a single stage and many: int8 NHWC chain form and the fp32 / int32-accumulator form, both equal to the oracle"""
+    torch = torch_dev
+    n, cin, hw, cout, k, stride, pad = shape
+    monkeypatch.setenv("ONHIP_TILE", tile + "x1x0x0x0x1")
+    d = cases.cd(cin, cout, k, stride, pad, hw, n=n, act=act, input_scale=0.037)
+    name = f"dma_{tile}_{cin}_{cout}_{k}_{stride}"
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    lut = cases.silu_lut()
+    oh, ow = d.out_hw()
+    launches = hip.load().onhip_direct_lds_launches()
+    # fp32 NCHW out with the raw accumulators
+    acc = torch.empty((d.n, d.cout, oh, ow), dtype=torch.int32, device="cuda")
+    y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, lut), acc32=acc)
+    torch.cuda.synchronize()
+    ref, ref_acc = oracle.conv2d_w8a32(d, x, w8, b32, aux, lut, want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), ref_acc), "int32 accumulators differ"
+    assert np.array_equal(y.cpu().numpy(), ref), "de-quantised outputs differ"
+    # int8 NHWC in and out
+    dq = ConvDesc.from_buffer_copy(d)
+    dq.out_s8, dq.output_scale = 1, 0.045
+    refq = oracle.conv2d_w8a32(dq, x, w8, b32, aux, lut)
+    xq = hip.quantize_nhwc_s8(dev(torch, x), d.input_scale)
+    wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
+    out = torch.full((d.n, oh, ow, (d.cout + 15) // 16 * 16), 77, dtype=torch.int8, device="cuda")
+    hip.conv2d_w8a8_nhwc(dq, xq, wp, dev(torch, b32), dev(torch, aux), dev(torch, lut), out=out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got[..., :d.cout], np.transpose(refq, (0, 2, 3, 1)))
+    assert not got[..., d.cout:].any()
+    assert hip.load().onhip_direct_lds_launches() == launches + 2, "the forced tile did not run the direct-to-LDS kernel"
+
+
 _TUNE_CHILD = r"""
 import sys, numpy as np, torch
 sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests/golden")

@@ -348,3 +348,20 @@ def test_calibration_percentile_rank(oracle):
     kept = np.concatenate([np.sort(np.abs(x[i * elems:(i + 1) * elems]))[::-1][:keep] for i in range(images)])
     rank = int((np.float32(1) - p) * images * elems)
     assert t == np.sort(kept)[::-1][rank]
+
+
+def test_cheap_rounding_of_the_quantisers_is_roundf():
+    """the device quantisers round with (int) (t + copysign(0.49999997, t)) instead of roundf: the same integer for every
+    float the clamp lets through.  All ties k + 0.5, their float neighbours, the values around one half, and ten million
+    random floats in [-128.5, 128.5]; the exhaustive check of all 2.2e9 floats in that range was run once in C."""
+    half = np.float32(np.frombuffer(np.uint32(0x3EFFFFFF).tobytes(), np.float32)[0])
+    assert half == np.nextafter(np.float32(0.5), np.float32(0))
+    ties = (np.arange(-129, 129, dtype=np.float32) + np.float32(0.5))
+    pts = np.concatenate([ties, np.nextafter(ties, np.float32(1e9)), np.nextafter(ties, np.float32(-1e9)),
+                          np.arange(-129, 130, dtype=np.float32), np.array([0.0, -0.0, 1e-40, -1e-40, 0.49999997, -0.49999997], np.float32)])
+    u = datagen.unit(datagen.seed_for("round", "t"), 10_000_000)
+    pts = np.concatenate([pts, ((u - 0.5) * 257.0).astype(np.float32)])
+    pts = pts[np.abs(pts) <= 128.5]
+    cheap = np.trunc(pts + np.copysign(half, pts)).astype(np.int64)          # float32 addition, then truncation
+    want = (np.sign(pts) * np.floor(np.abs(pts.astype(np.float64)) + 0.5)).astype(np.int64)   # round half away from zero
+    assert np.array_equal(cheap, want)
