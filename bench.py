@@ -533,7 +533,7 @@ OTHER_CONFIGS = ["cfg1", "resnet50_b1", "mobilenetv2_b64", "mobilenetv2_b1", "vi
                  "yolov8s_int8_b16", "yolov8s_int8chain_b16", "yolov8s_int8chain_b1"]
 
 
-def run_workload(torch, hip, name, steps, warmup, layers_table=False):
+def run_workload(torch, hip, name, steps, warmup, layers_table=False, graph=True):
     """times one workload: `warmup` untimed passes (tile choices are measured there when tuning is on), `steps` timed
     passes between two device synchronisations, then every layer on its own with HIP events on the launch stream"""
     desc, dtype, layers = make_workload(torch, hip, name)
@@ -551,7 +551,37 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False):
             L.launch(hip)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / steps
+    eager_ms = wall * 1e3 / steps
+    ms_per_step, launch_mode = eager_ms, "one launch per layer from the host"
+    # The same pass recorded once into a HIP graph and replayed: where the layers are shorter than the host needs to queue
+    # one (about 7 us through this Python binding), the device otherwise idles between them.  The replayed pass is the
+    # same launches with the same tile choices (made during the warm-up); its last layer's output is compared with the
+    # eager pass before the figure is used.
+    if graph:
+        try:
+            outs = [getattr(L, "yq", None) if getattr(L, "yq", None) is not None else L.y for L in layers]
+            want = outs[-1].clone()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for L in layers:
+                    L.launch(hip)
+            for _ in range(2):
+                g.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                g.replay()
+            torch.cuda.synchronize()
+            graph_ms = (time.perf_counter() - t0) * 1e3 / steps
+            same = bool(torch.equal(outs[-1], want))
+            if same and graph_ms < eager_ms:
+                ms_per_step, launch_mode = graph_ms, "one HIP graph replay per pass (the layers' launches recorded once)"
+            elif not same:
+                print(f"[bench] {name}: graph replay differs from the eager pass; eager timing kept", file=sys.stderr)
+            del g
+        except Exception as e:   # capture refused (e.g. an allocation inside a launch): the eager figure stands
+            print(f"[bench] {name}: no graph replay ({type(e).__name__}: {e})", file=sys.stderr)
+            torch.cuda.synchronize()
 
     # Roofline of the dominant kernel.  Dense layers all run onhip::igemm_kernel (MFMA-bound); depthwise layers run
     # onhip::depthwise_*_kernel (HBM-bound).  Whichever group takes more time is reported: algorithmic work of its
@@ -589,7 +619,8 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False):
                 # the same fraction from the wall time of the timed passes (layers back to back, cold caches between them)
                 "frac_whole_step": round(step_frac, 4)}
     res = {"name": name, "desc": desc, "dtype": dtype, "unit": unit, "flops": flops, "abytes": abytes,
-           "ms_per_step": ms_per_step, "per_layer_ms": per_layer_ms, "roofline": roofline, "layers": layers,
+           "ms_per_step": ms_per_step, "eager_ms_per_step": eager_ms, "launch": launch_mode, "per_layer_ms": per_layer_ms,
+           "roofline": roofline, "layers": layers,
            "value": flops / (ms_per_step * 1e-3) / 1e12}
     if layers_table:
         print(f"{'layer':<18}{'shape':<32}{'ms':>9}{unit:>9}{'%mfma':>7}{'GB/s':>8}{'%hbm':>6}", file=sys.stderr)
@@ -606,7 +637,8 @@ def config_summary(res):
     rf = res["roofline"]
     per = res["per_layer_ms"]
     out = {"workload": res["name"], "what": res["desc"], "dtype": res["dtype"], "value": round(res["value"], 3), "unit": res["unit"],
-           "ms_per_step": round(res["ms_per_step"], 4), "ms_sum_of_layers": round(sum(per), 4), "layers": len(per),
+           "ms_per_step": round(res["ms_per_step"], 4), "launch": res["launch"], "eager_ms_per_step": round(res["eager_ms_per_step"], 4),
+           "ms_sum_of_layers": round(sum(per), 4), "layers": len(per),
            "roofline": {k: rf[k] for k in ("bound", "achieved", "peak", "unit", "frac", "frac_whole_step", "avg_launch_ms", "launches")},
            "algorithmic_GBps": round(res["abytes"] / (res["ms_per_step"] * 1e-3) / 1e9, 1),
            "hbm_frac_whole_step": round(res["abytes"] / (res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -627,6 +659,7 @@ def main():
     ap.add_argument("--no-tune", action="store_true", help="use the cost model instead of measured tile choice")
     ap.add_argument("--no-batch1", action="store_true", help="skip the extra batch-1 pass over the same stack")
     ap.add_argument("--only", action="store_true", help="time the named workload only, not the other configurations after it")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches only, no HIP graph replay of the pass")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path runs on a single MI355X and nothing in this build "
@@ -653,10 +686,11 @@ def main():
     if args.workload.startswith("resnet50_net_b") or args.workload.startswith("mobilenetv2_net_b"):
         return bench_net(torch, args)
 
-    res = run_workload(torch, hip, args.workload, args.steps, args.warmup, layers_table=args.layers)
+    res = run_workload(torch, hip, args.workload, args.steps, args.warmup, layers_table=args.layers, graph=not args.no_graph)
     layers, per_layer_ms, dtype, unit = res["layers"], res["per_layer_ms"], res["dtype"], res["unit"]
 
-    extra = {"tuning": "cost model only" if args.no_tune else
+    extra = {"launch": res["launch"], "eager_ms_per_step": round(res["eager_ms_per_step"], 4),
+             "tuning": "cost model only" if args.no_tune else
              "tile and split-K measured once per layer shape during the warm-up passes (onhip_set_tuning(1)); the library's "
              "default is the cost model"}
     if not args.no_tune and args.workload == "resnet50_b32" and not args.only:
@@ -707,7 +741,7 @@ def main():
         for name in OTHER_CONFIGS:
             torch.cuda.empty_cache()
             t0 = time.perf_counter()
-            r = run_workload(torch, hip, name, steps=10, warmup=3)
+            r = run_workload(torch, hip, name, steps=10, warmup=3, graph=not args.no_graph)
             c = config_summary(r)
             c["bench_seconds"] = round(time.perf_counter() - t0, 1)
             configs.append(c)
