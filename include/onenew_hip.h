@@ -202,6 +202,43 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
                            const int32_t *bias32, const float *weight_aux, const float *silu_lut,
                            int8_t *yq, void *stream);
 
+/* ---- bf16 / fp16 with 16-bit storage --------------------------------------------------------------------------
+ * The reference has the two types as enumerators only (ELEM_TYPE_E TYPE_FP16 / the cuda tile fields,
+ * common/nn_common.h:102,107) and no kernel that stores them, so the layouts are this library's: activations NHWC
+ * with the channel count padded to onhip_h16_pitch(c) (a multiple of 32; padding channels hold zeros), 16-byte
+ * aligned; weights [cout][kh*kw][pitch(cin)] from the pack functions; accumulation in fp32 on the matrix cores
+ * (v_mfma_f32_32x32x16_bf16 / _f16); bias, activation (the fp32 convolution's, same tables) in fp32 on the sums,
+ * then one rounding to nearest even into the output type.  d->compute (ONHIP_COMPUTE_BF16 or _F16) names the type
+ * of x, the weights, the residual operand and the 16-bit output.  Arithmetic replaced: the multiply-accumulate of
+ * device/x86/Conv/conv.c:1024-1056 (its fp32 form) and device/x86/MatMul/mat_mul.c:10-102 on rounded operands.
+ *
+ * y_kind: where the result goes.  _NHWC: 16-bit, pitch(cout) channels per pixel, the input of the next 16-bit
+ * layer; `residual`, when not NULL, is a tensor of that type and layout that is added to the rounded result in
+ * fp32 (followed by a ReLU when residual_relu != 0) and the sum rounded again: what separate Add and Relu operators
+ * (device/x86/Add/add.c, Relu/relu.c) would store on 16-bit tensors.  _F32_NHWC: fp32, cout channels per pixel, no
+ * padding (the rows of a MatMul result).  _F32_NCHW: fp32 in the reference's own layout, the way back out of a
+ * 16-bit chain. */
+enum { ONHIP_H16_OUT_NHWC = 0, ONHIP_H16_OUT_F32_NHWC = 1, ONHIP_H16_OUT_F32_NCHW = 2 };
+int32_t onhip_h16_pitch(int32_t channels);
+/* bytes of a packed weight tensor of `rows` filters (or MatMul columns) of cin channels and `taps` filter taps */
+size_t onhip_h16_packed_weight_bytes(int32_t rows, int32_t cin, int32_t taps);
+/* fp32 OIHW weights -> packed 16-bit (once per tensor) */
+int onhip_h16_pack_conv_weights(const onhip_conv_desc_t *d, const float *w, void *packed, void *stream);
+/* the right operand b [k][n] (row-major fp32) of a MatMul -> packed 16-bit [n][pitch(k)] */
+int onhip_h16_pack_matmul_weights(const float *b, int32_t k, int32_t n, int32_t compute, void *packed, void *stream);
+/* fp32 NCHW <-> 16-bit NHWC with padded channels; fp32 rows [rows][k] <-> 16-bit rows [rows][pitch(k)] */
+int onhip_h16_from_nchw_f32(const float *x, int32_t n, int32_t c, int32_t h, int32_t w, int32_t compute, void *y, void *stream);
+int onhip_h16_to_nchw_f32(const void *x, int32_t n, int32_t c, int32_t h, int32_t w, int32_t compute, float *y, void *stream);
+int onhip_h16_from_rows_f32(const float *x, long long rows, int32_t k, int32_t compute, void *y, void *stream);
+int onhip_h16_to_rows_f32(const void *x, long long rows, int32_t k, int32_t compute, float *y, void *stream);
+/* dense convolution, at most 64 filter taps, tensors below 2 GiB */
+int onhip_conv2d_h16(const onhip_conv_desc_t *d, const void *x, const void *w_packed, const float *bias, const float *lut,
+                     const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream);
+/* y[rows][n] = x[rows][k] * b[k][n] (+ bias[n]) (then the table GELU of device/x86/Gelu/gelu.c when gelu_lut is given):
+ * the MatMul -> Add -> Gelu chain of a transformer's linear layers with x, b and (for _NHWC) y in 16 bits */
+int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, const void *x, const void *w_packed,
+                     const float *bias, const float *gelu_lut, const void *residual, void *y, int32_t y_kind, void *stream);
+
 /* Batched MatMul with optional fused bias and table GELU.  Replaces mat_mul.c eval (:10) and,
  * with bias/gelu_lut, the chain MatMul -> Add -> Gelu (device/x86/Gelu/gelu.c:9). */
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

@@ -296,7 +296,7 @@ static const int kNumRowbTiles = 6;
 
 // (bm, bn) is a tile this build has a kernel for
 static bool tile_exists(const Choice &c) {
-    if (c.dma) return dma_i8_tile_ok(c.bm, c.bn);
+    if (c.dma) return dma_tile_ok(c.bm, c.bn);
     const int (*list)[2] = c.rowb ? kRowbTiles : kTiles;
     const int n = c.rowb ? kNumRowbTiles : kNumTiles;
     for (int t = 0; t < n; ++t)
@@ -307,10 +307,12 @@ static bool tile_exists(const Choice &c) {
 static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Choice &c) {
     if (!tile_exists(c)) return false;   // e.g. a line of the cache file written by another build or by hand
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
+    const bool h16 = cfg.dtype != DT_I8 && (cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP);   // 16-bit storage: that kernel only
     if (c.dma) {
         static const bool off = getenv("ONHIP_NO_DMA") != nullptr;   // tuning hook: the register-staged kernel only
-        return !off && c.split == 1 && c.tail <= 1 && !c.rowb && !c.fin && dma_i8_ok(cfg, p);
+        return (!off || h16) && c.split == 1 && c.tail <= 1 && !c.rowb && !c.fin && dma_ok(cfg, p);
     }
+    if (h16) return false;
     if (c.rowb && (c.split != 1 || !rowb_f32_ok(cfg, p))) return false;
     if (c.fin) {
         static const bool off = getenv("ONHIP_NO_FIN") != nullptr;   // tuning hook: finishing launches only
@@ -357,13 +359,14 @@ static thread_local int tl_hint_bm = 0, tl_hint_bn = 0;
 // register-staged kernel, which has one.
 static bool dma_model_choice(const IgemmLaunch &cfg, const IgemmParams &p, Choice *out) {
     static const int order[4][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
+    const bool only = cfg.dtype != DT_I8;   // the 16-bit types have no other kernel for these operands
     for (int t = 0; t < 4; ++t) {
         const Choice c = {order[t][0], order[t][1], 1, 0, 0, 0, 1};
         if (!candidate_ok(cfg, p, c)) return false;
         if (c.bm == 128 && p.M <= 64) continue;
         const long long tiles = (long long) ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
         if (tiles >= 320 || t == 3) {
-            if (tiles < 96 && p.k_units >= 128) return false;
+            if (tiles < 96 && p.k_units >= 128 && !only) return false;
             *out = c;
             return true;
         }
@@ -373,7 +376,8 @@ static bool dma_model_choice(const IgemmLaunch &cfg, const IgemmParams &p, Choic
 
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     Choice best = {64, 64, 1, 0, 0, 0};
-    if (cfg.dtype == DT_I8 && !tl_hint_bm && dma_model_choice(cfg, p, &best)) return best;
+    const bool vec = cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP;
+    if (vec && (cfg.dtype != DT_I8 || !tl_hint_bm) && dma_model_choice(cfg, p, &best)) return best;
     for (int pass = tl_hint_bm ? 0 : 1; pass < 2; ++pass) {   // pass 0: the hinted tile; pass 1: every tile
         double best_cost = 1e300;
         for (int t = 0; t < kNumTiles; ++t)
@@ -402,7 +406,7 @@ static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStr
         p.partial = nullptr;
         p.arrive = nullptr;
         g_dma_launches.fetch_add(1, std::memory_order_relaxed);
-        return dma_i8_launch(cfg, p, st);
+        return dma_launch(cfg, p, st);
     }
     auto launch = [&]() {
         const int rc = c.rowb ? rowb_f32_launch(cfg, p, st) : igemm_launch(cfg, p, st);
@@ -462,6 +466,10 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     if (const char *env = getenv("ONHIP_TILE")) {   // tuning hook: ONHIP_TILE=BMxBN[xSPLIT[xTAIL[xROWB[xFIN[xDMA]]]]]
         Choice c = {0, 0, 1, 0, 0, 0, 0};
         if (sscanf(env, "%dx%dx%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin, &c.dma) >= 2) {
+            if (cfg.dtype != DT_I8 && (cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP)) {   // 16-bit storage: one kernel, its tiles
+                c = {c.bm, c.bn, 1, 0, 0, 0, 1};
+                if (!candidate_ok(cfg, p, c)) c = model_choice(cfg, p);
+            }
             if (c.dma && !candidate_ok(cfg, p, c)) {   // not a problem (or a tile) for that kernel: the register-staged one
                 c.dma = 0;
                 if (c.bm == 128 && c.bn == 64) c.bm = 64;
@@ -1047,6 +1055,153 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     p.ep.lut = gelu_lut;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     return plan_and_launch(cfg, p, st);
+}
+
+// ---- 16-bit storage: bf16 / fp16 operands and results in memory, fp32 accumulation ---------------------------------------
+static int h16_dtype(int compute, int *dt) {
+    if (compute == ONHIP_COMPUTE_BF16) { *dt = DT_BF16; return ONHIP_OK; }
+    if (compute == ONHIP_COMPUTE_F16) { *dt = DT_F16; return ONHIP_OK; }
+    return set_error(ONHIP_ERR_ARG, "16-bit storage: compute type %d is neither bf16 nor fp16", compute);
+}
+
+int32_t onhip_h16_pitch(int32_t channels) { return channels < 1 ? 0 : (channels + 31) / 32 * 32; }
+
+size_t onhip_h16_packed_weight_bytes(int32_t rows, int32_t cin, int32_t taps) {
+    if (rows < 1 || cin < 1 || taps < 1) return 0;
+    return (size_t) rows * taps * onhip_h16_pitch(cin) * 2;
+}
+
+int onhip_h16_pack_conv_weights(const onhip_conv_desc_t *d, const float *w, void *packed, void *stream) {
+    int32_t OH, OW;
+    int dt, rc = check_conv(d, &OH, &OW);
+    if (rc) return rc;
+    if ((rc = h16_dtype(d->compute, &dt))) return rc;
+    if (d->group != 1) return set_error(ONHIP_ERR_ARG, "16-bit storage: dense convolutions only");
+    if (!w || !packed || reinterpret_cast<uintptr_t>(packed) % 16) return set_error(ONHIP_ERR_ARG, "16-bit pack: null or unaligned pointer");
+    const int taps = d->kh * d->kw;
+    return pack_w16_launch(dt, w, d->cout, d->cin, taps, onhip_h16_pitch(d->cin), (long long) d->cin * taps, taps, 1, packed,
+                           reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_h16_pack_matmul_weights(const float *b, int32_t k, int32_t n, int32_t compute, void *packed, void *stream) {
+    int dt, rc = h16_dtype(compute, &dt);
+    if (rc) return rc;
+    if (!b || !packed || k < 1 || n < 1 || reinterpret_cast<uintptr_t>(packed) % 16) return set_error(ONHIP_ERR_ARG, "16-bit pack: bad argument");
+    return pack_w16_launch(dt, b, n, k, 1, onhip_h16_pitch(k), 1, n, 0, packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_h16_from_nchw_f32(const float *x, int32_t n, int32_t c, int32_t h, int32_t w, int32_t compute, void *y, void *stream) {
+    int dt, rc = h16_dtype(compute, &dt);
+    if (rc) return rc;
+    if (!x || !y || n < 1 || c < 1 || h < 1 || w < 1 || reinterpret_cast<uintptr_t>(y) % 16) return set_error(ONHIP_ERR_ARG, "16-bit conversion: bad argument");
+    return nchw_to_nhwc16_launch(dt, x, n, c, h, w, onhip_h16_pitch(c), y, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_h16_to_nchw_f32(const void *x, int32_t n, int32_t c, int32_t h, int32_t w, int32_t compute, float *y, void *stream) {
+    int dt, rc = h16_dtype(compute, &dt);
+    if (rc) return rc;
+    if (!x || !y || n < 1 || c < 1 || h < 1 || w < 1 || reinterpret_cast<uintptr_t>(x) % 16) return set_error(ONHIP_ERR_ARG, "16-bit conversion: bad argument");
+    return nhwc16_to_nchw_launch(dt, x, n, c, h, w, onhip_h16_pitch(c), y, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_h16_from_rows_f32(const float *x, long long rows, int32_t k, int32_t compute, void *y, void *stream) {
+    int dt, rc = h16_dtype(compute, &dt);
+    if (rc) return rc;
+    if (!x || !y || rows < 1 || k < 1) return set_error(ONHIP_ERR_ARG, "16-bit conversion: bad argument");
+    return rows_to_h16_launch(dt, x, rows, k, onhip_h16_pitch(k), y, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_h16_to_rows_f32(const void *x, long long rows, int32_t k, int32_t compute, float *y, void *stream) {
+    int dt, rc = h16_dtype(compute, &dt);
+    if (rc) return rc;
+    if (!x || !y || rows < 1 || k < 1) return set_error(ONHIP_ERR_ARG, "16-bit conversion: bad argument");
+    return rows_from_h16_launch(dt, x, rows, k, onhip_h16_pitch(k), y, reinterpret_cast<hipStream_t>(stream));
+}
+
+// gelu != 0: lut is the GELU table and is applied whatever the descriptor says (the linear layer's fused form)
+static int conv2d_h16_impl(const onhip_conv_desc_t *d, const void *x, const void *w_packed, const float *bias, const float *lut,
+                           int gelu, const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream) {
+    int32_t OH, OW;
+    int rc = check_conv(d, &OH, &OW);
+    if (rc) return rc;
+    IgemmLaunch cfg;
+    memset(&cfg, 0, sizeof(cfg));
+    if ((rc = h16_dtype(d->compute, &cfg.dtype))) return rc;
+    if (d->group != 1) return set_error(ONHIP_ERR_ARG, "conv 16-bit: dense convolutions only");
+    if (!x || !w_packed || !y || (d->has_bias && !bias)) return set_error(ONHIP_ERR_ARG, "conv 16-bit: null tensor pointer");
+    if (y_kind < ONHIP_H16_OUT_NHWC || y_kind > ONHIP_H16_OUT_F32_NCHW) return set_error(ONHIP_ERR_ARG, "conv 16-bit: output kind %d", y_kind);
+    if (residual && y_kind != ONHIP_H16_OUT_NHWC) return set_error(ONHIP_ERR_ARG, "conv 16-bit: the residual operand goes with the 16-bit output");
+    if (residual == y) return set_error(ONHIP_ERR_ARG, "conv 16-bit: the residual operand may not be the output buffer");
+    if (d->act_type == SILU && !lut) return set_error(ONHIP_ERR_ARG, "conv 16-bit: SILU needs the table");
+    if (d->kh * d->kw > 64) return set_error(ONHIP_ERR_ARG, "conv 16-bit: filters of more than 64 taps are not supported");
+    if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(w_packed) % 16 || reinterpret_cast<uintptr_t>(y) % 16 ||
+        reinterpret_cast<uintptr_t>(residual) % 16)
+        return set_error(ONHIP_ERR_ARG, "conv 16-bit: tensors must be 16-byte aligned");
+    const int cp = onhip_h16_pitch(d->cin), cop = onhip_h16_pitch(d->cout);
+    if ((long long) d->n * d->h * d->w * cp * 2 >= (1LL << 31) || (long long) d->n * OH * OW * cop * 4 >= (1LL << 31) ||
+        (long long) d->cout * d->kh * d->kw * cp * 2 >= (1LL << 31))
+        return set_error(ONHIP_ERR_ARG, "conv 16-bit: tensors of 2 GiB or more are not supported");
+    cfg.bl = BL_KVEC;
+    cfg.batch = 1;
+    IgemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.units_per_tap = cp / 8;
+    p.k_units = d->kh * d->kw * p.units_per_tap;
+    p.M = d->cout;
+    p.N = d->n * OH * OW;
+    p.K = p.k_units * 8;
+    p.A = w_packed;
+    p.lda = p.k_units * 16;      // bytes, like every quantity of the vector loader
+    p.B = x;
+    p.H = d->h; p.W = d->w; p.OW = OW; p.OHW = OH * OW; p.HW = d->h * d->w;
+    p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
+    p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
+    p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
+    p.use_tapmask = 1;
+    p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
+    p.pix_stride = cp * 2;
+    p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * cp * 2;
+    p.a_slice_bytes = (long long) p.M * p.lda;
+    p.b_slice_bytes = (long long) d->n * d->h * d->w * cp * 2;
+    p.C = y;
+    if (y_kind == ONHIP_H16_OUT_F32_NCHW) {
+        p.out_mode = OUT_CONV;
+        p.c_img_stride = (long long) d->cout * OH * OW;
+        p.c_stride_m = (long long) OH * OW;
+    } else {
+        // element (pixel n, channel m) at n * pitch + m
+        p.out_mode = OUT_PLAIN;
+        p.c_stride_m = 1;
+        p.c_stride_n = y_kind == ONHIP_H16_OUT_NHWC ? cop : d->cout;
+        p.out_h16 = y_kind == ONHIP_H16_OUT_NHWC;
+    }
+    p.c_slice_bytes = (long long) d->n * OH * OW * cop * 4;
+    p.bias = d->has_bias ? bias : nullptr;
+    p.bias_mode = d->has_bias ? BIAS_M : BIAS_NONE;
+    p.ep = make_epilogue(*d, lut);
+    if (gelu) p.ep.act = ONHIP_ACT_GELU_LUT;
+    p.res16 = residual;
+    p.res_relu = residual_relu;
+    return plan_and_launch(cfg, p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_conv2d_h16(const onhip_conv_desc_t *d, const void *x, const void *w_packed, const float *bias, const float *lut,
+                     const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream) {
+    return conv2d_h16_impl(d, x, w_packed, bias, lut, 0, residual, residual_relu, y, y_kind, stream);
+}
+
+int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, const void *x, const void *w_packed, const float *bias,
+                     const float *gelu_lut, const void *residual, void *y, int32_t y_kind, void *stream) {
+    if (rows < 1 || rows >= (1LL << 31) || k < 1 || n < 1) return set_error(ONHIP_ERR_ARG, "linear 16-bit: bad shape");
+    if (y_kind == ONHIP_H16_OUT_F32_NCHW) return set_error(ONHIP_ERR_ARG, "linear 16-bit: rows come out as rows");
+    // rows of a matrix are the pixels of a one-row image with k channels, the weights a 1x1 filter bank
+    onhip_conv_desc_t d;
+    memset(&d, 0, sizeof(d));
+    d.n = 1; d.cin = k; d.h = 1; d.w = (int32_t) rows; d.cout = n; d.kh = d.kw = 1; d.stride_h = d.stride_w = 1;
+    d.group = 1; d.has_bias = bias != nullptr; d.compute = compute;
+    d.act_type = NOT_ACT;
+    // the table GELU of device/x86/Gelu/gelu.c on the fp32 sums, as in the fp32 MatMul's fused form
+    return conv2d_h16_impl(&d, x, w_packed, bias, gelu_lut, gelu_lut != nullptr, residual, 0, y, y_kind, stream);
 }
 
 int onhip_copy_f32(const float *src, float *dst, long long n, void *stream) {

@@ -569,6 +569,87 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
     }
 }
 
+// two fp32 values rounded to the 16-bit type (nearest even) and packed, low half first; and back
+template <int DT> __device__ __forceinline__ unsigned pack_h16(float lo, float hi) {
+    if constexpr (DT == DT_BF16) {
+        const bf16x2 t = {(__bf16) lo, (__bf16) hi};
+        return __builtin_bit_cast(unsigned, t);
+    } else {
+        const f16x2 t = {(_Float16) lo, (_Float16) hi};
+        return __builtin_bit_cast(unsigned, t);
+    }
+}
+template <int DT> __device__ __forceinline__ float unpack_h16(unsigned w, int half) {
+    if constexpr (DT == DT_BF16) return __uint_as_float(half ? (w & 0xffff0000u) : (w << 16));
+    else {
+        const f16x2 t = __builtin_bit_cast(f16x2, w);
+        return (float) (half ? t.y : t.x);
+    }
+}
+
+// 16-bit NHWC output (bf16 or fp16; element (pixel n, channel m) at (n * pitch + m) * 2 bytes, pitch = p.c_stride_n a
+// multiple of 8): bias and activation in fp32 on the accumulators, rounding to the 16-bit type, then the tile is
+// transposed through LDS so that a thread stores 8 consecutive channels of one pixel with a single 128-bit access.  A
+// lane holds four consecutive channels of a pixel (accumulator registers 4q .. 4q+3), which go to LDS as 8 bytes.
+// An optional residual operand (p.res16, same layout as the output) is added in fp32 to the rounded value on the way
+// out, followed by a ReLU when p.res_relu says so, and the sum is rounded again: what a separate Add (+ Relu) operator
+// on the 16-bit tensors would store.  Channels between M and the pitch are written as zero.
+// stage: BN * (2 BM + 16) bytes of LDS nobody reads any more.  rows: LDS holding the BM per-row biases of the tile
+// (zero where there is none).
+template <int DT, int EPI, int BM, int BN, int TM, int TN>
+__device__ __forceinline__ void write_tile_nhwc_h16(const IgemmParams &p, f32x16 (&acc)[TM][TN], unsigned char *stage, int m0,
+                                                    int n0, int m_wave, int n_wave, int li, int lh, int tid,
+                                                    const float *rows) {
+    static_assert(DT == DT_BF16 || DT == DT_F16, "16-bit floating-point outputs");
+    constexpr int PITCH = 2 * BM + 16;
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int ml = m_wave - m0 + a * 32 + 8 * q + 4 * lh;   // first of the lane's four channels, tile-local
+            const float4 bias = *reinterpret_cast<const float4 *>(rows + ml);
+            const float bv[4] = {bias.x, bias.y, bias.z, bias.w};
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                float y[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float v = act_fast<EPI>(__fadd_rn(acc[a][b][4 * q + j], bv[j]), p.ep);
+                    y[j] = (m0 + ml + j < p.M) ? v : 0.0f;
+                }
+                const int nl = n_wave - n0 + b * 32 + li;
+                *reinterpret_cast<uint2 *>(stage + nl * PITCH + ml * 2) = make_uint2(pack_h16<DT>(y[0], y[1]), pack_h16<DT>(y[2], y[3]));
+            }
+        }
+    __syncthreads();
+    constexpr int GROUPS = BM / 8;
+    const rsrc_t rc = make_rsrc(p.C, RSRC_RANGE);
+    const rsrc_t rr = make_rsrc(p.res16, p.res16 ? RSRC_RANGE : 0u);
+    const int pitch = (int) p.c_stride_n;
+    const bool with_res = p.res16 != nullptr, relu = p.res_relu != 0;
+#pragma unroll
+    for (int f0 = 0; f0 < BN * GROUPS; f0 += THREADS) {
+        const int f = f0 + tid;
+        const int nl = f / GROUPS, g = f % GROUPS;
+        uint4 v = *reinterpret_cast<const uint4 *>(stage + nl * PITCH + g * 16);
+        const int n = n0 + nl, m = m0 + g * 8;
+        const bool ok = ((BN * GROUPS) % THREADS == 0 || f < BN * GROUPS) && n < p.N && m < pitch;
+        const unsigned off = ok ? (unsigned) (n * pitch + m) * 2u : OOB;
+        if (with_res) {   // uniform
+            const u32x4 r = __builtin_amdgcn_raw_buffer_load_b128(rr, off, 0, 0);
+            unsigned *w = reinterpret_cast<unsigned *>(&v);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float lo = __fadd_rn(unpack_h16<DT>(w[i], 0), unpack_h16<DT>(r[i], 0));
+                float hi = __fadd_rn(unpack_h16<DT>(w[i], 1), unpack_h16<DT>(r[i], 1));
+                if (relu) { lo = lo > 0.0f ? lo : 0.0f; hi = hi > 0.0f ? hi : 0.0f; }
+                w[i] = pack_h16<DT>(lo, hi);
+            }
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{v.x, v.y, v.z, v.w}, rc, off, 0, 0);
+    }
+}
+
 __device__ __forceinline__ unsigned to_bits(float v) { return __float_as_uint(v); }
 __device__ __forceinline__ unsigned to_bits(int v) { return (unsigned) v; }
 

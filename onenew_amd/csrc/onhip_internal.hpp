@@ -196,6 +196,11 @@ struct IgemmParams {
     int32_t *acc_out;          // optional raw accumulators, same addressing as C
     int out_s8;
     float out_inv_scale;       // 1.0f / output_scale
+    // 16-bit storage (bf16 / fp16 operands read as 16-byte vectors): out_h16 != 0 stores the result in the operands'
+    // type, NHWC with a channel pitch of c_stride_n; res16, when not null, is a tensor of that type and layout added on
+    // the way out (followed by a ReLU when res_relu is set)
+    int out_h16;
+    const void *res16;
     // split-K workspace: partial sums [split][M][N] fp32 (nullptr when unsplit)
     float *partial;
     // reduction inside the launch by the last slice of a tile to arrive: one counter per tile (uncached memory, like
@@ -222,9 +227,9 @@ bool rowb_f32_ok(const IgemmLaunch &cfg, const IgemmParams &p);
 int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
 // int8 kernel with operand tiles loaded from global memory straight into LDS (igemm_dma.hip): NHWC int8 activations whose
 // padded channel count is a multiple of 64, tiles 128x128, 128x64, 64x128, 64x64, no split-K
-bool dma_i8_ok(const IgemmLaunch &cfg, const IgemmParams &p);
-bool dma_i8_tile_ok(int bm, int bn);
-int dma_i8_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
+bool dma_ok(const IgemmLaunch &cfg, const IgemmParams &p);
+bool dma_tile_ok(int bm, int bn);
+int dma_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
 
 // ---- other kernels -------------------------------------------------------------------------------------
 int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w,
@@ -237,6 +242,13 @@ int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, flo
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
 int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
 int forget_quantised_tables(const void *base, size_t bytes);   // api.hip: the cache of tables behind an output quantiser
+// 16-bit storage (h16.hip): dt is DT_BF16 or DT_F16
+int pack_w16_launch(int dt, const float *w, long long rows, int cin, int taps, int cp, long long s_row, long long s_ch,
+                    long long s_tap, void *packed, hipStream_t stream);
+int nchw_to_nhwc16_launch(int dt, const float *x, int n, int c, int h, int w, int cp, void *y, hipStream_t stream);
+int nhwc16_to_nchw_launch(int dt, const void *x, int n, int c, int h, int w, int cp, float *y, hipStream_t stream);
+int rows_to_h16_launch(int dt, const float *x, long long rows, int k, int kp, void *y, hipStream_t stream);
+int rows_from_h16_launch(int dt, const void *x, long long rows, int k, int kp, float *y, hipStream_t stream);
 int pack_w8_launch(const int8_t *w8, int cout, int cin, int kh, int kw, int cp, int k_units, int8_t *packed,
                    hipStream_t stream);
 int gemm_nt_launch(int m, int k, int n, const float *a, const float *w, const float *bias, float *out,

@@ -37,6 +37,9 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_conv2d_w8a8_nhwc", "onhip_quant_weight_bias",
            "onhip_calib_workspace_bytes", "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
+           "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
+           "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
+           "onhip_conv2d_h16", "onhip_linear_h16",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
@@ -94,6 +97,18 @@ def load():
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
     L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
     L.onhip_plugin_forget.argtypes = [vp, C.c_size_t]
+    i32 = C.c_int32
+    L.onhip_h16_pitch.argtypes = [i32]
+    L.onhip_h16_packed_weight_bytes.argtypes = [i32, i32, i32]
+    L.onhip_h16_packed_weight_bytes.restype = C.c_size_t
+    L.onhip_h16_pack_conv_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    L.onhip_h16_pack_matmul_weights.argtypes = [vp, i32, i32, i32, vp, vp]
+    L.onhip_h16_from_nchw_f32.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp]
+    L.onhip_h16_to_nchw_f32.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp]
+    L.onhip_h16_from_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
+    L.onhip_h16_to_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
+    L.onhip_conv2d_h16.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, i32, vp, i32, vp]
+    L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
     _lib = L
@@ -399,6 +414,103 @@ def matmul(a, b, bias=None, gelu_lut=None, compute=abi.COMPUTE_F32, out=None):
         out = torch.empty(tuple(a.shape[:-1]) + (N,), dtype=torch.float32, device=a.device)
     _check(load().onhip_matmul(C.byref(d), _ptr(a), _ptr(b), _ptr(bias), _ptr(gelu_lut), _ptr(out), _stream()),
            "onhip_matmul")
+    return out
+
+
+# ---- bf16 / fp16 with 16-bit storage: tensors travel as torch.bfloat16 / torch.float16, NHWC with padded channels ----
+H16_OUT_NHWC, H16_OUT_F32_NHWC, H16_OUT_F32_NCHW = 0, 1, 2
+
+
+def h16_pitch(c):
+    return (c + 31) // 32 * 32
+
+
+def _h16_torch_dtype(compute):
+    import torch
+    if compute == abi.COMPUTE_BF16:
+        return torch.bfloat16
+    if compute == abi.COMPUTE_F16:
+        return torch.float16
+    raise OnhipError(f"16-bit storage: compute type {compute} is neither bf16 nor fp16")
+
+
+def h16_pack_conv_weights(d, w):
+    """fp32 OIHW weights -> [cout][kh*kw][pitch(cin)] in d.compute's 16-bit type"""
+    import torch
+    out = torch.empty((d.cout, d.kh * d.kw, h16_pitch(d.cin)), dtype=_h16_torch_dtype(d.compute), device=w.device)
+    _check(load().onhip_h16_pack_conv_weights(C.byref(d), _ptr(w), _ptr(out), _stream()), "onhip_h16_pack_conv_weights")
+    return out
+
+
+def h16_pack_matmul_weights(b, compute):
+    """the right operand [K, N] (fp32) of a MatMul -> [N][pitch(K)] 16-bit"""
+    import torch
+    k, n = b.shape
+    out = torch.empty((n, h16_pitch(k)), dtype=_h16_torch_dtype(compute), device=b.device)
+    _check(load().onhip_h16_pack_matmul_weights(_ptr(b), k, n, compute, _ptr(out), _stream()), "onhip_h16_pack_matmul_weights")
+    return out
+
+
+def h16_from_nchw(x, compute):
+    import torch
+    n, c, h, w = x.shape
+    out = torch.empty((n, h, w, h16_pitch(c)), dtype=_h16_torch_dtype(compute), device=x.device)
+    _check(load().onhip_h16_from_nchw_f32(_ptr(x), n, c, h, w, compute, _ptr(out), _stream()), "onhip_h16_from_nchw_f32")
+    return out
+
+
+def h16_to_nchw(x, c, compute):
+    import torch
+    n, h, w, cp = x.shape
+    assert cp == h16_pitch(c)
+    out = torch.empty((n, c, h, w), dtype=torch.float32, device=x.device)
+    _check(load().onhip_h16_to_nchw_f32(_ptr(x), n, c, h, w, compute, _ptr(out), _stream()), "onhip_h16_to_nchw_f32")
+    return out
+
+
+def h16_from_rows(x, compute):
+    import torch
+    rows, k = x.shape
+    out = torch.empty((rows, h16_pitch(k)), dtype=_h16_torch_dtype(compute), device=x.device)
+    _check(load().onhip_h16_from_rows_f32(_ptr(x), rows, k, compute, _ptr(out), _stream()), "onhip_h16_from_rows_f32")
+    return out
+
+
+def h16_to_rows(x, k, compute):
+    import torch
+    rows = x.shape[0]
+    out = torch.empty((rows, k), dtype=torch.float32, device=x.device)
+    _check(load().onhip_h16_to_rows_f32(_ptr(x), rows, k, compute, _ptr(out), _stream()), "onhip_h16_to_rows_f32")
+    return out
+
+
+def conv2d_h16(d, x, w_packed, bias=None, lut=None, residual=None, residual_relu=False, y_kind=H16_OUT_NHWC, out=None):
+    """x: 16-bit NHWC [n][h][w][pitch(cin)]; result by y_kind: 16-bit NHWC, fp32 NHWC [n][oh][ow][cout] or fp32 NCHW"""
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        if y_kind == H16_OUT_NHWC:
+            out = torch.empty((d.n, oh, ow, h16_pitch(d.cout)), dtype=x.dtype, device=x.device)
+        elif y_kind == H16_OUT_F32_NHWC:
+            out = torch.empty((d.n, oh, ow, d.cout), dtype=torch.float32, device=x.device)
+        else:
+            out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device=x.device)
+    _check(load().onhip_conv2d_h16(C.byref(d), _ptr(x), _ptr(w_packed), _ptr(bias), _ptr(lut), _ptr(residual),
+                                   int(residual_relu), _ptr(out), y_kind, _stream()), "onhip_conv2d_h16")
+    return out
+
+
+def linear_h16(x, w_packed, k, n, compute, bias=None, gelu_lut=None, residual=None, y_kind=H16_OUT_NHWC, out=None):
+    """x: 16-bit rows [rows][pitch(k)], w_packed from h16_pack_matmul_weights; y = x @ b (+ bias) (GELU table)"""
+    import torch
+    rows = x.shape[0]
+    if out is None:
+        if y_kind == H16_OUT_NHWC:
+            out = torch.empty((rows, h16_pitch(n)), dtype=x.dtype, device=x.device)
+        else:
+            out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
+    _check(load().onhip_linear_h16(rows, k, n, compute, _ptr(x), _ptr(w_packed), _ptr(bias), _ptr(gelu_lut), _ptr(residual),
+                                   _ptr(out), y_kind, _stream()), "onhip_linear_h16")
     return out
 
 
