@@ -279,6 +279,64 @@ class VitGlueLayer:
         return fl, lambda: oracle.transpose_f32(x, self.perm)
 
 
+class ConvH16Layer:
+    """dense convolution with bf16 / fp16 storage: 16-bit NHWC in, 16-bit NHWC out, weights packed once"""
+    kind = "conv_h16"
+
+    def __init__(self, torch, hip, name, d, compute, tag):
+        from onenew_amd import abi, datagen
+        d = abi.ConvDesc.from_buffer_copy(d)
+        d.compute = compute
+        w = datagen.normal(datagen.seed_for(f"{tag}/{name}", "w"), (d.cout, d.cin, d.kh, d.kw), 0.0, float(np.sqrt(2.0 / (d.cin * d.kh * d.kw))))
+        b = datagen.normal(datagen.seed_for(f"{tag}/{name}", "b"), (d.cout,), 0.0, 0.01)
+        self.name, self.d = name, d
+        x = device_uniform(torch, datagen.seed_for(f"{tag}/{name}", "x"), (d.n, d.cin, d.h, d.w))
+        self.x = hip.h16_from_nchw(x, compute)
+        del x
+        self.wp, self.b = hip.h16_pack_conv_weights(d, torch.from_numpy(w).cuda()), torch.from_numpy(b).cuda()
+        oh, ow = d.out_hw()
+        self.y = torch.empty((d.n, oh, ow, hip.h16_pitch(d.cout)), dtype=self.x.dtype, device="cuda")
+        # every tensor once at 2 bytes per element, unpadded (the channel padding the layout adds is not counted as work)
+        self.flops, self.bytes = d.flops(), d.algorithmic_bytes(eb_x=2, eb_w=2, eb_y=2)
+        self.dense = True
+        self.shape = f"M={d.cout} N={d.n * oh * ow} K={d.k_per_out()}"
+
+    def launch(self, hip):
+        hip.conv2d_h16(self.d, self.x, self.wp, self.b, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        return ConvF32Layer.cpu_runner(self, ops, oracle, tag)
+
+
+class LinearH16Layer:
+    """a transformer's linear layer with bf16 / fp16 storage: rows in, rows out, fused bias and table GELU"""
+    kind = "linear_h16"
+
+    def __init__(self, torch, hip, name, md, has_bias, gelu, compute, tag):
+        import cases
+        from onenew_amd import datagen
+        self.name, self.md, self.compute = name, md, compute
+        rows = md.batch * md.m
+        a = datagen.normal(datagen.seed_for(tag, name, "a"), (md.batch, md.m, md.k), 0.0, 1.0)
+        b = datagen.normal(datagen.seed_for(tag, name, "b"), (md.k, md.n), 0.0, 0.02)
+        self.host = (a, b)
+        self.a = hip.h16_from_rows(torch.from_numpy(a.reshape(rows, md.k)).cuda(), compute)
+        self.bp = hip.h16_pack_matmul_weights(torch.from_numpy(b).cuda(), compute)
+        self.bias = torch.from_numpy(datagen.normal(datagen.seed_for(tag, name, "bias"), (md.n,), 0.0, 0.02)).cuda() \
+            if has_bias else None
+        self.lut = torch.from_numpy(cases.gelu_lut()).cuda() if gelu else None
+        self.y = torch.empty((rows, hip.h16_pitch(md.n)), dtype=self.a.dtype, device="cuda")
+        self.flops, self.bytes = md.flops(), md.algorithmic_bytes(eb=2, bias=has_bias)
+        self.dense = True
+        self.shape = f"B={md.batch} M={md.m} N={md.n} K={md.k}"
+
+    def launch(self, hip):
+        hip.linear_h16(self.a, self.bp, self.md.k, self.md.n, self.compute, bias=self.bias, gelu_lut=self.lut, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        return MatmulLayer.cpu_runner(self, ops, oracle, tag)
+
+
 class MatmulLayer:
     kind = "matmul"
 
@@ -326,6 +384,17 @@ def make_workload(torch, hip, name):
     def conv_stack(layers):
         return [ConvF32Layer(torch, hip, n, d, tag) for n, d in layers]
 
+    if name.startswith("resnet50_b") and name.endswith(("_bf16", "_f16")):
+        n = int(name.split("_b")[1].split("_")[0])
+        compute, dtype = (abi.COMPUTE_BF16, "bf16") if name.endswith("_bf16") else (abi.COMPUTE_F16, "f16")
+        return (f"ResNet-50 conv stack {dtype} with 16-bit storage (NHWC in and out, fp32 accumulate), batch {n}, 224x224, "
+                f"53 conv layers, fused ReLU", dtype,
+                [ConvH16Layer(torch, hip, ln, d, compute, tag) for ln, d in stacks.with_batch(stacks.resnet50(), n)])
+    if name in ("cfg1_bf16", "cfg1_f16"):
+        import cases
+        compute, dtype = (abi.COMPUTE_BF16, "bf16") if name.endswith("_bf16") else (abi.COMPUTE_F16, "f16")
+        return (f"Conv2d+ReLU {dtype} with 16-bit storage 64->64 56x56 3x3 s1 p1, batch 1", dtype,
+                [ConvH16Layer(torch, hip, "cfg1", cases.conv_f32_cases()["cfg1_64x56_3x3"], compute, tag)])
     if name.startswith("resnet50_b"):
         n = int(name.split("_b")[1])
         return (f"ResNet-50 conv stack fp32, batch {n}, 224x224, 53 conv layers, fused ReLU", "f32",
@@ -383,6 +452,13 @@ def make_workload(torch, hip, name):
         elif rest.endswith("_f16"):
             compute, dtype, rest = abi.COMPUTE_F16, "f16", rest[:-4]
         n = int(rest)
+        if compute != abi.COMPUTE_F32:
+            # 16-bit storage for the four linear layers; the two attention products (per head, both operands activations)
+            # keep fp32 storage with operands rounded on the way into LDS
+            layers = [LinearH16Layer(torch, hip, ln, md, hb, g, compute, tag) if md.b_shared else
+                      MatmulLayer(torch, hip, ln, md, hb, g, compute, tag) for ln, md, hb, g in stacks.vit_tiny(n)]
+            return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads: qkv / proj / fc1 (fused bias + table "
+                    f"GELU) / fc2 with 16-bit storage, scores and context with fp32 storage", dtype, layers)
         layers = [MatmulLayer(torch, hip, ln, md, hb, g, compute, tag) for ln, md, hb, g in stacks.vit_tiny(n)]
         return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads; fc1 with fused bias + table GELU",
                 dtype, layers)
@@ -524,12 +600,12 @@ def bench_net(torch, args):
 
 
 METRIC = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vit_tiny_glue_ops_fp32_tflops",
-          "resnet50": "resnet50_conv_stack_fp32_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
+          "resnet50": "resnet50_conv_stack_{dtype}_tflops", "mobilenetv2": "mobilenetv2_conv_stack_fp32_tflops",
           "yolov8s_int8chain": "yolov8s_conv_stack_w8a8_tops", "yolov8s": "yolov8s_conv_stack_w8a32_tops",
-          "vit": "vit_tiny_matmul_{dtype}_tflops", "cfg1": "conv2d_relu_fp32_tflops"}
+          "vit": "vit_tiny_matmul_{dtype}_tflops", "cfg1": "conv2d_relu_{dtype}_tflops"}
 
 # the other configurations of the benchmark, timed after the headline one in a default run
-OTHER_CONFIGS = ["cfg1", "resnet50_b1", "mobilenetv2_b64", "mobilenetv2_b1", "vit_tiny_b64", "vit_tiny_b64_bf16", "vit_tiny_b1",
+OTHER_CONFIGS = ["cfg1", "cfg1_bf16", "resnet50_b1", "resnet50_b32_bf16", "mobilenetv2_b64", "mobilenetv2_b1", "vit_tiny_b64", "vit_tiny_b64_bf16", "vit_tiny_b1",
                  "yolov8s_int8_b16", "yolov8s_int8chain_b16", "yolov8s_int8chain_b1"]
 
 
@@ -594,7 +670,9 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False, graph=True
     grp = groups[dom_dense]
     g_ms = sum(t for _, t in grp)
     g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
-    kernel = (f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
+    kernel = ("onhip::igemm_dma_kernel (operand tiles straight into LDS, 16-bit storage, MFMA implicit GEMM)"
+              if dom_dense and grp[0][0].kind in ("conv_h16", "linear_h16") else
+              f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
               "element-wise / pooling / normalisation kernels (elementwise.hip, vit_glue.hip)" if grp[0][0].kind == "glue"
               else "onhip::depthwise_tiled_kernel")
     # the bound is the roof the group's arithmetic intensity puts it under
@@ -726,7 +804,7 @@ def main():
     cpu = None if args.no_cpu else cpu_baseline(layers, args.workload, unit)
 
     key = next(k for k in METRIC if args.workload.startswith(k))
-    line = {"metric": METRIC[key].format(dtype=dtype), "value": round(res["value"], 3), "unit": unit, "n_gpus": 1,
+    line = {"metric": METRIC[key].format(dtype="fp32" if dtype == "f32" and "{dtype}_tflops" in METRIC[key] and key != "vit" else dtype), "value": round(res["value"], 3), "unit": unit, "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
             "config": {"workload": res["desc"], "layers": len(layers), "ops_per_step": res["flops"],

@@ -171,7 +171,8 @@ static const int kNumSplits = 13;
 // rowb != 0: the kernel that feeds B from global memory straight into the MFMAs (igemm_rowb.hip), tile bm x bn
 // fin != 0 (with split > 1 or tail > 1): the slices of a tile are added up by the last of them to arrive, inside the
 // launch, instead of by a finishing launch (igemm_kernel, `arrive`)
-// dma != 0: the int8 kernel that loads its operand tiles straight into LDS (igemm_dma.hip), tile bm x bn, never split
+// dma != 0: the kernel that loads its operand tiles straight into LDS (igemm_dma_kernel.hpp), tile bm x bn, never split;
+// 1 = ring of stages within 64 KiB of LDS, 2 = the long ring
 struct Choice { int bm, bn, split, tail, rowb, fin, dma; };
 
 static std::mutex g_tune_mu;
@@ -296,7 +297,7 @@ static const int kNumRowbTiles = 6;
 
 // (bm, bn) is a tile this build has a kernel for
 static bool tile_exists(const Choice &c) {
-    if (c.dma) return dma_tile_ok(c.bm, c.bn);
+    if (c.dma) return c.dma <= 2 && dma_tile_ok(c.bm, c.bn);
     const int (*list)[2] = c.rowb ? kRowbTiles : kTiles;
     const int n = c.rowb ? kNumRowbTiles : kNumTiles;
     for (int t = 0; t < n; ++t)
@@ -402,6 +403,7 @@ static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStr
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
     if (c.dma) {
         cfg.bm = c.bm; cfg.bn = c.bn; cfg.split = 1;
+        cfg.ring = c.dma > 1;
         p.k_split_units = p.k_units;
         p.partial = nullptr;
         p.arrive = nullptr;
@@ -467,7 +469,7 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
         Choice c = {0, 0, 1, 0, 0, 0, 0};
         if (sscanf(env, "%dx%dx%dx%dx%dx%dx%d", &c.bm, &c.bn, &c.split, &c.tail, &c.rowb, &c.fin, &c.dma) >= 2) {
             if (cfg.dtype != DT_I8 && (cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP)) {   // 16-bit storage: one kernel, its tiles
-                c = {c.bm, c.bn, 1, 0, 0, 0, 1};
+                c = {c.bm, c.bn, 1, 0, 0, 0, c.dma > 1 ? 2 : 1};
                 if (!candidate_ok(cfg, p, c)) c = model_choice(cfg, p);
             }
             if (c.dma && !candidate_ok(cfg, p, c)) {   // not a problem (or a tile) for that kernel: the register-staged one
@@ -559,8 +561,8 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     }
     // the int8 kernel that loads its tiles straight into LDS
     static const int kDmaTiles[][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
-    for (int t = 0; t < 4 && !rc; ++t) {
-        const Choice c = {kDmaTiles[t][0], kDmaTiles[t][1], 1, 0, 0, 0, 1};
+    for (int t = 0; t < 8 && !rc; ++t) {
+        const Choice c = {kDmaTiles[t % 4][0], kDmaTiles[t % 4][1], 1, 0, 0, 0, 1 + t / 4};   // both ring lengths
         if (candidate_ok(cfg, p, c)) try_choice(c);
     }
     (void) hipEventDestroy(e0);

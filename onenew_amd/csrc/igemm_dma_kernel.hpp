@@ -62,7 +62,10 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
     constexpr int A_LOADS = BM / ROWS_PER_LOAD / 4, B_LOADS = BN / ROWS_PER_LOAD / 4;   // per wavefront and stage
     static_assert(A_LOADS >= 1 && B_LOADS >= 1, "every wavefront loads part of both operands");
     constexpr int STAGE = (BM + BN) * KS, PER_STAGE = A_LOADS + B_LOADS;
-    static_assert(NST >= 2 && NST * STAGE <= 65536, "stage offsets must fit the 16-bit immediate of ds_read");
+    // a ds_read reaches 64 KiB beyond its address register: a ring longer than that gets one set of read addresses per
+    // 64 KiB window, and a stage's offset inside its window is the instruction's immediate
+    static_assert(NST >= 2 && NST * STAGE <= 160 * 1024, "the ring must fit the 160 KiB of LDS of a compute unit");
+    constexpr int NSETS = (NST * STAGE + 65535) / 65536;
     // after the K loop the same memory holds the store's staging area, the quantised activation table and the per-row constants
     constexpr int OUT_STAGE = DT == DT_I8 ? BN * (BM + 16) : BN * (2 * BM + 16), ROWS_AT = OUT_STAGE + 8192, OUT_BYTES = ROWS_AT + 2 * BM * 4;
     static_assert(ROWS_AT % 16 == 0, "the per-row constants are read 16 bytes at a time");
@@ -169,40 +172,44 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
     for (int s = 0; s < NST - 1; ++s) issue(s, s);
 
     const unsigned lds0 = (unsigned) (size_t) (__attribute__((address_space(3))) unsigned char *) lds;
-    unsigned a_addr[TM][KSTEPS], b_addr[TN][KSTEPS];
+    unsigned a_addr[NSETS][TM][KSTEPS], b_addr[NSETS][TN][KSTEPS];
 #pragma unroll
-    for (int a = 0; a < TM; ++a) {
-        const int row = wm * TM * 32 + a * 32 + li;
+    for (int w = 0; w < NSETS; ++w) {
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) a_addr[a][s] = lds0 + row * KS + (((2 * s + lh) ^ dma_swz<KS>(row)) * 16);
-    }
+        for (int a = 0; a < TM; ++a) {
+            const int row = wm * TM * 32 + a * 32 + li;
 #pragma unroll
-    for (int b = 0; b < TN; ++b) {
-        const int row = wn * TN * 32 + b * 32 + li;
+            for (int s = 0; s < KSTEPS; ++s) a_addr[w][a][s] = lds0 + w * 65536 + row * KS + (((2 * s + lh) ^ dma_swz<KS>(row)) * 16);
+        }
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) b_addr[b][s] = lds0 + BM * KS + row * KS + (((2 * s + lh) ^ dma_swz<KS>(row)) * 16);
+        for (int b = 0; b < TN; ++b) {
+            const int row = wn * TN * 32 + b * 32 + li;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s)
+                b_addr[w][b][s] = lds0 + w * 65536 + BM * KS + row * KS + (((2 * s + lh) ^ dma_swz<KS>(row)) * 16);
+        }
     }
 
     auto stage_body = [&](int kt, auto bufc) __attribute__((always_inline)) {
-        constexpr int SB = decltype(bufc)::value * STAGE;
+        constexpr int SET = (decltype(bufc)::value * STAGE) >> 16, SB = (decltype(bufc)::value * STAGE) & 0xffff;
         // this wavefront's loads of stage kt have landed once at most the loads of the NST - 2 later stages are out;
         // the barrier says the same of everybody's, and that everybody has read stage kt - 1, whose buffer is loaded next
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NST - 2) * PER_STAGE) : "memory");
         __builtin_amdgcn_s_barrier();
         i32x4 av[2][TM], bv[2][TN];
 #pragma unroll
-        for (int a = 0; a < TM; ++a) av[0][a] = lds_read_b128<SB>(a_addr[a][0]);
+        for (int a = 0; a < TM; ++a) av[0][a] = lds_read_b128<SB>(a_addr[SET][a][0]);
 #pragma unroll
-        for (int b = 0; b < TN; ++b) bv[0][b] = lds_read_b128<SB>(b_addr[b][0]);
+        for (int b = 0; b < TN; ++b) bv[0][b] = lds_read_b128<SB>(b_addr[SET][b][0]);
         issue(kt + NST - 1, (decltype(bufc)::value + NST - 1) % NST);
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             const int cur = s & 1, nxt = cur ^ 1;
             if (s + 1 < KSTEPS) {
 #pragma unroll
-                for (int a = 0; a < TM; ++a) av[nxt][a] = lds_read_b128<SB>(a_addr[a][s + 1]);
+                for (int a = 0; a < TM; ++a) av[nxt][a] = lds_read_b128<SB>(a_addr[SET][a][s + 1]);
 #pragma unroll
-                for (int b = 0; b < TN; ++b) bv[nxt][b] = lds_read_b128<SB>(b_addr[b][s + 1]);
+                for (int b = 0; b < TN; ++b) bv[nxt][b] = lds_read_b128<SB>(b_addr[SET][b][s + 1]);
                 wait_operands<TM + TN>(av[cur], bv[cur]);
             } else {
                 wait_operands<0>(av[cur], bv[cur]);
@@ -311,19 +318,29 @@ template <int DT>
 int dma_launch_dt(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
     const int ks = dma_stage_bytes(p);
     const int key = cfg.bm * 1000 + cfg.bn;
+    // cfg.ring != 0: the long rings, more than 64 KiB of LDS for one workgroup (one or two workgroups per compute unit,
+    // three to seven stages of loads in flight each); otherwise rings of at most 64 KiB
     if (ks == 128) {
-        switch (key) {
+        switch (key + (cfg.ring ? 1000000 : 0)) {
             case 128128: return dma_launch_one<DT, 128, 128, 128, 2>(p, stream);
             case 128064: return dma_launch_one<DT, 128, 64, 128, 2>(p, stream);
             case 64128: return dma_launch_one<DT, 64, 128, 128, 2>(p, stream);
             case 64064: return dma_launch_one<DT, 64, 64, 128, 3>(p, stream);
+            case 1128128: return dma_launch_one<DT, 128, 128, 128, 4>(p, stream);
+            case 1128064: return dma_launch_one<DT, 128, 64, 128, 5>(p, stream);
+            case 1064128: return dma_launch_one<DT, 64, 128, 128, 5>(p, stream);
+            case 1064064: return dma_launch_one<DT, 64, 64, 128, 5>(p, stream);
         }
     } else {
-        switch (key) {
+        switch (key + (cfg.ring ? 1000000 : 0)) {
             case 128128: return dma_launch_one<DT, 128, 128, 64, 3>(p, stream);
             case 128064: return dma_launch_one<DT, 128, 64, 64, 4>(p, stream);
             case 64128: return dma_launch_one<DT, 64, 128, 64, 4>(p, stream);
             case 64064: return dma_launch_one<DT, 64, 64, 64, 4>(p, stream);
+            case 1128128: return dma_launch_one<DT, 128, 128, 64, 6>(p, stream);
+            case 1128064: return dma_launch_one<DT, 128, 64, 64, 8>(p, stream);
+            case 1064128: return dma_launch_one<DT, 64, 128, 64, 8>(p, stream);
+            case 1064064: return dma_launch_one<DT, 64, 64, 64, 8>(p, stream);
         }
     }
     return set_error(ONHIP_ERR_ARG, "igemm: no direct-to-LDS kernel for tile %dx%d", cfg.bm, cfg.bn);

@@ -219,6 +219,7 @@ struct IgemmLaunch {
     int bm, bn;     // tile
     int batch;      // grid.z
     int split;      // grid.y
+    int ring;       // direct-to-LDS kernel: 0 = ring of stage buffers within 64 KiB of LDS, 1 = the long ring
 };
 
 int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);

@@ -186,6 +186,74 @@ def test_vit_tiny_batch64_every_matmul(layer, compute, torch_dev, oracle):
         assert np.array_equal(yg.cpu().numpy(), oracle.lut_act(y, lut)), name
 
 
+# ---- 16-bit storage at full size ---------------------------------------------------------------------------------------
+def _round16(torch, t, compute):
+    """the operand as the 16-bit kernels see it, back in fp32 (torch's conversion is round-to-nearest-even, the
+    oracle's rule; the small tests compare the library's conversions with the oracle's bit for bit)"""
+    return t.to(torch.bfloat16 if compute == abi.COMPUTE_BF16 else torch.float16).float()
+
+
+@pytest.mark.parametrize("compute", [abi.COMPUTE_BF16, abi.COMPUTE_F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("layer", [i for i, v in enumerate(VIT) if v[1].b_shared], ids=[v[0] for v in VIT if v[1].b_shared])
+def test_vit_tiny_batch64_linear_layers_16bit_storage(layer, compute, torch_dev, oracle):
+    """qkv / proj / fc1 / fc2 at batch 64 with operands and result stored in 16 bits: the fp32 output against the oracle on
+    rounded operands (1e-4) and on the unrounded ones (1e-2); the 16-bit output is the rounding of the fp32 one"""
+    torch = torch_dev
+    name, md, has_bias, gelu = VIT[layer]
+    print(f"vit b64 {name} 16-bit storage compute {compute}", flush=True)
+    rows = md.batch * md.m
+    a = datagen.normal(_seed("vit", name, "a"), (rows, md.k), 0.0, 1.0)
+    b = datagen.normal(_seed("vit", name, "b"), (md.k, md.n), 0.0, 0.02)
+    bias = datagen.normal(_seed("vit", name, "bias"), (md.n,), 0.0, 0.02) if has_bias else None
+    lut = cases.gelu_lut() if gelu else None
+    cu = lambda t: None if t is None else torch.from_numpy(t).cuda()
+    ah, bp = hip.h16_from_rows(cu(a), compute), hip.h16_pack_matmul_weights(cu(b), compute)
+    pre = hip.linear_h16(ah, bp, md.k, md.n, compute, bias=cu(bias), y_kind=hip.H16_OUT_F32_NHWC)
+    y32 = hip.linear_h16(ah, bp, md.k, md.n, compute, bias=cu(bias), gelu_lut=cu(lut), y_kind=hip.H16_OUT_F32_NHWC)
+    y16 = hip.linear_h16(ah, bp, md.k, md.n, compute, bias=cu(bias), gelu_lut=cu(lut))
+    torch.cuda.synchronize()
+    rnd = oracle.round_bf16 if compute == abi.COMPUTE_BF16 else oracle.round_f16
+    ref16 = oracle.matmul_f32(rnd(a), rnd(b), bias=bias)
+    ref32 = oracle.matmul_f32(a, b, bias=bias)
+    scale = float(np.abs(ref32).max())
+    pre = pre.cpu().numpy()
+    assert np.abs(pre - ref16).max() <= 1e-4 * scale, name
+    assert np.abs(pre - ref32).max() <= 1e-2 * scale, name
+    y32 = y32.cpu().numpy()
+    assert np.array_equal(y32, oracle.lut_act(pre, lut) if gelu else pre)
+    got = y16.float().cpu().numpy()
+    assert np.array_equal(got[:, :md.n], rnd(y32)) and not got[:, md.n:].any()
+
+
+@pytest.mark.parametrize("layer", range(len(RESNET)), ids=[n for n, _ in RESNET])
+def test_resnet50_batch32_every_layer_bf16_storage(layer, torch_dev):
+    """every convolution of the stack with bf16 NHWC tensors: sampled outputs of the fp32 form against the float64 sum over
+    the rounded operands; the bf16 output (what the next layer reads) is the rounding of the fp32 one everywhere"""
+    torch = torch_dev
+    name, d = RESNET[layer]
+    print(f"resnet50 b32 bf16 {name}", flush=True)
+    d = ConvDesc.from_buffer_copy(d)
+    d.compute = abi.COMPUTE_BF16
+    x = _device_uniform(torch, _seed("rn50b32h", name, "x"), (d.n, d.cin, d.h, d.w))
+    w = datagen.normal(_seed("rn50b32h", name, "w"), (d.cout, d.cin, d.kh, d.kw), 0.0, float(np.sqrt(2.0 / (d.cin * d.kh * d.kw))))
+    b = datagen.normal(_seed("rn50b32h", name, "b"), (d.cout,), 0.0, 0.01)
+    wd, bd = torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()
+    xh, wp = hip.h16_from_nchw(x, d.compute), hip.h16_pack_conv_weights(d, wd)
+    y32 = hip.conv2d_h16(d, xh, wp, bd, y_kind=hip.H16_OUT_F32_NCHW)
+    y16 = hip.conv2d_h16(d, xh, wp, bd)
+    torch.cuda.synchronize()
+    flat, n, m, i, j = _sample_index(_seed("rn50b32h", name, "probe"), d)
+    got = y32.reshape(-1)[torch.from_numpy(flat).cuda()].cpu().numpy().astype(np.float64)
+    p = _patches(torch, _round16(torch, x, d.compute), d, n, i, j).astype(np.float64)
+    wr = _round16(torch, wd, d.compute).cpu().numpy().astype(np.float64)
+    ref = _act_f64(d, np.einsum("sckl,sckl->s", p, wr[m]) + b[m].astype(np.float64))
+    scale = max(float(np.abs(ref).max()), 1e-6)
+    assert np.abs(got - ref).max() <= 1e-4 * scale, f"{name}: {np.abs(got - ref).max():.3e} against {scale:.3e}"
+    want16 = y32.permute(0, 2, 3, 1).to(torch.bfloat16)
+    assert torch.equal(y16[..., :d.cout], want16), name
+    assert not bool(y16[..., d.cout:].any())
+
+
 # ---- YOLOv8s int8, batch 16 ---------------------------------------------------------------------------------------
 
 def _yolo_operands(torch, i, name, d):

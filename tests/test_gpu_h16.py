@@ -114,10 +114,13 @@ def run_conv_h16(torch, oracle, d, name, tile, monkeypatch, lut=None):
 
 
 @pytest.mark.parametrize("compute", TYPES)
+@pytest.mark.parametrize("ring", [1, 2])
 @pytest.mark.parametrize("tile", ["128x128", "128x64", "64x128", "64x64"])
 @pytest.mark.parametrize("shape", CONV_SHAPES)
-def test_conv_h16_every_tile(compute, tile, shape, torch_dev, oracle, monkeypatch):
+def test_conv_h16_every_tile(compute, ring, tile, shape, torch_dev, oracle, monkeypatch):
+    """ring: 1 = stage buffers within 64 KiB of LDS, 2 = the long ring (up to 144 KiB)"""
     torch = torch_dev
+    tile = f"{tile}x1x0x0x0x{ring}"
     n, cin, hw, cout, k, stride, pad = shape
     d = with_compute(cases.cd(cin, cout, k, stride, pad, hw, n=n, act=abi.RELU), compute)
     name = f"h16_{cin}_{cout}_{k}_{stride}"

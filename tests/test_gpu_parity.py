@@ -1105,13 +1105,14 @@ def test_conv_w8a8_nhwc_chain_form(name, tile, torch_dev, oracle, monkeypatch):
 @pytest.mark.parametrize("shape", [(2, 64, 19, 72, 3, 1, 1), (1, 128, 23, 200, 3, 2, 1), (3, 192, 9, 130, 1, 1, 0), (2, 128, 12, 64, 5, 1, 2),
                                    (1, 256, 7, 33, 3, 1, 1), (2, 64, 16, 128, 1, 2, 0)])
 @pytest.mark.parametrize("act", [abi.SILU, abi.RELU, abi.NOT_ACT])
-def test_conv_int8_direct_to_lds_kernel_every_tile(tile, shape, act, torch_dev, oracle, monkeypatch):
+@pytest.mark.parametrize("ring", [1, 2])
+def test_conv_int8_direct_to_lds_kernel_every_tile(ring, tile, shape, act, torch_dev, oracle, monkeypatch):
     """the int8 kernel that loads its tiles from global memory straight into LDS, every tile it has, on shapes with ragged
     rows and columns, strides, padding, 64- and 128-byte stages (channels a multiple of 64 / of 128), one and many taps,
     a single stage and many: int8 NHWC chain form and the fp32 / int32-accumulator form, both equal to the oracle"""
     torch = torch_dev
     n, cin, hw, cout, k, stride, pad = shape
-    monkeypatch.setenv("ONHIP_TILE", tile + "x1x0x0x0x1")
+    monkeypatch.setenv("ONHIP_TILE", tile + f"x1x0x0x0x{ring}")   # ring 2: the long ring of stage buffers (more than 64 KiB of LDS)
     d = cases.cd(cin, cout, k, stride, pad, hw, n=n, act=act, input_scale=0.037)
     name = f"dma_{tile}_{cin}_{cout}_{k}_{stride}"
     x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
