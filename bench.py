@@ -337,6 +337,42 @@ class LinearH16Layer:
         return MatmulLayer.cpu_runner(self, ops, oracle, tag)
 
 
+class AttentionLayer:
+    """scores = q k^T * scale, Softmax, context = scores v of every (batch, head) in one launch, q / k / v read as slices of
+    the qkv projection's output and the context written with the heads merged; counted as the two MatMuls it replaces"""
+    kind = "attention"
+
+    def __init__(self, torch, hip, name, md_scores, md_context, heads, tag):
+        from onenew_amd import datagen
+        self.name = name
+        bh, t, hd = md_scores.batch, md_scores.m, md_scores.k
+        b = bh // heads
+        self.qkv = device_uniform(torch, datagen.seed_for(tag, name, "qkv"), (b, t, 3, heads, hd), -1.5, 1.5)
+        self.q, self.k, self.v = (self.qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        self.scale = 1.0 / float(np.sqrt(hd))
+        self.y = torch.empty((b, t, heads * hd), dtype=torch.float32, device="cuda")
+        self.mds = (md_scores, md_context)
+        self.flops = md_scores.flops() + md_context.flops()
+        self.bytes = md_scores.algorithmic_bytes() + md_context.algorithmic_bytes()   # of the unfused chain's two MatMuls
+        self.dense = True
+        self.shape = f"B={b} H={heads} T={t} D={hd}"
+
+    def launch(self, hip):
+        hip.attention(self.q, self.k, self.v, scale=self.scale, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        # reference semantics: the two MatMuls and the Softmax between them as separate operators
+        ms, mc = self.mds
+        from onenew_amd import datagen
+        q = datagen.normal(datagen.seed_for(tag, self.name, "cq"), (ms.batch, ms.m, ms.k), 0.0, 1.0)
+        kt = datagen.normal(datagen.seed_for(tag, self.name, "ck"), (ms.batch, ms.k, ms.n), 0.0, 1.0)
+        v = datagen.normal(datagen.seed_for(tag, self.name, "cv"), (mc.batch, mc.k, mc.n), 0.0, 1.0)
+
+        def run():
+            return oracle.matmul_f32(oracle.softmax_f32(oracle.matmul_f32(q, kt)), v)
+        return self.flops, run
+
+
 class MatmulLayer:
     kind = "matmul"
 
@@ -459,8 +495,15 @@ def make_workload(torch, hip, name):
                       MatmulLayer(torch, hip, ln, md, hb, g, compute, tag) for ln, md, hb, g in stacks.vit_tiny(n)]
             return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads: qkv / proj / fc1 (fused bias + table "
                     f"GELU) / fc2 with 16-bit storage, scores and context with fp32 storage", dtype, layers)
-        layers = [MatmulLayer(torch, hip, ln, md, hb, g, compute, tag) for ln, md, hb, g in stacks.vit_tiny(n)]
-        return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads; fc1 with fused bias + table GELU",
+        spec = {ln: (md, hb, g) for ln, md, hb, g in stacks.vit_tiny(n)}
+        layers = []
+        for ln, md, hb, g in stacks.vit_tiny(n):
+            if ln == "scores":
+                layers.append(AttentionLayer(torch, hip, "attention", md, spec["context"][0], 3, tag))
+            elif ln != "context":
+                layers.append(MatmulLayer(torch, hip, ln, md, hb, g, compute, tag))
+        return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads: qkv, attention (scores, Softmax and "
+                f"context in one launch, head split and merge in its strides), proj, fc1 with fused bias + table GELU, fc2",
                 dtype, layers)
     raise SystemExit(f"unknown workload {name}")
 

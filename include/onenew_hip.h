@@ -244,6 +244,23 @@ int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, cons
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
                  const float *gelu_lut, float *out, void *stream);
 
+/* Attention of every (batch, head) in one launch:  out = Softmax(q k^T * scale) v, Softmax over the keys.  Replaces the
+ * operator chain MatMul (device/x86/MatMul/mat_mul.c:10-102) -> [Mul by a constant] -> Softmax (device/x86/Softmax/
+ * softmax.c:26-59) -> MatMul of a transformer block, together with the Transposes (device/x86/Transpose/transpose.c)
+ * that split q, k, v into heads, transpose k and merge the heads again: every operand is addressed through the element
+ * strides of (batch, head, token), the head dimension being contiguous, so q, k and v may be slices of one projection
+ * output [batch][tokens][3 * heads * head_dim] and out the merged [batch][tokens][heads * head_dim].  The scores stay in
+ * registers.  head_dim 32 or 64, at most 256 tokens, rows 16-byte aligned (strides multiples of 4); other shapes are
+ * refused and stay with the separate operators.  compute: ONHIP_COMPUTE_F32. */
+typedef struct onhip_attention_desc {
+    int32_t batch, heads, tokens, head_dim;
+    long long q_strides[3], k_strides[3], v_strides[3], out_strides[3];
+    float scale;      /* 1.0f when the graph has no Mul between the first MatMul and the Softmax */
+    int32_t compute;
+} onhip_attention_desc_t;
+int onhip_attention(const onhip_attention_desc_t *d, const float *q, const float *k, const float *v, float *out,
+                    void *stream);
+
 /* out[m][n] = sum_k a[m][k] * w[n][k] + bias[n].  Replaces gemm.c eval (:9). */
 int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float *w,
                    const float *bias, float *out, void *stream);

@@ -213,6 +213,13 @@ class MatmulDesc(C.Structure):
             + (4 * self.n if bias else 0)
 
 
+class AttentionDesc(C.Structure):
+    """onhip_attention_desc_t"""
+    _fields_ = [("batch", C.c_int32), ("heads", C.c_int32), ("tokens", C.c_int32), ("head_dim", C.c_int32),
+                ("q_strides", C.c_longlong * 3), ("k_strides", C.c_longlong * 3), ("v_strides", C.c_longlong * 3),
+                ("out_strides", C.c_longlong * 3), ("scale", C.c_float), ("compute", C.c_int32)]
+
+
 def check_layout():
     assert C.sizeof(BUFFER_INFO_S) == 16
     assert C.sizeof(OPERAND_S) == 312 and OPERAND_S.shapes.offset == 276 and OPERAND_S.data_type.offset == 308

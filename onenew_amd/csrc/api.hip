@@ -1206,6 +1206,24 @@ int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, cons
     return conv2d_h16_impl(&d, x, w_packed, bias, gelu_lut, gelu_lut != nullptr, residual, 0, y, y_kind, stream);
 }
 
+int onhip_attention(const onhip_attention_desc_t *d, const float *q, const float *k, const float *v, float *out, void *stream) {
+    if (!d || d->batch < 1 || d->heads < 1 || d->tokens < 1) return set_error(ONHIP_ERR_ARG, "attention: bad shape");
+    if (!q || !k || !v || !out) return set_error(ONHIP_ERR_ARG, "attention: null tensor pointer");
+    if (d->compute != ONHIP_COMPUTE_F32) return set_error(ONHIP_ERR_ARG, "attention: fp32 only");
+    if (d->head_dim != 32 && d->head_dim != 64) return set_error(ONHIP_ERR_ARG, "attention: head dimension %d (32 and 64 are fused)", d->head_dim);
+    if (d->tokens > 256) return set_error(ONHIP_ERR_ARG, "attention: %d tokens (at most 256 are fused)", d->tokens);
+    if ((long long) d->batch * d->heads > 65535) return set_error(ONHIP_ERR_ARG, "attention: more than 65535 (batch, head) pairs");
+    const long long *strides[4] = {d->q_strides, d->k_strides, d->v_strides, d->out_strides};
+    const void *ptrs[4] = {q, k, v, out};
+    for (int t = 0; t < 4; ++t) {
+        if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return set_error(ONHIP_ERR_ARG, "attention: tensors must be 16-byte aligned");
+        for (int i = 0; i < 3; ++i)
+            if (strides[t][i] < 0 || strides[t][i] % 4) return set_error(ONHIP_ERR_ARG, "attention: strides must be non-negative multiples of 4");
+        if (strides[t][2] < d->head_dim) return set_error(ONHIP_ERR_ARG, "attention: token stride below the head dimension");
+    }
+    return attention_f32_launch(*d, q, k, v, out, reinterpret_cast<hipStream_t>(stream));
+}
+
 int onhip_copy_f32(const float *src, float *dst, long long n, void *stream) {
     if (!src || !dst || n < 0) return set_error(ONHIP_ERR_ARG, "copy: bad argument");
     return copy_f32_launch(src, dst, n, reinterpret_cast<hipStream_t>(stream));

@@ -243,6 +243,9 @@ int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, flo
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
 int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
 int forget_quantised_tables(const void *base, size_t bytes);   // api.hip: the cache of tables behind an output quantiser
+// attention.hip
+int attention_f32_launch(const onhip_attention_desc_t &d, const float *q, const float *k, const float *v, float *out,
+                         hipStream_t stream);
 // 16-bit storage (h16.hip): dt is DT_BF16 or DT_F16
 int pack_w16_launch(int dt, const float *w, long long rows, int cin, int taps, int cp, long long s_row, long long s_ch,
                     long long s_tap, void *packed, hipStream_t stream);

@@ -39,7 +39,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
-           "onhip_conv2d_h16", "onhip_linear_h16",
+           "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
@@ -108,6 +108,7 @@ def load():
     L.onhip_h16_from_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
     L.onhip_h16_to_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
     L.onhip_conv2d_h16.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, i32, vp, i32, vp]
+    L.onhip_attention.argtypes = [C.POINTER(abi.AttentionDesc), vp, vp, vp, vp, vp]
     L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
@@ -511,6 +512,25 @@ def linear_h16(x, w_packed, k, n, compute, bias=None, gelu_lut=None, residual=No
             out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
     _check(load().onhip_linear_h16(rows, k, n, compute, _ptr(x), _ptr(w_packed), _ptr(bias), _ptr(gelu_lut), _ptr(residual),
                                    _ptr(out), y_kind, _stream()), "onhip_linear_h16")
+    return out
+
+
+def attention(q, k, v, scale=1.0, out=None, merged_out=True):
+    """out = Softmax(q k^T * scale) v per (batch, head).  q, k, v: views [batch, heads, tokens, head_dim] of fp32 tensors in
+    any (batch, head, token) stride order with a contiguous head dimension (e.g. slices of a [batch, tokens, 3, heads,
+    head_dim] projection output, permuted); the result is [batch, tokens, heads * head_dim] (heads merged) or, with
+    merged_out=False, [batch, heads, tokens, head_dim]"""
+    import torch
+    b, h, t, hd = q.shape
+    if out is None:
+        out = torch.empty((b, t, h * hd) if merged_out else (b, h, t, hd), dtype=torch.float32, device=q.device)
+    d = abi.AttentionDesc(batch=b, heads=h, tokens=t, head_dim=hd, scale=scale, compute=abi.COMPUTE_F32)
+    for name, ten in (("q_strides", q), ("k_strides", k), ("v_strides", v)):
+        if ten.stride(3) != 1:
+            raise OnhipError("attention: the head dimension must be contiguous")
+        setattr(d, name, (C.c_longlong * 3)(ten.stride(0), ten.stride(1), ten.stride(2)))
+    d.out_strides = (C.c_longlong * 3)(t * h * hd, hd, h * hd) if merged_out else (C.c_longlong * 3)(h * t * hd, t * hd, hd)
+    _check(load().onhip_attention(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _stream()), "onhip_attention")
     return out
 
 

@@ -1,0 +1,78 @@
+"""onhip_attention against the oracle's operator chain  Transpose -> MatMul -> [Mul] -> Softmax -> MatMul -> Transpose
+(the reference's ViT block runs exactly these operators one after the other), through the C-ABI; the first case is the
+ViT-Tiny configuration at its full batch of 64.  Tolerance 1e-4
+(normalised maximum and per element), the tolerance of the fp32 MatMul and of the Softmax's expf."""
+import numpy as np
+import pytest
+
+import cases
+from onenew_amd import hip
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_dev():
+    import torch
+    hip.init(0)
+    return torch
+
+
+def oracle_chain(oracle, qkv, b, t, h, hd, scale):
+    """qkv: [b, t, 3, h, hd] as the projection writes it -> merged context [b, t, h * hd]"""
+    x = oracle.transpose_f32(qkv.reshape(b, t, 3 * h, hd), (0, 2, 1, 3)).reshape(b, 3, h, t, hd)   # head split
+    q, k, v = x[:, 0], x[:, 1], x[:, 2]
+    kt = oracle.transpose_f32(np.ascontiguousarray(k), (0, 1, 3, 2))
+    s = oracle.matmul_f32(np.ascontiguousarray(q).reshape(b * h, t, hd), kt.reshape(b * h, hd, t))
+    if scale != 1.0:
+        s = (s * np.float32(scale)).astype(np.float32)
+    p = oracle.softmax_f32(s)
+    ctx = oracle.matmul_f32(p, np.ascontiguousarray(v).reshape(b * h, t, hd)).reshape(b, h, t, hd)
+    return oracle.transpose_f32(ctx, (0, 2, 1, 3)).reshape(b, t, h * hd)                            # head merge
+
+
+@pytest.mark.parametrize("shape", [(64, 3, 197, 64, 0.125), (2, 3, 197, 64, 0.125), (1, 1, 17, 32, 1.0), (3, 2, 64, 64, 0.125), (1, 4, 129, 32, 0.25),
+                                   (2, 1, 256, 64, 0.125), (1, 2, 5, 64, 1.0), (1, 3, 224, 64, 0.125), (2, 2, 33, 32, 0.5)])
+def test_attention_equals_the_operator_chain(shape, torch_dev, oracle):
+    torch = torch_dev
+    b, h, t, hd, scale = shape
+    print(f"attention {shape}", flush=True)
+    qkv = cases.datagen.normal(cases.datagen.seed_for("attn", *shape[:4]), (b, t, 3, h, hd), 0.0, 1.5)
+    dev = torch.from_numpy(qkv).cuda()
+    q, k, v = (dev[:, :, i].permute(0, 2, 1, 3) for i in range(3))       # views [b, h, t, hd] of the projection output
+    out = hip.attention(q, k, v, scale=scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    ref = oracle_chain(oracle, qkv, b, t, h, hd, scale).astype(np.float64)
+    top = np.abs(ref).max()
+    assert np.abs(got - ref).max() <= 1e-4 * top, f"{np.abs(got - ref).max():.3e} against {top:.3e}"
+    assert np.all(np.abs(got - ref) <= 1e-4 * np.abs(ref) + 1e-5)
+    # heads kept apart, operands as separate contiguous tensors
+    out2 = hip.attention(q.contiguous(), k.contiguous(), v.contiguous(), scale=scale, merged_out=False)
+    torch.cuda.synchronize()
+    assert torch.equal(out2.permute(0, 2, 1, 3).reshape(b, t, h * hd), out)
+
+
+def test_attention_rows_are_probabilities(torch_dev):
+    """v = identity columns: the output is the Softmax itself; rows sum to one, and large scores do not overflow"""
+    torch = torch_dev
+    t, hd = 64, 64
+    q = torch.randn((1, 1, t, hd), generator=torch.Generator().manual_seed(5)).cuda() * 30.0
+    k = torch.randn((1, 1, t, hd), generator=torch.Generator().manual_seed(6)).cuda()
+    v = torch.eye(t, hd, device="cuda").reshape(1, 1, t, hd).contiguous()
+    p = hip.attention(q, k, v, merged_out=False)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(p).all()) and bool((p >= 0).all())
+    assert torch.allclose(p.sum(-1), torch.ones(1, 1, t, device="cuda"), atol=1e-5)
+
+
+def test_attention_refuses_what_it_does_not_fuse(torch_dev):
+    torch = torch_dev
+    z = lambda *s: torch.zeros(s, device="cuda")
+    with pytest.raises(hip.OnhipError, match="head dimension 48"):
+        hip.attention(z(1, 1, 8, 48), z(1, 1, 8, 48), z(1, 1, 8, 48))
+    with pytest.raises(hip.OnhipError, match="at most 256"):
+        hip.attention(z(1, 1, 257, 64), z(1, 1, 257, 64), z(1, 1, 257, 64))
+    with pytest.raises(hip.OnhipError, match="multiples of 4"):
+        base = z(1, 1, 8, 66)
+        hip.attention(base[..., :64], z(1, 1, 8, 64), z(1, 1, 8, 64))
