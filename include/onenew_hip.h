@@ -244,6 +244,22 @@ int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, cons
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
                  const float *gelu_lut, float *out, void *stream);
 
+/* The second half of an inverted-residual block in one launch: depthwise 3x3 convolution (pads 1, stride 1 or 2, bias,
+ * activation) -> 1x1 convolution (bias, activation) [-> Add of a residual tensor shaped like the output].  Replaces two
+ * (three) operator evaluations, device/x86/Conv/conv.c depthwise path :757-899 and 1x1 path :1024-1056 (and
+ * device/x86/Add/add.c), without the depthwise result ever being written to memory.  The depthwise values are those of
+ * the separate operator bit for bit (same operations in the same order); the 1x1 sums are fp32 in MFMA order like
+ * onhip_conv2d_f32's.  No counterpart as one function in the reference.
+ * onhip_dw_project_supported: 0 = this pair of descriptors is not taken (run the two convolutions), 1 = taken,
+ * 2 = taken and expected to be faster than the two launches.  pw_packed: the 1x1 weights [cout][cin] re-laid once by
+ * onhip_dw_project_pack_weights (onhip_dw_project_packed_weight_bytes(cin, cout) bytes, 16-byte aligned). */
+int onhip_dw_project_supported(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw);
+size_t onhip_dw_project_packed_weight_bytes(int32_t ce, int32_t co);
+int onhip_dw_project_pack_weights(const float *pw_w, int32_t ce, int32_t co, float *packed, void *stream);
+int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const float *x, const float *dw_w,
+                         const float *dw_b, const float *pw_packed, const float *pw_b, const float *residual, float *y,
+                         void *stream);
+
 /* Attention of every (batch, head) in one launch:  out = Softmax(q k^T * scale) v, Softmax over the keys.  Replaces the
  * operator chain MatMul (device/x86/MatMul/mat_mul.c:10-102) -> [Mul by a constant] -> Softmax (device/x86/Softmax/
  * softmax.c:26-59) -> MatMul of a transformer block, together with the Transposes (device/x86/Transpose/transpose.c)
@@ -403,6 +419,12 @@ int onhip_plugin_set_stream(void *stream);
  * [base, base + bytes), so that other data at the same address later is packed afresh.  The device-resident runtime calls it when a net is freed.  No counterpart in the
  * reference (its weights live in host vectors for the life of the process). */
 int onhip_plugin_forget(const void *base, size_t bytes);
+/* `eval` keeps a device copy of every weight and table it was handed in host memory and, on each call, hashes the host
+ * buffer to see whether the copy is still current: all of it by default (about 0.05 ms per MiB), so weights updated in
+ * place are picked up.  on != 0: only 4096 sampled words are hashed, for a caller whose weights never change while the
+ * library is loaded (the reference keeps them in vectors filled once at load, host/op.h).  No counterpart in the
+ * reference. */
+int onhip_plugin_trust_weights(int on);
 /* Drops the device copies of weights the plugin level keeps between calls. */
 int onhip_plugin_release(void);
 

@@ -1206,6 +1206,62 @@ int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, cons
     return conv2d_h16_impl(&d, x, w_packed, bias, gelu_lut, gelu_lut != nullptr, residual, 0, y, y_kind, stream);
 }
 
+// the depthwise 3x3 -> 1x1 pair the fused kernel takes; *why (when not null) says what rules a pair out
+static bool dw_project_shapes_ok(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const char **why) {
+    const char *w = nullptr;
+    int32_t OH = 0, OW = 0;
+    if (!dw || !pw || check_conv(dw, &OH, &OW)) w = "bad depthwise descriptor";
+    else if (dw->group == 1 || dw->group != dw->cin || dw->cout != dw->cin) w = "the first convolution must be depthwise";
+    else if (dw->kh != 3 || dw->kw != 3 || dw->pad_t != 1 || dw->pad_l != 1 || dw->pad_b != 1 || dw->pad_r != 1) w = "depthwise 3x3 with pads 1 only";
+    else if (dw->stride_h != dw->stride_w || (dw->stride_h != 1 && dw->stride_h != 2)) w = "depthwise stride 1 or 2";
+    else if (dw->cin % 16) w = "depthwise channels must be a multiple of 16";
+    else if (!dw->has_bias) w = "the depthwise convolution must have a bias";
+    else if (dw->compute != ONHIP_COMPUTE_F32 || pw->compute != ONHIP_COMPUTE_F32 || dw->act_type == SILU || pw->act_type == SILU) w = "fp32 without table activations";
+    else if (pw->group != 1 || pw->kh != 1 || pw->kw != 1 || pw->stride_h != 1 || pw->stride_w != 1 || pw->pad_t || pw->pad_l || pw->pad_b || pw->pad_r)
+        w = "the second convolution must be 1x1, stride 1, unpadded";
+    else if (pw->cin != dw->cout || pw->n != dw->n || pw->h != OH || pw->w != OW) w = "the second convolution does not take the first one's output";
+    else if (pw->cout < 1 || pw->cout > 128) w = "at most 128 output channels";
+    else if (dwproj_band_rows(*dw, OH, OW, pw->cout) < 1) w = "output rows of more than 128 pixels";
+    else if ((long long) dw->n * dw->cin * dw->h * dw->w * 4 >= (1LL << 31) || (long long) pw->n * pw->cout * OH * OW * 4 >= (1LL << 31)) w = "tensors of 2 GiB or more";
+    if (why) *why = w;
+    return w == nullptr;
+}
+
+int onhip_dw_project_supported(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw) {
+    if (!dw_project_shapes_ok(dw, pw, nullptr)) return 0;
+    // Measured on MobileNetV2 at batch 64 (separate launches against this one): 96 channels 112x112 stride 2, 117 us
+    // against 98 us; stride 1 at 112x112 and 56x56, 83 and 79 us against 120 and 94 us.  The stride-2 depthwise kernel
+    // reads every other column it loads, which the patch here does not pay for; otherwise the two launches, each near
+    // half of the memory bandwidth, beat this kernel's serial chunk pipeline.  Recommended for the first case only.
+    int32_t OH = 0, OW = 0;
+    (void) onhip_conv_out_shape(dw, &OH, &OW);
+    const int rows = dwproj_band_rows(*dw, OH, OW, pw->cout);
+    const long long wgs = (long long) dw->n * ((OH + rows - 1) / rows);
+    return dw->stride_h == 2 && wgs >= 1024 && rows * OW >= 96 ? 2 : 1;
+}
+
+size_t onhip_dw_project_packed_weight_bytes(int32_t ce, int32_t co) {
+    return ce < 1 || co < 1 ? 0 : (size_t) ce * ((co + 31) / 32 * 32) * sizeof(float);
+}
+
+int onhip_dw_project_pack_weights(const float *pw_w, int32_t ce, int32_t co, float *packed, void *stream) {
+    if (!pw_w || !packed || ce < 1 || co < 1 || reinterpret_cast<uintptr_t>(packed) % 16) return set_error(ONHIP_ERR_ARG, "dw + project pack: bad argument");
+    return dwproj_pack_launch(pw_w, ce, co, packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const float *x, const float *dw_w, const float *dw_b,
+                         const float *pw_packed, const float *pw_b, const float *residual, float *y, void *stream) {
+    const char *why = nullptr;
+    if (!dw_project_shapes_ok(dw, pw, &why)) return set_error(ONHIP_ERR_ARG, "dw + project: %s", why);
+    if (!x || !dw_w || !dw_b || !pw_packed || !y || (pw->has_bias && !pw_b)) return set_error(ONHIP_ERR_ARG, "dw + project: null tensor pointer");
+    if (reinterpret_cast<uintptr_t>(pw_packed) % 16) return set_error(ONHIP_ERR_ARG, "dw + project: packed weights must be 16-byte aligned");
+    if (residual == y) return set_error(ONHIP_ERR_ARG, "dw + project: the residual operand may not be the output buffer");
+    int32_t OH = 0, OW = 0;
+    (void) onhip_conv_out_shape(dw, &OH, &OW);
+    return dwproj_f32_launch(*dw, *pw, OH, OW, x, dw_w, dw_b, pw_packed, pw->has_bias ? pw_b : nullptr, residual, make_epilogue(*dw, nullptr),
+                             make_epilogue(*pw, nullptr), y, reinterpret_cast<hipStream_t>(stream));
+}
+
 int onhip_attention(const onhip_attention_desc_t *d, const float *q, const float *k, const float *v, float *out, void *stream) {
     if (!d || d->batch < 1 || d->heads < 1 || d->tokens < 1) return set_error(ONHIP_ERR_ARG, "attention: bad shape");
     if (!q || !k || !v || !out) return set_error(ONHIP_ERR_ARG, "attention: null tensor pointer");

@@ -39,12 +39,12 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
-           "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention",
+           "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", "onhip_dw_project_supported", "onhip_dw_project_packed_weight_bytes", "onhip_dw_project_pack_weights", "onhip_dw_project_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
            "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_gelu_eval", "onhip_layernorm_eval",
-           "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_set_async", "onhip_plugin_set_stream", "onhip_plugin_forget", "onhip_plugin_release"]
+           "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_set_async", "onhip_plugin_set_stream", "onhip_plugin_forget", "onhip_plugin_trust_weights", "onhip_plugin_release"]
 
 
 def load():
@@ -109,6 +109,11 @@ def load():
     L.onhip_h16_to_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
     L.onhip_conv2d_h16.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, i32, vp, i32, vp]
     L.onhip_attention.argtypes = [C.POINTER(abi.AttentionDesc), vp, vp, vp, vp, vp]
+    L.onhip_dw_project_supported.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc)]
+    L.onhip_dw_project_packed_weight_bytes.argtypes = [i32, i32]
+    L.onhip_dw_project_packed_weight_bytes.restype = C.c_size_t
+    L.onhip_dw_project_pack_weights.argtypes = [vp, i32, i32, vp, vp]
+    L.onhip_dw_project_f32.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp]
     L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
@@ -512,6 +517,29 @@ def linear_h16(x, w_packed, k, n, compute, bias=None, gelu_lut=None, residual=No
             out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
     _check(load().onhip_linear_h16(rows, k, n, compute, _ptr(x), _ptr(w_packed), _ptr(bias), _ptr(gelu_lut), _ptr(residual),
                                    _ptr(out), y_kind, _stream()), "onhip_linear_h16")
+    return out
+
+
+def dw_project_supported(dw, pw):
+    return load().onhip_dw_project_supported(C.byref(dw), C.byref(pw))
+
+
+def dw_project_pack_weights(pw_w):
+    """1x1 weights [cout, cin(, 1, 1)] -> the k-major layout of the fused depthwise + 1x1 kernel"""
+    import torch
+    co, ce = pw_w.shape[0], pw_w.shape[1]
+    out = torch.empty(load().onhip_dw_project_packed_weight_bytes(ce, co) // 4, dtype=torch.float32, device=pw_w.device)
+    _check(load().onhip_dw_project_pack_weights(_ptr(pw_w), ce, co, _ptr(out), _stream()), "onhip_dw_project_pack_weights")
+    return out
+
+
+def dw_project_f32(dw, pw, x, dw_w, dw_b, pw_packed, pw_b=None, residual=None, out=None):
+    import torch
+    oh, ow = dw.out_hw()
+    if out is None:
+        out = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device=x.device)
+    _check(load().onhip_dw_project_f32(C.byref(dw), C.byref(pw), _ptr(x), _ptr(dw_w), _ptr(dw_b), _ptr(pw_packed), _ptr(pw_b),
+                                       _ptr(residual), _ptr(out), _stream()), "onhip_dw_project_f32")
     return out
 
 

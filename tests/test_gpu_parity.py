@@ -699,6 +699,24 @@ def test_plugin_conv_eval_host_buffers(name, torch_dev, golden):
     cases.check_against(golden, name, y, exact=exact, rtol=1e-4, atol=atol)
 
 
+def test_plugin_conv_eval_sees_a_weight_changed_in_place(torch_dev, oracle):
+    """the device copy of host weights is checked against all of the host buffer on every call: one weight changed in
+    place, at a position a sparse sample of the buffer would skip, must show in the next result"""
+    d = cases.conv_f32_cases()["cfg1_64x56_3x3"]
+    x, w, b = cases.conv_inputs("plugin_inplace", d)
+    op = ops.Conv(ops.Plugin(hip.plugin_path("Conv")).eval, d, w, b)
+    y0 = op(x).copy()
+    flat = op.weight.reshape(-1)
+    assert flat.size // 2 > 4096                      # large enough for a 4096-word sample to have gaps
+    flat[3] += np.float32(0.75)                       # word 1 of the buffer: between two sampled words
+    y1 = op(x).copy()
+    w2 = w.copy()
+    w2.reshape(-1)[3] += np.float32(0.75)
+    ref = oracle.conv2d_f32(d, x, w2, b)
+    assert not np.array_equal(y0, y1), "the stale device copy of the weights was used"
+    assert_close_f32(y1, ref, tag="weights changed in place")
+
+
 @pytest.mark.parametrize("name", ["q3x3_silu", "q3x3_nobias", "qdw3x3_s2", "q3x3_bigacc", "yolo_sppf_1x1_1024"])
 def test_plugin_conv_eval_w8a32(name, torch_dev, golden):
     d = cases.conv_w8a32_cases()[name]
