@@ -659,6 +659,7 @@ static bool wants_packed(const onhip_conv_desc_t *d) {
 
 size_t onhip_conv2d_packed_weight_bytes(const onhip_conv_desc_t *d) {
     if (!d || d->cin < 1 || d->cout < 1 || d->kh < 1 || d->kw < 1 || !wants_packed(d)) return 0;
+    if (stem_f32_shape(*d)) return (size_t) ((d->kh * d->kw * 3 + 1) / 2 * 2) * 64 * sizeof(float);   // [reduction index][64]
     return (size_t) d->cout * d->kh * d->kw * packed_cp(d) * sizeof(float);
 }
 
@@ -668,6 +669,8 @@ int onhip_conv2d_pack_weights(const onhip_conv_desc_t *d, const float *w, float 
     if (rc) return rc;
     if (!w || !packed) return set_error(ONHIP_ERR_ARG, "conv pack: null pointer");
     if (!wants_packed(d)) return set_error(ONHIP_ERR_ARG, "conv pack: this convolution takes its weights as they are");
+    // a first-layer convolution (three input channels): the layout of the kernel that runs it, whatever the image size
+    if (stem_f32_shape(*d)) return stem_pack_launch(*d, w, packed, reinterpret_cast<hipStream_t>(stream));
     return pack_wf32_launch(w, d->cout, d->cin, d->kh * d->kw, packed_cp(d), packed, reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -702,6 +705,15 @@ static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const flo
         if (!rc && addend) rc = add_relu_in_place(d, OH, OW, addend, relu_after, y, stream);
         return rc;
     }
+    // First-layer convolutions: packed weights have that kernel's layout, so it runs them whatever the image size (and
+    // the Add of a residual block, which no first layer has, as a pass of its own); weights as given only where rows of
+    // 96 pixels and more fill its workgroups.
+    if (stem_f32_ok(*d, OH, OW) && (packed || (OW >= 96 && !addend))) {
+        rc = stem_f32_launch(*d, OH, OW, x, w, packed, bias, ep, y, st);
+        if (!rc && addend) rc = add_relu_in_place(d, OH, OW, addend, relu_after, y, stream);
+        return rc;
+    }
+    if (packed && stem_f32_shape(*d)) return set_error(ONHIP_ERR_ARG, "conv: first-layer tensors of 2^29 elements or more are not supported with packed weights");
     IgemmLaunch cfg;
     memset(&cfg, 0, sizeof(cfg));
     rc = dtype_of_compute(d->compute, &cfg.dtype);

@@ -249,6 +249,12 @@ int dwproj_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int co);
 int dwproj_f32_launch(const onhip_conv_desc_t &dw, const onhip_conv_desc_t &pw, int OH, int OW, const float *x, const float *dw_w,
                       const float *dw_b, const float *pw_t, const float *pw_b, const float *res, const Epilogue &dw_ep,
                       const Epilogue &pw_ep, float *y, hipStream_t stream);
+// stem.hip: first-layer convolutions (three input channels) from an LDS patch
+bool stem_f32_shape(const onhip_conv_desc_t &d);
+bool stem_f32_ok(const onhip_conv_desc_t &d, int OH, int OW);
+int stem_pack_launch(const onhip_conv_desc_t &d, const float *w, float *packed, hipStream_t stream);
+int stem_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const float *w, int packed, const float *bias,
+                    const Epilogue &ep, float *y, hipStream_t stream);
 // attention.hip
 int attention_f32_launch(const onhip_attention_desc_t &d, const float *q, const float *k, const float *v, float *out,
                          hipStream_t stream);

@@ -481,6 +481,28 @@ def test_conv_w8a32_batched(torch_dev, oracle):
     assert np.array_equal(y.cpu().numpy(), oracle.conv2d_w8a32(d, x, w8, b32, aux, cases.silu_lut()))
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 7, 2, 3, 224, 224, abi.RELU, 1), (1, 32, 3, 2, 1, 224, 224, abi.CLIP, 1),
+                                   (1, 40, 3, 1, 1, 20, 200, abi.RELU, 1), (1, 8, 7, 1, 3, 9, 130, abi.NOT_ACT, 1),
+                                   (2, 33, 3, 2, 1, 37, 300, abi.LEAKYRELU, 1), (1, 64, 7, 2, 3, 64, 260, abi.RELU, 0)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_conv_f32_first_layer_kernel(shape, packed, torch_dev, oracle):
+    """three input channels, rows of at least 96 output pixels: the kernel that multiplies out of an LDS patch of the
+    input (one and several 128-pixel segments per row, ragged last segment, both filter sizes, both strides, with and
+    without bias, weights as given and tap-major packed); 1e-4 against the oracle like every fp32 convolution"""
+    torch = torch_dev
+    n, cout, k, stride, pad, h, w, act, bias = shape
+    d = cases.cd(3, cout, k, stride, pad, h, w=w, n=n, act=act, bias=bias, clip_min=0.0, clip_max=0.8, leaky_relu_alpha=0.1)
+    name = f"stem_{cout}_{k}_{stride}_{h}x{w}"
+    x, wt, b = cases.conv_inputs(name, d)
+    wd = dev(torch, wt)
+    if packed:
+        y = hip.conv2d_f32(d, dev(torch, x), hip.pack_conv_weights(d, wd), dev(torch, b), packed=True)
+    else:
+        y = hip.conv2d_f32(d, dev(torch, x), wd, dev(torch, b))
+    torch.cuda.synchronize()
+    assert_close_f32(y.cpu().numpy(), oracle.conv2d_f32(d, x, wt, b), tag=name)
+
+
 @pytest.mark.parametrize("compute,name", [(abi.COMPUTE_BF16, "cfg1_64x56_3x3"), (abi.COMPUTE_F16, "cfg1_64x56_3x3"),
                                           (abi.COMPUTE_BF16, "c7x7_s2_p3"), (abi.COMPUTE_F16, "c1x1_unaligned_clip")])
 def test_conv_reduced_precision_modes(compute, name, torch_dev, oracle):
