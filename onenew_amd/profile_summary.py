@@ -35,10 +35,12 @@ CLOCK_HZ = 2.4e9           # peak engine clock the MFMA peak is quoted at
 GLUE = ("add_kernel", "relu_kernel", "maxpool", "gap_kernel", "layernorm", "softmax", "transpose_kernel", "gelu_lut")
 LEGEND = ("Kernel names: `onhip::igemm_kernel<dtype, loader, BM, BN, WM, WN, PF, RES>` (dtype 0 fp32, 1 bf16, 2 f16, 3 int8; loader 0 "
           "gather, 1 int8 vectors, 2 plain, 3 tap-major packed, 4 int8 vectors with scalar taps; PF register sets of tiles in flight; "
-          "RES the variant whose store adds a residual operand), `onhip::igemm_dma_i8_kernel<BM, BN, WM, WN, KS, NST>` (int8, operand "
-          "tiles loaded straight into LDS, KS bytes of K per stage, ring of NST stages), `onhip::rowb_f32_kernel<WM, WN>` (fp32, B "
+          "RES the variant whose store adds a residual operand), `onhip::igemm_dma_kernel<dtype, BM, BN, WM, WN, KS, NST>` (int8 and "
+          "16-bit storage: operand tiles loaded straight into LDS, KS bytes of K per stage, ring of NST stages), `onhip::rowb_f32_kernel<WM, WN>` (fp32, B "
           "straight from memory, tile 32 WM x 128 WN), `onhip::splitk_finish_kernel`, `onhip::depthwise_tiled_kernel<int8, stride, "
-          "act>`, `onhip::quantize_nhwc_kernel<CBW>`, and the element-wise kernels.")
+          "act>`, `onhip::quantize_nhwc_kernel<CBW>`, `onhip::stem_f32_kernel<filter size, act, two row tiles>` (first-layer "
+          "convolutions from an LDS patch), `onhip::attention_f32_kernel<key tiles, head dim>`, `onhip::dwproj_f32_kernel<act, row "
+          "tiles, vector width>` (depthwise 3x3 + 1x1 in one launch), and the element-wise kernels.")
 
 
 def short(name):
@@ -48,9 +50,9 @@ def short(name):
 
 
 def family(name):
-    if "igemm" in name or "splitk_finish" in name or "rowb_f32" in name or "attention" in name:
+    if "igemm" in name or "splitk_finish" in name or "rowb_f32" in name or "attention" in name or "stem_f32" in name:
         return "igemm"
-    if "depthwise" in name:
+    if "depthwise" in name or "dwproj" in name:
         return "depthwise"
     if "quantize_nhwc" in name:
         return "quantize"
