@@ -708,7 +708,8 @@ static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const flo
     // First-layer convolutions: packed weights have that kernel's layout, so it runs them whatever the image size (and
     // the Add of a residual block, which no first layer has, as a pass of its own); weights as given only where rows of
     // 96 pixels and more fill its workgroups.
-    if (stem_f32_ok(*d, OH, OW) && (packed || (OW >= 96 && !addend))) {
+    static const bool no_stem = getenv("ONHIP_NO_STEM") != nullptr;   // tuning hook: unpacked weights on the implicit-GEMM kernels
+    if (stem_f32_ok(*d, OH, OW) && (packed || (OW >= 96 && !addend && !no_stem))) {
         rc = stem_f32_launch(*d, OH, OW, x, w, packed, bias, ep, y, st);
         if (!rc && addend) rc = add_relu_in_place(d, OH, OW, addend, relu_after, y, stream);
         return rc;
