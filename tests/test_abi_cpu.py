@@ -58,8 +58,12 @@ def test_errors_without_gpu_are_codes_not_crashes():
     assert lib.onhip_conv_out_shape(C.byref(d), C.byref(oh), C.byref(ow)) == 0 and (oh.value, ow.value) == (8, 8)
     d.group, d.cout = 4, 8       # depthwise needs cin == cout
     assert lib.onhip_conv_out_shape(C.byref(d), C.byref(oh), C.byref(ow)) == -1
+    # tap-major [cout][taps][channels padded to 4] ...
+    assert lib.onhip_conv2d_packed_weight_bytes(C.byref(abi.ConvDesc(n=1, cin=5, h=8, w=8, cout=8, kh=7, kw=7, stride_h=2,
+                                                                      stride_w=2, group=1, has_bias=1))) == 8 * 49 * 8 * 4
+    # ... except a first layer (three input channels, 7x7 or 3x3): [3 * taps rounded up to even][64], the layout of its kernel
     assert lib.onhip_conv2d_packed_weight_bytes(C.byref(abi.ConvDesc(n=1, cin=3, h=8, w=8, cout=8, kh=7, kw=7, stride_h=2,
-                                                                      stride_w=2, group=1, has_bias=1))) == 8 * 49 * 4 * 4
+                                                                      stride_w=2, group=1, has_bias=1))) == 148 * 64 * 4
     one = abi.ConvDesc(n=1, cin=8, h=8, w=8, cout=8, kh=1, kw=1, stride_h=1, stride_w=1, group=1, has_bias=1)
     assert lib.onhip_conv2d_packed_weight_bytes(C.byref(one)) == 0
     assert lib.onhip_conv_eval(None, None, None) == -1
