@@ -372,18 +372,21 @@ class AttentionLayer:
     the qkv projection's output and the context written with the heads merged; counted as the two MatMuls it replaces"""
     kind = "attention"
 
-    def __init__(self, torch, hip, name, md_scores, md_context, heads, tag):
+    def __init__(self, torch, hip, name, md_scores, md_context, heads, tag, dtype=None):
         from onenew_amd import datagen
         self.name = name
         bh, t, hd = md_scores.batch, md_scores.m, md_scores.k
         b = bh // heads
         self.qkv = device_uniform(torch, datagen.seed_for(tag, name, "qkv"), (b, t, 3, heads, hd), -1.5, 1.5)
+        if dtype is not None:   # 16-bit storage: q, k, v slices of a 16-bit projection output, 16-bit result
+            self.qkv = self.qkv.to(dtype)
         self.q, self.k, self.v = (self.qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         self.scale = 1.0 / float(np.sqrt(hd))
-        self.y = torch.empty((b, t, heads * hd), dtype=torch.float32, device="cuda")
+        self.y = torch.empty((b, t, heads * hd), dtype=self.qkv.dtype, device="cuda")
         self.mds = (md_scores, md_context)
         self.flops = md_scores.flops() + md_context.flops()
-        self.bytes = md_scores.algorithmic_bytes() + md_context.algorithmic_bytes()   # of the unfused chain's two MatMuls
+        eb = 4 if dtype is None else 2
+        self.bytes = md_scores.algorithmic_bytes(eb=eb) + md_context.algorithmic_bytes(eb=eb)   # of the unfused chain's two MatMuls
         self.dense = True
         self.shape = f"B={b} H={heads} T={t} D={hd}"
 
@@ -533,12 +536,17 @@ def make_workload(torch, hip, name):
             compute, dtype, rest = abi.COMPUTE_F16, "f16", rest[:-4]
         n = int(rest)
         if compute != abi.COMPUTE_F32:
-            # 16-bit storage for the four linear layers; the two attention products (per head, both operands activations)
-            # keep fp32 storage with operands rounded on the way into LDS
-            layers = [LinearH16Layer(torch, hip, ln, md, hb, g, compute, tag) if md.b_shared else
-                      MatmulLayer(torch, hip, ln, md, hb, g, compute, tag) for ln, md, hb, g in stacks.vit_tiny(n)]
-            return (f"ViT-Tiny block MatMuls {dtype}, batch {n}, 197 tokens x 192, 3 heads: qkv / proj / fc1 (fused bias + table "
-                    f"GELU) / fc2 with 16-bit storage, scores and context with fp32 storage", dtype, layers)
+            # 16-bit storage throughout: the four linear layers and the attention between them
+            tdt = torch.bfloat16 if compute == abi.COMPUTE_BF16 else torch.float16
+            spec = {ln: md for ln, md, _, _ in stacks.vit_tiny(n)}
+            layers = []
+            for ln, md, hb, g in stacks.vit_tiny(n):
+                if ln == "scores":
+                    layers.append(AttentionLayer(torch, hip, "attention", md, spec["context"], 3, tag, dtype=tdt))
+                elif ln != "context":
+                    layers.append(LinearH16Layer(torch, hip, ln, md, hb, g, compute, tag))
+            return (f"ViT-Tiny block MatMuls {dtype} with 16-bit storage, batch {n}, 197 tokens x 192, 3 heads: qkv, attention "
+                    f"(scores, Softmax and context in one launch), proj, fc1 (fused bias + table GELU), fc2", dtype, layers)
         spec = {ln: (md, hb, g) for ln, md, hb, g in stacks.vit_tiny(n)}
         layers = []
         for ln, md, hb, g in stacks.vit_tiny(n):

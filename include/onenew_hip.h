@@ -266,15 +266,18 @@ int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *p
  * that split q, k, v into heads, transpose k and merge the heads again: every operand is addressed through the element
  * strides of (batch, head, token), the head dimension being contiguous, so q, k and v may be slices of one projection
  * output [batch][tokens][3 * heads * head_dim] and out the merged [batch][tokens][heads * head_dim].  The scores stay in
- * registers.  head_dim 32 or 64, at most 256 tokens, rows 16-byte aligned (strides multiples of 4); other shapes are
- * refused and stay with the separate operators.  compute: ONHIP_COMPUTE_F32. */
+ * registers.  compute ONHIP_COMPUTE_F32: fp32 tensors, head_dim 32 or 64.  ONHIP_COMPUTE_BF16 / _F16: q, k, v and out
+ * are tensors of that 16-bit type (e.g. slices of a 16-bit projection output), head_dim 64; products on the 16-bit
+ * matrix-core instructions with fp32 accumulation, scores and Softmax in fp32, the probabilities rounded to the operand
+ * type for the second product.  At most 256 tokens, rows 16-byte aligned (strides multiples of a 16-byte vector); other
+ * shapes are refused and stay with the separate operators. */
 typedef struct onhip_attention_desc {
     int32_t batch, heads, tokens, head_dim;
     long long q_strides[3], k_strides[3], v_strides[3], out_strides[3];
     float scale;      /* 1.0f when the graph has no Mul between the first MatMul and the Softmax */
     int32_t compute;
 } onhip_attention_desc_t;
-int onhip_attention(const onhip_attention_desc_t *d, const float *q, const float *k, const float *v, float *out,
+int onhip_attention(const onhip_attention_desc_t *d, const void *q, const void *k, const void *v, void *out,
                     void *stream);
 
 /* out[m][n] = sum_k a[m][k] * w[n][k] + bias[n].  Replaces gemm.c eval (:9). */

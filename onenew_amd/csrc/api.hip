@@ -1275,22 +1275,32 @@ int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *p
                              make_epilogue(*pw, nullptr), y, reinterpret_cast<hipStream_t>(stream));
 }
 
-int onhip_attention(const onhip_attention_desc_t *d, const float *q, const float *k, const float *v, float *out, void *stream) {
+int onhip_attention(const onhip_attention_desc_t *d, const void *q, const void *k, const void *v, void *out, void *stream) {
     if (!d || d->batch < 1 || d->heads < 1 || d->tokens < 1) return set_error(ONHIP_ERR_ARG, "attention: bad shape");
     if (!q || !k || !v || !out) return set_error(ONHIP_ERR_ARG, "attention: null tensor pointer");
-    if (d->compute != ONHIP_COMPUTE_F32) return set_error(ONHIP_ERR_ARG, "attention: fp32 only");
-    if (d->head_dim != 32 && d->head_dim != 64) return set_error(ONHIP_ERR_ARG, "attention: head dimension %d (32 and 64 are fused)", d->head_dim);
+    const bool f32 = d->compute == ONHIP_COMPUTE_F32;
+    int dt = DT_F32;
+    if (!f32) {
+        const int rc = h16_dtype(d->compute, &dt);
+        if (rc) return rc;
+    }
+    if (d->head_dim != 64 && !(f32 && d->head_dim == 32))
+        return set_error(ONHIP_ERR_ARG, "attention: head dimension %d (fp32: 32 and 64 are fused, 16-bit: 64)", d->head_dim);
     if (d->tokens > 256) return set_error(ONHIP_ERR_ARG, "attention: %d tokens (at most 256 are fused)", d->tokens);
     if ((long long) d->batch * d->heads > 65535) return set_error(ONHIP_ERR_ARG, "attention: more than 65535 (batch, head) pairs");
     const long long *strides[4] = {d->q_strides, d->k_strides, d->v_strides, d->out_strides};
     const void *ptrs[4] = {q, k, v, out};
+    const int vec = f32 ? 4 : 8;   // elements of a 16-byte access
     for (int t = 0; t < 4; ++t) {
         if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return set_error(ONHIP_ERR_ARG, "attention: tensors must be 16-byte aligned");
         for (int i = 0; i < 3; ++i)
-            if (strides[t][i] < 0 || strides[t][i] % 4) return set_error(ONHIP_ERR_ARG, "attention: strides must be non-negative multiples of 4");
+            if (strides[t][i] < 0 || strides[t][i] % vec) return set_error(ONHIP_ERR_ARG, "attention: strides must be non-negative multiples of %d", vec);
         if (strides[t][2] < d->head_dim) return set_error(ONHIP_ERR_ARG, "attention: token stride below the head dimension");
     }
-    return attention_f32_launch(*d, q, k, v, out, reinterpret_cast<hipStream_t>(stream));
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (f32) return attention_f32_launch(*d, reinterpret_cast<const float *>(q), reinterpret_cast<const float *>(k),
+                                         reinterpret_cast<const float *>(v), reinterpret_cast<float *>(out), st);
+    return attention_h16_launch(dt, *d, q, k, v, out, st);
 }
 
 int onhip_copy_f32(const float *src, float *dst, long long n, void *stream) {

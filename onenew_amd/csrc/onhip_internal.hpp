@@ -258,6 +258,8 @@ int stem_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, 
 // attention.hip
 int attention_f32_launch(const onhip_attention_desc_t &d, const float *q, const float *k, const float *v, float *out,
                          hipStream_t stream);
+int attention_h16_launch(int dt, const onhip_attention_desc_t &d, const void *q, const void *k, const void *v, void *out,
+                         hipStream_t stream);
 // 16-bit storage (h16.hip): dt is DT_BF16 or DT_F16
 int pack_w16_launch(int dt, const float *w, long long rows, int cin, int taps, int cp, long long s_row, long long s_ch,
                     long long s_tap, void *packed, hipStream_t stream);

@@ -20,13 +20,12 @@
 namespace onhip {
 
 constexpr int ST_TW = 128;   // output pixels per workgroup
-constexpr int ST_MP = 68;    // floats per reduction index in the weight tile: rows 16-byte aligned, a transposing write two-way at worst
 
 struct StemParams {
     const float *x, *w, *bias;
     float *y;
     int n, h, w_in, oh, ow, cout, stride, pt, pl;
-    int packed;        // weights as stem_pack_kernel lays them out ([reduction index][64]) instead of [cout][3][k][k]
+    int packed;        // weights as stem_pack_kernel lays them out (the LDS image) instead of [cout][3][k][k]
     int segs;          // row segments of 128 pixels per output row
     int pw;            // patch columns: 127 * stride + k
     Div31 div_pw;
@@ -39,7 +38,9 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
     constexpr int ROWS = CIN * KS;                       // patch rows: (channel, filter row)
     constexpr int PATCH_MAX = ROWS * (127 * 2 + KS) + 8;   // strides up to 2 fit; larger strides are refused by the host
     __shared__ __attribute__((aligned(16))) float patch[PATCH_MAX];
-    __shared__ __attribute__((aligned(16))) float At[KP * ST_MP];
+    // weights in the order the matrix cores read them: [step][row tile][lane half][32 rows] (one conflict-free read per
+    // operand: the 64 lanes of a wavefront hit 64 different banks)
+    __shared__ __attribute__((aligned(16))) float At[KP * 64];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lh = lane >> 5;
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
     // Every load of a phase is issued before the first one is used (fixed trip counts, values held in registers): a loop
     // that loads and stores element by element would pay the memory latency once per element.
     // Weights -> At[k][m], k = tap * 3 + channel; the pad index and rows past cout are zero.  Packed weights
-    // (stem_pack_kernel) already have that layout, 64 output channels per reduction index: a straight 16-byte copy.
+    // (stem_pack_kernel) already are the LDS image: a straight 16-byte copy.
     {
         constexpr int W_PER_T = KP * 64 / 256, W4_PER_T = (KP * 64 / 4 + 255) / 256;
         static_assert(KP * 64 % 256 == 0, "whole passes over the weight tile");
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
 #pragma unroll
             for (int t = 0; t < W4_PER_T; ++t) {
                 const int f = tid + t * 256;
-                if (f < KP * 16) *reinterpret_cast<float4 *>(At + (f >> 4) * ST_MP + (f & 15) * 4) = wq[t];
+                if (f < KP * 16) reinterpret_cast<float4 *>(At)[f] = wq[t];
             }
         } else {
             float wv[W_PER_T];
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
             for (int t = 0; t < W_PER_T; ++t) {
                 const int f = tid + t * 256;
                 const int m = f / KP, k = f - m * KP;
-                At[k * ST_MP + m] = wv[t];
+                At[(((k >> 1) * 2 + (m >> 5)) * 2 + (k & 1)) * 32 + (m & 31)] = wv[t];
             }
         }
         if (tid < 8) patch[ROWS * pw + tid] = 0.0f;   // the pad index reads just past the last row
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
     const rsrc_t rb = make_rsrc(p.bias, p.bias ? (unsigned) (p.cout * 4) : 0u);
     const bool has_bias = p.bias != nullptr;
     const float *pb = patch + (wave * 32 + li) * p.stride;
-    const float *ab = At + lh * ST_MP + li;
+    const float *ab = At + lh * 32 + li;
 
     issue(item_begin);
     for (int item = item_begin; item < item_end; ++item) {
@@ -147,8 +148,8 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
             const int t0 = k0 / CIN, c0 = k0 % CIN, t1 = (k1 < K ? k1 : 0) / CIN, c1 = (k1 < K ? k1 : 0) % CIN;
             const int o0 = (c0 * KS + t0 / KS) * pw + t0 % KS, o1 = (c1 * KS + t1 / KS) * pw + t1 % KS;
             const float bv = pb[lh ? o1 : o0];   // index K (the pad) multiplies a zero weight
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[2 * s * ST_MP], bv, acc[0], 0, 0, 0);
-            if constexpr (TWO) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[2 * s * ST_MP + 32], bv, acc[1], 0, 0, 0);
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[s * 128], bv, acc[0], 0, 0, 0);
+            if constexpr (TWO) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[s * 128 + 64], bv, acc[1], 0, 0, 0);
         }
 
         // store: lane = pixel, rows 8 (r / 4) + 4 lh + r % 4 of each 32-channel tile
@@ -174,11 +175,12 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
     }
 }
 
-// weights [cout][3][k][k] -> [kp][64], reduction index tap * 3 + channel, zeros in the pad index and past cout
+// weights [cout][3][k][k] -> [step][row tile][lane half][32 rows] (kp * 64 floats), reduction index 2 * step + lane half =
+// tap * 3 + channel, row = 32 * tile + position; zeros in the pad index and past cout
 __global__ __launch_bounds__(256) void stem_pack_kernel(const float *w, int cout, int taps, int kp, float *packed) {
     const int f = blockIdx.x * 256 + threadIdx.x;
     if (f >= kp * 64) return;
-    const int k = f >> 6, m = f & 63;
+    const int k = (f >> 7) * 2 + ((f >> 5) & 1), m = ((f >> 6) & 1) * 32 + (f & 31);
     const int tap = k / 3, c = k - tap * 3;
     packed[f] = (m < cout && k < taps * 3) ? w[(m * 3 + c) * taps + tap] : 0.0f;
 }

@@ -546,18 +546,22 @@ def dw_project_f32(dw, pw, x, dw_w, dw_b, pw_packed, pw_b=None, residual=None, o
 def attention(q, k, v, scale=1.0, out=None, merged_out=True):
     """out = Softmax(q k^T * scale) v per (batch, head).  q, k, v: views [batch, heads, tokens, head_dim] of fp32 tensors in
     any (batch, head, token) stride order with a contiguous head dimension (e.g. slices of a [batch, tokens, 3, heads,
-    head_dim] projection output, permuted); the result is [batch, tokens, heads * head_dim] (heads merged) or, with
+    head_dim] projection output, permuted), fp32 or both operands and result in bfloat16 / float16; the result is [batch, tokens, heads * head_dim] (heads merged) or, with
     merged_out=False, [batch, heads, tokens, head_dim]"""
     import torch
     b, h, t, hd = q.shape
+    compute = {torch.float32: abi.COMPUTE_F32, torch.bfloat16: abi.COMPUTE_BF16, torch.float16: abi.COMPUTE_F16}[q.dtype]
     if out is None:
-        out = torch.empty((b, t, h * hd) if merged_out else (b, h, t, hd), dtype=torch.float32, device=q.device)
-    d = abi.AttentionDesc(batch=b, heads=h, tokens=t, head_dim=hd, scale=scale, compute=abi.COMPUTE_F32)
+        out = torch.empty((b, t, h * hd) if merged_out else (b, h, t, hd), dtype=q.dtype, device=q.device)
+    d = abi.AttentionDesc(batch=b, heads=h, tokens=t, head_dim=hd, scale=scale, compute=compute)
     for name, ten in (("q_strides", q), ("k_strides", k), ("v_strides", v)):
         if ten.stride(3) != 1:
             raise OnhipError("attention: the head dimension must be contiguous")
         setattr(d, name, (C.c_longlong * 3)(ten.stride(0), ten.stride(1), ten.stride(2)))
-    d.out_strides = (C.c_longlong * 3)(t * h * hd, hd, h * hd) if merged_out else (C.c_longlong * 3)(h * t * hd, t * hd, hd)
+    if out.dim() == 3 and merged_out:   # [b, t, pitch]: the merged layout, possibly with a channel pitch above heads * head_dim
+        d.out_strides = (C.c_longlong * 3)(out.stride(0), hd, out.stride(1))
+    else:
+        d.out_strides = (C.c_longlong * 3)(h * t * hd, t * hd, hd)
     _check(load().onhip_attention(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _stream()), "onhip_attention")
     return out
 

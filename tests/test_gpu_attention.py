@@ -53,6 +53,41 @@ def test_attention_equals_the_operator_chain(shape, torch_dev, oracle):
     assert torch.equal(out2.permute(0, 2, 1, 3).reshape(b, t, h * hd), out)
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+@pytest.mark.parametrize("shape", [(64, 3, 197, 64, 0.125), (2, 3, 197, 64, 0.125), (1, 2, 40, 64, 1.0), (3, 1, 256, 64, 0.125),
+                                   (1, 4, 129, 64, 0.25), (2, 2, 7, 64, 0.5)])
+def test_attention_with_16_bit_operands(shape, dtype, torch_dev, oracle):
+    """q, k, v and the result in bf16 / fp16: within 1e-2 of the oracle's fp32 operator chain on the same (rounded)
+    operands, and within one and a half units in the last place of the 16-bit type (normalised) of a float64 model of what
+    the kernel is specified to compute: exact scores and Softmax, probabilities rounded to the operand type, exact second
+    product, one rounding of the result"""
+    torch = torch_dev
+    b, h, t, hd, scale = shape
+    tdt = getattr(torch, dtype)
+    print(f"attention {dtype} {shape}", flush=True)
+    qkv = cases.datagen.normal(cases.datagen.seed_for("attn16", *shape[:4]), (b, t, 3, h, hd), 0.0, 1.0)
+    dev = torch.from_numpy(qkv).cuda().to(tdt)
+    rounded = dev.float().cpu().numpy()
+    q, k, v = (dev[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    out = hip.attention(q, k, v, scale=scale)
+    torch.cuda.synchronize()
+    assert out.dtype == tdt
+    got = out.float().cpu().numpy().astype(np.float64)
+    ref = oracle_chain(oracle, rounded, b, t, h, hd, scale).astype(np.float64)
+    top = np.abs(ref).max()
+    assert np.abs(got - ref).max() <= 1e-2 * top, f"{np.abs(got - ref).max():.3e} against {top:.3e}"
+    # the float64 model
+    x = rounded.astype(np.float64).transpose(0, 2, 3, 1, 4)                      # [b, 3, h, t, hd]
+    qq, kk, vv = x[:, 0], x[:, 1], x[:, 2]
+    sc = np.einsum("bhqd,bhkd->bhqk", qq, kk) * scale
+    pr = np.exp(sc - sc.max(-1, keepdims=True))
+    pr = pr / pr.sum(-1, keepdims=True)
+    pr16 = torch.from_numpy(pr).to(tdt).double().numpy()
+    model = np.einsum("bhqk,bhkd->bhqd", pr16, vv).transpose(0, 2, 1, 3).reshape(b, t, h * hd)
+    ulp = 2.0 ** -8 if dtype == "bfloat16" else 2.0 ** -11
+    assert np.abs(got - model).max() <= 1.5 * ulp * top + 1e-6, f"{np.abs(got - model).max():.3e} against {ulp * top:.3e}"
+
+
 def test_attention_rows_are_probabilities(torch_dev):
     """v = identity columns: the output is the Softmax itself; rows sum to one, and large scores do not overflow"""
     torch = torch_dev
