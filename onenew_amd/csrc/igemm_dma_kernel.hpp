@@ -15,8 +15,10 @@
 //     would wait for all of them (vmcnt(0)) before every read, which undoes the ring.  Waits are placed by hand:
 //     vmcnt((NST - 2) * loads per stage) before the one barrier of a stage, lgkmcnt per K step.
 //
-// Requirements (dma_ok): int8, K-vector loader, a whole number of stages per filter tap (channels padded to 16 a
-// multiple of KS), at most 64 taps, no split-K.  Everything else runs igemm_kernel.  The accumulator layout is that of
+// Requirements (dma_ok): K-vector loader, at most 64 taps, no split-K, and either a whole number of stages per filter tap
+// (channel pitch in bytes a multiple of KS) or, int8 only (MULTI), taps of 16 or 32 bytes: a 64-byte stage then holds
+// four or two taps, the tap is a per-lane quantity, and the last stage may reach past the end of K (the weights it reads
+// there meet activations that are zero).  Everything else runs igemm_kernel.  The accumulator layout is that of
 // igemm_kernel, and so are the epilogues (write_tile, write_tile_nhwc_s8): same bits.
 //
 // Replaces, like igemm_kernel's int8 variant: the int32 GEMM and de-quantisation of device/x86/Conv/conv.c:1024-1056.
@@ -49,13 +51,16 @@ __device__ __forceinline__ void wait_operands(i32x4 (&av)[TM], i32x4 (&bv)[TN]) 
 
 template <int KS> __device__ __forceinline__ int dma_swz(int row) { return KS == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
 
-template <int DT, int BM, int BN, int WM, int WN, int KS, int NST>
+template <int DT, int BM, int BN, int WM, int WN, int KS, int NST, bool MULTI = false>
 __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p) {
     // device pass only: the host pass cannot parse the inline assembly's register constraints, and a kernel whose body it
     // rejects gets no launch stub
 #if defined(__HIP_DEVICE_COMPILE__)
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     static_assert(DT == DT_I8 || DT == DT_BF16 || DT == DT_F16, "operand types stored as 16-byte vectors of K");
+    // MULTI: a filter tap is shorter than a stage (16 or 32 bytes of K: up to 16 or 32 int8 channels), so a 64-byte stage
+    // holds four or two taps and the tap is a per-lane quantity, a function of the unit the lane fetches
+    static_assert(!MULTI || (DT == DT_I8 && KS == 64), "several taps per stage: int8, 64-byte stages");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int SLOTS = KS / 16, KSTEPS = SLOTS / 2;
     constexpr int ROWS_PER_LOAD = 1024 / KS;
@@ -107,13 +112,14 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
     const char *a_base = reinterpret_cast<const char *>(p.A);
     const char *b_base = reinterpret_cast<const char *>(p.B) - (size_t) p.b_shift_bytes;
     const unsigned a_bytes = (unsigned) p.a_slice_bytes, b_bytes = (unsigned) (p.b_slice_bytes + p.b_shift_bytes);
-    const int k_stages = p.k_units / SLOTS;
-    const int stages_per_tap = p.units_per_tap / SLOTS;
+    const int k_stages = MULTI ? (p.k_units + SLOTS - 1) / SLOTS : p.k_units / SLOTS;   // MULTI: the last stage may be ragged
+    const int stages_per_tap = MULTI ? 1 : p.units_per_tap / SLOTS;
 
     // this lane's share of a wave-wide load: row lane / SLOTS of the load's rows, slot lane % SLOTS, which holds the
     // row's unit slot ^ swz(row)
     const int lrow = lane / SLOTS, lslot = lane % SLOTS;
     unsigned a_voff[A_LOADS], b_voff[B_LOADS], b_mask_lo[B_LOADS], b_mask_hi[B_LOADS];
+    unsigned b_tap_sub[MULTI ? B_LOADS : 1], b_within[MULTI ? B_LOADS : 1];   // MULTI: tap within the stage, byte offset within the tap
 #pragma unroll
     for (int t = 0; t < A_LOADS; ++t) {
         const int row = (wave * A_LOADS + t) * ROWS_PER_LOAD + lrow;
@@ -124,7 +130,14 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
     for (int t = 0; t < B_LOADS; ++t) {
         const int row = (wave * B_LOADS + t) * ROWS_PER_LOAD + lrow;
         const ColState c = make_col<BL_KVEC>(p, n0 + row);
-        b_voff[t] = c.pixoff == OOB ? OOB : c.pixoff + (unsigned) ((lslot ^ dma_swz<KS>(row)) * 16);
+        const int unit = lslot ^ dma_swz<KS>(row);
+        if constexpr (MULTI) {
+            b_voff[t] = c.pixoff;
+            b_tap_sub[t] = (unsigned) unit / (unsigned) p.units_per_tap;      // units_per_tap is 1 or 2
+            b_within[t] = ((unsigned) unit % (unsigned) p.units_per_tap) * 16u;
+        } else {
+            b_voff[t] = c.pixoff == OOB ? OOB : c.pixoff + (unsigned) (unit * 16);
+        }
         b_mask_lo[t] = c.mask_lo;
         b_mask_hi[t] = c.mask_hi;
     }
@@ -144,6 +157,19 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
         for (int t = 0; t < A_LOADS; ++t)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t) (base + (wave * A_LOADS + t) * 1024), 16, a_voff[t],
                                                      (unsigned) (kt * KS), 0, 0);
+        if constexpr (MULTI) {
+            const unsigned taps_per_stage = (unsigned) SLOTS / (unsigned) p.units_per_tap;
+#pragma unroll
+            for (int t = 0; t < B_LOADS; ++t) {
+                const unsigned tap = (unsigned) kt * taps_per_stage + b_tap_sub[t];
+                const unsigned ti = fast_div(tap, p.magic_kw, p.pass_kw), tj = tap - ti * (unsigned) p.kw;
+                const unsigned word = tap >= 32u ? b_mask_hi[t] : b_mask_lo[t];
+                const bool in = live && tap < (unsigned) p.khkw && ((word >> (tap & 31u)) & 1u) != 0u && b_voff[t] != OOB;
+                const unsigned voff = in ? b_voff[t] + (ti * (unsigned) p.W + tj) * (unsigned) p.pix_stride + b_within[t] : OOB;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t) (base + BM * KS + (wave * B_LOADS + t) * 1024), 16, voff, 0, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < B_LOADS; ++t) {
             // the tap's bit of the lane's validity mask as a bit field, the choice between the pixel and "outside" as bit
@@ -299,8 +325,12 @@ inline int dma_stage_bytes(const IgemmParams &p) {
     const int tap_bytes = p.units_per_tap * 16;
     return tap_bytes % 128 == 0 ? 128 : tap_bytes % 64 == 0 ? 64 : 0;
 }
+// int8 with 16 or 32 bytes of K per filter tap (up to 16 / 32 channels): 64-byte stages that hold four or two taps
+inline bool dma_multi_tap(int dtype, const IgemmParams &p) {
+    return dtype == DT_I8 && (p.units_per_tap == 1 || p.units_per_tap == 2) && p.khkw <= 64;
+}
 
-template <int DT, int BM, int BN, int KS, int NST>
+template <int DT, int BM, int BN, int KS, int NST, bool MULTI = false>
 int dma_launch_one(const IgemmParams &p_in, hipStream_t stream) {
     IgemmParams p = p_in;
     const int tiles_m = (p.M + BM - 1) / BM;
@@ -309,15 +339,26 @@ int dma_launch_one(const IgemmParams &p_in, hipStream_t stream) {
     p.div_ohw = make_div31((unsigned) (p.OHW > 0 ? p.OHW : 1));
     p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
     p.div_tiles_m = make_div31((unsigned) tiles_m);
-    hipLaunchKernelGGL((igemm_dma_kernel<DT, BM, BN, 2, 2, KS, NST>), dim3((unsigned) tiles), dim3(THREADS), 0, stream, p);
+    hipLaunchKernelGGL((igemm_dma_kernel<DT, BM, BN, 2, 2, KS, NST, MULTI>), dim3((unsigned) tiles), dim3(THREADS), 0, stream, p);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }
 
 template <int DT>
 int dma_launch_dt(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream) {
-    const int ks = dma_stage_bytes(p);
     const int key = cfg.bm * 1000 + cfg.bn;
+    if constexpr (DT == DT_I8) {
+        if (dma_multi_tap(DT, p)) {   // short taps: one ring length
+            switch (key) {
+                case 128128: return dma_launch_one<DT, 128, 128, 64, 3, true>(p, stream);
+                case 128064: return dma_launch_one<DT, 128, 64, 64, 4, true>(p, stream);
+                case 64128: return dma_launch_one<DT, 64, 128, 64, 4, true>(p, stream);
+                case 64064: return dma_launch_one<DT, 64, 64, 64, 4, true>(p, stream);
+            }
+            return set_error(ONHIP_ERR_ARG, "igemm: no direct-to-LDS kernel for tile %dx%d", cfg.bm, cfg.bn);
+        }
+    }
+    const int ks = dma_stage_bytes(p);
     // cfg.ring != 0: the long rings, more than 64 KiB of LDS for one workgroup (one or two workgroups per compute unit,
     // three to seven stages of loads in flight each); otherwise rings of at most 64 KiB
     if (ks == 128) {

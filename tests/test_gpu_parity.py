@@ -1143,13 +1143,16 @@ def test_conv_w8a8_nhwc_chain_form(name, tile, torch_dev, oracle, monkeypatch):
 
 @pytest.mark.parametrize("tile", ["128x128", "128x64", "64x128", "64x64"])
 @pytest.mark.parametrize("shape", [(2, 64, 19, 72, 3, 1, 1), (1, 128, 23, 200, 3, 2, 1), (3, 192, 9, 130, 1, 1, 0), (2, 128, 12, 64, 5, 1, 2),
-                                   (1, 256, 7, 33, 3, 1, 1), (2, 64, 16, 128, 1, 2, 0)])
+                                   (1, 256, 7, 33, 3, 1, 1), (2, 64, 16, 128, 1, 2, 0),
+                                   # fewer than 64 channels: stages that hold several filter taps, ragged last stage
+                                   (2, 3, 30, 40, 3, 2, 1), (1, 32, 21, 64, 3, 1, 1), (2, 16, 17, 72, 5, 1, 2), (1, 32, 16, 100, 1, 1, 0),
+                                   (1, 8, 12, 33, 7, 2, 3), (1, 20, 9, 130, 3, 1, 1)])
 @pytest.mark.parametrize("act", [abi.SILU, abi.RELU, abi.NOT_ACT])
 @pytest.mark.parametrize("ring", [1, 2])
 def test_conv_int8_direct_to_lds_kernel_every_tile(ring, tile, shape, act, torch_dev, oracle, monkeypatch):
     """the int8 kernel that loads its tiles from global memory straight into LDS, every tile it has, on shapes with ragged
-    rows and columns, strides, padding, 64- and 128-byte stages (channels a multiple of 64 / of 128), one and many taps,
-    a single stage and many: int8 NHWC chain form and the fp32 / int32-accumulator form, both equal to the oracle"""
+    rows and columns, strides, padding, 64- and 128-byte stages (channels a multiple of 64 / of 128) and 64-byte stages of
+    two or four short taps (up to 32 / 16 channels), one and many taps, a single stage and many: int8 NHWC chain form and the fp32 / int32-accumulator form, both equal to the oracle"""
     torch = torch_dev
     n, cin, hw, cout, k, stride, pad = shape
     monkeypatch.setenv("ONHIP_TILE", tile + f"x1x0x0x0x{ring}")   # ring 2: the long ring of stage buffers (more than 64 KiB of LDS)
