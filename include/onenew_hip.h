@@ -405,6 +405,11 @@ int onhip_layernorm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_IN
 int onhip_softmax_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_attention` of libMatMul_hip.so: MatMul(q, Transpose(k)) -> Softmax (last axis) -> MatMul(., v) in one call
+ * (onhip_attention with scale 1).  params[1..3] / inputs[0..2]: q, k (before its Transpose), v, all
+ * [..., tokens, head_dim]; params[4] / outputs[0]: the result.  No counterpart in the reference, whose host runs the four
+ * operators one after the other (mat_mul.c, transpose.c, softmax.c). */
+int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /*
  * No counterpart in the reference, whose operators always finish before eval returns (device/cuda/MaxPool/
  * maxpool.cu:76).  on != 0: an eval whose output is device memory returns as soon as its kernels are queued on

@@ -96,6 +96,16 @@ int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int32_t *n_re
 int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n);
 
 /*
+ * Attention blocks: MatMul(q, Transpose(k)) -> Softmax (last axis) -> MatMul(., v), where nothing else reads the operands
+ * in between, run as one call of the MatMul plugin's `eval_attention` (libMatMul_hip.so; the scores stay on the chip, the
+ * transposed k is never written) when q, k and v are [..., tokens, head_dim] with head_dim 32 or 64 and at most 256
+ * tokens.  The reference's host runs the four operators one after the other (host/net.h:613-618); its optimiser has
+ * no such pattern (tools/optimize/op_fusion.hpp:477-591).  The operands folded away have no buffer
+ * (onrt_net_operand gives a null pointer for them).  ONENEW_RT_FUSE=0 keeps the operators separate.  n: how many blocks.
+ */
+int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n);
+
+/*
  * One inference as a HIP graph, on request: with ONENEW_RT_GRAPH=1 in the environment at load time.  The operators
  * of a net are the same launches with the same addresses on every run, so the second call of onrt_net_run records
  * them (stream capture on a stream the net owns; the first call has packed the weights, sized the workspaces and

@@ -399,6 +399,50 @@ static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFF
     return ONHIP_OK;
 }
 
+// MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v) as one call.  Slots: params[1..3] the operands q, k, v (all
+// [..., tokens, head_dim], k NOT transposed), params[4] the result [..., tokens, head_dim]; inputs[0..2], outputs[0] the
+// tensors (host or device memory like every eval).  Leading dimensions are (batch, head) pairs.
+static int matmul_attention_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const OPERAND_S *t[4];
+    for (int i = 0; i < 4; ++i) {
+        t[i] = reinterpret_cast<const OPERAND_S *>(params[1 + i].addr);
+        if (!t[i]) return set_error(ONHIP_ERR_ARG, "attention eval: empty params slot %d", 1 + i);
+    }
+    const int nd = t[0]->dim_num_of_shapes;
+    if (nd < 2 || nd > SHAPE_LEN) return set_error(ONHIP_ERR_ARG, "attention eval: rank %d", nd);
+    for (int i = 1; i < 4; ++i)
+        if (t[i]->dim_num_of_shapes != nd || memcmp(t[i]->shapes, t[0]->shapes, nd * sizeof(t[0]->shapes[0])))
+            return set_error(ONHIP_ERR_ARG, "attention eval: q, k, v and the result must have one shape");
+    onhip_attention_desc_t d;
+    memset(&d, 0, sizeof(d));
+    d.batch = 1;
+    for (int i = 0; i < nd - 2; ++i) d.batch *= t[0]->shapes[i];
+    d.heads = 1;
+    d.tokens = t[0]->shapes[nd - 2];
+    d.head_dim = t[0]->shapes[nd - 1];
+    d.scale = 1.0f;
+    d.compute = ONHIP_COMPUTE_F32;
+    const long long plane = (long long) d.tokens * d.head_dim;
+    for (long long *st : {d.q_strides, d.k_strides, d.v_strides, d.out_strides}) { st[0] = plane; st[1] = plane; st[2] = d.head_dim; }
+    const size_t bytes = (size_t) d.batch * plane * 4;
+    const void *in[3];
+    for (int i = 0; i < 3; ++i) {
+        if (!inputs[i].addr) return set_error(ONHIP_ERR_ARG, "attention eval: empty input slot %d", i);
+        const int rc = input_on_device(i, reinterpret_cast<const void *>(inputs[i].addr), bytes, &in[i]);
+        if (rc) return rc;
+    }
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        const int rc = stage_buf(2, bytes, &y);
+        if (rc) return rc;
+    }
+    const int rc = onhip_attention(&d, in[0], in[1], in[2], y, g_stream);
+    if (rc) return rc;
+    return out_on_dev ? wait_for_output() : copy_out(host_out, y, bytes);
+}
+
 static int gemm_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     const OPERAND_S *a_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
     const OPERAND_S *o_t = reinterpret_cast<const OPERAND_S *>(params[4].addr);
@@ -712,6 +756,9 @@ int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFE
 
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MatMul", matmul_eval_locked, params, inputs, outputs);
+}
+int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MatMul (attention)", matmul_attention_eval_locked, params, inputs, outputs);
 }
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Gemm", gemm_eval_locked, params, inputs, outputs);

@@ -6,3 +6,12 @@ extern "C" __attribute__((visibility("default"))) int eval(BUFFER_INFO_S *params
                                                            BUFFER_INFO_S *outputs) {
     return onhip_matmul_eval(params, inputs, outputs);
 }
+
+// Not in the reference: MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v) of an attention block as one call.  Slots:
+// params[1..3] / inputs[0..2] = q, k (as it is before its Transpose), v, all [..., tokens, head_dim]; params[4] /
+// outputs[0] = the result.  The device-resident runtime calls it when a model has that pattern and the shape is one the
+// fused kernel takes (head_dim 32 or 64, at most 256 tokens).
+extern "C" __attribute__((visibility("default"))) int eval_attention(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                     BUFFER_INFO_S *outputs) {
+    return onhip_matmul_attention_eval(params, inputs, outputs);
+}

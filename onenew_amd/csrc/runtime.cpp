@@ -118,6 +118,7 @@ struct Tensor {
     bool is_init = false;
     bool produced = false;   // an io input, an initialiser or the output of an operator already ordered
     std::string alias;       // an operand folded away with its producer reads as this one (fuse_residual_blocks)
+    bool never_written = false;   // an operand inside a fused attention block: it has no buffer and no value
 };
 
 struct Node {
@@ -161,7 +162,8 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    int fused_blocks = 0, folded_relus = 0, folded_acts = 0;
+    onenew_eval_fn matmul_attention = nullptr;                    // optional entry point of the MatMul plugin
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -419,7 +421,7 @@ int allocate(onrt_net &net) {
     // operands: fp32 elements (elem_size * sizeof(float) in the reference), views excepted
     for (auto &kv : net.tensors) {
         Tensor &t = kv.second;
-        if (t.is_init || t.desc.not_need_buf || !t.alias.empty()) continue;
+        if (t.is_init || t.desc.not_need_buf || !t.alias.empty() || t.never_written) continue;
         t.bytes = (size_t) numel(t.desc) * 4;
         act_total += (t.bytes + 255) & ~(size_t) 255;
     }
@@ -428,7 +430,7 @@ int allocate(onrt_net &net) {
         size_t off = 0;
         for (auto &kv : net.tensors) {
             Tensor &t = kv.second;
-            if (t.is_init || t.desc.not_need_buf || !t.alias.empty()) continue;
+            if (t.is_init || t.desc.not_need_buf || !t.alias.empty() || t.never_written) continue;
             t.dev = static_cast<char *>(net.act_arena) + off;
             off += (t.bytes + 255) & ~(size_t) 255;
         }
@@ -515,6 +517,7 @@ int bind_plugins(onrt_net &net) {
             net.conv_add = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add"));
             net.conv_add_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add_relu"));
         }
+        if (type == "MatMul") net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
     }
     return ONRT_OK;
 }
@@ -691,6 +694,76 @@ int fuse_residual_blocks(onrt_net &net) {
     return ONRT_OK;
 }
 
+// ---- attention ------------------------------------------------------------------------------------------
+// MatMul(q, Transpose(k)) -> Softmax (last axis) -> MatMul(., v), with nothing else reading the operands in between,
+// becomes one call of the MatMul plugin's `eval_attention` on q, k (as it is before the Transpose) and v: the scores
+// stay on the chip and the Transpose of k is never materialised.  Only for the shapes the fused kernel takes (q, k, v
+// all [..., tokens, head_dim] with head_dim 32 or 64 and at most 256 tokens); every other attention block keeps its four
+// operators (device/x86/MatMul/mat_mul.c, Transpose/transpose.c, Softmax/softmax.c).  The fused call takes the place of
+// the second MatMul in the order, where q, k and v are all complete.  ONENEW_RT_FUSE=0 keeps every operator separate.
+int fuse_attention(onrt_net &net) {
+    if (!fusing_enabled() || !net.matmul_attention) return ONRT_OK;
+    auto producer_of = [&](const std::string &name) {
+        for (int idx : net.order)
+            for (const std::string &o : net.nodes[idx].out)
+                if (o == name) return idx;
+        return -1;
+    };
+    std::map<int, int> runs_instead;   // second MatMul -> the first one, which takes its place
+    std::vector<bool> dropped(net.nodes.size(), false);
+    for (int idx : net.order) {
+        Node &m1 = net.nodes[idx];
+        if (strcmp(m1.kind->type, "MatMul") || m1.in.size() != 2 || m1.out.size() != 1 || m1.fuse) continue;
+        // the second operand comes from a Transpose of the last two axes that nothing else reads
+        const int ti = producer_of(m1.in[1]);
+        if (ti < 0 || strcmp(net.nodes[ti].kind->type, "Transpose") || sole_reader(net, m1.in[1], "MatMul") != idx) continue;
+        const Node &tr = net.nodes[ti];
+        const TRANSPOSE_CONFIG_S *tc = reinterpret_cast<const TRANSPOSE_CONFIG_S *>(tr.cfg.data());
+        const std::string &q = m1.in[0], &k = tr.in[0];
+        const Tensor &qt = net.tensors[q], &kt = net.tensors[k];
+        const int nd = qt.desc.dim_num_of_shapes;
+        if (nd < 2 || tc->perm_num != nd || kt.desc.dim_num_of_shapes != nd || qt.is_init || kt.is_init) continue;
+        bool swap_last = tc->perm[nd - 1] == nd - 2 && tc->perm[nd - 2] == nd - 1;
+        for (int i = 0; i < nd - 2; ++i) swap_last = swap_last && tc->perm[i] == i;
+        if (!swap_last || memcmp(qt.desc.shapes, kt.desc.shapes, nd * sizeof(qt.desc.shapes[0]))) continue;
+        const int tokens = qt.desc.shapes[nd - 2], head_dim = qt.desc.shapes[nd - 1];
+        if ((head_dim != 32 && head_dim != 64) || tokens > 256) continue;
+        long long pairs = 1;
+        for (int i = 0; i < nd - 2; ++i) pairs *= qt.desc.shapes[i];
+        if (pairs > 65535) continue;
+        // scores -> Softmax over the keys -> second MatMul with v
+        const int si = sole_reader(net, m1.out[0], "Softmax");
+        if (si < 0 || net.nodes[si].in.size() != 1 || net.nodes[si].out.size() != 1) continue;
+        const SOFTMAX_CONFIG_S *sc = reinterpret_cast<const SOFTMAX_CONFIG_S *>(net.nodes[si].cfg.data());
+        if (sc->axis != -1 && sc->axis != nd - 1) continue;
+        const int m2i = sole_reader(net, net.nodes[si].out[0], "MatMul");
+        if (m2i < 0 || runs_instead.count(m2i)) continue;
+        Node &m2 = net.nodes[m2i];
+        if (m2.in.size() != 2 || m2.out.size() != 1 || m2.in[0] != net.nodes[si].out[0] || m2.in[1] == m2.in[0]) continue;
+        const Tensor &vt = net.tensors[m2.in[1]], &ot = net.tensors[m2.out[0]];
+        if (vt.is_init || vt.desc.dim_num_of_shapes != nd || ot.desc.dim_num_of_shapes != nd ||
+            memcmp(vt.desc.shapes, qt.desc.shapes, nd * sizeof(qt.desc.shapes[0])) ||
+            memcmp(ot.desc.shapes, qt.desc.shapes, nd * sizeof(qt.desc.shapes[0])))
+            continue;
+        m1.fuse = 3;
+        m1.in = {q, k, m2.in[1]};
+        m1.fused_out = m2.out[0];
+        m1.eval = net.matmul_attention;
+        for (const std::string &gone : {tr.out[0], m1.out[0], net.nodes[si].out[0]}) net.tensors[gone].never_written = true;
+        dropped[ti] = dropped[idx] = dropped[si] = true;
+        runs_instead[m2i] = idx;
+        ++net.fused_attentions;
+    }
+    std::vector<int> order;
+    for (int idx : net.order) {
+        auto it = runs_instead.find(idx);
+        if (it != runs_instead.end()) order.push_back(it->second);
+        else if (!dropped[idx]) order.push_back(idx);
+    }
+    net.order.swap(order);
+    return ONRT_OK;
+}
+
 // ---- slot arrays (op::rt_prepare, host/op.h:109-168, and prepare_init_operand_data of each operator) ----
 int fill_slots(onrt_net &net) {
     const size_t lut_len = net.silu_lut.size();
@@ -708,7 +781,7 @@ int fill_slots(onrt_net &net) {
             nd.params[1 + slot].addr = (int64_t) &t.desc;
             nd.inputs[slot].addr = (int64_t) t.dev;
         }
-        if (nd.fuse) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
+        if (nd.fuse == 1 || nd.fuse == 2) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
             Tensor &t = net.tensors[nd.fused_out.empty() ? nd.out[k] : nd.fused_out];
@@ -736,6 +809,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = bind_plugins(net);
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
+    if (!rc) rc = fuse_attention(net);
     if (!rc) rc = allocate(net);
     if (!rc) rc = build_tables(net);
     if (!rc) rc = fill_slots(net);
@@ -756,9 +830,10 @@ int plan(onrt_net &net) {
     int rc = read_model(net);
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
-    net.conv_add = net.conv_add_relu = plan_stub_eval;   // as with the Conv plugin of this package
+    net.conv_add = net.conv_add_relu = net.matmul_attention = plan_stub_eval;   // as with the plugins of this package
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
+    if (!rc) rc = fuse_attention(net);
     return rc;
 }
 
@@ -944,6 +1019,12 @@ static void forget_graph(onrt_net &net) {
 ONRT_API int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n) {
     if (!net || !n) return fail(ONRT_ERR_ARG, "folded activations: null argument");
     *n = (int32_t) net->folded_acts;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "fused attentions: null argument");
+    *n = (int32_t) net->fused_attentions;
     return ONRT_OK;
 }
 

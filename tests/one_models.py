@@ -98,6 +98,23 @@ def quantised_block():
     return m.tobytes(), [_r("xq", (1, 16, 18, 18))]
 
 
+def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output=False):
+    """q, k, v as three inputs [batch, heads, tokens, head_dim]: Transpose of k, MatMul, Softmax, MatMul, the pattern the
+    runtime runs as one attention call (unless the scores are also a net output)"""
+    m = onefile.OneModel()
+    shape = (batch, heads, tokens, head_dim)
+    for n in ("q", "k", "v"):
+        m.input(n, shape)
+    m.transpose("kt", "k", "k_t", (0, 1, 3, 2))
+    m.matmul("scores", "q", "k_t", "scores_out")
+    m.softmax("attn", "scores_out", "attn_out")
+    m.matmul("ctx", "attn_out", "v", "ctx_out")
+    m.output("ctx_out", shape)
+    if scores_also_output:
+        m.output("scores_out", (batch, heads, tokens, tokens))
+    return m.tobytes(), [_r(n + str(tokens), shape, 0.5) for n in ("q", "k", "v")]
+
+
 MODELS = {"quantised_block": quantised_block, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
 
 

@@ -180,6 +180,29 @@ def test_residual_block_is_folded_into_the_convolution(torch_dev, monkeypatch):
     assert np.array_equal(fused.run(x2)[0], plain.run(x2)[0])
 
 
+@pytest.mark.parametrize("model", ["attention_heads", "vit_block", "ragged"])
+def test_attention_block_runs_as_one_call(model, torch_dev, monkeypatch):
+    """the net loaded with the attention block folded into one call of the MatMul plugin's eval_attention against the
+    same net run operator by operator: outputs within 1e-4, the operands in between have no buffer, a second run on
+    another input reads its operands afresh"""
+    data, ins = {"attention_heads": one_models.attention_heads, "vit_block": one_models.vit_block,
+                 "ragged": lambda: one_models.attention_heads(heads=2, tokens=197, head_dim=32, batch=1)}[model]()
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    plain = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    fused = rt.Net(data)
+    assert plain.fused_attentions() == 0 and fused.fused_attentions() == 1
+    assert len(fused.ops()) == len(plain.ops()) - 3
+    assert fused.operand("scores_out")[1] is None and fused.operand("attn_out")[1] is None
+    for scale in (1.0, -0.7):
+        xs = [x * np.float32(scale) for x in ins]
+        for got, ref in zip(fused.run(*xs), plain.run(*xs)):
+            assert _close(got, ref, 1e-4)
+            assert np.all(np.abs(got - ref) <= 1e-4 * np.abs(ref) + 1e-5)
+    plain.close()
+    fused.close()
+
+
 @pytest.mark.parametrize("name", list(one_models.MODELS) + ["resnet50", "mobilenetv2"])
 def test_graph_replay_matches_plain_launches(name, torch_dev, monkeypatch):
     """loaded with ONENEW_RT_GRAPH=1 a net replays a recorded HIP graph of its operators from its second run on: five runs on changing inputs, with

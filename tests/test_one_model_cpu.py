@@ -183,6 +183,23 @@ def test_plan_folds_residual_blocks_and_relus():
     assert net.outputs[0][1] == (3, 1000)
 
 
+def test_plan_runs_an_attention_block_as_one_call(monkeypatch):
+    """MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v): one call where the fused kernel takes the shape, four operators
+    where it does not (head dimension, token count), where an operand in between has another reader, or with fusing off"""
+    data, _ = one_models.attention_heads()
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_attentions() == 1 and [t for t, _ in net.ops()] == ["MatMul"]
+    data, _ = one_models.vit_block()                       # q = k = v = one tensor, behind a Reshape
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_attentions() == 1 and len(net.ops()) == len(onefile.parse(data)["nodes"]) - 3
+    for kw in (dict(head_dim=48), dict(tokens=300), dict(scores_also_output=True)):
+        net = rt.Net(one_models.attention_heads(**kw)[0], plan_only=True)
+        assert net.fused_attentions() == 0 and len(net.ops()) == 4, kw
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    net = rt.Net(one_models.attention_heads()[0], plan_only=True)
+    assert net.fused_attentions() == 0 and len(net.ops()) == 4
+
+
 def test_plan_keeps_what_must_not_be_folded(monkeypatch):
     """a convolution whose result is a net output, or has two readers, or meets a broadcast Add, stays as it is; with
     ONENEW_RT_FUSE=0 so does everything"""
