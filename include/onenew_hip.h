@@ -410,6 +410,12 @@ int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S 
  * [..., tokens, head_dim]; params[4] / outputs[0]: the result.  No counterpart in the reference, whose host runs the four
  * operators one after the other (mat_mul.c, transpose.c, softmax.c). */
 int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_bias` / `eval_bias_gelu` of libMatMul_hip.so: MatMul -> Add of a bias over the last axis (-> Gelu) in one call
+ * (onhip_matmul with bias and table).  Slots as for the MatMul `eval` plus params[3] / inputs[2] = the bias, the
+ * result's operand in params[4], the Gelu table in inputs[11].  Bit-equal to the three reference operators in sequence
+ * (mat_mul.c, add.c, gelu.c) as this library computes them. */
+int onhip_matmul_bias_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_matmul_bias_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /*
  * No counterpart in the reference, whose operators always finish before eval returns (device/cuda/MaxPool/
  * maxpool.cu:76).  on != 0: an eval whose output is device memory returns as soon as its kernels are queued on

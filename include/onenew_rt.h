@@ -106,6 +106,14 @@ int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n);
 int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n);
 
 /*
+ * Linear layers: MatMul -> Add of an initialiser over the last axis (-> Gelu), where nothing else reads the operands in
+ * between, run as one call of the MatMul plugin's `eval_bias` / `eval_bias_gelu`, bit-equal to the separate operators
+ * (device/x86/MatMul/mat_mul.c, Add/add.c:56-70, Gelu/gelu.c).  The operands folded away read as the layer's result.
+ * ONENEW_RT_FUSE=0 keeps the operators separate.  n: how many layers.
+ */
+int onrt_net_fused_linears(const onrt_net_t *net, int32_t *n);
+
+/*
  * One inference as a HIP graph, on request: with ONENEW_RT_GRAPH=1 in the environment at load time.  The operators
  * of a net are the same launches with the same addresses on every run, so the second call of onrt_net_run records
  * them (stream capture on a stream the net owns; the first call has packed the weights, sized the workspaces and

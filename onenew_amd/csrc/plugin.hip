@@ -355,11 +355,15 @@ static int conv_add_relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *input
     return conv_eval_fused(params, inputs, outputs, 2);
 }
 
-static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+// mode 0: MatMul.  mode 1: MatMul -> Add of a bias over the last axis (params[3] / inputs[2], n elements; the result's
+// operand moves to params[4]).  mode 2: -> Gelu as well, through the table in inputs[11] like the Gelu operator.
+static int matmul_eval_mode(int mode, BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     const OPERAND_S *a_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
     const OPERAND_S *b_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
-    const OPERAND_S *o_t = reinterpret_cast<const OPERAND_S *>(params[3].addr);
-    if (!a_t || !b_t || !o_t) return set_error(ONHIP_ERR_ARG, "MatMul eval: empty params slot");
+    const OPERAND_S *bias_t = mode ? reinterpret_cast<const OPERAND_S *>(params[3].addr) : nullptr;
+    const OPERAND_S *o_t = reinterpret_cast<const OPERAND_S *>(params[mode ? 4 : 3].addr);
+    if (!a_t || !b_t || !o_t || (mode && (!bias_t || !inputs[2].addr))) return set_error(ONHIP_ERR_ARG, "MatMul eval: empty params slot");
+    if (mode == 2 && !inputs[BUF_MAXNUM - 1].addr) return set_error(ONHIP_ERR_ARG, "MatMul eval: no Gelu table in inputs[11]");
     const int nd = a_t->dim_num_of_shapes;
     if (nd < 2 || nd > SHAPE_LEN || o_t->dim_num_of_shapes < 1 || o_t->dim_num_of_shapes > SHAPE_LEN)
         return set_error(ONHIP_ERR_ARG, "MatMul eval: rank %d", nd);
@@ -392,11 +396,31 @@ static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFF
         rc = stage_buf(2, o_bytes, &y);
         if (rc) return rc;
     }
-    rc = onhip_matmul(&d, (const float *) a, (const float *) b, nullptr, nullptr, (float *) y, g_stream);
+    const void *bias = nullptr, *lut = nullptr;
+    if (mode) {
+        if (numel(bias_t) != d.n) return set_error(ONHIP_ERR_ARG, "MatMul eval: bias of %lld elements for %d columns", numel(bias_t), d.n);
+        const void *bias_host = reinterpret_cast<const void *>(inputs[2].addr);
+        rc = bias_t->is_fixed_val ? const_on_device(bias_host, (size_t) d.n * 4, &bias) : input_on_device(2, bias_host, (size_t) d.n * 4, &bias);
+        if (rc) return rc;
+    }
+    if (mode == 2) {
+        rc = const_on_device(reinterpret_cast<const void *>(inputs[BUF_MAXNUM - 1].addr), 8192 * 4, &lut);
+        if (rc) return rc;
+    }
+    rc = onhip_matmul(&d, (const float *) a, (const float *) b, (const float *) bias, (const float *) lut, (float *) y, g_stream);
     if (rc) return rc;
     if (!out_on_dev) return copy_out(host_out, y, o_bytes);
-    else return wait_for_output();
-    return ONHIP_OK;
+    return wait_for_output();
+}
+
+static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return matmul_eval_mode(0, params, inputs, outputs);
+}
+static int matmul_bias_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return matmul_eval_mode(1, params, inputs, outputs);
+}
+static int matmul_bias_gelu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return matmul_eval_mode(2, params, inputs, outputs);
 }
 
 // MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v) as one call.  Slots: params[1..3] the operands q, k, v (all
@@ -756,6 +780,12 @@ int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFE
 
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MatMul", matmul_eval_locked, params, inputs, outputs);
+}
+int onhip_matmul_bias_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MatMul (+ bias)", matmul_bias_eval_locked, params, inputs, outputs);
+}
+int onhip_matmul_bias_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MatMul (+ bias + Gelu)", matmul_bias_gelu_eval_locked, params, inputs, outputs);
 }
 int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MatMul (attention)", matmul_attention_eval_locked, params, inputs, outputs);

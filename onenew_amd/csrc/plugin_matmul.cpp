@@ -15,3 +15,16 @@ extern "C" __attribute__((visibility("default"))) int eval_attention(BUFFER_INFO
                                                                      BUFFER_INFO_S *outputs) {
     return onhip_matmul_attention_eval(params, inputs, outputs);
 }
+
+// Not in the reference: MatMul -> Add of a bias over the last axis (-> Gelu) as one call, the linear layers of a
+// transformer block.  Slots as for `eval`, plus params[3] / inputs[2] = the bias (as many elements as the result has
+// columns); the result's operand moves to params[4]; eval_bias_gelu reads the Gelu table from inputs[11] like the Gelu
+// operator (host/ops/gelu.h:80-96).  Values equal those of the separate operators bit for bit.
+extern "C" __attribute__((visibility("default"))) int eval_bias(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                BUFFER_INFO_S *outputs) {
+    return onhip_matmul_bias_eval(params, inputs, outputs);
+}
+extern "C" __attribute__((visibility("default"))) int eval_bias_gelu(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                     BUFFER_INFO_S *outputs) {
+    return onhip_matmul_bias_gelu_eval(params, inputs, outputs);
+}

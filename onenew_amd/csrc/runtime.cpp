@@ -162,8 +162,8 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    onenew_eval_fn matmul_attention = nullptr;                    // optional entry point of the MatMul plugin
-    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0;
+    onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr;   // optional entry points of the MatMul plugin
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -517,7 +517,11 @@ int bind_plugins(onrt_net &net) {
             net.conv_add = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add"));
             net.conv_add_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add_relu"));
         }
-        if (type == "MatMul") net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
+        if (type == "MatMul") {
+            net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
+            net.matmul_bias = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_bias"));
+            net.matmul_bias_gelu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_bias_gelu"));
+        }
     }
     return ONRT_OK;
 }
@@ -764,6 +768,54 @@ int fuse_attention(onrt_net &net) {
     return ONRT_OK;
 }
 
+// ---- linear layers ----------------------------------------------------------------------------------------
+// MatMul -> Add of an initialiser over the last axis (-> Gelu), where nothing else reads the operands in between, becomes
+// one call of the MatMul plugin's `eval_bias` / `eval_bias_gelu`: bias and table activation are applied in the store of
+// the product, bit-equal to the separate operators (device/x86/MatMul/mat_mul.c, Add/add.c:56-70 broadcast of the smaller
+// operand along the leading axes, Gelu/gelu.c).  The reference's optimiser builds the Gelu node itself out of five
+// primitives (tools/optimize/op_fusion.hpp:195-222); folding it into the MatMul goes one operator further, at load time.
+// Only a bias that add.c would broadcast: rank 3 to 6 result, bias [n] (leading axes of extent 1 allowed).
+int fuse_linear(onrt_net &net) {
+    if (!fusing_enabled() || !net.matmul_bias) return ONRT_OK;
+    std::vector<bool> dropped(net.nodes.size(), false);
+    for (int idx : net.order) {
+        Node &mm = net.nodes[idx];
+        if (strcmp(mm.kind->type, "MatMul") || mm.in.size() != 2 || mm.out.size() != 1 || mm.fuse) continue;
+        const int ai = sole_reader(net, mm.out[0], "Add");
+        if (ai < 0) continue;
+        const Node &add = net.nodes[ai];
+        if (add.in.size() != 2 || add.out.size() != 1 || add.in[0] == add.in[1]) continue;
+        const std::string &bias = add.in[0] == mm.out[0] ? add.in[1] : add.in[0];
+        const Tensor &bt = net.tensors[bias], &yt = net.tensors[mm.out[0]], &st = net.tensors[add.out[0]];
+        const int rank = yt.desc.dim_num_of_shapes, brank = bt.desc.dim_num_of_shapes;
+        if (!bt.is_init || rank < 3 || rank > 6 || brank < 1 || brank > rank) continue;
+        const int n = yt.desc.shapes[rank - 1];
+        bool last_axis_only = bt.desc.shapes[brank - 1] == n && numel(bt.desc) == n && numel(yt.desc) > n;
+        if (!last_axis_only || memcmp(st.desc.shapes, yt.desc.shapes, sizeof(yt.desc.shapes))) continue;
+        mm.fuse = 4;
+        mm.in.push_back(bias);
+        mm.fused_out = add.out[0];
+        mm.eval = net.matmul_bias;
+        net.tensors[mm.out[0]].alias = mm.fused_out;
+        dropped[ai] = true;
+        const int gi = net.matmul_bias_gelu ? sole_reader(net, add.out[0], "Gelu") : -1;
+        if (gi >= 0 && net.nodes[gi].in.size() == 1 && net.nodes[gi].out.size() == 1) {
+            mm.fuse = 5;
+            mm.fused_out = net.nodes[gi].out[0];
+            mm.eval = net.matmul_bias_gelu;
+            net.tensors[add.out[0]].alias = mm.fused_out;
+            net.tensors[mm.out[0]].alias = mm.fused_out;
+            dropped[gi] = true;
+        }
+        ++net.fused_linears;
+    }
+    std::vector<int> order;
+    for (int idx : net.order)
+        if (!dropped[idx]) order.push_back(idx);
+    net.order.swap(order);
+    return ONRT_OK;
+}
+
 // ---- slot arrays (op::rt_prepare, host/op.h:109-168, and prepare_init_operand_data of each operator) ----
 int fill_slots(onrt_net &net) {
     const size_t lut_len = net.silu_lut.size();
@@ -794,7 +846,7 @@ int fill_slots(onrt_net &net) {
         nd.params[BUF_MAXNUM - 1].addr = (int64_t) &net.useful;
         if (!strcmp(nd.kind->type, "Conv") && reinterpret_cast<const CONV_CONFIG_S *>(nd.cfg.data())->act_type == SILU)
             nd.inputs[BUF_MAXNUM - 1].addr = (int64_t) net.tables;
-        if (!strcmp(nd.kind->type, "Gelu")) nd.inputs[BUF_MAXNUM - 1].addr = (int64_t) (static_cast<float *>(net.tables) + lut_len);
+        if (!strcmp(nd.kind->type, "Gelu") || nd.fuse == 5) nd.inputs[BUF_MAXNUM - 1].addr = (int64_t) (static_cast<float *>(net.tables) + lut_len);
     }
     return ONRT_OK;
 }
@@ -810,6 +862,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = fuse_attention(net);
+    if (!rc) rc = fuse_linear(net);
     if (!rc) rc = allocate(net);
     if (!rc) rc = build_tables(net);
     if (!rc) rc = fill_slots(net);
@@ -830,10 +883,11 @@ int plan(onrt_net &net) {
     int rc = read_model(net);
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
-    net.conv_add = net.conv_add_relu = net.matmul_attention = plan_stub_eval;   // as with the plugins of this package
+    net.conv_add = net.conv_add_relu = net.matmul_attention = net.matmul_bias = net.matmul_bias_gelu = plan_stub_eval;   // as with the plugins of this package
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = fuse_attention(net);
+    if (!rc) rc = fuse_linear(net);
     return rc;
 }
 
@@ -1025,6 +1079,12 @@ ONRT_API int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n) {
 ONRT_API int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n) {
     if (!net || !n) return fail(ONRT_ERR_ARG, "fused attentions: null argument");
     *n = (int32_t) net->fused_attentions;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_fused_linears(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "fused linear layers: null argument");
+    *n = (int32_t) net->fused_linears;
     return ONRT_OK;
 }
 

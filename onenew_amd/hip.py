@@ -42,7 +42,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", "onhip_dw_project_supported", "onhip_dw_project_packed_weight_bytes", "onhip_dw_project_pack_weights", "onhip_dw_project_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
-           "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
+           "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
            "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_gelu_eval", "onhip_layernorm_eval",
            "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_set_async", "onhip_plugin_set_stream", "onhip_plugin_forget", "onhip_plugin_trust_weights", "onhip_plugin_release"]
 
@@ -115,7 +115,7 @@ def load():
     L.onhip_dw_project_pack_weights.argtypes = [vp, i32, i32, vp, vp]
     L.onhip_dw_project_f32.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp]
     L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
-    for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_gemm_eval"):
+    for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
     _lib = L
     return L

@@ -180,6 +180,37 @@ def test_residual_block_is_folded_into_the_convolution(torch_dev, monkeypatch):
     assert np.array_equal(fused.run(x2)[0], plain.run(x2)[0])
 
 
+def test_linear_layers_run_as_one_call_bit_for_bit(torch_dev, monkeypatch):
+    """MatMul -> Add of a bias -> Gelu and MatMul -> Add of a bias as one call each: the operands behind them hold exactly
+    what the separate operators produce (the bias is added to the finished sum, the table is read with the same index)"""
+    m = onefile.OneModel()
+    rng = np.random.default_rng(3)
+    w = lambda *s: (rng.normal(size=s) * 0.2).astype(np.float32)   # noqa: E731
+    m.input("x", (2, 50, 48))
+    m.matmul("fc1", "x", w(48, 96), "fc1_out")
+    m.add("fc1_bias", "fc1_out", w(96), "fc1_b")
+    m.gelu("act", "fc1_b", "act_out")
+    m.matmul("fc2", "act_out", w(96, 40), "fc2_out")
+    m.add("fc2_bias", "fc2_out", w(1, 1, 40), "fc2_b")                # leading axes of extent 1
+    m.matmul("fc3", "fc2_b", w(40, 24), "fc3_out")
+    m.add("not_a_bias", "fc3_out", w(2, 50, 24), "y")                 # a full tensor: stays an Add
+    m.output("act_out", (2, 50, 96))
+    m.output("y", (2, 50, 24))
+    data, x = m.tobytes(), rng.normal(size=(2, 50, 48)).astype(np.float32)
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    plain = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    fused = rt.Net(data)
+    assert plain.fused_linears() == 0 and fused.fused_linears() == 2
+    assert [t for t, _ in fused.ops()] == ["MatMul", "MatMul", "MatMul", "Add"]
+    for got, ref in zip(fused.run(x), plain.run(x)):
+        assert np.array_equal(got, ref)
+    assert np.array_equal(fused.fetch("fc2_b"), plain.fetch("fc2_b"))
+    assert fused.operand("fc1_out")[1] == fused.operand("fc1_b")[1] == fused.operand("act_out")[1]
+    plain.close()
+    fused.close()
+
+
 @pytest.mark.parametrize("model", ["attention_heads", "vit_block", "ragged"])
 def test_attention_block_runs_as_one_call(model, torch_dev, monkeypatch):
     """the net loaded with the attention block folded into one call of the MatMul plugin's eval_attention against the
@@ -192,7 +223,10 @@ def test_attention_block_runs_as_one_call(model, torch_dev, monkeypatch):
     monkeypatch.delenv("ONENEW_RT_FUSE")
     fused = rt.Net(data)
     assert plain.fused_attentions() == 0 and fused.fused_attentions() == 1
-    assert len(fused.ops()) == len(plain.ops()) - 3
+    # vit_block also has two linear layers (MatMul -> Add -> Gelu and MatMul -> Add): three more operators folded away
+    linears = 2 if model == "vit_block" else 0
+    assert plain.fused_linears() == 0 and fused.fused_linears() == linears
+    assert len(fused.ops()) == len(plain.ops()) - 3 - (3 if linears else 0)
     assert fused.operand("scores_out")[1] is None and fused.operand("attn_out")[1] is None
     for scale in (1.0, -0.7):
         xs = [x * np.float32(scale) for x in ins]
