@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
 Workloads: resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
-cfg1, resnet50_net_b{1,32} and mobilenetv2_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
+cfg1, resnet50_net_b{1,32}, mobilenetv2_net_b{1,64} and vit_tiny_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
 the HBM traffic counters are scaled by).
 
 A step is one pass over every layer of the workload: one launch per layer, inputs, weights and outputs
@@ -639,13 +639,14 @@ def cpu_baseline(layers, tag, unit, budget_s=12.0):
 
 def bench_net(torch, args):
     """A whole model (ResNet-50: 53 Conv, MaxPool, 16 Add, 16 Relu, GlobalAveragePool, Gemm; MobileNetV2: 52 Conv of
-    which 17 depthwise, 10 Add, GlobalAveragePool, Gemm) as a .one file through the device-resident runtime
+    which 17 depthwise, 10 Add, GlobalAveragePool, Gemm; ViT-Tiny: patch Conv, 12 encoder blocks of LayerNormalization /
+    MatMul / Add / Transpose / Softmax / Gelu, mean over the tokens, Gemm) as a .one file through the device-resident runtime
     (libonenew_rt.so): every operator back to back on the device, input and output in device memory.  A step is one
     inference of the batch."""
     from onenew_amd import rt, stacks
     n = int(args.workload.split("_b")[1])
-    model = "ResNet-50" if args.workload.startswith("resnet50") else "MobileNetV2"
-    make = stacks.resnet50_model if model == "ResNet-50" else stacks.mobilenet_v2_model
+    model = "ResNet-50" if args.workload.startswith("resnet50") else "MobileNetV2" if args.workload.startswith("mobilenetv2") else "ViT-Tiny"
+    make = {"ResNet-50": stacks.resnet50_model, "MobileNetV2": stacks.mobilenet_v2_model, "ViT-Tiny": stacks.vit_tiny_model}[model]
     data, in_shape, flops = make(n)
     net = rt.Net(data)
     x = torch.randn(in_shape, dtype=torch.float32, device="cuda")
@@ -856,7 +857,7 @@ def main():
                           "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
         return
 
-    if args.workload.startswith("resnet50_net_b") or args.workload.startswith("mobilenetv2_net_b"):
+    if args.workload.startswith(("resnet50_net_b", "mobilenetv2_net_b", "vit_tiny_net_b")):
         return bench_net(torch, args)
 
     res = run_workload(torch, hip, args.workload, args.steps, args.warmup, layers_table=args.layers, graph=not args.no_graph)

@@ -213,3 +213,67 @@ def mobilenet_v2_model(batch=1, classes=1000, tag="mobilenetv2_model"):
     m.output("logits", (batch, classes))
     return m.tobytes(), (batch, 3, 224, 224), flops
 
+
+
+def vit_tiny_model(batch=1, blocks=12, classes=1000, tag="vit_tiny_model"):
+    """A ViT-Tiny/16 encoder as a .one file with the operators this package runs: 16x16 stride-16 patch convolution,
+    position embedding, `blocks` pre-norm encoder blocks (LayerNormalization, three projections with bias, head split
+    Transposes, MatMul / Softmax / MatMul attention over 3 heads of 64 with the 1/8 scale folded into the q projection,
+    head merge, output projection, residual Add, LayerNormalization, MLP with table Gelu, residual Add), final
+    LayerNormalization, mean over the 196 tokens (no class token: the package has no Concat), Gemm head.  Seeded weights.
+    Returns (bytes, input shape, multiply-accumulates x 2 per inference)."""
+    import numpy as np
+    from . import datagen, onefile
+
+    m = onefile.OneModel()
+    T, D, H, hd = 196, 192, 3, 64
+    flops = 0
+
+    def w(name, shape, std):
+        return datagen.normal(datagen.seed_for(tag, name), shape, 0.0, std)
+
+    def linear(name, x, k, n, gain=1.0, gelu=False):
+        nonlocal flops
+        flops += 2 * batch * T * k * n
+        y = m.matmul(name, x, w(name + ".w", (k, n), gain / float(np.sqrt(k))), name + "_mm")
+        y = m.add(name + ".bias", y, w(name + ".b", (n,), 0.02), name + "_out")
+        return m.gelu(name + ".gelu", y, name + "_act") if gelu else y
+
+    x = m.input("input", (batch, 3, 224, 224))
+    flops += 2 * batch * D * T * 3 * 256
+    x = m.conv("patch", x, w("patch.w", (D, 3, 16, 16), 1.0 / float(np.sqrt(768))), w("patch.b", (D,), 0.02), "patch_out", stride=16)
+    x = m.reshape("tokens.flat", x, "tokens_flat", (batch, D, T, 1))
+    x = m.transpose("tokens.t", x, "tokens_t", (0, 2, 1, 3))
+    x = m.reshape("tokens", x, "tokens", (batch, T, D))
+    x = m.add("pos", x, w("pos", (T, D), 0.02), "embedded")
+    for b in range(blocks):
+        p = f"b{b}."
+        y = m.layernorm(p + "ln1", x, 1.0 + w(p + "ln1.g", (D,), 0.05), w(p + "ln1.b", (D,), 0.05), p + "ln1_out")
+        heads = {}
+        for which in ("q", "k", "v"):
+            t = linear(p + which, y, D, D, gain=0.125 if which == "q" else 1.0)
+            t = m.reshape(p + which + ".split", t, p + which + "_split", (batch, T, H, hd))
+            heads[which] = m.transpose(p + which + ".heads", t, p + which + "_heads", (0, 2, 1, 3))
+        flops += 2 * 2 * batch * H * T * T * hd
+        kt = m.transpose(p + "k.t", heads["k"], p + "k_t", (0, 1, 3, 2))
+        s = m.matmul(p + "scores", heads["q"], kt, p + "scores_out")
+        a = m.softmax(p + "attn", s, p + "attn_out")
+        c = m.matmul(p + "ctx", a, heads["v"], p + "ctx_out")
+        c = m.transpose(p + "merge", c, p + "merged", (0, 2, 1, 3))
+        c = m.reshape(p + "merge.flat", c, p + "merged_flat", (batch, T, D))
+        c = linear(p + "proj", c, D, D, gain=0.5)
+        x = m.add(p + "res1", c, x, p + "res1_out")
+        y = m.layernorm(p + "ln2", x, 1.0 + w(p + "ln2.g", (D,), 0.05), w(p + "ln2.b", (D,), 0.05), p + "ln2_out")
+        y = linear(p + "fc1", y, D, 4 * D, gelu=True)
+        y = linear(p + "fc2", y, 4 * D, D, gain=0.5)
+        x = m.add(p + "res2", y, x, p + "res2_out")
+    x = m.layernorm("ln", x, 1.0 + w("ln.g", (D,), 0.05), w("ln.b", (D,), 0.05), "ln_out")
+    x = m.reshape("pool.shape", x, "pool_in_t", (batch, T, D, 1))
+    x = m.transpose("pool.t", x, "pool_in", (0, 2, 1, 3))
+    x = m.reshape("pool.grid", x, "pool_grid", (batch, D, 14, 14))
+    x = m.global_avgpool("pool", x, "pooled")
+    x = m.flatten("flatten", x, "flat", axis=1)
+    flops += 2 * batch * classes * D
+    m.gemm("head", x, w("head.w", (classes, D), 0.05), w("head.b", (classes,), 0.01), "logits")
+    m.output("logits", (batch, classes))
+    return m.tobytes(), (batch, 3, 224, 224), flops

@@ -180,6 +180,25 @@ def test_residual_block_is_folded_into_the_convolution(torch_dev, monkeypatch):
     assert np.array_equal(fused.run(x2)[0], plain.run(x2)[0])
 
 
+def test_vit_encoder_through_the_runtime(torch_dev, monkeypatch):
+    """a ViT-Tiny encoder (two of its twelve blocks) as a .one file: logits against the CPU restatement of the graph, with
+    every attention block and every linear layer folded into one call each and with every operator on its own"""
+    from onenew_amd import stacks
+    data, shape, _ = stacks.vit_tiny_model(2, blocks=2)
+    x = np.random.default_rng(5).normal(size=shape).astype(np.float32)
+    ref = one_model.run(data, [x])[0]
+    fused = rt.Net(data)
+    assert fused.fused_attentions() == 2 and fused.fused_linears() == 12
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    plain = rt.Net(data)
+    assert len(plain.ops()) == len(onefile.parse(data)["nodes"]) and len(fused.ops()) == len(plain.ops()) - 2 * 3 - 14
+    for net in (fused, plain):
+        got = net.run(x)[0]
+        assert got.shape == ref.shape and _close(got, ref, 1e-3), float(np.abs(got - ref).max())
+        assert np.array_equal(np.argsort(got, axis=1)[:, -5:], np.argsort(ref, axis=1)[:, -5:])
+        net.close()
+
+
 def test_linear_layers_run_as_one_call_bit_for_bit(torch_dev, monkeypatch):
     """MatMul -> Add of a bias -> Gelu and MatMul -> Add of a bias as one call each: the operands behind them hold exactly
     what the separate operators produce (the bias is added to the finished sum, the table is read with the same index)"""
