@@ -243,6 +243,11 @@ int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, cons
  * with bias/gelu_lut, the chain MatMul -> Add -> Gelu (device/x86/Gelu/gelu.c:9). */
 int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
                  const float *gelu_lut, float *out, void *stream);
+/* MatMul -> Add of a bias over the last axis (bias may be NULL) -> Add of a tensor shaped like the result (the skip
+ * connection of a transformer block), the sum formed in the product's store: mat_mul.c eval (:10) followed by two
+ * device/x86/Add/add.c evals, bit-equal to them.  addend must not be the output buffer. */
+int onhip_matmul_add(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
+                     const float *addend, float *out, void *stream);
 
 /* The second half of an inverted-residual block in one launch: depthwise 3x3 convolution (pads 1, stride 1 or 2, bias,
  * activation) -> 1x1 convolution (bias, activation) [-> Add of a residual tensor shaped like the output].  Replaces two
@@ -407,7 +412,9 @@ int onhip_transpose_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_IN
 int onhip_gemm_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* `eval_attention` of libMatMul_hip.so: MatMul(q, Transpose(k)) -> Softmax (last axis) -> MatMul(., v) in one call
  * (onhip_attention with scale 1).  params[1..3] / inputs[0..2]: q, k (before its Transpose), v, all
- * [..., tokens, head_dim]; params[4] / outputs[0]: the result.  No counterpart in the reference, whose host runs the four
+ * [..., tokens, head_dim]; params[4] / outputs[0]: the result.  inputs[4]: null, or the address of four int32 flags (q, k,
+ * v, result); non-zero = that rank-4 tensor is stored [batch, tokens, heads, head_dim], as on the other side of a
+ * head-split / head-merge Transpose (0, 2, 1, 3), and its operand carries that shape.  No counterpart in the reference, whose host runs the four
  * operators one after the other (mat_mul.c, transpose.c, softmax.c). */
 int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* `eval_bias` / `eval_bias_gelu` of libMatMul_hip.so: MatMul -> Add of a bias over the last axis (-> Gelu) in one call
@@ -416,6 +423,10 @@ int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BU
  * (mat_mul.c, add.c, gelu.c) as this library computes them. */
 int onhip_matmul_bias_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_matmul_bias_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_bias_add` of libMatMul_hip.so: MatMul -> Add of a bias over the last axis -> Add of a tensor shaped like the
+ * result, in one call (onhip_matmul_add).  Slots as for `eval_bias`; the second addend travels in inputs[3] (it has the
+ * result's operand, so no params slot of its own), as the addend of the Conv plugin's `eval_add` does. */
+int onhip_matmul_bias_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /*
  * No counterpart in the reference, whose operators always finish before eval returns (device/cuda/MaxPool/
  * maxpool.cu:76).  on != 0: an eval whose output is device memory returns as soon as its kernels are queued on

@@ -100,7 +100,10 @@ int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n);
  * in between, run as one call of the MatMul plugin's `eval_attention` (libMatMul_hip.so; the scores stay on the chip, the
  * transposed k is never written) when q, k and v are [..., tokens, head_dim] with head_dim 32 or 64 and at most 256
  * tokens.  The reference's host runs the four operators one after the other (host/net.h:613-618); its optimiser has
- * no such pattern (tools/optimize/op_fusion.hpp:477-591).  The operands folded away have no buffer
+ * no such pattern (tools/optimize/op_fusion.hpp:477-591).  A head-split Transpose (0, 2, 1, 3) that only feeds q, k or v
+ * of such a block, and a head-merge one that alone reads its result, go as well: the call walks the [batch, tokens, heads,
+ * head_dim] tensor on their far side through strides (device/x86/Transpose/transpose.c never runs for them).
+ * The operands folded away have no buffer
  * (onrt_net_operand gives a null pointer for them).  ONENEW_RT_FUSE=0 keeps the operators separate.  n: how many blocks.
  */
 int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n);
@@ -112,6 +115,10 @@ int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n);
  * ONENEW_RT_FUSE=0 keeps the operators separate.  n: how many layers.
  */
 int onrt_net_fused_linears(const onrt_net_t *net, int32_t *n);
+/* Of those layers, the ones (without Gelu) whose result goes, with no other reader, into an Add with an activation of the
+ * same shape (the skip connection around a transformer block's projection): that Add joins the call (`eval_bias_add`,
+ * the addend in inputs[3]), which then runs where the second Add stood.  n: how many. */
+int onrt_net_fused_skips(const onrt_net_t *net, int32_t *n);
 
 /*
  * One inference as a HIP graph, on request: with ONENEW_RT_GRAPH=1 in the environment at load time.  The operators

@@ -1027,8 +1027,8 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
     return conv2d_w8a32_impl(&dd, nullptr, xq, w8_packed, 1, bias32, weight_aux, silu_lut, yq, nullptr, nullptr, 0, 1, stream);
 }
 
-int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
-                 const float *gelu_lut, float *out, void *stream) {
+static int matmul_impl(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
+                       const float *gelu_lut, const float *addend, float *out, void *stream) {
     if (!d || d->batch < 1 || d->m < 1 || d->k < 1 || d->n < 1) return set_error(ONHIP_ERR_ARG, "matmul: bad shape");
     if (!a || !b || !out) return set_error(ONHIP_ERR_ARG, "matmul: null tensor pointer");
     int batch = d->batch, M = d->m;
@@ -1069,7 +1069,30 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
     p.ep.act = gelu_lut ? ONHIP_ACT_GELU_LUT : NOT_ACT;
     p.ep.lut = gelu_lut;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (addend == out) return set_error(ONHIP_ERR_ARG, "matmul: the addend may not be the output buffer");
+    if (addend && cfg.dtype != DT_F32) {   // reduced-precision operands: the Add as a pass over the result
+        rc = plan_and_launch(cfg, p, st);
+        if (rc) return rc;
+        onhip_add_desc_t ad;
+        memset(&ad, 0, sizeof(ad));
+        ad.ndim = 2;
+        ad.large_shape[0] = ad.small_shape[0] = batch * M;
+        ad.large_shape[1] = ad.small_shape[1] = d->n;
+        return onhip_add_f32(&ad, out, addend, out, stream);
+    }
+    p.res = addend;   // laid out like the result; added after the bias, as the Add operator after it would
     return plan_and_launch(cfg, p, st);
+}
+
+int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
+                 const float *gelu_lut, float *out, void *stream) {
+    return matmul_impl(d, a, b, bias, gelu_lut, nullptr, out, stream);
+}
+
+int onhip_matmul_add(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
+                     const float *addend, float *out, void *stream) {
+    if (!addend) return set_error(ONHIP_ERR_ARG, "matmul_add: null addend");
+    return matmul_impl(d, a, b, bias, nullptr, addend, out, stream);
 }
 
 // ---- 16-bit storage: bf16 / fp16 operands and results in memory, fp32 accumulation ---------------------------------------

@@ -46,7 +46,7 @@ struct DevBuf {
     size_t bytes = 0;
 };
 // persistent staging buffers: [0] input, [1] second input, [2] output, [3] workspace
-static DevBuf g_stage[4];
+static DevBuf g_stage[6];   // 0, 1: inputs; 2: the output; 3: workspace; 4, 5: third and fourth input of a fused MatMul
 // uploaded constants keyed by (host address, bytes); the fingerprint of the content detects a host buffer that was
 // freed and reused for other data at the same address, or weights updated in place
 struct ConstEntry {
@@ -357,6 +357,7 @@ static int conv_add_relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *input
 
 // mode 0: MatMul.  mode 1: MatMul -> Add of a bias over the last axis (params[3] / inputs[2], n elements; the result's
 // operand moves to params[4]).  mode 2: -> Gelu as well, through the table in inputs[11] like the Gelu operator.
+// mode 3: mode 1 -> Add of the tensor in inputs[3], which has the result's shape.
 static int matmul_eval_mode(int mode, BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     const OPERAND_S *a_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
     const OPERAND_S *b_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
@@ -400,14 +401,22 @@ static int matmul_eval_mode(int mode, BUFFER_INFO_S *params, BUFFER_INFO_S *inpu
     if (mode) {
         if (numel(bias_t) != d.n) return set_error(ONHIP_ERR_ARG, "MatMul eval: bias of %lld elements for %d columns", numel(bias_t), d.n);
         const void *bias_host = reinterpret_cast<const void *>(inputs[2].addr);
-        rc = bias_t->is_fixed_val ? const_on_device(bias_host, (size_t) d.n * 4, &bias) : input_on_device(2, bias_host, (size_t) d.n * 4, &bias);
+        rc = bias_t->is_fixed_val ? const_on_device(bias_host, (size_t) d.n * 4, &bias) : input_on_device(4, bias_host, (size_t) d.n * 4, &bias);
         if (rc) return rc;
     }
     if (mode == 2) {
         rc = const_on_device(reinterpret_cast<const void *>(inputs[BUF_MAXNUM - 1].addr), 8192 * 4, &lut);
         if (rc) return rc;
     }
-    rc = onhip_matmul(&d, (const float *) a, (const float *) b, (const float *) bias, (const float *) lut, (float *) y, g_stream);
+    if (mode == 3) {
+        if (!inputs[3].addr) return set_error(ONHIP_ERR_ARG, "MatMul eval: no addend in inputs[3]");
+        const void *addend;
+        rc = input_on_device(5, reinterpret_cast<const void *>(inputs[3].addr), o_bytes, &addend);
+        if (rc) return rc;
+        rc = onhip_matmul_add(&d, (const float *) a, (const float *) b, (const float *) bias, (const float *) addend, (float *) y, g_stream);
+    } else {
+        rc = onhip_matmul(&d, (const float *) a, (const float *) b, (const float *) bias, (const float *) lut, (float *) y, g_stream);
+    }
     if (rc) return rc;
     if (!out_on_dev) return copy_out(host_out, y, o_bytes);
     return wait_for_output();
@@ -422,33 +431,57 @@ static int matmul_bias_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
 static int matmul_bias_gelu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return matmul_eval_mode(2, params, inputs, outputs);
 }
+static int matmul_bias_add_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return matmul_eval_mode(3, params, inputs, outputs);
+}
 
 // MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v) as one call.  Slots: params[1..3] the operands q, k, v (all
 // [..., tokens, head_dim], k NOT transposed), params[4] the result [..., tokens, head_dim]; inputs[0..2], outputs[0] the
 // tensors (host or device memory like every eval).  Leading dimensions are (batch, head) pairs.
+// inputs[4]: null, or the address of four int32 flags for q, k, v and the result; a non-zero flag says that this tensor
+// (rank 4) is stored [batch, tokens, heads, head_dim], i.e. as it is before a head-split Transpose (0, 2, 1, 3) or after
+// the head-merge one, and its operand in params carries that shape; the call walks it with strides.
 static int matmul_attention_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     const OPERAND_S *t[4];
     for (int i = 0; i < 4; ++i) {
         t[i] = reinterpret_cast<const OPERAND_S *>(params[1 + i].addr);
         if (!t[i]) return set_error(ONHIP_ERR_ARG, "attention eval: empty params slot %d", 1 + i);
     }
+    const int32_t *flags = reinterpret_cast<const int32_t *>(inputs[4].addr);
+    const bool token_major = flags && (flags[0] || flags[1] || flags[2] || flags[3]);
     const int nd = t[0]->dim_num_of_shapes;
-    if (nd < 2 || nd > SHAPE_LEN) return set_error(ONHIP_ERR_ARG, "attention eval: rank %d", nd);
-    for (int i = 1; i < 4; ++i)
-        if (t[i]->dim_num_of_shapes != nd || memcmp(t[i]->shapes, t[0]->shapes, nd * sizeof(t[0]->shapes[0])))
+    if (nd < 2 || nd > SHAPE_LEN || (token_major && nd != 4)) return set_error(ONHIP_ERR_ARG, "attention eval: rank %d", nd);
+    // every tensor's shape as [..., tokens, head_dim], the two middle axes of a token-major one exchanged
+    int32_t shape[4][SHAPE_LEN];
+    for (int i = 0; i < 4; ++i) {
+        if (t[i]->dim_num_of_shapes != nd) return set_error(ONHIP_ERR_ARG, "attention eval: q, k, v and the result must have one rank");
+        for (int a = 0; a < nd; ++a) shape[i][a] = t[i]->shapes[a];
+        if (token_major && flags[i]) { shape[i][1] = t[i]->shapes[2]; shape[i][2] = t[i]->shapes[1]; }
+        if (memcmp(shape[i], shape[0], nd * sizeof(int32_t)))
             return set_error(ONHIP_ERR_ARG, "attention eval: q, k, v and the result must have one shape");
+    }
     onhip_attention_desc_t d;
     memset(&d, 0, sizeof(d));
     d.batch = 1;
-    for (int i = 0; i < nd - 2; ++i) d.batch *= t[0]->shapes[i];
+    for (int i = 0; i < nd - 2; ++i) d.batch *= shape[0][i];
     d.heads = 1;
-    d.tokens = t[0]->shapes[nd - 2];
-    d.head_dim = t[0]->shapes[nd - 1];
+    d.tokens = shape[0][nd - 2];
+    d.head_dim = shape[0][nd - 1];
     d.scale = 1.0f;
     d.compute = ONHIP_COMPUTE_F32;
     const long long plane = (long long) d.tokens * d.head_dim;
-    for (long long *st : {d.q_strides, d.k_strides, d.v_strides, d.out_strides}) { st[0] = plane; st[1] = plane; st[2] = d.head_dim; }
-    const size_t bytes = (size_t) d.batch * plane * 4;
+    long long *strides[4] = {d.q_strides, d.k_strides, d.v_strides, d.out_strides};
+    for (long long *st : strides) { st[0] = plane; st[1] = plane; st[2] = d.head_dim; }
+    if (token_major) {
+        d.batch = shape[0][0];
+        d.heads = shape[0][1];
+        for (int i = 0; i < 4; ++i) {
+            strides[i][0] = (long long) d.heads * plane;
+            strides[i][1] = flags[i] ? d.head_dim : plane;
+            strides[i][2] = flags[i] ? (long long) d.heads * d.head_dim : d.head_dim;
+        }
+    }
+    const size_t bytes = (size_t) d.batch * d.heads * plane * 4;
     const void *in[3];
     for (int i = 0; i < 3; ++i) {
         if (!inputs[i].addr) return set_error(ONHIP_ERR_ARG, "attention eval: empty input slot %d", i);
@@ -786,6 +819,9 @@ int onhip_matmul_bias_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
 }
 int onhip_matmul_bias_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MatMul (+ bias + Gelu)", matmul_bias_gelu_eval_locked, params, inputs, outputs);
+}
+int onhip_matmul_bias_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MatMul (+ bias + Add)", matmul_bias_add_eval_locked, params, inputs, outputs);
 }
 int onhip_matmul_attention_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MatMul (attention)", matmul_attention_eval_locked, params, inputs, outputs);

@@ -128,6 +128,7 @@ struct Node {
     onenew_eval_fn eval = nullptr;
     int fuse = 0;            // Conv: 1 = the Add after it is folded in, 2 = and the Relu after that
     std::string addend, fused_out;
+    int32_t token_major[4] = {0, 0, 0, 0};   // fused attention: q, k, v, result stored [batch, tokens, heads, head_dim]
     BUFFER_INFO_S params[BUF_MAXNUM], inputs[BUF_MAXNUM], outputs[BUF_MAXNUM];
     const BASE_CONFIG_S *base() const { return reinterpret_cast<const BASE_CONFIG_S *>(cfg.data()); }
 };
@@ -162,8 +163,8 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr;   // optional entry points of the MatMul plugin
-    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0;
+    onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr, matmul_bias_add = nullptr;   // optional entry points of the MatMul plugin
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -521,6 +522,7 @@ int bind_plugins(onrt_net &net) {
             net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
             net.matmul_bias = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_bias"));
             net.matmul_bias_gelu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_bias_gelu"));
+            net.matmul_bias_add = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_bias_add"));
         }
     }
     return ONRT_OK;
@@ -705,6 +707,7 @@ int fuse_residual_blocks(onrt_net &net) {
 // all [..., tokens, head_dim] with head_dim 32 or 64 and at most 256 tokens); every other attention block keeps its four
 // operators (device/x86/MatMul/mat_mul.c, Transpose/transpose.c, Softmax/softmax.c).  The fused call takes the place of
 // the second MatMul in the order, where q, k and v are all complete.  ONENEW_RT_FUSE=0 keeps every operator separate.
+// Head-split and head-merge Transposes around the block fold into the call's strides (see below).
 int fuse_attention(onrt_net &net) {
     if (!fusing_enabled() || !net.matmul_attention) return ONRT_OK;
     auto producer_of = [&](const std::string &name) {
@@ -749,9 +752,36 @@ int fuse_attention(onrt_net &net) {
             memcmp(vt.desc.shapes, qt.desc.shapes, nd * sizeof(qt.desc.shapes[0])) ||
             memcmp(ot.desc.shapes, qt.desc.shapes, nd * sizeof(qt.desc.shapes[0])))
             continue;
+        // A head-split Transpose (0, 2, 1, 3) in front of q, k or v that nothing else reads, and a head-merge one behind the
+        // result: the call reads / writes the [batch, tokens, heads, head_dim] tensor on the other side of it through
+        // strides (flags in inputs[4]), and the Transpose goes.
+        auto swaps_heads = [&](int node) {
+            if (node < 0 || dropped[node] || nd != 4 || strcmp(net.nodes[node].kind->type, "Transpose")) return false;
+            const TRANSPOSE_CONFIG_S *c = reinterpret_cast<const TRANSPOSE_CONFIG_S *>(net.nodes[node].cfg.data());
+            return c->perm_num == 4 && c->perm[0] == 0 && c->perm[1] == 2 && c->perm[2] == 1 && c->perm[3] == 3 &&
+                   !net.tensors[net.nodes[node].in[0]].is_init;
+        };
+        std::string src[3] = {q, k, m2.in[1]}, result = m2.out[0];
+        const int reader[3] = {idx, ti, m2i};
+        const char *reader_type[3] = {"MatMul", "Transpose", "MatMul"};
+        for (int i = 0; i < 3; ++i) {
+            const int pi = producer_of(src[i]);
+            if (!swaps_heads(pi) || sole_reader(net, src[i], reader_type[i]) != reader[i]) continue;
+            net.tensors[src[i]].never_written = true;
+            src[i] = net.nodes[pi].in[0];
+            m1.token_major[i] = 1;
+            dropped[pi] = true;
+        }
+        const int oi = sole_reader(net, result, "Transpose");
+        if (swaps_heads(oi)) {
+            net.tensors[result].never_written = true;
+            result = net.nodes[oi].out[0];
+            m1.token_major[3] = 1;
+            dropped[oi] = true;
+        }
         m1.fuse = 3;
-        m1.in = {q, k, m2.in[1]};
-        m1.fused_out = m2.out[0];
+        m1.in = {src[0], src[1], src[2]};
+        m1.fused_out = result;
         m1.eval = net.matmul_attention;
         for (const std::string &gone : {tr.out[0], m1.out[0], net.nodes[si].out[0]}) net.tensors[gone].never_written = true;
         dropped[ti] = dropped[idx] = dropped[si] = true;
@@ -775,9 +805,13 @@ int fuse_attention(onrt_net &net) {
 // operand along the leading axes, Gelu/gelu.c).  The reference's optimiser builds the Gelu node itself out of five
 // primitives (tools/optimize/op_fusion.hpp:195-222); folding it into the MatMul goes one operator further, at load time.
 // Only a bias that add.c would broadcast: rank 3 to 6 result, bias [n] (leading axes of extent 1 allowed).
+// A second Add after the bias (no Gelu in between) whose other operand is an activation shaped like the result, the skip
+// connection around a transformer block's projection, goes into the same call (`eval_bias_add`, the addend in
+// inputs[3]); that call takes the place of the second Add in the order, where the addend is complete.
 int fuse_linear(onrt_net &net) {
     if (!fusing_enabled() || !net.matmul_bias) return ONRT_OK;
     std::vector<bool> dropped(net.nodes.size(), false);
+    std::map<int, int> runs_instead;   // second Add -> the MatMul that takes its place
     for (int idx : net.order) {
         Node &mm = net.nodes[idx];
         if (strcmp(mm.kind->type, "MatMul") || mm.in.size() != 2 || mm.out.size() != 1 || mm.fuse) continue;
@@ -808,10 +842,32 @@ int fuse_linear(onrt_net &net) {
             dropped[gi] = true;
         }
         ++net.fused_linears;
+        if (mm.fuse != 4 || !net.matmul_bias_add) continue;
+        const int si = sole_reader(net, add.out[0], "Add");
+        if (si < 0 || runs_instead.count(si)) continue;
+        const Node &skip = net.nodes[si];
+        if (skip.in.size() != 2 || skip.out.size() != 1 || skip.in[0] == skip.in[1]) continue;
+        const std::string &other = skip.in[0] == add.out[0] ? skip.in[1] : skip.in[0];
+        const Tensor &ot = net.tensors[other], &rt = net.tensors[skip.out[0]];
+        if (ot.is_init || !ot.alias.empty() || memcmp(ot.desc.shapes, st.desc.shapes, sizeof(st.desc.shapes)) ||
+            ot.desc.dim_num_of_shapes != st.desc.dim_num_of_shapes || memcmp(rt.desc.shapes, st.desc.shapes, sizeof(st.desc.shapes)))
+            continue;
+        mm.fuse = 6;
+        mm.addend = other;
+        mm.fused_out = skip.out[0];
+        mm.eval = net.matmul_bias_add;
+        net.tensors[add.out[0]].alias = mm.fused_out;
+        net.tensors[mm.out[0]].alias = mm.fused_out;
+        dropped[idx] = true;
+        runs_instead[si] = idx;
+        ++net.fused_skips;
     }
     std::vector<int> order;
-    for (int idx : net.order)
-        if (!dropped[idx]) order.push_back(idx);
+    for (int idx : net.order) {
+        auto it = runs_instead.find(idx);
+        if (it != runs_instead.end()) order.push_back(it->second);
+        else if (!dropped[idx]) order.push_back(idx);
+    }
     net.order.swap(order);
     return ONRT_OK;
 }
@@ -833,7 +889,8 @@ int fill_slots(onrt_net &net) {
             nd.params[1 + slot].addr = (int64_t) &t.desc;
             nd.inputs[slot].addr = (int64_t) t.dev;
         }
-        if (nd.fuse == 1 || nd.fuse == 2) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
+        if (nd.fuse == 3) nd.inputs[4].addr = (int64_t) nd.token_major;
+        if (nd.fuse == 1 || nd.fuse == 2 || nd.fuse == 6) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
             Tensor &t = net.tensors[nd.fused_out.empty() ? nd.out[k] : nd.fused_out];
@@ -883,7 +940,7 @@ int plan(onrt_net &net) {
     int rc = read_model(net);
     if (!rc) rc = order_nodes(net);
     if (!rc) rc = infer_shapes(net);
-    net.conv_add = net.conv_add_relu = net.matmul_attention = net.matmul_bias = net.matmul_bias_gelu = plan_stub_eval;   // as with the plugins of this package
+    net.conv_add = net.conv_add_relu = net.matmul_attention = net.matmul_bias = net.matmul_bias_gelu = net.matmul_bias_add = plan_stub_eval;   // as with the plugins of this package
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = fuse_attention(net);
@@ -1085,6 +1142,12 @@ ONRT_API int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n) {
 ONRT_API int onrt_net_fused_linears(const onrt_net_t *net, int32_t *n) {
     if (!net || !n) return fail(ONRT_ERR_ARG, "fused linear layers: null argument");
     *n = (int32_t) net->fused_linears;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_fused_skips(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "fused skip connections: null argument");
+    *n = (int32_t) net->fused_skips;
     return ONRT_OK;
 }
 

@@ -36,13 +36,13 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quantize_nhwc_s8",
            "onhip_conv2d_w8a8_nhwc", "onhip_quant_weight_bias",
            "onhip_calib_workspace_bytes", "onhip_calib_abs_max", "onhip_calib_histogram", "onhip_calib_threshold", "onhip_calib_percentile",
-           "onhip_matmul", "onhip_gemm_f32", "onhip_copy_f32",
+           "onhip_matmul", "onhip_matmul_add", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
            "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", "onhip_dw_project_supported", "onhip_dw_project_packed_weight_bytes", "onhip_dw_project_pack_weights", "onhip_dw_project_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
-           "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
+           "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
            "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_gelu_eval", "onhip_layernorm_eval",
            "onhip_softmax_eval", "onhip_transpose_eval", "onhip_plugin_set_async", "onhip_plugin_set_stream", "onhip_plugin_forget", "onhip_plugin_trust_weights", "onhip_plugin_release"]
 
@@ -94,6 +94,7 @@ def load():
     L.onhip_quantize_nhwc_s8.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float, vp, vp]
     L.onhip_conv2d_w8a8_nhwc.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
+    L.onhip_matmul_add.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
     L.onhip_copy_f32.argtypes = [vp, vp, C.c_longlong, vp]
     L.onhip_plugin_forget.argtypes = [vp, C.c_size_t]
@@ -115,7 +116,7 @@ def load():
     L.onhip_dw_project_pack_weights.argtypes = [vp, i32, i32, vp, vp]
     L.onhip_dw_project_f32.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp]
     L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
-    for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_gemm_eval"):
+    for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
     _lib = L
     return L
@@ -407,8 +408,9 @@ def conv2d_w8a32(d, x, w8, bias32, weight_aux, silu_lut=None, out=None, acc32=No
     return out
 
 
-def matmul(a, b, bias=None, gelu_lut=None, compute=abi.COMPUTE_F32, out=None):
-    """out = a @ b (b either [K, N] or batched like a), optional fused bias over N and table GELU"""
+def matmul(a, b, bias=None, gelu_lut=None, compute=abi.COMPUTE_F32, out=None, addend=None):
+    """out = a @ b (b either [K, N] or batched like a), optional fused bias over N and table GELU, or (addend given) bias
+    and the Add of a tensor shaped like the result"""
     import torch
     M, K = a.shape[-2], a.shape[-1]
     N = b.shape[-1]
@@ -418,6 +420,12 @@ def matmul(a, b, bias=None, gelu_lut=None, compute=abi.COMPUTE_F32, out=None):
     d = MatmulDesc(batch=batch, m=M, k=K, n=N, b_shared=int(b.numel() == K * N), compute=compute)
     if out is None:
         out = torch.empty(tuple(a.shape[:-1]) + (N,), dtype=torch.float32, device=a.device)
+    if addend is not None:
+        if gelu_lut is not None or tuple(addend.shape) != tuple(out.shape):
+            raise ValueError("matmul: an addend takes the result's shape and excludes the GELU table")
+        _check(load().onhip_matmul_add(C.byref(d), _ptr(a), _ptr(b), _ptr(bias), _ptr(addend), _ptr(out), _stream()),
+               "onhip_matmul_add")
+        return out
     _check(load().onhip_matmul(C.byref(d), _ptr(a), _ptr(b), _ptr(bias), _ptr(gelu_lut), _ptr(out), _stream()),
            "onhip_matmul")
     return out

@@ -98,11 +98,31 @@ def quantised_block():
     return m.tobytes(), [_r("xq", (1, 16, 18, 18))]
 
 
-def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output=False):
+def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output=False, split_heads=()):
     """q, k, v as three inputs [batch, heads, tokens, head_dim]: Transpose of k, MatMul, Softmax, MatMul, the pattern the
-    runtime runs as one attention call (unless the scores are also a net output)"""
+    runtime runs as one attention call (unless the scores are also a net output).  split_heads: which of "q", "k", "v"
+    arrive as [batch, tokens, heads, head_dim] and go through a head-split Transpose (0, 2, 1, 3) first, and whether the
+    result ("o") goes through the head-merge Transpose afterwards."""
     m = onefile.OneModel()
     shape = (batch, heads, tokens, head_dim)
+    flat = (batch, tokens, heads, head_dim)
+    if split_heads:
+        for n in ("q", "k", "v"):
+            if n in split_heads:
+                m.input(n + "_flat", flat)
+                m.transpose(n + "_split", n + "_flat", n, (0, 2, 1, 3))
+            else:
+                m.input(n, shape)
+        m.transpose("kt", "k", "k_t", (0, 1, 3, 2))
+        m.matmul("scores", "q", "k_t", "scores_out")
+        m.softmax("attn", "scores_out", "attn_out")
+        m.matmul("ctx", "attn_out", "v", "ctx_out")
+        if "o" in split_heads:
+            m.transpose("merge", "ctx_out", "merged", (0, 2, 1, 3))
+            m.output("merged", flat)
+        else:
+            m.output("ctx_out", shape)
+        return m.tobytes(), [_r(n + str(tokens), flat if n in split_heads else shape, 0.5) for n in ("q", "k", "v")]
     for n in ("q", "k", "v"):
         m.input(n, shape)
     m.transpose("kt", "k", "k_t", (0, 1, 3, 2))

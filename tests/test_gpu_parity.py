@@ -551,6 +551,30 @@ def test_matmul_bias_gelu_fused(compute, batch, torch_dev, oracle):
         assert np.mean(y == ref) > 0.98 and np.abs(y - ref).max() < 5e-3
 
 
+@pytest.mark.parametrize("compute", [abi.COMPUTE_F32, abi.COMPUTE_BF16])
+@pytest.mark.parametrize("shape", [((4, 197, 192), (192, 192)), ((2, 196, 768), (768, 192)), ((3, 37, 50), (3, 50, 21))])
+def test_matmul_bias_add_fused(shape, compute, torch_dev, oracle):
+    """MatMul -> Add of a bias -> Add of a skip tensor in one call == the three operators one after the other (the sums are
+    formed in the same order on the same values: bit for bit), and, in fp32, the oracle's chain within 1e-4"""
+    torch = torch_dev
+    a, w = cases.matmul_inputs("vit_proj", *shape)
+    n = shape[1][-1]
+    bias = cases.datagen.normal(cases.datagen.seed_for("vit_proj", "bias", n), (n,), 0.0, 0.05)
+    skip = cases.datagen.normal(cases.datagen.seed_for("vit_proj", "skip", n), shape[0][:-1] + (n,), 0.0, 1.0)
+    for b in (bias, None):
+        kw = dict(bias=dev(torch, b)) if b is not None else {}
+        y = hip.matmul(dev(torch, a), dev(torch, w), addend=dev(torch, skip), compute=compute, **kw)
+        pre = hip.matmul(dev(torch, a), dev(torch, w), compute=compute, **kw)
+        torch.cuda.synchronize()
+        y, pre = y.cpu().numpy(), pre.cpu().numpy()
+        assert np.array_equal(y, oracle.add_f32(pre, skip))
+        if compute == abi.COMPUTE_F32:
+            assert_close_f32(y, oracle.add_f32(oracle.matmul_f32(a, w, bias=b), skip), rel=1e-4, tag="proj + skip")
+    with pytest.raises(hip.OnhipError):
+        out = dev(torch, skip)
+        hip.matmul(dev(torch, a), dev(torch, w), addend=out, out=out)
+
+
 @pytest.mark.parametrize("name", list(cases.gemm_cases()))
 def test_gemm_f32(name, torch_dev, oracle, golden):
     torch = torch_dev

@@ -188,10 +188,10 @@ def test_vit_encoder_through_the_runtime(torch_dev, monkeypatch):
     x = np.random.default_rng(5).normal(size=shape).astype(np.float32)
     ref = one_model.run(data, [x])[0]
     fused = rt.Net(data)
-    assert fused.fused_attentions() == 2 and fused.fused_linears() == 12
+    assert fused.fused_attentions() == 2 and fused.fused_linears() == 12 and fused.fused_skips() == 4
     monkeypatch.setenv("ONENEW_RT_FUSE", "0")
     plain = rt.Net(data)
-    assert len(plain.ops()) == len(onefile.parse(data)["nodes"]) and len(fused.ops()) == len(plain.ops()) - 2 * 3 - 14
+    assert len(plain.ops()) == len(onefile.parse(data)["nodes"]) and len(fused.ops()) == len(plain.ops()) - 2 * 7 - 14 - 4
     for net in (fused, plain):
         got = net.run(x)[0]
         assert got.shape == ref.shape and _close(got, ref, 1e-3), float(np.abs(got - ref).max())
@@ -200,8 +200,9 @@ def test_vit_encoder_through_the_runtime(torch_dev, monkeypatch):
 
 
 def test_linear_layers_run_as_one_call_bit_for_bit(torch_dev, monkeypatch):
-    """MatMul -> Add of a bias -> Gelu and MatMul -> Add of a bias as one call each: the operands behind them hold exactly
-    what the separate operators produce (the bias is added to the finished sum, the table is read with the same index)"""
+    """MatMul -> Add of a bias -> Gelu, MatMul -> Add of a bias, and MatMul -> Add of a bias -> Add of a skip connection as
+    one call each: the operands behind them hold exactly what the separate operators produce (the bias is added to the
+    finished sum, the table is read with the same index, the skip tensor is added last)"""
     m = onefile.OneModel()
     rng = np.random.default_rng(3)
     w = lambda *s: (rng.normal(size=s) * 0.2).astype(np.float32)   # noqa: E731
@@ -213,19 +214,56 @@ def test_linear_layers_run_as_one_call_bit_for_bit(torch_dev, monkeypatch):
     m.add("fc2_bias", "fc2_out", w(1, 1, 40), "fc2_b")                # leading axes of extent 1
     m.matmul("fc3", "fc2_b", w(40, 24), "fc3_out")
     m.add("not_a_bias", "fc3_out", w(2, 50, 24), "y")                 # a full tensor: stays an Add
+    m.matmul("proj", "act_out", w(96, 48), "proj_out")
+    m.add("proj_bias", "proj_out", w(48), "proj_b")
+    m.add("skip", "x", "proj_b", "z")                                  # the block's input around it
+    m.matmul("fc4", "z", w(48, 48), "fc4_out")
+    m.add("fc4_bias", "fc4_out", w(48), "fc4_b")
+    m.add("skip_with_two_readers", "fc4_b", "z", "z2")                 # fc4_b is also an output: that Add stays
     m.output("act_out", (2, 50, 96))
     m.output("y", (2, 50, 24))
+    m.output("z", (2, 50, 48))
+    m.output("fc4_b", (2, 50, 48))
+    m.output("z2", (2, 50, 48))
     data, x = m.tobytes(), rng.normal(size=(2, 50, 48)).astype(np.float32)
     monkeypatch.setenv("ONENEW_RT_FUSE", "0")
     plain = rt.Net(data)
     monkeypatch.delenv("ONENEW_RT_FUSE")
     fused = rt.Net(data)
-    assert plain.fused_linears() == 0 and fused.fused_linears() == 2
-    assert [t for t, _ in fused.ops()] == ["MatMul", "MatMul", "MatMul", "Add"]
+    assert plain.fused_linears() == 0 and fused.fused_linears() == 4
+    assert plain.fused_skips() == 0 and fused.fused_skips() == 1
+    assert [t for t, _ in fused.ops()] == ["MatMul", "MatMul", "MatMul", "Add", "MatMul", "MatMul", "Add"]
     for got, ref in zip(fused.run(x), plain.run(x)):
         assert np.array_equal(got, ref)
     assert np.array_equal(fused.fetch("fc2_b"), plain.fetch("fc2_b"))
     assert fused.operand("fc1_out")[1] == fused.operand("fc1_b")[1] == fused.operand("act_out")[1]
+    assert fused.operand("proj_out")[1] == fused.operand("proj_b")[1] == fused.operand("z")[1]
+    # a second run on another input: the folded call reads the skip tensor afresh
+    x2 = (x * np.float32(-0.5) + np.float32(0.1)).astype(np.float32)
+    for got, ref in zip(fused.run(x2), plain.run(x2)):
+        assert np.array_equal(got, ref)
+    plain.close()
+    fused.close()
+
+
+@pytest.mark.parametrize("split", ["qkvo", "kv", "qo", "o"])
+def test_attention_block_takes_in_the_head_transposes(split, torch_dev, monkeypatch):
+    """head-split Transposes (0, 2, 1, 3) in front of q, k, v and the head-merge one behind the result fold into the
+    attention call's strides: as many operators fewer, the net's output within 1e-4 of the net run operator by operator
+    (which has the same values as the plain attention block, in another order in memory)"""
+    data, ins = one_models.attention_heads(heads=3, tokens=50, head_dim=64, batch=2, split_heads=tuple(split))
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    plain = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    fused = rt.Net(data)
+    assert fused.fused_attentions() == 1 and [t for t, _ in fused.ops()] == ["MatMul"]
+    assert len(plain.ops()) == 4 + len(split)
+    for name in [n for n in "qkv" if n in split]:
+        assert fused.operand(name)[1] is None
+    for scale in (1.0, -0.6):
+        xs = [x * np.float32(scale) for x in ins]
+        for got, ref in zip(fused.run(*xs), plain.run(*xs)):
+            assert got.shape == ref.shape and np.all(np.abs(got - ref) <= 1e-4 * np.abs(ref) + 1e-5)
     plain.close()
     fused.close()
 
@@ -242,10 +280,11 @@ def test_attention_block_runs_as_one_call(model, torch_dev, monkeypatch):
     monkeypatch.delenv("ONENEW_RT_FUSE")
     fused = rt.Net(data)
     assert plain.fused_attentions() == 0 and fused.fused_attentions() == 1
-    # vit_block also has two linear layers (MatMul -> Add -> Gelu and MatMul -> Add): three more operators folded away
+    # vit_block also has two linear layers (MatMul -> Add -> Gelu and MatMul -> Add -> Add of the skip connection): four
+    # more operators folded away
     linears = 2 if model == "vit_block" else 0
     assert plain.fused_linears() == 0 and fused.fused_linears() == linears
-    assert len(fused.ops()) == len(plain.ops()) - 3 - (3 if linears else 0)
+    assert len(fused.ops()) == len(plain.ops()) - 3 - (4 if linears else 0)
     assert fused.operand("scores_out")[1] is None and fused.operand("attn_out")[1] is None
     for scale in (1.0, -0.7):
         xs = [x * np.float32(scale) for x in ins]

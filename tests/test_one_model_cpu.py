@@ -191,9 +191,14 @@ def test_plan_runs_an_attention_block_as_one_call(monkeypatch):
     assert net.fused_attentions() == 1 and [t for t, _ in net.ops()] == ["MatMul"]
     data, _ = one_models.vit_block()                       # q = k = v = one tensor, behind a Reshape
     net = rt.Net(data, plan_only=True)
-    # and two linear layers in front: MatMul -> Add -> Gelu, MatMul -> Add (three more operators folded away)
-    assert net.fused_attentions() == 1 and net.fused_linears() == 2
-    assert len(net.ops()) == len(onefile.parse(data)["nodes"]) - 3 - 3
+    # and two linear layers in front: MatMul -> Add -> Gelu, MatMul -> Add -> Add of the skip connection (four more
+    # operators folded away)
+    assert net.fused_attentions() == 1 and net.fused_linears() == 2 and net.fused_skips() == 1
+    assert len(net.ops()) == len(onefile.parse(data)["nodes"]) - 3 - 4
+    # head-split Transposes in front of q, k, v and the head-merge one behind the result go into the same call
+    for split in ("qkvo", "k", "qo"):
+        net = rt.Net(one_models.attention_heads(split_heads=tuple(split))[0], plan_only=True)
+        assert net.fused_attentions() == 1 and [t for t, _ in net.ops()] == ["MatMul"], split
     for kw in (dict(head_dim=48), dict(tokens=300), dict(scores_also_output=True)):
         net = rt.Net(one_models.attention_heads(**kw)[0], plan_only=True)
         assert net.fused_attentions() == 0 and len(net.ops()) == 4, kw
