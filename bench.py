@@ -309,6 +309,37 @@ class DwProjectLayer:
         return f1 + f2, lambda: (r1(), r2())
 
 
+class IrBlockLayer:
+    """a whole inverted-residual block (1x1 expansion + CLIP, depthwise 3x3 + CLIP, 1x1 projection) in one launch: neither
+    wide tensor leaves the chip; work and bytes are counted as the three separate convolutions' (every tensor of the
+    unfused chain once), so the figures stay comparable with the layer-by-layer stack"""
+    kind = "ir_block"
+
+    def __init__(self, torch, hip, name, ex, dw, pw, tag):
+        from onenew_amd import datagen
+        self.name, self.ex, self.dw, self.pw = name.replace(".expand", "") + ".block", ex, dw, pw
+        self.x = device_uniform(torch, datagen.seed_for(f"{tag}/{name}", "x"), (ex.n, ex.cin, ex.h, ex.w))
+        g = lambda role, shape, std: torch.from_numpy(datagen.normal(datagen.seed_for(f"{tag}/{name}", role), shape, 0.0, std)).cuda()
+        self.ex_w, self.ex_b = g("w", (ex.cout, ex.cin, 1, 1), float(np.sqrt(2.0 / ex.cin))), g("b", (ex.cout,), 0.01)
+        self.dw_w, self.dw_b = g("dw", (dw.cout, 1, 3, 3), float(np.sqrt(2.0 / 9))), g("db", (dw.cout,), 0.01)
+        self.pw_w, self.pw_b = g("pw", (pw.cout, pw.cin, 1, 1), float(np.sqrt(2.0 / pw.cin))), g("pb", (pw.cout,), 0.01)
+        self.packed = hip.ir_block_pack_weights(self.ex_w, self.pw_w)
+        oh, ow = dw.out_hw()
+        self.y = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device="cuda")
+        self.flops = ex.flops() + dw.flops() + pw.flops()
+        self.bytes = ex.algorithmic_bytes() + dw.algorithmic_bytes() + pw.algorithmic_bytes()
+        self.dense = False           # counted against the memory traffic of the chain it replaces
+        self.shape = f"C={ex.cin}>{dw.cin}>{pw.cout} N={dw.n * oh * ow} s{dw.stride_h}"
+
+    def launch(self, hip):
+        hip.ir_block_f32(self.ex, self.dw, self.pw, self.x, self.packed, self.ex_b, self.dw_w, self.dw_b, self.pw_b, out=self.y)
+
+    def cpu_runner(self, ops, oracle, tag):
+        runs = [ConvF32Layer.cpu_runner(type("L", (), {"d": d, "name": self.name + sfx})(), ops, oracle, tag)
+                for d, sfx in ((self.ex, "/ex"), (self.dw, "/dw"), (self.pw, "/pw"))]
+        return sum(f for f, _ in runs), lambda: [r() for _, r in runs]
+
+
 class ConvH16Layer:
     """dense convolution with bf16 / fp16 storage: 16-bit NHWC in, 16-bit NHWC out, weights packed once"""
     kind = "conv_h16"
@@ -501,9 +532,16 @@ def make_workload(torch, hip, name):
     if name.startswith("mobilenetv2_b"):
         n = int(name.split("_b")[1].split("_")[0])
         spec = stacks.with_batch(stacks.mobilenet_v2(), n)
-        layers, fused, i = [], 0, 0
+        layers, fused, blocks, i = [], 0, 0, 0
         while i < len(spec):
             ln, d = spec[i]
+            # expansion, depthwise and projection in one launch where the block kernel takes the shapes
+            if (not name.endswith("_unfused") and not name.endswith("_noblocks") and i + 2 < len(spec) and d.group == 1
+                    and hip.ir_block_supported(d, spec[i + 1][1], spec[i + 2][1]) >= 2):
+                layers.append(IrBlockLayer(torch, hip, ln, d, spec[i + 1][1], spec[i + 2][1], tag))
+                blocks += 1
+                i += 3
+                continue
             # a depthwise convolution and the projection behind it in one launch where the library recommends it
             want = 1 if name.endswith("_fusedall") else 2
             if (not name.endswith("_unfused") and d.group != 1 and i + 1 < len(spec)
@@ -514,8 +552,8 @@ def make_workload(torch, hip, name):
             else:
                 layers.append(ConvF32Layer(torch, hip, ln, d, tag))
                 i += 1
-        return (f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers (17 depthwise), ReLU6 as CLIP; {fused} depthwise + "
-                f"projection pairs as one launch each", "f32", layers)
+        return (f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers (17 depthwise), ReLU6 as CLIP; {blocks} whole inverted-residual blocks "
+                f"and {fused} depthwise + projection pairs as one launch each", "f32", layers)
     if name == "cfg1":
         import cases
         return ("Conv2d+ReLU fp32 64->64 56x56 3x3 s1 p1, batch 1", "f32",

@@ -265,6 +265,25 @@ int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *p
                          const float *dw_b, const float *pw_packed, const float *pw_b, const float *residual, float *y,
                          void *stream);
 
+/* A whole inverted-residual block in one launch: 1x1 convolution (bias, activation) -> depthwise 3x3 (pads 1, stride 1 or
+ * 2, bias, activation) -> 1x1 convolution (bias, activation) [-> Add of a residual tensor shaped like the output].
+ * Replaces three (four) operator evaluations, device/x86/Conv/conv.c 1x1 path :1024-1056 twice and depthwise path :757-899
+ * (and device/x86/Add/add.c); neither wide tensor of the block is written to memory.  fp32; the depthwise stage performs
+ * the separate operator's operations in its order, the two 1x1 stages sum in MFMA order, so the block equals the chain of
+ * operators within fp32 summation error.  No counterpart as one function in the reference.
+ * onhip_ir_block_supported: 0 = this triple is not taken (16, 24, 32 or 64 input channels, expanded channels a multiple
+ * of 16, at most 64 output channels, rows of a multiple of 4 and at most 128 output pixels, biases on the first two
+ * convolutions), 1 = taken, 2 = taken and expected to be faster than the three launches (at least 256 bands of output rows
+ * over the batch).  packed: both 1x1 weight tensors ([ce][cin] and [co][ce]) re-laid once by
+ * onhip_ir_block_pack_weights (onhip_ir_block_packed_weight_bytes(cin, ce, co) bytes, 16-byte aligned). */
+int onhip_ir_block_supported(const onhip_conv_desc_t *expand, const onhip_conv_desc_t *dw, const onhip_conv_desc_t *project);
+size_t onhip_ir_block_packed_weight_bytes(int32_t cin, int32_t ce, int32_t co);
+int onhip_ir_block_pack_weights(const float *expand_w, const float *project_w, int32_t cin, int32_t ce, int32_t co, float *packed,
+                                void *stream);
+int onhip_ir_block_f32(const onhip_conv_desc_t *expand, const onhip_conv_desc_t *dw, const onhip_conv_desc_t *project, const float *x,
+                       const float *packed, const float *expand_b, const float *dw_w, const float *dw_b, const float *project_b,
+                       const float *residual, float *y, void *stream);
+
 /* Attention of every (batch, head) in one launch:  out = Softmax(q k^T * scale) v, Softmax over the keys.  Replaces the
  * operator chain MatMul (device/x86/MatMul/mat_mul.c:10-102) -> [Mul by a constant] -> Softmax (device/x86/Softmax/
  * softmax.c:26-59) -> MatMul of a transformer block, together with the Transposes (device/x86/Transpose/transpose.c)

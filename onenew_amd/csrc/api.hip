@@ -1298,6 +1298,63 @@ int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *p
                              make_epilogue(*pw, nullptr), y, reinterpret_cast<hipStream_t>(stream));
 }
 
+// the expansion -> depthwise -> projection triple the one-launch block kernel takes
+static bool ir_block_shapes_ok(const onhip_conv_desc_t *ex, const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const char **why) {
+    const char *w = nullptr;
+    int32_t EH = 0, EW = 0, OH = 0, OW = 0;
+    if (!dw_project_shapes_ok(dw, pw, &w)) {
+    } else if (!ex || check_conv(ex, &EH, &EW)) w = "bad expansion descriptor";
+    else if (ex->group != 1 || ex->kh != 1 || ex->kw != 1 || ex->stride_h != 1 || ex->stride_w != 1 || ex->pad_t || ex->pad_l || ex->pad_b || ex->pad_r)
+        w = "the first convolution must be 1x1, stride 1, unpadded";
+    else if (ex->compute != ONHIP_COMPUTE_F32 || ex->act_type == SILU || !ex->has_bias) w = "the expansion must be fp32 with a bias and no table activation";
+    else if (ex->cout != dw->cin || ex->n != dw->n || ex->h != dw->h || ex->w != dw->w) w = "the depthwise convolution does not take the expansion's output";
+    else if (!irblock_cin_ok(ex->cin)) w = "16, 24, 32 or 64 input channels";
+    else if (pw->cout > 64) w = "at most 64 output channels";
+    else if (onhip_conv_out_shape(dw, &OH, &OW) || irblock_band_rows(*dw, OH, OW, ex->cin) < 1) w = "no band of output rows fits the kernel (row length a multiple of 4, at most 128 output pixels)";
+    else if ((long long) ex->n * ex->cin * ex->h * ex->w * 4 >= (1LL << 31)) w = "tensors of 2 GiB or more";
+    if (why) *why = w;
+    return w == nullptr;
+}
+
+int onhip_ir_block_supported(const onhip_conv_desc_t *expand, const onhip_conv_desc_t *dw, const onhip_conv_desc_t *project) {
+    if (!ir_block_shapes_ok(expand, dw, project, nullptr)) return 0;
+    // One workgroup per band of output rows and image, a few tens of microseconds each whatever the batch: below one
+    // workgroup per compute unit the three separate launches, which spread over the whole chip, finish first (MobileNetV2
+    // at batch 1: 28 workgroups).  Measured on MobileNetV2 at batch 64, one launch against three: 130 / 191 us (16 -> 96 ->
+    // 24 channels, 112 x 112, stride 2), 104 / 121 (24 -> 144 -> 24, 56 x 56), 76 / 86, 44 / 54, 44 / 52.
+    int32_t OH = 0, OW = 0;
+    (void) onhip_conv_out_shape(dw, &OH, &OW);
+    const int rows = irblock_band_rows(*dw, OH, OW, expand->cin);
+    return (long long) dw->n * ((OH + rows - 1) / rows) >= 256 ? 2 : 1;
+}
+
+size_t onhip_ir_block_packed_weight_bytes(int32_t cin, int32_t ce, int32_t co) {
+    return cin < 1 || ce < 1 || co < 1 ? 0 : ((size_t) ce * cin + (size_t) ce * ((co + 31) / 32 * 32)) * sizeof(float);
+}
+
+int onhip_ir_block_pack_weights(const float *expand_w, const float *project_w, int32_t cin, int32_t ce, int32_t co, float *packed, void *stream) {
+    if (!expand_w || !project_w || !packed || cin < 4 || cin % 4 || ce < 16 || ce % 16 || co < 1 || reinterpret_cast<uintptr_t>(packed) % 16)
+        return set_error(ONHIP_ERR_ARG, "inverted-residual block pack: bad argument");
+    return irblock_pack_launch(expand_w, project_w, cin, ce, co, packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_ir_block_f32(const onhip_conv_desc_t *expand, const onhip_conv_desc_t *dw, const onhip_conv_desc_t *project, const float *x,
+                       const float *packed, const float *expand_b, const float *dw_w, const float *dw_b, const float *project_b,
+                       const float *residual, float *y, void *stream) {
+    const char *why = nullptr;
+    if (!ir_block_shapes_ok(expand, dw, project, &why)) return set_error(ONHIP_ERR_ARG, "inverted-residual block: %s", why);
+    if (!x || !packed || !expand_b || !dw_w || !dw_b || !y || (project->has_bias && !project_b))
+        return set_error(ONHIP_ERR_ARG, "inverted-residual block: null tensor pointer");
+    if (reinterpret_cast<uintptr_t>(packed) % 16 || reinterpret_cast<uintptr_t>(x) % 16)
+        return set_error(ONHIP_ERR_ARG, "inverted-residual block: input and packed weights must be 16-byte aligned");
+    if (residual == y || x == y) return set_error(ONHIP_ERR_ARG, "inverted-residual block: the output buffer may not be an input");
+    int32_t OH = 0, OW = 0;
+    (void) onhip_conv_out_shape(dw, &OH, &OW);
+    return irblock_f32_launch(*expand, *dw, *project, OH, OW, x, packed, expand_b, dw_w, dw_b, project->has_bias ? project_b : nullptr, residual,
+                              make_epilogue(*expand, nullptr), make_epilogue(*dw, nullptr), make_epilogue(*project, nullptr), y,
+                              reinterpret_cast<hipStream_t>(stream));
+}
+
 int onhip_attention(const onhip_attention_desc_t *d, const void *q, const void *k, const void *v, void *out, void *stream) {
     if (!d || d->batch < 1 || d->heads < 1 || d->tokens < 1) return set_error(ONHIP_ERR_ARG, "attention: bad shape");
     if (!q || !k || !v || !out) return set_error(ONHIP_ERR_ARG, "attention: null tensor pointer");

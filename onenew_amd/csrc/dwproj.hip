@@ -194,21 +194,32 @@ __global__ __launch_bounds__(256, 2) void dwproj_f32_kernel(const DwProjParams p
 
     // store: lane = pixel of the band (rows of a band are contiguous in NCHW), rows 8 (r / 4) + 4 lh + r % 4 of each tile
     const bool col_ok = q < min(p.band_rows, p.oh - oh0) * p.ow;
+    const bool plain = !has_bias || p.pw_ep.act == NOT_ACT;   // conv.c:18-27: without a bias the activation is skipped too
+    // every bias and residual value is requested before the first one is used: one memory round trip for the store
+    float bias[MT][16], resv[MT][16];
+    unsigned off[MT][16];
 #pragma unroll
-    for (int a = 0; a < MT; ++a) {
-        if (a * 32 >= p.co) break;   // uniform
+    for (int a = 0; a < MT; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m = a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
             const bool ok = col_ok && m < p.co;
-            const unsigned off = ok ? (unsigned) ((img * p.co + m) * OHW + oh0 * p.ow + q) * 4u : OOB;
-            float v = acc[a][r];
-            const float vb = __fadd_rn(v, buf_load_f32(rb, ok ? (unsigned) m * 4u : OOB, 0));
-            v = has_bias ? apply_act(vb, p.pw_ep) : v;   // conv.c:18-27: without a bias the activation is skipped too
-            if (has_res) v = __fadd_rn(v, buf_load_f32(rr, off, 0));
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), ry, off, 0, 0);
+            off[a][r] = ok ? (unsigned) ((img * p.co + m) * OHW + oh0 * p.ow + q) * 4u : OOB;
+            bias[a][r] = buf_load_f32(rb, (unsigned) m * 4u, 0);   // past the last channel, or no bias: zero
+            resv[a][r] = buf_load_f32(rr, off[a][r], 0);          // no residual: an empty buffer, zeros
         }
-    }
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = acc[a][r];
+            const float vb = __fadd_rn(v, bias[a][r]);
+            v = has_bias ? vb : v;
+            if (!plain) v = apply_act(v, p.pw_ep);
+            const float vr = __fadd_rn(v, resv[a][r]);
+            v = has_res ? vr : v;
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), ry, off[a][r], 0, 0);
+        }
 }
 
 __global__ __launch_bounds__(256) void dwproj_pack_kernel(const float *w, int ce, int co, int cop, float *packed) {

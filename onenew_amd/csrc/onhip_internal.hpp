@@ -243,6 +243,14 @@ int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, flo
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
 int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
 int forget_quantised_tables(const void *base, size_t bytes);   // api.hip: the cache of tables behind an output quantiser
+// irblock.hip: 1x1 expansion -> depthwise 3x3 -> 1x1 projection in one launch
+int irblock_pack_launch(const float *w_exp, const float *w_proj, int cin, int ce, int co, float *packed, hipStream_t stream);
+int irblock_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int cin);
+bool irblock_cin_ok(int cin);
+int irblock_f32_launch(const onhip_conv_desc_t &ex, const onhip_conv_desc_t &dw, const onhip_conv_desc_t &pw, int OH, int OW, const float *x,
+                       const float *packed, const float *exp_b, const float *dw_w, const float *dw_b, const float *pw_b, const float *res,
+                       const Epilogue &exp_ep, const Epilogue &dw_ep, const Epilogue &pw_ep, float *y, hipStream_t stream);
+
 // dwproj.hip: depthwise 3x3 -> 1x1 convolution in one launch
 int dwproj_pack_launch(const float *w, int ce, int co, float *packed, hipStream_t stream);
 int dwproj_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int co);

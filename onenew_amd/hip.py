@@ -40,6 +40,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
            "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", "onhip_dw_project_supported", "onhip_dw_project_packed_weight_bytes", "onhip_dw_project_pack_weights", "onhip_dw_project_f32",
+           "onhip_ir_block_supported", "onhip_ir_block_packed_weight_bytes", "onhip_ir_block_pack_weights", "onhip_ir_block_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
@@ -115,6 +116,11 @@ def load():
     L.onhip_dw_project_packed_weight_bytes.restype = C.c_size_t
     L.onhip_dw_project_pack_weights.argtypes = [vp, i32, i32, vp, vp]
     L.onhip_dw_project_f32.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp]
+    L.onhip_ir_block_supported.argtypes = [C.POINTER(ConvDesc)] * 3
+    L.onhip_ir_block_packed_weight_bytes.argtypes = [i32, i32, i32]
+    L.onhip_ir_block_packed_weight_bytes.restype = C.c_size_t
+    L.onhip_ir_block_pack_weights.argtypes = [vp, vp, i32, i32, i32, vp, vp]
+    L.onhip_ir_block_f32.argtypes = [C.POINTER(ConvDesc)] * 3 + [vp] * 9
     L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
@@ -548,6 +554,32 @@ def dw_project_f32(dw, pw, x, dw_w, dw_b, pw_packed, pw_b=None, residual=None, o
         out = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device=x.device)
     _check(load().onhip_dw_project_f32(C.byref(dw), C.byref(pw), _ptr(x), _ptr(dw_w), _ptr(dw_b), _ptr(pw_packed), _ptr(pw_b),
                                        _ptr(residual), _ptr(out), _stream()), "onhip_dw_project_f32")
+    return out
+
+
+def ir_block_supported(ex, dw, pw):
+    return load().onhip_ir_block_supported(C.byref(ex), C.byref(dw), C.byref(pw))
+
+
+def ir_block_pack_weights(expand_w, project_w):
+    """the two 1x1 weight tensors of an inverted-residual block, [ce, cin(, 1, 1)] and [cout, ce(, 1, 1)] -> the layout of
+    the one-launch block kernel"""
+    import torch
+    ce, cin, co = expand_w.shape[0], expand_w.shape[1], project_w.shape[0]
+    out = torch.empty(load().onhip_ir_block_packed_weight_bytes(cin, ce, co) // 4, dtype=torch.float32, device=expand_w.device)
+    _check(load().onhip_ir_block_pack_weights(_ptr(expand_w), _ptr(project_w), cin, ce, co, _ptr(out), _stream()),
+           "onhip_ir_block_pack_weights")
+    return out
+
+
+def ir_block_f32(ex, dw, pw, x, packed, expand_b, dw_w, dw_b, project_b=None, residual=None, out=None):
+    """1x1 expansion -> depthwise 3x3 -> 1x1 projection [-> Add of residual] in one launch"""
+    import torch
+    oh, ow = dw.out_hw()
+    if out is None:
+        out = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device=x.device)
+    _check(load().onhip_ir_block_f32(C.byref(ex), C.byref(dw), C.byref(pw), _ptr(x), _ptr(packed), _ptr(expand_b), _ptr(dw_w), _ptr(dw_b),
+                                     _ptr(project_b), _ptr(residual), _ptr(out), _stream()), "onhip_ir_block_f32")
     return out
 
 

@@ -143,6 +143,54 @@ def test_mobilenetv2_batch64_every_layer(layer, torch_dev, oracle):
         _check_dense_f32(torch_dev, "mbv2b64", name, d, w_std=0.05)
 
 
+# the inverted-residual blocks the benchmark runs as one launch each (expansion, depthwise, projection)
+IR_BLOCKS = [i for i in range(len(MOBILENET) - 2)
+             if MOBILENET[i][1].group == 1 and MOBILENET[i + 1][1].group != 1 and MOBILENET[i][1].kh == 1]
+
+
+@pytest.mark.parametrize("first", IR_BLOCKS, ids=[MOBILENET[i][0].replace(".expand", "") for i in IR_BLOCKS])
+def test_mobilenetv2_batch64_blocks_in_one_launch(first, torch_dev, oracle):
+    """every block the library recommends for the one-launch kernel at batch 64: three whole images against the oracle's
+    chain of the three convolutions (1e-4 of the largest value), and the other images through the fact that an image's
+    result depends on its own input alone"""
+    torch = torch_dev
+    (name, ex), (_, dw), (_, pw) = MOBILENET[first], MOBILENET[first + 1], MOBILENET[first + 2]
+    want = hip.ir_block_supported(ex, dw, pw)
+    print(f"mobilenetv2 b64 block {name}: supported = {want}", flush=True)
+    if want < 2:
+        pytest.skip("not a shape of the one-launch block kernel: the benchmark runs its three convolutions")
+    x = _device_uniform(torch, _seed("mbv2blk", name, "x"), (ex.n, ex.cin, ex.h, ex.w))
+    r = lambda role, shape, std, mean=0.0: datagen.normal(_seed("mbv2blk", name, role), shape, mean, std)   # noqa: E731
+    ex_w, ex_b = r("exw", (ex.cout, ex.cin, 1, 1), float(np.sqrt(2.0 / ex.cin))), r("exb", (ex.cout,), 0.3, 0.3)
+    dw_w, dw_b = r("dww", (dw.cout, 1, 3, 3), 0.4), r("dwb", (dw.cout,), 0.2)
+    pw_w, pw_b = r("pww", (pw.cout, pw.cin, 1, 1), float(np.sqrt(1.0 / pw.cin))), r("pwb", (pw.cout,), 0.1)
+    cu = lambda a: torch.from_numpy(a).cuda()   # noqa: E731
+    packed = hip.ir_block_pack_weights(cu(ex_w), cu(pw_w))
+    args = (packed, cu(ex_b), cu(dw_w), cu(dw_b), cu(pw_b))
+    y = hip.ir_block_f32(ex, dw, pw, x, *args)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y).all())
+    one = [ConvDesc.from_buffer_copy(d) for d in (ex, dw, pw)]
+    for d in one:
+        d.n = 1
+    pick = sorted({0, ex.n - 1, int(datagen.integers(_seed("mbv2blk", name, "img"), (1,), 0, ex.n - 1)[0])})
+    for img in pick:
+        wide = oracle.conv2d_f32(one[0], x[img:img + 1].cpu().numpy(), ex_w, ex_b)
+        ref = oracle.conv2d_f32(one[2], oracle.conv2d_f32(one[1], wide, dw_w, dw_b), pw_w, pw_b).astype(np.float64)
+        got = y[img:img + 1].cpu().numpy().astype(np.float64)
+        top = np.abs(ref).max()
+        assert np.abs(got - ref).max() <= 1e-4 * top, f"{name} image {img}: {np.abs(got - ref).max():.3e} against {top:.3e}"
+        assert np.all(np.abs(got - ref) <= 1e-4 * np.abs(ref) + 1e-5 * top), name
+    a, c = pick[0], (pick[0] + 1) % ex.n
+    x2 = x.clone()
+    x2[c] = x[a]
+    y2 = hip.ir_block_f32(ex, dw, pw, x2, *args)
+    torch.cuda.synchronize()
+    assert torch.equal(y2[c], y[a])
+    keep = [k for k in range(ex.n) if k != c]
+    assert torch.equal(y2[keep], y[keep])
+
+
 # ---- ViT-Tiny MatMuls at B = 64 -------------------------------------------------------------------------------
 
 VIT = stacks.vit_tiny(64)
