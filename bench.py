@@ -808,7 +808,8 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False, graph=True
               if dom_dense and grp[0][0].kind in ("conv_h16", "linear_h16") else
               f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
               "element-wise / pooling / normalisation kernels (elementwise.hip, vit_glue.hip)" if grp[0][0].kind == "glue"
-              else "onhip::depthwise_tiled_kernel")
+              else "onhip::irblock_f32_kernel (expansion + depthwise + projection in one launch) and onhip::depthwise_tiled_kernel"
+              if any(L.kind == "ir_block" for L, _ in grp) else "onhip::depthwise_tiled_kernel")
     # the bound is the roof the group's arithmetic intensity puts it under
     mfma_bound = dom_dense and g_flops / g_bytes >= PEAK[dtype] * 1e12 / (HBM_PEAK_GBS * 1e9)
     if mfma_bound:

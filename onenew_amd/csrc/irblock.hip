@@ -10,7 +10,8 @@
 //     W_exp[16 x cin] . Xs[cin x patch pixels] (v_mfma_f32_16x16x4_f32: A = weights[m = lane % 16][k = lane / 16], packed
 //     once so that a lane's values are consecutive words; B = Xs[k = lane / 16][pixel = lane % 16]; D = [m = 4 (lane / 16)
 //     + r][pixel = lane % 16]) whose result goes, with bias and activation, into the LDS patch the depthwise stage reads:
-//     [channel][input row][1 + w + 1], a zero column on either side, rows above / below the image left zero.  Halo rows
+//     [channel / 4][input row][1 + w + 1][channel % 4], a zero column on either side, rows above / below the image left
+//     zero; a lane's four values are one 16-byte store, and the depthwise stage reads a tap of four channels at once.  Halo rows
 //     are expanded by both neighbouring bands: (rows + 2) / rows (stride 1) of the expansion's arithmetic, none of its
 //     memory traffic;
 //   * depthwise and projection as in dwproj.hip: taps added in ascending (i, j) order to a zero sum, multiply and add
@@ -31,7 +32,8 @@ namespace onhip {
 
 constexpr int IR_BN = 128;        // output pixels of a band, at most
 constexpr int IR_KC = 16;         // expanded channels per chunk
-constexpr int IR_XSLOTS = 12;     // 16-byte input loads per thread, at most
+constexpr int IR_XSLOTS = 12;
+constexpr int IR_TPW = 9;         // pixel tiles of the expansion per wavefront, at most     // 16-byte input loads per thread, at most
 constexpr int IR_LDS_HALF = 80 * 1024;   // bytes of LDS a workgroup may take: two workgroups per compute unit
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256, 2) void irblock_f32_kernel(const IrParams p) {
     const int chunks = p.ce / IR_KC;
 
     // the whole patch to zero once: padding columns and the rows outside the image stay that way
-    for (int f = tid; f < NBUF * p.patch_floats; f += 256) patch0[f] = 0.0f;
+    for (int f = tid; f < NBUF * p.patch_floats / 4; f += 256) reinterpret_cast<float4 *>(patch0)[f] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 
     // block input: channel c, floats [0, P) of the rows ih_first .. (contiguous in memory), rows outside the image zero
     {
@@ -149,15 +151,25 @@ __global__ __launch_bounds__(256, 2) void irblock_f32_kernel(const IrParams p) {
             for (int a = 0; a < MT; ++a) pa[c][a] = buf_load_f32(rpw, (unsigned) (c * p.cop + a * 32 + li) * 4u, soff);
     };
     // chunk's expansion into the patch: wavefront w takes the pixel tiles w, w + 4, ..., two at a time (two independent
-    // chains of MFMAs)
-    auto expand_tiles = [&](float *patch, int t0, auto nt) __attribute__((always_inline)) {
-        constexpr int NT = decltype(nt)::value;
+    // chains of MFMAs).  Where a lane's four values of tile j (one pixel, the four channels 4 (lane / 16) .. + 3, which are
+    // one channel group of the patch) go is the same for every chunk: eo[j], in floats, or -1 for a pixel past the band's
+    // input or in a row outside the image.
+    int eo[IR_TPW];
+#pragma unroll
+    for (int j = 0; j < IR_TPW; ++j) {
+        const int px = 16 * (wave + 4 * j) + l16;
+        const int ir = (int) div31((unsigned) px, p.div_w), col = px - ir * p.w;
+        const bool ok = px < p.P && (unsigned) (ih_first + ir) < (unsigned) p.h;
+        eo[j] = ok ? ((lq * p.in_rows + ir) * pitch + 1 + col) * 4 : -1;
+    }
+    auto expand_tiles = [&](float *patch, auto j0, auto nt) __attribute__((always_inline)) {
+        constexpr int NT = decltype(nt)::value, J0 = decltype(j0)::value;
         f32x4 e[NT];
         float xv[NT][KS];
 #pragma unroll
         for (int u = 0; u < NT; ++u) {
             e[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            const float *xb = Xs + lq * p.xs_pitch + 16 * (t0 + 4 * u) + l16;
+            const float *xb = Xs + lq * p.xs_pitch + 16 * (wave + 4 * (J0 + u)) + l16;
 #pragma unroll
             for (int s = 0; s < KS; ++s) xv[u][s] = xb[4 * s * p.xs_pitch];
         }
@@ -167,19 +179,29 @@ __global__ __launch_bounds__(256, 2) void irblock_f32_kernel(const IrParams p) {
             for (int u = 0; u < NT; ++u) e[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(aexp[s], xv[u][s], e[u], 0, 0, 0);
 #pragma unroll
         for (int u = 0; u < NT; ++u) {
-            const int px = 16 * (t0 + 4 * u) + l16;
-            const int ir = (int) div31((unsigned) px, p.div_w), col = px - ir * p.w;
-            if (px < p.P && (unsigned) (ih_first + ir) < (unsigned) p.h) {
-                float *dst = patch + (4 * lq) * plane + ir * pitch + 1 + col;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) dst[r * plane] = ir_act<EPI>(__fadd_rn(e[u][r], eb[r]), p.exp_ep);
+            if (eo[J0 + u] >= 0) {
+                float4 o;
+                o.x = ir_act<EPI>(__fadd_rn(e[u][0], eb[0]), p.exp_ep);
+                o.y = ir_act<EPI>(__fadd_rn(e[u][1], eb[1]), p.exp_ep);
+                o.z = ir_act<EPI>(__fadd_rn(e[u][2], eb[2]), p.exp_ep);
+                o.w = ir_act<EPI>(__fadd_rn(e[u][3], eb[3]), p.exp_ep);
+                *reinterpret_cast<float4 *>(patch + eo[J0 + u]) = o;
             }
         }
     };
+    auto expand_from = [&](float *patch, auto j0) __attribute__((always_inline)) {
+        constexpr int J0 = decltype(j0)::value;
+        if (wave + 4 * J0 < p.tiles) {   // uniform
+            if (J0 + 1 < IR_TPW && wave + 4 * (J0 + 1) < p.tiles) expand_tiles(patch, j0, std::integral_constant<int, (J0 + 1 < IR_TPW ? 2 : 1)>());
+            else expand_tiles(patch, j0, std::integral_constant<int, 1>());
+        }
+    };
     auto expand = [&](float *patch) __attribute__((always_inline)) {
-        int t = wave;
-        for (; t + 4 < p.tiles; t += 8) expand_tiles(patch, t, std::integral_constant<int, 2>());
-        if (t < p.tiles) expand_tiles(patch, t, std::integral_constant<int, 1>());
+        expand_from(patch, std::integral_constant<int, 0>());
+        expand_from(patch, std::integral_constant<int, 2>());
+        expand_from(patch, std::integral_constant<int, 4>());
+        expand_from(patch, std::integral_constant<int, 6>());
+        expand_from(patch, std::integral_constant<int, 8>());
     };
 
     // v_mfma_f32_32x32x1_2b_f32: two 32x32 blocks (pixels 0..31 and 32..63 of the wavefront's 64), one reduction index per
@@ -195,26 +217,32 @@ __global__ __launch_bounds__(256, 2) void irblock_f32_kernel(const IrParams p) {
     auto depthwise_project = [&](int chunk, const float *patch) __attribute__((always_inline)) {
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            float wd[4][9], bd[4], tv[4][9];
+            // one channel group (four channels side by side in the patch): nine 16-byte reads give the lane its window in
+            // all four
+            float wd[4][9], bd[4];
+            float4 tv[9];
+            const int g = kh * 2 + half;
 #pragma unroll
             for (int cc = 0; cc < 4; ++cc) {
-                const int k = kh * 8 + half * 4 + cc;
-                const int c = chunk * IR_KC + k;   // uniform: scalar loads
+                const int c = chunk * IR_KC + g * 4 + cc;   // uniform: scalar loads
 #pragma unroll
                 for (int i = 0; i < 9; ++i) wd[cc][i] = p.dw_w[c * 9 + i];
                 bd[cc] = p.dw_b[c];
-                const float *tp = patch + k * plane + win;
-#pragma unroll
-                for (int i = 0; i < 3; ++i)
-#pragma unroll
-                    for (int t = 0; t < 3; ++t) tv[cc][i * 3 + t] = tp[i * pitch + t];
             }
+            const float4 *tp = reinterpret_cast<const float4 *>(patch) + g * plane + win;
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+#pragma unroll
+                for (int t = 0; t < 3; ++t) tv[i * 3 + t] = tp[i * pitch + t];
             __builtin_amdgcn_sched_barrier(0);   // every window is requested before the arithmetic starts
 #pragma unroll
             for (int cc = 0; cc < 4; ++cc) {
                 float sum = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 9; ++i) sum = __fadd_rn(sum, __fmul_rn(wd[cc][i], tv[cc][i]));
+                for (int i = 0; i < 9; ++i) {
+                    const float tap = cc == 0 ? tv[i].x : cc == 1 ? tv[i].y : cc == 2 ? tv[i].z : tv[i].w;
+                    sum = __fadd_rn(sum, __fmul_rn(wd[cc][i], tap));
+                }
                 float v = ir_act<EPI>(__fadd_rn(sum, bd[cc]), p.dw_ep);
                 v = q_ok ? v : 0.0f;
 #pragma unroll
@@ -347,7 +375,7 @@ int irblock_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int cin) {
         const int P = in_rows * dw.w;
         const long long slots = ((long long) cin * (P / 4) + 255) / 256;
         const long long lds = ((long long) cin * ir_xs_pitch(P) + 4 + (long long) IR_KC * in_rows * (dw.w + 2) + 4) * 4;
-        if (lds > IR_LDS_HALF || slots > IR_XSLOTS) continue;
+        if (lds > IR_LDS_HALF || slots > IR_XSLOTS || (P + 15) / 16 > 4 * IR_TPW) continue;
         if (!tallest) tallest = rows;
         if ((long long) dw.n * ((OH + rows - 1) / rows) >= 256) return rows;
     }
