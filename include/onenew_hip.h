@@ -417,6 +417,14 @@ int onhip_conv_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S 
  * `eval_add` and `eval_add_relu` beside `eval`, for the device-resident runtime. */
 int onhip_conv_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_block` / `eval_block_takes` of libConv_hip.so: Conv (1x1) -> Conv (depthwise 3x3) -> Conv (1x1) [-> Add] in one
+ * call (onhip_ir_block_f32).  Slots as for the first convolution's `eval` (host/op.h:109-168), the block's result operand
+ * in params[4] and outputs[0]; inputs[3] = the addend or null; params[5], params[6], inputs[5], inputs[6] = the depthwise
+ * convolution's CONV_CONFIG_S, weight operand, weights and bias; params[7], params[8], inputs[7], inputs[8] = the same of
+ * the last convolution.  onhip_conv_block_takes reads the params only and returns 1 when onhip_ir_block_supported says 2
+ * for these shapes, else 0.  No counterpart in the reference, whose host runs the operators one by one. */
+int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_conv_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Add (add.c:18), Relu (relu.c:8), MaxPool (maxpool.c:7), GlobalAveragePool (global_avgpool.c:7) */
 int onhip_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);

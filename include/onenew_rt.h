@@ -96,6 +96,15 @@ int onrt_net_fused_count(const onrt_net_t *net, int32_t *n_blocks, int32_t *n_re
 int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n);
 
 /*
+ * Inverted-residual blocks: Conv (1x1) -> Conv (depthwise 3x3) -> Conv (1x1) [-> Add], each result read by the next
+ * alone, run as one call of the Conv plugin's `eval_block` (libConv_hip.so; neither wide tensor in between is written)
+ * where its `eval_block_takes` recommends that for the shapes: MobileNetV2's blocks on the 112, 56 and 28 pixel planes at
+ * large batch.  The reference's host runs the operators one after the other (host/net.h:613-618).  The operands folded
+ * away have no buffer.  ONENEW_RT_FUSE=0 keeps the operators separate.  n: how many blocks.
+ */
+int onrt_net_fused_ir_blocks(const onrt_net_t *net, int32_t *n);
+
+/*
  * Attention blocks: MatMul(q, Transpose(k)) -> Softmax (last axis) -> MatMul(., v), where nothing else reads the operands
  * in between, run as one call of the MatMul plugin's `eval_attention` (libMatMul_hip.so; the scores stay on the chip, the
  * transposed k is never written) when q, k and v are [..., tokens, head_dim] with head_dim 32 or 64 and at most 256

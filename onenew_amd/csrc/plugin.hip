@@ -99,14 +99,24 @@ struct PackedEntry {
     float *dev;
     size_t bytes;
     bool int8;
+    const void *other;   // a pack made of two weight tensors (the 1x1 layers of a fused block): the one it is not keyed by
 };
 static std::map<const void *, PackedEntry> g_packed;
 
 static void drop_packed(const void *w_dev) {
     auto it = g_packed.find(w_dev);
-    if (it == g_packed.end()) return;
-    (void) hipFree(it->second.dev);
-    g_packed.erase(it);
+    if (it != g_packed.end()) {
+        (void) hipFree(it->second.dev);
+        g_packed.erase(it);
+    }
+    for (it = g_packed.begin(); it != g_packed.end();) {
+        if (it->second.other == w_dev) {
+            (void) hipFree(it->second.dev);
+            it = g_packed.erase(it);
+        } else {
+            ++it;
+        }
+    }
 }
 
 // *out = packed copy of the device weights w_dev for convolution d, or nullptr if d takes them as they are.
@@ -125,7 +135,23 @@ static int packed_weights(const onhip_conv_desc_t *d, const float *w_dev, const 
                                                     reinterpret_cast<int8_t *>(p), g_stream)
                   : onhip_conv2d_pack_weights(d, w_dev, p, g_stream);
     if (rc) { (void) hipFree(p); return rc; }
-    g_packed[w_dev] = PackedEntry{p, bytes, int8};
+    g_packed[w_dev] = PackedEntry{p, bytes, int8, nullptr};
+    *out = p;
+    return ONHIP_OK;
+}
+
+// the two 1x1 weight tensors of an inverted-residual block in the layout of onhip_ir_block_f32, packed when first seen,
+// keyed by the projection's device address
+static int packed_block_weights(const float *ex_w, const float *pw_w, int cin, int ce, int co, const float **out) {
+    const size_t bytes = onhip_ir_block_packed_weight_bytes(cin, ce, co);
+    auto it = g_packed.find(pw_w);
+    if (it != g_packed.end() && it->second.bytes == bytes && it->second.other == ex_w) { *out = it->second.dev; return ONHIP_OK; }
+    drop_packed(pw_w);
+    float *p = nullptr;
+    ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&p), bytes));
+    const int rc = onhip_ir_block_pack_weights(ex_w, pw_w, cin, ce, co, p, g_stream);
+    if (rc) { (void) hipFree(p); return rc; }
+    g_packed[pw_w] = PackedEntry{p, bytes, false, ex_w};
     *out = p;
     return ONHIP_OK;
 }
@@ -343,6 +369,93 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
     if (!out_on_dev) return copy_out(host_out, y, out_bytes);
     else return wait_for_output();
     return ONHIP_OK;
+}
+
+// One convolution of a fused block as the library describes it: configuration, input extent, weight operand.
+static void block_conv_desc(onhip_conv_desc_t *d, const CONV_CONFIG_S *cfg, int n, int cin, int h, int w, const OPERAND_S *w_t) {
+    memset(d, 0, sizeof(*d));
+    d->n = n; d->cin = cin; d->h = h; d->w = w;
+    d->cout = w_t->shapes[0]; d->kh = w_t->shapes[2]; d->kw = w_t->shapes[3];
+    d->stride_h = (int32_t) cfg->strides[0]; d->stride_w = (int32_t) cfg->strides[1];
+    d->pad_t = (int32_t) cfg->pads[0]; d->pad_l = (int32_t) cfg->pads[1];
+    d->pad_b = (int32_t) cfg->pads[2]; d->pad_r = (int32_t) cfg->pads[3];
+    d->group = !cfg->has_bias ? 1 : (cfg->group == 1 ? 1 : cin);   // conv.c:18-29, as in conv_eval_fused
+    d->has_bias = cfg->has_bias ? 1 : 0;
+    d->act_type = cfg->act_type;
+    d->clip_min = cfg->clip_min; d->clip_max = cfg->clip_max;
+    d->leaky_relu_alpha = cfg->leaky_relu_alpha;
+    d->hard_sigmoid_alpha = cfg->hard_sigmoid_alpha; d->hard_sigmoid_beta = cfg->hard_sigmoid_beta;
+    d->compute = ONHIP_COMPUTE_F32;
+}
+
+// Conv (1x1) -> Conv (depthwise 3x3) -> Conv (1x1) [-> Add] as one call of onhip_ir_block_f32.  Slots: params[0..4] /
+// inputs[0..2] as for the first convolution's `eval`, params[4] the block's result operand; inputs[3] the addend or
+// null; params[5] the depthwise CONV_CONFIG_S, params[6] its weight operand, inputs[5] / inputs[6] its weights and bias;
+// params[7] the last convolution's CONV_CONFIG_S, params[8] its weight operand, inputs[7] / inputs[8] its weights and
+// bias (null without).  query: no tensor is touched; the return value is 1 when the library recommends the one-launch
+// kernel for these shapes and 0 otherwise.
+static int conv_block_eval_mode(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, bool query) {
+    const CONV_CONFIG_S *cfg[3] = {reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr), reinterpret_cast<const CONV_CONFIG_S *>(params[5].addr),
+                                   reinterpret_cast<const CONV_CONFIG_S *>(params[7].addr)};
+    const OPERAND_S *in_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *w_t[3] = {reinterpret_cast<const OPERAND_S *>(params[2].addr), reinterpret_cast<const OPERAND_S *>(params[6].addr),
+                               reinterpret_cast<const OPERAND_S *>(params[8].addr)};
+    const OPERAND_S *out_t = reinterpret_cast<const OPERAND_S *>(params[4].addr);
+    if (!cfg[0] || !cfg[1] || !cfg[2] || !in_t || !w_t[0] || !w_t[1] || !w_t[2] || !out_t) {
+        if (query) return 0;
+        return set_error(ONHIP_ERR_ARG, "Conv block eval: empty params slot");
+    }
+    if (cfg[0]->ifmap_quant2 == TYPE_INT8 || cfg[1]->ifmap_quant2 == TYPE_INT8 || cfg[2]->ifmap_quant2 == TYPE_INT8) {
+        if (query) return 0;
+        return set_error(ONHIP_ERR_ARG, "Conv block eval: fp32 convolutions only");
+    }
+    onhip_conv_desc_t d[3];
+    int n = out_t->shapes[0] < in_t->shapes[0] ? out_t->shapes[0] : in_t->shapes[0];
+    n = n < 1 ? 1 : n;
+    int32_t oh = 0, ow = 0, h2 = 0, w2 = 0, h3 = 0, w3 = 0;
+    block_conv_desc(&d[0], cfg[0], n, in_t->shapes[1], in_t->shapes[2], in_t->shapes[3], w_t[0]);
+    bool ok = onhip_conv_out_shape(&d[0], &h2, &w2) == ONHIP_OK;
+    if (ok) {
+        block_conv_desc(&d[1], cfg[1], n, d[0].cout, h2, w2, w_t[1]);
+        ok = onhip_conv_out_shape(&d[1], &h3, &w3) == ONHIP_OK;
+    }
+    if (ok) {
+        block_conv_desc(&d[2], cfg[2], n, d[1].cout, h3, w3, w_t[2]);
+        ok = onhip_conv_out_shape(&d[2], &oh, &ow) == ONHIP_OK && out_t->shapes[1] == d[2].cout && out_t->shapes[2] == oh && out_t->shapes[3] == ow;
+    }
+    if (query) return ok && onhip_ir_block_supported(&d[0], &d[1], &d[2]) >= 2 ? 1 : 0;
+    if (!ok) return set_error(ONHIP_ERR_ARG, "Conv block eval: the three convolutions and the result operand do not fit together");
+    if (!onhip_ir_block_supported(&d[0], &d[1], &d[2])) return set_error(ONHIP_ERR_ARG, "Conv block eval: not a block the one-launch kernel takes");
+    const size_t in_bytes = (size_t) n * d[0].cin * d[0].h * d[0].w * 4, out_bytes = (size_t) n * d[2].cout * oh * ow * 4;
+    const void *x, *ex_w, *ex_b, *dw_w, *dw_b, *pw_w, *pw_b = nullptr, *addend = nullptr;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[1].addr), (size_t) d[0].cout * d[0].cin * 4, &ex_w);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[2].addr), (size_t) d[0].cout * 4, &ex_b);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[5].addr), (size_t) d[1].cout * d[1].kh * d[1].kw * 4, &dw_w);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[6].addr), (size_t) d[1].cout * 4, &dw_b);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[7].addr), (size_t) d[2].cout * d[2].cin * 4, &pw_w);
+    if (!rc && d[2].has_bias) rc = const_on_device(reinterpret_cast<const void *>(inputs[8].addr), (size_t) d[2].cout * 4, &pw_b);
+    if (!rc && inputs[3].addr) rc = input_on_device(5, reinterpret_cast<const void *>(inputs[3].addr), out_bytes, &addend);
+    if (rc) return rc;
+    if (!ex_w || !ex_b || !dw_w || !dw_b || !pw_w) return set_error(ONHIP_ERR_ARG, "Conv block eval: empty weight or bias slot");
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, out_bytes, &y);
+        if (rc) return rc;
+    }
+    const float *packed = nullptr;
+    rc = packed_block_weights((const float *) ex_w, (const float *) pw_w, d[0].cin, d[0].cout, d[2].cout, &packed);
+    if (rc) return rc;
+    rc = onhip_ir_block_f32(&d[0], &d[1], &d[2], (const float *) x, packed, (const float *) ex_b, (const float *) dw_w, (const float *) dw_b,
+                            (const float *) pw_b, (const float *) addend, (float *) y, g_stream);
+    if (rc) return rc;
+    return out_on_dev ? wait_for_output() : copy_out(host_out, y, out_bytes);
+}
+
+static int conv_block_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return conv_block_eval_mode(params, inputs, outputs, false);
 }
 
 static int conv_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
@@ -809,6 +922,13 @@ int onhip_conv_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INF
 
 int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Conv + Add + Relu", conv_add_relu_eval_locked, params, inputs, outputs);
+}
+int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv -> depthwise Conv -> Conv", conv_block_eval_locked, params, inputs, outputs);
+}
+int onhip_conv_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    if (!params) return 0;
+    return conv_block_eval_mode(params, inputs, outputs, true);
 }
 
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {

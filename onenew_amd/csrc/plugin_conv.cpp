@@ -15,6 +15,20 @@ extern "C" __attribute__((visibility("default"))) int eval_add(BUFFER_INFO_S *pa
     return onhip_conv_add_eval(params, inputs, outputs);
 }
 
+// Not in the reference: a whole inverted-residual block, Conv (1x1) -> Conv (depthwise 3x3) -> Conv (1x1) [-> Add], as one
+// call.  Slots as for the first convolution's `eval` with the block's result operand in params[4] and outputs[0];
+// inputs[3] = the addend or null; params[5], params[6], inputs[5], inputs[6] = the depthwise convolution's CONV_CONFIG_S,
+// weight operand, weights and bias; params[7], params[8], inputs[7], inputs[8] = the same of the last convolution.
+// eval_block_takes: same params, no tensors touched; 1 when the library recommends the call for these shapes, else 0.
+extern "C" __attribute__((visibility("default"))) int eval_block(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                 BUFFER_INFO_S *outputs) {
+    return onhip_conv_block_eval(params, inputs, outputs);
+}
+extern "C" __attribute__((visibility("default"))) int eval_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                       BUFFER_INFO_S *outputs) {
+    return onhip_conv_block_takes(params, inputs, outputs);
+}
+
 extern "C" __attribute__((visibility("default"))) int eval_add_relu(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
                                                                     BUFFER_INFO_S *outputs) {
     return onhip_conv_add_relu_eval(params, inputs, outputs);

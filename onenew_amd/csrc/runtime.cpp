@@ -129,6 +129,7 @@ struct Node {
     int fuse = 0;            // Conv: 1 = the Add after it is folded in, 2 = and the Relu after that
     std::string addend, fused_out;
     int32_t token_major[4] = {0, 0, 0, 0};   // fused attention: q, k, v, result stored [batch, tokens, heads, head_dim]
+    int block_dw = -1, block_pw = -1;        // fused inverted-residual block (fuse 7): its depthwise and last convolutions
     BUFFER_INFO_S params[BUF_MAXNUM], inputs[BUF_MAXNUM], outputs[BUF_MAXNUM];
     const BASE_CONFIG_S *base() const { return reinterpret_cast<const BASE_CONFIG_S *>(cfg.data()); }
 };
@@ -163,8 +164,9 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
+    onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr;
     onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr, matmul_bias_add = nullptr;   // optional entry points of the MatMul plugin
-    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0;
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -517,6 +519,8 @@ int bind_plugins(onrt_net &net) {
         if (type == "Conv") {
             net.conv_add = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add"));
             net.conv_add_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add_relu"));
+            net.conv_block = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block"));
+            net.conv_block_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block_takes"));
         }
         if (type == "MatMul") {
             net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
@@ -689,6 +693,77 @@ int fuse_residual_blocks(onrt_net &net) {
         dropped[idx] = true;
         runs_instead[ai] = idx;
         ++net.fused_blocks;
+    }
+    std::vector<int> order;
+    for (int idx : net.order) {
+        auto it = runs_instead.find(idx);
+        if (it != runs_instead.end()) order.push_back(it->second);
+        else if (!dropped[idx]) order.push_back(idx);
+    }
+    net.order.swap(order);
+    return ONRT_OK;
+}
+
+// ---- inverted-residual blocks ---------------------------------------------------------------------------
+// Conv (1x1) -> Conv (depthwise) -> Conv (1x1) [-> Add, already folded into the last convolution], each result read by
+// the next alone, becomes one call of the Conv plugin's `eval_block` where the plugin's `eval_block_takes` recommends it
+// for the shapes (large batches of MobileNetV2's early blocks): neither wide tensor in between is written.  The call
+// takes the place of the last convolution in the order.  Runs after the residual fold; ONENEW_RT_FUSE=0 keeps every
+// operator separate, and a plan without plugins (no device) folds none.
+void block_slots(onrt_net &net, Node &a, const Node &b, const Node &c, const Tensor &result) {
+    a.params[0].addr = (int64_t) a.cfg.data();
+    a.params[1].addr = (int64_t) &net.tensors[a.in[0]].desc;
+    a.params[2].addr = (int64_t) &net.tensors[a.in[1]].desc;
+    a.params[3].addr = (int64_t) &net.tensors[a.in[2]].desc;
+    a.params[4].addr = (int64_t) &result.desc;
+    a.params[5].addr = (int64_t) b.cfg.data();
+    a.params[6].addr = (int64_t) &net.tensors[b.in[1]].desc;
+    a.params[7].addr = (int64_t) c.cfg.data();
+    a.params[8].addr = (int64_t) &net.tensors[c.in[1]].desc;
+}
+
+int fuse_ir_blocks(onrt_net &net) {
+    if (!fusing_enabled() || !net.conv_block || !net.conv_block_takes) return ONRT_OK;
+    auto result_of = [](const Node &n) { return n.fused_out.empty() ? n.out[0] : n.fused_out; };
+    auto plain_conv = [&](const Node &n, size_t min_in) {
+        if (strcmp(n.kind->type, "Conv") || n.out.size() != 1 || n.in.size() < min_in || n.in.size() > 3) return false;
+        for (size_t k = 1; k < n.in.size(); ++k)
+            if (n.in[k].empty() || !net.tensors[n.in[k]].is_init) return false;
+        return !net.tensors[n.in[0]].is_init;
+    };
+    std::map<int, int> runs_instead;   // last convolution -> the first one, which takes its place
+    std::vector<bool> dropped(net.nodes.size(), false);
+    for (int idx : net.order) {
+        Node &a = net.nodes[idx];
+        if (a.fuse || dropped[idx] || !plain_conv(a, 3)) continue;
+        const int bi = sole_reader(net, result_of(a), "Conv");
+        if (bi < 0 || dropped[bi]) continue;
+        Node &b = net.nodes[bi];
+        if (b.fuse || !plain_conv(b, 3) || b.in[0] != result_of(a)) continue;
+        const int ci = sole_reader(net, result_of(b), "Conv");
+        if (ci < 0 || dropped[ci] || runs_instead.count(ci)) continue;
+        Node &c = net.nodes[ci];
+        if (c.fuse > 1 || !plain_conv(c, 2) || c.in[0] != result_of(b)) continue;
+        const Tensor &result = net.tensors[result_of(c)];
+        for (BUFFER_INFO_S &s : a.params) s.addr = 0;
+        block_slots(net, a, b, c, result);
+        const bool takes = net.conv_block_takes(a.params, a.inputs, a.outputs) == 1;
+        for (BUFFER_INFO_S &s : a.params) s.addr = 0;
+        if (!takes) continue;
+        for (const std::string &gone : {a.out[0], result_of(a), b.out[0], result_of(b)}) {
+            net.tensors[gone].never_written = true;
+            net.tensors[gone].alias.clear();
+        }
+        a.fuse = 7;
+        a.block_dw = bi;
+        a.block_pw = ci;
+        a.addend = c.fuse == 1 ? c.addend : std::string();
+        a.fused_out = result_of(c);
+        if (c.out[0] != a.fused_out) net.tensors[c.out[0]].alias = a.fused_out;
+        a.eval = net.conv_block;
+        dropped[idx] = dropped[bi] = true;
+        runs_instead[ci] = idx;
+        ++net.fused_ir_blocks;
     }
     std::vector<int> order;
     for (int idx : net.order) {
@@ -890,6 +965,15 @@ int fill_slots(onrt_net &net) {
             nd.inputs[slot].addr = (int64_t) t.dev;
         }
         if (nd.fuse == 3) nd.inputs[4].addr = (int64_t) nd.token_major;
+        if (nd.fuse == 7) {
+            const Node &b = net.nodes[nd.block_dw], &c = net.nodes[nd.block_pw];
+            block_slots(net, nd, b, c, net.tensors[nd.fused_out]);
+            nd.inputs[3].addr = nd.addend.empty() ? 0 : (int64_t) net.tensors[nd.addend].dev;
+            nd.inputs[5].addr = (int64_t) net.tensors[b.in[1]].dev;
+            nd.inputs[6].addr = (int64_t) net.tensors[b.in[2]].dev;
+            nd.inputs[7].addr = (int64_t) net.tensors[c.in[1]].dev;
+            nd.inputs[8].addr = c.in.size() > 2 ? (int64_t) net.tensors[c.in[2]].dev : 0;
+        }
         if (nd.fuse == 1 || nd.fuse == 2 || nd.fuse == 6) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
@@ -918,6 +1002,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = bind_plugins(net);
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
+    if (!rc) rc = fuse_ir_blocks(net);
     if (!rc) rc = fuse_attention(net);
     if (!rc) rc = fuse_linear(net);
     if (!rc) rc = allocate(net);
@@ -1142,6 +1227,12 @@ ONRT_API int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n) {
 ONRT_API int onrt_net_fused_linears(const onrt_net_t *net, int32_t *n) {
     if (!net || !n) return fail(ONRT_ERR_ARG, "fused linear layers: null argument");
     *n = (int32_t) net->fused_linears;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_fused_ir_blocks(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "fused inverted-residual blocks: null argument");
+    *n = (int32_t) net->fused_ir_blocks;
     return ONRT_OK;
 }
 

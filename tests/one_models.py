@@ -39,6 +39,24 @@ def mobile_block():
     return m.tobytes(), [_r("xm", (1, 8, 14, 14))]
 
 
+def inverted_residual_blocks(batch=8, size=32):
+    """two MobileNetV2-style blocks on a plane large enough for the one-launch block kernel to be recommended at this batch:
+    1x1 expansion + CLIP, depthwise 3x3 + CLIP (stride 1, then 2), linear 1x1 projection; the first with the skip connection"""
+    m = onefile.OneModel()
+    m.input("x", (batch, 16, size, size))
+    m.conv("e1", "x", _r("e1w", (64, 16, 1, 1), 0.3), _r("e1b", (64,), 0.3), "e1_out", act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("d1", "e1_out", _r("d1w", (64, 1, 3, 3), 0.3), _r("d1b", (64,), 0.1), "d1_out", pad=1, group=64, act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("p1", "d1_out", _r("p1w", (16, 64, 1, 1), 0.15), _r("p1b", (16,), 0.1), "p1_out")
+    m.add("skip", "p1_out", "x", "b1_out")
+    m.conv("e2", "b1_out", _r("e2w", (96, 16, 1, 1), 0.3), _r("e2b", (96,), 0.3), "e2_out", act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("d2", "e2_out", _r("d2w", (96, 1, 3, 3), 0.3), _r("d2b", (96,), 0.1), "d2_out", stride=2, pad=1, group=96, act=abi.CLIP,
+           clip=(0.0, 6.0))
+    m.conv("p2", "d2_out", _r("p2w", (24, 96, 1, 1), 0.1), None, "out")
+    m.output("out", (batch, 24, size // 2, size // 2))
+    m.output("b1_out", (batch, 16, size, size))
+    return m.tobytes(), [_r("xir", (batch, 16, size, size))]
+
+
 def vit_block():
     """layer norm, projection with a weight initialiser and a bias Add, table GELU, residual, then a token-mixing
     pair of MatMuls over two activations with Transpose and Softmax, and a Reshape view"""

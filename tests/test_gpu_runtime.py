@@ -246,6 +246,50 @@ def test_linear_layers_run_as_one_call_bit_for_bit(torch_dev, monkeypatch):
     fused.close()
 
 
+def test_inverted_residual_blocks_run_as_one_call(torch_dev, monkeypatch):
+    """Conv 1x1 -> depthwise Conv -> Conv 1x1 (-> Add) of two MobileNetV2-style blocks as one call of the Conv plugin's
+    eval_block each, where the plugin recommends it (enough bands of rows over the batch): against the net run operator by
+    operator within 1e-4 and against the CPU restatement of the graph; at a small batch the operators stay separate"""
+    data, ins = one_models.inverted_residual_blocks(batch=16, size=32)
+    fused, plain, got, want = _both_ways(data, ins, monkeypatch)
+    assert plain.fused_ir_blocks() == 0 and fused.fused_ir_blocks() == 2
+    assert [t for t, _ in fused.ops()] == ["Conv", "Conv"] and len(plain.ops()) == 7
+    for name in ("e1_out", "d1_out", "e2_out", "d2_out"):
+        assert fused.operand(name)[1] is None
+    ref = one_model.run(data, ins)
+    for g, w_, r in zip(got, want, ref):
+        assert g.shape == w_.shape and np.all(np.abs(g - w_) <= 1e-4 * np.abs(w_) + 1e-5 * np.abs(w_).max())
+        assert _close(g, r, 5e-4)
+    x2 = [(ins[0] * np.float32(-0.7) + np.float32(0.2)).astype(np.float32)]
+    for g, w_ in zip(fused.run(*x2), plain.run(*x2)):
+        assert np.all(np.abs(g - w_) <= 1e-4 * np.abs(w_) + 1e-5 * np.abs(w_).max())
+    fused.close()
+    plain.close()
+    small = rt.Net(one_models.inverted_residual_blocks(batch=1, size=32)[0])
+    assert small.fused_ir_blocks() == 0 and len(small.ops()) == 6
+    small.close()
+
+
+def test_mobilenetv2_batch64_with_its_blocks_in_one_call(torch_dev, monkeypatch):
+    """the whole MobileNetV2 model at batch 64, where the early inverted-residual blocks run as one call each: logits
+    against the same file run operator by operator (1e-3 of the largest logit, same top-5 on every image)"""
+    from onenew_amd import stacks
+    data, shape, _ = stacks.mobilenet_v2_model(64)
+    x = np.random.default_rng(64).uniform(-1.0, 1.0, size=shape).astype(np.float32)
+    fused = rt.Net(data)
+    assert fused.fused_ir_blocks() == 6
+    got = fused.run(x)[0]
+    fused.close()
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    plain = rt.Net(data)
+    assert plain.fused_ir_blocks() == 0
+    want = plain.run(x)[0]
+    plain.close()
+    assert got.shape == want.shape == (64, 1000)
+    assert np.abs(got - want).max() <= 1e-3 * np.abs(want).max()
+    assert np.array_equal(np.argsort(got, axis=1)[:, -5:], np.argsort(want, axis=1)[:, -5:])
+
+
 @pytest.mark.parametrize("split", ["qkvo", "kv", "qo", "o"])
 def test_attention_block_takes_in_the_head_transposes(split, torch_dev, monkeypatch):
     """head-split Transposes (0, 2, 1, 3) in front of q, k, v and the head-merge one behind the result fold into the
