@@ -72,7 +72,7 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
     static_assert(NST >= 2 && NST * STAGE <= 160 * 1024, "the ring must fit the 160 KiB of LDS of a compute unit");
     constexpr int NSETS = (NST * STAGE + 65535) / 65536;
     // after the K loop the same memory holds the store's staging area, the quantised activation table and the per-row constants
-    constexpr int OUT_STAGE = DT == DT_I8 ? BN * (BM + 16) : BN * (2 * BM + 16), ROWS_AT = OUT_STAGE + 8192, OUT_BYTES = ROWS_AT + 2 * BM * 4;
+    constexpr int OUT_STAGE = DT == DT_I8 ? BN * (BM + 16) : BN * (2 * BM + 16), ROWS_AT = OUT_STAGE + (DT == DT_I8 ? 8192 : 16384), OUT_BYTES = ROWS_AT + 2 * BM * 4;
     static_assert(ROWS_AT % 16 == 0, "the per-row constants are read 16 bytes at a time");
     constexpr int LDS_BYTES = NST * STAGE > OUT_BYTES ? NST * STAGE : OUT_BYTES;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];

@@ -602,6 +602,23 @@ __device__ __forceinline__ void write_tile_nhwc_h16(const IgemmParams &p, f32x16
                                                     const float *rows) {
     static_assert(DT == DT_BF16 || DT == DT_F16, "16-bit floating-point outputs");
     constexpr int PITCH = 2 * BM + 16;
+    // Table activations: the 8192 fp32 entries rounded to the output type, 16 KiB of LDS behind the staging area (the
+    // caller leaves them free).  The value stored is round(table[i]) either way; the gathers then hit LDS instead of
+    // sending 64 addresses per instruction to memory.
+    typedef const __attribute__((address_space(3))) unsigned short *lds_u16_t;
+    lds_u16_t tab = nullptr;
+    if constexpr (EPI == EPI_LUT) {
+        unsigned char *tl = stage + BN * PITCH;
+        const float4 *src = reinterpret_cast<const float4 *>(p.ep.lut);
+        float4 t[8192 / 4 / THREADS];
+#pragma unroll
+        for (int i = 0; i < 8192 / 4 / THREADS; ++i) t[i] = src[tid + i * THREADS];
+#pragma unroll
+        for (int i = 0; i < 8192 / 4 / THREADS; ++i)
+            reinterpret_cast<uint2 *>(tl)[tid + i * THREADS] = make_uint2(pack_h16<DT>(t[i].x, t[i].y), pack_h16<DT>(t[i].z, t[i].w));
+        __syncthreads();
+        tab = (lds_u16_t) tl;
+    }
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -609,16 +626,41 @@ __device__ __forceinline__ void write_tile_nhwc_h16(const IgemmParams &p, f32x16
             const int ml = m_wave - m0 + a * 32 + 8 * q + 4 * lh;   // first of the lane's four channels, tile-local
             const float4 bias = *reinterpret_cast<const float4 *>(rows + ml);
             const float bv[4] = {bias.x, bias.y, bias.z, bias.w};
+            float y[TN][4];
+            if constexpr (EPI == EPI_LUT) {
+                // act_fast<EPI_LUT>'s rules; the table reads of the row group all in flight together
+                float v[TN][4];
+                unsigned short l[TN][4];
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        v[b][j] = __fadd_rn(acc[a][b][4 * q + j], bv[j]);
+                        int idx = (int) __fmul_rn(__fadd_rn(v[b][j], 8.0f), 512.0f);
+                        idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
+                        l[b][j] = tab[idx];
+                    }
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float lv = unpack_h16<DT>((unsigned) l[b][j], 0);
+                        const float r = v[b][j] < -8.0f ? 0.0f : v[b][j] >= 8.0f ? v[b][j] : lv;
+                        y[b][j] = (m0 + ml + j < p.M) ? r : 0.0f;
+                    }
+            } else {
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float v = act_fast<EPI>(__fadd_rn(acc[a][b][4 * q + j], bv[j]), p.ep);
+                        y[b][j] = (m0 + ml + j < p.M) ? v : 0.0f;
+                    }
+            }
 #pragma unroll
             for (int b = 0; b < TN; ++b) {
-                float y[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float v = act_fast<EPI>(__fadd_rn(acc[a][b][4 * q + j], bv[j]), p.ep);
-                    y[j] = (m0 + ml + j < p.M) ? v : 0.0f;
-                }
                 const int nl = n_wave - n0 + b * 32 + li;
-                *reinterpret_cast<uint2 *>(stage + nl * PITCH + ml * 2) = make_uint2(pack_h16<DT>(y[0], y[1]), pack_h16<DT>(y[2], y[3]));
+                *reinterpret_cast<uint2 *>(stage + nl * PITCH + ml * 2) = make_uint2(pack_h16<DT>(y[b][0], y[b][1]), pack_h16<DT>(y[b][2], y[b][3]));
             }
         }
     __syncthreads();
