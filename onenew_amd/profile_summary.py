@@ -51,6 +51,8 @@ def short(name):
 
 
 def family(name):
+    if "_pack_kernel" in name:   # weight re-layouts: once per model, not part of a pass
+        return None
     if "igemm" in name or "splitk_finish" in name or "rowb_f32" in name or "attention" in name or "stem_f32" in name:
         return "igemm"
     if "depthwise" in name or "dwproj" in name or "irblock" in name:
@@ -98,26 +100,37 @@ def summarise(workload, raw, out_dir):
             continue
         L.append(f"| `{n}` | {r['Calls']} | {float(r['TotalDurationNs']) / 1e6:.3f} | {float(r['AverageNs']) / 1e3:.2f} | "
                  f"{float(r['Percentage']):.2f} | {float(r['MinNs']) / 1e3:.2f} | {float(r['MaxNs']) / 1e3:.2f} |")
-    passes = bench["warmup"] + bench["steps"] + 3 + max(10, bench["steps"])
-    nl = bench["config"]["layers"]
+    whole_model = "layers" not in bench["config"]      # a .one file through the runtime: one timed loop, no per-layer timing
+    passes = bench["warmup"] + bench["steps"] + (0 if whole_model else 3 + max(10, bench["steps"]))
+    nl = bench["config"].get("layers", bench["config"].get("operators"))
     groups = collections.defaultdict(list)
     for r in stats:
         fam = family(r["Name"])
         if fam:
             groups[fam].append(r)
     L.append("")
-    L.append(f"The traced run makes {passes} passes over the {nl} layers ({bench['warmup']} warm-up + {bench['steps']} timed steps, then "
-             f"3 + {max(10, bench['steps'])} per layer for the event-timed roofline figures), plus the launches that measure tile choices "
-             f"where the cache did not have them.")
+    if whole_model:
+        # the operator that runs once per inference has the fewest calls: that count is the number of inferences traced
+        # (warm-up, timed steps, and the runs bench.py makes before them to fill the tile cache and check the outputs)
+        passes = min([int(r["Calls"]) for rs in groups.values() for r in rs if "splitk_finish" not in r["Name"]] or [passes])
+        L.append(f"The traced run makes {passes} inferences of the {nl} operators ({bench['warmup']} warm-up + {bench['steps']} timed, the rest "
+                 f"before them: tile choices, output checks).")
+    else:
+        L.append(f"The traced run makes {passes} passes over the {nl} layers ({bench['warmup']} warm-up + {bench['steps']} timed steps, then "
+                 f"3 + {max(10, bench['steps'])} per layer for the event-timed roofline figures), plus the launches that measure tile choices "
+                 f"where the cache did not have them.")
     for g, rs in groups.items():
         ns = sum(float(r["TotalDurationNs"]) for r in rs)
         main = sum(int(r["Calls"]) for r in rs if "splitk_finish" not in r["Name"])
         L.append(f"- {g}: {main} layer launches, {ns / 1e6:.3f} ms in total (split-K reduction included) = "
                  f"**{ns / main / 1e3:.2f} us per layer launch**, {ns / passes / 1e6:.4f} ms per pass.")
     rf = bench["roofline"]
-    L.append(f"- `bench.py` in the same run (HIP events on the launch stream): roofline group `{rf['kernel']}`, "
-             f"{rf['launches']} launches per pass, average {rf['avg_launch_ms'] * 1e3:.2f} us per launch, "
-             f"{rf['achieved']} {rf['unit']}; whole pass {bench['ms_per_step']} ms wall, {bench['value']} {bench['unit']}.")
+    if whole_model:
+        L.append(f"- `bench.py` in the same run: {bench['ms_per_step']} ms per inference, {bench['value']} {bench['unit']} ({rf['kernel']}).")
+    else:
+        L.append(f"- `bench.py` in the same run (HIP events on the launch stream): roofline group `{rf['kernel']}`, "
+                 f"{rf['launches']} launches per pass, average {rf['avg_launch_ms'] * 1e3:.2f} us per launch, "
+                 f"{rf['achieved']} {rf['unit']}; whole pass {bench['ms_per_step']} ms wall, {bench['value']} {bench['unit']}.")
     L.append("")
     out = {"workload": workload, "groups": {}}
     if copy_f and copy_w and fetch:
@@ -144,8 +157,9 @@ def summarise(workload, raw, out_dir):
             out["groups"][g] = {"launches_counted": launches[g], "hbm_bytes_per_launch": round(per)}
         dom = "igemm" if "igemm" in rf["kernel"] else "depthwise" if "depthwise" in rf["kernel"] else "glue"
         out["hbm_bytes_per_launch"] = out["groups"].get(dom, {}).get("hbm_bytes_per_launch")
-        L.append(f"- algorithmic bytes per step (every tensor once): {bench['config']['algorithmic_bytes_per_step'] / 1e6:.1f} MB over {nl} layers "
-                 f"= {bench['config']['algorithmic_bytes_per_step'] / nl / 1e6:.2f} MB per layer launch.")
+        if "algorithmic_bytes_per_step" in bench["config"]:
+            L.append(f"- algorithmic bytes per step (every tensor once): {bench['config']['algorithmic_bytes_per_step'] / 1e6:.1f} MB over {nl} layers "
+                     f"= {bench['config']['algorithmic_bytes_per_step'] / nl / 1e6:.2f} MB per layer launch.")
         L.append("")
     if sq:
         L.append("## Matrix-core and LDS counters (`--pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT SQ_WAVE_CYCLES "
