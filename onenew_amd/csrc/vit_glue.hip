@@ -95,6 +95,70 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(const float *__rest
     }
 }
 
+// The same for rows of a multiple of four floats, 16-byte aligned: a thread's share of the workgroup's rows (up to
+// LN_VEC 16-byte pieces) is requested in one go and held in registers, so the staging costs one memory round trip instead of
+// one per loop iteration; sums in memory order by one thread per row as above; the normalised rows leave as 16-byte stores.
+constexpr int LN_VEC = 8;
+
+__global__ __launch_bounds__(256) void layernorm_rows4_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                              const float *__restrict__ b, float *__restrict__ y, int rows,
+                                                              int reduce, int rpw, float inv_n) {
+    __shared__ float tile[LN_LDS_FLOATS];
+    __shared__ float s_mean[64], s_inv[64];
+    const int row0 = blockIdx.x * rpw;
+    const int nr = min(rpw, rows - row0);
+    const int pitch = reduce + 1, groups = reduce / 4;
+    const int total = nr * groups;
+    const float4 *src = reinterpret_cast<const float4 *>(x + (long long) row0 * reduce);
+    float4 v[LN_VEC];
+    int at[LN_VEC], col[LN_VEC];
+#pragma unroll
+    for (int i = 0; i < LN_VEC; ++i) {
+        const int f = threadIdx.x + i * 256;
+        const bool live = f < total;
+        const int ff = live ? f : 0;
+        const int r = ff / groups;
+        col[i] = (ff - r * groups) * 4;
+        at[i] = live ? r * pitch + col[i] : -1;
+        v[i] = live ? src[ff] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+#pragma unroll
+    for (int i = 0; i < LN_VEC; ++i)
+        if (at[i] >= 0) {
+            tile[at[i]] = v[i].x; tile[at[i] + 1] = v[i].y; tile[at[i] + 2] = v[i].z; tile[at[i] + 3] = v[i].w;
+        }
+    __syncthreads();
+    if ((int) threadIdx.x < nr) {
+        const float *t = tile + threadIdx.x * pitch;
+        float psum = 0.0f, psq = 0.0f;
+        for (int i = 0; i < reduce; ++i) {
+            psum = __fadd_rn(psum, t[i]);
+            psq = __fadd_rn(psq, __fmul_rn(t[i], t[i]));
+        }
+        ln_stats(psum, psq, inv_n, &s_mean[threadIdx.x], &s_inv[threadIdx.x]);
+    }
+    __syncthreads();
+    float4 *dst = reinterpret_cast<float4 *>(y + (long long) row0 * reduce);
+    float4 wv[LN_VEC], bv[LN_VEC];
+#pragma unroll
+    for (int i = 0; i < LN_VEC; ++i) {
+        wv[i] = *reinterpret_cast<const float4 *>(w + col[i]);
+        bv[i] = *reinterpret_cast<const float4 *>(b + col[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < LN_VEC; ++i) {
+        if (at[i] < 0) continue;
+        const int r = at[i] / pitch;
+        const float m = s_mean[r], s = s_inv[r];
+        float4 o;
+        o.x = __fadd_rn(__fmul_rn(__fmul_rn(__fsub_rn(v[i].x, m), s), wv[i].x), bv[i].x);
+        o.y = __fadd_rn(__fmul_rn(__fmul_rn(__fsub_rn(v[i].y, m), s), wv[i].y), bv[i].y);
+        o.z = __fadd_rn(__fmul_rn(__fmul_rn(__fsub_rn(v[i].z, m), s), wv[i].z), bv[i].z);
+        o.w = __fadd_rn(__fmul_rn(__fmul_rn(__fsub_rn(v[i].w, m), s), wv[i].w), bv[i].w);
+        dst[threadIdx.x + i * 256] = o;
+    }
+}
+
 // one thread per row straight from memory: rows too long for LDS (stride 1), or the "axis 1" form of
 // layer_normalization.c:28-60 where the elements of a row lie `stride` apart and neighbouring threads read
 // neighbouring addresses
@@ -222,6 +286,17 @@ int onhip_layernorm_f32(int32_t rows, int32_t reduce, int32_t strided, const flo
     if (strided) {
         hipLaunchKernelGGL(layernorm_thread_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, x, weight, bias, y, rows,
                            reduce, 1LL, (long long) rows, inv_n);
+    } else if (reduce % 4 == 0 && reduce >= 32 && reduce + 1 <= LN_LDS_FLOATS / 4 &&
+               ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(bias)) & 15) == 0) {
+        // as many rows per workgroup as a thread's LN_VEC registers of 16 bytes cover, at most 64, and few enough that
+        // every compute unit gets a workgroup
+        int rpw = LN_VEC * 256 / (reduce / 4);
+        rpw = rpw > 64 ? 64 : rpw;
+        if (rpw > LN_LDS_FLOATS / (reduce + 1)) rpw = LN_LDS_FLOATS / (reduce + 1);
+        const int spread = (rows + 511) / 512;
+        if (rpw > spread) rpw = spread < 1 ? 1 : spread;
+        hipLaunchKernelGGL(layernorm_rows4_kernel, dim3((rows + rpw - 1) / rpw), dim3(256), 0, st, x, weight, bias, y, rows,
+                           reduce, rpw, inv_n);
     } else if (reduce + 1 <= LN_LDS_FLOATS / 4) {
         int rpw = LN_LDS_FLOATS / (reduce + 1);
         if (rpw > 64) rpw = 64;
