@@ -122,6 +122,16 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
     const float *pb = patch + (wave * 32 + li) * p.stride;
     const float *ab = At + lh * 32 + li;
 
+    // the biases of this lane's rows: the same for every item
+    float bias_r[TWO ? 2 : 1][16];
+#pragma unroll
+    for (int a = 0; a < (TWO ? 2 : 1); ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+            bias_r[a][r] = buf_load_f32(rb, m < p.cout ? (unsigned) m * 4u : OOB, 0);
+        }
+
     issue(item_begin);
     for (int item = item_begin; item < item_end; ++item) {
         __syncthreads();   // everybody has read the previous patch (and, the first time, written the weights)
@@ -168,7 +178,7 @@ __global__ __launch_bounds__(256, 2) void stem_f32_kernel(const StemParams p) {
                 const float v = acc[a][r];
                 // bias after the full sum; without a bias the value is left alone (the sign of a zero sum) and, like the
                 // reference (conv.c:18-27), so is the activation: p.ep says NOT_ACT then
-                const float vb = __fadd_rn(v, buf_load_f32(rb, ok ? (unsigned) m * 4u : OOB, 0));
+                const float vb = __fadd_rn(v, bias_r[a][r]);
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(act_fast<EPI>(has_bias ? vb : v, p.ep)), ry, off, 0, 0);
             }
         }
