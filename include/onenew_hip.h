@@ -272,9 +272,9 @@ int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *p
  * the separate operator's operations in its order, the two 1x1 stages sum in MFMA order, so the block equals the chain of
  * operators within fp32 summation error.  No counterpart as one function in the reference.
  * onhip_ir_block_supported: 0 = this triple is not taken (16, 24, 32 or 64 input channels, expanded channels a multiple
- * of 16, at most 64 output channels, rows of a multiple of 4 and at most 128 output pixels, biases on the first two
- * convolutions), 1 = taken, 2 = taken and expected to be faster than the three launches (at least 256 bands of output rows
- * over the batch).  packed: both 1x1 weight tensors ([ce][cin] and [co][ce]) re-laid once by
+ * of 16, at most 64 output channels, rows of a multiple of 2 and at most 128 output pixels, biases on the first two
+ * convolutions), 1 = taken, 2 = taken and expected to be faster than the three launches (at most 32 input channels and at
+ * least 256 bands of output rows over the batch).  packed: both 1x1 weight tensors ([ce][cin] and [co][ce]) re-laid once by
  * onhip_ir_block_pack_weights (onhip_ir_block_packed_weight_bytes(cin, ce, co) bytes, 16-byte aligned). */
 int onhip_ir_block_supported(const onhip_conv_desc_t *expand, const onhip_conv_desc_t *dw, const onhip_conv_desc_t *project);
 size_t onhip_ir_block_packed_weight_bytes(int32_t cin, int32_t ce, int32_t co);

@@ -38,6 +38,7 @@ constexpr int IR_LDS_HALF = 80 * 1024;   // bytes of LDS a workgroup may take: t
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x32 __attribute__((ext_vector_type(32)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 struct IrParams {
     const float *x;        // [n][cin][h][w]
@@ -54,7 +55,8 @@ struct IrParams {
     int P;                 // in_rows * w: pixels of a band's input
     int xs_pitch;          // floats between the channels of Xs (P rounded up so that four rows fall into four bank groups)
     int tiles;             // ceil(P / 16)
-    int groups;            // 16-byte loads per channel: P / 4
+    int vec;               // floats per load of the block input: 4 (rows a multiple of 4 floats) or 2
+    int groups;            // loads per channel: P / vec
     int slots;             // loads per thread: ceil(cin * groups / 256)
     unsigned x_bytes;
     int xs_floats, patch_floats;   // LDS: Xs, then one or two patches
@@ -106,17 +108,25 @@ __global__ __launch_bounds__(256, 2) void irblock_f32_kernel(const IrParams p) {
             const bool live = f < p.cin * p.groups;
             const int ff = live ? f : 0;
             const int c = (int) div31((unsigned) ff, p.div_groups), g = ff - c * p.groups;
-            const int ir = (int) div31((unsigned) (4 * g), p.div_w);
+            const int ir = (int) div31((unsigned) (p.vec * g), p.div_w);   // a load lies inside one row: w is a multiple of vec
             const int ih = ih_first + ir;
             const bool in = live && (unsigned) ih < (unsigned) p.h;
-            // 4 g = ir * w + column: the float offset from the start of row ih_first
-            const unsigned off = in ? (unsigned) (((img * p.cin + c) * p.h + ih_first) * p.w + 4 * g) * 4u : OOB;
-            xr[i] = buf_load_b128(rx, off, 0);
-            l_off[i] = live ? c * p.xs_pitch + 4 * g : -1;
+            // vec * g = ir * w + column: the float offset from the start of row ih_first
+            const unsigned off = in ? (unsigned) (((img * p.cin + c) * p.h + ih_first) * p.w + p.vec * g) * 4u : OOB;
+            if (p.vec == 4) {   // uniform
+                xr[i] = buf_load_b128(rx, off, 0);
+            } else {
+                const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(rx, off, 0, 0);
+                xr[i] = make_uint4(t.x, t.y, 0u, 0u);
+            }
+            l_off[i] = live ? c * p.xs_pitch + p.vec * g : -1;
         }
 #pragma unroll
         for (int i = 0; i < IR_XSLOTS; ++i)
-            if (l_off[i] >= 0) *reinterpret_cast<uint4 *>(Xs + l_off[i]) = xr[i];
+            if (l_off[i] >= 0) {
+                if (p.vec == 4) *reinterpret_cast<uint4 *>(Xs + l_off[i]) = xr[i];
+                else *reinterpret_cast<uint2 *>(Xs + l_off[i]) = make_uint2(xr[i].x, xr[i].y);
+            }
     }
 
     // this lane's pixel of the band in the depthwise stage: patch offset of the window's top-left corner (a lane past the
@@ -361,7 +371,8 @@ static int ir_xs_pitch(int P) {
 
 // the band of output rows one workgroup takes, or 0 when the kernel does not fit the shape
 int irblock_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int cin) {
-    if (OW > IR_BN || dw.w % 4) return 0;
+    if (OW > IR_BN || dw.w % 2) return 0;
+    const int vec = dw.w % 4 ? 2 : 4;
     int rows = IR_BN / OW;
     rows = rows > OH ? OH : rows;
     if (const char *env = getenv("ONHIP_IR_ROWS")) {   // tuning hook: at most this many output rows per band
@@ -373,7 +384,7 @@ int irblock_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int cin) {
     for (; rows >= 1; --rows) {
         const int in_rows = (rows - 1) * dw.stride_h + 3;
         const int P = in_rows * dw.w;
-        const long long slots = ((long long) cin * (P / 4) + 255) / 256;
+        const long long slots = ((long long) cin * (P / vec) + 255) / 256;
         const long long lds = ((long long) cin * ir_xs_pitch(P) + 4 + (long long) IR_KC * in_rows * (dw.w + 2) + 4) * 4;
         if (lds > IR_LDS_HALF || slots > IR_XSLOTS || (P + 15) / 16 > 4 * IR_TPW) continue;
         if (!tallest) tallest = rows;
@@ -444,7 +455,8 @@ int irblock_f32_launch(const onhip_conv_desc_t &ex, const onhip_conv_desc_t &dw,
     p.P = p.in_rows * p.w;
     p.xs_pitch = ir_xs_pitch(p.P);
     p.tiles = (p.P + 15) / 16;
-    p.groups = p.P / 4;
+    p.vec = p.w % 4 ? 2 : 4;
+    p.groups = p.P / p.vec;
     p.slots = (p.cin * p.groups + 255) / 256;
     p.x_bytes = (unsigned) ((size_t) ex.n * ex.cin * ex.h * ex.w * 4);
     p.div_ow = make_div31((unsigned) OW);

@@ -43,12 +43,14 @@ def operands(tag, ex, dw, pw):
 
 
 # (n, input channels, expanded channels, h, w, output channels, stride, residual): MobileNetV2's blocks on the 112, 56 and
-# 28 pixel planes at a small batch, then ragged ones (odd heights, a last band shorter than the others, bands of one row
+# 28 pixel planes at a small batch (and one on the 14 pixel plane, rows of an even number of floats that is not a multiple
+# of four), then ragged ones (odd heights, a last band shorter than the others, bands of one row
 # and of the whole image, output channels not a multiple of 32, 64 input channels)
 SHAPES = [(2, 16, 96, 112, 112, 24, 2, False), (1, 24, 144, 56, 56, 24, 1, True), (2, 24, 144, 56, 56, 32, 2, False),
           (2, 32, 192, 28, 28, 32, 1, True), (2, 32, 192, 28, 28, 64, 2, False), (1, 16, 48, 20, 20, 40, 1, False),
           (2, 32, 64, 9, 12, 64, 2, False), (1, 24, 32, 37, 36, 24, 1, True), (1, 64, 128, 8, 8, 64, 1, True),
-          (1, 64, 128, 16, 16, 33, 1, False), (1, 16, 16, 5, 128, 8, 1, False), (3, 32, 160, 11, 44, 17, 2, False)]
+          (1, 64, 128, 16, 16, 33, 1, False), (1, 16, 16, 5, 128, 8, 1, False), (3, 32, 160, 11, 44, 17, 2, False),
+          (2, 64, 384, 14, 14, 64, 1, True), (1, 32, 64, 9, 18, 40, 2, False), (1, 16, 32, 6, 6, 16, 1, False)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -104,7 +106,7 @@ def test_depthwise_stage_is_the_reference_depthwise_bit_for_bit(shape, act, torc
 def test_block_says_what_it_does_not_take(torch_dev):
     torch = torch_dev
     z = torch.zeros(64, device="cuda")
-    ex, dw, pw = descs(1, 64, 384, 14, 14, 64, 1)          # rows of 14 pixels: not a multiple of 4
+    ex, dw, pw = descs(1, 64, 128, 7, 7, 64, 1)            # rows of 7 pixels: an odd number of floats
     assert hip.ir_block_supported(ex, dw, pw) == 0
     with pytest.raises(hip.OnhipError, match="band of output rows"):
         hip.ir_block_f32(ex, dw, pw, z, z, z, z, z, z)
