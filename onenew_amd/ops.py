@@ -30,7 +30,9 @@ class Plugin:
         self.eval.argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
         # entry points beside `eval` that the HIP Conv plugin has and the reference's plugins do not: the convolution
         # with the Add (and Relu) of a residual block folded in, the other operand of the Add in inputs[3]
-        for extra in ("eval_add", "eval_add_relu"):
+        # and a whole inverted-residual block (eval_block, eval_block_takes); the MatMul plugin's fused forms
+        for extra in ("eval_add", "eval_add_relu", "eval_block", "eval_block_takes", "eval_attention", "eval_bias", "eval_bias_gelu",
+                      "eval_bias_add"):
             fn = getattr(self.lib, extra, None) if hasattr(self.lib, extra) else None
             if fn is not None:
                 fn.restype = C.c_int
@@ -193,6 +195,56 @@ class Conv(_Op):
         return out
 
 
+class ConvBlock(_Op):
+    """Conv (1x1) -> Conv (depthwise 3x3) -> Conv (1x1) [-> Add] through the HIP Conv plugin's `eval_block`: the slots of the
+    first convolution's `eval` with the block's result operand in params[4], then the depthwise convolution's CONV_CONFIG_S,
+    weight operand, weights and bias in params[5], params[6], inputs[5], inputs[6] and the last convolution's in params[7],
+    params[8], inputs[7], inputs[8]; the addend in inputs[3].  No counterpart among the reference's host classes."""
+
+    def __init__(self, plugin, descs, weights, biases):
+        super().__init__(plugin.eval_block)
+        self.takes_fn = plugin.eval_block_takes
+        self.convs = [Conv(None, d, w, b) for d, w, b in zip(descs, weights, biases)]
+        ex, dw, pw = self.convs
+        oh, ow = pw.desc.out_hw()
+        self.out_shape = (pw.desc.n, pw.desc.cout, oh, ow)
+        self.out_operand = make_operand(self.out_shape, b"out")
+        self._slot(self.params_vec, 0, ex.conv_cfg)
+        self._slot(self.params_vec, 1, ex.in_operand)
+        self._slot(self.params_vec, 2, ex.weight_operand)
+        self._slot(self.params_vec, 3, ex.bias_operand)
+        self._slot(self.params_vec, 4, self.out_operand)
+        self._slot(self.inputs_vec, 1, ex.weight)
+        self._slot(self.inputs_vec, 2, ex.bias)
+        for base, conv in ((5, dw), (7, pw)):
+            self._slot(self.params_vec, base, conv.conv_cfg)
+            self._slot(self.params_vec, base + 1, conv.weight_operand)
+            self._slot(self.inputs_vec, base, conv.weight)
+            if conv.desc.has_bias:
+                self._slot(self.inputs_vec, base + 1, conv.bias)
+
+    def takes(self):
+        """1 when the library recommends the one-launch kernel for these shapes"""
+        return self.takes_fn(self.params_vec, self.inputs_vec, self.outputs_vec)
+
+    def __call__(self, x, addend=None, out=None):
+        xin = np.ascontiguousarray(x, dtype=np.float32)
+        if out is None:
+            out = aligned_empty(self.out_shape, np.float32)
+        self._slot(self.inputs_vec, 0, xin)
+        self._slot(self.outputs_vec, 0, out)
+        kept = 2
+        if addend is not None:
+            self._slot(self.inputs_vec, 3, np.ascontiguousarray(addend, dtype=np.float32))
+            kept = 3
+        rc = self.forward()
+        del self._keep[-kept:]
+        self.inputs_vec[3].addr = 0
+        if rc != 0:
+            raise RuntimeError(f"Conv eval_block returned {rc}")
+        return out
+
+
 class MatMul(_Op):
     """host/ops/mat_mul.h: out = A[..., M, K] @ B, B either [K, N] shared or batched like A."""
 
@@ -220,6 +272,68 @@ class MatMul(_Op):
         del self._keep[-6:]
         if rc != 0:
             raise RuntimeError(f"MatMul eval returned {rc}")
+        return out
+
+
+class MatMulFused(_Op):
+    """The HIP MatMul plugin's entry points beside `eval` (no counterpart among the reference's host classes):
+    linear(): MatMul -> Add of a bias [-> Gelu | -> Add of a tensor shaped like the result] through eval_bias /
+    eval_bias_gelu / eval_bias_add (bias in params[3] / inputs[2], result operand in params[4], Gelu table in inputs[11],
+    second addend in inputs[3]); attention(): MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v) through eval_attention
+    (q, k, v in params[1..3] / inputs[0..2], result in params[4], four int32 layout flags behind inputs[4])."""
+
+    def __init__(self, plugin):
+        super().__init__(None)
+        self.plugin = plugin
+        self.cfg = MATMUL_CONFIG_S()
+        self.cfg.op_base_cfg.op_type = b"MatMul"
+        self._slot(self.params_vec, 0, self.cfg)
+
+    def _run(self, fn, what):
+        rc = fn(self.params_vec, self.inputs_vec, self.outputs_vec)
+        for vec in (self.params_vec, self.inputs_vec, self.outputs_vec):
+            for i in range(1 if vec is self.params_vec else 0, BUF_MAXNUM):
+                vec[i].addr = 0
+        del self._keep[1:]
+        if rc != 0:
+            raise RuntimeError(f"MatMul {what} returned {rc}")
+
+    def linear(self, a, w, bias, gelu_lut=None, addend=None):
+        a, w, bias = (np.ascontiguousarray(t, dtype=np.float32) for t in (a, w, bias))
+        oshape = a.shape[:-1] + (w.shape[-1],)
+        out = aligned_empty(oshape, np.float32)
+        for i, o in enumerate([make_operand(a.shape, b"a"), make_operand(w.shape, b"w", fixed=True),
+                               make_operand(bias.shape, b"bias", fixed=True), make_operand(oshape, b"out")]):
+            self._slot(self.params_vec, 1 + i, o)
+        for i, t in enumerate((a, w, bias)):
+            self._slot(self.inputs_vec, i, t)
+        self._slot(self.outputs_vec, 0, out)
+        fn, what = self.plugin.eval_bias, "eval_bias"
+        if gelu_lut is not None:
+            self._slot(self.inputs_vec, BUF_MAXNUM - 1, np.ascontiguousarray(gelu_lut, dtype=np.float32))
+            fn, what = self.plugin.eval_bias_gelu, "eval_bias_gelu"
+        elif addend is not None:
+            self._slot(self.inputs_vec, 3, np.ascontiguousarray(addend, dtype=np.float32))
+            fn, what = self.plugin.eval_bias_add, "eval_bias_add"
+        self._run(fn, what)
+        return out
+
+    def attention(self, q, k, v, token_major=(0, 0, 0, 0)):
+        """q, k, v: [batch, heads, tokens, head_dim], or [batch, tokens, heads, head_dim] where the flag is set; so the
+        result (flag 3)"""
+        q, k, v = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v))
+        b, h, t, d = q.shape if not token_major[0] else (q.shape[0], q.shape[2], q.shape[1], q.shape[3])
+        oshape = (b, t, h, d) if token_major[3] else (b, h, t, d)
+        out = aligned_empty(oshape, np.float32)
+        for i, o in enumerate([make_operand(q.shape, b"q"), make_operand(k.shape, b"k"), make_operand(v.shape, b"v"),
+                               make_operand(oshape, b"out")]):
+            self._slot(self.params_vec, 1 + i, o)
+        for i, tns in enumerate((q, k, v)):
+            self._slot(self.inputs_vec, i, tns)
+        if any(token_major):
+            self._slot(self.inputs_vec, 4, np.asarray(token_major, dtype=np.int32))
+        self._slot(self.outputs_vec, 0, out)
+        self._run(self.plugin.eval_attention, "eval_attention")
         return out
 
 

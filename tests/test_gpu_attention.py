@@ -111,3 +111,24 @@ def test_attention_refuses_what_it_does_not_fuse(torch_dev):
     with pytest.raises(hip.OnhipError, match="multiples of 4"):
         base = z(1, 1, 8, 66)
         hip.attention(base[..., :64], z(1, 1, 8, 64), z(1, 1, 8, 64))
+
+
+@pytest.mark.parametrize("flags", [(0, 0, 0, 0), (1, 1, 1, 1), (0, 1, 0, 1)])
+def test_plugin_eval_attention_host_buffers(flags, torch_dev, oracle):
+    """the MatMul plugin's eval_attention on tensors in host memory, with and without the layout flags that say a tensor
+    is stored [batch, tokens, heads, head_dim] (the far side of a head-split / head-merge Transpose): 1e-4 against the
+    oracle's chain Transpose -> MatMul -> Softmax -> MatMul"""
+    from onenew_amd import ops
+    b, h, t, hd = 2, 3, 50, 64
+    g = cases.datagen
+    q, k, v = (g.normal(g.seed_for("plug_attn", n, *flags), (b, h, t, hd), 0.0, 0.5) for n in "qkv")
+    kt = oracle.transpose_f32(k, (0, 1, 3, 2))
+    p = oracle.softmax_f32(oracle.matmul_f32(q.reshape(b * h, t, hd), kt.reshape(b * h, hd, t)))
+    ref = oracle.matmul_f32(p, v.reshape(b * h, t, hd)).reshape(b, h, t, hd)
+    given = [np.ascontiguousarray(x.transpose(0, 2, 1, 3)) if f else x for x, f in zip((q, k, v), flags)]
+    op = ops.MatMulFused(ops.Plugin(hip.plugin_path("MatMul")))
+    got = op.attention(*given, token_major=flags)
+    if flags[3]:
+        got = got.transpose(0, 2, 1, 3)
+    assert got.shape == ref.shape
+    assert np.abs(got.astype(np.float64) - ref).max() <= 1e-4 * np.abs(ref).max()

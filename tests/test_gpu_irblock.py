@@ -103,6 +103,28 @@ def test_depthwise_stage_is_the_reference_depthwise_bit_for_bit(shape, act, torc
     assert np.array_equal(got, ref), f"{(got != ref).sum()} of {ref.size} depthwise values differ"
 
 
+@pytest.mark.parametrize("shape", [(2, 16, 96, 28, 28, 24, 2, False), (1, 32, 64, 20, 20, 32, 1, True)])
+def test_plugin_eval_block_host_buffers(shape, torch_dev, oracle):
+    """the Conv plugin's eval_block on tensors in host memory, slots filled like the host fills a Conv's (weights and
+    biases as fixed operands, the block's result operand in params[4]): within 1e-4 of the oracle's operator chain, a second
+    call (cached weights) identical, and eval_block_takes saying that so small a batch is not recommended"""
+    from onenew_amd import ops
+    n, cin, ce, h, w, co, stride, with_res = shape
+    ex, dw, pw = descs(n, cin, ce, h, w, co, stride)
+    x, ex_w, ex_b, dw_w, dw_b, pw_w, pw_b = operands(f"irplugin{shape}", ex, dw, pw)
+    oh, ow = dw.out_hw()
+    res = cases.datagen.normal(cases.datagen.seed_for("irplugin", "res", *shape[:7]), (n, co, oh, ow), 0.0, 1.0) if with_res else None
+    block = ops.ConvBlock(ops.Plugin(hip.plugin_path("Conv")), (ex, dw, pw), (ex_w, dw_w, pw_w), (ex_b, dw_b, pw_b))
+    assert block.takes() == 0
+    y = block(x, addend=res).copy()
+    assert np.array_equal(block(x, addend=res), y)
+    ref = oracle.conv2d_f32(pw, oracle.conv2d_f32(dw, oracle.conv2d_f32(ex, x, ex_w, ex_b), dw_w, dw_b), pw_w, pw_b)
+    if with_res:
+        ref = ref + res
+    top = np.abs(ref).max()
+    assert np.abs(y.astype(np.float64) - ref).max() <= 1e-4 * top
+
+
 def test_block_says_what_it_does_not_take(torch_dev):
     torch = torch_dev
     z = torch.zeros(64, device="cuda")

@@ -575,6 +575,24 @@ def test_matmul_bias_add_fused(shape, compute, torch_dev, oracle):
         hip.matmul(dev(torch, a), dev(torch, w), addend=out, out=out)
 
 
+def test_plugin_matmul_fused_entries_host_buffers(torch_dev, oracle):
+    """eval_bias, eval_bias_gelu and eval_bias_add of the MatMul plugin on tensors in host memory: each equal, bit for bit,
+    to the operators it replaces as this library computes them (MatMul through `eval`, then the oracle's Add / table Gelu /
+    Add on that result)"""
+    a, w = cases.matmul_inputs("plug_linear", (3, 37, 48), (48, 40))
+    bias = cases.datagen.normal(cases.datagen.seed_for("plug_linear", "bias"), (40,), 0.0, 0.2)
+    skip = cases.datagen.normal(cases.datagen.seed_for("plug_linear", "skip"), (3, 37, 40), 0.0, 1.0)
+    lut = cases.gelu_lut()
+    plug = ops.Plugin(hip.plugin_path("MatMul"))
+    plain = ops.MatMul(plug.eval)(a, w)
+    fused = ops.MatMulFused(plug)
+    with_bias = oracle.add_f32(plain, bias)
+    assert np.array_equal(fused.linear(a, w, bias), with_bias)
+    assert np.array_equal(fused.linear(a, w, bias, gelu_lut=lut), oracle.lut_act(with_bias, lut))
+    assert np.array_equal(fused.linear(a, w, bias, addend=skip), oracle.add_f32(with_bias, skip))
+    assert_close_f32(with_bias, oracle.matmul_f32(a, w, bias=bias), rel=1e-4, tag="plugin linear")
+
+
 @pytest.mark.parametrize("name", list(cases.gemm_cases()))
 def test_gemm_f32(name, torch_dev, oracle, golden):
     torch = torch_dev
