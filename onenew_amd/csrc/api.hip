@@ -995,6 +995,12 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
         rc = quantised_table(ep.lut, p.out_inv_scale, st, &p.ep.qlut);
         if (rc) return rc;
     }
+    // 3x3, stride 1, few channels, int8 in and out: the kernel that keeps the band's input in LDS and the weights in registers
+    // tuning hooks: ONHIP_NO_PATCH keeps to the implicit-GEMM kernels, and so does a forced tile of theirs; ONHIP_PATCH_ALL
+    // sends every shape the LDS-patch kernel can take to it, not only those it is measured to win
+    const bool no_patch = getenv("ONHIP_NO_PATCH") != nullptr || getenv("ONHIP_TILE") != nullptr;
+    if (nhwc_out && !no_patch && i8patch_ok(p, getenv("ONHIP_PATCH_ALL") != nullptr)) return i8patch_launch(p, st);
+    if (nhwc_out && !no_patch && i8direct_ok(p)) return i8direct_launch(p, st);
     return plan_and_launch(cfg, p, st);
 }
 

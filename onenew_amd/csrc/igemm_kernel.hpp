@@ -436,11 +436,12 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
 // between M and the pitch are written as zero.  stage: BN * (BM + 16) bytes of LDS nobody reads any more.
 // rows: when not null, LDS holding the tile's per-row constants, BM de-quantisation factors weight_aux / 127 followed by
 // the BM int32 biases as floats (rows m0 .. m0 + BM - 1), which the caller computed once per row; otherwise every lane
-// fetches and divides for its own 16 x TM rows.
+// fetches and divides for its own 16 x TM rows.  table_ready: the caller (a persistent workgroup) has already copied the
+// quantised activation table to stage + BN * (BM + 16).
 template <int EPI, int BM, int BN, int TM, int TN, bool QLUT_IN_LDS, class ACC>
 __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&acc)[TM][TN], unsigned char *stage, int m0,
                                                    int n0, int m_wave, int n_wave, int li, int lh, int tid,
-                                                   const float *rows = nullptr) {
+                                                   const float *rows = nullptr, bool table_ready = false) {
     constexpr int PITCH = BM + 16;
     const unsigned lh16 = (unsigned) lh * 16u;
     float aux[TM][16];      // the factor weight_aux / 127 of each of the lane's rows
@@ -480,10 +481,13 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
     lds_s8_t qtab_lds = nullptr;
     if (EPI == EPI_LUT && p.ep.qlut && QLUT_IN_LDS) {
         unsigned char *ql = stage + BN * PITCH;
-        const uint4 *src = reinterpret_cast<const uint4 *>(p.ep.qlut);
+        if (!table_ready) {   // uniform
+            const uint4 *src = reinterpret_cast<const uint4 *>(p.ep.qlut);
 #pragma unroll
-        for (int i = 0; i < 8192 / 16 / THREADS; ++i) reinterpret_cast<uint4 *>(ql)[tid + i * THREADS] = src[tid + i * THREADS];
-        __syncthreads();
+            for (int i = 0; i < 8192 / 16 / THREADS; ++i) reinterpret_cast<uint4 *>(ql)[tid + i * THREADS] = src[tid + i * THREADS];
+            if (tid == 0) ql[-1] = 0;   // the entry "below the table": see the gather
+            __syncthreads();
+        }
         qtab_lds = (lds_s8_t) ql;
     }
     const bool has_bias = p.bias32 != nullptr;
@@ -507,7 +511,38 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
                     f = has_bias ? fbias : f;
                     x[b][j] = __fmul_rn(f, aux[a][r]);
                 }
-            if (table) {   // act_fast<EPI_LUT>'s rules with the table behind the output quantiser
+            if (table && QLUT_IN_LDS) {
+                // act_fast<EPI_LUT>'s rules with the table behind the output quantiser and in LDS.  (x + 8) * 512 as one
+                // fused multiply-add: the product by 512 is exact, so both round x + 8 once.  Rounded DOWN to an integer
+                // and held to -1 .. 8191, the index says "below the table" (x < -8: the result is 0) as -1, and the byte
+                // before the table, the last of the staging area's padding that no store or read touches, holds that 0.
+                unsigned l[TN][4];
+                bool beyond = false;
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        int idx;
+                        asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(idx) : "v"(__builtin_fmaf(x[b][j], 512.0f, 4096.0f)));
+                        idx = max(-1, min(idx, 8191));
+                        l[b][j] = (unsigned char) qtab_lds[idx];
+                        beyond |= x[b][j] >= 8.0f;
+                    }
+                // beyond the table the activation is the identity: rare enough that a wavefront usually skips this whole
+                if (__builtin_amdgcn_ballot_w64(beyond) != 0ull) {
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const unsigned hi = (unsigned) requant_s8(x[b][j], p.out_inv_scale) & 0xffu;
+                            l[b][j] = x[b][j] >= 8.0f ? hi : l[b][j];
+                        }
+                }
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) q8[b][j] = (int) l[b][j];
+            } else if (table) {   // the same from the table in global memory
                 int l[TN][4];
 #pragma unroll
                 for (int b = 0; b < TN; ++b)
@@ -515,8 +550,7 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
                     for (int j = 0; j < 4; ++j) {
                         int idx = (int) __fmul_rn(__fadd_rn(x[b][j], 8.0f), 512.0f);
                         idx = idx < 0 ? 0 : idx > 8191 ? 8191 : idx;
-                        if constexpr (QLUT_IN_LDS) l[b][j] = qtab_lds[idx];
-                        else l[b][j] = qtab[idx];
+                        l[b][j] = qtab[idx];
                     }
                 bool beyond = false;
 #pragma unroll
@@ -526,7 +560,6 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
                         q8[b][j] = x[b][j] < -8.0f ? 0 : l[b][j];
                         beyond |= x[b][j] >= 8.0f;
                     }
-                // beyond the table the activation is the identity: rare enough that a wavefront usually skips this whole
                 if (__builtin_amdgcn_ballot_w64(beyond) != 0ull) {
 #pragma unroll
                     for (int b = 0; b < TN; ++b)
@@ -542,16 +575,16 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
 #pragma unroll
                     for (int j = 0; j < 4; ++j) q8[b][j] = requant_s8(act_fast<EPI>(x[b][j], p.ep), p.out_inv_scale);
             }
+            // channels past the last are stored as zero: a mask over the word of four
+            const int left = p.M - (m0 + ml);
+            const unsigned keep = left >= 4 ? 0xffffffffu : left <= 0 ? 0u : (1u << (8 * left)) - 1u;
 #pragma unroll
             for (int b = 0; b < TN; ++b) {
                 unsigned packed = 0;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int v = (m0 + ml + j < p.M) ? q8[b][j] : 0;
-                    packed |= ((unsigned) v & 0xffu) << (8 * j);
-                }
+                for (int j = 0; j < 4; ++j) packed |= ((unsigned) q8[b][j] & 0xffu) << (8 * j);
                 const int nl = n_wave - n0 + b * 32 + li;
-                *reinterpret_cast<unsigned *>(stage + nl * PITCH + ml) = packed;
+                *reinterpret_cast<unsigned *>(stage + nl * PITCH + ml) = packed & keep;
             }
         }
     __syncthreads();

@@ -243,6 +243,13 @@ int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, flo
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
 int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
 int forget_quantised_tables(const void *base, size_t bytes);   // api.hip: the cache of tables behind an output quantiser
+// i8patch.hip: int8 NHWC 3x3 convolutions with few channels from an LDS-resident input patch
+struct IgemmParams;
+bool i8patch_ok(const IgemmParams &p, bool any_shape);
+int i8patch_launch(const IgemmParams &p, hipStream_t stream);
+bool i8direct_ok(const IgemmParams &p);
+int i8direct_launch(const IgemmParams &p, hipStream_t stream);
+
 // irblock.hip: 1x1 expansion -> depthwise 3x3 -> 1x1 projection in one launch
 int irblock_pack_launch(const float *w_exp, const float *w_proj, int cin, int ce, int co, float *packed, hipStream_t stream);
 int irblock_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int cin);
