@@ -172,15 +172,15 @@ __global__ __launch_bounds__(256, 2) void i8patch_kernel(const IgemmParams p, co
     }
 }
 
-// The same convolution without the patch: every lane loads the 16 bytes of its pixel under each filter tap straight from
+// The same convolution, and 1x1 convolutions, without the patch: every lane loads the 16 bytes of its pixel under each filter tap straight from
 // global memory (zeros outside the image from the buffer descriptor's range check).  For strides above 1, where windows
 // share few pixels, and for 16 bytes per pixel (up to 16 input channels: a network's first layer), where two taps fill
 // one MFMA step: K index 32 k + 16 half of step k is tap (32 k + 16 half) / CB, byte (32 k + 16 half) % CB of the pixel,
 // and the packed weights ([m][tap][CB]) are read at that same index.  A persistent workgroup walks blocks of BN output
 // pixels of the whole batch; the next block's loads are in flight while this one is stored.
-template <int CB, int WM, int TN, int OCC>
+template <int CB, int TAPS, int WM, int TM, int TN, int OCC>
 __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p, const int blocks) {
-    constexpr int NK = (9 * CB + 31) / 32, WN = 4 / WM, BM = 32 * WM, BN = 32 * TN * WN;
+    constexpr int NK = (TAPS * CB + 31) / 32, WN = 4 / WM, BM = 32 * TM * WM, BN = 32 * TN * WN;
     constexpr int STAGE = BN * (BM + 16);
     __shared__ __attribute__((aligned(16))) unsigned char lds[STAGE + 8192 + 2 * BM * 4];
     unsigned char *const stage = lds;
@@ -190,15 +190,18 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
     const int li = lane & 31, lh = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
 
-    i32x4 areg[NK];
+    i32x4 areg[TM][NK];
     {
         const rsrc_t ra = make_rsrc(p.A, (unsigned) p.a_slice_bytes);
-        const int m = 32 * wm + li;
 #pragma unroll
-        for (int k = 0; k < NK; ++k) {
-            const int kk = 32 * k + 16 * lh;
-            const uint4 q = buf_load_b128(ra, m < p.M && kk < 9 * CB ? (unsigned) (m * p.lda + kk) : OOB, 0);
-            areg[k] = i32x4{(int) q.x, (int) q.y, (int) q.z, (int) q.w};
+        for (int a = 0; a < TM; ++a) {
+            const int m = 32 * (TM * wm + a) + li;
+#pragma unroll
+            for (int k = 0; k < NK; ++k) {
+                const int kk = 32 * k + 16 * lh;
+                const uint4 q = buf_load_b128(ra, m < p.M && kk < TAPS * CB ? (unsigned) (m * p.lda + kk) : OOB, 0);
+                areg[a][k] = i32x4{(int) q.x, (int) q.y, (int) q.z, (int) q.w};
+            }
         }
     }
     if (tid < BM) {
@@ -219,9 +222,10 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
     int tap_i[NK], tap_j[NK], tap_byte[NK];
 #pragma unroll
     for (int k = 0; k < NK; ++k) {
-        const int kk = 32 * k + 16 * lh, tap = kk / CB;   // a power of two
-        tap_i[k] = tap < 9 ? (tap * 11) >> 5 : 1 << 28;   // tap / 3 for tap < 10; past the last tap: outside any image
-        tap_j[k] = tap - 3 * ((tap * 11) >> 5);
+        const int kk = 32 * k + 16 * lh, tap = kk / CB;
+        const int ti = TAPS == 9 ? (tap * 11) >> 5 : 0;    // tap / 3 for tap < 10
+        tap_i[k] = tap < TAPS ? ti : 1 << 28;              // past the last tap: outside any image
+        tap_j[k] = tap - (TAPS == 9 ? 3 : 1) * ti;
         tap_byte[k] = kk % CB;
     }
     const rsrc_t rx = make_rsrc(p.B, (unsigned) p.b_slice_bytes);
@@ -247,59 +251,67 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
     int blk = blockIdx.x;
     if (blk < blocks) issue(blk);
     for (; blk < blocks; blk += gridDim.x) {
-        i32x16 acc[1][TN];
+        i32x16 acc[TM][TN];
 #pragma unroll
-        for (int b = 0; b < TN; ++b) {
+        for (int a = 0; a < TM; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[0][b][r] = 0;
+            for (int b = 0; b < TN; ++b) {
 #pragma unroll
-            for (int k = 0; k < NK; ++k) {
-                const i32x4 bv = i32x4{(int) bx[b][k].x, (int) bx[b][k].y, (int) bx[b][k].z, (int) bx[b][k].w};
-                acc[0][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[k], bv, acc[0][b], 0, 0, 0);
+                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const i32x4 bv = i32x4{(int) bx[b][k].x, (int) bx[b][k].y, (int) bx[b][k].z, (int) bx[b][k].w};
+                    acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[a][k], bv, acc[a][b], 0, 0, 0);
+                }
             }
-        }
         if (blk + (int) gridDim.x < blocks) issue(blk + gridDim.x);   // uniform
         __syncthreads();   // the previous block's store has left the staging area (and, the first time, the table is there)
-        const int n0 = blk * BN, m_wave = 32 * wm, n_wave = n0 + 32 * TN * wn;
+        const int n0 = blk * BN, m_wave = 32 * TM * wm, n_wave = n0 + 32 * TN * wn;
         switch (p.ep.act) {
             case NOT_ACT:
-            case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, 1, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, 1, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, 1, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+            case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+            case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+            case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
             case SILU:
-            case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, 1, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, 1, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+            case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+            default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN, true>(p, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
         }
     }
 }
 
 // the int8 NHWC chain form of a 3x3 convolution of any stride and padding with 16 or 32 bytes per input pixel and at most
-// 64 output channels
+// 64 output channels; of a 1x1 convolution with 64, 96 or 128 bytes per pixel and at most 64 output channels (with two
+// row tiles per wavefront, up to 128 channels, it was measured level with the implicit-GEMM kernels or behind them)
 bool i8direct_ok(const IgemmParams &p) {
     if (!p.out_s8 || p.out_mode != OUT_PLAIN || p.c_stride_m != 1 || p.acc_out) return false;
-    if (p.kh != 3 || p.kw != 3 || p.M > 64) return false;
-    if (p.pix_stride != 16 && p.pix_stride != 32) return false;
-    if (p.lda != 9 * p.pix_stride || p.b_slice_bytes >= (1LL << 31) - 64) return false;
-    return true;
+    if (p.lda != p.khkw * p.pix_stride || p.b_slice_bytes >= (1LL << 31) - 64) return false;
+    if (p.kh == 3 && p.kw == 3) return p.M <= 64 && (p.pix_stride == 16 || p.pix_stride == 32);
+    if (p.kh == 1 && p.kw == 1) return p.M <= 64 && (p.pix_stride == 64 || p.pix_stride == 96 || p.pix_stride == 128);
+    return false;
 }
 
-template <int CB, int WM, int TN, int OCC>
+template <int CB, int TAPS, int WM, int TM, int TN, int OCC>
 static int i8direct_launch_one(IgemmParams p, hipStream_t stream) {
     constexpr int BN = 32 * TN * (4 / WM);
     const int blocks = (p.N + BN - 1) / BN;
     p.div_ohw = make_div31((unsigned) p.OHW);
     p.div_ow = make_div31((unsigned) p.OW);
     const int grid = blocks < 256 * OCC ? blocks : 256 * OCC;   // OCC workgroups per compute unit
-    hipLaunchKernelGGL((i8direct_kernel<CB, WM, TN, OCC>), dim3((unsigned) grid), dim3(256), 0, stream, p, blocks);
+    hipLaunchKernelGGL((i8direct_kernel<CB, TAPS, WM, TM, TN, OCC>), dim3((unsigned) grid), dim3(256), 0, stream, p, blocks);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }
 
 int i8direct_launch(const IgemmParams &p, hipStream_t stream) {
+    if (p.kh == 1) {
+        if (p.pix_stride == 64) return i8direct_launch_one<64, 1, 2, 1, 2, 2>(p, stream);
+        if (p.pix_stride == 96) return i8direct_launch_one<96, 1, 2, 1, 2, 2>(p, stream);
+        return i8direct_launch_one<128, 1, 2, 1, 2, 2>(p, stream);
+    }
     // measured on a first layer (3 -> 32 channels, stride 2) and the layer after it (32 -> 64): three workgroups per
     // compute unit help the former, whose time is the store's arithmetic; smaller or larger blocks help neither
-    if (p.pix_stride == 16) return p.M <= 32 ? i8direct_launch_one<16, 1, 2, 3>(p, stream) : i8direct_launch_one<16, 2, 2, 2>(p, stream);
-    return p.M <= 32 ? i8direct_launch_one<32, 1, 2, 2>(p, stream) : i8direct_launch_one<32, 2, 2, 2>(p, stream);
+    if (p.pix_stride == 16) return p.M <= 32 ? i8direct_launch_one<16, 9, 1, 1, 2, 3>(p, stream) : i8direct_launch_one<16, 9, 2, 1, 2, 2>(p, stream);
+    return p.M <= 32 ? i8direct_launch_one<32, 9, 1, 1, 2, 2>(p, stream) : i8direct_launch_one<32, 9, 2, 1, 2, 2>(p, stream);
 }
 
 static int i8patch_rows(const IgemmParams &p, int *big);

@@ -39,7 +39,7 @@ LEGEND = ("Kernel names: `onhip::igemm_kernel<dtype, loader, BM, BN, WM, WN, PF,
           "16-bit storage: operand tiles loaded straight into LDS, KS bytes of K per stage, ring of NST stages), `onhip::rowb_f32_kernel<WM, WN>` (fp32, B "
           "straight from memory, tile 32 WM x 128 WN), `onhip::splitk_finish_kernel`, `onhip::depthwise_tiled_kernel<int8, stride, "
           "act>`, `onhip::quantize_nhwc_kernel<CBW>`, `onhip::stem_f32_kernel<filter size, act, two row tiles>` (first-layer "
-          "convolutions from an LDS patch), `onhip::i8patch_kernel<bytes per pixel, WM, pixel tiles>` and `onhip::i8direct_kernel<bytes per pixel, WM, pixel "
+          "convolutions from an LDS patch), `onhip::i8patch_kernel<bytes per pixel, WM, pixel tiles>` and `onhip::i8direct_kernel<bytes per pixel, taps, WM, TM, pixel "
           "tiles, workgroups per CU>` (int8 chain form, 3x3 with few channels: input rows in LDS / windows loaded per tap), `onhip::attention_f32_kernel<key tiles, head dim>`, `onhip::dwproj_f32_kernel<act, row "
           "tiles, vector width>` (depthwise 3x3 + 1x1 in one launch), `onhip::irblock_f32_kernel<act, input channels / 4, row tiles, "
           "patches>` (1x1 expansion + depthwise 3x3 + 1x1 projection in one launch), and the element-wise kernels.")

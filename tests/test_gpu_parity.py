@@ -1283,22 +1283,26 @@ def test_tune_cache_file_is_validated_and_rewritten(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", [
-    # (n, cin, h, w, cout, stride, pad): 16 bytes per pixel (two taps per MFMA step), first layers
-    (2, 3, 30, 30, 32, 2, 1), (1, 3, 33, 47, 16, 2, 1), (3, 8, 17, 21, 40, 1, 1), (2, 16, 12, 19, 64, 2, 0), (1, 4, 9, 70, 24, 1, 2),
+    # (n, cin, h, w, cout, k, stride, pad): 16 bytes per pixel (two taps per MFMA step), first layers
+    (2, 3, 30, 30, 32, 3, 2, 1), (1, 3, 33, 47, 16, 3, 2, 1), (3, 8, 17, 21, 40, 3, 1, 1), (2, 16, 12, 19, 64, 3, 2, 0), (1, 4, 9, 70, 24, 3, 1, 2),
     # 32 bytes per pixel: stride 1 with pads 1 (the rows of a band kept in LDS), other strides and pads (loaded per tap)
-    (2, 32, 20, 20, 32, 1, 1), (1, 24, 13, 37, 16, 1, 1), (2, 32, 16, 160, 32, 1, 1), (1, 32, 7, 256, 24, 1, 1), (3, 20, 5, 6, 64, 1, 1),
-    (2, 32, 21, 23, 64, 2, 1), (1, 32, 18, 18, 48, 1, 0), (2, 17, 15, 15, 32, 2, 1), (1, 32, 40, 80, 64, 1, 1),
+    (2, 32, 20, 20, 32, 3, 1, 1), (1, 24, 13, 37, 16, 3, 1, 1), (2, 32, 16, 160, 32, 3, 1, 1), (1, 32, 7, 256, 24, 3, 1, 1), (3, 20, 5, 6, 64, 3, 1, 1),
+    (2, 32, 21, 23, 64, 3, 2, 1), (1, 32, 18, 18, 48, 3, 1, 0), (2, 17, 15, 15, 32, 3, 2, 1), (1, 32, 40, 80, 64, 3, 1, 1),
     # 64 bytes per pixel, stride 1, pads 1
-    (2, 64, 20, 20, 64, 1, 1), (1, 48, 11, 80, 32, 1, 1), (1, 64, 9, 13, 40, 1, 1)])
+    (2, 64, 20, 20, 64, 3, 1, 1), (1, 48, 11, 80, 32, 3, 1, 1), (1, 64, 9, 13, 40, 3, 1, 1),
+    # 1x1 with 64, 96 or 128 bytes per pixel, a stride, a pad; more than 64 output channels (the implicit-GEMM kernels')
+    (2, 64, 20, 20, 64, 1, 1, 0), (1, 50, 13, 37, 40, 1, 1, 0), (2, 96, 9, 31, 48, 1, 1, 0), (1, 90, 16, 16, 64, 1, 2, 0),
+    (3, 128, 7, 11, 33, 1, 1, 0), (1, 128, 24, 24, 64, 1, 1, 1), (2, 100, 5, 5, 16, 1, 1, 0), (1, 128, 12, 12, 80, 1, 1, 0)])
 @pytest.mark.parametrize("act", [abi.SILU, abi.RELU, abi.NOT_ACT])
 def test_conv_int8_chain_3x3_with_few_channels(shape, act, torch_dev, oracle, monkeypatch):
-    """3x3 convolutions of the int8 NHWC chain form with at most 64 input channels and 64 output channels: whichever kernel
+    """3x3 convolutions of the int8 NHWC chain form with at most 64 input channels and 64 output channels, and 1x1
+    convolutions with at most 128 and 64: whichever kernel
     takes them (input rows of a band in LDS, or windows loaded per tap, or the implicit-GEMM kernels), the bytes are the
     oracle's, and the same with the LDS kernel given every shape it can take and with those two kernels switched off; ragged sizes, pixels past the last block, pads 0 to 2"""
     torch = torch_dev
-    n, cin, h, w, cout, stride, pad = shape
-    d = cases.cd(cin, cout, 3, stride, pad, h, w=w, n=n, act=act, input_scale=0.041, out_s8=1, output_scale=0.052)
-    x, w8, b32, aux = cases.conv_inputs(f"few_{cin}_{cout}_{h}_{w}_{stride}_{pad}", d, quant=True)
+    n, cin, h, w, cout, k, stride, pad = shape
+    d = cases.cd(cin, cout, k, stride, pad, h, w=w, n=n, act=act, input_scale=0.041, out_s8=1, output_scale=0.052)
+    x, w8, b32, aux = cases.conv_inputs(f"few_{cin}_{cout}_{h}_{w}_{k}_{stride}_{pad}", d, quant=True)
     lut = cases.silu_lut()
     oh, ow = d.out_hw()
     ref = np.transpose(oracle.conv2d_w8a32(d, x, w8, b32, aux, lut), (0, 2, 3, 1))
