@@ -34,6 +34,19 @@ struct PatchGeom {
     Div31 div_ow, div_rowvecs, div_parts;
 };
 
+// Which items of 0 .. total - 1 a persistent workgroup takes: workgroups are dealt to the 8 XCDs in turn, each with an L2 of
+// its own, so XCD x gets the x-th contiguous eighth of the items and its workgroups walk that eighth together; items next
+// to each other (bands and blocks of neighbouring image rows, which share input rows) then meet in one L2 at about the
+// same time.  With a grid that is not a multiple of 8: plain striding.
+struct ItemWalk { int first, end, step; };
+__device__ __forceinline__ ItemWalk xcd_walk(int total) {
+    const int g = (int) gridDim.x;
+    if (g % 8 != 0) return {(int) blockIdx.x, total, g};
+    const int xcd = (int) blockIdx.x & 7, chunk = (total + 7) >> 3;
+    const int lo = xcd * chunk, hi = min(total, lo + chunk);
+    return {lo + ((int) blockIdx.x >> 3), hi, g >> 3};
+}
+
 // WM = 1: the four wavefronts side by side over the pixels (up to 32 output channels); WM = 2: two rows of two (up to 64),
 // so a wavefront holds the weights of one 32-row tile only.  TN: 32-pixel tiles per wavefront.
 template <int CB, int WM, int TN>
@@ -122,15 +135,16 @@ __global__ __launch_bounds__(256, 2) void i8patch_kernel(const IgemmParams p, co
     };
 
     IgemmParams ps = p;   // the store's view of the problem: the band's pixels only
-    int band = blockIdx.x;
-    if (band < g.total) issue(band);
-    for (; band < g.total; band += gridDim.x) {
+    const ItemWalk walk = xcd_walk(g.total);
+    int band = walk.first;
+    if (band < walk.end) issue(band);
+    for (; band < walk.end; band += walk.step) {
         __syncthreads();   // everybody is done with the previous band's patch and staging area
 #pragma unroll
         for (int i = 0; i < P8_SLOTS; ++i)
             if (l_off[i] >= 0) *reinterpret_cast<uint4 *>(patch + l_off[i]) = xr[i];
         __syncthreads();
-        if (band + (int) gridDim.x < g.total) issue(band + gridDim.x);   // uniform
+        if (band + walk.step < walk.end) issue(band + walk.step);   // uniform
 
         i32x16 acc[1][TN];
 #pragma unroll
@@ -248,9 +262,10 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
         }
     };
 
-    int blk = blockIdx.x;
-    if (blk < blocks) issue(blk);
-    for (; blk < blocks; blk += gridDim.x) {
+    const ItemWalk walk = xcd_walk(blocks);
+    int blk = walk.first;
+    if (blk < walk.end) issue(blk);
+    for (; blk < walk.end; blk += walk.step) {
         i32x16 acc[TM][TN];
 #pragma unroll
         for (int a = 0; a < TM; ++a)
@@ -264,7 +279,7 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
                     acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[a][k], bv, acc[a][b], 0, 0, 0);
                 }
             }
-        if (blk + (int) gridDim.x < blocks) issue(blk + gridDim.x);   // uniform
+        if (blk + walk.step < walk.end) issue(blk + walk.step);   // uniform
         __syncthreads();   // the previous block's store has left the staging area (and, the first time, the table is there)
         const int n0 = blk * BN, m_wave = 32 * TM * wm, n_wave = n0 + 32 * TN * wn;
         switch (p.ep.act) {
@@ -296,7 +311,7 @@ static int i8direct_launch_one(IgemmParams p, hipStream_t stream) {
     const int blocks = (p.N + BN - 1) / BN;
     p.div_ohw = make_div31((unsigned) p.OHW);
     p.div_ow = make_div31((unsigned) p.OW);
-    const int grid = blocks < 256 * OCC ? blocks : 256 * OCC;   // OCC workgroups per compute unit
+    const int grid = blocks < 256 * OCC ? (blocks + 7) / 8 * 8 : 256 * OCC;   // OCC workgroups per compute unit; a multiple of 8 (xcd_walk)
     hipLaunchKernelGGL((i8direct_kernel<CB, TAPS, WM, TM, TN, OCC>), dim3((unsigned) grid), dim3(256), 0, stream, p, blocks);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
@@ -342,8 +357,8 @@ static int i8patch_launch_one(const IgemmParams &p, PatchGeom g, hipStream_t str
                                             80 * 1024));
         allowed.store(80 * 1024);
     }
-    int grid = 512;   // two workgroups per compute unit
-    grid = grid > g.total ? g.total : grid;
+    int grid = 512;   // two workgroups per compute unit; a multiple of 8 (xcd_walk)
+    grid = grid > g.total ? (g.total + 7) / 8 * 8 : grid;
     hipLaunchKernelGGL((i8patch_kernel<CB, WM, TN>), dim3((unsigned) grid), dim3(256), lds, stream, p, g);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
