@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
 Workloads: resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
-cfg1, resnet50_net_b{1,32}, mobilenetv2_net_b{1,64} and vit_tiny_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
+cfg1, resnet50_net_b{1,32}, resnet50_int8_net_b{1,32} (the same with W8A32 convolutions), mobilenetv2_net_b{1,64} and vit_tiny_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
 the HBM traffic counters are scaled by).
 
 A step is one pass over every layer of the workload: one launch per layer, inputs, weights and outputs
@@ -685,6 +685,9 @@ def bench_net(torch, args):
     n = int(args.workload.split("_b")[1])
     model = "ResNet-50" if args.workload.startswith("resnet50") else "MobileNetV2" if args.workload.startswith("mobilenetv2") else "ViT-Tiny"
     make = {"ResNet-50": stacks.resnet50_model, "MobileNetV2": stacks.mobilenet_v2_model, "ViT-Tiny": stacks.vit_tiny_model}[model]
+    int8 = "_int8_net_" in args.workload   # the convolutions in the W8A32 form of the offline quantiser
+    if int8:
+        make = lambda batch: stacks.resnet50_model(batch, quantised=True)   # noqa: E731
     data, in_shape, flops = make(n)
     net = rt.Net(data)
     x = torch.randn(in_shape, dtype=torch.float32, device="cuda")
@@ -719,15 +722,15 @@ def bench_net(torch, args):
             cpu = {"value": round(flops1 / (ms * 1e-3) / 1e12, 5), "unit": "TFLOP/s", "cores": 8, "kind": "reference",
                    "sample": f"40 inferences of the same model at batch 1 through the reference's host operator classes "
                              f"and x86 kernels, median {ms:.2f} ms", "ms_per_inference": round(ms, 3)}
-    line = {"metric": f"{args.workload.split('_net_')[0]}_net_fp32_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TFLOP/s",
+    line = {"metric": f"{args.workload.split('_net_')[0]}_net_{'w8a32_tops' if int8 else 'fp32_tflops'}", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TOP/s" if int8 else "TFLOP/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": f"{model} .one model fp32, batch {n}, 224x224, {len(ops)} operators through the "
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8" if int8 else "f32", "data": "synthetic",
+            "config": {"workload": f"{model} .one model {'W8A32 (int8 weights and activations, int32 accumulate; ' + str(net.int8_links()) + ' operands between convolutions travel as int8)' if int8 else 'fp32'}, batch {n}, 224x224, {len(ops)} operators through the "
                                    f"device-resident runtime, input and logits in HBM", "operators": len(ops),
                        "ops_per_step": flops, "model_bytes": len(data)},
             "roofline": {"kernel": "whole inference: every operator of the graph on the default stream", "bound": "mfma",
-                         "achieved": round(flops / (dev * 1e-3) / 1e12, 3), "peak": PEAK["f32"], "unit": "TFLOP/s",
-                         "frac": round(flops / (dev * 1e-3) / 1e12 / PEAK["f32"], 4), "traffic": None,
+                         "achieved": round(flops / (dev * 1e-3) / 1e12, 3), "peak": PEAK["i8" if int8 else "f32"], "unit": "TOP/s" if int8 else "TFLOP/s",
+                         "frac": round(flops / (dev * 1e-3) / 1e12 / PEAK["i8" if int8 else "f32"], 4), "traffic": None,
                          "launches": len(ops), "device_ms_per_inference": round(dev, 4)},
             "cpu_baseline": cpu, "images_per_s": round(n / (ms_per_step * 1e-3), 1)}
     print(json.dumps(line))
@@ -896,7 +899,7 @@ def main():
                           "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
         return
 
-    if args.workload.startswith(("resnet50_net_b", "mobilenetv2_net_b", "vit_tiny_net_b")):
+    if args.workload.startswith(("resnet50_net_b", "resnet50_int8_net_b", "mobilenetv2_net_b", "vit_tiny_net_b")):
         return bench_net(torch, args)
 
     res = run_workload(torch, hip, args.workload, args.steps, args.warmup, layers_table=args.layers, graph=not args.no_graph)

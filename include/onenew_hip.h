@@ -202,6 +202,17 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
                            const int32_t *bias32, const float *weight_aux, const float *silu_lut,
                            int8_t *yq, void *stream);
 
+/* One link of an int8 chain inside a model: the activations come as fp32 NCHW (x, quantised with d->input_scale into the
+ * workspace as in onhip_conv2d_w8a32) or as int8 NHWC with channels padded to 16 (xq), exactly one of the two; the
+ * result leaves as fp32 NCHW (d->out_s8 == 0) or as int8 NHWC quantised with d->output_scale (d->out_s8 == 1: what a
+ * consumer whose input_scale is that value would make of the fp32 result, conv.c:961-973).  Weights packed by
+ * onhip_conv2d_w8a32_pack_weights.  Depthwise is refused.  No counterpart in the reference, whose W8A32 operators
+ * (device/x86/Conv/conv.c:939-1067) always take and return fp32; the device-resident runtime calls it for edges between
+ * two int8 convolutions. */
+int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,
+                         const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
 /* ---- bf16 / fp16 with 16-bit storage --------------------------------------------------------------------------
  * The reference has the two types as enumerators only (ELEM_TYPE_E TYPE_FP16 / the cuda tile fields,
  * common/nn_common.h:102,107) and no kernel that stores them, so the layouts are this library's: activations NHWC
@@ -424,6 +435,11 @@ int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFE
  * the last convolution.  onhip_conv_block_takes reads the params only and returns 1 when onhip_ir_block_supported says 2
  * for these shapes, else 0.  No counterpart in the reference, whose host runs the operators one by one. */
 int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_link` of libConv_hip.so: a dense int8 (W8A32) Conv whose input and/or result travel as int8 NHWC (channels padded
+ * to 16) instead of fp32 NCHW, see onhip_conv2d_w8_link.  Slots as for `eval`; inputs[4] = host pointer to
+ * {int32 in_s8, int32 out_s8, float out_scale}; inputs[5] = null, or host pointer to an int32 1 / 2 for the Add (and
+ * Relu) of a residual block with its other operand in inputs[3] (fp32 results only).  No counterpart in the reference. */
+int onhip_conv_link_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_conv_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Add (add.c:18), Relu (relu.c:8), MaxPool (maxpool.c:7), GlobalAveragePool (global_avgpool.c:7) */

@@ -1033,6 +1033,15 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
     return conv2d_w8a32_impl(&dd, nullptr, xq, w8_packed, 1, bias32, weight_aux, silu_lut, yq, nullptr, nullptr, 0, 1, stream);
 }
 
+int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,
+                         const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    if (!d) return set_error(ONHIP_ERR_ARG, "conv w8 link: null descriptor");
+    if ((x != nullptr) == (xq != nullptr)) return set_error(ONHIP_ERR_ARG, "conv w8 link: exactly one of x and xq");
+    return conv2d_w8a32_impl(d, x, xq, w8_packed, 1, bias32, weight_aux, silu_lut, y, nullptr, workspace, workspace_bytes,
+                             d->out_s8 ? 1 : 0, stream);
+}
+
 static int matmul_impl(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
                        const float *gelu_lut, const float *addend, float *out, void *stream) {
     if (!d || d->batch < 1 || d->m < 1 || d->k < 1 || d->n < 1) return set_error(ONHIP_ERR_ARG, "matmul: bad shape");

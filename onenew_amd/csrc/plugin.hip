@@ -238,9 +238,17 @@ static long long numel(const OPERAND_S *o) {
     return n;
 }
 
+// What travels along the edges of an int8 convolution inside a chain of them (inputs[4] of `eval_link`): in_s8 != 0, the
+// input tensor is int8 NHWC with channels padded to 16, quantised with this operator's input_scale by its producer;
+// out_s8 != 0, the result is stored that way for consumers whose input_scale is out_scale.
+struct ConvLink {
+    int32_t in_s8, out_s8;
+    float out_scale;
+};
+
 // fuse 0: the Conv of the reference.  1: inputs[3] holds a tensor of the output's shape that is added to the result
-// (the Add of a residual block); 2: and a Relu after that.
-static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, int fuse) {
+// (the Add of a residual block); 2: and a Relu after that.  link: null, or the int8 forms of the edges.
+static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, int fuse, const ConvLink *link = nullptr) {
     const CONV_CONFIG_S *cfg = reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr);
     const OPERAND_S *in_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
     const OPERAND_S *w_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
@@ -281,8 +289,14 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
     if (w_t->shapes[1] != kc)
         return set_error(ONHIP_ERR_ARG, "Conv eval: weight has %d input channels, expected %d", w_t->shapes[1], kc);
 
-    const size_t in_bytes = (size_t) d.n * d.cin * d.h * d.w * 4;
-    const size_t out_bytes = (size_t) d.n * d.cout * OH * OW * 4;
+    const bool in_s8 = link && link->in_s8, out_s8 = link && link->out_s8;
+    if (link) {
+        if (!int8 || d.group != 1) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges are for dense int8 convolutions");
+        if (out_s8 && fuse) return set_error(ONHIP_ERR_ARG, "Conv eval: an int8 result cannot take the Add of a residual block");
+        if (out_s8 && !(link->out_scale > 0.0f)) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 result without a scale");
+    }
+    const size_t in_bytes = in_s8 ? (size_t) d.n * d.h * d.w * ((d.cin + 15) / 16 * 16) : (size_t) d.n * d.cin * d.h * d.w * 4;
+    const size_t out_bytes = out_s8 ? (size_t) d.n * OH * OW * ((d.cout + 15) / 16 * 16) : (size_t) d.n * d.cout * OH * OW * 4;
     const size_t w_elems = (size_t) d.cout * kc * d.kh * d.kw;
     const void *x, *w, *b = nullptr, *lut = nullptr, *aux = nullptr;
     rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
@@ -332,7 +346,13 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         const float *wp = nullptr;
         rc = packed_weights(&d, (const float *) w, &wp, true);
         if (rc) return rc;
-        if (wp)
+        if (link) {
+            if (!wp) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges need the packed weight form");
+            d.out_s8 = out_s8 ? 1 : 0;
+            d.output_scale = link->out_scale;
+            rc = onhip_conv2d_w8_link(&d, in_s8 ? nullptr : (const float *) x, in_s8 ? (const int8_t *) x : nullptr, (const int8_t *) wp,
+                                      (const int32_t *) b, (const float *) aux, (const float *) lut, y, ws, ws_bytes, g_stream);
+        } else if (wp)
             rc = onhip_conv2d_w8a32_packed(&d, (const float *) x, (const int8_t *) wp, (const int32_t *) b,
                                            (const float *) aux, (const float *) lut, y, nullptr, ws, ws_bytes, g_stream);
         else
@@ -466,6 +486,15 @@ static int conv_add_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BU
 }
 static int conv_add_relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return conv_eval_fused(params, inputs, outputs, 2);
+}
+// inputs[4]: a ConvLink in host memory; inputs[5]: null, or one int32 in host memory, 1 / 2 = the Add (and Relu) of a
+// residual block with its other operand in inputs[3]
+static int conv_link_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    const ConvLink *link = reinterpret_cast<const ConvLink *>(inputs[4].addr);
+    if (!link) return set_error(ONHIP_ERR_ARG, "Conv eval: no edge description in inputs[4]");
+    const int32_t *fuse = reinterpret_cast<const int32_t *>(inputs[5].addr);
+    if (fuse && (*fuse < 0 || *fuse > 2)) return set_error(ONHIP_ERR_ARG, "Conv eval: fold code %d", *fuse);
+    return conv_eval_fused(params, inputs, outputs, fuse ? *fuse : 0, link);
 }
 
 // mode 0: MatMul.  mode 1: MatMul -> Add of a bias over the last axis (params[3] / inputs[2], n elements; the result's
@@ -922,6 +951,9 @@ int onhip_conv_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INF
 
 int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Conv + Add + Relu", conv_add_relu_eval_locked, params, inputs, outputs);
+}
+int onhip_conv_link_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv (int8 edges)", conv_link_eval_locked, params, inputs, outputs);
 }
 int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Conv -> depthwise Conv -> Conv", conv_block_eval_locked, params, inputs, outputs);

@@ -33,3 +33,11 @@ extern "C" __attribute__((visibility("default"))) int eval_add_relu(BUFFER_INFO_
                                                                     BUFFER_INFO_S *outputs) {
     return onhip_conv_add_relu_eval(params, inputs, outputs);
 }
+
+// Not in the reference: a dense int8 convolution inside a chain of them, taking and/or leaving its activations as int8
+// NHWC.  Slots as for `eval`; inputs[4] = {int32 in_s8, int32 out_s8, float out_scale} in host memory; inputs[5] = null
+// or an int32 fold code (1 Add, 2 Add + Relu, the other operand in inputs[3]).
+extern "C" __attribute__((visibility("default"))) int eval_link(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                BUFFER_INFO_S *outputs) {
+    return onhip_conv_link_eval(params, inputs, outputs);
+}

@@ -119,6 +119,7 @@ struct Tensor {
     bool produced = false;   // an io input, an initialiser or the output of an operator already ordered
     std::string alias;       // an operand folded away with its producer reads as this one (fuse_residual_blocks)
     bool never_written = false;   // an operand inside a fused attention block: it has no buffer and no value
+    bool as_s8 = false;           // written and read as int8 NHWC, channels padded to 16 (link_int8_convs)
 };
 
 struct Node {
@@ -130,6 +131,10 @@ struct Node {
     std::string addend, fused_out;
     int32_t token_major[4] = {0, 0, 0, 0};   // fused attention: q, k, v, result stored [batch, tokens, heads, head_dim]
     int block_dw = -1, block_pw = -1;        // fused inverted-residual block (fuse 7): its depthwise and last convolutions
+    // an int8 convolution whose input and/or result travel as int8 NHWC (link_int8_convs): what `eval_link` reads from
+    // inputs[4] ({in_s8, out_s8, out_scale}) and inputs[5] (the fold code, when an Add is folded in)
+    struct { int32_t in_s8, out_s8; float out_scale; } link = {0, 0, 0.0f};
+    int32_t link_fuse = 0;
     BUFFER_INFO_S params[BUF_MAXNUM], inputs[BUF_MAXNUM], outputs[BUF_MAXNUM];
     const BASE_CONFIG_S *base() const { return reinterpret_cast<const BASE_CONFIG_S *>(cfg.data()); }
 };
@@ -164,9 +169,9 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr;
+    onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr, conv_link = nullptr;
     onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr, matmul_bias_add = nullptr;   // optional entry points of the MatMul plugin
-    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0;
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0, int8_links = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -426,6 +431,10 @@ int allocate(onrt_net &net) {
         Tensor &t = kv.second;
         if (t.is_init || t.desc.not_need_buf || !t.alias.empty() || t.never_written) continue;
         t.bytes = (size_t) numel(t.desc) * 4;
+        if (t.as_s8) {   // [n, h, w, channels padded to 16] bytes, where that is more
+            const size_t s8 = (size_t) t.desc.shapes[0] * t.desc.shapes[2] * t.desc.shapes[3] * (((size_t) t.desc.shapes[1] + 15) / 16 * 16);
+            if (s8 > t.bytes) t.bytes = s8;
+        }
         act_total += (t.bytes + 255) & ~(size_t) 255;
     }
     if (act_total) {
@@ -521,6 +530,7 @@ int bind_plugins(onrt_net &net) {
             net.conv_add_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add_relu"));
             net.conv_block = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block"));
             net.conv_block_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block_takes"));
+            net.conv_link = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_link"));
         }
         if (type == "MatMul") {
             net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
@@ -775,6 +785,61 @@ int fuse_ir_blocks(onrt_net &net) {
     return ONRT_OK;
 }
 
+// ---- int8 edges -------------------------------------------------------------------------------------------
+// The reference's W8A32 convolution takes fp32, quantises it with its input_scale (device/x86/Conv/conv.c:961-973) and
+// returns fp32 (:1049-1056).  Where the result of a dense int8 Conv is read by dense int8 Convs only, all with the same
+// input_scale, that quantisation moves into the producer's store: the operand travels as int8 NHWC (a quarter of the
+// bytes, and no staging pass in the consumers), holding exactly the bytes each consumer would have made of the fp32
+// tensor, so the model's results do not change.  The Conv plugin's `eval_link` runs both ends.  Not for depthwise
+// convolutions (no NHWC int8 form), results that an Add is folded into, model outputs, or operands any other operator
+// reads.  Runs after the other folds; ONENEW_RT_FUSE=0 keeps every operand fp32 (layer-by-layer comparisons), and so
+// does ONENEW_RT_LINK=0 with the other folds in place.
+int link_int8_convs(onrt_net &net) {
+    if (!fusing_enabled() || !net.conv_link) return ONRT_OK;
+    if (const char *env = getenv("ONENEW_RT_LINK"))   // "0": the other folds without this one (measurements)
+        if (!strcmp(env, "0")) return ONRT_OK;
+    auto result_of = [](const Node &n) { return n.fused_out.empty() ? n.out[0] : n.fused_out; };
+    auto dense_int8 = [&](const Node &n) -> const CONV_CONFIG_S * {
+        if (strcmp(n.kind->type, "Conv") || n.out.size() != 1 || n.in.size() < 2 || n.in.size() > 3 || n.fuse > 2) return nullptr;
+        for (size_t k = 1; k < n.in.size(); ++k)
+            if (n.in[k].empty() || !net.tensors[n.in[k]].is_init) return nullptr;
+        if (net.tensors[n.in[0]].is_init) return nullptr;
+        const CONV_CONFIG_S *cfg = reinterpret_cast<const CONV_CONFIG_S *>(n.cfg.data());
+        if (cfg->ifmap_quant2 != TYPE_INT8 || (cfg->has_bias && cfg->group != 1)) return nullptr;   // conv.c:18-29: depthwise
+        return cfg;
+    };
+    for (int idx : net.order) {
+        Node &p = net.nodes[idx];
+        if (!dense_int8(p) || p.fuse != 0) continue;
+        const std::string name = result_of(p);
+        if (is_net_output(net, name) || net.tensors[name].desc.not_need_buf) continue;
+        const std::vector<int> readers = readers_of(net, name);
+        bool ok = !readers.empty();
+        float scale = 0.0f;
+        for (int ri : readers) {
+            const Node &c = net.nodes[ri];
+            const CONV_CONFIG_S *cc = dense_int8(c);
+            if (!cc || c.in[0] != name || !(cc->input_scale > 0.0f) || (scale != 0.0f && cc->input_scale != scale)) { ok = false; break; }
+            scale = cc->input_scale;
+        }
+        for (int oi : net.order)   // nor may it be the other operand of a folded Add
+            if (net.nodes[oi].addend == name) ok = false;
+        if (!ok) continue;
+        p.link.out_s8 = 1;
+        p.link.out_scale = scale;
+        p.eval = net.conv_link;
+        for (int ri : readers) {
+            Node &c = net.nodes[ri];
+            c.link.in_s8 = 1;
+            c.link_fuse = c.fuse;
+            c.eval = net.conv_link;
+        }
+        net.tensors[name].as_s8 = true;
+        ++net.int8_links;
+    }
+    return ONRT_OK;
+}
+
 // ---- attention ------------------------------------------------------------------------------------------
 // MatMul(q, Transpose(k)) -> Softmax (last axis) -> MatMul(., v), with nothing else reading the operands in between,
 // becomes one call of the MatMul plugin's `eval_attention` on q, k (as it is before the Transpose) and v: the scores
@@ -975,6 +1040,10 @@ int fill_slots(onrt_net &net) {
             nd.inputs[8].addr = c.in.size() > 2 ? (int64_t) net.tensors[c.in[2]].dev : 0;
         }
         if (nd.fuse == 1 || nd.fuse == 2 || nd.fuse == 6) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
+        if (nd.link.in_s8 || nd.link.out_s8) {
+            nd.inputs[4].addr = (int64_t) &nd.link;
+            nd.inputs[5].addr = nd.link_fuse ? (int64_t) &nd.link_fuse : 0;
+        }
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
             Tensor &t = net.tensors[nd.fused_out.empty() ? nd.out[k] : nd.fused_out];
@@ -1005,6 +1074,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = fuse_ir_blocks(net);
     if (!rc) rc = fuse_attention(net);
     if (!rc) rc = fuse_linear(net);
+    if (!rc) rc = link_int8_convs(net);
     if (!rc) rc = allocate(net);
     if (!rc) rc = build_tables(net);
     if (!rc) rc = fill_slots(net);
@@ -1227,6 +1297,12 @@ ONRT_API int onrt_net_fused_attentions(const onrt_net_t *net, int32_t *n) {
 ONRT_API int onrt_net_fused_linears(const onrt_net_t *net, int32_t *n) {
     if (!net || !n) return fail(ONRT_ERR_ARG, "fused linear layers: null argument");
     *n = (int32_t) net->fused_linears;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_quantised_links(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "null argument");
+    *n = (int32_t) net->int8_links;
     return ONRT_OK;
 }
 

@@ -116,6 +116,44 @@ def quantised_block():
     return m.tobytes(), [_r("xq", (1, 16, 18, 18))]
 
 
+def quantised_chain(n=1, hw=18, different_scales=False, extra_reader=False):
+    """dense W8A32 convolutions feeding each other: q1 -> (q2, q2b with one input_scale) , q2 -> q3, and a residual
+    block qa -> qb + skip -> Relu behind q3; the operands between them can travel as int8.  different_scales: q2b
+    quantises its input differently from q2; extra_reader: a Relu also reads q1's result"""
+    from oracle import oracle
+    m = onefile.OneModel()
+    m.input("x", (n, 16, hw, hw))
+
+    def q(tag, shape, scale):
+        w = _r(tag + "w", shape, scale)
+        b = _r(tag + "b", (shape[0],), 0.2)
+        return oracle.quant_weight_bias(w, b)
+
+    w8, b32, aux = q("c1", (32, 16, 3, 3), 0.1)
+    m.conv("q1", "x", w8, b32, "q1_out", pad=1, act=abi.SILU, quant=(aux, 0.031))
+    w8, b32, aux = q("c2", (64, 32, 1, 1), 0.2)
+    m.conv("q2", "q1_out", w8, b32, "q2_out", act=abi.RELU, quant=(aux, 0.024))
+    w8, b32, aux = q("c2b", (24, 32, 3, 3), 0.1)
+    m.conv("q2b", "q1_out", w8, b32, "q2b_out", stride=2, pad=1, act=abi.NOT_ACT, quant=(aux, 0.029 if different_scales else 0.024))
+    m.relu("relu_b", "q2b_out", "out_b")
+    oh = (hw + 2 - 3) // 2 + 1
+    m.output("out_b", (n, 24, oh, oh))
+    if extra_reader:
+        m.relu("relu_x", "q1_out", "out_x")
+        m.output("out_x", (n, 32, hw, hw))
+    w8, b32, aux = q("c3", (32, 64, 3, 3), 0.08)
+    m.conv("q3", "q2_out", w8, b32, "q3_out", pad=1, act=abi.NOT_ACT, quant=(aux, 0.04))
+    # a residual block of int8 convolutions on q3's fp32 result
+    w8, b32, aux = q("ca", (32, 32, 1, 1), 0.2)
+    m.conv("qa", "q3_out", w8, b32, "qa_out", act=abi.RELU, quant=(aux, 0.06))
+    w8, b32, aux = q("cb", (32, 32, 3, 3), 0.1)
+    m.conv("qb", "qa_out", w8, b32, "qb_out", pad=1, act=abi.NOT_ACT, quant=(aux, 0.035))
+    m.add("sum", "qb_out", "q3_out", "sum_out")
+    m.relu("relu_s", "sum_out", "out")
+    m.output("out", (n, 32, hw, hw))
+    return m.tobytes(), [_r("xqc", (n, 16, hw, hw))]
+
+
 def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output=False, split_heads=()):
     """q, k, v as three inputs [batch, heads, tokens, head_dim]: Transpose of k, MatMul, Softmax, MatMul, the pattern the
     runtime runs as one attention call (unless the scores are also a net output).  split_heads: which of "q", "k", "v"
@@ -153,7 +191,7 @@ def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output
     return m.tobytes(), [_r(n + str(tokens), shape, 0.5) for n in ("q", "k", "v")]
 
 
-MODELS = {"quantised_block": quantised_block, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
+MODELS = {"quantised_block": quantised_block, "quantised_chain": quantised_chain, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
 
 
 def unfused_activations(optimised=False):

@@ -48,7 +48,7 @@ def test_model_outputs_match_oracle(name, torch_dev, monkeypatch):
     for (oname, _), got in zip(net.outputs, outs):
         assert got.shape == ref[oname].shape
         assert _close(got, ref[oname], 5e-4), oname                          # up to five MFMA operators deep, 1e-4 each
-        if name == "quantised_block":
+        if name in ("quantised_block", "quantised_chain"):
             assert np.array_equal(got, ref[oname])                           # integer accumulation: the chain is exact
     # every intermediate operand sits in device memory and holds what the oracle computed at that point
     for op_type, cfg in m["nodes"]:
@@ -691,3 +691,41 @@ def test_unoptimised_file_runs_like_the_optimised_one(torch_dev, monkeypatch):
     monkeypatch.delenv("ONENEW_RT_FUSE")
     assert unfused.folded_activations() == 4 and [t for t, _ in unfused.ops()] == ["Conv"] * 5 + ["Relu"]
     assert np.array_equal(unfused.run(*ins)[0], want[0])
+
+
+@pytest.mark.gpu
+def test_int8_convolutions_exchange_int8_operands(torch_dev, monkeypatch):
+    """dense int8 convolutions that feed each other hand their operand over as int8 NHWC, quantised by the producer with
+    the consumers' input_scale: three operands in the chain model (one with two readers, one into a convolution with a
+    folded Add + Relu), the results equal to the oracle's and to the runtime's with every operand fp32, bit for bit;
+    at batch 3 too.  Consumers with different scales, or any other reader, keep the operand fp32"""
+    for n in (1, 3):
+        data, ins = one_models.quantised_chain(n=n)
+        net = rt.Net(data)
+        assert net.int8_links() == 3 and net.fused_blocks() == 1
+        outs = net.run(*ins)
+        outs2 = net.run(*ins)                       # buffers reused
+        ref = one_model.run(data, ins, keep_all=True)
+        for (oname, _), got, got2 in zip(net.outputs, outs, outs2):
+            assert np.array_equal(got, ref[oname]), oname
+            assert np.array_equal(got2, got)
+        net.close()
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    data, ins = one_models.quantised_chain()
+    plain = rt.Net(data)
+    assert plain.int8_links() == 0
+    plain_outs = plain.run(*ins)
+    plain.close()
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    net = rt.Net(data)
+    for a, b in zip(net.run(*ins), plain_outs):
+        assert np.array_equal(a, b)
+    net.close()
+    for kw, links in (({"different_scales": True}, 2), ({"extra_reader": True}, 2)):
+        data, ins = one_models.quantised_chain(**kw)
+        net = rt.Net(data)
+        assert net.int8_links() == links, kw
+        ref = one_model.run(data, ins, keep_all=True)
+        for (oname, _), got in zip(net.outputs, net.run(*ins)):
+            assert np.array_equal(got, ref[oname]), (kw, oname)
+        net.close()
