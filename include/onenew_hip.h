@@ -322,8 +322,10 @@ int onhip_gemm_f32(int32_t m, int32_t k, int32_t n, const float *a, const float 
 /* ---- the operators around the convolutions of a residual network (device pointers) ------------ */
 
 /* Broadcasting add: out = large + small, out has the shape of `large`; `small` is aligned to the
- * same rank (host pads its shape with leading 1s) and each of its extents is 1 or equal.  relu != 0
- * applies max(x, 0) to the sum: the Add -> Relu pair that closes a residual block, in one pass.
+ * same rank (host pads its shape with leading 1s) and each of its extents is 1 or equal.  relu == 1
+ * applies "x > 0 ? x : 0" to the sum: the Add -> Relu pair that closes a residual block, in one pass; relu == 2 applies
+ * the Relu operator's own two rules by element index (device/x86/Relu/relu.c:27-52: "0 > x ? 0 : x" below n - n % 32,
+ * "x > 0 ? x : 0" from there on; they differ on NaN and negative zero), what a separate Relu would store.
  * Replaces device/x86/Add/add.c eval (:18-80) and fun_0 / fun_1 / fun_2_dim3..6 (:87-365). */
 typedef struct {
     int32_t ndim;            /* 1..6 */

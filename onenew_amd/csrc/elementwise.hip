@@ -23,10 +23,17 @@ struct AddParams {
     Div31 div[6];             // by the extents of the large operand, innermost first
     int extent[6];
     int small_stride[6];      // innermost first; 0 where the small operand is broadcast
-    int relu;
+    int relu;                 // 1: "r > 0 ? r : 0" on every element; 2: relu.c's two rules by element index (relu_body below
+                              // n_body = n - n % 32, relu_tail from there on)
+    long long n_body;
     Div31 div_small;          // MODE 3: by the number of float4 groups of the small operand
     int small4;
 };
+
+__device__ __forceinline__ float add_then_relu(float r, int relu, long long i, long long n_body) {
+    if (relu == 2) return i < n_body ? relu_body(r) : relu_tail(r);
+    return (relu && !(r > 0)) ? 0.0f : r;
+}
 
 template <int MODE>
 __global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__restrict__ large,
@@ -38,13 +45,12 @@ __global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__re
             const float4 a = reinterpret_cast<const float4 *>(large)[i4], b = reinterpret_cast<const float4 *>(small)[i4];
             // operand order of add.c:96: small + large
             float4 r = make_float4(__fadd_rn(b.x, a.x), __fadd_rn(b.y, a.y), __fadd_rn(b.z, a.z), __fadd_rn(b.w, a.w));
-            if (p.relu) { r.x = r.x > 0 ? r.x : 0; r.y = r.y > 0 ? r.y : 0; r.z = r.z > 0 ? r.z : 0; r.w = r.w > 0 ? r.w : 0; }
+            if (p.relu == 2 && i4 * 4 < p.n_body) {   // n_body is a multiple of 32: the four share a rule
+                r.x = relu_body(r.x); r.y = relu_body(r.y); r.z = relu_body(r.z); r.w = relu_body(r.w);
+            } else if (p.relu) { r.x = r.x > 0 ? r.x : 0; r.y = r.y > 0 ? r.y : 0; r.z = r.z > 0 ? r.z : 0; r.w = r.w > 0 ? r.w : 0; }
             reinterpret_cast<float4 *>(out)[i4] = r;
         } else if (i4 * 4 < p.n) {
-            for (long long i = i4 * 4; i < p.n; ++i) {
-                const float r = __fadd_rn(small[i], large[i]);
-                out[i] = (p.relu && !(r > 0)) ? 0.0f : r;
-            }
+            for (long long i = i4 * 4; i < p.n; ++i) out[i] = add_then_relu(__fadd_rn(small[i], large[i]), p.relu, i, p.n_body);
         }
     } else if constexpr (MODE == 3) {
         const long long i4 = (long long) blockIdx.x * 256 + threadIdx.x;
@@ -53,7 +59,9 @@ __global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__re
         const unsigned j4 = (unsigned) i4 - q * (unsigned) p.small4;
         const float4 a = reinterpret_cast<const float4 *>(large)[i4], b = reinterpret_cast<const float4 *>(small)[j4];
         float4 r = make_float4(__fadd_rn(a.x, b.x), __fadd_rn(a.y, b.y), __fadd_rn(a.z, b.z), __fadd_rn(a.w, b.w));
-        if (p.relu) { r.x = r.x > 0 ? r.x : 0; r.y = r.y > 0 ? r.y : 0; r.z = r.z > 0 ? r.z : 0; r.w = r.w > 0 ? r.w : 0; }
+        if (p.relu == 2 && i4 * 4 < p.n_body) {
+            r.x = relu_body(r.x); r.y = relu_body(r.y); r.z = relu_body(r.z); r.w = relu_body(r.w);
+        } else if (p.relu) { r.x = r.x > 0 ? r.x : 0; r.y = r.y > 0 ? r.y : 0; r.z = r.z > 0 ? r.z : 0; r.w = r.w > 0 ? r.w : 0; }
         reinterpret_cast<float4 *>(out)[i4] = r;
     } else {
         const long long i = (long long) blockIdx.x * 256 + threadIdx.x;
@@ -70,8 +78,7 @@ __global__ __launch_bounds__(256) void add_kernel(AddParams p, const float *__re
                 }
             }
         }
-        const float r = __fadd_rn(large[i], small[j]);
-        out[i] = (p.relu && !(r > 0)) ? 0.0f : r;
+        out[i] = add_then_relu(__fadd_rn(large[i], small[j]), p.relu, i, p.n_body);
     }
 }
 
@@ -214,7 +221,8 @@ int onhip_add_f32(const onhip_add_desc_t *d, const float *large, const float *sm
     if (n >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "add: tensors of 2^31 elements or more are not supported");
     p.n = n;
     p.ndim = d->ndim;
-    p.relu = d->relu ? 1 : 0;
+    p.relu = d->relu == 2 ? 2 : d->relu ? 1 : 0;
+    p.n_body = n - n % 32;
     int stride = 1;
     for (int k = 0; k < d->ndim; ++k) {        // innermost first
         const int dim = d->ndim - 1 - k;

@@ -358,14 +358,14 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         else
             rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
                                     (const float *) lut, y, nullptr, ws, ws_bytes, g_stream);
-        if (!rc && fuse) {   // the int8 store does not fold the addend in: the two operators as passes over y
+        if (!rc && fuse) {   // the int8 store does not fold the addend in: the two operators as one pass over y
             onhip_add_desc_t ad;
             memset(&ad, 0, sizeof(ad));
             ad.ndim = 4;
             const int32_t shape[4] = {d.n, d.cout, OH, OW};
             for (int i = 0; i < 4; ++i) ad.large_shape[i] = ad.small_shape[i] = shape[i];
+            ad.relu = fuse == 2 ? 2 : 0;   // the Relu operator's rules by element index, in the same pass
             rc = onhip_add_f32(&ad, (const float *) y, (const float *) addend, (float *) y, g_stream);
-            if (!rc && fuse == 2) rc = onhip_relu_f32((const float *) y, (float *) y, (long long) (out_bytes / 4), g_stream);
         }
     } else if (fuse) {
         const float *wp = nullptr;

@@ -1317,3 +1317,28 @@ def test_conv_int8_chain_3x3_with_few_channels(shape, act, torch_dev, oracle, mo
         got = out.cpu().numpy()
         assert np.array_equal(got[..., :d.cout], ref), f"kernels off: {off}"
         assert not got[..., d.cout:].any()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 8, 7, 9), (1, 3, 5, 5), (4, 64), (1, 32, 14, 14)])
+def test_add_then_relu_by_the_relu_operators_own_rules(shape, torch_dev):
+    """onhip_add_f32 with relu = 2: the Relu operator's two rules by element index (relu.c:27-52) in the same pass, equal
+    bit for bit to onhip_add_f32 followed by onhip_relu_f32, NaNs and negative zeros included, before and after the
+    boundary at n - n % 32"""
+    torch = torch_dev
+    rng = np.random.default_rng(11)
+    a = rng.normal(size=shape).astype(np.float32)
+    b = rng.normal(size=shape).astype(np.float32)
+    fa, fb = a.reshape(-1), b.reshape(-1)
+    n = fa.size
+    for i in (0, 5, n - n % 32 - 1, n - n % 32, n - 1):     # sums that are NaN and -0 on both sides of the boundary
+        if 0 <= i < n:
+            fa[i], fb[i] = np.float32("nan"), np.float32(1.0)
+    for i in (1, 6, n - n % 32 - 2, n - n % 32 + 1, n - 2):
+        if 0 <= i < n and not np.isnan(fa[i]):
+            fa[i], fb[i] = np.float32(-0.0), np.float32(-0.0)
+    ta, tb = dev(torch, a), dev(torch, b)
+    two = hip.relu_f32(hip.add_f32(ta, tb))
+    one = hip.add_f32(ta, tb, relu=2)
+    torch.cuda.synchronize()
+    assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32))
