@@ -206,12 +206,14 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
  * workspace as in onhip_conv2d_w8a32) or as int8 NHWC with channels padded to 16 (xq), exactly one of the two; the
  * result leaves as fp32 NCHW (d->out_s8 == 0) or as int8 NHWC quantised with d->output_scale (d->out_s8 == 1: what a
  * consumer whose input_scale is that value would make of the fp32 result, conv.c:961-973).  Weights packed by
- * onhip_conv2d_w8a32_pack_weights.  Depthwise is refused.  No counterpart in the reference, whose W8A32 operators
- * (device/x86/Conv/conv.c:939-1067) always take and return fp32; the device-resident runtime calls it for edges between
- * two int8 convolutions. */
+ * onhip_conv2d_w8a32_pack_weights.  Depthwise is refused.  addend, when not null (fp32 results only): a tensor of the
+ * result's shape added to it in the store (device/x86/Add/add.c:96), followed, with relu_after != 0, by relu as
+ * device/x86/Relu/relu.c:27-52 (both of its rules, by element index): the three operators' bytes in one pass.  No
+ * counterpart in the reference, whose W8A32 operators (device/x86/Conv/conv.c:939-1067) always take and return fp32; the
+ * device-resident runtime calls it for edges between two int8 convolutions and for the one that closes a residual block. */
 int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,
-                         const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y, void *workspace,
-                         size_t workspace_bytes, void *stream);
+                         const int32_t *bias32, const float *weight_aux, const float *silu_lut, const float *addend,
+                         int32_t relu_after, void *y, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- bf16 / fp16 with 16-bit storage --------------------------------------------------------------------------
  * The reference has the two types as enumerators only (ELEM_TYPE_E TYPE_FP16 / the cuda tile fields,

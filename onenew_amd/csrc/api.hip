@@ -309,6 +309,8 @@ static bool candidate_ok(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
     if (!tile_exists(c)) return false;   // e.g. a line of the cache file written by another build or by hand
     const int k_tiles = (p.k_units + k_tile_units(cfg.dtype) - 1) / k_tile_units(cfg.dtype);
     const bool h16 = cfg.dtype != DT_I8 && (cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP);   // 16-bit storage: that kernel only
+    // int8 with a residual operand: the register-staged kernel, whole K in one workgroup
+    if (p.res && cfg.dtype == DT_I8 && (c.dma || c.split > 1 || c.tail > 1 || c.fin || c.rowb)) return false;
     if (c.dma) {
         static const bool off = getenv("ONHIP_NO_DMA") != nullptr;   // tuning hook: the register-staged kernel only
         return (!off || h16) && c.split == 1 && c.tail <= 1 && !c.rowb && !c.fin && dma_ok(cfg, p);
@@ -892,13 +894,16 @@ int onhip::forget_quantised_tables(const void *base, size_t bytes) {
 // nhwc_out != 0: the int8 result is written NHWC with its channels padded to 16, ready to be the next xq
 static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8, int packed_w,
                              const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y,
-                             int32_t *acc32, void *workspace, size_t workspace_bytes, int nhwc_out, void *stream) {
+                             int32_t *acc32, void *workspace, size_t workspace_bytes, int nhwc_out, void *stream,
+                             const float *addend = nullptr, int relu_after = 0) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
     if ((!x && !xq) || !w8 || !y || !weight_aux || (d->has_bias && !bias32))
         return set_error(ONHIP_ERR_ARG, "conv w8a32: null tensor pointer");
     if (nhwc_out && !d->out_s8) return set_error(ONHIP_ERR_ARG, "conv w8a8: the NHWC output form is int8 (out_s8 = 1)");
+    if (addend && (d->out_s8 || acc32 || d->group != 1))
+        return set_error(ONHIP_ERR_ARG, "conv w8a32: an addend goes with dense convolutions and fp32 results");
     if ((xq || nhwc_out) && d->group != 1) return set_error(ONHIP_ERR_ARG, "conv w8a8: depthwise is not available in the NHWC int8 form");
     // the reference pads all four sides by pads[0] (conv.c:979-999) while shapes come from the four
     // pads: only uniform padding is self-consistent
@@ -995,6 +1000,12 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
         rc = quantised_table(ep.lut, p.out_inv_scale, st, &p.ep.qlut);
         if (rc) return rc;
     }
+    if (addend) {   // the Add (and Relu) after the convolution, in its store
+        const long long n_out = (long long) d->n * d->cout * OH * OW;
+        p.res = addend;
+        p.res_relu = relu_after ? 1 : 0;
+        p.res_body = (unsigned) (n_out - n_out % 32);   // relu.c:27-52
+    }
     // 3x3, stride 1, few channels, int8 in and out: the kernel that keeps the band's input in LDS and the weights in registers
     // tuning hooks: ONHIP_NO_PATCH keeps to the implicit-GEMM kernels, and so does a forced tile of theirs; ONHIP_PATCH_ALL
     // sends every shape the LDS-patch kernel can take to it, not only those it is measured to win
@@ -1034,12 +1045,12 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
 }
 
 int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,
-                         const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y, void *workspace,
-                         size_t workspace_bytes, void *stream) {
+                         const int32_t *bias32, const float *weight_aux, const float *silu_lut, const float *addend,
+                         int32_t relu_after, void *y, void *workspace, size_t workspace_bytes, void *stream) {
     if (!d) return set_error(ONHIP_ERR_ARG, "conv w8 link: null descriptor");
     if ((x != nullptr) == (xq != nullptr)) return set_error(ONHIP_ERR_ARG, "conv w8 link: exactly one of x and xq");
     return conv2d_w8a32_impl(d, x, xq, w8_packed, 1, bias32, weight_aux, silu_lut, y, nullptr, workspace, workspace_bytes,
-                             d->out_s8 ? 1 : 0, stream);
+                             d->out_s8 ? 1 : 0, stream, addend, relu_after);
 }
 
 static int matmul_impl(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

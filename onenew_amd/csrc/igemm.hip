@@ -21,7 +21,9 @@ int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t strea
     if (p.a_slice_bytes >= (1LL << 31) || p.b_slice_bytes + 2 * p.b_shift_bytes >= (1LL << 31) ||
         p.c_slice_bytes >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "igemm: an operand slice of 2 GiB or more is not supported");
-    if (p.res && cfg.dtype != DT_F32) return set_error(ONHIP_ERR_ARG, "igemm: the residual store exists for fp32 operands");
+    if (p.res && cfg.dtype != DT_F32 && cfg.dtype != DT_I8)
+        return set_error(ONHIP_ERR_ARG, "igemm: the residual store exists for fp32 and int8 operands");
+    if (p.res && cfg.dtype == DT_I8 && cfg.split > 1) return set_error(ONHIP_ERR_ARG, "igemm i8: no split-K with a residual operand");
     switch (cfg.dtype) {
         case DT_F32: return igemm_launch_f32(cfg, p, stream);
         case DT_BF16: return igemm_launch_bf16(cfg, p, stream);

@@ -359,8 +359,21 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
             const int n = n_wave + b * 32 + li;
             col_voff4[b] = n < p.N ? out_col_offset(p, n, 4) + (unsigned) (4 * lh) * row_bytes4 : OOB;
         }
+        // RES: the residual operand of a folded Add (fp32 results): a row tile's addends are requested together
+        const rsrc_t rres = make_rsrc(RES ? reinterpret_cast<const char *>(p.res) + (size_t) batch * p.c_batch_stride * 4 : nullptr,
+                                      RES ? RSRC_RANGE : 0u);
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
+        for (int a = 0; a < TM; ++a) {
+            float rv[RES ? 16 : 1][RES ? TN : 1];
+            if constexpr (RES) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
+                    const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
+#pragma unroll
+                    for (int b = 0; b < TN; ++b) rv[r][b] = buf_load_f32(rres, row_ok ? col_voff[b] : OOB, (unsigned) m_uni * row_bytes);
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
@@ -377,7 +390,8 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                     float f = __fmul_rn((float) av, p.in_scale);
                     const float fbias = __fadd_rn(f, fb);
                     f = p.bias32 ? fbias : f;
-                    const float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
+                    float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
+                    if constexpr (RES) y = add_res(y, rv[r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
                     const unsigned voff = row_ok ? col_voff[b] : OOB;
                     if (p.out_s8)
                         __builtin_amdgcn_raw_buffer_store_b8((unsigned char) requant_s8(y, p.out_inv_scale), rc, voff,
@@ -386,6 +400,7 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), rc, voff, (unsigned) m_uni * row_bytes, 0);
                 }
             }
+        }
     } else {
         float rv[RES ? TM : 1][RES ? 16 : 1][RES ? TN : 1];
         if constexpr (RES) {
@@ -761,7 +776,7 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
 // ---- the kernel --------------------------------------------------------------------------------
 template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1, bool RES = false>
 __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
-    static_assert(!RES || DT == DT_F32, "the residual store exists for fp32 operands");
+    static_assert(!RES || DT == DT_F32 || DT == DT_I8, "the residual store exists for fp32 and int8 operands (fp32 results)");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     static_assert(TM >= 1 && TN >= 1 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile / wave grid mismatch");

@@ -346,19 +346,22 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         const float *wp = nullptr;
         rc = packed_weights(&d, (const float *) w, &wp, true);
         if (rc) return rc;
-        if (link) {
+        bool added = false;   // the addend went into the convolution's store
+        if (link || (fuse && wp)) {
             if (!wp) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges need the packed weight form");
             d.out_s8 = out_s8 ? 1 : 0;
-            d.output_scale = link->out_scale;
+            d.output_scale = link ? link->out_scale : 0.0f;
             rc = onhip_conv2d_w8_link(&d, in_s8 ? nullptr : (const float *) x, in_s8 ? (const int8_t *) x : nullptr, (const int8_t *) wp,
-                                      (const int32_t *) b, (const float *) aux, (const float *) lut, y, ws, ws_bytes, g_stream);
+                                      (const int32_t *) b, (const float *) aux, (const float *) lut, (const float *) addend, fuse == 2,
+                                      y, ws, ws_bytes, g_stream);
+            added = true;
         } else if (wp)
             rc = onhip_conv2d_w8a32_packed(&d, (const float *) x, (const int8_t *) wp, (const int32_t *) b,
                                            (const float *) aux, (const float *) lut, y, nullptr, ws, ws_bytes, g_stream);
         else
             rc = onhip_conv2d_w8a32(&d, (const float *) x, (const int8_t *) w, (const int32_t *) b, (const float *) aux,
                                     (const float *) lut, y, nullptr, ws, ws_bytes, g_stream);
-        if (!rc && fuse) {   // the int8 store does not fold the addend in: the two operators as one pass over y
+        if (!rc && fuse && !added) {   // unpacked weights: the two operators as one pass over y
             onhip_add_desc_t ad;
             memset(&ad, 0, sizeof(ad));
             ad.ndim = 4;

@@ -1342,3 +1342,47 @@ def test_add_then_relu_by_the_relu_operators_own_rules(shape, torch_dev):
     one = hip.add_f32(ta, tb, relu=2)
     torch.cuda.synchronize()
     assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 64, 14, 14, 256, 1, 1, 0), (1, 32, 9, 11, 40, 3, 1, 1), (3, 128, 7, 7, 100, 1, 1, 0), (1, 16, 20, 20, 64, 3, 2, 1),
+                                   (2, 256, 6, 6, 33, 1, 1, 0)])
+@pytest.mark.parametrize("act", [abi.NOT_ACT, abi.RELU, abi.SILU])
+@pytest.mark.parametrize("relu_after", [False, True])
+def test_int8_convolution_with_the_add_and_relu_in_its_store(shape, act, relu_after, torch_dev, oracle):
+    """onhip_conv2d_w8_link with an addend: fp32 or int8 NHWC activations in, the Add (and the Relu, by its own two rules)
+    of a residual block in the convolution's fp32 store, equal bit for bit to the W8A32 convolution followed by the Add
+    and Relu operators; NaN and negative-zero sums included"""
+    torch = torch_dev
+    n, cin, h, w, cout, k, stride, pad = shape
+    d = cases.cd(cin, cout, k, stride, pad, h, w=w, n=n, act=act, input_scale=0.043)
+    x, w8, b32, aux = cases.conv_inputs(f"resq_{cin}_{cout}_{h}_{w}_{k}_{stride}", d, quant=True)
+    lut = cases.silu_lut()
+    oh, ow = d.out_hw()
+    y = hip.conv2d_w8a32(d, dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, lut))
+    torch.cuda.synchronize()
+    yh = y.cpu().numpy()
+    rng = np.random.default_rng(3)
+    addend = rng.normal(size=yh.shape).astype(np.float32)
+    fa, fy = addend.reshape(-1), yh.reshape(-1)
+    nel = fa.size
+    for i in (0, 7, nel - nel % 32 - 1, nel - nel % 32, nel - 1):
+        if 0 <= i < nel:
+            fa[i] = np.float32("nan")
+    for i in (3, nel - nel % 32 - 2, nel - nel % 32 + 1, nel - 2):
+        if 0 <= i < nel and fy[i] == 0:
+            fa[i] = np.float32(-0.0)
+    ta = dev(torch, addend)
+    want = hip.add_f32(y, ta)
+    if relu_after:
+        want = hip.relu_f32(want)
+    wp = hip.pack_conv_weights_w8(d, dev(torch, w8))
+    got = hip.conv2d_w8_link(d, wp, dev(torch, b32), dev(torch, aux), dev(torch, lut), x=dev(torch, x), addend=ta, relu_after=relu_after)
+    xq = hip.quantize_nhwc_s8(dev(torch, x), d.input_scale)
+    got_q = hip.conv2d_w8_link(d, wp, dev(torch, b32), dev(torch, aux), dev(torch, lut), xq=xq, addend=ta, relu_after=relu_after)
+    plain = hip.conv2d_w8_link(d, wp, dev(torch, b32), dev(torch, aux), dev(torch, lut), xq=xq)
+    torch.cuda.synchronize()
+    bits = lambda t: t.cpu().numpy().view(np.uint32)   # noqa: E731
+    assert np.array_equal(bits(got), bits(want))
+    assert np.array_equal(bits(got_q), bits(want))
+    assert np.array_equal(bits(plain), bits(y))
