@@ -208,12 +208,14 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
  * consumer whose input_scale is that value would make of the fp32 result, conv.c:961-973).  Weights packed by
  * onhip_conv2d_w8a32_pack_weights.  Depthwise is refused.  addend, when not null (fp32 results only): a tensor of the
  * result's shape added to it in the store (device/x86/Add/add.c:96), followed, with relu_after != 0, by relu as
- * device/x86/Relu/relu.c:27-52 (both of its rules, by element index): the three operators' bytes in one pass.  No
+ * device/x86/Relu/relu.c:27-52 (both of its rules, by element index): the three operators' bytes in one pass.  y_twin,
+ * when not null (with an addend, cout a multiple of 16, d->out_s8 == 0): the fp32 result is also stored there as int8
+ * NHWC quantised with d->output_scale, for the int8 convolutions among the tensor's readers.  No
  * counterpart in the reference, whose W8A32 operators (device/x86/Conv/conv.c:939-1067) always take and return fp32; the
  * device-resident runtime calls it for edges between two int8 convolutions and for the one that closes a residual block. */
 int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,
                          const int32_t *bias32, const float *weight_aux, const float *silu_lut, const float *addend,
-                         int32_t relu_after, void *y, void *workspace, size_t workspace_bytes, void *stream);
+                         int32_t relu_after, void *y, int8_t *y_twin, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- bf16 / fp16 with 16-bit storage --------------------------------------------------------------------------
  * The reference has the two types as enumerators only (ELEM_TYPE_E TYPE_FP16 / the cuda tile fields,
@@ -441,7 +443,8 @@ int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFE
 int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* `eval_link` of libConv_hip.so: a dense int8 (W8A32) Conv whose input and/or result travel as int8 NHWC (channels padded
  * to 16) instead of fp32 NCHW, see onhip_conv2d_w8_link.  Slots as for `eval`; inputs[4] = host pointer to
- * {int32 in_s8, int32 out_s8, float out_scale}; inputs[5] = null, or host pointer to an int32 1 / 2 for the Add (and
+ * {int32 in_s8, int32 out_s8, float out_scale, int32 twin} (twin != 0: outputs[1] = device buffer for the int8 copy of an
+ * fp32 result with a folded Add); inputs[5] = null, or host pointer to an int32 1 / 2 for the Add (and
  * Relu) of a residual block with its other operand in inputs[3] (fp32 results only).  No counterpart in the reference. */
 int onhip_conv_link_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_conv_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);

@@ -895,7 +895,7 @@ int onhip::forget_quantised_tables(const void *base, size_t bytes) {
 static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8, int packed_w,
                              const int32_t *bias32, const float *weight_aux, const float *silu_lut, void *y,
                              int32_t *acc32, void *workspace, size_t workspace_bytes, int nhwc_out, void *stream,
-                             const float *addend = nullptr, int relu_after = 0) {
+                             const float *addend = nullptr, int relu_after = 0, int8_t *twin = nullptr) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
@@ -904,6 +904,9 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     if (nhwc_out && !d->out_s8) return set_error(ONHIP_ERR_ARG, "conv w8a8: the NHWC output form is int8 (out_s8 = 1)");
     if (addend && (d->out_s8 || acc32 || d->group != 1))
         return set_error(ONHIP_ERR_ARG, "conv w8a32: an addend goes with dense convolutions and fp32 results");
+    if (twin && (!addend || d->cout % 16 || !(d->output_scale > 0.0f) || reinterpret_cast<uintptr_t>(twin) % 4 ||
+                 (long long) d->n * OH * OW * d->cout >= (1LL << 31)))
+        return set_error(ONHIP_ERR_ARG, "conv w8a32: the int8 twin goes with an addend, output channels in sixteens and an output_scale");
     if ((xq || nhwc_out) && d->group != 1) return set_error(ONHIP_ERR_ARG, "conv w8a8: depthwise is not available in the NHWC int8 form");
     // the reference pads all four sides by pads[0] (conv.c:979-999) while shapes come from the four
     // pads: only uniform padding is self-consistent
@@ -1005,6 +1008,9 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
         p.res = addend;
         p.res_relu = relu_after ? 1 : 0;
         p.res_body = (unsigned) (n_out - n_out % 32);   // relu.c:27-52
+        p.twin = twin;
+        p.twin_pitch = d->cout;
+        p.twin_inv_scale = twin ? 1.0f / d->output_scale : 0.0f;
     }
     // 3x3, stride 1, few channels, int8 in and out: the kernel that keeps the band's input in LDS and the weights in registers
     // tuning hooks: ONHIP_NO_PATCH keeps to the implicit-GEMM kernels, and so does a forced tile of theirs; ONHIP_PATCH_ALL
@@ -1046,11 +1052,11 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
 
 int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,
                          const int32_t *bias32, const float *weight_aux, const float *silu_lut, const float *addend,
-                         int32_t relu_after, void *y, void *workspace, size_t workspace_bytes, void *stream) {
+                         int32_t relu_after, void *y, int8_t *y_twin, void *workspace, size_t workspace_bytes, void *stream) {
     if (!d) return set_error(ONHIP_ERR_ARG, "conv w8 link: null descriptor");
     if ((x != nullptr) == (xq != nullptr)) return set_error(ONHIP_ERR_ARG, "conv w8 link: exactly one of x and xq");
     return conv2d_w8a32_impl(d, x, xq, w8_packed, 1, bias32, weight_aux, silu_lut, y, nullptr, workspace, workspace_bytes,
-                             d->out_s8 ? 1 : 0, stream, addend, relu_after);
+                             d->out_s8 ? 1 : 0, stream, addend, relu_after, y_twin);
 }
 
 static int matmul_impl(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,

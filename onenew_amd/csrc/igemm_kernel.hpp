@@ -362,6 +362,10 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
         // RES: the residual operand of a folded Add (fp32 results): a row tile's addends are requested together
         const rsrc_t rres = make_rsrc(RES ? reinterpret_cast<const char *>(p.res) + (size_t) batch * p.c_batch_stride * 4 : nullptr,
                                       RES ? RSRC_RANGE : 0u);
+        const rsrc_t rtwin = make_rsrc(RES ? p.twin : nullptr, RES && p.twin ? RSRC_RANGE : 0u);
+        unsigned tw[TN];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) tw[b] = 0;
 #pragma unroll
         for (int a = 0; a < TM; ++a) {
             float rv[RES ? 16 : 1][RES ? TN : 1];
@@ -391,7 +395,19 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                     const float fbias = __fadd_rn(f, fb);
                     f = p.bias32 ? fbias : f;
                     float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
-                    if constexpr (RES) y = add_res(y, rv[r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
+                    if constexpr (RES) {
+                        y = add_res(y, rv[r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
+                        // the int8 twin: registers 4 q .. 4 q + 3 are four consecutive channels of the lane's pixel
+                        if (p.twin) {   // uniform
+                            tw[b] |= ((unsigned) requant_s8(y, p.twin_inv_scale) & 0xffu) << (8 * (r % 4));
+                            if (r % 4 == 3) {
+                                const int n = n_wave + b * 32 + li, m4 = m_wave + a * 32 + 8 * (r / 4) + 4 * lh;
+                                const bool ok = n < p.N && m4 < p.M;
+                                __builtin_amdgcn_raw_buffer_store_b32(tw[b], rtwin, ok ? (unsigned) (n * p.twin_pitch + m4) : OOB, 0, 0);
+                                tw[b] = 0;
+                            }
+                        }
+                    }
                     const unsigned voff = row_ok ? col_voff[b] : OOB;
                     if (p.out_s8)
                         __builtin_amdgcn_raw_buffer_store_b8((unsigned char) requant_s8(y, p.out_inv_scale), rc, voff,

@@ -201,6 +201,12 @@ struct IgemmParams {
     // the way out (followed by a ReLU when res_relu is set)
     int out_h16;
     const void *res16;
+    // int8 kernels with a residual operand: when not null, the fp32 result (after the Add and the Relu) is ALSO stored
+    // here as int8 NHWC, element (pixel n, channel m) at n * twin_pitch + m, quantised with twin_inv_scale: the form the
+    // int8 convolutions that read the tensor would make of it (M a multiple of 16, so no padding channels exist)
+    int8_t *twin;
+    int twin_pitch;
+    float twin_inv_scale;
     // split-K workspace: partial sums [split][M][N] fp32 (nullptr when unsplit)
     float *partial;
     // reduction inside the launch by the last slice of a tile to arrive: one counter per tile (uncached memory, like

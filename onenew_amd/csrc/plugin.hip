@@ -241,9 +241,12 @@ static long long numel(const OPERAND_S *o) {
 // What travels along the edges of an int8 convolution inside a chain of them (inputs[4] of `eval_link`): in_s8 != 0, the
 // input tensor is int8 NHWC with channels padded to 16, quantised with this operator's input_scale by its producer;
 // out_s8 != 0, the result is stored that way for consumers whose input_scale is out_scale.
+// twin != 0 (fp32 results with a folded Add only): outputs[1] receives the result once more, as int8 NHWC quantised with
+// out_scale, for the int8 convolutions among its readers.
 struct ConvLink {
     int32_t in_s8, out_s8;
     float out_scale;
+    int32_t twin;
 };
 
 // fuse 0: the Conv of the reference.  1: inputs[3] holds a tensor of the output's shape that is added to the result
@@ -351,9 +354,15 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
             if (!wp) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges need the packed weight form");
             d.out_s8 = out_s8 ? 1 : 0;
             d.output_scale = link ? link->out_scale : 0.0f;
+            int8_t *twin = nullptr;
+            if (link && link->twin) {
+                twin = reinterpret_cast<int8_t *>(outputs[1].addr);
+                if (!twin || !is_device_ptr(twin) || !fuse || out_s8)
+                    return set_error(ONHIP_ERR_ARG, "Conv eval: the int8 twin needs a device buffer in outputs[1], a folded Add and an fp32 result");
+            }
             rc = onhip_conv2d_w8_link(&d, in_s8 ? nullptr : (const float *) x, in_s8 ? (const int8_t *) x : nullptr, (const int8_t *) wp,
                                       (const int32_t *) b, (const float *) aux, (const float *) lut, (const float *) addend, fuse == 2,
-                                      y, ws, ws_bytes, g_stream);
+                                      y, twin, ws, ws_bytes, g_stream);
             added = true;
         } else if (wp)
             rc = onhip_conv2d_w8a32_packed(&d, (const float *) x, (const int8_t *) wp, (const int32_t *) b,

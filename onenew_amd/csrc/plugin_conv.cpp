@@ -35,8 +35,9 @@ extern "C" __attribute__((visibility("default"))) int eval_add_relu(BUFFER_INFO_
 }
 
 // Not in the reference: a dense int8 convolution inside a chain of them, taking and/or leaving its activations as int8
-// NHWC.  Slots as for `eval`; inputs[4] = {int32 in_s8, int32 out_s8, float out_scale} in host memory; inputs[5] = null
-// or an int32 fold code (1 Add, 2 Add + Relu, the other operand in inputs[3]).
+// NHWC.  Slots as for `eval`; inputs[4] = {int32 in_s8, int32 out_s8, float out_scale, int32 twin} in host memory (twin:
+// outputs[1] = device buffer that receives an fp32 result with a folded Add once more as int8 NHWC); inputs[5] = null or
+// an int32 fold code (1 Add, 2 Add + Relu, the other operand in inputs[3]).
 extern "C" __attribute__((visibility("default"))) int eval_link(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
                                                                 BUFFER_INFO_S *outputs) {
     return onhip_conv_link_eval(params, inputs, outputs);

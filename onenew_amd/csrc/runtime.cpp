@@ -120,6 +120,8 @@ struct Tensor {
     std::string alias;       // an operand folded away with its producer reads as this one (fuse_residual_blocks)
     bool never_written = false;   // an operand inside a fused attention block: it has no buffer and no value
     bool as_s8 = false;           // written and read as int8 NHWC, channels padded to 16 (link_int8_convs)
+    bool has_twin = false;        // fp32, and stored once more as int8 NHWC for the int8 convolutions among its readers
+    void *twin_dev = nullptr;
 };
 
 struct Node {
@@ -133,8 +135,9 @@ struct Node {
     int block_dw = -1, block_pw = -1;        // fused inverted-residual block (fuse 7): its depthwise and last convolutions
     // an int8 convolution whose input and/or result travel as int8 NHWC (link_int8_convs): what `eval_link` reads from
     // inputs[4] ({in_s8, out_s8, out_scale}) and inputs[5] (the fold code, when an Add is folded in)
-    struct { int32_t in_s8, out_s8; float out_scale; } link = {0, 0, 0.0f};
+    struct { int32_t in_s8, out_s8; float out_scale; int32_t twin; } link = {0, 0, 0.0f, 0};
     int32_t link_fuse = 0;
+    bool reads_twin = false;   // its input is the int8 copy of an fp32 operand
     BUFFER_INFO_S params[BUF_MAXNUM], inputs[BUF_MAXNUM], outputs[BUF_MAXNUM];
     const BASE_CONFIG_S *base() const { return reinterpret_cast<const BASE_CONFIG_S *>(cfg.data()); }
 };
@@ -436,6 +439,7 @@ int allocate(onrt_net &net) {
             if (s8 > t.bytes) t.bytes = s8;
         }
         act_total += (t.bytes + 255) & ~(size_t) 255;
+        if (t.has_twin) act_total += ((size_t) numel(t.desc) + 255) & ~(size_t) 255;   // a byte per element, no padding channels
     }
     if (act_total) {
         ONRT_HIP(hipMalloc(&net.act_arena, act_total));
@@ -445,6 +449,10 @@ int allocate(onrt_net &net) {
             if (t.is_init || t.desc.not_need_buf || !t.alias.empty() || t.never_written) continue;
             t.dev = static_cast<char *>(net.act_arena) + off;
             off += (t.bytes + 255) & ~(size_t) 255;
+            if (t.has_twin) {
+                t.twin_dev = static_cast<char *>(net.act_arena) + off;
+                off += ((size_t) numel(t.desc) + 255) & ~(size_t) 255;
+            }
         }
     }
     for (auto &kv : net.tensors) {
@@ -837,6 +845,43 @@ int link_int8_convs(onrt_net &net) {
         net.tensors[name].as_s8 = true;
         ++net.int8_links;
     }
+    // The result of an int8 Conv with a folded Add (the output of a residual block) stays fp32, because the next block's
+    // Add reads it; the int8 Convs among its readers get an int8 copy, written by the same store (outputs[1] of
+    // `eval_link`), instead of each quantising the fp32 tensor again.  Output channels in sixteens, so that the copy has
+    // no padding channels.
+    for (int idx : net.order) {
+        Node &p = net.nodes[idx];
+        const CONV_CONFIG_S *pc = dense_int8(p);
+        if (!pc || (p.fuse != 1 && p.fuse != 2) || p.link.out_s8) continue;
+        const std::string name = result_of(p);
+        Tensor &t = net.tensors[name];
+        if (t.desc.not_need_buf || t.desc.shapes[1] % 16 || !t.alias.empty()) continue;
+        float scale = 0.0f;
+        bool ok = true;
+        std::vector<int> takers;
+        for (int ri : readers_of(net, name)) {
+            const Node &c = net.nodes[ri];
+            const CONV_CONFIG_S *cc = dense_int8(c);
+            if (!cc || c.in[0] != name || c.link.in_s8) continue;            // reads the fp32 tensor
+            if (!(cc->input_scale > 0.0f) || (scale != 0.0f && cc->input_scale != scale)) { ok = false; break; }
+            scale = cc->input_scale;
+            takers.push_back(ri);
+        }
+        if (!ok || takers.empty()) continue;
+        p.link.twin = 1;
+        p.link.out_scale = scale;
+        p.link_fuse = p.fuse;
+        p.eval = net.conv_link;
+        t.has_twin = true;
+        for (int ri : takers) {
+            Node &c = net.nodes[ri];
+            c.link.in_s8 = 1;
+            c.link_fuse = c.fuse;
+            c.reads_twin = true;
+            c.eval = net.conv_link;
+        }
+        ++net.int8_links;
+    }
     return ONRT_OK;
 }
 
@@ -1040,9 +1085,10 @@ int fill_slots(onrt_net &net) {
             nd.inputs[8].addr = c.in.size() > 2 ? (int64_t) net.tensors[c.in[2]].dev : 0;
         }
         if (nd.fuse == 1 || nd.fuse == 2 || nd.fuse == 6) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
-        if (nd.link.in_s8 || nd.link.out_s8) {
+        if (nd.link.in_s8 || nd.link.out_s8 || nd.link.twin) {
             nd.inputs[4].addr = (int64_t) &nd.link;
             nd.inputs[5].addr = nd.link_fuse ? (int64_t) &nd.link_fuse : 0;
+            if (nd.reads_twin) nd.inputs[0].addr = (int64_t) net.tensors[nd.in[0]].twin_dev;
         }
         int out_slot = 1 + (int) nd.in.size();   // host/op.h:131-137
         for (size_t k = 0; k < nd.out.size(); ++k, ++out_slot) {
@@ -1051,6 +1097,7 @@ int fill_slots(onrt_net &net) {
             nd.params[out_slot].addr = (int64_t) &t.desc;
             nd.outputs[k].addr = (int64_t) t.dev;
         }
+        if (nd.link.twin) nd.outputs[1].addr = (int64_t) net.tensors[nd.fused_out.empty() ? nd.out[0] : nd.fused_out].twin_dev;
         // per-model tunables in the last params slot (host/ops/conv.h:66-69, host/ops/maxpool.h:57-62); the
         // HIP operators bring their own workspace, so the shared scratch buffer stays unallocated
         nd.params[BUF_MAXNUM - 1].addr = (int64_t) &net.useful;

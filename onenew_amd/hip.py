@@ -94,7 +94,7 @@ def load():
     L.onhip_calib_percentile.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), vp, C.c_size_t, vp]
     L.onhip_quantize_nhwc_s8.argtypes = [vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float, vp, vp]
     L.onhip_conv2d_w8a8_nhwc.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp]
-    L.onhip_conv2d_w8_link.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, C.c_int32, vp, vp, C.c_size_t, vp]
+    L.onhip_conv2d_w8_link.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, C.c_int32, vp, vp, vp, C.c_size_t, vp]
     L.onhip_matmul.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_matmul_add.argtypes = [C.POINTER(MatmulDesc), vp, vp, vp, vp, vp, vp]
     L.onhip_gemm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
@@ -399,9 +399,10 @@ def conv2d_w8a8_nhwc(d, xq, w8_packed, bias32, weight_aux, silu_lut=None, out=No
     return out
 
 
-def conv2d_w8_link(d, w8_packed, bias32, weight_aux, silu_lut=None, x=None, xq=None, addend=None, relu_after=False, out=None):
+def conv2d_w8_link(d, w8_packed, bias32, weight_aux, silu_lut=None, x=None, xq=None, addend=None, relu_after=False, out=None, twin=None):
     """one link of an int8 chain: fp32 NCHW (x) or int8 NHWC (xq) in; fp32 NCHW out, optionally with an addend (and a
-    Relu) folded into the store, or int8 NHWC out (d.out_s8 = 1, d.output_scale)"""
+    Relu) folded into the store and an int8 NHWC copy quantised with d.output_scale in `twin`, or int8 NHWC out
+    (d.out_s8 = 1, d.output_scale)"""
     import torch
     oh, ow = d.out_hw()
     src = x if x is not None else xq
@@ -413,7 +414,7 @@ def conv2d_w8_link(d, w8_packed, bias32, weight_aux, silu_lut=None, x=None, xq=N
     need = conv2d_w8a32_workspace(d)
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=src.device)
     _check(load().onhip_conv2d_w8_link(C.byref(d), _ptr(x), _ptr(xq), _ptr(w8_packed), _ptr(bias32), _ptr(weight_aux), _ptr(silu_lut),
-                                       _ptr(addend), int(relu_after), _ptr(out), _ptr(ws), ws.numel(), _stream()), "onhip_conv2d_w8_link")
+                                       _ptr(addend), int(relu_after), _ptr(out), _ptr(twin), _ptr(ws), ws.numel(), _stream()), "onhip_conv2d_w8_link")
     return out
 
 

@@ -116,10 +116,11 @@ def quantised_block():
     return m.tobytes(), [_r("xq", (1, 16, 18, 18))]
 
 
-def quantised_chain(n=1, hw=18, different_scales=False, extra_reader=False):
+def quantised_chain(n=1, hw=18, different_scales=False, extra_reader=False, tail=False):
     """dense W8A32 convolutions feeding each other: q1 -> (q2, q2b with one input_scale) , q2 -> q3, and a residual
     block qa -> qb + skip -> Relu behind q3; the operands between them can travel as int8.  different_scales: q2b
-    quantises its input differently from q2; extra_reader: a Relu also reads q1's result"""
+    quantises its input differently from q2; extra_reader: a Relu also reads q1's result; tail: two more int8
+    convolutions read the residual block's fp32 result (which stays an output)"""
     from oracle import oracle
     m = onefile.OneModel()
     m.input("x", (n, 16, hw, hw))
@@ -151,6 +152,13 @@ def quantised_chain(n=1, hw=18, different_scales=False, extra_reader=False):
     m.add("sum", "qb_out", "q3_out", "sum_out")
     m.relu("relu_s", "sum_out", "out")
     m.output("out", (n, 32, hw, hw))
+    if tail:
+        w8, b32, aux = q("ct", (48, 32, 3, 3), 0.1)
+        m.conv("qt", "out", w8, b32, "out_t", pad=1, act=abi.RELU, quant=(aux, 0.045))
+        m.output("out_t", (n, 48, hw, hw))
+        w8, b32, aux = q("cu", (16, 32, 1, 1), 0.2)
+        m.conv("qu", "out", w8, b32, "out_u", stride=2, act=abi.NOT_ACT, quant=(aux, 0.045))
+        m.output("out_u", (n, 16, (hw - 1) // 2 + 1, (hw - 1) // 2 + 1))
     return m.tobytes(), [_r("xqc", (n, 16, hw, hw))]
 
 

@@ -1386,3 +1386,15 @@ def test_int8_convolution_with_the_add_and_relu_in_its_store(shape, act, relu_af
     assert np.array_equal(bits(got), bits(want))
     assert np.array_equal(bits(got_q), bits(want))
     assert np.array_equal(bits(plain), bits(y))
+    if cout % 16 == 0:
+        # the same store also leaves the result as int8 NHWC, as the input quantiser of a reader would make it (the NaN
+        # sums aside: no quantiser is defined on them)
+        dt = ConvDesc.from_buffer_copy(d)
+        dt.output_scale = 0.06
+        twin = torch.full((n, oh, ow, cout), 77, dtype=torch.int8, device="cuda")
+        got_t = hip.conv2d_w8_link(dt, wp, dev(torch, b32), dev(torch, aux), dev(torch, lut), xq=xq, addend=ta, relu_after=relu_after, twin=twin)
+        ref_t = hip.quantize_nhwc_s8(want, 0.06)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(got_t), bits(want))
+        ok = ~np.isnan(np.transpose(want.cpu().numpy(), (0, 2, 3, 1)))
+        assert np.array_equal(twin.cpu().numpy()[ok], ref_t.cpu().numpy()[ok])

@@ -721,6 +721,15 @@ def test_int8_convolutions_exchange_int8_operands(torch_dev, monkeypatch):
     for a, b in zip(net.run(*ins), plain_outs):
         assert np.array_equal(a, b)
     net.close()
+    # the fp32 result of the residual block, read by two more int8 convolutions: they get its int8 copy from the same store
+    for n in (1, 2):
+        data, ins = one_models.quantised_chain(n=n, tail=True)
+        net = rt.Net(data)
+        assert net.int8_links() == 4
+        ref = one_model.run(data, ins, keep_all=True)
+        for (oname, _), got in zip(net.outputs, net.run(*ins)):
+            assert np.array_equal(got, ref[oname]), ("tail", oname)
+        net.close()
     for kw, links in (({"different_scales": True}, 2), ({"extra_reader": True}, 2)):
         data, ins = one_models.quantised_chain(**kw)
         net = rt.Net(data)
