@@ -109,6 +109,23 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
         }
     }
 
+    // the quantised activation table that the int8 NHWC store gathers from (8 KiB, 32 bytes per thread): requested here,
+    // before any operand load (being the oldest loads in flight, the K loop's counted waits cover them), and written
+    // to LDS behind the staging area once the K loop has left it, instead of a memory round trip plus a barrier of its own
+    // at the head of every tile's store
+    uint4 table_q[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    bool table_pre = false;
+    if constexpr (DT == DT_I8) {
+        table_pre = p.out_s8 && p.out_mode == OUT_PLAIN && p.c_stride_m == 1 && !p.acc_out && p.ep.qlut != nullptr &&
+                    (p.ep.act == SILU || p.ep.act == ONHIP_ACT_GELU_LUT);   // uniform
+        if (table_pre) {
+            const rsrc_t rq = make_rsrc(p.ep.qlut, 8192u);
+            table_q[0] = buf_load_b128(rq, (unsigned) tid * 16u, 0);
+            table_q[1] = buf_load_b128(rq, (unsigned) (tid + THREADS) * 16u, 0);
+        }
+    }
+    asm volatile("" ::: "memory");   // these loads stay ahead of the operand loads: the stage waits count loads in issue order
+
     const char *a_base = reinterpret_cast<const char *>(p.A);
     const char *b_base = reinterpret_cast<const char *>(p.B) - (size_t) p.b_shift_bytes;
     const unsigned a_bytes = (unsigned) p.a_slice_bytes, b_bytes = (unsigned) (p.b_slice_bytes + p.b_shift_bytes);
@@ -278,6 +295,14 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
             rows[tid] = row_bias;
         }
     }
+    if constexpr (DT == DT_I8) {
+        if (table_pre) {
+            unsigned char *ql = lds + BN * (BM + 16);   // where write_tile_nhwc_s8 looks for it
+            reinterpret_cast<uint4 *>(ql)[tid] = table_q[0];
+            reinterpret_cast<uint4 *>(ql)[tid + THREADS] = table_q[1];
+            if (tid == 0) ql[-1] = 0;                   // its "below the table" entry
+        }
+    }
     __syncthreads();
 
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
@@ -285,12 +310,12 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
         if (p.out_s8 && p.out_mode == OUT_PLAIN && p.c_stride_m == 1 && !p.acc_out) {
             switch (p.ep.act) {
                 case NOT_ACT:
-                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows); break;
-                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows); break;
-                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows); break;
+                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows, table_pre); break;
+                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows, table_pre); break;
+                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows, table_pre); break;
                 case SILU:
-                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows); break;
-                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows); break;
+                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows, table_pre); break;
+                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN, true>(p, acc, lds, m0, n0, m_wave, n_wave, li, lh, tid, rows, table_pre); break;
             }
             return;
         }
