@@ -676,16 +676,20 @@ def cpu_baseline(layers, tag, unit, budget_s=12.0):
 
 
 def bench_net(torch, args):
+    print(json.dumps(net_result(torch, args.workload, args.steps, args.warmup, not args.no_cpu)))
+
+
+def net_result(torch, workload, steps, warmup, with_cpu):
     """A whole model (ResNet-50: 53 Conv, MaxPool, 16 Add, 16 Relu, GlobalAveragePool, Gemm; MobileNetV2: 52 Conv of
     which 17 depthwise, 10 Add, GlobalAveragePool, Gemm; ViT-Tiny: patch Conv, 12 encoder blocks of LayerNormalization /
     MatMul / Add / Transpose / Softmax / Gelu, mean over the tokens, Gemm) as a .one file through the device-resident runtime
     (libonenew_rt.so): every operator back to back on the device, input and output in device memory.  A step is one
     inference of the batch."""
     from onenew_amd import rt, stacks
-    n = int(args.workload.split("_b")[1])
-    model = "ResNet-50" if args.workload.startswith("resnet50") else "MobileNetV2" if args.workload.startswith("mobilenetv2") else "ViT-Tiny"
+    n = int(workload.split("_b")[1])
+    model = "ResNet-50" if workload.startswith("resnet50") else "MobileNetV2" if workload.startswith("mobilenetv2") else "ViT-Tiny"
     make = {"ResNet-50": stacks.resnet50_model, "MobileNetV2": stacks.mobilenet_v2_model, "ViT-Tiny": stacks.vit_tiny_model}[model]
-    int8 = "_int8_net_" in args.workload   # the convolutions in the W8A32 form of the offline quantiser
+    int8 = "_int8_net_" in workload   # the convolutions in the W8A32 form of the offline quantiser
     if int8:
         make = lambda batch: stacks.resnet50_model(batch, quantised=True)   # noqa: E731
     data, in_shape, flops = make(n)
@@ -693,18 +697,18 @@ def bench_net(torch, args):
     x = torch.randn(in_shape, dtype=torch.float32, device="cuda")
     y = torch.empty((n, 1000), dtype=torch.float32, device="cuda")
     ins, outs = [x.data_ptr()], [y.data_ptr()]
-    for _ in range(max(2, args.warmup)):     # the first inferences measure tile choices and pack the weights
+    for _ in range(max(2, warmup)):     # the first inferences measure tile choices and pack the weights
         net.run_raw(ins, outs)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         net.run_raw(ins, outs)
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
     # device time of one inference: events around it on the default stream, where the plugins launch
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     dev_ms = []
-    for _ in range(max(5, args.steps)):
+    for _ in range(max(5, steps)):
         e0.record(torch.cuda.default_stream())
         net.run_raw(ins, outs)
         e1.record(torch.cuda.default_stream())
@@ -713,7 +717,7 @@ def bench_net(torch, args):
     dev = float(np.median(dev_ms))
     ops = net.ops()
     cpu = None
-    if not args.no_cpu:
+    if with_cpu:
         from oracle import one_model
         if one_model.have_ref_runner():
             data1, shape1, flops1 = make(1)
@@ -722,8 +726,8 @@ def bench_net(torch, args):
             cpu = {"value": round(flops1 / (ms * 1e-3) / 1e12, 5), "unit": "TFLOP/s", "cores": 8, "kind": "reference",
                    "sample": f"40 inferences of the same model at batch 1 through the reference's host operator classes "
                              f"and x86 kernels, median {ms:.2f} ms", "ms_per_inference": round(ms, 3)}
-    line = {"metric": f"{args.workload.split('_net_')[0]}_net_{'w8a32_tops' if int8 else 'fp32_tflops'}", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TOP/s" if int8 else "TFLOP/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+    line = {"metric": f"{workload.split('_net_')[0]}_net_{'w8a32_tops' if int8 else 'fp32_tflops'}", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 3), "unit": "TOP/s" if int8 else "TFLOP/s",
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8" if int8 else "f32", "data": "synthetic",
             "config": {"workload": f"{model} .one model {'W8A32 (int8 weights and activations, int32 accumulate; ' + str(net.int8_links()) + ' operands between convolutions travel as int8)' if int8 else 'fp32'}, batch {n}, 224x224, {len(ops)} operators through the "
                                    f"device-resident runtime, input and logits in HBM", "operators": len(ops),
@@ -733,7 +737,8 @@ def bench_net(torch, args):
                          "frac": round(flops / (dev * 1e-3) / 1e12 / PEAK["i8" if int8 else "f32"], 4), "traffic": None,
                          "launches": len(ops), "device_ms_per_inference": round(dev, 4)},
             "cpu_baseline": cpu, "images_per_s": round(n / (ms_per_step * 1e-3), 1)}
-    print(json.dumps(line))
+    net.close()
+    return line
 
 
 METRIC = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vit_tiny_glue_ops_fp32_tflops",
@@ -742,6 +747,7 @@ METRIC = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vi
           "vit": "vit_tiny_matmul_{dtype}_tflops", "cfg1": "conv2d_relu_{dtype}_tflops"}
 
 # the other configurations of the benchmark, timed after the headline one in a default run
+NET_CONFIGS = ["resnet50_net_b32", "resnet50_int8_net_b32", "mobilenetv2_net_b64", "vit_tiny_net_b64"]
 OTHER_CONFIGS = ["cfg1", "cfg1_bf16", "resnet50_b1", "resnet50_b32_bf16", "mobilenetv2_b64", "mobilenetv2_b1", "vit_tiny_b64", "vit_tiny_b64_bf16", "vit_tiny_b1",
                  "yolov8s_int8_b16", "yolov8s_int8chain_b16", "yolov8s_int8chain_b1"]
 
@@ -964,6 +970,16 @@ def main():
             print(f"[bench] {name}: {c['value']} {c['unit']}, {c['ms_per_step']} ms per step, roofline {c['roofline']['bound']} "
                   f"{c['roofline']['frac']}", file=sys.stderr, flush=True)
             del r
+        # whole models as .one files through the device-resident runtime (fewer inferences, no CPU leg)
+        for name in NET_CONFIGS:
+            torch.cuda.empty_cache()
+            t0 = time.perf_counter()
+            r = net_result(torch, name, steps=10, warmup=3, with_cpu=False)
+            c = {"workload": name, "what": r["config"]["workload"], "dtype": r["dtype"], "value": r["value"], "unit": r["unit"],
+                 "ms_per_step": r["ms_per_step"], "images_per_s": r["images_per_s"], "operators": r["config"]["operators"],
+                 "device_ms_per_inference": r["roofline"]["device_ms_per_inference"], "bench_seconds": round(time.perf_counter() - t0, 1)}
+            configs.append(c)
+            print(f"[bench] {name}: {c['value']} {c['unit']}, {c['ms_per_step']} ms per inference of the batch", file=sys.stderr, flush=True)
         line["configs"] = configs
     print(json.dumps(line))
 
