@@ -31,7 +31,8 @@ class Plugin:
         # entry points beside `eval` that the HIP Conv plugin has and the reference's plugins do not: the convolution
         # with the Add (and Relu) of a residual block folded in, the other operand of the Add in inputs[3]
         # and a whole inverted-residual block (eval_block, eval_block_takes); the MatMul plugin's fused forms
-        for extra in ("eval_add", "eval_add_relu", "eval_block", "eval_block_takes", "eval_attention", "eval_bias", "eval_bias_gelu",
+        # (eval_link: an int8 convolution whose activations travel as int8 NHWC on one or both sides)
+        for extra in ("eval_add", "eval_add_relu", "eval_block", "eval_block_takes", "eval_link", "eval_attention", "eval_bias", "eval_bias_gelu",
                       "eval_bias_add"):
             fn = getattr(self.lib, extra, None) if hasattr(self.lib, extra) else None
             if fn is not None:
@@ -192,6 +193,44 @@ class Conv(_Op):
         self.inputs_vec[3].addr = 0
         if rc != 0:
             raise RuntimeError(f"Conv eval returned {rc}")
+        return out
+
+
+class ConvLink(Conv):
+    """A dense W8A32 Conv through the HIP Conv plugin's `eval_link`: the slots of `eval` plus inputs[4] = {int32 in_s8,
+    int32 out_s8, float out_scale, int32 twin} and inputs[5] = null or an int32 fold code (1: Add, 2: Add + Relu, the
+    other operand in inputs[3]).  in_s8: x is int8 [n, h, w, channels padded to 16]; out_s8: the result is stored that
+    way, quantised with out_scale.  No counterpart among the reference's host classes."""
+
+    class _Flags(C.Structure):
+        _fields_ = [("in_s8", C.c_int32), ("out_s8", C.c_int32), ("out_scale", C.c_float), ("twin", C.c_int32)]
+
+    def __init__(self, plugin, desc, weight, bias, weight_aux, silu_lut=None):
+        super().__init__(plugin.eval_link, desc, weight, bias, weight_aux=weight_aux, silu_lut=silu_lut)
+
+    def __call__(self, x, in_s8=False, out_scale=None, addend=None, relu_after=False):
+        d = self.desc
+        oh, ow = d.out_hw()
+        flags = self._Flags(int(in_s8), int(out_scale is not None), float(out_scale or 0.0), 0)
+        fold = C.c_int32(0 if addend is None else 2 if relu_after else 1)
+        xin = np.ascontiguousarray(x, dtype=np.int8 if in_s8 else np.float32)
+        if out_scale is not None:
+            out = aligned_empty((d.n, oh, ow, (d.cout + 15) // 16 * 16), np.int8)
+        else:
+            out = aligned_empty((d.n, d.cout, oh, ow), np.float32)
+        self._slot(self.inputs_vec, 0, xin)
+        self._slot(self.outputs_vec, 0, out)
+        self._slot(self.inputs_vec, 4, flags)
+        kept = 3
+        if addend is not None:
+            self._slot(self.inputs_vec, 3, np.ascontiguousarray(addend, dtype=np.float32))
+            self._slot(self.inputs_vec, 5, fold)
+            kept = 5
+        rc = self.forward()
+        del self._keep[-kept:]
+        self.inputs_vec[3].addr = self.inputs_vec[4].addr = self.inputs_vec[5].addr = 0
+        if rc != 0:
+            raise RuntimeError(f"Conv eval_link returned {rc}")
         return out
 
 

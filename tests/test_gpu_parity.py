@@ -1398,3 +1398,27 @@ def test_int8_convolution_with_the_add_and_relu_in_its_store(shape, act, relu_af
         assert np.array_equal(bits(got_t), bits(want))
         ok = ~np.isnan(np.transpose(want.cpu().numpy(), (0, 2, 3, 1)))
         assert np.array_equal(twin.cpu().numpy()[ok], ref_t.cpu().numpy()[ok])
+
+
+@pytest.mark.gpu
+def test_plugin_eval_link_host_buffers(torch_dev, oracle):
+    """eval_link of the Conv plugin on tensors in host memory: fp32 in / int8 NHWC out equals the consumer's quantiser on
+    the W8A32 result of `eval`; int8 NHWC in / fp32 out with the Add and Relu folded equals Add and Relu on it, bit for bit"""
+    torch = torch_dev
+    d = cases.cd(24, 40, 3, 1, 1, 13, n=2, act=abi.SILU, input_scale=0.037)
+    x, w8, b32, aux = cases.conv_inputs("plug_link", d, quant=True)
+    lut = cases.silu_lut()
+    plug = ops.Plugin(hip.plugin_path("Conv"))
+    y = ops.Conv(plug.eval, d, w8, b32, weight_aux=aux, silu_lut=lut)(x)
+    assert np.array_equal(y, oracle.conv2d_w8a32(d, x, w8, b32, aux, lut))
+    link = ops.ConvLink(plug, d, w8, b32, aux, silu_lut=lut)
+    yq = link(x, out_scale=0.052)
+    dq = ConvDesc.from_buffer_copy(d)
+    dq.out_s8, dq.output_scale = 1, 0.052
+    refq = np.transpose(oracle.conv2d_w8a32(dq, x, w8, b32, aux, lut), (0, 2, 3, 1))
+    assert yq.shape == (2, 13, 13, 48) and np.array_equal(yq[..., :40], refq) and not yq[..., 40:].any()
+    xq = hip.quantize_nhwc_s8(dev(torch, x), d.input_scale).cpu().numpy()
+    skip = cases.datagen.normal(cases.datagen.seed_for("plug_link", "skip"), y.shape, 0.0, 1.0)
+    assert np.array_equal(link(xq, in_s8=True), y)
+    assert np.array_equal(link(xq, in_s8=True, addend=skip), oracle.add_f32(y, skip))
+    assert np.array_equal(link(x, addend=skip, relu_after=True), oracle.relu_f32(oracle.add_f32(y, skip)))
