@@ -1288,6 +1288,8 @@ def test_tune_cache_file_is_validated_and_rewritten(tmp_path):
     # 32 bytes per pixel: stride 1 with pads 1 (the rows of a band kept in LDS), other strides and pads (loaded per tap)
     (2, 32, 20, 20, 32, 3, 1, 1), (1, 24, 13, 37, 16, 3, 1, 1), (2, 32, 16, 160, 32, 3, 1, 1), (1, 32, 7, 256, 24, 3, 1, 1), (3, 20, 5, 6, 64, 3, 1, 1),
     (2, 32, 21, 23, 64, 3, 2, 1), (1, 32, 18, 18, 48, 3, 1, 0), (2, 17, 15, 15, 32, 3, 2, 1), (1, 32, 40, 80, 64, 3, 1, 1),
+    # rows too long for a band in LDS (loaded per tap instead); fewer blocks than XCDs; one pixel
+    (1, 32, 4, 300, 32, 3, 1, 1), (3, 32, 3, 3, 16, 3, 1, 1), (1, 16, 1, 1, 32, 3, 1, 1),
     # 64 bytes per pixel, stride 1, pads 1
     (2, 64, 20, 20, 64, 3, 1, 1), (1, 48, 11, 80, 32, 3, 1, 1), (1, 64, 9, 13, 40, 3, 1, 1),
     # 1x1 with 64, 96 or 128 bytes per pixel, a stride, a pad; more than 64 output channels (the implicit-GEMM kernels')
