@@ -1,15 +1,17 @@
-// int8 3x3 convolutions (stride 1, pads 1, NHWC int8 in and out: the chain form) with few channels: 32 or 64 bytes per
-// input pixel, at most 64 output channels.  The implicit-GEMM kernels read every input pixel nine times, once per filter
-// tap, through L2 into LDS; with so few channels that traffic, not the matrix cores, sets their time.  Here
+// Two kernels for the convolutions of an int8 NHWC chain (int8 in and out) that have few channels: i8patch_kernel, 3x3
+// with stride 1 and pads 1, 32 or 64 bytes per input pixel, at most 64 output channels, described here; and
+// i8direct_kernel further down (3x3 of any stride with 16 or 32 bytes per pixel, 1x1 with 64 to 128).  The implicit-GEMM
+// kernels read every input pixel nine times, once per filter tap, through L2 into LDS, and pay a tile's whole set-up and
+// store for two or three K stages; with so few channels that, not the matrix cores, sets their time.  Here
 //
 //   * a persistent workgroup walks bands of whole output rows (up to 256 pixels) of the batch; the band's input rows plus
 //     halo, (rows + 2) x (w + 2) pixels with zeros outside the image, are loaded ONCE into an LDS patch (NHWC rows are
 //     contiguous: plain 16-byte loads), the next band's into registers while this one is multiplied;
-//   * all weights of the layer (at most 64 x 9 x 64 bytes) sit in the registers of every wavefront for the life of the
-//     workgroup: lane (row lane % 32, half lane / 32) holds bytes 32 s + 16 half .. + 15 of every (row tile, tap, step s);
+//   * the weights of a wavefront's 32-row tile (at most 32 x 9 x 64 bytes) sit in its registers for the life of the
+//     workgroup: lane (row lane % 32, half lane / 32) holds bytes 32 s + 16 half .. + 15 of every (tap, step s);
 //   * v_mfma_i32_32x32x32_i8: B = 16 bytes of the pixel under tap (i, j), read from the patch at a per-lane base (computed
-//     once per workgroup) plus a compile-time offset, no address arithmetic in the loop; wavefront w owns the pixels
-//     32 TN w .. of the band and every row tile;
+//     once per workgroup) plus a compile-time offset, no address arithmetic in the loop; the four wavefronts stand side
+//     by side over the band's pixels (WM = 1) or two by two over row tiles and pixels (WM = 2, up to 64 channels);
 //   * the store is the int8 NHWC store of the implicit-GEMM kernels (write_tile_nhwc_s8: de-quantisation, bias, activation
 //     or quantised table, re-quantisation, transposition through LDS, 16-byte stores), so the results are the same bytes.
 // Arithmetic: device/x86/Conv/conv.c:961-973 (the input quantiser, here the producer's), :1024-1056 (int32 sums, then
