@@ -357,6 +357,11 @@ typedef struct {
 int onhip_maxpool_out_shape(const onhip_pool_desc_t *d, int32_t *oh, int32_t *ow);
 int onhip_maxpool_f32(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const float *x, float *y,
                       void *stream);
+/* The same on int8 NHWC activations (element (image, row, column, channel) at ((image * h + row) * w + column) * cp +
+ * channel, cp = c rounded up to 16; 16-byte aligned): y = the byte-wise maximum over the window.  Because the activation
+ * quantiser (device/x86/Conv/conv.c:961-973) is monotonic, this is what that quantiser makes of maxpool.c's fp32 result
+ * on the de-quantised input: a MaxPool between int8 convolutions needs no fp32 tensor.  No counterpart in the reference. */
+int onhip_maxpool_s8_nhwc(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const int8_t *x, int8_t *y, void *stream);
 
 /* y[n][c] = (sum of the plane in memory order) * (1.0f / (h*w)).  Replaces
  * device/x86/GlobalAveragePool/global_avgpool.c eval (:7-45). */
@@ -453,6 +458,9 @@ int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_
 int onhip_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_maxpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_s8` of libMaxPool_hip.so: slots and operand descriptors as for `eval` (NCHW shapes), the tensors int8 NHWC with
+ * channels padded to 16 (onhip_maxpool_s8_nhwc).  For the device-resident runtime, between int8 convolutions. */
+int onhip_maxpool_s8_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_global_avgpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Gelu (gelu.c:9), LayerNormalization (layer_normalization.c:10), Softmax (softmax.c:12), Transpose (transpose.c:13) */
 int onhip_gelu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);

@@ -108,7 +108,9 @@ int onrt_net_fused_ir_blocks(const onrt_net_t *net, int32_t *n);
  * int8 edges: the result of a dense int8 (W8A32) Conv that only dense int8 Convs with one and the same input_scale read
  * travels as int8 NHWC, quantised in the producer's store exactly as each consumer would have quantised the fp32 tensor
  * (device/x86/Conv/conv.c:961-973), through the Conv plugin's `eval_link`: a quarter of the bytes, no staging pass in the
- * consumers, the same results.  The reference's operators always exchange fp32 (conv.c:939-1067).  ONENEW_RT_FUSE=0
+ * consumers, the same results.  Likewise the int8 copy that the store of an int8 Conv with a folded Add leaves for the
+ * int8 readers of its fp32 result, and both operands of a MaxPool between int8 convolutions (pooled as bytes: the
+ * quantiser is monotonic).  The reference's operators always exchange fp32 (conv.c:939-1067).  ONENEW_RT_FUSE=0
  * keeps every operand fp32.  n: how many operands travel that way.
  */
 int onrt_net_quantised_links(const onrt_net_t *net, int32_t *n);

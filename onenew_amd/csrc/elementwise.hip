@@ -131,6 +131,45 @@ __global__ __launch_bounds__(256) void maxpool_kernel(PoolParams p, const float 
     y[o] = m;
 }
 
+// Max pooling on int8 NHWC activations (channels padded to 16): a thread takes 16 channels of one output pixel, one
+// 16-byte load per tap.  The quantiser of conv.c:961-973 never decreases with its argument, so the maximum of the quantised
+// values is the quantised maximum: what an int8 convolution reading the fp32 result of maxpool.c would make of it (the
+// -3276800 the reference starts from quantises to -128, below which no int8 lies).  cg: 16-byte groups per pixel.
+__device__ __forceinline__ unsigned max_s8x4(unsigned a, unsigned b) {
+    unsigned r = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int x = (int) (a << (24 - 8 * k)) >> 24, y = (int) (b << (24 - 8 * k)) >> 24;
+        r |= ((unsigned) (x > y ? x : y) & 0xffu) << (8 * k);
+    }
+    return r;
+}
+
+__global__ __launch_bounds__(256) void maxpool_nhwc_s8_kernel(PoolParams p, const uint4 *__restrict__ x, uint4 *__restrict__ y,
+                                                              long long total, int cg, Div31 div_cg) {
+    const long long o = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (o >= total) return;
+    const unsigned pix = ew_div((unsigned) o, div_cg);
+    const int g = (int) ((unsigned) o - pix * (unsigned) cg);
+    const unsigned t = ew_div(pix, p.div_ow);
+    const int ow = (int) (pix - t * (unsigned) p.OW);
+    const unsigned img = ew_div(t, p.div_oh);        // planes = images here
+    const int oh = (int) (t - img * (unsigned) p.OH);
+    const int ih0 = oh * p.sh - p.pad, iw0 = ow * p.sw - p.pad;
+    uint4 m = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);   // -128 in every byte
+    for (int i = 0; i < p.kh; ++i) {
+        const int ih = ih0 + i;
+        if ((unsigned) ih >= (unsigned) p.H) continue;
+        for (int j = 0; j < p.kw; ++j) {
+            const int iw = iw0 + j;
+            if ((unsigned) iw >= (unsigned) p.W) continue;
+            const uint4 v = x[((long long) (img * (unsigned) p.H + (unsigned) ih) * p.W + iw) * cg + g];
+            m.x = max_s8x4(m.x, v.x); m.y = max_s8x4(m.y, v.y); m.z = max_s8x4(m.z, v.z); m.w = max_s8x4(m.w, v.w);
+        }
+    }
+    y[o] = m;
+}
+
 // The pooling of a ResNet stem, 3x3 stride 2 padding 1 on rows of a multiple of four floats: a thread produces two
 // neighbouring outputs from one 16-byte load and one single float per input row (columns 4p-1 .. 4p+3 cover both
 // windows), instead of nine single loads per output.  The maximum does not depend on the order of its operands, and a
@@ -305,6 +344,29 @@ int onhip_maxpool_f32(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const 
         hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0,
                            reinterpret_cast<hipStream_t>(stream), p, x, y, total);
     }
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+int onhip_maxpool_s8_nhwc(const onhip_pool_desc_t *d, int32_t oh, int32_t ow, const int8_t *x, int8_t *y, void *stream) {
+    int32_t moh, mow;
+    int rc = onhip_maxpool_out_shape(d, &moh, &mow);
+    if (rc) return rc;
+    if (!x || !y) return set_error(ONHIP_ERR_ARG, "maxpool: null pointer");
+    if (oh < 1 || ow < 1 || oh > moh || ow > mow)
+        return set_error(ONHIP_ERR_ARG, "maxpool: output %dx%d does not fit (at most %dx%d)", oh, ow, moh, mow);
+    if (!aligned16(x) || !aligned16(y)) return set_error(ONHIP_ERR_ARG, "maxpool: int8 tensors must be 16-byte aligned");
+    const int cg = (d->c + 15) / 16;
+    PoolParams p;
+    p.planes = d->n; p.H = d->h; p.W = d->w; p.OH = oh; p.OW = ow;
+    p.kh = d->kh; p.kw = d->kw; p.sw = d->stride_w; p.sh = d->stride_h; p.pad = d->pad;
+    p.div_ow = make_div31((unsigned) ow);
+    p.div_oh = make_div31((unsigned) oh);
+    const long long total = (long long) d->n * oh * ow * cg;
+    if (total >= (1LL << 31) || (long long) d->n * d->h * d->w * cg >= (1LL << 31))
+        return set_error(ONHIP_ERR_ARG, "maxpool: tensors of 2^31 groups or more are not supported");
+    hipLaunchKernelGGL(maxpool_nhwc_s8_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       p, reinterpret_cast<const uint4 *>(x), reinterpret_cast<uint4 *>(y), total, cg, make_div31((unsigned) cg));
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }

@@ -762,7 +762,15 @@ static int relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER
     return finish_output(host_out, y, (size_t) n * 4, out_on_dev);
 }
 
+static int maxpool_eval_mode(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, bool s8);
 static int maxpool_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return maxpool_eval_mode(params, inputs, outputs, false);
+}
+static int maxpool_s8_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return maxpool_eval_mode(params, inputs, outputs, true);
+}
+// s8: the tensors are int8 NHWC with channels padded to 16
+static int maxpool_eval_mode(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, bool s8) {
     const MAX_POOL_CONFIG_S *cfg = reinterpret_cast<const MAX_POOL_CONFIG_S *>(params[0].addr);
     const OPERAND_S *it = reinterpret_cast<const OPERAND_S *>(params[1].addr);
     const OPERAND_S *ot = reinterpret_cast<const OPERAND_S *>(params[2].addr);
@@ -776,7 +784,9 @@ static int maxpool_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUF
     d.stride_w = (int32_t) cfg->strides[0]; d.stride_h = (int32_t) cfg->strides[1];
     d.pad = (int32_t) cfg->pads[0];
     const int32_t oh = ot->shapes[2], ow = ot->shapes[3];
-    const size_t in_bytes = (size_t) d.n * d.c * d.h * d.w * 4, out_bytes = (size_t) d.n * d.c * oh * ow * 4;
+    const size_t cp = ((size_t) d.c + 15) / 16 * 16;
+    const size_t in_bytes = s8 ? (size_t) d.n * d.h * d.w * cp : (size_t) d.n * d.c * d.h * d.w * 4;
+    const size_t out_bytes = s8 ? (size_t) d.n * oh * ow * cp : (size_t) d.n * d.c * oh * ow * 4;
     const void *x;
     int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
     if (rc) return rc;
@@ -787,7 +797,8 @@ static int maxpool_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUF
         rc = stage_buf(2, out_bytes, &y);
         if (rc) return rc;
     }
-    rc = onhip_maxpool_f32(&d, oh, ow, (const float *) x, (float *) y, g_stream);
+    if (s8) rc = onhip_maxpool_s8_nhwc(&d, oh, ow, (const int8_t *) x, (int8_t *) y, g_stream);
+    else rc = onhip_maxpool_f32(&d, oh, ow, (const float *) x, (float *) y, g_stream);
     if (rc) return rc;
     return finish_output(host_out, y, out_bytes, out_on_dev);
 }
@@ -1004,6 +1015,10 @@ int onhip_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S 
 
 int onhip_maxpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("MaxPool", maxpool_eval_locked, params, inputs, outputs);
+}
+
+int onhip_maxpool_s8_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("MaxPool (int8)", maxpool_s8_eval_locked, params, inputs, outputs);
 }
 
 int onhip_global_avgpool_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {

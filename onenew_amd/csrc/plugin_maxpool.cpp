@@ -6,3 +6,10 @@ extern "C" __attribute__((visibility("default"))) int eval(BUFFER_INFO_S *params
                                                            BUFFER_INFO_S *outputs) {
     return onhip_maxpool_eval(params, inputs, outputs);
 }
+
+// Not in the reference: the same operator on int8 NHWC tensors (channels padded to 16), between int8 convolutions whose
+// operands travel that way.  Slots and operand descriptors (NCHW shapes) as for `eval`.
+extern "C" __attribute__((visibility("default"))) int eval_s8(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                              BUFFER_INFO_S *outputs) {
+    return onhip_maxpool_s8_eval(params, inputs, outputs);
+}

@@ -173,6 +173,7 @@ struct onrt_net {
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
     onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr, conv_link = nullptr;
+    onenew_eval_fn maxpool_s8 = nullptr;   // optional entry point of the MaxPool plugin
     onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr, matmul_bias_add = nullptr;   // optional entry points of the MatMul plugin
     int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0, int8_links = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
@@ -540,6 +541,7 @@ int bind_plugins(onrt_net &net) {
             net.conv_block_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block_takes"));
             net.conv_link = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_link"));
         }
+        if (type == "MaxPool") net.maxpool_s8 = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_s8"));
         if (type == "MatMul") {
             net.matmul_attention = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_attention"));
             net.matmul_bias = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_bias"));
@@ -844,6 +846,45 @@ int link_int8_convs(onrt_net &net) {
         }
         net.tensors[name].as_s8 = true;
         ++net.int8_links;
+    }
+    // A MaxPool between int8 convolutions (the pooling behind a quantised stem): the quantiser is monotonic, so pooling the
+    // producer's int8 result gives the bytes the consumers would make of the pooled fp32 tensor; both operands travel
+    // as int8 and the MaxPool plugin's `eval_s8` runs.  Producer: a dense int8 Conv whose result only the MaxPool reads;
+    // readers of the MaxPool: dense int8 Convs with one input_scale.
+    for (int idx : net.order) {
+        Node &p = net.nodes[idx];
+        if (!net.maxpool_s8 || !dense_int8(p) || p.fuse != 0 || p.link.out_s8) continue;
+        const std::string name = result_of(p);
+        const int mi = sole_reader(net, name, "MaxPool");
+        if (mi < 0 || net.tensors[name].desc.not_need_buf) continue;
+        Node &mp = net.nodes[mi];
+        if (mp.in.size() != 1 || mp.out.size() != 1 || mp.in[0] != name) continue;
+        const std::string pooled = mp.out[0];
+        if (is_net_output(net, pooled) || net.tensors[pooled].desc.not_need_buf) continue;
+        const std::vector<int> readers = readers_of(net, pooled);
+        bool ok = !readers.empty();
+        float scale = 0.0f;
+        for (int ri : readers) {
+            const Node &c = net.nodes[ri];
+            const CONV_CONFIG_S *cc = dense_int8(c);
+            if (!cc || c.in[0] != pooled || !(cc->input_scale > 0.0f) || (scale != 0.0f && cc->input_scale != scale)) { ok = false; break; }
+            scale = cc->input_scale;
+        }
+        for (int oi : net.order)
+            if (net.nodes[oi].addend == pooled || net.nodes[oi].addend == name) ok = false;
+        if (!ok) continue;
+        p.link.out_s8 = 1;
+        p.link.out_scale = scale;
+        p.eval = net.conv_link;
+        mp.eval = net.maxpool_s8;
+        for (int ri : readers) {
+            Node &c = net.nodes[ri];
+            c.link.in_s8 = 1;
+            c.link_fuse = c.fuse;
+            c.eval = net.conv_link;
+        }
+        net.tensors[name].as_s8 = net.tensors[pooled].as_s8 = true;
+        net.int8_links += 2;
     }
     // The result of an int8 Conv with a folded Add (the output of a residual block) stays fp32, because the next block's
     // Add reads it; the int8 Convs among its readers get an int8 copy, written by the same store (outputs[1] of

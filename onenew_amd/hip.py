@@ -41,7 +41,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
            "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", "onhip_dw_project_supported", "onhip_dw_project_packed_weight_bytes", "onhip_dw_project_pack_weights", "onhip_dw_project_f32",
            "onhip_ir_block_supported", "onhip_ir_block_packed_weight_bytes", "onhip_ir_block_pack_weights", "onhip_ir_block_f32",
-           "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_global_avgpool_f32",
+           "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_maxpool_s8_nhwc", "onhip_maxpool_s8_eval", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
            "onhip_maxpool_eval", "onhip_global_avgpool_eval", "onhip_gelu_eval", "onhip_layernorm_eval",
@@ -80,6 +80,7 @@ def load():
     L.onhip_add_f32.argtypes = [vp, vp, vp, vp, vp]
     L.onhip_relu_f32.argtypes = [vp, vp, C.c_longlong, vp]
     L.onhip_maxpool_f32.argtypes = [vp, C.c_int32, C.c_int32, vp, vp, vp]
+    L.onhip_maxpool_s8_nhwc.argtypes = [vp, C.c_int32, C.c_int32, vp, vp, vp]
     L.onhip_global_avgpool_f32.argtypes = [C.c_int32] * 4 + [vp, vp, vp]
     L.onhip_gelu_lut_f32.argtypes = [vp, vp, vp, C.c_longlong, vp]
     L.onhip_layernorm_f32.argtypes = [C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp, vp]
@@ -220,6 +221,16 @@ def add_f32(large, small, relu=False, out=None):
     if out is None:
         out = torch.empty_like(large)
     _check(load().onhip_add_f32(C.byref(d), _ptr(large), _ptr(small), _ptr(out), _stream()), "onhip_add_f32")
+    return out
+
+
+def maxpool_s8_nhwc(d, xq, out=None):
+    """max pooling (PoolDesc d) on int8 NHWC activations [n, h, w, c rounded up to 16]"""
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        out = torch.empty((d.n, oh, ow, xq.shape[3]), dtype=torch.int8, device=xq.device)
+    _check(load().onhip_maxpool_s8_nhwc(C.byref(d), oh, ow, _ptr(xq), _ptr(out), _stream()), "onhip_maxpool_s8_nhwc")
     return out
 
 

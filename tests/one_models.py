@@ -162,6 +162,32 @@ def quantised_chain(n=1, hw=18, different_scales=False, extra_reader=False, tail
     return m.tobytes(), [_r("xqc", (n, 16, hw, hw))]
 
 
+def quantised_stem(n=1, hw=21):
+    """a quantised stem: dense int8 Conv (7x7 stride 2, Relu) -> MaxPool 3x3 stride 2 -> two dense int8 convolutions with
+    one input_scale; the operands either side of the MaxPool can travel as int8"""
+    from oracle import oracle
+    m = onefile.OneModel()
+    m.input("x", (n, 3, hw, hw))
+
+    def q(tag, shape, scale):
+        w = _r(tag + "w", shape, scale)
+        b = _r(tag + "b", (shape[0],), 0.2)
+        return oracle.quant_weight_bias(w, b)
+
+    w8, b32, aux = q("s0", (24, 3, 7, 7), 0.1)
+    m.conv("stem", "x", w8, b32, "stem_out", stride=2, pad=3, act=abi.RELU, quant=(aux, 0.02))
+    h1 = (hw + 6 - 7) // 2 + 1
+    m.maxpool("pool", "stem_out", "pool_out", 3, 2, 1)
+    h2 = (h1 + 2 - 3) // 2 + 1
+    w8, b32, aux = q("s1", (32, 24, 1, 1), 0.2)
+    m.conv("c1", "pool_out", w8, b32, "out_a", act=abi.RELU, quant=(aux, 0.03))
+    m.output("out_a", (n, 32, h2, h2))
+    w8, b32, aux = q("s2", (16, 24, 3, 3), 0.1)
+    m.conv("c2", "pool_out", w8, b32, "out_b", pad=1, act=abi.NOT_ACT, quant=(aux, 0.03))
+    m.output("out_b", (n, 16, h2, h2))
+    return m.tobytes(), [_r("xstem", (n, 3, hw, hw))]
+
+
 def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output=False, split_heads=()):
     """q, k, v as three inputs [batch, heads, tokens, head_dim]: Transpose of k, MatMul, Softmax, MatMul, the pattern the
     runtime runs as one attention call (unless the scores are also a net output).  split_heads: which of "q", "k", "v"
@@ -199,7 +225,7 @@ def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output
     return m.tobytes(), [_r(n + str(tokens), shape, 0.5) for n in ("q", "k", "v")]
 
 
-MODELS = {"quantised_block": quantised_block, "quantised_chain": quantised_chain, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
+MODELS = {"quantised_block": quantised_block, "quantised_chain": quantised_chain, "quantised_stem": quantised_stem, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
 
 
 def unfused_activations(optimised=False):

@@ -1424,3 +1424,20 @@ def test_plugin_eval_link_host_buffers(torch_dev, oracle):
     assert np.array_equal(link(xq, in_s8=True), y)
     assert np.array_equal(link(xq, in_s8=True, addend=skip), oracle.add_f32(y, skip))
     assert np.array_equal(link(x, addend=skip, relu_after=True), oracle.relu_f32(oracle.add_f32(y, skip)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 24, 11, 11, 3, 2, 1), (1, 64, 56, 56, 3, 2, 1), (3, 5, 9, 14, 2, 2, 0), (1, 16, 7, 7, 3, 1, 1), (2, 40, 6, 6, 5, 1, 2)])
+def test_maxpool_on_int8_nhwc_is_the_quantised_fp32_maxpool(shape, torch_dev):
+    """onhip_maxpool_s8_nhwc on the quantised tensor equals the quantiser applied to onhip_maxpool_f32's result (the
+    quantiser is monotonic), padding channels stay zero... except where a window holds no input at all"""
+    torch = torch_dev
+    n, c, h, w, k, stride, pad = shape
+    x = cases.datagen.normal(cases.datagen.seed_for("mp8", str(shape)), (n, c, h, w), 0.0, 1.5)
+    d = abi.PoolDesc(n=n, c=c, h=h, w=w, kh=k, kw=k, stride_w=stride, stride_h=stride, pad=pad)
+    scale = 0.031
+    y = hip.maxpool_f32(d, dev(torch, x))
+    want = hip.quantize_nhwc_s8(y, scale)
+    got = hip.maxpool_s8_nhwc(d, hip.quantize_nhwc_s8(dev(torch, x), scale))
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy()[..., :c], want.cpu().numpy()[..., :c])

@@ -48,7 +48,7 @@ def test_model_outputs_match_oracle(name, torch_dev, monkeypatch):
     for (oname, _), got in zip(net.outputs, outs):
         assert got.shape == ref[oname].shape
         assert _close(got, ref[oname], 5e-4), oname                          # up to five MFMA operators deep, 1e-4 each
-        if name in ("quantised_block", "quantised_chain"):
+        if name in ("quantised_block", "quantised_chain", "quantised_stem"):
             assert np.array_equal(got, ref[oname])                           # integer accumulation: the chain is exact
     # every intermediate operand sits in device memory and holds what the oracle computed at that point
     for op_type, cfg in m["nodes"]:
@@ -737,4 +737,18 @@ def test_int8_convolutions_exchange_int8_operands(torch_dev, monkeypatch):
         ref = one_model.run(data, ins, keep_all=True)
         for (oname, _), got in zip(net.outputs, net.run(*ins)):
             assert np.array_equal(got, ref[oname]), (kw, oname)
+        net.close()
+
+
+@pytest.mark.gpu
+def test_maxpool_between_int8_convolutions_runs_on_int8(torch_dev):
+    """Conv (int8) -> MaxPool -> two int8 convolutions with one input_scale: both operands around the MaxPool travel as
+    int8 NHWC and the pooling runs on bytes; the outputs equal the oracle's fp32 evaluation bit for bit"""
+    for n, hw in ((2, 21), (1, 40)):
+        data, ins = one_models.quantised_stem(n=n, hw=hw)
+        net = rt.Net(data)
+        assert net.int8_links() == 2
+        ref = one_model.run(data, ins, keep_all=True)
+        for (oname, _), got in zip(net.outputs, net.run(*ins)):
+            assert np.array_equal(got, ref[oname]), oname
         net.close()
