@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void i8patch_kernel(const IgemmParams p, co
 // one MFMA step: K index 32 k + 16 half of step k is tap (32 k + 16 half) / CB, byte (32 k + 16 half) % CB of the pixel,
 // and the packed weights ([m][tap][CB]) are read at that same index.  A persistent workgroup walks blocks of BN output
 // pixels of the whole batch; the next block's loads are in flight while this one is stored.
-template <int CB, int TAPS, int WM, int TM, int TN, int OCC>
+template <int CB, int TAPS, int KW, int WM, int TM, int TN, int OCC>
 __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p, const int blocks) {
     constexpr int NK = (TAPS * CB + 31) / 32, WN = 4 / WM, BM = 32 * TM * WM, BN = 32 * TN * WN;
     constexpr int STAGE = BN * (BM + 16);
@@ -234,15 +234,21 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
         if (tid == 0) stage[STAGE - 1] = 0;   // the store's "below the table" entry, in padding that nothing else touches
     }
 
-    // where step k's bytes lie relative to the window's first pixel: the same for every block
-    int tap_i[NK], tap_j[NK], tap_byte[NK];
-#pragma unroll
-    for (int k = 0; k < NK; ++k) {
+    // where step k's bytes lie relative to the window's first pixel: the same for every block.  Filters of many taps
+    // (MANY: a 7x7 first layer, 25 steps) work the three numbers out per load instead of holding them, and load a block's
+    // pixels when its turn comes rather than a block ahead: the registers go to the weights.
+    constexpr bool MANY = NK > 12;
+    int tap_i[MANY ? 1 : NK], tap_j[MANY ? 1 : NK], tap_byte[MANY ? 1 : NK];
+    auto tap_of = [&](int k, int &ti, int &tj, int &tb) __attribute__((always_inline)) {
         const int kk = 32 * k + 16 * lh, tap = kk / CB;
-        const int ti = TAPS == 9 ? (tap * 11) >> 5 : 0;    // tap / 3 for tap < 10
-        tap_i[k] = tap < TAPS ? ti : 1 << 28;              // past the last tap: outside any image
-        tap_j[k] = tap - (TAPS == 9 ? 3 : 1) * ti;
-        tap_byte[k] = kk % CB;
+        const int i = tap / KW;
+        ti = tap < TAPS ? i : 1 << 28;              // past the last tap: outside any image
+        tj = tap - KW * i;
+        tb = kk % CB;
+    };
+    if constexpr (!MANY) {
+#pragma unroll
+        for (int k = 0; k < NK; ++k) tap_of(k, tap_i[k], tap_j[k], tap_byte[k]);
     }
     const rsrc_t rx = make_rsrc(p.B, (unsigned) p.b_slice_bytes);
     uint4 bx[TN][NK];
@@ -257,17 +263,21 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
             const int iy0 = live ? oy * p.sh - p.pt : -(1 << 29), ix0 = ox * p.sw - p.pl;
 #pragma unroll
             for (int k = 0; k < NK; ++k) {
-                const int iy = iy0 + tap_i[k], ix = ix0 + tap_j[k];
+                int ti, tj, tb;
+                if constexpr (MANY) tap_of(k, ti, tj, tb);
+                else { ti = tap_i[k]; tj = tap_j[k]; tb = tap_byte[k]; }
+                const int iy = iy0 + ti, ix = ix0 + tj;
                 const bool ok = (unsigned) iy < (unsigned) p.H && (unsigned) ix < (unsigned) p.W;
-                bx[b][k] = buf_load_b128(rx, ok ? (unsigned) (((img * p.H + iy) * p.W + ix) * CB + tap_byte[k]) : OOB, 0);
+                bx[b][k] = buf_load_b128(rx, ok ? (unsigned) (((img * p.H + iy) * p.W + ix) * CB + tb) : OOB, 0);
             }
         }
     };
 
     const ItemWalk walk = xcd_walk(blocks);
     int blk = walk.first;
-    if (blk < walk.end) issue(blk);
+    if (!MANY && blk < walk.end) issue(blk);
     for (; blk < walk.end; blk += walk.step) {
+        if constexpr (MANY) issue(blk);
         i32x16 acc[TM][TN];
 #pragma unroll
         for (int a = 0; a < TM; ++a)
@@ -281,7 +291,7 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
                     acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[a][k], bv, acc[a][b], 0, 0, 0);
                 }
             }
-        if (blk + walk.step < walk.end) issue(blk + walk.step);   // uniform
+        if (!MANY && blk + walk.step < walk.end) issue(blk + walk.step);   // uniform
         __syncthreads();   // the previous block's store has left the staging area (and, the first time, the table is there)
         const int n0 = blk * BN, m_wave = 32 * TM * wm, n_wave = n0 + 32 * TN * wn;
         switch (p.ep.act) {
@@ -297,38 +307,40 @@ __global__ __launch_bounds__(256, OCC) void i8direct_kernel(const IgemmParams p,
 }
 
 // the int8 NHWC chain form of a 3x3 convolution of any stride and padding with 16 or 32 bytes per input pixel and at most
-// 64 output channels; of a 1x1 convolution with 64, 96 or 128 bytes per pixel and at most 64 output channels (with two
+// 64 output channels; of a 7x7 convolution with 16 bytes per pixel and at most 64; of a 1x1 convolution with 64, 96 or 128 bytes per pixel and at most 64 output channels (with two
 // row tiles per wavefront, up to 128 channels, it was measured level with the implicit-GEMM kernels or behind them)
 bool i8direct_ok(const IgemmParams &p) {
     if (!p.out_s8 || p.out_mode != OUT_PLAIN || p.c_stride_m != 1 || p.acc_out) return false;
     if (p.lda != p.khkw * p.pix_stride || p.b_slice_bytes >= (1LL << 31) - 64) return false;
     if (p.kh == 3 && p.kw == 3) return p.M <= 64 && (p.pix_stride == 16 || p.pix_stride == 32);
+    if (p.kh == 7 && p.kw == 7) return p.M <= 64 && p.pix_stride == 16;   // a first layer: up to 16 input channels
     if (p.kh == 1 && p.kw == 1) return p.M <= 64 && (p.pix_stride == 64 || p.pix_stride == 96 || p.pix_stride == 128);
     return false;
 }
 
-template <int CB, int TAPS, int WM, int TM, int TN, int OCC>
+template <int CB, int TAPS, int KW, int WM, int TM, int TN, int OCC>
 static int i8direct_launch_one(IgemmParams p, hipStream_t stream) {
     constexpr int BN = 32 * TN * (4 / WM);
     const int blocks = (p.N + BN - 1) / BN;
     p.div_ohw = make_div31((unsigned) p.OHW);
     p.div_ow = make_div31((unsigned) p.OW);
     const int grid = blocks < 256 * OCC ? (blocks + 7) / 8 * 8 : 256 * OCC;   // OCC workgroups per compute unit; a multiple of 8 (xcd_walk)
-    hipLaunchKernelGGL((i8direct_kernel<CB, TAPS, WM, TM, TN, OCC>), dim3((unsigned) grid), dim3(256), 0, stream, p, blocks);
+    hipLaunchKernelGGL((i8direct_kernel<CB, TAPS, KW, WM, TM, TN, OCC>), dim3((unsigned) grid), dim3(256), 0, stream, p, blocks);
     ONHIP_CHECK_HIP(hipGetLastError());
     return ONHIP_OK;
 }
 
 int i8direct_launch(const IgemmParams &p, hipStream_t stream) {
+    if (p.kh == 7) return p.M <= 32 ? i8direct_launch_one<16, 49, 7, 1, 1, 1, 2>(p, stream) : i8direct_launch_one<16, 49, 7, 2, 1, 1, 2>(p, stream);
     if (p.kh == 1) {
-        if (p.pix_stride == 64) return i8direct_launch_one<64, 1, 2, 1, 2, 2>(p, stream);
-        if (p.pix_stride == 96) return i8direct_launch_one<96, 1, 2, 1, 2, 2>(p, stream);
-        return i8direct_launch_one<128, 1, 2, 1, 2, 2>(p, stream);
+        if (p.pix_stride == 64) return i8direct_launch_one<64, 1, 1, 2, 1, 2, 2>(p, stream);
+        if (p.pix_stride == 96) return i8direct_launch_one<96, 1, 1, 2, 1, 2, 2>(p, stream);
+        return i8direct_launch_one<128, 1, 1, 2, 1, 2, 2>(p, stream);
     }
     // measured on a first layer (3 -> 32 channels, stride 2) and the layer after it (32 -> 64): three workgroups per
     // compute unit help the former, whose time is the store's arithmetic; smaller or larger blocks help neither
-    if (p.pix_stride == 16) return p.M <= 32 ? i8direct_launch_one<16, 9, 1, 1, 2, 3>(p, stream) : i8direct_launch_one<16, 9, 2, 1, 2, 2>(p, stream);
-    return p.M <= 32 ? i8direct_launch_one<32, 9, 1, 1, 2, 2>(p, stream) : i8direct_launch_one<32, 9, 2, 1, 2, 2>(p, stream);
+    if (p.pix_stride == 16) return p.M <= 32 ? i8direct_launch_one<16, 9, 3, 1, 1, 2, 3>(p, stream) : i8direct_launch_one<16, 9, 3, 2, 1, 2, 2>(p, stream);
+    return p.M <= 32 ? i8direct_launch_one<32, 9, 3, 1, 1, 2, 2>(p, stream) : i8direct_launch_one<32, 9, 3, 2, 1, 2, 2>(p, stream);
 }
 
 static int i8patch_rows(const IgemmParams &p, int *big);

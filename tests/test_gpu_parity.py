@@ -1288,6 +1288,8 @@ def test_tune_cache_file_is_validated_and_rewritten(tmp_path):
     # 32 bytes per pixel: stride 1 with pads 1 (the rows of a band kept in LDS), other strides and pads (loaded per tap)
     (2, 32, 20, 20, 32, 3, 1, 1), (1, 24, 13, 37, 16, 3, 1, 1), (2, 32, 16, 160, 32, 3, 1, 1), (1, 32, 7, 256, 24, 3, 1, 1), (3, 20, 5, 6, 64, 3, 1, 1),
     (2, 32, 21, 23, 64, 3, 2, 1), (1, 32, 18, 18, 48, 3, 1, 0), (2, 17, 15, 15, 32, 3, 2, 1), (1, 32, 40, 80, 64, 3, 1, 1),
+    # 7x7 first layers (49 taps of 16 bytes, 25 MFMA steps), one and two row tiles
+    (2, 3, 30, 30, 64, 7, 2, 3), (1, 3, 33, 47, 24, 7, 2, 3), (1, 8, 20, 20, 32, 7, 1, 3), (2, 16, 9, 9, 40, 7, 2, 0),
     # rows too long for a band in LDS (loaded per tap instead); fewer blocks than XCDs; one pixel
     (1, 32, 4, 300, 32, 3, 1, 1), (3, 32, 3, 3, 16, 3, 1, 1), (1, 16, 1, 1, 32, 3, 1, 1),
     # 64 bytes per pixel, stride 1, pads 1
@@ -1297,8 +1299,8 @@ def test_tune_cache_file_is_validated_and_rewritten(tmp_path):
     (3, 128, 7, 11, 33, 1, 1, 0), (1, 128, 24, 24, 64, 1, 1, 1), (2, 100, 5, 5, 16, 1, 1, 0), (1, 128, 12, 12, 80, 1, 1, 0)])
 @pytest.mark.parametrize("act", [abi.SILU, abi.RELU, abi.NOT_ACT])
 def test_conv_int8_chain_3x3_with_few_channels(shape, act, torch_dev, oracle, monkeypatch):
-    """3x3 convolutions of the int8 NHWC chain form with at most 64 input channels and 64 output channels, and 1x1
-    convolutions with at most 128 and 64: whichever kernel
+    """3x3 convolutions of the int8 NHWC chain form with at most 64 input channels and 64 output channels, 7x7 first
+    layers, and 1x1 convolutions with at most 128 and 64: whichever kernel
     takes them (input rows of a band in LDS, or windows loaded per tap, or the implicit-GEMM kernels), the bytes are the
     oracle's, and the same with the LDS kernel given every shape it can take and with those two kernels switched off; ragged sizes, pixels past the last block, pads 0 to 2"""
     torch = torch_dev
