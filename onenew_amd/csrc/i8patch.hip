@@ -4,9 +4,10 @@
 // kernels read every input pixel nine times, once per filter tap, through L2 into LDS, and pay a tile's whole set-up and
 // store for two or three K stages; with so few channels that, not the matrix cores, sets their time.  Here
 //
-//   * a persistent workgroup walks bands of whole output rows (up to 256 pixels) of the batch; the band's input rows plus
-//     halo, (rows + 2) x (w + 2) pixels with zeros outside the image, are loaded ONCE into an LDS patch (NHWC rows are
-//     contiguous: plain 16-byte loads), the next band's into registers while this one is multiplied;
+//   * a persistent workgroup walks bands of whole output rows of the batch; the band's input rows plus halo,
+//     (rows + 2) x (w + 2) pixels with zeros outside the image, are loaded ONCE into an LDS patch (NHWC rows are
+//     contiguous: plain 16-byte loads), the next band's into registers while this one is multiplied and stored, a block
+//     of 128 or 256 pixels per pass (rows and block chosen so that the last block of a band is as full as possible);
 //   * the weights of a wavefront's 32-row tile (at most 32 x 9 x 64 bytes) sit in its registers for the life of the
 //     workgroup: lane (row lane % 32, half lane / 32) holds bytes 32 s + 16 half .. + 15 of every (tap, step s);
 //   * v_mfma_i32_32x32x32_i8: B = 16 bytes of the pixel under tap (i, j), read from the patch at a per-lane base (computed
@@ -27,6 +28,7 @@ namespace onhip {
 constexpr int P8_SLOTS = 8;   // 16-byte patch loads per thread, at most
 
 struct PatchGeom {
+    int passes;          // blocks of BN pixels a band is multiplied and stored in
     int rows;            // output rows of a band
     int bands;           // bands per image
     int total;           // bands of the batch
@@ -110,17 +112,6 @@ __global__ __launch_bounds__(256, 2) void i8patch_kernel(const IgemmParams p, co
         g_off[i] = (r * W + pc - 1) * CB + part * 16;              // bytes from the start of the input row above the band
         l_off[i] = live ? ff * 16 : -1;
     }
-    // this lane's pixels in the MFMAs: byte offset in the patch of the window's top-left pixel, per pixel tile
-    int boff[TN];
-    bool tile_on[TN];
-#pragma unroll
-    for (int b = 0; b < TN; ++b) {
-        const int q0 = 32 * (TN * wn + b);
-        tile_on[b] = q0 < band_px;                                // uniform
-        const int q = q0 + li < band_px ? q0 + li : 0;
-        const int r = (int) div31((unsigned) q, g.div_ow), c = q - r * W;
-        boff[b] = (r * g.prow_px + c) * CB + 16 * lh;
-    }
     const int row_bytes = g.prow_px * CB;
 
     const rsrc_t rx = make_rsrc(p.B, (unsigned) p.b_slice_bytes);
@@ -148,42 +139,57 @@ __global__ __launch_bounds__(256, 2) void i8patch_kernel(const IgemmParams p, co
         __syncthreads();
         if (band + walk.step < walk.end) issue(band + walk.step);   // uniform
 
-        i32x16 acc[1][TN];
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[0][b][r] = 0;
-#pragma unroll
-        for (int b = 0; b < TN; ++b) {
-            if (!tile_on[b]) continue;
-#pragma unroll
-            for (int i = 0; i < 3; ++i) {
-                const unsigned char *prow_base = patch + boff[b] + i * row_bytes;
-                i32x4 bv[3][S];
-#pragma unroll
-                for (int j = 0; j < 3; ++j)
-#pragma unroll
-                    for (int s = 0; s < S; ++s) bv[j][s] = *reinterpret_cast<const i32x4 *>(prow_base + j * CB + 32 * s);
-#pragma unroll
-                for (int j = 0; j < 3; ++j)
-#pragma unroll
-                    for (int s = 0; s < S; ++s)
-                        acc[0][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[3 * i + j][s], bv[j][s], acc[0][b], 0, 0, 0);
-            }
-        }
-
         const int img = band / g.bands, oy0 = (band - img * g.bands) * g.rows;
-        const int n0 = (img * H + oy0) * W;
-        ps.N = n0 + min(g.rows, H - oy0) * W;
-        const int m_wave = 32 * wm, n_wave = n0 + 32 * TN * wn;
-        switch (p.ep.act) {
-            case NOT_ACT:
-            case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            case SILU:
-            case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
-            default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+        const int n_band = (img * H + oy0) * W;
+        ps.N = n_band + min(g.rows, H - oy0) * W;
+        for (int pass = 0; pass < g.passes; ++pass) {
+            if (n_band + pass * BN >= ps.N) break;   // uniform: a ragged last band ends early
+            if (pass > 0) __syncthreads();           // the previous pass's store has left the staging area
+            // this lane's pixels in the MFMAs: byte offset in the patch of the window's top-left pixel, per pixel tile
+            int boff[TN];
+            bool tile_on[TN];
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                const int q0 = pass * BN + 32 * (TN * wn + b);
+                tile_on[b] = q0 < band_px;                                // uniform
+                const int q = q0 + li < band_px ? q0 + li : 0;
+                const int r = (int) div31((unsigned) q, g.div_ow), c = q - r * W;
+                boff[b] = (r * g.prow_px + c) * CB + 16 * lh;
+            }
+            i32x16 acc[1][TN];
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[0][b][r] = 0;
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                if (!tile_on[b]) continue;
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    const unsigned char *prow_base = patch + boff[b] + i * row_bytes;
+                    i32x4 bv[3][S];
+#pragma unroll
+                    for (int j = 0; j < 3; ++j)
+#pragma unroll
+                        for (int s = 0; s < S; ++s) bv[j][s] = *reinterpret_cast<const i32x4 *>(prow_base + j * CB + 32 * s);
+#pragma unroll
+                    for (int j = 0; j < 3; ++j)
+#pragma unroll
+                        for (int s = 0; s < S; ++s)
+                            acc[0][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[3 * i + j][s], bv[j][s], acc[0][b], 0, 0, 0);
+                }
+            }
+            const int n0 = n_band + pass * BN;
+            const int m_wave = 32 * wm, n_wave = n0 + 32 * TN * wn;
+            switch (p.ep.act) {
+                case NOT_ACT:
+                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+                case SILU:
+                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, 1, TN, true>(ps, acc, stage, 0, n0, m_wave, n_wave, li, lh, tid, rows, true); break;
+            }
         }
     }
 }
@@ -354,7 +360,7 @@ bool i8patch_ok(const IgemmParams &p, bool any_shape) {
     if (!p.out_s8 || p.out_mode != OUT_PLAIN || p.c_stride_m != 1 || p.acc_out) return false;
     if (p.kh != 3 || p.kw != 3 || p.sh != 1 || p.sw != 1 || p.pt != 1 || p.pl != 1) return false;
     if (p.pix_stride != 32 && p.pix_stride != 64) return false;
-    if (p.M > 64 || p.OW != p.W || p.OHW != p.HW || p.W > 256 || p.W < 4) return false;
+    if (p.M > 64 || p.OW != p.W || p.OHW != p.HW || p.W < 4) return false;
     if (p.lda != 9 * p.pix_stride) return false;
     int big = 0;
     return i8patch_rows(p, &big) > 0;
@@ -378,20 +384,23 @@ static int i8patch_launch_one(const IgemmParams &p, PatchGeom g, hipStream_t str
     return ONHIP_OK;
 }
 
-// whole rows per band: 128 or 256 pixels' worth, whichever fills its 32-pixel tiles better, within the patch loads a thread
-// has registers for and the LDS two workgroups share; 0: none fits
+// whole rows per band and the block (128 or 256 pixels) the band is multiplied and stored in, pass after pass: the pair
+// whose last block is fullest (a store costs the same for an empty pixel), the larger block unless it is 7 % emptier
+// (measured: three rows of 160 pixels in two blocks of 256 beat four rows in five blocks of 128, 22.9 against 24.3 us),
+// more rows per band (fewer halo rows) between equals; within the patch loads a thread has registers for and the LDS two workgroups share.  0: no row fits
 static int i8patch_rows(const IgemmParams &p, int *big) {
     const int W = p.W, H = p.H, cb = p.pix_stride, bm = p.M > 32 ? 64 : 32;
     int best_rows = 0;
-    double best_fill = 0.0;
+    double best = 0.0;
     for (int bn = 128; bn <= 256; bn += 128) {
-        int rows = bn / W;
-        rows = rows > H ? H : rows;
-        if (rows < 1) continue;
-        const long long vecs = (long long) (rows + 2) * (W + 2) * cb / 16;
-        if (vecs > 256LL * P8_SLOTS || (long long) bn * (bm + 16) + 8192 + 2 * bm * 4 + vecs * 16 > 80 * 1024) continue;
-        const double fill = (double) rows * W / bn;
-        if (fill > best_fill + 0.05) { best_fill = fill; best_rows = rows; *big = bn == 256; }
+        if (bn == 256 && cb == 64 && bm == 64) continue;   // four pixel tiles per wavefront and 72 registers of weights do not fit
+        for (int rows = 1; rows <= H && rows <= 32; ++rows) {
+            const long long vecs = (long long) (rows + 2) * (W + 2) * cb / 16;
+            if (vecs > 256LL * P8_SLOTS || (long long) bn * (bm + 16) + 8192 + 2 * bm * 4 + vecs * 16 > 80 * 1024) break;
+            const int passes = (rows * W + bn - 1) / bn;
+            const double score = (double) rows * W / ((double) passes * bn) + 0.001 * rows + (bn == 256 ? 0.07 : 0.0);
+            if (score > best) { best = score; best_rows = rows; *big = bn == 256; }
+        }
     }
     return best_rows;
 }
@@ -403,6 +412,7 @@ int i8patch_launch(const IgemmParams &p, hipStream_t stream) {
     int big = 0;
     g.rows = i8patch_rows(p, &big);
     if (!g.rows) return set_error(ONHIP_ERR_ARG, "int8 patch kernel: rows of %d pixels do not fit", W);
+    g.passes = (g.rows * W + (big ? 256 : 128) - 1) / (big ? 256 : 128);
     g.bands = (H + g.rows - 1) / g.rows;
     g.total = images * g.bands;
     g.prow_px = W + 2;
@@ -416,7 +426,7 @@ int i8patch_launch(const IgemmParams &p, hipStream_t stream) {
         return big ? i8patch_launch_one<64, 1, 2>(p, g, stream) : i8patch_launch_one<64, 1, 1>(p, g, stream);
     }
     if (cb == 32) return big ? i8patch_launch_one<32, 2, 4>(p, g, stream) : i8patch_launch_one<32, 2, 2>(p, g, stream);
-    return big ? i8patch_launch_one<64, 2, 4>(p, g, stream) : i8patch_launch_one<64, 2, 2>(p, g, stream);
+    return i8patch_launch_one<64, 2, 2>(p, g, stream);
 }
 
 }  // namespace onhip
