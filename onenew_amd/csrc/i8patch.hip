@@ -354,16 +354,21 @@ static int i8patch_rows(const IgemmParams &p, int *big);
 // the problems this kernel takes: the int8 NHWC chain form of a 3x3 convolution, stride 1, pads 1, 32 or 64 bytes per
 // input pixel, at most 64 output channels
 bool i8patch_ok(const IgemmParams &p, bool any_shape) {
-    // measured: ahead of the implicit-GEMM kernels with 32 bytes per pixel and one row tile, behind them (by a tenth) with
-    // 64 bytes per pixel and two
-    if (!any_shape && (p.pix_stride != 32 || p.M > 32)) return false;
     if (!p.out_s8 || p.out_mode != OUT_PLAIN || p.c_stride_m != 1 || p.acc_out) return false;
     if (p.kh != 3 || p.kw != 3 || p.sh != 1 || p.sw != 1 || p.pt != 1 || p.pl != 1) return false;
     if (p.pix_stride != 32 && p.pix_stride != 64) return false;
     if (p.M > 64 || p.OW != p.W || p.OHW != p.HW || p.W < 4) return false;
     if (p.lda != 9 * p.pix_stride) return false;
     int big = 0;
-    return i8patch_rows(p, &big) > 0;
+    const int rows = i8patch_rows(p, &big);
+    if (rows < 1) return false;
+    if (any_shape) return true;
+    // measured against the implicit-GEMM kernels (batch 16): ahead with 32 bytes per pixel and one row tile (160 x 160:
+    // 22.9 against 36.3 us) and with 64 bytes and two (80 x 80: 16.0 against 17.0), the other two combinations not
+    // measured; behind wherever the batch has fewer bands than the chip has compute units (40 x 40: 16 against 9 us)
+    const bool measured = (p.pix_stride == 32 && p.M <= 32) || (p.pix_stride == 64 && p.M > 32);
+    const long long bands = (long long) (p.N / p.OHW) * ((p.H + rows - 1) / rows);
+    return measured && bands >= 256;
 }
 
 template <int CB, int WM, int TN>
