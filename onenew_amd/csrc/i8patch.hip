@@ -54,7 +54,7 @@ __device__ __forceinline__ ItemWalk xcd_walk(int total) {
 // WM = 1: the four wavefronts side by side over the pixels (up to 32 output channels); WM = 2: two rows of two (up to 64),
 // so a wavefront holds the weights of one 32-row tile only.  TN: 32-pixel tiles per wavefront.
 template <int CB, int WM, int TN>
-__global__ __launch_bounds__(256, 2) void i8patch_kernel(const IgemmParams p, const PatchGeom g) {
+__global__ __launch_bounds__(256, (CB == 32 && TN == 1 ? 3 : 2)) void i8patch_kernel(const IgemmParams p, const PatchGeom g) {
     constexpr int S = CB / 32, PARTS = CB / 16, WN = 4 / WM, BM = 32 * WM, BN = 32 * TN * WN;
     constexpr int STAGE = BN * (BM + 16);
     extern __shared__ __attribute__((aligned(16))) unsigned char p8_lds[];
@@ -382,7 +382,7 @@ static int i8patch_launch_one(const IgemmParams &p, PatchGeom g, hipStream_t str
                                             80 * 1024));
         allowed.store(80 * 1024);
     }
-    int grid = 512;   // two workgroups per compute unit; a multiple of 8 (xcd_walk)
+    int grid = CB == 32 && TN == 1 ? 768 : 512;   // three or two workgroups per compute unit; a multiple of 8 (xcd_walk)
     grid = grid > g.total ? (g.total + 7) / 8 * 8 : grid;
     hipLaunchKernelGGL((i8patch_kernel<CB, WM, TN>), dim3((unsigned) grid), dim3(256), lds, stream, p, g);
     ONHIP_CHECK_HIP(hipGetLastError());
@@ -391,8 +391,10 @@ static int i8patch_launch_one(const IgemmParams &p, PatchGeom g, hipStream_t str
 
 // whole rows per band and the block (128 or 256 pixels) the band is multiplied and stored in, pass after pass: the pair
 // whose last block is fullest (a store costs the same for an empty pixel), the larger block unless it is 7 % emptier
-// (measured: three rows of 160 pixels in two blocks of 256 beat four rows in five blocks of 128, 22.9 against 24.3 us),
-// more rows per band (fewer halo rows) between equals; within the patch loads a thread has registers for and the LDS two workgroups share.  0: no row fits
+// (measured: three rows of 160 pixels in two blocks of 256 beat four rows in five blocks of 128, 22.9 against 24.3 us,
+// with two workgroups per compute unit each) -- except with 32 bytes per pixel and one row tile, where the 128-pixel
+// variant fits three workgroups per compute unit and wins (21.7 us) --, more rows per band (fewer halo rows) between
+// equals; within the patch loads a thread has registers for and the LDS two workgroups share.  0: no row fits
 static int i8patch_rows(const IgemmParams &p, int *big) {
     const int W = p.W, H = p.H, cb = p.pix_stride, bm = p.M > 32 ? 64 : 32;
     int best_rows = 0;
@@ -403,7 +405,7 @@ static int i8patch_rows(const IgemmParams &p, int *big) {
             const long long vecs = (long long) (rows + 2) * (W + 2) * cb / 16;
             if (vecs > 256LL * P8_SLOTS || (long long) bn * (bm + 16) + 8192 + 2 * bm * 4 + vecs * 16 > 80 * 1024) break;
             const int passes = (rows * W + bn - 1) / bn;
-            const double score = (double) rows * W / ((double) passes * bn) + 0.001 * rows + (bn == 256 ? 0.07 : 0.0);
+            const double score = (double) rows * W / ((double) passes * bn) + 0.001 * rows + (bn == 256 && !(cb == 32 && bm == 32) ? 0.07 : 0.0);
             if (score > best) { best = score; best_rows = rows; *big = bn == 256; }
         }
     }
