@@ -97,6 +97,10 @@ long long onhip_split_tail_launches(void);
 /* Diagnostic, no counterpart in the reference: how many int8 launches so far ran the kernel that loads its operand tiles
  * from global memory straight into LDS (NHWC int8 activations with a multiple of 64 padded channels). */
 long long onhip_direct_lds_launches(void);
+/* Diagnostic, no counterpart in the reference: how many launches of onhip_conv2d_f32_noalloc so far cut K into slices and
+ * therefore put their partial sums into the library's built-in scratch array (a call the cost model gives a single
+ * slice never touches the array). */
+long long onhip_noalloc_scratch_launches(void);
 /* The model-wide GEMM tile of a .one file: BLOCK_INFO_S.cuda_gemm_tile_{m,n} (common/nn_common.h:28-39), which the
  * reference's tuner fills for its x86 kernels (tools/optimize/auto_tuning.hpp:9-75) and its converter defaults to
  * 16 x 16 (tools/onnx2one/onnx2one.cpp:1346-1349).  onhip_set_tile_hint(bm, bn) makes the cost model of the calling

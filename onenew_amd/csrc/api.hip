@@ -86,6 +86,7 @@ static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 static const int kMaxDevices = 64;
 static void *g_noalloc_ptr[kMaxDevices];      // address of `scratch` on each device, once looked up there
 static thread_local void *tl_noalloc = nullptr;   // non-null while this thread runs the entry point: get_scratch hands it out
+static std::atomic<long long> g_noalloc_scratch_uses{0};   // launches whose partial sums went to the built-in array
 
 // address of this device's copy of `scratch`; looked up with that device current, no allocation involved
 static int noalloc_scratch(void **out) {
@@ -109,6 +110,7 @@ static int get_scratch(size_t bytes, void **out) {
             return set_error(ONHIP_ERR_WORKSPACE, "conv (no allocation): the split-K partial sums of this problem take %zu bytes, "
                              "the built-in scratch holds %zu; use onhip_conv2d_f32", bytes, kNoAllocScratchBytes);
         *out = tl_noalloc;
+        g_noalloc_scratch_uses.fetch_add(1, std::memory_order_relaxed);
         return ONHIP_OK;
     }
     std::lock_guard<std::mutex> lock(g_scratch_mu);
@@ -643,6 +645,8 @@ long long onhip_scratch_bytes(void) {
 long long onhip_direct_lds_launches(void) { return g_dma_launches.load(std::memory_order_relaxed); }
 
 long long onhip_split_tail_launches(void) { return g_tail_launches.load(std::memory_order_relaxed); }
+
+long long onhip_noalloc_scratch_launches(void) { return g_noalloc_scratch_uses.load(std::memory_order_relaxed); }
 
 int onhip_conv_out_shape(const onhip_conv_desc_t *d, int32_t *oh, int32_t *ow) {
     if (!oh || !ow) return set_error(ONHIP_ERR_ARG, "conv: null output pointer");

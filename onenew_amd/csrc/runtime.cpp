@@ -567,26 +567,37 @@ bool is_net_output(const onrt_net &net, const std::string &name) {
     return std::find(net.out_names.begin(), net.out_names.end(), name) != net.out_names.end();
 }
 
-// index of the only node reading `name`, if it is of the given type and the operand is not a net output; else -1
+// index of the only node reading `name`, if it is of the given type and the operand is not a net output; else -1.
+// The other operand of an Add folded into a convolution or a MatMul (Node::addend) is a read like any input: the Add
+// itself is no longer in the order, and what it read must still be written.
 int sole_reader(const onrt_net &net, const std::string &name, const char *type) {
     if (is_net_output(net, name)) return -1;
     int found = -1;
-    for (int idx : net.order)
-        for (const std::string &in : net.nodes[idx].in)
+    for (int idx : net.order) {
+        const Node &nd = net.nodes[idx];
+        for (const std::string &in : nd.in)
             if (in == name) {
                 if (found >= 0) return -1;   // a second reader, or the same node twice
                 found = idx;
             }
+        if (!nd.addend.empty() && nd.addend == name) {
+            if (found >= 0) return -1;
+            found = idx;
+        }
+    }
     if (found < 0 || strcmp(net.nodes[found].kind->type, type)) return -1;
     return found;
 }
 
-// every node that reads `name`, in execution order
+// every node that reads `name` (as an input or as the other operand of a folded Add), in execution order
 std::vector<int> readers_of(const onrt_net &net, const std::string &name) {
     std::vector<int> out;
-    for (int idx : net.order)
-        for (const std::string &in : net.nodes[idx].in)
+    for (int idx : net.order) {
+        const Node &nd = net.nodes[idx];
+        for (const std::string &in : nd.in)
             if (in == name) out.push_back(idx);
+        if (!nd.addend.empty() && nd.addend == name) out.push_back(idx);
+    }
     return out;
 }
 
@@ -755,9 +766,10 @@ int fuse_ir_blocks(onrt_net &net) {
     std::vector<bool> dropped(net.nodes.size(), false);
     for (int idx : net.order) {
         Node &a = net.nodes[idx];
-        if (a.fuse || dropped[idx] || !plain_conv(a, 3)) continue;
+        // a convolution that already closes a fused block keeps that role: its result is that block's output
+        if (a.fuse || dropped[idx] || runs_instead.count(idx) || !plain_conv(a, 3)) continue;
         const int bi = sole_reader(net, result_of(a), "Conv");
-        if (bi < 0 || dropped[bi]) continue;
+        if (bi < 0 || dropped[bi] || runs_instead.count(bi)) continue;
         Node &b = net.nodes[bi];
         if (b.fuse || !plain_conv(b, 3) || b.in[0] != result_of(a)) continue;
         const int ci = sole_reader(net, result_of(b), "Conv");
@@ -1126,6 +1138,13 @@ int fill_slots(onrt_net &net) {
             nd.inputs[8].addr = c.in.size() > 2 ? (int64_t) net.tensors[c.in[2]].dev : 0;
         }
         if (nd.fuse == 1 || nd.fuse == 2 || nd.fuse == 6) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
+        // the other operand of a folded Add must be a tensor some operator writes (or an input): one that a later fold
+        // took the buffer away from would be added as zeros, silently
+        if (!nd.addend.empty() && !net.plan_only) {
+            const Tensor &ad = net.tensors[nd.addend];
+            if (!ad.dev || ad.never_written)
+                return fail(ONRT_ERR_FORMAT, "%s: the operand %s of the Add folded into it has no buffer", nd.base()->op_name, nd.addend.c_str());
+        }
         if (nd.link.in_s8 || nd.link.out_s8 || nd.link.twin) {
             nd.inputs[4].addr = (int64_t) &nd.link;
             nd.inputs[5].addr = nd.link_fuse ? (int64_t) &nd.link_fuse : 0;
@@ -1177,6 +1196,17 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
 
 int plan_stub_eval(BUFFER_INFO_S *, BUFFER_INFO_S *, BUFFER_INFO_S *) { return ONRT_ERR_ARG; }
 
+// stands in for the Conv plugin's `eval_block_takes` in a plan made with ONENEW_RT_PLAN_BLOCKS=1: every 1x1 -> depthwise ->
+// 1x1 chain counts as taken, whatever its size (the plugin's own answer depends on the batch and the device)
+int plan_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *, BUFFER_INFO_S *) {
+    const CONV_CONFIG_S *a = reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr);
+    const CONV_CONFIG_S *b = reinterpret_cast<const CONV_CONFIG_S *>(params[5].addr);
+    const CONV_CONFIG_S *c = reinterpret_cast<const CONV_CONFIG_S *>(params[7].addr);
+    if (!a || !b || !c) return 0;
+    const bool one_by_one = a->kernel_shape[0] == 1 && a->kernel_shape[1] == 1 && c->kernel_shape[0] == 1 && c->kernel_shape[1] == 1;
+    return one_by_one && a->group == 1 && c->group == 1 && b->group > 1 ? 1 : 0;
+}
+
 // the host-side part of prepare: what would run, in which order, on which shapes
 int plan(onrt_net &net) {
     net.plan_only = true;
@@ -1186,6 +1216,12 @@ int plan(onrt_net &net) {
     net.conv_add = net.conv_add_relu = net.matmul_attention = net.matmul_bias = net.matmul_bias_gelu = net.matmul_bias_add = plan_stub_eval;   // as with the plugins of this package
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
+    if (const char *env = getenv("ONENEW_RT_PLAN_BLOCKS"))   // "1": the inverted-residual fold as well, on the graph's shape alone
+        if (!rc && !strcmp(env, "1")) {
+            net.conv_block = plan_stub_eval;
+            net.conv_block_takes = plan_block_takes;
+            rc = fuse_ir_blocks(net);
+        }
     if (!rc) rc = fuse_attention(net);
     if (!rc) rc = fuse_linear(net);
     return rc;

@@ -29,7 +29,7 @@ def plugin_path(op):
     return os.path.join(LIBDIR, f"lib{op}_hip.so")
 
 
-EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_direct_lds_launches", "onhip_scratch_bytes", "onhip_set_tile_hint", "onhip_tile_candidate", "onhip_conv_out_shape", "onhip_conv2d_f32",
+EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_direct_lds_launches", "onhip_noalloc_scratch_launches", "onhip_scratch_bytes", "onhip_set_tile_hint", "onhip_tile_candidate", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
            "onhip_conv2d_f32_add", "onhip_conv2d_f32_noalloc", "onhip_conv_add_eval", "onhip_conv_add_relu_eval", "onhip_conv_block_eval", "onhip_conv_block_takes", "onhip_conv_link_eval", "onhip_conv2d_w8_link",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
@@ -58,6 +58,7 @@ def load():
     L = C.CDLL(path, mode=C.RTLD_GLOBAL)
     L.onhip_split_tail_launches.restype = C.c_longlong
     L.onhip_direct_lds_launches.restype = C.c_longlong
+    L.onhip_noalloc_scratch_launches.restype = C.c_longlong
     L.onhip_scratch_bytes.restype = C.c_longlong
     vp = C.c_void_p
     L.onhip_init.argtypes = [C.c_int]

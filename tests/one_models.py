@@ -57,6 +57,35 @@ def inverted_residual_blocks(batch=8, size=32):
     return m.tobytes(), [_r("xir", (batch, 16, size, size))]
 
 
+def separable_chain(batch=16, size=32, ch=32):
+    """a depthwise-separable stack pw -> dw -> pw -> dw -> pw (MobileNetV1 style, at most 64 channels): the last 1x1 of the
+    first triple is also the first 1x1 of the next, so one-launch blocks must not overlap"""
+    m = onefile.OneModel()
+    m.input("x", (batch, 16, size, size))
+    act = dict(act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("pw1", "x", _r("s_pw1w", (ch, 16, 1, 1), 0.3), _r("s_pw1b", (ch,), 0.3), "pw1_out", **act)
+    m.conv("dw1", "pw1_out", _r("s_dw1w", (ch, 1, 3, 3), 0.3), _r("s_dw1b", (ch,), 0.1), "dw1_out", pad=1, group=ch, **act)
+    m.conv("pw2", "dw1_out", _r("s_pw2w", (ch, ch, 1, 1), 0.2), _r("s_pw2b", (ch,), 0.2), "pw2_out", **act)
+    m.conv("dw2", "pw2_out", _r("s_dw2w", (ch, 1, 3, 3), 0.3), _r("s_dw2b", (ch,), 0.1), "dw2_out", pad=1, group=ch, **act)
+    m.conv("pw3", "dw2_out", _r("s_pw3w", (24, ch, 1, 1), 0.2), _r("s_pw3b", (24,), 0.1), "out")
+    m.output("out", (batch, 24, size, size))
+    return m.tobytes(), [_r("xsep", (batch, 16, size, size))]
+
+
+def block_with_inner_skip(batch=16, size=32, ch=32):
+    """1x1 -> depthwise -> 1x1 whose result is added to the FIRST convolution's result: that operand has a second reader
+    (the Add folded into the last convolution), so the triple must stay three operators"""
+    m = onefile.OneModel()
+    m.input("x", (batch, 16, size, size))
+    act = dict(act=abi.CLIP, clip=(0.0, 6.0))
+    m.conv("a", "x", _r("k_aw", (ch, 16, 1, 1), 0.3), _r("k_ab", (ch,), 0.3), "a_out", **act)
+    m.conv("b", "a_out", _r("k_bw", (ch, 1, 3, 3), 0.3), _r("k_bb", (ch,), 0.1), "b_out", pad=1, group=ch, **act)
+    m.conv("c", "b_out", _r("k_cw", (ch, ch, 1, 1), 0.2), _r("k_cb", (ch,), 0.2), "c_out")
+    m.add("skip", "c_out", "a_out", "out")
+    m.output("out", (batch, ch, size, size))
+    return m.tobytes(), [_r("xskip", (batch, 16, size, size))]
+
+
 def vit_block():
     """layer norm, projection with a weight initialiser and a bias Add, table GELU, residual, then a token-mixing
     pair of MatMuls over two activations with Transpose and Softmax, and a Reshape view"""

@@ -270,6 +270,29 @@ def test_inverted_residual_blocks_run_as_one_call(torch_dev, monkeypatch):
     small.close()
 
 
+def test_one_launch_blocks_do_not_overlap_nor_swallow_a_folded_adds_operand(torch_dev, monkeypatch):
+    """pw -> dw -> pw -> dw -> pw with at most 64 channels at a batch where the plugin recommends the block kernel: one block
+    is folded (the middle 1x1 closes it and opens no second one), the output equals the operator-by-operator run within
+    1e-4; a triple whose first result the folded Add of its last convolution reads keeps its operators and its values"""
+    data, ins = one_models.separable_chain(batch=16, size=32)
+    fused, plain, got, want = _both_ways(data, ins, monkeypatch)
+    assert plain.fused_ir_blocks() == 0 and fused.fused_ir_blocks() == 1
+    assert [n for _, n in fused.ops()] == ["pw1", "dw2", "pw3"]
+    for g, w_ in zip(got, want):
+        assert g.shape == w_.shape and np.all(np.abs(g - w_) <= 1e-4 * np.abs(w_) + 1e-5 * np.abs(w_).max())
+    assert _close(got[0], one_model.run(data, ins)[0], 5e-4)
+    fused.close()
+    plain.close()
+    data, ins = one_models.block_with_inner_skip(batch=16, size=32)
+    fused, plain, got, want = _both_ways(data, ins, monkeypatch)
+    assert fused.fused_ir_blocks() == 0 and fused.fused_blocks() == 1
+    assert [n for _, n in fused.ops()] == ["a", "b", "c"]
+    assert np.all(np.abs(got[0] - want[0]) <= 1e-4 * np.abs(want[0]) + 1e-5 * np.abs(want[0]).max())
+    assert _close(got[0], one_model.run(data, ins)[0], 5e-4)
+    fused.close()
+    plain.close()
+
+
 def test_mobilenetv2_batch64_with_its_blocks_in_one_call(torch_dev, monkeypatch):
     """the whole MobileNetV2 model at batch 64, where the early inverted-residual blocks run as one call each: logits
     against the same file run operator by operator (1e-3 of the largest logit, same top-5 on every image)"""

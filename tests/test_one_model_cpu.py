@@ -183,6 +183,29 @@ def test_plan_folds_residual_blocks_and_relus():
     assert net.outputs[0][1] == (3, 1000)
 
 
+def test_plan_keeps_one_launch_blocks_apart_and_counts_folded_adds_as_reads(monkeypatch):
+    """the inverted-residual fold on the graph alone (ONENEW_RT_PLAN_BLOCKS=1 takes every 1x1 -> depthwise -> 1x1 chain):
+    in pw -> dw -> pw -> dw -> pw the middle 1x1 closes the first block and must not open a second one over it; a triple
+    whose first result is also the other operand of the Add folded into its last convolution stays three operators"""
+    monkeypatch.setenv("ONENEW_RT_PLAN_BLOCKS", "1")
+    data, _ = one_models.separable_chain()
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_ir_blocks() == 1
+    assert [n for _, n in net.ops()] == ["pw1", "dw2", "pw3"]
+    data, _ = one_models.block_with_inner_skip()
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 1 and net.fused_ir_blocks() == 0
+    assert [n for _, n in net.ops()] == ["a", "b", "c"]
+    # MobileNetV2's blocks: the skip connection reads the block's input, not an operand inside it; all 16 expanding
+    # blocks are chains of this shape (the first block has no expansion)
+    from onenew_amd import stacks
+    data, _, _ = stacks.mobilenet_v2_model(2)
+    net = rt.Net(data, plan_only=True)
+    assert net.fused_blocks() == 10 and net.fused_ir_blocks() == 16
+    monkeypatch.delenv("ONENEW_RT_PLAN_BLOCKS")
+    assert rt.Net(one_models.separable_chain()[0], plan_only=True).fused_ir_blocks() == 0
+
+
 def test_plan_runs_an_attention_block_as_one_call(monkeypatch):
     """MatMul(q, Transpose(k)) -> Softmax -> MatMul(., v): one call where the fused kernel takes the shape, four operators
     where it does not (head dimension, token count), where an operand in between has another reader, or with fusing off"""

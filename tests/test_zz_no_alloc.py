@@ -44,8 +44,11 @@ def test_no_alloc_entry_point_matches_the_allocating_one():
             oh, ow = d.out_hw()
             out = torch.full((d.n, d.cout, oh, ow), float("nan"), dtype=torch.float32, device="cuda")
             torch.cuda.synchronize()
+            used = hip.load().onhip_noalloc_scratch_launches()
             hip.conv2d_f32_noalloc(d, x, wp, out, b, packed=packed)
             torch.cuda.synchronize()
+            # the case is only a test of the built-in array if the cost model did cut K for it
+            assert hip.load().onhip_noalloc_scratch_launches() == used + 1, f"{tag}: the call did not use the built-in scratch array"
             got, want = out.cpu().numpy(), ref.cpu().numpy()
             assert np.isfinite(got).all()
             scale = float(np.abs(want).max())
