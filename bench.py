@@ -279,36 +279,6 @@ class VitGlueLayer:
         return fl, lambda: oracle.transpose_f32(x, self.perm)
 
 
-class DwProjectLayer:
-    """depthwise 3x3 + CLIP and the 1x1 projection after it in one launch (the depthwise result stays on the chip); work
-    and bytes are counted as the two separate convolutions' (every tensor of the unfused pair once)"""
-    kind = "dw_project"
-
-    def __init__(self, torch, hip, name, dw, pw, tag):
-        from onenew_amd import datagen
-        dname = name.replace(".dw", "")
-        self.name, self.dw, self.pw = dname + ".dw+proj", dw, pw
-        self.x = device_uniform(torch, datagen.seed_for(f"{tag}/{name}", "x"), (dw.n, dw.cin, dw.h, dw.w))
-        g = lambda role, shape, std: torch.from_numpy(datagen.normal(datagen.seed_for(f"{tag}/{name}", role), shape, 0.0, std)).cuda()
-        self.dw_w, self.dw_b = g("w", (dw.cout, 1, 3, 3), float(np.sqrt(2.0 / 9))), g("b", (dw.cout,), 0.01)
-        self.pw_w, self.pw_b = g("pw", (pw.cout, pw.cin, 1, 1), float(np.sqrt(2.0 / pw.cin))), g("pb", (pw.cout,), 0.01)
-        self.packed = hip.dw_project_pack_weights(self.pw_w)
-        oh, ow = dw.out_hw()
-        self.y = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device="cuda")
-        self.flops = dw.flops() + pw.flops()
-        self.bytes = dw.algorithmic_bytes() + pw.algorithmic_bytes()
-        self.dense = False           # bound by memory traffic like the depthwise layer it contains
-        self.shape = f"C={dw.cin} M={pw.cout} N={dw.n * oh * ow} s{dw.stride_h}"
-
-    def launch(self, hip):
-        hip.dw_project_f32(self.dw, self.pw, self.x, self.dw_w, self.dw_b, self.packed, self.pw_b, out=self.y)
-
-    def cpu_runner(self, ops, oracle, tag):
-        f1, r1 = ConvF32Layer.cpu_runner(type("L", (), {"d": self.dw, "name": self.name + "/dw"})(), ops, oracle, tag)
-        f2, r2 = ConvF32Layer.cpu_runner(type("L", (), {"d": self.pw, "name": self.name + "/pw"})(), ops, oracle, tag)
-        return f1 + f2, lambda: (r1(), r2())
-
-
 class IrBlockLayer:
     """a whole inverted-residual block (1x1 expansion + CLIP, depthwise 3x3 + CLIP, 1x1 projection) in one launch: neither
     wide tensor leaves the chip; work and bytes are counted as the three separate convolutions' (every tensor of the
@@ -532,28 +502,20 @@ def make_workload(torch, hip, name):
     if name.startswith("mobilenetv2_b"):
         n = int(name.split("_b")[1].split("_")[0])
         spec = stacks.with_batch(stacks.mobilenet_v2(), n)
-        layers, fused, blocks, i = [], 0, 0, 0
+        layers, blocks, i = [], 0, 0
         while i < len(spec):
             ln, d = spec[i]
             # expansion, depthwise and projection in one launch where the block kernel takes the shapes
-            if (not name.endswith("_unfused") and not name.endswith("_noblocks") and i + 2 < len(spec) and d.group == 1
+            if (not name.endswith("_unfused") and i + 2 < len(spec) and d.group == 1
                     and hip.ir_block_supported(d, spec[i + 1][1], spec[i + 2][1]) >= 2):
                 layers.append(IrBlockLayer(torch, hip, ln, d, spec[i + 1][1], spec[i + 2][1], tag))
                 blocks += 1
                 i += 3
                 continue
-            # a depthwise convolution and the projection behind it in one launch where the library recommends it
-            want = 1 if name.endswith("_fusedall") else 2
-            if (not name.endswith("_unfused") and d.group != 1 and i + 1 < len(spec)
-                    and hip.dw_project_supported(d, spec[i + 1][1]) >= want):
-                layers.append(DwProjectLayer(torch, hip, ln, d, spec[i + 1][1], tag))
-                fused += 1
-                i += 2
-            else:
-                layers.append(ConvF32Layer(torch, hip, ln, d, tag))
-                i += 1
+            layers.append(ConvF32Layer(torch, hip, ln, d, tag))
+            i += 1
         return (f"MobileNetV2 conv stack fp32, batch {n}, 224x224, 52 conv layers (17 depthwise), ReLU6 as CLIP; {blocks} whole inverted-residual blocks "
-                f"and {fused} depthwise + projection pairs as one launch each", "f32", layers)
+                f"as one launch each", "f32", layers)
     if name == "cfg1":
         import cases
         return ("Conv2d+ReLU fp32 64->64 56x56 3x3 s1 p1, batch 1", "f32",

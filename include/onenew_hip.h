@@ -97,6 +97,12 @@ long long onhip_split_tail_launches(void);
 /* Diagnostic, no counterpart in the reference: how many int8 launches so far ran the kernel that loads its operand tiles
  * from global memory straight into LDS (NHWC int8 activations with a multiple of 64 padded channels). */
 long long onhip_direct_lds_launches(void);
+/* Diagnostic, no counterpart in the reference: how the calling thread's last dense convolution / MatMul launch ran:
+ * out = {tile rows, tile columns, K slices of every tile (1 = none), K slices of the leftover tiles only (0 = none),
+ * 1 if the fp32 kernel that reads B straight from memory ran, 1 if the slices were added up inside the launch,
+ * 1 / 2 if the kernel that loads operand tiles straight into LDS ran (short / long ring)}; zeros before the first such
+ * launch; launches of the other kernel families (depthwise, first-layer, few-channel int8) leave it as it is. */
+void onhip_last_launch_choice(int32_t out[7]);
 /* Diagnostic, no counterpart in the reference: how many launches of onhip_conv2d_f32_noalloc so far cut K into slices and
  * therefore put their partial sums into the library's built-in scratch array (a call the cost model gives a single
  * slice never touches the array). */
@@ -267,22 +273,6 @@ int onhip_matmul(const onhip_matmul_desc_t *d, const float *a, const float *b, c
  * device/x86/Add/add.c evals, bit-equal to them.  addend must not be the output buffer. */
 int onhip_matmul_add(const onhip_matmul_desc_t *d, const float *a, const float *b, const float *bias,
                      const float *addend, float *out, void *stream);
-
-/* The second half of an inverted-residual block in one launch: depthwise 3x3 convolution (pads 1, stride 1 or 2, bias,
- * activation) -> 1x1 convolution (bias, activation) [-> Add of a residual tensor shaped like the output].  Replaces two
- * (three) operator evaluations, device/x86/Conv/conv.c depthwise path :757-899 and 1x1 path :1024-1056 (and
- * device/x86/Add/add.c), without the depthwise result ever being written to memory.  The depthwise values are those of
- * the separate operator bit for bit (same operations in the same order); the 1x1 sums are fp32 in MFMA order like
- * onhip_conv2d_f32's.  No counterpart as one function in the reference.
- * onhip_dw_project_supported: 0 = this pair of descriptors is not taken (run the two convolutions), 1 = taken,
- * 2 = taken and expected to be faster than the two launches.  pw_packed: the 1x1 weights [cout][cin] re-laid once by
- * onhip_dw_project_pack_weights (onhip_dw_project_packed_weight_bytes(cin, cout) bytes, 16-byte aligned). */
-int onhip_dw_project_supported(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw);
-size_t onhip_dw_project_packed_weight_bytes(int32_t ce, int32_t co);
-int onhip_dw_project_pack_weights(const float *pw_w, int32_t ce, int32_t co, float *packed, void *stream);
-int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const float *x, const float *dw_w,
-                         const float *dw_b, const float *pw_packed, const float *pw_b, const float *residual, float *y,
-                         void *stream);
 
 /* A whole inverted-residual block in one launch: 1x1 convolution (bias, activation) -> depthwise 3x3 (pads 1, stride 1 or
  * 2, bias, activation) -> 1x1 convolution (bias, activation) [-> Add of a residual tensor shaped like the output].

@@ -401,10 +401,22 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
 static std::atomic<long long> g_tail_launches{0};
 static std::atomic<long long> g_dma_launches{0};
 
+// what the calling thread's last implicit-GEMM launch ran as (onhip_last_launch_choice): tile, K slices as launched,
+// slices of the leftover tiles, and which kernel
+static thread_local int tl_last_choice[7] = {0, 0, 0, 0, 0, 0, 0};
+
 // Runs the problem the way the choice says.
 static int launch_choice(IgemmLaunch cfg, IgemmParams p, const Choice &c, hipStream_t st) {
     int dpc = 0, left = 0;
     p.part_begin = p.dp_tiles = p.tail_tiles = 0;
+    struct Note {   // filled in on every way out of this function
+        const IgemmLaunch &cfg; const IgemmParams &p; const Choice &c;
+        ~Note() {
+            const bool tail = p.tail_tiles > 0;
+            const int v[7] = {c.bm, c.bn, c.dma || tail ? 1 : cfg.split, tail ? cfg.split : 0, c.dma ? 0 : c.rowb, p.arrive ? 1 : 0, c.dma};
+            for (int i = 0; i < 7; ++i) tl_last_choice[i] = v[i];
+        }
+    } note{cfg, p, c};
     if (c.dma) {
         cfg.bm = c.bm; cfg.bn = c.bn; cfg.split = 1;
         cfg.ring = c.dma > 1;
@@ -645,6 +657,10 @@ long long onhip_scratch_bytes(void) {
 long long onhip_direct_lds_launches(void) { return g_dma_launches.load(std::memory_order_relaxed); }
 
 long long onhip_split_tail_launches(void) { return g_tail_launches.load(std::memory_order_relaxed); }
+
+void onhip_last_launch_choice(int32_t out[7]) {
+    for (int i = 0; i < 7; ++i) out[i] = tl_last_choice[i];
+}
 
 long long onhip_noalloc_scratch_launches(void) { return g_noalloc_scratch_uses.load(std::memory_order_relaxed); }
 
@@ -1278,7 +1294,8 @@ int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, cons
     return conv2d_h16_impl(&d, x, w_packed, bias, gelu_lut, gelu_lut != nullptr, residual, 0, y, y_kind, stream);
 }
 
-// the depthwise 3x3 -> 1x1 pair the fused kernel takes; *why (when not null) says what rules a pair out
+// the depthwise 3x3 -> 1x1 pair at the end of a block the one-launch block kernel takes; *why (when not null) says what
+// rules a pair out
 static bool dw_project_shapes_ok(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const char **why) {
     const char *w = nullptr;
     int32_t OH = 0, OW = 0;
@@ -1293,45 +1310,9 @@ static bool dw_project_shapes_ok(const onhip_conv_desc_t *dw, const onhip_conv_d
         w = "the second convolution must be 1x1, stride 1, unpadded";
     else if (pw->cin != dw->cout || pw->n != dw->n || pw->h != OH || pw->w != OW) w = "the second convolution does not take the first one's output";
     else if (pw->cout < 1 || pw->cout > 128) w = "at most 128 output channels";
-    else if (dwproj_band_rows(*dw, OH, OW, pw->cout) < 1) w = "output rows of more than 128 pixels";
     else if ((long long) dw->n * dw->cin * dw->h * dw->w * 4 >= (1LL << 31) || (long long) pw->n * pw->cout * OH * OW * 4 >= (1LL << 31)) w = "tensors of 2 GiB or more";
     if (why) *why = w;
     return w == nullptr;
-}
-
-int onhip_dw_project_supported(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw) {
-    if (!dw_project_shapes_ok(dw, pw, nullptr)) return 0;
-    // Measured on MobileNetV2 at batch 64 (separate launches against this one): 96 channels 112x112 stride 2, 117 us
-    // against 98 us; stride 1 at 112x112 and 56x56, 83 and 79 us against 120 and 94 us.  The stride-2 depthwise kernel
-    // reads every other column it loads, which the patch here does not pay for; otherwise the two launches, each near
-    // half of the memory bandwidth, beat this kernel's serial chunk pipeline.  Recommended for the first case only.
-    int32_t OH = 0, OW = 0;
-    (void) onhip_conv_out_shape(dw, &OH, &OW);
-    const int rows = dwproj_band_rows(*dw, OH, OW, pw->cout);
-    const long long wgs = (long long) dw->n * ((OH + rows - 1) / rows);
-    return dw->stride_h == 2 && wgs >= 1024 && rows * OW >= 96 ? 2 : 1;
-}
-
-size_t onhip_dw_project_packed_weight_bytes(int32_t ce, int32_t co) {
-    return ce < 1 || co < 1 ? 0 : (size_t) ce * ((co + 31) / 32 * 32) * sizeof(float);
-}
-
-int onhip_dw_project_pack_weights(const float *pw_w, int32_t ce, int32_t co, float *packed, void *stream) {
-    if (!pw_w || !packed || ce < 1 || co < 1 || reinterpret_cast<uintptr_t>(packed) % 16) return set_error(ONHIP_ERR_ARG, "dw + project pack: bad argument");
-    return dwproj_pack_launch(pw_w, ce, co, packed, reinterpret_cast<hipStream_t>(stream));
-}
-
-int onhip_dw_project_f32(const onhip_conv_desc_t *dw, const onhip_conv_desc_t *pw, const float *x, const float *dw_w, const float *dw_b,
-                         const float *pw_packed, const float *pw_b, const float *residual, float *y, void *stream) {
-    const char *why = nullptr;
-    if (!dw_project_shapes_ok(dw, pw, &why)) return set_error(ONHIP_ERR_ARG, "dw + project: %s", why);
-    if (!x || !dw_w || !dw_b || !pw_packed || !y || (pw->has_bias && !pw_b)) return set_error(ONHIP_ERR_ARG, "dw + project: null tensor pointer");
-    if (reinterpret_cast<uintptr_t>(pw_packed) % 16) return set_error(ONHIP_ERR_ARG, "dw + project: packed weights must be 16-byte aligned");
-    if (residual == y) return set_error(ONHIP_ERR_ARG, "dw + project: the residual operand may not be the output buffer");
-    int32_t OH = 0, OW = 0;
-    (void) onhip_conv_out_shape(dw, &OH, &OW);
-    return dwproj_f32_launch(*dw, *pw, OH, OW, x, dw_w, dw_b, pw_packed, pw->has_bias ? pw_b : nullptr, residual, make_epilogue(*dw, nullptr),
-                             make_epilogue(*pw, nullptr), y, reinterpret_cast<hipStream_t>(stream));
 }
 
 // the expansion -> depthwise -> projection triple the one-launch block kernel takes

@@ -264,12 +264,6 @@ int irblock_f32_launch(const onhip_conv_desc_t &ex, const onhip_conv_desc_t &dw,
                        const float *packed, const float *exp_b, const float *dw_w, const float *dw_b, const float *pw_b, const float *res,
                        const Epilogue &exp_ep, const Epilogue &dw_ep, const Epilogue &pw_ep, float *y, hipStream_t stream);
 
-// dwproj.hip: depthwise 3x3 -> 1x1 convolution in one launch
-int dwproj_pack_launch(const float *w, int ce, int co, float *packed, hipStream_t stream);
-int dwproj_band_rows(const onhip_conv_desc_t &dw, int OH, int OW, int co);
-int dwproj_f32_launch(const onhip_conv_desc_t &dw, const onhip_conv_desc_t &pw, int OH, int OW, const float *x, const float *dw_w,
-                      const float *dw_b, const float *pw_t, const float *pw_b, const float *res, const Epilogue &dw_ep,
-                      const Epilogue &pw_ep, float *y, hipStream_t stream);
 // stem.hip: first-layer convolutions (three input channels) from an LDS patch
 bool stem_f32_shape(const onhip_conv_desc_t &d);
 bool stem_f32_ok(const onhip_conv_desc_t &d, int OH, int OW);

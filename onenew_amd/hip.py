@@ -29,7 +29,7 @@ def plugin_path(op):
     return os.path.join(LIBDIR, f"lib{op}_hip.so")
 
 
-EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_direct_lds_launches", "onhip_noalloc_scratch_launches", "onhip_scratch_bytes", "onhip_set_tile_hint", "onhip_tile_candidate", "onhip_conv_out_shape", "onhip_conv2d_f32",
+EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_direct_lds_launches", "onhip_noalloc_scratch_launches", "onhip_last_launch_choice", "onhip_scratch_bytes", "onhip_set_tile_hint", "onhip_tile_candidate", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
            "onhip_conv2d_f32_add", "onhip_conv2d_f32_noalloc", "onhip_conv_add_eval", "onhip_conv_add_relu_eval", "onhip_conv_block_eval", "onhip_conv_block_takes", "onhip_conv_link_eval", "onhip_conv2d_w8_link",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
@@ -39,7 +39,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_matmul", "onhip_matmul_add", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
-           "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", "onhip_dw_project_supported", "onhip_dw_project_packed_weight_bytes", "onhip_dw_project_pack_weights", "onhip_dw_project_f32",
+           "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", 
            "onhip_ir_block_supported", "onhip_ir_block_packed_weight_bytes", "onhip_ir_block_pack_weights", "onhip_ir_block_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_maxpool_s8_nhwc", "onhip_maxpool_s8_eval", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
@@ -114,11 +114,6 @@ def load():
     L.onhip_h16_to_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
     L.onhip_conv2d_h16.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, i32, vp, i32, vp]
     L.onhip_attention.argtypes = [C.POINTER(abi.AttentionDesc), vp, vp, vp, vp, vp]
-    L.onhip_dw_project_supported.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc)]
-    L.onhip_dw_project_packed_weight_bytes.argtypes = [i32, i32]
-    L.onhip_dw_project_packed_weight_bytes.restype = C.c_size_t
-    L.onhip_dw_project_pack_weights.argtypes = [vp, i32, i32, vp, vp]
-    L.onhip_dw_project_f32.argtypes = [C.POINTER(ConvDesc), C.POINTER(ConvDesc), vp, vp, vp, vp, vp, vp, vp, vp]
     L.onhip_ir_block_supported.argtypes = [C.POINTER(ConvDesc)] * 3
     L.onhip_ir_block_packed_weight_bytes.argtypes = [i32, i32, i32]
     L.onhip_ir_block_packed_weight_bytes.restype = C.c_size_t
@@ -566,29 +561,6 @@ def linear_h16(x, w_packed, k, n, compute, bias=None, gelu_lut=None, residual=No
     return out
 
 
-def dw_project_supported(dw, pw):
-    return load().onhip_dw_project_supported(C.byref(dw), C.byref(pw))
-
-
-def dw_project_pack_weights(pw_w):
-    """1x1 weights [cout, cin(, 1, 1)] -> the k-major layout of the fused depthwise + 1x1 kernel"""
-    import torch
-    co, ce = pw_w.shape[0], pw_w.shape[1]
-    out = torch.empty(load().onhip_dw_project_packed_weight_bytes(ce, co) // 4, dtype=torch.float32, device=pw_w.device)
-    _check(load().onhip_dw_project_pack_weights(_ptr(pw_w), ce, co, _ptr(out), _stream()), "onhip_dw_project_pack_weights")
-    return out
-
-
-def dw_project_f32(dw, pw, x, dw_w, dw_b, pw_packed, pw_b=None, residual=None, out=None):
-    import torch
-    oh, ow = dw.out_hw()
-    if out is None:
-        out = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device=x.device)
-    _check(load().onhip_dw_project_f32(C.byref(dw), C.byref(pw), _ptr(x), _ptr(dw_w), _ptr(dw_b), _ptr(pw_packed), _ptr(pw_b),
-                                       _ptr(residual), _ptr(out), _stream()), "onhip_dw_project_f32")
-    return out
-
-
 def ir_block_supported(ex, dw, pw):
     return load().onhip_ir_block_supported(C.byref(ex), C.byref(dw), C.byref(pw))
 
@@ -652,6 +624,13 @@ def copy_f32(src, dst):
     """plain device copy (the yardstick for HBM traffic counters)"""
     _check(load().onhip_copy_f32(_ptr(src), _ptr(dst), src.numel(), _stream()), "onhip_copy_f32")
     return dst
+
+
+def last_launch_choice():
+    """(bm, bn, split, tail, rowb, fin, dma) of the calling thread's last dense convolution / MatMul launch"""
+    v = (C.c_int32 * 7)()
+    load().onhip_last_launch_choice(v)
+    return tuple(int(t) for t in v)
 
 
 def split_tail_launches():

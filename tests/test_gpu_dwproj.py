@@ -11,7 +11,11 @@ import pytest
 import cases
 from onenew_amd import abi, hip
 
-pytestmark = pytest.mark.gpu
+# The kernel these tests cover (depthwise 3x3 + 1x1 projection in one launch, onhip_dw_project_f32) was taken out of the
+# library: the whole-block kernel (onhip_ir_block_f32, tests/test_gpu_irblock.py) runs every block it was faster on, and
+# on every other shape it lost to the two separate launches.  The tests stay as the record of what it had to satisfy.
+pytestmark = [pytest.mark.gpu, pytest.mark.skip(reason="onhip_dw_project_f32 is no longer part of the library: superseded by the "
+                                                       "one-launch block kernel, slower than two launches elsewhere")]
 
 
 @pytest.fixture(scope="module")

@@ -1,6 +1,10 @@
 """The benchmark configurations at their stated sizes, every layer: ResNet-50 batch 32 (53 convolutions), MobileNetV2
 batch 64 (52, of which 17 depthwise), the ViT-Tiny MatMuls at B = 64 in fp32 and bf16, YOLOv8s int8 batch 16 (63
-convolutions, fp32-in/out W8A32 form and int8 NHWC chain form).  What the benchmark times is what is checked here.
+convolutions, fp32-in/out W8A32 form and int8 NHWC chain form).  The dense fp32 layers are checked twice: with the tile
+and split the cost model gives (a host calling `eval` gets those) and with the ones the library measures when tuning is
+on, which is what the benchmark times; and, on the layers where the measured choice varies from box to box, under
+each kernel variant it can fall on (B straight from memory, K slices added up inside the launch, leftover tiles cut
+along K).
 
 Tensors of this size are drawn on the device (seeded) and only what the check needs comes back to the host: for a
 dense convolution the input patches of a few thousand sampled outputs, which are then evaluated on the CPU - float64
@@ -121,6 +125,14 @@ def _check_depthwise_f32(torch, oracle, tag, name, d):
     assert torch.equal(y2[keep], y[keep])
 
 
+@pytest.fixture
+def measured_choices():
+    """tile, split and kernel variant measured per problem shape on first use, as bench.py runs the stacks"""
+    prev = hip.set_tuning(1)
+    yield
+    hip.set_tuning(prev)
+
+
 RESNET = stacks.with_batch(stacks.resnet50(), 32)
 MOBILENET = stacks.with_batch(stacks.mobilenet_v2(), 64)
 YOLO = stacks.with_batch(stacks.yolov8s(), 16)
@@ -131,6 +143,55 @@ def test_resnet50_batch32_every_layer(layer, torch_dev):
     name, d = RESNET[layer]
     print(f"resnet50 b32 {name}", flush=True)
     _check_dense_f32(torch_dev, "rn50b32", name, d)
+
+
+@pytest.mark.parametrize("layer", range(len(RESNET)), ids=[n for n, _ in RESNET])
+def test_resnet50_batch32_every_layer_measured_choice(layer, torch_dev, measured_choices):
+    """the same check with the launch the library measures to be the fastest for the shape: what bench.py times"""
+    name, d = RESNET[layer]
+    _check_dense_f32(torch_dev, "rn50b32", name, d)
+    print(f"resnet50 b32 {name}: measured choice (bm, bn, split, tail, rowb, fin, dma) = {hip.last_launch_choice()}", flush=True)
+
+
+def _layer(stack, name):
+    return next(d for n, d in stack if n == name)
+
+
+# (layer, ONHIP_TILE, what must have run): the kernel variants the measured choice takes on these layers on one box or
+# another - B straight from memory (rowb) on 1x1 stride-1 layers, K slices reduced by the last slice to arrive (fin)
+# or by a finishing launch, the leftover tiles alone cut along K (tail)
+FORCED = [("l1.0.conv1", "64x256x1x0x1", dict(rowb=1)), ("l1.0.conv3", "64x128x1x0x1", dict(rowb=1)),
+          ("l1.1.conv1", "128x128x1x0x1", dict(rowb=1)), ("l2.0.conv1", "128x128x1x0x1", dict(rowb=1)),
+          ("l2.1.conv3", "64x128x1x0x1", dict(rowb=1)), ("l3.0.conv1", "128x128x1x0x1", dict(rowb=1)),
+          ("l4.0.conv1", "128x128x1x0x1", dict(rowb=1)), ("l2.0.down", "64x128", dict(rowb=0, split=1)),
+          ("l3.1.conv2", "64x64x3x0x0x1", dict(split=3, fin=1)), ("l3.1.conv2", "64x64x3", dict(split=3, fin=0)),
+          ("l3.0.conv2", "64x64x3x0x0x1", dict(split=3, fin=1)), ("l3.1.conv1", "64x64x2x0x0x1", dict(split=2, fin=1)),
+          ("l3.1.conv3", "64x128x1x2x0x1", dict()), ("l4.0.conv2", "64x64x6x0x0x1", dict(split=6, fin=1)),
+          ("l4.1.conv2", "64x64x6x0x0x1", dict(split=6, fin=1)), ("l4.1.conv2", "128x128x12x0x0x1", dict(split=12, fin=1)),
+          ("l4.1.conv1", "64x64x4x0x0x1", dict(split=4, fin=1)), ("l4.1.conv3", "64x64x2x0x0x1", dict(split=2, fin=1)),
+          ("l4.0.down", "64x64x2x0x0x1", dict(split=2, fin=1)), ("l2.1.conv2", "64x64x1x4x0x1", dict(tail=4, fin=1)),
+          ("l2.1.conv2", "64x64x1x4", dict(tail=4, fin=0)), ("l1.1.conv2", "64x64x1x8x0x1", dict(tail=8, fin=1)),
+          ("l2.1.conv1", "64x64x1x2x0x1", dict()), ("l3.0.conv1", "64x128x1x2x0x1", dict())]
+
+
+@pytest.mark.parametrize("name,tile,ran", FORCED, ids=[f"{n}-{t}" for n, t, _ in FORCED])
+def test_resnet50_batch32_forced_kernel_variants(name, tile, ran, torch_dev, monkeypatch):
+    monkeypatch.setenv("ONHIP_TILE", tile)
+    print(f"resnet50 b32 {name} forced {tile}", flush=True)
+    _check_dense_f32(torch_dev, "rn50b32", name, _layer(RESNET, name))
+    got = dict(zip(("bm", "bn", "split", "tail", "rowb", "fin", "dma"), hip.last_launch_choice()))
+    print(f"  ran as {got}", flush=True)
+    want = [int(v) for v in tile.split("x")[:2]]
+    assert [got["bm"], got["bn"]] == want, (tile, got)
+    for key, v in ran.items():
+        assert got[key] == v, f"{name} {tile}: {key} = {got[key]}, expected {v} ({got})"
+
+
+@pytest.mark.parametrize("layer", [i for i, (_, d) in enumerate(MOBILENET) if d.group == 1], ids=[n for n, d in MOBILENET if d.group == 1])
+def test_mobilenetv2_batch64_every_dense_layer_measured_choice(layer, torch_dev, measured_choices):
+    name, d = MOBILENET[layer]
+    _check_dense_f32(torch_dev, "mbv2b64", name, d, w_std=0.05)
+    print(f"mobilenetv2 b64 {name}: measured choice = {hip.last_launch_choice()}", flush=True)
 
 
 @pytest.mark.parametrize("layer", range(len(MOBILENET)), ids=[n for n, _ in MOBILENET])
@@ -196,10 +257,13 @@ def test_mobilenetv2_batch64_blocks_in_one_launch(first, torch_dev, oracle):
 VIT = stacks.vit_tiny(64)
 
 
+@pytest.mark.parametrize("tuned", [0, 1], ids=["cost_model", "measured_choice"])
 @pytest.mark.parametrize("compute", [abi.COMPUTE_F32, abi.COMPUTE_BF16, abi.COMPUTE_F16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("layer", range(len(VIT)), ids=[v[0] for v in VIT])
-def test_vit_tiny_batch64_every_matmul(layer, compute, torch_dev, oracle):
+def test_vit_tiny_batch64_every_matmul(layer, compute, tuned, torch_dev, oracle, request):
     torch = torch_dev
+    prev = hip.set_tuning(tuned)
+    request.addfinalizer(lambda: hip.set_tuning(prev))
     name, md, has_bias, gelu = VIT[layer]
     print(f"vit b64 {name} compute {compute}", flush=True)
     ashape = (md.batch, md.m, md.k)
