@@ -169,7 +169,8 @@ int onhip_conv2d_f32_noalloc(const onhip_conv_desc_t *d, const float *x, const f
 int onhip_conv2d_f32_add(const onhip_conv_desc_t *d, const float *x, const float *w, int32_t packed, const float *bias,
                          const float *silu_lut, const float *addend, int32_t relu_after, float *y, void *stream);
 
-/* Bytes of device scratch onhip_conv2d_w8a32 needs for `d` (the int8 copy of the activations). */
+/* Bytes of device scratch onhip_conv2d_w8a32 (and onhip_conv2d_w8_link on fp32 activations) needs for `d`: the int8
+ * copy of the activations.  A depthwise convolution uses it only in onhip_conv2d_w8_link with fp32 in and int8 out. */
 size_t onhip_conv2d_w8a32_workspace(const onhip_conv_desc_t *d);
 
 /* W8A32 convolution: fp32 activations quantised with d->input_scale, int8 weights
@@ -203,8 +204,10 @@ int onhip_conv2d_w8a32_packed(const onhip_conv_desc_t *d, const float *x, const 
  * from the activations de-quantised with d->input_scale — the quantiser every reference Conv applies
  * to its input (conv.c:961-973), moved into the producer's epilogue, so a chain of these calls gives
  * the consumer the same int8 values as a chain of reference convolutions.  No counterpart as a
- * separate function in the reference.  Dense convolutions only; weights from
- * onhip_conv2d_w8a32_pack_weights.  onhip_quantize_nhwc_s8 makes the first xq of a chain from
+ * separate function in the reference.  Dense convolutions take their weights from
+ * onhip_conv2d_w8a32_pack_weights; depthwise convolutions (d->group == d->cin, the arithmetic of
+ * conv.c:617-755) take them as the reference holds them, [c][1][kh][kw] int8, and write padding
+ * channels as zero.  onhip_quantize_nhwc_s8 makes the first xq of a chain from
  * NCHW fp32 (q 16-byte aligned, n*h*w*round_up(c,16) bytes). */
 int onhip_quantize_nhwc_s8(const float *x, int32_t n, int32_t c, int32_t h, int32_t w, float scale,
                            int8_t *q, void *stream);
@@ -212,11 +215,18 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
                            const int32_t *bias32, const float *weight_aux, const float *silu_lut,
                            int8_t *yq, void *stream);
 
+/* 1 when the depthwise convolution `d` is available with int8 NHWC activations (onhip_conv2d_w8a8_nhwc,
+ * onhip_conv2d_w8_link): any filter and stride with uniform padding, as long as the kernel's table of weights fits its
+ * LDS ((kh * kw + 3) * round_up(channels, 16) floats within 64 KiB); 0 otherwise and for dense convolutions.  No
+ * counterpart in the reference. */
+int onhip_conv2d_w8a8_depthwise_supported(const onhip_conv_desc_t *d);
+
 /* One link of an int8 chain inside a model: the activations come as fp32 NCHW (x, quantised with d->input_scale into the
  * workspace as in onhip_conv2d_w8a32) or as int8 NHWC with channels padded to 16 (xq), exactly one of the two; the
  * result leaves as fp32 NCHW (d->out_s8 == 0) or as int8 NHWC quantised with d->output_scale (d->out_s8 == 1: what a
  * consumer whose input_scale is that value would make of the fp32 result, conv.c:961-973).  Weights packed by
- * onhip_conv2d_w8a32_pack_weights.  Depthwise is refused.  addend, when not null (fp32 results only): a tensor of the
+ * onhip_conv2d_w8a32_pack_weights; for a depthwise convolution w8_packed is the weights as the reference holds them,
+ * and no addend or twin.  addend, when not null (fp32 results only): a tensor of the
  * result's shape added to it in the store (device/x86/Add/add.c:96), followed, with relu_after != 0, by relu as
  * device/x86/Relu/relu.c:27-52 (both of its rules, by element index): the three operators' bytes in one pass.  y_twin,
  * when not null (with an addend, cout a multiple of 16, d->out_s8 == 0): the fp32 result is also stored there as int8
@@ -440,12 +450,16 @@ int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFE
  * the last convolution.  onhip_conv_block_takes reads the params only and returns 1 when onhip_ir_block_supported says 2
  * for these shapes, else 0.  No counterpart in the reference, whose host runs the operators one by one. */
 int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
-/* `eval_link` of libConv_hip.so: a dense int8 (W8A32) Conv whose input and/or result travel as int8 NHWC (channels padded
+/* `eval_link` of libConv_hip.so: an int8 (W8A32) Conv, dense or depthwise, whose input and/or result travel as int8 NHWC (channels padded
  * to 16) instead of fp32 NCHW, see onhip_conv2d_w8_link.  Slots as for `eval`; inputs[4] = host pointer to
  * {int32 in_s8, int32 out_s8, float out_scale, int32 twin} (twin != 0: outputs[1] = device buffer for the int8 copy of an
  * fp32 result with a folded Add); inputs[5] = null, or host pointer to an int32 1 / 2 for the Add (and
  * Relu) of a residual block with its other operand in inputs[3] (fp32 results only).  No counterpart in the reference. */
 int onhip_conv_link_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_link_takes` of libConv_hip.so: reads params[0..2] only (CONV_CONFIG_S, input operand, weight operand) and returns
+ * 1 when `eval_link` can run this convolution with int8 NHWC activations on either side (every dense int8 convolution;
+ * depthwise ones where onhip_conv2d_w8a8_depthwise_supported says so), else 0.  No counterpart in the reference. */
+int onhip_conv_link_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_conv_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* Add (add.c:18), Relu (relu.c:8), MaxPool (maxpool.c:7), GlobalAveragePool (global_avgpool.c:7) */

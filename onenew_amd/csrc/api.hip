@@ -831,11 +831,12 @@ static void w8a32_layout(const onhip_conv_desc_t *d, int *cp, int *k_units, size
 }
 
 size_t onhip_conv2d_w8a32_workspace(const onhip_conv_desc_t *d) {
-    if (!d || d->group != 1) return 0;
+    if (!d) return 0;
     int cp, ku;
     size_t pb, qb;
     w8a32_layout(d, &cp, &ku, &pb, &qb);
-    return pb + qb;
+    // depthwise: only the form with fp32 activations in and an int8 NHWC result out stages anything (the quantised input)
+    return d->group != 1 ? qb : pb + qb;
 }
 
 size_t onhip_conv2d_w8a32_packed_weight_bytes(const onhip_conv_desc_t *d) {
@@ -927,7 +928,6 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     if (twin && (!addend || d->cout % 16 || !(d->output_scale > 0.0f) || reinterpret_cast<uintptr_t>(twin) % 4 ||
                  (long long) d->n * OH * OW * d->cout >= (1LL << 31)))
         return set_error(ONHIP_ERR_ARG, "conv w8a32: the int8 twin goes with an addend, output channels in sixteens and an output_scale");
-    if ((xq || nhwc_out) && d->group != 1) return set_error(ONHIP_ERR_ARG, "conv w8a8: depthwise is not available in the NHWC int8 form");
     // the reference pads all four sides by pads[0] (conv.c:979-999) while shapes come from the four
     // pads: only uniform padding is self-consistent
     if (d->pad_t != d->pad_l || d->pad_t != d->pad_b || d->pad_t != d->pad_r)
@@ -938,8 +938,27 @@ static int conv2d_w8a32_impl(const onhip_conv_desc_t *d, const float *x, const i
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const Epilogue ep = make_epilogue(*d, silu_lut);
     if (d->group != 1) {
-        if (packed_w) return set_error(ONHIP_ERR_ARG, "conv w8a32: depthwise weights have no packed form");
-        return depthwise_w8a32_launch(*d, OH, OW, x, w8, bias32, weight_aux, ep, y, acc32, st);
+        // depthwise weights have no packed form: every entry point takes them as the reference holds them
+        if (!xq && !nhwc_out) return depthwise_w8a32_launch(*d, OH, OW, x, w8, bias32, weight_aux, ep, y, acc32, st);
+        // an int8 NHWC tensor on either side: the kernel of the chain form.  fp32 activations are quantised into the
+        // workspace first (the staging pass of the dense W8A32 form); an fp32 result is written NCHW by the kernel
+        if (acc32) return set_error(ONHIP_ERR_ARG, "conv w8a8: depthwise accumulators are available in the fp32 form only");
+        if (!dw_s8_ok(*d, OH, OW)) return set_error(ONHIP_ERR_ARG, "conv w8a8: depthwise with %d channels and a %dx%d filter is not available in the NHWC int8 form", d->cout, d->kh, d->kw);
+        const int cpd = (d->cin + 15) / 16 * 16;
+        const int8_t *q8 = xq;
+        if (!xq) {
+            const size_t need = (size_t) d->n * d->h * d->w * cpd;
+            if (!workspace || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16)
+                return set_error(ONHIP_ERR_WORKSPACE, "conv w8a8: depthwise needs a 16-byte aligned workspace of %zu bytes for the quantised input, %zu given",
+                                 need, workspace ? workspace_bytes : (size_t) 0);
+            rc = quantize_nhwc_launch(x, d->n, d->cin, d->h, d->w, cpd, 1.0f / d->input_scale, reinterpret_cast<int8_t *>(workspace), st);
+            if (rc) return rc;
+            q8 = reinterpret_cast<const int8_t *>(workspace);
+        } else if (reinterpret_cast<uintptr_t>(xq) % 16) {
+            return set_error(ONHIP_ERR_ARG, "conv w8a8: int8 activations must be 16-byte aligned");
+        }
+        if (nhwc_out && reinterpret_cast<uintptr_t>(y) % 16) return set_error(ONHIP_ERR_ARG, "conv w8a8: the int8 result must be 16-byte aligned");
+        return dw_s8_launch(*d, OH, OW, q8, w8, bias32, weight_aux, ep, y, st);
     }
 
     int cp, k_units;
@@ -1068,6 +1087,13 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
     onhip_conv_desc_t dd = *d;
     dd.out_s8 = 1;
     return conv2d_w8a32_impl(&dd, nullptr, xq, w8_packed, 1, bias32, weight_aux, silu_lut, yq, nullptr, nullptr, 0, 1, stream);
+}
+
+int onhip_conv2d_w8a8_depthwise_supported(const onhip_conv_desc_t *d) {
+    int32_t OH = 0, OW = 0;
+    if (!d || d->group == 1 || check_conv(d, &OH, &OW)) return 0;
+    if (d->pad_t != d->pad_l || d->pad_t != d->pad_b || d->pad_t != d->pad_r) return 0;
+    return dw_s8_ok(*d, OH, OW) ? 1 : 0;
 }
 
 int onhip_conv2d_w8_link(const onhip_conv_desc_t *d, const float *x, const int8_t *xq, const int8_t *w8_packed,

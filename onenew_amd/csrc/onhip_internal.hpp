@@ -244,6 +244,10 @@ int depthwise_f32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float
 int depthwise_w8a32_launch(const onhip_conv_desc_t &d, int OH, int OW, const float *x, const int8_t *w8,
                            const int32_t *bias32, const float *weight_aux, const Epilogue &ep, void *y,
                            int32_t *acc32, hipStream_t stream);
+// dw_s8.hip: depthwise convolution on int8 NHWC activations (the chain form's twin of depthwise_w8a32_launch)
+bool dw_s8_ok(const onhip_conv_desc_t &d, int OH, int OW);
+int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, const int8_t *w8, const int32_t *bias32,
+                 const float *weight_aux, const Epilogue &ep, void *y, hipStream_t stream);
 int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
                          hipStream_t stream);
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);

@@ -294,7 +294,8 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
 
     const bool in_s8 = link && link->in_s8, out_s8 = link && link->out_s8;
     if (link) {
-        if (!int8 || d.group != 1) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges are for dense int8 convolutions");
+        if (!int8) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges are for int8 convolutions");
+        if (d.group != 1 && (fuse || link->twin)) return set_error(ONHIP_ERR_ARG, "Conv eval: a depthwise int8 convolution takes no folded Add");
         if (out_s8 && fuse) return set_error(ONHIP_ERR_ARG, "Conv eval: an int8 result cannot take the Add of a residual block");
         if (out_s8 && !(link->out_scale > 0.0f)) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 result without a scale");
     }
@@ -351,7 +352,8 @@ static int conv_eval_fused(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_
         if (rc) return rc;
         bool added = false;   // the addend went into the convolution's store
         if (link || (fuse && wp)) {
-            if (!wp) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges need the packed weight form");
+            if (!wp && d.group == 1) return set_error(ONHIP_ERR_ARG, "Conv eval: int8 edges need the packed weight form");
+            if (!wp) wp = (const float *) w;   // depthwise: the weights as they are
             d.out_s8 = out_s8 ? 1 : 0;
             d.output_scale = link ? link->out_scale : 0.0f;
             int8_t *twin = nullptr;
@@ -574,6 +576,22 @@ static int matmul_eval_mode(int mode, BUFFER_INFO_S *params, BUFFER_INFO_S *inpu
     if (rc) return rc;
     if (!out_on_dev) return copy_out(host_out, y, o_bytes);
     return wait_for_output();
+}
+
+// `eval_link_takes`: reads params[0..2] only (configuration, input operand, weight operand); 1 when this convolution
+// can take and leave int8 NHWC activations through `eval_link`, 0 when it cannot (fp32, or a depthwise shape beyond the
+// int8 NHWC depthwise kernel)
+static int conv_link_takes(BUFFER_INFO_S *params) {
+    const CONV_CONFIG_S *cfg = reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr);
+    const OPERAND_S *in_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *w_t = reinterpret_cast<const OPERAND_S *>(params[2].addr);
+    if (!cfg || !in_t || !w_t || cfg->ifmap_quant2 != TYPE_INT8) return 0;
+    if (!cfg->has_bias || cfg->group == 1) return 1;   // conv.c:18-29: dense
+    onhip_conv_desc_t d;
+    block_conv_desc(&d, cfg, in_t->shapes[0] < 1 ? 1 : in_t->shapes[0], in_t->shapes[1], in_t->shapes[2], in_t->shapes[3], w_t);
+    int32_t oh = 0, ow = 0;
+    if (onhip_conv_out_shape(&d, &oh, &ow) != ONHIP_OK) return 0;
+    return onhip_conv2d_w8a8_depthwise_supported(&d);
 }
 
 static int matmul_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
@@ -974,6 +992,9 @@ int onhip_conv_add_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INF
 
 int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Conv + Add + Relu", conv_add_relu_eval_locked, params, inputs, outputs);
+}
+int onhip_conv_link_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *, BUFFER_INFO_S *) {
+    return params ? conv_link_takes(params) : 0;
 }
 int onhip_conv_link_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     return guarded("Conv (int8 edges)", conv_link_eval_locked, params, inputs, outputs);

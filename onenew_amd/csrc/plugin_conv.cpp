@@ -42,3 +42,10 @@ extern "C" __attribute__((visibility("default"))) int eval_link(BUFFER_INFO_S *p
                                                                 BUFFER_INFO_S *outputs) {
     return onhip_conv_link_eval(params, inputs, outputs);
 }
+
+// eval_link_takes: params[0..2] only, no tensors touched; 1 when eval_link can run this convolution (dense int8, or a
+// depthwise int8 shape the NHWC kernel takes), else 0.
+extern "C" __attribute__((visibility("default"))) int eval_link_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                      BUFFER_INFO_S *outputs) {
+    return onhip_conv_link_takes(params, inputs, outputs);
+}

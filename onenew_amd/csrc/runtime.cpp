@@ -172,7 +172,7 @@ struct onrt_net {
     long long runs = 0, graph_launches = 0;
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
-    onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr, conv_link = nullptr;
+    onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr, conv_link = nullptr, conv_link_takes = nullptr;
     onenew_eval_fn maxpool_s8 = nullptr;   // optional entry point of the MaxPool plugin
     onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr, matmul_bias_add = nullptr;   // optional entry points of the MatMul plugin
     int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0, int8_links = 0;
@@ -540,6 +540,7 @@ int bind_plugins(onrt_net &net) {
             net.conv_block = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block"));
             net.conv_block_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block_takes"));
             net.conv_link = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_link"));
+            net.conv_link_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_link_takes"));
         }
         if (type == "MaxPool") net.maxpool_s8 = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_s8"));
         if (type == "MatMul") {
@@ -812,27 +813,42 @@ int fuse_ir_blocks(onrt_net &net) {
 // returns fp32 (:1049-1056).  Where the result of a dense int8 Conv is read by dense int8 Convs only, all with the same
 // input_scale, that quantisation moves into the producer's store: the operand travels as int8 NHWC (a quarter of the
 // bytes, and no staging pass in the consumers), holding exactly the bytes each consumer would have made of the fp32
-// tensor, so the model's results do not change.  The Conv plugin's `eval_link` runs both ends.  Not for depthwise
-// convolutions (no NHWC int8 form), results that an Add is folded into, model outputs, or operands any other operator
-// reads.  Runs after the other folds; ONENEW_RT_FUSE=0 keeps every operand fp32 (layer-by-layer comparisons), and so
+// tensor, so the model's results do not change.  The Conv plugin's `eval_link` runs both ends.  Depthwise int8
+// convolutions (device/x86/Conv/conv.c:617-755) take part where the plugin's `eval_link_takes` says its NHWC kernel has
+// the shape, so a quantised MobileNetV2 moves int8 from the stem to the last projection.  Not for results that an Add is
+// folded into, model outputs, or operands any other operator reads.  Runs after the other folds; ONENEW_RT_FUSE=0 keeps every operand fp32 (layer-by-layer comparisons), and so
 // does ONENEW_RT_LINK=0 with the other folds in place.
 int link_int8_convs(onrt_net &net) {
     if (!fusing_enabled() || !net.conv_link) return ONRT_OK;
     if (const char *env = getenv("ONENEW_RT_LINK"))   // "0": the other folds without this one (measurements)
         if (!strcmp(env, "0")) return ONRT_OK;
     auto result_of = [](const Node &n) { return n.fused_out.empty() ? n.out[0] : n.fused_out; };
-    auto dense_int8 = [&](const Node &n) -> const CONV_CONFIG_S * {
+    // an int8 convolution `eval_link` can run: dense, or (with_depthwise) a depthwise one without a folded Add that the
+    // plugin's NHWC kernel takes
+    auto int8_conv = [&](const Node &n, bool with_depthwise) -> const CONV_CONFIG_S * {
         if (strcmp(n.kind->type, "Conv") || n.out.size() != 1 || n.in.size() < 2 || n.in.size() > 3 || n.fuse > 2) return nullptr;
         for (size_t k = 1; k < n.in.size(); ++k)
             if (n.in[k].empty() || !net.tensors[n.in[k]].is_init) return nullptr;
         if (net.tensors[n.in[0]].is_init) return nullptr;
         const CONV_CONFIG_S *cfg = reinterpret_cast<const CONV_CONFIG_S *>(n.cfg.data());
-        if (cfg->ifmap_quant2 != TYPE_INT8 || (cfg->has_bias && cfg->group != 1)) return nullptr;   // conv.c:18-29: depthwise
+        if (cfg->ifmap_quant2 != TYPE_INT8) return nullptr;
+        if (cfg->has_bias && cfg->group != 1) {   // conv.c:18-29: depthwise
+            if (!with_depthwise || n.fuse != 0 || !net.conv_link_takes) return nullptr;
+            BUFFER_INFO_S prm[BUF_MAXNUM], none[BUF_MAXNUM];
+            memset(prm, 0, sizeof(prm));
+            memset(none, 0, sizeof(none));
+            prm[0].addr = (int64_t) n.cfg.data();
+            prm[1].addr = (int64_t) &net.tensors[n.in[0]].desc;
+            prm[2].addr = (int64_t) &net.tensors[n.in[1]].desc;
+            if (net.conv_link_takes(prm, none, none) != 1) return nullptr;
+        }
         return cfg;
     };
+    auto dense_int8 = [&](const Node &n) { return int8_conv(n, false); };
+    auto any_int8 = [&](const Node &n) { return int8_conv(n, true); };
     for (int idx : net.order) {
         Node &p = net.nodes[idx];
-        if (!dense_int8(p) || p.fuse != 0) continue;
+        if (!any_int8(p) || p.fuse != 0) continue;
         const std::string name = result_of(p);
         if (is_net_output(net, name) || net.tensors[name].desc.not_need_buf) continue;
         const std::vector<int> readers = readers_of(net, name);
@@ -840,7 +856,7 @@ int link_int8_convs(onrt_net &net) {
         float scale = 0.0f;
         for (int ri : readers) {
             const Node &c = net.nodes[ri];
-            const CONV_CONFIG_S *cc = dense_int8(c);
+            const CONV_CONFIG_S *cc = any_int8(c);
             if (!cc || c.in[0] != name || !(cc->input_scale > 0.0f) || (scale != 0.0f && cc->input_scale != scale)) { ok = false; break; }
             scale = cc->input_scale;
         }
@@ -914,7 +930,7 @@ int link_int8_convs(onrt_net &net) {
         std::vector<int> takers;
         for (int ri : readers_of(net, name)) {
             const Node &c = net.nodes[ri];
-            const CONV_CONFIG_S *cc = dense_int8(c);
+            const CONV_CONFIG_S *cc = any_int8(c);
             if (!cc || c.in[0] != name || c.link.in_s8) continue;            // reads the fp32 tensor
             if (!(cc->input_scale > 0.0f) || (scale != 0.0f && cc->input_scale != scale)) { ok = false; break; }
             scale = cc->input_scale;

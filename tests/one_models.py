@@ -191,6 +191,49 @@ def quantised_chain(n=1, hw=18, different_scales=False, extra_reader=False, tail
     return m.tobytes(), [_r("xqc", (n, 16, hw, hw))]
 
 
+def quantised_mobile(n=1, hw=24, scales_differ=False):
+    """MobileNetV2 in small, every convolution W8A32: dense 3x3 stride-2 stem, a depthwise + projection pair, an expanding
+    block with a stride-2 depthwise layer and one with the skip connection (its sum is read by an int8 convolution and is
+    a net output), 5x5 depthwise in the last block.  Every operand between two convolutions can travel as int8, the
+    depthwise ones included.  scales_differ: the second depthwise layer quantises its input with another scale than the
+    expansion's other reader, so that operand stays fp32"""
+    from oracle import oracle
+    m = onefile.OneModel()
+    m.input("x", (n, 3, hw, hw))
+    clip = dict(act=abi.CLIP, clip=(0.0, 6.0))
+
+    def q(tag, shape, scale):
+        w = _r("qm_" + tag + "w", shape, scale)
+        b = _r("qm_" + tag + "b", (shape[0],), 0.2)
+        return oracle.quant_weight_bias(w, b)
+
+    def cv(name, x, out, shape, wscale, in_scale, **kw):
+        w8, b32, aux = q(name, shape, wscale)
+        m.conv(name, x, w8, b32, out, quant=(aux, in_scale), **kw)
+
+    h1 = (hw + 2 - 3) // 2 + 1
+    cv("stem", "x", "stem_out", (20, 3, 3, 3), 0.3, 0.02, stride=2, pad=1, **clip)
+    cv("dw0", "stem_out", "dw0_out", (20, 1, 3, 3), 0.3, 0.03, pad=1, group=20, **clip)
+    cv("pw0", "dw0_out", "pw0_out", (16, 20, 1, 1), 0.2, 0.04)
+    cv("e1", "pw0_out", "e1_out", (48, 16, 1, 1), 0.3, 0.05, **clip)
+    cv("dw1", "e1_out", "dw1_out", (48, 1, 3, 3), 0.3, 0.035, stride=2, pad=1, group=48, **clip)
+    if scales_differ:   # a second reader of the expansion with another input_scale: e1_out stays fp32
+        cv("side", "e1_out", "side_out", (8, 48, 1, 1), 0.2, 0.05, act=abi.RELU)
+        m.output("side_out", (n, 8, h1, h1))
+    h2 = (h1 + 2 - 3) // 2 + 1
+    cv("p1", "dw1_out", "p1_out", (24, 48, 1, 1), 0.2, 0.045)
+    cv("e2", "p1_out", "e2_out", (72, 24, 1, 1), 0.3, 0.05, **clip)
+    cv("dw2", "e2_out", "dw2_out", (72, 1, 3, 3), 0.3, 0.04, pad=1, group=72, **clip)
+    cv("p2", "dw2_out", "p2_out", (24, 72, 1, 1), 0.2, 0.045)
+    m.add("skip", "p2_out", "p1_out", "b2_out")
+    m.output("b2_out", (n, 24, h2, h2))
+    cv("e3", "b2_out", "e3_out", (40, 24, 1, 1), 0.3, 0.06, act=abi.SILU)
+    cv("dw3", "e3_out", "dw3_out", (40, 1, 5, 5), 0.2, 0.03, pad=2, group=40, act=abi.RELU)
+    cv("p3", "dw3_out", "out", (32, 40, 1, 1), 0.2, 0.05)
+    m.output("out", (n, 32, h2, h2))
+    return m.tobytes(), [_r("xqm", (n, 3, hw, hw))]
+
+
 def quantised_stem(n=1, hw=21):
     """a quantised stem: dense int8 Conv (7x7 stride 2, Relu) -> MaxPool 3x3 stride 2 -> two dense int8 convolutions with
     one input_scale; the operands either side of the MaxPool can travel as int8"""
@@ -254,7 +297,7 @@ def attention_heads(heads=3, tokens=40, head_dim=64, batch=2, scores_also_output
     return m.tobytes(), [_r(n + str(tokens), shape, 0.5) for n in ("q", "k", "v")]
 
 
-MODELS = {"quantised_block": quantised_block, "quantised_chain": quantised_chain, "quantised_stem": quantised_stem, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
+MODELS = {"quantised_block": quantised_block, "quantised_mobile": quantised_mobile, "quantised_chain": quantised_chain, "quantised_stem": quantised_stem, "resnet_block": resnet_block, "mobile_block": mobile_block, "vit_block": vit_block, "two_inputs": two_inputs}
 
 
 def unfused_activations(optimised=False):

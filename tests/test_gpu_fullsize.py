@@ -432,3 +432,42 @@ def test_yolov8s_int8_batch16_every_layer(layer, torch_dev, oracle):
     # and, over the whole tensor, the chain form is the quantisation of the fp32 form's result (same accumulators)
     want = hip.quantize_nhwc_s8(y_full, dq.output_scale)
     assert torch.equal(out[..., :d.cout], want[..., :d.cout]), f"{name}: chain form is not the quantised fp32 form everywhere"
+
+
+# ---- MobileNetV2 depthwise layers in the int8 NHWC chain form, batch 64 -------------------------------------------------
+DW_LAYERS = [i for i, (_, d) in enumerate(MOBILENET) if d.group != 1]
+
+
+@pytest.mark.parametrize("layer", DW_LAYERS, ids=[MOBILENET[i][0] for i in DW_LAYERS])
+def test_mobilenetv2_batch64_depthwise_int8_chain_form(layer, torch_dev, oracle):
+    """every depthwise layer with int8 NHWC activations in and out (conv.c:617-755 + the consumer's quantiser :961-973):
+    three whole images against the oracle bit for bit, and over the whole batch the int8 result is the quantisation of what
+    the fp32-in / fp32-out form of the same layer returns (that form is checked against the oracle the same way)"""
+    torch = torch_dev
+    name, d0 = MOBILENET[layer]
+    print(f"mobilenetv2 b64 int8 {name}", flush=True)
+    d = ConvDesc.from_buffer_copy(d0)
+    d.input_scale = 0.021
+    x = _device_uniform(torch, _seed("mbv2q", name, "x"), (d.n, d.cin, d.h, d.w)) * 3.0      # a few per cent clip at +-127
+    w8 = datagen.integers(_seed("mbv2q", name, "w"), (d.cout, 1, d.kh, d.kw), -127, 127).astype(np.int8)
+    b32 = datagen.integers(_seed("mbv2q", name, "b"), (d.cout,), -300, 300).astype(np.int32)
+    aux = datagen.uniform(_seed("mbv2q", name, "aux"), (d.cout,), 0.5, 3.0)
+    cu = lambda t: torch.from_numpy(t).cuda()   # noqa: E731
+    w8d, b32d, auxd = cu(w8), cu(b32), cu(aux)
+    y32 = hip.conv2d_w8a32(d, x, w8d, b32d, auxd)
+    dq = ConvDesc.from_buffer_copy(d)
+    dq.out_s8, dq.output_scale = 1, 0.045
+    xq = hip.quantize_nhwc_s8(x, d.input_scale)
+    oh, ow = d.out_hw()
+    cp = (d.cout + 15) // 16 * 16
+    out = torch.full((d.n, oh, ow, cp), 77, dtype=torch.int8, device="cuda")
+    hip.conv2d_w8a8_nhwc(dq, xq, w8d, b32d, auxd, out=out)
+    torch.cuda.synchronize()
+    d1 = ConvDesc.from_buffer_copy(dq)
+    d1.n = 1
+    for img in sorted({0, d.n - 1, int(datagen.integers(_seed("mbv2q", name, "img"), (1,), 0, d.n - 1)[0])}):
+        ref = oracle.conv2d_w8a32(d1, x[img:img + 1].cpu().numpy(), w8, b32, aux)            # int8 NCHW
+        assert np.array_equal(out[img, :, :, :d.cout].cpu().numpy(), np.transpose(ref[0], (1, 2, 0))), f"{name}: image {img}"
+    want = hip.quantize_nhwc_s8(y32, dq.output_scale)
+    assert torch.equal(out[..., :d.cout], want[..., :d.cout]), f"{name}: not the quantised fp32 form everywhere"
+    assert not bool(out[..., d.cout:].any())

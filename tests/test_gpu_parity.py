@@ -1443,3 +1443,60 @@ def test_maxpool_on_int8_nhwc_is_the_quantised_fp32_maxpool(shape, torch_dev):
     got = hip.maxpool_s8_nhwc(d, hip.quantize_nhwc_s8(dev(torch, x), scale))
     torch.cuda.synchronize()
     assert np.array_equal(got.cpu().numpy()[..., :c], want.cpu().numpy()[..., :c])
+
+
+# ---- depthwise convolutions in the int8 NHWC chain form ---------------------------------------------------------
+# (channels, height, width, filter, stride, pad, activation, batch): channel counts inside and beyond one 16-channel
+# group, MobileNetV2's (32, 96, 144, 960), strides 1 / 2 (the unrolled 3x3 kernels) and 3, 5x5 and 7x7 (the generic one),
+# planes narrower than a wavefront and wider, output rows that do not fill the last strip of a lane
+DW_CHAIN = [(12, 11, 11, 3, 1, 1, abi.SILU, 2), (10, 14, 14, 3, 2, 1, abi.CLIP, 3), (6, 9, 9, 5, 1, 2, abi.NOT_ACT, 2),
+            (32, 28, 28, 3, 1, 1, abi.CLIP, 2), (96, 30, 26, 3, 2, 1, abi.CLIP, 2), (144, 13, 17, 3, 1, 1, abi.RELU, 1),
+            (960, 7, 7, 3, 1, 1, abi.CLIP, 3), (24, 70, 70, 3, 1, 1, abi.LEAKYRELU, 1), (40, 15, 15, 3, 3, 1, abi.HARDSILU, 2),
+            (17, 12, 12, 7, 2, 3, abi.RELU, 2), (48, 5, 5, 3, 1, 1, abi.SILU, 9), (200, 9, 20, 5, 2, 2, abi.CLIP, 2),
+            (16, 6, 130, 3, 2, 1, abi.NOT_ACT, 1), (64, 1, 1, 3, 1, 1, abi.RELU, 70)]
+
+
+def _dw_chain_desc(shape):
+    c, h, w, k, s, pad, act, n = shape
+    d = cases.cd(c, c, k, s, pad, h, w, act=act, group=c, n=n, input_scale=0.013, clip_min=0.0, clip_max=6.0,
+                 leaky_relu_alpha=0.1, hard_sigmoid_alpha=0.2, hard_sigmoid_beta=0.5)
+    return d
+
+
+@pytest.mark.parametrize("shape", DW_CHAIN, ids=["x".join(map(str, s)) for s in DW_CHAIN])
+def test_depthwise_w8a8_nhwc_chain_form(shape, torch_dev, oracle):
+    """depthwise int8 convolutions with int8 NHWC on both sides (conv.c:617-755 followed by the consumer's quantiser,
+    :961-973): the reference's int8 values exactly, padding channels zero, and the two mixed forms of a model edge (fp32
+    NCHW in / int8 NHWC out, int8 NHWC in / fp32 NCHW out) equal to the reference's fp32 result and its quantisation"""
+    torch = torch_dev
+    d = _dw_chain_desc(shape)
+    name = "dwchain_" + "x".join(map(str, shape))
+    x, w8, b32, aux = cases.conv_inputs(name, d, quant=True)
+    lut = cases.silu_lut()
+    ref32 = oracle.conv2d_w8a32(d, x, w8, b32, aux, lut)                    # fp32 NCHW
+    dq = ConvDesc.from_buffer_copy(d)
+    dq.out_s8, dq.output_scale = 1, 0.037
+    ref8 = oracle.conv2d_w8a32(dq, x, w8, b32, aux, lut)                    # int8 NCHW
+    assert np.array_equal(ref8, oracle.quantize_s8(ref32, dq.output_scale))
+    xd, wd, bd, ad, ld = dev(torch, x), dev(torch, w8), dev(torch, b32), dev(torch, aux), dev(torch, lut)
+    xq = hip.quantize_nhwc_s8(xd, d.input_scale)
+    oh, ow = d.out_hw()
+    cp = (d.cout + 15) // 16 * 16
+    out = torch.full((d.n, oh, ow, cp), 77, dtype=torch.int8, device="cuda")
+    hip.conv2d_w8a8_nhwc(dq, xq, wd, bd, ad, ld, out=out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got[..., :d.cout], np.transpose(ref8, (0, 2, 3, 1))), f"{name}: int8 values differ"
+    assert not got[..., d.cout:].any(), f"{name}: padding channels are not zero"
+    # int8 in, fp32 out
+    y32 = hip.conv2d_w8_link(d, wd, bd, ad, ld, xq=xq)
+    torch.cuda.synchronize()
+    assert np.array_equal(y32.cpu().numpy(), ref32), f"{name}: fp32 result from int8 activations differs"
+    # fp32 in, int8 out
+    y8 = hip.conv2d_w8_link(dq, wd, bd, ad, ld, x=xd)
+    torch.cuda.synchronize()
+    assert np.array_equal(y8.cpu().numpy(), got), f"{name}: int8 result from fp32 activations differs"
+    # and the fp32 form is untouched by all this
+    y = hip.conv2d_w8a32(d, xd, wd, bd, ad, ld)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), ref32)

@@ -48,7 +48,7 @@ def test_model_outputs_match_oracle(name, torch_dev, monkeypatch):
     for (oname, _), got in zip(net.outputs, outs):
         assert got.shape == ref[oname].shape
         assert _close(got, ref[oname], 5e-4), oname                          # up to five MFMA operators deep, 1e-4 each
-        if name in ("quantised_block", "quantised_chain", "quantised_stem"):
+        if name in ("quantised_block", "quantised_chain", "quantised_stem", "quantised_mobile"):
             assert np.array_equal(got, ref[oname])                           # integer accumulation: the chain is exact
     # every intermediate operand sits in device memory and holds what the oracle computed at that point
     for op_type, cfg in m["nodes"]:
@@ -775,3 +775,41 @@ def test_maxpool_between_int8_convolutions_runs_on_int8(torch_dev):
         for (oname, _), got in zip(net.outputs, net.run(*ins)):
             assert np.array_equal(got, ref[oname]), oname
         net.close()
+
+
+@pytest.mark.gpu
+def test_depthwise_int8_convolutions_take_part_in_the_int8_edges(torch_dev, monkeypatch):
+    """a quantised MobileNetV2-style model: the operands around its depthwise convolutions (conv.c:617-755) travel as int8
+    NHWC like those between dense ones, so everything from the stem to the last projection is int8 except the sum of the
+    skip connection; the outputs equal the oracle's evaluation with every operand fp32 and the runtime's own with the
+    edges off, bit for bit.  A reader with another input_scale keeps that one operand fp32."""
+    for n, hw in ((2, 24), (1, 37)):
+        data, ins = one_models.quantised_mobile(n=n, hw=hw)
+        net = rt.Net(data)
+        # stem, dw0, pw0, e1, dw1 | p1 (read by e2 and, as the Add's operand, by p2: stays fp32), e2, dw2 | e3, dw3
+        assert net.int8_links() == 9, net.int8_links()
+        outs = net.run(*ins)
+        outs2 = net.run(*ins)
+        ref = one_model.run(data, ins, keep_all=True)
+        for (oname, _), got, got2 in zip(net.outputs, outs, outs2):
+            assert np.array_equal(got, ref[oname]), oname
+            assert np.array_equal(got2, got)
+        net.close()
+    data, ins = one_models.quantised_mobile()
+    monkeypatch.setenv("ONENEW_RT_LINK", "0")
+    plain = rt.Net(data)
+    assert plain.int8_links() == 0
+    want = plain.run(*ins)
+    plain.close()
+    monkeypatch.delenv("ONENEW_RT_LINK")
+    net = rt.Net(data)
+    for a, b in zip(net.run(*ins), want):
+        assert np.array_equal(a, b)
+    net.close()
+    data, ins = one_models.quantised_mobile(scales_differ=True)
+    net = rt.Net(data)
+    assert net.int8_links() == 8
+    ref = one_model.run(data, ins, keep_all=True)
+    for (oname, _), got in zip(net.outputs, net.run(*ins)):
+        assert np.array_equal(got, ref[oname]), ("scales differ", oname)
+    net.close()
