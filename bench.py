@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--layers]
 
 Workloads: resnet50_b{1,32} (default: the ResNet-50 conv stack, fp32, batch 32),
-cfg1, resnet50_net_b{1,32}, resnet50_int8_net_b{1,32} (the same with W8A32 convolutions), mobilenetv2_net_b{1,64} and vit_tiny_net_b{1,64} (the whole model as a .one file through the runtime), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
+cfg1, resnet50_net_b{1,32}, mobilenetv2_net_b{1,64} and vit_tiny_net_b{1,64} (the whole model as a .one file through the runtime), resnet50_int8_net_b{1,32} and mobilenetv2_int8_net_b{1,64} (the same files through the model-level quantisation step: W8A32 convolutions with calibrated scales), mobilenetv2_b{1,64}, yolov8s_int8_b{1,16}, vit_tiny_b{1,64}[_bf16|_f16], and `copy` (the yardstick
 the HBM traffic counters are scaled by).
 
 A step is one pass over every layer of the workload: one launch per layer, inputs, weights and outputs
@@ -651,12 +651,21 @@ def net_result(torch, workload, steps, warmup, with_cpu):
     n = int(workload.split("_b")[1])
     model = "ResNet-50" if workload.startswith("resnet50") else "MobileNetV2" if workload.startswith("mobilenetv2") else "ViT-Tiny"
     make = {"ResNet-50": stacks.resnet50_model, "MobileNetV2": stacks.mobilenet_v2_model, "ViT-Tiny": stacks.vit_tiny_model}[model]
-    int8 = "_int8_net_" in workload   # the convolutions in the W8A32 form of the offline quantiser
-    if int8:
-        make = lambda batch: stacks.resnet50_model(batch, quantised=True)   # noqa: E731
+    int8 = "_int8_net_" in workload   # every convolution in the W8A32 form the offline quantiser writes
     data, in_shape, flops = make(n)
-    net = rt.Net(data)
     x = torch.randn(in_shape, dtype=torch.float32, device="cuda")
+    calibration = None
+    if int8:
+        # the model-level quantisation step on the fp32 file (tools/optimize/model_quant.hpp:625-679): activation scales
+        # from the KL search over two calibration batches drawn like the input, weights / bias / weight_aux per channel
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1234)
+        cal = [torch.randn(in_shape, generator=g, dtype=torch.float32, device="cuda") for _ in range(2)]
+        t0 = time.perf_counter()
+        data = rt.quantise(data, [c.data_ptr() for c in cal], rt.QUANT_KL)
+        calibration = {"method": "KL", "batches": len(cal), "seconds": round(time.perf_counter() - t0, 2)}
+        del cal
+    net = rt.Net(data)
     y = torch.empty((n, 1000), dtype=torch.float32, device="cuda")
     ins, outs = [x.data_ptr()], [y.data_ptr()]
     for _ in range(max(2, warmup)):     # the first inferences measure tile choices and pack the weights
@@ -699,6 +708,8 @@ def net_result(torch, workload, steps, warmup, with_cpu):
                          "frac": round(flops / (dev * 1e-3) / 1e12 / PEAK["i8" if int8 else "f32"], 4), "traffic": None,
                          "launches": len(ops), "device_ms_per_inference": round(dev, 4)},
             "cpu_baseline": cpu, "images_per_s": round(n / (ms_per_step * 1e-3), 1)}
+    if calibration:
+        line["calibration"] = calibration
     net.close()
     return line
 
@@ -709,7 +720,7 @@ METRIC = {"resnet50_glue": "resnet50_glue_ops_fp32_tflops", "vit_tiny_glue": "vi
           "vit": "vit_tiny_matmul_{dtype}_tflops", "cfg1": "conv2d_relu_{dtype}_tflops"}
 
 # the other configurations of the benchmark, timed after the headline one in a default run
-NET_CONFIGS = ["resnet50_net_b32", "resnet50_int8_net_b32", "mobilenetv2_net_b64", "vit_tiny_net_b64"]
+NET_CONFIGS = ["resnet50_net_b32", "resnet50_int8_net_b32", "mobilenetv2_net_b64", "mobilenetv2_int8_net_b64", "vit_tiny_net_b64"]
 OTHER_CONFIGS = ["cfg1", "cfg1_bf16", "resnet50_b1", "resnet50_b32_bf16", "mobilenetv2_b64", "mobilenetv2_b1", "vit_tiny_b64", "vit_tiny_b64_bf16", "vit_tiny_b1",
                  "yolov8s_int8_b16", "yolov8s_int8chain_b16", "yolov8s_int8chain_b1"]
 
@@ -867,7 +878,7 @@ def main():
                           "bytes_written_per_launch": src.numel() * 4, "launches": args.warmup + args.steps}))
         return
 
-    if args.workload.startswith(("resnet50_net_b", "resnet50_int8_net_b", "mobilenetv2_net_b", "vit_tiny_net_b")):
+    if args.workload.startswith(("resnet50_net_b", "resnet50_int8_net_b", "mobilenetv2_net_b", "mobilenetv2_int8_net_b", "vit_tiny_net_b")):
         return bench_net(torch, args)
 
     res = run_workload(torch, hip, args.workload, args.steps, args.warmup, layers_table=args.layers, graph=not args.no_graph)

@@ -191,6 +191,30 @@ int onrt_net_get_tiles(const onrt_net_t *net, int32_t tiles[3]);
 int onrt_net_set_tiles(onrt_net_t *net, const int32_t tiles[3]);
 int onrt_one_set_tiles(void *one_buf, size_t bytes, const int32_t tiles[3]);
 
+/*
+ * Model-level quantisation, the counterpart of model_quant (tools/optimize/model_quant.hpp:625-679): from an fp32 .one
+ * image and calibration inputs to the W8A32 image the reference's optimiser writes.  The fp32 model is loaded with every
+ * operator separate and run on each calibration input; for the input operand of every Conv the statistics of `method`
+ * are taken on the device (the calibration passes of the kernel library, libonenew_hip.so beside the plugins):
+ *   ONRT_QUANT_KL / ONRT_QUANT_MSE: the largest magnitude over `images` (first pass, :276-300), then the 2048-bin
+ *     histogram of |x| over `images2` (second pass, :302-337; NULL = the same inputs again - the reference goes on
+ *     reading its image list where the first pass stopped), then the KL (:345-431) or MSE (:585-618) threshold search;
+ *   ONRT_QUANT_PERCENT: the 99.998 % magnitude over all of `images` (:83-185).
+ * Then, as :657-670 and :31-81, every Conv gets input_scale = threshold / 127 and ifmap_quant2 = int8, its weights become
+ * int8 (at the front of the initialiser, which keeps its fp32 size and type) with weight_aux = max |w| per output channel,
+ * its bias int32 (quant_weight_bias, :6-29).  images / images2: n_images x (number of model inputs) pointers, input k of
+ * calibration item i at [i * inputs + k], each a tensor of that input's shape in host or device memory.
+ * quant_one_buf receives `bytes` bytes: the quantised image, loadable like any other.  A Conv that is int8 already is
+ * refused.  The bytes behind the int8 weights inside their initialiser are zero here (the reference leaves the remains of
+ * its in-place conversion there; nothing reads them).
+ */
+#define ONRT_QUANT_KL 0
+#define ONRT_QUANT_MSE 1
+#define ONRT_QUANT_PERCENT 2
+int onrt_one_quantise(const void *one_buf, size_t bytes, const char *op_lib_dir, int32_t method,
+                      const void *const *images, int32_t n_images, const void *const *images2, int32_t n_images2,
+                      void *quant_one_buf);
+
 #ifdef __cplusplus
 }
 #endif

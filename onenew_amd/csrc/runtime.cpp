@@ -559,7 +559,9 @@ int bind_plugins(onrt_net &net) {
 // reference's kernel would apply the activation: a convolution with a bias (conv.c:18-27 returns before do_act without
 // one) and no activation yet, whose result only the Relu reads.  As in the optimised file, the activation is then
 // do_act's "x > 0 ? x : 0" (a NaN becomes 0) instead of relu.c's vector rule.  ONENEW_RT_FUSE=0 leaves the file as it is.
+thread_local bool tl_load_unfused = false;   // set around the load inside onrt_one_quantise: every operand gets a buffer
 bool fusing_enabled() {
+    if (tl_load_unfused) return false;
     const char *env = getenv("ONENEW_RT_FUSE");
     return !(env && !strcmp(env, "0"));
 }
@@ -1586,6 +1588,188 @@ ONRT_API int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *cons
     }
     // a blocking copy has already waited for the operators; otherwise wait here: results are complete on return
     if (!copied) ONRT_HIP(hipStreamSynchronize(nullptr));
+    return ONRT_OK;
+}
+
+// ---- model-level quantisation (tools/optimize/model_quant.hpp:625-679) ----------------------------------------------
+// The reference copies the fp32 file, runs it on the calibration images collecting, for the input operand of every Conv,
+// the statistics of the chosen method (abs-max and a 2048-bin histogram for KL :197-435 and MSE :437-623; the largest
+// magnitudes for the percentile :83-185), turns them into a clipping threshold per operand, writes
+// input_scale = threshold / 127 and ifmap_quant2 = int8 into every Conv (:657-670) and quantises every Conv's weights and
+// bias in place (:31-81, :6-29).  Here the fp32 model runs on the device through the operator plugins with every
+// operator separate, the statistics are taken where the operands lie (the calibration kernels of the kernel library),
+// and the file image is rewritten on the host.
+namespace {
+typedef size_t (*calib_ws_fn)(int);
+typedef int (*calib_absmax_fn)(const float *, long long, float *, void *, size_t, void *);
+typedef int (*calib_hist_fn)(const float *, long long, float, float *, void *, size_t, void *);
+typedef int (*calib_thr_fn)(int, const float *, long long, float, float *);
+typedef int (*calib_pct_fn)(const float *, int, int, float *, void *, size_t, void *);
+typedef int (*quant_wb_fn)(const float *, const float *, int32_t, int32_t, int8_t *, int32_t *, float *);
+typedef const char *(*last_error_fn)(void);
+
+struct KernelLib {
+    calib_ws_fn ws = nullptr;
+    calib_absmax_fn abs_max = nullptr;
+    calib_hist_fn hist = nullptr;
+    calib_thr_fn thr = nullptr;
+    calib_pct_fn pct = nullptr;
+    quant_wb_fn quant_wb = nullptr;
+    last_error_fn err = nullptr;
+};
+
+int bind_kernel_lib(const std::string &dir, KernelLib *k) {
+    const std::string path = dir + "/libonenew_hip.so";
+    void *h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!h) return fail(ONRT_ERR_PLUGIN, "quantise: %s", dlerror());
+    k->ws = reinterpret_cast<calib_ws_fn>(dlsym(h, "onhip_calib_workspace_bytes"));
+    k->abs_max = reinterpret_cast<calib_absmax_fn>(dlsym(h, "onhip_calib_abs_max"));
+    k->hist = reinterpret_cast<calib_hist_fn>(dlsym(h, "onhip_calib_histogram"));
+    k->thr = reinterpret_cast<calib_thr_fn>(dlsym(h, "onhip_calib_threshold"));
+    k->pct = reinterpret_cast<calib_pct_fn>(dlsym(h, "onhip_calib_percentile"));
+    k->quant_wb = reinterpret_cast<quant_wb_fn>(dlsym(h, "onhip_quant_weight_bias"));
+    k->err = reinterpret_cast<last_error_fn>(dlsym(h, "onhip_last_error"));
+    if (!k->ws || !k->abs_max || !k->hist || !k->thr || !k->pct || !k->quant_wb || !k->err)
+        return fail(ONRT_ERR_PLUGIN, "quantise: %s lacks the calibration entry points", path.c_str());
+    return ONRT_OK;
+}
+
+// offset in the file of the data of the initialiser called `name` and its descriptor, or 0
+size_t find_initialiser(const std::vector<char> &file, const char *name, OPERAND_S *desc) {
+    const ONE_MODEL_DESC_S *h = reinterpret_cast<const ONE_MODEL_DESC_S *>(file.data());
+    size_t off = (size_t) h->init_info_offset;
+    for (int i = 0; i < h->init_cnt; ++i) {
+        OPERAND_S d;
+        memcpy(&d, file.data() + off, sizeof(d));
+        d.operand_name[OPERAND_NAME_LEN - 1] = 0;
+        if (!strcmp(d.operand_name, name)) {
+            *desc = d;
+            return off + sizeof(OPERAND_S);
+        }
+        off += align64(sizeof(OPERAND_S) + (size_t) numel(d) * elem_bytes(d.data_type));
+    }
+    return 0;
+}
+}  // namespace
+
+ONRT_API int onrt_one_quantise(const void *one_buf, size_t bytes, const char *op_lib_dir, int32_t method,
+                               const void *const *images, int32_t n_images, const void *const *images2, int32_t n_images2,
+                               void *quant_one_buf) {
+    if (!one_buf || !quant_one_buf || !images || n_images < 1) return fail(ONRT_ERR_ARG, "quantise: null argument or no calibration image");
+    if (method != ONRT_QUANT_KL && method != ONRT_QUANT_MSE && method != ONRT_QUANT_PERCENT) return fail(ONRT_ERR_ARG, "quantise: unknown method %d", method);
+    if (!images2) { images2 = images; n_images2 = n_images; }
+    if (n_images2 < 1) return fail(ONRT_ERR_ARG, "quantise: no image for the second pass");
+    // the fp32 model with every operator separate: each Conv's input operand is a tensor of its own in device memory
+    onrt_net_t *net = nullptr;
+    tl_load_unfused = true;
+    int rc = onrt_net_load_buf(one_buf, bytes, op_lib_dir, &net);
+    tl_load_unfused = false;
+    if (rc) return rc;
+    struct Guard { onrt_net_t *n; void *ws = nullptr; std::vector<void *> bufs; ~Guard() { for (void *b : bufs) (void) hipFree(b); if (ws) (void) hipFree(ws); onrt_net_free(n); } } guard{net};
+    KernelLib k;
+    rc = bind_kernel_lib(net->lib_dir, &k);
+    if (rc) return rc;
+    // the input operands of the Conv nodes, in file order, each once
+    std::vector<std::string> names;
+    for (const Node &nd : net->nodes) {
+        if (strcmp(nd.kind->type, "Conv")) continue;
+        if (reinterpret_cast<const CONV_CONFIG_S *>(nd.cfg.data())->ifmap_quant2 == TYPE_INT8)
+            return fail(ONRT_ERR_ARG, "quantise: Conv %s is quantised already", nd.base()->op_name);
+        if (std::find(names.begin(), names.end(), nd.in[0]) == names.end()) names.push_back(nd.in[0]);
+    }
+    if (names.empty()) return fail(ONRT_ERR_ARG, "quantise: the model has no Conv");
+    for (const std::string &nm : names) {
+        const Tensor &t = net->tensors[nm];
+        if (!t.dev || numel(t.desc) < 1 || numel(t.desc) >= (1LL << 31)) return fail(ONRT_ERR_FORMAT, "quantise: operand %s has no buffer", nm.c_str());
+    }
+    const size_t n_in = net->in_names.size();
+    std::vector<void *> outs(net->out_names.size(), nullptr);
+    const size_t ws_bytes = k.ws(method == ONRT_QUANT_PERCENT ? n_images : 1);
+    ONRT_HIP(hipMalloc(&guard.ws, ws_bytes ? ws_bytes : 16));
+    std::map<std::string, float> threshold;
+    auto lib_fail = [&](const char *what) { return fail(ONRT_ERR_RUNTIME, "quantise: %s: %s", what, k.err()); };
+    if (method == ONRT_QUANT_PERCENT) {
+        // one pass: every image's copy of every operand is kept, [image][element], for the selection over all of them
+        std::map<std::string, float *> store;
+        for (const std::string &nm : names) {
+            void *b = nullptr;
+            ONRT_HIP(hipMalloc(&b, (size_t) n_images * numel(net->tensors[nm].desc) * 4));
+            guard.bufs.push_back(b);
+            store[nm] = static_cast<float *>(b);
+        }
+        for (int i = 0; i < n_images; ++i) {
+            rc = onrt_net_run(net, images + (size_t) i * n_in, outs.data());
+            if (rc) return rc;
+            for (const std::string &nm : names) {
+                const size_t n = (size_t) numel(net->tensors[nm].desc);
+                ONRT_HIP(hipMemcpy(store[nm] + (size_t) i * n, net->tensors[nm].dev, n * 4, hipMemcpyDeviceToDevice));
+            }
+        }
+        for (const std::string &nm : names) {
+            float thr = 0.0f;
+            if (k.pct(store[nm], n_images, (int) numel(net->tensors[nm].desc), &thr, guard.ws, ws_bytes, nullptr)) return lib_fail("percentile");
+            threshold[nm] = thr;
+        }
+    } else {
+        std::map<std::string, float> max_abs;
+        std::map<std::string, std::vector<float>> hist;
+        for (const std::string &nm : names) { max_abs[nm] = 0.0f; hist[nm].assign(2048, 0.0f); }
+        for (int i = 0; i < n_images; ++i) {          // model_quant.hpp:276-300: the largest magnitude of every operand
+            rc = onrt_net_run(net, images + (size_t) i * n_in, outs.data());
+            if (rc) return rc;
+            for (const std::string &nm : names)
+                if (k.abs_max(static_cast<const float *>(net->tensors[nm].dev), numel(net->tensors[nm].desc), &max_abs[nm], guard.ws, ws_bytes, nullptr)) return lib_fail("abs-max");
+        }
+        for (int i = 0; i < n_images2; ++i) {         // :302-337: the histogram of every operand over [0, that maximum]
+            rc = onrt_net_run(net, images2 + (size_t) i * n_in, outs.data());
+            if (rc) return rc;
+            for (const std::string &nm : names)
+                if (k.hist(static_cast<const float *>(net->tensors[nm].dev), numel(net->tensors[nm].desc), max_abs[nm], hist[nm].data(), guard.ws, ws_bytes, nullptr)) return lib_fail("histogram");
+        }
+        for (const std::string &nm : names) {
+            float thr = 0.0f;
+            // the reference counts "elements per image x calibrate_img_num" (:341, :583)
+            if (k.thr(method == ONRT_QUANT_KL ? 0 : 1, hist[nm].data(), numel(net->tensors[nm].desc) * (long long) n_images2, max_abs[nm], &thr)) return lib_fail("threshold");
+            threshold[nm] = thr;
+        }
+    }
+    // the quantised image: the file with every Conv's scale, type and weight_aux set and its weights and bias rewritten
+    std::vector<char> out(net->file);
+    const ONE_MODEL_DESC_S *h = reinterpret_cast<const ONE_MODEL_DESC_S *>(out.data());
+    size_t off = (size_t) h->node_cfg_offset;
+    for (int i = 0; i < h->node_cnt; ++i) {
+        const OpKind *kind = find_kind(out.data() + off);
+        if (!kind) return fail(ONRT_ERR_FORMAT, "quantise: node %d has an unknown type", i);
+        if (!strcmp(kind->type, "Conv")) {
+            CONV_CONFIG_S *cfg = reinterpret_cast<CONV_CONFIG_S *>(out.data() + off);
+            const std::string in0(cfg->op_base_cfg.in_operand_name[0]);
+            cfg->input_scale = threshold[in0] / 127;      // model_quant.hpp:668
+            cfg->ifmap_quant2 = TYPE_INT8;
+            OPERAND_S wd, bd;
+            const size_t w_off = find_initialiser(out, cfg->op_base_cfg.in_operand_name[1], &wd);
+            if (!w_off || wd.data_type != TYPE_FP32 || wd.dim_num_of_shapes != 4) return fail(ONRT_ERR_FORMAT, "quantise: Conv %s has no fp32 weight initialiser of rank 4", cfg->op_base_cfg.op_name);
+            const int cout = wd.shapes[0], inner = wd.shapes[1] * wd.shapes[2] * wd.shapes[3];
+            if (cout < 1 || cout > 4096 || inner < 1) return fail(ONRT_ERR_FORMAT, "quantise: Conv %s has %d output channels (weight_aux holds 4096)", cfg->op_base_cfg.op_name, cout);
+            size_t b_off = 0;
+            if (cfg->has_bias) {
+                b_off = find_initialiser(out, cfg->op_base_cfg.in_operand_name[2], &bd);
+                if (!b_off || numel(bd) != cout) return fail(ONRT_ERR_FORMAT, "quantise: Conv %s has no bias initialiser of %d elements", cfg->op_base_cfg.op_name, cout);
+            }
+            std::vector<float> w((size_t) cout * inner), b(cout);
+            memcpy(w.data(), out.data() + w_off, w.size() * 4);
+            if (b_off) memcpy(b.data(), out.data() + b_off, b.size() * 4);
+            std::vector<int8_t> w8(w.size());
+            std::vector<int32_t> b32(cout);
+            if (k.quant_wb(w.data(), b_off ? b.data() : nullptr, cout, inner, w8.data(), b32.data(), cfg->weight_aux)) return lib_fail("weight quantiser");
+            // int8 weights at the front of the fp32-sized initialiser, int32 bias in the fp32 bias (:16-25); the bytes behind
+            // the weights, which nothing reads, are cleared (the reference leaves what the in-place conversion left there)
+            memset(out.data() + w_off, 0, w.size() * 4);
+            memcpy(out.data() + w_off, w8.data(), w8.size());
+            if (b_off) memcpy(out.data() + b_off, b32.data(), b32.size() * 4);
+        }
+        off += align64(kind->cfg_size);
+    }
+    memcpy(quant_one_buf, out.data(), out.size());
     return ONRT_OK;
 }
 

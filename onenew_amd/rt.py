@@ -8,7 +8,7 @@ from . import hip
 
 EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
            "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf",
-           "onrt_net_folded_activations", "onrt_net_fused_attentions", "onrt_net_fused_linears", "onrt_net_fused_skips", "onrt_net_fused_ir_blocks", "onrt_net_quantised_links", "onrt_net_tune_tiles", "onrt_net_get_tiles", "onrt_net_set_tiles", "onrt_one_set_tiles"]
+           "onrt_net_folded_activations", "onrt_net_fused_attentions", "onrt_net_fused_linears", "onrt_net_fused_skips", "onrt_net_fused_ir_blocks", "onrt_net_quantised_links", "onrt_net_tune_tiles", "onrt_net_get_tiles", "onrt_net_set_tiles", "onrt_one_set_tiles", "onrt_one_quantise"]
 
 _lib = None
 
@@ -54,6 +54,7 @@ def load():
     L.onrt_net_get_tiles.argtypes = [vp, i32p]
     L.onrt_net_set_tiles.argtypes = [vp, i32p]
     L.onrt_one_set_tiles.argtypes = [C.c_char_p, C.c_size_t, i32p]
+    L.onrt_one_quantise.argtypes = [C.c_char_p, C.c_size_t, C.c_char_p, C.c_int32, C.POINTER(vp), C.c_int32, C.POINTER(vp), C.c_int32, C.c_char_p]
     _lib = L
     return L
 
@@ -69,6 +70,38 @@ def with_tiles(one_bytes, tiles):
     t = (C.c_int32 * 3)(*tiles)
     _check(load().onrt_one_set_tiles(buf, len(one_bytes), t), "onrt_one_set_tiles")
     return buf.raw
+
+
+QUANT_KL, QUANT_MSE, QUANT_PERCENT = 0, 1, 2
+
+
+def quantise(one_bytes, images, method=QUANT_KL, images2=None, op_lib_dir=None):
+    """the W8A32 image of an fp32 .one model (onrt_one_quantise, the counterpart of tools/optimize/model_quant.hpp:625-679).
+    images: calibration items, each a numpy array (one-input models) or a list of arrays in input order, or device
+    addresses given as ints; images2: the items of the second pass of KL / MSE (default: the same ones)."""
+    vp = C.c_void_p
+    keep = []
+
+    def pointers(items):
+        flat = []
+        for item in items:
+            for a in (item if isinstance(item, (list, tuple)) else [item]):
+                if isinstance(a, int):
+                    flat.append(a)
+                else:
+                    a = np.ascontiguousarray(a, dtype=np.float32)
+                    keep.append(a)
+                    flat.append(a.ctypes.data)
+        return (vp * len(flat))(*[vp(p) for p in flat])
+
+    one_bytes = bytes(one_bytes)
+    p1 = pointers(images)
+    p2 = pointers(images2) if images2 is not None else None
+    out = C.create_string_buffer(len(one_bytes))
+    lib_dir = (op_lib_dir or os.path.dirname(lib_path())).encode()
+    _check(load().onrt_one_quantise(one_bytes, len(one_bytes), lib_dir, int(method), p1, len(images), p2,
+                                    len(images2) if images2 is not None else 0, out), "onrt_one_quantise")
+    return out.raw
 
 
 class Net:

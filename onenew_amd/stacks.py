@@ -120,12 +120,10 @@ def with_batch(layers, n):
     return out
 
 
-def resnet50_model(batch=1, classes=1000, tag="resnet50_model", quantised=False):
+def resnet50_model(batch=1, classes=1000, tag="resnet50_model"):
     """The whole ResNet-50 as a .one file, in the form the offline optimiser leaves it: batch norm folded into the
     convolutions, ReLU fused into stem / conv1 / conv2 (33 of the 53), the residual Add and its ReLU as nodes of
     their own, MaxPool 3x3 s2 after the stem, GlobalAveragePool, Flatten, Gemm.  Seeded He-scaled weights.
-    quantised: every convolution in the W8A32 form the offline quantiser writes (tools/optimize/model_quant.hpp:6-29:
-    int8 weights, int32 bias, per-channel weight_aux) with one synthetic input_scale for every operand.
     Returns (bytes, input shape, multiply-accumulates x 2 per inference)."""
     import numpy as np
     from . import datagen, onefile
@@ -142,10 +140,6 @@ def resnet50_model(batch=1, classes=1000, tag="resnet50_model", quantised=False)
         flops += 2 * batch * cout * out_hw * out_hw * cin * k * k
         w = weights(name + ".w", (cout, cin, k, k), cin * k * k) * gain   # the residual branch is damped: no batch norm here
         b = datagen.normal(datagen.seed_for(tag, name + ".b"), (cout,), 0.0, 0.01)
-        if quantised:
-            from . import hip
-            w8, b32, aux = hip.quant_weight_bias(w, b)
-            return m.conv(name, x, w8, b32, name + "_out", stride=s, pad=p, act=act, quant=(aux, 0.05))
         return m.conv(name, x, w, b, name + "_out", stride=s, pad=p, act=act)
 
     x = m.input("input", (batch, 3, 224, 224))

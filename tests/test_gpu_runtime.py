@@ -813,3 +813,136 @@ def test_depthwise_int8_convolutions_take_part_in_the_int8_edges(torch_dev, monk
     for (oname, _), got in zip(net.outputs, net.run(*ins)):
         assert np.array_equal(got, ref[oname]), ("scales differ", oname)
     net.close()
+
+
+def _conv_nodes(parsed):
+    return [cfg for t, cfg in parsed["nodes"] if t == "Conv"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("method", ["kl", "mse", "percent"])
+@pytest.mark.parametrize("model", ["resnet_block", "mobile_block", "unfused_activations", "ir_blocks"])
+def test_model_level_quantisation_writes_what_the_oracles_steps_give(model, method, torch_dev, oracle, monkeypatch):
+    """onrt_one_quantise (tools/optimize/model_quant.hpp:625-679) on small fp32 models: every Conv of the image it returns
+    carries input_scale = threshold / 127 with the threshold the oracle's calibrators compute from the same activations
+    (the fp32 net's own operands on the calibration inputs), int8 weights, int32 bias and weight_aux equal to the oracle's
+    quant_weight_bias, and nothing else in the file differs; the quantised image then runs through the runtime with the
+    results of the oracle's executor (bit for bit where every operator after the first Conv is exact)"""
+    builder = {"resnet_block": one_models.resnet_block, "mobile_block": one_models.mobile_block,
+               "unfused_activations": one_models.unfused_activations,
+               "ir_blocks": lambda: one_models.inverted_residual_blocks(batch=2, size=32)}[model]
+    if method == "percent" and model != "ir_blocks":
+        # model_quant.hpp:107-118 keeps (1 - 0.99998) * 10 * elements values per image: nothing below 5000 elements, and the
+        # threshold of such an operand is 0
+        pytest.skip("the percentile rule keeps no value of operands this small")
+    data, ins = builder()
+    rng = np.random.default_rng(77)
+    images = [[(a * np.float32(s) + rng.normal(size=a.shape).astype(np.float32) * np.float32(0.1)).astype(np.float32) for a in ins]
+              for s in (1.0, 0.7, -1.2)]
+    second = [[(a * np.float32(0.9)).astype(np.float32) for a in item] for item in images[:2]]
+    code = {"kl": rt.QUANT_KL, "mse": rt.QUANT_MSE, "percent": rt.QUANT_PERCENT}[method]
+    q = rt.quantise(data, images, code, images2=None if method == "percent" else second)
+    assert len(q) == len(data)
+    src, dst = onefile.parse(data), onefile.parse(q)
+    # the activations the calibration saw: the fp32 net, operator by operator
+    monkeypatch.setenv("ONENEW_RT_FUSE", "0")
+    net = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_FUSE")
+    names = []
+    for cfg in _conv_nodes(src):
+        n = cfg.op_base_cfg.in_operand_name[0].value.decode()
+        if n not in names:
+            names.append(n)
+    seen = {n: [] for n in names}
+    seen2 = {n: [] for n in names}
+    for store, items in ((seen, images), (seen2, second)):
+        for item in items:
+            net.run(*item)
+            for n in names:
+                store[n].append(net.fetch(n).copy())
+    net.close()
+    thr = {}
+    for n in names:
+        if method == "percent":
+            x = np.stack(seen[n])
+            thr[n] = oracle.calib_percentile(x, len(images), x[0].size)
+        else:
+            mx = 0.0
+            for a in seen[n]:
+                mx = oracle.calib_abs_max(a, mx)
+            hist = None
+            for a in seen2[n]:
+                hist = oracle.calib_histogram(a, mx, hist)
+            thr[n] = oracle.calib_threshold(method, hist, seen2[n][0].size * len(second), mx)
+    assert [t for t, _ in src["nodes"]] == [t for t, _ in dst["nodes"]]
+    touched = set()
+    for (t, a), (_, b) in zip(src["nodes"], dst["nodes"]):
+        if t != "Conv":
+            assert bytes(a) == bytes(b)
+            continue
+        name = a.op_base_cfg.op_name.decode()
+        want_scale = np.float32(thr[a.op_base_cfg.in_operand_name[0].value.decode()]) / np.float32(127)
+        assert np.float32(b.input_scale) == want_scale, (name, b.input_scale, want_scale)
+        assert b.ifmap_quant2 == abi.TYPE_INT8 and b.input_scale > 0
+        wname = a.op_base_cfg.in_operand_name[1].value.decode()
+        w = src["inits"][wname]
+        bias = src["inits"][a.op_base_cfg.in_operand_name[2].value.decode()] if a.has_bias else None
+        w8, b32, aux = oracle.quant_weight_bias(w, bias)
+        got_w = dst["inits"][wname]
+        assert got_w.shape == w.shape and got_w.dtype == np.float32
+        raw = got_w.reshape(-1).view(np.int8)
+        assert np.array_equal(raw[:w.size], w8.reshape(-1)) and not raw[w.size:].any(), name
+        assert np.array_equal(np.array(b.weight_aux[:w.shape[0]], np.float32), aux), name
+        touched.add(wname)
+        if bias is not None:
+            bname = a.op_base_cfg.in_operand_name[2].value.decode()
+            assert np.array_equal(dst["inits"][bname].view(np.int32), b32), name
+            touched.add(bname)
+        # everything else of the node is as it was
+        a2 = type(a).from_buffer_copy(a)
+        a2.input_scale, a2.ifmap_quant2 = b.input_scale, b.ifmap_quant2
+        for i in range(len(a2.weight_aux)):
+            a2.weight_aux[i] = b.weight_aux[i]
+        assert bytes(a2) == bytes(b), name
+    for n, arr in src["inits"].items():
+        if n not in touched:
+            assert np.array_equal(arr.view(np.uint8), dst["inits"][n].view(np.uint8)), n
+    assert src["inputs"] == dst["inputs"] and src["outputs"] == dst["outputs"]
+    # the quantised image runs: against the oracle's executor on the same image
+    qnet = rt.Net(q)
+    if model == "unfused_activations":
+        # the oracle's executor has no Clip / Sigmoid / Mul nodes (it reads optimised files); the same model written by the
+        # optimiser carries the same weights and, given the same scales, must give the same results
+        opt, _ = one_models.unfused_activations(optimised=True)
+        buf = bytearray(opt)
+        po, off = onefile.parse(opt), onefile.parse(opt)["header"].node_cfg_offset
+        scales = {b.op_base_cfg.op_name.decode(): b for b in _conv_nodes(dst)}
+        for t, cfg in po["nodes"]:
+            assert t == "Conv"
+            qc = scales[cfg.op_base_cfg.op_name.decode()]
+            cfg.input_scale, cfg.ifmap_quant2 = qc.input_scale, qc.ifmap_quant2
+            for i in range(len(cfg.weight_aux)):
+                cfg.weight_aux[i] = qc.weight_aux[i]
+            buf[off:off + C.sizeof(cfg)] = bytes(cfg)
+            off += onefile.align64(C.sizeof(cfg))
+        ref_model = bytes(buf)
+        # weights and biases: the optimised builder draws the same ones, so copy the quantised initialisers over by name
+        pq = onefile.parse(ref_model)
+        m2 = bytearray(ref_model)
+        ioff = pq["header"].init_info_offset
+        for name, arr in pq["inits"].items():
+            start = ioff + C.sizeof(abi.OPERAND_S)
+            m2[start:start + arr.nbytes] = dst["inits"][name].tobytes()
+            ioff += onefile.align64(C.sizeof(abi.OPERAND_S) + arr.nbytes)
+        ref = one_model.run(bytes(m2), ins)
+    else:
+        ref = one_model.run(q, ins)
+    for got, want in zip(qnet.run(*ins), ref):
+        if model == "resnet_block":          # a Gemm (MFMA summation order) ends this one
+            assert _close(got, want, 1e-4)
+        else:
+            assert np.array_equal(got, want)
+    qnet.close()
+    # and an image that is quantised already is refused
+    with pytest.raises(rt.OnrtError, match="quantised already"):
+        rt.quantise(q, images, code)
