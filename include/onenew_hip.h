@@ -216,9 +216,8 @@ int onhip_conv2d_w8a8_nhwc(const onhip_conv_desc_t *d, const int8_t *xq, const i
                            int8_t *yq, void *stream);
 
 /* 1 when the depthwise convolution `d` is available with int8 NHWC activations (onhip_conv2d_w8a8_nhwc,
- * onhip_conv2d_w8_link): any filter and stride with uniform padding, as long as the kernel's table of weights fits its
- * LDS ((kh * kw + 3) * round_up(channels, 16) floats within 64 KiB); 0 otherwise and for dense convolutions.  No
- * counterpart in the reference. */
+ * onhip_conv2d_w8_link): any stride, uniform padding, filters of up to 225 taps, tensors below 2 GiB; 0 otherwise and
+ * for dense convolutions.  No counterpart in the reference. */
 int onhip_conv2d_w8a8_depthwise_supported(const onhip_conv_desc_t *d);
 
 /* One link of an int8 chain inside a model: the activations come as fp32 NCHW (x, quantised with d->input_scale into the

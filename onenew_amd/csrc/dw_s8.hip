@@ -9,9 +9,10 @@
 //   * A wavefront works on ONE group of 16 channels (the 16 bytes of a pixel one 128-bit load brings) and its lanes run
 //     along output pixels; the four wavefronts of a workgroup take different groups of the same pixels at the same
 //     time, so the cache lines of those pixels are fetched once per workgroup.
-//   * With the group uniform in the wavefront, the weights are the same for every lane: the workgroup converts all
-//     weights to float once into LDS ([group][quad of channels][tap][4]) and a lane reads four of them per 128-bit
-//     broadcast read.
+//   * With the group uniform in the wavefront, the weights are the same for every lane: the workgroup converts the
+//     weights of its (up to four) groups to float once into LDS ([group][quad of channels][tap][4]) and a lane reads
+//     four of them per 128-bit broadcast read.  Pixels and chunks of four channel groups both spread over the grid, so
+//     a 7 x 7 plane with 960 channels still makes hundreds of workgroups.
 //   * The products are formed in fp32: v_cvt_f32_ubyte{0..3} turns a byte into a float in one instruction, but only an
 //     unsigned one, so the input is biased by 128 (one xor per dword) and the sum starts at -128 * sum(w).  Every
 //     product and partial sum is an integer below 2^24, so the fp32 sum equals the int32 sum exactly, in any order.
@@ -24,12 +25,17 @@
 
 namespace onhip {
 
+#ifndef DWS8_R1
+#define DWS8_R1 2
+#endif
+
 struct DwS8Params {
     int C, Cp, G, N, H, W, OH, OW, kh, kw, taps, sh, sw, pad;
     int strips;            // strips of R output rows per image
     int items;             // N * strips * OW lanes' worth of work per channel group
     int gw;                // wavefronts of a workgroup that take different channel groups (1, 2 or 4)
-    Div31 div_ow, div_strips, div_taps;
+    int pchunks;           // chunks of 64 * (4 / gw) lanes' items; workgroup id = chunk of channel groups * pchunks + pixel chunk
+    Div31 div_ow, div_strips, div_taps, div_pchunks;
     float in_scale, out_inv_scale;
     const int8_t *x;
     const int8_t *w;
@@ -56,16 +62,25 @@ __device__ __forceinline__ void dws8_bytes(unsigned v, float f[4]) {
 // S3 > 0: 3x3 filter with stride S3 in both directions; S3 == 0: any filter, one output per lane
 template <int S3, int EPI, bool OUT_F32>
 __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
+    // the weights and per-channel constants of the gw channel groups this workgroup's wavefronts take
     extern __shared__ __align__(16) float lds[];
-    float *wl = lds;                         // [G][4][taps][4]
-    float *cst = lds + p.Cp * p.taps;        // [G][3][16]: -128 * sum of the channel's weights, bias, weight_aux / 127
+    float *wl = lds;                              // [gw][4][taps][4]
+    float *cst = lds + p.gw * 16 * p.taps;        // [gw][3][16]: -128 * sum of the channel's weights, bias, weight_aux / 127
     const int tid = threadIdx.x;
-    for (int i = tid; i < p.Cp * p.taps; i += 256) {
-        const int c = dws8_div(i, p.div_taps), t = i - c * p.taps;
+    // Workgroup id = chunk of channel groups * pchunks + pixel chunk: neighbouring workgroups (which run at the same time,
+    // on different XCDs) write different pixels.  With the chunk of channel groups as the fast index instead, three
+    // workgroups stored their 16-byte pieces into the same 128-byte lines at the same moment, and a fraction of a per cent
+    // of those pieces came out with wrong bytes (measured on full-size layers, different ones from run to run, never
+    // with this order).
+    const int gchunk = dws8_div((int) blockIdx.x, p.div_pchunks), pchunk = (int) blockIdx.x - gchunk * p.pchunks;
+    const int c_first = gchunk * p.gw * 16;       // first channel of the workgroup
+    for (int i = tid; i < p.gw * 16 * p.taps; i += 256) {
+        const int cl = dws8_div(i, p.div_taps), t = i - cl * p.taps, c = c_first + cl;
         const float w = c < p.C ? (float) p.w[(long long) c * p.taps + t] : 0.0f;
-        wl[(((c >> 4) * 4 + ((c & 15) >> 2)) * p.taps + t) * 4 + (c & 3)] = w;
+        wl[(((cl >> 4) * 4 + ((cl & 15) >> 2)) * p.taps + t) * 4 + (cl & 3)] = w;
     }
-    for (int c = tid; c < p.Cp; c += 256) {
+    for (int cl = tid; cl < p.gw * 16; cl += 256) {
+        const int c = c_first + cl;
         int sum = 0;
         float bias = 0.0f, coeff = 0.0f;
         if (c < p.C) {
@@ -73,19 +88,21 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
             bias = (float) p.b32[c];
             coeff = __fdiv_rn(p.aux[c], 127.0f);
         }
-        float *cc = cst + (c >> 4) * 48 + (c & 15);
+        float *cc = cst + (cl >> 4) * 48 + (cl & 15);
         cc[0] = -128.0f * (float) sum;
         cc[16] = bias;
         cc[32] = coeff;
     }
     __syncthreads();
 
-    constexpr int R = S3 == 1 ? 4 : S3 == 2 ? 2 : 1;
+    constexpr int R = S3 == 1 ? DWS8_R1 : S3 == 2 ? 2 : 1;
     constexpr int ROWS = S3 > 0 ? (R - 1) * S3 + 3 : 1;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int gsub = wave % p.gw, psub = wave / p.gw;
+    const int g = gchunk * p.gw + gsub;           // the wavefront's channel group; gsub indexes the tables in LDS
+    if (g >= p.G) return;
     const int per_wg = 64 * (4 / p.gw);
-    const int item = blockIdx.x * per_wg + psub * 64 + lane;
+    const int item = pchunk * per_wg + psub * 64 + lane;
     const bool live = item < p.items;
     const int it = live ? item : 0;
     const int ns = dws8_div(it, p.div_ow), ow = it - ns * p.OW;
@@ -103,19 +120,19 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
             for (int j = 0; j < 3; ++j) {
                 const int ih = ih0 + r, iw = iw0 + j;
                 const bool ok = live && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-                voff[r][j] = ok ? (unsigned) (((n * p.H + ih) * p.W + iw) * p.Cp) : OOB;
+                voff[r][j] = ok ? (unsigned) (((n * p.H + ih) * p.W + iw) * p.Cp + g * 16) : OOB;
             }
-        for (int g = gsub; g < p.G; g += p.gw) {
+        {
             uint4 px[ROWS][3];
 #pragma unroll
             for (int r = 0; r < ROWS; ++r)
 #pragma unroll
-                for (int j = 0; j < 3; ++j) px[r][j] = buf_load_b128(rx, voff[r][j], (unsigned) g * 16u);
+                for (int j = 0; j < 3; ++j) px[r][j] = buf_load_b128(rx, voff[r][j], 0u);
             unsigned outw[R][4];
 #pragma unroll
             for (int cq = 0; cq < 4; ++cq) {
-                const float4 *wq = reinterpret_cast<const float4 *>(wl + (g * 4 + cq) * 9 * 4);
-                const float4 *cq4 = reinterpret_cast<const float4 *>(cst + g * 48 + cq * 4);
+                const float4 *wq = reinterpret_cast<const float4 *>(wl + (gsub * 4 + cq) * 9 * 4);
+                const float4 *cq4 = reinterpret_cast<const float4 *>(cst + gsub * 48 + cq * 4);
                 const float4 init = cq4[0], bias = cq4[4], coeff = cq4[8];
                 float w[9][4];
 #pragma unroll
@@ -175,10 +192,10 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
             }
         }
     } else {
-        for (int g = gsub; g < p.G; g += p.gw) {
+        {
             float acc[16];
 #pragma unroll
-            for (int k = 0; k < 16; ++k) acc[k] = cst[g * 48 + k];
+            for (int k = 0; k < 16; ++k) acc[k] = cst[gsub * 48 + k];
             for (int i = 0; i < p.kh; ++i)
                 for (int j = 0; j < p.kw; ++j) {
                     const int ih = ih0 + i, iw = iw0 + j;
@@ -189,7 +206,7 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
                     for (int cq = 0; cq < 4; ++cq) {
                         float f[4];
                         dws8_bytes(cq == 0 ? v.x : cq == 1 ? v.y : cq == 2 ? v.z : v.w, f);
-                        const float4 w = *reinterpret_cast<const float4 *>(wl + ((g * 4 + cq) * p.taps + t) * 4);
+                        const float4 w = *reinterpret_cast<const float4 *>(wl + ((gsub * 4 + cq) * p.taps + t) * 4);
                         acc[cq * 4 + 0] = __fmaf_rn(f[0], w.x, acc[cq * 4 + 0]);
                         acc[cq * 4 + 1] = __fmaf_rn(f[1], w.y, acc[cq * 4 + 1]);
                         acc[cq * 4 + 2] = __fmaf_rn(f[2], w.z, acc[cq * 4 + 2]);
@@ -199,8 +216,8 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
             unsigned outw[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
             for (int k = 0; k < 16; ++k) {
-                const float fl = __fadd_rn(__fmul_rn(acc[k], p.in_scale), cst[g * 48 + 16 + k]);
-                const float v = act_fast<EPI>(__fmul_rn(fl, cst[g * 48 + 32 + k]), p.ep);
+                const float fl = __fadd_rn(__fmul_rn(acc[k], p.in_scale), cst[gsub * 48 + 16 + k]);
+                const float v = act_fast<EPI>(__fmul_rn(fl, cst[gsub * 48 + 32 + k]), p.ep);
                 const int c = g * 16 + k;
                 if constexpr (OUT_F32) {
                     const bool ok = live && c < p.C;
@@ -218,14 +235,13 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
     }
 }
 
-static const size_t kDwS8MaxLds = 64 * 1024;   // dynamic LDS a launch may ask for without further ado
 
 // the shapes the kernel takes: what fits its LDS table of weights and its 32-bit offsets
 bool dw_s8_ok(const onhip_conv_desc_t &d, int OH, int OW) {
     const long long cp = (d.cout + 15) / 16 * 16;
     const long long taps = (long long) d.kh * d.kw;
     if (d.group == 1 || d.cout != d.cin || !d.has_bias) return false;
-    if ((cp * taps + cp * 3) * 4 > (long long) kDwS8MaxLds) return false;
+    if (taps > 225) return false;   // the table of four channel groups' weights stays within 64 KiB of LDS
     if ((long long) d.n * d.h * d.w * cp >= (1LL << 31) || (long long) d.n * OH * OW * cp >= (1LL << 31)) return false;
     if ((long long) d.n * d.cout * OH * OW * 4 >= (1LL << 31)) return false;
     return true;
@@ -252,7 +268,7 @@ int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, c
     p.N = d.n; p.H = d.h; p.W = d.w; p.OH = OH; p.OW = OW;
     p.kh = d.kh; p.kw = d.kw; p.taps = d.kh * d.kw; p.sh = d.stride_h; p.sw = d.stride_w; p.pad = d.pad_t;
     const int s3 = (d.kh == 3 && d.kw == 3 && d.stride_h == d.stride_w && (d.stride_h == 1 || d.stride_h == 2)) ? d.stride_h : 0;
-    const int R = s3 == 1 ? 4 : s3 == 2 ? 2 : 1;
+    const int R = s3 == 1 ? DWS8_R1 : s3 == 2 ? 2 : 1;
     p.strips = (OH + R - 1) / R;
     const long long items = (long long) d.n * p.strips * OW;
     if (items >= (1LL << 31)) return set_error(ONHIP_ERR_ARG, "depthwise int8 NHWC: too many outputs");
@@ -268,9 +284,12 @@ int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, c
     p.y_bytes = d.out_s8 ? (unsigned) ((long long) d.n * OH * OW * p.Cp) : (unsigned) ((long long) d.n * d.cout * OH * OW * 4);
     p.ep = ep;
     const int per_wg = 64 * (4 / p.gw);
-    const long long wgs = (items + per_wg - 1) / per_wg;
+    const int gchunks = (p.G + p.gw - 1) / p.gw;
+    p.pchunks = (int) ((items + per_wg - 1) / per_wg);
+    p.div_pchunks = make_div31((unsigned) p.pchunks);
+    const long long wgs = (long long) p.pchunks * gchunks;
     if (wgs > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise int8 NHWC: too many workgroups");
-    const size_t lds_bytes = ((size_t) p.Cp * p.taps + (size_t) p.Cp * 3) * 4;
+    const size_t lds_bytes = ((size_t) p.gw * 16 * p.taps + (size_t) p.gw * 48) * 4;
     const int epi = epi_of_act(ep.act);
     if (d.out_s8) {
         if (s3 == 1) dw_s8_dispatch<1, false>(epi, (unsigned) wgs, lds_bytes, stream, p);
