@@ -281,8 +281,8 @@ class VitGlueLayer:
 
 class IrBlockLayer:
     """a whole inverted-residual block (1x1 expansion + CLIP, depthwise 3x3 + CLIP, 1x1 projection) in one launch: neither
-    wide tensor leaves the chip; work and bytes are counted as the three separate convolutions' (every tensor of the
-    unfused chain once), so the figures stay comparable with the layer-by-layer stack"""
+    wide tensor leaves the chip.  Work is counted as the three convolutions'; bytes as what the launch itself has to move
+    (input, weights, output), with the bytes of the three-launch chain it replaces kept beside them (`chain_bytes`)"""
     kind = "ir_block"
 
     def __init__(self, torch, hip, name, ex, dw, pw, tag):
@@ -297,8 +297,12 @@ class IrBlockLayer:
         oh, ow = dw.out_hw()
         self.y = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device="cuda")
         self.flops = ex.flops() + dw.flops() + pw.flops()
-        self.bytes = ex.algorithmic_bytes() + dw.algorithmic_bytes() + pw.algorithmic_bytes()
-        self.dense = False           # counted against the memory traffic of the chain it replaces
+        # what this launch has to move: the block's input, its weights and biases, its output (every tensor once) ...
+        self.bytes = 4 * (self.x.numel() + self.y.numel() + self.ex_w.numel() + self.ex_b.numel() + self.dw_w.numel()
+                          + self.dw_b.numel() + self.pw_w.numel() + self.pw_b.numel())
+        # ... and what the three separate convolutions it replaces move (both wide tensors written and read back)
+        self.chain_bytes = ex.algorithmic_bytes() + dw.algorithmic_bytes() + pw.algorithmic_bytes()
+        self.dense = False           # grouped with the depthwise layers: the memory-bound part of the network
         self.shape = f"C={ex.cin}>{dw.cin}>{pw.cout} N={dw.n * oh * ow} s{dw.stride_h}"
 
     def launch(self, hip):
@@ -731,7 +735,7 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False, graph=True
     desc, dtype, layers = make_workload(torch, hip, name)
     unit = "TOP/s" if dtype == "i8" else "TFLOP/s"
     flops = sum(L.flops for L in layers)
-    abytes = sum(L.bytes for L in layers)
+    abytes = sum(L.bytes for L in layers)           # what the launches of a pass have to move (fused launches: their own tensors)
 
     for _ in range(warmup):
         for L in layers:
@@ -786,6 +790,7 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False, graph=True
     grp = groups[dom_dense]
     g_ms = sum(t for _, t in grp)
     g_flops, g_bytes = sum(L.flops for L, _ in grp), sum(L.bytes for L, _ in grp)
+    g_chain_bytes = sum(getattr(L, "chain_bytes", L.bytes) for L, _ in grp)
     kernel = ("onhip::igemm_dma_kernel (operand tiles straight into LDS, 16-bit storage, MFMA implicit GEMM)"
               if dom_dense and grp[0][0].kind in ("conv_h16", "linear_h16") else
               f"onhip::igemm_kernel ({dtype} MFMA implicit GEMM)" if dom_dense else
@@ -813,6 +818,12 @@ def run_workload(torch, hip, name, steps, warmup, layers_table=False, graph=True
                 "arithmetic_intensity": round(g_flops / g_bytes, 2),
                 # the same fraction from the wall time of the timed passes (layers back to back, cold caches between them)
                 "frac_whole_step": round(step_frac, 4)}
+    if g_chain_bytes != g_bytes and not mfma_bound:
+        # launches that replace a chain of operators: `achieved` / `frac` count the bytes those launches themselves move;
+        # this is the rate at which the bytes of the chains they replace would have had to move in the same time
+        roofline["unfused_chain_equivalent"] = {"achieved": round(g_chain_bytes / (g_ms * 1e-3) / 1e9, 3), "unit": "GB/s",
+                                                "frac": round(g_chain_bytes / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                                "bytes_per_launch": g_chain_bytes / len(grp)}
     res = {"name": name, "desc": desc, "dtype": dtype, "unit": unit, "flops": flops, "abytes": abytes,
            "ms_per_step": ms_per_step, "eager_ms_per_step": eager_ms, "launch": launch_mode, "per_layer_ms": per_layer_ms,
            "roofline": roofline, "layers": layers,
@@ -834,7 +845,8 @@ def config_summary(res):
     out = {"workload": res["name"], "what": res["desc"], "dtype": res["dtype"], "value": round(res["value"], 3), "unit": res["unit"],
            "ms_per_step": round(res["ms_per_step"], 4), "launch": res["launch"], "eager_ms_per_step": round(res["eager_ms_per_step"], 4),
            "ms_sum_of_layers": round(sum(per), 4), "layers": len(per),
-           "roofline": {k: rf[k] for k in ("bound", "achieved", "peak", "unit", "frac", "frac_whole_step", "avg_launch_ms", "launches")},
+           "roofline": {k: rf[k] for k in ("bound", "achieved", "peak", "unit", "frac", "frac_whole_step", "avg_launch_ms", "launches", "traffic",
+                                           "unfused_chain_equivalent") if k in rf},
            "algorithmic_GBps": round(res["abytes"] / (res["ms_per_step"] * 1e-3) / 1e9, 1),
            "hbm_frac_whole_step": round(res["abytes"] / (res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     lowai = [(L, t) for L, t in zip(res["layers"], per) if not L.dense]

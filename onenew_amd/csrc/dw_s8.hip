@@ -72,7 +72,16 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
     // workgroups stored their 16-byte pieces into the same 128-byte lines at the same moment, and a fraction of a per cent
     // of those pieces came out with wrong bytes (measured on full-size layers, different ones from run to run, never
     // with this order).
-    const int gchunk = dws8_div((int) blockIdx.x, p.div_pchunks), pchunk = (int) blockIdx.x - gchunk * p.pchunks;
+    // Consecutive workgroup ids go round-robin over the 8 XCDs, each with an L2 of its own: every XCD gets a contiguous
+    // run of the numbering, so that the chunks either side of a boundary (which may share a line, and share their halo
+    // rows) meet in one L2.
+    int lid;
+    {
+        const int nb = (int) gridDim.x, bid = (int) blockIdx.x;
+        const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
+        lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+    }
+    const int gchunk = dws8_div(lid, p.div_pchunks), pchunk = lid - gchunk * p.pchunks;
     const int c_first = gchunk * p.gw * 16;       // first channel of the workgroup
     for (int i = tid; i < p.gw * 16 * p.taps; i += 256) {
         const int cl = dws8_div(i, p.div_taps), t = i - cl * p.taps, c = c_first + cl;
