@@ -395,6 +395,29 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
             }
         if (best_cost < 1e300) break;
     }
+    // What measuring the candidates keeps finding on top of the tile and split above (fp32, one batch slice):
+    //  * no split, and a few tiles left over after whole rounds of 256: those tiles alone cut along K so that the leftover,
+    //    too, puts about a workgroup on every compute unit (launch_choice);
+    //  * K slices added up by the last slice of a tile to arrive instead of by a finishing launch, where the launch has
+    //    tiles enough that those last arrivers spread over the chip (at batch 1, with a handful of tiles, the finishing
+    //    launch's spread over every compute unit wins).  Same sums in the same order either way.
+    if (cfg.dtype == DT_F32 && !vec && !best.rowb && !best.dma) {
+        int dpc = 0, left = 0;
+        if (best.split == 1 && tail_geometry(cfg, p, best.bm, best.bn, &dpc, &left)) {
+            int want = 256 / left;
+            want = want > 16 ? 16 : want;
+            for (int ts = want; ts >= 2; ts /= 2) {
+                const Choice c = {best.bm, best.bn, 1, ts, 0, 0, 0};
+                if (candidate_ok(cfg, p, c)) { best = c; break; }
+            }
+        }
+        const long long tiles = (long long) ((p.M + best.bm - 1) / best.bm) * ((p.N + best.bn - 1) / best.bn);
+        if ((best.split > 1 || best.tail > 1) && tiles >= 128) {
+            Choice c = best;
+            c.fin = 1;
+            if (candidate_ok(cfg, p, c)) best = c;
+        }
+    }
     return best;
 }
 

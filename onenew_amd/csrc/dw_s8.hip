@@ -67,11 +67,7 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
     float *wl = lds;                              // [gw][4][taps][4]
     float *cst = lds + p.gw * 16 * p.taps;        // [gw][3][16]: -128 * sum of the channel's weights, bias, weight_aux / 127
     const int tid = threadIdx.x;
-    // Workgroup id = chunk of channel groups * pchunks + pixel chunk: neighbouring workgroups (which run at the same time,
-    // on different XCDs) write different pixels.  With the chunk of channel groups as the fast index instead, three
-    // workgroups stored their 16-byte pieces into the same 128-byte lines at the same moment, and a fraction of a per cent
-    // of those pieces came out with wrong bytes (measured on full-size layers, different ones from run to run, never
-    // with this order).
+    // Workgroup id = chunk of channel groups * pchunks + pixel chunk.
     // Consecutive workgroup ids go round-robin over the 8 XCDs, each with an L2 of its own: every XCD gets a contiguous
     // run of the numbering, so that the chunks either side of a boundary (which may share a line, and share their halo
     // rows) meet in one L2.
@@ -195,8 +191,12 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
                 for (int q = 0; q < R; ++q) {
                     const int oh = oh0 + q;
                     const bool ok = live && oh < p.OH;
+                    // The group's offset goes into the vector offset, the scalar offset stays the constant 0: after a 128-bit
+                    // buffer store whose scalar offset is a REGISTER the compiler leaves no gap before the next instruction
+                    // that writes one of the data registers, and on this GPU that instruction then changes what some lanes
+                    // store (seen here as the first dword of a pixel's 16 bytes holding the next row's index, now and then).
                     __builtin_amdgcn_raw_buffer_store_b128(u32x4{outw[q][0], outw[q][1], outw[q][2], outw[q][3]}, ry,
-                                                           ok ? (unsigned) (((n * p.OH + oh) * p.OW + ow) * p.Cp) : OOB, (unsigned) g * 16u, 0);
+                                                           ok ? (unsigned) (((n * p.OH + oh) * p.OW + ow) * p.Cp + g * 16) : OOB, 0, 0);
                 }
             }
         }
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
             }
             if constexpr (!OUT_F32)
                 __builtin_amdgcn_raw_buffer_store_b128(u32x4{outw[0], outw[1], outw[2], outw[3]}, ry,
-                                                       live ? (unsigned) (((n * p.OH + oh0) * p.OW + ow) * p.Cp) : OOB, (unsigned) g * 16u, 0);
+                                                       live ? (unsigned) (((n * p.OH + oh0) * p.OW + ow) * p.Cp + g * 16) : OOB, 0, 0);
         }
     }
 }

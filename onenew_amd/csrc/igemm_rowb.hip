@@ -48,9 +48,12 @@ __device__ __forceinline__ void rowb_store(const IgemmParams &p, f32x16 (&acc)[4
             const float vm = __fadd_rn(a, bias_m[r]), vn = __fadd_rn(a, bias_n[j]);
             v[j] = act_fast<EPI>(bias_m_on ? vm : bias_n_on ? vn : a, p.ep);
         }
+        // row offset in the vector offset, scalar offset the constant 0: a 128-bit buffer store with a register as its
+        // scalar offset gets no gap from the compiler before the next write to its data registers, which on this GPU can
+        // change what some lanes store
         __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]),
                                                      __float_as_uint(v[3])},
-                                               rc, row_ok ? col_voff : OOB, (unsigned) m_uni * (unsigned) p.c_stride_m * 4u, 0);
+                                               rc, row_ok ? col_voff + (unsigned) m_uni * (unsigned) p.c_stride_m * 4u : OOB, 0, 0);
     }
 }
 
@@ -66,7 +69,7 @@ __device__ __forceinline__ void rowb_store_partial(const IgemmParams &p, f32x16 
         const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
         const float v0 = acc[0][r], v1 = acc[1][r], v2 = acc[2][r], v3 = acc[3][r];
         __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)},
-                                               rp, row_ok ? cv : OOB, (unsigned) m_uni * (unsigned) width * 4u, 0);
+                                               rp, row_ok ? cv + (unsigned) m_uni * (unsigned) width * 4u : OOB, 0, 0);
     }
 }
 
