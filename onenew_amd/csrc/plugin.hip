@@ -657,7 +657,9 @@ static int matmul_attention_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *in
     const void *in[3];
     for (int i = 0; i < 3; ++i) {
         if (!inputs[i].addr) return set_error(ONHIP_ERR_ARG, "attention eval: empty input slot %d", i);
-        const int rc = input_on_device(i, reinterpret_cast<const void *>(inputs[i].addr), bytes, &in[i]);
+        // q and k in the first two staging buffers, v in the fifth: the third one holds the result (the kernel reads v
+        // of one head while it writes the result of another)
+        const int rc = input_on_device(i < 2 ? i : 4, reinterpret_cast<const void *>(inputs[i].addr), bytes, &in[i]);
         if (rc) return rc;
     }
     void *host_out = reinterpret_cast<void *>(outputs[0].addr);

@@ -132,3 +132,19 @@ def test_plugin_eval_attention_host_buffers(flags, torch_dev, oracle):
         got = got.transpose(0, 2, 1, 3)
     assert got.shape == ref.shape
     assert np.abs(got.astype(np.float64) - ref).max() <= 1e-4 * np.abs(ref).max()
+
+
+def test_plugin_eval_attention_result_does_not_share_a_staging_buffer_with_v(torch_dev, oracle):
+    """host buffers, the result token-major and v head-major, many heads and tokens: the result of one head is written while
+    v of the next is still being read, so the two must not sit in one staging buffer (they once did: now and then wrong)"""
+    from onenew_amd import ops
+    b, h, t, hd = 3, 6, 200, 64
+    g = cases.datagen
+    q, k, v = (g.normal(g.seed_for("plug_attn_big", n), (b, h, t, hd), 0.0, 0.5) for n in "qkv")
+    kt = oracle.transpose_f32(k, (0, 1, 3, 2))
+    p = oracle.softmax_f32(oracle.matmul_f32(q.reshape(b * h, t, hd), kt.reshape(b * h, hd, t)))
+    ref = oracle.matmul_f32(p, v.reshape(b * h, t, hd)).reshape(b, h, t, hd)
+    op = ops.MatMulFused(ops.Plugin(hip.plugin_path("MatMul")))
+    for _ in range(3):
+        got = op.attention(q, k, v, token_major=(0, 0, 0, 1)).transpose(0, 2, 1, 3)
+        assert np.abs(got.astype(np.float64) - ref).max() <= 1e-4 * np.abs(ref).max()
