@@ -1169,6 +1169,9 @@ static int matmul_impl(const onhip_matmul_desc_t *d, const float *a, const float
     p.bias_mode = bias ? BIAS_N : BIAS_NONE;
     p.ep.act = gelu_lut ? ONHIP_ACT_GELU_LUT : NOT_ACT;
     p.ep.lut = gelu_lut;
+    // more rows than columns: the left operand is the large one (activations against a weight matrix), so tiles are
+    // numbered along N first and an XCD reads its rows of A once for all column blocks
+    p.n_fast = M > d->n ? 1 : 0;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (addend == out) return set_error(ONHIP_ERR_ARG, "matmul: the addend may not be the output buffer");
     if (addend && cfg.dtype != DT_F32) {   // reduced-precision operands: the Add as a pass over the result

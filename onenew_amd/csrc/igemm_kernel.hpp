@@ -843,7 +843,12 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
             whole_k = p.dp_tiles > 0;
         }
     }
-    const int tile_n = (int) div31((unsigned) lid, p.div_tiles_m), tile_m = lid - tile_n * tiles_m;
+    int tile_n = (int) div31((unsigned) lid, p.div_tiles_m), tile_m = lid - tile_n * tiles_m;
+    if (p.n_fast && p.dp_tiles == 0) {   // uniform: rows of A stay in the XCD's L2 while it sweeps the column blocks
+        const int tiles_n = (p.N + BN - 1) / BN;
+        tile_m = (int) div31((unsigned) lid, p.div_tiles_n);
+        tile_n = lid - tile_m * tiles_n;
+    }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int batch = blockIdx.z;
     const int u_begin = whole_k ? 0 : slice * p.k_split_units;
@@ -1262,6 +1267,7 @@ static int launch_one(const IgemmLaunch &cfg, const IgemmParams &p_in, hipStream
     p.div_ohw = make_div31((unsigned) (p.OHW > 0 ? p.OHW : 1));
     p.div_ow = make_div31((unsigned) (p.OW > 0 ? p.OW : 1));
     p.div_tiles_m = make_div31((unsigned) tiles_m);
+    p.div_tiles_n = make_div31((unsigned) ((p.N + BN - 1) / BN));
     dim3 grid(tiles, cfg.split, cfg.batch);
     if (p.dp_tiles > 0) {   // whole tiles first, then the K slices of the leftover tiles (igemm_kernel)
         if (cfg.batch != 1 || p.dp_tiles + p.tail_tiles != tiles || !p.partial || p.part_begin != p.dp_tiles / tiles_m * BN)

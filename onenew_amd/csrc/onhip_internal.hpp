@@ -215,6 +215,11 @@ struct IgemmParams {
     int n_slices;
     // exact division of any x < 2^31 by OHW, OW and the number of row tiles (filled in by the launcher)
     Div31 div_ohw, div_ow, div_tiles_m;
+    // n_fast != 0 (tiled kernel, launches without leftover-tile slices): tiles are numbered along N first, so that an XCD's
+    // run of tiles covers a band of rows of A against every column block of B.  For products whose A (many rows) does not
+    // fit an L2 while B (a weight matrix) does: each XCD then reads its rows of A once instead of all of A per column block.
+    int n_fast;
+    Div31 div_tiles_n;
 };
 
 enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2, DT_I8 = 3 };
