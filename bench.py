@@ -326,9 +326,17 @@ class ConvH16Layer:
         b = datagen.normal(datagen.seed_for(f"{tag}/{name}", "b"), (d.cout,), 0.0, 0.01)
         self.name, self.d = name, d
         x = device_uniform(torch, datagen.seed_for(f"{tag}/{name}", "x"), (d.n, d.cin, d.h, d.w))
-        self.x = hip.h16_from_nchw(x, compute)
+        # a first layer (at most 8 input channels, filter rows of at most 8 columns) is kept in the storage form made for
+        # it, 8 channels per pixel instead of 32: what a 16-bit pipeline is fed with at its head
+        self.first = hip.load().onhip_h16_first_width(d) > 0
+        if self.first:
+            self.x = hip.h16_first_from_nchw(d, x)
+            self.wp = hip.h16_first_pack_weights(d, torch.from_numpy(w).cuda())
+        else:
+            self.x = hip.h16_from_nchw(x, compute)
+            self.wp = hip.h16_pack_conv_weights(d, torch.from_numpy(w).cuda())
         del x
-        self.wp, self.b = hip.h16_pack_conv_weights(d, torch.from_numpy(w).cuda()), torch.from_numpy(b).cuda()
+        self.b = torch.from_numpy(b).cuda()
         oh, ow = d.out_hw()
         self.y = torch.empty((d.n, oh, ow, hip.h16_pitch(d.cout)), dtype=self.x.dtype, device="cuda")
         # every tensor once at 2 bytes per element, unpadded (the channel padding the layout adds is not counted as work)
@@ -337,7 +345,10 @@ class ConvH16Layer:
         self.shape = f"M={d.cout} N={d.n * oh * ow} K={d.k_per_out()}"
 
     def launch(self, hip):
-        hip.conv2d_h16(self.d, self.x, self.wp, self.b, out=self.y)
+        if self.first:
+            hip.conv2d_h16_first(self.d, self.x, self.wp, self.b, out=self.y)
+        else:
+            hip.conv2d_h16(self.d, self.x, self.wp, self.b, out=self.y)
 
     def cpu_runner(self, ops, oracle, tag):
         return ConvF32Layer.cpu_runner(self, ops, oracle, tag)

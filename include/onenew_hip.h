@@ -268,6 +268,22 @@ int onhip_h16_to_rows_f32(const void *x, long long rows, int32_t k, int32_t comp
 /* dense convolution, at most 64 filter taps, tensors below 2 GiB */
 int onhip_conv2d_h16(const onhip_conv_desc_t *d, const void *x, const void *w_packed, const float *bias, const float *lut,
                      const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream);
+/* First layers (dense, at most 8 input channels, filter rows of at most 8 columns, any stride and padding) in a storage
+ * form of their own: with the 32-channel pitch above a three-channel image is 29/32 zeros, in memory and in the
+ * arithmetic.  Here the image is stored [n][h][wp][cpp] (wp = onhip_h16_first_width: the padded row, an even number of
+ * columns; cpp = onhip_h16_first_channels: 4 channels per pixel for up to four input channels, else 8; stored column s =
+ * image column s - pad_l, zeros outside) and the weights [cout][kh][8 columns][cpp], so that a filter row meets 16 cpp
+ * contiguous bytes of the stored row and the reduction runs over kh x 8 cpp values.  The same
+ * arithmetic as onhip_conv2d_h16 (device/x86/Conv/conv.c:300-415 on operands rounded to the 16-bit type, fp32 sums, bias
+ * and activation in fp32); the result leaves in the layouts of y_kind, i.e. as the next layer's ordinary input. */
+int32_t onhip_h16_first_width(const onhip_conv_desc_t *d);            /* 0: not a shape of this form */
+int32_t onhip_h16_first_channels(const onhip_conv_desc_t *d);
+size_t onhip_h16_first_input_bytes(const onhip_conv_desc_t *d);
+size_t onhip_h16_first_weight_bytes(const onhip_conv_desc_t *d);
+int onhip_h16_first_from_nchw_f32(const onhip_conv_desc_t *d, const float *x, void *x_first, void *stream);
+int onhip_h16_first_pack_weights(const onhip_conv_desc_t *d, const float *w, void *packed, void *stream);
+int onhip_conv2d_h16_first(const onhip_conv_desc_t *d, const void *x_first, const void *w_packed, const float *bias,
+                           const float *lut, void *y, int32_t y_kind, void *stream);
 /* y[rows][n] = x[rows][k] * b[k][n] (+ bias[n]) (then the table GELU of device/x86/Gelu/gelu.c when gelu_lut is given):
  * the MatMul -> Add -> Gelu chain of a transformer's linear layers with x, b and (for _NHWC) y in 16 bits */
 int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, const void *x, const void *w_packed,

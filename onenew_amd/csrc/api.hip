@@ -1261,8 +1261,26 @@ int onhip_h16_to_rows_f32(const void *x, long long rows, int32_t k, int32_t comp
 }
 
 // gelu != 0: lut is the GELU table and is applied whatever the descriptor says (the linear layer's fused form)
+// the stored row width of the first-layer form: every output column's 8-pixel window lies inside its row
+static int h16_first_width(const onhip_conv_desc_t *d, int OW) {
+    const int padded = d->pad_l + d->w + d->pad_r, reach = (OW - 1) * d->stride_w + 8;
+    return ((padded > reach ? padded : reach) + 1) & ~1;   // even: rows of 4-channel pixels then start on 16 bytes
+}
+// channels stored per pixel: 4 (8 bytes) for up to four input channels, else 8
+static int h16_first_cpp(const onhip_conv_desc_t *d) { return d->cin <= 4 ? 4 : 8; }
+
+static int h16_first_check(const onhip_conv_desc_t *d, int32_t *OH, int32_t *OW) {
+    const int rc = check_conv(d, OH, OW);
+    if (rc) return rc;
+    if (d->group != 1 || d->cin > 8 || d->kw > 8 || d->kh > 64)
+        return set_error(ONHIP_ERR_ARG, "16-bit first layer: dense, at most 8 input channels, filter rows of at most 8 columns, at most 64 of them");
+    return ONHIP_OK;
+}
+
+// first != 0: x is the first-layer form [n][h][wp][cpp] and w_packed [cout][kh][8][cpp] (onhip_h16_first_*)
 static int conv2d_h16_impl(const onhip_conv_desc_t *d, const void *x, const void *w_packed, const float *bias, const float *lut,
-                           int gelu, const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream) {
+                           int gelu, const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream,
+                           int first = 0) {
     int32_t OH, OW;
     int rc = check_conv(d, &OH, &OW);
     if (rc) return rc;
@@ -1280,31 +1298,47 @@ static int conv2d_h16_impl(const onhip_conv_desc_t *d, const void *x, const void
         reinterpret_cast<uintptr_t>(residual) % 16)
         return set_error(ONHIP_ERR_ARG, "conv 16-bit: tensors must be 16-byte aligned");
     const int cp = onhip_h16_pitch(d->cin), cop = onhip_h16_pitch(d->cout);
-    if ((long long) d->n * d->h * d->w * cp * 2 >= (1LL << 31) || (long long) d->n * OH * OW * cop * 4 >= (1LL << 31) ||
+    const int wp = first ? h16_first_width(d, OW) : d->w;
+    if ((long long) d->n * d->h * wp * (first ? h16_first_cpp(d) : cp) * 2 >= (1LL << 31) || (long long) d->n * OH * OW * cop * 4 >= (1LL << 31) ||
         (long long) d->cout * d->kh * d->kw * cp * 2 >= (1LL << 31))
         return set_error(ONHIP_ERR_ARG, "conv 16-bit: tensors of 2 GiB or more are not supported");
     cfg.bl = BL_KVEC;
     cfg.batch = 1;
     IgemmParams p;
     memset(&p, 0, sizeof(p));
-    p.units_per_tap = cp / 8;
-    p.k_units = d->kh * d->kw * p.units_per_tap;
     p.M = d->cout;
     p.N = d->n * OH * OW;
-    p.K = p.k_units * 8;
     p.A = w_packed;
-    p.lda = p.k_units * 16;      // bytes, like every quantity of the vector loader
     p.B = x;
-    p.H = d->h; p.W = d->w; p.OW = OW; p.OHW = OH * OW; p.HW = d->h * d->w;
-    p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
-    p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t; p.pl = d->pad_l;
-    p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
+    p.H = d->h; p.OW = OW; p.OHW = OH * OW;
+    p.sh = d->stride_h; p.sw = d->stride_w; p.pt = d->pad_t;
     p.use_tapmask = 1;
+    if (first) {
+        // A filter row is one tap of 8 pixels x 4 or 8 channels = 64 or 128 contiguous bytes of the stored row, beginning at
+        // stored column ow * stride_w (the left padding is in the stored row, so no column is ever outside it); pixels are
+        // 8 or 16 bytes apart.  The reduction index runs over (filter row, column, channel), zeros where the filter has none.
+        p.units_per_tap = h16_first_cpp(d);
+        p.tap_spans_pixels = 1;
+        p.W = wp;
+        p.kh = d->kh; p.kw = 1; p.khkw = d->kh;
+        p.pl = 0;
+        p.pix_stride = h16_first_cpp(d) * 2;
+    } else {
+        p.units_per_tap = cp / 8;
+        p.W = d->w;
+        p.kh = d->kh; p.kw = d->kw; p.khkw = d->kh * d->kw;
+        p.pl = d->pad_l;
+        p.pix_stride = cp * 2;
+    }
+    p.HW = p.H * p.W;
+    p.k_units = p.khkw * p.units_per_tap;
+    p.K = p.k_units * 8;
+    p.lda = p.k_units * 16;      // bytes, like every quantity of the vector loader
+    p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
     p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
-    p.pix_stride = cp * 2;
-    p.b_shift_bytes = ((long long) d->pad_t * d->w + d->pad_l) * cp * 2;
+    p.b_shift_bytes = ((long long) p.pt * p.W + p.pl) * p.pix_stride;
     p.a_slice_bytes = (long long) p.M * p.lda;
-    p.b_slice_bytes = (long long) d->n * d->h * d->w * cp * 2;
+    p.b_slice_bytes = (long long) d->n * p.H * p.W * p.pix_stride;
     p.C = y;
     if (y_kind == ONHIP_H16_OUT_F32_NCHW) {
         p.out_mode = OUT_CONV;
@@ -1330,6 +1364,48 @@ static int conv2d_h16_impl(const onhip_conv_desc_t *d, const void *x, const void
 int onhip_conv2d_h16(const onhip_conv_desc_t *d, const void *x, const void *w_packed, const float *bias, const float *lut,
                      const void *residual, int32_t residual_relu, void *y, int32_t y_kind, void *stream) {
     return conv2d_h16_impl(d, x, w_packed, bias, lut, 0, residual, residual_relu, y, y_kind, stream);
+}
+
+int32_t onhip_h16_first_channels(const onhip_conv_desc_t *d) { return d && onhip_h16_first_width(d) ? h16_first_cpp(d) : 0; }
+
+int32_t onhip_h16_first_width(const onhip_conv_desc_t *d) {
+    int32_t OH, OW;
+    if (!d || h16_first_check(d, &OH, &OW)) return 0;
+    return h16_first_width(d, OW);
+}
+
+size_t onhip_h16_first_input_bytes(const onhip_conv_desc_t *d) {
+    const int32_t wp = onhip_h16_first_width(d);
+    return wp ? (size_t) d->n * d->h * wp * h16_first_cpp(d) * 2 : 0;
+}
+
+size_t onhip_h16_first_weight_bytes(const onhip_conv_desc_t *d) {
+    return onhip_h16_first_width(d) ? (size_t) d->cout * d->kh * 8 * h16_first_cpp(d) * 2 : 0;
+}
+
+int onhip_h16_first_from_nchw_f32(const onhip_conv_desc_t *d, const float *x, void *x_first, void *stream) {
+    int32_t OH, OW;
+    int dt, rc = h16_first_check(d, &OH, &OW);
+    if (rc || (rc = h16_dtype(d->compute, &dt))) return rc;
+    if (!x || !x_first || reinterpret_cast<uintptr_t>(x_first) % 16) return set_error(ONHIP_ERR_ARG, "16-bit first layer: null or misaligned tensor");
+    return first_from_nchw_launch(dt, x, d->n, d->cin, d->h, d->w, h16_first_width(d, OW), h16_first_cpp(d), d->pad_l, x_first,
+                                  reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_h16_first_pack_weights(const onhip_conv_desc_t *d, const float *w, void *packed, void *stream) {
+    int32_t OH, OW;
+    int dt, rc = h16_first_check(d, &OH, &OW);
+    if (rc || (rc = h16_dtype(d->compute, &dt))) return rc;
+    if (!w || !packed || reinterpret_cast<uintptr_t>(packed) % 16) return set_error(ONHIP_ERR_ARG, "16-bit first layer: null or misaligned weights");
+    return first_pack_w16_launch(dt, w, d->cout, d->cin, d->kh, d->kw, h16_first_cpp(d), packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_conv2d_h16_first(const onhip_conv_desc_t *d, const void *x_first, const void *w_packed, const float *bias, const float *lut,
+                           void *y, int32_t y_kind, void *stream) {
+    int32_t OH, OW;
+    const int rc = h16_first_check(d, &OH, &OW);
+    if (rc) return rc;
+    return conv2d_h16_impl(d, x_first, w_packed, bias, lut, 0, nullptr, 0, y, y_kind, stream, 1);
 }
 
 int onhip_linear_h16(long long rows, int32_t k, int32_t n, int32_t compute, const void *x, const void *w_packed, const float *bias,

@@ -66,6 +66,67 @@ int nchw_to_nhwc16_launch(int dt, const float *x, int n, int c, int h, int w, in
     return ONHIP_OK;
 }
 
+// ---- first layers: fp32 NCHW (at most 8 channels) -> 16-bit [n][h][wp][cpp], cpp = 4 or 8 channels per pixel ----------
+// Stored column s holds image column s - pad_l (zeros outside the image, zeros in the channels past c), so that the 8
+// stored pixels from column ow * stride_w on are the whole receptive-field row of output column ow: 16 cpp contiguous
+// bytes.  One thread per stored pixel; the loads of a wavefront are runs of 64 pixels of a channel plane.
+template <int DT, int CPP>
+__global__ __launch_bounds__(256) void first_from_nchw_kernel(const float *x, int c, int h, int w, int wp, int pad_l, unsigned short *y) {
+    const int s = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    const long long img = blockIdx.z;
+    if (s >= wp) return;
+    const int col = s - pad_l;
+    float v[CPP];
+#pragma unroll
+    for (int e = 0; e < CPP; ++e) v[e] = e < c && col >= 0 && col < w ? x[((img * c + e) * h + row) * (long long) w + col] : 0.0f;
+    unsigned short *dst = y + ((img * h + row) * (long long) wp + s) * CPP;
+    if constexpr (CPP == 8)
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(pack_h16<DT>(v[0], v[1]), pack_h16<DT>(v[2], v[3]), pack_h16<DT>(v[4], v[5]), pack_h16<DT>(v[6], v[7]));
+    else
+        *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_h16<DT>(v[0], v[1]), pack_h16<DT>(v[2], v[3]));
+}
+
+int first_from_nchw_launch(int dt, const float *x, int n, int c, int h, int w, int wp, int cpp, int pad_l, void *y, hipStream_t stream) {
+    if (n > 65535 || h > 65535) return set_error(ONHIP_ERR_ARG, "16-bit first layer: %d images of %d rows", n, h);
+    const dim3 grid((wp + 255) / 256, h, n);
+    unsigned short *out = reinterpret_cast<unsigned short *>(y);
+    if (dt == DT_BF16 && cpp == 8) hipLaunchKernelGGL((first_from_nchw_kernel<DT_BF16, 8>), grid, dim3(256), 0, stream, x, c, h, w, wp, pad_l, out);
+    else if (dt == DT_BF16) hipLaunchKernelGGL((first_from_nchw_kernel<DT_BF16, 4>), grid, dim3(256), 0, stream, x, c, h, w, wp, pad_l, out);
+    else if (cpp == 8) hipLaunchKernelGGL((first_from_nchw_kernel<DT_F16, 8>), grid, dim3(256), 0, stream, x, c, h, w, wp, pad_l, out);
+    else hipLaunchKernelGGL((first_from_nchw_kernel<DT_F16, 4>), grid, dim3(256), 0, stream, x, c, h, w, wp, pad_l, out);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
+// fp32 OIHW weights -> [cout][kh][8 columns][cpp channels] 16-bit: filter row i of an output channel as the bytes that
+// meet a receptive-field row of the layout above (columns past kw and channels past cin are zeros)
+template <int DT, int CPP>
+__global__ __launch_bounds__(256) void first_pack_w16_kernel(const float *w, int cin, int kh, int kw, unsigned short *packed, int total) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;   // one (row, filter row, column) per thread
+    if (idx >= total) return;
+    const int j = idx % 8, i = (idx / 8) % kh, row = idx / (8 * kh);
+    float v[CPP];
+#pragma unroll
+    for (int e = 0; e < CPP; ++e) v[e] = e < cin && j < kw ? w[((long long) (row * cin + e) * kh + i) * kw + j] : 0.0f;
+    unsigned short *dst = packed + (long long) idx * CPP;
+    if constexpr (CPP == 8)
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(pack_h16<DT>(v[0], v[1]), pack_h16<DT>(v[2], v[3]), pack_h16<DT>(v[4], v[5]), pack_h16<DT>(v[6], v[7]));
+    else
+        *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_h16<DT>(v[0], v[1]), pack_h16<DT>(v[2], v[3]));
+}
+
+int first_pack_w16_launch(int dt, const float *w, int cout, int cin, int kh, int kw, int cpp, void *packed, hipStream_t stream) {
+    const int total = cout * kh * 8;
+    const dim3 grid((total + 255) / 256);
+    unsigned short *out = reinterpret_cast<unsigned short *>(packed);
+    if (dt == DT_BF16 && cpp == 8) hipLaunchKernelGGL((first_pack_w16_kernel<DT_BF16, 8>), grid, dim3(256), 0, stream, w, cin, kh, kw, out, total);
+    else if (dt == DT_BF16) hipLaunchKernelGGL((first_pack_w16_kernel<DT_BF16, 4>), grid, dim3(256), 0, stream, w, cin, kh, kw, out, total);
+    else if (cpp == 8) hipLaunchKernelGGL((first_pack_w16_kernel<DT_F16, 8>), grid, dim3(256), 0, stream, w, cin, kh, kw, out, total);
+    else hipLaunchKernelGGL((first_pack_w16_kernel<DT_F16, 4>), grid, dim3(256), 0, stream, w, cin, kh, kw, out, total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
 // ---- 16-bit NHWC (pitch cp) -> fp32 NCHW ---------------------------------------------------------------------------
 // The mirror image: a thread reads one 16-byte block and writes its 8 channels to 8 planes; the 16 lanes that share a
 // channel block write 16 consecutive floats of a plane.

@@ -8,7 +8,7 @@ bool dma_ok(const IgemmLaunch &cfg, const IgemmParams &p) {
     if (cfg.dtype != DT_I8 && cfg.dtype != DT_BF16 && cfg.dtype != DT_F16) return false;
     if (cfg.batch != 1 || (cfg.bl != BL_KVEC && cfg.bl != BL_KVEC_TAP)) return false;
     if (!p.use_tapmask || p.units_per_tap < 1 || p.k_units != p.khkw * p.units_per_tap) return false;
-    if (p.lda != p.k_units * 16 || p.pix_stride != p.units_per_tap * 16) return false;
+    if (p.lda != p.k_units * 16 || (p.pix_stride != p.units_per_tap * 16 && !p.tap_spans_pixels)) return false;
     if (reinterpret_cast<uintptr_t>(p.A) % 16 || reinterpret_cast<uintptr_t>(p.B) % 16) return false;
     return dma_stage_bytes(p) != 0 || dma_multi_tap(cfg.dtype, p);
 }

@@ -172,6 +172,9 @@ struct IgemmParams {
     long long a_slice_bytes, b_slice_bytes, c_slice_bytes;  // extent one batch slice can address (< 2 GiB)
     // vector geometry (BL_KVEC)
     int units_per_tap;         // units per filter tap (Cp / 16 for NHWC int8); k_units for a plain matrix
+    int tap_spans_pixels;      // K-vector loaders: a tap's units_per_tap * 16 bytes of K start at the tap's pixel and run on
+                               // into the pixels after it in the row (pix_stride is then less than that): first layers stored
+                               // with few channels per pixel, a filter row being one tap
     unsigned magic_upt, pass_upt;
     int use_tapmask;           // kh*kw <= 64: per-lane tap validity is a 64-bit mask built once per tile
     int pix_stride;            // bytes between consecutive n ("pixels"): Cp, or ldb * elem
@@ -287,6 +290,8 @@ int attention_h16_launch(int dt, const onhip_attention_desc_t &d, const void *q,
 // 16-bit storage (h16.hip): dt is DT_BF16 or DT_F16
 int pack_w16_launch(int dt, const float *w, long long rows, int cin, int taps, int cp, long long s_row, long long s_ch,
                     long long s_tap, void *packed, hipStream_t stream);
+int first_from_nchw_launch(int dt, const float *x, int n, int c, int h, int w, int wp, int cpp, int pad_l, void *y, hipStream_t stream);
+int first_pack_w16_launch(int dt, const float *w, int cout, int cin, int kh, int kw, int cpp, void *packed, hipStream_t stream);
 int nchw_to_nhwc16_launch(int dt, const float *x, int n, int c, int h, int w, int cp, void *y, hipStream_t stream);
 int nhwc16_to_nchw_launch(int dt, const void *x, int n, int c, int h, int w, int cp, float *y, hipStream_t stream);
 int rows_to_h16_launch(int dt, const float *x, long long rows, int k, int kp, void *y, hipStream_t stream);

@@ -39,7 +39,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_matmul", "onhip_matmul_add", "onhip_gemm_f32", "onhip_copy_f32",
            "onhip_h16_pitch", "onhip_h16_packed_weight_bytes", "onhip_h16_pack_conv_weights", "onhip_h16_pack_matmul_weights",
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
-           "onhip_conv2d_h16", "onhip_linear_h16", "onhip_attention", 
+           "onhip_conv2d_h16", "onhip_h16_first_width", "onhip_h16_first_channels", "onhip_h16_first_input_bytes", "onhip_h16_first_weight_bytes", "onhip_h16_first_from_nchw_f32", "onhip_h16_first_pack_weights", "onhip_conv2d_h16_first", "onhip_linear_h16", "onhip_attention", 
            "onhip_ir_block_supported", "onhip_ir_block_packed_weight_bytes", "onhip_ir_block_pack_weights", "onhip_ir_block_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_maxpool_s8_nhwc", "onhip_maxpool_s8_eval", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
@@ -113,6 +113,16 @@ def load():
     L.onhip_h16_from_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
     L.onhip_h16_to_rows_f32.argtypes = [vp, C.c_longlong, i32, i32, vp, vp]
     L.onhip_conv2d_h16.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, i32, vp, i32, vp]
+    L.onhip_h16_first_width.argtypes = [C.POINTER(ConvDesc)]
+    L.onhip_h16_first_width.restype = i32
+    L.onhip_h16_first_channels.argtypes = [C.POINTER(ConvDesc)]
+    L.onhip_h16_first_channels.restype = i32
+    for f in (L.onhip_h16_first_input_bytes, L.onhip_h16_first_weight_bytes):
+        f.argtypes = [C.POINTER(ConvDesc)]
+        f.restype = C.c_size_t
+    L.onhip_h16_first_from_nchw_f32.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    L.onhip_h16_first_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    L.onhip_conv2d_h16_first.argtypes = [C.POINTER(ConvDesc), vp, vp, vp, vp, vp, i32, vp]
     L.onhip_attention.argtypes = [C.POINTER(abi.AttentionDesc), vp, vp, vp, vp, vp]
     L.onhip_ir_block_supported.argtypes = [C.POINTER(ConvDesc)] * 3
     L.onhip_ir_block_packed_weight_bytes.argtypes = [i32, i32, i32]
@@ -544,6 +554,42 @@ def conv2d_h16(d, x, w_packed, bias=None, lut=None, residual=None, residual_relu
             out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device=x.device)
     _check(load().onhip_conv2d_h16(C.byref(d), _ptr(x), _ptr(w_packed), _ptr(bias), _ptr(lut), _ptr(residual),
                                    int(residual_relu), _ptr(out), y_kind, _stream()), "onhip_conv2d_h16")
+    return out
+
+
+def h16_first_from_nchw(d, x):
+    """fp32 NCHW image of a first layer -> its 16-bit storage form [n][h][wp][4 or 8]"""
+    import torch
+    lib = load()
+    wp = lib.onhip_h16_first_width(C.byref(d))
+    if wp < 1:
+        raise OnhipError("16-bit first layer: " + load().onhip_last_error().decode())
+    out = torch.empty((d.n, d.h, wp, lib.onhip_h16_first_channels(C.byref(d))), dtype=_h16_torch_dtype(d.compute), device=x.device)
+    _check(lib.onhip_h16_first_from_nchw_f32(C.byref(d), _ptr(x), _ptr(out), _stream()), "onhip_h16_first_from_nchw_f32")
+    return out
+
+
+def h16_first_pack_weights(d, w):
+    """fp32 OIHW weights of a first layer -> [cout][kh][8][4 or 8] 16-bit"""
+    import torch
+    out = torch.empty((d.cout, d.kh, 8, load().onhip_h16_first_channels(C.byref(d))), dtype=_h16_torch_dtype(d.compute), device=w.device)
+    _check(load().onhip_h16_first_pack_weights(C.byref(d), _ptr(w), _ptr(out), _stream()), "onhip_h16_first_pack_weights")
+    return out
+
+
+def conv2d_h16_first(d, x_first, w_packed, bias=None, lut=None, y_kind=H16_OUT_NHWC, out=None):
+    """conv2d_h16 on the first-layer storage form (h16_first_from_nchw, h16_first_pack_weights)"""
+    import torch
+    oh, ow = d.out_hw()
+    if out is None:
+        if y_kind == H16_OUT_NHWC:
+            out = torch.empty((d.n, oh, ow, h16_pitch(d.cout)), dtype=x_first.dtype, device=x_first.device)
+        elif y_kind == H16_OUT_F32_NHWC:
+            out = torch.empty((d.n, oh, ow, d.cout), dtype=torch.float32, device=x_first.device)
+        else:
+            out = torch.empty((d.n, d.cout, oh, ow), dtype=torch.float32, device=x_first.device)
+    _check(load().onhip_conv2d_h16_first(C.byref(d), _ptr(x_first), _ptr(w_packed), _ptr(bias), _ptr(lut), _ptr(out), y_kind,
+                                         _stream()), "onhip_conv2d_h16_first")
     return out
 
 

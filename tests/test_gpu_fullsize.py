@@ -366,6 +366,33 @@ def test_resnet50_batch32_every_layer_bf16_storage(layer, torch_dev):
     assert not bool(y16[..., d.cout:].any())
 
 
+def test_resnet50_batch32_stem_bf16_in_the_first_layer_form(torch_dev):
+    """the stem as the bf16 benchmark runs it (8 channels per pixel, a filter row per tap): sampled outputs against the
+    float64 sum over the rounded operands; the bf16 store is the rounding of the fp32 one"""
+    torch = torch_dev
+    name, d = RESNET[0]
+    assert d.cin == 3 and d.kh == 7
+    d = ConvDesc.from_buffer_copy(d)
+    d.compute = abi.COMPUTE_BF16
+    x = _device_uniform(torch, _seed("rn50b32h", name, "x"), (d.n, d.cin, d.h, d.w))
+    w = datagen.normal(_seed("rn50b32h", name, "w"), (d.cout, d.cin, d.kh, d.kw), 0.0, float(np.sqrt(2.0 / (d.cin * d.kh * d.kw))))
+    b = datagen.normal(_seed("rn50b32h", name, "b"), (d.cout,), 0.0, 0.01)
+    wd, bd = torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()
+    xf, wp = hip.h16_first_from_nchw(d, x), hip.h16_first_pack_weights(d, wd)
+    y32 = hip.conv2d_h16_first(d, xf, wp, bd, y_kind=hip.H16_OUT_F32_NCHW)
+    y16 = hip.conv2d_h16_first(d, xf, wp, bd)
+    torch.cuda.synchronize()
+    flat, n, m, i, j = _sample_index(_seed("rn50b32h", name, "probe"), d)
+    got = y32.reshape(-1)[torch.from_numpy(flat).cuda()].cpu().numpy().astype(np.float64)
+    p = _patches(torch, _round16(torch, x, d.compute), d, n, i, j).astype(np.float64)
+    wr = _round16(torch, wd, d.compute).cpu().numpy().astype(np.float64)
+    ref = _act_f64(d, np.einsum("sckl,sckl->s", p, wr[m]) + b[m].astype(np.float64))
+    scale = max(float(np.abs(ref).max()), 1e-6)
+    assert np.abs(got - ref).max() <= 1e-4 * scale, f"{name}: {np.abs(got - ref).max():.3e} against {scale:.3e}"
+    assert torch.equal(y16[..., :d.cout], y32.permute(0, 2, 3, 1).to(torch.bfloat16))
+    assert not bool(y16[..., d.cout:].any())
+
+
 # ---- YOLOv8s int8, batch 16 ---------------------------------------------------------------------------------------
 
 def _yolo_operands(torch, i, name, d):

@@ -135,6 +135,70 @@ def test_conv_h16_every_tile(compute, ring, tile, shape, torch_dev, oracle, monk
     assert not got16[..., cout:].any(), "channel padding of the output must be zero"
 
 
+# (n, cin, h, w, cout, kh, kw, stride, pad): first layers in their own storage form; the ResNet-50 / MobileNetV2 / YOLOv8
+# stems in small, a ragged one (cin 1, 5 x 8 filter, stride 3, more padding than the filter needs), stride 1
+FIRST_SHAPES = [(2, 3, 30, 30, 64, 7, 7, 2, 3), (1, 3, 20, 36, 32, 3, 3, 2, 1), (2, 1, 17, 23, 9, 5, 8, 3, 4),
+                (1, 8, 12, 12, 40, 3, 3, 1, 1), (3, 4, 9, 40, 130, 1, 2, 1, 0), (2, 3, 11, 13, 24, 3, 3, 1, 1),
+                (1, 5, 15, 15, 16, 4, 4, 3, 2)]
+
+
+@pytest.mark.parametrize("compute", TYPES)
+@pytest.mark.parametrize("tile", [None, "128x128", "128x64", "64x128", "64x64x1x0x0x0x2"])
+@pytest.mark.parametrize("shape", FIRST_SHAPES)
+def test_conv_h16_first_layer_form(compute, tile, shape, torch_dev, oracle, monkeypatch):
+    """onhip_conv2d_h16_first against the oracle on rounded operands, and bit for bit against onhip_conv2d_h16 on the
+    32-channel form where both take the shape with the same tile (same products, zeros added in between)"""
+    torch = torch_dev
+    if tile:
+        monkeypatch.setenv("ONHIP_TILE", tile)
+    n, cin, h, w, cout, kh, kw, stride, pad = shape
+    d = ConvDesc(n=n, cin=cin, h=h, w=w, cout=cout, kh=kh, kw=kw, stride_h=stride, stride_w=stride, pad_t=pad, pad_l=pad,
+                 pad_b=pad, pad_r=pad, group=1, has_bias=1, act_type=abi.RELU, compute=compute)
+    name = f"h16first_{cin}_{cout}_{kh}x{kw}_{stride}"
+    print(f"case {name} tile {tile} compute {compute}", flush=True)
+    rnd = rounder(oracle, compute)
+    x, wt, b = cases.conv_inputs(name, d)
+    xf = hip.h16_first_from_nchw(d, dev(torch, x))
+    wp_cols = xf.shape[2]
+    oh, ow = d.out_hw()
+    cpp = 4 if cin <= 4 else 8
+    assert wp_cols == hip.load().onhip_h16_first_width(d) >= max(w + 2 * pad, (ow - 1) * stride + 8) and wp_cols % 2 == 0
+    assert xf.shape[3] == hip.load().onhip_h16_first_channels(d) == cpp
+    # the storage form itself: rounded pixels at column + pad_l, zeros around them and in the channels past cin
+    got = xf.float().cpu().numpy()
+    want = np.zeros((n, h, wp_cols, cpp), np.float32)
+    want[:, :, pad:pad + w, :cin] = np.transpose(rnd(x), (0, 2, 3, 1))
+    assert np.array_equal(got, want)
+    wpk = hip.h16_first_pack_weights(d, dev(torch, wt))
+    wwant = np.zeros((cout, kh, 8, cpp), np.float32)
+    wwant[:, :, :kw, :cin] = np.transpose(rnd(wt), (0, 2, 3, 1))
+    assert np.array_equal(wpk.float().cpu().numpy(), wwant)
+    launches = hip.load().onhip_direct_lds_launches()
+    y_nchw = hip.conv2d_h16_first(d, xf, wpk, dev(torch, b), y_kind=hip.H16_OUT_F32_NCHW).cpu().numpy()
+    out16 = torch.full((n, oh, ow, hip.h16_pitch(cout)), 7.0, dtype=xf.dtype, device="cuda")
+    hip.conv2d_h16_first(d, xf, wpk, dev(torch, b), y_kind=hip.H16_OUT_NHWC, out=out16)
+    torch.cuda.synchronize()
+    assert hip.load().onhip_direct_lds_launches() == launches + 2, "the first-layer form did not run on the direct-to-LDS kernel"
+    ref = oracle.conv2d_f32(d, rnd(x), rnd(wt), b)
+    assert norm_diff(y_nchw, ref) <= 1e-4, f"vs oracle on rounded operands: {norm_diff(y_nchw, ref):.3e}"
+    assert norm_diff(y_nchw, oracle.conv2d_f32(d, x, wt, b)) <= 1e-2
+    got16 = out16.float().cpu().numpy()
+    assert np.array_equal(got16[..., :cout], rnd(np.transpose(y_nchw, (0, 2, 3, 1))))
+    assert not got16[..., cout:].any(), "channel padding of the output must be zero"
+
+
+def test_conv_h16_first_layer_form_refuses_what_it_cannot_store(torch_dev):
+    d = ConvDesc(n=1, cin=9, h=8, w=8, cout=8, kh=3, kw=3, stride_h=1, stride_w=1, pad_t=1, pad_l=1, pad_b=1, pad_r=1,
+                 group=1, has_bias=0, act_type=abi.NOT_ACT, compute=abi.COMPUTE_BF16)
+    assert hip.load().onhip_h16_first_width(d) == 0          # nine channels
+    d.cin, d.kw, d.pad_l, d.pad_r = 3, 9, 4, 4
+    assert hip.load().onhip_h16_first_width(d) == 0          # filter rows of nine columns
+    d.kw, d.pad_l, d.pad_r, d.compute = 3, 1, 1, abi.COMPUTE_F32
+    x = torch_dev.zeros((1, 3, 8, 8), device="cuda")
+    with pytest.raises(hip.OnhipError):
+        hip.h16_first_from_nchw(d, x)                        # not a 16-bit type
+
+
 @pytest.mark.parametrize("compute", TYPES)
 @pytest.mark.parametrize("act", ["none", "clip", "silu", "leaky", "nobias"])
 def test_conv_h16_activations(compute, act, torch_dev, oracle, monkeypatch):
