@@ -40,7 +40,7 @@ LEGEND = ("Kernel names: `onhip::igemm_kernel<dtype, loader, BM, BN, WM, WN, PF,
           "straight from memory, tile 32 WM x 128 WN), `onhip::splitk_finish_kernel`, `onhip::depthwise_tiled_kernel<int8, stride, "
           "act>`, `onhip::quantize_nhwc_kernel<CBW>`, `onhip::stem_f32_kernel<filter size, act, two row tiles>` (first-layer "
           "convolutions from an LDS patch), `onhip::i8patch_kernel<bytes per pixel, WM, pixel tiles>` and `onhip::i8direct_kernel<bytes per pixel, taps, WM, TM, pixel "
-          "tiles, workgroups per CU>` (int8 chain form, 3x3 with few channels: input rows in LDS / windows loaded per tap), `onhip::attention_f32_kernel<key tiles, head dim>`, `onhip::irblock_f32_kernel<act, input channels / 4, row tiles, "
+          "tiles, workgroups per CU>` (int8 chain form, 3x3 with few channels: input rows in LDS / windows loaded per tap), `onhip::attention_f32_kernel<16-key tiles, head dim>`, `onhip::dw_s8_nhwc_kernel<3x3 stride, epilogue, fp32 out>` (depthwise on int8 NHWC), `onhip::irblock_f32_kernel<act, input channels / 4, row tiles, "
           "patches>` (1x1 expansion + depthwise 3x3 + 1x1 projection in one launch), and the element-wise kernels.")
 
 
@@ -55,7 +55,7 @@ def family(name):
         return None
     if "igemm" in name or "splitk_finish" in name or "rowb_f32" in name or "attention" in name or "stem_f32" in name or "i8patch" in name or "i8direct" in name:
         return "igemm"
-    if "depthwise" in name or "irblock" in name:
+    if "depthwise" in name or "irblock" in name or "dw_s8" in name:
         return "depthwise"
     if "quantize_nhwc" in name:
         return "quantize"
