@@ -245,6 +245,226 @@ __global__ __launch_bounds__(256) void dw_s8_nhwc_kernel(const DwS8Params p) {
 }
 
 
+// ---- 3x3 filters on the matrix cores ------------------------------------------------------------------------------------
+// The kernel above needs about 47 vector instructions per output byte (byte -> float conversions, nine multiply-adds,
+// the store's arithmetic) and is bound by them: counters put its vector pipes at 60 % busy and its memory pipes nearly
+// idle.  The matrix cores do a depthwise filter tap as a product with a DIAGONAL matrix: for 32 channels and 32 pixels,
+//     v_mfma_i32_32x32x32_i8:  D[m][n] += sum_k A[m][k] B[k][n],  A[m][k] = (m == k) ? w[channel m][tap] : 0,
+//                                                                B[k][n] = x[pixel n under the tap][channel k]
+// 31 of 32 products are with zero, and it is still a third of the vector instructions' time, on a pipe that runs beside
+// them.  B is exactly what memory holds: a lane's operand, 16 consecutive reduction indices of one column, is the 16
+// bytes of one channel group of one NHWC pixel; the nine taps are nine loads at shifted pixels (zeros outside the image
+// from the buffer descriptor: int8 zero is the real zero, no bias trick).  The int32 sums are exact, so the bytes are
+// those of the kernel above and of the reference (conv.c:727-752, :961-973).
+//   * A workgroup owns a band of output rows of one image and up to 8 channel groups.  It copies the input rows the band
+//     reads (halo included) into LDS with consecutive lanes on consecutive 16-byte units of memory, so memory is read once
+//     and in runs; the nine shifted operands of a block of 32 output pixels are then nine ds_read_b128.  (Loaded straight
+//     from memory they are nine loads of 32 useful bytes per cache line, the L1 does not hold the lines of the wavefronts
+//     of a compute unit, and the layer is bound by refetching them: 57 us for 144 channels on 56 x 56 x 64 either way.)
+//   * A wavefront owns one block of 32 channels (two 16-channel groups) and walks the band's blocks of 32 output pixels;
+//     its nine diagonal matrices (36 registers) and its lanes' 16 biases and 16 factors are set up once.
+//   * The accumulator gives a lane one pixel and the channels 8 q + 4 (lane / 32) + k: for the int8 NHWC store the two lane
+//     halves exchange two dwords, after which each holds the 16 consecutive bytes of one channel group (one 128-bit
+//     store); for the fp32 NCHW store the layout is already right (32 consecutive pixels of a channel per store).
+struct DwMfmaParams {
+    DwS8Params b;
+    int gc;                // channel groups (16 channels) per workgroup: 2, 4 or 8, i.e. one block of 32 channels per wavefront
+    int gchunks;           // chunks of gc groups
+    int pitch_u;           // 16-byte units a pixel takes in LDS: gc + 1, odd, so that neighbouring pixels start in different banks
+    int brows;             // output rows of a band
+    int bands;             // bands per image
+    int rows, lw;          // input rows and columns of a band, halo included
+    int gc_last;           // groups of the last chunk (G - (gchunks - 1) * gc)
+    int gsh, gsh_last;     // log2 of gc, and of gc_last rounded up to a power of two
+    int consts_at;         // byte offset of the per-wavefront channel constants in LDS
+    Div31 div_row, div_rowl;   // by the units of a staged row, lw << gsh, and the same for the last chunk
+    Div31 div_gchunks, div_bands;
+};
+
+// a 16-byte LDS read the compiler neither delays to its use nor waits for on its own: the nine operand reads of a pixel
+// block are issued together and waited for once (left to the compiler, each read sits right before its MFMA with a wait
+// in between: nine LDS latencies per block)
+__device__ __forceinline__ i32x4 dws8_lds_read(unsigned addr) {
+    i32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
+template <int EPI, bool OUT_F32>
+__global__ __launch_bounds__(256) void dw_s8_mfma_kernel(const DwMfmaParams mp) {
+    constexpr int UNR = 4;
+    const DwS8Params &p = mp.b;
+    extern __shared__ __align__(16) unsigned char tile[];          // [rows][lw][pitch_u][16 bytes], then [4 wavefronts][2][32] floats
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    int lid;
+    {
+        const int nb = (int) gridDim.x, bid = (int) blockIdx.x;
+        const int q = nb >> 3, rmd = nb & 7, xcd = bid & 7, idx = bid >> 3;
+        lid = xcd * q + (xcd < rmd ? xcd : rmd) + idx;
+    }
+    // chunks of the same pixels next to each other (they share cache lines), then the bands of an image (they share rows)
+    const int nbnd = dws8_div(lid, mp.div_gchunks), gchunk = lid - nbnd * mp.gchunks;
+    const int n = dws8_div(nbnd, mp.div_bands), band = nbnd - n * mp.bands;
+    const int g_first = gchunk * mp.gc;
+    const rsrc_t rx = make_rsrc(p.x, p.x_bytes);
+    const rsrc_t ry = make_rsrc(p.y, p.y_bytes);
+
+    // the band's input rows into LDS: consecutive lanes on consecutive 16-byte units of memory (runs of 16 gc bytes per
+    // pixel); everything outside the image, and groups past the last, as zeros from the buffer descriptor
+    const int ih_base = band * mp.brows * p.sh - p.pad;
+    const bool last_chunk = gchunk == mp.gchunks - 1;                // uniform
+    const int groups_here = last_chunk ? mp.gc_last : mp.gc;
+    // units are numbered (row, column, group) with the groups of a pixel rounded up to a power of two (gc is one; the
+    // last chunk may have fewer): one division per unit, the rest is shifts
+    const int gsh = last_chunk ? mp.gsh_last : mp.gsh;
+    const Div31 drow = last_chunk ? mp.div_rowl : mp.div_row;
+    const int row_units = mp.lw << gsh, units = mp.rows * row_units;
+    for (int base = 0; base < units; base += 256 * UNR) {
+        uint4 v[UNR];
+        unsigned dst[UNR];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            const int u = base + k * 256 + tid;
+            const int row = dws8_div(u, drow), rem = u - row * row_units;
+            const int col = rem >> gsh, unit = rem & ((1 << gsh) - 1);
+            const int ih = ih_base + row, iw = col - p.pad;
+            const bool ok = u < units && unit < groups_here && (unsigned) ih < (unsigned) p.H && (unsigned) iw < (unsigned) p.W;
+            v[k] = buf_load_b128(rx, ok ? (unsigned) (((n * p.H + ih) * p.W + iw) * p.Cp + (g_first + unit) * 16) : OOB, 0u);
+            dst[k] = u < units ? (unsigned) (((row * mp.lw + col) * mp.pitch_u + unit) * 16) : 0xffffffffu;
+        }
+#pragma unroll
+        for (int k = 0; k < UNR; ++k)
+            if (dst[k] != 0xffffffffu) *reinterpret_cast<uint4 *>(tile + dst[k]) = v[k];
+    }
+
+    // The wavefront's block of 32 channels: with fewer than four blocks in the chunk the wavefronts share them and split
+    // the pixels (three blocks: the fourth wavefront only helps with the copy).
+    const int nbl = (groups_here + 1) >> 1;
+    const int wave_c = nbl >= 3 ? 4 : nbl, cbl = wave % wave_c, psub = wave / wave_c, pstep = 4 / wave_c;
+    const int cb0 = g_first * 16 + cbl * 32;                        // first channel of the block
+    const bool group_ok = g_first + cbl * 2 + lh < p.G;             // the lane half's channel group exists
+    // the nine diagonal matrices: row li, reduction indices 16 lh .. 16 lh + 15; the diagonal passes through this lane
+    // when li / 16 == lh, at byte li % 16
+    i32x4 amat[9];
+    {
+        const int c = cb0 + li;
+        const bool on = cbl < nbl && (li >> 4) == lh && c < p.C;
+        const rsrc_t rw = make_rsrc(p.w, (unsigned) (p.C * 9));
+        unsigned wb[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+            wb[t] = (unsigned) __builtin_amdgcn_raw_buffer_load_b8(rw, on ? (unsigned) (c * 9 + t) : OOB, 0, 0) & 0xffu;
+        const int dw = (li & 15) >> 2, sh = 8 * (li & 3);
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int v = (int) (wb[t] << sh);
+            amat[t] = i32x4{dw == 0 ? v : 0, dw == 1 ? v : 0, dw == 2 ? v : 0, dw == 3 ? v : 0};
+        }
+    }
+    // bias (as a float) and factor weight_aux / 127 of the block's 32 channels: lane li of the lower half fetches and divides
+    // for channel li, the lanes pick their 16 channels 8 q + 4 lh + k up from LDS after the barrier
+    float *wconst = reinterpret_cast<float *>(tile + mp.consts_at) + wave * 64;
+    if (lh == 0) {
+        const rsrc_t rb = make_rsrc(p.b32, (unsigned) (p.C * 4)), ra = make_rsrc(p.aux, (unsigned) (p.C * 4));
+        const unsigned off = (unsigned) (cb0 + li) * 4u;               // past C: zeros
+        wconst[li] = (float) (int) __builtin_amdgcn_raw_buffer_load_b32(rb, off, 0, 0);
+        wconst[32 + li] = __fdiv_rn(buf_load_f32(ra, off, 0), 127.0f);
+    }
+    // which bytes of the lane's four output words are channels of the tensor (the rest are written as zero)
+    unsigned keep[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        keep[q] = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) keep[q] |= cb0 + 8 * q + 4 * lh + k < p.C ? 0xffu << (8 * k) : 0u;
+    }
+    __syncthreads();
+    if (cbl >= nbl) return;
+    const unsigned lds0 = (unsigned) (size_t) (__attribute__((address_space(3))) unsigned char *) tile;
+    float bias[16], coeff[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float4 b4 = *reinterpret_cast<const float4 *>(wconst + 8 * q + 4 * lh);
+        const float4 c4 = *reinterpret_cast<const float4 *>(wconst + 32 + 8 * q + 4 * lh);
+        bias[4 * q] = b4.x; bias[4 * q + 1] = b4.y; bias[4 * q + 2] = b4.z; bias[4 * q + 3] = b4.w;
+        coeff[4 * q] = c4.x; coeff[4 * q + 1] = c4.y; coeff[4 * q + 2] = c4.z; coeff[4 * q + 3] = c4.w;
+    }
+    // int8 output behind no activation, Relu or Clip: activation, the product with 1 / output_scale and the quantiser's
+    // clamp are one median of three on v / output_scale.  The product is monotonic and so is its rounding, so clamping
+    // before it to [a, b] and after it to [fl(a / s), fl(b / s)] give the same float; two nested clamps are one.  (A NaN
+    // comes out as the lower bound here and as 0 from the separate steps; no finite scale or weight produces one.)
+    float q_lo = -128.0f, q_hi = 127.0f;
+    if constexpr (EPI == EPI_RELU) q_lo = 0.0f;
+    if constexpr (EPI == EPI_CLIP) {
+        q_lo = fmaxf(__fmul_rn(p.ep.clip_min, p.out_inv_scale), -128.0f);
+        q_hi = fminf(__fmul_rn(p.ep.clip_max, p.out_inv_scale), 127.0f);
+    }
+
+    const int oh_first = band * mp.brows;
+    const int band_pix = min(mp.brows, p.OH - oh_first) * p.OW;     // output pixels of this band
+    const int pblocks = (band_pix + 31) >> 5;
+    for (int pb = psub; pb < pblocks; pb += pstep) {
+        const int pi = pb * 32 + li;
+        const bool live = pi < band_pix;
+        const int pc = live ? pi : 0;
+        const int orow = dws8_div(pc, p.div_ow), ow = pc - orow * p.OW;
+        const int oh = oh_first + orow;
+        const unsigned in0 = (unsigned) (((orow * p.sh) * mp.lw + ow * p.sw) * mp.pitch_u + cbl * 2 + lh) * 16u;
+        i32x4 xv[9];
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+#pragma unroll
+            for (int j = 0; j < 3; ++j) xv[i * 3 + j] = dws8_lds_read(lds0 + in0 + (unsigned) ((i * mp.lw + j) * mp.pitch_u) * 16u);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(xv[0]), "+v"(xv[1]), "+v"(xv[2]), "+v"(xv[3]), "+v"(xv[4]), "+v"(xv[5]), "+v"(xv[6]), "+v"(xv[7]), "+v"(xv[8])
+                     :: "memory");
+        i32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(amat[t], xv[t], acc, 0, 0, 0);
+
+        unsigned word[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            int b8[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int r = 4 * q + k, c = cb0 + 8 * q + 4 * lh + k;
+                // conv.c:739 and :746-752: acc * s + bias32, then * (aux / 127): separately rounded
+                const float fl = __fadd_rn(__fmul_rn((float) acc[r], p.in_scale), bias[r]);
+                const float pre = __fmul_rn(fl, coeff[r]);
+                if constexpr (OUT_F32) {
+                    const bool ok = live && c < p.C;
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(act_fast<EPI>(pre, p.ep)), ry,
+                                                          ok ? (unsigned) (((n * p.C + c) * p.OH + oh) * p.OW + ow) * 4u : OOB, 0, 0);
+                } else if constexpr (EPI == EPI_GENERIC) {
+                    b8[k] = quant_s8(act_fast<EPI>(pre, p.ep), p.out_inv_scale);
+                } else {
+                    b8[k] = round_half_away_small(__builtin_amdgcn_fmed3f(__fmul_rn(pre, p.out_inv_scale), q_lo, q_hi));
+                }
+            }
+            if constexpr (!OUT_F32) {
+                // the low bytes of four integers into one word: three byte permutes
+                const unsigned p01 = __builtin_amdgcn_perm((unsigned) b8[1], (unsigned) b8[0], 0x0c0c0400u);
+                const unsigned p23 = __builtin_amdgcn_perm((unsigned) b8[3], (unsigned) b8[2], 0x0c0c0400u);
+                word[q] = __builtin_amdgcn_perm(p23, p01, 0x05040100u) & keep[q];
+            }
+        }
+        if constexpr (!OUT_F32) {
+            // word[q] = channels 8 q + 4 lh .. + 3.  Lane half 0 stores channels 0..15 = {own 0, partner 0, own 1, partner 1},
+            // half 1 channels 16..31 = {partner 2, own 2, partner 3, own 3}: each half sends the two words the other needs
+            const unsigned r0 = (unsigned) __shfl_xor((int) (lh ? word[0] : word[2]), 32, 64);
+            const unsigned r1 = (unsigned) __shfl_xor((int) (lh ? word[1] : word[3]), 32, 64);
+            const u32x4 out = lh ? u32x4{r0, word[2], r1, word[3]} : u32x4{word[0], r0, word[1], r1};
+            // the whole offset in the vector offset, scalar offset the constant 0: see the store of the kernel above
+            __builtin_amdgcn_raw_buffer_store_b128(out, ry, live && group_ok ? (unsigned) (((n * p.OH + oh) * p.OW + ow) * p.Cp + cb0 + lh * 16) : OOB,
+                                                   0, 0);
+        }
+    }
+}
+
 // the shapes the kernel takes: what fits its LDS table of weights and its 32-bit offsets
 bool dw_s8_ok(const onhip_conv_desc_t &d, int OH, int OW) {
     const long long cp = (d.cout + 15) / 16 * 16;
@@ -254,6 +474,16 @@ bool dw_s8_ok(const onhip_conv_desc_t &d, int OH, int OW) {
     if ((long long) d.n * d.h * d.w * cp >= (1LL << 31) || (long long) d.n * OH * OW * cp >= (1LL << 31)) return false;
     if ((long long) d.n * d.cout * OH * OW * 4 >= (1LL << 31)) return false;
     return true;
+}
+
+template <bool OUT_F32>
+static void dw_s8_mfma_dispatch(int epi, unsigned wgs, size_t lds, hipStream_t st, const DwMfmaParams &p) {
+    switch (epi) {
+        case EPI_NONE: hipLaunchKernelGGL((dw_s8_mfma_kernel<EPI_NONE, OUT_F32>), dim3(wgs), dim3(256), lds, st, p); break;
+        case EPI_RELU: hipLaunchKernelGGL((dw_s8_mfma_kernel<EPI_RELU, OUT_F32>), dim3(wgs), dim3(256), lds, st, p); break;
+        case EPI_CLIP: hipLaunchKernelGGL((dw_s8_mfma_kernel<EPI_CLIP, OUT_F32>), dim3(wgs), dim3(256), lds, st, p); break;
+        default: hipLaunchKernelGGL((dw_s8_mfma_kernel<EPI_GENERIC, OUT_F32>), dim3(wgs), dim3(256), lds, st, p); break;
+    }
 }
 
 template <int S3, bool OUT_F32>
@@ -292,6 +522,43 @@ int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, c
     p.x_bytes = (unsigned) ((long long) d.n * d.h * d.w * p.Cp);
     p.y_bytes = d.out_s8 ? (unsigned) ((long long) d.n * OH * OW * p.Cp) : (unsigned) ((long long) d.n * d.cout * OH * OW * 4);
     p.ep = ep;
+    const int epi = epi_of_act(ep.act);
+    if (d.kh == 3 && d.kw == 3 && !getenv("ONHIP_DW_NO_MFMA")) {   // 3x3, any stride: the matrix-core kernel
+        DwMfmaParams mp;
+        memset(&mp, 0, sizeof(mp));
+        mp.b = p;
+        mp.gc = p.G >= 8 ? 8 : p.G > 2 ? (p.G + 1) / 2 * 2 : 2;
+        if (mp.gc == 6) mp.gc = 4;                                 // blocks of 32 channels in ones, twos or fours per workgroup
+        mp.gchunks = (p.G + mp.gc - 1) / mp.gc;
+        mp.pitch_u = mp.gc + 1;
+        mp.lw = (OW - 1) * d.stride_w + 3;
+        const long long row_bytes = (long long) mp.lw * mp.pitch_u * 16;
+        auto rows_of = [&](int brows) { return (brows - 1) * d.stride_h + 3; };
+        // the tallest band whose input fits 48 KiB of LDS (three workgroups per compute unit), shortened while that leaves
+        // the chip fewer than 1024 workgroups
+        int brows = OH;
+        while (brows > 1 && (rows_of(brows) * row_bytes > 48 * 1024 || (long long) d.n * ((OH + brows - 1) / brows) * mp.gchunks < 1024)) --brows;
+        if (rows_of(brows) * row_bytes <= 64 * 1024) {
+            mp.brows = brows;
+            mp.bands = (OH + brows - 1) / brows;
+            mp.rows = rows_of(brows);
+            mp.gc_last = p.G - (mp.gchunks - 1) * mp.gc;
+            mp.gsh = mp.gc == 8 ? 3 : mp.gc == 4 ? 2 : 1;
+            mp.gsh_last = mp.gc_last > 4 ? 3 : mp.gc_last > 2 ? 2 : mp.gc_last > 1 ? 1 : 0;
+            mp.div_row = make_div31((unsigned) (mp.lw << mp.gsh));
+            mp.div_rowl = make_div31((unsigned) (mp.lw << mp.gsh_last));
+            mp.consts_at = (int) (mp.rows * row_bytes);
+            mp.div_gchunks = make_div31((unsigned) mp.gchunks);
+            mp.div_bands = make_div31((unsigned) mp.bands);
+            const long long wgs = (long long) d.n * mp.bands * mp.gchunks;
+            if (wgs > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise int8 NHWC: too many workgroups");
+            const size_t lds = (size_t) mp.rows * row_bytes + 4 * 64 * sizeof(float);
+            if (d.out_s8) dw_s8_mfma_dispatch<false>(epi, (unsigned) wgs, lds, stream, mp);
+            else dw_s8_mfma_dispatch<true>(epi, (unsigned) wgs, lds, stream, mp);
+            ONHIP_CHECK_HIP(hipGetLastError());
+            return ONHIP_OK;
+        }
+    }
     const int per_wg = 64 * (4 / p.gw);
     const int gchunks = (p.G + p.gw - 1) / p.gw;
     p.pchunks = (int) ((items + per_wg - 1) / per_wg);
@@ -299,7 +566,6 @@ int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, c
     const long long wgs = (long long) p.pchunks * gchunks;
     if (wgs > 0x7fffffffLL) return set_error(ONHIP_ERR_ARG, "depthwise int8 NHWC: too many workgroups");
     const size_t lds_bytes = ((size_t) p.gw * 16 * p.taps + (size_t) p.gw * 48) * 4;
-    const int epi = epi_of_act(ep.act);
     if (d.out_s8) {
         if (s3 == 1) dw_s8_dispatch<1, false>(epi, (unsigned) wgs, lds_bytes, stream, p);
         else if (s3 == 2) dw_s8_dispatch<2, false>(epi, (unsigned) wgs, lds_bytes, stream, p);
