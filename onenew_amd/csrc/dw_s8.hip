@@ -529,15 +529,20 @@ int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, c
         mp.b = p;
         mp.gc = p.G >= 8 ? 8 : p.G > 2 ? (p.G + 1) / 2 * 2 : 2;
         if (mp.gc == 6) mp.gc = 4;                                 // blocks of 32 channels in ones, twos or fours per workgroup
+        // 9 or 10 groups in chunks of 8 leave a chunk of one or two whose workgroups copy as many rows as the full ones; in
+        // chunks of 4, with the smaller tiles five workgroups fit a compute unit (144 channels on 56 x 56 x 64: 39 -> 30 us)
+        long long lds_cap = 48 * 1024;
+        if (p.G == 9 || p.G == 10) { mp.gc = 4; lds_cap = 32 * 1024; }
         mp.gchunks = (p.G + mp.gc - 1) / mp.gc;
         mp.pitch_u = mp.gc + 1;
         mp.lw = (OW - 1) * d.stride_w + 3;
         const long long row_bytes = (long long) mp.lw * mp.pitch_u * 16;
         auto rows_of = [&](int brows) { return (brows - 1) * d.stride_h + 3; };
         // the tallest band whose input fits 48 KiB of LDS (three workgroups per compute unit), shortened while that leaves
-        // the chip fewer than 1024 workgroups
+        // the chip fewer than 1024 workgroups.  (Measured and not kept: two pixel blocks per trip with their MFMA chains
+        // interleaved, 10 to 25 % slower for its registers; bands down to 16 KiB for more workgroups per unit, slower.)
         int brows = OH;
-        while (brows > 1 && (rows_of(brows) * row_bytes > 48 * 1024 || (long long) d.n * ((OH + brows - 1) / brows) * mp.gchunks < 1024)) --brows;
+        while (brows > 1 && (rows_of(brows) * row_bytes > lds_cap || (long long) d.n * ((OH + brows - 1) / brows) * mp.gchunks < 1024)) --brows;
         if (rows_of(brows) * row_bytes <= 64 * 1024) {
             mp.brows = brows;
             mp.bands = (OH + brows - 1) / brows;
