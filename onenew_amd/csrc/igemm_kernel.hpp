@@ -521,8 +521,13 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
         }
         qtab_lds = (lds_s8_t) ql;
     }
-    const bool has_bias = p.bias32 != nullptr;
     const bool table = EPI == EPI_LUT && p.ep.qlut != nullptr;   // uniform: the table entries arrive quantised
+    float q_lo = -128.0f, q_hi = 127.0f;                         // the merged clamp of the branch without a table
+    if constexpr (EPI == EPI_RELU) q_lo = 0.0f;
+    if constexpr (EPI == EPI_CLIP) {
+        q_lo = fmaxf(__fmul_rn(p.ep.clip_min, p.out_inv_scale), -128.0f);
+        q_hi = fminf(__fmul_rn(p.ep.clip_max, p.out_inv_scale), 127.0f);
+    }
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -537,9 +542,9 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int r = 4 * q + j;
-                    float f = __fmul_rn((float) acc[a][b][r], p.in_scale);
-                    const float fbias = __fadd_rn(f, fb32[a][r]);
-                    f = has_bias ? fbias : f;
+                    // without a bias fb32 is 0, and adding it changes nothing that reaches an int8 result (the sum of an
+                    // integer times a positive scale is never -0)
+                    const float f = __fadd_rn(__fmul_rn((float) acc[a][b][r], p.in_scale), fb32[a][r]);
                     x[b][j] = __fmul_rn(f, aux[a][r]);
                 }
             if (table && QLUT_IN_LDS) {
@@ -600,6 +605,16 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
                             q8[b][j] = x[b][j] >= 8.0f ? hi : q8[b][j];
                         }
                 }
+            } else if constexpr (EPI == EPI_NONE || EPI == EPI_RELU || EPI == EPI_CLIP) {
+                // activation, product with 1 / output_scale and the quantiser's clamp as ONE median of three on
+                // x / output_scale: the product and its rounding are monotonic, so clamping to [a, b] before it and to
+                // [fl(a / s), fl(b / s)] after it give the same float, and two nested clamps are one.  (A NaN comes out as
+                // the lower bound here and as 0 from the separate steps; no finite scale or weight produces one.)
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        q8[b][j] = round_half_away_small(__builtin_amdgcn_fmed3f(__fmul_rn(x[b][j], p.out_inv_scale), q_lo, q_hi));
             } else {
 #pragma unroll
                 for (int b = 0; b < TN; ++b)
@@ -611,9 +626,10 @@ __device__ __forceinline__ void write_tile_nhwc_s8(const IgemmParams &p, ACC (&a
             const unsigned keep = left >= 4 ? 0xffffffffu : left <= 0 ? 0u : (1u << (8 * left)) - 1u;
 #pragma unroll
             for (int b = 0; b < TN; ++b) {
-                unsigned packed = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) packed |= ((unsigned) q8[b][j] & 0xffu) << (8 * j);
+                // the low bytes of four integers into one word: three byte permutes
+                const unsigned p01 = __builtin_amdgcn_perm((unsigned) q8[b][1], (unsigned) q8[b][0], 0x0c0c0400u);
+                const unsigned p23 = __builtin_amdgcn_perm((unsigned) q8[b][3], (unsigned) q8[b][2], 0x0c0c0400u);
+                const unsigned packed = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
                 const int nl = n_wave - n0 + b * 32 + li;
                 *reinterpret_cast<unsigned *>(stage + nl * PITCH + ml) = packed & keep;
             }
