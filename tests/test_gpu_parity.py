@@ -1453,12 +1453,17 @@ DW_CHAIN = [(12, 11, 11, 3, 1, 1, abi.SILU, 2), (10, 14, 14, 3, 2, 1, abi.CLIP, 
             (32, 28, 28, 3, 1, 1, abi.CLIP, 2), (96, 30, 26, 3, 2, 1, abi.CLIP, 2), (144, 13, 17, 3, 1, 1, abi.RELU, 1),
             (960, 7, 7, 3, 1, 1, abi.CLIP, 3), (24, 70, 70, 3, 1, 1, abi.LEAKYRELU, 1), (40, 15, 15, 3, 3, 1, abi.HARDSILU, 2),
             (17, 12, 12, 7, 2, 3, abi.RELU, 2), (48, 5, 5, 3, 1, 1, abi.SILU, 9), (200, 9, 20, 5, 2, 2, abi.CLIP, 2),
-            (16, 6, 130, 3, 2, 1, abi.NOT_ACT, 1), (64, 1, 1, 3, 1, 1, abi.RELU, 70)]
+            (16, 6, 130, 3, 2, 1, abi.NOT_ACT, 1), (64, 1, 1, 3, 1, 1, abi.RELU, 70),
+            # 3x3 without padding and with more than it needs; 33 channels: Clip bounds inside the int8 range (see below)
+            (20, 9, 9, 3, 1, 0, abi.RELU, 2), (33, 10, 8, 3, 2, 2, abi.CLIP, 2), (272, 31, 33, 3, 1, 1, abi.CLIP, 1)]
 
 
 def _dw_chain_desc(shape):
     c, h, w, k, s, pad, act, n = shape
-    d = cases.cd(c, c, k, s, pad, h, w, act=act, group=c, n=n, input_scale=0.013, clip_min=0.0, clip_max=6.0,
+    # 33 channels: Clip to [-1, 2.5], i.e. to [-27, 68] output steps, so that the activation's bounds and not the
+    # quantiser's are what clamps
+    lo, hi = (-1.0, 2.5) if c == 33 else (0.0, 6.0)
+    d = cases.cd(c, c, k, s, pad, h, w, act=act, group=c, n=n, input_scale=0.013, clip_min=lo, clip_max=hi,
                  leaky_relu_alpha=0.1, hard_sigmoid_alpha=0.2, hard_sigmoid_beta=0.5)
     return d
 
