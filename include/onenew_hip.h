@@ -318,6 +318,26 @@ int onhip_ir_block_f32(const onhip_conv_desc_t *expand, const onhip_conv_desc_t 
                        const float *packed, const float *expand_b, const float *dw_w, const float *dw_b, const float *project_b,
                        const float *residual, float *y, void *stream);
 
+/* A dense convolution and the 1x1 convolution that reads its result, in one launch:  y = b(a(x)) [+ addend, then Relu].
+ * Replaces two operator evaluations (device/x86/Conv/conv.c:300-415 twice: im2col + SGEMM + bias + activation, the second
+ * with a 1x1 filter) and, with `addend`, the Add and Relu after them (device/x86/Add/add.c, device/x86/Relu/relu.c:27-52);
+ * the tensor between the two convolutions is never written to memory: a workgroup holds all of a's output channels for its
+ * 64 pixels and multiplies them by b's weights before it stores.  fp32; both products sum in MFMA order, so the pair equals
+ * the two operators within fp32 summation error.  No counterpart as one function in the reference.
+ * a: dense, at most 64 output channels, not a plain 1x1 and not a first layer (three input channels),
+ * weights in the tap-major packed form of onhip_conv2d_pack_weights; b: 1x1, stride 1, no padding, over a's result, weights
+ * ([cout][cin]) re-laid once by onhip_conv2d_pw_pack_weights into the order the kernel's matrix instructions read them
+ * (onhip_conv2d_pw_packed_weight_bytes(b) bytes, 16-byte aligned); activations none, Relu or Clip.
+ * onhip_conv2d_pw_supported: 0 = not taken, 1 = taken, 2 = taken and expected to be faster than the two launches (at least
+ * 16384 output pixels over the batch).  addend (may be NULL): a tensor shaped like y, added after b's activation;
+ * relu_after != 0: relu.c's rule on the sum.  addend must not be y. */
+int onhip_conv2d_pw_supported(const onhip_conv_desc_t *a, const onhip_conv_desc_t *b);
+size_t onhip_conv2d_pw_packed_weight_bytes(const onhip_conv_desc_t *b);
+int onhip_conv2d_pw_pack_weights(const onhip_conv_desc_t *b, const float *wb, float *packed, void *stream);
+int onhip_conv2d_pw_f32(const onhip_conv_desc_t *a, const onhip_conv_desc_t *b, const float *x, const float *wa_packed,
+                        const float *bias_a, const float *wb_packed, const float *bias_b, const float *addend,
+                        int32_t relu_after, float *y, void *stream);
+
 /* Attention of every (batch, head) in one launch:  out = Softmax(q k^T * scale) v, Softmax over the keys.  Replaces the
  * operator chain MatMul (device/x86/MatMul/mat_mul.c:10-102) -> [Mul by a constant] -> Softmax (device/x86/Softmax/
  * softmax.c:26-59) -> MatMul of a transformer block, together with the Transposes (device/x86/Transpose/transpose.c)

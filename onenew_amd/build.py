@@ -19,7 +19,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-c++20-extensions",
              "-ffp-contract=off",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-KERNEL_SOURCES = ["depthwise.hip", "dw_s8.hip", "igemm_f32.hip", "igemm_f32_res.hip", "igemm_bf16.hip", "igemm_f16.hip", "igemm_i8.hip", "igemm_i8_res.hip", "igemm_rowb.hip", "igemm_dma.hip", "igemm_dma_bf16.hip", "igemm_dma_f16.hip", "igemm.hip", "direct.hip", "h16.hip", "attention.hip", "attention_h16.hip", "stem.hip", "irblock.hip", "i8patch.hip", "calib.hip", "elementwise.hip", "vit_glue.hip", "api.hip",
+KERNEL_SOURCES = ["depthwise.hip", "dw_s8.hip", "igemm_f32.hip", "igemm_f32_res.hip", "igemm_f32_pw.hip", "igemm_bf16.hip", "igemm_f16.hip", "igemm_i8.hip", "igemm_i8_res.hip", "igemm_rowb.hip", "igemm_dma.hip", "igemm_dma_bf16.hip", "igemm_dma_f16.hip", "igemm.hip", "direct.hip", "h16.hip", "attention.hip", "attention_h16.hip", "stem.hip", "irblock.hip", "i8patch.hip", "calib.hip", "elementwise.hip", "vit_glue.hip", "api.hip",
                   "plugin.hip"]
 PLUGINS = {"Conv": "plugin_conv.cpp", "MatMul": "plugin_matmul.cpp", "Gemm": "plugin_gemm.cpp",
            "Add": "plugin_add.cpp", "Relu": "plugin_relu.cpp", "MaxPool": "plugin_maxpool.cpp",

@@ -846,6 +846,102 @@ int onhip_conv2d_f32_noalloc(const onhip_conv_desc_t *d, const float *x, const f
     return rc;
 }
 
+// ---- a convolution and the 1x1 convolution after it in one launch ------------------------------------------------------------
+static bool act_none_relu_clip(int act) { return act == NOT_ACT || act == RELU6 || act == RELU || act == CLIP; }
+
+// what the pair must look like; *why names the first condition that fails
+static bool conv_pw_shapes_ok(const onhip_conv_desc_t *a, const onhip_conv_desc_t *b, int OH, int OW, const char **why) {
+    *why = nullptr;
+    if (a->compute != ONHIP_COMPUTE_F32 || b->compute != ONHIP_COMPUTE_F32) *why = "fp32 only";
+    else if (a->group != 1 || b->group != 1) *why = "dense convolutions only";
+    else if (!wants_packed(a) || stem_f32_shape(*a)) *why = "the first convolution must be one that takes tap-major packed weights";
+    else if (a->cout > 64) *why = "the first convolution must have at most 64 output channels";
+    else if (b->kh != 1 || b->kw != 1 || b->stride_h != 1 || b->stride_w != 1 || b->pad_t || b->pad_l || b->pad_b || b->pad_r)
+        *why = "the second convolution must be 1x1, stride 1, without padding";
+    else if (b->cin != a->cout || b->n != a->n || b->h != OH || b->w != OW) *why = "the second convolution does not read the first one's result";
+    else if (!act_none_relu_clip(a->act_type) || !act_none_relu_clip(b->act_type)) *why = "activations other than none, Relu and Clip";
+    else if (a->kh * a->kw > 64) *why = "filters of more than 64 taps";
+    else if ((long long) a->n * b->cout * OH * OW >= (1LL << 29) || (long long) a->n * a->cin * a->h * a->w >= (1LL << 29))
+        *why = "tensors of 2^29 elements or more";
+    return *why == nullptr;
+}
+
+int onhip_conv2d_pw_supported(const onhip_conv_desc_t *a, const onhip_conv_desc_t *b) {
+    int32_t OH, OW, OH2, OW2;
+    if (check_conv(a, &OH, &OW) || check_conv(b, &OH2, &OW2)) return 0;
+    const char *why;
+    if (!conv_pw_shapes_ok(a, b, OH, OW, &why)) return 0;
+    // expected to pay: the first result is wide in pixels and narrow in channels, so that writing and re-reading it
+    // and a launch of its own cost more than the occupancy its registers take from the first product
+    return (long long) a->n * OH * OW >= 16384 ? 2 : 1;
+}
+
+size_t onhip_conv2d_pw_packed_weight_bytes(const onhip_conv_desc_t *b) {
+    if (!b || b->cout < 1 || b->cin < 1 || b->cin > 64) return 0;
+    return (size_t) ((b->cout + 63) / 64) * 64 * 64 * sizeof(float);
+}
+
+int onhip_conv2d_pw_pack_weights(const onhip_conv_desc_t *b, const float *wb, float *packed, void *stream) {
+    if (!onhip_conv2d_pw_packed_weight_bytes(b)) return set_error(ONHIP_ERR_ARG, "conv + 1x1 pack: a 1x1 convolution over at most 64 channels");
+    if (!wb || !packed || reinterpret_cast<uintptr_t>(packed) % 16) return set_error(ONHIP_ERR_ARG, "conv + 1x1 pack: null or unaligned pointer");
+    return pack_pw2_launch(wb, b->cout, b->cin, packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+int onhip_conv2d_pw_f32(const onhip_conv_desc_t *a, const onhip_conv_desc_t *b, const float *x, const float *wa_packed,
+                        const float *bias_a, const float *wb_packed, const float *bias_b, const float *addend, int32_t relu_after,
+                        float *y, void *stream) {
+    int32_t OH, OW, OH2, OW2;
+    int rc = check_conv(a, &OH, &OW);
+    if (!rc) rc = check_conv(b, &OH2, &OW2);
+    if (rc) return rc;
+    const char *why;
+    if (!conv_pw_shapes_ok(a, b, OH, OW, &why)) return set_error(ONHIP_ERR_ARG, "conv + 1x1: %s", why);
+    if (!x || !wa_packed || !wb_packed || !y || (a->has_bias && !bias_a) || (b->has_bias && !bias_b))
+        return set_error(ONHIP_ERR_ARG, "conv + 1x1: null tensor pointer");
+    if (addend == y) return set_error(ONHIP_ERR_ARG, "conv + 1x1: the addend may not be the output buffer");
+    IgemmParams p;
+    memset(&p, 0, sizeof(p));
+    const int cp = packed_cp(a);
+    p.M = a->cout;
+    p.N = a->n * OH * OW;
+    p.H = a->h; p.W = a->w; p.OW = OW; p.OHW = OH * OW; p.HW = a->h * a->w;
+    p.kh = a->kh; p.kw = a->kw; p.khkw = a->kh * a->kw;
+    p.sh = a->stride_h; p.sw = a->stride_w; p.pt = a->pad_t; p.pl = a->pad_l;
+    p.magic_khkw = magic_for(p.khkw); p.pass_khkw = pass_for(p.khkw);
+    p.magic_kw = magic_for(p.kw); p.pass_kw = pass_for(p.kw);
+    p.use_tapmask = 1;
+    p.K = p.khkw * cp;
+    p.units_per_tap = cp / 4;
+    p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
+    p.k_units = p.K / 4;
+    p.A = wa_packed;
+    p.lda = p.K;
+    p.B = x;
+    p.b_img_stride = (long long) a->cin * a->h * a->w;
+    p.b_shift_bytes = ((long long) a->pad_t * a->w + a->pad_l) * 4;
+    p.a_slice_bytes = (long long) p.M * p.K * 4;
+    p.b_slice_bytes = (long long) a->n * p.b_img_stride * 4;
+    p.c_slice_bytes = (long long) a->n * b->cout * OH * OW * 4;
+    p.C = y;
+    p.out_mode = OUT_CONV;
+    p.c_img_stride = (long long) b->cout * OH * OW;
+    p.c_stride_m = (long long) OH * OW;
+    p.bias = bias_a;
+    p.bias_mode = a->has_bias ? BIAS_M : BIAS_NONE;
+    p.ep = make_epilogue(*a, nullptr);
+    p.w2 = wb_packed;
+    p.bias2 = b->has_bias ? bias_b : nullptr;
+    p.m2 = b->cout;
+    p.ep2 = make_epilogue(*b, nullptr);
+    if (addend) {
+        const long long n_out = (long long) a->n * b->cout * OH * OW;
+        p.res = addend;
+        p.res_relu = relu_after ? 1 : 0;
+        p.res_body = (unsigned) (n_out - n_out % 32);   // relu.c:27-52
+    }
+    return igemm_launch_f32_pw(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 static void w8a32_layout(const onhip_conv_desc_t *d, int *cp, int *k_units, size_t *packed_bytes, size_t *q_bytes) {
     *cp = (d->cin + 15) / 16 * 16;
     *k_units = d->kh * d->kw * (*cp / 16);

@@ -68,6 +68,29 @@ int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float 
     return ONHIP_OK;
 }
 
+// ---- fp32 1x1 weights [m2][cmid] (cmid <= 64) -> the A operand order of igemm_kernel's second product ---------------
+// [block of 64 rows][half of 32 rows][step s < 8][lane (lh, li)][4 floats]: lane (li, lh) of half wm holds columns
+// 4 (2 s + lh) .. + 3 of row block * 64 + wm * 32 + li; zeros beyond m2 rows and cmid columns
+__global__ __launch_bounds__(256) void pack_pw2_kernel(const float *w, int m2, int cmid, float4 *packed, long long total) {
+    const long long idx = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int lane = (int) (idx % 64), s = (int) ((idx / 64) % 8);
+    const int half = (int) (idx / 512);
+    const int row = half * 32 + lane % 32, col = 4 * (2 * s + lane / 32);
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (row < m2 && col + j < cmid) ? w[(long long) row * cmid + col + j] : 0.0f;
+    packed[idx] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+int pack_pw2_launch(const float *w, int m2, int cmid, float *packed, hipStream_t stream) {
+    const long long total = (long long) ((m2 + 63) / 64) * 2 * 8 * 64;
+    hipLaunchKernelGGL(pack_pw2_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, stream, w, m2, cmid,
+                       reinterpret_cast<float4 *>(packed), total);
+    ONHIP_CHECK_HIP(hipGetLastError());
+    return ONHIP_OK;
+}
+
 // ---- int8 weights [cout][cin][kh][kw] -> [cout][k_units * 16], k = (tap * cp + channel), zero padded ---
 __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t *w8, int cin, int khkw, int cp, int row_bytes,
                                                       int8_t *packed, long long total) {

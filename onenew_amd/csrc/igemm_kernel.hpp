@@ -805,9 +805,113 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
     }
 }
 
+// ---- a second, 1x1 product over the finished tile (the PW2 variant of the kernel, fp32, tile 64 x 64) ---------------------
+// The workgroup's tile holds every row of the first product (M <= 64) for its 64 columns, so it is the whole B operand
+// of a 1x1 convolution over that result for these columns: out[m2][64] = w2[m2][M] * act(tile + bias).  The tile goes to
+// LDS in the B layout of the K loop ([unit of 4 rows][column][16 B]; a lane's accumulator registers 4q .. 4q+3 are four
+// consecutive rows of one column, i.e. exactly one unit), every wavefront takes the 16 units of its 32 columns into
+// registers once, and then walks the rows of w2 in blocks of 64 (32 per wavefront) with its A operands loaded straight
+// from memory, where they lie in the MFMA's own layout (lane li = row, lanes 32-63 the odd unit of a step; w2 is packed
+// that way once): no LDS traffic and no barrier in this loop.  The reduction runs in the order of the K loop (unit pairs ascending, the four elements of a
+// unit one MFMA each), so the result has the bits of the two launches it replaces when those use this tile.
+// tl: LDS of at least 16 * 64 * 16 bytes that no wavefront reads any more (the caller has synchronised).
+template <int EPI, bool RES>
+__device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &acc1, uint4 *tl, int n0, int wm, int wn, int li, int lh) {
+    const unsigned lh16 = (unsigned) lh * 16u;
+    const int cmid = p.M;
+    // the first product's bias: rows 8 (r / 4) + 4 lh + r % 4 of the wavefront's 32
+    const rsrc_t rb1 = make_rsrc(p.bias, p.bias_mode == BIAS_M ? (unsigned) (cmid * 4) : 0u);
+    float b1[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) b1[r] = buf_load_f32(rb1, lh16, (unsigned) (wm * 32 + 8 * (r / 4) + (r % 4)) * 4u);
+    // A of the second product, re-laid once by pack_pw2_launch into the order this loop reads it: for every block of 64
+    // rows, half wm and step s the 64 lanes' 16 bytes side by side (lane (li, lh): row block * 64 + wm * 32 + li, unit
+    // 2 s + lh; zeros beyond m2 rows and M columns), so a load instruction is one contiguous KiB
+    const int mblocks = (p.m2 + 63) / 64;
+    const rsrc_t rw2 = make_rsrc(p.w2, (unsigned) (mblocks * 64 * 64 * 4));
+    const unsigned lane16 = (unsigned) (lh * 32 + li) * 16u;
+    uint4 wa[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) wa[s] = buf_load_b128(rw2, lane16, (unsigned) (wm * 8 + s) * 1024u);
+    const unsigned bias1_mask = p.bias_mode == BIAS_M ? 0xffffffffu : 0u;
+    // the first product's activation is none, Relu or Clip (the launcher refuses others): apply_act's comparisons as
+    // selects under two uniform flags, so that the sixteen values take no branch
+    const bool lo_on = p.ep.act == RELU || p.ep.act == CLIP, hi_on = p.ep.act == CLIP;
+    const float lo = p.ep.act == CLIP ? p.ep.clip_min : 0.0f, hi = p.ep.clip_max;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = 4 * q + j;
+            const float a = acc1[r];
+            // an absent bias must not touch the value (the sign of a zero sum): a select between bit patterns, which
+            // the compiler does not turn into a branch around the addition
+            const unsigned ab = __float_as_uint(a), sb = __float_as_uint(__fadd_rn(a, b1[r]));
+            float x = __uint_as_float(ab ^ ((ab ^ sb) & bias1_mask));
+            x = (lo_on & !(x > lo)) ? lo : x;
+            x = (hi_on & !(x < hi)) ? hi : x;
+            v[j] = wm * 32 + 8 * q + 4 * lh + j < cmid ? x : 0.0f;
+        }
+        tl[(wm * 8 + 2 * q + lh) * 64 + wn * 32 + li] = make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3]));
+    }
+    __syncthreads();
+    uint4 tb[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) tb[s] = tl[(2 * s + lh) * 64 + wn * 32 + li];
+
+    const rsrc_t rc = make_rsrc(p.C, RSRC_RANGE);
+    const rsrc_t rres = make_rsrc(RES ? p.res : nullptr, RES ? RSRC_RANGE : 0u);
+    const rsrc_t rb2 = make_rsrc(p.bias2, p.bias2 ? (unsigned) (p.m2 * 4) : 0u);
+    const bool bias2_on = p.bias2 != nullptr;
+    const unsigned row_bytes = (unsigned) p.c_stride_m * 4u;
+    const int n = n0 + wn * 32 + li;
+    const unsigned col_voff = n < p.N ? out_col_offset(p, n, 4) + (unsigned) (4 * lh) * row_bytes : OOB;
+    // One operand set: the 16 bytes of step s are requested again, for the next block of rows, as soon as the step's
+    // four MFMAs have been issued, so every load has most of a block's matrix work (and the stores) to arrive.  A block
+    // past the end loads nothing (its rows are beyond m2).
+    for (int mb = 0; mb < mblocks; ++mb) {
+        const int m_wave = mb * 64 + wm * 32;   // uniform
+        const bool m_edge = m_wave + 32 > p.m2;
+        float b2[16], rv[RES ? 16 : 1];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) b2[r] = buf_load_f32(rb2, lh16, (unsigned) (m_wave + 8 * (r / 4) + (r % 4)) * 4u);
+        if constexpr (RES) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m_uni = m_wave + 8 * (r / 4) + (r % 4);
+                rv[r] = buf_load_f32(rres, (!m_edge || m_uni + 4 * lh < p.m2) ? col_voff : OOB, (unsigned) m_uni * row_bytes);
+            }
+        }
+        f32x16 acc2;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc2[r] = 0.0f;
+        const unsigned next_voff = mb + 1 < mblocks ? lane16 : OOB;
+        const unsigned next_soff = (unsigned) (((mb + 1) * 2 + wm) * 8) * 1024u;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+#pragma unroll
+            for (int part = 0; part < 4; ++part) Traits<DT_F32>::mma_part(acc2, wa[s], tb[s], part);
+            wa[s] = buf_load_b128(rw2, next_voff, next_soff + 1024u * s);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m_uni = m_wave + 8 * (r / 4) + (r % 4);
+            const bool row_ok = !m_edge || m_uni + 4 * lh < p.m2;
+            float v = acc2[r];
+            v = bias2_on ? __fadd_rn(v, b2[r]) : v;
+            v = act_fast<EPI>(v, p.ep2);
+            if constexpr (RES) v = add_res(v, rv[r], p.res_relu, (col_voff + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff : OOB, (unsigned) m_uni * row_bytes, 0);
+        }
+    }
+}
+
 // ---- the kernel --------------------------------------------------------------------------------
-template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1, bool RES = false>
-__global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
+template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1, bool RES = false, bool PW2 = false>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (RES ? 3 : 4) : 1))) void igemm_kernel(const IgemmParams p) {
+    static_assert(!PW2 || (DT == DT_F32 && BM == 64 && BN == 64 && WM == 2 && WN == 2), "the second product exists for fp32 tiles of 64 x 64");
     static_assert(!RES || DT == DT_F32 || DT == DT_I8, "the residual store exists for fp32 and int8 operands (fp32 results)");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -1107,6 +1211,20 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(const IgemmParams p) {
     for (; kt + U <= k_tiles; kt += U) group(kt, CHECKED, std::false_type{});
     if (kt < k_tiles) group(kt, CHECKED, std::true_type{});
 
+    if constexpr (PW2) {
+        // the launcher gives this variant one row tile, all of K and no batch: the tile is the whole first product
+        static_assert(sizeof(lds) >= 16 * 64 * 16, "the tile as a B operand fits the operand buffers");
+        __syncthreads();   // every wavefront is done with the operand buffers
+        uint4 *tl = &lds[0][0];
+        switch (p.ep2.act) {
+            case NOT_ACT:
+            case RELU6: pw2_stage<EPI_NONE, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
+            case RELU: pw2_stage<EPI_RELU, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
+            case CLIP: pw2_stage<EPI_CLIP, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
+            default: pw2_stage<EPI_GENERIC, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
+        }
+        return;
+    }
     const int m_wave = m0 + wm * (BM / WM), n_wave = n0 + wn * (BN / WN);
     if (p.partial && !whole_k) {
         if (DT == DT_I8 || !p.arrive) {   // a finishing launch adds the slices up

@@ -223,6 +223,14 @@ struct IgemmParams {
     // fit an L2 while B (a weight matrix) does: each XCD then reads its rows of A once instead of all of A per column block.
     int n_fast;
     Div31 div_tiles_n;
+    // a second, 1x1 product over the finished tile (igemm_kernel's PW2 variant, one row tile: M <= 64): the M rows of the
+    // first product, with `bias` and `ep` applied, are the reduction of w2 ([m2][M], in pack_pw2_launch's order).  C, the
+    // c_* strides and res then describe the m2-row result, bias2 and ep2 its epilogue; the M-row tensor between the two
+    // never exists
+    const float *w2;
+    const float *bias2;
+    int m2;
+    Epilogue ep2;
 };
 
 enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2, DT_I8 = 3 };
@@ -237,6 +245,9 @@ struct IgemmLaunch {
 };
 
 int igemm_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
+// fp32 convolution followed by a 1x1 convolution over its result in one launch (igemm_f32_pw.hip): p as for the tap-major
+// packed loader with M <= 64 rows, plus w2 / bias2 / m2 / ep2
+int igemm_launch_f32_pw(const IgemmParams &p, hipStream_t stream);
 // fp32 kernel for plain problems with B rows contiguous along N (igemm_rowb.hip): tiles 64x128, 128x128, 64x256
 bool rowb_f32_ok(const IgemmLaunch &cfg, const IgemmParams &p);
 int rowb_f32_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStream_t stream);
@@ -259,6 +270,7 @@ int dw_s8_launch(const onhip_conv_desc_t &d, int OH, int OW, const int8_t *xq, c
 int quantize_nhwc_launch(const float *x, int n, int c, int h, int w, int cp, float inv_scale, int8_t *q,
                          hipStream_t stream);
 int pack_wf32_launch(const float *w, int cout, int cin, int khkw, int cp, float *packed, hipStream_t stream);
+int pack_pw2_launch(const float *w, int m2, int cmid, float *packed, hipStream_t stream);   // ceil(m2 / 64) * 16 KiB
 int build_qlut_launch(const float *lut, float out_inv_scale, signed char *qlut, hipStream_t stream);
 int forget_quantised_tables(const void *base, size_t bytes);   // api.hip: the cache of tables behind an output quantiser
 // i8patch.hip: int8 NHWC 3x3 convolutions with few channels from an LDS-resident input patch

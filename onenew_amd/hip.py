@@ -41,6 +41,7 @@ EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_ta
            "onhip_h16_from_nchw_f32", "onhip_h16_to_nchw_f32", "onhip_h16_from_rows_f32", "onhip_h16_to_rows_f32",
            "onhip_conv2d_h16", "onhip_h16_first_width", "onhip_h16_first_channels", "onhip_h16_first_input_bytes", "onhip_h16_first_weight_bytes", "onhip_h16_first_from_nchw_f32", "onhip_h16_first_pack_weights", "onhip_conv2d_h16_first", "onhip_linear_h16", "onhip_attention", 
            "onhip_ir_block_supported", "onhip_ir_block_packed_weight_bytes", "onhip_ir_block_pack_weights", "onhip_ir_block_f32",
+           "onhip_conv2d_pw_supported", "onhip_conv2d_pw_packed_weight_bytes", "onhip_conv2d_pw_pack_weights", "onhip_conv2d_pw_f32",
            "onhip_add_f32", "onhip_relu_f32", "onhip_maxpool_out_shape", "onhip_maxpool_f32", "onhip_maxpool_s8_nhwc", "onhip_maxpool_s8_eval", "onhip_global_avgpool_f32",
            "onhip_gelu_lut_f32", "onhip_layernorm_f32", "onhip_softmax_f32", "onhip_transpose_f32",
            "onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval", "onhip_add_eval", "onhip_relu_eval",
@@ -129,6 +130,11 @@ def load():
     L.onhip_ir_block_packed_weight_bytes.restype = C.c_size_t
     L.onhip_ir_block_pack_weights.argtypes = [vp, vp, i32, i32, i32, vp, vp]
     L.onhip_ir_block_f32.argtypes = [C.POINTER(ConvDesc)] * 3 + [vp] * 9
+    L.onhip_conv2d_pw_supported.argtypes = [C.POINTER(ConvDesc)] * 2
+    L.onhip_conv2d_pw_packed_weight_bytes.argtypes = [C.POINTER(ConvDesc)]
+    L.onhip_conv2d_pw_packed_weight_bytes.restype = C.c_size_t
+    L.onhip_conv2d_pw_pack_weights.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    L.onhip_conv2d_pw_f32.argtypes = [C.POINTER(ConvDesc)] * 2 + [vp] * 6 + [i32, vp, vp]
     L.onhip_linear_h16.argtypes = [C.c_longlong, i32, i32, i32, vp, vp, vp, vp, vp, vp, i32, vp]
     for name in ("onhip_conv_eval", "onhip_matmul_eval", "onhip_matmul_attention_eval", "onhip_matmul_bias_eval", "onhip_matmul_bias_gelu_eval", "onhip_matmul_bias_add_eval", "onhip_gemm_eval"):
         getattr(L, name).argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
@@ -630,6 +636,31 @@ def ir_block_f32(ex, dw, pw, x, packed, expand_b, dw_w, dw_b, project_b=None, re
         out = torch.empty((dw.n, pw.cout, oh, ow), dtype=torch.float32, device=x.device)
     _check(load().onhip_ir_block_f32(C.byref(ex), C.byref(dw), C.byref(pw), _ptr(x), _ptr(packed), _ptr(expand_b), _ptr(dw_w), _ptr(dw_b),
                                      _ptr(project_b), _ptr(residual), _ptr(out), _stream()), "onhip_ir_block_f32")
+    return out
+
+
+def conv2d_pw_supported(a, b):
+    """0: the pair is not taken; 1: taken; 2: taken and expected to beat the two launches"""
+    return load().onhip_conv2d_pw_supported(C.byref(a), C.byref(b))
+
+
+def conv2d_pw_pack_weights(b, wb):
+    """the 1x1 convolution's weights in the order conv2d_pw_f32 reads them"""
+    import torch
+    out = torch.empty(load().onhip_conv2d_pw_packed_weight_bytes(C.byref(b)) // 4, dtype=torch.float32, device=wb.device)
+    _check(load().onhip_conv2d_pw_pack_weights(C.byref(b), _ptr(wb), _ptr(out), _stream()), "onhip_conv2d_pw_pack_weights")
+    return out
+
+
+def conv2d_pw_f32(a, b, x, wa_packed, bias_a, wb_packed, bias_b, addend=None, relu_after=False, out=None):
+    """convolution a (packed weights) and the 1x1 convolution b over its result (weights from conv2d_pw_pack_weights)
+    [-> Add of addend -> Relu] in one launch"""
+    import torch
+    oh, ow = a.out_hw()
+    if out is None:
+        out = torch.empty((a.n, b.cout, oh, ow), dtype=torch.float32, device=x.device)
+    _check(load().onhip_conv2d_pw_f32(C.byref(a), C.byref(b), _ptr(x), _ptr(wa_packed), _ptr(bias_a), _ptr(wb_packed), _ptr(bias_b),
+                                      _ptr(addend), 1 if relu_after else 0, _ptr(out), _stream()), "onhip_conv2d_pw_f32")
     return out
 
 

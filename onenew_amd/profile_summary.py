@@ -33,9 +33,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SIMDS = 256 * 4            # MI355X: 256 compute units of 4 SIMDs
 CLOCK_HZ = 2.4e9           # peak engine clock the MFMA peak is quoted at
 GLUE = ("add_kernel", "relu_kernel", "maxpool", "gap_kernel", "layernorm", "softmax", "transpose_kernel", "gelu_lut")
-LEGEND = ("Kernel names: `onhip::igemm_kernel<dtype, loader, BM, BN, WM, WN, PF, RES>` (dtype 0 fp32, 1 bf16, 2 f16, 3 int8; loader 0 "
+LEGEND = ("Kernel names: `onhip::igemm_kernel<dtype, loader, BM, BN, WM, WN, PF, RES, PW2>` (dtype 0 fp32, 1 bf16, 2 f16, 3 int8; loader 0 "
           "gather, 1 int8 vectors, 2 plain, 3 tap-major packed, 4 int8 vectors with scalar taps; PF register sets of tiles in flight; "
-          "RES the variant whose store adds a residual operand), `onhip::igemm_dma_kernel<dtype, BM, BN, WM, WN, KS, NST>` (int8 and "
+          "RES the variant whose store adds a residual operand; PW2 the variant that multiplies its finished tile by a second, 1x1 weight "
+          "matrix before storing: a convolution and the 1x1 convolution after it in one launch), `onhip::igemm_dma_kernel<dtype, BM, BN, WM, WN, KS, NST>` (int8 and "
           "16-bit storage: operand tiles loaded straight into LDS, KS bytes of K per stage, ring of NST stages), `onhip::rowb_f32_kernel<WM, WN>` (fp32, B "
           "straight from memory, tile 32 WM x 128 WN), `onhip::splitk_finish_kernel`, `onhip::depthwise_tiled_kernel<int8, stride, "
           "act>`, `onhip::quantize_nhwc_kernel<CBW>`, `onhip::stem_f32_kernel<filter size, act, two row tiles>` (first-layer "
