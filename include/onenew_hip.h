@@ -485,6 +485,15 @@ int onhip_conv_add_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFE
  * the last convolution.  onhip_conv_block_takes reads the params only and returns 1 when onhip_ir_block_supported says 2
  * for these shapes, else 0.  No counterpart in the reference, whose host runs the operators one by one. */
 int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+/* `eval_pair` / `eval_pair_relu` / `eval_pair_takes` of libConv_hip.so: Conv (dense, at most 64 output channels, not a plain
+ * 1x1) -> Conv (1x1) [-> Add [-> Relu]] in one call (onhip_conv2d_pw_f32).  Slots as for the first convolution's `eval`, the
+ * pair's result operand in params[4] and outputs[0]; inputs[3] = the addend or null; params[5], params[6], inputs[5],
+ * inputs[6] = the second convolution's CONV_CONFIG_S, weight operand, weights and bias.  onhip_conv_pair_relu_eval applies
+ * relu.c's rule to the sum (an addend is required); onhip_conv_pair_takes reads the params only and returns 1 when
+ * onhip_conv2d_pw_supported says 2 for these shapes, else 0.  No counterpart in the reference. */
+int onhip_conv_pair_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_conv_pair_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
+int onhip_conv_pair_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs);
 /* `eval_link` of libConv_hip.so: an int8 (W8A32) Conv, dense or depthwise, whose input and/or result travel as int8 NHWC (channels padded
  * to 16) instead of fp32 NCHW, see onhip_conv2d_w8_link.  Slots as for `eval`; inputs[4] = host pointer to
  * {int32 in_s8, int32 out_s8, float out_scale, int32 twin} (twin != 0: outputs[1] = device buffer for the int8 copy of an

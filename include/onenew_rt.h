@@ -105,6 +105,16 @@ int onrt_net_folded_activations(const onrt_net_t *net, int32_t *n);
 int onrt_net_fused_ir_blocks(const onrt_net_t *net, int32_t *n);
 
 /*
+ * Convolution pairs: Conv (dense, at most 64 output channels, not a plain 1x1) -> Conv (1x1) [-> Add [-> Relu], folded into
+ * the second convolution], the first result read by the second alone, run as one call of the Conv plugin's `eval_pair` /
+ * `eval_pair_relu` (libConv_hip.so; the tensor in between is not written) where its `eval_pair_takes` recommends that for
+ * the shapes: the 3x3 and the last convolution of ResNet-50's first-stage bottlenecks at large batch.  The reference's host
+ * runs the operators one after the other (host/net.h:613-618).  The operand folded away has no buffer.  ONENEW_RT_FUSE=0
+ * keeps the operators separate, ONENEW_RT_FUSE_PAIRS=0 these pairs alone.  n: how many pairs.
+ */
+int onrt_net_fused_pairs(const onrt_net_t *net, int32_t *n);
+
+/*
  * int8 edges: the result of a dense int8 (W8A32) Conv that only dense int8 Convs with one and the same input_scale read
  * travels as int8 NHWC, quantised in the producer's store exactly as each consumer would have quantised the fp32 tensor
  * (device/x86/Conv/conv.c:961-973), through the Conv plugin's `eval_link`: a quarter of the bytes, no staging pass in the

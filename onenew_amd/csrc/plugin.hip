@@ -156,6 +156,21 @@ static int packed_block_weights(const float *ex_w, const float *pw_w, int cin, i
     return ONHIP_OK;
 }
 
+// the 1x1 convolution of a fused pair: its weights in the order onhip_conv2d_pw_f32 reads them, next to their device copy
+static int packed_pair_weights(const onhip_conv_desc_t *b, const float *w_dev, const float **out) {
+    const size_t bytes = onhip_conv2d_pw_packed_weight_bytes(b);
+    auto it = g_packed.find(w_dev);
+    if (it != g_packed.end() && it->second.bytes == bytes && it->second.other == w_dev) { *out = it->second.dev; return ONHIP_OK; }
+    drop_packed(w_dev);
+    float *p = nullptr;
+    ONHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&p), bytes));
+    const int rc = onhip_conv2d_pw_pack_weights(b, w_dev, p, g_stream);
+    if (rc) { (void) hipFree(p); return rc; }
+    g_packed[w_dev] = PackedEntry{p, bytes, false, w_dev};
+    *out = p;
+    return ONHIP_OK;
+}
+
 static int ensure_ready() {
     if (g_ready) return ONHIP_OK;
     int dev = 0;
@@ -486,6 +501,74 @@ static int conv_block_eval_mode(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BU
                             (const float *) pw_b, (const float *) addend, (float *) y, g_stream);
     if (rc) return rc;
     return out_on_dev ? wait_for_output() : copy_out(host_out, y, out_bytes);
+}
+
+// Conv (dense, at most 64 output channels, not a plain 1x1) -> Conv (1x1) [-> Add [-> Relu]] as one call of
+// onhip_conv2d_pw_f32.  Slots: params[0..4] / inputs[0..2] as for the first convolution's `eval`, params[4] the pair's result
+// operand; inputs[3] the addend or null; params[5] the second convolution's CONV_CONFIG_S, params[6] its weight operand,
+// inputs[5] / inputs[6] its weights and bias (null without).  relu: relu.c's rule on the sum (with an addend only).
+// query: no tensor is touched; 1 when the library recommends the one-launch kernel for these shapes, else 0.
+static int conv_pair_eval_mode(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs, bool query, bool relu) {
+    const CONV_CONFIG_S *cfg[2] = {reinterpret_cast<const CONV_CONFIG_S *>(params[0].addr), reinterpret_cast<const CONV_CONFIG_S *>(params[5].addr)};
+    const OPERAND_S *in_t = reinterpret_cast<const OPERAND_S *>(params[1].addr);
+    const OPERAND_S *w_t[2] = {reinterpret_cast<const OPERAND_S *>(params[2].addr), reinterpret_cast<const OPERAND_S *>(params[6].addr)};
+    const OPERAND_S *out_t = reinterpret_cast<const OPERAND_S *>(params[4].addr);
+    if (!cfg[0] || !cfg[1] || !in_t || !w_t[0] || !w_t[1] || !out_t) {
+        if (query) return 0;
+        return set_error(ONHIP_ERR_ARG, "Conv pair eval: empty params slot");
+    }
+    if (cfg[0]->ifmap_quant2 == TYPE_INT8 || cfg[1]->ifmap_quant2 == TYPE_INT8) {
+        if (query) return 0;
+        return set_error(ONHIP_ERR_ARG, "Conv pair eval: fp32 convolutions only");
+    }
+    onhip_conv_desc_t d[2];
+    int n = out_t->shapes[0] < in_t->shapes[0] ? out_t->shapes[0] : in_t->shapes[0];
+    n = n < 1 ? 1 : n;
+    int32_t oh = 0, ow = 0, h2 = 0, w2 = 0;
+    block_conv_desc(&d[0], cfg[0], n, in_t->shapes[1], in_t->shapes[2], in_t->shapes[3], w_t[0]);
+    bool ok = cfg[0]->group == 1 && cfg[1]->group == 1 && w_t[0]->shapes[1] == in_t->shapes[1] && onhip_conv_out_shape(&d[0], &h2, &w2) == ONHIP_OK;
+    if (ok) {
+        block_conv_desc(&d[1], cfg[1], n, d[0].cout, h2, w2, w_t[1]);
+        ok = w_t[1]->shapes[1] == d[0].cout && onhip_conv_out_shape(&d[1], &oh, &ow) == ONHIP_OK && out_t->shapes[1] == d[1].cout &&
+             out_t->shapes[2] == oh && out_t->shapes[3] == ow;
+    }
+    if (query) return ok && onhip_conv2d_pw_supported(&d[0], &d[1]) >= 2 ? 1 : 0;
+    if (!ok) return set_error(ONHIP_ERR_ARG, "Conv pair eval: the two convolutions and the result operand do not fit together");
+    if (!onhip_conv2d_pw_supported(&d[0], &d[1])) return set_error(ONHIP_ERR_ARG, "Conv pair eval: not a pair the one-launch kernel takes");
+    const size_t in_bytes = (size_t) n * d[0].cin * d[0].h * d[0].w * 4, out_bytes = (size_t) n * d[1].cout * oh * ow * 4;
+    const void *x, *wa, *ba = nullptr, *wb, *bb = nullptr, *addend = nullptr;
+    int rc = input_on_device(0, reinterpret_cast<const void *>(inputs[0].addr), in_bytes, &x);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[1].addr), (size_t) d[0].cout * d[0].cin * d[0].kh * d[0].kw * 4, &wa);
+    if (!rc && d[0].has_bias) rc = const_on_device(reinterpret_cast<const void *>(inputs[2].addr), (size_t) d[0].cout * 4, &ba);
+    if (!rc) rc = const_on_device(reinterpret_cast<const void *>(inputs[5].addr), (size_t) d[1].cout * d[1].cin * 4, &wb);
+    if (!rc && d[1].has_bias) rc = const_on_device(reinterpret_cast<const void *>(inputs[6].addr), (size_t) d[1].cout * 4, &bb);
+    if (!rc && inputs[3].addr) rc = input_on_device(5, reinterpret_cast<const void *>(inputs[3].addr), out_bytes, &addend);
+    if (rc) return rc;
+    if (!wa || !wb || (d[0].has_bias && !ba) || (d[1].has_bias && !bb)) return set_error(ONHIP_ERR_ARG, "Conv pair eval: empty weight or bias slot");
+    if (relu && !addend) return set_error(ONHIP_ERR_ARG, "Conv pair eval: a Relu after the Add needs the addend in inputs[3]");
+    void *host_out = reinterpret_cast<void *>(outputs[0].addr);
+    void *y = host_out;
+    const bool out_on_dev = is_device_ptr(host_out);
+    if (!out_on_dev) {
+        rc = stage_buf(2, out_bytes, &y);
+        if (rc) return rc;
+    }
+    const float *wa_packed = nullptr, *wb_packed = nullptr;
+    rc = packed_weights(&d[0], (const float *) wa, &wa_packed);
+    if (!rc && !wa_packed) rc = set_error(ONHIP_ERR_ARG, "Conv pair eval: the first convolution has no packed weight form");
+    if (!rc) rc = packed_pair_weights(&d[1], (const float *) wb, &wb_packed);
+    if (rc) return rc;
+    rc = onhip_conv2d_pw_f32(&d[0], &d[1], (const float *) x, wa_packed, (const float *) ba, wb_packed, (const float *) bb,
+                             (const float *) addend, relu ? 1 : 0, (float *) y, g_stream);
+    if (rc) return rc;
+    return out_on_dev ? wait_for_output() : copy_out(host_out, y, out_bytes);
+}
+
+static int conv_pair_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return conv_pair_eval_mode(params, inputs, outputs, false, false);
+}
+static int conv_pair_relu_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return conv_pair_eval_mode(params, inputs, outputs, false, true);
 }
 
 static int conv_block_eval_locked(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
@@ -1007,6 +1090,17 @@ int onhip_conv_block_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_I
 int onhip_conv_block_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
     if (!params) return 0;
     return conv_block_eval_mode(params, inputs, outputs, true);
+}
+
+int onhip_conv_pair_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv -> 1x1 Conv", conv_pair_eval_locked, params, inputs, outputs);
+}
+int onhip_conv_pair_relu_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    return guarded("Conv -> 1x1 Conv -> Add -> Relu", conv_pair_relu_eval_locked, params, inputs, outputs);
+}
+int onhip_conv_pair_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {
+    if (!params) return 0;
+    return conv_pair_eval_mode(params, inputs, outputs, true, false);
 }
 
 int onhip_matmul_eval(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs, BUFFER_INFO_S *outputs) {

@@ -29,6 +29,24 @@ extern "C" __attribute__((visibility("default"))) int eval_block_takes(BUFFER_IN
     return onhip_conv_block_takes(params, inputs, outputs);
 }
 
+// Not in the reference: a dense convolution with at most 64 output channels and the 1x1 convolution over its result
+// [-> Add [-> Relu]] as one call.  Slots as for the first convolution's `eval` with the pair's result operand in params[4]
+// and outputs[0]; inputs[3] = the addend or null; params[5], params[6], inputs[5], inputs[6] = the second convolution's
+// CONV_CONFIG_S, weight operand, weights and bias.  eval_pair_relu: with the Relu after the Add.  eval_pair_takes: same
+// params, no tensors touched; 1 when the library recommends the call for these shapes, else 0.
+extern "C" __attribute__((visibility("default"))) int eval_pair(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                BUFFER_INFO_S *outputs) {
+    return onhip_conv_pair_eval(params, inputs, outputs);
+}
+extern "C" __attribute__((visibility("default"))) int eval_pair_relu(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                     BUFFER_INFO_S *outputs) {
+    return onhip_conv_pair_relu_eval(params, inputs, outputs);
+}
+extern "C" __attribute__((visibility("default"))) int eval_pair_takes(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
+                                                                      BUFFER_INFO_S *outputs) {
+    return onhip_conv_pair_takes(params, inputs, outputs);
+}
+
 extern "C" __attribute__((visibility("default"))) int eval_add_relu(BUFFER_INFO_S *params, BUFFER_INFO_S *inputs,
                                                                     BUFFER_INFO_S *outputs) {
     return onhip_conv_add_relu_eval(params, inputs, outputs);

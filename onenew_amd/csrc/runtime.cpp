@@ -132,7 +132,8 @@ struct Node {
     int fuse = 0;            // Conv: 1 = the Add after it is folded in, 2 = and the Relu after that
     std::string addend, fused_out;
     int32_t token_major[4] = {0, 0, 0, 0};   // fused attention: q, k, v, result stored [batch, tokens, heads, head_dim]
-    int block_dw = -1, block_pw = -1;        // fused inverted-residual block (fuse 7): its depthwise and last convolutions
+    int block_dw = -1, block_pw = -1;        // fused inverted-residual block (fuse 7): its depthwise and last convolutions;
+                                             // fused pair (fuse 8): block_pw is its 1x1 convolution
     // an int8 convolution whose input and/or result travel as int8 NHWC (link_int8_convs): what `eval_link` reads from
     // inputs[4] ({in_s8, out_s8, out_scale}) and inputs[5] (the fold code, when an Add is folded in)
     struct { int32_t in_s8, out_s8; float out_scale; int32_t twin; } link = {0, 0, 0.0f, 0};
@@ -173,9 +174,10 @@ struct onrt_net {
     size_t init_bytes = 0;
     onenew_eval_fn conv_add = nullptr, conv_add_relu = nullptr;   // optional entry points of the Conv plugin
     onenew_eval_fn conv_block = nullptr, conv_block_takes = nullptr, conv_link = nullptr, conv_link_takes = nullptr;
+    onenew_eval_fn conv_pair = nullptr, conv_pair_relu = nullptr, conv_pair_takes = nullptr;
     onenew_eval_fn maxpool_s8 = nullptr;   // optional entry point of the MaxPool plugin
     onenew_eval_fn matmul_attention = nullptr, matmul_bias = nullptr, matmul_bias_gelu = nullptr, matmul_bias_add = nullptr;   // optional entry points of the MatMul plugin
-    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0, int8_links = 0;
+    int fused_blocks = 0, folded_relus = 0, folded_acts = 0, fused_attentions = 0, fused_linears = 0, fused_skips = 0, fused_ir_blocks = 0, fused_pairs = 0, int8_links = 0;
     void *init_arena = nullptr, *act_arena = nullptr, *tables = nullptr;
     std::vector<float> silu_lut, gelu_lut;
 };
@@ -539,6 +541,9 @@ int bind_plugins(onrt_net &net) {
             net.conv_add_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_add_relu"));
             net.conv_block = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block"));
             net.conv_block_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_block_takes"));
+            net.conv_pair = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_pair"));
+            net.conv_pair_relu = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_pair_relu"));
+            net.conv_pair_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_pair_takes"));
             net.conv_link = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_link"));
             net.conv_link_takes = reinterpret_cast<onenew_eval_fn>(dlsym(it->second, "eval_link_takes"));
         }
@@ -799,6 +804,75 @@ int fuse_ir_blocks(onrt_net &net) {
         dropped[idx] = dropped[bi] = true;
         runs_instead[ci] = idx;
         ++net.fused_ir_blocks;
+    }
+    std::vector<int> order;
+    for (int idx : net.order) {
+        auto it = runs_instead.find(idx);
+        if (it != runs_instead.end()) order.push_back(it->second);
+        else if (!dropped[idx]) order.push_back(idx);
+    }
+    net.order.swap(order);
+    return ONRT_OK;
+}
+
+// ---- a convolution and the 1x1 convolution after it ---------------------------------------------------------
+// Conv -> Conv (1x1) [-> Add [-> Relu], already folded into the second convolution], the first result read by the second
+// alone, becomes one call of the Conv plugin's `eval_pair` (`eval_pair_relu`) where the plugin's `eval_pair_takes`
+// recommends it for the shapes (the 3x3 and the last convolution of ResNet-50's 64-channel bottlenecks at a batch that
+// fills the chip): the tensor in between is not written.  The call takes the place of the second convolution in the
+// order.  Runs after the residual and the inverted-residual folds, whose convolutions it leaves alone as first ones;
+// ONENEW_RT_FUSE=0 keeps every operator separate, ONENEW_RT_FUSE_PAIRS=0 these pairs alone.
+void pair_slots(onrt_net &net, Node &a, const Node &b, const Tensor &result) {
+    a.params[0].addr = (int64_t) a.cfg.data();
+    a.params[1].addr = (int64_t) &net.tensors[a.in[0]].desc;
+    a.params[2].addr = (int64_t) &net.tensors[a.in[1]].desc;
+    a.params[3].addr = (int64_t) &net.tensors[a.in[2]].desc;
+    a.params[4].addr = (int64_t) &result.desc;
+    a.params[5].addr = (int64_t) b.cfg.data();
+    a.params[6].addr = (int64_t) &net.tensors[b.in[1]].desc;
+}
+
+int fuse_conv_pairs(onrt_net &net) {
+    if (!fusing_enabled() || !net.conv_pair || !net.conv_pair_relu || !net.conv_pair_takes) return ONRT_OK;
+    if (const char *env = getenv("ONENEW_RT_FUSE_PAIRS"))   // "0": this fold alone switched off
+        if (!strcmp(env, "0")) return ONRT_OK;
+    auto result_of = [](const Node &n) { return n.fused_out.empty() ? n.out[0] : n.fused_out; };
+    auto plain_conv = [&](const Node &n, size_t min_in) {
+        if (strcmp(n.kind->type, "Conv") || n.out.size() != 1 || n.in.size() < min_in || n.in.size() > 3) return false;
+        for (size_t k = 1; k < n.in.size(); ++k)
+            if (n.in[k].empty() || !net.tensors[n.in[k]].is_init) return false;
+        return !net.tensors[n.in[0]].is_init;
+    };
+    std::map<int, int> runs_instead;   // second convolution -> the first one, which takes its place
+    std::vector<bool> dropped(net.nodes.size(), false);
+    for (int idx : net.order) {
+        Node &a = net.nodes[idx];
+        if (a.fuse || dropped[idx] || runs_instead.count(idx) || !plain_conv(a, 3)) continue;
+        const int bi = sole_reader(net, result_of(a), "Conv");
+        if (bi < 0 || dropped[bi] || runs_instead.count(bi)) continue;
+        Node &b = net.nodes[bi];
+        if (b.fuse > 2 || !plain_conv(b, 2) || b.in[0] != result_of(a)) continue;
+        // the other operand of a folded Add must not be the tensor that disappears
+        if (b.fuse && (b.addend == a.out[0] || b.addend == result_of(a))) continue;
+        const Tensor &result = net.tensors[result_of(b)];
+        for (BUFFER_INFO_S &s : a.params) s.addr = 0;
+        pair_slots(net, a, b, result);
+        const bool takes = net.conv_pair_takes(a.params, a.inputs, a.outputs) == 1;
+        for (BUFFER_INFO_S &s : a.params) s.addr = 0;
+        if (!takes) continue;
+        for (const std::string &gone : {a.out[0], result_of(a)}) {
+            net.tensors[gone].never_written = true;
+            net.tensors[gone].alias.clear();
+        }
+        a.fuse = 8;
+        a.block_pw = bi;
+        a.addend = b.fuse ? b.addend : std::string();
+        a.fused_out = result_of(b);
+        if (b.out[0] != a.fused_out) net.tensors[b.out[0]].alias = a.fused_out;
+        a.eval = b.fuse == 2 ? net.conv_pair_relu : net.conv_pair;
+        dropped[idx] = true;
+        runs_instead[bi] = idx;
+        ++net.fused_pairs;
     }
     std::vector<int> order;
     for (int idx : net.order) {
@@ -1155,6 +1229,13 @@ int fill_slots(onrt_net &net) {
             nd.inputs[7].addr = (int64_t) net.tensors[c.in[1]].dev;
             nd.inputs[8].addr = c.in.size() > 2 ? (int64_t) net.tensors[c.in[2]].dev : 0;
         }
+        if (nd.fuse == 8) {
+            const Node &b = net.nodes[nd.block_pw];
+            pair_slots(net, nd, b, net.tensors[nd.fused_out]);
+            nd.inputs[3].addr = nd.addend.empty() ? 0 : (int64_t) net.tensors[nd.addend].dev;
+            nd.inputs[5].addr = (int64_t) net.tensors[b.in[1]].dev;
+            nd.inputs[6].addr = b.in.size() > 2 ? (int64_t) net.tensors[b.in[2]].dev : 0;
+        }
         if (nd.fuse == 1 || nd.fuse == 2 || nd.fuse == 6) nd.inputs[3].addr = (int64_t) net.tensors[nd.addend].dev;
         // the other operand of a folded Add must be a tensor some operator writes (or an input): one that a later fold
         // took the buffer away from would be added as zeros, silently
@@ -1197,6 +1278,7 @@ int prepare(onrt_net &net, const char *op_lib_dir) {
     if (!rc) rc = fold_activations_into_conv(net);
     if (!rc) rc = fuse_residual_blocks(net);
     if (!rc) rc = fuse_ir_blocks(net);
+    if (!rc) rc = fuse_conv_pairs(net);
     if (!rc) rc = fuse_attention(net);
     if (!rc) rc = fuse_linear(net);
     if (!rc) rc = link_int8_convs(net);
@@ -1451,6 +1533,12 @@ ONRT_API int onrt_net_quantised_links(const onrt_net_t *net, int32_t *n) {
 ONRT_API int onrt_net_fused_ir_blocks(const onrt_net_t *net, int32_t *n) {
     if (!net || !n) return fail(ONRT_ERR_ARG, "fused inverted-residual blocks: null argument");
     *n = (int32_t) net->fused_ir_blocks;
+    return ONRT_OK;
+}
+
+ONRT_API int onrt_net_fused_pairs(const onrt_net_t *net, int32_t *n) {
+    if (!net || !n) return fail(ONRT_ERR_ARG, "fused convolution pairs: null argument");
+    *n = (int32_t) net->fused_pairs;
     return ONRT_OK;
 }
 

@@ -31,7 +31,7 @@ def plugin_path(op):
 
 EXPORTS = ["onhip_init", "onhip_last_error", "onhip_set_tuning", "onhip_split_tail_launches", "onhip_direct_lds_launches", "onhip_noalloc_scratch_launches", "onhip_last_launch_choice", "onhip_scratch_bytes", "onhip_set_tile_hint", "onhip_tile_candidate", "onhip_conv_out_shape", "onhip_conv2d_f32",
            "onhip_conv2d_packed_weight_bytes", "onhip_conv2d_pack_weights", "onhip_conv2d_f32_packed",
-           "onhip_conv2d_f32_add", "onhip_conv2d_f32_noalloc", "onhip_conv_add_eval", "onhip_conv_add_relu_eval", "onhip_conv_block_eval", "onhip_conv_block_takes", "onhip_conv_link_eval", "onhip_conv_link_takes", "onhip_conv2d_w8_link", "onhip_conv2d_w8a8_depthwise_supported",
+           "onhip_conv2d_f32_add", "onhip_conv2d_f32_noalloc", "onhip_conv_add_eval", "onhip_conv_add_relu_eval", "onhip_conv_block_eval", "onhip_conv_block_takes", "onhip_conv_pair_eval", "onhip_conv_pair_relu_eval", "onhip_conv_pair_takes", "onhip_conv_link_eval", "onhip_conv_link_takes", "onhip_conv2d_w8_link", "onhip_conv2d_w8a8_depthwise_supported",
            "onhip_conv2d_w8a32_workspace", "onhip_conv2d_w8a32", "onhip_conv2d_w8a32_packed_weight_bytes",
            "onhip_conv2d_w8a32_pack_weights", "onhip_conv2d_w8a32_packed", "onhip_quantize_nhwc_s8",
            "onhip_conv2d_w8a8_nhwc", "onhip_quant_weight_bias",

@@ -30,9 +30,10 @@ class Plugin:
         self.eval.argtypes = [C.POINTER(BUFFER_INFO_S)] * 3
         # entry points beside `eval` that the HIP Conv plugin has and the reference's plugins do not: the convolution
         # with the Add (and Relu) of a residual block folded in, the other operand of the Add in inputs[3]
-        # and a whole inverted-residual block (eval_block, eval_block_takes); the MatMul plugin's fused forms
+        # and a whole inverted-residual block (eval_block, eval_block_takes) or a convolution and the 1x1 convolution after
+        # it (eval_pair, eval_pair_relu, eval_pair_takes); the MatMul plugin's fused forms
         # (eval_link: an int8 convolution whose activations travel as int8 NHWC on one or both sides)
-        for extra in ("eval_add", "eval_add_relu", "eval_block", "eval_block_takes", "eval_link", "eval_attention", "eval_bias", "eval_bias_gelu",
+        for extra in ("eval_add", "eval_add_relu", "eval_block", "eval_block_takes", "eval_pair", "eval_pair_relu", "eval_pair_takes", "eval_link", "eval_attention", "eval_bias", "eval_bias_gelu",
                       "eval_bias_add"):
             fn = getattr(self.lib, extra, None) if hasattr(self.lib, extra) else None
             if fn is not None:

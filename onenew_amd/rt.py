@@ -8,7 +8,7 @@ from . import hip
 
 EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
            "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf",
-           "onrt_net_folded_activations", "onrt_net_fused_attentions", "onrt_net_fused_linears", "onrt_net_fused_skips", "onrt_net_fused_ir_blocks", "onrt_net_quantised_links", "onrt_net_tune_tiles", "onrt_net_get_tiles", "onrt_net_set_tiles", "onrt_one_set_tiles", "onrt_one_quantise"]
+           "onrt_net_folded_activations", "onrt_net_fused_attentions", "onrt_net_fused_linears", "onrt_net_fused_skips", "onrt_net_fused_ir_blocks", "onrt_net_fused_pairs", "onrt_net_quantised_links", "onrt_net_tune_tiles", "onrt_net_get_tiles", "onrt_net_set_tiles", "onrt_one_set_tiles", "onrt_one_quantise"]
 
 _lib = None
 
@@ -47,6 +47,7 @@ def load():
     L.onrt_net_fused_linears.argtypes = [vp, i32p]
     L.onrt_net_fused_skips.argtypes = [vp, i32p]
     L.onrt_net_fused_ir_blocks.argtypes = [vp, i32p]
+    L.onrt_net_fused_pairs.argtypes = [vp, i32p]
     L.onrt_net_quantised_links.argtypes = [vp, i32p]
     L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
     L.onrt_net_run.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
@@ -182,6 +183,12 @@ class Net:
         """number of Conv (1x1) -> depthwise Conv -> Conv (1x1) [-> Add] blocks that run as one call"""
         n = C.c_int32()
         _check(load().onrt_net_fused_ir_blocks(self._h, C.byref(n)), "onrt_net_fused_ir_blocks")
+        return n.value
+
+    def fused_pairs(self):
+        """number of Conv -> Conv (1x1) [-> Add [-> Relu]] pairs that run as one call"""
+        n = C.c_int32()
+        _check(load().onrt_net_fused_pairs(self._h, C.byref(n)), "onrt_net_fused_pairs")
         return n.value
 
     def int8_links(self):

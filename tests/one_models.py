@@ -57,6 +57,29 @@ def inverted_residual_blocks(batch=8, size=32):
     return m.tobytes(), [_r("xir", (batch, 16, size, size))]
 
 
+def bottleneck_pairs(batch=16, size=32):
+    """two ResNet-style bottlenecks with 16 channels inside, on a plane large enough at this batch for the library to
+    recommend the 3x3 convolution and the 1x1 after it as one launch: the first with a projection on the skip path (which
+    comes before the last convolution in the file, as in ResNet-50, so the Add is folded into the projection and the pair
+    has none), the second with the identity skip (the pair takes the Add and the Relu)"""
+    m = onefile.OneModel()
+    m.input("x", (batch, 32, size, size))
+    m.conv("c1", "x", _r("bp_c1w", (16, 32, 1, 1), 0.25), _r("bp_c1b", (16,), 0.2), "c1_out", act=abi.RELU)
+    m.conv("c2", "c1_out", _r("bp_c2w", (16, 16, 3, 3), 0.12), _r("bp_c2b", (16,), 0.2), "c2_out", pad=1, act=abi.RELU)
+    m.conv("dn", "x", _r("bp_dnw", (64, 32, 1, 1), 0.2), _r("bp_dnb", (64,), 0.1), "dn_out")
+    m.conv("c3", "c2_out", _r("bp_c3w", (64, 16, 1, 1), 0.2), _r("bp_c3b", (64,), 0.1), "c3_out")
+    m.add("add1", "c3_out", "dn_out", "add1_out")
+    m.relu("relu1", "add1_out", "r1")
+    m.conv("c4", "r1", _r("bp_c4w", (16, 64, 1, 1), 0.2), _r("bp_c4b", (16,), 0.2), "c4_out", act=abi.RELU)
+    m.conv("c5", "c4_out", _r("bp_c5w", (16, 16, 3, 3), 0.12), _r("bp_c5b", (16,), 0.2), "c5_out", pad=1, act=abi.RELU)
+    m.conv("c6", "c5_out", _r("bp_c6w", (64, 16, 1, 1), 0.2), _r("bp_c6b", (64,), 0.1), "c6_out")
+    m.add("add2", "c6_out", "r1", "add2_out")
+    m.relu("relu2", "add2_out", "out")
+    m.output("out", (batch, 64, size, size))
+    m.output("r1", (batch, 64, size, size))
+    return m.tobytes(), [_r("xbp", (batch, 32, size, size))]
+
+
 def separable_chain(batch=16, size=32, ch=32):
     """a depthwise-separable stack pw -> dw -> pw -> dw -> pw (MobileNetV1 style, at most 64 channels): the last 1x1 of the
     first triple is also the first 1x1 of the next, so one-launch blocks must not overlap"""

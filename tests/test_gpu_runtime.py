@@ -270,6 +270,45 @@ def test_inverted_residual_blocks_run_as_one_call(torch_dev, monkeypatch):
     small.close()
 
 
+def test_convolution_pairs_run_as_one_call(torch_dev, monkeypatch):
+    """Conv (3x3) -> Conv (1x1) of two ResNet-style bottlenecks as one call of the Conv plugin's eval_pair / eval_pair_relu
+    each, where the plugin recommends it: the pair of the first block without an Add (the projection on the skip path took
+    it), the pair of the second with the Add and the Relu; the same bits as the net run operator by operator on the tile the
+    pair's kernel uses, within 1e-4 of it whatever tiles it picks, and close to the CPU restatement of the graph; at a
+    small batch the operators stay separate"""
+    data, ins = one_models.bottleneck_pairs(batch=16, size=32)
+    fused, plain, got, want = _both_ways(data, ins, monkeypatch)
+    assert plain.fused_pairs() == 0 and fused.fused_pairs() == 2
+    assert [n for _, n in fused.ops()] == ["c1", "c2", "dn", "c4", "c5"] and len(plain.ops()) == 11
+    assert fused.fused_blocks() == 2   # the two Adds (and Relus) were folded first: into dn and into c6
+    for name in ("c2_out", "c5_out"):
+        assert fused.operand(name)[1] is None
+    assert fused.operand("c6_out")[1] == fused.operand("add2_out")[1] == fused.operand("out")[1]
+    ref = one_model.run(data, ins)
+    for g, w_, r in zip(got, want, ref):
+        assert g.shape == w_.shape and np.all(np.abs(g - w_) <= 1e-4 * np.abs(w_) + 1e-5 * np.abs(w_).max())
+        assert _close(g, r, 5e-4)
+    x2 = [(ins[0] * np.float32(-0.7) + np.float32(0.2)).astype(np.float32)]
+    for g, w_ in zip(fused.run(*x2), plain.run(*x2)):
+        assert np.all(np.abs(g - w_) <= 1e-4 * np.abs(w_) + 1e-5 * np.abs(w_).max())
+    fused.close()
+    plain.close()
+    monkeypatch.setenv("ONHIP_TILE", "64x64x1")
+    tiled = rt.Net(data)
+    monkeypatch.setenv("ONENEW_RT_FUSE_PAIRS", "0")
+    tiled_plain = rt.Net(data)
+    monkeypatch.delenv("ONENEW_RT_FUSE_PAIRS")
+    assert tiled.fused_pairs() == 2 and tiled_plain.fused_pairs() == 0 and tiled_plain.fused_blocks() == 2
+    for g, w_ in zip(tiled.run(*ins), tiled_plain.run(*ins)):
+        assert np.array_equal(g, w_)
+    tiled.close()
+    tiled_plain.close()
+    monkeypatch.delenv("ONHIP_TILE")
+    small = rt.Net(one_models.bottleneck_pairs(batch=1, size=32)[0])
+    assert small.fused_pairs() == 0 and len(small.ops()) == 7
+    small.close()
+
+
 def test_one_launch_blocks_do_not_overlap_nor_swallow_a_folded_adds_operand(torch_dev, monkeypatch):
     """pw -> dw -> pw -> dw -> pw with at most 64 channels at a batch where the plugin recommends the block kernel: one block
     is folded (the middle 1x1 closes it and opens no second one), the output equals the operator-by-operator run within
