@@ -345,10 +345,14 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
     const double per_cu = ceil(wgs / 256.0);
     const int regs_occ = c.bm * c.bn >= 128 * 128 ? 3 : c.bm * c.bn >= 64 * 128 ? 4 : 6;
     const double resident = per_cu < regs_occ ? per_cu : regs_occ;
-    const double overhead = cfg.bl == BL_GATHER ? 1.35 : 1.18;   // measured steady-state inefficiency
+    // measured steady-state inefficiency; a workgroup alone on its CU (one wavefront per SIMD, in lock step at every
+    // barrier) needs 690 cycles for the 512 of a K tile where several resident ones need about 600
+    const double overhead = (cfg.bl == BL_GATHER ? 1.35 : 1.18) * (resident <= 1.0 ? 1.15 : 1.0);
     const double mfma = per * tile_mfma_cycles(cfg.dtype, c.bm, c.bn) * overhead;
     const double fixed = 2600.0 + 12.0 * (c.bm * c.bn / 256);     // first loads in flight + epilogue stores
-    double cycles = per_cu * mfma + ceil(per_cu / resident) * fixed;
+    // the fixed part of co-resident workgroups overlaps; a last, partly filled group of them pays its share of it, not
+    // all of it (with all of it the 64 x 128 tile won over 64 x 64 on short-K layers, where it measures 15 % slower)
+    double cycles = per_cu * mfma + per_cu / resident * fixed;
     if (c.split > 1) cycles += 9000.0 + (double) (c.split + 1) * p.M * p.N * cfg.batch * 4.0 / 1500.0;
     return cycles;
 }
@@ -403,9 +407,13 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     //    launch's spread over every compute unit wins).  Same sums in the same order either way.
     if (cfg.dtype == DT_F32 && !vec && !best.rowb && !best.dma) {
         int dpc = 0, left = 0;
-        if (best.split == 1 && tail_geometry(cfg, p, best.bm, best.bn, &dpc, &left)) {
+        // ... where K is long enough to be cut: measured on the ResNet-50 layers at batch 32, a leftover cut along a K of
+        // 256 or less loses 2-7 us on every layer (the slices are all fill and drain), one of 512 gains only when cut in
+        // at most four
+        if (best.split == 1 && p.k_units > 64 && tail_geometry(cfg, p, best.bm, best.bn, &dpc, &left)) {
             int want = 256 / left;
             want = want > 16 ? 16 : want;
+            if (p.k_units <= 128 && want > 4) want = 4;
             for (int ts = want; ts >= 2; ts /= 2) {
                 const Choice c = {best.bm, best.bn, 1, ts, 0, 0, 0};
                 if (candidate_ok(cfg, p, c)) { best = c; break; }
