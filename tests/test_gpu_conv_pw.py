@@ -82,6 +82,44 @@ def test_pair_equals_the_operator_chain(shape, torch_dev, oracle):
     close(y.cpu().numpy(), ref)
 
 
+def _random_shapes(count=24):
+    """seeded draws over everything the entry point takes: 1-64 middle channels, 1-200 output channels, 1-3 images, filters
+    of 1-5 rows and columns (never a plain 1x1), strides 1-3, paddings up to the filter's reach, every activation pair"""
+    rng = np.random.default_rng(20251)
+    out = []
+    while len(out) < count:
+        n, cin, cmid, cout = int(rng.integers(1, 4)), int(rng.integers(1, 40)), int(rng.integers(1, 65)), int(rng.integers(1, 201))
+        kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        pads = tuple(int(rng.integers(0, k)) for k in (kh, kw, kh, kw))
+        if kh == 1 and kw == 1 and not any(pads):
+            continue
+        h, w, s = int(rng.integers(kh, 24)), int(rng.integers(kw, 24)), int(rng.integers(1, 4))
+        act_a, act_b = (int(rng.choice([N, R, CL])) for _ in range(2))
+        out.append((n, cin, cmid, h, w, cout, (kh, kw), s, pads, act_a, act_b, bool(rng.integers(0, 2)), bool(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("shape", _random_shapes())
+def test_pair_random_shapes(shape, torch_dev, oracle):
+    torch = torch_dev
+    n, cin, cmid, h, w, cout, k, s, p, act_a, act_b, with_res, relu = shape
+    print(f"conv + 1x1, drawn shape {shape}", flush=True)
+    a, b = descs(n, cin, cmid, h, w, cout, k, s, p, act_a, act_b)
+    assert hip.conv2d_pw_supported(a, b) >= 1
+    x, wa, ba, wb, bb = operands(f"convpw_rand{shape}", a, b)
+    oh, ow = a.out_hw()
+    res = cases.datagen.normal(cases.datagen.seed_for("convpw_rand", "res", *shape[:6]), (n, cout, oh, ow), 0.0, 1.0) if with_res else None
+    y = hip.conv2d_pw_f32(a, b, dev(torch, x), hip.pack_conv_weights(a, dev(torch, wa)), dev(torch, ba),
+                          hip.conv2d_pw_pack_weights(b, dev(torch, wb)), dev(torch, bb), dev(torch, res), relu and with_res)
+    torch.cuda.synchronize()
+    ref = oracle.conv2d_f32(b, oracle.conv2d_f32(a, x, wa, ba), wb, bb).astype(np.float64)
+    if with_res:
+        ref = ref + res
+        if relu:
+            ref = np.maximum(ref, 0.0)
+    close(y.cpu().numpy(), ref)
+
+
 @pytest.mark.parametrize("bias_a,bias_b", [(0, 1), (1, 0), (0, 0)])
 def test_pair_without_biases(bias_a, bias_b, torch_dev, oracle):
     """a convolution without bias has no activation either (conv.c:18-27), in both places"""
