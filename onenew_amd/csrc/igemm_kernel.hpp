@@ -363,9 +363,11 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
         const rsrc_t rres = make_rsrc(RES ? reinterpret_cast<const char *>(p.res) + (size_t) batch * p.c_batch_stride * 4 : nullptr,
                                       RES ? RSRC_RANGE : 0u);
         const rsrc_t rtwin = make_rsrc(RES ? p.twin : nullptr, RES && p.twin ? RSRC_RANGE : 0u);
-        unsigned tw[TN];
+        unsigned tq[TN][4];
 #pragma unroll
-        for (int b = 0; b < TN; ++b) tw[b] = 0;
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tq[b][j] = 0;
 #pragma unroll
         for (int a = 0; a < TM; ++a) {
             float rv[RES ? 16 : 1][RES ? TN : 1];
@@ -397,14 +399,20 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                     float y = act_fast<EPI>(__fmul_rn(f, coeff), p.ep);
                     if constexpr (RES) {
                         y = add_res(y, rv[r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
-                        // the int8 twin: registers 4 q .. 4 q + 3 are four consecutive channels of the lane's pixel
+                        // the int8 twin: registers 4 q .. 4 q + 3 are four consecutive channels of the lane's pixel.  The
+                        // quantiser's product and clamp as a multiply and a median of three (a NaN comes out as -128 here
+                        // and as 0 from the comparisons of requant_s8; no finite operand produces one), the four low
+                        // bytes packed with three byte permutes
                         if (p.twin) {   // uniform
-                            tw[b] |= ((unsigned) requant_s8(y, p.twin_inv_scale) & 0xffu) << (8 * (r % 4));
+                            tq[b][r % 4] = (unsigned) round_half_away_small(
+                                __builtin_amdgcn_fmed3f(__fmul_rn(y, p.twin_inv_scale), -128.0f, 127.0f));
                             if (r % 4 == 3) {
                                 const int n = n_wave + b * 32 + li, m4 = m_wave + a * 32 + 8 * (r / 4) + 4 * lh;
                                 const bool ok = n < p.N && m4 < p.M;
-                                __builtin_amdgcn_raw_buffer_store_b32(tw[b], rtwin, ok ? (unsigned) (n * p.twin_pitch + m4) : OOB, 0, 0);
-                                tw[b] = 0;
+                                const unsigned p01 = __builtin_amdgcn_perm(tq[b][1], tq[b][0], 0x0c0c0400u);
+                                const unsigned p23 = __builtin_amdgcn_perm(tq[b][3], tq[b][2], 0x0c0c0400u);
+                                __builtin_amdgcn_raw_buffer_store_b32(__builtin_amdgcn_perm(p23, p01, 0x05040100u), rtwin,
+                                                                      ok ? (unsigned) (n * p.twin_pitch + m4) : OOB, 0, 0);
                             }
                         }
                     }
