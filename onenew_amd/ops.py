@@ -285,6 +285,56 @@ class ConvBlock(_Op):
         return out
 
 
+class ConvPair(_Op):
+    """Conv (dense, at most 64 output channels) -> Conv (1x1) [-> Add [-> Relu]] through the HIP Conv plugin's `eval_pair` /
+    `eval_pair_relu`: the slots of the first convolution's `eval` with the pair's result operand in params[4], then the second
+    convolution's CONV_CONFIG_S, weight operand, weights and bias in params[5], params[6], inputs[5], inputs[6]; the addend
+    in inputs[3].  No counterpart among the reference's host classes."""
+
+    def __init__(self, plugin, descs, weights, biases):
+        super().__init__(plugin.eval_pair)
+        self.relu_fn, self.takes_fn = plugin.eval_pair_relu, plugin.eval_pair_takes
+        self.convs = [Conv(None, d, w, b) for d, w, b in zip(descs, weights, biases)]
+        first, second = self.convs
+        oh, ow = second.desc.out_hw()
+        self.out_shape = (second.desc.n, second.desc.cout, oh, ow)
+        self.out_operand = make_operand(self.out_shape, b"out")
+        self._slot(self.params_vec, 0, first.conv_cfg)
+        self._slot(self.params_vec, 1, first.in_operand)
+        self._slot(self.params_vec, 2, first.weight_operand)
+        self._slot(self.params_vec, 3, first.bias_operand)
+        self._slot(self.params_vec, 4, self.out_operand)
+        self._slot(self.inputs_vec, 1, first.weight)
+        if first.desc.has_bias:
+            self._slot(self.inputs_vec, 2, first.bias)
+        self._slot(self.params_vec, 5, second.conv_cfg)
+        self._slot(self.params_vec, 6, second.weight_operand)
+        self._slot(self.inputs_vec, 5, second.weight)
+        if second.desc.has_bias:
+            self._slot(self.inputs_vec, 6, second.bias)
+
+    def takes(self):
+        """1 when the library recommends the one-launch kernel for these shapes"""
+        return self.takes_fn(self.params_vec, self.inputs_vec, self.outputs_vec)
+
+    def __call__(self, x, addend=None, relu=False, out=None):
+        xin = np.ascontiguousarray(x, dtype=np.float32)
+        if out is None:
+            out = aligned_empty(self.out_shape, np.float32)
+        self._slot(self.inputs_vec, 0, xin)
+        self._slot(self.outputs_vec, 0, out)
+        kept = 2
+        if addend is not None:
+            self._slot(self.inputs_vec, 3, np.ascontiguousarray(addend, dtype=np.float32))
+            kept = 3
+        rc = (self.relu_fn if relu else self.eval)(self.params_vec, self.inputs_vec, self.outputs_vec)
+        del self._keep[-kept:]
+        self.inputs_vec[3].addr = 0
+        if rc != 0:
+            raise RuntimeError(f"Conv eval_pair returned {rc}")
+        return out
+
+
 class MatMul(_Op):
     """host/ops/mat_mul.h: out = A[..., M, K] @ B, B either [K, N] shared or batched like A."""
 

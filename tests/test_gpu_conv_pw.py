@@ -186,6 +186,27 @@ def test_resnet50_first_stage_pair_at_batch_32(torch_dev, monkeypatch):
     assert torch.equal(y_res, two_res), f"{(y_res != two_res).sum().item()} of {y.numel()} values differ"
 
 
+@pytest.mark.parametrize("shape", [(2, 16, 32, 20, 20, 64, 3, 1, 1, R, N, True, True), (1, 8, 48, 9, 11, 100, 3, 2, 1, CL, R, False, False)])
+def test_plugin_eval_pair_host_buffers(shape, torch_dev, oracle):
+    """the Conv plugin's eval_pair / eval_pair_relu on tensors in host memory, slots filled like the host fills a Conv's
+    (weights and biases as fixed operands, the pair's result operand in params[4]): within 1e-4 of the oracle's operator
+    chain, a second call (cached weights) identical, and eval_pair_takes saying that so small a batch is not recommended"""
+    from onenew_amd import ops
+    n, cin, cmid, h, w, cout, k, s, p, act_a, act_b, with_res, relu = shape
+    a, b = descs(n, cin, cmid, h, w, cout, k, s, p, act_a, act_b)
+    x, wa, ba, wb, bb = operands(f"convpw_plugin{shape}", a, b)
+    oh, ow = a.out_hw()
+    res = cases.datagen.normal(cases.datagen.seed_for("convpw_plugin", "res", *shape[:6]), (n, cout, oh, ow), 0.0, 1.0) if with_res else None
+    pair = ops.ConvPair(ops.Plugin(hip.plugin_path("Conv")), (a, b), (wa, wb), (ba, bb))
+    assert pair.takes() == 0
+    y = pair(x, addend=res, relu=relu).copy()
+    assert np.array_equal(pair(x, addend=res, relu=relu), y)
+    ref = oracle.conv2d_f32(b, oracle.conv2d_f32(a, x, wa, ba), wb, bb).astype(np.float64)
+    if with_res:
+        ref = np.maximum(ref + res, 0.0) if relu else ref + res
+    close(y, ref)
+
+
 def test_pair_refuses_what_it_cannot_run(torch_dev):
     torch = torch_dev
     ok_a, ok_b = descs(1, 16, 32, 10, 10, 64, 3, 1, 1, R, N)
