@@ -559,12 +559,21 @@ static int plan_and_launch(const IgemmLaunch &cfg, const IgemmParams &p, hipStre
     ONHIP_CHECK_HIP(hipEventCreate(&e0));
     ONHIP_CHECK_HIP(hipEventCreate(&e1));
     Choice best = guess;
-    float best_ms = 1e30f;
+    float best_ms = 1e30f, guess_ms = 1e30f;
     int rc = ONHIP_OK;
+    // The model's own choice is measured first (it need not be among the candidates below), and another one takes its
+    // place only by beating it by 2 %: the measurements repeat within about 3 %, and without the margin a launch that is
+    // no faster replaces the model's on a coin toss (seen as a tuned stack slower than the untuned one).
+    rc = time_choice(cfg, p, guess, st, e0, e1, &guess_ms);
+    best_ms = guess_ms;
+    auto same = [](const Choice &a, const Choice &b) {
+        return a.bm == b.bm && a.bn == b.bn && a.split == b.split && a.tail == b.tail && a.rowb == b.rowb && a.fin == b.fin && a.dma == b.dma;
+    };
     auto try_choice = [&](const Choice &c) {
+        if (same(c, guess)) return;
         float ms = 0.f;
         rc = time_choice(cfg, p, c, st, e0, e1, &ms);
-        if (!rc && ms < best_ms) { best_ms = ms; best = c; }
+        if (!rc && ms < best_ms && ms < 0.98f * guess_ms) { best_ms = ms; best = c; }
     };
     for (int t = 0; t < kNumTiles && !rc; ++t) {
         for (int s = 0; s < kNumSplits && !rc; ++s) {
