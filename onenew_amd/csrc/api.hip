@@ -348,7 +348,10 @@ static double model_cost(const IgemmLaunch &cfg, const IgemmParams &p, const Cho
     // measured steady-state inefficiency; a workgroup alone on its CU (one wavefront per SIMD, in lock step at every
     // barrier) needs 690 cycles for the 512 of a K tile where several resident ones need about 600
     const double overhead = (cfg.bl == BL_GATHER ? 1.35 : 1.18) * (resident <= 1.0 ? 1.15 : 1.0);
-    const double mfma = per * tile_mfma_cycles(cfg.dtype, c.bm, c.bn) * overhead;
+    // fp32: the wider tiles leave fewer wavefronts resident and measure behind the 64 x 64 one wherever the two come
+    // out even here (ViT-Tiny's first MLP product at batch 64: 50 against 44 us)
+    const double wide = cfg.dtype == DT_F32 && c.bm * c.bn > 64 * 64 ? 1.05 : 1.0;
+    const double mfma = per * tile_mfma_cycles(cfg.dtype, c.bm, c.bn) * overhead * wide;
     const double fixed = 2600.0 + 12.0 * (c.bm * c.bn / 256);     // first loads in flight + epilogue stores
     // the fixed part of co-resident workgroups overlaps; a last, partly filled group of them pays its share of it, not
     // all of it (with all of it the 64 x 128 tile won over 64 x 64 on short-K layers, where it measures 15 % slower)
@@ -387,6 +390,14 @@ static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     Choice best = {64, 64, 1, 0, 0, 0};
     const bool vec = cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP;
     if (vec && (cfg.dtype != DT_I8 || !tl_hint_bm) && dma_model_choice(cfg, p, &best)) return best;
+    // fp32 1x1 convolutions with at most 32 input channels (MobileNetV2's first expansions and projection): B straight from
+    // memory, no LDS round trip for an operand that is used once per 32 rows (measured 10-35 % ahead of the tiled kernel on
+    // every such layer at batch 64); the tile by the row count
+    if (cfg.dtype == DT_F32 && cfg.bl == BL_PLAIN && p.K <= 32 && !tl_hint_bm && !p.res) {
+        const Choice c = p.M <= 32 ? Choice{32, 256, 1, 0, 1, 0, 0} : p.M % 96 == 0 ? Choice{96, 128, 1, 0, 1, 0, 0} : Choice{64, 256, 1, 0, 1, 0, 0};
+        const long long tiles = (long long) ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
+        if (tiles >= 512 && candidate_ok(cfg, p, c)) return c;   // measured at batch 64 only: at least two workgroups per CU
+    }
     for (int pass = tl_hint_bm ? 0 : 1; pass < 2; ++pass) {   // pass 0: the hinted tile; pass 1: every tile
         double best_cost = 1e300;
         for (int t = 0; t < kNumTiles; ++t)
