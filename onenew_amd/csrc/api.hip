@@ -371,25 +371,42 @@ static thread_local int tl_hint_bm = 0, tl_hint_bn = 0;
 // register-staged kernel, which has one.
 static bool dma_model_choice(const IgemmLaunch &cfg, const IgemmParams &p, Choice *out) {
     static const int order[4][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
+    // what a tile's steady state costs per output against the largest one's (measured on the YOLOv8s layers)
+    static const double eff[4] = {1.0, 1.08, 1.10, 1.20};
     const bool only = cfg.dtype != DT_I8;   // the 16-bit types have no other kernel for these operands
+    // int8 with a large fp32 result (the reference's W8A32 form on big planes): the register-staged kernel's store of
+    // fp32 rows is the faster one from about 6.5 million outputs up (every such YOLOv8s layer at batch 16, 5-35 %)
+    if (!only && !p.out_s8 && (long long) p.M * p.N >= (long long) 256 * 25600) return false;
+    // The largest tile does not always win: among the tiles that give every CU a workgroup and then some, the one with the
+    // least work in its rounds of 256 workgroups (800 tiles of 128 x 128 are four rounds, 1600 of 128 x 64 seven half as
+    // long).  Problems with so few tiles that only a split along K reaches all CUs go to the register-staged kernel.
+    int best = -1;
+    double best_cost = 1e300;
     for (int t = 0; t < 4; ++t) {
         const Choice c = {order[t][0], order[t][1], 1, 0, 0, 0, 1};
         if (!candidate_ok(cfg, p, c)) return false;
         if (c.bm == 128 && p.M <= 64) continue;
         const long long tiles = (long long) ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
-        if (tiles >= 320 || t == 3) {
-            if (tiles < 96 && p.k_units >= 128 && !only) return false;
-            *out = c;
-            return true;
-        }
+        if (tiles < 320 && t != 3) continue;
+        if (t == 3 && tiles < 96 && p.k_units >= 128 && !only) return false;
+        const double cost = (double) ((tiles + 255) / 256) * c.bm * c.bn * eff[t];
+        if (cost < best_cost) { best_cost = cost; best = t; }
     }
-    return false;
+    if (best < 0) return false;
+    *out = Choice{order[best][0], order[best][1], 1, 0, 0, 0, 1};
+    return true;
 }
 
 static Choice model_choice(const IgemmLaunch &cfg, const IgemmParams &p) {
     Choice best = {64, 64, 1, 0, 0, 0};
     const bool vec = cfg.bl == BL_KVEC || cfg.bl == BL_KVEC_TAP;
     if (vec && (cfg.dtype != DT_I8 || !tl_hint_bm) && dma_model_choice(cfg, p, &best)) return best;
+    // int8 with a large fp32 result (see dma_model_choice): 64 x 128 on the register-staged kernel, 32 rows where there
+    // are no more
+    if (vec && cfg.dtype == DT_I8 && !tl_hint_bm && !p.out_s8 && (long long) p.M * p.N >= (long long) 256 * 25600) {
+        const Choice c = {p.M <= 32 ? 32 : 64, 128, 1, 0, 0, 0, 0};
+        if (candidate_ok(cfg, p, c)) return c;
+    }
     // fp32 1x1 convolutions with at most 32 input channels (MobileNetV2's first expansions and projection): B straight from
     // memory, no LDS round trip for an operand that is used once per 32 rows (measured 10-35 % ahead of the tiled kernel on
     // every such layer at batch 64); the tile by the row count
