@@ -136,7 +136,8 @@ int onhip_conv2d_f32(const onhip_conv_desc_t *d, const float *x, const float *w,
  * runs fastest on weights re-laid out tap-major, [cout][kh*kw][cin padded to the MFMA unit]: every
  * group of input channels then shares one filter tap and the im2col arithmetic shrinks to one
  * scalar description per group.  onhip_conv2d_packed_weight_bytes returns the size of that copy
- * (0 when the convolution takes its weights as they are: 1x1 without padding, depthwise);
+ * (0 when the convolution takes its weights as they are: 1x1 without padding, depthwise, and, first
+ * layers with three input channels apart, fewer than four input channels or more than 64 filter taps);
  * onhip_conv2d_pack_weights writes it (device kernel on `stream`); onhip_conv2d_f32_packed is
  * onhip_conv2d_f32 on such a copy.  Results of the two entry points agree to fp32 rounding (the
  * summation order over K differs).  No counterpart in the reference, whose only weight

@@ -743,8 +743,17 @@ static int packed_cp(const onhip_conv_desc_t *d) {
     return (d->cin + kpu - 1) / kpu * kpu;
 }
 
+// Dense convolutions other than the plain 1x1 have a packed weight form: the first-layer kernel's own, or the tap-major one.
+// Not the tap-major one where it would cost more than it saves: fewer than four input channels (a tap is padded to four:
+// a third more reduction) and filters of more than 64 taps (validity by coordinates instead of the lane's mask); the
+// element gather on the weights as they are measures 25 % ahead there (ViT's 16 x 16 patch convolution: 63 against 83 us).
+// a 1x1 filter without padding: the input itself is the B operand, no window arithmetic
+static bool plain_pointwise(const onhip_conv_desc_t *d) {
+    return d->kh == 1 && d->kw == 1 && !d->pad_t && !d->pad_l && !d->pad_b && !d->pad_r;
+}
 static bool wants_packed(const onhip_conv_desc_t *d) {
-    return d->group == 1 && !(d->kh == 1 && d->kw == 1 && !d->pad_t && !d->pad_l && !d->pad_b && !d->pad_r);
+    if (d->group != 1 || plain_pointwise(d)) return false;
+    return stem_f32_shape(*d) || (d->cin >= 4 && d->kh * d->kw <= 64);
 }
 
 size_t onhip_conv2d_packed_weight_bytes(const onhip_conv_desc_t *d) {
@@ -829,7 +838,7 @@ static int conv2d_f32_impl(const onhip_conv_desc_t *d, const float *x, const flo
         p.units_per_tap = cp / kpu;
         p.magic_upt = magic_for(p.units_per_tap); p.pass_upt = pass_for(p.units_per_tap);
     } else {
-        cfg.bl = wants_packed(d) ? BL_GATHER : BL_PLAIN;
+        cfg.bl = plain_pointwise(d) ? BL_PLAIN : BL_GATHER;
         p.K = d->cin * p.khkw;
     }
     if ((unsigned long long) p.K * (unsigned) p.khkw >= (1ULL << 32))

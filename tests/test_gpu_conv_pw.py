@@ -88,7 +88,7 @@ def _random_shapes(count=24):
     rng = np.random.default_rng(20251)
     out = []
     while len(out) < count:
-        n, cin, cmid, cout = int(rng.integers(1, 4)), int(rng.integers(1, 40)), int(rng.integers(1, 65)), int(rng.integers(1, 201))
+        n, cin, cmid, cout = int(rng.integers(1, 4)), int(rng.integers(4, 40)), int(rng.integers(1, 65)), int(rng.integers(1, 201))
         kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
         pads = tuple(int(rng.integers(0, k)) for k in (kh, kw, kh, kw))
         if kh == 1 and kw == 1 and not any(pads):
@@ -216,6 +216,7 @@ def test_pair_refuses_what_it_cannot_run(torch_dev):
     bad = [descs(1, 16, 96, 10, 10, 64, 3, 1, 1, R, N),          # more than 64 middle channels
            descs(1, 16, 32, 10, 10, 64, 1, 1, 0, R, N),          # the first convolution is a plain 1x1
            descs(1, 3, 32, 32, 32, 64, 7, 2, 3, R, N),           # a first layer
+           descs(1, 3, 32, 10, 10, 64, 5, 1, 2, R, N),           # fewer than four input channels: no tap-major weights
            descs(1, 16, 32, 10, 10, 64, 3, 1, 1, abi.SILU, N),   # a table activation
            descs(1, 16, 32, 10, 10, 64, 3, 1, 1, R, abi.LEAKYRELU)]
     for a, b in bad:

@@ -220,8 +220,17 @@ def test_depthwise_stride_leaves_rows_and_columns_unread(shape, quant, torch_dev
     assert np.array_equal(y.cpu().numpy(), ref)
 
 
-PACKED_CASES = [n for n, d in cases.conv_f32_cases().items()
-                if d.group == 1 and not (d.kh == 1 and d.kw == 1 and d.pad_t == 0)]
+def _has_packed_form(d):
+    """dense, not a plain 1x1; the first-layer kernel's shapes, or at least four input channels and at most 64 taps"""
+    if d.group != 1 or (d.kh == 1 and d.kw == 1 and d.pad_t == 0):
+        return False
+    first_layer = d.cin == 3 and d.cout <= 64 and d.kh == d.kw and d.kh in (3, 7) and d.stride_h == d.stride_w and d.stride_h <= 2
+    return first_layer or (d.cin >= 4 and d.kh * d.kw <= 64)
+
+
+PACKED_CASES = [n for n, d in cases.conv_f32_cases().items() if _has_packed_form(d)]
+UNPACKED_DENSE_CASES = [n for n, d in cases.conv_f32_cases().items()
+                        if d.group == 1 and not (d.kh == 1 and d.kw == 1 and d.pad_t == 0) and not _has_packed_form(d)]
 
 
 @pytest.mark.parametrize("name", PACKED_CASES)
@@ -241,6 +250,19 @@ def test_conv_f32_packed_weights(name, torch_dev, oracle):
     assert_close_f32(y.cpu().numpy(), oracle.conv2d_f32(dn, x, w, b), tag=name + " packed")
 
 
+@pytest.mark.parametrize("name", UNPACKED_DENSE_CASES)
+def test_conv_f32_shapes_without_a_packed_form(name, torch_dev):
+    """fewer than four input channels or more than 64 filter taps (first-layer shapes apart): the library says that the
+    weights are taken as they are, and refuses to pack them or to be handed packed ones"""
+    torch = torch_dev
+    d = cases.conv_f32_cases()[name]
+    x, w, b = cases.conv_inputs(name, d)
+    wd = dev(torch, w)
+    assert hip.pack_conv_weights(d, wd) is None
+    with pytest.raises(hip.OnhipError):
+        hip.conv2d_f32(d, dev(torch, x), wd, dev(torch, b), None, packed=True)
+
+
 @pytest.mark.parametrize("compute", [abi.COMPUTE_BF16, abi.COMPUTE_F16])
 def test_conv_packed_reduced_precision(compute, torch_dev, oracle):
     torch = torch_dev
@@ -249,7 +271,8 @@ def test_conv_packed_reduced_precision(compute, torch_dev, oracle):
         d.compute = compute
         x, w, b = cases.conv_inputs(name, d)
         wp = hip.pack_conv_weights(d, dev(torch, w))
-        y = hip.conv2d_f32(d, dev(torch, x), wp, dev(torch, b), None, packed=True)
+        assert (wp is None) == (d.cin < 4)   # three input channels at reduced precision: no packed form, the element gather
+        y = hip.conv2d_f32(d, dev(torch, x), wp if wp is not None else dev(torch, w), dev(torch, b), None, packed=wp is not None)
         torch.cuda.synchronize()
         rnd = oracle.round_bf16 if compute == abi.COMPUTE_BF16 else oracle.round_f16
         assert_close_f32(y.cpu().numpy(), oracle.conv2d_f32(d, rnd(x), rnd(w), b), rel=1e-4, tag=name + " packed")
