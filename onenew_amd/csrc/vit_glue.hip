@@ -259,6 +259,27 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeParams p, const
     y[o] = x[src];
 }
 
+// A batch of plain matrix transposes, x [batch][rows][cols] -> y [batch][cols][rows], through a 32 x 33 LDS tile: both
+// the reads and the writes are runs of 32 consecutive floats (the element-wise kernel above reads one float per 32-byte
+// sector there: 8 x the bytes).  Grid (column tiles, row tiles, batch).
+__global__ __launch_bounds__(256) void transpose_tiled_kernel(const float *__restrict__ x, float *__restrict__ y, int rows, int cols) {
+    __shared__ float tile[32][33];
+    const long long base = (long long) blockIdx.z * rows * cols;
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+    for (int i = ty; i < 32; i += 8) {
+        const int r = r0 + i, c = c0 + tx;
+        if (r < rows && c < cols) tile[i][tx] = x[base + (long long) r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = ty; i < 32; i += 8) {
+        const int c = c0 + i, r = r0 + tx;
+        if (c < cols && r < rows) y[base + (long long) c * rows + r] = tile[tx][i];
+    }
+}
+
 }  // namespace onhip
 
 using namespace onhip;
@@ -343,6 +364,27 @@ int onhip_transpose_f32(const onhip_transpose_desc_t *d, const float *x, float *
         p.extent[k] = d->in_shape[id];
         p.div[k] = make_div31((unsigned) d->in_shape[id]);
         p.in_stride[k] = in_stride[id];
+    }
+    // Extents of one dropped and output dimensions that are neighbours in the input as well merged, what is left may be a
+    // batch of plain matrix transposes (ViT: [batch, channels, tokens, 1] <-> [batch, tokens, channels, 1]; k^T of the
+    // attention): those go through the LDS tile.
+    {
+        long long ext[6], str[6];
+        int m = 0;
+        for (int k = 0; k < d->ndim; ++k) {
+            if (p.extent[k] == 1) continue;
+            if (m > 0 && (long long) p.in_stride[k] == str[m - 1] * ext[m - 1]) ext[m - 1] *= p.extent[k];
+            else { ext[m] = p.extent[k]; str[m] = p.in_stride[k]; ++m; }
+        }
+        const bool matrix = (m == 2 || m == 3) && str[1] == 1 && str[0] == ext[1] && (m == 2 || str[2] == ext[0] * ext[1]);
+        const long long batch = m == 3 ? ext[2] : 1;
+        if (matrix && ext[0] >= 8 && ext[1] >= 8 && batch <= 65535 && (ext[0] + 31) / 32 <= 65535 && ext[0] < (1LL << 31) && ext[1] < (1LL << 31)) {
+            // x [batch][rows = ext[0]][cols = ext[1]] (cols contiguous) -> y [batch][cols][rows]
+            const dim3 grid((unsigned) ((ext[1] + 31) / 32), (unsigned) ((ext[0] + 31) / 32), (unsigned) batch);
+            hipLaunchKernelGGL(transpose_tiled_kernel, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x, y, (int) ext[0], (int) ext[1]);
+            ONHIP_CHECK_HIP(hipGetLastError());
+            return ONHIP_OK;
+        }
     }
     hipLaunchKernelGGL(transpose_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
                        p, x, y);

@@ -1149,6 +1149,22 @@ def test_transpose_matches_numpy_and_plugin(name, torch_dev):
         assert np.array_equal(ops.Transpose(ops.Plugin(hip.plugin_path("Transpose")).eval, perm)(x), np.transpose(x, perm))
 
 
+# shapes that reduce to a batch of plain matrix transposes (the LDS-tile kernel): ViT's tokens <-> channels with its unit
+# dimension, ragged tiles, a single matrix, batch dimensions that merge, rows of fewer than 8 floats (element-wise kernel)
+TRANSPOSE_EXTRA = [((3, 192, 196, 1), (0, 2, 1, 3)), ((3, 196, 192, 1), (0, 2, 1, 3)), ((2, 37, 65), (0, 2, 1)), ((100, 70), (1, 0)),
+                   ((2, 3, 33, 40), (0, 1, 3, 2)), ((5, 1, 64, 9), (0, 1, 3, 2)), ((4, 300, 5), (0, 2, 1)), ((1, 32, 32), (0, 2, 1)),
+                   ((2, 8, 1, 50, 1), (0, 3, 2, 1, 4))]
+
+
+@pytest.mark.parametrize("shape,perm", TRANSPOSE_EXTRA)
+def test_transpose_batches_of_matrices(shape, perm, torch_dev):
+    torch = torch_dev
+    x = cases.transpose_input(f"tr_extra{shape}{perm}", shape)
+    y = hip.transpose_f32(dev(torch, x), perm)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), np.transpose(x, perm))
+
+
 # chain-form shapes beyond the W8A32 case list: output channels that end inside a 16-channel group and inside a
 # row tile, channel counts whose K tiles do / do not straddle filter taps (64-channel multiples or not)
 CHAIN_EXTRA = {
