@@ -182,6 +182,16 @@ int onrt_net_operand(const onrt_net_t *net, const char *name, int32_t *ndim, int
  * (read the result in place through onrt_net_operand).
  */
 int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs);
+/*
+ * The same inference without the wait at its end, for callers that keep the device busy with one batch after the other:
+ * the copies into the net's input buffers, the operators and the copies of the outputs are queued on the default stream
+ * (where the plugins launch) and the call returns; results are complete once that stream is (hipStreamSynchronize(NULL),
+ * or any later work queued on it).  Every inputs[i] and non-NULL outputs[i] must be device memory; handed the net's own
+ * buffers (onrt_net_operand) the call copies nothing.  A call must not be handed input memory that an earlier, still
+ * running call is writing as its output.  Not for a net loaded with ONENEW_RT_GRAPH=1.  No counterpart in the reference,
+ * whose host waits for every operator (host/net.h:613-627).
+ */
+int onrt_net_enqueue(onrt_net_t *net, const void *const *inputs, void *const *outputs);
 
 /*
  * The model-wide GEMM tile: BLOCK_INFO_S.cuda_gemm_tile_{m,n,k} in the file header (common/nn_common.h:28-39;

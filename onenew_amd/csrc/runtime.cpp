@@ -1637,6 +1637,46 @@ ONRT_API int onrt_net_tune_tiles(onrt_net_t *net, int32_t reps, int32_t tiles[3]
     return rc;
 }
 
+namespace {
+bool on_device(const void *p) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void) hipGetLastError();   // plain host memory: clear the sticky error
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+}  // namespace
+
+ONRT_API int onrt_net_enqueue(onrt_net_t *net, const void *const *inputs, void *const *outputs) {
+    if (!net || (!inputs && !net->in_names.empty()) || (!outputs && !net->out_names.empty())) return fail(ONRT_ERR_ARG, "enqueue: null argument");
+    if (net->plan_only) return fail(ONRT_ERR_ARG, "enqueue: this net is a plan (onrt_net_plan_buf): load it to run it");
+    if (net->stream) return fail(ONRT_ERR_ARG, "enqueue: not for a net loaded with ONENEW_RT_GRAPH=1, whose runs go to a stream of its own");
+    for (size_t i = 0; i < net->in_names.size(); ++i)
+        if (!inputs[i] || !on_device(inputs[i])) return fail(ONRT_ERR_ARG, "enqueue: input %zu is not device memory", i);
+    for (size_t i = 0; i < net->out_names.size(); ++i)
+        if (outputs[i] && !on_device(outputs[i])) return fail(ONRT_ERR_ARG, "enqueue: output %zu is not device memory", i);
+    // everything in the order of the default stream, where the plugins launch: copies in, operators, copies out
+    for (size_t i = 0; i < net->in_names.size(); ++i) {
+        const Tensor &t = net->tensors[net->in_names[i]];
+        if (inputs[i] != t.dev) ONRT_HIP(hipMemcpyAsync(t.dev, inputs[i], t.bytes, hipMemcpyDeviceToDevice, nullptr));
+    }
+    set_async(*net, 1);
+    const int rc = run_operators(*net);
+    set_async(*net, 0);
+    ++net->runs;
+    if (rc) {
+        (void) hipDeviceSynchronize();
+        return rc;
+    }
+    for (size_t i = 0; i < net->out_names.size(); ++i) {
+        if (!outputs[i]) continue;
+        const Tensor &t = net->tensors[net->out_names[i]];
+        if (outputs[i] != t.dev) ONRT_HIP(hipMemcpyAsync(outputs[i], t.dev, t.bytes, hipMemcpyDeviceToDevice, nullptr));
+    }
+    return ONRT_OK;
+}
+
 ONRT_API int onrt_net_run(onrt_net_t *net, const void *const *inputs, void *const *outputs) {
     if (!net || (!inputs && !net->in_names.empty()) || (!outputs && !net->out_names.empty())) return fail(ONRT_ERR_ARG, "run: null argument");
     if (net->plan_only) return fail(ONRT_ERR_ARG, "run: this net is a plan (onrt_net_plan_buf): load it to run it");

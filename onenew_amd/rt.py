@@ -7,7 +7,7 @@ import numpy as np
 from . import hip
 
 EXPORTS = ["onrt_last_error", "onrt_net_load_file", "onrt_net_load_buf", "onrt_net_free", "onrt_net_io_count",
-           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf",
+           "onrt_net_io_info", "onrt_net_op_count", "onrt_net_op_info", "onrt_net_operand", "onrt_net_run", "onrt_net_enqueue", "onrt_net_fused_count", "onrt_net_graph_launches", "onrt_net_plan_buf",
            "onrt_net_folded_activations", "onrt_net_fused_attentions", "onrt_net_fused_linears", "onrt_net_fused_skips", "onrt_net_fused_ir_blocks", "onrt_net_fused_pairs", "onrt_net_quantised_links", "onrt_net_tune_tiles", "onrt_net_get_tiles", "onrt_net_set_tiles", "onrt_one_set_tiles", "onrt_one_quantise"]
 
 _lib = None
@@ -51,6 +51,7 @@ def load():
     L.onrt_net_quantised_links.argtypes = [vp, i32p]
     L.onrt_net_operand.argtypes = [vp, C.c_char_p, i32p, i32p, C.POINTER(vp)]
     L.onrt_net_run.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
+    L.onrt_net_enqueue.argtypes = [vp, C.POINTER(vp), C.POINTER(vp)]
     L.onrt_net_tune_tiles.argtypes = [vp, C.c_int32, i32p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.onrt_net_get_tiles.argtypes = [vp, i32p]
     L.onrt_net_set_tiles.argtypes = [vp, i32p]
@@ -245,6 +246,13 @@ class Net:
         ins = (vp * max(1, len(in_ptrs)))(*[vp(p) for p in in_ptrs])
         outs = (vp * max(1, len(out_ptrs)))(*[vp(p or 0) for p in out_ptrs])
         _check(load().onrt_net_run(self._h, ins, outs), "onrt_net_run")
+
+    def enqueue_raw(self, in_ptrs, out_ptrs):
+        """run_raw without the wait at the end: device addresses only, results complete when the default stream is"""
+        vp = C.c_void_p
+        ins = (vp * max(1, len(in_ptrs)))(*[vp(p) for p in in_ptrs])
+        outs = (vp * max(1, len(out_ptrs)))(*[vp(p or 0) for p in out_ptrs])
+        _check(load().onrt_net_enqueue(self._h, ins, outs), "onrt_net_enqueue")
 
     def run(self, *arrays):
         """numpy inputs in input order -> list of numpy outputs"""

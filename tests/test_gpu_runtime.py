@@ -270,6 +270,40 @@ def test_inverted_residual_blocks_run_as_one_call(torch_dev, monkeypatch):
     small.close()
 
 
+def test_inferences_queued_without_a_wait(torch_dev, monkeypatch):
+    """onrt_net_enqueue: the same inference queued on the default stream, no wait at its end.  Three of them back to back
+    on the net's own buffers (nothing copied) and on caller tensors (copies queued in stream order) give the bits of
+    onrt_net_run; host memory and a net with a stream of its own are refused"""
+    torch = torch_dev
+    data, ins = one_models.resnet_block()
+    net = rt.Net(data)
+    (want,) = net.run(*ins)
+    x = torch.from_numpy(ins[0]).cuda()
+    y = torch.zeros(want.shape, dtype=torch.float32, device="cuda")
+    for _ in range(3):
+        net.enqueue_raw([x.data_ptr()], [y.data_ptr()])
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), want)
+    (_, in_dev), (_, out_dev) = net.operand(net.inputs[0][0]), net.operand(net.outputs[0][0])
+    x2 = (ins[0] * np.float32(0.5) - np.float32(0.25)).astype(np.float32)
+    (want2,) = net.run(x2)                       # leaves x2 in the net's input buffer
+    for _ in range(3):
+        net.enqueue_raw([in_dev], [out_dev])
+    torch.cuda.synchronize()
+    assert np.array_equal(net.fetch(net.outputs[0][0]).reshape(want2.shape), want2)
+    with pytest.raises(rt.OnrtError):
+        net.enqueue_raw([ins[0].ctypes.data], [y.data_ptr()])
+    host_out = np.empty(want.shape, np.float32)
+    with pytest.raises(rt.OnrtError):
+        net.enqueue_raw([x.data_ptr()], [host_out.ctypes.data])
+    net.close()
+    monkeypatch.setenv("ONENEW_RT_GRAPH", "1")
+    graphed = rt.Net(data)
+    with pytest.raises(rt.OnrtError):
+        graphed.enqueue_raw([x.data_ptr()], [y.data_ptr()])
+    graphed.close()
+
+
 def test_convolution_pairs_run_as_one_call(torch_dev, monkeypatch):
     """Conv (3x3) -> Conv (1x1) of two ResNet-style bottlenecks as one call of the Conv plugin's eval_pair / eval_pair_relu
     each, where the plugin recommends it: the pair of the first block without an Add (the projection on the skip path took
