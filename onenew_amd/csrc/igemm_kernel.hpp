@@ -314,9 +314,11 @@ __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
 // RES: the kernel variant for the last convolution of a residual block; the element of p.res at each output's place
 // is added after the activation (add_res).  All of a wavefront's addends are requested at once, ahead of the bias:
 // one memory round trip, paid for in registers, which is why the variant is a kernel of its own.
-template <int DT, int EPI, int TM, int TN, bool RES, class ACC>
+// sbias, when not null: this wavefront's rows of the per-row bias in LDS, where the kernel put them before its K loop
+// (-0.0f for a launch without one), so that the store does not begin with a trip to memory.
+template <int DT, int EPI, int TM, int TN, bool RES, bool BIAS_LDS = false, class ACC>
 __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][TN], int batch, int m_wave, int n_wave,
-                                           int li, int lh) {
+                                           int li, int lh, const float *sbias = nullptr) {
     const int esz = (DT == DT_I8 && p.out_s8) ? 1 : 4;
     const rsrc_t rc = make_rsrc(reinterpret_cast<const char *>(p.C) + (size_t) batch * p.c_batch_stride * esz,
                                 RSRC_RANGE);
@@ -441,30 +443,48 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                 }
         }
         float bias_m[TM][16];
+        if constexpr (BIAS_LDS) {
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
+            for (int a = 0; a < TM; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                bias_m[a][r] = buf_load_f32(rbias_m, lh16, (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u);
-#pragma unroll
-        for (int a = 0; a < TM; ++a)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);   // row of lanes with lh == 0
-                const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
-#pragma unroll
-                for (int b = 0; b < TN; ++b) {
-                    float v = acc[a][b][r];
-                    // bias after the full sum; absent bias must not touch the value (the sign of a zero sum)
-                    const float vm = __fadd_rn(v, bias_m[a][r]), vn = __fadd_rn(v, bias_n[b]);
-                    v = bias_m_on ? vm : bias_n_on ? vn : v;
-                    v = act_fast<EPI>(v, p.ep);
-                    if constexpr (RES)
-                        v = add_res(v, rv[a][r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
-                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff[b] : OOB,
-                                                          (unsigned) m_uni * row_bytes, 0);
+                for (int q = 0; q < 4; ++q) {
+                    const float4 t = *reinterpret_cast<const float4 *>(sbias + a * 32 + 8 * q + 4 * lh);
+                    bias_m[a][4 * q + 0] = t.x; bias_m[a][4 * q + 1] = t.y; bias_m[a][4 * q + 2] = t.z; bias_m[a][4 * q + 3] = t.w;
                 }
-            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    bias_m[a][r] = buf_load_f32(rbias_m, lh16, (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u);
+        }
+        // One add per value whatever the bias: the addend is the row's or the column's bias, or -0.0f, which leaves every
+        // value as it is (the sign of a zero sum included).  Rows are tested against M in the last row tile only.
+        float bias_sel[TN];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) bias_sel[b] = bias_n_on ? bias_n[b] : -0.0f;
+        auto store_rows = [&](auto edge) __attribute__((always_inline)) {
+            constexpr bool EDGE = decltype(edge)::value;
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);   // row of lanes with lh == 0
+                    const bool row_ok = !EDGE || m_uni + 4 * lh < p.M;
+#pragma unroll
+                    for (int b = 0; b < TN; ++b) {
+                        // bias after the full sum
+                        float v = __fadd_rn(acc[a][b][r], (BIAS_LDS ? !bias_n_on : bias_m_on) ? bias_m[a][r] : bias_sel[b]);
+                        v = act_fast<EPI>(v, p.ep);
+                        if constexpr (RES)
+                            v = add_res(v, rv[a][r][b], p.res_relu, (col_voff[b] + (unsigned) m_uni * row_bytes) >> 2, p.res_body);
+                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rc, row_ok ? col_voff[b] : OOB,
+                                                              (unsigned) m_uni * row_bytes, 0);
+                    }
+                }
+        };
+        if (m_edge) store_rows(std::true_type{});
+        else store_rows(std::false_type{});
     }
 }
 
@@ -943,6 +963,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     typedef typename Traits<DT>::acc_t acc_t;
 
     __shared__ uint4 lds[2][A_LDS + B_LDS];
+    // the tile's rows of a per-row bias (fp32 / 16-bit operand kernels): requested first of all, in LDS before the K loop
+    constexpr bool BIAS_LDS = DT != DT_I8 && !PW2;
+    __shared__ __attribute__((aligned(16))) float s_bias[BIAS_LDS ? BM : 4];
 
     const int tid = threadIdx.x;
     // the wavefront index is uniform; saying so keeps everything derived from it in scalar registers
@@ -1158,10 +1181,19 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     Operands op0, op1;
     constexpr std::true_type CHECKED{};
     constexpr std::false_type UNCHECKED{};
+    float bias_row = -0.0f;   // the addend that changes nothing
+    if constexpr (BIAS_LDS) {
+        const bool on = p.bias_mode == BIAS_M;
+        const float bv = buf_load_f32(make_rsrc(p.bias, on ? (unsigned) (p.M * 4) : 0u), tid < BM ? (unsigned) (m0 + tid) * 4u : OOB, 0);
+        bias_row = on ? bv : -0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(0, i);
     issue(0, CHECKED, std::integral_constant<int, 0>{});
     stage(0, 0, CHECKED, std::integral_constant<int, 0>{});
+    if constexpr (BIAS_LDS) {
+        if (tid < BM) s_bias[tid] = bias_row;   // read after the K loop, many barriers from here
+    }
     // tiles 1 .. PF: tile t into set t % PF
     [&]<int... T>(std::integer_sequence<int, T...>) __attribute__((always_inline)) {
         ((void) ([&]() __attribute__((always_inline)) {
@@ -1318,12 +1350,12 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     }
     switch (p.ep.act) {
         case NOT_ACT:
-        case RELU6: write_tile<DT, EPI_NONE, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
-        case RELU: write_tile<DT, EPI_RELU, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
-        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case RELU6: write_tile<DT, EPI_NONE, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
+        case RELU: write_tile<DT, EPI_RELU, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
+        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
         case SILU:
-        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
-        default: write_tile<DT, EPI_GENERIC, TM, TN, RES>(p, acc, batch, m_wave, n_wave, li, lh); break;
+        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
+        default: write_tile<DT, EPI_GENERIC, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
     }
 }
 
