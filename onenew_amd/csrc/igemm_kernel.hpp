@@ -314,7 +314,7 @@ __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
 // RES: the kernel variant for the last convolution of a residual block; the element of p.res at each output's place
 // is added after the activation (add_res).  All of a wavefront's addends are requested at once, ahead of the bias:
 // one memory round trip, paid for in registers, which is why the variant is a kernel of its own.
-// sbias, when not null: this wavefront's rows of the per-row bias in LDS, where the kernel put them before its K loop
+// sbias, when not null: this wavefront's rows of the per-row bias in LDS, where the kernel put them after its K loop
 // (-0.0f for a launch without one), so that the store does not begin with a trip to memory.
 template <int DT, int EPI, int TM, int TN, bool RES, bool BIAS_LDS = false, class ACC>
 __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][TN], int batch, int m_wave, int n_wave,
@@ -844,14 +844,18 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
 // unit one MFMA each), so the result has the bits of the two launches it replaces when those use this tile.
 // tl: LDS of at least 16 * 64 * 16 bytes that no wavefront reads any more (the caller has synchronised).
 template <int EPI, bool RES>
-__device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &acc1, uint4 *tl, int n0, int wm, int wn, int li, int lh) {
+__device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &acc1, uint4 *tl, const float *sbias, int n0, int wm, int wn,
+                                          int li, int lh) {
     const unsigned lh16 = (unsigned) lh * 16u;
     const int cmid = p.M;
-    // the first product's bias: rows 8 (r / 4) + 4 lh + r % 4 of the wavefront's 32
-    const rsrc_t rb1 = make_rsrc(p.bias, p.bias_mode == BIAS_M ? (unsigned) (cmid * 4) : 0u);
+    // the first product's bias, rows 8 (r / 4) + 4 lh + r % 4 of the wavefront's 32: requested before the K loop, in LDS,
+    // -0.0f (the addend that changes nothing, not even the sign of a zero sum) where there is none
     float b1[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) b1[r] = buf_load_f32(rb1, lh16, (unsigned) (wm * 32 + 8 * (r / 4) + (r % 4)) * 4u);
+    for (int q = 0; q < 4; ++q) {
+        const float4 t = *reinterpret_cast<const float4 *>(sbias + wm * 32 + 8 * q + 4 * lh);
+        b1[4 * q + 0] = t.x; b1[4 * q + 1] = t.y; b1[4 * q + 2] = t.z; b1[4 * q + 3] = t.w;
+    }
     // A of the second product, re-laid once by pack_pw2_launch into the order this loop reads it: for every block of 64
     // rows, half wm and step s the 64 lanes' 16 bytes side by side (lane (li, lh): row block * 64 + wm * 32 + li, unit
     // 2 s + lh; zeros beyond m2 rows and M columns), so a load instruction is one contiguous KiB
@@ -861,7 +865,6 @@ __device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &ac
     uint4 wa[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) wa[s] = buf_load_b128(rw2, lane16, (unsigned) (wm * 8 + s) * 1024u);
-    const unsigned bias1_mask = p.bias_mode == BIAS_M ? 0xffffffffu : 0u;
     // the first product's activation is none, Relu or Clip (the launcher refuses others): apply_act's comparisons as
     // selects under two uniform flags, so that the sixteen values take no branch
     const bool lo_on = p.ep.act == RELU || p.ep.act == CLIP, hi_on = p.ep.act == CLIP;
@@ -872,11 +875,7 @@ __device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &ac
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int r = 4 * q + j;
-            const float a = acc1[r];
-            // an absent bias must not touch the value (the sign of a zero sum): a select between bit patterns, which
-            // the compiler does not turn into a branch around the addition
-            const unsigned ab = __float_as_uint(a), sb = __float_as_uint(__fadd_rn(a, b1[r]));
-            float x = __uint_as_float(ab ^ ((ab ^ sb) & bias1_mask));
+            float x = __fadd_rn(acc1[r], b1[r]);
             x = (lo_on & !(x > lo)) ? lo : x;
             x = (hi_on & !(x < hi)) ? hi : x;
             v[j] = wm * 32 + 8 * q + 4 * lh + j < cmid ? x : 0.0f;
@@ -963,8 +962,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     typedef typename Traits<DT>::acc_t acc_t;
 
     __shared__ uint4 lds[2][A_LDS + B_LDS];
-    // the tile's rows of a per-row bias (fp32 / 16-bit operand kernels): requested first of all, in LDS before the K loop
-    constexpr bool BIAS_LDS = DT != DT_I8 && !PW2;
+    // the tile's rows of a per-row bias (fp32 / 16-bit operand kernels; with PW2 the first product's): requested with the
+    // first operand tiles, in LDS when the K loop is over
+    constexpr bool BIAS_LDS = DT != DT_I8;
     __shared__ __attribute__((aligned(16))) float s_bias[BIAS_LDS ? BM : 4];
 
     const int tid = threadIdx.x;
@@ -1181,19 +1181,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     Operands op0, op1;
     constexpr std::true_type CHECKED{};
     constexpr std::false_type UNCHECKED{};
-    float bias_row = -0.0f;   // the addend that changes nothing
-    if constexpr (BIAS_LDS) {
-        const bool on = p.bias_mode == BIAS_M;
-        const float bv = buf_load_f32(make_rsrc(p.bias, on ? (unsigned) (p.M * 4) : 0u), tid < BM ? (unsigned) (m0 + tid) * 4u : OOB, 0);
-        bias_row = on ? bv : -0.0f;
-    }
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(0, i);
     issue(0, CHECKED, std::integral_constant<int, 0>{});
     stage(0, 0, CHECKED, std::integral_constant<int, 0>{});
-    if constexpr (BIAS_LDS) {
-        if (tid < BM) s_bias[tid] = bias_row;   // read after the K loop, many barriers from here
-    }
     // tiles 1 .. PF: tile t into set t % PF
     [&]<int... T>(std::integer_sequence<int, T...>) __attribute__((always_inline)) {
         ((void) ([&]() __attribute__((always_inline)) {
@@ -1202,6 +1193,13 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
             issue(T + 1, CHECKED, std::integral_constant<int, (T + 1) % PF>{});
         }()), ...);
     }(std::make_integer_sequence<int, PF>{});
+    // the tile's bias rows, behind the first operand loads (nothing waits for them before the K loop is over)
+    float bias_row = -0.0f;   // the addend that changes nothing
+    if constexpr (BIAS_LDS) {
+        const bool on = p.bias_mode == BIAS_M;
+        const float bv = buf_load_f32(make_rsrc(p.bias, on ? (unsigned) (p.M * 4) : 0u), tid < BM ? (unsigned) (m0 + tid) * 4u : OOB, 0);
+        bias_row = on ? bv : -0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(PF + 1, i);   // for the first load of the loop: tile 1 + PF
     __syncthreads();
@@ -1250,18 +1248,22 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     for (; kt < n_plain; kt += U) group(kt, UNCHECKED, std::false_type{});
     for (; kt + U <= k_tiles; kt += U) group(kt, CHECKED, std::false_type{});
     if (kt < k_tiles) group(kt, CHECKED, std::true_type{});
+    if constexpr (BIAS_LDS) {
+        if (tid < BM) s_bias[tid] = bias_row;
+        if constexpr (!PW2) __syncthreads();
+    }
 
     if constexpr (PW2) {
         // the launcher gives this variant one row tile, all of K and no batch: the tile is the whole first product
         static_assert(sizeof(lds) >= 16 * 64 * 16, "the tile as a B operand fits the operand buffers");
-        __syncthreads();   // every wavefront is done with the operand buffers
+        __syncthreads();   // every wavefront is done with the operand buffers (and the bias rows are in place)
         uint4 *tl = &lds[0][0];
         switch (p.ep2.act) {
             case NOT_ACT:
-            case RELU6: pw2_stage<EPI_NONE, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
-            case RELU: pw2_stage<EPI_RELU, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
-            case CLIP: pw2_stage<EPI_CLIP, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
-            default: pw2_stage<EPI_GENERIC, RES>(p, acc[0][0], tl, n0, wm, wn, li, lh); break;
+            case RELU6: pw2_stage<EPI_NONE, RES>(p, acc[0][0], tl, s_bias, n0, wm, wn, li, lh); break;
+            case RELU: pw2_stage<EPI_RELU, RES>(p, acc[0][0], tl, s_bias, n0, wm, wn, li, lh); break;
+            case CLIP: pw2_stage<EPI_CLIP, RES>(p, acc[0][0], tl, s_bias, n0, wm, wn, li, lh); break;
+            default: pw2_stage<EPI_GENERIC, RES>(p, acc[0][0], tl, s_bias, n0, wm, wn, li, lh); break;
         }
         return;
     }
