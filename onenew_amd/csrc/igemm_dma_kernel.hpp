@@ -335,12 +335,12 @@ __global__ __launch_bounds__(THREADS) void igemm_dma_kernel(const IgemmParams p)
     }
     switch (p.ep.act) {
         case NOT_ACT:
-        case RELU6: write_tile<DT, EPI_NONE, TM, TN, false>(p, acc, 0, m_wave, n_wave, li, lh); break;
-        case RELU: write_tile<DT, EPI_RELU, TM, TN, false>(p, acc, 0, m_wave, n_wave, li, lh); break;
-        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, false>(p, acc, 0, m_wave, n_wave, li, lh); break;
+        case RELU6: write_tile<DT, EPI_NONE, TM, TN, false, DT == DT_I8>(p, acc, 0, m_wave, n_wave, li, lh, rows + (m_wave - m0), rows + BM + (m_wave - m0)); break;
+        case RELU: write_tile<DT, EPI_RELU, TM, TN, false, DT == DT_I8>(p, acc, 0, m_wave, n_wave, li, lh, rows + (m_wave - m0), rows + BM + (m_wave - m0)); break;
+        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, false, DT == DT_I8>(p, acc, 0, m_wave, n_wave, li, lh, rows + (m_wave - m0), rows + BM + (m_wave - m0)); break;
         case SILU:
-        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, false>(p, acc, 0, m_wave, n_wave, li, lh); break;
-        default: write_tile<DT, EPI_GENERIC, TM, TN, false>(p, acc, 0, m_wave, n_wave, li, lh); break;
+        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, false, DT == DT_I8>(p, acc, 0, m_wave, n_wave, li, lh, rows + (m_wave - m0), rows + BM + (m_wave - m0)); break;
+        default: write_tile<DT, EPI_GENERIC, TM, TN, false, DT == DT_I8>(p, acc, 0, m_wave, n_wave, li, lh, rows + (m_wave - m0), rows + BM + (m_wave - m0)); break;
     }
 #endif
 }

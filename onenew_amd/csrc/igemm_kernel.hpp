@@ -314,11 +314,13 @@ __device__ __forceinline__ int requant_s8(float y, float inv_scale) {
 // RES: the kernel variant for the last convolution of a residual block; the element of p.res at each output's place
 // is added after the activation (add_res).  All of a wavefront's addends are requested at once, ahead of the bias:
 // one memory round trip, paid for in registers, which is why the variant is a kernel of its own.
-// sbias, when not null: this wavefront's rows of the per-row bias in LDS, where the kernel put them after its K loop
-// (-0.0f for a launch without one), so that the store does not begin with a trip to memory.
+// BIAS_LDS: the per-row constants of this wavefront's rows wait in LDS, where the kernel put them when its K loop was
+// over, so that the store does not begin with a trip to memory: sbias the per-row bias (-0.0f for a launch without
+// one); for int8 operands the de-quantisation factors weight_aux / 127, divided once per row and not by every lane,
+// and srow2 the int32 biases as floats.
 template <int DT, int EPI, int TM, int TN, bool RES, bool BIAS_LDS = false, class ACC>
 __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][TN], int batch, int m_wave, int n_wave,
-                                           int li, int lh, const float *sbias = nullptr) {
+                                           int li, int lh, const float *sbias = nullptr, const float *srow2 = nullptr) {
     const int esz = (DT == DT_I8 && p.out_s8) ? 1 : 4;
     const rsrc_t rc = make_rsrc(reinterpret_cast<const char *>(p.C) + (size_t) batch * p.c_batch_stride * esz,
                                 RSRC_RANGE);
@@ -345,16 +347,32 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
         const rsrc_t racc = make_rsrc(p.acc_out ? p.acc_out + (size_t) batch * p.c_batch_stride : nullptr,
                                       p.acc_out ? RSRC_RANGE : 0u);
         const unsigned row_bytes4 = (unsigned) p.c_stride_m * 4u;
-        float aux[TM][16];
-        int b32[TM][16];
+        float aux[TM][16];    // weight_aux / 127 of each of the lane's rows
+        float fb32[TM][16];   // and the row's int32 bias as a float
+        if constexpr (BIAS_LDS) {
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
+            for (int a = 0; a < TM; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const unsigned soff = (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u;
-                aux[a][r] = buf_load_f32(raux, lh16, soff);
-                b32[a][r] = (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
-            }
+                for (int q = 0; q < 4; ++q) {
+                    const float4 c = *reinterpret_cast<const float4 *>(sbias + a * 32 + 8 * q + 4 * lh);
+                    const float4 f = *reinterpret_cast<const float4 *>(srow2 + a * 32 + 8 * q + 4 * lh);
+                    aux[a][4 * q] = c.x; aux[a][4 * q + 1] = c.y; aux[a][4 * q + 2] = c.z; aux[a][4 * q + 3] = c.w;
+                    fb32[a][4 * q] = f.x; fb32[a][4 * q + 1] = f.y; fb32[a][4 * q + 2] = f.z; fb32[a][4 * q + 3] = f.w;
+                }
+        } else {
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const unsigned soff = (unsigned) (m_wave + a * 32 + 8 * (r / 4) + (r % 4)) * 4u;
+                    aux[a][r] = buf_load_f32(raux, lh16, soff);
+                    fb32[a][r] = (float) (int) __builtin_amdgcn_raw_buffer_load_b32(rb32, lh16, soff, 0);
+                }
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) aux[a][r] = __fdiv_rn(aux[a][r], 127.0f);
+        }
         unsigned col_voff4[TN];
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
@@ -387,8 +405,8 @@ __device__ __forceinline__ void write_tile(const IgemmParams &p, ACC (&acc)[TM][
                 const int m_uni = m_wave + a * 32 + 8 * (r / 4) + (r % 4);
                 const bool row_ok = !m_edge || m_uni + 4 * lh < p.M;
                 // conv.c:1041-1056: acc * s, + bias, * (aux / 127): three separately rounded operations
-                const float coeff = __fdiv_rn(aux[a][r], 127.0f);
-                const float fb = (float) b32[a][r];
+                const float coeff = aux[a][r];
+                const float fb = fb32[a][r];
 #pragma unroll
                 for (int b = 0; b < TN; ++b) {
                     const int av = acc[a][b][r];
@@ -962,10 +980,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     typedef typename Traits<DT>::acc_t acc_t;
 
     __shared__ uint4 lds[2][A_LDS + B_LDS];
-    // the tile's rows of a per-row bias (fp32 / 16-bit operand kernels; with PW2 the first product's): requested with the
-    // first operand tiles, in LDS when the K loop is over
-    constexpr bool BIAS_LDS = DT != DT_I8;
-    __shared__ __attribute__((aligned(16))) float s_bias[BIAS_LDS ? BM : 4];
+    // the tile's rows of the store's per-row constants: the bias (fp32 / 16-bit operand kernels; with PW2 the first
+    // product's), or weight_aux / 127 followed by the int32 bias as a float (int8).  Requested with the first operand
+    // tiles, in LDS when the K loop is over
+    constexpr bool BIAS_LDS = true;
+    __shared__ __attribute__((aligned(16))) float s_bias[DT == DT_I8 ? 2 * BM : BM];
 
     const int tid = threadIdx.x;
     // the wavefront index is uniform; saying so keeps everything derived from it in scalar registers
@@ -1195,10 +1214,17 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     }(std::make_integer_sequence<int, PF>{});
     // the tile's bias rows, behind the first operand loads (nothing waits for them before the K loop is over)
     float bias_row = -0.0f;   // the addend that changes nothing
-    if constexpr (BIAS_LDS) {
-        const bool on = p.bias_mode == BIAS_M;
-        const float bv = buf_load_f32(make_rsrc(p.bias, on ? (unsigned) (p.M * 4) : 0u), tid < BM ? (unsigned) (m0 + tid) * 4u : OOB, 0);
-        bias_row = on ? bv : -0.0f;
+    float aux_row = 0.0f;
+    {
+        const unsigned row_off = tid < BM ? (unsigned) (m0 + tid) * 4u : OOB;   // rows beyond M read as zero
+        if constexpr (DT == DT_I8) {
+            aux_row = buf_load_f32(make_rsrc(p.weight_aux, p.weight_aux ? (unsigned) (p.M * 4) : 0u), row_off, 0);
+            bias_row = (float) (int) __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(p.bias32, p.bias32 ? (unsigned) (p.M * 4) : 0u), row_off, 0, 0);
+        } else {
+            const bool on = p.bias_mode == BIAS_M;
+            const float bv = buf_load_f32(make_rsrc(p.bias, on ? (unsigned) (p.M * 4) : 0u), row_off, 0);
+            bias_row = on ? bv : -0.0f;
+        }
     }
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) prep_item(PF + 1, i);   // for the first load of the loop: tile 1 + PF
@@ -1248,10 +1274,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
     for (; kt < n_plain; kt += U) group(kt, UNCHECKED, std::false_type{});
     for (; kt + U <= k_tiles; kt += U) group(kt, CHECKED, std::false_type{});
     if (kt < k_tiles) group(kt, CHECKED, std::true_type{});
-    if constexpr (BIAS_LDS) {
-        if (tid < BM) s_bias[tid] = bias_row;
-        if constexpr (!PW2) __syncthreads();
+    if (tid < BM) {
+        if constexpr (DT == DT_I8) {
+            s_bias[tid] = __fdiv_rn(aux_row, 127.0f);   // conv.c:1049-1056: the factor is weight_aux / 127, rounded once
+            s_bias[BM + tid] = bias_row;
+        } else {
+            s_bias[tid] = bias_row;
+        }
     }
+    if constexpr (!PW2) __syncthreads();
 
     if constexpr (PW2) {
         // the launcher gives this variant one row tile, all of K and no batch: the tile is the whole first product
@@ -1340,24 +1371,24 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (
             __syncthreads();   // every wavefront is done with the operand buffers
             switch (p.ep.act) {
                 case NOT_ACT:
-                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
-                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
-                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case RELU6: write_tile_nhwc_s8<EPI_NONE, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid, s_bias); break;
+                case RELU: write_tile_nhwc_s8<EPI_RELU, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid, s_bias); break;
+                case CLIP: write_tile_nhwc_s8<EPI_CLIP, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid, s_bias); break;
                 case SILU:
-                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
-                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid); break;
+                case ONHIP_ACT_GELU_LUT: write_tile_nhwc_s8<EPI_LUT, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid, s_bias); break;
+                default: write_tile_nhwc_s8<EPI_GENERIC, BM, BN, TM, TN, QL>(p, acc, stage, m0, n0, m_wave, n_wave, li, lh, tid, s_bias); break;
             }
             return;
         }
     }
     switch (p.ep.act) {
         case NOT_ACT:
-        case RELU6: write_tile<DT, EPI_NONE, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
-        case RELU: write_tile<DT, EPI_RELU, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
-        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
+        case RELU6: write_tile<DT, EPI_NONE, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM), s_bias + BM + wm * (BM / WM)); break;
+        case RELU: write_tile<DT, EPI_RELU, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM), s_bias + BM + wm * (BM / WM)); break;
+        case CLIP: write_tile<DT, EPI_CLIP, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM), s_bias + BM + wm * (BM / WM)); break;
         case SILU:
-        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
-        default: write_tile<DT, EPI_GENERIC, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM)); break;
+        case ONHIP_ACT_GELU_LUT: write_tile<DT, EPI_LUT, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM), s_bias + BM + wm * (BM / WM)); break;
+        default: write_tile<DT, EPI_GENERIC, TM, TN, RES, BIAS_LDS>(p, acc, batch, m_wave, n_wave, li, lh, s_bias + wm * (BM / WM), s_bias + BM + wm * (BM / WM)); break;
     }
 }
 
