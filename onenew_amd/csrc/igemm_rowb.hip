@@ -21,22 +21,25 @@ namespace onhip {
 // K tile: 16 reduction steps = 2 slabs of 8; A units per row and tile: 4
 constexpr int RB_KT = 16;
 
+// sbias: the per-row bias of this wavefront's 32 rows in LDS (-0.0f, the addend that changes nothing, without one)
 template <int EPI>
-__device__ __forceinline__ void rowb_store(const IgemmParams &p, f32x16 (&acc)[4], int batch, int m_wave, int n_quad, int lh) {
+__device__ __forceinline__ void rowb_store(const IgemmParams &p, f32x16 (&acc)[4], int batch, int m_wave, int n_quad, int lh,
+                                           const float *sbias) {
     const rsrc_t rc = make_rsrc(reinterpret_cast<const char *>(p.C) + (size_t) batch * p.c_batch_stride * 4, RSRC_RANGE);
     const bool col_ok = n_quad < p.N;
     const int nn = col_ok ? n_quad : 0;
     const unsigned col_voff = col_ok ? out_col_offset(p, nn, 4) + (unsigned) (4 * lh) * (unsigned) p.c_stride_m * 4u : OOB;
-    const bool bias_m_on = p.bias_mode == BIAS_M, bias_n_on = p.bias_mode == BIAS_N;
-    const rsrc_t rbias_m = make_rsrc(p.bias, bias_m_on ? (unsigned) (p.M * 4) : 0u);
+    const bool bias_n_on = p.bias_mode == BIAS_N;
     const rsrc_t rbias_n = make_rsrc(p.bias, bias_n_on ? (unsigned) (p.N * 4) : 0u);
     const uint4 bn = buf_load_b128(rbias_n, (unsigned) nn * 4u, 0);
     const float bias_n[4] = {__uint_as_float(bn.x), __uint_as_float(bn.y), __uint_as_float(bn.z), __uint_as_float(bn.w)};
     const bool m_edge = m_wave + 32 > p.M;
     float bias_m[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-        bias_m[r] = buf_load_f32(rbias_m, (unsigned) lh * 16u, (unsigned) (m_wave + 8 * (r / 4) + (r % 4)) * 4u);
+    for (int q = 0; q < 4; ++q) {
+        const float4 t = *reinterpret_cast<const float4 *>(sbias + 8 * q + 4 * lh);
+        bias_m[4 * q + 0] = t.x; bias_m[4 * q + 1] = t.y; bias_m[4 * q + 2] = t.z; bias_m[4 * q + 3] = t.w;
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int m_uni = m_wave + 8 * (r / 4) + (r % 4);   // row of the lanes with lh == 0
@@ -44,9 +47,8 @@ __device__ __forceinline__ void rowb_store(const IgemmParams &p, f32x16 (&acc)[4
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float a = acc[j][r];
-            const float vm = __fadd_rn(a, bias_m[r]), vn = __fadd_rn(a, bias_n[j]);
-            v[j] = act_fast<EPI>(bias_m_on ? vm : bias_n_on ? vn : a, p.ep);
+            // one add whatever the bias: the row's (or -0.0f) unless the launch has a per-column one
+            v[j] = act_fast<EPI>(__fadd_rn(acc[j][r], bias_n_on ? bias_n[j] : bias_m[r]), p.ep);
         }
         // row offset in the vector offset, scalar offset the constant 0: a 128-bit buffer store with a register as its
         // scalar offset gets no gap from the compiler before the next write to its data registers, which on this GPU can
@@ -79,6 +81,7 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
     constexpr int A_SLOTS = BM * 4, A_PER_T = (A_SLOTS + NT - 1) / NT;
     constexpr int A_LD = BM + 1;   // a spare slot per unit row: the four units of a row are stored by neighbouring threads
     __shared__ uint4 lds[2][4 * A_LD];
+    __shared__ __attribute__((aligned(16))) float s_bias[BM];   // the tile's rows of a per-row bias, for the store
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -204,6 +207,13 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
     issue_a(1);
     issue_b(qb1, 1, 0);
     issue_b(qb1, 1, 1);
+    // the bias rows behind the first operand loads; in LDS when the K loop is over
+    float bias_row;
+    {
+        const bool on = p.bias_mode == BIAS_M;
+        const float bv = buf_load_f32(make_rsrc(p.bias, on ? (unsigned) (p.M * 4) : 0u), tid < BM ? (unsigned) (m0 + tid) * 4u : OOB, 0);
+        bias_row = on ? bv : -0.0f;
+    }
     __syncthreads();
     read_a(oa0, 0);
     int kt = 0;
@@ -218,14 +228,17 @@ __global__ __launch_bounds__(64 * WM * WN) void rowb_f32_kernel(const IgemmParam
         rowb_store_partial(p, acc, slice, m_wave, n_quad, lh);
         return;
     }
+    if (tid < BM) s_bias[tid] = bias_row;
+    __syncthreads();
+    const float *sbias = s_bias + wm * 32;
     switch (p.ep.act) {
         case NOT_ACT:
-        case RELU6: rowb_store<EPI_NONE>(p, acc, batch, m_wave, n_quad, lh); break;
-        case RELU: rowb_store<EPI_RELU>(p, acc, batch, m_wave, n_quad, lh); break;
-        case CLIP: rowb_store<EPI_CLIP>(p, acc, batch, m_wave, n_quad, lh); break;
+        case RELU6: rowb_store<EPI_NONE>(p, acc, batch, m_wave, n_quad, lh, sbias); break;
+        case RELU: rowb_store<EPI_RELU>(p, acc, batch, m_wave, n_quad, lh, sbias); break;
+        case CLIP: rowb_store<EPI_CLIP>(p, acc, batch, m_wave, n_quad, lh, sbias); break;
         case SILU:
-        case ONHIP_ACT_GELU_LUT: rowb_store<EPI_LUT>(p, acc, batch, m_wave, n_quad, lh); break;
-        default: rowb_store<EPI_GENERIC>(p, acc, batch, m_wave, n_quad, lh); break;
+        case ONHIP_ACT_GELU_LUT: rowb_store<EPI_LUT>(p, acc, batch, m_wave, n_quad, lh, sbias); break;
+        default: rowb_store<EPI_GENERIC>(p, acc, batch, m_wave, n_quad, lh, sbias); break;
     }
 }
 
