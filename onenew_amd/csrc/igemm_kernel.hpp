@@ -855,10 +855,10 @@ __device__ __forceinline__ void write_partial(const IgemmParams &p, ACC (&acc)[T
 // The workgroup's tile holds every row of the first product (M <= 64) for its 64 columns, so it is the whole B operand
 // of a 1x1 convolution over that result for these columns: out[m2][64] = w2[m2][M] * act(tile + bias).  The tile goes to
 // LDS in the B layout of the K loop ([unit of 4 rows][column][16 B]; a lane's accumulator registers 4q .. 4q+3 are four
-// consecutive rows of one column, i.e. exactly one unit), every wavefront takes the 16 units of its 32 columns into
-// registers once, and then walks the rows of w2 in blocks of 64 (32 per wavefront) with its A operands loaded straight
-// from memory, where they lie in the MFMA's own layout (lane li = row, lanes 32-63 the odd unit of a step; w2 is packed
-// that way once): no LDS traffic and no barrier in this loop.  The reduction runs in the order of the K loop (unit pairs ascending, the four elements of a
+// consecutive rows of one column, i.e. exactly one unit), and every wavefront then walks the rows of w2 in blocks of
+// 64 (32 per wavefront), its B operand read from that tile one step ahead and its A operands loaded straight from
+// memory, where they lie in the MFMA's own layout (lane li = row, lanes 32-63 the odd unit of a step; w2 is packed
+// that way once): no barrier in this loop.  The reduction runs in the order of the K loop (unit pairs ascending, the four elements of a
 // unit one MFMA each), so the result has the bits of the two launches it replaces when those use this tile.
 // tl: LDS of at least 16 * 64 * 16 bytes that no wavefront reads any more (the caller has synchronised).
 template <int EPI, bool RES>
@@ -901,9 +901,10 @@ __device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &ac
         tl[(wm * 8 + 2 * q + lh) * 64 + wn * 32 + li] = make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3]));
     }
     __syncthreads();
-    uint4 tb[8];
-#pragma unroll
-    for (int s = 0; s < 8; ++s) tb[s] = tl[(2 * s + lh) * 64 + wn * 32 + li];
+    // B of the second product stays in LDS: the 16 bytes of a step are read one step ahead (eight registers, not the 32
+    // of the whole operand, which cost the kernel a wavefront per SIMD)
+    const uint4 *tbp = tl + lh * 64 + wn * 32 + li;
+    uint4 tb_next = tbp[0];
 
     const rsrc_t rc = make_rsrc(p.C, RSRC_RANGE);
     const rsrc_t rres = make_rsrc(RES ? p.res : nullptr, RES ? RSRC_RANGE : 0u);
@@ -935,8 +936,10 @@ __device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &ac
         const unsigned next_soff = (unsigned) (((mb + 1) * 2 + wm) * 8) * 1024u;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
+            const uint4 tb = tb_next;
+            tb_next = tbp[((s + 1) & 7) * 128];   // step s + 1, or step 0 of the next block of rows
 #pragma unroll
-            for (int part = 0; part < 4; ++part) Traits<DT_F32>::mma_part(acc2, wa[s], tb[s], part);
+            for (int part = 0; part < 4; ++part) Traits<DT_F32>::mma_part(acc2, wa[s], tb, part);
             wa[s] = buf_load_b128(rw2, next_voff, next_soff + 1024u * s);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -955,7 +958,7 @@ __device__ __forceinline__ void pw2_stage(const IgemmParams &p, const f32x16 &ac
 
 // ---- the kernel --------------------------------------------------------------------------------
 template <int DT, int BL, int BM, int BN, int WM, int WN, int PF = 1, bool RES = false, bool PW2 = false>
-__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? (RES ? 3 : 4) : 1))) void igemm_kernel(const IgemmParams p) {
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(PW2 ? 4 : 1))) void igemm_kernel(const IgemmParams p) {
     static_assert(!PW2 || (DT == DT_F32 && BM == 64 && BN == 64 && WM == 2 && WN == 2), "the second product exists for fp32 tiles of 64 x 64");
     static_assert(!RES || DT == DT_F32 || DT == DT_I8, "the residual store exists for fp32 and int8 operands (fp32 results)");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
